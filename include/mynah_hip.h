@@ -1,0 +1,283 @@
+/* mynah_hip.h -- C ABI of the gfx950 (MI355X) HIP backend for Mynah TTS's decode-step kernels.
+ *
+ * Plain C: pointers, sizes, ints.  No C++ or framework types cross this boundary.
+ * Conventions are the reference seam's (src/backend.c:137-139, :472):
+ *   - every call returns 0 on success, -1 on failure, and writes a NUL-terminated message into
+ *     `error` (capacity `error_capacity`; either may be NULL/0);
+ *   - `state` is the opaque handle produced by mynah_backend_hip_open and destroyed by the close
+ *     function it hands back;
+ *   - "dev" pointers are device memory from mynah_hip_dev_alloc; weights, biases and LayerNorm
+ *     gains are HOST pointers to immutable memory that outlives the backend, converted and cached
+ *     on the device the first time they are seen, keyed by (address, byte size)
+ *     (gpu/cuda/backend_cuda.cu:133-143,193-219);
+ *   - resident ops enqueue on one internal stream and return without synchronising; only
+ *     mynah_hip_sync, mynah_hip_d2h, mynah_hip_download, mynah_hip_argmax_dev and the host-pointer
+ *     matmul/sgemm block.
+ *
+ * Section 1 mirrors, symbol for symbol, what src/backend.c declares for a GPU backend
+ * (src/backend.c:72-135) so `#if defined(MYNAH_ENABLE_HIP)` blocks can bind it unchanged.
+ * Section 2 fills the gap the single-stream seam leaves: weight-stationary batched twins and a
+ * whole-step entry for B concurrent streams (the reference only batches on the CPU,
+ * src/graph.c:3127-3284, src/qmat.c:820-888).
+ */
+#ifndef MYNAH_HIP_H
+#define MYNAH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Section 1 -- the reference seam (src/backend.h)
+ * ------------------------------------------------------------------------------------------ */
+
+/* src/backend.h:10-25 */
+typedef int (*mynah_backend_matmul_fn)(void *, const float *, float *, size_t, size_t, size_t,
+                                       const float *, const float *, char *, size_t);
+typedef void (*mynah_backend_close_fn)(void *);
+typedef int (*mynah_backend_self_test_fn)(void *, char *, size_t);
+typedef int (*mynah_backend_sgemm_fn)(void *, int trans_a, int trans_b, size_t m, size_t n, size_t k,
+                                      float alpha, const float *a, size_t lda, const float *b, size_t ldb,
+                                      float beta, float *c, size_t ldc, char *, size_t);
+
+/* Counterpart of mynah_backend_cuda_open (src/backend.c:106-109, gpu/cuda/backend_cuda.cu:540-565).
+ * matmul: out[rows,ow] = in[rows,iw] W[ow,iw]^T + bias, all HOST pointers, synchronous
+ *         (src/backend.h:32-35).  rows <= 16 takes the quantized matvec selected by MYNAH_QUANT,
+ *         like mynah_qmat_linear_resolved (src/qmat.c:768-818); more rows use the f32 GEMM.
+ * sgemm:  row-major C = alpha op(A) op(B) + beta C on HOST pointers (src/backend.h:15-25).
+ * self_test: the matmul/sgemm KATs of gpu/cuda/backend_cuda.cu:514-529 and the resident-op KATs
+ *         of gpu/metal/backend_metal_ops.m:1038-1107 (codec ops excluded). */
+int mynah_backend_hip_open(void **state, mynah_backend_matmul_fn *matmul, mynah_backend_sgemm_fn *sgemm,
+                           mynah_backend_close_fn *close, mynah_backend_self_test_fn *self_test,
+                           char *error, size_t error_capacity);
+
+/* src/backend.h:181-186 */
+int mynah_hip_dev_alloc(void *state, size_t n, float **dev_ptr, char *error, size_t error_capacity);
+void mynah_hip_dev_free(void *state, float *dev_ptr);
+/* src/backend.h:156-163.  h2d is asynchronous on the backend stream (the source is staged through
+ * pinned memory before the call returns); d2h synchronises first. */
+int mynah_hip_h2d(void *state, const float *host, float *dev_ptr, size_t n, char *error, size_t error_capacity);
+int mynah_hip_d2h(void *state, const float *dev_ptr, float *host, size_t n, char *error, size_t error_capacity);
+/* src/backend.h:78-85: upload returns a pointer into backend-owned scratch, valid until the next upload. */
+int mynah_hip_upload(void *state, const float *host, size_t n, float **dev_ptr, char *error, size_t error_capacity);
+int mynah_hip_download(void *state, const float *dev_ptr, float *host, size_t n, char *error, size_t error_capacity);
+/* src/backend.h:86-93 */
+int mynah_hip_sync(void *state, char *error, size_t error_capacity);
+int mynah_hip_batch_begin(void *state, char *error, size_t error_capacity);
+
+/* src/backend.h:53-58: in-place resident ops, no copy, no sync.
+ * layer_norm_inplace: gain only, eps 1e-5 (src/graph.c:147-150). */
+int mynah_hip_gelu_inplace(void *state, float *dev_data, size_t n, char *error, size_t error_capacity);
+int mynah_hip_residual_inplace(void *state, float *dev_out, const float *dev_in, size_t n, char *error, size_t error_capacity);
+int mynah_hip_layer_norm_inplace(void *state, const float *dev_in, float *dev_out, const float *gain,
+                                 size_t rows, size_t width, char *error, size_t error_capacity);
+/* out[rows,ow] = in[rows,iw] W[ow,iw]^T + bias; dev in/out, HOST W/bias.  rows <= 16 runs the
+ * weight-stationary quantized matvec (activation quantisation fused), else the f32 GEMM. */
+int mynah_hip_matmul_d2d(void *state, const float *dev_in, float *dev_out, size_t rows, size_t iw, size_t ow,
+                         const float *weight, const float *bias, char *error, size_t error_capacity);
+/* HOST input, dev output (src/backend.h:57). */
+int mynah_hip_matmul_to_dev(void *state, const float *host_in, float *dev_out, size_t rows, size_t iw, size_t ow,
+                            const float *weight, const float *bias, char *error, size_t error_capacity);
+/* src/backend.h:66-71 */
+int mynah_hip_matvec_dev(void *state, const float *dev_in, float *dev_out, size_t K, size_t N,
+                         const float *weight, const float *bias, char *error, size_t error_capacity);
+/* src/backend.h:95-128: device-buffer forms. layer_norm_dev honours `bias` (may be NULL). */
+int mynah_hip_matmul_dev(void *state, const float *dev_in, float *dev_out, size_t rows, size_t iw, size_t ow,
+                         const float *weight, const float *bias, char *error, size_t error_capacity);
+int mynah_hip_sgemm_dev(void *state, int trans_a, int trans_b, size_t m, size_t n, size_t k, float alpha,
+                        const float *dev_a, size_t lda, const float *dev_b, size_t ldb, float beta,
+                        float *dev_c, size_t ldc, char *error, size_t error_capacity);
+int mynah_hip_gelu_dev(void *state, float *dev_data, size_t n, char *error, size_t error_capacity);
+int mynah_hip_layer_norm_dev(void *state, const float *dev_in, float *dev_out, const float *gain,
+                             const float *bias, size_t rows, size_t width, char *error, size_t error_capacity);
+int mynah_hip_softmax_dev(void *state, float *dev_data, size_t rows, size_t cols, size_t valid,
+                          char *error, size_t error_capacity);
+int mynah_hip_residual_add_dev(void *state, float *dev_out, const float *dev_in, size_t n,
+                               char *error, size_t error_capacity);
+
+/* src/backend.h:135-154.  Self: dev_qkv = [q | k | v] (3 * heads * head_width floats); the k and v
+ * parts are first stored at row `position` of the per-layer caches (rows are `cache_stride` floats
+ * apart), then rows [0, valid) are attended.  Cross: read-only caches.  heads * head_width may be
+ * anything up to 4096, head_width <= 1024. */
+int mynah_hip_self_attention_dev(void *state, const float *dev_qkv, float *dev_k_cache, float *dev_v_cache,
+                                 size_t position, size_t cache_stride, size_t valid, size_t heads,
+                                 size_t head_width, float scale, float *dev_out,
+                                 char *error, size_t error_capacity);
+int mynah_hip_cross_attention_dev(void *state, const float *dev_q, const float *dev_k_cache,
+                                  const float *dev_v_cache, size_t valid, size_t cache_stride, size_t heads,
+                                  size_t head_width, float scale, float *dev_out,
+                                  char *error, size_t error_capacity);
+
+/* src/backend.h:165-179.  clip: clamp to [-1, 1], NaN -> 0 (gpu/metal/backend_metal_ops.m:1090-1101).
+ * argmax: candidates i < codebook_size plus eos_id iff allow_eos; strict > from -FLT_MAX, the first
+ * index wins ties (src/backend.c:825-847).  Synchronises and returns one scalar. */
+int mynah_hip_copy_dev(void *state, float *dev_dst, const float *dev_src, size_t n, char *error, size_t error_capacity);
+int mynah_hip_scale_dev(void *state, float *dev_data, size_t n, float scale, char *error, size_t error_capacity);
+int mynah_hip_clip_dev(void *state, float *dev_data, size_t n, char *error, size_t error_capacity);
+int mynah_hip_argmax_dev(void *state, const float *dev_logits, size_t vocab, size_t codebook_size, size_t eos_id,
+                         int allow_eos, unsigned *argmax, char *error, size_t error_capacity);
+
+/* ------------------------------------------------------------------------------------------
+ * Section 2 -- what the single-stream seam lacks
+ * ------------------------------------------------------------------------------------------ */
+
+#define MYNAH_HIP_MAX_BATCH 16   /* MYNAH_MAX_BATCH, src/graph.c:12 */
+
+/* Weight storage, the strings of MYNAH_QUANT (src/qmat.c:571-576); numeric values are QMAT_* (src/qmat.c:36). */
+enum { MYNAH_HIP_F32 = 0, MYNAH_HIP_INT8 = 1, MYNAH_HIP_INT4 = 2, MYNAH_HIP_F16 = 3 };
+/* Quantiser arithmetic: 0 evaluates src/qmat.c:39-113 as written (IEEE, compiler independent);
+ * 1 reproduces what the reference's stock build (gcc -O3 -ffast-math, Makefile:5) stores:
+ * scale = amax * f32(1/127) and inv = 127/amax (int4: amax * f32(1/7), 6.9999995f/amax). */
+enum { MYNAH_HIP_ARITH_STRICT = 0, MYNAH_HIP_ARITH_STOCK = 1 };
+
+/* Selects the storage used for weights first seen AFTER the call (already cached weights keep
+ * theirs).  The open call initialises it from MYNAH_QUANT ("int8" | "int4" | "f16", else f32) and
+ * MYNAH_QUANT_ARITH ("stock", else strict).  int4 falls back to f32 when iw % 32 != 0
+ * (src/qmat.c:630); quantised storage is used only for rows <= 16 and iw <= 8192 (src/qmat.c:32-33). */
+int mynah_hip_set_quant(void *state, int qtype, int arith, char *error, size_t error_capacity);
+
+/* Host-side load-time conversion used by the weight cache, exposed so callers (and tests) can
+ * check or pre-pack bytes.  Restates quantize_weight_int8/int4 (src/qmat.c:39-91) and the
+ * (__fp16) cast (src/qmat.c:655, IEEE round-to-nearest-even). */
+void mynah_hip_quantize_weight_int8(const float *w, size_t n, size_t k, int8_t *q, float *scales, int arith);
+int mynah_hip_quantize_weight_int4(const float *w, size_t n, size_t k, uint8_t *q, float *scales, int arith);
+void mynah_hip_convert_weight_f16(const float *w, size_t count, uint16_t *out);
+
+/* Weight-stationary batched linear: `batch` single-row activations of different streams, one pass
+ * over the weight.  Twin of mynah_qmat_linear_batched (src/qmat.h:53-58, src/qmat.c:820-888):
+ * dev_in[b] / dev_out[b] are scattered device rows; every out[b] is bit-identical to the same row
+ * run alone (src/qmat.c:1107-1179).  batch <= MYNAH_HIP_MAX_BATCH. */
+int mynah_hip_matmul_d2d_batched(void *state, const float *const *dev_in, float *const *dev_out, size_t batch,
+                                 size_t iw, size_t ow, const float *weight, const float *bias,
+                                 char *error, size_t error_capacity);
+
+/* Parity probe for the quantised matvec: like mynah_hip_matmul_d2d with rows == 1, and additionally
+ * stores the int8 activation (iw bytes), its scale (1 float) and the int32 accumulators
+ * (int8: ow values; int4: ow * iw/32 per-group values) to the given device buffers (any may be NULL). */
+int mynah_hip_matmul_d2d_probe(void *state, const float *dev_in, float *dev_out, size_t iw, size_t ow,
+                               const float *weight, const float *bias, int8_t *dev_qx, float *dev_sx,
+                               int32_t *dev_acc, char *error, size_t error_capacity);
+
+/* Batched single-token attention.  Arrays have `batch` entries and live on the HOST; the caches are
+ * device pointers.  Same per-stream contract as the single-stream calls above; every stream's output
+ * is bit-identical to that stream run alone. */
+int mynah_hip_self_attention_dev_batched(void *state, const float *const *dev_qkv, float *const *dev_k_cache,
+                                         float *const *dev_v_cache, const size_t *position, size_t cache_stride,
+                                         const size_t *valid, size_t batch, size_t heads, size_t head_width,
+                                         float scale, float *const *dev_out, char *error, size_t error_capacity);
+int mynah_hip_cross_attention_dev_batched(void *state, const float *const *dev_q, const float *const *dev_k_cache,
+                                          const float *const *dev_v_cache, const size_t *valid, size_t cache_stride,
+                                          size_t batch, size_t heads, size_t head_width, float scale,
+                                          float *const *dev_out, char *error, size_t error_capacity);
+
+/* Embedding gather (src/graph.c:729-737 text rows, :764-804 audio frame): out[t,:] = sum over `tables`
+ * of table_j[ids[t*tables + j], :] scaled by `scale` (1 for text, 1/16 for the stacked audio frame),
+ * optionally + position[t0 + t, :] (src/graph.c:649-651, :3156-3157).  f32 tables are HOST pointers
+ * cached on the device; ids are a HOST array.  With one table and scale 1 the row is copied bit for bit. */
+int mynah_hip_embed_gather(void *state, const float *const *tables, const size_t *table_rows, size_t table_count,
+                           const int32_t *ids, size_t tokens, size_t width, float scale, const float *position,
+                           size_t position_offset, float *dev_out, char *error, size_t error_capacity);
+
+/* ---- whole decode step ------------------------------------------------------------------- */
+
+/* Pre-resolved decoder weights: HOST pointers, the fields of decoder_layer_resolved / decoder_cache
+ * (src/graph.c:2795-2861) plus the generalisations the synthetic configurations need (LayerNorm
+ * bias, several cross-attention heads).  Per-layer tensors are arrays of `layers` pointers. */
+typedef struct {
+    size_t layers, width, heads, head_width, ffn_width;
+    size_t cross_heads, cross_head_width;   /* xattn_width = cross_heads * cross_head_width; 0 heads = no cross sublayer */
+    size_t capacity;                        /* rows of each self K/V cache per layer */
+    const float *const *norm_self;          /* [layers] -> [width] gain */
+    const float *const *norm_self_bias;     /* NULL, or [layers] -> [width] (NULL entries allowed) */
+    const float *const *norm_xattn_query;
+    const float *const *norm_xattn_query_bias;
+    const float *const *norm_pos_ff;
+    const float *const *norm_pos_ff_bias;
+    const float *const *qkv_w;              /* [3*width, width] */
+    const float *const *o_self_w;           /* [width, width] */
+    const float *const *q_cross_w;          /* [xattn_width, width] */
+    const float *const *o_cross_w;          /* [width, xattn_width] */
+    const float *const *ffn_up_w;           /* [ffn_width, width] */
+    const float *const *ffn_down_w;         /* [width, ffn_width] */
+    const float *norm_out;                  /* [width] gain, NULL = no final norm */
+    const float *norm_out_bias;             /* NULL or [width] */
+    const float *position;                  /* [capacity, width] position embeddings, or NULL */
+} mynah_hip_decoder_desc;
+
+typedef struct mynah_hip_decoder mynah_hip_decoder;
+
+/* One live stream of a batched step: the device-side fields of decoder_cache (src/graph.c:2853-2857). */
+typedef struct {
+    float *dev_self_k;          /* [layers, capacity, width] */
+    float *dev_self_v;
+    const float *dev_cross_k;   /* [layers, memory_length, xattn_width] */
+    const float *dev_cross_v;
+    size_t length;              /* tokens already cached; this step appends row `length` */
+    size_t memory_length;
+    const float *dev_input;     /* [width] the embedded frame, before the position add */
+    float *dev_output;          /* [width] after the final norm */
+} mynah_hip_decoder_slot;
+
+/* Converts and caches every weight under the current quant setting and builds the resident step. */
+int mynah_hip_decoder_create(void *state, const mynah_hip_decoder_desc *desc, mynah_hip_decoder **out,
+                             char *error, size_t error_capacity);
+void mynah_hip_decoder_destroy(void *state, mynah_hip_decoder *decoder);
+
+/* One decode step for `batch` streams: the fused order of decoder_step_batch (src/graph.c:3127-3284)
+ * -- per layer LN -> QKV -> self-attention + KV append -> O -> +res -> LN -> Q -> cross-attention ->
+ * O -> +res -> LN -> up -> GELU -> down -> +res, final LN -- with one pass over each weight for all
+ * streams.  Enqueues and returns (no sync).  Fails with "decoder cache capacity exceeded" when a
+ * slot's length >= capacity (src/graph.c:3152-3155) and with "decoder batch exceeds
+ * MYNAH_MAX_BATCH" above 16 (:3133-3136).  Slot lengths are read, not advanced. */
+int mynah_hip_decoder_step(void *state, mynah_hip_decoder *decoder, const mynah_hip_decoder_slot *slots,
+                           size_t batch, char *error, size_t error_capacity);
+
+/* Output head for the step's final-normed rows: logits[b] = W[rows,width] hidden[b] + bias, then a
+ * softmax over each consecutive group of `vocab` logits (mynah_softmax_f32, src/kernels.c:391-420).
+ * dev_probs[b] may be NULL (logits only).  W/bias HOST pointers. */
+int mynah_hip_output_head(void *state, const float *const *dev_hidden, size_t batch, size_t width,
+                          const float *weight, const float *bias, size_t rows, size_t vocab,
+                          float *const *dev_logits, float *const *dev_probs, char *error, size_t error_capacity);
+
+/* ---- text-encoder prefill (dense, MFMA) --------------------------------------------------- */
+
+typedef struct {
+    size_t layers, width, heads, head_width, ffn_width, vocab, max_positions;
+    const float *tok_table;       /* HOST f32 [vocab, width]; stored as f16 on the device */
+    const float *pos_table;       /* HOST f32 [max_positions, width]; stored as f16 */
+    const float *const *qkv_w, *const *o_w, *const *up_w, *const *down_w;   /* [layers] HOST f32, stored f16 */
+    const float *const *norm1, *const *norm1_bias, *const *norm2, *const *norm2_bias;
+    const float *norm_out, *norm_out_bias;
+} mynah_hip_encoder_desc;
+typedef struct mynah_hip_encoder mynah_hip_encoder;
+
+int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_desc *desc, mynah_hip_encoder **out,
+                             char *error, size_t error_capacity);
+void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *encoder);
+/* ids: HOST int32 [tokens]; dev_embed_f16 (optional): [tokens,width] f16 bits of the gathered token rows;
+ * dev_out: f32 [tokens,width].  Bidirectional attention, plain FFN (the kernel == 1 branch of
+ * causal_conv_ffn, src/graph.c:302-316), pre-LayerNorm, f16 operands with f32 accumulation. */
+int mynah_hip_encoder_prefill(void *state, mynah_hip_encoder *encoder, const int32_t *ids, size_t tokens,
+                              uint16_t *dev_embed_f16, float *dev_out, char *error, size_t error_capacity);
+
+/* ---- measurement helpers ------------------------------------------------------------------ */
+
+/* HIP events on the backend's own stream (a torch/other-runtime event would not see it).
+ * timer_begin records, timer_end records + synchronises and returns elapsed milliseconds. */
+int mynah_hip_timer_begin(void *state, char *error, size_t error_capacity);
+int mynah_hip_timer_end(void *state, float *milliseconds, char *error, size_t error_capacity);
+/* Streams `bytes` of backend-owned scratch through the chip (read+write) so that the last-level
+ * cache holds none of the caller's data: used between timed iterations. */
+int mynah_hip_flush_cache(void *state, size_t bytes, char *error, size_t error_capacity);
+/* 0 = launch every stage kernel individually, 1 (default) = replay the step as a captured HIP graph. */
+int mynah_hip_set_graph_mode(void *state, int enabled, char *error, size_t error_capacity);
+/* Bytes of device memory held by the weight cache (packed weights + scales + vectors). */
+size_t mynah_hip_cached_weight_bytes(void *state);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,454 @@
+"""Host-side bindings of the gfx950 HIP backend for Mynah TTS's decode-step kernels.
+
+The product is the C-ABI shared library libmynah_hip.so (sources in csrc/, declarations in
+include/mynah_hip.h).  This module only loads it through ctypes and mirrors the reference's
+backend seam (src/backend.h) with the same names, argument meaning and error behaviour
+(0 / -1 + message), so the parity tests read like the reference's own self-tests.
+
+There is no CPU fallback: if the library is missing or no MI355X is present, loading or opening
+fails loudly.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmynah_hip.so")
+HEADER_PATH = os.path.join(HERE, "..", "include", "mynah_hip.h")
+
+F32, INT8, INT4, F16 = 0, 1, 2, 3
+ARITH_STRICT, ARITH_STOCK = 0, 1
+MAX_BATCH = 16
+QTYPE_NAMES = {F32: "f32", INT8: "int8", INT4: "int4", F16: "f16"}
+
+_sz = C.c_size_t
+_vp = C.c_void_p
+_err = (C.c_char_p, _sz)
+
+MATMUL_FN = C.CFUNCTYPE(C.c_int, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, C.c_char_p, _sz)
+SGEMM_FN = C.CFUNCTYPE(C.c_int, _vp, C.c_int, C.c_int, _sz, _sz, _sz, C.c_float, _vp, _sz, _vp, _sz, C.c_float,
+                       _vp, _sz, C.c_char_p, _sz)
+CLOSE_FN = C.CFUNCTYPE(None, _vp)
+SELF_TEST_FN = C.CFUNCTYPE(C.c_int, _vp, C.c_char_p, _sz)
+
+
+class DecoderDesc(C.Structure):
+    _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn_width", _sz),
+                ("cross_heads", _sz), ("cross_head_width", _sz), ("capacity", _sz),
+                ("norm_self", _vp), ("norm_self_bias", _vp), ("norm_xattn_query", _vp), ("norm_xattn_query_bias", _vp),
+                ("norm_pos_ff", _vp), ("norm_pos_ff_bias", _vp),
+                ("qkv_w", _vp), ("o_self_w", _vp), ("q_cross_w", _vp), ("o_cross_w", _vp), ("ffn_up_w", _vp),
+                ("ffn_down_w", _vp), ("norm_out", _vp), ("norm_out_bias", _vp), ("position", _vp)]
+
+
+class DecoderSlot(C.Structure):
+    _fields_ = [("dev_self_k", _vp), ("dev_self_v", _vp), ("dev_cross_k", _vp), ("dev_cross_v", _vp),
+                ("length", _sz), ("memory_length", _sz), ("dev_input", _vp), ("dev_output", _vp)]
+
+
+class EncoderDesc(C.Structure):
+    _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn_width", _sz),
+                ("vocab", _sz), ("max_positions", _sz), ("tok_table", _vp), ("pos_table", _vp),
+                ("qkv_w", _vp), ("o_w", _vp), ("up_w", _vp), ("down_w", _vp),
+                ("norm1", _vp), ("norm1_bias", _vp), ("norm2", _vp), ("norm2_bias", _vp),
+                ("norm_out", _vp), ("norm_out_bias", _vp)]
+
+
+def load_library(path=LIB_PATH):
+    """dlopen the backend.  Raises (never falls back) when it has not been built."""
+    if not os.path.exists(path):
+        raise RuntimeError(
+            "libmynah_hip.so is not built: run `python mynah-tts_amd/build.py` (needs hipcc for gfx950). "
+            "There is no CPU fallback for the HIP backend.")
+    lib = C.CDLL(path)
+    lib.mynah_backend_hip_open.argtypes = [C.POINTER(_vp), C.POINTER(MATMUL_FN), C.POINTER(SGEMM_FN),
+                                           C.POINTER(CLOSE_FN), C.POINTER(SELF_TEST_FN), *_err]
+    lib.mynah_hip_dev_alloc.argtypes = [_vp, _sz, C.POINTER(_vp), *_err]
+    lib.mynah_hip_dev_free.argtypes = [_vp, _vp]
+    lib.mynah_hip_dev_free.restype = None
+    lib.mynah_hip_h2d.argtypes = [_vp, _vp, _vp, _sz, *_err]
+    lib.mynah_hip_d2h.argtypes = [_vp, _vp, _vp, _sz, *_err]
+    lib.mynah_hip_upload.argtypes = [_vp, _vp, _sz, C.POINTER(_vp), *_err]
+    lib.mynah_hip_download.argtypes = [_vp, _vp, _vp, _sz, *_err]
+    lib.mynah_hip_sync.argtypes = [_vp, *_err]
+    lib.mynah_hip_batch_begin.argtypes = [_vp, *_err]
+    lib.mynah_hip_gelu_inplace.argtypes = [_vp, _vp, _sz, *_err]
+    lib.mynah_hip_gelu_dev.argtypes = [_vp, _vp, _sz, *_err]
+    lib.mynah_hip_residual_inplace.argtypes = [_vp, _vp, _vp, _sz, *_err]
+    lib.mynah_hip_residual_add_dev.argtypes = [_vp, _vp, _vp, _sz, *_err]
+    lib.mynah_hip_layer_norm_inplace.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, *_err]
+    lib.mynah_hip_layer_norm_dev.argtypes = [_vp, _vp, _vp, _vp, _vp, _sz, _sz, *_err]
+    for name in ("mynah_hip_matmul_d2d", "mynah_hip_matmul_dev", "mynah_hip_matmul_to_dev"):
+        getattr(lib, name).argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, *_err]
+    lib.mynah_hip_matvec_dev.argtypes = [_vp, _vp, _vp, _sz, _sz, _vp, _vp, *_err]
+    lib.mynah_hip_sgemm_dev.argtypes = [_vp, C.c_int, C.c_int, _sz, _sz, _sz, C.c_float, _vp, _sz, _vp, _sz,
+                                        C.c_float, _vp, _sz, *_err]
+    lib.mynah_hip_softmax_dev.argtypes = [_vp, _vp, _sz, _sz, _sz, *_err]
+    lib.mynah_hip_self_attention_dev.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_float, _vp, *_err]
+    lib.mynah_hip_cross_attention_dev.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp, *_err]
+    lib.mynah_hip_copy_dev.argtypes = [_vp, _vp, _vp, _sz, *_err]
+    lib.mynah_hip_scale_dev.argtypes = [_vp, _vp, _sz, C.c_float, *_err]
+    lib.mynah_hip_clip_dev.argtypes = [_vp, _vp, _sz, *_err]
+    lib.mynah_hip_argmax_dev.argtypes = [_vp, _vp, _sz, _sz, _sz, C.c_int, C.POINTER(C.c_uint), *_err]
+    lib.mynah_hip_set_quant.argtypes = [_vp, C.c_int, C.c_int, *_err]
+    lib.mynah_hip_quantize_weight_int8.argtypes = [_vp, _sz, _sz, _vp, _vp, C.c_int]
+    lib.mynah_hip_quantize_weight_int8.restype = None
+    lib.mynah_hip_quantize_weight_int4.argtypes = [_vp, _sz, _sz, _vp, _vp, C.c_int]
+    lib.mynah_hip_convert_weight_f16.argtypes = [_vp, _sz, _vp]
+    lib.mynah_hip_convert_weight_f16.restype = None
+    lib.mynah_hip_matmul_d2d_batched.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, *_err]
+    lib.mynah_hip_matmul_d2d_probe.argtypes = [_vp, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _vp, _vp, *_err]
+    lib.mynah_hip_self_attention_dev_batched.argtypes = [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _sz, C.c_float,
+                                                         _vp, *_err]
+    lib.mynah_hip_cross_attention_dev_batched.argtypes = [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp,
+                                                          *_err]
+    lib.mynah_hip_embed_gather.argtypes = [_vp, _vp, _vp, _sz, _vp, _sz, _sz, C.c_float, _vp, _sz, _vp, *_err]
+    lib.mynah_hip_decoder_create.argtypes = [_vp, C.POINTER(DecoderDesc), C.POINTER(_vp), *_err]
+    lib.mynah_hip_decoder_destroy.argtypes = [_vp, _vp]
+    lib.mynah_hip_decoder_destroy.restype = None
+    lib.mynah_hip_decoder_step.argtypes = [_vp, _vp, C.POINTER(DecoderSlot), _sz, *_err]
+    lib.mynah_hip_output_head.argtypes = [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _vp, *_err]
+    lib.mynah_hip_encoder_create.argtypes = [_vp, C.POINTER(EncoderDesc), C.POINTER(_vp), *_err]
+    lib.mynah_hip_encoder_destroy.argtypes = [_vp, _vp]
+    lib.mynah_hip_encoder_destroy.restype = None
+    lib.mynah_hip_encoder_prefill.argtypes = [_vp, _vp, _vp, _sz, _vp, _vp, *_err]
+    lib.mynah_hip_timer_begin.argtypes = [_vp, *_err]
+    lib.mynah_hip_timer_end.argtypes = [_vp, C.POINTER(C.c_float), *_err]
+    lib.mynah_hip_flush_cache.argtypes = [_vp, _sz, *_err]
+    lib.mynah_hip_set_graph_mode.argtypes = [_vp, C.c_int, *_err]
+    lib.mynah_hip_cached_weight_bytes.argtypes = [_vp]
+    lib.mynah_hip_cached_weight_bytes.restype = _sz
+    return lib
+
+
+class BackendError(RuntimeError):
+    pass
+
+
+def _np_ptr(a):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+class DeviceBuffer:
+    """n floats of device memory owned through mynah_hip_dev_alloc / dev_free."""
+
+    def __init__(self, backend, n):
+        self.backend, self.n = backend, int(n)
+        p = _vp()
+        backend._call("mynah_hip_dev_alloc", _sz(self.n), C.byref(p))
+        self.ptr = p.value
+
+    def at(self, offset_floats):
+        return self.ptr + 4 * int(offset_floats)
+
+    def write(self, host, offset=0):
+        host = np.ascontiguousarray(host)
+        assert host.nbytes % 4 == 0 and host.nbytes // 4 + offset <= self.n
+        self.backend._call("mynah_hip_h2d", _np_ptr(host), _vp(self.at(offset)), _sz(host.nbytes // 4))
+        return self
+
+    def read(self, n=None, offset=0, dtype=np.float32):
+        n = self.n - offset if n is None else n
+        out = np.empty(n, np.float32)
+        self.backend._call("mynah_hip_d2h", _vp(self.at(offset)), _np_ptr(out), _sz(n))
+        return out.view(dtype)
+
+    def free(self):
+        if self.ptr:
+            self.backend.lib.mynah_hip_dev_free(self.backend.state, _vp(self.ptr))
+            self.ptr = None
+
+
+class Backend:
+    """mynah_backend_open(MYNAH_TTS_DEVICE_HIP) as the reference's backend.c would wire it
+    (src/backend.c:367-475): one opaque state plus the function pointers handed back by open."""
+
+    def __init__(self, quant=None, arith=None):
+        self.lib = load_library()
+        self.state = _vp()
+        self._matmul, self._sgemm = MATMUL_FN(), SGEMM_FN()
+        self._close, self._self_test = CLOSE_FN(), SELF_TEST_FN()
+        err = C.create_string_buffer(512)
+        rc = self.lib.mynah_backend_hip_open(C.byref(self.state), C.byref(self._matmul), C.byref(self._sgemm),
+                                             C.byref(self._close), C.byref(self._self_test), err, 512)
+        if rc != 0:
+            raise BackendError("mynah_backend_hip_open failed: " + err.value.decode())
+        self._keep = []   # host arrays whose addresses key the device weight cache
+        if quant is not None or arith is not None:
+            self.set_quant(F32 if quant is None else quant, ARITH_STRICT if arith is None else arith)
+
+    # -- plumbing
+    def _call(self, name, *args):
+        err = C.create_string_buffer(512)
+        rc = getattr(self.lib, name)(self.state, *args, err, 512)
+        if rc != 0:
+            raise BackendError("%s: %s" % (name, err.value.decode()))
+        return rc
+
+    def keep(self, array):
+        """Pin a host tensor for the life of the backend (the cache keys on its address)."""
+        a = np.ascontiguousarray(array, np.float32)
+        self._keep.append(a)
+        return a
+
+    def close(self):
+        if self.state:
+            self._close(self.state)
+            self.state = _vp()
+
+    def alloc(self, n):
+        return DeviceBuffer(self, n)
+
+    def sync(self):
+        self._call("mynah_hip_sync")
+
+    def set_quant(self, qtype, arith=ARITH_STRICT):
+        self._call("mynah_hip_set_quant", C.c_int(qtype), C.c_int(arith))
+
+    # -- host-pointer seam ops
+    def self_test(self):
+        err = C.create_string_buffer(512)
+        rc = self._self_test(self.state, err, 512)
+        return rc, err.value.decode()
+
+    def matmul(self, inp, weight, bias=None):
+        inp = np.ascontiguousarray(inp, np.float32)
+        rows, iw = inp.shape
+        ow = weight.shape[0]
+        out = np.empty((rows, ow), np.float32)
+        err = C.create_string_buffer(512)
+        rc = self._matmul(self.state, _np_ptr(inp), _np_ptr(out), rows, iw, ow, _np_ptr(weight), _np_ptr(bias), err, 512)
+        if rc != 0:
+            raise BackendError(err.value.decode())
+        return out
+
+    def sgemm(self, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc):
+        err = C.create_string_buffer(512)
+        rc = self._sgemm(self.state, ta, tb, m, n, k, alpha, _np_ptr(a), lda, _np_ptr(b), ldb, beta, _np_ptr(c), ldc,
+                         err, 512)
+        if rc != 0:
+            raise BackendError(err.value.decode())
+        return c
+
+    # -- resident seam ops (device buffers in, host weights)
+    def matmul_d2d(self, din, dout, rows, iw, ow, weight, bias=None):
+        self._call("mynah_hip_matmul_d2d", _vp(din), _vp(dout), _sz(rows), _sz(iw), _sz(ow), _np_ptr(weight), _np_ptr(bias))
+
+    def matmul_d2d_batched(self, dins, douts, iw, ow, weight, bias=None):
+        B = len(dins)
+        arr = _vp * B
+        self._call("mynah_hip_matmul_d2d_batched", arr(*dins), arr(*douts), _sz(B), _sz(iw), _sz(ow), _np_ptr(weight),
+                   _np_ptr(bias))
+
+    def matmul_probe(self, din, dout, iw, ow, weight, bias, dqx, dsx, dacc):
+        self._call("mynah_hip_matmul_d2d_probe", _vp(din), _vp(dout), _sz(iw), _sz(ow), _np_ptr(weight), _np_ptr(bias),
+                   _vp(dqx), _vp(dsx), _vp(dacc))
+
+    def layer_norm_inplace(self, din, dout, gain, rows, width):
+        self._call("mynah_hip_layer_norm_inplace", _vp(din), _vp(dout), _np_ptr(gain), _sz(rows), _sz(width))
+
+    def layer_norm_dev(self, din, dout, gain, bias, rows, width):
+        self._call("mynah_hip_layer_norm_dev", _vp(din), _vp(dout), _np_ptr(gain), _np_ptr(bias), _sz(rows), _sz(width))
+
+    def gelu_inplace(self, d, n):
+        self._call("mynah_hip_gelu_inplace", _vp(d), _sz(n))
+
+    def residual_inplace(self, dout, din, n):
+        self._call("mynah_hip_residual_inplace", _vp(dout), _vp(din), _sz(n))
+
+    def softmax_dev(self, d, rows, cols, valid):
+        self._call("mynah_hip_softmax_dev", _vp(d), _sz(rows), _sz(cols), _sz(valid))
+
+    def copy_dev(self, dst, src, n):
+        self._call("mynah_hip_copy_dev", _vp(dst), _vp(src), _sz(n))
+
+    def scale_dev(self, d, n, scale):
+        self._call("mynah_hip_scale_dev", _vp(d), _sz(n), C.c_float(scale))
+
+    def clip_dev(self, d, n):
+        self._call("mynah_hip_clip_dev", _vp(d), _sz(n))
+
+    def argmax_dev(self, dlogits, vocab, codebook_size, eos_id, allow_eos):
+        out = C.c_uint(0)
+        self._call("mynah_hip_argmax_dev", _vp(dlogits), _sz(vocab), _sz(codebook_size), _sz(eos_id), C.c_int(int(allow_eos)),
+                   C.byref(out))
+        return out.value
+
+    def self_attention_dev(self, dqkv, dk, dv, position, stride, valid, heads, hw, scale, dout):
+        self._call("mynah_hip_self_attention_dev", _vp(dqkv), _vp(dk), _vp(dv), _sz(position), _sz(stride), _sz(valid),
+                   _sz(heads), _sz(hw), C.c_float(scale), _vp(dout))
+
+    def cross_attention_dev(self, dq, dk, dv, valid, stride, heads, hw, scale, dout):
+        self._call("mynah_hip_cross_attention_dev", _vp(dq), _vp(dk), _vp(dv), _sz(valid), _sz(stride), _sz(heads), _sz(hw),
+                   C.c_float(scale), _vp(dout))
+
+    def self_attention_dev_batched(self, dqkv, dk, dv, positions, stride, valids, heads, hw, scale, douts):
+        B = len(dqkv)
+        arr, szs = _vp * B, _sz * B
+        self._call("mynah_hip_self_attention_dev_batched", arr(*dqkv), arr(*dk), arr(*dv), szs(*positions), _sz(stride),
+                   szs(*valids), _sz(B), _sz(heads), _sz(hw), C.c_float(scale), arr(*douts))
+
+    def cross_attention_dev_batched(self, dq, dk, dv, valids, stride, heads, hw, scale, douts):
+        B = len(dq)
+        arr, szs = _vp * B, _sz * B
+        self._call("mynah_hip_cross_attention_dev_batched", arr(*dq), arr(*dk), arr(*dv), szs(*valids), _sz(stride), _sz(B),
+                   _sz(heads), _sz(hw), C.c_float(scale), arr(*douts))
+
+    def embed_gather(self, tables, ids, width, scale, position, position_offset, dout):
+        ids = np.ascontiguousarray(ids, np.int32)
+        T = len(tables)
+        tokens = ids.size // T
+        arr = _vp * T
+        rows = (_sz * T)(*[t.shape[0] for t in tables])
+        self._call("mynah_hip_embed_gather", arr(*[_np_ptr(t) for t in tables]), rows, _sz(T), _np_ptr(ids), _sz(tokens),
+                   _sz(width), C.c_float(scale), _np_ptr(position), _sz(position_offset), _vp(dout))
+
+    def output_head(self, dhidden, width, weight, bias, rows, vocab, dlogits, dprobs):
+        B = len(dhidden)
+        arr = _vp * B
+        self._call("mynah_hip_output_head", arr(*dhidden), _sz(B), _sz(width), _np_ptr(weight), _np_ptr(bias), _sz(rows),
+                   _sz(vocab), arr(*dlogits), None if dprobs is None else arr(*dprobs))
+
+    # -- measurement
+    def timer_begin(self):
+        self._call("mynah_hip_timer_begin")
+
+    def timer_end(self):
+        ms = C.c_float(0)
+        self._call("mynah_hip_timer_end", C.byref(ms))
+        return ms.value
+
+    def flush_cache(self, nbytes=512 << 20):
+        self._call("mynah_hip_flush_cache", _sz(nbytes))
+
+    def set_graph_mode(self, enabled):
+        self._call("mynah_hip_set_graph_mode", C.c_int(int(enabled)))
+
+    def cached_weight_bytes(self):
+        return self.lib.mynah_hip_cached_weight_bytes(self.state)
+
+
+def _ptr_array(arrays):
+    """C array of host pointers (one per layer); None entries stay NULL."""
+    arr = (_vp * len(arrays))(*[_np_ptr(a) for a in arrays])
+    return arr
+
+
+class Decoder:
+    """mynah_hip_decoder_create + step: the batched resident decode step."""
+
+    def __init__(self, backend, cfg, weights):
+        self.backend, self.cfg = backend, cfg
+        L = cfg["layers"]
+        self._hold = []
+
+        def per_layer(name):
+            if weights.get(name) is None:
+                return None
+            rows = [backend.keep(weights[name][l]) for l in range(L)]
+            arr = _ptr_array(rows)
+            self._hold.append(arr)
+            return C.cast(arr, _vp)
+
+        def single(name):
+            if weights.get(name) is None:
+                return None
+            return _np_ptr(backend.keep(weights[name]))
+
+        d = DecoderDesc()
+        d.layers, d.width, d.heads, d.head_width, d.ffn_width = L, cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
+        d.cross_heads, d.cross_head_width, d.capacity = cfg["cross_heads"], cfg["cross_head_width"], cfg["capacity"]
+        d.norm_self, d.norm_self_bias = per_layer("norm_self_g"), per_layer("norm_self_b")
+        d.norm_xattn_query, d.norm_xattn_query_bias = per_layer("norm_cross_g"), per_layer("norm_cross_b")
+        d.norm_pos_ff, d.norm_pos_ff_bias = per_layer("norm_ff_g"), per_layer("norm_ff_b")
+        d.qkv_w, d.o_self_w = per_layer("qkv"), per_layer("o_self")
+        d.q_cross_w, d.o_cross_w = per_layer("q_cross"), per_layer("o_cross")
+        d.ffn_up_w, d.ffn_down_w = per_layer("ffn_up"), per_layer("ffn_down")
+        d.norm_out, d.norm_out_bias, d.position = single("norm_out_g"), single("norm_out_b"), single("position")
+        self.desc = d
+        h = _vp()
+        backend._call("mynah_hip_decoder_create", C.byref(d), C.byref(h))
+        self.handle = h
+
+    def step(self, slots):
+        """slots: list of dicts with k, v, ck, cv (device addresses), length, memory_length, inp, out."""
+        B = len(slots)
+        arr = (DecoderSlot * B)()
+        for i, s in enumerate(slots):
+            arr[i] = DecoderSlot(s["k"], s["v"], s.get("ck"), s.get("cv"), s["length"], s.get("memory_length", 0),
+                                 s["inp"], s["out"])
+        self.backend._call("mynah_hip_decoder_step", self.handle, arr, _sz(B))
+
+    def destroy(self):
+        if self.handle:
+            self.backend.lib.mynah_hip_decoder_destroy(self.backend.state, self.handle)
+            self.handle = None
+
+
+class Encoder:
+    """mynah_hip_encoder_create + prefill: the dense MFMA text-encoder path."""
+
+    def __init__(self, backend, cfg, weights):
+        self.backend, self.cfg = backend, cfg
+        L = cfg["layers"]
+        self._hold = []
+
+        def per_layer(name):
+            if weights.get(name) is None:
+                return None
+            rows = [backend.keep(weights[name][l]) for l in range(L)]
+            arr = _ptr_array(rows)
+            self._hold.append(arr)
+            return C.cast(arr, _vp)
+
+        def single(name):
+            return None if weights.get(name) is None else _np_ptr(backend.keep(weights[name]))
+
+        e = EncoderDesc()
+        e.layers, e.width, e.heads, e.head_width, e.ffn_width = L, cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
+        e.vocab, e.max_positions = cfg["vocab"], cfg["max_positions"]
+        e.tok_table, e.pos_table = single("tok_table"), single("pos_table")
+        e.qkv_w, e.o_w, e.up_w, e.down_w = per_layer("qkv"), per_layer("o"), per_layer("up"), per_layer("down")
+        e.norm1, e.norm1_bias = per_layer("norm1_g"), per_layer("norm1_b")
+        e.norm2, e.norm2_bias = per_layer("norm2_g"), per_layer("norm2_b")
+        e.norm_out, e.norm_out_bias = single("norm_out_g"), single("norm_out_b")
+        self.desc = e
+        h = _vp()
+        backend._call("mynah_hip_encoder_create", C.byref(e), C.byref(h))
+        self.handle = h
+
+    def prefill(self, ids, dembed, dout):
+        ids = np.ascontiguousarray(ids, np.int32)
+        self.backend._call("mynah_hip_encoder_prefill", self.handle, _np_ptr(ids), _sz(ids.size), _vp(dembed), _vp(dout))
+
+    def destroy(self):
+        if self.handle:
+            self.backend.lib.mynah_hip_encoder_destroy(self.backend.state, self.handle)
+            self.handle = None
+
+
+# ---- host-side converters (exposed by the library, used by callers that pre-pack and by tests)
+def quantize_weight_int8(lib, w, arith=ARITH_STRICT):
+    w = np.ascontiguousarray(w, np.float32)
+    n, k = w.shape
+    q = np.empty((n, k), np.int8)
+    s = np.empty(n, np.float32)
+    lib.mynah_hip_quantize_weight_int8(_np_ptr(w), n, k, _np_ptr(q), _np_ptr(s), arith)
+    return q, s
+
+
+def quantize_weight_int4(lib, w, arith=ARITH_STRICT):
+    w = np.ascontiguousarray(w, np.float32)
+    n, k = w.shape
+    q = np.empty((n, k // 2), np.uint8)
+    s = np.empty((n, max(k // 32, 1)), np.float32)
+    rc = lib.mynah_hip_quantize_weight_int4(_np_ptr(w), n, k, _np_ptr(q), _np_ptr(s), arith)
+    return rc, q, s
+
+
+def convert_weight_f16(lib, w):
+    w = np.ascontiguousarray(w, np.float32)
+    out = np.empty(w.shape, np.uint16)
+    lib.mynah_hip_convert_weight_f16(_np_ptr(w), w.size, _np_ptr(out))
+    return out

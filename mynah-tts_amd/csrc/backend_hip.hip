@@ -1,0 +1,851 @@
+// C ABI of the gfx950 backend: state, pointer-keyed weight cache, and the seam's resident ops.
+#include <float.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <new>
+
+#include "kernels.h"
+
+namespace mynah {
+
+// ------------------------------------------------------------------------------------------ helpers
+int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity) {
+    if (st->pinned_bytes >= bytes) return 0;
+    if (st->pinned != nullptr) {
+        MYNAH_TRY(hipStreamSynchronize(st->stream));
+        (void)hipHostFree(st->pinned);
+        st->pinned = nullptr;
+        st->pinned_bytes = 0;
+    }
+    size_t cap = 1u << 20;
+    while (cap < bytes) cap <<= 1;
+    MYNAH_TRY(hipHostMalloc(&st->pinned, cap, hipHostMallocDefault));
+    st->pinned_bytes = cap;
+    return 0;
+}
+
+static int ensure_scratch(State *st, size_t bytes, char *error, size_t capacity) {
+    if (st->scratch_bytes >= bytes) return 0;
+    if (st->scratch != nullptr) {
+        MYNAH_TRY(hipStreamSynchronize(st->stream));
+        (void)hipFree(st->scratch);
+        st->scratch = nullptr;
+        st->scratch_bytes = 0;
+    }
+    size_t cap = 1u << 20;
+    while (cap < bytes) cap <<= 1;
+    MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->scratch), cap));
+    st->scratch_bytes = cap;
+    return 0;
+}
+
+// Host memory -> device, stream ordered.  Sources of at most the pinned staging size are staged so
+// the call can return before the copy runs; larger ones (weights at load time) copy synchronously.
+static int copy_to_device(State *st, void *dst, const void *src, size_t bytes, char *error, size_t capacity) {
+    if (bytes == 0) return 0;
+    MYNAH_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, st->stream));
+    // pageable source: the runtime has consumed `src` when the call returns
+    return 0;
+}
+
+int ensure_attention_workspace(State *st, size_t batch, size_t heads, size_t head_width, size_t max_valid,
+                               char *error, size_t capacity) {
+    const size_t chunks = (max_valid + kAttnChunk - 1) / kAttnChunk + 1;
+    const size_t need = batch * heads * chunks * (head_width + 2);
+    if (st->attn_partial_floats < need) {
+        if (st->attn_partial != nullptr) {
+            MYNAH_TRY(hipStreamSynchronize(st->stream));
+            (void)hipFree(st->attn_partial);
+            st->attn_partial = nullptr;
+            st->attn_partial_floats = 0;
+        }
+        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->attn_partial), need * sizeof(float)));
+        st->attn_partial_floats = need;
+    }
+    if (st->attn_counters == nullptr) {
+        const size_t count = (size_t)kMaxBatch * 4096;   // heads * batch upper bound
+        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->attn_counters), count * sizeof(unsigned)));
+        MYNAH_TRY(hipMemsetAsync(st->attn_counters, 0, count * sizeof(unsigned), st->stream));
+    }
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------ weight cache
+// Keyed by (host address, byte size, conversion), on the contract that the host memory is an
+// immutable model tensor that outlives the backend (gpu/cuda/backend_cuda.cu:193-219).
+int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qtype, const CachedWeight **out,
+                  char *error, size_t capacity) {
+    if (host == nullptr || n == 0 || k == 0 || n > SIZE_MAX / k / sizeof(float)) {
+        set_error(error, capacity, "invalid weight tensor");
+        return -1;
+    }
+    int qtype = want_qtype;
+    if (qtype == MYNAH_HIP_INT4 && (k % 32u) != 0) qtype = MYNAH_HIP_F32;   // src/qmat.c:630
+    if (qtype != MYNAH_HIP_F32 && k > kQuantMaxK) qtype = MYNAH_HIP_F32;    // src/qmat.c:33,774
+    if (qtype != MYNAH_HIP_F32 && !linear_fast_supported(qtype, n, k)) qtype = MYNAH_HIP_F32;
+    const WeightKey key{host, n * k * sizeof(float), 1 + qtype * 2 + (qtype == MYNAH_HIP_INT8 || qtype == MYNAH_HIP_INT4 ? st->arith : 0)};
+    std::lock_guard<std::mutex> lock(st->mu);
+    auto it = st->weights.find(key);
+    if (it != st->weights.end()) {
+        *out = &it->second;
+        return 0;
+    }
+    CachedWeight cw;
+    cw.qtype = qtype;
+    cw.n = n;
+    cw.k = k;
+    const size_t count = n * k;
+    if (qtype == MYNAH_HIP_F32) {
+        cw.bytes = count * sizeof(float);
+        MYNAH_TRY(hipMalloc(&cw.data, cw.bytes));
+        MYNAH_TRY(hipMemcpy(cw.data, host, cw.bytes, hipMemcpyHostToDevice));
+    } else if (qtype == MYNAH_HIP_F16) {
+        std::vector<uint16_t> packed(count);
+        for (size_t i = 0; i < count; ++i) packed[i] = f32_to_f16_rne(host[i]);
+        cw.bytes = count * sizeof(uint16_t);
+        MYNAH_TRY(hipMalloc(&cw.data, cw.bytes));
+        MYNAH_TRY(hipMemcpy(cw.data, packed.data(), cw.bytes, hipMemcpyHostToDevice));
+    } else if (qtype == MYNAH_HIP_INT8) {
+        std::vector<int8_t> packed(count);
+        std::vector<float> scales(n);
+        quantize_weight_int8(host, n, k, packed.data(), scales.data(), st->arith);
+        cw.bytes = count + n * sizeof(float);
+        MYNAH_TRY(hipMalloc(&cw.data, count));
+        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&cw.scales), n * sizeof(float)));
+        MYNAH_TRY(hipMemcpy(cw.data, packed.data(), count, hipMemcpyHostToDevice));
+        MYNAH_TRY(hipMemcpy(cw.scales, scales.data(), n * sizeof(float), hipMemcpyHostToDevice));
+    } else {
+        const size_t groups = k / 32u;
+        std::vector<uint8_t> packed(count / 2u);
+        std::vector<float> scales(n * groups);
+        if (quantize_weight_int4(host, n, k, packed.data(), scales.data(), st->arith) != 0) {
+            set_error(error, capacity, "int4 weight needs a width that is a multiple of 32");
+            return -1;
+        }
+        cw.bytes = count / 2u + n * groups * sizeof(float);
+        MYNAH_TRY(hipMalloc(&cw.data, count / 2u));
+        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&cw.scales), n * groups * sizeof(float)));
+        MYNAH_TRY(hipMemcpy(cw.data, packed.data(), count / 2u, hipMemcpyHostToDevice));
+        MYNAH_TRY(hipMemcpy(cw.scales, scales.data(), n * groups * sizeof(float), hipMemcpyHostToDevice));
+    }
+    st->weight_bytes += cw.bytes;
+    auto ins = st->weights.emplace(key, cw);
+    *out = &ins.first->second;   // unordered_map never moves its nodes: the pointer stays valid
+    return 0;
+}
+
+int cached_vector(State *st, const float *host, size_t n, const float **dev, char *error, size_t capacity) {
+    if (host == nullptr) {
+        *dev = nullptr;
+        return 0;
+    }
+    const WeightKey key{host, n * sizeof(float), 0};
+    std::lock_guard<std::mutex> lock(st->mu);
+    auto it = st->weights.find(key);
+    if (it != st->weights.end()) {
+        *dev = static_cast<const float *>(it->second.data);
+        return 0;
+    }
+    CachedWeight cw;
+    cw.n = 1;
+    cw.k = n;
+    cw.bytes = n * sizeof(float);
+    MYNAH_TRY(hipMalloc(&cw.data, cw.bytes));
+    MYNAH_TRY(hipMemcpy(cw.data, host, cw.bytes, hipMemcpyHostToDevice));
+    st->weight_bytes += cw.bytes;
+    st->weights.emplace(key, cw);
+    *dev = static_cast<const float *>(cw.data);
+    return 0;
+}
+
+// out[b] = W in[b] (+bias) for `batch` device rows: fused matvec tiles, or the generic f32 GEMM.
+static int linear_rows(State *st, const float *const *in, float *const *out, size_t batch, size_t iw, size_t ow,
+                       const float *weight, const float *bias, int8_t *probe_qx, float *probe_sx, int32_t *probe_acc,
+                       char *error, size_t capacity) {
+    const float *dbias = nullptr;
+    if (cached_vector(st, bias, ow, &dbias, error, capacity) != 0) return -1;
+    const CachedWeight *cw = nullptr;
+    const int want = batch <= kQuantMaxRows ? st->qtype : MYNAH_HIP_F32;
+    if (cached_matrix(st, weight, ow, iw, want, &cw, error, capacity) != 0) return -1;
+    if (!linear_fast_supported(cw->qtype, ow, iw)) {
+        for (size_t b = 0; b < batch; ++b)
+            if (launch_gemm_f32(st, in[b], out[b], 1, iw, ow, static_cast<const float *>(cw->data), dbias, error, capacity) != 0)
+                return -1;
+        return 0;
+    }
+    for (size_t b0 = 0; b0 < batch; b0 += kBatchTile) {
+        LinearArgs a{};
+        a.w = cw->data;
+        a.scales = cw->scales;
+        a.bias = dbias;
+        a.qtype = cw->qtype;
+        a.n = (int)ow;
+        a.k = (int)iw;
+        a.batch = (int)(batch - b0 < (size_t)kBatchTile ? batch - b0 : (size_t)kBatchTile);
+        for (int b = 0; b < a.batch; ++b) {
+            a.in[b] = in[b0 + b];
+            a.out[b] = out[b0 + b];
+        }
+        a.arith = st->arith;
+        a.epilogue = EPI_NONE;
+        a.probe_qx = probe_qx;
+        a.probe_sx = probe_sx;
+        a.probe_acc = probe_acc;
+        if (launch_linear(st, a, error, capacity) != 0) return -1;
+    }
+    return 0;
+}
+
+static int check_rows(const void *in, const void *out, size_t rows, size_t iw, size_t ow, const float *weight,
+                      char *error, size_t capacity) {
+    if (in == nullptr || out == nullptr || weight == nullptr || rows == 0 || iw == 0 || ow == 0 ||
+        iw > 0x7fffffffu || ow > 0x7fffffffu || rows > 0x7fffffffu) {
+        set_error(error, capacity, "invalid matmul arguments");
+        return -1;
+    }
+    return 0;
+}
+
+static int matmul_device(State *st, const float *din, float *dout, size_t rows, size_t iw, size_t ow,
+                         const float *weight, const float *bias, char *error, size_t capacity) {
+    if (check_rows(din, dout, rows, iw, ow, weight, error, capacity) != 0) return -1;
+    if (rows <= kQuantMaxRows) {
+        const float *in[kMaxBatch];
+        float *out[kMaxBatch];
+        for (size_t r = 0; r < rows; ++r) {
+            in[r] = din + r * iw;
+            out[r] = dout + r * ow;
+        }
+        return linear_rows(st, in, out, rows, iw, ow, weight, bias, nullptr, nullptr, nullptr, error, capacity);
+    }
+    const float *dbias = nullptr;
+    if (cached_vector(st, bias, ow, &dbias, error, capacity) != 0) return -1;
+    const CachedWeight *cw = nullptr;
+    if (cached_matrix(st, weight, ow, iw, MYNAH_HIP_F32, &cw, error, capacity) != 0) return -1;
+    return launch_gemm_f32(st, din, dout, rows, iw, ow, static_cast<const float *>(cw->data), dbias, error, capacity);
+}
+
+// host in / host out, synchronous (mynah_backend_matmul, src/backend.h:32-35)
+static int hip_matmul(void *opaque, const float *input, float *output, size_t rows, size_t iw, size_t ow,
+                      const float *weight, const float *bias, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (check_rows(input, output, rows, iw, ow, weight, error, capacity) != 0) return -1;
+    const size_t in_n = rows * iw, out_n = rows * ow;
+    if (ensure_scratch(st, (in_n + out_n) * sizeof(float), error, capacity) != 0) return -1;
+    float *din = st->scratch, *dout = st->scratch + in_n;
+    MYNAH_TRY(hipMemcpyAsync(din, input, in_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
+    if (matmul_device(st, din, dout, rows, iw, ow, weight, bias, error, capacity) != 0) return -1;
+    MYNAH_TRY(hipMemcpyAsync(output, dout, out_n * sizeof(float), hipMemcpyDeviceToHost, st->stream));
+    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    return 0;
+}
+
+static int hip_sgemm(void *opaque, int ta, int tb, size_t m, size_t n, size_t k, float alpha, const float *a, size_t lda,
+                     const float *b, size_t ldb, float beta, float *c, size_t ldc, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (a == nullptr || b == nullptr || c == nullptr || m == 0 || n == 0) {
+        set_error(error, capacity, "invalid sgemm arguments");
+        return -1;
+    }
+    const size_t a_n = (ta ? k : m) * lda, b_n = (tb ? n : k) * ldb, c_n = m * ldc;
+    if (ensure_scratch(st, (a_n + b_n + c_n) * sizeof(float), error, capacity) != 0) return -1;
+    float *da = st->scratch, *db = da + a_n, *dc = db + b_n;
+    MYNAH_TRY(hipMemcpyAsync(da, a, a_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
+    MYNAH_TRY(hipMemcpyAsync(db, b, b_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
+    if (beta != 0.0f) MYNAH_TRY(hipMemcpyAsync(dc, c, c_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
+    if (launch_sgemm(st, ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc, error, capacity) != 0) return -1;
+    MYNAH_TRY(hipMemcpyAsync(c, dc, c_n * sizeof(float), hipMemcpyDeviceToHost, st->stream));
+    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    return 0;
+}
+
+static void hip_close(void *opaque) {
+    State *st = static_cast<State *>(opaque);
+    if (st == nullptr) return;
+    (void)hipStreamSynchronize(st->stream);
+    for (auto &kv : st->weights) {
+        if (kv.second.data != nullptr) (void)hipFree(kv.second.data);
+        if (kv.second.scales != nullptr) (void)hipFree(kv.second.scales);
+    }
+    if (st->scratch != nullptr) (void)hipFree(st->scratch);
+    if (st->pinned != nullptr) (void)hipHostFree(st->pinned);
+    if (st->flush != nullptr) (void)hipFree(st->flush);
+    if (st->attn_partial != nullptr) (void)hipFree(st->attn_partial);
+    if (st->attn_counters != nullptr) (void)hipFree(st->attn_counters);
+    if (st->ptr_table != nullptr) (void)hipFree(st->ptr_table);
+    if (st->ptr_table_host != nullptr) (void)hipHostFree(st->ptr_table_host);
+    if (st->ev0 != nullptr) (void)hipEventDestroy(st->ev0);
+    if (st->ev1 != nullptr) (void)hipEventDestroy(st->ev1);
+    if (st->stream != nullptr) (void)hipStreamDestroy(st->stream);
+    delete st;
+}
+
+static int attention_table(State *st, int is_self, const float *const *q, float *const *kc, float *const *vc,
+                           const size_t *position, const size_t *valid, size_t stride, size_t batch, size_t heads,
+                           size_t hw, float scale, float *const *out, char *error, size_t capacity) {
+    if (batch == 0) return 0;
+    if (batch > (size_t)kMaxBatch) {
+        set_error(error, capacity, "attention batch exceeds MYNAH_MAX_BATCH");
+        return -1;
+    }
+    if (heads == 0 || hw == 0 || hw > 1024 || heads * hw > 4096 || stride > 0x7fffffffu) {
+        set_error(error, capacity, "attention: unsupported head shape");
+        return -1;
+    }
+    size_t max_valid = 1;
+    AttnArgs a{};
+    for (size_t b = 0; b < batch; ++b) {
+        if (q[b] == nullptr || kc[b] == nullptr || vc[b] == nullptr || out[b] == nullptr || valid[b] > 0x7ffffff0u) {
+            set_error(error, capacity, "attention: null buffer");
+            return -1;
+        }
+        if (is_self && (position[b] >= valid[b])) {
+            set_error(error, capacity, "attention: position must lie inside the valid range");
+            return -1;
+        }
+        a.q[b] = q[b];
+        a.k_cache[b] = kc[b];
+        a.v_cache[b] = vc[b];
+        a.out[b] = out[b];
+        a.position[b] = is_self ? (int)position[b] : -1;
+        a.valid[b] = (int)valid[b];
+        if (valid[b] > max_valid) max_valid = valid[b];
+    }
+    if (ensure_attention_workspace(st, batch, heads, hw, max_valid, error, capacity) != 0) return -1;
+    a.slots = nullptr;
+    a.batch = (int)batch;
+    a.heads = (int)heads;
+    a.head_width = (int)hw;
+    a.stride = (int)stride;
+    a.q_stride = 0;
+    a.scale = scale;
+    a.is_self = is_self;
+    a.max_chunks = (int)((max_valid + kAttnChunk - 1) / kAttnChunk);
+    a.partial = st->attn_partial;
+    a.counters = st->attn_counters;
+    // the vector path needs 16-byte aligned rows everywhere
+    bool aligned = true;
+    for (size_t b = 0; b < batch; ++b)
+        aligned = aligned && ((reinterpret_cast<uintptr_t>(q[b]) | reinterpret_cast<uintptr_t>(kc[b]) |
+                               reinterpret_cast<uintptr_t>(vc[b]) | reinterpret_cast<uintptr_t>(out[b])) & 15u) == 0;
+    if (!aligned) a.q_stride = 1;   // any value that is not a multiple of 4 selects the scalar path
+    return launch_attention(st, a, error, capacity);
+}
+
+static int backend_self_test(void *opaque, char *error, size_t capacity);
+
+}  // namespace mynah
+
+using namespace mynah;
+
+// =========================================================================================== open
+extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn *matmul, mynah_backend_sgemm_fn *sgemm,
+                                      mynah_backend_close_fn *close, mynah_backend_self_test_fn *self_test, char *error,
+                                      size_t capacity) {
+    if (state_out == nullptr) {
+        set_error(error, capacity, "invalid backend state pointer");
+        return -1;
+    }
+    *state_out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count == 0) {
+        set_error(error, capacity, "no HIP device");
+        return -1;
+    }
+    MYNAH_TRY(hipSetDevice(0));
+    hipDeviceProp_t prop;
+    MYNAH_TRY(hipGetDeviceProperties(&prop, 0));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        if (error != nullptr && capacity > 0)
+            snprintf(error, capacity, "HIP backend is built for gfx950 (MI355X); found %s", prop.gcnArchName);
+        return -1;
+    }
+    State *st = new (std::nothrow) State();
+    if (st == nullptr) {
+        set_error(error, capacity, "out of memory creating HIP backend");
+        return -1;
+    }
+    st->cu_count = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    if (hip_check(hipStreamCreate(&st->stream), "stream create", error, capacity) != 0 ||
+        hip_check(hipEventCreate(&st->ev0), "event create", error, capacity) != 0 ||
+        hip_check(hipEventCreate(&st->ev1), "event create", error, capacity) != 0) {
+        hip_close(st);
+        return -1;
+    }
+    const char *quant = getenv("MYNAH_QUANT");   // same strings as src/qmat.c:571-576
+    if (quant != nullptr && strcmp(quant, "int8") == 0) st->qtype = MYNAH_HIP_INT8;
+    else if (quant != nullptr && strcmp(quant, "int4") == 0) st->qtype = MYNAH_HIP_INT4;
+    else if (quant != nullptr && strcmp(quant, "f16") == 0) st->qtype = MYNAH_HIP_F16;
+    const char *arith = getenv("MYNAH_QUANT_ARITH");
+    if (arith != nullptr && strcmp(arith, "stock") == 0) st->arith = MYNAH_HIP_ARITH_STOCK;
+    const char *graph = getenv("MYNAH_HIP_GRAPH");
+    if (graph != nullptr && strcmp(graph, "0") == 0) st->graph_mode = 0;
+    *state_out = st;
+    if (matmul != nullptr) *matmul = hip_matmul;
+    if (sgemm != nullptr) *sgemm = hip_sgemm;
+    if (close != nullptr) *close = hip_close;
+    if (self_test != nullptr) *self_test = backend_self_test;
+    if (error != nullptr && capacity > 0) error[0] = '\0';
+    return 0;
+}
+
+// =========================================================================================== memory
+extern "C" int mynah_hip_dev_alloc(void *opaque, size_t n, float **dev_ptr, char *error, size_t capacity) {
+    (void)opaque;
+    if (dev_ptr == nullptr || n == 0 || n > SIZE_MAX / sizeof(float)) {
+        set_error(error, capacity, "invalid device allocation size");
+        return -1;
+    }
+    return hip_check(hipMalloc(reinterpret_cast<void **>(dev_ptr), n * sizeof(float)), "malloc", error, capacity);
+}
+
+extern "C" void mynah_hip_dev_free(void *opaque, float *dev_ptr) {
+    State *st = static_cast<State *>(opaque);
+    if (dev_ptr == nullptr) return;
+    if (st != nullptr) (void)hipStreamSynchronize(st->stream);
+    (void)hipFree(dev_ptr);
+}
+
+extern "C" int mynah_hip_h2d(void *opaque, const float *host, float *dev_ptr, size_t n, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (host == nullptr || dev_ptr == nullptr) {
+        set_error(error, capacity, "invalid h2d arguments");
+        return -1;
+    }
+    return copy_to_device(st, dev_ptr, host, n * sizeof(float), error, capacity);
+}
+
+extern "C" int mynah_hip_d2h(void *opaque, const float *dev_ptr, float *host, size_t n, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (host == nullptr || dev_ptr == nullptr) {
+        set_error(error, capacity, "invalid d2h arguments");
+        return -1;
+    }
+    MYNAH_TRY(hipMemcpyAsync(host, dev_ptr, n * sizeof(float), hipMemcpyDeviceToHost, st->stream));
+    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    return 0;
+}
+
+extern "C" int mynah_hip_upload(void *opaque, const float *host, size_t n, float **dev_ptr, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (host == nullptr || dev_ptr == nullptr || n == 0) {
+        set_error(error, capacity, "invalid upload arguments");
+        return -1;
+    }
+    if (ensure_scratch(st, n * sizeof(float), error, capacity) != 0) return -1;
+    *dev_ptr = st->scratch;
+    return copy_to_device(st, st->scratch, host, n * sizeof(float), error, capacity);
+}
+
+extern "C" int mynah_hip_download(void *opaque, const float *dev_ptr, float *host, size_t n, char *error, size_t capacity) {
+    return mynah_hip_d2h(opaque, dev_ptr, host, n, error, capacity);
+}
+
+extern "C" int mynah_hip_sync(void *opaque, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    return hip_check(hipStreamSynchronize(st->stream), "sync", error, capacity);
+}
+
+extern "C" int mynah_hip_batch_begin(void *opaque, char *error, size_t capacity) {
+    (void)opaque;   // a command-buffer hint on Metal; nothing to do on a HIP stream (src/backend.c:571-577)
+    if (error != nullptr && capacity > 0) error[0] = '\0';
+    return 0;
+}
+
+// =========================================================================================== resident ops
+extern "C" int mynah_hip_gelu_inplace(void *opaque, float *d, size_t n, char *error, size_t capacity) {
+    if (d == nullptr) { set_error(error, capacity, "invalid gelu arguments"); return -1; }
+    return launch_gelu(static_cast<State *>(opaque), d, n, error, capacity);
+}
+extern "C" int mynah_hip_gelu_dev(void *opaque, float *d, size_t n, char *error, size_t capacity) {
+    return mynah_hip_gelu_inplace(opaque, d, n, error, capacity);
+}
+extern "C" int mynah_hip_residual_inplace(void *opaque, float *dout, const float *din, size_t n, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (dout == nullptr || din == nullptr) { set_error(error, capacity, "invalid residual arguments"); return -1; }
+    // The engine passes a HOST row of the mmapped position table in the device slot (src/graph.c:1118-1120):
+    // resolve it through the pointer-keyed cache when the address is not device memory.
+    hipPointerAttribute_t attr;
+    const hipError_t r = hipPointerGetAttributes(&attr, din);
+    if (r != hipSuccess || (attr.type != hipMemoryTypeDevice && attr.type != hipMemoryTypeManaged)) {
+        (void)hipGetLastError();
+        const float *cached = nullptr;
+        if (cached_vector(st, din, n, &cached, error, capacity) != 0) return -1;
+        din = cached;
+    }
+    return launch_residual(st, dout, din, n, error, capacity);
+}
+extern "C" int mynah_hip_residual_add_dev(void *opaque, float *dout, const float *din, size_t n, char *error, size_t capacity) {
+    return mynah_hip_residual_inplace(opaque, dout, din, n, error, capacity);
+}
+extern "C" int mynah_hip_layer_norm_dev(void *opaque, const float *din, float *dout, const float *gain, const float *bias,
+                                        size_t rows, size_t width, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (din == nullptr || dout == nullptr || gain == nullptr || width == 0 || width > 0x7fffffffu) {
+        set_error(error, capacity, "invalid layer norm arguments");
+        return -1;
+    }
+    const float *dgain = nullptr, *dbias = nullptr;
+    if (cached_vector(st, gain, width, &dgain, error, capacity) != 0) return -1;
+    if (cached_vector(st, bias, width, &dbias, error, capacity) != 0) return -1;
+    return launch_layernorm(st, din, dout, dgain, dbias, rows, width, error, capacity);
+}
+extern "C" int mynah_hip_layer_norm_inplace(void *opaque, const float *din, float *dout, const float *gain, size_t rows,
+                                            size_t width, char *error, size_t capacity) {
+    return mynah_hip_layer_norm_dev(opaque, din, dout, gain, nullptr, rows, width, error, capacity);
+}
+extern "C" int mynah_hip_matmul_d2d(void *opaque, const float *din, float *dout, size_t rows, size_t iw, size_t ow,
+                                    const float *weight, const float *bias, char *error, size_t capacity) {
+    return matmul_device(static_cast<State *>(opaque), din, dout, rows, iw, ow, weight, bias, error, capacity);
+}
+extern "C" int mynah_hip_matmul_dev(void *opaque, const float *din, float *dout, size_t rows, size_t iw, size_t ow,
+                                    const float *weight, const float *bias, char *error, size_t capacity) {
+    return matmul_device(static_cast<State *>(opaque), din, dout, rows, iw, ow, weight, bias, error, capacity);
+}
+extern "C" int mynah_hip_matvec_dev(void *opaque, const float *din, float *dout, size_t K, size_t N, const float *weight,
+                                    const float *bias, char *error, size_t capacity) {
+    return matmul_device(static_cast<State *>(opaque), din, dout, 1, K, N, weight, bias, error, capacity);
+}
+extern "C" int mynah_hip_matmul_to_dev(void *opaque, const float *host_in, float *dout, size_t rows, size_t iw, size_t ow,
+                                       const float *weight, const float *bias, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (check_rows(host_in, dout, rows, iw, ow, weight, error, capacity) != 0) return -1;
+    if (ensure_scratch(st, rows * iw * sizeof(float), error, capacity) != 0) return -1;
+    if (copy_to_device(st, st->scratch, host_in, rows * iw * sizeof(float), error, capacity) != 0) return -1;
+    return matmul_device(st, st->scratch, dout, rows, iw, ow, weight, bias, error, capacity);
+}
+extern "C" int mynah_hip_sgemm_dev(void *opaque, int ta, int tb, size_t m, size_t n, size_t k, float alpha, const float *da,
+                                   size_t lda, const float *db, size_t ldb, float beta, float *dc, size_t ldc, char *error,
+                                   size_t capacity) {
+    if (da == nullptr || db == nullptr || dc == nullptr) { set_error(error, capacity, "invalid sgemm arguments"); return -1; }
+    return launch_sgemm(static_cast<State *>(opaque), ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc, error, capacity);
+}
+extern "C" int mynah_hip_softmax_dev(void *opaque, float *d, size_t rows, size_t cols, size_t valid, char *error, size_t capacity) {
+    if (d == nullptr || cols > 0x7fffffffu) { set_error(error, capacity, "invalid softmax arguments"); return -1; }
+    return launch_softmax(static_cast<State *>(opaque), d, rows, cols, valid, error, capacity);
+}
+extern "C" int mynah_hip_copy_dev(void *opaque, float *dst, const float *src, size_t n, char *error, size_t capacity) {
+    if (dst == nullptr || src == nullptr) { set_error(error, capacity, "invalid copy arguments"); return -1; }
+    return launch_copy(static_cast<State *>(opaque), dst, src, n, error, capacity);
+}
+extern "C" int mynah_hip_scale_dev(void *opaque, float *d, size_t n, float scale, char *error, size_t capacity) {
+    if (d == nullptr) { set_error(error, capacity, "invalid scale arguments"); return -1; }
+    return launch_scale(static_cast<State *>(opaque), d, n, scale, error, capacity);
+}
+extern "C" int mynah_hip_clip_dev(void *opaque, float *d, size_t n, char *error, size_t capacity) {
+    if (d == nullptr) { set_error(error, capacity, "invalid clip arguments"); return -1; }
+    return launch_clip(static_cast<State *>(opaque), d, n, error, capacity);
+}
+extern "C" int mynah_hip_argmax_dev(void *opaque, const float *dlogits, size_t vocab, size_t codebook_size, size_t eos_id,
+                                    int allow_eos, unsigned *argmax, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (dlogits == nullptr || argmax == nullptr || vocab == 0 || codebook_size > vocab || eos_id > 0xffffffffu ||
+        vocab > 0x7fffffffu) {   // src/backend.c:829-830
+        set_error(error, capacity, "invalid argmax arguments");
+        return -1;
+    }
+    if (ensure_scratch(st, 256, error, capacity) != 0) return -1;
+    if (ensure_pinned(st, 256, error, capacity) != 0) return -1;
+    unsigned *dres = reinterpret_cast<unsigned *>(st->scratch);
+    if (launch_argmax(st, dlogits, vocab, codebook_size, eos_id >= 0x7fffffffu ? 0x7ffffffeu : eos_id, allow_eos, dres, error, capacity) != 0)
+        return -1;
+    MYNAH_TRY(hipMemcpyAsync(st->pinned, dres, sizeof(unsigned), hipMemcpyDeviceToHost, st->stream));
+    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    *argmax = *static_cast<unsigned *>(st->pinned);
+    return 0;
+}
+
+extern "C" int mynah_hip_self_attention_dev(void *opaque, const float *dqkv, float *dk, float *dv, size_t position,
+                                            size_t cache_stride, size_t valid, size_t heads, size_t head_width, float scale,
+                                            float *dout, char *error, size_t capacity) {
+    const float *q[1] = {dqkv};
+    float *k[1] = {dk}, *v[1] = {dv}, *o[1] = {dout};
+    return attention_table(static_cast<State *>(opaque), 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width,
+                           scale, o, error, capacity);
+}
+extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, const float *dk, const float *dv, size_t valid,
+                                             size_t cache_stride, size_t heads, size_t head_width, float scale, float *dout,
+                                             char *error, size_t capacity) {
+    const float *q[1] = {dq};
+    float *k[1] = {const_cast<float *>(dk)}, *v[1] = {const_cast<float *>(dv)}, *o[1] = {dout};
+    return attention_table(static_cast<State *>(opaque), 0, q, k, v, nullptr, &valid, cache_stride, 1, heads, head_width,
+                           scale, o, error, capacity);
+}
+
+// =========================================================================================== section 2
+extern "C" int mynah_hip_set_quant(void *opaque, int qtype, int arith, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (qtype < MYNAH_HIP_F32 || qtype > MYNAH_HIP_F16 || arith < 0 || arith > 1) {
+        set_error(error, capacity, "unknown quantisation mode");
+        return -1;
+    }
+    st->qtype = qtype;
+    st->arith = arith;
+    return 0;
+}
+
+extern "C" int mynah_hip_matmul_d2d_batched(void *opaque, const float *const *din, float *const *dout, size_t batch, size_t iw,
+                                            size_t ow, const float *weight, const float *bias, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (batch == 0) return 0;   // src/qmat.c:826
+    if (batch > (size_t)kMaxBatch) {
+        set_error(error, capacity, "batch exceeds MYNAH_MAX_BATCH");
+        return -1;
+    }
+    if (check_rows(din, dout, batch, iw, ow, weight, error, capacity) != 0) return -1;
+    for (size_t b = 0; b < batch; ++b)
+        if (din[b] == nullptr || dout[b] == nullptr) {
+            set_error(error, capacity, "invalid matmul arguments");
+            return -1;
+        }
+    return linear_rows(st, din, dout, batch, iw, ow, weight, bias, nullptr, nullptr, nullptr, error, capacity);
+}
+
+extern "C" int mynah_hip_matmul_d2d_probe(void *opaque, const float *din, float *dout, size_t iw, size_t ow,
+                                          const float *weight, const float *bias, int8_t *dqx, float *dsx, int32_t *dacc,
+                                          char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (check_rows(din, dout, 1, iw, ow, weight, error, capacity) != 0) return -1;
+    const float *in[1] = {din};
+    float *out[1] = {dout};
+    return linear_rows(st, in, out, 1, iw, ow, weight, bias, dqx, dsx, dacc, error, capacity);
+}
+
+extern "C" int mynah_hip_self_attention_dev_batched(void *opaque, const float *const *dqkv, float *const *dk, float *const *dv,
+                                                    const size_t *position, size_t cache_stride, const size_t *valid,
+                                                    size_t batch, size_t heads, size_t head_width, float scale,
+                                                    float *const *dout, char *error, size_t capacity) {
+    if (dqkv == nullptr || dk == nullptr || dv == nullptr || position == nullptr || valid == nullptr || dout == nullptr) {
+        set_error(error, capacity, "attention: null buffer");
+        return -1;
+    }
+    return attention_table(static_cast<State *>(opaque), 1, dqkv, dk, dv, position, valid, cache_stride, batch, heads,
+                           head_width, scale, dout, error, capacity);
+}
+extern "C" int mynah_hip_cross_attention_dev_batched(void *opaque, const float *const *dq, const float *const *dk,
+                                                     const float *const *dv, const size_t *valid, size_t cache_stride,
+                                                     size_t batch, size_t heads, size_t head_width, float scale,
+                                                     float *const *dout, char *error, size_t capacity) {
+    if (dq == nullptr || dk == nullptr || dv == nullptr || valid == nullptr || dout == nullptr || batch > (size_t)kMaxBatch) {
+        set_error(error, capacity, "attention: null buffer or batch exceeds MYNAH_MAX_BATCH");
+        return -1;
+    }
+    float *k[kMaxBatch], *v[kMaxBatch];
+    for (size_t b = 0; b < batch; ++b) {
+        k[b] = const_cast<float *>(dk[b]);
+        v[b] = const_cast<float *>(dv[b]);
+    }
+    return attention_table(static_cast<State *>(opaque), 0, dq, k, v, nullptr, valid, cache_stride, batch, heads, head_width,
+                           scale, dout, error, capacity);
+}
+
+extern "C" int mynah_hip_embed_gather(void *opaque, const float *const *tables, const size_t *table_rows, size_t table_count,
+                                      const int32_t *ids, size_t tokens, size_t width, float scale, const float *position,
+                                      size_t position_offset, float *dout, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (tables == nullptr || table_rows == nullptr || ids == nullptr || dout == nullptr || table_count == 0 || table_count > 32 ||
+        width == 0 || width > 0x7fffffffu) {
+        set_error(error, capacity, "invalid gather arguments");
+        return -1;
+    }
+    if (tokens == 0) return 0;
+    for (size_t t = 0; t < tokens; ++t)
+        for (size_t j = 0; j < table_count; ++j) {
+            const int32_t id = ids[t * table_count + j];
+            if (id < 0 || (size_t)id >= table_rows[j]) {   // src/graph.c:730-735
+                set_error(error, capacity, "text token id is outside vocabulary");
+                return -1;
+            }
+        }
+    const float *dtables[32];
+    for (size_t j = 0; j < table_count; ++j) {
+        const CachedWeight *cw = nullptr;
+        if (cached_matrix(st, tables[j], table_rows[j], width, MYNAH_HIP_F32, &cw, error, capacity) != 0) return -1;
+        dtables[j] = static_cast<const float *>(cw->data);
+    }
+    const float *dpos = nullptr;
+    if (position != nullptr) {
+        if (cached_vector(st, position + position_offset * width, tokens * width, &dpos, error, capacity) != 0) return -1;
+    }
+    const size_t id_bytes = tokens * table_count * sizeof(int32_t);
+    if (ensure_scratch(st, id_bytes, error, capacity) != 0) return -1;
+    if (copy_to_device(st, st->scratch, ids, id_bytes, error, capacity) != 0) return -1;
+    return launch_gather(st, dtables, table_count, reinterpret_cast<const int32_t *>(st->scratch), tokens, width, scale, dpos,
+                         dout, error, capacity);
+}
+
+extern "C" int mynah_hip_output_head(void *opaque, const float *const *dhidden, size_t batch, size_t width, const float *weight,
+                                     const float *bias, size_t rows, size_t vocab, float *const *dlogits,
+                                     float *const *dprobs, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (batch == 0) return 0;
+    if (batch > (size_t)kMaxBatch || dhidden == nullptr || dlogits == nullptr || vocab == 0 || rows % vocab != 0) {
+        set_error(error, capacity, "invalid output head arguments");
+        return -1;
+    }
+    if (linear_rows(st, dhidden, dlogits, batch, width, rows, weight, bias, nullptr, nullptr, nullptr, error, capacity) != 0)
+        return -1;
+    if (dprobs != nullptr)
+        for (size_t b = 0; b < batch; ++b)
+            if (dprobs[b] != nullptr &&
+                launch_softmax_heads(st, dlogits[b], dprobs[b], rows / vocab, vocab, error, capacity) != 0)
+                return -1;
+    return 0;
+}
+
+// =========================================================================================== measurement
+__global__ void __launch_bounds__(256) k_flush(uint4 *p, size_t n16) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (; i < n16; i += stride) {
+        uint4 v = p[i];
+        v.x += 1u;
+        p[i] = v;
+    }
+}
+
+extern "C" int mynah_hip_timer_begin(void *opaque, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    return hip_check(hipEventRecord(st->ev0, st->stream), "event record", error, capacity);
+}
+extern "C" int mynah_hip_timer_end(void *opaque, float *ms, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    MYNAH_TRY(hipEventRecord(st->ev1, st->stream));
+    MYNAH_TRY(hipEventSynchronize(st->ev1));
+    MYNAH_TRY(hipEventElapsedTime(ms, st->ev0, st->ev1));
+    return 0;
+}
+extern "C" int mynah_hip_flush_cache(void *opaque, size_t bytes, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (bytes < (1u << 20)) bytes = 1u << 20;
+    if (st->flush_bytes < bytes) {
+        if (st->flush != nullptr) {
+            MYNAH_TRY(hipStreamSynchronize(st->stream));
+            (void)hipFree(st->flush);
+            st->flush = nullptr;
+            st->flush_bytes = 0;
+        }
+        MYNAH_TRY(hipMalloc(&st->flush, bytes));
+        MYNAH_TRY(hipMemsetAsync(st->flush, 0, bytes, st->stream));
+        st->flush_bytes = bytes;
+    }
+    hipLaunchKernelGGL(k_flush, dim3(2048), dim3(256), 0, st->stream, static_cast<uint4 *>(st->flush), bytes / 16);
+    return hip_check(hipGetLastError(), "flush launch", error, capacity);
+}
+extern "C" int mynah_hip_set_graph_mode(void *opaque, int enabled, char *error, size_t capacity) {
+    (void)error; (void)capacity;
+    static_cast<State *>(opaque)->graph_mode = enabled ? 1 : 0;
+    return 0;
+}
+extern "C" size_t mynah_hip_cached_weight_bytes(void *opaque) { return static_cast<State *>(opaque)->weight_bytes; }
+
+// =========================================================================================== self test
+namespace mynah {
+
+static bool near(float a, float b, float tol) { return fabsf(a - b) <= tol; }
+
+// The matmul/sgemm KATs of gpu/cuda/backend_cuda.cu:514-529 (same numbers as src/backend.c:290-310) and
+// the resident-op KATs of gpu/metal/backend_metal_ops.m:1038-1107 (codec ops excluded).
+// Arrays are static: the weight cache keys on the host address and never refreshes it.
+static int backend_self_test(void *opaque, char *error, size_t capacity) {
+    static const float in[6] = {1, 2, 3, -1, 0.5f, 2};
+    static const float w[12] = {1, 0, 0, 0, 1, 0, 0, 0, 1, 1, 1, 1};
+    static const float bi[4] = {0.5f, -0.5f, 1, 2};
+    const float want[8] = {1.5f, 1.5f, 4, 8, -0.5f, 0, 3, 3.5f};
+    float got[8] = {0};
+    if (hip_matmul(opaque, in, got, 2, 3, 4, w, bi, error, capacity) != 0) return -1;
+    for (int i = 0; i < 8; ++i)
+        if (!near(got[i], want[i], 1e-5f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP matmul mismatch %d: %f != %f", i, got[i], want[i]);
+            return -1;
+        }
+    float so[8] = {0};
+    if (hip_sgemm(opaque, 0, 1, 2, 4, 3, 1.0f, in, 3, w, 3, 0.0f, so, 4, error, capacity) != 0) return -1;
+    const float sw[8] = {1, 2, 3, 6, -1, 0.5f, 2, 1.5f};
+    for (int i = 0; i < 8; ++i)
+        if (!near(so[i], sw[i], 1e-5f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP sgemm mismatch %d: %f != %f", i, so[i], sw[i]);
+            return -1;
+        }
+
+    static const float vin[2] = {1.0f, 2.0f};
+    static const float eye[4] = {1.0f, 0.0f, 0.0f, 1.0f};
+    static const float b2[2] = {0.5f, -0.5f};
+    static const float qkv1[6] = {1.0f, 0.0f, 1.0f, 0.0f, 2.0f, 3.0f};
+    static const float qkv2[6] = {1.0f, 0.0f, 0.0f, 1.0f, 4.0f, 5.0f};
+    static const float gain[2] = {1.0f, 1.0f};
+    float *din = nullptr, *dout = nullptr, *dtmp = nullptr, *dqkv = nullptr, *dsk = nullptr, *dsv = nullptr;
+    float o[2];
+    int rc = -1;
+    const float e1 = expf(1.0f);
+    do {
+        if (mynah_hip_dev_alloc(opaque, 2, &din, error, capacity) != 0 || mynah_hip_dev_alloc(opaque, 2, &dout, error, capacity) != 0 ||
+            mynah_hip_dev_alloc(opaque, 2, &dtmp, error, capacity) != 0 || mynah_hip_dev_alloc(opaque, 6, &dqkv, error, capacity) != 0 ||
+            mynah_hip_dev_alloc(opaque, 4, &dsk, error, capacity) != 0 || mynah_hip_dev_alloc(opaque, 4, &dsv, error, capacity) != 0)
+            break;
+        if (mynah_hip_h2d(opaque, vin, din, 2, error, capacity) != 0 ||
+            mynah_hip_matmul_d2d(opaque, din, dout, 1, 2, 2, eye, b2, error, capacity) != 0 ||
+            mynah_hip_d2h(opaque, dout, o, 2, error, capacity) != 0)
+            break;
+        if (!near(o[0], 1.5f, 1e-5f) || !near(o[1], 1.5f, 1e-5f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP matmul_d2d mismatch: %.8g %.8g (want 1.5 1.5)", o[0], o[1]);
+            break;
+        }
+        if (mynah_hip_h2d(opaque, qkv1, dqkv, 6, error, capacity) != 0 ||
+            mynah_hip_self_attention_dev(opaque, dqkv, dsk, dsv, 0, 2, 1, 1, 2, 1.0f, dout, error, capacity) != 0 ||
+            mynah_hip_d2h(opaque, dout, o, 2, error, capacity) != 0)
+            break;
+        if (!near(o[0], 2.0f, 1e-5f) || !near(o[1], 3.0f, 1e-5f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP 1-token attention mismatch: %.8g %.8g (want 2 3)", o[0], o[1]);
+            break;
+        }
+        if (mynah_hip_h2d(opaque, qkv2, dqkv, 6, error, capacity) != 0 ||
+            mynah_hip_self_attention_dev(opaque, dqkv, dsk, dsv, 1, 2, 2, 1, 2, 1.0f, dout, error, capacity) != 0 ||
+            mynah_hip_d2h(opaque, dout, o, 2, error, capacity) != 0)
+            break;
+        if (!near(o[0], (2.0f * e1 + 4.0f) / (e1 + 1.0f), 1e-5f) || !near(o[1], (3.0f * e1 + 5.0f) / (e1 + 1.0f), 1e-5f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP 2-token attention mismatch: %.8g %.8g", o[0], o[1]);
+            break;
+        }
+        if (mynah_hip_cross_attention_dev(opaque, din, dsk, dsv, 1, 2, 1, 2, 1.0f, dout, error, capacity) != 0 ||
+            mynah_hip_d2h(opaque, dout, o, 2, error, capacity) != 0)
+            break;
+        if (!near(o[0], 2.0f, 1e-5f) || !near(o[1], 3.0f, 1e-5f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP cross attention mismatch: %.8g %.8g", o[0], o[1]);
+            break;
+        }
+        const float zeros[2] = {0.0f, 0.0f};
+        if (mynah_hip_h2d(opaque, zeros, dtmp, 2, error, capacity) != 0 || mynah_hip_sync(opaque, error, capacity) != 0 ||
+            mynah_hip_gelu_inplace(opaque, dout, 2, error, capacity) != 0 ||
+            mynah_hip_residual_inplace(opaque, dtmp, dout, 2, error, capacity) != 0 ||
+            mynah_hip_layer_norm_inplace(opaque, dout, dtmp, gain, 1, 2, error, capacity) != 0 ||
+            mynah_hip_d2h(opaque, dtmp, o, 2, error, capacity) != 0)
+            break;
+        // gelu(2), gelu(3) normalised over two elements: -1/+1 up to eps
+        if (!near(o[0], -1.0f, 1e-3f) || !near(o[1], 1.0f, 1e-3f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP gelu/residual/layer norm chain mismatch: %.8g %.8g", o[0], o[1]);
+            break;
+        }
+        const float clip_values[2] = {-2.0f, NAN};
+        if (mynah_hip_h2d(opaque, clip_values, dtmp, 2, error, capacity) != 0 || mynah_hip_sync(opaque, error, capacity) != 0 ||
+            mynah_hip_clip_dev(opaque, dtmp, 2, error, capacity) != 0 || mynah_hip_d2h(opaque, dtmp, o, 2, error, capacity) != 0)
+            break;
+        if (o[0] != -1.0f || o[1] != 0.0f) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP clip mismatch: %.8g %.8g (want -1 0)", o[0], o[1]);
+            break;
+        }
+        rc = 0;
+    } while (0);
+    mynah_hip_dev_free(opaque, din);
+    mynah_hip_dev_free(opaque, dout);
+    mynah_hip_dev_free(opaque, dtmp);
+    mynah_hip_dev_free(opaque, dqkv);
+    mynah_hip_dev_free(opaque, dsk);
+    mynah_hip_dev_free(opaque, dsv);
+    if (rc != 0 && error != nullptr && capacity > 0 && error[0] == '\0') snprintf(error, capacity, "HIP resident ops self-test mismatch");
+    return rc;
+}
+
+}  // namespace mynah

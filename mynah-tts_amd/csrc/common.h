@@ -1,0 +1,109 @@
+// Shared host/device definitions for the gfx950 backend.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include <cstdio>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/mynah_hip.h"
+
+namespace mynah {
+
+constexpr int kWave = 64;            // CDNA wavefront
+constexpr int kMaxBatch = MYNAH_HIP_MAX_BATCH;
+constexpr int kBatchTile = 8;        // streams served by one pass over a weight tile
+constexpr size_t kQuantMaxRows = 16; // QMAT_SMALL_COUNT, src/qmat.c:32
+constexpr size_t kQuantMaxK = 8192;  // QMAT_K_MAX, src/qmat.c:33
+constexpr int kAttnChunk = 64;       // cache positions handled by one attention workgroup
+
+// ---- error plumbing (0 / -1 + message, src/backend.c:137-139) ----
+inline void set_error(char *error, size_t capacity, const char *message) {
+    if (error != nullptr && capacity > 0) snprintf(error, capacity, "%s", message);
+}
+inline int hip_check(hipError_t r, const char *what, char *error, size_t capacity) {
+    if (r == hipSuccess) return 0;
+    if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP %s: %s", what, hipGetErrorString(r));
+    return -1;
+}
+#define MYNAH_TRY(expr) do { if (hip_check((expr), #expr, error, capacity) != 0) return -1; } while (0)
+
+// ---- device-resident copy of one host tensor, converted at first sight ----
+struct CachedWeight {
+    int qtype = MYNAH_HIP_F32;   // storage actually used
+    size_t n = 0, k = 0;
+    void *data = nullptr;        // f32 [n,k] | int8 [n,k] | nibbles [n,k/2] | f16 [n,k]
+    float *scales = nullptr;     // int8 [n] | int4 [n,k/32]
+    size_t bytes = 0;
+};
+
+struct WeightKey {
+    const void *host;
+    size_t bytes;
+    int kind;   // 0 plain f32 vector/matrix, 1 + qtype*2 + arith for converted matrices
+    bool operator==(const WeightKey &o) const { return host == o.host && bytes == o.bytes && kind == o.kind; }
+};
+struct WeightKeyHash {
+    size_t operator()(const WeightKey &k) const {
+        return std::hash<const void *>()(k.host) ^ (k.bytes * 0x9e3779b97f4a7c15ull) ^ ((size_t)k.kind << 56);
+    }
+};
+
+// Per-step dynamic data of the resident decode step; lives in device memory so a captured graph can
+// be replayed with new lengths and pointers.
+struct StepSlots {
+    float *self_k[kMaxBatch];
+    float *self_v[kMaxBatch];
+    const float *cross_k[kMaxBatch];
+    const float *cross_v[kMaxBatch];
+    const float *input[kMaxBatch];
+    float *output[kMaxBatch];
+    int length[kMaxBatch];
+    int memory_length[kMaxBatch];
+};
+
+struct State {
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    int cu_count = 256;
+    int qtype = MYNAH_HIP_F32;
+    int arith = MYNAH_HIP_ARITH_STRICT;
+    int graph_mode = 1;
+    std::mutex mu;
+    std::unordered_map<WeightKey, CachedWeight, WeightKeyHash> weights;
+    size_t weight_bytes = 0;
+    // upload scratch (src/backend.h:78-81) and pinned staging for h2d/d2h
+    float *scratch = nullptr;
+    size_t scratch_bytes = 0;
+    void *pinned = nullptr;
+    size_t pinned_bytes = 0;
+    // cache-flush buffer
+    void *flush = nullptr;
+    size_t flush_bytes = 0;
+    // attention split-L partials + arrival counters
+    float *attn_partial = nullptr;
+    size_t attn_partial_floats = 0;
+    unsigned *attn_counters = nullptr;
+    // small device block for batched pointer tables of the section-2 calls
+    void *ptr_table = nullptr;
+    void *ptr_table_host = nullptr;   // pinned
+};
+
+// weight cache (backend_hip.hip)
+int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qtype, const CachedWeight **out,
+                  char *error, size_t capacity);
+int cached_vector(State *st, const float *host, size_t n, const float **dev, char *error, size_t capacity);
+int ensure_attention_workspace(State *st, size_t batch, size_t heads, size_t head_width, size_t max_valid,
+                               char *error, size_t capacity);
+int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity);
+
+// host quantisers (quantize_host.cpp)
+void quantize_weight_int8(const float *w, size_t n, size_t k, int8_t *q, float *scales, int arith);
+int quantize_weight_int4(const float *w, size_t n, size_t k, uint8_t *q, float *scales, int arith);
+uint16_t f32_to_f16_rne(float value);
+
+}  // namespace mynah

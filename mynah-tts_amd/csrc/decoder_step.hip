@@ -1,0 +1,286 @@
+// The resident batched decode step: decoder_step_batch (src/graph.c:3127-3284) as eight fused
+// kernels per layer, replayed as one HIP graph.
+//
+//   per layer   1  LN(norm_self) + act-quant + QKV matvec                      -> qkv
+//               2  self-attention with KV append (split over cache chunks)     -> attn
+//               3  act-quant + O matvec + residual                             -> x
+//               4  LN(norm_xattn_query) + act-quant + Q matvec                 -> qx
+//               5  cross-attention over the encoder memory                     -> ctx
+//               6  act-quant + O matvec + residual                             -> x
+//               7  LN(norm_pos_ff) + act-quant + up matvec + tanh-GELU         -> hidden
+//               8  act-quant + down matvec + residual                          -> x
+//   begin / end    x = input + position[length]   /   out = LN(norm_out)(x)
+//
+// Everything that changes from step to step (cache pointers, lengths, input/output rows) lives in a
+// small device-side slot table written by the begin kernel, so the captured graph is replayed
+// unchanged for the life of a (decoder, batch size) pair.
+#include <string.h>
+
+#include <new>
+
+#include "kernels.h"
+
+namespace mynah {
+
+struct LayerWeights {
+    const CachedWeight *qkv, *o_self, *q_cross, *o_cross, *up, *down;
+    const float *norm_self, *norm_self_b, *norm_cross, *norm_cross_b, *norm_ff, *norm_ff_b;
+};
+
+}  // namespace mynah
+
+struct mynah_hip_decoder {
+    size_t layers, width, heads, head_width, ffn, cross_heads, cross_head_width, xw, capacity;
+    std::vector<mynah::LayerWeights> lw;
+    const float *norm_out = nullptr, *norm_out_b = nullptr, *position = nullptr;
+    // workspaces, kMaxBatch rows each
+    float *x = nullptr, *qkv = nullptr, *attn = nullptr, *qx = nullptr, *ctx = nullptr, *hidden = nullptr;
+    mynah::StepSlots *dev_slots = nullptr;
+    hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};
+    int eager_steps[mynah::kMaxBatch + 1] = {};   // a batch size runs eagerly once before it is captured
+    int arith = 0;
+};
+
+namespace mynah {
+
+static int enqueue_linear(State *st, const mynah_hip_decoder *d, const CachedWeight *w, const float *in, size_t in_stride,
+                          float *out, size_t out_stride, int batch, const float *ln_gain, const float *ln_bias, int epilogue,
+                          char *error, size_t capacity) {
+    for (int b0 = 0; b0 < batch; b0 += kBatchTile) {
+        LinearArgs a{};
+        a.w = w->data;
+        a.scales = w->scales;
+        a.bias = nullptr;   // no decoder linear has a bias (src/graph.c:3169-3272 pass NULL)
+        a.qtype = w->qtype;
+        a.n = (int)w->n;
+        a.k = (int)w->k;
+        a.batch = batch - b0 < kBatchTile ? batch - b0 : kBatchTile;
+        for (int b = 0; b < a.batch; ++b) {
+            a.in[b] = in + (size_t)(b0 + b) * in_stride;
+            a.out[b] = out + (size_t)(b0 + b) * out_stride;
+        }
+        a.ln_gain = ln_gain;
+        a.ln_bias = ln_bias;
+        a.epilogue = epilogue;
+        a.arith = d->arith;
+        if (launch_linear(st, a, error, capacity) != 0) return -1;
+    }
+    return 0;
+}
+
+static int enqueue_attention(State *st, const mynah_hip_decoder *d, int is_self, size_t layer, int batch, char *error,
+                             size_t capacity) {
+    AttnArgs a{};
+    a.slots = d->dev_slots;
+    a.layer = layer;
+    a.capacity = d->capacity;
+    a.batch = batch;
+    a.is_self = is_self;
+    a.partial = st->attn_partial;
+    a.counters = st->attn_counters;
+    if (is_self) {
+        a.q[0] = d->qkv;
+        a.out[0] = d->attn;
+        a.heads = (int)d->heads;
+        a.head_width = (int)d->head_width;
+        a.stride = (int)d->width;
+        a.q_stride = (int)(3 * d->width);
+        a.scale = 1.0f / sqrtf((float)d->head_width);
+        a.max_chunks = (int)((d->capacity + kAttnChunk - 1) / kAttnChunk);
+    } else {
+        a.q[0] = d->qx;
+        a.out[0] = d->ctx;
+        a.heads = (int)d->cross_heads;
+        a.head_width = (int)d->cross_head_width;
+        a.stride = (int)d->xw;
+        a.q_stride = (int)d->xw;
+        a.scale = 1.0f / sqrtf((float)d->cross_head_width);
+        a.max_chunks = (int)((d->capacity + kAttnChunk - 1) / kAttnChunk);   // memory_length <= capacity is checked per step
+    }
+    return launch_attention(st, a, error, capacity);
+}
+
+// The layer loop; everything here is replayable (no per-step scalars in kernel arguments).
+static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char *error, size_t capacity) {
+    const size_t w = d->width;
+    for (size_t l = 0; l < d->layers; ++l) {
+        const LayerWeights &lw = d->lw[l];
+        if (enqueue_linear(st, d, lw.qkv, d->x, w, d->qkv, 3 * w, batch, lw.norm_self, lw.norm_self_b, EPI_NONE, error, capacity) != 0) return -1;
+        if (enqueue_attention(st, d, 1, l, batch, error, capacity) != 0) return -1;
+        if (enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
+        if (d->xw != 0) {
+            if (enqueue_linear(st, d, lw.q_cross, d->x, w, d->qx, d->xw, batch, lw.norm_cross, lw.norm_cross_b, EPI_NONE, error, capacity) != 0) return -1;
+            if (enqueue_attention(st, d, 0, l, batch, error, capacity) != 0) return -1;
+            if (enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
+        }
+        if (enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity) != 0) return -1;
+        if (enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
+    }
+    return launch_step_end(st, d->dev_slots, batch, w, d->x, w, d->norm_out, d->norm_out_b, error, capacity);
+}
+
+static int per_layer_vector(State *st, const float *const *arr, size_t layer, size_t n, const float **dev, char *error,
+                            size_t capacity) {
+    *dev = nullptr;
+    if (arr == nullptr || arr[layer] == nullptr) return 0;
+    return cached_vector(st, arr[layer], n, dev, error, capacity);
+}
+
+}  // namespace mynah
+
+using namespace mynah;
+
+extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
+    State *st = static_cast<State *>(opaque);
+    if (d == nullptr) return;
+    if (st != nullptr) (void)hipStreamSynchronize(st->stream);
+    for (auto &g : d->graphs)
+        if (g != nullptr) (void)hipGraphExecDestroy(g);
+    float *bufs[] = {d->x, d->qkv, d->attn, d->qx, d->ctx, d->hidden};
+    for (float *p : bufs)
+        if (p != nullptr) (void)hipFree(p);
+    if (d->dev_slots != nullptr) (void)hipFree(d->dev_slots);
+    delete d;
+}
+
+extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_desc *desc, mynah_hip_decoder **out, char *error,
+                                        size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (out != nullptr) *out = nullptr;
+    if (st == nullptr || desc == nullptr || out == nullptr || desc->layers == 0 || desc->width == 0 || desc->heads == 0 ||
+        desc->heads * desc->head_width != desc->width || desc->ffn_width == 0 || desc->capacity == 0 ||
+        desc->capacity > 0x7ffffff0u || desc->norm_self == nullptr || desc->norm_pos_ff == nullptr || desc->qkv_w == nullptr ||
+        desc->o_self_w == nullptr || desc->ffn_up_w == nullptr || desc->ffn_down_w == nullptr) {
+        set_error(error, capacity, "invalid decoder description");
+        return -1;
+    }
+    const size_t xw = desc->cross_heads * desc->cross_head_width;
+    if (xw != 0 && (desc->q_cross_w == nullptr || desc->o_cross_w == nullptr || desc->norm_xattn_query == nullptr)) {
+        set_error(error, capacity, "decoder description lacks cross-attention weights");
+        return -1;
+    }
+    if (desc->head_width > 1024 || desc->cross_head_width > 1024 || desc->width > 4096 || xw > 4096) {
+        set_error(error, capacity, "decoder head shape not supported");
+        return -1;
+    }
+    if (!linear_fast_supported(MYNAH_HIP_F32, desc->width, desc->width) ||
+        !linear_fast_supported(MYNAH_HIP_F32, desc->width, desc->ffn_width) ||
+        (xw != 0 && !linear_fast_supported(MYNAH_HIP_F32, desc->width, xw))) {
+        set_error(error, capacity, "decoder widths must be multiples of 256 and at most 3072 for the resident step");
+        return -1;
+    }
+    mynah_hip_decoder *d = new (std::nothrow) mynah_hip_decoder();
+    if (d == nullptr) {
+        set_error(error, capacity, "out of memory creating decoder");
+        return -1;
+    }
+    d->layers = desc->layers; d->width = desc->width; d->heads = desc->heads; d->head_width = desc->head_width;
+    d->ffn = desc->ffn_width; d->cross_heads = desc->cross_heads; d->cross_head_width = desc->cross_head_width;
+    d->xw = xw; d->capacity = desc->capacity; d->arith = st->arith;
+    d->lw.resize(desc->layers);
+    const size_t w = d->width;
+    int rc = 0;
+    for (size_t l = 0; l < d->layers && rc == 0; ++l) {
+        LayerWeights &lw = d->lw[l];
+        rc |= cached_matrix(st, desc->qkv_w[l], 3 * w, w, st->qtype, &lw.qkv, error, capacity);
+        rc |= cached_matrix(st, desc->o_self_w[l], w, w, st->qtype, &lw.o_self, error, capacity);
+        if (xw != 0) {
+            rc |= cached_matrix(st, desc->q_cross_w[l], xw, w, st->qtype, &lw.q_cross, error, capacity);
+            rc |= cached_matrix(st, desc->o_cross_w[l], w, xw, st->qtype, &lw.o_cross, error, capacity);
+            rc |= per_layer_vector(st, desc->norm_xattn_query, l, w, &lw.norm_cross, error, capacity);
+            rc |= per_layer_vector(st, desc->norm_xattn_query_bias, l, w, &lw.norm_cross_b, error, capacity);
+        }
+        rc |= cached_matrix(st, desc->ffn_up_w[l], d->ffn, w, st->qtype, &lw.up, error, capacity);
+        rc |= cached_matrix(st, desc->ffn_down_w[l], w, d->ffn, st->qtype, &lw.down, error, capacity);
+        rc |= per_layer_vector(st, desc->norm_self, l, w, &lw.norm_self, error, capacity);
+        rc |= per_layer_vector(st, desc->norm_self_bias, l, w, &lw.norm_self_b, error, capacity);
+        rc |= per_layer_vector(st, desc->norm_pos_ff, l, w, &lw.norm_ff, error, capacity);
+        rc |= per_layer_vector(st, desc->norm_pos_ff_bias, l, w, &lw.norm_ff_b, error, capacity);
+        if (rc == 0 && (lw.norm_self == nullptr || lw.norm_ff == nullptr || (xw != 0 && lw.norm_cross == nullptr))) {
+            set_error(error, capacity, "decoder description lacks a LayerNorm gain");
+            rc = -1;
+        }
+    }
+    if (rc == 0) rc |= cached_vector(st, desc->norm_out, w, &d->norm_out, error, capacity);
+    if (rc == 0) rc |= cached_vector(st, desc->norm_out_bias, w, &d->norm_out_b, error, capacity);
+    if (rc == 0 && desc->position != nullptr) rc |= cached_vector(st, desc->position, d->capacity * w, &d->position, error, capacity);
+    const size_t B = kMaxBatch;
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->x), B * w * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->qkv), B * 3 * w * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->attn), B * w * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->qx), B * (xw ? xw : 4) * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->ctx), B * (xw ? xw : 4) * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->hidden), B * d->ffn * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->dev_slots), sizeof(StepSlots)), "malloc", error, capacity);
+    const size_t hw_max = d->head_width > d->cross_head_width ? d->head_width : d->cross_head_width;
+    const size_t heads_max = d->heads > d->cross_heads ? d->heads : d->cross_heads;
+    if (rc == 0) rc |= ensure_attention_workspace(st, B, heads_max, hw_max, d->capacity, error, capacity);
+    if (rc != 0) {
+        mynah_hip_decoder_destroy(opaque, d);
+        return -1;
+    }
+    *out = d;
+    return 0;
+}
+
+extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch,
+                                      char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (batch == 0) return 0;   // src/graph.c:3132
+    if (batch > (size_t)kMaxBatch) {
+        set_error(error, capacity, "decoder batch exceeds MYNAH_MAX_BATCH");   // src/graph.c:3133-3136
+        return -1;
+    }
+    if (st == nullptr || d == nullptr || slots == nullptr) {
+        set_error(error, capacity, "invalid decoder step arguments");
+        return -1;
+    }
+    StepSlots s;
+    memset(&s, 0, sizeof s);
+    for (size_t b = 0; b < batch; ++b) {
+        const mynah_hip_decoder_slot &in = slots[b];
+        if (in.length >= d->capacity) {
+            set_error(error, capacity, "decoder cache capacity exceeded");   // src/graph.c:3152-3155
+            return -1;
+        }
+        if (in.dev_self_k == nullptr || in.dev_self_v == nullptr || in.dev_input == nullptr || in.dev_output == nullptr ||
+            (d->xw != 0 && in.memory_length != 0 && (in.dev_cross_k == nullptr || in.dev_cross_v == nullptr))) {
+            set_error(error, capacity, "decoder slot has a null buffer");
+            return -1;
+        }
+        if (in.memory_length > d->capacity) {
+            set_error(error, capacity, "decoder memory length exceeds the attention workspace (capacity)");
+            return -1;
+        }
+        s.self_k[b] = in.dev_self_k;
+        s.self_v[b] = in.dev_self_v;
+        s.cross_k[b] = in.dev_cross_k;
+        s.cross_v[b] = in.dev_cross_v;
+        s.input[b] = in.dev_input;
+        s.output[b] = in.dev_output;
+        s.length[b] = (int)in.length;
+        s.memory_length[b] = (int)in.memory_length;
+    }
+    const int B = (int)batch;
+    if (launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
+    if (!st->graph_mode || d->eager_steps[B] == 0) {
+        // the first step of a batch size also performs one-time kernel attribute set-up, which does not belong in a capture
+        d->eager_steps[B] = 1;
+        return enqueue_layers(st, d, B, error, capacity);
+    }
+    if (d->graphs[B] == nullptr) {
+        hipGraph_t graph = nullptr;
+        MYNAH_TRY(hipStreamBeginCapture(st->stream, hipStreamCaptureModeThreadLocal));
+        const int rc = enqueue_layers(st, d, B, error, capacity);
+        const hipError_t end = hipStreamEndCapture(st->stream, &graph);
+        if (rc != 0) {
+            if (graph != nullptr) (void)hipGraphDestroy(graph);
+            return -1;
+        }
+        MYNAH_TRY(end);
+        const hipError_t inst = hipGraphInstantiate(&d->graphs[B], graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        MYNAH_TRY(inst);
+    }
+    return hip_check(hipGraphLaunch(d->graphs[B], st->stream), "graph launch", error, capacity);
+}

@@ -1,0 +1,86 @@
+// Launch wrappers of the device kernels (kernels_linear.hip, kernels_attention.hip, kernels_misc.hip).
+#pragma once
+
+#include "common.h"
+
+namespace mynah {
+
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_RESIDUAL = 2 };
+
+// One weight-stationary pass: out[b][n] = epilogue(W * prologue(in[b])) for up to kBatchTile streams.
+struct LinearArgs {
+    const void *w;          // packed weight, storage `qtype`
+    const float *scales;    // int8 [n] | int4 [n, k/32]
+    const float *bias;      // [n] or null
+    int qtype;
+    int n, k;
+    int batch;              // streams in this pass (<= kBatchTile)
+    const float *in[kBatchTile];
+    float *out[kBatchTile];
+    const float *ln_gain;   // non-null: LayerNorm prologue (eps 1e-5)
+    const float *ln_bias;   // may be null
+    int epilogue;           // EPI_*
+    int arith;              // MYNAH_HIP_ARITH_*: how the activation scale is formed
+    int8_t *probe_qx;       // parity probes (null in production)
+    float *probe_sx;
+    int32_t *probe_acc;
+};
+
+// True when the fused matvec kernel supports this shape/storage; otherwise use linear_generic.
+bool linear_fast_supported(int qtype, size_t n, size_t k);
+int launch_linear(State *st, const LinearArgs &args, char *error, size_t capacity);
+// Any shape, f32 weights: out[r,n] = in[r,k] W[n,k]^T + bias (rows may be large).
+int launch_gemm_f32(State *st, const float *in, float *out, size_t rows, size_t k, size_t n, const float *w,
+                    const float *bias, char *error, size_t capacity);
+int launch_sgemm(State *st, int ta, int tb, size_t m, size_t n, size_t k, float alpha, const float *a, size_t lda,
+                 const float *b, size_t ldb, float beta, float *c, size_t ldc, char *error, size_t capacity);
+
+// Single-token attention for up to kMaxBatch streams.  Pointers come either from the by-value table
+// (seam calls) or from `slots` in device memory (resident step, replayable as a graph).
+struct AttnArgs {
+    const StepSlots *slots;        // non-null: resident-step mode
+    size_t layer;                  // slots mode: cache offsets are layer * capacity * stride etc.
+    size_t capacity;
+    const float *q[kMaxBatch];     // table mode: q rows (self: the qkv row)
+    float *k_cache[kMaxBatch];
+    float *v_cache[kMaxBatch];
+    float *out[kMaxBatch];
+    int position[kMaxBatch];       // self only: row to append
+    int valid[kMaxBatch];
+    int batch;
+    int heads, head_width;
+    int stride;                    // floats between cache rows
+    int q_stride;                  // slots mode: floats between streams in the q/qkv and out workspaces
+    float scale;
+    int is_self;
+    int max_chunks;                // grid.x
+    float *partial;                // [batch, heads, max_chunks, head_width + 2]
+    unsigned *counters;            // [batch, heads], zero between launches
+};
+int launch_attention(State *st, const AttnArgs &args, char *error, size_t capacity);
+
+int launch_layernorm(State *st, const float *in, float *out, const float *gain, const float *bias, size_t rows,
+                     size_t width, char *error, size_t capacity);
+int launch_gelu(State *st, float *data, size_t n, char *error, size_t capacity);
+int launch_residual(State *st, float *out, const float *in, size_t n, char *error, size_t capacity);
+int launch_copy(State *st, float *dst, const float *src, size_t n, char *error, size_t capacity);
+int launch_scale(State *st, float *data, size_t n, float scale, char *error, size_t capacity);
+int launch_clip(State *st, float *data, size_t n, char *error, size_t capacity);
+int launch_softmax(State *st, float *data, size_t rows, size_t cols, size_t valid, char *error, size_t capacity);
+int launch_softmax_heads(State *st, const float *logits, float *probs, size_t rows, size_t cols, char *error,
+                         size_t capacity);
+int launch_argmax(State *st, const float *logits, size_t vocab, size_t codebook, size_t eos, int allow_eos,
+                  unsigned *dev_result, char *error, size_t capacity);
+int launch_gather(State *st, const float *const *dev_tables, size_t table_count, const int32_t *dev_ids,
+                  size_t tokens, size_t width, float scale, const float *dev_position, float *out, char *error,
+                  size_t capacity);
+int launch_stream_copy(State *st, const void *src, void *dst, size_t bytes, char *error, size_t capacity);
+
+// Resident step: writes the slot table to device memory and forms x[b] = input[b] + position[length[b]].
+int launch_step_begin(State *st, const StepSlots &slots, StepSlots *dev_slots, int batch, size_t width,
+                      const float *dev_position, float *x, size_t x_stride, char *error, size_t capacity);
+// Final norm of the step: out = slots->output[b]; gain may be null (plain copy).
+int launch_step_end(State *st, const StepSlots *dev_slots, int batch, size_t width, const float *x, size_t x_stride,
+                    const float *gain, const float *bias, char *error, size_t capacity);
+
+}  // namespace mynah

@@ -1,0 +1,271 @@
+// Small resident ops of the seam: LayerNorm, GELU, residual, copy/scale/clip, softmax, constrained
+// argmax, embedding gather, and the begin/end kernels of the resident decode step.
+#include <float.h>
+
+#include "kernels.h"
+
+namespace mynah {
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    return v;
+}
+
+// Sum over a 256-thread workgroup in a fixed order: lanes by butterfly, then waves 0..3.
+__device__ __forceinline__ float block_sum(float v, float *s4) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return ((s4[0] + s4[1]) + s4[2]) + s4[3];
+}
+__device__ __forceinline__ float block_max(float v, float *s4) {
+    v = wave_max(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+}
+
+// mynah_layernorm_f32 (src/kernels.c:186-244): mean, then the variance of (x - mean), eps inside the
+// square root, y = (x - mean) * scale * gain (+ bias).  One workgroup per row.
+__device__ __forceinline__ void layernorm_row(const float *x, float *y, const float *gain, const float *bias, int width,
+                                              float *s4) {
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < width; i += 256) s += x[i];
+    const float mean = block_sum(s, s4) / (float)width;
+    float v = 0.0f;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const float d = x[i] - mean;
+        v = __builtin_fmaf(d, d, v);
+    }
+    const float variance = block_sum(v, s4);
+    const float scale = 1.0f / sqrtf(variance / (float)width + 1.0e-5f);
+    for (int i = threadIdx.x; i < width; i += 256) {
+        float z = ((x[i] - mean) * scale) * gain[i];
+        if (bias != nullptr) z += bias[i];
+        y[i] = z;
+    }
+}
+
+__global__ void __launch_bounds__(256) k_layernorm(const float *in, float *out, const float *gain, const float *bias, int width) {
+    __shared__ float s4[4];
+    layernorm_row(in + (size_t)blockIdx.x * width, out + (size_t)blockIdx.x * width, gain, bias, width, s4);
+}
+
+__global__ void __launch_bounds__(256) k_gelu(float *data, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const float x = data[i];
+        const float cubic = x * x * x;
+        const float c = 0.7978845608f * (x + 0.044715f * cubic);
+        data[i] = 0.5f * x * (1.0f + tanhf(c));
+    }
+}
+__global__ void __launch_bounds__(256) k_residual(float *out, const float *in, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] += in[i];
+}
+__global__ void __launch_bounds__(256) k_copy(float *dst, const float *src, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+__global__ void __launch_bounds__(256) k_scale(float *data, size_t n, float scale) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) data[i] *= scale;
+}
+// clamp to [-1, 1]; NaN becomes 0 (gpu/metal/backend_metal_ops.m:1090-1101)
+__global__ void __launch_bounds__(256) k_clip(float *data, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const float v = data[i];
+        data[i] = (v != v) ? 0.0f : (v > 1.0f ? 1.0f : (v < -1.0f ? -1.0f : v));
+    }
+}
+
+// mynah_backend_softmax_dev (src/backend.c:602-619): in place, first `valid` columns, zero tail.
+__global__ void __launch_bounds__(256) k_softmax_masked(float *data, int cols, int valid) {
+    __shared__ float s4[4];
+    float *row = data + (size_t)blockIdx.x * cols;
+    const int v = valid < cols ? valid : cols;
+    float mx = -1e30f;
+    for (int i = threadIdx.x; i < v; i += 256) mx = fmaxf(mx, row[i]);
+    mx = block_max(mx, s4);
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < v; i += 256) {
+        const float e = expf(row[i] - mx);
+        row[i] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, s4);
+    const float inv = 1.0f / sum;
+    for (int i = threadIdx.x; i < v; i += 256) row[i] *= inv;
+    for (int i = v + threadIdx.x; i < cols; i += 256) row[i] = 0.0f;
+}
+
+// mynah_softmax_f32 (src/kernels.c:391-420) per head: p = expf(x - max) * (1 / total).
+__global__ void __launch_bounds__(256) k_softmax_heads(const float *logits, float *probs, int cols) {
+    __shared__ float s4[4];
+    const float *row = logits + (size_t)blockIdx.x * cols;
+    float *prow = probs + (size_t)blockIdx.x * cols;
+    float mx = -FLT_MAX;
+    for (int i = threadIdx.x; i < cols; i += 256) mx = fmaxf(mx, row[i]);
+    mx = block_max(mx, s4);
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < cols; i += 256) sum += expf(row[i] - mx);
+    sum = block_sum(sum, s4);
+    const float inv = 1.0f / sum;
+    for (int i = threadIdx.x; i < cols; i += 256) prow[i] = expf(row[i] - mx) * inv;
+}
+
+// mynah_backend_argmax_dev (src/backend.c:825-847): strict > from -FLT_MAX, first index on ties,
+// result 0 when no candidate beats -FLT_MAX.  One workgroup.
+__global__ void __launch_bounds__(256) k_argmax(const float *logits, int vocab, int codebook, int eos, int allow_eos,
+                                                unsigned *result) {
+    __shared__ float s_val[256];
+    __shared__ int s_idx[256];
+    float best = -FLT_MAX;
+    int at = 0x7fffffff;
+    for (int i = threadIdx.x; i < vocab; i += 256) {
+        if (!(i < codebook || (allow_eos && i == eos))) continue;
+        const float v = logits[i];
+        if (v > best) { best = v; at = i; }   // ascending i inside a thread: first max kept
+    }
+    s_val[threadIdx.x] = best;
+    s_idx[threadIdx.x] = at;
+    __syncthreads();
+    for (int half = 128; half > 0; half >>= 1) {
+        if (threadIdx.x < half) {
+            const float ov = s_val[threadIdx.x + half];
+            const int oi = s_idx[threadIdx.x + half];
+            const float mv = s_val[threadIdx.x];
+            const int mi = s_idx[threadIdx.x];
+            if (ov > mv || (ov == mv && oi < mi)) { s_val[threadIdx.x] = ov; s_idx[threadIdx.x] = oi; }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) result[0] = s_idx[0] == 0x7fffffff ? 0u : (unsigned)s_idx[0];
+}
+
+// Embedding gather: sum of table rows (bit-exact copy for one table and scale 1) + optional position.
+struct GatherTables { const float *t[32]; };
+__global__ void __launch_bounds__(256) k_gather(GatherTables tables, int table_count, const int32_t *ids, int width, float scale,
+                                                const float *position, float *out) {
+    const int t = blockIdx.x;
+    for (int d = threadIdx.x; d < width; d += 256) {
+        float v = tables.t[0][(size_t)ids[(size_t)t * table_count] * width + d];
+        for (int j = 1; j < table_count; ++j) v += tables.t[j][(size_t)ids[(size_t)t * table_count + j] * width + d];
+        if (scale != 1.0f) v *= scale;
+        if (position != nullptr) v += position[(size_t)t * width + d];
+        out[(size_t)t * width + d] = v;
+    }
+}
+
+// Decode-step begin: record the slot table, x[b] = input[b] + position[length[b]] (src/graph.c:3156-3157).
+__global__ void __launch_bounds__(256) k_step_begin(const StepSlots slots, StepSlots *dev_slots, int width, const float *position,
+                                                    float *x, size_t x_stride) {
+    const int b = blockIdx.x;
+    if (b == 0 && threadIdx.x == 0) *dev_slots = slots;
+    const float *in = slots.input[b];
+    const float *pe = position != nullptr ? position + (size_t)slots.length[b] * width : nullptr;
+    for (int d = threadIdx.x; d < width; d += 256) x[(size_t)b * x_stride + d] = pe != nullptr ? in[d] + pe[d] : in[d];
+}
+
+__global__ void __launch_bounds__(256) k_step_end(const StepSlots *slots, int width, const float *x, size_t x_stride,
+                                                  const float *gain, const float *bias) {
+    __shared__ float s4[4];
+    const int b = blockIdx.x;
+    float *out = slots->output[b];
+    const float *row = x + (size_t)b * x_stride;
+    if (gain == nullptr) {
+        for (int d = threadIdx.x; d < width; d += 256) out[d] = row[d];
+        return;
+    }
+    layernorm_row(row, out, gain, bias, width, s4);
+}
+
+inline unsigned blocks_for(size_t n) { return (unsigned)((n + 255) / 256); }
+
+}  // namespace
+
+int launch_layernorm(State *st, const float *in, float *out, const float *gain, const float *bias, size_t rows,
+                     size_t width, char *error, size_t capacity) {
+    if (rows == 0 || width == 0) return 0;
+    hipLaunchKernelGGL(k_layernorm, dim3((unsigned)rows), dim3(256), 0, st->stream, in, out, gain, bias, (int)width);
+    return hip_check(hipGetLastError(), "layernorm launch", error, capacity);
+}
+int launch_gelu(State *st, float *data, size_t n, char *error, size_t capacity) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_gelu, dim3(blocks_for(n)), dim3(256), 0, st->stream, data, n);
+    return hip_check(hipGetLastError(), "gelu launch", error, capacity);
+}
+int launch_residual(State *st, float *out, const float *in, size_t n, char *error, size_t capacity) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_residual, dim3(blocks_for(n)), dim3(256), 0, st->stream, out, in, n);
+    return hip_check(hipGetLastError(), "residual launch", error, capacity);
+}
+int launch_copy(State *st, float *dst, const float *src, size_t n, char *error, size_t capacity) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_copy, dim3(blocks_for(n)), dim3(256), 0, st->stream, dst, src, n);
+    return hip_check(hipGetLastError(), "copy launch", error, capacity);
+}
+int launch_scale(State *st, float *data, size_t n, float scale, char *error, size_t capacity) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_scale, dim3(blocks_for(n)), dim3(256), 0, st->stream, data, n, scale);
+    return hip_check(hipGetLastError(), "scale launch", error, capacity);
+}
+int launch_clip(State *st, float *data, size_t n, char *error, size_t capacity) {
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_clip, dim3(blocks_for(n)), dim3(256), 0, st->stream, data, n);
+    return hip_check(hipGetLastError(), "clip launch", error, capacity);
+}
+int launch_softmax(State *st, float *data, size_t rows, size_t cols, size_t valid, char *error, size_t capacity) {
+    if (rows == 0 || cols == 0) return 0;
+    hipLaunchKernelGGL(k_softmax_masked, dim3((unsigned)rows), dim3(256), 0, st->stream, data, (int)cols, (int)valid);
+    return hip_check(hipGetLastError(), "softmax launch", error, capacity);
+}
+int launch_softmax_heads(State *st, const float *logits, float *probs, size_t rows, size_t cols, char *error,
+                         size_t capacity) {
+    if (rows == 0 || cols == 0) return 0;
+    hipLaunchKernelGGL(k_softmax_heads, dim3((unsigned)rows), dim3(256), 0, st->stream, logits, probs, (int)cols);
+    return hip_check(hipGetLastError(), "softmax launch", error, capacity);
+}
+int launch_argmax(State *st, const float *logits, size_t vocab, size_t codebook, size_t eos, int allow_eos,
+                  unsigned *dev_result, char *error, size_t capacity) {
+    hipLaunchKernelGGL(k_argmax, dim3(1), dim3(256), 0, st->stream, logits, (int)vocab, (int)codebook, (int)eos, allow_eos,
+                       dev_result);
+    return hip_check(hipGetLastError(), "argmax launch", error, capacity);
+}
+int launch_gather(State *st, const float *const *dev_tables, size_t table_count, const int32_t *dev_ids, size_t tokens,
+                  size_t width, float scale, const float *dev_position, float *out, char *error, size_t capacity) {
+    if (tokens == 0) return 0;
+    if (table_count < 1 || table_count > 32) {
+        set_error(error, capacity, "gather: between 1 and 32 tables");
+        return -1;
+    }
+    GatherTables t;
+    for (size_t j = 0; j < 32; ++j) t.t[j] = j < table_count ? dev_tables[j] : nullptr;
+    hipLaunchKernelGGL(k_gather, dim3((unsigned)tokens), dim3(256), 0, st->stream, t, (int)table_count, dev_ids, (int)width, scale,
+                       dev_position, out);
+    return hip_check(hipGetLastError(), "gather launch", error, capacity);
+}
+int launch_step_begin(State *st, const StepSlots &slots, StepSlots *dev_slots, int batch, size_t width,
+                      const float *dev_position, float *x, size_t x_stride, char *error, size_t capacity) {
+    hipLaunchKernelGGL(k_step_begin, dim3((unsigned)batch), dim3(256), 0, st->stream, slots, dev_slots, (int)width, dev_position, x,
+                       x_stride);
+    return hip_check(hipGetLastError(), "step begin launch", error, capacity);
+}
+int launch_step_end(State *st, const StepSlots *dev_slots, int batch, size_t width, const float *x, size_t x_stride,
+                    const float *gain, const float *bias, char *error, size_t capacity) {
+    hipLaunchKernelGGL(k_step_end, dim3((unsigned)batch), dim3(256), 0, st->stream, dev_slots, (int)width, x, x_stride, gain, bias);
+    return hip_check(hipGetLastError(), "step end launch", error, capacity);
+}
+
+}  // namespace mynah

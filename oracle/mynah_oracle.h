@@ -1,0 +1,140 @@
+/* TEST INFRASTRUCTURE ONLY -- a CPU restatement of the reference's decode-step arithmetic.
+ *
+ * Nothing in the shipped library (mynah-tts_amd/csrc, include/) includes, links or calls
+ * this file.  It exists so tests, the smoke check and the benchmark's CPU-baseline leg have
+ * an independent statement of what the reference computes.  Each function cites the
+ * reference file:line it restates (paths relative to the reference tree).
+ *
+ * Pinning status (which independent evidence checks each function; see tests/test_oracle_*.py):
+ *   quantizers, int dots, matvec_q8/q4, act-quant   -- bit-compared with the compiled reference
+ *                                                     (oracle/_ref, both flag sets) + brute force ties
+ *   layernorm, gelu, softmax, argmax, residual      -- reference self-test KATs (src/kernels.c:439-517)
+ *                                                     + float64 closed forms + compiled reference
+ *   self/cross attention                            -- Metal resident-op KATs
+ *                                                     (gpu/metal/backend_metal_ops.m:1049-1079) + float64
+ *                                                     softmax(QK^T)V + compiled reference decode step
+ *   decoder step                                    -- compiled reference decoder_step_batch (f32/int8/int4,
+ *                                                     B=1 and ragged B=8) + batched==solo bit identity
+ *   f16 rounding                                    -- numpy.float16 (IEEE RNE) over all 65536 halves and
+ *                                                     random floats; ingot KATs 0x3c00<->1.0
+ *   matvec_f16                                      -- no x86 reference build exists (src/qmat.c:25-28);
+ *                                                     pinned by float64 dot of exactly-widened halves
+ *   encoder prefill (bidirectional, plain FFN, f16-rounded weights, synthetic config)
+ *                                                   -- float64 numpy restatement + attention/LN/GELU pins
+ *                                                     above; the reference has no function with this exact
+ *                                                     composition (its encoder is causal with conv FFN), and
+ *                                                     its rows>1 GEMM is OpenBLAS, absent here: parity of the
+ *                                                     GEMM rounding order is UNPINNED, tolerance 2e-3.
+ */
+#ifndef MYNAH_ORACLE_H
+#define MYNAH_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ORC_F32 = 0, ORC_INT8 = 1, ORC_INT4 = 2, ORC_F16 = 3 };   /* src/qmat.c:36 */
+enum { ORC_STRICT = 0, ORC_STOCK = 1 };   /* quantizer arithmetic: source as written / stock -ffast-math build */
+
+/* ---- load-time weight conversion ---- */
+void orc_quantize_weight_int8(const float *w, size_t n, size_t k, int8_t *q, float *scales, int variant);
+int orc_quantize_weight_int4(const float *w, size_t n, size_t k, uint8_t *q, float *scales, int variant);
+uint16_t orc_f32_to_f16(float value);
+float orc_f16_to_f32(uint16_t bits);
+void orc_f32_to_f16_array(const float *in, uint16_t *out, size_t n);
+
+/* ---- per-vector activation quantization ---- */
+float orc_quantize_act_int8(int8_t *qx, const float *x, size_t k, int variant);
+
+/* ---- matvec kernels ---- */
+int32_t orc_dot_q8_i32(const int8_t *qx, const int8_t *w, size_t k);
+void orc_matvec_q8(float *out, int32_t *acc_out, const int8_t *qx, float sx, const int8_t *weights,
+                   const float *scales, const float *bias, size_t rows, size_t cols);
+void orc_matvec_q4(float *out, int32_t *group_acc_out, const int8_t *qx, float sx, const uint8_t *weights,
+                   const float *scales, const float *bias, size_t rows, size_t cols);
+void orc_matvec_f16(float *out, const float *x, const uint16_t *weights, const float *bias,
+                    size_t rows, size_t cols);
+void orc_matvec_f32(float *out, const float *x, const float *weights, const float *bias,
+                    size_t rows, size_t cols);
+
+typedef struct {
+    int qtype;           /* ORC_* */
+    size_t n, k;         /* out rows, in columns */
+    const void *data;    /* f32 [n,k] | int8 [n,k] | packed nibbles [n,k/2] | f16 bits [n,k] */
+    const float *scales; /* int8: [n]; int4: [n,k/32]; else NULL */
+} orc_weight;
+
+/* out[n] = W x (+bias): act-quant for int8/int4, f32 activations for f16/f32. */
+void orc_linear(const orc_weight *w, const float *x, float *out, const float *bias, int act_variant);
+
+/* ---- f32 elementwise kernels ---- */
+void orc_layernorm(const float *in, const float *gain, const float *bias, float *out,
+                   size_t rows, size_t width, float eps);
+void orc_gelu_scalar(float *data, size_t n);
+void orc_gelu_pade(float *data, size_t n);
+int orc_softmax(const float *logits, float *probs, size_t n);
+void orc_softmax_row_inplace(float *values, size_t n);
+void orc_softmax_masked(float *data, size_t rows, size_t cols, size_t valid);
+void orc_residual_add(float *out, const float *in, size_t n);
+int orc_argmax_constrained(const float *logits, size_t vocab, size_t codebook_size, size_t eos_id,
+                           int allow_eos, unsigned *argmax);
+
+/* ---- single-token attention ---- */
+void orc_self_attention(const float *qkv, float *k_cache, float *v_cache, size_t position,
+                        size_t cache_stride, size_t valid, size_t heads, size_t head_width,
+                        float scale, float *out, float *scores_scratch);
+void orc_cross_attention(const float *q, const float *k_cache, const float *v_cache, size_t valid,
+                         size_t cache_stride, size_t heads, size_t head_width, float scale,
+                         float *out, float *scores_scratch);
+
+/* ---- whole decode step ---- */
+typedef struct {
+    size_t layers, width, heads, head_width, ffn;
+    size_t cross_heads, cross_head_width;   /* xw = cross_heads * cross_head_width */
+    size_t capacity;
+    const orc_weight *qkv, *o_self, *q_cross, *o_cross, *ffn_up, *ffn_down;   /* [layers] each */
+    const float *norm_self_g, *norm_self_b;     /* [layers,width]; *_b may be NULL (gain-only) */
+    const float *norm_cross_g, *norm_cross_b;
+    const float *norm_ff_g, *norm_ff_b;
+    const float *norm_out_g, *norm_out_b;       /* [width] */
+    const float *position;                      /* [capacity,width] or NULL (no position add) */
+    int act_variant;
+} orc_decoder;
+
+/* B slots, one token each.  self_k/self_v[b]: [layers,capacity,width] appended at lengths[b];
+ * cross_k/cross_v[b]: [layers,memory_lengths[b],xw].  outs[b]: [width] after the final norm.
+ * hidden_out[b] (optional): the pre-final-norm residual stream.  lengths are NOT advanced. */
+int orc_decoder_step(const orc_decoder *d, size_t batch, float *const *self_k, float *const *self_v,
+                     const float *const *cross_k, const float *const *cross_v,
+                     const size_t *lengths, const size_t *memory_lengths,
+                     const float *const *inputs, float *const *outs);
+
+/* final-normed hidden [width] -> logits [heads_out*vocab] -> softmax per head. */
+void orc_output_head(const orc_weight *w_out, const float *bias, const float *hidden, size_t heads_out,
+                     size_t vocab, float *logits, float *probs, int act_variant);
+
+/* ---- encoder prefill (synthetic config: bidirectional, plain FFN, pre-LN, f16-rounded weights) ---- */
+typedef struct {
+    size_t layers, width, heads, head_width, ffn, vocab, max_positions;
+    const uint16_t *tok_table;   /* f16 bits [vocab,width] */
+    const uint16_t *pos_table;   /* f16 bits [max_positions,width] */
+    const uint16_t *qkv_w, *o_w, *up_w, *down_w;   /* f16 bits, per layer concatenated */
+    const float *norm1_g, *norm1_b, *norm2_g, *norm2_b;   /* [layers,width]; *_b may be NULL */
+    const float *norm_out_g, *norm_out_b;          /* [width] or NULL gain => no final norm */
+} orc_encoder;
+
+/* embed_out: f16 bits [T,width] of the gathered token rows (bit-exact artefact);
+ * out: f32 [T,width].  threads >= 1 splits GEMM rows over pthreads (results are thread-count independent). */
+int orc_encoder_prefill(const orc_encoder *e, const int32_t *ids, size_t T, uint16_t *embed_out,
+                        float *out, int threads);
+
+/* f32 row-major C[m,n] = A[m,k] * B[n,k]^T, k-contiguous dots (used by the encoder and tests). */
+void orc_gemm_nt(const float *a, const float *b, float *c, size_t m, size_t n, size_t k, int threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,429 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes bindings for the CPU oracle (liboracle.so) and, when built,
+the compiled reference (oracle/_ref/libmynah_ref*.so).
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this module.
+The shipped package never does.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+F32, INT8, INT4, F16 = 0, 1, 2, 3
+STRICT, STOCK = 0, 1
+
+_f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_i8p = np.ctypeslib.ndpointer(dtype=np.int8, flags="C_CONTIGUOUS")
+_u8p = np.ctypeslib.ndpointer(dtype=np.uint8, flags="C_CONTIGUOUS")
+_u16p = np.ctypeslib.ndpointer(dtype=np.uint16, flags="C_CONTIGUOUS")
+_i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+_sz = C.c_size_t
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def build_oracle():
+    subprocess.run(["make", "-C", HERE, "oracle"], check=True, stdout=subprocess.DEVNULL)
+
+
+def _load_oracle():
+    path = os.path.join(HERE, "liboracle.so")
+    if not os.path.exists(path):
+        build_oracle()
+    lib = C.CDLL(path)
+    lib.orc_quantize_weight_int8.argtypes = [_f32p, _sz, _sz, _i8p, _f32p, C.c_int]
+    lib.orc_quantize_weight_int8.restype = None
+    lib.orc_quantize_weight_int4.argtypes = [_f32p, _sz, _sz, _u8p, _f32p, C.c_int]
+    lib.orc_quantize_weight_int4.restype = C.c_int
+    lib.orc_f32_to_f16_array.argtypes = [_f32p, _u16p, _sz]
+    lib.orc_f32_to_f16_array.restype = None
+    lib.orc_f16_to_f32.argtypes = [C.c_uint16]
+    lib.orc_f16_to_f32.restype = C.c_float
+    lib.orc_quantize_act_int8.argtypes = [_i8p, _f32p, _sz, C.c_int]
+    lib.orc_quantize_act_int8.restype = C.c_float
+    lib.orc_matvec_q8.argtypes = [_f32p, C.c_void_p, _i8p, C.c_float, _i8p, _f32p, C.c_void_p, _sz, _sz]
+    lib.orc_matvec_q8.restype = None
+    lib.orc_matvec_q4.argtypes = [_f32p, C.c_void_p, _i8p, C.c_float, _u8p, _f32p, C.c_void_p, _sz, _sz]
+    lib.orc_matvec_q4.restype = None
+    lib.orc_matvec_f16.argtypes = [_f32p, _f32p, _u16p, C.c_void_p, _sz, _sz]
+    lib.orc_matvec_f16.restype = None
+    lib.orc_matvec_f32.argtypes = [_f32p, _f32p, _f32p, C.c_void_p, _sz, _sz]
+    lib.orc_matvec_f32.restype = None
+    lib.orc_layernorm.argtypes = [_f32p, _f32p, C.c_void_p, _f32p, _sz, _sz, C.c_float]
+    lib.orc_layernorm.restype = None
+    lib.orc_gelu_scalar.argtypes = [_f32p, _sz]
+    lib.orc_gelu_pade.argtypes = [_f32p, _sz]
+    lib.orc_softmax.argtypes = [_f32p, _f32p, _sz]
+    lib.orc_softmax.restype = C.c_int
+    lib.orc_softmax_row_inplace.argtypes = [_f32p, _sz]
+    lib.orc_softmax_masked.argtypes = [_f32p, _sz, _sz, _sz]
+    lib.orc_residual_add.argtypes = [_f32p, _f32p, _sz]
+    lib.orc_argmax_constrained.argtypes = [_f32p, _sz, _sz, _sz, C.c_int, C.POINTER(C.c_uint)]
+    lib.orc_argmax_constrained.restype = C.c_int
+    lib.orc_self_attention.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, _sz, _sz, C.c_float, _f32p, _f32p]
+    lib.orc_cross_attention.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, _sz, C.c_float, _f32p, _f32p]
+    lib.orc_decoder_step.restype = C.c_int
+    lib.orc_output_head.restype = None
+    lib.orc_encoder_prefill.restype = C.c_int
+    lib.orc_gemm_nt.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, C.c_int]
+    return lib
+
+
+lib = _load_oracle()
+
+
+class OrcWeight(C.Structure):
+    _fields_ = [("qtype", C.c_int), ("n", _sz), ("k", _sz), ("data", C.c_void_p), ("scales", C.c_void_p)]
+
+
+class OrcDecoder(C.Structure):
+    _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn", _sz),
+                ("cross_heads", _sz), ("cross_head_width", _sz), ("capacity", _sz),
+                ("qkv", C.POINTER(OrcWeight)), ("o_self", C.POINTER(OrcWeight)),
+                ("q_cross", C.POINTER(OrcWeight)), ("o_cross", C.POINTER(OrcWeight)),
+                ("ffn_up", C.POINTER(OrcWeight)), ("ffn_down", C.POINTER(OrcWeight)),
+                ("norm_self_g", C.c_void_p), ("norm_self_b", C.c_void_p),
+                ("norm_cross_g", C.c_void_p), ("norm_cross_b", C.c_void_p),
+                ("norm_ff_g", C.c_void_p), ("norm_ff_b", C.c_void_p),
+                ("norm_out_g", C.c_void_p), ("norm_out_b", C.c_void_p),
+                ("position", C.c_void_p), ("act_variant", C.c_int)]
+
+
+class OrcEncoder(C.Structure):
+    _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn", _sz),
+                ("vocab", _sz), ("max_positions", _sz),
+                ("tok_table", C.c_void_p), ("pos_table", C.c_void_p),
+                ("qkv_w", C.c_void_p), ("o_w", C.c_void_p), ("up_w", C.c_void_p), ("down_w", C.c_void_p),
+                ("norm1_g", C.c_void_p), ("norm1_b", C.c_void_p), ("norm2_g", C.c_void_p),
+                ("norm2_b", C.c_void_p), ("norm_out_g", C.c_void_p), ("norm_out_b", C.c_void_p)]
+
+
+# ----------------------------------------------------------------------------- numpy-level helpers
+def quantize_weight_int8(w, variant=STRICT):
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    n, k = w.shape
+    q = np.empty((n, k), np.int8)
+    s = np.empty(n, np.float32)
+    lib.orc_quantize_weight_int8(w, n, k, q, s, variant)
+    return q, s
+
+
+def quantize_weight_int4(w, variant=STRICT):
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    n, k = w.shape
+    q = np.empty((n, k // 2), np.uint8)
+    s = np.empty((n, k // 32), np.float32)
+    if lib.orc_quantize_weight_int4(w, n, k, q, s, variant) != 0:
+        raise ValueError("int4 needs k % 32 == 0")
+    return q, s
+
+
+def f32_to_f16_bits(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib.orc_f32_to_f16_array(x.reshape(-1), out.reshape(-1), x.size)
+    return out
+
+
+def quantize_act_int8(x, variant=STRICT):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    qx = np.empty(x.shape, np.int8)
+    sx = lib.orc_quantize_act_int8(qx, x, x.size, variant)
+    return qx, np.float32(sx)
+
+
+def matvec_q8(qx, sx, q, scales, bias=None):
+    n, k = q.shape
+    out = np.empty(n, np.float32)
+    acc = np.empty(n, np.int32)
+    lib.orc_matvec_q8(out, _ptr(acc), qx, float(sx), q, scales, _ptr(bias), n, k)
+    return out, acc
+
+
+def matvec_q4(qx, sx, q, scales, bias=None):
+    n, k2 = q.shape
+    k = k2 * 2
+    out = np.empty(n, np.float32)
+    acc = np.empty((n, k // 32), np.int32)
+    lib.orc_matvec_q4(out, _ptr(acc), qx, float(sx), q, np.ascontiguousarray(scales), _ptr(bias), n, k)
+    return out, acc
+
+
+def matvec_f16(x, wbits, bias=None):
+    n, k = wbits.shape
+    out = np.empty(n, np.float32)
+    lib.orc_matvec_f16(out, np.ascontiguousarray(x, np.float32), wbits, _ptr(bias), n, k)
+    return out
+
+
+def matvec_f32(x, w, bias=None):
+    n, k = w.shape
+    out = np.empty(n, np.float32)
+    lib.orc_matvec_f32(out, np.ascontiguousarray(x, np.float32), np.ascontiguousarray(w, np.float32), _ptr(bias), n, k)
+    return out
+
+
+def layernorm(x, gain, bias=None, eps=1e-5):
+    x = np.ascontiguousarray(x, np.float32)
+    x2 = x.reshape(-1, x.shape[-1])
+    out = np.empty_like(x2)
+    lib.orc_layernorm(x2, np.ascontiguousarray(gain, np.float32), _ptr(bias), out, x2.shape[0], x2.shape[1], eps)
+    return out.reshape(x.shape)
+
+
+def gelu_scalar(x):
+    y = np.array(x, dtype=np.float32, copy=True).reshape(-1)
+    lib.orc_gelu_scalar(y, y.size)
+    return y.reshape(np.shape(x))
+
+
+def gelu_pade(x):
+    y = np.array(x, dtype=np.float32, copy=True).reshape(-1)
+    lib.orc_gelu_pade(y, y.size)
+    return y.reshape(np.shape(x))
+
+
+def softmax(x):
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty_like(x)
+    rc = lib.orc_softmax(x, out, x.size)
+    return rc, out
+
+
+def softmax_row_inplace(x):
+    y = np.array(x, dtype=np.float32, copy=True)
+    lib.orc_softmax_row_inplace(y, y.size)
+    return y
+
+
+def softmax_masked(x, valid):
+    y = np.array(x, dtype=np.float32, copy=True)
+    lib.orc_softmax_masked(y, y.shape[0], y.shape[1], valid)
+    return y
+
+
+def argmax_constrained(logits, codebook_size, eos_id, allow_eos):
+    out = C.c_uint(0)
+    rc = lib.orc_argmax_constrained(np.ascontiguousarray(logits, np.float32), logits.size, codebook_size, eos_id,
+                                    int(allow_eos), C.byref(out))
+    return rc, out.value
+
+
+def self_attention(qkv, k_cache, v_cache, position, stride, valid, heads, hw, scale):
+    out = np.empty(heads * hw, np.float32)
+    scratch = np.empty(valid + 1, np.float32)
+    lib.orc_self_attention(qkv, k_cache, v_cache, position, stride, valid, heads, hw, scale, out, scratch)
+    return out
+
+
+def cross_attention(q, k_cache, v_cache, valid, stride, heads, hw, scale):
+    out = np.empty(heads * hw, np.float32)
+    scratch = np.empty(valid + 1, np.float32)
+    lib.orc_cross_attention(q, k_cache, v_cache, valid, stride, heads, hw, scale, out, scratch)
+    return out
+
+
+class PackedWeight:
+    """A weight matrix converted once on the host; keeps the numpy arrays alive for ctypes."""
+
+    def __init__(self, w, qtype, variant=STRICT):
+        w = np.ascontiguousarray(w, np.float32)
+        self.qtype, self.n, self.k = qtype, w.shape[0], w.shape[1]
+        self.scales = None
+        if qtype == F32:
+            self.data = w
+        elif qtype == F16:
+            self.data = f32_to_f16_bits(w)
+        elif qtype == INT8:
+            self.data, self.scales = quantize_weight_int8(w, variant)
+        elif qtype == INT4:
+            self.data, self.scales = quantize_weight_int4(w, variant)
+        else:
+            raise ValueError(qtype)
+
+    def struct(self):
+        return OrcWeight(self.qtype, self.n, self.k, _ptr(self.data), _ptr(self.scales))
+
+    def nbytes(self):
+        return self.data.nbytes + (0 if self.scales is None else self.scales.nbytes)
+
+
+def linear(pw, x, bias=None, act_variant=STRICT):
+    out = np.empty(pw.n, np.float32)
+    s = pw.struct()
+    lib.orc_linear(C.byref(s), _ptr(np.ascontiguousarray(x, np.float32)), _ptr(out), _ptr(bias), act_variant)
+    return out
+
+
+class Decoder:
+    """Synthetic decoder stack: holds packed weights and runs orc_decoder_step."""
+
+    def __init__(self, cfg, weights, qtype, variant=STRICT):
+        # weights: dict of per-layer f32 arrays (see tests/synth.py)
+        self.cfg = cfg
+        L = cfg["layers"]
+        self.packed = {name: [PackedWeight(weights[name][l], qtype, variant) for l in range(L)]
+                       for name in ("qkv", "o_self", "q_cross", "o_cross", "ffn_up", "ffn_down")}
+        self._arrays = {name: (OrcWeight * L)(*[p.struct() for p in self.packed[name]]) for name in self.packed}
+        self.norms = {k: (None if weights.get(k) is None else np.ascontiguousarray(weights[k], np.float32))
+                      for k in ("norm_self_g", "norm_self_b", "norm_cross_g", "norm_cross_b", "norm_ff_g",
+                                "norm_ff_b", "norm_out_g", "norm_out_b", "position")}
+        d = OrcDecoder()
+        d.layers, d.width, d.heads, d.head_width, d.ffn = L, cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
+        d.cross_heads, d.cross_head_width, d.capacity = cfg["cross_heads"], cfg["cross_head_width"], cfg["capacity"]
+        for name in self._arrays:
+            setattr(d, name, self._arrays[name])
+        for k, v in self.norms.items():
+            setattr(d, k, _ptr(v))
+        d.act_variant = variant
+        self.d = d
+
+    def step(self, self_k, self_v, cross_k, cross_v, lengths, memory_lengths, inputs):
+        B = len(inputs)
+        outs = [np.empty(self.cfg["width"], np.float32) for _ in range(B)]
+        pp = C.c_void_p * B
+        szs = _sz * B
+        rc = lib.orc_decoder_step(C.byref(self.d), _sz(B), pp(*[_ptr(a) for a in self_k]), pp(*[_ptr(a) for a in self_v]),
+                                  pp(*[_ptr(a) for a in cross_k]), pp(*[_ptr(a) for a in cross_v]),
+                                  szs(*lengths), szs(*memory_lengths), pp(*[_ptr(a) for a in inputs]),
+                                  pp(*[_ptr(a) for a in outs]))
+        if rc != 0:
+            raise RuntimeError("decoder cache capacity exceeded")
+        return outs
+
+
+def output_head(pw, hidden, heads_out, vocab, bias=None, act_variant=STRICT):
+    logits = np.empty(heads_out * vocab, np.float32)
+    probs = np.empty(heads_out * vocab, np.float32)
+    s = pw.struct()
+    lib.orc_output_head(C.byref(s), _ptr(bias), _ptr(np.ascontiguousarray(hidden, np.float32)), _sz(heads_out),
+                        _sz(vocab), _ptr(logits), _ptr(probs), C.c_int(act_variant))
+    return logits, probs
+
+
+def encoder_prefill(cfg, w, ids, threads=8):
+    """w: dict with f16-bit tables/weights (uint16) and f32 norms.  Returns (embed_bits, out)."""
+    e = OrcEncoder()
+    e.layers, e.width, e.heads, e.head_width, e.ffn = cfg["layers"], cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
+    e.vocab, e.max_positions = cfg["vocab"], cfg["max_positions"]
+    keep = []
+    for name in ("tok_table", "pos_table", "qkv_w", "o_w", "up_w", "down_w"):
+        a = np.ascontiguousarray(w[name], np.uint16)
+        keep.append(a)
+        setattr(e, name, _ptr(a))
+    for name in ("norm1_g", "norm1_b", "norm2_g", "norm2_b", "norm_out_g", "norm_out_b"):
+        a = None if w.get(name) is None else np.ascontiguousarray(w[name], np.float32)
+        keep.append(a)
+        setattr(e, name, _ptr(a))
+    ids = np.ascontiguousarray(ids, np.int32)
+    T = ids.size
+    embed = np.empty((T, cfg["width"]), np.uint16)
+    out = np.empty((T, cfg["width"]), np.float32)
+    rc = lib.orc_encoder_prefill(C.byref(e), _ptr(ids), _sz(T), _ptr(embed), _ptr(out), C.c_int(threads))
+    if rc != 0:
+        raise ValueError("invalid ids or length")
+    return embed, out
+
+
+# ----------------------------------------------------------------------------- compiled reference
+class RefDecoderDesc(C.Structure):
+    _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn", _sz), ("xw", _sz),
+                ("capacity", _sz),
+                ("norm_self", C.c_void_p), ("norm_xq", C.c_void_p), ("norm_ff", C.c_void_p),
+                ("qkv_w", C.c_void_p), ("o_w", C.c_void_p), ("qx_w", C.c_void_p), ("ox_w", C.c_void_p),
+                ("up_w", C.c_void_p), ("down_w", C.c_void_p), ("norm_out", C.c_void_p), ("position", C.c_void_p)]
+
+
+def ref_available(strict=False):
+    return os.path.exists(os.path.join(HERE, "_ref", "libmynah_ref_strict.so" if strict else "libmynah_ref.so"))
+
+
+_ref_cache = {}
+
+
+def load_ref(strict=False):
+    """The reference's own CPU code, compiled from the reference tree by oracle/Makefile `ref`."""
+    key = bool(strict)
+    if key in _ref_cache:
+        return _ref_cache[key]
+    path = os.path.join(HERE, "_ref", "libmynah_ref_strict.so" if strict else "libmynah_ref.so")
+    r = C.CDLL(path)
+    r.ref_quantize_weight_int8.argtypes = [_f32p, _sz, _sz, _i8p, _f32p]
+    r.ref_quantize_weight_int8.restype = None
+    r.ref_quantize_weight_int4.argtypes = [_f32p, _sz, _sz, _u8p, _f32p]
+    r.ref_quantize_weight_int4.restype = None
+    r.ref_quantize_act_int8.argtypes = [_i8p, _f32p, _sz]
+    r.ref_quantize_act_int8.restype = C.c_float
+    r.ref_matvec_q8.argtypes = [_f32p, _i8p, C.c_float, _i8p, _f32p, C.c_void_p, _sz, _sz]
+    r.ref_matvec_q8.restype = None
+    r.ref_matvec_q4.argtypes = [_f32p, _i8p, C.c_float, _u8p, _f32p, C.c_void_p, _sz, _sz]
+    r.ref_matvec_q4.restype = None
+    r.ref_matvec_rows_blocked.argtypes = [_f32p, _i8p, C.c_float, C.c_void_p, _f32p, C.c_void_p, _sz, _sz, C.c_int]
+    r.ref_matvec_q_rows.argtypes = [_f32p, _i8p, C.c_float, C.c_void_p, _f32p, C.c_void_p, _sz, _sz, C.c_int]
+    r.ref_num_threads.restype = C.c_int
+    r.mynah_qmat_self_test.argtypes = [C.c_char_p, _sz]
+    r.mynah_qmat_self_test.restype = C.c_int
+    r.mynah_kernels_self_test.argtypes = [C.c_char_p, _sz]
+    r.mynah_kernels_self_test.restype = C.c_int
+    r.mynah_layernorm_f32.argtypes = [_f32p, _f32p, C.c_void_p, _f32p, _sz, _sz, C.c_float]
+    r.mynah_layernorm_f32.restype = None
+    r.mynah_gelu_f32_scalar.argtypes = [_f32p, _sz]
+    r.mynah_gelu_f32.argtypes = [_f32p, _sz]
+    r.mynah_softmax_f32.argtypes = [_f32p, _f32p, _sz]
+    r.mynah_softmax_f32.restype = C.c_int
+    r.mynah_matvec_bias_f32.argtypes = [_f32p, _f32p, C.c_void_p, _f32p, _sz, _sz]
+    r.ref_softmax_row_inplace.argtypes = [_f32p, _sz]
+    r.ref_decoder_new.argtypes = [C.POINTER(RefDecoderDesc), C.c_int, _sz, _sz]
+    r.ref_decoder_new.restype = C.c_void_p
+    r.ref_decoder_free.argtypes = [C.c_void_p]
+    r.ref_decoder_step.restype = C.c_int
+    _ref_cache[key] = r
+    return r
+
+
+class RefDecoder:
+    """The reference's decoder_step_batch on synthetic weights (gain-only LayerNorm, one cross head)."""
+
+    def __init__(self, cfg, weights, qtype, batch, max_memory, strict=False):
+        assert cfg["cross_heads"] == 1, "the reference's decode step has a single cross-attention head"
+        self.r = load_ref(strict)
+        self.cfg, self.batch = cfg, batch
+        self.keep = {}
+        d = RefDecoderDesc()
+        d.layers, d.width, d.heads, d.head_width, d.ffn = cfg["layers"], cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
+        d.xw, d.capacity = cfg["cross_head_width"], cfg["capacity"]
+        names = {"norm_self": "norm_self_g", "norm_xq": "norm_cross_g", "norm_ff": "norm_ff_g", "qkv_w": "qkv",
+                 "o_w": "o_self", "qx_w": "q_cross", "ox_w": "o_cross", "up_w": "ffn_up", "down_w": "ffn_down",
+                 "norm_out": "norm_out_g", "position": "position"}
+        for field, key in names.items():
+            a = np.ascontiguousarray(weights[key], np.float32)
+            self.keep[field] = a
+            setattr(d, field, _ptr(a))
+        self.desc = d
+        self.h = self.r.ref_decoder_new(C.byref(d), qtype, batch, max_memory)
+        if not self.h:
+            raise RuntimeError("ref_decoder_new failed")
+
+    def step(self, self_k, self_v, cross_k, cross_v, lengths, memory_lengths, inputs):
+        B = self.batch
+        outs = [np.empty(self.cfg["width"], np.float32) for _ in range(B)]
+        pp = C.c_void_p * B
+        szs = _sz * B
+        lens = szs(*lengths)
+        err = C.create_string_buffer(256)
+        rc = self.r.ref_decoder_step(C.c_void_p(self.h), pp(*[_ptr(a) for a in self_k]), pp(*[_ptr(a) for a in self_v]),
+                                     pp(*[_ptr(a) for a in cross_k]), pp(*[_ptr(a) for a in cross_v]), lens,
+                                     szs(*memory_lengths), pp(*[_ptr(a) for a in inputs]),
+                                     pp(*[_ptr(a) for a in outs]), err, _sz(256))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        return outs, list(lens)
+
+    def close(self):
+        if self.h:
+            self.r.ref_decoder_free(C.c_void_p(self.h))
+            self.h = None

@@ -1,0 +1,157 @@
+/* TEST INFRASTRUCTURE ONLY -- never linked into, loaded by, or timed as the product.
+ *
+ * Drives the reference's own batched decode step on synthetic weights, without a
+ * model pack.  The reference engine source is NOT copied: the include below
+ * resolves through -I<reference>/src (oracle/Makefile) and the object lives only
+ * in oracle/_ref/.
+ *
+ * Reference functions reached through this shim (file:line in the reference tree):
+ *   decoder_step_batch        src/graph.c:3127-3284  (B slots, weight-stationary projections)
+ *   layer_norm                src/graph.c:147-150    (gain only, eps 1e-5)
+ *   softmax_row_inplace       src/graph.c:245-257
+ *   batch_scratch_init        src/graph.c:121-144
+ *   mynah_backend_open(CPU)   src/backend.c:367-475
+ *   mynah_qmat_cache_new      src/qmat.c:567-591
+ *
+ * The shim fills a decoder_cache (src/graph.c:2813-2861) per slot by hand:
+ * only plain-pointer fields are touched by decoder_step_batch.
+ */
+#include "graph.c"
+
+typedef struct {
+    size_t layers, width, heads, head_width, ffn, xw, capacity;
+    /* per-layer tensors, concatenated over layers */
+    const float *norm_self;   /* [layers, width] */
+    const float *norm_xq;     /* [layers, width] */
+    const float *norm_ff;     /* [layers, width] */
+    const float *qkv_w;       /* [layers, 3*width, width] */
+    const float *o_w;         /* [layers, width, width] */
+    const float *qx_w;        /* [layers, xw, width] */
+    const float *ox_w;        /* [layers, width, xw] */
+    const float *up_w;        /* [layers, ffn, width] */
+    const float *down_w;      /* [layers, width, ffn] */
+    const float *norm_out;    /* [width] */
+    const float *position;    /* [capacity, width] */
+} ref_decoder_desc;
+
+typedef struct {
+    mynah_tts_model model;
+    ref_decoder_desc desc;
+    decoder_layer_resolved *resolved;
+    decoder_cache caches[MYNAH_MAX_BATCH];
+    batch_scratch scratch;
+    size_t batch;
+} ref_decoder;
+
+void ref_decoder_free(ref_decoder *d) {
+    if (d == NULL) return;
+    for (size_t b = 0; b < MYNAH_MAX_BATCH; ++b) {
+        decoder_cache *c = &d->caches[b];
+        free(c->scratch_x); free(c->scratch_nrm); free(c->scratch_qkv); free(c->scratch_attn);
+        free(c->scratch_proj); free(c->scratch_q_x); free(c->scratch_xctx);
+        free(c->scratch_hidden); free(c->scratch_scores);
+    }
+    batch_scratch_free(&d->scratch);
+    free(d->resolved);
+    if (d->model.qcache != NULL) mynah_qmat_cache_free(d->model.qcache);
+    if (d->model.backend != NULL) mynah_backend_close(d->model.backend);
+    free(d);
+}
+
+/* qtype: 0 f32, 1 int8, 2 int4 (the reference's QMAT_* values, src/qmat.c:36). */
+ref_decoder *ref_decoder_new(const ref_decoder_desc *desc, int qtype, size_t batch,
+                             size_t max_memory_length) {
+    if (batch == 0 || batch > MYNAH_MAX_BATCH) return NULL;
+    ref_decoder *d = (ref_decoder *)calloc(1, sizeof(*d));
+    if (d == NULL) return NULL;
+    char error[256];
+    d->desc = *desc;
+    d->batch = batch;
+    if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &d->model.backend, error, sizeof error) != 0) goto fail;
+    d->model.qcache = mynah_qmat_cache_new(qtype);
+    if (d->model.qcache == NULL) goto fail;
+    d->resolved = (decoder_layer_resolved *)calloc(desc->layers, sizeof(*d->resolved));
+    if (d->resolved == NULL) goto fail;
+    const size_t w = desc->width, f = desc->ffn, xw = desc->xw;
+    for (size_t l = 0; l < desc->layers; ++l) {
+        decoder_layer_resolved *r = &d->resolved[l];
+        r->norm_self = desc->norm_self + l * w;
+        r->norm_xattn_query = desc->norm_xq + l * w;
+        r->norm_pos_ff = desc->norm_ff + l * w;
+        r->qkv_w = desc->qkv_w + l * 3u * w * w;
+        r->o_self_w = desc->o_w + l * w * w;
+        r->q_cross_w = desc->qx_w + l * xw * w;
+        r->o_cross_w = desc->ox_w + l * w * xw;
+        r->ffn_up_w = desc->up_w + l * f * w;
+        r->ffn_down_w = desc->down_w + l * w * f;
+        snprintf(r->qkv, sizeof r->qkv, "synthetic.layer%zu.qkv", l);
+        snprintf(r->o_self, sizeof r->o_self, "synthetic.layer%zu.o_self", l);
+        snprintf(r->q_cross, sizeof r->q_cross, "synthetic.layer%zu.q_cross", l);
+        snprintf(r->o_cross, sizeof r->o_cross, "synthetic.layer%zu.o_cross", l);
+        snprintf(r->ffn_up, sizeof r->ffn_up, "synthetic.layer%zu.ffn_up", l);
+        snprintf(r->ffn_down, sizeof r->ffn_down, "synthetic.layer%zu.ffn_down", l);
+    }
+    size_t score_len = desc->capacity > max_memory_length ? desc->capacity : max_memory_length;
+    for (size_t b = 0; b < batch; ++b) {
+        decoder_cache *c = &d->caches[b];
+        c->layers = desc->layers; c->width = w; c->heads = desc->heads;
+        c->head_width = desc->head_width; c->ffn_width = f; c->xattn_width = xw;
+        c->capacity = desc->capacity;
+        c->position = desc->position;
+        c->resolved = d->resolved;
+        c->norm_out = desc->norm_out;
+        c->scratch_rows = 1;
+        c->scratch_x = (float *)calloc(w, sizeof(float));
+        c->scratch_nrm = (float *)calloc(w, sizeof(float));
+        c->scratch_qkv = (float *)calloc(3u * w, sizeof(float));
+        c->scratch_attn = (float *)calloc(w, sizeof(float));
+        c->scratch_proj = (float *)calloc(w, sizeof(float));
+        c->scratch_q_x = (float *)calloc(xw, sizeof(float));
+        c->scratch_xctx = (float *)calloc(xw, sizeof(float));
+        c->scratch_hidden = (float *)calloc(f, sizeof(float));
+        c->scratch_scores = (float *)calloc(score_len + 1u, sizeof(float));
+        if (!c->scratch_x || !c->scratch_nrm || !c->scratch_qkv || !c->scratch_attn || !c->scratch_proj ||
+            !c->scratch_q_x || !c->scratch_xctx || !c->scratch_hidden || !c->scratch_scores) goto fail;
+    }
+    const size_t k_max = f > w ? f : w;
+    if (batch_scratch_init(&d->scratch, batch, k_max > xw ? k_max : xw, error, sizeof error) != 0) goto fail;
+    return d;
+fail:
+    ref_decoder_free(d);
+    return NULL;
+}
+
+/* One batched step.  self_k/self_v[b]: [layers, capacity, width] (caller-owned, appended in
+ * place at row lengths[b]); cross_k/cross_v[b]: [layers, memory_lengths[b], xw].
+ * lengths[b] is advanced by one on success, exactly as the reference does (src/graph.c:3281). */
+int ref_decoder_step(ref_decoder *d, float *const *self_k, float *const *self_v,
+                     float *const *cross_k, float *const *cross_v,
+                     size_t *lengths, const size_t *memory_lengths,
+                     const float *const *inputs, float *const *outs,
+                     char *error, size_t error_capacity) {
+    decoder_cache *ptrs[MYNAH_MAX_BATCH];
+    for (size_t b = 0; b < d->batch; ++b) {
+        decoder_cache *c = &d->caches[b];
+        c->self_k = self_k[b]; c->self_v = self_v[b];
+        c->cross_k = cross_k[b]; c->cross_v = cross_v[b];
+        c->length = lengths[b];
+        c->memory_length = memory_lengths[b];
+        ptrs[b] = c;
+    }
+    const int rc = decoder_step_batch(&d->model, ptrs, inputs, outs, d->batch,
+                                      d->batch > 1u ? &d->scratch : NULL, error, error_capacity);
+    for (size_t b = 0; b < d->batch; ++b) {
+        decoder_cache *c = &d->caches[b];
+        lengths[b] = c->length;
+        c->self_k = c->self_v = c->cross_k = c->cross_v = NULL;
+    }
+    return rc;
+}
+
+void ref_layer_norm_gain(const float *input, float *output, size_t rows, size_t width, const float *gain) {
+    layer_norm(input, output, rows, width, gain);
+}
+
+void ref_softmax_row_inplace(float *values, size_t length) { softmax_row_inplace(values, length); }
+
+float ref_gelu_tanh(float x) { return gelu_tanh(x); }
