@@ -266,7 +266,9 @@ class Decoder:
         # weights: dict of per-layer f32 arrays (see tests/synth.py)
         self.cfg = cfg
         L = cfg["layers"]
-        self.packed = {name: [PackedWeight(weights[name][l], qtype, variant) for l in range(L)]
+        has_cross = cfg["cross_heads"] * cfg["cross_head_width"] != 0
+        self.packed = {name: [PackedWeight(weights[name][l], qtype if (has_cross or "cross" not in name) else F32, variant)
+                              for l in range(L)]
                        for name in ("qkv", "o_self", "q_cross", "o_cross", "ffn_up", "ffn_down")}
         self._arrays = {name: (OrcWeight * L)(*[p.struct() for p in self.packed[name]]) for name in self.packed}
         self.norms = {k: (None if weights.get(k) is None else np.ascontiguousarray(weights[k], np.float32))

@@ -1,0 +1,345 @@
+"""GPU parity of the seam's resident ops against the oracle, through the C ABI."""
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(2304, 768), (768, 768), (3072, 768), (768, 3072)]   # the benchmark's int8 matvec sweep
+
+
+def _announce(msg):
+    print("[gpu-case] " + msg, flush=True)
+
+
+def test_backend_self_test(backend):
+    """matmul / sgemm KATs (gpu/cuda/backend_cuda.cu:514-529) and resident-op KATs
+    (gpu/metal/backend_metal_ops.m:1038-1107) inside the library."""
+    _announce("self_test")
+    rc, msg = backend.self_test()
+    assert rc == 0, msg
+
+
+def test_matmul_kat_through_function_pointer(backend):
+    _announce("matmul KAT")
+    x = np.array([[1.0, 2.0, 3.0], [-1.0, 0.5, 2.0]], np.float32)
+    w = backend.keep(np.array([[1, 0, 0], [0, 1, 0], [0, 0, 1], [1, 1, 1]], np.float32))
+    b = backend.keep(np.array([0.5, -0.5, 1.0, 2.0], np.float32))
+    out = backend.matmul(x, w, b)
+    assert np.allclose(out, [[1.5, 1.5, 4.0, 8.0], [-0.5, 0.0, 3.0, 3.5]], atol=1e-5)
+    c = np.zeros((2, 4), np.float32)
+    backend.sgemm(0, 1, 2, 4, 3, 1.0, x, 3, w, 3, 0.0, c, 4)
+    assert np.allclose(c, [[1, 2, 3, 6], [-1, 0.5, 2, 1.5]], atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("arith", [0, 1])
+def test_int8_matvec_bit_exact_integers(backend, pkg, orc, nerr, shape, arith):
+    """Packed weights, int8 activations, activation scale and int32 accumulators bit-exact; f32 output 1e-5."""
+    n, k = shape
+    _announce("int8 matvec %dx%d arith=%d" % (n, k, arith))
+    rng = np.random.default_rng(100 + n + k)
+    w = backend.keep((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    x = rng.standard_normal(k).astype(np.float32)
+    bias = backend.keep((rng.standard_normal(n) * 0.1).astype(np.float32))
+    # the library's own load-time quantiser == the oracle's == (tested on the CPU) the compiled reference's
+    q, s = pkg.quantize_weight_int8(backend.lib, w, arith)
+    oq, os_ = orc.quantize_weight_int8(w, arith)
+    assert np.array_equal(q, oq) and np.array_equal(s.view(np.uint32), os_.view(np.uint32))
+    backend.set_quant(pkg.INT8, arith)
+    din, dout = backend.alloc(k).write(x), backend.alloc(n)
+    dqx, dsx, dacc = backend.alloc(k // 4), backend.alloc(1), backend.alloc(n)
+    backend.matmul_probe(din.ptr, dout.ptr, k, n, w, bias, dqx.ptr, dsx.ptr, dacc.ptr)
+    got = dout.read()
+    qx = dqx.read(dtype=np.int8)
+    sx = dsx.read()[0]
+    acc = dacc.read(dtype=np.int32)
+    oqx, osx = orc.quantize_act_int8(x, arith)
+    want, oacc = orc.matvec_q8(oqx, osx, oq, os_, bias)
+    assert np.array_equal(qx, oqx), "int8 activations differ"
+    assert np.float32(sx).view(np.uint32) == np.float32(osx).view(np.uint32), "activation scale differs"
+    assert np.array_equal(acc, oacc), "int32 accumulators differ"
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "f32 epilogue differs bitwise"
+    assert nerr(got, want) < 1e-5
+    for b in (din, dout, dqx, dsx, dacc):
+        b.free()
+    backend.set_quant(pkg.F32)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_int4_matvec_group_accumulators(backend, pkg, orc, nerr, shape):
+    n, k = shape
+    _announce("int4 matvec %dx%d" % (n, k))
+    rng = np.random.default_rng(200 + n + k)
+    w = backend.keep((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    x = rng.standard_normal(k).astype(np.float32)
+    rc, q, s = pkg.quantize_weight_int4(backend.lib, w, 0)
+    oq, os_ = orc.quantize_weight_int4(w, 0)
+    assert rc == 0 and np.array_equal(q, oq) and np.array_equal(s.view(np.uint32), os_.view(np.uint32))
+    backend.set_quant(pkg.INT4)
+    din, dout = backend.alloc(k).write(x), backend.alloc(n)
+    dqx, dsx, dacc = backend.alloc(k // 4), backend.alloc(1), backend.alloc(n * (k // 32))
+    backend.matmul_probe(din.ptr, dout.ptr, k, n, w, None, dqx.ptr, dsx.ptr, dacc.ptr)
+    got = dout.read()
+    acc = dacc.read(dtype=np.int32).reshape(n, k // 32)
+    oqx, osx = orc.quantize_act_int8(x)
+    want, oacc = orc.matvec_q4(oqx, osx, oq, os_)
+    assert np.array_equal(dqx.read(dtype=np.int8), oqx)
+    assert np.array_equal(acc, oacc), "per-group int32 accumulators differ"
+    # the group sum is a lane-local sequence followed by a butterfly, not the reference's single sequence
+    assert nerr(got, want) < 1e-5
+    for b in (din, dout, dqx, dsx, dacc):
+        b.free()
+    backend.set_quant(pkg.F32)
+
+
+@pytest.mark.parametrize("qtype_name,tol", [("f32", 1e-5), ("f16", 1e-5)])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_float_matvec(backend, pkg, orc, nerr, shape, qtype_name, tol):
+    """f32 weights within 1e-5; f16 weights (exact widening, f32 FMA, f32 activations) within 1e-5 of the
+    oracle's matvec_f16 and within 2e-3 of the f32-weight result."""
+    n, k = shape
+    _announce("%s matvec %dx%d" % (qtype_name, n, k))
+    rng = np.random.default_rng(300 + n + k)
+    w = backend.keep((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    x = rng.standard_normal(k).astype(np.float32)
+    bias = backend.keep((rng.standard_normal(n) * 0.1).astype(np.float32))
+    qtype = pkg.F32 if qtype_name == "f32" else pkg.F16
+    backend.set_quant(qtype)
+    din, dout = backend.alloc(k).write(x), backend.alloc(n)
+    backend.matmul_d2d(din.ptr, dout.ptr, 1, k, n, w, bias)
+    got = dout.read()
+    if qtype == pkg.F32:
+        want = orc.matvec_f32(x, w, bias)
+    else:
+        bits = pkg.convert_weight_f16(backend.lib, w)
+        assert np.array_equal(bits, orc.f32_to_f16_bits(w)), "f16 weight bits differ"
+        want = orc.matvec_f16(x, bits, bias)
+        assert nerr(got, orc.matvec_f32(x, w, bias)) < 2e-3
+    assert nerr(got, want) < tol
+    din.free()
+    dout.free()
+    backend.set_quant(pkg.F32)
+
+
+@pytest.mark.parametrize("qtype_name", ["int8", "int4", "f16", "f32"])
+def test_batched_matvec_bit_identical_to_solo(backend, pkg, qtype_name):
+    """self_test_batched (src/qmat.c:1107-1179) on the GPU: B=5 scattered rows, memcmp against one-at-a-time;
+    then B = 8 and B = 13 (two weight passes)."""
+    qtype = {"int8": pkg.INT8, "int4": pkg.INT4, "f16": pkg.F16, "f32": pkg.F32}[qtype_name]
+    n, k = 768, 768
+    _announce("batched matvec %s" % qtype_name)
+    rng = np.random.default_rng(400)
+    w = backend.keep((rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+    bias = backend.keep((rng.standard_normal(n) * 0.1).astype(np.float32))
+    backend.set_quant(qtype)
+    for B in (5, 8, 13):
+        xs = rng.standard_normal((B, k)).astype(np.float32)
+        xs[B // 2] = 0.0                                   # an all-zero activation row (sx == 0)
+        dins = [backend.alloc(k).write(xs[b]) for b in range(B)]
+        douts = [backend.alloc(n) for _ in range(B)]
+        solo = []
+        for b in range(B):
+            backend.matmul_d2d(dins[b].ptr, douts[b].ptr, 1, k, n, w, bias)
+            solo.append(douts[b].read())
+        backend.matmul_d2d_batched([d.ptr for d in dins], [d.ptr for d in douts], k, n, w, bias)
+        for b in range(B):
+            got = douts[b].read()
+            assert np.array_equal(got.view(np.uint32), solo[b].view(np.uint32)), "B=%d stream %d" % (B, b)
+        assert np.array_equal(solo[B // 2], bias)          # zero activation -> exactly the bias
+        for d in dins + douts:
+            d.free()
+    backend.set_quant(pkg.F32)
+
+
+def test_matmul_rows_and_generic_shapes(backend, pkg, orc, nerr):
+    """rows > 1 through matmul_d2d (prefill-like), shapes the fused matvec does not take, host-pointer matmul."""
+    _announce("generic matmul shapes")
+    rng = np.random.default_rng(500)
+    for rows, k, n in ((1, 100, 37), (3, 48, 50), (40, 768, 96), (16, 768, 768), (17, 256, 64)):
+        w = backend.keep((rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+        bias = backend.keep(rng.standard_normal(n).astype(np.float32))
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        want = np.stack([orc.matvec_f32(r, w, bias) for r in x])
+        din, dout = backend.alloc(rows * k).write(x), backend.alloc(rows * n)
+        backend.matmul_d2d(din.ptr, dout.ptr, rows, k, n, w, bias)
+        assert nerr(dout.read().reshape(rows, n), want) < 1e-5, (rows, k, n)
+        assert nerr(backend.matmul(x, w, bias), want) < 1e-5
+        din.free()
+        dout.free()
+    # int4 request on a width that is not a multiple of 32 silently stays f32 (src/qmat.c:630)
+    backend.set_quant(pkg.INT4)
+    w = backend.keep((rng.standard_normal((64, 48)) * 0.05).astype(np.float32))
+    x = rng.standard_normal((1, 48)).astype(np.float32)
+    assert nerr(backend.matmul(x, w), orc.matvec_f32(x[0], w)[None]) < 1e-5
+    backend.set_quant(pkg.F32)
+
+
+def test_layernorm_gelu_residual_softmax(backend, orc, nerr):
+    _announce("layernorm/gelu/residual/softmax")
+    rng = np.random.default_rng(600)
+    x = (rng.standard_normal((5, 768)) * 3 + 0.5).astype(np.float32)
+    gain = backend.keep((1 + 0.1 * rng.standard_normal(768)).astype(np.float32))
+    beta = backend.keep((0.02 * rng.standard_normal(768)).astype(np.float32))
+    din, dout = backend.alloc(x.size).write(x), backend.alloc(x.size)
+    backend.layer_norm_inplace(din.ptr, dout.ptr, gain, 5, 768)
+    assert nerr(dout.read().reshape(5, 768), orc.layernorm(x, gain)) < 1e-5
+    backend.layer_norm_dev(din.ptr, dout.ptr, gain, beta, 5, 768)
+    assert nerr(dout.read().reshape(5, 768), orc.layernorm(x, gain, beta)) < 1e-5
+    # KAT: layernorm(1..4) = -+1.34164 (src/kernels.c:473-482; eps 1e-5 here)
+    g4 = backend.keep(np.ones(4, np.float32))
+    d4 = backend.alloc(4).write(np.array([1, 2, 3, 4], np.float32))
+    backend.layer_norm_inplace(d4.ptr, d4.ptr, g4, 1, 4)
+    r = d4.read()
+    assert abs(r[0] + 1.34164) < 1e-4 and abs(r[3] - 1.34164) < 1e-4
+    # GELU: gelu(0) = 0, gelu(1) = 0.8411920 (src/kernels.c:493-499) and 3072 values vs the scalar libm form
+    v = np.concatenate([np.array([-1.0, 0.0, 1.0]), np.linspace(-9, 9, 3069)]).astype(np.float32)
+    dv = backend.alloc(v.size).write(v)
+    backend.gelu_inplace(dv.ptr, v.size)
+    gv = dv.read()
+    assert abs(gv[1]) < 1e-6 and abs(gv[2] - 0.8411920) < 1e-5
+    assert np.max(np.abs(gv - orc.gelu_scalar(v))) < 1e-5 * np.max(np.abs(v))
+    # residual
+    a = rng.standard_normal(768).astype(np.float32)
+    b = rng.standard_normal(768).astype(np.float32)
+    da, db = backend.alloc(768).write(a), backend.alloc(768).write(b)
+    backend.residual_inplace(da.ptr, db.ptr, 768)
+    assert np.array_equal(da.read(), a + b)
+    # a HOST row in the device slot (src/graph.c:1118-1120) resolves through the weight cache
+    hostrow = backend.keep(rng.standard_normal(768).astype(np.float32))
+    backend.residual_inplace(da.ptr, hostrow.ctypes.data, 768)
+    assert np.array_equal(da.read(), (a + b) + hostrow)
+    # masked softmax (src/backend.c:602-619) on 8 x 1024
+    logits = (rng.standard_normal((8, 1024)) * 4).astype(np.float32)
+    dl = backend.alloc(logits.size).write(logits)
+    backend.softmax_dev(dl.ptr, 8, 1024, 700)
+    got = dl.read().reshape(8, 1024)
+    assert nerr(got, orc.softmax_masked(logits, 700)) < 1e-5 and not got[:, 700:].any()
+    # copy / scale / clip
+    dc = backend.alloc(768)
+    backend.copy_dev(dc.ptr, da.ptr, 768)
+    assert np.array_equal(dc.read(), da.read())
+    backend.scale_dev(dc.ptr, 768, 0.25)
+    assert np.array_equal(dc.read(), da.read() * np.float32(0.25))
+    dclip = backend.alloc(4).write(np.array([-2.0, np.nan, 0.5, 7.0], np.float32))
+    backend.clip_dev(dclip.ptr, 4)
+    assert dclip.read().tolist() == [-1.0, 0.0, 0.5, 1.0]
+    for d in (din, dout, d4, dv, da, db, dl, dc, dclip):
+        d.free()
+
+
+def test_argmax(backend, orc):
+    _announce("argmax")
+    rng = np.random.default_rng(700)
+    logits = rng.standard_normal(2048).astype(np.float32)
+    logits[100] = logits[900] = 9.0        # tie: the first index wins
+    logits[2030] = 11.0                    # above codebook: only counts when it is the eos id
+    d = backend.alloc(2048).write(logits)
+    for codebook, eos, allow in ((2016, 2030, False), (2016, 2030, True), (2016, 2040, True), (50, 2030, False), (2048, 0, False)):
+        assert backend.argmax_dev(d.ptr, 2048, codebook, eos, allow) == orc.argmax_constrained(logits, codebook, eos, allow)[1]
+    dinf = backend.alloc(8).write(np.full(8, -np.inf, np.float32))
+    assert backend.argmax_dev(dinf.ptr, 8, 8, 0, False) == 0
+    dnan = backend.alloc(2).write(np.array([np.nan, 1.0], np.float32))
+    assert backend.argmax_dev(dnan.ptr, 2, 2, 0, False) == 1
+    with pytest.raises(Exception):
+        backend.argmax_dev(d.ptr, 2048, 4096, 0, False)     # codebook > vocab (src/backend.c:829-830)
+    for x in (d, dinf, dnan):
+        x.free()
+
+
+@pytest.mark.parametrize("heads,hw,L", [(12, 64, 1), (12, 64, 63), (12, 64, 64), (12, 64, 65), (12, 64, 300),
+                                        (12, 64, 1024), (1, 768, 200), (3, 20, 70), (1, 2, 5)])
+def test_self_and_cross_attention(backend, orc, nerr, heads, hw, L):
+    """Split-L attention against the reference's two-pass order, incl. chunk edges (63/64/65), one wide head
+    (what the engine passes for cross attention) and head widths that are not multiples of 4."""
+    _announce("attention heads=%d hw=%d L=%d" % (heads, hw, L))
+    rng = np.random.default_rng(800 + heads + hw + L)
+    width = heads * hw
+    scale = 1.0 / math.sqrt(hw)
+    qkv = rng.standard_normal(3 * width).astype(np.float32)
+    kc = np.zeros((L + 2, width), np.float32)
+    vc = np.zeros((L + 2, width), np.float32)
+    kc[:L - 1] = rng.standard_normal((L - 1, width))
+    vc[:L - 1] = rng.standard_normal((L - 1, width))
+    kc[L:] = 77.0     # rows beyond `valid` must be ignored and left alone
+    vc[L:] = -77.0
+    ok, ov = kc.copy(), vc.copy()
+    want = orc.self_attention(qkv, ok, ov, L - 1, width, L, heads, hw, scale)
+    dq, dk, dv, do = backend.alloc(qkv.size).write(qkv), backend.alloc(kc.size).write(kc), backend.alloc(vc.size).write(vc), backend.alloc(width)
+    backend.self_attention_dev(dq.ptr, dk.ptr, dv.ptr, L - 1, width, L, heads, hw, scale, do.ptr)
+    assert nerr(do.read(), want) < 1e-5
+    assert np.array_equal(dk.read().reshape(kc.shape), ok), "KV append must write exactly row `position` of K"
+    assert np.array_equal(dv.read().reshape(vc.shape), ov), "KV append must write exactly row `position` of V"
+    # cross: read-only over the same caches
+    wantx = orc.cross_attention(qkv[:width], ok, ov, L, width, heads, hw, scale)
+    backend.cross_attention_dev(dq.ptr, dk.ptr, dv.ptr, L, width, heads, hw, scale, do.ptr)
+    assert nerr(do.read(), wantx) < 1e-5
+    assert np.array_equal(dk.read().reshape(kc.shape), ok)
+    for d in (dq, dk, dv, do):
+        d.free()
+
+
+def test_batched_attention_bit_identical_to_solo(backend, orc, nerr):
+    _announce("batched attention")
+    rng = np.random.default_rng(900)
+    heads, hw = 12, 64
+    width = heads * hw
+    scale = 0.125
+    lengths = [64, 2048, 777, 65, 1, 300, 1999, 128]
+    B = len(lengths)
+    bufs = []
+    for L in lengths:
+        qkv = rng.standard_normal(3 * width).astype(np.float32)
+        kc = rng.standard_normal((L, width)).astype(np.float32)
+        vc = rng.standard_normal((L, width)).astype(np.float32)
+        bufs.append((qkv, kc, vc, backend.alloc(qkv.size).write(qkv), backend.alloc(kc.size).write(kc),
+                     backend.alloc(vc.size).write(vc), backend.alloc(width)))
+    solo = []
+    for (qkv, kc, vc, dq, dk, dv, do), L in zip(bufs, lengths):
+        backend.self_attention_dev(dq.ptr, dk.ptr, dv.ptr, L - 1, width, L, heads, hw, scale, do.ptr)
+        solo.append(do.read())
+        ok, ov = kc.copy(), vc.copy()
+        assert nerr(solo[-1], orc.self_attention(qkv, ok, ov, L - 1, width, L, heads, hw, scale)) < 1e-5
+    backend.self_attention_dev_batched([b[3].ptr for b in bufs], [b[4].ptr for b in bufs], [b[5].ptr for b in bufs],
+                                       [L - 1 for L in lengths], width, lengths, heads, hw, scale, [b[6].ptr for b in bufs])
+    for b, buf in enumerate(bufs):
+        assert np.array_equal(buf[6].read().view(np.uint32), solo[b].view(np.uint32)), "self stream %d" % b
+    solo = []
+    for (qkv, kc, vc, dq, dk, dv, do), L in zip(bufs, lengths):
+        backend.cross_attention_dev(dq.ptr, dk.ptr, dv.ptr, L, width, heads, hw, scale, do.ptr)
+        solo.append(do.read())
+    backend.cross_attention_dev_batched([b[3].ptr for b in bufs], [b[4].ptr for b in bufs], [b[5].ptr for b in bufs],
+                                        lengths, width, heads, hw, scale, [b[6].ptr for b in bufs])
+    for b, buf in enumerate(bufs):
+        assert np.array_equal(buf[6].read().view(np.uint32), solo[b].view(np.uint32)), "cross stream %d" % b
+    for buf in bufs:
+        for d in buf[3:]:
+            d.free()
+
+
+def test_embedding_gather_bit_exact(backend):
+    """Text rows are a memcpy (src/graph.c:729-737); the audio frame is a sum of table rows / count (:764-804)."""
+    _announce("gather")
+    rng = np.random.default_rng(1000)
+    table = backend.keep((rng.standard_normal((4096, 768)) * 0.02).astype(np.float32))
+    pos = backend.keep((rng.standard_normal((512, 768)) * 0.02).astype(np.float32))
+    ids = rng.integers(0, 4096, 256).astype(np.int32)
+    dout = backend.alloc(256 * 768)
+    backend.embed_gather([table], ids, 768, 1.0, None, 0, dout.ptr)
+    assert np.array_equal(dout.read().reshape(256, 768).view(np.uint32), table[ids].view(np.uint32))
+    backend.embed_gather([table], ids, 768, 1.0, pos, 3, dout.ptr)
+    assert np.array_equal(dout.read().reshape(256, 768), table[ids] + pos[3:259])
+    tables = [backend.keep((rng.standard_normal((2024, 768)) * 0.02).astype(np.float32)) for _ in range(16)]
+    fid = rng.integers(0, 2024, (2, 16)).astype(np.int32)
+    backend.embed_gather(tables, fid, 768, 1.0 / 16.0, None, 0, dout.ptr)
+    want = np.zeros((2, 768), np.float32)
+    for t in range(2):
+        acc = tables[0][fid[t, 0]].copy()
+        for j in range(1, 16):
+            acc = acc + tables[j][fid[t, j]]
+        want[t] = acc * np.float32(1.0 / 16.0)
+    assert np.array_equal(dout.read(2 * 768).reshape(2, 768), want)
+    with pytest.raises(Exception):
+        backend.embed_gather([table], np.array([4096], np.int32), 768, 1.0, None, 0, dout.ptr)   # out of vocabulary
+    dout.free()

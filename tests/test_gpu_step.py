@@ -1,0 +1,196 @@
+"""GPU parity of the resident batched decode step against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _announce(msg):
+    print("[gpu-case] " + msg, flush=True)
+
+
+class Harness:
+    """Uploads a set of synthetic streams and runs mynah_hip_decoder_step on them."""
+
+    def __init__(self, pkg, backend, cfg, weights, streams):
+        self.backend, self.cfg, self.streams = backend, cfg, streams
+        self.dec = pkg.Decoder(backend, cfg, weights)
+        self.bufs = []
+        for s in streams:
+            b = {n: backend.alloc(max(s[n].size, 4)).write(s[n]) if s[n].size else backend.alloc(4) for n in ("k", "v", "ck", "cv", "x")}
+            b["out"] = backend.alloc(cfg["width"])
+            self.bufs.append(b)
+
+    def slots(self, which=None):
+        which = range(len(self.streams)) if which is None else which
+        return [{"k": self.bufs[i]["k"].ptr, "v": self.bufs[i]["v"].ptr, "ck": self.bufs[i]["ck"].ptr, "cv": self.bufs[i]["cv"].ptr,
+                 "length": self.streams[i]["length"], "memory_length": self.streams[i]["memory_length"],
+                 "inp": self.bufs[i]["x"].ptr, "out": self.bufs[i]["out"].ptr} for i in which]
+
+    def step(self, which=None):
+        self.dec.step(self.slots(which))
+        which = range(len(self.streams)) if which is None else which
+        return [self.bufs[i]["out"].read() for i in which]
+
+    def reset_cache(self, i):
+        self.bufs[i]["k"].write(self.streams[i]["k"])
+        self.bufs[i]["v"].write(self.streams[i]["v"])
+
+    def cache_rows(self, i):
+        shape = self.streams[i]["k"].shape
+        return self.bufs[i]["k"].read().reshape(shape), self.bufs[i]["v"].read().reshape(shape)
+
+    def close(self):
+        self.dec.destroy()
+        for b in self.bufs:
+            for d in b.values():
+                d.free()
+
+
+def _oracle_step(orc, cfg, weights, streams, qtype):
+    odec = orc.Decoder(cfg, weights, qtype)
+    ks = [s["k"].copy() for s in streams]
+    vs = [s["v"].copy() for s in streams]
+    outs = odec.step(ks, vs, [s["ck"] for s in streams], [s["cv"] for s in streams], [s["length"] for s in streams],
+                     [s["memory_length"] for s in streams], [s["x"] for s in streams])
+    return outs, ks, vs
+
+
+QT = {"f32": 0, "int8": 1, "int4": 2, "f16": 3}
+# f32/f16 activations stay f32 end to end: 1e-5 normalised (f16: against the oracle run on the same f16 bits).
+# int8/int4 re-quantise the activation of every projection; one last-bit difference in a LayerNorm output can move
+# an int8 activation by one step, which the next layers amplify, so whole-step agreement is bounded at 2e-2 while the
+# per-projection integers are checked bit-exactly in test_gpu_seam.py.
+TOL = {"f32": 1e-5, "f16": 1e-5, "int8": 2e-2, "int4": 2e-2}
+
+
+@pytest.mark.parametrize("qtype_name", ["f32", "f16", "int8", "int4"])
+def test_one_block_batch1_kv256(pkg, backend, orc, synth, nerr, qtype_name):
+    """One decoder block, batch 1, KV length 256, LayerNorm gain and bias (the f32 case is the benchmark's
+    CPU-runnable configuration)."""
+    _announce("one block b=1 kv=256 %s" % qtype_name)
+    cfg = synth.decoder_config(layers=1, capacity=258, cross_heads=0)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, [256], [0], seed=1)
+    backend.set_quant(QT[qtype_name])
+    h = Harness(pkg, backend, cfg, weights, streams)
+    got = h.step()
+    want, ks, vs = _oracle_step(orc, cfg, weights, streams, QT[qtype_name])
+    assert nerr(got[0], want[0]) < TOL[qtype_name]
+    gk, gv = h.cache_rows(0)
+    assert nerr(gk[0, 256], ks[0][0, 256]) < TOL[qtype_name] and nerr(gv[0, 256], vs[0][0, 256]) < TOL[qtype_name]
+    mask = np.ones(258, bool)
+    mask[256] = False
+    assert np.array_equal(gk[:, mask], streams[0]["k"][:, mask]) and np.array_equal(gv[:, mask], streams[0]["v"][:, mask])
+    h.close()
+    backend.set_quant(0)
+
+
+@pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4", "f16"])
+def test_two_layers_ragged_batch8_and_bit_identity(pkg, backend, orc, synth, nerr, qtype_name):
+    """Ragged B=8 (incl. an empty cache and chunk-edge lengths) against the oracle, eager and graph replay,
+    and every stream bit-identical to the same stream run alone on the GPU."""
+    _announce("two layers ragged b=8 %s" % qtype_name)
+    lengths = [5, 64, 0, 129, 63, 2, 300, 65]
+    mems = [7, 64, 3, 32, 65, 1, 27, 200]
+    cfg = synth.decoder_config(layers=2, capacity=304)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=1)
+    backend.set_quant(QT[qtype_name])
+    h = Harness(pkg, backend, cfg, weights, streams)
+    want, ks, vs = _oracle_step(orc, cfg, weights, streams, QT[qtype_name])
+    first = h.step()                        # eager (first use of this batch size)
+    for b in range(8):
+        assert nerr(first[b], want[b]) < TOL[qtype_name], "stream %d" % b
+    for b in (0, 3, 6):
+        gk, gv = h.cache_rows(b)
+        L = lengths[b]
+        for layer in range(2):
+            assert nerr(gk[layer, L], ks[b][layer, L]) < TOL[qtype_name]
+            assert nerr(gv[layer, L], vs[b][layer, L]) < TOL[qtype_name]
+    # graph capture + three replays, interleaved with host reads, must reproduce the eager result bit for bit
+    for replay in range(4):
+        for b in range(8):
+            h.reset_cache(b)
+        again = h.step()
+        for b in range(8):
+            assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32)), "replay %d stream %d" % (replay, b)
+    # batched == solo, bitwise, for every stream
+    for b in range(8):
+        h.reset_cache(b)
+        solo = h.step([b])[0]
+        assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
+    # a different batch composition (B = 3) keeps each stream's bits as well
+    for b in (1, 4, 7):
+        h.reset_cache(b)
+    sub = h.step([7, 1, 4])
+    for got, b in zip(sub, (7, 1, 4)):
+        assert np.array_equal(got.view(np.uint32), first[b].view(np.uint32))
+    h.close()
+    backend.set_quant(0)
+
+
+def test_twelve_layers_int8_multi_step(pkg, backend, orc, synth, nerr):
+    """The benchmark stack (12 layers, 12x64 cross heads, int8) at reduced cache length, two consecutive steps
+    so that the second step attends over the row the first one appended."""
+    _announce("12 layers int8 two steps")
+    cfg = synth.decoder_config(layers=12, capacity=132)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, [128, 40], [64, 48], seed=1)
+    backend.set_quant(1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    odec = orc.Decoder(cfg, weights, orc.INT8)
+    ks = [s["k"].copy() for s in streams]
+    vs = [s["v"].copy() for s in streams]
+    lengths = [128, 40]
+    for step in range(2):
+        for i, s in enumerate(streams):
+            s["length"] = lengths[i]
+        want = odec.step(ks, vs, [s["ck"] for s in streams], [s["cv"] for s in streams], lengths, [64, 48], [s["x"] for s in streams])
+        got = h.step()
+        for b in range(2):
+            assert nerr(got[b], want[b]) < 5e-2, "step %d stream %d" % (step, b)
+        lengths = [n + 1 for n in lengths]
+    h.close()
+    backend.set_quant(0)
+
+
+def test_step_error_paths(pkg, backend, synth):
+    _announce("step error paths")
+    cfg = synth.decoder_config(layers=1, capacity=8)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, [7], [4], seed=1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    h.step()                                             # the last row still fits
+    streams[0]["length"] = 8
+    with pytest.raises(pkg.BackendError, match="capacity exceeded"):      # src/graph.c:3152-3155
+        h.step()
+    streams[0]["length"] = 7
+    with pytest.raises(pkg.BackendError, match="MYNAH_MAX_BATCH"):        # src/graph.c:3133-3136
+        h.dec.step(h.slots([0] * 17))
+    h.dec.step([])                                       # empty batch is a no-op (src/graph.c:3132)
+    h.close()
+
+
+def test_output_head(pkg, backend, orc, synth, nerr):
+    """Final-normed rows -> 8 x 1024 logits -> per-head softmax, int8 and f32 weights."""
+    _announce("output head")
+    rng = np.random.default_rng(1100)
+    w = backend.keep((rng.standard_normal((8192, 768)) * 0.02).astype(np.float32))
+    hidden = rng.standard_normal((3, 768)).astype(np.float32)
+    for qtype in (pkg.F32, pkg.INT8, pkg.INT4):
+        backend.set_quant(qtype)
+        dh = [backend.alloc(768).write(hidden[b]) for b in range(3)]
+        dl = [backend.alloc(8192) for _ in range(3)]
+        dp = [backend.alloc(8192) for _ in range(3)]
+        backend.output_head([d.ptr for d in dh], 768, w, None, 8192, 1024, [d.ptr for d in dl], [d.ptr for d in dp])
+        pw = orc.PackedWeight(w, qtype)
+        for b in range(3):
+            logits, probs = orc.output_head(pw, hidden[b], 8, 1024)
+            assert nerr(dl[b].read(), logits) < 1e-5
+            got = dp[b].read()
+            assert nerr(got, probs) < 1e-5
+            assert np.allclose(got.reshape(8, 1024).sum(-1), 1.0, atol=1e-5)
+        for d in dh + dl + dp:
+            d.free()
+    backend.set_quant(0)
