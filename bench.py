@@ -1,0 +1,187 @@
+"""Decode-step benchmark: us per step and achieved HBM GB/s of the int8 12-layer decoder stack on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--quant int8] [--skip-b8]
+
+Workload (named in config.workload): the 12-layer d=768 decoder stack (12 heads x 64, FFN 3072, a 12 x 64
+cross-attention sublayer per layer), int8 weights, batch 1, self-KV length 1024, cross-KV length 256, followed by the
+final LayerNorm, the 768 -> 8 x 1024 output projection and the per-head softmax.  Synthetic seeded data, random
+weights.  A "step" is one decode step of that stack for the whole batch.
+
+HBM honesty: the int8 weights (106 MB) and one stream's KV (94 MB) would fit in the 256 MB last-level cache, so the
+timed loop rotates over several independent copies of weights AND caches (ROTATE sets, > 600 MB in total): every step
+streams its bytes from HBM.  Inputs are resident in HBM before the timed region starts; nothing crosses PCIe in it.
+
+The JSON line also carries the same stack at batch 8 with ragged cache lengths (continuous batching) under "b8",
+the roofline of the step and the CPU baseline (the reference's own CPU decode step, compiled from its sources).
+"""
+import argparse
+import json
+import os
+import subprocess
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+METRIC = "decode-step µs + achieved HBM GB/s (% of 8 TB/s peak), int8 b=1 and b=8"
+PEAK_GBPS = 8000.0
+ROTATE = 3
+
+
+def build_sets(pkg, synth, backend, cfg, qtype, lengths, mems, head_rows, rotate):
+    """`rotate` independent copies of the decoder weights, the output head and the per-stream caches."""
+    base = synth.decoder_weights(cfg, seed=0)
+    rng = np.random.default_rng(7)
+    head = (rng.standard_normal((head_rows, cfg["width"]), dtype=np.float32) * np.float32(0.02))
+    sets = []
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=1)
+    for r in range(rotate):
+        weights = {k: (None if v is None else np.array(v, copy=True)) for k, v in base.items()}   # new host addresses
+        dec = pkg.Decoder(backend, cfg, weights)
+        head_w = backend.keep(np.array(head, copy=True))
+        slots, outs, logits, probs = [], [], [], []
+        for s in streams:
+            bufs = {n: backend.alloc(max(s[n].size, 4)).write(s[n]) for n in ("k", "v", "ck", "cv", "x")}
+            out = backend.alloc(cfg["width"])
+            slots.append({"k": bufs["k"].ptr, "v": bufs["v"].ptr, "ck": bufs["ck"].ptr, "cv": bufs["cv"].ptr,
+                          "length": s["length"], "memory_length": s["memory_length"], "inp": bufs["x"].ptr, "out": out.ptr})
+            outs.append(out)
+            logits.append(backend.alloc(head_rows))
+            probs.append(backend.alloc(head_rows))
+        sets.append({"dec": dec, "head": head_w, "slots": slots, "outs": outs, "logits": logits, "probs": probs})
+    return sets, streams
+
+
+def run_steps(backend, sets, cfg, head_rows, vocab, count, start=0):
+    for i in range(start, start + count):
+        s = sets[i % len(sets)]
+        s["dec"].step(s["slots"])
+        backend.output_head([o.ptr for o in s["outs"]], cfg["width"], s["head"], None, head_rows, vocab,
+                            [d.ptr for d in s["logits"]], [d.ptr for d in s["probs"]])
+
+
+def time_config(pkg, synth, backend, qtype, lengths, mems, capacity, steps, warmup, rotate=ROTATE):
+    cfg = synth.decoder_config(layers=12, capacity=capacity)
+    head_rows, vocab = 8 * 1024, 1024
+    backend.set_quant(qtype)
+    t0 = time.time()
+    sets, streams = build_sets(pkg, synth, backend, cfg, qtype, lengths, mems, head_rows, rotate)
+    setup_s = time.time() - t0
+    run_steps(backend, sets, cfg, head_rows, vocab, max(warmup, 2 * rotate))      # eager pass + graph capture for every set
+    backend.sync()
+    backend.timer_begin()
+    run_steps(backend, sets, cfg, head_rows, vocab, steps)
+    ms = backend.timer_end()
+    step_us = ms * 1000.0 / steps
+    b = synth.decoder_step_bytes(cfg, qtype, [s["length"] for s in streams], [s["memory_length"] for s in streams])
+    head_bytes = synth.weight_bytes(head_rows, cfg["width"], qtype)
+    total = b["total"] + head_bytes
+    probs = sets[0]["probs"][0].read()
+    assert np.all(np.isfinite(probs)) and abs(float(probs[:vocab].sum()) - 1.0) < 1e-3, "benchmark output is not a distribution"
+    for s in sets:
+        s["dec"].destroy()
+    return {"step_us": step_us, "bytes": total, "weight_bytes": b["weights"] + head_bytes, "kv_bytes": b["kv"],
+            "gbps": total / (step_us * 1e-6) / 1e9, "setup_s": setup_s}
+
+
+def cpu_baseline(steps=5, warmup=2):
+    """The reference's own CPU decode step (compiled from its sources into oracle/_ref), timed on this box's host
+    cores in a child process: all online cores, then one thread."""
+    out = {}
+    cores = os.cpu_count() or 1
+    for label, threads in (("all", cores), ("one", 1)):
+        cmd = [sys.executable, os.path.join(ROOT, "oracle", "cpu_baseline.py"), "--kind", "reference", "--threads", str(threads),
+               "--steps", str(steps), "--warmup", str(warmup)]
+        try:
+            proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
+            out[label] = json.loads(proc.stdout.strip().splitlines()[-1])
+        except Exception as e:   # the baseline is reported, never required for the GPU number
+            out[label] = {"error": str(e)[:200]}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--quant", default="int8", choices=["int8", "int4", "f16", "f32"])
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--skip-b8", action="store_true")
+    ap.add_argument("--no-graph", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X: the decode step has no multi-GPU form (streams shard by request, with no "
+              "exchange step); run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    pkg = entry.load_package()
+    import mynah_tts_amd.synth as synth
+    qtype = {"f32": pkg.F32, "int8": pkg.INT8, "int4": pkg.INT4, "f16": pkg.F16}[args.quant]
+    backend = pkg.Backend(quant=qtype)
+    if args.no_graph:
+        backend.set_graph_mode(False)
+
+    b1 = time_config(pkg, synth, backend, qtype, [1023], [256], 1024, args.steps, args.warmup)
+    b8 = None
+    if not args.skip_b8:
+        self_len, cross_len = synth.ragged_lengths(8, seed=3)
+        b8 = time_config(pkg, synth, backend, qtype, [n - 1 for n in self_len], cross_len, 2048, max(args.steps // 3, 20),
+                         max(args.warmup // 3, 6), rotate=ROTATE)
+        b8["self_lengths"], b8["cross_lengths"] = self_len, cross_len
+    backend.close()
+
+    result = {
+        "metric": METRIC,
+        "value": round(b1["gbps"], 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(b1["step_us"] / 1000.0, 6),
+        "step_us": round(b1["step_us"], 2),
+        "pct_of_peak": round(100.0 * b1["gbps"] / PEAK_GBPS, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"int8": "int8 weights x int8 activations -> int32, f32 epilogue", "int4": "int4 x int8 -> int32 per group",
+                  "f16": "f16 weights, f32 accumulate", "f32": "f32"}[args.quant],
+        "data": "synthetic (seeded N(0,1) activations and caches, N(0,0.02) weights quantised at load time)",
+        "config": {"workload": "12-layer d=768 decoder stack decode step, %s weights, batch 1, self-KV 1024, cross-KV 256 "
+                               "(12x64 heads), final LayerNorm + 768->8x1024 output head + softmax" % args.quant,
+                   "batch": 1, "layers": 12, "width": 768, "self_kv": 1024, "cross_kv": 256, "quant": args.quant,
+                   "graph": not args.no_graph, "rotating_sets": ROTATE},
+        "roofline": {"bound": "hbm", "kernel": "decode step = one HIP graph of 97 stage kernels + 3 head kernels "
+                                               "(k_linear int8 matvecs and k_attention carry the bytes)",
+                     "achieved": round(b1["gbps"], 2), "peak": PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(b1["gbps"] / PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_step": b1["bytes"], "weight_bytes": b1["weight_bytes"], "kv_bytes": b1["kv_bytes"]},
+    }
+    if b8 is not None:
+        result["b8"] = {"step_us": round(b8["step_us"], 2), "gbps": round(b8["gbps"], 2),
+                        "pct_of_peak": round(100.0 * b8["gbps"] / PEAK_GBPS, 2), "algorithmic_bytes_per_step": b8["bytes"],
+                        "weight_bytes": b8["weight_bytes"], "kv_bytes": b8["kv_bytes"], "self_lengths": b8["self_lengths"],
+                        "cross_lengths": b8["cross_lengths"],
+                        "us_per_stream_step": round(b8["step_us"] / 8.0, 2)}
+    if not args.no_cpu:
+        cpu = cpu_baseline()
+        allc = cpu.get("all", {})
+        result["cpu_baseline"] = {
+            "value": round(allc.get("median_us", float("nan")), 1), "unit": "us per decode step (batch 1)",
+            "cores": allc.get("threads"), "kind": allc.get("kind", "reference"),
+            "sample": "median of 5 steps after 2 warm-ups of the reference's own decoder_step_batch (stock flags, its pthread "
+                      "pool) on the same 12-layer int8 stack, self-KV 1024, cross-KV 256; that function has gain-only LayerNorm and "
+                      "one 768-wide cross head (same bytes and flops) and no output head",
+            "one_thread_us": round(cpu.get("one", {}).get("median_us", float("nan")), 1),
+            "online_cores": allc.get("online_cores"),
+            "gpu_speedup": round(allc.get("median_us", float("nan")) / b1["step_us"], 1) if "median_us" in allc else None,
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -19,7 +19,8 @@ constexpr int kMaxBatch = MYNAH_HIP_MAX_BATCH;
 constexpr int kBatchTile = 8;        // streams served by one pass over a weight tile
 constexpr size_t kQuantMaxRows = 16; // QMAT_SMALL_COUNT, src/qmat.c:32
 constexpr size_t kQuantMaxK = 8192;  // QMAT_K_MAX, src/qmat.c:33
-constexpr int kAttnChunk = 64;       // cache positions handled by one attention workgroup
+constexpr int kAttnChunk = 64;       // cache positions handled by one workgroup of the stand-alone attention kernels
+constexpr int kStepUnitRows = 128;   // cache rows per attention unit (workgroup) of the fused resident step
 
 // ---- error plumbing (0 / -1 + message, src/backend.c:137-139) ----
 inline void set_error(char *error, size_t capacity, const char *message) {

@@ -1,19 +1,21 @@
-// The resident batched decode step: decoder_step_batch (src/graph.c:3127-3284) as eight fused
+// The resident batched decode step: decoder_step_batch (src/graph.c:3127-3284) as six fused
 // kernels per layer, replayed as one HIP graph.
 //
-//   per layer   1  LN(norm_self) + act-quant + QKV matvec                      -> qkv
-//               2  self-attention with KV append (split over cache chunks)     -> attn
-//               3  act-quant + O matvec + residual                             -> x
-//               4  LN(norm_xattn_query) + act-quant + Q matvec                 -> qx
-//               5  cross-attention over the encoder memory                     -> ctx
-//               6  act-quant + O matvec + residual                             -> x
-//               7  LN(norm_pos_ff) + act-quant + up matvec + tanh-GELU         -> hidden
-//               8  act-quant + down matvec + residual                          -> x
+//   per layer   1  LN(norm_self) + act-quant + per-head Q/K/V rows + KV append + split-L self-attention -> partials
+//               2  fold partials + act-quant + O matvec + residual                                       -> x
+//               3  LN(norm_xattn_query) + act-quant + per-head Q rows + split-L cross-attention          -> partials
+//               4  fold partials + act-quant + O matvec + residual                                       -> x
+//               5  LN(norm_pos_ff) + act-quant + up matvec + tanh-GELU                                   -> hidden
+//               6  act-quant + down matvec + residual                                                    -> x
 //   begin / end    x = input + position[length]   /   out = LN(norm_out)(x)
+//
+// Head shapes the fused attention kernel does not take (head width other than 64) run the same step as
+// eight kernels per layer: projection, stand-alone attention, projection.
 //
 // Everything that changes from step to step (cache pointers, lengths, input/output rows) lives in a
 // small device-side slot table written by the begin kernel, so the captured graph is replayed
 // unchanged for the life of a (decoder, batch size) pair.
+#include <stdlib.h>
 #include <string.h>
 
 #include <new>
@@ -36,6 +38,10 @@ struct mynah_hip_decoder {
     // workspaces, kMaxBatch rows each
     float *x = nullptr, *qkv = nullptr, *attn = nullptr, *qx = nullptr, *ctx = nullptr, *hidden = nullptr;
     mynah::StepSlots *dev_slots = nullptr;
+    float *partial = nullptr;   // split-L attention partials of the fused path
+    float *partial_ml = nullptr;
+    int max_units = 0;
+    bool fused_attention = false;
     hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};
     int eager_steps[mynah::kMaxBatch + 1] = {};   // a batch size runs eagerly once before it is captured
     int arith = 0;
@@ -43,11 +49,22 @@ struct mynah_hip_decoder {
 
 namespace mynah {
 
+// fold: 0 = plain input rows, 1 = fold of the self-attention partials, 2 = fold of the cross-attention partials
 static int enqueue_linear(State *st, const mynah_hip_decoder *d, const CachedWeight *w, const float *in, size_t in_stride,
                           float *out, size_t out_stride, int batch, const float *ln_gain, const float *ln_bias, int epilogue,
-                          char *error, size_t capacity) {
+                          char *error, size_t capacity, int fold = 0) {
     for (int b0 = 0; b0 < batch; b0 += kBatchTile) {
         LinearArgs a{};
+        if (fold != 0) {
+            a.fold_partial = d->partial;
+            a.fold_partial_ml = d->partial_ml;
+            a.fold_slots = d->dev_slots;
+            a.fold_heads = (int)(fold == 1 ? d->heads : d->cross_heads);
+            a.fold_head_width = (int)(fold == 1 ? d->head_width : d->cross_head_width);
+            a.fold_max_units = d->max_units;
+            a.fold_is_self = fold == 1 ? 1 : 0;
+            a.fold_stream0 = b0;
+        }
         a.w = w->data;
         a.scales = w->scales;
         a.bias = nullptr;   // no decoder linear has a bias (src/graph.c:3169-3272 pass NULL)
@@ -100,9 +117,48 @@ static int enqueue_attention(State *st, const mynah_hip_decoder *d, int is_self,
     return launch_attention(st, a, error, capacity);
 }
 
+static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_self, size_t layer, int batch, const CachedWeight *w,
+                                  const float *ln_gain, const float *ln_bias, char *error, size_t capacity) {
+    StepAttnArgs a{};
+    a.slots = d->dev_slots;
+    a.x = d->x;
+    a.batch = batch;
+    a.width = (int)d->width;
+    a.ln_gain = ln_gain;
+    a.ln_bias = ln_bias;
+    a.w = w->data;
+    a.scales = w->scales;
+    a.qtype = w->qtype;
+    a.arith = d->arith;
+    a.is_self = is_self;
+    a.heads = (int)(is_self ? d->heads : d->cross_heads);
+    a.head_width = (int)(is_self ? d->head_width : d->cross_head_width);
+    a.layer = layer;
+    a.capacity = d->capacity;
+    a.max_units = d->max_units;
+    a.scale = 1.0f / sqrtf((float)a.head_width);
+    a.partial = d->partial;
+    a.partial_ml = d->partial_ml;
+    return launch_step_attention(st, a, error, capacity);
+}
+
 // The layer loop; everything here is replayable (no per-step scalars in kernel arguments).
 static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char *error, size_t capacity) {
     const size_t w = d->width;
+    if (d->fused_attention) {
+        for (size_t l = 0; l < d->layers; ++l) {
+            const LayerWeights &lw = d->lw[l];
+            if (enqueue_step_attention(st, d, 1, l, batch, lw.qkv, lw.norm_self, lw.norm_self_b, error, capacity) != 0) return -1;
+            if (enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, 1) != 0) return -1;
+            if (d->xw != 0) {
+                if (enqueue_step_attention(st, d, 0, l, batch, lw.q_cross, lw.norm_cross, lw.norm_cross_b, error, capacity) != 0) return -1;
+                if (enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, 2) != 0) return -1;
+            }
+            if (enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity) != 0) return -1;
+            if (enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
+        }
+        return launch_step_end(st, d->dev_slots, batch, w, d->x, w, d->norm_out, d->norm_out_b, error, capacity);
+    }
     for (size_t l = 0; l < d->layers; ++l) {
         const LayerWeights &lw = d->lw[l];
         if (enqueue_linear(st, d, lw.qkv, d->x, w, d->qkv, 3 * w, batch, lw.norm_self, lw.norm_self_b, EPI_NONE, error, capacity) != 0) return -1;
@@ -136,7 +192,7 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
     for (auto &g : d->graphs)
         if (g != nullptr) (void)hipGraphExecDestroy(g);
-    float *bufs[] = {d->x, d->qkv, d->attn, d->qx, d->ctx, d->hidden};
+    float *bufs[] = {d->x, d->qkv, d->attn, d->qx, d->ctx, d->hidden, d->partial, d->partial_ml};
     for (float *p : bufs)
         if (p != nullptr) (void)hipFree(p);
     if (d->dev_slots != nullptr) (void)hipFree(d->dev_slots);
@@ -215,6 +271,22 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
     const size_t hw_max = d->head_width > d->cross_head_width ? d->head_width : d->cross_head_width;
     const size_t heads_max = d->heads > d->cross_heads ? d->heads : d->cross_heads;
     if (rc == 0) rc |= ensure_attention_workspace(st, B, heads_max, hw_max, d->capacity, error, capacity);
+    if (rc == 0) {
+        const char *env = getenv("MYNAH_HIP_FUSED_ATTENTION");
+        const LayerWeights &l0 = d->lw[0];
+        d->fused_attention = !(env != nullptr && strcmp(env, "0") == 0) &&
+                             step_attention_supported(l0.qkv->qtype, w, d->heads, d->head_width) &&
+                             (xw == 0 || (l0.q_cross->qtype == l0.qkv->qtype &&
+                                          step_attention_supported(l0.q_cross->qtype, w, d->cross_heads, d->cross_head_width)));
+        d->max_units = (int)((d->capacity + kStepUnitRows - 1) / kStepUnitRows) + 1;
+        if (d->fused_attention) {
+            const size_t floats = B * heads_max * (size_t)d->max_units * hw_max;
+            rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial), floats * sizeof(float)), "malloc", error, capacity);
+            if (rc == 0)
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial_ml), B * heads_max * 2 * (size_t)d->max_units * sizeof(float)),
+                                "malloc", error, capacity);
+        }
+    }
     if (rc != 0) {
         mynah_hip_decoder_destroy(opaque, d);
         return -1;

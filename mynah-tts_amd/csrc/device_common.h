@@ -1,0 +1,429 @@
+// Device-side building blocks shared by the matvec and attention kernels (gfx950, wave64).
+#pragma once
+
+#include "kernels.h"
+
+namespace mynah {
+
+constexpr int kThreads = 256;             // every fused kernel runs 4 waves per workgroup
+
+// ---- wavefront reductions on the DPP data path (no LDS round trips) -------------------------------------
+// Lane permutations inside a row of 16 lanes: xor 1, xor 2, mirror within 8, mirror within 16.  After the
+// four steps every lane of a row holds the row's total (float addition is commutative, so all lanes of a
+// row compute bit-identical values).  Rows are then combined through v_readlane in the fixed order
+// ((r0 + r1) + r2) + r3.  All 64 lanes must be active.
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // row_half_mirror
+constexpr int kDppMirror = 0x140;     // row_mirror
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_f(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_f<kDppXor1>(v);
+    v += dpp_f<kDppXor2>(v);
+    v += dpp_f<kDppHalfMirror>(v);
+    v += dpp_f<kDppMirror>(v);
+    return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = fmaxf(v, dpp_f<kDppXor1>(v));
+    v = fmaxf(v, dpp_f<kDppXor2>(v));
+    v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_f<kDppMirror>(v));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    return ((lane_f(v, 0) + lane_f(v, 16)) + lane_f(v, 32)) + lane_f(v, 48);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = row16_max(v);
+    return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
+}
+
+// Sum over aligned groups of 1 << lg lanes (lg uniform, 0..6); every lane of a group gets the group's total.
+__device__ __forceinline__ float group_sum_f(float v, int lg) {
+    if (lg >= 1) v += dpp_f<kDppXor1>(v);
+    if (lg >= 2) v += dpp_f<kDppXor2>(v);
+    if (lg >= 3) v += dpp_f<kDppHalfMirror>(v);
+    if (lg >= 4) v += dpp_f<kDppMirror>(v);
+    if (lg >= 5) {
+        const float r0 = lane_f(v, 0), r1 = lane_f(v, 16), r2 = lane_f(v, 32), r3 = lane_f(v, 48);
+        if (lg == 5) v = (threadIdx.x & 32) ? r2 + r3 : r0 + r1;
+        else v = ((r0 + r1) + r2) + r3;
+    }
+    return v;
+}
+__device__ __forceinline__ int group_sum_i(int v, int lg) {
+    if (lg >= 1) v += dpp_i<kDppXor1>(v);
+    if (lg >= 2) v += dpp_i<kDppXor2>(v);
+    if (lg >= 3) v += dpp_i<kDppHalfMirror>(v);
+    if (lg >= 4) v += dpp_i<kDppMirror>(v);
+    if (lg >= 5) {
+        const int r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+        const int r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+        if (lg == 5) v = (threadIdx.x & 32) ? r2 + r3 : r0 + r1;
+        else v = r0 + r1 + r2 + r3;
+    }
+    return v;
+}
+
+// Reduces BT independent values over the 256-thread workgroup in a fixed order: lanes by butterfly,
+// then waves 0..3.  The order never depends on how many of the BT slots are live.
+template <int BT, bool IS_MAX>
+__device__ __forceinline__ void block_reduce(float (&v)[BT], float *s_scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int b = 0; b < BT; ++b) v[b] = IS_MAX ? wave_max(v[b]) : wave_sum(v[b]);
+    __syncthreads();
+    if (lane == 0) {
+#pragma unroll
+        for (int b = 0; b < BT; ++b) s_scratch[wave * BT + b] = v[b];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < BT; ++b) {
+        const float a0 = s_scratch[b], a1 = s_scratch[BT + b], a2 = s_scratch[2 * BT + b], a3 = s_scratch[3 * BT + b];
+        v[b] = IS_MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : ((a0 + a1) + a2) + a3;
+    }
+}
+
+// round half away from zero by truncation, clamp to +-127 (src/qmat.c:106-110)
+__device__ __forceinline__ int quant_act(float x, float inv) {
+    const float v = x * inv;
+    int q = (int)(v >= 0.0f ? v + 0.5f : v - 0.5f);
+    q = q > 127 ? 127 : q;
+    q = q < -127 ? -127 : q;
+    return q;
+}
+
+// src/kernels.c:382-389
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float cubic = x * x * x;
+    const float c = 0.7978845608f * (x + 0.044715f * cubic);
+    return 0.5f * x * (1.0f + tanhf(c));
+}
+
+__device__ __forceinline__ int dot4(unsigned a, unsigned b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// offset-binary nibbles (q + 8) of one dword -> four signed bytes each for the even and odd elements
+__device__ __forceinline__ void unpack_q4(unsigned w, unsigned &even, unsigned &odd) {
+    const unsigned lo = w & 0x0f0f0f0fu;
+    const unsigned hi = (w >> 4) & 0x0f0f0f0fu;
+    even = ((lo | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+    odd = ((hi | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+}
+
+// exact widening of an IEEE half (v_cvt_f32_f16)
+__device__ __forceinline__ float half_bits_to_float(unsigned short h) {
+    _Float16 v;
+    __builtin_memcpy(&v, &h, sizeof v);
+    return (float)v;
+}
+
+template <int QT> struct Chunk;   // elements per 16-byte weight chunk
+template <> struct Chunk<MYNAH_HIP_F32> { static constexpr int n = 4; };
+template <> struct Chunk<MYNAH_HIP_F16> { static constexpr int n = 8; };
+template <> struct Chunk<MYNAH_HIP_INT8> { static constexpr int n = 16; };
+template <> struct Chunk<MYNAH_HIP_INT4> { static constexpr int n = 32; };
+
+template <int QT>
+constexpr bool kQuantised = (QT == MYNAH_HIP_INT8 || QT == MYNAH_HIP_INT4);
+
+// Lane-group width for a row of `chunks` 16-byte chunks: the widest power of two that still leaves
+// about three chunks per lane (k = 768 int8 -> 16 lanes, k = 3072 int8 -> 64 lanes).
+__host__ __device__ inline int lane_group_log2(int chunks) {
+    int lg = 6;
+    while (lg > 0 && (chunks >> lg) < 3) --lg;
+    return lg;
+}
+
+// One 16-byte weight chunk against the staged activations of BT streams.
+//   int8 : iacc += sum w*qx                         (dot_q8, src/qmat.c:136-152)
+//   int4 : facc += (float)(group int32) * scale[g]  (dot_q4, src/qmat.c:156-185; one chunk = one group of 32)
+//   f16  : facc = fma(widen(w), x, facc)            (matvec_f16, src/qmat.c:306-378)
+//   f32  : facc = fma(w, x, facc)
+// group_out (int4 probe): per-group integer of stream 0.
+template <int QT, int BT>
+__device__ __forceinline__ void dot_chunk(const uint4 wv, const float sc, const int c, const unsigned char *smem, const int k,
+                                          int (&iacc)[BT], float (&facc)[BT], int *group_out) {
+    if constexpr (QT == MYNAH_HIP_INT8) {
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const uint4 xv = *reinterpret_cast<const uint4 *>(smem + (size_t)b * k + (size_t)c * 16);
+            int s = iacc[b];
+            s = dot4(wv.x, xv.x, s);
+            s = dot4(wv.y, xv.y, s);
+            s = dot4(wv.z, xv.z, s);
+            s = dot4(wv.w, xv.w, s);
+            iacc[b] = s;
+        }
+    } else if constexpr (QT == MYNAH_HIP_INT4) {
+        unsigned e0, o0, e1, o1, e2, o2, e3, o3;
+        unpack_q4(wv.x, e0, o0);
+        unpack_q4(wv.y, e1, o1);
+        unpack_q4(wv.z, e2, o2);
+        unpack_q4(wv.w, e3, o3);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const uint4 *xp = reinterpret_cast<const uint4 *>(smem + (size_t)b * k + (size_t)c * 32);
+            const uint4 xa = xp[0], xb = xp[1];
+            int gi = 0;
+            gi = dot4(e0, xa.x, gi); gi = dot4(o0, xa.y, gi);
+            gi = dot4(e1, xa.z, gi); gi = dot4(o1, xa.w, gi);
+            gi = dot4(e2, xb.x, gi); gi = dot4(o2, xb.y, gi);
+            gi = dot4(e3, xb.z, gi); gi = dot4(o3, xb.w, gi);
+            const float term = (float)gi * sc;   // acc += (float)gi * scales[g]  (src/qmat.c:181)
+            facc[b] = facc[b] + term;
+            if (b == 0 && group_out != nullptr) *group_out = gi;
+        }
+    } else if constexpr (QT == MYNAH_HIP_F16) {
+        const unsigned wd[4] = {wv.x, wv.y, wv.z, wv.w};
+        float wf[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            wf[2 * i] = half_bits_to_float((unsigned short)(wd[i] & 0xffffu));
+            wf[2 * i + 1] = half_bits_to_float((unsigned short)(wd[i] >> 16));
+        }
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const float4 *xp = reinterpret_cast<const float4 *>(smem) + (size_t)b * (k >> 2) + (size_t)c * 2;
+            const float4 xa = xp[0], xb = xp[1];
+            float s = facc[b];
+            s = __builtin_fmaf(wf[0], xa.x, s); s = __builtin_fmaf(wf[1], xa.y, s);
+            s = __builtin_fmaf(wf[2], xa.z, s); s = __builtin_fmaf(wf[3], xa.w, s);
+            s = __builtin_fmaf(wf[4], xb.x, s); s = __builtin_fmaf(wf[5], xb.y, s);
+            s = __builtin_fmaf(wf[6], xb.z, s); s = __builtin_fmaf(wf[7], xb.w, s);
+            facc[b] = s;
+        }
+    } else {
+        const float w0 = __uint_as_float(wv.x), w1 = __uint_as_float(wv.y);
+        const float w2 = __uint_as_float(wv.z), w3 = __uint_as_float(wv.w);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const float4 xa = reinterpret_cast<const float4 *>(smem)[(size_t)b * (k >> 2) + c];
+            float s = facc[b];
+            s = __builtin_fmaf(w0, xa.x, s); s = __builtin_fmaf(w1, xa.y, s);
+            s = __builtin_fmaf(w2, xa.z, s); s = __builtin_fmaf(w3, xa.w, s);
+            facc[b] = s;
+        }
+    }
+}
+
+// Reduction over a lane group of G = 1 << lg lanes: the same tree for every batch size.
+template <int QT, int BT>
+__device__ __forceinline__ void group_reduce(int (&iacc)[BT], float (&facc)[BT], const int lg) {
+#pragma unroll
+    for (int b = 0; b < BT; ++b) {
+        if constexpr (QT == MYNAH_HIP_INT8) iacc[b] = group_sum_i(iacc[b], lg);
+        else facc[b] = group_sum_f(facc[b], lg);
+    }
+}
+
+// ((float)acc * scale[row]) * sx (src/qmat.c:224) / acc * sx (src/qmat.c:292) / acc
+template <int QT>
+__device__ __forceinline__ float finish_value(const int iacc, const float facc, const float wscale, const float sx) {
+    if constexpr (QT == MYNAH_HIP_INT8) return ((float)iacc * wscale) * sx;
+    else if constexpr (QT == MYNAH_HIP_INT4) return facc * sx;
+    else return facc;
+}
+
+// Where the prologue takes a stream's activation row from.
+struct ActSource {
+    const float *rows[kBatchTile];   // plain device rows (one per stream of the tile) ...
+    // ... or the fold of split-L attention partials (resident step): row[b] = sum_u o_u e^(m_u-M) / sum_u l_u e^(m_u-M)
+    const float *partial;            // non-null selects the fold: partial outputs [stream][head][max_units][head_width]
+    const float *partial_ml;         // chunk maxima and sums [stream][head][2][max_units]
+    const StepSlots *slots;
+    int heads, head_width, max_units, is_self, stream0;
+};
+
+// Units a stream's attention was split into: cache chunks of kStepUnitRows rows, plus the step's new row for
+// self-attention.  Depends on that stream's own length only.
+__device__ __forceinline__ int attention_units(const StepSlots *s, int stream, int is_self) {
+    if (is_self) return (s->length[stream] + kStepUnitRows - 1) / kStepUnitRows + 1;
+    const int chunks = (s->memory_length[stream] + kStepUnitRows - 1) / kStepUnitRows;
+    return chunks > 0 ? chunks : 1;
+}
+
+// One float4 of a stream's folded attention output.  Units are taken in order 0..units-1; the loads of
+// a block of units are independent of the running sums so they are in flight together.
+__device__ __forceinline__ float4 fold_partials(const ActSource &src, int stream, int f4) {
+    const int hw = src.head_width;
+    const int d = 4 * f4;
+    const int head = d / hw, dh = d - head * hw;
+    const size_t sh = (size_t)stream * src.heads + head;
+    const float *m = src.partial_ml + sh * 2 * src.max_units;
+    const float *l = m + src.max_units;
+    const float *o = src.partial + sh * src.max_units * hw + dh;
+    const int units = attention_units(src.slots, stream, src.is_self);
+    float M = -3.0e38f;
+#pragma unroll 8
+    for (int u = 0; u < units; ++u) M = fmaxf(M, m[u]);
+    float L = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+    for (int u = 0; u < units; ++u) {
+        const float w = expf(m[u] - M);
+        const float4 ou = *reinterpret_cast<const float4 *>(o + (size_t)u * hw);
+        L = __builtin_fmaf(l[u], w, L);
+        acc.x = __builtin_fmaf(ou.x, w, acc.x);
+        acc.y = __builtin_fmaf(ou.y, w, acc.y);
+        acc.z = __builtin_fmaf(ou.z, w, acc.z);
+        acc.w = __builtin_fmaf(ou.w, w, acc.w);
+    }
+    acc.x /= L; acc.y /= L; acc.z /= L; acc.w /= L;
+    return acc;
+}
+
+struct PrologueParams {
+    int k;                  // row length (multiple of 4; k/4 <= 256 * NVT)
+    int batch;              // live streams (<= BT)
+    const float *ln_gain;   // non-null: LayerNorm, eps 1e-5 (mynah_layernorm_f32, src/kernels.c:186-244)
+    const float *ln_bias;
+    int arith;
+    int8_t *probe_qx;       // parity probes for stream 0 (written by workgroup 0 only)
+    float *probe_sx;
+};
+
+// Stages the activations of up to BT streams in LDS, all 256 threads cooperating on every stream:
+// load (or fold) -> optional LayerNorm -> for int8/int4 weights the per-vector absmax int8 quantisation
+// (quantize_act_int8, src/qmat.c:94-113; int4 additionally de-interleaves even/odd elements per run of 8
+// so they line up with the low/high nibbles of a weight dword).  NVT = float4 per thread per stream.
+template <int QT, int BT, int NVT>
+__device__ __forceinline__ void stage_activations(const PrologueParams &p, const ActSource &src, unsigned char *smem, float *s_sx,
+                                                  float *s_scratch) {
+    const int tid = threadIdx.x;
+    const int nf4 = p.k >> 2;
+    float4 xr[BT][NVT];
+#pragma unroll
+    for (int b = 0; b < BT; ++b)
+#pragma unroll
+        for (int i = 0; i < NVT; ++i) {
+            const int f = tid + kThreads * i;
+            const bool on = b < p.batch && f < nf4;
+            if (!on) xr[b][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            else if (src.partial != nullptr) xr[b][i] = fold_partials(src, src.stream0 + b, f);
+            else xr[b][i] = reinterpret_cast<const float4 *>(src.rows[b])[f];
+        }
+    if (p.ln_gain != nullptr) {
+        float4 gv[NVT], bv[NVT];
+#pragma unroll
+        for (int i = 0; i < NVT; ++i) {
+            const int f = tid + kThreads * i;
+            gv[i] = f < nf4 ? reinterpret_cast<const float4 *>(p.ln_gain)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+            bv[i] = (f < nf4 && p.ln_bias != nullptr) ? reinterpret_cast<const float4 *>(p.ln_bias)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float s[BT];
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            s[b] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NVT; ++i) s[b] += (xr[b][i].x + xr[b][i].y) + (xr[b][i].z + xr[b][i].w);
+        }
+        block_reduce<BT, false>(s, s_scratch);
+        float mean[BT], v[BT];
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            mean[b] = s[b] / (float)p.k;
+            v[b] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NVT; ++i)
+                if (tid + kThreads * i < nf4) {
+                    const float d0 = xr[b][i].x - mean[b], d1 = xr[b][i].y - mean[b], d2 = xr[b][i].z - mean[b], d3 = xr[b][i].w - mean[b];
+                    v[b] = __builtin_fmaf(d0, d0, v[b]);
+                    v[b] = __builtin_fmaf(d1, d1, v[b]);
+                    v[b] = __builtin_fmaf(d2, d2, v[b]);
+                    v[b] = __builtin_fmaf(d3, d3, v[b]);
+                }
+        }
+        block_reduce<BT, false>(v, s_scratch);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const float rstd = 1.0f / sqrtf(v[b] / (float)p.k + 1.0e-5f);
+#pragma unroll
+            for (int i = 0; i < NVT; ++i) {
+                float4 y;
+                y.x = ((xr[b][i].x - mean[b]) * rstd) * gv[i].x;
+                y.y = ((xr[b][i].y - mean[b]) * rstd) * gv[i].y;
+                y.z = ((xr[b][i].z - mean[b]) * rstd) * gv[i].z;
+                y.w = ((xr[b][i].w - mean[b]) * rstd) * gv[i].w;
+                if (p.ln_bias != nullptr) {
+                    y.x += bv[i].x; y.y += bv[i].y; y.z += bv[i].z; y.w += bv[i].w;
+                }
+                xr[b][i] = y;   // lanes beyond the row hold gain 0 -> 0
+            }
+        }
+    }
+    if constexpr (kQuantised<QT>) {
+        float amax[BT];
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            amax[b] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NVT; ++i)
+                if (tid + kThreads * i < nf4)
+                    amax[b] = fmaxf(fmaxf(amax[b], fmaxf(fabsf(xr[b][i].x), fabsf(xr[b][i].y))), fmaxf(fabsf(xr[b][i].z), fabsf(xr[b][i].w)));
+        }
+        block_reduce<BT, true>(amax, s_scratch);
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            const float inv = amax[b] > 0.0f ? 127.0f / amax[b] : 0.0f;
+            unsigned char *dst = smem + (size_t)b * p.k;
+#pragma unroll
+            for (int i = 0; i < NVT; ++i) {
+                const int f = tid + kThreads * i;
+                if (f < nf4) {
+                    const int q0 = quant_act(xr[b][i].x, inv), q1 = quant_act(xr[b][i].y, inv);
+                    const int q2 = quant_act(xr[b][i].z, inv), q3 = quant_act(xr[b][i].w, inv);
+                    const int idx = 4 * f;
+                    if constexpr (QT == MYNAH_HIP_INT8) {
+                        *reinterpret_cast<unsigned *>(dst + idx) = (unsigned)(q0 & 0xff) | ((unsigned)(q1 & 0xff) << 8) |
+                                                                   ((unsigned)(q2 & 0xff) << 16) | ((unsigned)(q3 & 0xff) << 24);
+                    } else {
+                        const int block = idx & ~7, half = (idx & 4) >> 1;
+                        *reinterpret_cast<unsigned short *>(dst + block + half) = (unsigned short)((q0 & 0xff) | ((q2 & 0xff) << 8));
+                        *reinterpret_cast<unsigned short *>(dst + block + 4 + half) = (unsigned short)((q1 & 0xff) | ((q3 & 0xff) << 8));
+                    }
+                    if (p.probe_qx != nullptr && blockIdx.x == 0 && b == 0) {
+                        p.probe_qx[idx] = (int8_t)q0; p.probe_qx[idx + 1] = (int8_t)q1;
+                        p.probe_qx[idx + 2] = (int8_t)q2; p.probe_qx[idx + 3] = (int8_t)q3;
+                    }
+                }
+            }
+            if (tid == 0) {
+                // returned activation scale (src/qmat.c:112): amax/127, or amax * f32(1/127) as the stock build folds it
+                const float sx = amax[b] > 0.0f ? (p.arith == MYNAH_HIP_ARITH_STOCK ? amax[b] * (1.0f / 127.0f) : amax[b] / 127.0f) : 0.0f;
+                s_sx[b] = sx;
+                if (p.probe_sx != nullptr && blockIdx.x == 0 && b == 0) p.probe_sx[0] = sx;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < BT; ++b) {
+            float4 *dst = reinterpret_cast<float4 *>(smem) + (size_t)b * nf4;
+#pragma unroll
+            for (int i = 0; i < NVT; ++i) {
+                const int f = tid + kThreads * i;
+                if (f < nf4) dst[f] = xr[b][i];
+            }
+            if (tid == 0) s_sx[b] = 1.0f;
+        }
+    }
+    __syncthreads();
+}
+
+}  // namespace mynah

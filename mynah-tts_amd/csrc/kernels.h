@@ -21,6 +21,12 @@ struct LinearArgs {
     const float *ln_bias;   // may be null
     int epilogue;           // EPI_*
     int arith;              // MYNAH_HIP_ARITH_*: how the activation scale is formed
+    // Resident step only: take in[b] from the fold of split-L attention partials instead of a device row
+    // (stream fold_stream0 + b of the slot table; see kernels_step_attention.hip).
+    const float *fold_partial;
+    const float *fold_partial_ml;
+    const StepSlots *fold_slots;
+    int fold_heads, fold_head_width, fold_max_units, fold_is_self, fold_stream0;
     int8_t *probe_qx;       // parity probes (null in production)
     float *probe_sx;
     int32_t *probe_acc;
@@ -58,6 +64,27 @@ struct AttnArgs {
     unsigned *counters;            // [batch, heads], zero between launches
 };
 int launch_attention(State *st, const AttnArgs &args, char *error, size_t capacity);
+
+// Resident step: LayerNorm + activation quantisation + this head's slice of the Q (self: Q, K, V) projection +
+// attention over one cache chunk, per workgroup; writes split-L partials that the next matvec folds.
+struct StepAttnArgs {
+    const StepSlots *slots;
+    const float *x;           // [batch, width] residual stream
+    int batch, width;
+    const float *ln_gain, *ln_bias;
+    const void *w;            // self: [3*width, width] qkv weight; cross: [heads*head_width, width] q weight
+    const float *scales;
+    int qtype, arith;
+    int is_self;
+    int heads, head_width;
+    size_t layer, capacity;   // cache addressing (self: rows `capacity` apart per layer; cross: memory_length)
+    int max_units;            // per stream, incl. the new-row unit for self-attention
+    float scale;
+    float *partial;           // partial outputs [batch, heads, max_units, head_width]
+    float *partial_ml;        // chunk maxima and sums [batch, heads, 2, max_units]
+};
+int launch_step_attention(State *st, const StepAttnArgs &args, char *error, size_t capacity);
+bool step_attention_supported(int qtype, size_t width, size_t heads, size_t head_width);
 
 int launch_layernorm(State *st, const float *in, float *out, const float *gain, const float *bias, size_t rows,
                      size_t width, char *error, size_t capacity);

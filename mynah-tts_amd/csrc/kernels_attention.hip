@@ -6,182 +6,81 @@
 // workgroup owns (stream, head, chunk of 64 cache rows): 16 lanes read one 64-float K row as four
 // coalesced float4 each, scores are reduced inside the 16-lane group, the chunk's (max, sum, partial
 // output) goes to a small workspace, and the LAST workgroup of a (stream, head) to arrive folds the
-// chunks in chunk order with the usual log-sum-exp rescaling.  Which workgroup arrives last does not
+// chunks in a fixed order with the usual log-sum-exp rescaling.  Which workgroup arrives last does not
 // change the arithmetic, and the chunking depends only on the stream's own length, so a stream in a
 // batch is bit-identical to the same stream alone.
+//
+// A decode step is a chain of ~100 dependent kernels, each a few microseconds long, so what matters
+// inside a kernel is the number of dependent memory round trips.  The head_width == 64 path therefore
+// issues every global load it will need (q, its four K rows and its four V rows) before it waits for
+// anything, and the fold reads the partials with ordinary pipelined loads after the acquire fence.
 //
 // The self variant first appends this step's k/v at row `position` (src/graph.c:3180-3181): the
 // workgroup whose chunk contains that row writes its head's slice of the cache row and takes the
 // values from the qkv vector instead of reading them back.
-#include "kernels.h"
+#include "device_common.h"
 
 namespace mynah {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kPosLanes = 16;                    // lanes cooperating on one cache row
+constexpr int kPosLanes = 16;                     // lanes cooperating on one cache row
 constexpr int kPosPerPass = kThreads / kPosLanes; // 16 rows in flight per pass
+constexpr int kRowsPerThread = kAttnChunk / kPosPerPass;   // 4
 
-__device__ __forceinline__ float group16_sum(float v) {
-    v += __shfl_xor(v, 8);
-    v += __shfl_xor(v, 4);
-    v += __shfl_xor(v, 2);
-    v += __shfl_xor(v, 1);
-    return v;
-}
-
-// VEC: head_width % 4 == 0 and all rows 16-byte aligned -> float4 path
-template <bool VEC>
-__global__ void __launch_bounds__(kThreads) k_attention(const AttnArgs a) {
-    extern __shared__ __align__(16) float lds[];
-    const int hw = a.head_width;
-    float *s_q = lds;                      // [hw]
-    float *s_score = s_q + hw;             // [kAttnChunk]
-    float *s_red = s_score + kAttnChunk;   // [kPosPerPass][hw]
-    __shared__ float s_m, s_l;
-    __shared__ int s_last;
-
-    const int chunk = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
-    const int tid = threadIdx.x;
-    int valid, position;
+struct Resolved {
     const float *q;
     float *kc, *vc, *out;
+    int valid, position;
+};
+
+__device__ __forceinline__ Resolved resolve(const AttnArgs &a, int b) {
+    Resolved r;
     if (a.slots != nullptr) {
         const StepSlots *s = a.slots;
         if (a.is_self) {
-            position = s->length[b];
-            valid = position + 1;
-            kc = s->self_k[b] + a.layer * a.capacity * (size_t)a.stride;
-            vc = s->self_v[b] + a.layer * a.capacity * (size_t)a.stride;
+            r.position = s->length[b];
+            r.valid = r.position + 1;
+            r.kc = s->self_k[b] + a.layer * a.capacity * (size_t)a.stride;
+            r.vc = s->self_v[b] + a.layer * a.capacity * (size_t)a.stride;
         } else {
-            position = -1;
-            valid = s->memory_length[b];
-            kc = const_cast<float *>(s->cross_k[b]) + a.layer * (size_t)valid * a.stride;
-            vc = const_cast<float *>(s->cross_v[b]) + a.layer * (size_t)valid * a.stride;
+            r.position = -1;
+            r.valid = s->memory_length[b];
+            r.kc = const_cast<float *>(s->cross_k[b]) + a.layer * (size_t)r.valid * a.stride;
+            r.vc = const_cast<float *>(s->cross_v[b]) + a.layer * (size_t)r.valid * a.stride;
         }
-        q = a.q[0] + (size_t)b * a.q_stride;
-        out = a.out[0] + (size_t)b * (a.heads * hw);
+        r.q = a.q[0] + (size_t)b * a.q_stride;
+        r.out = a.out[0] + (size_t)b * (a.heads * a.head_width);
     } else {
-        position = a.is_self ? a.position[b] : -1;
-        valid = a.valid[b];
-        q = a.q[b];
-        kc = a.k_cache[b];
-        vc = a.v_cache[b];
-        out = a.out[b];
+        r.position = a.is_self ? a.position[b] : -1;
+        r.valid = a.valid[b];
+        r.q = a.q[b];
+        r.kc = a.k_cache[b];
+        r.vc = a.v_cache[b];
+        r.out = a.out[b];
     }
-    const int nchunks = valid > 0 ? (valid + kAttnChunk - 1) / kAttnChunk : 1;
-    if (chunk >= nchunks) return;
+    return r;
+}
 
-    const int width = a.heads * hw;
-    const float *qh = q + (size_t)head * hw;
-    const float *knew = q + width + (size_t)head * hw;       // self only
-    const float *vnew = q + 2 * (size_t)width + (size_t)head * hw;
-    float *outh = out + (size_t)head * hw;
-
-    if (valid <= 0) {   // empty memory: the reference leaves the context at zero (src/graph.c:3242)
-        for (int d = tid; d < hw; d += kThreads) outh[d] = 0.0f;
-        return;
+// Softmax statistics of one chunk: s_score[0..63] holds scaled scores (-3e38 beyond `count`);
+// afterwards it holds exp(score - max), and (max, sum) are in s_ml.
+__device__ __forceinline__ void chunk_stats(float *s_score, float *s_ml, int count) {
+    if (threadIdx.x < 64) {
+        const float sc = s_score[threadIdx.x];
+        const float m = wave_max(sc);
+        const float e = (int)threadIdx.x < count ? expf(sc - m) : 0.0f;
+        const float l = wave_sum(e);
+        s_score[threadIdx.x] = e;
+        if (threadIdx.x == 0) { s_ml[0] = m; s_ml[1] = l; }
     }
+}
 
-    for (int d = tid; d < hw; d += kThreads) s_q[d] = qh[d];
-    __syncthreads();
-
-    const int p0 = chunk * kAttnChunk;
-    const int count = min(kAttnChunk, valid - p0);
-    const int j = tid & (kPosLanes - 1);     // lane inside the row group
-    const int g = tid / kPosLanes;           // row group 0..15
-
-    // ---- scores
-    for (int pi = g; pi < kAttnChunk; pi += kPosPerPass) {
-        const int p = p0 + pi;
-        const bool in_range = pi < count;
-        const bool fresh = in_range && p == position;
-        const float *krow = fresh ? knew : kc + (size_t)p * a.stride + (size_t)head * hw;
-        float dot = 0.0f;
-        if (in_range) {
-            if constexpr (VEC) {
-                for (int d = 4 * j; d < hw; d += 4 * kPosLanes) {
-                    const float4 kv = *reinterpret_cast<const float4 *>(krow + d);
-                    const float4 qv = *reinterpret_cast<const float4 *>(s_q + d);
-                    dot = __builtin_fmaf(qv.x, kv.x, dot);
-                    dot = __builtin_fmaf(qv.y, kv.y, dot);
-                    dot = __builtin_fmaf(qv.z, kv.z, dot);
-                    dot = __builtin_fmaf(qv.w, kv.w, dot);
-                    if (fresh) *reinterpret_cast<float4 *>(kc + (size_t)p * a.stride + (size_t)head * hw + d) = kv;
-                }
-            } else {
-                for (int d = j; d < hw; d += kPosLanes) {
-                    const float kv = krow[d];
-                    dot = __builtin_fmaf(s_q[d], kv, dot);
-                    if (fresh) kc[(size_t)p * a.stride + (size_t)head * hw + d] = kv;
-                }
-            }
-        }
-        dot = group16_sum(dot);
-        if (j == 0) s_score[pi] = in_range ? dot * a.scale : -3.0e38f;
-    }
-    __syncthreads();
-
-    // ---- chunk softmax statistics (one wave, 64 scores)
-    if (tid < 64) {
-        const float sc = s_score[tid];
-        float m = sc;
-#pragma unroll
-        for (int x = 32; x > 0; x >>= 1) m = fmaxf(m, __shfl_xor(m, x));
-        const float e = tid < count ? expf(sc - m) : 0.0f;
-        float l = e;
-#pragma unroll
-        for (int x = 32; x > 0; x >>= 1) l += __shfl_xor(l, x);
-        s_score[tid] = e;
-        if (tid == 0) { s_m = m; s_l = l; }
-    }
-    __syncthreads();
-
-    // ---- weighted sum of V rows: each row group accumulates its rows, then groups are folded in order
-    if constexpr (VEC) {
-        for (int d = 4 * j; d < hw; d += 4 * kPosLanes) {
-            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-            for (int pi = g; pi < count; pi += kPosPerPass) {
-                const int p = p0 + pi;
-                const bool fresh = p == position;
-                const float *vrow = fresh ? vnew : vc + (size_t)p * a.stride + (size_t)head * hw;
-                const float4 vv = *reinterpret_cast<const float4 *>(vrow + d);
-                const float e = s_score[pi];
-                acc.x = __builtin_fmaf(e, vv.x, acc.x);
-                acc.y = __builtin_fmaf(e, vv.y, acc.y);
-                acc.z = __builtin_fmaf(e, vv.z, acc.z);
-                acc.w = __builtin_fmaf(e, vv.w, acc.w);
-                if (fresh) *reinterpret_cast<float4 *>(vc + (size_t)p * a.stride + (size_t)head * hw + d) = vv;
-            }
-            *reinterpret_cast<float4 *>(s_red + (size_t)g * hw + d) = acc;
-        }
-    } else {
-        for (int d = j; d < hw; d += kPosLanes) {
-            float acc = 0.0f;
-            for (int pi = g; pi < count; pi += kPosPerPass) {
-                const int p = p0 + pi;
-                const bool fresh = p == position;
-                const float vv = fresh ? vnew[d] : vc[(size_t)p * a.stride + (size_t)head * hw + d];
-                acc = __builtin_fmaf(s_score[pi], vv, acc);
-                if (fresh) vc[(size_t)p * a.stride + (size_t)head * hw + d] = vv;
-            }
-            s_red[(size_t)g * hw + d] = acc;
-        }
-    }
-    __syncthreads();
-
-    const float m_c = s_m, l_c = s_l;
-    if (nchunks == 1) {
-        for (int d = tid; d < hw; d += kThreads) {
-            float o = 0.0f;
-#pragma unroll
-            for (int gg = 0; gg < kPosPerPass; ++gg) o += s_red[(size_t)gg * hw + d];
-            outh[d] = o / l_c;
-        }
-        return;
-    }
-
-    // ---- several chunks: publish the partial, the last arrival folds them
+// Publishes this chunk's (max, sum, partial output) and lets the last arrival of the (stream, head)
+// fold all chunks: out = sum_c o_c e^(m_c - M) / sum_c l_c e^(m_c - M), chunks taken in four interleaved
+// sequences (c = g, g+4, ...) that are then added in order g = 0..3 -- fixed, whoever folds.
+__device__ __forceinline__ void publish_and_fold(const AttnArgs &a, int b, int head, int chunk, int nchunks, int hw,
+                                                 const float *s_red, float m_c, float l_c, float *outh, float *s_w,
+                                                 float *s_fold, int *s_last) {
+    const int tid = threadIdx.x;
     const size_t pstride = (size_t)hw + 2;
     float *part = a.partial + (((size_t)b * a.heads + head) * a.max_chunks) * pstride;
     float *mine = part + (size_t)chunk * pstride;
@@ -192,56 +91,280 @@ __global__ void __launch_bounds__(kThreads) k_attention(const AttnArgs a) {
         mine[2 + d] = o;
     }
     if (tid == 0) { mine[0] = m_c; mine[1] = l_c; }
-    __threadfence();
-    __syncthreads();
+    __syncthreads();   // every store of this workgroup has reached the L2 (workgroup-scope release) ...
     if (tid == 0) {
+        __threadfence();   // ... and one device-scope release publishes them: a fence per wave would serialise hundreds of L2 write-backs
         unsigned *counter = a.counters + (size_t)b * a.heads + head;
         const unsigned before = atomicAdd(counter, 1u);
-        s_last = (before == (unsigned)(nchunks - 1)) ? 1 : 0;
-        if (s_last) *counter = 0u;   // every other chunk has already arrived: ready for the next launch
+        const int last = (before == (unsigned)(nchunks - 1)) ? 1 : 0;
+        if (last) *counter = 0u;   // every other chunk has already arrived: ready for the next launch
+        *s_last = last;
     }
     __syncthreads();
-    if (!s_last) return;
-    __threadfence();
+    if (!*s_last) return;
+    __threadfence();   // acquire: the partials below are read with ordinary loads
 
+    // s_w[c] = m_c, s_w[max_chunks + c] = l_c
+    for (int c = tid; c < nchunks; c += kThreads) {
+        s_w[c] = part[(size_t)c * pstride];
+        s_w[a.max_chunks + c] = part[(size_t)c * pstride + 1];
+    }
+    __syncthreads();
     float M = -3.0e38f;
-    for (int c = 0; c < nchunks; ++c) M = fmaxf(M, __hip_atomic_load(part + (size_t)c * pstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    for (int c = 0; c < nchunks; ++c) M = fmaxf(M, s_w[c]);
+    __syncthreads();
+    for (int c = tid; c < nchunks; c += kThreads) s_w[c] = expf(s_w[c] - M);
+    __syncthreads();
     float L = 0.0f;
-    for (int c = 0; c < nchunks; ++c) {
-        const float mc = __hip_atomic_load(part + (size_t)c * pstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const float lc = __hip_atomic_load(part + (size_t)c * pstride + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        L = __builtin_fmaf(lc, expf(mc - M), L);
-    }
-    for (int d = tid; d < hw; d += kThreads) {
+    for (int c = 0; c < nchunks; ++c) L = __builtin_fmaf(s_w[a.max_chunks + c], s_w[c], L);
+
+    const int gsize = hw <= 64 ? 64 : (hw <= 128 ? 128 : 256);
+    const int ngroups = kThreads / gsize;
+    const int g = tid / gsize;
+    for (int d0 = 0; d0 < hw; d0 += gsize) {
+        const int d = d0 + (tid % gsize);
         float o = 0.0f;
-        for (int c = 0; c < nchunks; ++c) {
-            const float mc = __hip_atomic_load(part + (size_t)c * pstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const float oc = __hip_atomic_load(part + (size_t)c * pstride + 2 + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            o = __builtin_fmaf(oc, expf(mc - M), o);
+        if (d < hw)
+            for (int c = g; c < nchunks; c += ngroups) o = __builtin_fmaf(part[(size_t)c * pstride + 2 + d], s_w[c], o);
+        s_fold[tid] = o;
+        __syncthreads();
+        if (g == 0 && d < hw) {
+            float total = s_fold[tid];
+            for (int gg = 1; gg < ngroups; ++gg) total += s_fold[gg * gsize + tid];
+            outh[d] = total / L;
         }
-        outh[d] = o / L;
+        __syncthreads();
     }
+}
+
+// ------------------------------------------------------------------------------------------------
+// head_width == 64, aligned rows: everything prefetched, no LDS staging of q.
+__global__ void __launch_bounds__(kThreads) k_attention_hw64(const AttnArgs a) {
+    extern __shared__ __align__(16) float lds[];
+    float *s_score = lds;                     // [64]
+    float *s_red = s_score + kAttnChunk;      // [16][64]
+    float *s_w = s_red + kPosPerPass * 64;    // [2 * max_chunks]
+    float *s_fold = s_w + 2 * a.max_chunks;   // [256]
+    __shared__ float s_ml[2];
+    __shared__ int s_last;
+    constexpr int hw = 64;
+
+    const int chunk = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const Resolved r = resolve(a, b);
+    const int nchunks = r.valid > 0 ? (r.valid + kAttnChunk - 1) / kAttnChunk : 1;
+    if (chunk >= nchunks) return;
+    const int width = a.heads * hw;
+    float *outh = r.out + (size_t)head * hw;
+    if (r.valid <= 0) {   // empty memory: the reference leaves the context at zero (src/graph.c:3242)
+        if (tid < hw) outh[tid] = 0.0f;
+        return;
+    }
+    const int p0 = chunk * kAttnChunk;
+    const int count = min(kAttnChunk, r.valid - p0);
+    const int j = tid & (kPosLanes - 1);
+    const int g = tid / kPosLanes;
+    const size_t col = (size_t)head * hw + 4 * j;
+
+    // ---- every load this workgroup needs, issued before anything is consumed
+    const float4 qv = *reinterpret_cast<const float4 *>(r.q + col);
+    float4 kv[kRowsPerThread], vv[kRowsPerThread];
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; ++i) {
+        const int pi = g + kPosPerPass * i;
+        const int p = p0 + pi;
+        const bool in_range = pi < count;
+        const bool fresh = in_range && p == r.position;
+        const float *krow = fresh ? r.q + width + col : r.kc + (size_t)p * a.stride + col;
+        const float *vrow = fresh ? r.q + 2 * (size_t)width + col : r.vc + (size_t)p * a.stride + col;
+        kv[i] = in_range ? *reinterpret_cast<const float4 *>(krow) : make_float4(0.f, 0.f, 0.f, 0.f);
+        vv[i] = in_range ? *reinterpret_cast<const float4 *>(vrow) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    // ---- scores (+ append of the new row)
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; ++i) {
+        const int pi = g + kPosPerPass * i;
+        const int p = p0 + pi;
+        const bool in_range = pi < count;
+        float dot = 0.0f;
+        dot = __builtin_fmaf(qv.x, kv[i].x, dot);
+        dot = __builtin_fmaf(qv.y, kv[i].y, dot);
+        dot = __builtin_fmaf(qv.z, kv[i].z, dot);
+        dot = __builtin_fmaf(qv.w, kv[i].w, dot);
+        dot = row16_sum(dot);
+        if (j == 0) s_score[pi] = in_range ? dot * a.scale : -3.0e38f;
+        if (in_range && p == r.position) {
+            *reinterpret_cast<float4 *>(r.kc + (size_t)p * a.stride + col) = kv[i];
+            *reinterpret_cast<float4 *>(r.vc + (size_t)p * a.stride + col) = vv[i];
+        }
+    }
+    __syncthreads();
+    chunk_stats(s_score, s_ml, count);
+    __syncthreads();
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; ++i) {
+        const float e = s_score[g + kPosPerPass * i];   // 0 beyond `count`
+        acc.x = __builtin_fmaf(e, vv[i].x, acc.x);
+        acc.y = __builtin_fmaf(e, vv[i].y, acc.y);
+        acc.z = __builtin_fmaf(e, vv[i].z, acc.z);
+        acc.w = __builtin_fmaf(e, vv[i].w, acc.w);
+    }
+    *reinterpret_cast<float4 *>(s_red + (size_t)g * hw + 4 * j) = acc;
+    __syncthreads();
+    const float m_c = s_ml[0], l_c = s_ml[1];
+    if (nchunks == 1) {
+        if (tid < hw) {
+            float o = 0.0f;
+#pragma unroll
+            for (int gg = 0; gg < kPosPerPass; ++gg) o += s_red[(size_t)gg * hw + tid];
+            outh[tid] = o / l_c;
+        }
+        return;
+    }
+    publish_and_fold(a, b, head, chunk, nchunks, hw, s_red, m_c, l_c, outh, s_w, s_fold, &s_last);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Any head width (the engine passes one 768-wide head for cross attention, src/graph.c:3443-3448;
+// self-test shapes are 2 wide).  VEC: head_width % 4 == 0 and all rows 16-byte aligned.
+template <bool VEC>
+__global__ void __launch_bounds__(kThreads) k_attention_any(const AttnArgs a) {
+    extern __shared__ __align__(16) float lds[];
+    const int hw = a.head_width;
+    float *s_q = lds;                           // [hw]
+    float *s_score = s_q + hw;                  // [64]
+    float *s_red = s_score + kAttnChunk;        // [16][hw]
+    float *s_w = s_red + (size_t)kPosPerPass * hw;   // [2 * max_chunks]
+    float *s_fold = s_w + 2 * a.max_chunks;     // [256]
+    __shared__ float s_ml[2];
+    __shared__ int s_last;
+
+    const int chunk = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x;
+    const Resolved r = resolve(a, b);
+    const int nchunks = r.valid > 0 ? (r.valid + kAttnChunk - 1) / kAttnChunk : 1;
+    if (chunk >= nchunks) return;
+    const int width = a.heads * hw;
+    const float *qh = r.q + (size_t)head * hw;
+    const float *knew = r.q + width + (size_t)head * hw;
+    const float *vnew = r.q + 2 * (size_t)width + (size_t)head * hw;
+    float *outh = r.out + (size_t)head * hw;
+    if (r.valid <= 0) {
+        for (int d = tid; d < hw; d += kThreads) outh[d] = 0.0f;
+        return;
+    }
+    for (int d = tid; d < hw; d += kThreads) s_q[d] = qh[d];
+    __syncthreads();
+
+    const int p0 = chunk * kAttnChunk;
+    const int count = min(kAttnChunk, r.valid - p0);
+    const int j = tid & (kPosLanes - 1);
+    const int g = tid / kPosLanes;
+
+    for (int pi = g; pi < kAttnChunk; pi += kPosPerPass) {
+        const int p = p0 + pi;
+        const bool in_range = pi < count;
+        const bool fresh = in_range && p == r.position;
+        const float *krow = fresh ? knew : r.kc + (size_t)p * a.stride + (size_t)head * hw;
+        float dot = 0.0f;
+        if (in_range) {
+            if constexpr (VEC) {
+                for (int d = 4 * j; d < hw; d += 4 * kPosLanes) {
+                    const float4 kv = *reinterpret_cast<const float4 *>(krow + d);
+                    const float4 qv = *reinterpret_cast<const float4 *>(s_q + d);
+                    dot = __builtin_fmaf(qv.x, kv.x, dot);
+                    dot = __builtin_fmaf(qv.y, kv.y, dot);
+                    dot = __builtin_fmaf(qv.z, kv.z, dot);
+                    dot = __builtin_fmaf(qv.w, kv.w, dot);
+                    if (fresh) *reinterpret_cast<float4 *>(r.kc + (size_t)p * a.stride + (size_t)head * hw + d) = kv;
+                }
+            } else {
+                for (int d = j; d < hw; d += kPosLanes) {
+                    const float kv = krow[d];
+                    dot = __builtin_fmaf(s_q[d], kv, dot);
+                    if (fresh) r.kc[(size_t)p * a.stride + (size_t)head * hw + d] = kv;
+                }
+            }
+        }
+        dot = row16_sum(dot);
+        if (j == 0) s_score[pi] = in_range ? dot * a.scale : -3.0e38f;
+    }
+    __syncthreads();
+    chunk_stats(s_score, s_ml, count);
+    __syncthreads();
+
+    if constexpr (VEC) {
+        for (int d = 4 * j; d < hw; d += 4 * kPosLanes) {
+            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int pi = g; pi < count; pi += kPosPerPass) {
+                const int p = p0 + pi;
+                const bool fresh = p == r.position;
+                const float *vrow = fresh ? vnew : r.vc + (size_t)p * a.stride + (size_t)head * hw;
+                const float4 vv = *reinterpret_cast<const float4 *>(vrow + d);
+                const float e = s_score[pi];
+                acc.x = __builtin_fmaf(e, vv.x, acc.x);
+                acc.y = __builtin_fmaf(e, vv.y, acc.y);
+                acc.z = __builtin_fmaf(e, vv.z, acc.z);
+                acc.w = __builtin_fmaf(e, vv.w, acc.w);
+                if (fresh) *reinterpret_cast<float4 *>(r.vc + (size_t)p * a.stride + (size_t)head * hw + d) = vv;
+            }
+            *reinterpret_cast<float4 *>(s_red + (size_t)g * hw + d) = acc;
+        }
+    } else {
+        for (int d = j; d < hw; d += kPosLanes) {
+            float acc = 0.0f;
+            for (int pi = g; pi < count; pi += kPosPerPass) {
+                const int p = p0 + pi;
+                const bool fresh = p == r.position;
+                const float vv = fresh ? vnew[d] : r.vc[(size_t)p * a.stride + (size_t)head * hw + d];
+                acc = __builtin_fmaf(s_score[pi], vv, acc);
+                if (fresh) r.vc[(size_t)p * a.stride + (size_t)head * hw + d] = vv;
+            }
+            s_red[(size_t)g * hw + d] = acc;
+        }
+    }
+    __syncthreads();
+
+    const float m_c = s_ml[0], l_c = s_ml[1];
+    if (nchunks == 1) {
+        for (int d = tid; d < hw; d += kThreads) {
+            float o = 0.0f;
+#pragma unroll
+            for (int gg = 0; gg < kPosPerPass; ++gg) o += s_red[(size_t)gg * hw + d];
+            outh[d] = o / l_c;
+        }
+        return;
+    }
+    publish_and_fold(a, b, head, chunk, nchunks, hw, s_red, m_c, l_c, outh, s_w, s_fold, &s_last);
 }
 
 }  // namespace
 
 int launch_attention(State *st, const AttnArgs &a, char *error, size_t capacity) {
     if (a.batch < 1 || a.batch > kMaxBatch || a.heads < 1 || a.head_width < 1 || a.head_width > 1024 ||
-        a.max_chunks < 1 || a.partial == nullptr || a.counters == nullptr) {
+        a.max_chunks < 1 || a.max_chunks > 4096 || a.partial == nullptr || a.counters == nullptr) {
         set_error(error, capacity, "attention: invalid shape");
         return -1;
     }
-    const size_t lds = ((size_t)a.head_width * (1 + kPosPerPass) + kAttnChunk) * sizeof(float);
     const bool vec = (a.head_width % 4) == 0 && (a.stride % 4) == 0 && (a.q_stride % 4) == 0;
+    const bool fast = vec && a.head_width == 64;
+    const size_t hw = (size_t)a.head_width;
+    const size_t lds = ((fast ? 0 : hw) + kAttnChunk + (size_t)kPosPerPass * hw + 2 * (size_t)a.max_chunks + kThreads) * sizeof(float);
     const dim3 grid((unsigned)a.max_chunks, (unsigned)a.heads, (unsigned)a.batch);
     static bool raised[2] = {false, false};
-    if (lds > 48 * 1024 && !raised[vec ? 1 : 0]) {
-        const void *fn = vec ? reinterpret_cast<const void *>(&k_attention<true>) : reinterpret_cast<const void *>(&k_attention<false>);
-        MYNAH_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    if (lds > 48 * 1024 && !fast && !raised[vec ? 1 : 0]) {
+        const void *fn = vec ? reinterpret_cast<const void *>(&k_attention_any<true>) : reinterpret_cast<const void *>(&k_attention_any<false>);
+        MYNAH_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised[vec ? 1 : 0] = true;
     }
-    if (vec) hipLaunchKernelGGL(k_attention<true>, grid, dim3(kThreads), lds, st->stream, a);
-    else hipLaunchKernelGGL(k_attention<false>, grid, dim3(kThreads), lds, st->stream, a);
+    if (lds > 128 * 1024) {
+        set_error(error, capacity, "attention: head width and cache length exceed the workgroup's LDS");
+        return -1;
+    }
+    if (fast) hipLaunchKernelGGL(k_attention_hw64, grid, dim3(kThreads), lds, st->stream, a);
+    else if (vec) hipLaunchKernelGGL(k_attention_any<true>, grid, dim3(kThreads), lds, st->stream, a);
+    else hipLaunchKernelGGL(k_attention_any<false>, grid, dim3(kThreads), lds, st->stream, a);
     return hip_check(hipGetLastError(), "attention launch", error, capacity);
 }
 

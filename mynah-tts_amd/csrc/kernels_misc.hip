@@ -2,21 +2,10 @@
 // argmax, embedding gather, and the begin/end kernels of the resident decode step.
 #include <float.h>
 
-#include "kernels.h"
+#include "device_common.h"
 
 namespace mynah {
 namespace {
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
-    return v;
-}
 
 // Sum over a 256-thread workgroup in a fixed order: lanes by butterfly, then waves 0..3.
 __device__ __forceinline__ float block_sum(float v, float *s4) {
