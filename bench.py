@@ -113,6 +113,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--skip-b8", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run the library's plain read+write kernel over 256 MiB three times (a known-size reference for "
+                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: the decode step has no multi-GPU form (streams shard by request, with no "
@@ -125,6 +128,10 @@ def main():
     backend = pkg.Backend(quant=qtype)
     if args.no_graph:
         backend.set_graph_mode(False)
+    if args.calibrate:
+        for _ in range(3):
+            backend.flush_cache(256 << 20)
+        backend.sync()
 
     b1 = time_config(pkg, synth, backend, qtype, [1023], [256], 1024, args.steps, args.warmup)
     b8 = None

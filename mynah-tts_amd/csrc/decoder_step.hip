@@ -117,6 +117,10 @@ static int enqueue_attention(State *st, const mynah_hip_decoder *d, int is_self,
     return launch_attention(st, a, error, capacity);
 }
 
+// Up to this many streams the output projection folds the attention partials itself; above it a separate fold
+// kernel runs once (every workgroup folding every stream would outweigh one extra launch).
+constexpr int kConsumerFoldMaxBatch = 2;
+
 static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_self, size_t layer, int batch, const CachedWeight *w,
                                   const float *ln_gain, const float *ln_bias, char *error, size_t capacity) {
     StepAttnArgs a{};
@@ -139,7 +143,9 @@ static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_
     a.scale = 1.0f / sqrtf((float)a.head_width);
     a.partial = d->partial;
     a.partial_ml = d->partial_ml;
-    return launch_step_attention(st, a, error, capacity);
+    if (launch_step_attention(st, a, error, capacity) != 0) return -1;
+    if (batch > kConsumerFoldMaxBatch) return launch_step_fold(st, a, is_self ? d->attn : d->ctx, error, capacity);
+    return 0;
 }
 
 // The layer loop; everything here is replayable (no per-step scalars in kernel arguments).
@@ -149,10 +155,11 @@ static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char
         for (size_t l = 0; l < d->layers; ++l) {
             const LayerWeights &lw = d->lw[l];
             if (enqueue_step_attention(st, d, 1, l, batch, lw.qkv, lw.norm_self, lw.norm_self_b, error, capacity) != 0) return -1;
-            if (enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, 1) != 0) return -1;
+            const bool consumer_fold = batch <= kConsumerFoldMaxBatch;
+            if (enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 1 : 0) != 0) return -1;
             if (d->xw != 0) {
                 if (enqueue_step_attention(st, d, 0, l, batch, lw.q_cross, lw.norm_cross, lw.norm_cross_b, error, capacity) != 0) return -1;
-                if (enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, 2) != 0) return -1;
+                if (enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 2 : 0) != 0) return -1;
             }
             if (enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity) != 0) return -1;
             if (enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;

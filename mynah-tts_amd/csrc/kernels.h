@@ -84,6 +84,8 @@ struct StepAttnArgs {
     float *partial_ml;        // chunk maxima and sums [batch, heads, 2, max_units]
 };
 int launch_step_attention(State *st, const StepAttnArgs &args, char *error, size_t capacity);
+// Folds the partials of the same arguments into out[batch][heads * head_width] (large batches only).
+int launch_step_fold(State *st, const StepAttnArgs &args, float *out, char *error, size_t capacity);
 bool step_attention_supported(int qtype, size_t width, size_t heads, size_t head_width);
 
 int launch_layernorm(State *st, const float *in, float *out, const float *gain, const float *bias, size_t rows,

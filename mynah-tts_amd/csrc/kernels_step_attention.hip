@@ -211,14 +211,23 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         if (j == 0) s_score[pi] = pi < count ? dot * a.scale : -3.0e38f;
     }
     __syncthreads();
-    if (tid < 64) {   // 128 scores: two per lane
-        const float s0 = s_score[tid], s1 = s_score[tid + 64];
-        const float m = wave_max(fmaxf(s0, s1));
-        const float e0 = tid < count ? expf(s0 - m) : 0.0f;
-        const float e1 = tid + 64 < count ? expf(s1 - m) : 0.0f;
-        const float l = wave_sum(e0 + e1);
-        s_score[tid] = e0;
-        s_score[tid + 64] = e1;
+    if (tid < 64) {   // kStepUnitRows scores, kStepUnitRows / 64 per lane
+        constexpr int kPerLane = kStepUnitRows / 64;
+        float sc[kPerLane], m = -3.0e38f;
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i) {
+            sc[i] = s_score[tid + 64 * i];
+            m = fmaxf(m, sc[i]);
+        }
+        m = wave_max(m);
+        float l = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kPerLane; ++i) {
+            const float e = tid + 64 * i < count ? expf(sc[i] - m) : 0.0f;
+            s_score[tid + 64 * i] = e;
+            l += e;
+        }
+        l = wave_sum(l);
         if (tid == 0) { s_ml[0] = m; s_ml[1] = l; }
     }
     __syncthreads();
@@ -240,6 +249,20 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         out_o[tid] = o;
         if (tid == 0) { out_m[unit] = s_ml[0]; out_l[unit] = s_ml[1]; }
     }
+}
+
+// Stand-alone fold of the partials into out[stream][heads * 64]: used instead of the consumer-side fold when
+// the batch is large enough that every workgroup of the output projection folding every stream would cost more
+// than one extra launch.  Same arithmetic (fold_partials), so the result does not depend on which path ran.
+__global__ void __launch_bounds__(kThreads) k_step_fold(const float *partial, const float *partial_ml, const StepSlots *slots, int heads,
+                                                        int max_units, int is_self, float *out) {
+    const int stream = blockIdx.y;
+    const int f4 = blockIdx.x * kThreads + threadIdx.x;
+    if (f4 >= heads * (kHw / 4)) return;
+    ActSource src;
+    src.partial = partial; src.partial_ml = partial_ml; src.slots = slots; src.heads = heads; src.head_width = kHw;
+    src.max_units = max_units; src.is_self = is_self; src.stream0 = 0;
+    reinterpret_cast<float4 *>(out + (size_t)stream * heads * kHw)[f4] = fold_partials(src, stream, f4);
 }
 
 template <int QT>
@@ -264,6 +287,13 @@ bool step_attention_supported(int qtype, size_t width, size_t heads, size_t head
     const int chunks = (int)width / epc;
     const int group = 1 << lane_group_log2(chunks);
     return (chunks + group - 1) / group <= 4;   // one register group of four chunks per lane and pass
+}
+
+int launch_step_fold(State *st, const StepAttnArgs &a, float *out, char *error, size_t capacity) {
+    const int f4 = a.heads * (kHw / 4);
+    const dim3 grid((unsigned)((f4 + kThreads - 1) / kThreads), (unsigned)a.batch);
+    hipLaunchKernelGGL(k_step_fold, grid, dim3(kThreads), 0, st->stream, a.partial, a.partial_ml, a.slots, a.heads, a.max_units, a.is_self, out);
+    return hip_check(hipGetLastError(), "step fold launch", error, capacity);
 }
 
 int launch_step_attention(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
