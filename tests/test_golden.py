@@ -1,0 +1,91 @@
+"""The oracle against the committed outputs of the compiled reference (tests/golden/reference_vectors.npz, written by
+tests/golden/make_golden.py).  These run wherever the reference tree itself is absent.
+
+Bars: integers and scales bit-exact; f32 results of the strict build within 1e-6 (normalised max error,
+max|a-b|/max|b|) -- the oracle is compiled with the same IEEE rules; the stock (-ffast-math) build within 1e-5.
+"""
+import os
+import zlib
+
+import numpy as np
+import pytest
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def gold():
+    return np.load(GOLDEN, allow_pickle=False)
+
+
+def _bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+@pytest.mark.parametrize("tag", ["stock", "strict"])
+def test_quantisers_bit_exact(orc, gold, tag):
+    variant = orc.STOCK if tag == "stock" else orc.STRICT
+    w = gold["quant_w"]
+    q8, s8 = orc.quantize_weight_int8(w, variant)
+    assert np.array_equal(q8, gold["quant_%s_q8" % tag])
+    assert np.array_equal(_bits(s8), _bits(gold["quant_%s_s8" % tag]))
+    q4, s4 = orc.quantize_weight_int4(w, variant)
+    assert np.array_equal(q4, gold["quant_%s_q4" % tag])
+    assert np.array_equal(_bits(s4).reshape(-1), _bits(gold["quant_%s_s4" % tag]).reshape(-1))
+    qx, sx = orc.quantize_act_int8(gold["quant_x"], variant)
+    assert np.array_equal(qx, gold["quant_%s_qx" % tag])
+    assert _bits(np.float32(sx)) == _bits(gold["quant_%s_sx" % tag])
+    for i in range(w.shape[0]):
+        qr, sr = orc.quantize_act_int8(w[i], variant)
+        assert np.array_equal(qr, gold["quant_%s_qrows" % tag][i]), "row %d" % i
+        assert _bits(np.float32(sr)) == _bits(gold["quant_%s_srows" % tag][i]), "row %d" % i
+
+
+@pytest.mark.parametrize("tag", ["stock", "strict"])
+def test_integer_matvecs(orc, gold, nerr, tag):
+    qx, sx, bias = gold["quant_%s_qx" % tag], float(gold["quant_%s_sx" % tag]), gold["quant_bias"]
+    y8, _ = orc.matvec_q8(qx, sx, gold["quant_%s_q8" % tag], gold["quant_%s_s8" % tag], bias)
+    y4, _ = orc.matvec_q4(qx, sx, gold["quant_%s_q4" % tag], gold["quant_%s_s4" % tag], bias)
+    if tag == "strict":      # same IEEE rules, same formula order: the f32 epilogue reproduces bit for bit
+        assert np.array_equal(_bits(y8), _bits(gold["quant_strict_y8"]))
+        assert np.array_equal(_bits(y4), _bits(gold["quant_strict_y4"]))
+    else:
+        assert nerr(y8, gold["quant_stock_y8"]) < 1e-6
+        assert nerr(y4, gold["quant_stock_y4"]) < 1e-6
+
+
+def test_layernorm_gelu_softmax(orc, gold, nerr):
+    x = gold["kern_x"]
+    for r in range(x.shape[0]):
+        assert nerr(orc.layernorm(x[r], gold["kern_gain"], gold["kern_beta"]), gold["kern_layernorm"][r]) < 1e-6
+    assert nerr(orc.gelu_scalar(x.reshape(-1)), gold["kern_gelu"].reshape(-1)) < 1e-6
+    rc, sm = orc.softmax(x[0])
+    assert rc == 0 and nerr(sm, gold["kern_softmax"]) < 1e-6
+
+
+@pytest.mark.parametrize("qname", ["f32", "int8", "int4"])
+@pytest.mark.parametrize("tag", ["stock", "strict"])
+def test_decode_step(orc, synth, gold, nerr, qname, tag):
+    lengths = [int(n) for n in gold["step_lengths"]]
+    mems = [int(n) for n in gold["step_mems"]]
+    cfg = synth.decoder_config(layers=2, capacity=max(lengths) + 3, cross_heads=1)
+    weights = synth.decoder_weights(cfg, seed=0, ln_bias=False)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=1)
+    c = 0
+    for a in [weights[k] for k in sorted(weights) if weights[k] is not None] + \
+             [s[n] for s in streams for n in ("k", "v", "ck", "cv", "x")]:
+        c = zlib.crc32(np.ascontiguousarray(a).tobytes(), c)
+    if np.uint32(c) != gold["step_input_crc"]:
+        pytest.skip("numpy's generator produced different synthetic inputs than when the fixture was written")
+    qtype = {"f32": orc.F32, "int8": orc.INT8, "int4": orc.INT4}[qname]
+    dec = orc.Decoder(cfg, weights, qtype, orc.STOCK if tag == "stock" else orc.STRICT)
+    ks = [s["k"].copy() for s in streams]
+    vs = [s["v"].copy() for s in streams]
+    outs = dec.step(ks, vs, [s["ck"] for s in streams], [s["cv"] for s in streams], lengths, mems, [s["x"] for s in streams])
+    # f32: 1e-5.  Quantised: identical packed weights on both sides, but a last-bit LayerNorm difference can flip
+    # one int8 activation by 1, which moves an output by up to ~1e-3 of its vector's scale.
+    tol = 1e-5 if qname == "f32" else 5e-3
+    for b in range(len(lengths)):
+        assert nerr(outs[b], gold["step_%s_%s_out" % (qname, tag)][b]) < tol, "stream %d" % b
+        assert nerr(ks[b][:, lengths[b]], gold["step_%s_%s_newk" % (qname, tag)][b]) < tol
+        assert nerr(vs[b][:, lengths[b]], gold["step_%s_%s_newv" % (qname, tag)][b]) < tol
