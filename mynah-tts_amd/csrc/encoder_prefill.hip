@@ -1,17 +1,454 @@
-// Text-encoder prefill on the matrix cores (placeholder translation unit: filled in below).
-#include "kernels.h"
-
-struct mynah_hip_encoder { int unused; };
+// Text-encoder prefill on the matrix cores: the dense, many-rows twin of the decode step.
+//
+// encode_text / transformer_stack (src/graph.c:713-748, :634-711) run, per layer, LayerNorm -> QKV
+// linear -> per-head scaled QK^T -> row softmax -> PV -> O -> residual -> LayerNorm -> FFN -> residual
+// through an f32 BLAS.  Here the weights are f16 (converted once at load, IEEE round to nearest even,
+// third_party/ingot/src/dtype.c:246-268), the activations entering a product are rounded to f16, and
+// every product accumulates in f32 on v_mfma_f32_32x32x16_f16.  The residual stream, the LayerNorm
+// statistics, the softmax and the GELU stay f32.  Bidirectional attention and the plain FFN
+// (kernel == 1 branch of causal_conv_ffn, src/graph.c:302-316).
+//
+// Layout in device memory (T tokens padded to a multiple of 64 rows; pad rows are kept finite and are
+// masked out as attention keys, so they never reach a real row):
+//   x    f32 [Tpad, w]       residual stream
+//   nrm  f16 [Tpad, w]       LayerNorm output = A operand of the QKV / FFN-up products
+//   qk   f16 [Tpad, 2w]      q | k of every token, row-major (K-contiguous operands of QK^T)
+//   vt   f16 [w, TpadMax]    v transposed: vt[h*64+d][t], so PV's B operand is K(=t)-contiguous too
+//   ctx  f16 [Tpad, w]       attention output = A operand of the O product
+//   hid  f16 [Tpad, ffn]     GELU(up) = A operand of the FFN-down product
+//
+// All products are "NT": C[m][n] = sum_k A[m][k] * W[n][k], both operands K-contiguous, which is how
+// the 32x32x16 MFMA wants them: lane l supplies row (l % 32) of A (or of W) and the eight consecutive
+// k values 8*(l / 32) .. +7 of the 16-deep step.
+#include "device_common.h"
 
 using namespace mynah;
 
-extern "C" int mynah_hip_encoder_create(void *, const mynah_hip_encoder_desc *, mynah_hip_encoder **out, char *error, size_t capacity) {
-    if (out != nullptr) *out = nullptr;
-    set_error(error, capacity, "encoder prefill is not available in this build");
-    return -1;
+struct mynah_hip_encoder {
+    size_t layers = 0, width = 0, heads = 0, head_width = 0, ffn = 0, vocab = 0, max_positions = 0, tpad_max = 0;
+    const CachedWeight *tok = nullptr, *pos = nullptr;
+    std::vector<const CachedWeight *> qkv, o, up, down;
+    std::vector<const float *> n1g, n1b, n2g, n2b;
+    const float *nog = nullptr, *nob = nullptr;
+    float *x = nullptr;
+    _Float16 *nrm = nullptr, *qk = nullptr, *vt = nullptr, *ctx = nullptr, *hid = nullptr;
+    int *ids = nullptr;
+    int *ids_host = nullptr;   // pinned
+    size_t max_lds = 0;
+};
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kTile = 64;            // workgroup tile of the products: 64 x 64, K step 64
+constexpr int kLdsStride = 72;       // halfs per staged row: 64 + 8 keeps 16-byte reads of 32 rows off each other's banks
+constexpr int kQTile = 32;           // queries per attention workgroup
+constexpr int kScorePad = 8;         // floats appended to a score row (bank spread for the row-wise softmax)
+
+enum { ENC_QKV = 0, ENC_RESIDUAL = 1, ENC_GELU = 2 };
+
+struct GemmArgs {
+    const _Float16 *a;     // [M, K] row-major, lda = K
+    const _Float16 *w;     // [N, K]
+    int M, N, K;
+    float *x;              // ENC_RESIDUAL: x[m][n] += c, ldx = N
+    _Float16 *out;         // ENC_QKV: qk [M, 2*width];  ENC_GELU: hid [M, N]
+    _Float16 *vt;          // ENC_QKV: v transposed [width, vt_stride]
+    int width, vt_stride;
+};
+
+// Row of C held in accumulator register r of lane l for a 32x32 MFMA tile; the column is l % 32.
+__device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+template <int EPI>
+__global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
+    __shared__ __align__(16) _Float16 s_a[2][kTile * kLdsStride];
+    __shared__ __align__(16) _Float16 s_w[2][kTile * kLdsStride];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+    const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
+    // staging: thread -> (row tid / 8 and + 32, 16-byte chunk tid % 8) of both tiles
+    const int srow = tid >> 3, schunk = tid & 7;
+    const uint4 *ga0 = reinterpret_cast<const uint4 *>(g.a + (size_t)(m0 + srow) * g.K) + schunk;
+    const uint4 *ga1 = reinterpret_cast<const uint4 *>(g.a + (size_t)(m0 + srow + 32) * g.K) + schunk;
+    const uint4 *gw0 = reinterpret_cast<const uint4 *>(g.w + (size_t)(n0 + srow) * g.K) + schunk;
+    const uint4 *gw1 = reinterpret_cast<const uint4 *>(g.w + (size_t)(n0 + srow + 32) * g.K) + schunk;
+    const int soff0 = srow * kLdsStride + schunk * 8, soff1 = (srow + 32) * kLdsStride + schunk * 8;
+
+    uint4 ra0 = ga0[0], ra1 = ga1[0], rw0 = gw0[0], rw1 = gw1[0];
+    *reinterpret_cast<uint4 *>(&s_a[0][soff0]) = ra0;
+    *reinterpret_cast<uint4 *>(&s_a[0][soff1]) = ra1;
+    *reinterpret_cast<uint4 *>(&s_w[0][soff0]) = rw0;
+    *reinterpret_cast<uint4 *>(&s_w[0][soff1]) = rw1;
+    __syncthreads();
+
+    floatx16 acc = {0};
+    const int nk = g.K / kTile;
+    const int frag = (lane & 31) * kLdsStride + 8 * (lane >> 5);
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) {   // next K step's tiles travel while this one is multiplied
+            const int step = (kt + 1) * (kTile / 8);
+            ra0 = ga0[step]; ra1 = ga1[step]; rw0 = gw0[step]; rw1 = gw1[step];
+        }
+        const _Float16 *pa = &s_a[cur][wm * 32 * kLdsStride + frag];
+        const _Float16 *pw = &s_w[cur][wn * 32 * kLdsStride + frag];
+#pragma unroll
+        for (int j = 0; j < kTile / 16; ++j) {
+            const half8 fa = *reinterpret_cast<const half8 *>(pa + 16 * j);
+            const half8 fw = *reinterpret_cast<const half8 *>(pw + 16 * j);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fw, acc, 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            const int nxt = cur ^ 1;   // last read one iteration ago, before the barrier that ended it
+            *reinterpret_cast<uint4 *>(&s_a[nxt][soff0]) = ra0;
+            *reinterpret_cast<uint4 *>(&s_a[nxt][soff1]) = ra1;
+            *reinterpret_cast<uint4 *>(&s_w[nxt][soff0]) = rw0;
+            *reinterpret_cast<uint4 *>(&s_w[nxt][soff1]) = rw1;
+        }
+        __syncthreads();
+    }
+
+    const int n = n0 + wn * 32 + (lane & 31);
+    const int mbase = m0 + wm * 32;
+    if constexpr (EPI == ENC_RESIDUAL) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float *p = g.x + (size_t)(mbase + acc_row(r, lane)) * g.N + n;
+            *p = *p + acc[r];
+        }
+    } else if constexpr (EPI == ENC_GELU) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) g.out[(size_t)(mbase + acc_row(r, lane)) * g.N + n] = (_Float16)gelu_tanh(acc[r]);
+    } else {
+        if (n < 2 * g.width) {   // uniform per workgroup: width is a multiple of the tile
+#pragma unroll
+            for (int r = 0; r < 16; ++r) g.out[(size_t)(mbase + acc_row(r, lane)) * (2 * g.width) + n] = (_Float16)acc[r];
+        } else {
+            _Float16 *col = g.vt + (size_t)(n - 2 * g.width) * g.vt_stride + mbase;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {   // registers 4q .. 4q+3 are four consecutive tokens
+                half4 v = {(_Float16)acc[4 * q], (_Float16)acc[4 * q + 1], (_Float16)acc[4 * q + 2], (_Float16)acc[4 * q + 3]};
+                *reinterpret_cast<half4 *>(col + 8 * q + 4 * (lane >> 5)) = v;
+            }
+        }
+    }
 }
-extern "C" void mynah_hip_encoder_destroy(void *, mynah_hip_encoder *) {}
-extern "C" int mynah_hip_encoder_prefill(void *, mynah_hip_encoder *, const int32_t *, size_t, uint16_t *, float *, char *error, size_t capacity) {
-    set_error(error, capacity, "encoder prefill is not available in this build");
-    return -1;
+
+// Token gather + position add (src/graph.c:729-737, :649-651).  Rows [tokens, tpad) are zeroed.
+__global__ void __launch_bounds__(kThreads) k_enc_embed(const int *ids, const _Float16 *tok, const _Float16 *pos, float *x,
+                                                        uint16_t *embed_out, int tokens, int width) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x * 8; c < width; c += kThreads * 8) {
+        float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
+        if (t < tokens) {
+            const uint4 traw = *reinterpret_cast<const uint4 *>(tok + (size_t)ids[t] * width + c);
+            const half8 tv = *reinterpret_cast<const half8 *>(&traw);
+            const half8 pv = *reinterpret_cast<const half8 *>(pos + (size_t)t * width + c);
+            if (embed_out != nullptr) *reinterpret_cast<uint4 *>(embed_out + (size_t)t * width + c) = traw;
+            lo = make_float4((float)tv[0] + (float)pv[0], (float)tv[1] + (float)pv[1], (float)tv[2] + (float)pv[2], (float)tv[3] + (float)pv[3]);
+            hi = make_float4((float)tv[4] + (float)pv[4], (float)tv[5] + (float)pv[5], (float)tv[6] + (float)pv[6], (float)tv[7] + (float)pv[7]);
+        }
+        *reinterpret_cast<float4 *>(x + (size_t)t * width + c) = lo;
+        *reinterpret_cast<float4 *>(x + (size_t)t * width + c + 4) = hi;
+    }
+}
+
+// Row LayerNorm, one wavefront per row, two-pass statistics (src/kernels.c:186-244), eps 1e-5.
+// Writes f16 (operand of the next product) or f32 (the encoder's output).
+template <bool F16_OUT>
+__global__ void __launch_bounds__(kThreads) k_enc_layernorm(const float *x, const float *gain, const float *bias, void *out, int rows, int width) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float4 *xr = reinterpret_cast<const float4 *>(x + (size_t)row * width);
+    const int n4 = width / 4;
+    float s = 0.0f;
+    for (int i = lane; i < n4; i += 64) {
+        const float4 v = xr[i];
+        s += (v.x + v.y) + (v.z + v.w);
+    }
+    const float mean = wave_sum(s) / (float)width;
+    float q = 0.0f;
+    for (int i = lane; i < n4; i += 64) {
+        const float4 v = xr[i];
+        const float a = v.x - mean, b = v.y - mean, c = v.z - mean, d = v.w - mean;
+        q += (a * a + b * b) + (c * c + d * d);
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + 1.0e-5f);
+    for (int i = lane; i < n4; i += 64) {
+        const float4 v = xr[i];
+        const float4 gg = reinterpret_cast<const float4 *>(gain)[i];
+        float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (bias != nullptr) bb = reinterpret_cast<const float4 *>(bias)[i];
+        const float y0 = (v.x - mean) * rstd * gg.x + bb.x, y1 = (v.y - mean) * rstd * gg.y + bb.y;
+        const float y2 = (v.z - mean) * rstd * gg.z + bb.z, y3 = (v.w - mean) * rstd * gg.w + bb.w;
+        if constexpr (F16_OUT) {
+            half4 h = {(_Float16)y0, (_Float16)y1, (_Float16)y2, (_Float16)y3};
+            reinterpret_cast<half4 *>(static_cast<_Float16 *>(out) + (size_t)row * width)[i] = h;
+        } else {
+            reinterpret_cast<float4 *>(static_cast<float *>(out) + (size_t)row * width)[i] = make_float4(y0, y1, y2, y3);
+        }
+    }
+}
+
+// One (32-query tile, head): S = scale * Q K^T over all keys (f32, in LDS) -> row softmax numerators
+// (f16, written over the row's own storage) and denominators -> O = P V / denom.
+// Wavefront w takes key tiles w, w+4, ... for the scores and, for PV, output columns 32*(w & 1) .. +31
+// over the key half (w >> 1); the two halves meet in LDS.
+__global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, const _Float16 *vt, _Float16 *ctx, int tokens, int tpad,
+                                                            int width, int vt_stride, float scale) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ float s_inv[kQTile];
+    __shared__ __align__(16) float s_half[2][16][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int q0 = blockIdx.x * kQTile, head = blockIdx.y;
+    const int sstride = tpad + kScorePad;                    // floats per score row
+    float *S = reinterpret_cast<float *>(smem);
+
+    // ---- scores
+    {
+        const int ld = 2 * width;
+        const _Float16 *qrow = qk + (size_t)(q0 + (lane & 31)) * ld + head * 64 + 8 * (lane >> 5);
+        half8 fq[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) fq[j] = *reinterpret_cast<const half8 *>(qrow + 16 * j);
+        for (int tile = wave; tile < tpad / 32; tile += 4) {
+            const _Float16 *krow = qk + (size_t)(tile * 32 + (lane & 31)) * ld + width + head * 64 + 8 * (lane >> 5);
+            floatx16 acc = {0};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const half8 fk = *reinterpret_cast<const half8 *>(krow + 16 * j);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fq[j], fk, acc, 0, 0, 0);
+            }
+            const int key = tile * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) S[acc_row(r, lane) * sstride + key] = key < tokens ? acc[r] * scale : -3.0e38f;
+        }
+    }
+    __syncthreads();
+
+    // ---- softmax of row tid / 8 by eight adjacent lanes (softmax_row_inplace, src/graph.c:245-257)
+    {
+        const int row = tid >> 3, part = tid & 7;
+        float *srow = S + row * sstride;
+        _Float16 *prow = reinterpret_cast<_Float16 *>(srow);
+        float m = -3.0e38f;
+        for (int c = part; c < tpad; c += 8) m = fmaxf(m, srow[c]);
+        m = fmaxf(m, __shfl_xor(m, 1));
+        m = fmaxf(m, __shfl_xor(m, 2));
+        m = fmaxf(m, __shfl_xor(m, 4));
+        float l = 0.0f;
+        // Numerators go back as f16 into the first half of the row's own bytes.  Element c (2 bytes at
+        // 2c) lands on floats already consumed: the eight lanes of a row walk c in lock step (one
+        // wavefront, in order), reading floats c .. c+7 of a sweep before writing halfs c .. c+7.
+        for (int c = part; c < tpad; c += 8) {
+            const float e = c < tokens ? expf(srow[c] - m) : 0.0f;
+            l += e;
+            prow[c] = (_Float16)e;
+        }
+        l += __shfl_xor(l, 1);
+        l += __shfl_xor(l, 2);
+        l += __shfl_xor(l, 4);
+        if (part == 0) s_inv[row] = 1.0f / l;
+    }
+    __syncthreads();
+
+    // ---- P V
+    {
+        const int wn = wave & 1, kh = wave >> 1;
+        const int kspan = tpad / 2;                              // multiple of 32
+        const _Float16 *prow = reinterpret_cast<const _Float16 *>(S + (lane & 31) * sstride) + kh * kspan + 8 * (lane >> 5);
+        const _Float16 *vrow = vt + (size_t)(head * 64 + wn * 32 + (lane & 31)) * vt_stride + kh * kspan + 8 * (lane >> 5);
+        floatx16 acc = {0};
+        for (int k = 0; k < kspan; k += 16) {
+            const half8 fp = *reinterpret_cast<const half8 *>(prow + k);
+            const half8 fv = *reinterpret_cast<const half8 *>(vrow + k);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fp, fv, acc, 0, 0, 0);
+        }
+        if (kh == 1) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_half[wn][r][lane] = acc[r];
+        }
+        __syncthreads();
+        if (kh == 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = acc_row(r, lane);
+                const float o = (acc[r] + s_half[wn][r][lane]) * s_inv[row];
+                ctx[(size_t)(q0 + row) * width + head * 64 + wn * 32 + (lane & 31)] = (_Float16)o;
+            }
+        }
+    }
+}
+
+template <int EPI>
+int launch_gemm(State *st, const GemmArgs &g, char *error, size_t capacity) {
+    if (g.M % kTile != 0 || g.N % kTile != 0 || g.K % kTile != 0 || g.M <= 0 || g.N <= 0 || g.K <= 0) {
+        set_error(error, capacity, "encoder product: shape is not a multiple of the 64 x 64 x 64 tile");
+        return -1;
+    }
+    hipLaunchKernelGGL((k_enc_gemm<EPI>), dim3(g.N / kTile, g.M / kTile), dim3(kThreads), 0, st->stream, g);
+    return hip_check(hipGetLastError(), "encoder product launch", error, capacity);
+}
+
+int f16_matrix(State *st, const float *host, size_t n, size_t k, const CachedWeight **out, char *error, size_t capacity) {
+    if (cached_matrix(st, host, n, k, MYNAH_HIP_F16, out, error, capacity) != 0) return -1;
+    if ((*out)->qtype != MYNAH_HIP_F16) {
+        set_error(error, capacity, "encoder: weight shape cannot be stored as f16");
+        return -1;
+    }
+    return 0;
+}
+
+size_t attention_lds_bytes(size_t tpad) { return (size_t)kQTile * (tpad + kScorePad) * sizeof(float); }
+
+}  // namespace
+
+extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_desc *d, mynah_hip_encoder **out, char *error, size_t capacity) {
+    State *st = static_cast<State *>(state);
+    if (out != nullptr) *out = nullptr;
+    if (st == nullptr || d == nullptr || out == nullptr) {
+        set_error(error, capacity, "encoder_create: null argument");
+        return -1;
+    }
+    if (d->layers == 0 || d->width == 0 || d->heads == 0 || d->heads * d->head_width != d->width || d->head_width != 64 ||
+        d->width % kTile != 0 || d->ffn_width % kTile != 0 || d->ffn_width == 0 || d->vocab == 0 || d->max_positions == 0 ||
+        d->width > 8192 || d->ffn_width > 32768 || d->max_positions > 4096 || d->tok_table == nullptr || d->pos_table == nullptr ||
+        d->qkv_w == nullptr || d->o_w == nullptr || d->up_w == nullptr || d->down_w == nullptr || d->norm1 == nullptr || d->norm2 == nullptr) {
+        set_error(error, capacity, "encoder_create: unsupported shape (needs 64-wide heads, widths that are multiples of 64) or missing weights");
+        return -1;
+    }
+    auto *e = new mynah_hip_encoder();
+    e->layers = d->layers; e->width = d->width; e->heads = d->heads; e->head_width = d->head_width; e->ffn = d->ffn_width;
+    e->vocab = d->vocab; e->max_positions = d->max_positions;
+    e->tpad_max = (d->max_positions + kTile - 1) / kTile * kTile;
+    int lds = 0;
+    if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, 0) != hipSuccess || lds <= 0) lds = 65536;
+    e->max_lds = (size_t)lds;
+    auto fail = [&](void) { mynah_hip_encoder_destroy(state, e); return -1; };
+    if (attention_lds_bytes(e->tpad_max) + 10 * 1024 > e->max_lds) {
+        set_error(error, capacity, "encoder_create: max_positions needs more LDS per workgroup than this device has");
+        return fail();
+    }
+    if (f16_matrix(st, d->tok_table, d->vocab, d->width, &e->tok, error, capacity) != 0) return fail();
+    if (f16_matrix(st, d->pos_table, d->max_positions, d->width, &e->pos, error, capacity) != 0) return fail();
+    for (size_t l = 0; l < d->layers; ++l) {
+        const CachedWeight *cw = nullptr;
+        const float *v = nullptr;
+        if (d->qkv_w[l] == nullptr || d->o_w[l] == nullptr || d->up_w[l] == nullptr || d->down_w[l] == nullptr || d->norm1[l] == nullptr ||
+            d->norm2[l] == nullptr) {
+            set_error(error, capacity, "encoder_create: missing layer weight");
+            return fail();
+        }
+        if (f16_matrix(st, d->qkv_w[l], 3 * d->width, d->width, &cw, error, capacity) != 0) return fail();
+        e->qkv.push_back(cw);
+        if (f16_matrix(st, d->o_w[l], d->width, d->width, &cw, error, capacity) != 0) return fail();
+        e->o.push_back(cw);
+        if (f16_matrix(st, d->up_w[l], d->ffn_width, d->width, &cw, error, capacity) != 0) return fail();
+        e->up.push_back(cw);
+        if (f16_matrix(st, d->down_w[l], d->width, d->ffn_width, &cw, error, capacity) != 0) return fail();
+        e->down.push_back(cw);
+        if (cached_vector(st, d->norm1[l], d->width, &v, error, capacity) != 0) return fail();
+        e->n1g.push_back(v);
+        v = nullptr;
+        if (d->norm1_bias != nullptr && d->norm1_bias[l] != nullptr && cached_vector(st, d->norm1_bias[l], d->width, &v, error, capacity) != 0) return fail();
+        e->n1b.push_back(v);
+        if (cached_vector(st, d->norm2[l], d->width, &v, error, capacity) != 0) return fail();
+        e->n2g.push_back(v);
+        v = nullptr;
+        if (d->norm2_bias != nullptr && d->norm2_bias[l] != nullptr && cached_vector(st, d->norm2_bias[l], d->width, &v, error, capacity) != 0) return fail();
+        e->n2b.push_back(v);
+    }
+    if (d->norm_out != nullptr && cached_vector(st, d->norm_out, d->width, &e->nog, error, capacity) != 0) return fail();
+    if (d->norm_out != nullptr && d->norm_out_bias != nullptr && cached_vector(st, d->norm_out_bias, d->width, &e->nob, error, capacity) != 0) return fail();
+    const size_t tp = e->tpad_max, w = e->width, f = e->ffn;
+    auto alloc = [&](void **p, size_t bytes) {
+        if (hip_check(hipMalloc(p, bytes), "encoder workspace", error, capacity) != 0) return -1;
+        return hip_check(hipMemsetAsync(*p, 0, bytes, st->stream), "encoder workspace clear", error, capacity);
+    };
+    if (alloc(reinterpret_cast<void **>(&e->x), tp * w * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->nrm), tp * w * 2) != 0 ||
+        alloc(reinterpret_cast<void **>(&e->qk), tp * 2 * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->vt), w * tp * 2) != 0 ||
+        alloc(reinterpret_cast<void **>(&e->ctx), tp * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->hid), tp * f * 2) != 0 ||
+        alloc(reinterpret_cast<void **>(&e->ids), tp * sizeof(int)) != 0)
+        return fail();
+    if (hip_check(hipHostMalloc(reinterpret_cast<void **>(&e->ids_host), tp * sizeof(int), hipHostMallocDefault), "encoder ids staging", error, capacity) != 0)
+        return fail();
+    if (attention_lds_bytes(e->tpad_max) > 48 * 1024 &&
+        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_enc_attention), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)attention_lds_bytes(e->tpad_max)), "encoder attention LDS size", error, capacity) != 0)
+        return fail();
+    if (hip_check(hipStreamSynchronize(st->stream), "encoder create", error, capacity) != 0) return fail();
+    *out = e;
+    return 0;
+}
+
+extern "C" void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *e) {
+    State *st = static_cast<State *>(state);
+    if (e == nullptr) return;
+    if (st != nullptr) (void)hipStreamSynchronize(st->stream);
+    for (void *p : {(void *)e->x, (void *)e->nrm, (void *)e->qk, (void *)e->vt, (void *)e->ctx, (void *)e->hid, (void *)e->ids})
+        if (p != nullptr) (void)hipFree(p);
+    if (e->ids_host != nullptr) (void)hipHostFree(e->ids_host);
+    delete e;
+}
+
+extern "C" int mynah_hip_encoder_prefill(void *state, mynah_hip_encoder *e, const int32_t *ids, size_t tokens, uint16_t *dev_embed_f16,
+                                         float *dev_out, char *error, size_t capacity) {
+    State *st = static_cast<State *>(state);
+    if (st == nullptr || e == nullptr || ids == nullptr || dev_out == nullptr) {
+        set_error(error, capacity, "encoder_prefill: null argument");
+        return -1;
+    }
+    if (tokens == 0 || tokens > e->max_positions) {
+        set_error(error, capacity, "encoder_prefill: token count outside [1, max_positions]");
+        return -1;
+    }
+    for (size_t t = 0; t < tokens; ++t) {
+        if (ids[t] < 0 || (size_t)ids[t] >= e->vocab) {   // src/graph.c:730-735
+            set_error(error, capacity, "encoder_prefill: token id out of range");
+            return -1;
+        }
+    }
+    // the staging buffer of the previous call may still be in flight
+    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    for (size_t t = 0; t < tokens; ++t) e->ids_host[t] = ids[t];
+    MYNAH_TRY(hipMemcpyAsync(e->ids, e->ids_host, tokens * sizeof(int), hipMemcpyHostToDevice, st->stream));
+
+    const int T = (int)tokens, w = (int)e->width, f = (int)e->ffn;
+    const int tpad = (T + kTile - 1) / kTile * kTile;
+    const int vt_stride = (int)e->tpad_max;
+    hipLaunchKernelGGL(k_enc_embed, dim3(tpad), dim3(kThreads), 0, st->stream, e->ids, static_cast<const _Float16 *>(e->tok->data),
+                       static_cast<const _Float16 *>(e->pos->data), e->x, dev_embed_f16, T, w);
+    const dim3 ln_grid((tpad + 3) / 4);
+    const float scale = 1.0f / sqrtf((float)e->head_width);
+    const size_t lds = attention_lds_bytes((size_t)tpad);
+    for (size_t l = 0; l < e->layers; ++l) {
+        hipLaunchKernelGGL((k_enc_layernorm<true>), ln_grid, dim3(kThreads), 0, st->stream, e->x, e->n1g[l], e->n1b[l], (void *)e->nrm, tpad, w);
+        GemmArgs g{};
+        g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->qkv[l]->data); g.M = tpad; g.N = 3 * w; g.K = w;
+        g.out = e->qk; g.vt = e->vt; g.width = w; g.vt_stride = vt_stride;
+        if (launch_gemm<ENC_QKV>(st, g, error, capacity) != 0) return -1;
+        hipLaunchKernelGGL(k_enc_attention, dim3(tpad / kQTile, (unsigned)e->heads), dim3(kThreads), lds, st->stream, e->qk, e->vt, e->ctx, T, tpad,
+                           w, vt_stride, scale);
+        g = GemmArgs{};
+        g.a = e->ctx; g.w = static_cast<const _Float16 *>(e->o[l]->data); g.M = tpad; g.N = w; g.K = w; g.x = e->x;
+        if (launch_gemm<ENC_RESIDUAL>(st, g, error, capacity) != 0) return -1;
+        hipLaunchKernelGGL((k_enc_layernorm<true>), ln_grid, dim3(kThreads), 0, st->stream, e->x, e->n2g[l], e->n2b[l], (void *)e->nrm, tpad, w);
+        g = GemmArgs{};
+        g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->up[l]->data); g.M = tpad; g.N = f; g.K = w; g.out = e->hid;
+        if (launch_gemm<ENC_GELU>(st, g, error, capacity) != 0) return -1;
+        g = GemmArgs{};
+        g.a = e->hid; g.w = static_cast<const _Float16 *>(e->down[l]->data); g.M = tpad; g.N = w; g.K = f; g.x = e->x;
+        if (launch_gemm<ENC_RESIDUAL>(st, g, error, capacity) != 0) return -1;
+    }
+    if (e->nog != nullptr) {
+        hipLaunchKernelGGL((k_enc_layernorm<false>), dim3((T + 3) / 4), dim3(kThreads), 0, st->stream, e->x, e->nog, e->nob, (void *)dev_out, T, w);
+    } else {
+        MYNAH_TRY(hipMemcpyAsync(dev_out, e->x, (size_t)T * w * sizeof(float), hipMemcpyDeviceToDevice, st->stream));
+    }
+    return hip_check(hipGetLastError(), "encoder prefill launch", error, capacity);
 }
