@@ -88,6 +88,27 @@ def time_config(pkg, synth, backend, qtype, lengths, mems, capacity, steps, warm
             "gbps": total / (step_us * 1e-6) / 1e9, "setup_s": setup_s}
 
 
+def time_prefill(pkg, synth, backend, tokens=256, runs=30, warmup=5):
+    """Text-encoder prefill: 6 layers, d=768, 12x64 heads, FFN 3072, f16 weights, `tokens` tokens, on the matrix cores."""
+    cfg = synth.encoder_config()
+    enc = pkg.Encoder(backend, cfg, synth.encoder_weights(cfg, seed=4))
+    ids = np.random.default_rng(5).integers(0, cfg["vocab"], size=tokens).astype(np.int32)
+    dout = backend.alloc(tokens * cfg["width"])
+    for _ in range(warmup):
+        enc.prefill(ids, 0, dout.ptr)
+    backend.sync()
+    backend.timer_begin()
+    for _ in range(runs):
+        enc.prefill(ids, 0, dout.ptr)
+    us = backend.timer_end() * 1000.0 / runs
+    out = dout.read()
+    assert np.all(np.isfinite(out)), "prefill output is not finite"
+    enc.destroy()
+    w, f, L = cfg["width"], cfg["ffn"], cfg["layers"]
+    flops = L * (2 * tokens * (3 * w * w + w * w + 2 * f * w) + 4 * tokens * tokens * w)
+    return {"us": us, "flops": flops, "tflops": flops / (us * 1e-6) / 1e12, "tokens": tokens}
+
+
 def cpu_baseline(steps=5, warmup=2):
     """The reference's own CPU decode step (compiled from its sources into oracle/_ref), timed on this box's host
     cores in a child process: all online cores, then one thread."""
@@ -112,6 +133,7 @@ def main():
     ap.add_argument("--quant", default="int8", choices=["int8", "int4", "f16", "f32"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--skip-b8", action="store_true")
+    ap.add_argument("--skip-prefill", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the library's plain read+write kernel over 256 MiB three times (a known-size reference for "
@@ -140,6 +162,7 @@ def main():
         b8 = time_config(pkg, synth, backend, qtype, [n - 1 for n in self_len], cross_len, 2048, max(args.steps // 3, 20),
                          max(args.warmup // 3, 6), rotate=ROTATE)
         b8["self_lengths"], b8["cross_lengths"] = self_len, cross_len
+    prefill = None if args.skip_prefill else time_prefill(pkg, synth, backend)
     backend.close()
 
     result = {
@@ -174,6 +197,11 @@ def main():
                         "weight_bytes": b8["weight_bytes"], "kv_bytes": b8["kv_bytes"], "self_lengths": b8["self_lengths"],
                         "cross_lengths": b8["cross_lengths"],
                         "us_per_stream_step": round(b8["step_us"] / 8.0, 2)}
+    if prefill is not None:
+        result["prefill"] = {"workload": "text-encoder prefill, 6 layers d=768 12x64 heads FFN 3072, f16 weights and operands, f32 "
+                                         "accumulate, %d tokens" % prefill["tokens"],
+                             "us": round(prefill["us"], 2), "flops": prefill["flops"], "tflops": round(prefill["tflops"], 2),
+                             "bound": "mfma", "peak_tflops": 2500.0, "frac": round(prefill["tflops"] / 2500.0, 4)}
     if not args.no_cpu:
         cpu = cpu_baseline()
         allc = cpu.get("all", {})

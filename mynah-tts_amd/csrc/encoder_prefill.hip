@@ -16,6 +16,8 @@
 //   vt   f16 [w, TpadMax]    v transposed: vt[h*64+d][t], so PV's B operand is K(=t)-contiguous too
 //   ctx  f16 [Tpad, w]       attention output = A operand of the O product
 //   hid  f16 [Tpad, ffn]     GELU(up) = A operand of the FFN-down product
+//   part f32 [4, Tpad, w]    K-split partial sums of the O and FFN-down products; the row pass that follows
+//                            adds them to x in a fixed order (no atomics: results do not depend on scheduling)
 //
 // All products are "NT": C[m][n] = sum_k A[m][k] * W[n][k], both operands K-contiguous, which is how
 // the 32x32x16 MFMA wants them: lane l supplies row (l % 32) of A (or of W) and the eight consecutive
@@ -24,16 +26,28 @@
 
 using namespace mynah;
 
+// Per-call values read by the kernels from device memory, so that one captured graph per padded length
+// serves every call: the token count and the caller's output pointers.
+struct EncParams {
+    int tokens;
+    int reserved;
+    uint16_t *embed_out;
+    float *out;
+};
+
 struct mynah_hip_encoder {
     size_t layers = 0, width = 0, heads = 0, head_width = 0, ffn = 0, vocab = 0, max_positions = 0, tpad_max = 0;
     const CachedWeight *tok = nullptr, *pos = nullptr;
     std::vector<const CachedWeight *> qkv, o, up, down;
     std::vector<const float *> n1g, n1b, n2g, n2b;
     const float *nog = nullptr, *nob = nullptr;
-    float *x = nullptr;
+    float *x = nullptr, *part = nullptr;   // part: [splits, Tpad, w] partial products of the O and FFN-down products
     _Float16 *nrm = nullptr, *qk = nullptr, *vt = nullptr, *ctx = nullptr, *hid = nullptr;
-    int *ids = nullptr;
-    int *ids_host = nullptr;   // pinned
+    int *ids = nullptr;        // [tpad_max] token ids, followed by one EncParams
+    int *ids_host = nullptr;   // pinned twin of ids
+    EncParams *params = nullptr;
+    std::unordered_map<int, hipGraphExec_t> graphs;   // by padded length
+    std::unordered_map<int, int> eager_runs;          // a padded length runs eagerly once before it is captured
     size_t max_lds = 0;
 };
 
@@ -42,19 +56,20 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTile = 64;            // workgroup tile of the products: 64 x 64, K step 64
 constexpr int kLdsStride = 72;       // halfs per staged row: 64 + 8 keeps 16-byte reads of 32 rows off each other's banks
 constexpr int kQTile = 32;           // queries per attention workgroup
 constexpr int kScorePad = 8;         // floats appended to a score row (bank spread for the row-wise softmax)
 
-enum { ENC_QKV = 0, ENC_RESIDUAL = 1, ENC_GELU = 2 };
+enum { ENC_QKV = 0, ENC_PARTIAL = 1, ENC_GELU = 2 };
 
 struct GemmArgs {
     const _Float16 *a;     // [M, K] row-major, lda = K
     const _Float16 *w;     // [N, K]
     int M, N, K;
-    float *x;              // ENC_RESIDUAL: x[m][n] += c, ldx = N
+    float *part;           // ENC_PARTIAL: part[z][m][n] = this K split's share of the product (summed by the next LayerNorm pass)
     _Float16 *out;         // ENC_QKV: qk [M, 2*width];  ENC_GELU: hid [M, N]
     _Float16 *vt;          // ENC_QKV: v transposed [width, vt_stride]
     int width, vt_stride;
@@ -62,6 +77,30 @@ struct GemmArgs {
 
 // Row of C held in accumulator register r of lane l for a 32x32 MFMA tile; the column is l % 32.
 __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// One K step of both operand tiles on its way from global memory to LDS (four 16-byte pieces per thread).
+struct StagedTiles {
+    u32x4 a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0}, w0 = {0, 0, 0, 0}, w1 = {0, 0, 0, 0};
+    __device__ __forceinline__ void load(const u32x4 *ga0, const u32x4 *ga1, const u32x4 *gw0, const u32x4 *gw1, int chunk) {
+        a0 = ga0[chunk]; a1 = ga1[chunk]; w0 = gw0[chunk]; w1 = gw1[chunk];
+    }
+    __device__ __forceinline__ void store(_Float16 *sa, _Float16 *sw, int off0, int off1) const {
+        *reinterpret_cast<u32x4 *>(sa + off0) = a0;
+        *reinterpret_cast<u32x4 *>(sa + off1) = a1;
+        *reinterpret_cast<u32x4 *>(sw + off0) = w0;
+        *reinterpret_cast<u32x4 *>(sw + off1) = w1;
+    }
+};
+
+// acc += A-tile fragment x W-tile fragment over one 64-deep K step (four 32x32x16 MFMAs).
+__device__ __forceinline__ void mma_tile(floatx16 &acc, const _Float16 *pa, const _Float16 *pw) {
+#pragma unroll
+    for (int j = 0; j < kTile / 16; ++j) {
+        const half8 fa = *reinterpret_cast<const half8 *>(pa + 16 * j);
+        const half8 fw = *reinterpret_cast<const half8 *>(pw + 16 * j);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fw, acc, 0, 0, 0);
+    }
+}
 
 template <int EPI>
 __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
@@ -72,54 +111,55 @@ __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
     const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
     // staging: thread -> (row tid / 8 and + 32, 16-byte chunk tid % 8) of both tiles
     const int srow = tid >> 3, schunk = tid & 7;
-    const uint4 *ga0 = reinterpret_cast<const uint4 *>(g.a + (size_t)(m0 + srow) * g.K) + schunk;
-    const uint4 *ga1 = reinterpret_cast<const uint4 *>(g.a + (size_t)(m0 + srow + 32) * g.K) + schunk;
-    const uint4 *gw0 = reinterpret_cast<const uint4 *>(g.w + (size_t)(n0 + srow) * g.K) + schunk;
-    const uint4 *gw1 = reinterpret_cast<const uint4 *>(g.w + (size_t)(n0 + srow + 32) * g.K) + schunk;
+    const u32x4 *ga0 = reinterpret_cast<const u32x4 *>(g.a + (size_t)(m0 + srow) * g.K) + schunk;
+    const u32x4 *ga1 = reinterpret_cast<const u32x4 *>(g.a + (size_t)(m0 + srow + 32) * g.K) + schunk;
+    const u32x4 *gw0 = reinterpret_cast<const u32x4 *>(g.w + (size_t)(n0 + srow) * g.K) + schunk;
+    const u32x4 *gw1 = reinterpret_cast<const u32x4 *>(g.w + (size_t)(n0 + srow + 32) * g.K) + schunk;
     const int soff0 = srow * kLdsStride + schunk * 8, soff1 = (srow + 32) * kLdsStride + schunk * 8;
 
-    uint4 ra0 = ga0[0], ra1 = ga1[0], rw0 = gw0[0], rw1 = gw1[0];
-    *reinterpret_cast<uint4 *>(&s_a[0][soff0]) = ra0;
-    *reinterpret_cast<uint4 *>(&s_a[0][soff1]) = ra1;
-    *reinterpret_cast<uint4 *>(&s_w[0][soff0]) = rw0;
-    *reinterpret_cast<uint4 *>(&s_w[0][soff1]) = rw1;
+    // K range of this workgroup (blockIdx.z splits K; only ENC_PARTIAL launches more than one split)
+    const int nk = g.K / kTile / (int)gridDim.z;
+    const int kbase = (int)blockIdx.z * nk * (kTile / 8);   // in 16-byte chunks
+    ga0 += kbase; ga1 += kbase; gw0 += kbase; gw1 += kbase;
+
+    // Global -> register -> LDS pipeline, two K steps ahead of the multiply: the loop is bound by the
+    // latency of these loads, not by the matrix cores, so two steps are kept in flight.
+    StagedTiles p0, p1;   // p0: odd K steps, p1: even K steps (from 2 on)
+    {
+        const u32x4 a0 = ga0[0], a1 = ga1[0], w0 = gw0[0], w1 = gw1[0];
+        if (1 < nk) p0.load(ga0, ga1, gw0, gw1, kTile / 8);
+        if (2 < nk) p1.load(ga0, ga1, gw0, gw1, 2 * (kTile / 8));
+        *reinterpret_cast<u32x4 *>(&s_a[0][soff0]) = a0;
+        *reinterpret_cast<u32x4 *>(&s_a[0][soff1]) = a1;
+        *reinterpret_cast<u32x4 *>(&s_w[0][soff0]) = w0;
+        *reinterpret_cast<u32x4 *>(&s_w[0][soff1]) = w1;
+    }
     __syncthreads();
 
     floatx16 acc = {0};
-    const int nk = g.K / kTile;
     const int frag = (lane & 31) * kLdsStride + 8 * (lane >> 5);
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) {   // next K step's tiles travel while this one is multiplied
-            const int step = (kt + 1) * (kTile / 8);
-            ra0 = ga0[step]; ra1 = ga1[step]; rw0 = gw0[step]; rw1 = gw1[step];
-        }
-        const _Float16 *pa = &s_a[cur][wm * 32 * kLdsStride + frag];
-        const _Float16 *pw = &s_w[cur][wn * 32 * kLdsStride + frag];
-#pragma unroll
-        for (int j = 0; j < kTile / 16; ++j) {
-            const half8 fa = *reinterpret_cast<const half8 *>(pa + 16 * j);
-            const half8 fw = *reinterpret_cast<const half8 *>(pw + 16 * j);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fw, acc, 0, 0, 0);
-        }
-        if (kt + 1 < nk) {
-            const int nxt = cur ^ 1;   // last read one iteration ago, before the barrier that ended it
-            *reinterpret_cast<uint4 *>(&s_a[nxt][soff0]) = ra0;
-            *reinterpret_cast<uint4 *>(&s_a[nxt][soff1]) = ra1;
-            *reinterpret_cast<uint4 *>(&s_w[nxt][soff0]) = rw0;
-            *reinterpret_cast<uint4 *>(&s_w[nxt][soff1]) = rw1;
-        }
+    const int fa_off = wm * 32 * kLdsStride + frag, fw_off = wn * 32 * kLdsStride + frag;
+    for (int kt = 0; kt < nk; kt += 2) {
+        // even step: multiply buffer 0, stage step kt + 1 (in p0) into buffer 1, request step kt + 3
+        mma_tile(acc, &s_a[0][fa_off], &s_w[0][fw_off]);
+        if (kt + 1 < nk) p0.store(&s_a[1][0], &s_w[1][0], soff0, soff1);
+        if (kt + 3 < nk) p0.load(ga0, ga1, gw0, gw1, (kt + 3) * (kTile / 8));
         __syncthreads();
+        if (kt + 1 < nk) {
+            // odd step: multiply buffer 1, stage step kt + 2 (in p1) into buffer 0, request step kt + 4
+            mma_tile(acc, &s_a[1][fa_off], &s_w[1][fw_off]);
+            if (kt + 2 < nk) p1.store(&s_a[0][0], &s_w[0][0], soff0, soff1);
+            if (kt + 4 < nk) p1.load(ga0, ga1, gw0, gw1, (kt + 4) * (kTile / 8));
+            __syncthreads();
+        }
     }
 
     const int n = n0 + wn * 32 + (lane & 31);
     const int mbase = m0 + wm * 32;
-    if constexpr (EPI == ENC_RESIDUAL) {
+    if constexpr (EPI == ENC_PARTIAL) {
+        float *part = g.part + (size_t)blockIdx.z * g.M * g.N;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            float *p = g.x + (size_t)(mbase + acc_row(r, lane)) * g.N + n;
-            *p = *p + acc[r];
-        }
+        for (int r = 0; r < 16; ++r) part[(size_t)(mbase + acc_row(r, lane)) * g.N + n] = acc[r];
     } else if constexpr (EPI == ENC_GELU) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) g.out[(size_t)(mbase + acc_row(r, lane)) * g.N + n] = (_Float16)gelu_tanh(acc[r]);
@@ -139,9 +179,11 @@ __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
 }
 
 // Token gather + position add (src/graph.c:729-737, :649-651).  Rows [tokens, tpad) are zeroed.
-__global__ void __launch_bounds__(kThreads) k_enc_embed(const int *ids, const _Float16 *tok, const _Float16 *pos, float *x,
-                                                        uint16_t *embed_out, int tokens, int width) {
+__global__ void __launch_bounds__(kThreads) k_enc_embed(const int *ids, const EncParams *params, const _Float16 *tok, const _Float16 *pos,
+                                                        float *x, int width) {
     const int t = blockIdx.x;
+    const int tokens = params->tokens;
+    uint16_t *embed_out = params->embed_out;
     for (int c = threadIdx.x * 8; c < width; c += kThreads * 8) {
         float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
         if (t < tokens) {
@@ -157,50 +199,109 @@ __global__ void __launch_bounds__(kThreads) k_enc_embed(const int *ids, const _F
     }
 }
 
-// Row LayerNorm, one wavefront per row, two-pass statistics (src/kernels.c:186-244), eps 1e-5.
-// Writes f16 (operand of the next product) or f32 (the encoder's output).
-template <bool F16_OUT>
-__global__ void __launch_bounds__(kThreads) k_enc_layernorm(const float *x, const float *gain, const float *bias, void *out, int rows, int width) {
+// Row pass between two products, one wavefront per row: first the residual update
+// x += sum over K splits of the previous product's partials (src/graph.c:470, :316), then LayerNorm with
+// two-pass statistics (src/kernels.c:186-244, eps 1e-5) written as f16 (operand of the next product) or
+// f32 (the encoder's output, to params->out, rows below params->tokens only).  gain == nullptr: no
+// LayerNorm, the updated row is copied out as f32.  A lane keeps its NV float4 pieces of the row in
+// registers (width <= 256 * NV; the widest supported row, 4096, takes NV = 16).
+template <bool F16_OUT, int NV>
+__global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *part, int splits, size_t split_stride, const float *gain,
+                                                       const float *bias, _Float16 *out_f16, const EncParams *params, int rows, int width) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     if (row >= rows) return;
-    const float4 *xr = reinterpret_cast<const float4 *>(x + (size_t)row * width);
+    if constexpr (!F16_OUT) {
+        if (row >= params->tokens) return;
+    }
+    float4 *xr = reinterpret_cast<float4 *>(x + (size_t)row * width);
     const int n4 = width / 4;
-    float s = 0.0f;
-    for (int i = lane; i < n4; i += 64) {
-        const float4 v = xr[i];
-        s += (v.x + v.y) + (v.z + v.w);
+    float4 v[NV], gg[NV], bb[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = lane + 64 * u;
+        const bool in = i < n4;
+        v[u] = in ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        gg[u] = (in && gain != nullptr) ? reinterpret_cast<const float4 *>(gain)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        bb[u] = (in && bias != nullptr) ? reinterpret_cast<const float4 *>(bias)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    const float mean = wave_sum(s) / (float)width;
-    float q = 0.0f;
-    for (int i = lane; i < n4; i += 64) {
-        const float4 v = xr[i];
-        const float a = v.x - mean, b = v.y - mean, c = v.z - mean, d = v.w - mean;
-        q += (a * a + b * b) + (c * c + d * d);
-    }
-    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + 1.0e-5f);
-    for (int i = lane; i < n4; i += 64) {
-        const float4 v = xr[i];
-        const float4 gg = reinterpret_cast<const float4 *>(gain)[i];
-        float4 bb = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (bias != nullptr) bb = reinterpret_cast<const float4 *>(bias)[i];
-        const float y0 = (v.x - mean) * rstd * gg.x + bb.x, y1 = (v.y - mean) * rstd * gg.y + bb.y;
-        const float y2 = (v.z - mean) * rstd * gg.z + bb.z, y3 = (v.w - mean) * rstd * gg.w + bb.w;
-        if constexpr (F16_OUT) {
-            half4 h = {(_Float16)y0, (_Float16)y1, (_Float16)y2, (_Float16)y3};
-            reinterpret_cast<half4 *>(static_cast<_Float16 *>(out) + (size_t)row * width)[i] = h;
-        } else {
-            reinterpret_cast<float4 *>(static_cast<float *>(out) + (size_t)row * width)[i] = make_float4(y0, y1, y2, y3);
+    if (part != nullptr) {
+        float4 p[NV];
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int i = lane + 64 * u;
+            p[u] = i < n4 ? reinterpret_cast<const float4 *>(part + (size_t)row * width)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        for (int z = 1; z < splits; ++z) {   // fixed order: the sum does not depend on how the splits were scheduled
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                const int i = lane + 64 * u;
+                if (i < n4) {
+                    const float4 q = reinterpret_cast<const float4 *>(part + z * split_stride + (size_t)row * width)[i];
+                    p[u].x += q.x; p[u].y += q.y; p[u].z += q.z; p[u].w += q.w;
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int i = lane + 64 * u;
+            v[u].x += p[u].x; v[u].y += p[u].y; v[u].z += p[u].z; v[u].w += p[u].w;
+            if (i < n4) xr[i] = v[u];
         }
     }
+    if (gain == nullptr) {
+        if constexpr (!F16_OUT) {
+#pragma unroll
+            for (int u = 0; u < NV; ++u)
+                if (lane + 64 * u < n4) reinterpret_cast<float4 *>(params->out + (size_t)row * width)[lane + 64 * u] = v[u];
+        }
+        return;
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);   // pieces past the row are zero
+    const float mean = wave_sum(s) / (float)width;
+    float q = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        if (lane + 64 * u < n4) {
+            const float a = v[u].x - mean, b = v[u].y - mean, c = v[u].z - mean, d = v[u].w - mean;
+            q += (a * a + b * b) + (c * c + d * d);
+        }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + 1.0e-5f);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = lane + 64 * u;
+        if (i < n4) {
+            const float y0 = (v[u].x - mean) * rstd * gg[u].x + bb[u].x, y1 = (v[u].y - mean) * rstd * gg[u].y + bb[u].y;
+            const float y2 = (v[u].z - mean) * rstd * gg[u].z + bb[u].z, y3 = (v[u].w - mean) * rstd * gg[u].w + bb[u].w;
+            if constexpr (F16_OUT) {
+                half4 h = {(_Float16)y0, (_Float16)y1, (_Float16)y2, (_Float16)y3};
+                reinterpret_cast<half4 *>(out_f16 + (size_t)row * width)[i] = h;
+            } else {
+                reinterpret_cast<float4 *>(params->out + (size_t)row * width)[i] = make_float4(y0, y1, y2, y3);
+            }
+        }
+    }
+}
+
+template <bool F16_OUT>
+void launch_rows(State *st, int width, dim3 grid, float *x, const float *part, int splits, size_t split_stride, const float *gain,
+                 const float *bias, _Float16 *out_f16, const EncParams *params, int rows) {
+    if (width <= 1024)
+        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 4>), grid, dim3(kThreads), 0, st->stream, x, part, splits, split_stride, gain, bias, out_f16, params, rows, width);
+    else
+        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 16>), grid, dim3(kThreads), 0, st->stream, x, part, splits, split_stride, gain, bias, out_f16, params, rows, width);
 }
 
 // One (32-query tile, head): S = scale * Q K^T over all keys (f32, in LDS) -> row softmax numerators
 // (f16, written over the row's own storage) and denominators -> O = P V / denom.
 // Wavefront w takes key tiles w, w+4, ... for the scores and, for PV, output columns 32*(w & 1) .. +31
 // over the key half (w >> 1); the two halves meet in LDS.
-__global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, const _Float16 *vt, _Float16 *ctx, int tokens, int tpad,
-                                                            int width, int vt_stride, float scale) {
+__global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, const _Float16 *vt, _Float16 *ctx, const EncParams *params,
+                                                            int tpad, int width, int vt_stride, float scale) {
+    const int tokens = params->tokens;
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_inv[kQTile];
     __shared__ __align__(16) float s_half[2][16][64];
@@ -286,12 +387,13 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
 }
 
 template <int EPI>
-int launch_gemm(State *st, const GemmArgs &g, char *error, size_t capacity) {
-    if (g.M % kTile != 0 || g.N % kTile != 0 || g.K % kTile != 0 || g.M <= 0 || g.N <= 0 || g.K <= 0) {
+int launch_gemm(State *st, const GemmArgs &g, int splits, char *error, size_t capacity) {
+    if (g.M % kTile != 0 || g.N % kTile != 0 || g.M <= 0 || g.N <= 0 || g.K <= 0 || splits < 1 || g.K % (kTile * splits) != 0 ||
+        (splits > 1 && EPI != ENC_PARTIAL)) {
         set_error(error, capacity, "encoder product: shape is not a multiple of the 64 x 64 x 64 tile");
         return -1;
     }
-    hipLaunchKernelGGL((k_enc_gemm<EPI>), dim3(g.N / kTile, g.M / kTile), dim3(kThreads), 0, st->stream, g);
+    hipLaunchKernelGGL((k_enc_gemm<EPI>), dim3(g.N / kTile, g.M / kTile, splits), dim3(kThreads), 0, st->stream, g);
     return hip_check(hipGetLastError(), "encoder product launch", error, capacity);
 }
 
@@ -306,6 +408,54 @@ int f16_matrix(State *st, const float *host, size_t n, size_t k, const CachedWei
 
 size_t attention_lds_bytes(size_t tpad) { return (size_t)kQTile * (tpad + kScorePad) * sizeof(float); }
 
+constexpr int kMaxSplits = 4;
+int pick_splits(int k) {
+    for (int s = kMaxSplits; s > 1; --s)
+        if (k % (kTile * s) == 0 && k / (kTile * s) >= 3) return s;
+    return 1;
+}
+
+// Every kernel of one prefill over `tpad` padded rows, in stream order.  Everything that changes from call to
+// call (token count, output pointers) is read from e->params on the device, so the sequence can be captured once.
+int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size_t capacity) {
+    const int w = (int)e->width, f = (int)e->ffn;
+    const int vt_stride = (int)e->tpad_max;
+    hipLaunchKernelGGL(k_enc_embed, dim3(tpad), dim3(kThreads), 0, st->stream, e->ids, e->params, static_cast<const _Float16 *>(e->tok->data),
+                       static_cast<const _Float16 *>(e->pos->data), e->x, w);
+    const dim3 row_grid((tpad + 3) / 4);
+    const float scale = 1.0f / sqrtf((float)e->head_width);
+    const size_t lds = attention_lds_bytes((size_t)tpad);
+    const size_t split_stride = (size_t)tpad * w;
+    // K splits of the two width-wide products (few output tiles, long K): enough workgroups to occupy the chip
+    const int o_splits = pick_splits(w), down_splits = pick_splits(f);
+    const float *pending = nullptr;   // partials of the last product, not yet added to x
+    int pending_splits = 0;
+    for (size_t l = 0; l < e->layers; ++l) {
+        launch_rows<true>(st, w, row_grid, e->x, pending, pending_splits, split_stride, e->n1g[l], e->n1b[l], e->nrm, e->params, tpad);
+        GemmArgs g{};
+        g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->qkv[l]->data); g.M = tpad; g.N = 3 * w; g.K = w;
+        g.out = e->qk; g.vt = e->vt; g.width = w; g.vt_stride = vt_stride;
+        if (launch_gemm<ENC_QKV>(st, g, 1, error, capacity) != 0) return -1;
+        hipLaunchKernelGGL(k_enc_attention, dim3(tpad / kQTile, (unsigned)e->heads), dim3(kThreads), lds, st->stream, e->qk, e->vt, e->ctx, e->params,
+                           tpad, w, vt_stride, scale);
+        g = GemmArgs{};
+        g.a = e->ctx; g.w = static_cast<const _Float16 *>(e->o[l]->data); g.M = tpad; g.N = w; g.K = w; g.part = e->part;
+        if (launch_gemm<ENC_PARTIAL>(st, g, o_splits, error, capacity) != 0) return -1;
+        launch_rows<true>(st, w, row_grid, e->x, e->part, o_splits, split_stride, e->n2g[l], e->n2b[l], e->nrm, e->params, tpad);
+        g = GemmArgs{};
+        g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->up[l]->data); g.M = tpad; g.N = f; g.K = w; g.out = e->hid;
+        if (launch_gemm<ENC_GELU>(st, g, 1, error, capacity) != 0) return -1;
+        g = GemmArgs{};
+        g.a = e->hid; g.w = static_cast<const _Float16 *>(e->down[l]->data); g.M = tpad; g.N = w; g.K = f; g.part = e->part;
+        if (launch_gemm<ENC_PARTIAL>(st, g, down_splits, error, capacity) != 0) return -1;
+        pending = e->part;
+        pending_splits = down_splits;
+    }
+    // last residual update, then the final norm (src/graph.c:696-701) or a plain copy when the stack has none
+    launch_rows<false>(st, w, row_grid, e->x, pending, pending_splits, split_stride, e->nog, e->nob, nullptr, e->params, tpad);
+    return hip_check(hipGetLastError(), "encoder prefill launch", error, capacity);
+}
+
 }  // namespace
 
 extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_desc *d, mynah_hip_encoder **out, char *error, size_t capacity) {
@@ -317,7 +467,7 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
     }
     if (d->layers == 0 || d->width == 0 || d->heads == 0 || d->heads * d->head_width != d->width || d->head_width != 64 ||
         d->width % kTile != 0 || d->ffn_width % kTile != 0 || d->ffn_width == 0 || d->vocab == 0 || d->max_positions == 0 ||
-        d->width > 8192 || d->ffn_width > 32768 || d->max_positions > 4096 || d->tok_table == nullptr || d->pos_table == nullptr ||
+        d->width > 4096 || d->ffn_width > 32768 || d->max_positions > 4096 || d->tok_table == nullptr || d->pos_table == nullptr ||
         d->qkv_w == nullptr || d->o_w == nullptr || d->up_w == nullptr || d->down_w == nullptr || d->norm1 == nullptr || d->norm2 == nullptr) {
         set_error(error, capacity, "encoder_create: unsupported shape (needs 64-wide heads, widths that are multiples of 64) or missing weights");
         return -1;
@@ -373,10 +523,13 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
     if (alloc(reinterpret_cast<void **>(&e->x), tp * w * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->nrm), tp * w * 2) != 0 ||
         alloc(reinterpret_cast<void **>(&e->qk), tp * 2 * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->vt), w * tp * 2) != 0 ||
         alloc(reinterpret_cast<void **>(&e->ctx), tp * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->hid), tp * f * 2) != 0 ||
-        alloc(reinterpret_cast<void **>(&e->ids), tp * sizeof(int)) != 0)
+        alloc(reinterpret_cast<void **>(&e->ids), tp * sizeof(int) + sizeof(EncParams)) != 0 ||
+        alloc(reinterpret_cast<void **>(&e->part), kMaxSplits * tp * w * sizeof(float)) != 0)
         return fail();
-    if (hip_check(hipHostMalloc(reinterpret_cast<void **>(&e->ids_host), tp * sizeof(int), hipHostMallocDefault), "encoder ids staging", error, capacity) != 0)
+    if (hip_check(hipHostMalloc(reinterpret_cast<void **>(&e->ids_host), tp * sizeof(int) + sizeof(EncParams), hipHostMallocDefault),
+                  "encoder ids staging", error, capacity) != 0)
         return fail();
+    e->params = reinterpret_cast<EncParams *>(e->ids + tp);   // tp is a multiple of 64: 8-byte aligned
     if (attention_lds_bytes(e->tpad_max) > 48 * 1024 &&
         hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_enc_attention), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       (int)attention_lds_bytes(e->tpad_max)), "encoder attention LDS size", error, capacity) != 0)
@@ -390,7 +543,9 @@ extern "C" void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *e) {
     State *st = static_cast<State *>(state);
     if (e == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
-    for (void *p : {(void *)e->x, (void *)e->nrm, (void *)e->qk, (void *)e->vt, (void *)e->ctx, (void *)e->hid, (void *)e->ids})
+    for (auto &g : e->graphs)
+        if (g.second != nullptr) (void)hipGraphExecDestroy(g.second);
+    for (void *p : {(void *)e->x, (void *)e->nrm, (void *)e->qk, (void *)e->vt, (void *)e->ctx, (void *)e->hid, (void *)e->ids, (void *)e->part})
         if (p != nullptr) (void)hipFree(p);
     if (e->ids_host != nullptr) (void)hipHostFree(e->ids_host);
     delete e;
@@ -415,40 +570,38 @@ extern "C" int mynah_hip_encoder_prefill(void *state, mynah_hip_encoder *e, cons
     }
     // the staging buffer of the previous call may still be in flight
     MYNAH_TRY(hipStreamSynchronize(st->stream));
+    const size_t tp = e->tpad_max;
     for (size_t t = 0; t < tokens; ++t) e->ids_host[t] = ids[t];
+    EncParams *hp = reinterpret_cast<EncParams *>(e->ids_host + tp);
+    hp->tokens = (int)tokens;
+    hp->reserved = 0;
+    hp->embed_out = dev_embed_f16;
+    hp->out = dev_out;
     MYNAH_TRY(hipMemcpyAsync(e->ids, e->ids_host, tokens * sizeof(int), hipMemcpyHostToDevice, st->stream));
+    MYNAH_TRY(hipMemcpyAsync(e->params, hp, sizeof(EncParams), hipMemcpyHostToDevice, st->stream));
 
-    const int T = (int)tokens, w = (int)e->width, f = (int)e->ffn;
-    const int tpad = (T + kTile - 1) / kTile * kTile;
-    const int vt_stride = (int)e->tpad_max;
-    hipLaunchKernelGGL(k_enc_embed, dim3(tpad), dim3(kThreads), 0, st->stream, e->ids, static_cast<const _Float16 *>(e->tok->data),
-                       static_cast<const _Float16 *>(e->pos->data), e->x, dev_embed_f16, T, w);
-    const dim3 ln_grid((tpad + 3) / 4);
-    const float scale = 1.0f / sqrtf((float)e->head_width);
-    const size_t lds = attention_lds_bytes((size_t)tpad);
-    for (size_t l = 0; l < e->layers; ++l) {
-        hipLaunchKernelGGL((k_enc_layernorm<true>), ln_grid, dim3(kThreads), 0, st->stream, e->x, e->n1g[l], e->n1b[l], (void *)e->nrm, tpad, w);
-        GemmArgs g{};
-        g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->qkv[l]->data); g.M = tpad; g.N = 3 * w; g.K = w;
-        g.out = e->qk; g.vt = e->vt; g.width = w; g.vt_stride = vt_stride;
-        if (launch_gemm<ENC_QKV>(st, g, error, capacity) != 0) return -1;
-        hipLaunchKernelGGL(k_enc_attention, dim3(tpad / kQTile, (unsigned)e->heads), dim3(kThreads), lds, st->stream, e->qk, e->vt, e->ctx, T, tpad,
-                           w, vt_stride, scale);
-        g = GemmArgs{};
-        g.a = e->ctx; g.w = static_cast<const _Float16 *>(e->o[l]->data); g.M = tpad; g.N = w; g.K = w; g.x = e->x;
-        if (launch_gemm<ENC_RESIDUAL>(st, g, error, capacity) != 0) return -1;
-        hipLaunchKernelGGL((k_enc_layernorm<true>), ln_grid, dim3(kThreads), 0, st->stream, e->x, e->n2g[l], e->n2b[l], (void *)e->nrm, tpad, w);
-        g = GemmArgs{};
-        g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->up[l]->data); g.M = tpad; g.N = f; g.K = w; g.out = e->hid;
-        if (launch_gemm<ENC_GELU>(st, g, error, capacity) != 0) return -1;
-        g = GemmArgs{};
-        g.a = e->hid; g.w = static_cast<const _Float16 *>(e->down[l]->data); g.M = tpad; g.N = w; g.K = f; g.x = e->x;
-        if (launch_gemm<ENC_RESIDUAL>(st, g, error, capacity) != 0) return -1;
+    const int tpad = ((int)tokens + kTile - 1) / kTile * kTile;
+    if (!st->graph_mode || e->eager_runs[tpad] == 0) {
+        e->eager_runs[tpad] = 1;
+        return enqueue_prefill(st, e, tpad, error, capacity);
     }
-    if (e->nog != nullptr) {
-        hipLaunchKernelGGL((k_enc_layernorm<false>), dim3((T + 3) / 4), dim3(kThreads), 0, st->stream, e->x, e->nog, e->nob, (void *)dev_out, T, w);
-    } else {
-        MYNAH_TRY(hipMemcpyAsync(dev_out, e->x, (size_t)T * w * sizeof(float), hipMemcpyDeviceToDevice, st->stream));
+    hipGraphExec_t &exec = e->graphs[tpad];
+    if (exec == nullptr) {
+        hipGraph_t graph = nullptr;
+        MYNAH_TRY(hipStreamBeginCapture(st->stream, hipStreamCaptureModeThreadLocal));
+        const int rc = enqueue_prefill(st, e, tpad, error, capacity);
+        const hipError_t end = hipStreamEndCapture(st->stream, &graph);
+        if (rc != 0 || end != hipSuccess) {
+            if (graph != nullptr) (void)hipGraphDestroy(graph);
+            if (rc == 0) (void)hip_check(end, "encoder graph capture", error, capacity);
+            return -1;
+        }
+        const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        if (hip_check(inst, "encoder graph instantiate", error, capacity) != 0) {
+            exec = nullptr;
+            return -1;
+        }
     }
-    return hip_check(hipGetLastError(), "encoder prefill launch", error, capacity);
+    return hip_check(hipGraphLaunch(exec, st->stream), "encoder graph launch", error, capacity);
 }
