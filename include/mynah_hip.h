@@ -242,6 +242,22 @@ int mynah_hip_output_head(void *state, const float *const *dev_hidden, size_t ba
                           const float *weight, const float *bias, size_t rows, size_t vocab,
                           float *const *dev_logits, float *const *dev_probs, char *error, size_t error_capacity);
 
+/* Measurement helper (no counterpart in the reference): enqueue one stage of the step -- all layers, as its own
+ * captured graph, with the slot table of the last mynah_hip_decoder_step of this batch size -- so that a caller can
+ * time that kernel alone in the step's own setting between mynah_hip_timer_begin / _end.  Overwrites the decoder's
+ * workspaces like a step does. */
+enum {
+    MYNAH_HIP_STAGE_SELF_ATTENTION = 0,   /* LN + Q/K/V rows + KV append + self-attention partials */
+    MYNAH_HIP_STAGE_SELF_OUT = 1,         /* fold + O matvec + residual */
+    MYNAH_HIP_STAGE_CROSS_ATTENTION = 2,  /* LN + Q rows + cross-attention partials */
+    MYNAH_HIP_STAGE_CROSS_OUT = 3,        /* fold + O matvec + residual */
+    MYNAH_HIP_STAGE_FFN_UP = 4,           /* LN + up matvec + GELU */
+    MYNAH_HIP_STAGE_FFN_DOWN = 5,         /* down matvec + residual */
+    MYNAH_HIP_STAGE_COUNT = 6
+};
+int mynah_hip_decoder_stage_enqueue(void *state, mynah_hip_decoder *decoder, size_t batch, int stage,
+                                    char *error, size_t error_capacity);
+
 /* ---- text-encoder prefill (dense, MFMA) --------------------------------------------------- */
 
 typedef struct {

@@ -109,6 +109,7 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_decoder_destroy.restype = None
     lib.mynah_hip_decoder_step.argtypes = [_vp, _vp, C.POINTER(DecoderSlot), _sz, *_err]
     lib.mynah_hip_output_head.argtypes = [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _vp, *_err]
+    lib.mynah_hip_decoder_stage_enqueue.argtypes = [_vp, _vp, _sz, C.c_int, *_err]
     lib.mynah_hip_encoder_create.argtypes = [_vp, C.POINTER(EncoderDesc), C.POINTER(_vp), *_err]
     lib.mynah_hip_encoder_destroy.argtypes = [_vp, _vp]
     lib.mynah_hip_encoder_destroy.restype = None
@@ -379,6 +380,10 @@ class Decoder:
             arr[i] = DecoderSlot(s["k"], s["v"], s.get("ck"), s.get("cv"), s["length"], s.get("memory_length", 0),
                                  s["inp"], s["out"])
         self.backend._call("mynah_hip_decoder_step", self.handle, arr, _sz(B))
+
+    def stage_enqueue(self, batch, stage):
+        """Measurement helper: one stage of the step (all layers) as its own graph, see mynah_hip_decoder_stage_enqueue."""
+        self.backend._call("mynah_hip_decoder_stage_enqueue", self.handle, _sz(batch), C.c_int(stage))
 
     def destroy(self):
         if self.handle:

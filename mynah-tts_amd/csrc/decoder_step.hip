@@ -44,6 +44,7 @@ struct mynah_hip_decoder {
     bool fused_attention = false;
     hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};
     int eager_steps[mynah::kMaxBatch + 1] = {};   // a batch size runs eagerly once before it is captured
+    hipGraphExec_t stage_graphs[MYNAH_HIP_STAGE_COUNT][mynah::kMaxBatch + 1] = {};   // single-stage graphs (measurement only)
     int arith = 0;
 };
 
@@ -149,21 +150,33 @@ static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_
 }
 
 // The layer loop; everything here is replayable (no per-step scalars in kernel arguments).
-static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char *error, size_t capacity) {
+// `stages` selects which of the six per-layer stages are enqueued (bit MYNAH_HIP_STAGE_*); the step itself
+// passes kAllStages, the per-stage timing entry one bit at a time.
+constexpr unsigned kAllStages = 0x3fu;
+
+static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char *error, size_t capacity, unsigned stages = kAllStages) {
     const size_t w = d->width;
+    const auto on = [stages](int stage) { return (stages >> stage) & 1u; };
     if (d->fused_attention) {
         for (size_t l = 0; l < d->layers; ++l) {
             const LayerWeights &lw = d->lw[l];
-            if (enqueue_step_attention(st, d, 1, l, batch, lw.qkv, lw.norm_self, lw.norm_self_b, error, capacity) != 0) return -1;
+            if (on(MYNAH_HIP_STAGE_SELF_ATTENTION) &&
+                enqueue_step_attention(st, d, 1, l, batch, lw.qkv, lw.norm_self, lw.norm_self_b, error, capacity) != 0) return -1;
             const bool consumer_fold = batch <= kConsumerFoldMaxBatch;
-            if (enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 1 : 0) != 0) return -1;
+            if (on(MYNAH_HIP_STAGE_SELF_OUT) &&
+                enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 1 : 0) != 0) return -1;
             if (d->xw != 0) {
-                if (enqueue_step_attention(st, d, 0, l, batch, lw.q_cross, lw.norm_cross, lw.norm_cross_b, error, capacity) != 0) return -1;
-                if (enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 2 : 0) != 0) return -1;
+                if (on(MYNAH_HIP_STAGE_CROSS_ATTENTION) &&
+                    enqueue_step_attention(st, d, 0, l, batch, lw.q_cross, lw.norm_cross, lw.norm_cross_b, error, capacity) != 0) return -1;
+                if (on(MYNAH_HIP_STAGE_CROSS_OUT) &&
+                    enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 2 : 0) != 0) return -1;
             }
-            if (enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity) != 0) return -1;
-            if (enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
+            if (on(MYNAH_HIP_STAGE_FFN_UP) &&
+                enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity) != 0) return -1;
+            if (on(MYNAH_HIP_STAGE_FFN_DOWN) &&
+                enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
         }
+        if (stages != kAllStages) return 0;
         return launch_step_end(st, d->dev_slots, batch, w, d->x, w, d->norm_out, d->norm_out_b, error, capacity);
     }
     for (size_t l = 0; l < d->layers; ++l) {
@@ -199,6 +212,9 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
     for (auto &g : d->graphs)
         if (g != nullptr) (void)hipGraphExecDestroy(g);
+    for (auto &row : d->stage_graphs)
+        for (auto &g : row)
+            if (g != nullptr) (void)hipGraphExecDestroy(g);
     float *bufs[] = {d->x, d->qkv, d->attn, d->qx, d->ctx, d->hidden, d->partial, d->partial_ml};
     for (float *p : bufs)
         if (p != nullptr) (void)hipFree(p);
@@ -362,4 +378,45 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
         MYNAH_TRY(inst);
     }
     return hip_check(hipGraphLaunch(d->graphs[B], st->stream), "graph launch", error, capacity);
+}
+
+// Measurement helper: enqueue ONE stage of the step (all layers, back to back, as its own captured graph) on the
+// backend's stream, reusing the slot table of the last mynah_hip_decoder_step with this batch size.  The kernels,
+// their arguments and their order among themselves are those of the real step; only the other stages are left out,
+// so a caller can bracket a loop of these with mynah_hip_timer_begin / _end and get that kernel's launch time in the
+// step's own setting (dependent graph nodes, weights and caches coming from HBM).  It perturbs the decoder's
+// workspaces (x, hidden) like a step does and is not part of the decode path.
+extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *d, size_t batch, int stage, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    if (st == nullptr || d == nullptr || batch == 0 || batch > (size_t)kMaxBatch || stage < 0 || stage >= MYNAH_HIP_STAGE_COUNT) {
+        set_error(error, capacity, "invalid stage arguments");
+        return -1;
+    }
+    if (!d->fused_attention || d->eager_steps[batch] == 0) {
+        set_error(error, capacity, "stage timing needs the fused step and one earlier step with this batch size");
+        return -1;
+    }
+    if ((stage == MYNAH_HIP_STAGE_CROSS_ATTENTION || stage == MYNAH_HIP_STAGE_CROSS_OUT) && d->xw == 0) {
+        set_error(error, capacity, "decoder has no cross-attention sublayer");
+        return -1;
+    }
+    hipGraphExec_t &exec = d->stage_graphs[stage][batch];
+    if (exec == nullptr) {
+        hipGraph_t graph = nullptr;
+        MYNAH_TRY(hipStreamBeginCapture(st->stream, hipStreamCaptureModeThreadLocal));
+        const int rc = enqueue_layers(st, d, (int)batch, error, capacity, 1u << stage);
+        const hipError_t end = hipStreamEndCapture(st->stream, &graph);
+        if (rc != 0) {
+            if (graph != nullptr) (void)hipGraphDestroy(graph);
+            return -1;
+        }
+        MYNAH_TRY(end);
+        const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(graph);
+        if (hip_check(inst, "stage graph instantiate", error, capacity) != 0) {
+            exec = nullptr;
+            return -1;
+        }
+    }
+    return hip_check(hipGraphLaunch(exec, st->stream), "stage graph launch", error, capacity);
 }

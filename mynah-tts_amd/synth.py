@@ -112,4 +112,10 @@ def decoder_step_bytes(cfg, qtype, lengths, memory_lengths):
     for length, mem in zip(lengths, memory_lengths):
         kv += L * 2 * (length + 1) * w * 4      # rows [0, length] incl. the appended one
         kv += L * 2 * mem * xw * 4
-    return {"weights": weights, "kv": kv, "total": weights + kv}
+    # the same bytes split by stage kernel, per launch (one layer): order of the MYNAH_HIP_STAGE_* values
+    self_kv = sum(2 * (n + 1) * w * 4 for n in lengths)
+    cross_kv = sum(2 * m * xw * 4 for m in memory_lengths)
+    stages = [weight_bytes(3 * w, w, qtype) + self_kv, weight_bytes(w, w, qtype),
+              (weight_bytes(xw, w, qtype) + cross_kv) if xw else 0, weight_bytes(w, xw, qtype) if xw else 0,
+              weight_bytes(f, w, qtype), weight_bytes(w, f, qtype)]
+    return {"weights": weights, "kv": kv, "total": weights + kv, "stage_bytes_per_launch": stages}
