@@ -7,12 +7,14 @@
 //     LayerNorm(x) -> int8 activation quantisation -> this head's 64 rows of the Q projection
 //     -> scores against one 128-row unit of the K cache -> unit softmax statistics -> weighted V rows
 //     -> partial (max, sum, output[64]) to a workspace.
-// Units of a stream: its cache chunks, plus -- for self-attention -- one "new row" unit that also
-// computes this head's K and V rows of the step, appends them to the cache (src/graph.c:3180-3181) and
-// contributes the new row's own score.  The next kernel (the output projection) folds the partials in
-// its prologue, so no fence, atomic or second pass is needed here.  How a stream is cut into units
-// depends on its own length only, and a unit's arithmetic on nothing but its own inputs, so a stream in
-// a batch is bit-identical to the same stream alone.
+// Units of a stream: its cache chunks, plus -- for self-attention -- the step's new row, whose work is
+// split over two workgroups with fixed indices so that each can request all of its weight rows before
+// anything else has arrived: workgroup 0 computes this head's Q and K rows, appends K
+// (src/graph.c:3180-3181) and contributes the new row's own score; workgroup 1 computes the V row,
+// appends it and contributes it as that partial's output.  The next kernel (the output projection) folds
+// the partials in its prologue, so no fence, atomic or second pass is needed here.  How a stream is cut
+// into units depends on its own length only, and a unit's arithmetic on nothing but its own inputs, so a
+// stream in a batch is bit-identical to the same stream alone.
 //
 // The LayerNorm/quantisation is recomputed per workgroup (3 KB of input), and the 64 x 768 weight slice
 // of a head is read by every unit of that head.  Work items are ordered head-major and cut into eight
@@ -31,7 +33,8 @@ constexpr int kHw = 64;                          // head width handled by the fu
 constexpr int kPosLanes = 16;                    // lanes cooperating on one cache row
 constexpr int kPosPerPass = kThreads / kPosLanes;
 constexpr int kRowsPerThread = kStepUnitRows / kPosPerPass;   // 8
-constexpr int kPrefetchPasses = 4;
+constexpr int kPrefetchPasses = 4;    // passes of weight rows per register bank: one bank in flight for a cache-chunk or V
+                                      // workgroup, two for the Q+K workgroup of the new row (twice the rows)
 
 struct PassRegs {
     uint4 wv[4];
@@ -58,41 +61,59 @@ __device__ __forceinline__ void load_pass(PassRegs &p, const StepAttnArgs &a, in
     }
 }
 
-// Projection rows [row0, row0 + nrows) of this head (row numbering of weight_row) -> s_proj.
-// `pre` holds the first kPrefetchPasses passes when `preloaded`.
+// Requests passes [pass0, pass0 + kPrefetchPasses) of rows [row0, row0 + nrows) into `bank`.
 template <int QT>
-__device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&pre)[kPrefetchPasses], bool preloaded, int row0, int nrows,
+__device__ __forceinline__ void load_bank(PassRegs (&bank)[kPrefetchPasses], const StepAttnArgs &a, int pass0, int row0, int nrows, int head,
+                                          int lg, int chunks) {
+    const int rpp = 64 >> lg;
+    const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
+#pragma unroll
+    for (int p = 0; p < kPrefetchPasses; ++p)
+        if (pass0 + p < passes) load_pass<QT>(bank[p], a, pass0 + p, row0, nrows, head, lg, chunks);
+}
+
+// Passes [pass0, pass0 + kPrefetchPasses) of the projection rows [row0, row0 + nrows) of this head (row numbering
+// of weight_row), whose weights are in `bank` -> s_proj.
+template <int QT>
+__device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRegs (&bank)[kPrefetchPasses], int pass0, int row0, int nrows,
                                              int head, int lg, int chunks, const unsigned char *smem, const float sx, float *s_proj) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int G = 1 << lg, gl = lane & (G - 1), gidx = lane >> lg;
     const int rpp = 64 >> lg;
     const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
-    for (int pb = 0; pb < passes; pb += kPrefetchPasses) {
-        if (pb > 0 || !preloaded) {
 #pragma unroll
-            for (int p = 0; p < kPrefetchPasses; ++p)
-                if (pb + p < passes) load_pass<QT>(pre[p], a, pb + p, row0, nrows, head, lg, chunks);
-        }
+    for (int p = 0; p < kPrefetchPasses; ++p) {
+        const int pass = pass0 + p;
+        if (pass < passes) {
+            const int r = row0 + pass * 4 * rpp + wave * rpp + gidx;
+            int iacc[1] = {0};
+            float facc[1] = {0.0f};
 #pragma unroll
-        for (int p = 0; p < kPrefetchPasses; ++p) {
-            const int pass = pb + p;
-            if (pass < passes) {
-                const int r = row0 + pass * 4 * rpp + wave * rpp + gidx;
-                int iacc[1] = {0};
-                float facc[1] = {0.0f};
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int c = gl + u * G;
-                    if (c < chunks) dot_chunk<QT, 1>(pre[p].wv[u], pre[p].sc[u], c, smem, a.width, iacc, facc, nullptr);
-                }
-                group_reduce<QT, 1>(iacc, facc, lg);
-                if (gl == 0 && r < row0 + nrows) {
-                    float wscale = 1.0f;
-                    if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[weight_row(r, head, a.width)];
-                    s_proj[r] = finish_value<QT>(iacc[0], facc[0], wscale, sx);
-                }
+            for (int u = 0; u < 4; ++u) {
+                const int c = gl + u * G;
+                if (c < chunks) dot_chunk<QT, 1>(bank[p].wv[u], bank[p].sc[u], c, smem, a.width, iacc, facc, nullptr);
+            }
+            group_reduce<QT, 1>(iacc, facc, lg);
+            if (gl == 0 && r < row0 + nrows) {
+                float wscale = 1.0f;
+                if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[weight_row(r, head, a.width)];
+                s_proj[r] = finish_value<QT>(iacc[0], facc[0], wscale, sx);
             }
         }
+    }
+}
+
+// Projection rows [row0, row0 + nrows): passes [0, kPrefetchPasses) are in `bank` on entry, those from `next_pass`
+// on are fetched here, a bank at a time.
+template <int QT>
+__device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&bank)[kPrefetchPasses], int next_pass, int row0, int nrows,
+                                             int head, int lg, int chunks, const unsigned char *smem, const float sx, float *s_proj) {
+    const int rpp = 64 >> lg;
+    const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
+    project_bank<QT>(a, bank, 0, row0, nrows, head, lg, chunks, smem, sx, s_proj);
+    for (int pb = next_pass; pb < passes; pb += kPrefetchPasses) {
+        load_bank<QT>(bank, a, pb, row0, nrows, head, lg, chunks);
+        project_bank<QT>(a, bank, pb, row0, nrows, head, lg, chunks, smem, sx, s_proj);
     }
 }
 
@@ -109,32 +130,36 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const int tid = threadIdx.x;
     const StepSlots *slots = a.slots;
 
-    // ---- static work decode: item = (head * batch + stream) * max_units + unit, XCD x owns items [x*per_xcd, (x+1)*per_xcd)
-    const int items = a.heads * a.batch * a.max_units;
+    // ---- static work decode: item = (head * batch + stream) * wg_units + unit, XCD x owns items [x*per_xcd, (x+1)*per_xcd).
+    // Self-attention: unit 0 = Q+K of the new row, unit 1 = V of the new row, unit 2 + c = cache chunk c.
+    const int wg_units = a.max_units + (a.is_self ? 1 : 0);
+    const int items = a.heads * a.batch * wg_units;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int item = xcd * per_xcd + slot;
     if (slot >= per_xcd || item >= items) return;
-    const int unit = item % a.max_units;
-    const int hb = item / a.max_units;
+    const int unit = item % wg_units;
+    const int hb = item / wg_units;
     const int b = hb % a.batch;
     const int head = hb / a.batch;
+    const bool role_qk = a.is_self && unit == 0;
+    const bool role_v = a.is_self && unit == 1;
+    const int chunk = a.is_self ? unit - 2 : unit;   // cache chunk of this workgroup (chunk roles only)
+    const int pidx = a.is_self ? unit - 1 : unit;    // partial slot written by a chunk role (slot 0 = the new row)
 
     constexpr int kEpc = Chunk<QT>::n;
     const int chunks = a.width / kEpc;
 
-    // ---- requests that need neither activations nor the slot table: the head's Q weight rows
+    // ---- requests that need neither activations nor the slot table: this role's weight rows
     PassRegs pre[kPrefetchPasses];
-    const int rpp = 64 >> lg;
-    const int q_passes = (kHw + 4 * rpp - 1) / (4 * rpp);
-#pragma unroll
-    for (int p = 0; p < kPrefetchPasses; ++p)
-        if (p < q_passes) load_pass<QT>(pre[p], a, p, 0, kHw, head, lg, chunks);
+    if (role_qk) load_bank<QT>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
+    else if (role_v) load_bank<QT>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
+    else load_bank<QT>(pre, a, 0, 0, kHw, head, lg, chunks);
 
     // ---- slot table: is this unit live, and where are its cache rows?
-    const int units_b = attention_units(slots, b, a.is_self);
-    if (unit >= units_b) return;
     const int length = a.is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
-    const bool new_row = a.is_self && unit == units_b - 1;
+    const int nchunks = (length + kStepUnitRows - 1) / kStepUnitRows;
+    const bool new_row = role_qk || role_v;
+    if (!new_row && chunk >= (a.is_self ? nchunks : max(nchunks, 1))) return;
     const int stride = a.heads * kHw;   // floats between cache rows
     float *kc, *vc;
     if (a.is_self) {
@@ -147,15 +172,41 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const int j = tid & (kPosLanes - 1);
     const int g = tid / kPosLanes;
     const size_t col = (size_t)head * kHw + 4 * j;
-    const int p0 = unit * kStepUnitRows;
+    const int p0 = chunk * kStepUnitRows;
     const int count = new_row ? 0 : max(0, min(kStepUnitRows, length - p0));
+    // A chunk role keeps its cache rows here.  The Q+K role has no cache rows and parks its second bank of weight
+    // passes in the same registers (as raw bits), so that no role needs more registers than the largest one.
+    static_assert(2 * kRowsPerThread == 4 * kPrefetchPasses, "the second weight bank must fit the cache-row registers");
     float4 kv[kRowsPerThread], vv[kRowsPerThread];
+    float sc2[4 * kPrefetchPasses];   // int4 only: group scales of the second bank
+    if (role_qk) {
+        PassRegs bank2[kPrefetchPasses];
 #pragma unroll
-    for (int i = 0; i < kRowsPerThread; ++i) {
-        const int pi = g + kPosPerPass * i;
-        const bool in_range = pi < count;
-        kv[i] = in_range ? *reinterpret_cast<const float4 *>(kc + (size_t)(p0 + pi) * stride + col) : make_float4(0.f, 0.f, 0.f, 0.f);
-        vv[i] = in_range ? *reinterpret_cast<const float4 *>(vc + (size_t)(p0 + pi) * stride + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int p = 0; p < kPrefetchPasses; ++p) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { bank2[p].wv[u] = make_uint4(0, 0, 0, 0); bank2[p].sc[u] = 0.0f; }
+        }
+        load_bank<QT>(bank2, a, kPrefetchPasses, 0, 2 * kHw, head, lg, chunks);
+#pragma unroll
+        for (int p = 0; p < kPrefetchPasses; ++p) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = 4 * p + u;
+                if (idx < kRowsPerThread) kv[idx] = __builtin_bit_cast(float4, bank2[p].wv[u]);
+                else vv[idx - kRowsPerThread] = __builtin_bit_cast(float4, bank2[p].wv[u]);
+                sc2[idx] = bank2[p].sc[u];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4 * kPrefetchPasses; ++i) sc2[i] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < kRowsPerThread; ++i) {
+            const int pi = g + kPosPerPass * i;
+            const bool in_range = pi < count;
+            kv[i] = in_range ? *reinterpret_cast<const float4 *>(kc + (size_t)(p0 + pi) * stride + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+            vv[i] = in_range ? *reinterpret_cast<const float4 *>(vc + (size_t)(p0 + pi) * stride + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     }
 
     // ---- LayerNorm + activation quantisation of x[b], staged in LDS
@@ -169,31 +220,61 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         stage_activations<QT, 1, NVT>(p, src, smem, s_sx, s_scratch);
     }
 
-    // ---- this head's projection rows -> s_proj (q always; k and v for the new-row unit)
-    project_rows<QT>(a, pre, true, 0, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
-    if (new_row) project_rows<QT>(a, pre, false, kHw, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
-    __syncthreads();
-
     const size_t sh = (size_t)b * a.heads + head;
     float *out_m = a.partial_ml + sh * 2 * a.max_units;
     float *out_l = out_m + a.max_units;
-    float *out_o = a.partial + (sh * a.max_units + unit) * kHw;
 
-    if (new_row) {
-        // append this step's k / v (this head's slice) and contribute the new row's own score
-        if (tid < kHw) kc[(size_t)length * stride + (size_t)head * kHw + tid] = s_proj[kHw + tid];
-        else if (tid < 2 * kHw) vc[(size_t)length * stride + (size_t)head * kHw + (tid - kHw)] = s_proj[2 * kHw + (tid - kHw)];
+    if (role_qk) {
+        // this head's q and k of the new row; append k; the new row's own score opens partial 0
+        {
+            PassRegs bank2[kPrefetchPasses];
+#pragma unroll
+            for (int p = 0; p < kPrefetchPasses; ++p) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int idx = 4 * p + u;
+                    bank2[p].wv[u] = __builtin_bit_cast(uint4, idx < kRowsPerThread ? kv[idx] : vv[idx - kRowsPerThread]);
+                    bank2[p].sc[u] = sc2[idx];
+                }
+            }
+            project_bank<QT>(a, pre, 0, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+            project_bank<QT>(a, bank2, kPrefetchPasses, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+            const int rpp = 64 >> lg;
+            const int passes = (2 * kHw + 4 * rpp - 1) / (4 * rpp);
+            for (int pb = 2 * kPrefetchPasses; pb < passes; pb += kPrefetchPasses) {   // more than eight passes: wide (f32 / f16) rows
+                load_bank<QT>(pre, a, pb, 0, 2 * kHw, head, lg, chunks);
+                project_bank<QT>(a, pre, pb, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+            }
+        }
+        __syncthreads();
         if (tid < 64) {
-            float d = s_proj[tid] * s_proj[kHw + tid];
+            const float kval = s_proj[kHw + tid];
+            kc[(size_t)length * stride + (size_t)head * kHw + tid] = kval;
+            float d = s_proj[tid] * kval;
             d = wave_sum(d);
-            out_o[tid] = s_proj[2 * kHw + tid];   // exp(score - max) = 1
-            if (tid == 0) { out_m[unit] = d * a.scale; out_l[unit] = 1.0f; }
+            if (tid == 0) { out_m[0] = d * a.scale; out_l[0] = 1.0f; }   // exp(score - max) = 1
         }
         return;
     }
+    if (role_v) {
+        // this head's v of the new row: appended, and the output of partial 0
+        project_rows<QT>(a, pre, kPrefetchPasses, 2 * kHw, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+        __syncthreads();
+        if (tid < kHw) {
+            const float vval = s_proj[2 * kHw + tid];
+            vc[(size_t)length * stride + (size_t)head * kHw + tid] = vval;
+            a.partial[sh * a.max_units * kHw + tid] = vval;
+        }
+        return;
+    }
+
+    // ---- cache chunk: this head's q, then the chunk's scores
+    project_rows<QT>(a, pre, kPrefetchPasses, 0, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+    __syncthreads();
+    float *out_o = a.partial + (sh * a.max_units + pidx) * kHw;
     if (count <= 0) {   // empty memory (cross only): the context stays zero (src/graph.c:3242)
         if (tid < kHw) out_o[tid] = 0.0f;
-        if (tid == 0) { out_m[unit] = 0.0f; out_l[unit] = 1.0f; }
+        if (tid == 0) { out_m[pidx] = 0.0f; out_l[pidx] = 1.0f; }
         return;
     }
 
@@ -247,7 +328,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 #pragma unroll
         for (int gg = 0; gg < kPosPerPass; ++gg) o += s_red[(size_t)gg * kHw + tid];
         out_o[tid] = o;
-        if (tid == 0) { out_m[unit] = s_ml[0]; out_l[unit] = s_ml[1]; }
+        if (tid == 0) { out_m[pidx] = s_ml[0]; out_l[pidx] = s_ml[1]; }
     }
 }
 
@@ -269,7 +350,7 @@ template <int QT>
 int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const int chunks = a.width / Chunk<QT>::n;
     const int lg = lane_group_log2(chunks);
-    const int items = a.heads * a.batch * a.max_units;
+    const int items = a.heads * a.batch * (a.max_units + (a.is_self ? 1 : 0));   // self: the new row takes two workgroups
     const int per_xcd = (items + 7) / 8;
     const int grid = 8 * per_xcd;
     const size_t lds = (size_t)a.width * (kQuantised<QT> ? 1 : 4);
