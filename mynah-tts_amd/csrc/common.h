@@ -21,6 +21,11 @@ constexpr size_t kQuantMaxRows = 16; // QMAT_SMALL_COUNT, src/qmat.c:32
 constexpr size_t kQuantMaxK = 8192;  // QMAT_K_MAX, src/qmat.c:33
 constexpr int kAttnChunk = 64;       // cache positions handled by one workgroup of the stand-alone attention kernels
 constexpr int kStepUnitRows = 128;   // cache rows per attention unit (workgroup) of the fused resident step
+// Up to this many streams the resident step is laid out for latency: the output projection folds the attention
+// partials itself and attention workgroups request their weights before looking at the slot table.  Above it a
+// separate fold kernel runs once (every workgroup folding every stream would outweigh one extra launch) and
+// workgroups of units a stream does not have leave before requesting anything.
+constexpr int kConsumerFoldMaxBatch = 2;
 
 // ---- error plumbing (0 / -1 + message, src/backend.c:137-139) ----
 inline void set_error(char *error, size_t capacity, const char *message) {

@@ -118,9 +118,6 @@ static int enqueue_attention(State *st, const mynah_hip_decoder *d, int is_self,
     return launch_attention(st, a, error, capacity);
 }
 
-// Up to this many streams the output projection folds the attention partials itself; above it a separate fold
-// kernel runs once (every workgroup folding every stream would outweigh one extra launch).
-constexpr int kConsumerFoldMaxBatch = 2;
 
 static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_self, size_t layer, int batch, const CachedWeight *w,
                                   const float *ln_gain, const float *ln_bias, char *error, size_t capacity) {

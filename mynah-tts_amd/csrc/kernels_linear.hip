@@ -31,6 +31,16 @@
 namespace mynah {
 namespace {
 
+// Output row pointer of stream b (b < BT, not known at compile time): a select chain over the kernel arguments.
+template <int BT>
+__device__ __forceinline__ float *stream_out(const LinearArgs &a, int b) {
+    float *o = a.out[0];
+#pragma unroll
+    for (int i = 1; i < BT; ++i)
+        if (b == i) o = a.out[i];
+    return o;
+}
+
 template <int QT, int BT, int NVT>
 __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const int rows_per_wg, const int lg) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -55,6 +65,9 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
     uint4 wv[4];
     float sc[4];
     float pre_scale = 1.0f, pre_bias = 0.0f, pre_res[BT];
+#pragma unroll
+    for (int b = 0; b < BT; ++b) pre_res[b] = 0.0f;
+    const bool lanes_finish = BT > 1 && G >= BT;
     {
         const int row = row_begin + wave * rows_per_pass + gidx;
         const int rowc = row < row_end ? row : row_end - 1;
@@ -65,7 +78,15 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
             wv[u] = c < chunks ? wrow[c] : make_uint4(0, 0, 0, 0);
             sc[u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? a.scales[(size_t)rowc * chunks + c] : 0.0f;
         }
-        if (gl == 0) {
+        // Epilogue operands.  One stream: lane 0 of a group finishes the row.  Several streams: lane b of a group
+        // finishes stream b (when the group has that many lanes), so the epilogues of a row run side by side.
+        if (lanes_finish) {
+            if (gl < BT) {
+                if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
+                if (a.bias != nullptr) pre_bias = a.bias[rowc];
+                if (a.epilogue == EPI_RESIDUAL && gl < a.batch) pre_res[0] = stream_out<BT>(a, gl)[rowc];
+            }
+        } else if (gl == 0) {
             if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
             if (a.bias != nullptr) pre_bias = a.bias[rowc];
 #pragma unroll
@@ -117,7 +138,30 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
             }
         }
         group_reduce<QT, BT>(iacc, facc, lg);
-        if (gl == 0 && valid) {
+        if (lanes_finish) {
+            if (gl < a.batch && valid) {
+                int mi = iacc[0];
+                float mf = facc[0];
+#pragma unroll
+                for (int b = 1; b < BT; ++b)
+                    if (gl == b) { mi = iacc[b]; mf = facc[b]; }
+                float wscale = 1.0f, bias = 0.0f;
+                if (first) {
+                    wscale = pre_scale;
+                    bias = pre_bias;
+                } else {
+                    if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[row];
+                    if (a.bias != nullptr) bias = a.bias[row];
+                }
+                float val = finish_value<QT>(mi, mf, wscale, s_sx[gl]);
+                if (QT == MYNAH_HIP_INT8 && a.probe_acc != nullptr && gl == 0) a.probe_acc[row] = mi;
+                if (a.bias != nullptr) val += bias;
+                if (a.epilogue == EPI_GELU) val = gelu_tanh(val);
+                float *o = stream_out<BT>(a, gl) + row;
+                if (a.epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : *o) + val;
+                *o = val;
+            }
+        } else if (gl == 0 && valid) {
             float wscale = 1.0f, bias = 0.0f;
             if (first) {
                 wscale = pre_scale;

@@ -149,6 +149,15 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     constexpr int kEpc = Chunk<QT>::n;
     const int chunks = a.width / kEpc;
 
+    // With many streams most of the grid belongs to units that short streams do not have: there the slot table is
+    // looked at first, so that such a workgroup leaves without having requested anything.  With one or two streams
+    // nearly every unit is live and the weight rows are requested before the table has arrived (latency matters more).
+    if (a.batch > kConsumerFoldMaxBatch && !(a.is_self && unit < 2)) {
+        const int len = a.is_self ? slots->length[b] : slots->memory_length[b];
+        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+        if (chunk >= (a.is_self ? live : max(live, 1))) return;
+    }
+
     // ---- requests that need neither activations nor the slot table: this role's weight rows
     PassRegs pre[kPrefetchPasses];
     if (role_qk) load_bank<QT>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
