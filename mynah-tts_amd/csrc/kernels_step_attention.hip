@@ -33,8 +33,11 @@ constexpr int kHw = 64;                          // head width handled by the fu
 constexpr int kPosLanes = 16;                    // lanes cooperating on one cache row
 constexpr int kPosPerPass = kThreads / kPosLanes;
 constexpr int kRowsPerThread = kStepUnitRows / kPosPerPass;   // 8
-constexpr int kPrefetchPasses = 4;    // passes of weight rows per register bank: one bank in flight for a cache-chunk or V
-                                      // workgroup, two for the Q+K workgroup of the new row (twice the rows)
+// PF = passes of weight rows per register bank: one bank is in flight for a cache-chunk or V workgroup, two for the
+// Q+K workgroup of the new row (twice the rows).  4 when one or two streams are stepped (every weight row of a head is
+// requested at once: shortest path), 2 for larger batches (fewer registers: three workgroups per CU instead of two,
+// which is what matters once there are more workgroups than the chip holds at a time).  The arithmetic is the same.
+constexpr int kPrefetchLatency = 4, kPrefetchThroughput = 2;
 
 struct PassRegs {
     uint4 wv[4];
@@ -61,28 +64,28 @@ __device__ __forceinline__ void load_pass(PassRegs &p, const StepAttnArgs &a, in
     }
 }
 
-// Requests passes [pass0, pass0 + kPrefetchPasses) of rows [row0, row0 + nrows) into `bank`.
-template <int QT>
-__device__ __forceinline__ void load_bank(PassRegs (&bank)[kPrefetchPasses], const StepAttnArgs &a, int pass0, int row0, int nrows, int head,
+// Requests passes [pass0, pass0 + PF) of rows [row0, row0 + nrows) into `bank`.
+template <int QT, int PF>
+__device__ __forceinline__ void load_bank(PassRegs (&bank)[PF], const StepAttnArgs &a, int pass0, int row0, int nrows, int head,
                                           int lg, int chunks) {
     const int rpp = 64 >> lg;
     const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
 #pragma unroll
-    for (int p = 0; p < kPrefetchPasses; ++p)
+    for (int p = 0; p < PF; ++p)
         if (pass0 + p < passes) load_pass<QT>(bank[p], a, pass0 + p, row0, nrows, head, lg, chunks);
 }
 
-// Passes [pass0, pass0 + kPrefetchPasses) of the projection rows [row0, row0 + nrows) of this head (row numbering
+// Passes [pass0, pass0 + PF) of the projection rows [row0, row0 + nrows) of this head (row numbering
 // of weight_row), whose weights are in `bank` -> s_proj.
-template <int QT>
-__device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRegs (&bank)[kPrefetchPasses], int pass0, int row0, int nrows,
+template <int QT, int PF>
+__device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRegs (&bank)[PF], int pass0, int row0, int nrows,
                                              int head, int lg, int chunks, const unsigned char *smem, const float sx, float *s_proj) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int G = 1 << lg, gl = lane & (G - 1), gidx = lane >> lg;
     const int rpp = 64 >> lg;
     const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
 #pragma unroll
-    for (int p = 0; p < kPrefetchPasses; ++p) {
+    for (int p = 0; p < PF; ++p) {
         const int pass = pass0 + p;
         if (pass < passes) {
             const int r = row0 + pass * 4 * rpp + wave * rpp + gidx;
@@ -103,21 +106,21 @@ __device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRe
     }
 }
 
-// Projection rows [row0, row0 + nrows): passes [0, kPrefetchPasses) are in `bank` on entry, those from `next_pass`
+// Projection rows [row0, row0 + nrows): passes [0, PF) are in `bank` on entry, those from `next_pass`
 // on are fetched here, a bank at a time.
-template <int QT>
-__device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&bank)[kPrefetchPasses], int next_pass, int row0, int nrows,
+template <int QT, int PF>
+__device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&bank)[PF], int next_pass, int row0, int nrows,
                                              int head, int lg, int chunks, const unsigned char *smem, const float sx, float *s_proj) {
     const int rpp = 64 >> lg;
     const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
-    project_bank<QT>(a, bank, 0, row0, nrows, head, lg, chunks, smem, sx, s_proj);
-    for (int pb = next_pass; pb < passes; pb += kPrefetchPasses) {
-        load_bank<QT>(bank, a, pb, row0, nrows, head, lg, chunks);
-        project_bank<QT>(a, bank, pb, row0, nrows, head, lg, chunks, smem, sx, s_proj);
+    project_bank<QT, PF>(a, bank, 0, row0, nrows, head, lg, chunks, smem, sx, s_proj);
+    for (int pb = next_pass; pb < passes; pb += PF) {
+        load_bank<QT, PF>(bank, a, pb, row0, nrows, head, lg, chunks);
+        project_bank<QT, PF>(a, bank, pb, row0, nrows, head, lg, chunks, smem, sx, s_proj);
     }
 }
 
-template <int QT, int NVT>
+template <int QT, int NVT, int PF>
 __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a, const int lg, const int per_xcd) {
     extern __shared__ __align__(16) unsigned char smem[];   // staged activations: width bytes (int8/int4) or floats
     __shared__ __align__(16) float s_proj[3 * kHw];         // q | k | v of this head
@@ -159,10 +162,10 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     }
 
     // ---- requests that need neither activations nor the slot table: this role's weight rows
-    PassRegs pre[kPrefetchPasses];
-    if (role_qk) load_bank<QT>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
-    else if (role_v) load_bank<QT>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
-    else load_bank<QT>(pre, a, 0, 0, kHw, head, lg, chunks);
+    PassRegs pre[PF];
+    if (role_qk) load_bank<QT, PF>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
+    else if (role_v) load_bank<QT, PF>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
+    else load_bank<QT, PF>(pre, a, 0, 0, kHw, head, lg, chunks);
 
     // ---- slot table: is this unit live, and where are its cache rows?
     const int length = a.is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
@@ -185,19 +188,19 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const int count = new_row ? 0 : max(0, min(kStepUnitRows, length - p0));
     // A chunk role keeps its cache rows here.  The Q+K role has no cache rows and parks its second bank of weight
     // passes in the same registers (as raw bits), so that no role needs more registers than the largest one.
-    static_assert(2 * kRowsPerThread == 4 * kPrefetchPasses, "the second weight bank must fit the cache-row registers");
+    static_assert(2 * kRowsPerThread >= 4 * PF, "the second weight bank must fit the cache-row registers");
     float4 kv[kRowsPerThread], vv[kRowsPerThread];
-    float sc2[4 * kPrefetchPasses];   // int4 only: group scales of the second bank
+    float sc2[4 * PF];   // int4 only: group scales of the second bank
     if (role_qk) {
-        PassRegs bank2[kPrefetchPasses];
+        PassRegs bank2[PF];
 #pragma unroll
-        for (int p = 0; p < kPrefetchPasses; ++p) {
+        for (int p = 0; p < PF; ++p) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) { bank2[p].wv[u] = make_uint4(0, 0, 0, 0); bank2[p].sc[u] = 0.0f; }
         }
-        load_bank<QT>(bank2, a, kPrefetchPasses, 0, 2 * kHw, head, lg, chunks);
+        load_bank<QT, PF>(bank2, a, PF, 0, 2 * kHw, head, lg, chunks);
 #pragma unroll
-        for (int p = 0; p < kPrefetchPasses; ++p) {
+        for (int p = 0; p < PF; ++p) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int idx = 4 * p + u;
@@ -208,7 +211,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < 4 * kPrefetchPasses; ++i) sc2[i] = 0.0f;
+        for (int i = 0; i < 4 * PF; ++i) sc2[i] = 0.0f;
 #pragma unroll
         for (int i = 0; i < kRowsPerThread; ++i) {
             const int pi = g + kPosPerPass * i;
@@ -236,9 +239,9 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     if (role_qk) {
         // this head's q and k of the new row; append k; the new row's own score opens partial 0
         {
-            PassRegs bank2[kPrefetchPasses];
+            PassRegs bank2[PF];
 #pragma unroll
-            for (int p = 0; p < kPrefetchPasses; ++p) {
+            for (int p = 0; p < PF; ++p) {
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int idx = 4 * p + u;
@@ -246,13 +249,13 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
                     bank2[p].sc[u] = sc2[idx];
                 }
             }
-            project_bank<QT>(a, pre, 0, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
-            project_bank<QT>(a, bank2, kPrefetchPasses, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+            project_bank<QT, PF>(a, pre, 0, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+            project_bank<QT, PF>(a, bank2, PF, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
             const int rpp = 64 >> lg;
             const int passes = (2 * kHw + 4 * rpp - 1) / (4 * rpp);
-            for (int pb = 2 * kPrefetchPasses; pb < passes; pb += kPrefetchPasses) {   // more than eight passes: wide (f32 / f16) rows
-                load_bank<QT>(pre, a, pb, 0, 2 * kHw, head, lg, chunks);
-                project_bank<QT>(a, pre, pb, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+            for (int pb = 2 * PF; pb < passes; pb += PF) {   // passes beyond the two banks (wide f32 / f16 rows, or the two-pass banks)
+                load_bank<QT, PF>(pre, a, pb, 0, 2 * kHw, head, lg, chunks);
+                project_bank<QT, PF>(a, pre, pb, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
             }
         }
         __syncthreads();
@@ -267,7 +270,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     }
     if (role_v) {
         // this head's v of the new row: appended, and the output of partial 0
-        project_rows<QT>(a, pre, kPrefetchPasses, 2 * kHw, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+        project_rows<QT, PF>(a, pre, PF, 2 * kHw, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
         __syncthreads();
         if (tid < kHw) {
             const float vval = s_proj[2 * kHw + tid];
@@ -278,7 +281,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     }
 
     // ---- cache chunk: this head's q, then the chunk's scores
-    project_rows<QT>(a, pre, kPrefetchPasses, 0, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+    project_rows<QT, PF>(a, pre, PF, 0, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
     __syncthreads();
     float *out_o = a.partial + (sh * a.max_units + pidx) * kHw;
     if (count <= 0) {   // empty memory (cross only): the context stays zero (src/graph.c:3242)
@@ -363,8 +366,14 @@ int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const int per_xcd = (items + 7) / 8;
     const int grid = 8 * per_xcd;
     const size_t lds = (size_t)a.width * (kQuantised<QT> ? 1 : 4);
-    if (a.width <= 1024) hipLaunchKernelGGL((k_step_attention<QT, 1>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
-    else hipLaunchKernelGGL((k_step_attention<QT, 3>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+    const bool latency = a.batch <= kConsumerFoldMaxBatch;
+    if (a.width <= 1024) {
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+    } else {
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+    }
     return hip_check(hipGetLastError(), "step attention launch", error, capacity);
 }
 
