@@ -194,3 +194,90 @@ def test_output_head(pkg, backend, orc, synth, nerr):
         for d in dh + dl + dp:
             d.free()
     backend.set_quant(0)
+
+
+@pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4"])
+@pytest.mark.parametrize("arith_name", ["strict", "stock"])
+def test_step_against_compiled_reference_fixture(pkg, backend, synth, nerr, qtype_name, arith_name):
+    """The GPU step against the committed outputs of the reference's own decoder_step_batch (tests/golden): its real head
+    shape -- gain-only LayerNorm, ONE 768-wide cross-attention head -- ragged batch of 8.  That head width is not the
+    fused attention kernel's, so this also covers the eight-kernel form of the step.  No oracle in between."""
+    import os
+    import zlib
+    _announce("step vs reference fixture %s %s" % (qtype_name, arith_name))
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.npz"), allow_pickle=False)
+    lengths = [int(n) for n in gold["step_lengths"]]
+    mems = [int(n) for n in gold["step_mems"]]
+    cfg = synth.decoder_config(layers=2, capacity=max(lengths) + 3, cross_heads=1)
+    weights = synth.decoder_weights(cfg, seed=0, ln_bias=False)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=1)
+    c = 0
+    for a in [weights[k] for k in sorted(weights) if weights[k] is not None] + [s[n] for s in streams for n in ("k", "v", "ck", "cv", "x")]:
+        c = zlib.crc32(np.ascontiguousarray(a).tobytes(), c)
+    if np.uint32(c) != gold["step_input_crc"]:
+        pytest.skip("numpy's generator produced different synthetic inputs than when the fixture was written")
+    backend.set_quant(QT[qtype_name], 0 if arith_name == "strict" else 1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    got = h.step()
+    tol = TOL[qtype_name]
+    for b in range(8):
+        assert nerr(got[b], gold["step_%s_%s_out" % (qtype_name, arith_name)][b]) < tol, "stream %d" % b
+        gk, gv = h.cache_rows(b)
+        assert nerr(gk[:, lengths[b]], gold["step_%s_%s_newk" % (qtype_name, arith_name)][b]) < tol
+        assert nerr(gv[:, lengths[b]], gold["step_%s_%s_newv" % (qtype_name, arith_name)][b]) < tol
+    h.close()
+    backend.set_quant(0)
+
+
+def test_batch16_two_tiles(pkg, backend, orc, synth, nerr):
+    """MYNAH_MAX_BATCH streams: two weight passes of eight streams each; oracle parity and batched == solo bitwise."""
+    _announce("one layer ragged b=16 int8")
+    rng = np.random.default_rng(16)
+    lengths = [int(n) for n in rng.integers(0, 200, size=16)]
+    mems = [int(n) for n in rng.integers(1, 70, size=16)]
+    cfg = synth.decoder_config(layers=1, capacity=204)
+    weights = synth.decoder_weights(cfg, seed=5)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=6)
+    backend.set_quant(1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    want, ks, vs = _oracle_step(orc, cfg, weights, streams, 1)
+    first = h.step()
+    for b in range(16):
+        assert nerr(first[b], want[b]) < TOL["int8"], "stream %d" % b
+    for b in range(16):
+        h.reset_cache(b)
+    again = h.step()                       # captured graph
+    for b in range(16):
+        assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32))
+    for b in (0, 7, 8, 15):
+        h.reset_cache(b)
+        solo = h.step([b])[0]
+        assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
+    h.close()
+    backend.set_quant(0)
+
+
+def test_stage_enqueue_leaves_the_step_intact(pkg, backend, synth):
+    """The per-stage timing entry replays single stages of the step; a full step afterwards gives the same bits as before."""
+    _announce("stage enqueue")
+    cfg = synth.decoder_config(layers=2, capacity=140)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, [130, 17, 64], [20, 33, 1], seed=1)
+    backend.set_quant(1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    with pytest.raises(pkg.BackendError):            # needs one earlier step with this batch size
+        h.dec.stage_enqueue(3, 0)
+    first = h.step()
+    for stage in range(6):
+        for _ in range(2):
+            h.dec.stage_enqueue(3, stage)
+    backend.sync()
+    with pytest.raises(pkg.BackendError):
+        h.dec.stage_enqueue(3, 6)
+    for b in range(3):
+        h.reset_cache(b)
+    again = h.step()
+    for b in range(3):
+        assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32))
+    h.close()
+    backend.set_quant(0)
