@@ -130,9 +130,11 @@ STAGES = [("self-attention", "k_step_attention: LayerNorm + int8 act-quant + per
           ("ffn-up", "k_linear: LayerNorm + act-quant + up matvec + GELU"),
           ("ffn-down", "k_linear: act-quant + down matvec + residual")]
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, scaled by the same
-# counters over the library's plain 256 MiB read+write kernel); None until measured for the current kernels.
-MEASURED_TRAFFIC = {}
+# HBM bytes per launch (batch 1) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same counter
+# reads for the library's plain 256 MiB read+write kernel: x2.000 and x1.000); the summary with the commands is
+# profiles/decode_step_int8_hbm_counters.md.  Valid for the int8 workload these were measured on.
+MEASURED_TRAFFIC = {"self-attention": 8778004, "cross-attention": 2854000, "self-out": 873000, "cross-out": 873000,
+                    "ffn-up": 2583000, "ffn-down": 2692000}
 
 
 def roofline(r):
@@ -145,7 +147,7 @@ def roofline(r):
                      "share_of_step": round(us * r["layers"] / r["step_us"], 3)})
     top = max(rows, key=lambda x: x["share_of_step"])
     return {"bound": "hbm", "kernel": top["stage"] + " stage = " + top["kernel"], "achieved": top["gbps"], "peak": PEAK_GBPS,
-            "unit": "GB/s", "frac": top["frac"], "traffic": MEASURED_TRAFFIC.get(top["stage"]),
+            "unit": "GB/s", "frac": top["frac"], "traffic": MEASURED_TRAFFIC.get(top["stage"]) if r.get("traffic_valid") else None,
             "launch_us": top["launch_us"], "algorithmic_bytes_per_launch": top["algorithmic_bytes_per_launch"],
             "stages": rows,
             "whole_step": {"step_us": round(r["step_us"], 2), "algorithmic_bytes_per_step": r["bytes"], "weight_bytes": r["weight_bytes"],
@@ -199,6 +201,7 @@ def main():
         backend.sync()
 
     b1 = time_config(pkg, synth, backend, qtype, [1023], [256], 1024, args.steps, args.warmup)
+    b1["traffic_valid"] = args.quant == "int8"
     b8 = None
     if not args.skip_b8:
         self_len, cross_len = synth.ragged_lengths(8, seed=3)
