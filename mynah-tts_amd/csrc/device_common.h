@@ -80,13 +80,14 @@ __device__ __forceinline__ int group_sum_i(int v, int lg) {
 }
 
 // Reduces BT independent values over the 256-thread workgroup in a fixed order: lanes by butterfly,
-// then waves 0..3.  The order never depends on how many of the BT slots are live.
+// then waves 0..3.  The order never depends on how many of the BT slots are live.  `s_scratch` is 4 * BT floats
+// that no earlier reduction of this workgroup used (each reduction of a kernel gets its own region, so a single
+// barrier per reduction is enough).
 template <int BT, bool IS_MAX>
 __device__ __forceinline__ void block_reduce(float (&v)[BT], float *s_scratch) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int b = 0; b < BT; ++b) v[b] = IS_MAX ? wave_max(v[b]) : wave_sum(v[b]);
-    __syncthreads();
     if (lane == 0) {
 #pragma unroll
         for (int b = 0; b < BT; ++b) s_scratch[wave * BT + b] = v[b];
@@ -289,6 +290,8 @@ __device__ __forceinline__ float4 fold_partials(const ActSource &src, int stream
     return acc;
 }
 
+constexpr int kPrologueScratch = 12;   // floats of reduction scratch per stream slot
+
 struct PrologueParams {
     int k;                  // row length (multiple of 4; k/4 <= 256 * NVT)
     int batch;              // live streams (<= BT)
@@ -303,6 +306,7 @@ struct PrologueParams {
 // load (or fold) -> optional LayerNorm -> for int8/int4 weights the per-vector absmax int8 quantisation
 // (quantize_act_int8, src/qmat.c:94-113; int4 additionally de-interleaves even/odd elements per run of 8
 // so they line up with the low/high nibbles of a weight dword).  NVT = float4 per thread per stream.
+// s_scratch: kPrologueScratch * BT floats (one region per reduction: mean, variance, absmax).
 template <int QT, int BT, int NVT>
 __device__ __forceinline__ void stage_activations(const PrologueParams &p, const ActSource &src, unsigned char *smem, float *s_sx,
                                                   float *s_scratch) {
@@ -350,7 +354,7 @@ __device__ __forceinline__ void stage_activations(const PrologueParams &p, const
                     v[b] = __builtin_fmaf(d3, d3, v[b]);
                 }
         }
-        block_reduce<BT, false>(v, s_scratch);
+        block_reduce<BT, false>(v, s_scratch + 4 * BT);
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
             const float rstd = 1.0f / sqrtf(v[b] / (float)p.k + 1.0e-5f);
@@ -378,7 +382,7 @@ __device__ __forceinline__ void stage_activations(const PrologueParams &p, const
                 if (tid + kThreads * i < nf4)
                     amax[b] = fmaxf(fmaxf(amax[b], fmaxf(fabsf(xr[b][i].x), fabsf(xr[b][i].y))), fmaxf(fabsf(xr[b][i].z), fabsf(xr[b][i].w)));
         }
-        block_reduce<BT, true>(amax, s_scratch);
+        block_reduce<BT, true>(amax, s_scratch + 8 * BT);
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
             const float inv = amax[b] > 0.0f ? 127.0f / amax[b] : 0.0f;

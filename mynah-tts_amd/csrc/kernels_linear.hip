@@ -45,7 +45,7 @@ template <int QT, int BT, int NVT>
 __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const int rows_per_wg, const int lg) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_sx[BT];
-    __shared__ float s_scratch[4 * BT];
+    __shared__ float s_scratch[kPrologueScratch * BT];
     constexpr int kEpc = Chunk<QT>::n;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;

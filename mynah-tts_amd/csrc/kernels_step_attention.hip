@@ -124,11 +124,10 @@ template <int QT, int NVT, int PF>
 __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a, const int lg, const int per_xcd) {
     extern __shared__ __align__(16) unsigned char smem[];   // staged activations: width bytes (int8/int4) or floats
     __shared__ __align__(16) float s_proj[3 * kHw];         // q | k | v of this head
-    __shared__ __align__(16) float s_score[kStepUnitRows];
-    __shared__ __align__(16) float s_red[kPosPerPass * kHw];
+    __shared__ __align__(16) float s_red[4 * kHw];          // per-wavefront weighted V sums
+    __shared__ float s_wave_ml[8];                          // per-wavefront max | sum
     __shared__ float s_sx[1];
-    __shared__ float s_scratch[4];
-    __shared__ float s_ml[2];
+    __shared__ float s_scratch[kPrologueScratch];
 
     const int tid = threadIdx.x;
     const StepSlots *slots = a.slots;
@@ -290,8 +289,12 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         return;
     }
 
-    // ---- scores of this unit
+    // ---- scores, softmax statistics and weighted V rows, one wavefront at a time: a wavefront owns 32 rows of the unit
+    // (its four 16-lane row groups x 8 passes) and nothing leaves it until its own (max, sum, out[64]) is complete;
+    // the four results meet once in LDS.
     const float4 qv = *reinterpret_cast<const float4 *>(s_proj + 4 * j);
+    float sc[kRowsPerThread];
+    float m = -3.0e38f;
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
         const int pi = g + kPosPerPass * i;
@@ -300,47 +303,46 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         dot = __builtin_fmaf(qv.y, kv[i].y, dot);
         dot = __builtin_fmaf(qv.z, kv[i].z, dot);
         dot = __builtin_fmaf(qv.w, kv[i].w, dot);
-        dot = row16_sum(dot);
-        if (j == 0) s_score[pi] = pi < count ? dot * a.scale : -3.0e38f;
+        dot = row16_sum(dot);   // every lane of the row group holds the row's score
+        sc[i] = pi < count ? dot * a.scale : -3.0e38f;
+        m = fmaxf(m, sc[i]);
     }
-    __syncthreads();
-    if (tid < 64) {   // kStepUnitRows scores, kStepUnitRows / 64 per lane
-        constexpr int kPerLane = kStepUnitRows / 64;
-        float sc[kPerLane], m = -3.0e38f;
-#pragma unroll
-        for (int i = 0; i < kPerLane; ++i) {
-            sc[i] = s_score[tid + 64 * i];
-            m = fmaxf(m, sc[i]);
-        }
-        m = wave_max(m);
-        float l = 0.0f;
-#pragma unroll
-        for (int i = 0; i < kPerLane; ++i) {
-            const float e = tid + 64 * i < count ? expf(sc[i] - m) : 0.0f;
-            s_score[tid + 64 * i] = e;
-            l += e;
-        }
-        l = wave_sum(l);
-        if (tid == 0) { s_ml[0] = m; s_ml[1] = l; }
-    }
-    __syncthreads();
+    m = fmaxf(fmaxf(lane_f(m, 0), lane_f(m, 16)), fmaxf(lane_f(m, 32), lane_f(m, 48)));
+    float l = 0.0f;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
-        const float e = s_score[g + kPosPerPass * i];
+        const float e = g + kPosPerPass * i < count ? expf(sc[i] - m) : 0.0f;
+        l += e;
         acc.x = __builtin_fmaf(e, vv[i].x, acc.x);
         acc.y = __builtin_fmaf(e, vv[i].y, acc.y);
         acc.z = __builtin_fmaf(e, vv[i].z, acc.z);
         acc.w = __builtin_fmaf(e, vv[i].w, acc.w);
     }
-    *reinterpret_cast<float4 *>(s_red + (size_t)g * kHw + 4 * j) = acc;
+    l = ((lane_f(l, 0) + lane_f(l, 16)) + lane_f(l, 32)) + lane_f(l, 48);
+    acc.x += __shfl_xor(acc.x, 16); acc.y += __shfl_xor(acc.y, 16); acc.z += __shfl_xor(acc.z, 16); acc.w += __shfl_xor(acc.w, 16);
+    acc.x += __shfl_xor(acc.x, 32); acc.y += __shfl_xor(acc.y, 32); acc.z += __shfl_xor(acc.z, 32); acc.w += __shfl_xor(acc.w, 32);
+    const int lane = tid & 63, wave = tid >> 6;
+    if (lane < kPosLanes) *reinterpret_cast<float4 *>(s_red + wave * kHw + 4 * lane) = acc;
+    if (lane == 0) { s_wave_ml[wave] = m; s_wave_ml[4 + wave] = l; }
     __syncthreads();
-    if (tid < kHw) {
-        float o = 0.0f;
-#pragma unroll
-        for (int gg = 0; gg < kPosPerPass; ++gg) o += s_red[(size_t)gg * kHw + tid];
-        out_o[tid] = o;
-        if (tid == 0) { out_m[pidx] = s_ml[0]; out_l[pidx] = s_ml[1]; }
+    if (tid < kPosLanes) {   // merge the four wavefronts in order 0..3
+        const float m0 = s_wave_ml[0], m1 = s_wave_ml[1], m2 = s_wave_ml[2], m3 = s_wave_ml[3];
+        const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+        const float w0 = expf(m0 - M), w1 = expf(m1 - M), w2 = expf(m2 - M), w3 = expf(m3 - M);   // a wavefront without rows: exp(-3e38 - M) = 0
+        float L = s_wave_ml[4] * w0;
+        L = __builtin_fmaf(s_wave_ml[5], w1, L);
+        L = __builtin_fmaf(s_wave_ml[6], w2, L);
+        L = __builtin_fmaf(s_wave_ml[7], w3, L);
+        const float4 o0 = *reinterpret_cast<const float4 *>(s_red + 4 * tid), o1 = *reinterpret_cast<const float4 *>(s_red + kHw + 4 * tid);
+        const float4 o2 = *reinterpret_cast<const float4 *>(s_red + 2 * kHw + 4 * tid), o3 = *reinterpret_cast<const float4 *>(s_red + 3 * kHw + 4 * tid);
+        float4 o;
+        o.x = __builtin_fmaf(o3.x, w3, __builtin_fmaf(o2.x, w2, __builtin_fmaf(o1.x, w1, o0.x * w0)));
+        o.y = __builtin_fmaf(o3.y, w3, __builtin_fmaf(o2.y, w2, __builtin_fmaf(o1.y, w1, o0.y * w0)));
+        o.z = __builtin_fmaf(o3.z, w3, __builtin_fmaf(o2.z, w2, __builtin_fmaf(o1.z, w1, o0.z * w0)));
+        o.w = __builtin_fmaf(o3.w, w3, __builtin_fmaf(o2.w, w2, __builtin_fmaf(o1.w, w1, o0.w * w0)));
+        *reinterpret_cast<float4 *>(out_o + 4 * tid) = o;
+        if (tid == 0) { out_m[pidx] = M; out_l[pidx] = L; }
     }
 }
 
