@@ -307,12 +307,14 @@ struct PrologueParams {
 // (quantize_act_int8, src/qmat.c:94-113; int4 additionally de-interleaves even/odd elements per run of 8
 // so they line up with the low/high nibbles of a weight dword).  NVT = float4 per thread per stream.
 // s_scratch: kPrologueScratch * BT floats (one region per reduction: mean, variance, absmax).
-template <int QT, int BT, int NVT>
-__device__ __forceinline__ void stage_activations(const PrologueParams &p, const ActSource &src, unsigned char *smem, float *s_sx,
-                                                  float *s_scratch) {
+//
+// First half of the prologue: request (or fold) the activation rows and the LayerNorm vectors.  Split from the
+// arithmetic so that a kernel can put other requests between the two (they are served while these are in flight).
+template <int BT, int NVT>
+__device__ __forceinline__ void load_activations(const PrologueParams &p, const ActSource &src, float4 (&xr)[BT][NVT], float4 (&gv)[NVT],
+                                                 float4 (&bv)[NVT]) {
     const int tid = threadIdx.x;
     const int nf4 = p.k >> 2;
-    float4 xr[BT][NVT];
 #pragma unroll
     for (int b = 0; b < BT; ++b)
 #pragma unroll
@@ -323,14 +325,21 @@ __device__ __forceinline__ void stage_activations(const PrologueParams &p, const
             else if (src.partial != nullptr) xr[b][i] = fold_partials(src, src.stream0 + b, f);
             else xr[b][i] = reinterpret_cast<const float4 *>(src.rows[b])[f];
         }
-    if (p.ln_gain != nullptr) {
-        float4 gv[NVT], bv[NVT];
 #pragma unroll
-        for (int i = 0; i < NVT; ++i) {
-            const int f = tid + kThreads * i;
-            gv[i] = f < nf4 ? reinterpret_cast<const float4 *>(p.ln_gain)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
-            bv[i] = (f < nf4 && p.ln_bias != nullptr) ? reinterpret_cast<const float4 *>(p.ln_bias)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+    for (int i = 0; i < NVT; ++i) {
+        const int f = tid + kThreads * i;
+        gv[i] = (p.ln_gain != nullptr && f < nf4) ? reinterpret_cast<const float4 *>(p.ln_gain)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+        bv[i] = (p.ln_gain != nullptr && f < nf4 && p.ln_bias != nullptr) ? reinterpret_cast<const float4 *>(p.ln_bias)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+
+// Second half: optional LayerNorm -> quantisation (or plain copy) -> LDS.
+template <int QT, int BT, int NVT>
+__device__ __forceinline__ void finish_activations(const PrologueParams &p, float4 (&xr)[BT][NVT], const float4 (&gv)[NVT],
+                                                   const float4 (&bv)[NVT], unsigned char *smem, float *s_sx, float *s_scratch) {
+    const int tid = threadIdx.x;
+    const int nf4 = p.k >> 2;
+    if (p.ln_gain != nullptr) {
         float s[BT];
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
@@ -428,6 +437,14 @@ __device__ __forceinline__ void stage_activations(const PrologueParams &p, const
         }
     }
     __syncthreads();
+}
+
+template <int QT, int BT, int NVT>
+__device__ __forceinline__ void stage_activations(const PrologueParams &p, const ActSource &src, unsigned char *smem, float *s_sx,
+                                                  float *s_scratch) {
+    float4 xr[BT][NVT], gv[NVT], bv[NVT];
+    load_activations<BT, NVT>(p, src, xr, gv, bv);
+    finish_activations<QT, BT, NVT>(p, xr, gv, bv, smem, s_sx, s_scratch);
 }
 
 }  // namespace mynah

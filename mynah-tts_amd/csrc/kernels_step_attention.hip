@@ -41,13 +41,14 @@ constexpr int kPrefetchLatency = 4, kPrefetchThroughput = 2;
 
 struct PassRegs {
     uint4 wv[4];
-    float sc[4];
+    float sc[4];   // int4: group scales of the four chunks
+    float ws;      // int8: scale of the row
 };
 
 // Weight row of projection output r for this head: r = part * 64 + i, part 0/1/2 = q/k/v.
 __device__ __forceinline__ int weight_row(int r, int head, int width) { return (r >> 6) * width + head * kHw + (r & 63); }
 
-template <int QT>
+template <int QT, int PF>
 __device__ __forceinline__ void load_pass(PassRegs &p, const StepAttnArgs &a, int pass, int row0, int nrows, int head, int lg, int chunks) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int G = 1 << lg, gl = lane & (G - 1), gidx = lane >> lg;
@@ -62,6 +63,8 @@ __device__ __forceinline__ void load_pass(PassRegs &p, const StepAttnArgs &a, in
         p.wv[u] = c < chunks ? wrow[c] : make_uint4(0, 0, 0, 0);
         p.sc[u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? a.scales[(size_t)wrow_id * chunks + c] : 0.0f;
     }
+    // the row scale travels with the weights in the latency layout; the throughput layout fetches it at use (registers)
+    p.ws = (QT == MYNAH_HIP_INT8 && PF == kPrefetchLatency) ? a.scales[wrow_id] : 1.0f;
 }
 
 // Requests passes [pass0, pass0 + PF) of rows [row0, row0 + nrows) into `bank`.
@@ -72,7 +75,7 @@ __device__ __forceinline__ void load_bank(PassRegs (&bank)[PF], const StepAttnAr
     const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
 #pragma unroll
     for (int p = 0; p < PF; ++p)
-        if (pass0 + p < passes) load_pass<QT>(bank[p], a, pass0 + p, row0, nrows, head, lg, chunks);
+        if (pass0 + p < passes) load_pass<QT, PF>(bank[p], a, pass0 + p, row0, nrows, head, lg, chunks);
 }
 
 // Passes [pass0, pass0 + PF) of the projection rows [row0, row0 + nrows) of this head (row numbering
@@ -98,8 +101,8 @@ __device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRe
             }
             group_reduce<QT, 1>(iacc, facc, lg);
             if (gl == 0 && r < row0 + nrows) {
-                float wscale = 1.0f;
-                if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[weight_row(r, head, a.width)];
+                float wscale = bank[p].ws;
+                if constexpr (QT == MYNAH_HIP_INT8 && PF != kPrefetchLatency) wscale = a.scales[weight_row(r, head, a.width)];
                 s_proj[r] = finish_value<QT>(iacc[0], facc[0], wscale, sx);
             }
         }
@@ -166,6 +169,17 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     else if (role_v) load_bank<QT, PF>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
     else load_bank<QT, PF>(pre, a, 0, 0, kHw, head, lg, chunks);
 
+    // ---- ... and (latency layout) the activation row with its LayerNorm vectors
+    PrologueParams pro;
+    pro.k = a.width; pro.batch = 1; pro.ln_gain = a.ln_gain; pro.ln_bias = a.ln_bias; pro.arith = a.arith;
+    pro.probe_qx = nullptr; pro.probe_sx = nullptr;
+    float4 xr[1][NVT], gv[NVT], bv[NVT];
+    ActSource act;
+    act.rows[0] = a.x + (size_t)b * a.width;
+    act.partial = nullptr;
+    // latency layout: requested now, ahead of the slot table; throughput layout: after the cache rows (fewer live registers)
+    if constexpr (PF == kPrefetchLatency) load_activations<1, NVT>(pro, act, xr, gv, bv);
+
     // ---- slot table: is this unit live, and where are its cache rows?
     const int length = a.is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
     const int nchunks = (length + kStepUnitRows - 1) / kStepUnitRows;
@@ -190,12 +204,14 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     static_assert(2 * kRowsPerThread >= 4 * PF, "the second weight bank must fit the cache-row registers");
     float4 kv[kRowsPerThread], vv[kRowsPerThread];
     float sc2[4 * PF];   // int4 only: group scales of the second bank
+    float ws2[PF];       // int8 only: row scales of the second bank
     if (role_qk) {
         PassRegs bank2[PF];
 #pragma unroll
         for (int p = 0; p < PF; ++p) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) { bank2[p].wv[u] = make_uint4(0, 0, 0, 0); bank2[p].sc[u] = 0.0f; }
+            bank2[p].ws = 1.0f;
         }
         load_bank<QT, PF>(bank2, a, PF, 0, 2 * kHw, head, lg, chunks);
 #pragma unroll
@@ -207,10 +223,13 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
                 else vv[idx - kRowsPerThread] = __builtin_bit_cast(float4, bank2[p].wv[u]);
                 sc2[idx] = bank2[p].sc[u];
             }
+            ws2[p] = bank2[p].ws;
         }
     } else {
 #pragma unroll
         for (int i = 0; i < 4 * PF; ++i) sc2[i] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < PF; ++i) ws2[i] = 1.0f;
 #pragma unroll
         for (int i = 0; i < kRowsPerThread; ++i) {
             const int pi = g + kPosPerPass * i;
@@ -220,16 +239,9 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         }
     }
 
-    // ---- LayerNorm + activation quantisation of x[b], staged in LDS
-    {
-        PrologueParams p;
-        p.k = a.width; p.batch = 1; p.ln_gain = a.ln_gain; p.ln_bias = a.ln_bias; p.arith = a.arith;
-        p.probe_qx = nullptr; p.probe_sx = nullptr;
-        ActSource src;
-        src.rows[0] = a.x + (size_t)b * a.width;
-        src.partial = nullptr;
-        stage_activations<QT, 1, NVT>(p, src, smem, s_sx, s_scratch);
-    }
+    // ---- LayerNorm + activation quantisation of x[b], staged in LDS (the cache rows requested above stay in flight)
+    if constexpr (PF != kPrefetchLatency) load_activations<1, NVT>(pro, act, xr, gv, bv);
+    finish_activations<QT, 1, NVT>(pro, xr, gv, bv, smem, s_sx, s_scratch);
 
     const size_t sh = (size_t)b * a.heads + head;
     float *out_m = a.partial_ml + sh * 2 * a.max_units;
@@ -247,6 +259,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
                     bank2[p].wv[u] = __builtin_bit_cast(uint4, idx < kRowsPerThread ? kv[idx] : vv[idx - kRowsPerThread]);
                     bank2[p].sc[u] = sc2[idx];
                 }
+                bank2[p].ws = ws2[p];
             }
             project_bank<QT, PF>(a, pre, 0, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
             project_bank<QT, PF>(a, bank2, PF, 0, 2 * kHw, head, lg, chunks, smem, s_sx[0], s_proj);
