@@ -61,6 +61,21 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
     const size_t row_bytes = (size_t)chunks * 16;
     const int pass_stride = 4 * rows_per_pass;
 
+    // ------------------------------------------------------------------ activation rows first: the prologue's arithmetic
+    // waits for these only, so it runs while the weight rows requested after them are still on their way
+    PrologueParams pro;
+    pro.k = k; pro.batch = a.batch; pro.ln_gain = a.ln_gain; pro.ln_bias = a.ln_bias; pro.arith = a.arith;
+    pro.probe_qx = a.probe_qx; pro.probe_sx = a.probe_sx;
+    float4 xr[BT][NVT], gv[NVT], bv[NVT];
+    {
+        ActSource src;
+#pragma unroll
+        for (int b = 0; b < kBatchTile; ++b) src.rows[b] = a.in[b];
+        src.partial = a.fold_partial; src.partial_ml = a.fold_partial_ml; src.slots = a.fold_slots; src.heads = a.fold_heads; src.head_width = a.fold_head_width;
+        src.max_units = a.fold_max_units; src.is_self = a.fold_is_self; src.stream0 = a.fold_stream0;
+        load_activations<BT, NVT>(pro, src, xr, gv, bv);
+    }
+
     // ------------------------------------------------------------------ loads that need no activation
     uint4 wv[4];
     float sc[4];
@@ -94,18 +109,8 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
         }
     }
 
-    // ------------------------------------------------------------------ prologue
-    {
-        PrologueParams p;
-        p.k = k; p.batch = a.batch; p.ln_gain = a.ln_gain; p.ln_bias = a.ln_bias; p.arith = a.arith;
-        p.probe_qx = a.probe_qx; p.probe_sx = a.probe_sx;
-        ActSource src;
-#pragma unroll
-        for (int b = 0; b < kBatchTile; ++b) src.rows[b] = a.in[b];
-        src.partial = a.fold_partial; src.partial_ml = a.fold_partial_ml; src.slots = a.fold_slots; src.heads = a.fold_heads; src.head_width = a.fold_head_width;
-        src.max_units = a.fold_max_units; src.is_self = a.fold_is_self; src.stream0 = a.fold_stream0;
-        stage_activations<QT, BT, NVT>(p, src, smem, s_sx, s_scratch);
-    }
+    // ------------------------------------------------------------------ prologue arithmetic (the weight requests above stay in flight)
+    finish_activations<QT, BT, NVT>(pro, xr, gv, bv, smem, s_sx, s_scratch);
 
     // ------------------------------------------------------------------ body
     bool first = true;

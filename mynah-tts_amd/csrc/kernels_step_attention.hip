@@ -163,13 +163,9 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         if (chunk >= (a.is_self ? live : max(live, 1))) return;
     }
 
-    // ---- requests that need neither activations nor the slot table: this role's weight rows
-    PassRegs pre[PF];
-    if (role_qk) load_bank<QT, PF>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
-    else if (role_v) load_bank<QT, PF>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
-    else load_bank<QT, PF>(pre, a, 0, 0, kHw, head, lg, chunks);
-
-    // ---- ... and (latency layout) the activation row with its LayerNorm vectors
+    // ---- requests that need neither the slot table nor each other.  Latency layout: the activation row and its
+    // LayerNorm vectors go first -- the prologue's arithmetic waits for these only and runs while the weight rows,
+    // requested right after, are still on their way.  Throughput layout: after the cache rows (fewer live registers).
     PrologueParams pro;
     pro.k = a.width; pro.batch = 1; pro.ln_gain = a.ln_gain; pro.ln_bias = a.ln_bias; pro.arith = a.arith;
     pro.probe_qx = nullptr; pro.probe_sx = nullptr;
@@ -177,8 +173,11 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     ActSource act;
     act.rows[0] = a.x + (size_t)b * a.width;
     act.partial = nullptr;
-    // latency layout: requested now, ahead of the slot table; throughput layout: after the cache rows (fewer live registers)
     if constexpr (PF == kPrefetchLatency) load_activations<1, NVT>(pro, act, xr, gv, bv);
+    PassRegs pre[PF];
+    if (role_qk) load_bank<QT, PF>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
+    else if (role_v) load_bank<QT, PF>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
+    else load_bank<QT, PF>(pre, a, 0, 0, kHw, head, lg, chunks);
 
     // ---- slot table: is this unit live, and where are its cache rows?
     const int length = a.is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
