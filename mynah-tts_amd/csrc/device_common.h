@@ -290,6 +290,10 @@ __device__ __forceinline__ float4 fold_partials(const ActSource &src, int stream
     return acc;
 }
 
+// Keeps the memory requests written above this point above it: without it the compiler is free to sink a load to its
+// first use, i.e. behind whatever that use waits for.  Emits no instruction and waits for nothing.
+__device__ __forceinline__ void requests_issued() { __asm__ volatile("" ::: "memory"); }
+
 constexpr int kPrologueScratch = 12;   // floats of reduction scratch per stream slot
 
 struct PrologueParams {

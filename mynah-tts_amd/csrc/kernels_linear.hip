@@ -75,6 +75,7 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
         src.max_units = a.fold_max_units; src.is_self = a.fold_is_self; src.stream0 = a.fold_stream0;
         load_activations<BT, NVT>(pro, src, xr, gv, bv);
     }
+    requests_issued();
 
     // ------------------------------------------------------------------ loads that need no activation
     uint4 wv[4];
@@ -108,6 +109,8 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
             for (int b = 0; b < BT; ++b) pre_res[b] = (a.epilogue == EPI_RESIDUAL && b < a.batch) ? a.out[b][rowc] : 0.0f;
         }
     }
+
+    requests_issued();
 
     // ------------------------------------------------------------------ prologue arithmetic (the weight requests above stay in flight)
     finish_activations<QT, BT, NVT>(pro, xr, gv, bv, smem, s_sx, s_scratch);

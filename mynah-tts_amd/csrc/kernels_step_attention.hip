@@ -178,6 +178,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     if (role_qk) load_bank<QT, PF>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
     else if (role_v) load_bank<QT, PF>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
     else load_bank<QT, PF>(pre, a, 0, 0, kHw, head, lg, chunks);
+    if constexpr (PF == kPrefetchLatency) requests_issued();
 
     // ---- slot table: is this unit live, and where are its cache rows?
     const int length = a.is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
