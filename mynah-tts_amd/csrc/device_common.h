@@ -146,7 +146,7 @@ constexpr bool kQuantised = (QT == MYNAH_HIP_INT8 || QT == MYNAH_HIP_INT4);
 
 // Lane-group width for a row of `chunks` 16-byte chunks: the widest power of two that still leaves
 // about three chunks per lane (k = 768 int8 -> 16 lanes, k = 3072 int8 -> 64 lanes).
-__host__ __device__ inline int lane_group_log2(int chunks) {
+__host__ __device__ constexpr int lane_group_log2(int chunks) {
     int lg = 6;
     while (lg > 0 && (chunks >> lg) < 3) --lg;
     return lg;

@@ -41,15 +41,19 @@ __device__ __forceinline__ float *stream_out(const LinearArgs &a, int b) {
     return o;
 }
 
-template <int QT, int BT, int NVT>
-__global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const int rows_per_wg, const int lg) {
+// KFIX: row length known at compile time (0 = taken from the arguments).  With it the lane-group width and the number of
+// chunks per lane are constants, so the per-chunk range checks fold away and the weight requests are straight-line code;
+// the two row lengths of the decoder stack (768 and 3072) get such a build.
+template <int QT, int BT, int NVT, int KFIX>
+__global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_sx[BT];
     __shared__ float s_scratch[kPrologueScratch * BT];
     constexpr int kEpc = Chunk<QT>::n;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int k = a.k;
+    const int k = KFIX != 0 ? KFIX : a.k;
+    const int lg = KFIX != 0 ? lane_group_log2(KFIX / kEpc) : lg_arg;
 
     const int G = 1 << lg;
     const int gl = lane & (G - 1);
@@ -236,7 +240,7 @@ __global__ void __launch_bounds__(256) k_sgemm(int ta, int tb, int m, int n, int
     *dst = beta == 0.0f ? alpha * sum : alpha * sum + beta * *dst;
 }
 
-template <int QT, int BT, int NVT>
+template <int QT, int BT, int NVT, int KFIX>
 int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity) {
     constexpr int epc = Chunk<QT>::n;
     const int chunks = a.k / epc;
@@ -250,26 +254,28 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
     const size_t lds = (size_t)BT * a.k * (kQuantised<QT> ? 1 : 4);
     static bool raised = false;   // per instantiation
     if (lds > 48 * 1024 && !raised) {
-        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_linear<QT, BT, NVT>),
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_linear<QT, BT, NVT, KFIX>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((k_linear<QT, BT, NVT>), dim3(grid), dim3(kThreads), lds, st->stream, a, rows_per_wg, lg);
+    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX>), dim3(grid), dim3(kThreads), lds, st->stream, a, rows_per_wg, lg);
     return hip_check(hipGetLastError(), "linear launch", error, capacity);
 }
 
-template <int QT, int NVT>
+template <int QT, int NVT, int KFIX>
 int launch_linear_b(State *st, const LinearArgs &a, char *error, size_t capacity) {
-    if (a.batch <= 1) return launch_linear_t<QT, 1, NVT>(st, a, error, capacity);
-    if (a.batch == 2) return launch_linear_t<QT, 2, NVT>(st, a, error, capacity);
-    if (a.batch <= 4) return launch_linear_t<QT, 4, NVT>(st, a, error, capacity);
-    return launch_linear_t<QT, 8, NVT>(st, a, error, capacity);
+    if (a.batch <= 1) return launch_linear_t<QT, 1, NVT, KFIX>(st, a, error, capacity);
+    if (a.batch == 2) return launch_linear_t<QT, 2, NVT, KFIX>(st, a, error, capacity);
+    if (a.batch <= 4) return launch_linear_t<QT, 4, NVT, KFIX>(st, a, error, capacity);
+    return launch_linear_t<QT, 8, NVT, KFIX>(st, a, error, capacity);
 }
 
 template <int QT>
 int launch_linear_q(State *st, const LinearArgs &a, char *error, size_t capacity) {
-    if (a.k <= 1024) return launch_linear_b<QT, 1>(st, a, error, capacity);
-    return launch_linear_b<QT, 3>(st, a, error, capacity);
+    if (a.k == 768) return launch_linear_b<QT, 1, 768>(st, a, error, capacity);
+    if (a.k == 3072) return launch_linear_b<QT, 3, 3072>(st, a, error, capacity);
+    if (a.k <= 1024) return launch_linear_b<QT, 1, 0>(st, a, error, capacity);
+    return launch_linear_b<QT, 3, 0>(st, a, error, capacity);
 }
 
 }  // namespace

@@ -123,8 +123,10 @@ __device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&b
     }
 }
 
-template <int QT, int NVT, int PF>
-__global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a, const int lg, const int per_xcd) {
+// WFIX: model width known at compile time (0 = taken from the arguments): lane-group width, chunks per lane and passes
+// per bank become constants and the per-chunk range checks fold away.  The decoder stack's width (768) gets such a build.
+template <int QT, int NVT, int PF, int WFIX>
+__global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a_arg, const int lg_arg, const int per_xcd) {
     extern __shared__ __align__(16) unsigned char smem[];   // staged activations: width bytes (int8/int4) or floats
     __shared__ __align__(16) float s_proj[3 * kHw];         // q | k | v of this head
     __shared__ __align__(16) float s_red[4 * kHw];          // per-wavefront weighted V sums
@@ -132,6 +134,10 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     __shared__ float s_sx[1];
     __shared__ float s_scratch[kPrologueScratch];
 
+    constexpr int kEpc = Chunk<QT>::n;
+    const int lg = WFIX != 0 ? lane_group_log2(WFIX / kEpc) : lg_arg;
+    StepAttnArgs a = a_arg;
+    if constexpr (WFIX != 0) a.width = WFIX;
     const int tid = threadIdx.x;
     const StepSlots *slots = a.slots;
 
@@ -151,7 +157,6 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const int chunk = a.is_self ? unit - 2 : unit;   // cache chunk of this workgroup (chunk roles only)
     const int pidx = a.is_self ? unit - 1 : unit;    // partial slot written by a chunk role (slot 0 = the new row)
 
-    constexpr int kEpc = Chunk<QT>::n;
     const int chunks = a.width / kEpc;
 
     // With many streams most of the grid belongs to units that short streams do not have: there the slot table is
@@ -382,12 +387,16 @@ int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const int grid = 8 * per_xcd;
     const size_t lds = (size_t)a.width * (kQuantised<QT> ? 1 : 4);
     const bool latency = a.batch <= kConsumerFoldMaxBatch;
-    if (a.width <= 1024) {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+    const dim3 g(grid), t(kThreads);
+    if (a.width == 768) {
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 768>), g, t, lds, st->stream, a, lg, per_xcd);
+    } else if (a.width <= 1024) {
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 0>), g, t, lds, st->stream, a, lg, per_xcd);
     } else {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput>), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput, 0>), g, t, lds, st->stream, a, lg, per_xcd);
     }
     return hip_check(hipGetLastError(), "step attention launch", error, capacity);
 }
