@@ -330,7 +330,9 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
-        const float e = g + kPosPerPass * i < count ? expf(sc[i] - m) : 0.0f;
+        // hardware exponential (2^(x log2 e), relative error about 1e-6 for the arguments met here) for the unit's 128 weights;
+        // the few exponentials that combine partial results stay exact
+        const float e = g + kPosPerPass * i < count ? __expf(sc[i] - m) : 0.0f;
         l += e;
         acc.x = __builtin_fmaf(e, vv[i].x, acc.x);
         acc.y = __builtin_fmaf(e, vv[i].y, acc.y);
@@ -389,8 +391,8 @@ int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const bool latency = a.batch <= kConsumerFoldMaxBatch;
     const dim3 g(grid), t(kThreads);
     if (a.width == 768) {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 768>), g, t, lds, st->stream, a, lg, per_xcd);
+        // the fixed-shape build needs few enough registers (154 for int8) to hold three workgroups per CU with four-pass banks
+        hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768>), g, t, lds, st->stream, a, lg, per_xcd);
     } else if (a.width <= 1024) {
         if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 0>), g, t, lds, st->stream, a, lg, per_xcd);
         else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 0>), g, t, lds, st->stream, a, lg, per_xcd);
