@@ -44,8 +44,23 @@ __device__ __forceinline__ float *stream_out(const LinearArgs &a, int b) {
 // KFIX: row length known at compile time (0 = taken from the arguments).  With it the lane-group width and the number of
 // chunks per lane are constants, so the per-chunk range checks fold away and the weight requests are straight-line code;
 // the two row lengths of the decoder stack (768 and 3072) get such a build.
-template <int QT, int BT, int NVT, int KFIX>
+// SPEC: what the launch is known not to use, so that the corresponding code is not there at all (0 = everything
+// decided at run time).  SPEC_RESIDUAL: no LayerNorm, no bias, no probes, residual epilogue (the step's output and
+// FFN-down projections; the fold source stays a run-time choice).  SPEC_UP: LayerNorm, no fold, no bias, no probes,
+// GELU epilogue (the step's FFN-up projection).
+enum { SPEC_ANY = 0, SPEC_RESIDUAL = 1, SPEC_UP = 2 };
+
+template <int QT, int BT, int NVT, int KFIX, int SPEC>
 __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
+    // the arguments a specialised build does not look at
+    const float *const arg_bias = SPEC != SPEC_ANY ? nullptr : a.bias;
+    int8_t *const arg_probe_qx = SPEC != SPEC_ANY ? nullptr : a.probe_qx;
+    float *const arg_probe_sx = SPEC != SPEC_ANY ? nullptr : a.probe_sx;
+    int32_t *const arg_probe_acc = SPEC != SPEC_ANY ? nullptr : a.probe_acc;
+    const int arg_epilogue = SPEC == SPEC_UP ? EPI_GELU : SPEC == SPEC_RESIDUAL ? EPI_RESIDUAL : a.epilogue;
+    const float *const arg_ln_gain = SPEC == SPEC_RESIDUAL ? nullptr : a.ln_gain;
+    const float *const arg_ln_bias = SPEC == SPEC_RESIDUAL ? nullptr : a.ln_bias;
+    const float *const arg_fold_partial = SPEC == SPEC_UP ? nullptr : a.fold_partial;
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_sx[BT];
     __shared__ float s_scratch[kPrologueScratch * BT];
@@ -68,14 +83,14 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
     // ------------------------------------------------------------------ activation rows first: the prologue's arithmetic
     // waits for these only, so it runs while the weight rows requested after them are still on their way
     PrologueParams pro;
-    pro.k = k; pro.batch = a.batch; pro.ln_gain = a.ln_gain; pro.ln_bias = a.ln_bias; pro.arith = a.arith;
-    pro.probe_qx = a.probe_qx; pro.probe_sx = a.probe_sx;
+    pro.k = k; pro.batch = a.batch; pro.ln_gain = arg_ln_gain; pro.ln_bias = arg_ln_bias; pro.arith = a.arith;
+    pro.probe_qx = arg_probe_qx; pro.probe_sx = arg_probe_sx;
     float4 xr[BT][NVT], gv[NVT], bv[NVT];
     {
         ActSource src;
 #pragma unroll
         for (int b = 0; b < kBatchTile; ++b) src.rows[b] = a.in[b];
-        src.partial = a.fold_partial; src.partial_ml = a.fold_partial_ml; src.slots = a.fold_slots; src.heads = a.fold_heads; src.head_width = a.fold_head_width;
+        src.partial = arg_fold_partial; src.partial_ml = a.fold_partial_ml; src.slots = a.fold_slots; src.heads = a.fold_heads; src.head_width = a.fold_head_width;
         src.max_units = a.fold_max_units; src.is_self = a.fold_is_self; src.stream0 = a.fold_stream0;
         load_activations<BT, NVT>(pro, src, xr, gv, bv);
     }
@@ -103,14 +118,14 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
         if (lanes_finish) {
             if (gl < BT) {
                 if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
-                if (a.bias != nullptr) pre_bias = a.bias[rowc];
-                if (a.epilogue == EPI_RESIDUAL && gl < a.batch) pre_res[0] = stream_out<BT>(a, gl)[rowc];
+                if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
+                if (arg_epilogue == EPI_RESIDUAL && gl < a.batch) pre_res[0] = stream_out<BT>(a, gl)[rowc];
             }
         } else if (gl == 0) {
             if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
-            if (a.bias != nullptr) pre_bias = a.bias[rowc];
+            if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
 #pragma unroll
-            for (int b = 0; b < BT; ++b) pre_res[b] = (a.epilogue == EPI_RESIDUAL && b < a.batch) ? a.out[b][rowc] : 0.0f;
+            for (int b = 0; b < BT; ++b) pre_res[b] = (arg_epilogue == EPI_RESIDUAL && b < a.batch) ? a.out[b][rowc] : 0.0f;
         }
     }
 
@@ -145,7 +160,7 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
                 if (c < chunks) {
                     int group_int = 0;
                     dot_chunk<QT, BT>(wv[u], sc[u], c, smem, k, iacc, facc, &group_int);
-                    if (QT == MYNAH_HIP_INT4 && a.probe_acc != nullptr && valid) a.probe_acc[(size_t)row * chunks + c] = group_int;
+                    if (QT == MYNAH_HIP_INT4 && arg_probe_acc != nullptr && valid) arg_probe_acc[(size_t)row * chunks + c] = group_int;
                 }
             }
         }
@@ -163,14 +178,14 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
                     bias = pre_bias;
                 } else {
                     if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[row];
-                    if (a.bias != nullptr) bias = a.bias[row];
+                    if (arg_bias != nullptr) bias = arg_bias[row];
                 }
                 float val = finish_value<QT>(mi, mf, wscale, s_sx[gl]);
-                if (QT == MYNAH_HIP_INT8 && a.probe_acc != nullptr && gl == 0) a.probe_acc[row] = mi;
-                if (a.bias != nullptr) val += bias;
-                if (a.epilogue == EPI_GELU) val = gelu_tanh(val);
+                if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && gl == 0) arg_probe_acc[row] = mi;
+                if (arg_bias != nullptr) val += bias;
+                if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
                 float *o = stream_out<BT>(a, gl) + row;
-                if (a.epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : *o) + val;
+                if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : *o) + val;
                 *o = val;
             }
         } else if (gl == 0 && valid) {
@@ -180,17 +195,17 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
                 bias = pre_bias;
             } else {
                 if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[row];
-                if (a.bias != nullptr) bias = a.bias[row];
+                if (arg_bias != nullptr) bias = arg_bias[row];
             }
 #pragma unroll
             for (int b = 0; b < BT; ++b) {
                 if (b < a.batch) {
                     float val = finish_value<QT>(iacc[b], facc[b], wscale, s_sx[b]);
-                    if (QT == MYNAH_HIP_INT8 && a.probe_acc != nullptr && b == 0) a.probe_acc[row] = iacc[b];
-                    if (a.bias != nullptr) val += bias;
-                    if (a.epilogue == EPI_GELU) val = gelu_tanh(val);
+                    if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && b == 0) arg_probe_acc[row] = iacc[b];
+                    if (arg_bias != nullptr) val += bias;
+                    if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
                     float *o = a.out[b] + row;
-                    if (a.epilogue == EPI_RESIDUAL) val = (first ? pre_res[b] : *o) + val;
+                    if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[b] : *o) + val;
                     *o = val;
                 }
             }
@@ -240,7 +255,7 @@ __global__ void __launch_bounds__(256) k_sgemm(int ta, int tb, int m, int n, int
     *dst = beta == 0.0f ? alpha * sum : alpha * sum + beta * *dst;
 }
 
-template <int QT, int BT, int NVT, int KFIX>
+template <int QT, int BT, int NVT, int KFIX, int SPEC>
 int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity) {
     constexpr int epc = Chunk<QT>::n;
     const int chunks = a.k / epc;
@@ -254,28 +269,39 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
     const size_t lds = (size_t)BT * a.k * (kQuantised<QT> ? 1 : 4);
     static bool raised = false;   // per instantiation
     if (lds > 48 * 1024 && !raised) {
-        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_linear<QT, BT, NVT, KFIX>),
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_linear<QT, BT, NVT, KFIX, SPEC>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX>), dim3(grid), dim3(kThreads), lds, st->stream, a, rows_per_wg, lg);
+    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads), lds, st->stream, a, rows_per_wg, lg);
     return hip_check(hipGetLastError(), "linear launch", error, capacity);
 }
 
-template <int QT, int NVT, int KFIX>
+template <int QT, int NVT, int KFIX, int SPEC>
 int launch_linear_b(State *st, const LinearArgs &a, char *error, size_t capacity) {
-    if (a.batch <= 1) return launch_linear_t<QT, 1, NVT, KFIX>(st, a, error, capacity);
-    if (a.batch == 2) return launch_linear_t<QT, 2, NVT, KFIX>(st, a, error, capacity);
-    if (a.batch <= 4) return launch_linear_t<QT, 4, NVT, KFIX>(st, a, error, capacity);
-    return launch_linear_t<QT, 8, NVT, KFIX>(st, a, error, capacity);
+    if (a.batch <= 1) return launch_linear_t<QT, 1, NVT, KFIX, SPEC>(st, a, error, capacity);
+    if (a.batch == 2) return launch_linear_t<QT, 2, NVT, KFIX, SPEC>(st, a, error, capacity);
+    if (a.batch <= 4) return launch_linear_t<QT, 4, NVT, KFIX, SPEC>(st, a, error, capacity);
+    return launch_linear_t<QT, 8, NVT, KFIX, SPEC>(st, a, error, capacity);
 }
 
 template <int QT>
 int launch_linear_q(State *st, const LinearArgs &a, char *error, size_t capacity) {
-    if (a.k == 768) return launch_linear_b<QT, 1, 768>(st, a, error, capacity);
-    if (a.k == 3072) return launch_linear_b<QT, 3, 3072>(st, a, error, capacity);
-    if (a.k <= 1024) return launch_linear_b<QT, 1, 0>(st, a, error, capacity);
-    return launch_linear_b<QT, 3, 0>(st, a, error, capacity);
+    // what the arguments rule out decides the build (see SPEC above)
+    const bool plain = a.bias == nullptr && a.probe_qx == nullptr && a.probe_sx == nullptr && a.probe_acc == nullptr;
+    const bool residual = plain && a.epilogue == EPI_RESIDUAL && a.ln_gain == nullptr;
+    const bool up = plain && a.epilogue == EPI_GELU && a.ln_gain != nullptr && a.fold_partial == nullptr;
+    if (a.k == 768) {
+        if (residual) return launch_linear_b<QT, 1, 768, SPEC_RESIDUAL>(st, a, error, capacity);
+        if (up) return launch_linear_b<QT, 1, 768, SPEC_UP>(st, a, error, capacity);
+        return launch_linear_b<QT, 1, 768, SPEC_ANY>(st, a, error, capacity);
+    }
+    if (a.k == 3072) {
+        if (residual) return launch_linear_b<QT, 3, 3072, SPEC_RESIDUAL>(st, a, error, capacity);
+        return launch_linear_b<QT, 3, 3072, SPEC_ANY>(st, a, error, capacity);
+    }
+    if (a.k <= 1024) return launch_linear_b<QT, 1, 0, SPEC_ANY>(st, a, error, capacity);
+    return launch_linear_b<QT, 3, 0, SPEC_ANY>(st, a, error, capacity);
 }
 
 }  // namespace
