@@ -125,7 +125,8 @@ __device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&b
 
 // WFIX: model width known at compile time (0 = taken from the arguments): lane-group width, chunks per lane and passes
 // per bank become constants and the per-chunk range checks fold away.  The decoder stack's width (768) gets such a build.
-template <int QT, int NVT, int PF, int WFIX>
+// SELF: 1 / 0 = self / cross attention known at compile time (the cross build has no new-row roles at all), -1 = from the arguments.
+template <int QT, int NVT, int PF, int WFIX, int SELF>
 __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a_arg, const int lg_arg, const int per_xcd) {
     extern __shared__ __align__(16) unsigned char smem[];   // staged activations: width bytes (int8/int4) or floats
     __shared__ __align__(16) float s_proj[3 * kHw];         // q | k | v of this head
@@ -138,12 +139,13 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const int lg = WFIX != 0 ? lane_group_log2(WFIX / kEpc) : lg_arg;
     StepAttnArgs a = a_arg;
     if constexpr (WFIX != 0) a.width = WFIX;
+    const bool is_self = SELF >= 0 ? SELF == 1 : a.is_self != 0;
     const int tid = threadIdx.x;
     const StepSlots *slots = a.slots;
 
     // ---- static work decode: item = (head * batch + stream) * wg_units + unit, XCD x owns items [x*per_xcd, (x+1)*per_xcd).
     // Self-attention: unit 0 = Q+K of the new row, unit 1 = V of the new row, unit 2 + c = cache chunk c.
-    const int wg_units = a.max_units + (a.is_self ? 1 : 0);
+    const int wg_units = a.max_units + (is_self ? 1 : 0);
     const int items = a.heads * a.batch * wg_units;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int item = xcd * per_xcd + slot;
@@ -152,20 +154,20 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const int hb = item / wg_units;
     const int b = hb % a.batch;
     const int head = hb / a.batch;
-    const bool role_qk = a.is_self && unit == 0;
-    const bool role_v = a.is_self && unit == 1;
-    const int chunk = a.is_self ? unit - 2 : unit;   // cache chunk of this workgroup (chunk roles only)
-    const int pidx = a.is_self ? unit - 1 : unit;    // partial slot written by a chunk role (slot 0 = the new row)
+    const bool role_qk = is_self && unit == 0;
+    const bool role_v = is_self && unit == 1;
+    const int chunk = is_self ? unit - 2 : unit;   // cache chunk of this workgroup (chunk roles only)
+    const int pidx = is_self ? unit - 1 : unit;    // partial slot written by a chunk role (slot 0 = the new row)
 
     const int chunks = a.width / kEpc;
 
     // With many streams most of the grid belongs to units that short streams do not have: there the slot table is
     // looked at first, so that such a workgroup leaves without having requested anything.  With one or two streams
     // nearly every unit is live and the weight rows are requested before the table has arrived (latency matters more).
-    if (a.batch > kConsumerFoldMaxBatch && !(a.is_self && unit < 2)) {
-        const int len = a.is_self ? slots->length[b] : slots->memory_length[b];
+    if (a.batch > kConsumerFoldMaxBatch && !(is_self && unit < 2)) {
+        const int len = is_self ? slots->length[b] : slots->memory_length[b];
         const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-        if (chunk >= (a.is_self ? live : max(live, 1))) return;
+        if (chunk >= (is_self ? live : max(live, 1))) return;
     }
 
     // ---- requests that need neither the slot table nor each other.  Latency layout: the activation row and its
@@ -186,13 +188,13 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     if constexpr (PF == kPrefetchLatency) requests_issued();
 
     // ---- slot table: is this unit live, and where are its cache rows?
-    const int length = a.is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
+    const int length = is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
     const int nchunks = (length + kStepUnitRows - 1) / kStepUnitRows;
     const bool new_row = role_qk || role_v;
-    if (!new_row && chunk >= (a.is_self ? nchunks : max(nchunks, 1))) return;
+    if (!new_row && chunk >= (is_self ? nchunks : max(nchunks, 1))) return;
     const int stride = a.heads * kHw;   // floats between cache rows
     float *kc, *vc;
-    if (a.is_self) {
+    if (is_self) {
         kc = slots->self_k[b] + a.layer * a.capacity * (size_t)stride;
         vc = slots->self_v[b] + a.layer * a.capacity * (size_t)stride;
     } else {
@@ -392,13 +394,14 @@ int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const dim3 g(grid), t(kThreads);
     if (a.width == 768) {
         // the fixed-shape build needs few enough registers (154 for int8) to hold three workgroups per CU with four-pass banks
-        hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768>), g, t, lds, st->stream, a, lg, per_xcd);
+        if (a.is_self) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 1>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 0>), g, t, lds, st->stream, a, lg, per_xcd);
     } else if (a.width <= 1024) {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 0>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
     } else {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency, 0>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
     }
     return hip_check(hipGetLastError(), "step attention launch", error, capacity);
 }
