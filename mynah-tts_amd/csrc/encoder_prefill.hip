@@ -226,26 +226,25 @@ __global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *pa
         bb[u] = (in && bias != nullptr) ? reinterpret_cast<const float4 *>(bias)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     if (part != nullptr) {
-        float4 p[NV];
+        // all splits are requested at once and added in split order: the sum does not depend on how the splits were scheduled
+        constexpr int kSplits = 4;   // kMaxSplits of the products
+        float4 p[kSplits][NV];
 #pragma unroll
-        for (int u = 0; u < NV; ++u) {
-            const int i = lane + 64 * u;
-            p[u] = i < n4 ? reinterpret_cast<const float4 *>(part + (size_t)row * width)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-        for (int z = 1; z < splits; ++z) {   // fixed order: the sum does not depend on how the splits were scheduled
+        for (int z = 0; z < kSplits; ++z) {
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
                 const int i = lane + 64 * u;
-                if (i < n4) {
-                    const float4 q = reinterpret_cast<const float4 *>(part + z * split_stride + (size_t)row * width)[i];
-                    p[u].x += q.x; p[u].y += q.y; p[u].z += q.z; p[u].w += q.w;
-                }
+                p[z][u] = (z < splits && i < n4) ? reinterpret_cast<const float4 *>(part + z * split_stride + (size_t)row * width)[i]
+                                                : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         }
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
             const int i = lane + 64 * u;
-            v[u].x += p[u].x; v[u].y += p[u].y; v[u].z += p[u].z; v[u].w += p[u].w;
+            float4 t = p[0][u];
+#pragma unroll
+            for (int z = 1; z < kSplits; ++z) { t.x += p[z][u].x; t.y += p[z][u].y; t.z += p[z][u].z; t.w += p[z][u].w; }
+            v[u].x += t.x; v[u].y += t.y; v[u].z += t.z; v[u].w += t.w;
             if (i < n4) xr[i] = v[u];
         }
     }
@@ -310,24 +309,49 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
     const int sstride = tpad + kScorePad;                    // floats per score row
     float *S = reinterpret_cast<float *>(smem);
 
+    // ---- every global request of this workgroup is independent of the others and is issued here: the query
+    // fragments, the key fragments of this wavefront's first kKeyTiles score tiles and the V fragments of its first
+    // kValueSteps PV steps (all of them up to 512 tokens); they are consumed in that order while the rest arrives.
+    constexpr int kKeyTiles = 4, kValueSteps = 16;
+    const int ld = 2 * width;
+    const int ntiles = tpad / 32;
+    const int wn = wave & 1, kh = wave >> 1;
+    const int kspan = tpad / 2;                              // keys per PV half, multiple of 32
+    const _Float16 *qrow = qk + (size_t)(q0 + (lane & 31)) * ld + head * 64 + 8 * (lane >> 5);
+    const _Float16 *kbase = qk + (size_t)(lane & 31) * ld + width + head * 64 + 8 * (lane >> 5);
+    const _Float16 *vrow = vt + (size_t)(head * 64 + wn * 32 + (lane & 31)) * vt_stride + kh * kspan + 8 * (lane >> 5);
+    half8 fq[4], fk[kKeyTiles][4], fv[kValueSteps];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) fq[j] = *reinterpret_cast<const half8 *>(qrow + 16 * j);
+#pragma unroll
+    for (int t = 0; t < kKeyTiles; ++t) {
+        const int tile = wave + 4 * t;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            fk[t][j] = tile < ntiles ? *reinterpret_cast<const half8 *>(kbase + (size_t)tile * 32 * ld + 16 * j) : half8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int st = 0; st < kValueSteps; ++st)
+        fv[st] = 16 * st < kspan ? *reinterpret_cast<const half8 *>(vrow + 16 * st) : half8{0, 0, 0, 0, 0, 0, 0, 0};
+
     // ---- scores
     {
-        const int ld = 2 * width;
-        const _Float16 *qrow = qk + (size_t)(q0 + (lane & 31)) * ld + head * 64 + 8 * (lane >> 5);
-        half8 fq[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) fq[j] = *reinterpret_cast<const half8 *>(qrow + 16 * j);
-        for (int tile = wave; tile < tpad / 32; tile += 4) {
-            const _Float16 *krow = qk + (size_t)(tile * 32 + (lane & 31)) * ld + width + head * 64 + 8 * (lane >> 5);
+        auto score_tile = [&](int tile, const half8 (&k4)[4]) {
             floatx16 acc = {0};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const half8 fk = *reinterpret_cast<const half8 *>(krow + 16 * j);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fq[j], fk, acc, 0, 0, 0);
-            }
+            for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fq[j], k4[j], acc, 0, 0, 0);
             const int key = tile * 32 + (lane & 31);
 #pragma unroll
             for (int r = 0; r < 16; ++r) S[acc_row(r, lane) * sstride + key] = key < tokens ? acc[r] * scale : -3.0e38f;
+        };
+#pragma unroll
+        for (int t = 0; t < kKeyTiles; ++t)
+            if (wave + 4 * t < ntiles) score_tile(wave + 4 * t, fk[t]);
+        for (int tile = wave + 4 * kKeyTiles; tile < ntiles; tile += 4) {   // more than 512 tokens
+            half8 k4[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) k4[j] = *reinterpret_cast<const half8 *>(kbase + (size_t)tile * 32 * ld + 16 * j);
+            score_tile(tile, k4);
         }
     }
     __syncthreads();
@@ -347,7 +371,7 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
         // 2c) lands on floats already consumed: the eight lanes of a row walk c in lock step (one
         // wavefront, in order), reading floats c .. c+7 of a sweep before writing halfs c .. c+7.
         for (int c = part; c < tpad; c += 8) {
-            const float e = c < tokens ? expf(srow[c] - m) : 0.0f;
+            const float e = c < tokens ? __expf(srow[c] - m) : 0.0f;   // hardware exponential: the numerators are rounded to f16 anyway
             l += e;
             prow[c] = (_Float16)e;
         }
@@ -360,15 +384,19 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
 
     // ---- P V
     {
-        const int wn = wave & 1, kh = wave >> 1;
-        const int kspan = tpad / 2;                              // multiple of 32
         const _Float16 *prow = reinterpret_cast<const _Float16 *>(S + (lane & 31) * sstride) + kh * kspan + 8 * (lane >> 5);
-        const _Float16 *vrow = vt + (size_t)(head * 64 + wn * 32 + (lane & 31)) * vt_stride + kh * kspan + 8 * (lane >> 5);
         floatx16 acc = {0};
-        for (int k = 0; k < kspan; k += 16) {
+#pragma unroll
+        for (int st = 0; st < kValueSteps; ++st) {
+            if (16 * st < kspan) {
+                const half8 fp = *reinterpret_cast<const half8 *>(prow + 16 * st);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fp, fv[st], acc, 0, 0, 0);
+            }
+        }
+        for (int k = 16 * kValueSteps; k < kspan; k += 16) {   // more than 512 tokens
             const half8 fp = *reinterpret_cast<const half8 *>(prow + k);
-            const half8 fv = *reinterpret_cast<const half8 *>(vrow + k);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fp, fv, acc, 0, 0, 0);
+            const half8 fvk = *reinterpret_cast<const half8 *>(vrow + k);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fp, fvk, acc, 0, 0, 0);
         }
         if (kh == 1) {
 #pragma unroll
@@ -408,7 +436,7 @@ int f16_matrix(State *st, const float *host, size_t n, size_t k, const CachedWei
 
 size_t attention_lds_bytes(size_t tpad) { return (size_t)kQTile * (tpad + kScorePad) * sizeof(float); }
 
-constexpr int kMaxSplits = 4;
+constexpr int kMaxSplits = 4;   // k_enc_rows reads exactly this many partial planes at most
 int pick_splits(int k) {
     for (int s = kMaxSplits; s > 1; --s)
         if (k % (kTile * s) == 0 && k / (kTile * s) >= 3) return s;
