@@ -356,24 +356,40 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
     }
     __syncthreads();
 
-    // ---- softmax of row tid / 8 by eight adjacent lanes (softmax_row_inplace, src/graph.c:245-257)
+    // ---- softmax of row tid / 8 by eight adjacent lanes (softmax_row_inplace, src/graph.c:245-257).  A lane takes
+    // float4 pieces part, part + 8, ... of the row (up to kPieces of them in registers, i.e. 1024 keys), so the row is
+    // read from LDS once.  The numerators go back as f16 over the first half of the row's own bytes: the eight lanes
+    // of a row belong to one wavefront and all of their reads are done before the first of these writes is issued.
     {
+        constexpr int kPieces = 32;
         const int row = tid >> 3, part = tid & 7;
-        float *srow = S + row * sstride;
-        _Float16 *prow = reinterpret_cast<_Float16 *>(srow);
+        const float4 *srow = reinterpret_cast<const float4 *>(S + row * sstride);
+        half4 *prow = reinterpret_cast<half4 *>(S + row * sstride);
+        const int npieces = tpad / 4;
+        float4 v[kPieces];
         float m = -3.0e38f;
-        for (int c = part; c < tpad; c += 8) m = fmaxf(m, srow[c]);
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) {
+            const int c = part + 8 * i;
+            if (c < npieces) {
+                v[i] = srow[c];
+                m = fmaxf(fmaxf(m, fmaxf(v[i].x, v[i].y)), fmaxf(v[i].z, v[i].w));
+            }
+        }
         m = fmaxf(m, __shfl_xor(m, 1));
         m = fmaxf(m, __shfl_xor(m, 2));
         m = fmaxf(m, __shfl_xor(m, 4));
         float l = 0.0f;
-        // Numerators go back as f16 into the first half of the row's own bytes.  Element c (2 bytes at
-        // 2c) lands on floats already consumed: the eight lanes of a row walk c in lock step (one
-        // wavefront, in order), reading floats c .. c+7 of a sweep before writing halfs c .. c+7.
-        for (int c = part; c < tpad; c += 8) {
-            const float e = c < tokens ? __expf(srow[c] - m) : 0.0f;   // hardware exponential: the numerators are rounded to f16 anyway
-            l += e;
-            prow[c] = (_Float16)e;
+#pragma unroll
+        for (int i = 0; i < kPieces; ++i) {
+            const int c = part + 8 * i;
+            if (c < npieces) {
+                // hardware exponential: the numerators are rounded to f16 anyway; masked keys hold -3e38 and give 0
+                const float e0 = __expf(v[i].x - m), e1 = __expf(v[i].y - m), e2 = __expf(v[i].z - m), e3 = __expf(v[i].w - m);
+                l += (e0 + e1) + (e2 + e3);
+                const half4 h = {(_Float16)e0, (_Float16)e1, (_Float16)e2, (_Float16)e3};
+                prow[c] = h;
+            }
         }
         l += __shfl_xor(l, 1);
         l += __shfl_xor(l, 2);
@@ -508,8 +524,8 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
     if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, 0) != hipSuccess || lds <= 0) lds = 65536;
     e->max_lds = (size_t)lds;
     auto fail = [&](void) { mynah_hip_encoder_destroy(state, e); return -1; };
-    if (attention_lds_bytes(e->tpad_max) + 10 * 1024 > e->max_lds) {
-        set_error(error, capacity, "encoder_create: max_positions needs more LDS per workgroup than this device has");
+    if (e->tpad_max > 1024 || attention_lds_bytes(e->tpad_max) + 10 * 1024 > e->max_lds) {   // 1024: a softmax lane keeps 32 float4 pieces of its row
+        set_error(error, capacity, "encoder_create: max_positions beyond 1024, or more LDS per workgroup than this device has");
         return fail();
     }
     if (f16_matrix(st, d->tok_table, d->vocab, d->width, &e->tok, error, capacity) != 0) return fail();
