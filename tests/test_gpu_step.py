@@ -281,3 +281,35 @@ def test_stage_enqueue_leaves_the_step_intact(pkg, backend, synth):
         assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32))
     h.close()
     backend.set_quant(0)
+
+
+def test_full_size_ragged_batch8_int8(pkg, backend, orc, synth, nerr):
+    """The benchmark's batch-8 configuration at full size (12 layers, self KV up to 2048 rows, 12x64 cross heads, int8):
+    two streams against the oracle, graph replay == eager and batched == solo bit for bit."""
+    _announce("12 layers int8 ragged b=8 full size")
+    self_len, cross_len = synth.ragged_lengths(8, seed=3)
+    lengths = [n - 1 for n in self_len]
+    cfg = synth.decoder_config(layers=12, capacity=2048)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, cross_len, seed=1)
+    backend.set_quant(1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    first = h.step()
+    assert all(np.all(np.isfinite(o)) for o in first)
+    check = (1, 6)                                      # the shortest and the longest stream
+    odec = orc.Decoder(cfg, weights, orc.INT8)
+    for b in check:
+        s = streams[b]
+        want = odec.step([s["k"].copy()], [s["v"].copy()], [s["ck"]], [s["cv"]], [lengths[b]], [cross_len[b]], [s["x"]])[0]
+        assert nerr(first[b], want) < 5e-2, "stream %d" % b     # 12 layers of re-quantised activations, see TOL above
+    for b in range(8):
+        h.reset_cache(b)
+    again = h.step()                                    # captured graph
+    for b in range(8):
+        assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32)), "replay differs for stream %d" % b
+    for b in check:
+        h.reset_cache(b)
+        solo = h.step([b])[0]
+        assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
+    h.close()
+    backend.set_quant(0)
