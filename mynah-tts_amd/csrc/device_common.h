@@ -260,8 +260,15 @@ __device__ __forceinline__ int attention_units(const StepSlots *s, int stream, i
     return chunks > 0 ? chunks : 1;
 }
 
-// One float4 of a stream's folded attention output.  Units are taken in order 0..units-1; the loads of
-// a block of units are independent of the running sums so they are in flight together.
+// Keeps the memory requests written above this point above it: without it the compiler is free to sink a load to its
+// first use, i.e. behind whatever that use waits for.  Emits no instruction and waits for nothing.
+__device__ __forceinline__ void requests_issued() { __asm__ volatile("" ::: "memory"); }
+
+// One float4 of a stream's folded attention output.  Units are taken in order 0..units-1.  How many units the stream
+// has is in the slot table, a read that takes as long as the partials themselves: so the first kFoldAhead partial slots
+// (they exist whatever the stream's length: the workspace is sized for max_units) are requested before the count is
+// looked at, and masked by it afterwards.  Streams with more units continue from memory.
+constexpr int kFoldAhead = 10;
 __device__ __forceinline__ float4 fold_partials(const ActSource &src, int stream, int f4) {
     const int hw = src.head_width;
     const int d = 4 * f4;
@@ -270,14 +277,37 @@ __device__ __forceinline__ float4 fold_partials(const ActSource &src, int stream
     const float *m = src.partial_ml + sh * 2 * src.max_units;
     const float *l = m + src.max_units;
     const float *o = src.partial + sh * src.max_units * hw + dh;
+    float pm[kFoldAhead], pl[kFoldAhead];
+    float4 po[kFoldAhead];
+#pragma unroll
+    for (int u = 0; u < kFoldAhead; ++u) {
+        const bool in = u < src.max_units;
+        pm[u] = in ? m[u] : -3.0e38f;
+        pl[u] = in ? l[u] : 0.0f;
+        po[u] = in ? *reinterpret_cast<const float4 *>(o + (size_t)u * hw) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    requests_issued();
     const int units = attention_units(src.slots, stream, src.is_self);
     float M = -3.0e38f;
-#pragma unroll 8
-    for (int u = 0; u < units; ++u) M = fmaxf(M, m[u]);
+#pragma unroll
+    for (int u = 0; u < kFoldAhead; ++u)
+        if (u < units) M = fmaxf(M, pm[u]);
+    for (int u = kFoldAhead; u < units; ++u) M = fmaxf(M, m[u]);
     float L = 0.0f;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int u = 0; u < kFoldAhead; ++u) {
+        if (u < units) {
+            const float w = expf(pm[u] - M);
+            L = __builtin_fmaf(pl[u], w, L);
+            acc.x = __builtin_fmaf(po[u].x, w, acc.x);
+            acc.y = __builtin_fmaf(po[u].y, w, acc.y);
+            acc.z = __builtin_fmaf(po[u].z, w, acc.z);
+            acc.w = __builtin_fmaf(po[u].w, w, acc.w);
+        }
+    }
 #pragma unroll 4
-    for (int u = 0; u < units; ++u) {
+    for (int u = kFoldAhead; u < units; ++u) {
         const float w = expf(m[u] - M);
         const float4 ou = *reinterpret_cast<const float4 *>(o + (size_t)u * hw);
         L = __builtin_fmaf(l[u], w, L);
@@ -289,10 +319,6 @@ __device__ __forceinline__ float4 fold_partials(const ActSource &src, int stream
     acc.x /= L; acc.y /= L; acc.z /= L; acc.w /= L;
     return acc;
 }
-
-// Keeps the memory requests written above this point above it: without it the compiler is free to sink a load to its
-// first use, i.e. behind whatever that use waits for.  Emits no instruction and waits for nothing.
-__device__ __forceinline__ void requests_issued() { __asm__ volatile("" ::: "memory"); }
 
 constexpr int kPrologueScratch = 12;   // floats of reduction scratch per stream slot
 

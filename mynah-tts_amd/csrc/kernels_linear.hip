@@ -60,7 +60,7 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
     const int arg_epilogue = SPEC == SPEC_UP ? EPI_GELU : SPEC == SPEC_RESIDUAL ? EPI_RESIDUAL : a.epilogue;
     const float *const arg_ln_gain = SPEC == SPEC_RESIDUAL ? nullptr : a.ln_gain;
     const float *const arg_ln_bias = SPEC == SPEC_RESIDUAL ? nullptr : a.ln_bias;
-    const float *const arg_fold_partial = SPEC == SPEC_UP ? nullptr : a.fold_partial;
+    const float *const arg_fold_partial = (SPEC == SPEC_UP || BT > kConsumerFoldMaxBatch) ? nullptr : a.fold_partial;   // larger batches fold in a kernel of their own
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_sx[BT];
     __shared__ float s_scratch[kPrologueScratch * BT];
@@ -315,6 +315,11 @@ bool linear_fast_supported(int qtype, size_t n, size_t k) {
 int launch_linear(State *st, const LinearArgs &a, char *error, size_t capacity) {
     if (a.batch < 1 || a.batch > kBatchTile) {
         set_error(error, capacity, "linear: batch tile out of range");
+        return -1;
+    }
+    if (a.fold_partial != nullptr && (a.batch > kConsumerFoldMaxBatch || a.k != a.fold_heads * a.fold_head_width || a.fold_slots == nullptr ||
+                                      a.fold_partial_ml == nullptr)) {
+        set_error(error, capacity, "linear: the fold source takes at most two streams and rows of heads x head width");
         return -1;
     }
     if (!linear_fast_supported(a.qtype, (size_t)a.n, (size_t)a.k)) {
