@@ -669,3 +669,128 @@ int orc_encoder_prefill(const orc_encoder *e, const int32_t *ids, size_t T, uint
     free(qh); free(kh); free(vt); free(hc); free(wf);
     return 0;
 }
+
+/* ---- local transformer frame ------------------------------------------------------------------------------------ */
+
+unsigned orc_local_choose(float *logits, size_t vocab, size_t codebook_size, size_t eos_id, orc_local_item *item,
+                          unsigned *greedy, size_t *top_indices, float *top_values) {
+    const int sampling = item->temperature > 0.0f && item->topk > 1u;   /* src/graph.c:1549-1550 (rng_state always present here) */
+    const size_t top_count = item->topk < vocab ? item->topk : vocab;
+    /* src/graph.c:1556-1570: mask and first-max argmax */
+    float best = -FLT_MAX;
+    unsigned argmax = 0;
+    for (size_t c = 0; c < vocab; ++c) {
+        const int is_code = c < codebook_size;
+        const int is_eos = c == eos_id;
+        if (!is_code && !(is_eos && !item->forbid_eos)) {
+            logits[c] = -FLT_MAX;
+            continue;
+        }
+        if (logits[c] > best) {
+            best = logits[c];
+            argmax = (unsigned)c;
+        }
+    }
+    if (greedy != NULL) *greedy = argmax;
+    unsigned value = argmax;
+    if (sampling) {
+        /* src/graph.c:1577-1598: stable insertion of every candidate into a descending list of top_count */
+        size_t used = 0;
+        for (size_t c = 0; c < vocab; ++c) {
+            size_t insert = used;
+            while (insert > 0 && logits[c] > top_values[insert - 1u]) --insert;
+            if (used < top_count) {
+                for (size_t q = used; q > insert; --q) {
+                    top_indices[q] = top_indices[q - 1u];
+                    top_values[q] = top_values[q - 1u];
+                }
+                top_indices[insert] = c;
+                top_values[insert] = logits[c];
+                ++used;
+            } else if (insert < top_count) {
+                for (size_t q = top_count - 1u; q > insert; --q) {
+                    top_indices[q] = top_indices[q - 1u];
+                    top_values[q] = top_values[q - 1u];
+                }
+                top_indices[insert] = c;
+                top_values[insert] = logits[c];
+            }
+        }
+        /* src/graph.c:1599-1616 */
+        const float maximum = top_values[0];
+        float total = 0.0f;
+        for (size_t q = 0; q < used; ++q) {
+            top_values[q] = expf((top_values[q] - maximum) / item->temperature);
+            total += top_values[q];
+        }
+        uint64_t bits = item->rng_state;
+        bits ^= bits << 13;
+        bits ^= bits >> 7;
+        bits ^= bits << 17;
+        item->rng_state = bits == 0 ? UINT64_C(0x9e3779b97f4a7c15) : bits;
+        const float draw = ((float)((item->rng_state >> 40) & UINT64_C(0xffffff)) / (float)UINT64_C(0x1000000)) * total;
+        float cumulative = 0.0f;
+        for (size_t q = 0; q < used; ++q) {
+            cumulative += top_values[q];
+            if (draw <= cumulative || q + 1u == used) {
+                value = (unsigned)top_indices[q];
+                break;
+            }
+        }
+    }
+    return value;
+}
+
+int orc_local_frame(const orc_local *L, size_t batch, const float *const *decoder_last, orc_local_item *items,
+                    float *const *k, float *const *v, unsigned *values, unsigned *stored, int *saw_eos,
+                    size_t *eos_frame, float *logits_out) {
+    const orc_decoder *d = L->stack;
+    const size_t width = d->width, vocab = L->vocab;
+    if (batch == 0 || batch > 16 || d->cross_heads * d->cross_head_width != 0 || d->capacity < L->streams) return -1;
+    float *row_in = (float *)malloc(batch * width * sizeof(float));
+    float *row_out = (float *)malloc(batch * width * sizeof(float));
+    float *logits = (float *)malloc(vocab * sizeof(float));
+    size_t max_top = 1;
+    for (size_t b = 0; b < batch; ++b)
+        if (items[b].topk > max_top) max_top = items[b].topk;
+    if (max_top > vocab) max_top = vocab;
+    size_t *top_indices = (size_t *)malloc(max_top * sizeof(size_t));
+    float *top_values = (float *)malloc(max_top * sizeof(float));
+    const float *in_ptrs[16];
+    float *out_ptrs[16];
+    size_t lengths[16], no_memory[16];
+    for (size_t b = 0; b < batch; ++b) {
+        memcpy(row_in + b * width, decoder_last[b], width * sizeof(float));   /* src/graph.c:1421 */
+        in_ptrs[b] = row_in + b * width;
+        out_ptrs[b] = row_out + b * width;
+        saw_eos[b] = 0;
+        eos_frame[b] = SIZE_MAX;
+        no_memory[b] = 0;
+    }
+    int rc = 0;
+    for (size_t stream = 0; stream < L->streams && rc == 0; ++stream) {
+        for (size_t b = 0; b < batch; ++b) lengths[b] = stream;   /* cache.length restarts at 0 every frame (:1412) */
+        rc = orc_decoder_step(d, batch, k, v, NULL, NULL, lengths, no_memory, in_ptrs, out_ptrs);
+        if (rc != 0) break;
+        for (size_t b = 0; b < batch; ++b) {
+            /* the same projection weight for every item of this stream (:1536-1547) */
+            orc_linear(&L->projection[stream], out_ptrs[b], logits, L->projection_bias != NULL ? L->projection_bias[stream] : NULL,
+                       d->act_variant);
+            unsigned greedy = 0;
+            const unsigned value = orc_local_choose(logits, vocab, L->codebook_size, L->eos_id, &items[b], &greedy, top_indices,
+                                                    top_values);
+            if (logits_out != NULL) memcpy(logits_out + (b * L->streams + stream) * vocab, logits, vocab * sizeof(float));
+            if (greedy == L->eos_id || value == L->eos_id) {   /* :1572-1574, :1617-1622 */
+                saw_eos[b] = 1;
+                const size_t frame = stream / L->codebook_count;
+                if (frame < eos_frame[b]) eos_frame[b] = frame;
+            }
+            const unsigned emit = value < vocab ? value : 0u;                    /* :1626 */
+            values[b * L->streams + stream] = value;
+            stored[b * L->streams + stream] = value < L->codebook_size ? value : 0u;   /* :1627 */
+            memcpy(row_in + b * width, L->audio_table[stream] + (size_t)emit * width, width * sizeof(float));   /* :1651 */
+        }
+    }
+    free(row_in); free(row_out); free(logits); free(top_indices); free(top_values);
+    return rc;
+}

@@ -134,6 +134,37 @@ int orc_encoder_prefill(const orc_encoder *e, const int32_t *ids, size_t T, uint
 /* f32 row-major C[m,n] = A[m,k] * B[n,k]^T, k-contiguous dots (used by the encoder and tests). */
 void orc_gemm_nt(const float *a, const float *b, float *c, size_t m, size_t n, size_t k, int threads);
 
+/* ---- local transformer frame: 16 sequential streams, each a local step + projection + token choice ---- */
+typedef struct {
+    float temperature;     /* sampling iff temperature > 0 && topk > 1 (src/graph.c:1487-1489) */
+    size_t topk;
+    uint64_t rng_state;    /* xorshift64 state, advanced once per sampled stream */
+    int forbid_eos;        /* generated_raw_length < min_raw_length */
+} orc_local_item;
+
+/* One token from one row of logits, as sample_local_frame_batch chooses it (src/graph.c:1548-1616): constrained
+ * first-max argmax (disallowed candidates are overwritten with -FLT_MAX in `logits`), then for sampling items the
+ * top-k insertion sort, expf((l - max) / temperature), xorshift64 draw and cumulative pick.  Returns the value;
+ * *greedy receives the argmax (EOS detection looks at both).  top_indices / top_values: scratch of topk entries. */
+unsigned orc_local_choose(float *logits, size_t vocab, size_t codebook_size, size_t eos_id, orc_local_item *item,
+                          unsigned *greedy, size_t *top_indices, float *top_values);
+
+typedef struct {
+    const orc_decoder *stack;              /* the local transformer: no cross attention, no final norm */
+    size_t streams, vocab, codebook_size, eos_id, codebook_count;
+    const orc_weight *projection;          /* [streams] packed [vocab, width] */
+    const float *const *projection_bias;   /* [streams] [vocab] or NULL entries */
+    const float *const *audio_table;       /* [streams] f32 [vocab, width] */
+} orc_local;
+
+/* sample_local_frame_batch (src/graph.c:1374-1656) for `batch` items that all stay live.  decoder_last[b]: [width].
+ * k/v[b]: [layers, capacity, width] scratch caches (capacity >= streams).  values / stored: [batch, streams] the chosen
+ * token and the code handed on (special tokens collapsed to 0); saw_eos / eos_frame: [batch] (eos_frame = SIZE_MAX when
+ * none); logits_out (optional): [batch, streams, vocab] after the constraint mask. */
+int orc_local_frame(const orc_local *L, size_t batch, const float *const *decoder_last, orc_local_item *items,
+                    float *const *k, float *const *v, unsigned *values, unsigned *stored, int *saw_eos,
+                    size_t *eos_frame, float *logits_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -70,6 +70,8 @@ def _load_oracle():
     lib.orc_output_head.restype = None
     lib.orc_encoder_prefill.restype = C.c_int
     lib.orc_gemm_nt.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, C.c_int]
+    lib.orc_local_choose.restype = C.c_uint
+    lib.orc_local_frame.restype = C.c_int
     return lib
 
 
@@ -331,6 +333,75 @@ def encoder_prefill(cfg, w, ids, threads=8):
     return embed, out
 
 
+# ----------------------------------------------------------------------------- local transformer frame
+class OrcLocalItem(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("topk", _sz), ("rng_state", C.c_uint64), ("forbid_eos", C.c_int)]
+
+
+class OrcLocal(C.Structure):
+    _fields_ = [("stack", C.POINTER(OrcDecoder)), ("streams", _sz), ("vocab", _sz), ("codebook_size", _sz), ("eos_id", _sz),
+                ("codebook_count", _sz), ("projection", C.POINTER(OrcWeight)), ("projection_bias", C.c_void_p),
+                ("audio_table", C.c_void_p)]
+
+
+def local_choose(logits, codebook_size, eos_id, temperature, topk, rng_state, forbid_eos):
+    """One token from one row of logits.  Returns (value, greedy, new_rng_state, masked_logits)."""
+    lg = np.array(logits, dtype=np.float32, copy=True)
+    item = OrcLocalItem(float(temperature), int(topk), int(rng_state), int(bool(forbid_eos)))
+    greedy = C.c_uint(0)
+    n = max(1, min(int(topk), lg.size))
+    top_i = (_sz * n)()
+    top_v = (C.c_float * n)()
+    value = lib.orc_local_choose(_ptr(lg), _sz(lg.size), _sz(codebook_size), _sz(eos_id), C.byref(item), C.byref(greedy), top_i, top_v)
+    return int(value), int(greedy.value), int(item.rng_state), lg
+
+
+class LocalFrame:
+    """orc_local_frame on a local stack (an orc.Decoder without cross attention or final norm), per-stream projections
+    (PackedWeight list), optional biases and f32 audio tables."""
+
+    def __init__(self, stack, projections, biases, audio_tables, codebook_size, eos_id, codebook_count):
+        self.stack, self.projections = stack, projections
+        S = len(projections)
+        self.S, self.vocab = S, projections[0].struct().n
+        self._proj = (OrcWeight * S)(*[p.struct() for p in projections])
+        self._bias_arrays = None if biases is None else [np.ascontiguousarray(b, np.float32) for b in biases]
+        self._tables = [np.ascontiguousarray(t, np.float32) for t in audio_tables]
+        pp = C.c_void_p * S
+        self._bias_ptrs = None if biases is None else pp(*[_ptr(b) for b in self._bias_arrays])
+        self._table_ptrs = pp(*[_ptr(t) for t in self._tables])
+        L = OrcLocal()
+        L.stack = C.pointer(stack.d)
+        L.streams, L.vocab, L.codebook_size, L.eos_id, L.codebook_count = S, self.vocab, codebook_size, eos_id, codebook_count
+        L.projection = self._proj
+        L.projection_bias = None if biases is None else C.cast(self._bias_ptrs, C.c_void_p)
+        L.audio_table = C.cast(self._table_ptrs, C.c_void_p)
+        self.L = L
+
+    def frame(self, decoder_last, items, want_logits=False):
+        """items: list of dicts temperature/topk/rng_state/forbid_eos.  Returns dict with values, stored, saw_eos, eos_frame,
+        rng_state (advanced) and optionally logits [batch, streams, vocab]."""
+        B = len(decoder_last)
+        cfg = self.stack.cfg
+        arr = (OrcLocalItem * B)(*[OrcLocalItem(float(i["temperature"]), int(i["topk"]), int(i["rng_state"]), int(bool(i["forbid_eos"])))
+                                   for i in items])
+        ks = [np.zeros((cfg["layers"], cfg["capacity"], cfg["width"]), np.float32) for _ in range(B)]
+        vs = [np.zeros((cfg["layers"], cfg["capacity"], cfg["width"]), np.float32) for _ in range(B)]
+        rows = [np.ascontiguousarray(r, np.float32) for r in decoder_last]
+        pp = C.c_void_p * B
+        values = np.zeros((B, self.S), np.uint32)
+        stored = np.zeros((B, self.S), np.uint32)
+        saw = np.zeros(B, np.int32)
+        eosf = np.zeros(B, np.uint64)
+        logits = np.zeros((B, self.S, self.vocab), np.float32) if want_logits else None
+        rc = lib.orc_local_frame(C.byref(self.L), _sz(B), pp(*[_ptr(r) for r in rows]), arr, pp(*[_ptr(a) for a in ks]),
+                                 pp(*[_ptr(a) for a in vs]), _ptr(values), _ptr(stored), _ptr(saw), _ptr(eosf), _ptr(logits))
+        if rc != 0:
+            raise RuntimeError("orc_local_frame failed")
+        return {"values": values, "stored": stored, "saw_eos": saw, "eos_frame": eosf,
+                "rng_state": [int(arr[b].rng_state) for b in range(B)], "logits": logits}
+
+
 # ----------------------------------------------------------------------------- compiled reference
 class RefDecoderDesc(C.Structure):
     _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn", _sz), ("xw", _sz),
@@ -385,6 +456,54 @@ def load_ref(strict=False):
     r.ref_decoder_step.restype = C.c_int
     _ref_cache[key] = r
     return r
+
+
+class RefLocalDesc(C.Structure):
+    _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn", _sz), ("capacity", _sz),
+                ("norm_self", C.c_void_p), ("norm_ff", C.c_void_p), ("qkv_w", C.c_void_p), ("o_w", C.c_void_p),
+                ("up_w", C.c_void_p), ("down_w", C.c_void_p), ("position", C.c_void_p)]
+
+
+class RefLocal:
+    """The reference's local_step_batch (src/graph.c:1234-1343) on synthetic weights."""
+
+    def __init__(self, cfg, weights, qtype, batch, strict=False):
+        self.r = load_ref(strict)
+        self.r.ref_local_new.argtypes = [C.POINTER(RefLocalDesc), C.c_int, _sz]
+        self.r.ref_local_new.restype = C.c_void_p
+        self.r.ref_local_free.argtypes = [C.c_void_p]
+        self.r.ref_local_step.restype = C.c_int
+        self.cfg, self.batch = cfg, batch
+        self.keep = {}
+        d = RefLocalDesc()
+        d.layers, d.width, d.heads, d.head_width, d.ffn, d.capacity = (cfg["layers"], cfg["width"], cfg["heads"], cfg["head_width"],
+                                                                       cfg["ffn"], cfg["capacity"])
+        names = {"norm_self": "norm_self_g", "norm_ff": "norm_ff_g", "qkv_w": "qkv", "o_w": "o_self", "up_w": "ffn_up",
+                 "down_w": "ffn_down", "position": "position"}
+        for field, key in names.items():
+            a = np.ascontiguousarray(weights[key], np.float32)
+            self.keep[field] = a
+            setattr(d, field, _ptr(a))
+        self.h = self.r.ref_local_new(C.byref(d), qtype, batch)
+        if not self.h:
+            raise RuntimeError("ref_local_new failed")
+
+    def step(self, ks, vs, lengths, inputs):
+        B = self.batch
+        outs = [np.empty(self.cfg["width"], np.float32) for _ in range(B)]
+        pp = C.c_void_p * B
+        lens = (_sz * B)(*lengths)
+        err = C.create_string_buffer(256)
+        rc = self.r.ref_local_step(C.c_void_p(self.h), pp(*[_ptr(a) for a in ks]), pp(*[_ptr(a) for a in vs]), lens,
+                                   pp(*[_ptr(a) for a in inputs]), pp(*[_ptr(a) for a in outs]), err, _sz(256))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        return outs, list(lens)
+
+    def close(self):
+        if self.h:
+            self.r.ref_local_free(C.c_void_p(self.h))
+            self.h = None
 
 
 class RefDecoder:

@@ -7,6 +7,7 @@
  *
  * Reference functions reached through this shim (file:line in the reference tree):
  *   decoder_step_batch        src/graph.c:3127-3284  (B slots, weight-stationary projections)
+ *   local_step_batch          src/graph.c:1234-1343  (the local transformer's batched step)
  *   layer_norm                src/graph.c:147-150    (gain only, eps 1e-5)
  *   softmax_row_inplace       src/graph.c:245-257
  *   batch_scratch_init        src/graph.c:121-144
@@ -155,3 +156,104 @@ void ref_layer_norm_gain(const float *input, float *output, size_t rows, size_t 
 void ref_softmax_row_inplace(float *values, size_t length) { softmax_row_inplace(values, length); }
 
 float ref_gelu_tanh(float x) { return gelu_tanh(x); }
+
+/* ---- the local transformer's batched step (local_step_batch, src/graph.c:1234-1343) --------------------------
+ * Same pattern: a local_cache (src/graph.c:810-851) and a local_workspace (:928-937) per slot filled by hand;
+ * local_step_batch touches nothing else of the model but qcache and backend. */
+typedef struct {
+    size_t layers, width, heads, head_width, ffn, capacity;   /* layers <= 4 */
+    const float *norm_self;   /* [layers, width] */
+    const float *norm_ff;     /* [layers, width] */
+    const float *qkv_w;       /* [layers, 3*width, width] */
+    const float *o_w;         /* [layers, width, width] */
+    const float *up_w;        /* [layers, ffn, width] */
+    const float *down_w;      /* [layers, width, ffn] */
+    const float *position;    /* [capacity, width] */
+} ref_local_desc;
+
+typedef struct {
+    mynah_tts_model model;
+    local_cache caches[MYNAH_MAX_BATCH];
+    local_workspace workspaces[MYNAH_MAX_BATCH];
+    batch_scratch scratch;
+    size_t batch;
+} ref_local;
+
+void ref_local_free(ref_local *d) {
+    if (d == NULL) return;
+    for (size_t b = 0; b < MYNAH_MAX_BATCH; ++b) {
+        local_workspace *w = &d->workspaces[b];
+        free(w->x); free(w->nrm); free(w->qkv); free(w->attn); free(w->proj); free(w->hidden); free(w->scores);
+        free(w->gelu_scratch);
+    }
+    batch_scratch_free(&d->scratch);
+    if (d->model.qcache != NULL) mynah_qmat_cache_free(d->model.qcache);
+    if (d->model.backend != NULL) mynah_backend_close(d->model.backend);
+    free(d);
+}
+
+ref_local *ref_local_new(const ref_local_desc *desc, int qtype, size_t batch) {
+    if (batch == 0 || batch > MYNAH_MAX_BATCH || desc->layers == 0 || desc->layers > 4) return NULL;
+    ref_local *d = (ref_local *)calloc(1, sizeof(*d));
+    if (d == NULL) return NULL;
+    char error[256];
+    d->batch = batch;
+    if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &d->model.backend, error, sizeof error) != 0) goto fail;
+    d->model.qcache = mynah_qmat_cache_new(qtype);
+    if (d->model.qcache == NULL) goto fail;
+    const size_t w = desc->width, f = desc->ffn;
+    for (size_t b = 0; b < batch; ++b) {
+        local_cache *c = &d->caches[b];
+        c->layers = desc->layers; c->width = w; c->heads = desc->heads; c->head_width = desc->head_width;
+        c->ffn_width = f; c->capacity = desc->capacity; c->position = desc->position;
+        for (size_t l = 0; l < desc->layers; ++l) {
+            c->norm_self[l] = desc->norm_self + l * w;
+            c->norm_ff[l] = desc->norm_ff + l * w;
+            c->qkv_w[l] = desc->qkv_w + l * 3u * w * w;
+            c->o_w[l] = desc->o_w + l * w * w;
+            c->ffn_up_w[l] = desc->up_w + l * f * w;
+            c->ffn_down_w[l] = desc->down_w + l * w * f;
+            snprintf(c->qkv_name[l], sizeof c->qkv_name[l], "synthetic.local%zu.qkv", l);
+            snprintf(c->o_name[l], sizeof c->o_name[l], "synthetic.local%zu.o", l);
+            snprintf(c->ffn_up_name[l], sizeof c->ffn_up_name[l], "synthetic.local%zu.up", l);
+            snprintf(c->ffn_down_name[l], sizeof c->ffn_down_name[l], "synthetic.local%zu.down", l);
+        }
+        local_workspace *ws = &d->workspaces[b];
+        ws->x = (float *)calloc(w, sizeof(float));
+        ws->nrm = (float *)calloc(w, sizeof(float));
+        ws->qkv = (float *)calloc(3u * w, sizeof(float));
+        ws->attn = (float *)calloc(w, sizeof(float));
+        ws->proj = (float *)calloc(w, sizeof(float));
+        ws->hidden = (float *)calloc(f, sizeof(float));
+        ws->scores = (float *)calloc(desc->capacity + 1u, sizeof(float));
+        ws->gelu_scratch = (float *)calloc(f, sizeof(float));
+        if (!ws->x || !ws->nrm || !ws->qkv || !ws->attn || !ws->proj || !ws->hidden || !ws->scores || !ws->gelu_scratch) goto fail;
+    }
+    if (batch_scratch_init(&d->scratch, batch, f > w ? f : w, error, sizeof error) != 0) goto fail;
+    return d;
+fail:
+    ref_local_free(d);
+    return NULL;
+}
+
+/* One batched local step.  k/v[b]: [layers, capacity, width], appended in place at row lengths[b];
+ * lengths[b] comes back advanced by one (src/graph.c:1340). */
+int ref_local_step(ref_local *d, float *const *k, float *const *v, size_t *lengths, const float *const *inputs,
+                   float *const *outs, char *error, size_t error_capacity) {
+    local_cache *caches[MYNAH_MAX_BATCH];
+    local_workspace *workspaces[MYNAH_MAX_BATCH];
+    for (size_t b = 0; b < d->batch; ++b) {
+        d->caches[b].k = k[b];
+        d->caches[b].v = v[b];
+        d->caches[b].length = lengths[b];
+        caches[b] = &d->caches[b];
+        workspaces[b] = &d->workspaces[b];
+    }
+    const int rc = local_step_batch(&d->model, caches, workspaces, inputs, outs, d->batch,
+                                    d->batch > 1u ? &d->scratch : NULL, error, error_capacity);
+    for (size_t b = 0; b < d->batch; ++b) {
+        lengths[b] = d->caches[b].length;
+        d->caches[b].k = d->caches[b].v = NULL;
+    }
+    return rc;
+}
