@@ -258,6 +258,54 @@ enum {
 int mynah_hip_decoder_stage_enqueue(void *state, mynah_hip_decoder *decoder, size_t batch, int stage,
                                     char *error, size_t error_capacity);
 
+/* ---- local-transformer frame ---------------------------------------------------------------- */
+
+/* The per-frame token loop of sample_local_frame_batch (src/graph.c:1374-1656): for each of `streams` codebook
+ * positions one step of the local stack (local_step_batch, :1234-1343 -- a decoder stack without cross attention
+ * and without final norm, its KV cache restarting at 0 every frame), the width -> vocab projection of that position
+ * (:1536-1547, quantised like every other matvec), the token choice (:1548-1616) and the embedding of the chosen
+ * token as the next position's input (:1629-1652).  Everything stays on the device; the host sees the tokens once
+ * per frame instead of once per position. */
+typedef struct {
+    size_t streams;                          /* positions per frame (dep_q * stack_factor; 16) */
+    size_t vocab;                            /* projection rows (<= 8192) */
+    size_t codebook_size;                    /* candidates [0, codebook_size) are codes */
+    size_t eos_id;                           /* the one special token that may be allowed besides the codes */
+    size_t codebook_count;                   /* eos_frame = position / codebook_count (src/graph.c:1620) */
+    const float *const *projection_w;        /* [streams] -> HOST f32 [vocab, width] */
+    const float *const *projection_bias;     /* NULL, or [streams] -> HOST f32 [vocab] (NULL entries allowed) */
+    const float *const *audio_table;         /* [streams] -> HOST f32 [vocab, width]: input row of the next position */
+} mynah_hip_local_desc;
+
+/* One live utterance: the fields of local_batch_item (src/graph.c:1345-1372) the frame reads.  rng_state is the
+ * xorshift64 state itself (the reference holds a pointer; NULL there means "greedy", which is topk <= 1 here) and is
+ * advanced in place when the item samples.  forbid_eos is generated_raw_length < min_raw_length (:1504). */
+typedef struct {
+    const float *dev_decoder_last;   /* device [width]: the decoder's output row for this frame */
+    float temperature;
+    size_t topk;                     /* sampling needs temperature > 0 and topk > 1; min(topk, vocab) <= 256 then */
+    uint64_t rng_state;
+    int forbid_eos;
+} mynah_hip_local_item;
+
+typedef struct mynah_hip_local mynah_hip_local;
+
+/* `stack` describes the local transformer's layers (cross_heads = 0, norm_out = NULL, capacity >= streams,
+ * position = NULL or the local position table).  Converts and caches all weights; owns KV caches for
+ * MYNAH_HIP_MAX_BATCH items. */
+int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc *stack, const mynah_hip_local_desc *desc,
+                           mynah_hip_local **out, char *error, size_t error_capacity);
+void mynah_hip_local_destroy(void *state, mynah_hip_local *local);
+
+/* One frame for `batch` items.  HOST outputs: values[b*streams + s] = chosen token, stored[...] = the token if it
+ * is a code else 0 (src/graph.c:1627), saw_eos[b], eos_frame[b] (SIZE_MAX = none).  dev_logits_copy (optional,
+ * device f32 [batch, streams, vocab]) receives the masked logits every choice was made from.  Synchronous.
+ * Fails with "local frame batch exceeds MYNAH_MAX_BATCH" (:1379-1382) and "local sampler scratch too small"
+ * (:1416-1419; here: a sampling item's min(topk, vocab) above 256). */
+int mynah_hip_local_frame(void *state, mynah_hip_local *local, mynah_hip_local_item *items, size_t batch,
+                          unsigned *values, unsigned *stored, int *saw_eos, size_t *eos_frame,
+                          float *dev_logits_copy, char *error, size_t error_capacity);
+
 /* ---- text-encoder prefill (dense, MFMA) --------------------------------------------------- */
 
 typedef struct {

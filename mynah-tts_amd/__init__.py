@@ -55,6 +55,16 @@ class EncoderDesc(C.Structure):
                 ("norm_out", _vp), ("norm_out_bias", _vp)]
 
 
+class LocalItem(C.Structure):
+    _fields_ = [("dev_decoder_last", _vp), ("temperature", C.c_float), ("topk", _sz), ("rng_state", C.c_uint64),
+                ("forbid_eos", C.c_int)]
+
+
+class LocalDesc(C.Structure):
+    _fields_ = [("streams", _sz), ("vocab", _sz), ("codebook_size", _sz), ("eos_id", _sz), ("codebook_count", _sz),
+                ("projection_w", _vp), ("projection_bias", _vp), ("audio_table", _vp)]
+
+
 def load_library(path=LIB_PATH):
     """dlopen the backend.  Raises (never falls back) when it has not been built."""
     if not os.path.exists(path):
@@ -110,6 +120,10 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_decoder_step.argtypes = [_vp, _vp, C.POINTER(DecoderSlot), _sz, *_err]
     lib.mynah_hip_output_head.argtypes = [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _vp, *_err]
     lib.mynah_hip_decoder_stage_enqueue.argtypes = [_vp, _vp, _sz, C.c_int, *_err]
+    lib.mynah_hip_local_create.argtypes = [_vp, C.POINTER(DecoderDesc), C.POINTER(LocalDesc), C.POINTER(_vp), *_err]
+    lib.mynah_hip_local_destroy.argtypes = [_vp, _vp]
+    lib.mynah_hip_local_destroy.restype = None
+    lib.mynah_hip_local_frame.argtypes = [_vp, _vp, C.POINTER(LocalItem), _sz, _vp, _vp, _vp, _vp, _vp, *_err]
     lib.mynah_hip_encoder_create.argtypes = [_vp, C.POINTER(EncoderDesc), C.POINTER(_vp), *_err]
     lib.mynah_hip_encoder_destroy.argtypes = [_vp, _vp]
     lib.mynah_hip_encoder_destroy.restype = None
@@ -336,40 +350,46 @@ def _ptr_array(arrays):
     return arr
 
 
+def _decoder_desc(backend, cfg, weights, hold):
+    """Fills a DecoderDesc with host pointers the backend keeps alive; `hold` collects the pointer arrays."""
+    L = cfg["layers"]
+
+    def per_layer(name):
+        if weights.get(name) is None:
+            return None
+        rows = [backend.keep(weights[name][l]) for l in range(L)]
+        arr = _ptr_array(rows)
+        hold.append(arr)
+        return C.cast(arr, _vp)
+
+    def single(name):
+        if weights.get(name) is None:
+            return None
+        return _np_ptr(backend.keep(weights[name]))
+
+    d = DecoderDesc()
+    d.layers, d.width, d.heads, d.head_width, d.ffn_width = L, cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
+    d.cross_heads, d.cross_head_width, d.capacity = cfg["cross_heads"], cfg["cross_head_width"], cfg["capacity"]
+    d.norm_self, d.norm_self_bias = per_layer("norm_self_g"), per_layer("norm_self_b")
+    if cfg["cross_heads"]:
+        d.norm_xattn_query, d.norm_xattn_query_bias = per_layer("norm_cross_g"), per_layer("norm_cross_b")
+        d.q_cross_w, d.o_cross_w = per_layer("q_cross"), per_layer("o_cross")
+    d.norm_pos_ff, d.norm_pos_ff_bias = per_layer("norm_ff_g"), per_layer("norm_ff_b")
+    d.qkv_w, d.o_self_w = per_layer("qkv"), per_layer("o_self")
+    d.ffn_up_w, d.ffn_down_w = per_layer("ffn_up"), per_layer("ffn_down")
+    d.norm_out, d.norm_out_bias, d.position = single("norm_out_g"), single("norm_out_b"), single("position")
+    return d
+
+
 class Decoder:
     """mynah_hip_decoder_create + step: the batched resident decode step."""
 
     def __init__(self, backend, cfg, weights):
         self.backend, self.cfg = backend, cfg
-        L = cfg["layers"]
         self._hold = []
-
-        def per_layer(name):
-            if weights.get(name) is None:
-                return None
-            rows = [backend.keep(weights[name][l]) for l in range(L)]
-            arr = _ptr_array(rows)
-            self._hold.append(arr)
-            return C.cast(arr, _vp)
-
-        def single(name):
-            if weights.get(name) is None:
-                return None
-            return _np_ptr(backend.keep(weights[name]))
-
-        d = DecoderDesc()
-        d.layers, d.width, d.heads, d.head_width, d.ffn_width = L, cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
-        d.cross_heads, d.cross_head_width, d.capacity = cfg["cross_heads"], cfg["cross_head_width"], cfg["capacity"]
-        d.norm_self, d.norm_self_bias = per_layer("norm_self_g"), per_layer("norm_self_b")
-        d.norm_xattn_query, d.norm_xattn_query_bias = per_layer("norm_cross_g"), per_layer("norm_cross_b")
-        d.norm_pos_ff, d.norm_pos_ff_bias = per_layer("norm_ff_g"), per_layer("norm_ff_b")
-        d.qkv_w, d.o_self_w = per_layer("qkv"), per_layer("o_self")
-        d.q_cross_w, d.o_cross_w = per_layer("q_cross"), per_layer("o_cross")
-        d.ffn_up_w, d.ffn_down_w = per_layer("ffn_up"), per_layer("ffn_down")
-        d.norm_out, d.norm_out_bias, d.position = single("norm_out_g"), single("norm_out_b"), single("position")
-        self.desc = d
+        self.desc = _decoder_desc(backend, cfg, weights, self._hold)
         h = _vp()
-        backend._call("mynah_hip_decoder_create", C.byref(d), C.byref(h))
+        backend._call("mynah_hip_decoder_create", C.byref(self.desc), C.byref(h))
         self.handle = h
 
     def step(self, slots):
@@ -388,6 +408,49 @@ class Decoder:
     def destroy(self):
         if self.handle:
             self.backend.lib.mynah_hip_decoder_destroy(self.backend.state, self.handle)
+            self.handle = None
+
+
+class Local:
+    """mynah_hip_local_create + frame: the local transformer's per-frame token loop, resident on the device."""
+
+    def __init__(self, backend, cfg, weights, projections, biases, tables, codebook_size, eos_id, codebook_count):
+        self.backend, self.cfg = backend, cfg
+        self._hold = []
+        self.stack_desc = _decoder_desc(backend, cfg, weights, self._hold)
+        self.streams, self.vocab = len(projections), int(projections[0].shape[0])
+        d = LocalDesc()
+        d.streams, d.vocab, d.codebook_size, d.eos_id, d.codebook_count = self.streams, self.vocab, codebook_size, eos_id, codebook_count
+        for name, arrays in (("projection_w", projections), ("projection_bias", biases), ("audio_table", tables)):
+            if arrays is None:
+                continue
+            arr = _ptr_array([None if a is None else backend.keep(a) for a in arrays])
+            self._hold.append(arr)
+            setattr(d, name, C.cast(arr, _vp))
+        self.desc = d
+        h = _vp()
+        backend._call("mynah_hip_local_create", C.byref(self.stack_desc), C.byref(d), C.byref(h))
+        self.handle = h
+
+    def frame(self, items, dev_logits_copy=None):
+        """items: list of dicts {row (device address of the decoder's output row), temperature, topk, rng_state,
+        forbid_eos}.  Returns values, stored [B, streams], saw_eos, eos_frame, rng_state (advanced)."""
+        B = len(items)
+        arr = (LocalItem * B)()
+        for i, it in enumerate(items):
+            arr[i] = LocalItem(it["row"], it["temperature"], it["topk"], it["rng_state"], int(bool(it["forbid_eos"])))
+        values = np.zeros((B, self.streams), np.uint32)
+        stored = np.zeros((B, self.streams), np.uint32)
+        saw = np.zeros(B, np.int32)
+        eos_frame = np.zeros(B, np.uint64)
+        self.backend._call("mynah_hip_local_frame", self.handle, arr, _sz(B), _np_ptr(values), _np_ptr(stored), _np_ptr(saw),
+                           _np_ptr(eos_frame), dev_logits_copy)
+        return {"values": values, "stored": stored, "saw_eos": saw, "eos_frame": eos_frame,
+                "rng_state": [int(arr[i].rng_state) for i in range(B)]}
+
+    def destroy(self):
+        if self.handle:
+            self.backend.lib.mynah_hip_local_destroy(self.backend.state, self.handle)
             self.handle = None
 
 
