@@ -123,6 +123,40 @@ def time_prefill(pkg, synth, backend, tokens=256, runs=30, warmup=5):
     return {"us": us, "flops": flops, "tflops": flops / (us * 1e-6) / 1e12, "tokens": tokens}
 
 
+def time_local(pkg, synth, backend, qtype, batch, frames=40, warmup=5, streams=16, vocab=2048):
+    """The local transformer's frame (16 sequential positions: one 768-wide layer step + 768 -> 2048 projection + token
+    choice), resident on the device.  Every item samples (temperature 0.8, top-k 50).  The frame call is synchronous, so
+    the clock is the host's; the items go up and the tokens come down once per frame inside the timed region."""
+    cfg = synth.decoder_config(layers=1, capacity=streams + 1, cross_heads=0)
+    w = synth.decoder_weights(cfg, seed=7, ln_bias=False)
+    w["norm_out_g"] = w["norm_out_b"] = None
+    rng = np.random.default_rng(8)
+    proj = [(rng.standard_normal((vocab, cfg["width"]), dtype=np.float32) * np.float32(0.05)) for _ in range(streams)]
+    tables = [rng.standard_normal((vocab, cfg["width"]), dtype=np.float32) for _ in range(streams)]
+    loc = pkg.Local(backend, cfg, w, proj, None, tables, vocab - 32, vocab - 31, streams // 2)
+    drows = [backend.alloc(cfg["width"]).write(rng.standard_normal(cfg["width"], dtype=np.float32)) for _ in range(batch)]
+    items = [{"row": d.ptr, "temperature": 0.8, "topk": 50, "rng_state": 1000 + b, "forbid_eos": True} for b, d in enumerate(drows)]
+    out = None
+    for _ in range(warmup):
+        out = loc.frame(items)
+        for it, st in zip(items, out["rng_state"]):
+            it["rng_state"] = st
+    t0 = time.perf_counter()
+    for _ in range(frames):
+        out = loc.frame(items)
+        for it, st in zip(items, out["rng_state"]):
+            it["rng_state"] = st
+    us = (time.perf_counter() - t0) * 1e6 / frames
+    assert np.all(out["values"] < vocab - 32), "forbidden token chosen"
+    loc.destroy()
+    for d in drows:
+        d.free()
+    wd, f = cfg["width"], cfg["ffn"]
+    layer = sum(synth.weight_bytes(n, k, qtype) for n, k in ((3 * wd, wd), (wd, wd), (f, wd), (wd, f)))
+    nbytes = streams * (layer + synth.weight_bytes(vocab, wd, qtype))
+    return {"batch": batch, "frame_us": us, "position_us": us / streams, "bytes": nbytes, "gbps": nbytes / (us * 1e-6) / 1e9}
+
+
 STAGES = [("self-attention", "k_step_attention: LayerNorm + int8 act-quant + per-head Q/K/V rows + KV append + attention over the self cache"),
           ("self-out", "k_linear: fold of attention partials + act-quant + O matvec + residual"),
           ("cross-attention", "k_step_attention: LayerNorm + act-quant + per-head Q rows + attention over the cross cache"),
@@ -179,6 +213,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--skip-b8", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
+    ap.add_argument("--skip-local", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the library's plain read+write kernel over 256 MiB three times (a known-size reference for "
@@ -209,6 +244,7 @@ def main():
                          max(args.warmup // 3, 6), rotate=ROTATE)
         b8["self_lengths"], b8["cross_lengths"] = self_len, cross_len
     prefill = None if args.skip_prefill else time_prefill(pkg, synth, backend)
+    local = None if args.skip_local else [time_local(pkg, synth, backend, qtype, b) for b in (1, 8)]
     backend.close()
 
     result = {
@@ -244,6 +280,13 @@ def main():
                                          "accumulate, %d tokens" % prefill["tokens"],
                              "us": round(prefill["us"], 2), "flops": prefill["flops"], "tflops": round(prefill["tflops"], 2),
                              "bound": "mfma", "peak_tflops": 2500.0, "frac": round(prefill["tflops"] / 2500.0, 4)}
+    if local is not None:
+        result["local"] = {"workload": "local-transformer frame: 16 sequential positions of (one d=768 layer step, %s weights + "
+                                       "768->2048 projection + top-50 temperature sampling), tokens chosen on the device, one "
+                                       "host round trip per frame" % args.quant,
+                           "frames": [{"batch": r["batch"], "frame_us": round(r["frame_us"], 1), "position_us": round(r["position_us"], 2),
+                                       "algorithmic_bytes_per_frame": r["bytes"], "gbps": round(r["gbps"], 1),
+                                       "frac": round(r["gbps"] / PEAK_GBPS, 4)} for r in local]}
     if not args.no_cpu:
         cpu = cpu_baseline()
         allc = cpu.get("all", {})

@@ -151,7 +151,8 @@ static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_
 // passes kAllStages, the per-stage timing entry one bit at a time.
 constexpr unsigned kAllStages = 0x3fu;
 
-static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char *error, size_t capacity, unsigned stages = kAllStages) {
+static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char *error, size_t capacity, unsigned stages = kAllStages,
+                          bool with_end = true) {
     const size_t w = d->width;
     const auto on = [stages](int stage) { return (stages >> stage) & 1u; };
     if (d->fused_attention) {
@@ -173,7 +174,7 @@ static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char
             if (on(MYNAH_HIP_STAGE_FFN_DOWN) &&
                 enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
         }
-        if (stages != kAllStages) return 0;
+        if (stages != kAllStages || !with_end) return 0;
         return launch_step_end(st, d->dev_slots, batch, w, d->x, w, d->norm_out, d->norm_out_b, error, capacity);
     }
     for (size_t l = 0; l < d->layers; ++l) {
@@ -189,7 +190,14 @@ static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char
         if (enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity) != 0) return -1;
         if (enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
     }
+    if (!with_end) return 0;
     return launch_step_end(st, d->dev_slots, batch, w, d->x, w, d->norm_out, d->norm_out_b, error, capacity);
+}
+
+DecoderRows decoder_rows(mynah_hip_decoder *d) { return DecoderRows{d->x, d->dev_slots, d->position}; }
+
+int decoder_enqueue_layers(State *st, mynah_hip_decoder *d, int batch, char *error, size_t capacity) {
+    return enqueue_layers(st, d, batch, error, capacity, kAllStages, false);
 }
 
 static int per_layer_vector(State *st, const float *const *arr, size_t layer, size_t n, const float **dev, char *error,

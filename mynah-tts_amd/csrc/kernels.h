@@ -112,4 +112,16 @@ int launch_step_begin(State *st, const StepSlots &slots, StepSlots *dev_slots, i
 int launch_step_end(State *st, const StepSlots *dev_slots, int batch, size_t width, const float *x, size_t x_stride,
                     const float *gain, const float *bias, char *error, size_t capacity);
 
+// Resident decoder internals for a caller that drives the layers itself (the local frame): the residual rows
+// x[kMaxBatch][width] the layer kernels read and update, the device slot table they take caches and lengths from,
+// and the device position table.  decoder_enqueue_layers puts one step's layer kernels on the stream -- no begin
+// kernel, no output kernel, no graph launch -- and may be captured once every kernel shape has run eagerly.
+struct DecoderRows {
+    float *x;
+    StepSlots *slots;
+    const float *position;
+};
+DecoderRows decoder_rows(mynah_hip_decoder *decoder);
+int decoder_enqueue_layers(State *st, mynah_hip_decoder *decoder, int batch, char *error, size_t capacity);
+
 }  // namespace mynah

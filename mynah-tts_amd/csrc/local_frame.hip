@@ -7,16 +7,19 @@
 // (:1617-1628) and the lookup of the token's embedding as the next position's input (:1629-1652).  Its resident GPU path
 // crosses to the host once per stream (argmax_dev or a d2h of the logits, then an h2d of the embedding row).
 //
-// Here the whole frame stays on the device: the stack's step is the resident decode step of this library
-// (mynah_hip_decoder_step on a decoder without cross attention), the projection is the batched matvec, and one small
-// kernel per stream chooses the token for every item, keeps the generator state and the EOS flags in device memory and
-// gathers the next input row.  The host uploads the per-item parameters once and downloads the tokens once.
+// Here the whole frame stays on the device and is replayed as ONE captured graph per batch size: per position the layer
+// kernels of the resident decode step (a decoder without cross attention), the batched matvec for the projection, and
+// one small kernel that chooses the token for every item, keeps the generator state and the EOS flags in device memory,
+// forms the next position's input row (embedding + position) directly in the stack's residual rows and advances the
+// cache length in the device slot table.  The caches belong to this object, so nothing in the graph changes from frame
+// to frame; what does change (the items) is uploaded once before the graph and the tokens are downloaded once after it.
 //
 // The token choice follows the reference decision for decision: disallowed candidates count as -FLT_MAX, the first
 // maximum wins, the top-k list is ordered by (logit descending, index ascending) -- which is what the reference's
 // insertion loop produces -- the numerators are expf((l - max) / temperature), and total and cumulative sums are formed
 // sequentially in list order by one thread, so that the comparison `draw <= cumulative` sees the same float32 sums.
 #include <float.h>
+#include <string.h>
 
 #include <new>
 
@@ -39,188 +42,284 @@ struct LocalItemDev {
     unsigned long long eos_frame;   // ~0 = none
 };
 
+// Everything a frame brings from the host, uploaded in one copy.
+struct LocalFrameDev {
+    float *logits_copy;             // optional [batch, streams, vocab]: the masked logits, for parity tests
+    LocalItemDev items[kMaxBatch];  // generator state and EOS flags updated in place
+};
+
 struct SampleArgs {
-    LocalItemDev *items;          // [batch], generator state and EOS flags updated in place
-    const float *logits;          // [batch, logits_stride]
-    size_t logits_stride;
-    float *logits_copy;           // optional [batch, streams, vocab]: the masked logits, for parity tests
-    const float *audio_table;     // [vocab, width] of this stream
-    float *row_in;                // [batch, width]: next input of the stack
+    LocalFrameDev *frame;
+    const float *logits;          // [batch, vocab]
+    const float *audio_table;     // [vocab, width] of this position
+    const float *next_position;   // position row of the next step, or null
+    float *x;                     // [batch, width]: residual rows of the stack = its next input
+    StepSlots *slots;             // cache lengths advance here
     unsigned *values, *stored;    // [batch, streams]
     int stream, streams, vocab, codebook_size, eos_id, codebook_count, width;
 };
 
-// Monotone map float -> unsigned: a > b  <=>  key(a) > key(b)  (no NaNs among logits that matter).
+// Monotone map float -> unsigned: a > b  <=>  key(a) > key(b)  (no NaNs among logits that matter), and back.
 __device__ __forceinline__ unsigned order_key(float v) {
     const unsigned u = __float_as_uint(v);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
+__device__ __forceinline__ float key_value(unsigned key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+// (key, index) in one integer whose order is the order of the reference's candidate list: larger logit first, among
+// equal logits the smaller index first.  No two candidates share one, and every one is above zero.
+__device__ __forceinline__ unsigned long long candidate(unsigned key, int index) {
+    return ((unsigned long long)key << 32) | (unsigned long long)(0xffffffffu - (unsigned)index);
+}
+__device__ __forceinline__ int candidate_index(unsigned long long c) { return (int)(0xffffffffu - (unsigned)(c & 0xffffffffull)); }
+__device__ __forceinline__ unsigned candidate_key(unsigned long long c) { return (unsigned)(c >> 32); }
 
-// Exclusive prefix sum of one int per thread over the 256-thread workgroup; *total receives the sum.
-__device__ __forceinline__ int block_exclusive_scan(int v, int *s_scan, int *total) {
-    const int tid = threadIdx.x;
-    s_scan[tid] = v;
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-        const int add = tid >= off ? s_scan[tid - off] : 0;
-        __syncthreads();
-        s_scan[tid] += add;
-        __syncthreads();
+// How many of list[0, n) are above `mine` (pairs of entries per LDS read; the list is 16-byte aligned).
+__device__ __forceinline__ int count_above(const unsigned long long *list, int n, unsigned long long mine) {
+    const ulonglong2 *pairs = reinterpret_cast<const ulonglong2 *>(list);
+    int above = 0;
+#pragma unroll 4
+    for (int j = 0; j < n / 2; ++j) {
+        const ulonglong2 p = pairs[j];
+        above += (p.x > mine ? 1 : 0) + (p.y > mine ? 1 : 0);
     }
-    const int inclusive = s_scan[tid];
-    *total = s_scan[255];
-    __syncthreads();
-    return inclusive - v;
+    if (n & 1) above += list[n - 1] > mine ? 1 : 0;
+    return above;
 }
 
-__global__ void __launch_bounds__(256) k_local_begin(LocalItemDev *items, float *row_in, int width) {
+// Frame start: the slot table (caches of this object, every length 0), x[b] = decoder_last[b] + position[0]
+// (src/graph.c:1420-1422 and :1262-1264), EOS flags cleared (:1409-1410).
+__global__ void __launch_bounds__(256) k_local_begin(LocalFrameDev *frame, const StepSlots slots, StepSlots *dev_slots, float *x,
+                                                     const float *position, int width) {
     const int b = blockIdx.x;
-    const float *src = items[b].decoder_last;
-    for (int d = threadIdx.x; d < width; d += 256) row_in[(size_t)b * width + d] = src[d];   // src/graph.c:1420-1422
+    if (b == 0 && threadIdx.x == 0) *dev_slots = slots;
+    const float *src = frame->items[b].decoder_last;
+    for (int d = threadIdx.x; d < width; d += 256) x[(size_t)b * width + d] = position != nullptr ? src[d] + position[d] : src[d];
     if (threadIdx.x == 0) {
-        items[b].saw_eos = 0;
-        items[b].eos_frame = ~0ull;
+        frame->items[b].saw_eos = 0;
+        frame->items[b].eos_frame = ~0ull;
     }
 }
+
+// Token choice for one item per workgroup.
+//
+// Sampling needs the top_count largest candidates in list order.  Common case: every thread keeps the best of its own
+// (strided) candidates; each wavefront finds the ceil(top_count / 4)-th best among its 64 (bit by bit, with ballots),
+// and the smallest of the four is a lower bound of the wanted threshold with at least top_count candidates at or above
+// it, and usually not many more (some 60 for top-50 of 2048 logits).  Those are collected and ranked against each other,
+// all pairs.  When more than kFastCandidates qualify (large top-k, many equal logits) the
+// threshold is found exactly by radix selection instead and exactly top_count candidates are collected.  Both ways end in
+// the same list, ranked the same way.
+constexpr int kFastCandidates = 512;
 
 __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float *s_lg = reinterpret_cast<float *>(smem);                 // [vocab] masked logits
-    __shared__ int s_scan[256];
-    __shared__ unsigned s_hist[256];
-    __shared__ float s_best[4];
-    __shared__ int s_best_idx[4];
-    __shared__ unsigned s_sel_key[kMaxTopK];
-    __shared__ int s_sel_idx[kMaxTopK];
-    __shared__ float s_top_val[kMaxTopK];
+    unsigned *s_key = reinterpret_cast<unsigned *>(smem);          // [vocab] order keys of the masked logits
+    __shared__ unsigned long long s_head[4];                       // every wavefront's best candidate
+    __shared__ unsigned s_bound[4];
+    __shared__ __align__(16) unsigned long long s_cand[kFastCandidates];
+    __shared__ unsigned s_hist[4][256];
+    __shared__ __align__(16) float s_top_val[kMaxTopK + 8];
     __shared__ int s_top_idx[kMaxTopK];
-    __shared__ unsigned s_prefix;
-    __shared__ int s_remaining;
-    __shared__ unsigned s_value;
+    __shared__ unsigned s_wave_total[4];
+    __shared__ unsigned s_prefix, s_count;
+    __shared__ int s_remaining, s_pick;
+    __shared__ float s_draw;
 
-    const int tid = threadIdx.x, b = blockIdx.x;
-    LocalItemDev &item = a.items[b];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, b = blockIdx.x;
+    LocalItemDev &item = a.frame->items[b];
     const int V = a.vocab;
-    const float *lg = a.logits + (size_t)b * a.logits_stride;
+    const float *lg = a.logits + (size_t)b * V;
     const int forbid_eos = item.forbid_eos;
-
-    // ---- constraint mask (src/graph.c:1556-1563) and first-max argmax (:1564-1569)
-    float best = -FLT_MAX;
-    int best_idx = 0x7fffffff;
-    for (int c = tid; c < V; c += 256) {
-        const bool allowed = c < a.codebook_size || (c == a.eos_id && !forbid_eos);
-        const float v = allowed ? lg[c] : -FLT_MAX;
-        s_lg[c] = v;
-        if (a.logits_copy != nullptr) a.logits_copy[((size_t)b * a.streams + a.stream) * V + c] = v;
-        if (allowed && v > best) { best = v; best_idx = c; }   // strided ascending: the first of equal maxima stays
-    }
-    // lanes, then wavefronts: larger value wins, equal values keep the smaller index
-    for (int off = 32; off >= 1; off >>= 1) {
-        const float ov = __shfl_xor(best, off);
-        const int oi = __shfl_xor(best_idx, off);
-        if (ov > best || (ov == best && oi < best_idx)) { best = ov; best_idx = oi; }
-    }
-    if ((tid & 63) == 0) { s_best[tid >> 6] = best; s_best_idx[tid >> 6] = best_idx; }
-    __syncthreads();
-    best = s_best[0]; best_idx = s_best_idx[0];
-    for (int w = 1; w < 4; ++w)
-        if (s_best[w] > best || (s_best[w] == best && s_best_idx[w] < best_idx)) { best = s_best[w]; best_idx = s_best_idx[w]; }
-    const unsigned argmax = best_idx == 0x7fffffff ? 0u : (unsigned)best_idx;   // nothing above -FLT_MAX: the reference keeps 0
-
     const float temperature = item.temperature;
-    const int top_count = min((int)min(item.topk, (unsigned)V), kMaxTopK);
-    const bool sampling = temperature > 0.0f && item.topk > 1u;
-    if (tid == 0) s_value = argmax;
-    if (sampling) {
-        // ---- the top_count-th largest key by radix selection (four 8-bit digits, most significant first)
-        if (tid == 0) { s_prefix = 0u; s_remaining = top_count; }
-        for (int shift = 24; shift >= 0; shift -= 8) {
-            s_hist[tid] = 0u;
-            __syncthreads();
-            const unsigned prefix = s_prefix;
-            const unsigned high_mask = shift == 24 ? 0u : (0xffffffffu << (shift + 8));
-            for (int c = tid; c < V; c += 256) {
-                const unsigned key = order_key(s_lg[c]);
-                if ((key & high_mask) == (prefix & high_mask)) atomicAdd(&s_hist[(key >> shift) & 0xffu], 1u);
-            }
-            __syncthreads();
-            if (tid == 0) {
-                int remaining = s_remaining;
-                int digit = 255;
-                for (; digit > 0; --digit) {
-                    const int n = (int)s_hist[digit];
-                    if (n >= remaining) break;
-                    remaining -= n;
-                }
-                s_prefix = prefix | ((unsigned)digit << shift);
-                s_remaining = remaining;
-            }
-            __syncthreads();
-        }
-        const unsigned threshold = s_prefix;    // key of the top_count-th largest logit
-        const int take_equal = s_remaining;     // how many candidates with exactly that key belong to the list (earliest first)
+    const unsigned topk = item.topk;
+    float *logits_copy = a.frame->logits_copy;
+    const int top_count = min((int)min(topk, (unsigned)V), kMaxTopK);
+    const bool sampling = temperature > 0.0f && topk > 1u;
 
-        // ---- compaction in index order: [keys above the threshold ..., the first take_equal keys equal to it ...]
-        const int per = (V + 255) / 256;
-        const int c0 = tid * per, c1 = min(V, c0 + per);
-        int n_gt = 0, n_eq = 0;
-        for (int c = c0; c < c1; ++c) {
-            const unsigned key = order_key(s_lg[c]);
-            n_gt += key > threshold;
-            n_eq += key == threshold;
-        }
-        int total_gt = 0, total_eq = 0;
-        int pos_gt = block_exclusive_scan(n_gt, s_scan, &total_gt);
-        int pos_eq = block_exclusive_scan(n_eq, s_scan, &total_eq);
-        for (int c = c0; c < c1; ++c) {
-            const unsigned key = order_key(s_lg[c]);
-            if (key > threshold) {
-                s_sel_key[pos_gt] = key; s_sel_idx[pos_gt] = c; ++pos_gt;
-            } else if (key == threshold) {
-                if (pos_eq < take_equal) { s_sel_key[total_gt + pos_eq] = key; s_sel_idx[total_gt + pos_eq] = c; }
-                ++pos_eq;
+    // ---- constraint mask (src/graph.c:1556-1563); eight candidates per thread are requested at a time
+    unsigned long long mine = 0ull;
+    for (int c0 = tid; c0 < V; c0 += 8 * 256) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = c0 + 256 * i < V ? lg[c0 + 256 * i] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int c = c0 + 256 * i;
+            if (c < V) {
+                const bool allowed = c < a.codebook_size || (c == a.eos_id && !forbid_eos);
+                const float masked = allowed ? v[i] : -FLT_MAX;
+                const unsigned key = order_key(masked);
+                s_key[c] = key;
+                if (logits_copy != nullptr) logits_copy[((size_t)b * a.streams + a.stream) * V + c] = masked;
+                const unsigned long long cand = candidate(key, c);
+                mine = cand > mine ? cand : mine;
             }
         }
-        __syncthreads();
-        // ---- order the list by (logit descending, index ascending): the order the reference's insertion loop builds
-        for (int q = tid; q < top_count; q += 256) {
-            const unsigned key = s_sel_key[q];
-            const int idx = s_sel_idx[q];
-            int rank = 0;
-            for (int j = 0; j < top_count; ++j) rank += s_sel_key[j] > key || (s_sel_key[j] == key && s_sel_idx[j] < idx);
-            s_top_idx[rank] = idx;
-            s_top_val[rank] = s_lg[idx];
+    }
+    for (int p = 0; p < 4; ++p) s_hist[p][tid] = 0u;
+    if (tid == 0) { s_prefix = 0u; s_remaining = top_count; s_count = 0u; s_pick = top_count - 1; }
+    // ---- the head of the list: the largest candidate of the wavefront, then of the four
+    unsigned long long head = mine;
+    for (int off = 32; off >= 1; off >>= 1) {
+        const unsigned long long other = __shfl_xor(head, off);
+        head = other > head ? other : head;
+    }
+    // (sampling) the largest key that at least `want` of the wavefront's 64 bests reach
+    unsigned bound = 0u;
+    if (sampling) {
+        const int want = (top_count + 3) / 4;
+        const unsigned own = candidate_key(mine);
+        for (int bit = 31; bit >= 0; --bit) {
+            const unsigned trial = bound | (1u << bit);
+            if (__popcll(__ballot(own >= trial)) >= want) bound = trial;
+        }
+    }
+    if (lane == 0) { s_head[wave] = head; s_bound[wave] = bound; }
+    __syncthreads();
+    for (int w = 0; w < 4; ++w) {
+        head = s_head[w] > head ? s_head[w] : head;
+        bound = s_bound[w] < bound ? s_bound[w] : bound;
+    }
+    // first-max argmax (src/graph.c:1564-1569): a candidate counts only above -FLT_MAX, otherwise the reference keeps 0
+    const unsigned argmax = candidate_key(head) > order_key(-FLT_MAX) ? (unsigned)candidate_index(head) : 0u;
+    const float maximum = key_value(candidate_key(head));   // the list's first logit (src/graph.c:1599)
+    unsigned value = argmax;
+
+    if (sampling) {
+        // ---- collect the candidates at or above the bound: one LDS counter update per wavefront, places by ballot
+        unsigned in_wave = 0u;
+        for (int base = wave * 64; base < V; base += 256) {
+            const int c = base + lane;
+            in_wave += (unsigned)__popcll(__ballot(c < V && s_key[c] >= bound));
+        }
+        unsigned next_slot = 0u;
+        if (lane == 0) next_slot = atomicAdd(&s_count, in_wave);
+        next_slot = __shfl(next_slot, 0);
+        for (int base = wave * 64; base < V; base += 256) {
+            const int c = base + lane;
+            const unsigned key = c < V ? s_key[c] : 0u;
+            const bool take = c < V && key >= bound;
+            const unsigned long long mask = __ballot(take);
+            const unsigned slot = next_slot + (unsigned)__popcll(mask & ((1ull << lane) - 1ull));
+            if (take && slot < (unsigned)kFastCandidates) s_cand[slot] = candidate(key, c);
+            next_slot += (unsigned)__popcll(mask);
         }
         __syncthreads();
-        // ---- numerators in parallel, sums in list order by one thread (src/graph.c:1599-1616)
-        const float maximum = s_top_val[0];
+        int listed = (int)s_count;
+        if (listed > kFastCandidates) {
+            // ---- the top_count-th largest key by radix selection: four 8-bit digits, most significant first.  Per digit
+            // one LDS histogram of the candidates that share the digits chosen so far; the first wavefront then finds the
+            // bin in which the wanted rank falls (four bins per lane, suffix sums across lanes by shuffles).
+            for (int p = 0; p < 4; ++p) {
+                const int shift = 24 - 8 * p;
+                const unsigned prefix = s_prefix;
+                const int remaining = s_remaining;
+                const unsigned high_mask = p == 0 ? 0u : (0xffffffffu << (shift + 8));
+                for (int c = tid; c < V; c += 256) {
+                    const unsigned key = s_key[c];
+                    if ((key & high_mask) == prefix) atomicAdd(&s_hist[p][(key >> shift) & 0xffu], 1u);
+                }
+                __syncthreads();
+                if (wave == 0) {
+                    int h[4];
+                    for (int j = 0; j < 4; ++j) h[j] = (int)s_hist[p][4 * lane + j];
+                    const int own = h[0] + h[1] + h[2] + h[3];
+                    int suffix = own;   // candidates in the bins of this lane and of all higher lanes
+                    for (int off = 1; off < 64; off <<= 1) {
+                        const int other = __shfl_down(suffix, off);
+                        if (lane + off < 64) suffix += other;
+                    }
+                    int above = suffix - own;   // candidates in bins above the one looked at
+                    for (int j = 3; j >= 0; --j) {
+                        if (above < remaining && remaining <= above + h[j]) {   // true for exactly one bin of one lane
+                            s_prefix = prefix | ((unsigned)(4 * lane + j) << shift);
+                            s_remaining = remaining - above;
+                        }
+                        above += h[j];
+                    }
+                }
+                __syncthreads();
+            }
+            const unsigned threshold = s_prefix;    // key of the top_count-th largest logit
+            const int take_equal = s_remaining;     // how many candidates with exactly that key belong to the list (earliest first)
+            // compaction in index order: [keys above the threshold ..., the first take_equal keys equal to it ...]
+            const int per = (V + 255) / 256;
+            const int c0 = min(V, tid * per), c1 = min(V, c0 + per);
+            unsigned counts = 0u;   // low half: keys above the threshold in [c0, c1); high half: keys equal to it
+            for (int c = c0; c < c1; ++c) {
+                const unsigned key = s_key[c];
+                counts += (key > threshold ? 1u : 0u) + (key == threshold ? 0x10000u : 0u);
+            }
+            unsigned inclusive = counts;
+            for (int off = 1; off < 64; off <<= 1) {
+                const unsigned other = __shfl_up(inclusive, off);
+                if (lane >= off) inclusive += other;
+            }
+            if (lane == 63) s_wave_total[wave] = inclusive;
+            __syncthreads();
+            unsigned before = 0u, total = 0u;
+            for (int w = 0; w < 4; ++w) {
+                if (w < wave) before += s_wave_total[w];
+                total += s_wave_total[w];
+            }
+            const unsigned exclusive = before + inclusive - counts;
+            int pos_gt = (int)(exclusive & 0xffffu), pos_eq = (int)(exclusive >> 16);
+            const int total_gt = (int)(total & 0xffffu);
+            for (int c = c0; c < c1; ++c) {
+                const unsigned key = s_key[c];
+                if (key > threshold) {
+                    s_cand[pos_gt++] = candidate(key, c);
+                } else if (key == threshold) {
+                    if (pos_eq < take_equal) s_cand[total_gt + pos_eq] = candidate(key, c);
+                    ++pos_eq;
+                }
+            }
+            listed = top_count;
+            __syncthreads();
+        }
+        // ---- list position = how many collected candidates come before; numerators expf((l - max) / T) (src/graph.c:1599-1604)
+        for (int q = tid; q < listed; q += 256) {
+            const unsigned long long own = s_cand[q];
+            const int place = count_above(s_cand, listed, own);
+            if (place < top_count) {
+                s_top_idx[place] = candidate_index(own);
+                s_top_val[place] = expf((key_value(candidate_key(own)) - maximum) / temperature);
+            }
+        }
+        if (tid < 8) s_top_val[top_count + tid] = 0.0f;   // lets the running sum below go in whole groups of eight
         __syncthreads();
-        for (int q = tid; q < top_count; q += 256) s_top_val[q] = expf((s_top_val[q] - maximum) / temperature);
-        __syncthreads();
+        // ---- running sums in list order by one thread, kept in place (src/graph.c:1605-1616): float32 sums depend on
+        // the order, and the last running sum is the reference's total
         if (tid == 0) {
-            float total = 0.0f;
-            for (int q = 0; q < top_count; ++q) total += s_top_val[q];
+            float running = 0.0f;
+            for (int q0 = 0; q0 < top_count; q0 += 8) {
+                float part[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) part[i] = s_top_val[q0 + i];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    running += part[i];
+                    s_top_val[q0 + i] = running;
+                }
+            }
             unsigned long long bits = item.rng_state;
             bits ^= bits << 13;
             bits ^= bits >> 7;
             bits ^= bits << 17;
             bits = bits == 0ull ? 0x9e3779b97f4a7c15ull : bits;
             item.rng_state = bits;
-            const float draw = ((float)((bits >> 40) & 0xffffffull) / 16777216.0f) * total;
-            float cumulative = 0.0f;
-            unsigned value = argmax;
-            for (int q = 0; q < top_count; ++q) {
-                cumulative += s_top_val[q];
-                if (draw <= cumulative || q + 1 == top_count) {
-                    value = (unsigned)s_top_idx[q];
-                    break;
-                }
-            }
-            s_value = value;
+            s_draw = ((float)((bits >> 40) & 0xffffffull) / 16777216.0f) * running;
         }
+        __syncthreads();
+        // the first list position whose running sum reaches the draw; the last one if rounding leaves none
+        const float draw = s_draw;
+        for (int q = tid; q < top_count; q += 256)
+            if (draw <= s_top_val[q] && !(q > 0 && draw <= s_top_val[q - 1])) s_pick = q;
+        __syncthreads();
+        value = (unsigned)s_top_idx[s_pick];
     }
-    __syncthreads();
-    const unsigned value = s_value;
     // ---- EOS in either the greedy or the chosen token (src/graph.c:1572-1574,1617-1622), codes, next input row
     if (tid == 0) {
         if (argmax == (unsigned)a.eos_id || value == (unsigned)a.eos_id) {
@@ -230,10 +329,14 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
         }
         a.values[(size_t)b * a.streams + a.stream] = value;
         a.stored[(size_t)b * a.streams + a.stream] = value < (unsigned)a.codebook_size ? value : 0u;   // :1627
+        a.slots->length[b] = a.stream + 1;
     }
-    const unsigned emit = value < (unsigned)V ? value : 0u;                                              // :1626
-    const float *row = a.audio_table + (size_t)emit * a.width;
-    for (int d = tid; d < a.width; d += 256) a.row_in[(size_t)b * a.width + d] = row[d];              // :1651
+    if (a.stream + 1 < a.streams) {
+        const unsigned emit = value < (unsigned)V ? value : 0u;                                          // :1626
+        const float *row = a.audio_table + (size_t)emit * a.width;                                      // :1651
+        const float *pe = a.next_position;                                                             // :1262-1264
+        for (int d = tid; d < a.width; d += 256) a.x[(size_t)b * a.width + d] = pe != nullptr ? row[d] + pe[d] : row[d];
+    }
 }
 
 }  // namespace
@@ -242,22 +345,75 @@ struct mynah_hip_local {
     mynah_hip_decoder *stack = nullptr;
     size_t layers = 0, width = 0, capacity = 0;
     size_t streams = 0, vocab = 0, codebook_size = 0, eos_id = 0, codebook_count = 0;
-    std::vector<const float *> projection_w, projection_bias;   // host pointers (the weight cache keys on them)
-    std::vector<const float *> audio_table;                      // device f32 [vocab, width]
-    float *k = nullptr, *v = nullptr;                            // [kMaxBatch, layers, capacity, width]
-    float *row_in = nullptr, *row_out = nullptr, *logits = nullptr;
-    LocalItemDev *items = nullptr, *items_host = nullptr;        // device / pinned
-    unsigned *values = nullptr, *values_host = nullptr;          // [2, kMaxBatch, streams]: values | stored
+    std::vector<const CachedWeight *> projection;   // [streams], storage of the current quant setting
+    std::vector<const float *> projection_bias;     // [streams] device, or null
+    std::vector<const float *> audio_table;         // [streams] device f32 [vocab, width]
+    int arith = 0;
+    float *k = nullptr, *v = nullptr;               // [kMaxBatch, layers, capacity, width]
+    float *logits = nullptr;                        // [kMaxBatch, vocab]
+    LocalFrameDev *frame = nullptr, *frame_host = nullptr;   // device / pinned
+    unsigned *values = nullptr, *values_host = nullptr;      // [2, kMaxBatch, streams]: values | stored
+    hipGraphExec_t graphs[kMaxBatch + 1] = {};
+    int eager_frames[kMaxBatch + 1] = {};   // a batch size runs eagerly once (one-time kernel set-up) before it is captured
 };
+
+// One frame's kernels on the stream; replayable: nothing here depends on the items.
+static int enqueue_frame(State *st, mynah_hip_local *l, int B, char *error, size_t capacity) {
+    const DecoderRows rows = decoder_rows(l->stack);
+    const int width = (int)l->width;
+    StepSlots slots;
+    memset(&slots, 0, sizeof slots);
+    const size_t per_slot = l->layers * l->capacity * l->width;
+    for (int b = 0; b < B; ++b) {
+        slots.self_k[b] = l->k + (size_t)b * per_slot;
+        slots.self_v[b] = l->v + (size_t)b * per_slot;
+        slots.input[b] = rows.x + (size_t)b * width;
+        slots.output[b] = rows.x + (size_t)b * width;
+    }
+    hipLaunchKernelGGL(k_local_begin, dim3(B), dim3(256), 0, st->stream, l->frame, slots, rows.slots, rows.x, rows.position, width);
+    MYNAH_TRY(hipGetLastError());
+    for (size_t stream = 0; stream < l->streams; ++stream) {
+        if (decoder_enqueue_layers(st, l->stack, B, error, capacity) != 0) return -1;
+        const CachedWeight *cw = l->projection[stream];
+        for (int b0 = 0; b0 < B; b0 += kBatchTile) {
+            LinearArgs p{};
+            p.w = cw->data;
+            p.scales = cw->scales;
+            p.bias = l->projection_bias[stream];
+            p.qtype = cw->qtype;
+            p.n = (int)l->vocab;
+            p.k = width;
+            p.batch = B - b0 < kBatchTile ? B - b0 : kBatchTile;
+            for (int b = 0; b < p.batch; ++b) {
+                p.in[b] = rows.x + (size_t)(b0 + b) * width;
+                p.out[b] = l->logits + (size_t)(b0 + b) * l->vocab;
+            }
+            p.arith = l->arith;
+            p.epilogue = EPI_NONE;
+            if (launch_linear(st, p, error, capacity) != 0) return -1;
+        }
+        SampleArgs a{};
+        a.frame = l->frame; a.logits = l->logits; a.audio_table = l->audio_table[stream];
+        a.next_position = rows.position != nullptr ? rows.position + (stream + 1) * l->width : nullptr;
+        a.x = rows.x; a.slots = rows.slots; a.values = l->values; a.stored = l->values + (size_t)kMaxBatch * l->streams;
+        a.stream = (int)stream; a.streams = (int)l->streams; a.vocab = (int)l->vocab; a.codebook_size = (int)l->codebook_size;
+        a.eos_id = (int)l->eos_id; a.codebook_count = (int)l->codebook_count; a.width = width;
+        hipLaunchKernelGGL(k_local_sample, dim3(B), dim3(256), l->vocab * sizeof(float), st->stream, a);
+        MYNAH_TRY(hipGetLastError());
+    }
+    return 0;
+}
 
 extern "C" void mynah_hip_local_destroy(void *state, mynah_hip_local *l) {
     State *st = static_cast<State *>(state);
     if (l == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
+    for (auto &g : l->graphs)
+        if (g != nullptr) (void)hipGraphExecDestroy(g);
     if (l->stack != nullptr) mynah_hip_decoder_destroy(state, l->stack);
-    for (void *p : {(void *)l->k, (void *)l->v, (void *)l->row_in, (void *)l->row_out, (void *)l->logits, (void *)l->items, (void *)l->values})
+    for (void *p : {(void *)l->k, (void *)l->v, (void *)l->logits, (void *)l->frame, (void *)l->values})
         if (p != nullptr) (void)hipFree(p);
-    if (l->items_host != nullptr) (void)hipHostFree(l->items_host);
+    if (l->frame_host != nullptr) (void)hipHostFree(l->frame_host);
     if (l->values_host != nullptr) (void)hipHostFree(l->values_host);
     delete l;
 }
@@ -276,6 +432,7 @@ extern "C" int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc 
         set_error(error, capacity, "local_create: the stack must have no cross attention and no final norm, capacity >= streams, vocab <= 8192");
         return -1;
     }
+    // with a position table, position streams (one past the last step) is never read: the last choice forms no next row
     mynah_hip_local *l = new (std::nothrow) mynah_hip_local();
     if (l == nullptr) {
         set_error(error, capacity, "out of memory creating the local frame");
@@ -283,7 +440,7 @@ extern "C" int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc 
     }
     auto fail = [&]() { mynah_hip_local_destroy(state, l); return -1; };
     if (mynah_hip_decoder_create(state, stack, &l->stack, error, capacity) != 0) return fail();
-    l->layers = stack->layers; l->width = stack->width; l->capacity = stack->capacity;
+    l->layers = stack->layers; l->width = stack->width; l->capacity = stack->capacity; l->arith = st->arith;
     l->streams = desc->streams; l->vocab = desc->vocab; l->codebook_size = desc->codebook_size; l->eos_id = desc->eos_id;
     l->codebook_count = desc->codebook_count;
     for (size_t s = 0; s < desc->streams; ++s) {
@@ -292,13 +449,16 @@ extern "C" int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc 
             return fail();
         }
         const CachedWeight *cw = nullptr;
-        // converted and cached now, so that the first frame does not pay for it
         if (cached_matrix(st, desc->projection_w[s], desc->vocab, stack->width, st->qtype, &cw, error, capacity) != 0) return fail();
-        l->projection_w.push_back(desc->projection_w[s]);
-        const float *bias = desc->projection_bias != nullptr ? desc->projection_bias[s] : nullptr;
+        if (!linear_fast_supported(cw->qtype, desc->vocab, stack->width)) {
+            set_error(error, capacity, "local_create: projection shape not supported by the fused matvec");
+            return fail();
+        }
+        l->projection.push_back(cw);
         const float *dev_bias = nullptr;
-        if (cached_vector(st, bias, desc->vocab, &dev_bias, error, capacity) != 0) return fail();
-        l->projection_bias.push_back(bias);
+        if (cached_vector(st, desc->projection_bias != nullptr ? desc->projection_bias[s] : nullptr, desc->vocab, &dev_bias, error, capacity) != 0)
+            return fail();
+        l->projection_bias.push_back(dev_bias);
         if (cached_matrix(st, desc->audio_table[s], desc->vocab, stack->width, MYNAH_HIP_F32, &cw, error, capacity) != 0) return fail();
         if (cw->qtype != MYNAH_HIP_F32) {
             set_error(error, capacity, "local_create: audio table could not be kept as f32");
@@ -312,13 +472,11 @@ extern "C" int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc 
         return hip_check(hipMemset(*p, 0, bytes), "local frame workspace clear", error, capacity);
     };
     if (alloc(reinterpret_cast<void **>(&l->k), cache_floats * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&l->v), cache_floats * sizeof(float)) != 0 ||
-        alloc(reinterpret_cast<void **>(&l->row_in), B * l->width * sizeof(float)) != 0 ||
-        alloc(reinterpret_cast<void **>(&l->row_out), B * l->width * sizeof(float)) != 0 ||
         alloc(reinterpret_cast<void **>(&l->logits), B * l->vocab * sizeof(float)) != 0 ||
-        alloc(reinterpret_cast<void **>(&l->items), B * sizeof(LocalItemDev)) != 0 ||
+        alloc(reinterpret_cast<void **>(&l->frame), sizeof(LocalFrameDev)) != 0 ||
         alloc(reinterpret_cast<void **>(&l->values), 2 * B * l->streams * sizeof(unsigned)) != 0)
         return fail();
-    if (hip_check(hipHostMalloc(reinterpret_cast<void **>(&l->items_host), B * sizeof(LocalItemDev), hipHostMallocDefault), "local frame staging", error, capacity) != 0 ||
+    if (hip_check(hipHostMalloc(reinterpret_cast<void **>(&l->frame_host), sizeof(LocalFrameDev), hipHostMallocDefault), "local frame staging", error, capacity) != 0 ||
         hip_check(hipHostMalloc(reinterpret_cast<void **>(&l->values_host), 2 * B * l->streams * sizeof(unsigned), hipHostMallocDefault), "local frame staging", error, capacity) != 0)
         return fail();
     *out = l;
@@ -350,9 +508,11 @@ extern "C" int mynah_hip_local_frame(void *state, mynah_hip_local *l, mynah_hip_
             return -1;
         }
     }
+    const int B = (int)batch;
     MYNAH_TRY(hipStreamSynchronize(st->stream));   // the staging buffers of the previous frame may still be in flight
+    l->frame_host->logits_copy = dev_logits_copy;
     for (size_t b = 0; b < batch; ++b) {
-        LocalItemDev &d = l->items_host[b];
+        LocalItemDev &d = l->frame_host->items[b];
         d.decoder_last = items[b].dev_decoder_last;
         d.temperature = items[b].temperature;
         d.topk = items[b].topk > 0xffffffffu ? 0xffffffffu : (unsigned)items[b].topk;
@@ -361,51 +521,41 @@ extern "C" int mynah_hip_local_frame(void *state, mynah_hip_local *l, mynah_hip_
         d.saw_eos = 0;
         d.eos_frame = ~0ull;
     }
-    MYNAH_TRY(hipMemcpyAsync(l->items, l->items_host, batch * sizeof(LocalItemDev), hipMemcpyHostToDevice, st->stream));
-    const int B = (int)batch, width = (int)l->width;
-    hipLaunchKernelGGL(k_local_begin, dim3(B), dim3(256), 0, st->stream, l->items, l->row_in, width);
-    MYNAH_TRY(hipGetLastError());
-
-    mynah_hip_decoder_slot slots[kMaxBatch];
-    const float *proj_in[kMaxBatch];
-    float *proj_out[kMaxBatch];
-    const size_t per_slot = l->layers * l->capacity * l->width;
-    for (int b = 0; b < B; ++b) {
-        slots[b] = mynah_hip_decoder_slot{};
-        slots[b].dev_self_k = l->k + (size_t)b * per_slot;
-        slots[b].dev_self_v = l->v + (size_t)b * per_slot;
-        slots[b].memory_length = 0;
-        slots[b].dev_input = l->row_in + (size_t)b * width;
-        slots[b].dev_output = l->row_out + (size_t)b * width;
-        proj_in[b] = slots[b].dev_output;
-        proj_out[b] = l->logits + (size_t)b * l->vocab;
-    }
-    unsigned *dev_values = l->values, *dev_stored = l->values + (size_t)kMaxBatch * l->streams;
-    for (size_t stream = 0; stream < l->streams; ++stream) {
-        for (int b = 0; b < B; ++b) slots[b].length = stream;   // the local cache restarts at 0 every frame (src/graph.c:1412)
-        if (mynah_hip_decoder_step(state, l->stack, slots, batch, error, capacity) != 0) return -1;
-        if (mynah_hip_matmul_d2d_batched(state, proj_in, proj_out, batch, l->width, l->vocab, l->projection_w[stream],
-                                         l->projection_bias[stream], error, capacity) != 0)
-            return -1;
-        SampleArgs a{};
-        a.items = l->items; a.logits = l->logits; a.logits_stride = l->vocab; a.logits_copy = dev_logits_copy;
-        a.audio_table = l->audio_table[stream]; a.row_in = l->row_in; a.values = dev_values; a.stored = dev_stored;
-        a.stream = (int)stream; a.streams = (int)l->streams; a.vocab = (int)l->vocab; a.codebook_size = (int)l->codebook_size;
-        a.eos_id = (int)l->eos_id; a.codebook_count = (int)l->codebook_count; a.width = width;
-        hipLaunchKernelGGL(k_local_sample, dim3(B), dim3(256), l->vocab * sizeof(float), st->stream, a);
-        MYNAH_TRY(hipGetLastError());
+    MYNAH_TRY(hipMemcpyAsync(l->frame, l->frame_host, sizeof(LocalFrameDev), hipMemcpyHostToDevice, st->stream));
+    if (!st->graph_mode || l->eager_frames[B] == 0) {
+        l->eager_frames[B] = 1;
+        if (enqueue_frame(st, l, B, error, capacity) != 0) return -1;
+    } else {
+        if (l->graphs[B] == nullptr) {
+            hipGraph_t graph = nullptr;
+            MYNAH_TRY(hipStreamBeginCapture(st->stream, hipStreamCaptureModeThreadLocal));
+            const int rc = enqueue_frame(st, l, B, error, capacity);
+            const hipError_t end = hipStreamEndCapture(st->stream, &graph);
+            if (rc != 0) {
+                if (graph != nullptr) (void)hipGraphDestroy(graph);
+                return -1;
+            }
+            MYNAH_TRY(end);
+            const hipError_t inst = hipGraphInstantiate(&l->graphs[B], graph, nullptr, nullptr, 0);
+            (void)hipGraphDestroy(graph);
+            if (hip_check(inst, "local frame graph instantiate", error, capacity) != 0) {
+                l->graphs[B] = nullptr;
+                return -1;
+            }
+        }
+        MYNAH_TRY(hipGraphLaunch(l->graphs[B], st->stream));
     }
     MYNAH_TRY(hipMemcpyAsync(l->values_host, l->values, 2 * (size_t)kMaxBatch * l->streams * sizeof(unsigned), hipMemcpyDeviceToHost, st->stream));
-    MYNAH_TRY(hipMemcpyAsync(l->items_host, l->items, batch * sizeof(LocalItemDev), hipMemcpyDeviceToHost, st->stream));
+    MYNAH_TRY(hipMemcpyAsync(l->frame_host, l->frame, sizeof(LocalFrameDev), hipMemcpyDeviceToHost, st->stream));
     MYNAH_TRY(hipStreamSynchronize(st->stream));
     for (size_t b = 0; b < batch; ++b) {
         for (size_t s = 0; s < l->streams; ++s) {
             values[b * l->streams + s] = l->values_host[b * l->streams + s];
             stored[b * l->streams + s] = l->values_host[(size_t)kMaxBatch * l->streams + b * l->streams + s];
         }
-        items[b].rng_state = l->items_host[b].rng_state;
-        saw_eos[b] = l->items_host[b].saw_eos;
-        eos_frame[b] = l->items_host[b].eos_frame == ~0ull ? SIZE_MAX : (size_t)l->items_host[b].eos_frame;
+        items[b].rng_state = l->frame_host->items[b].rng_state;
+        saw_eos[b] = l->frame_host->items[b].saw_eos;
+        eos_frame[b] = l->frame_host->items[b].eos_frame == ~0ull ? SIZE_MAX : (size_t)l->frame_host->items[b].eos_frame;
     }
     return 0;
 }
