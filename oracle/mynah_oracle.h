@@ -25,6 +25,15 @@
  *                                                     composition (its encoder is causal with conv FFN), and
  *                                                     its rows>1 GEMM is OpenBLAS, absent here: parity of the
  *                                                     GEMM rounding order is UNPINNED, tolerance 2e-3.
+ *   local step (local_step_batch)                   -- compiled reference's own local_step_batch (f32/int8/int4, both
+ *                                                     flag sets, three positions of a batch of three)
+ *   local token choice and frame bookkeeping (sample_local_frame_batch)
+ *                                                   -- the function needs a whole model object and is not reachable
+ *                                                     in the compiled reference; pinned by what fixes it without it:
+ *                                                     xorshift64 against numpy uint64, mask / first-max hand cases,
+ *                                                     the sampled token against an independent numpy restatement
+ *                                                     (stable sort, float32 sequential sums) on seeded rows with ties,
+ *                                                     draw frequencies against softmax
  */
 #ifndef MYNAH_ORACLE_H
 #define MYNAH_ORACLE_H
