@@ -126,8 +126,13 @@ __device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&b
 // WFIX: model width known at compile time (0 = taken from the arguments): lane-group width, chunks per lane and passes
 // per bank become constants and the per-chunk range checks fold away.  The decoder stack's width (768) gets such a build.
 // SELF: 1 / 0 = self / cross attention known at compile time (the cross build has no new-row roles at all), -1 = from the arguments.
-template <int QT, int NVT, int PF, int WFIX, int SELF>
-__global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a_arg, const int lg_arg, const int per_xcd) {
+// PACKED: how a workgroup finds its work.  0: from its index alone (one or two streams: nearly every unit of the grid
+// exists, and the weight rows can be requested before the slot table has arrived).  1: from its index and the slot
+// table (more streams, ragged lengths: most of a grid sized for the longest possible stream would belong to units that
+// short streams do not have; here the workgroups are numbered over the units that exist, so those with nothing to do
+// are the last ones of the grid and leave after one read instead of holding places among the working ones).
+template <int QT, int NVT, int PF, int WFIX, int SELF, int PACKED>
+__global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a_arg, const int lg_arg, const int per_xcd_arg) {
     extern __shared__ __align__(16) unsigned char smem[];   // staged activations: width bytes (int8/int4) or floats
     __shared__ __align__(16) float s_proj[3 * kHw];         // q | k | v of this head
     __shared__ __align__(16) float s_red[4 * kHw];          // per-wavefront weighted V sums
@@ -145,15 +150,50 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 
     // ---- static work decode: item = (head * batch + stream) * wg_units + unit, XCD x owns items [x*per_xcd, (x+1)*per_xcd).
     // Self-attention: unit 0 = Q+K of the new row, unit 1 = V of the new row, unit 2 + c = cache chunk c.
-    const int wg_units = a.max_units + (is_self ? 1 : 0);
-    const int items = a.heads * a.batch * wg_units;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int item = xcd * per_xcd + slot;
-    if (slot >= per_xcd || item >= items) return;
-    const int unit = item % wg_units;
-    const int hb = item / wg_units;
-    const int b = hb % a.batch;
-    const int head = hb / a.batch;
+    int unit, b, head;
+    if constexpr (PACKED == 0) {
+        const int wg_units = a.max_units + (is_self ? 1 : 0);
+        const int items = a.heads * a.batch * wg_units;
+        const int item = xcd * per_xcd_arg + slot;
+        if (slot >= per_xcd_arg || item >= items) return;
+        unit = item % wg_units;
+        const int hb = item / wg_units;
+        b = hb % a.batch;
+        head = hb / a.batch;
+    } else {
+        // per head: [Q+K and V of every stream's new row (self only)] [the cache chunks that exist, stream by stream]
+        int chunk_items = 0;
+        for (int s = 0; s < a.batch; ++s) {
+            const int len = is_self ? slots->length[s] : slots->memory_length[s];
+            const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+            chunk_items += is_self ? live : max(live, 1);
+        }
+        const int row_items = is_self ? 2 * a.batch : 0;
+        const int per_head = row_items + chunk_items;
+        const int items = a.heads * per_head;
+        const int per_xcd = (items + 7) / 8;
+        const int item = xcd * per_xcd + slot;
+        if (slot >= per_xcd || item >= items) return;
+        head = item / per_head;
+        int r = item - head * per_head;
+        if (r < row_items) {
+            b = r >> 1;
+            unit = r & 1;
+        } else {
+            r -= row_items;
+            b = 0;
+            unit = 0;
+            int before = 0;
+            for (int s = 0; s < a.batch; ++s) {
+                const int len = is_self ? slots->length[s] : slots->memory_length[s];
+                const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+                const int n = is_self ? live : max(live, 1);
+                if (r >= before && r < before + n) { b = s; unit = r - before + (is_self ? 2 : 0); }
+                before += n;
+            }
+        }
+    }
     const bool role_qk = is_self && unit == 0;
     const bool role_v = is_self && unit == 1;
     const int chunk = is_self ? unit - 2 : unit;   // cache chunk of this workgroup (chunk roles only)
@@ -164,7 +204,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     // With many streams most of the grid belongs to units that short streams do not have: there the slot table is
     // looked at first, so that such a workgroup leaves without having requested anything.  With one or two streams
     // nearly every unit is live and the weight rows are requested before the table has arrived (latency matters more).
-    if (a.batch > kConsumerFoldMaxBatch && !(is_self && unit < 2)) {
+    if (PACKED == 0 && a.batch > kConsumerFoldMaxBatch && !(is_self && unit < 2)) {
         const int len = is_self ? slots->length[b] : slots->memory_length[b];
         const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
         if (chunk >= (is_self ? live : max(live, 1))) return;
@@ -394,14 +434,16 @@ int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const dim3 g(grid), t(kThreads);
     if (a.width == 768) {
         // the fixed-shape build needs few enough registers (154 for int8) to hold three workgroups per CU with four-pass banks
-        if (a.is_self) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 1>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        if (a.is_self && latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 1, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        else if (a.is_self) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 1, 1>), g, t, lds, st->stream, a, lg, per_xcd);
+        else if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 0, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 0, 1>), g, t, lds, st->stream, a, lg, per_xcd);
     } else if (a.width <= 1024) {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 0, -1, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 0, -1, 1>), g, t, lds, st->stream, a, lg, per_xcd);
     } else {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput, 0, -1>), g, t, lds, st->stream, a, lg, per_xcd);
+        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency, 0, -1, 0>), g, t, lds, st->stream, a, lg, per_xcd);
+        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput, 0, -1, 1>), g, t, lds, st->stream, a, lg, per_xcd);
     }
     return hip_check(hipGetLastError(), "step attention launch", error, capacity);
 }
