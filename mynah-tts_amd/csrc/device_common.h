@@ -83,9 +83,10 @@ __device__ __forceinline__ int group_sum_i(int v, int lg) {
 // then waves 0..3.  The order never depends on how many of the BT slots are live.  `s_scratch` is 4 * BT floats
 // that no earlier reduction of this workgroup used (each reduction of a kernel gets its own region, so a single
 // barrier per reduction is enough).
+// `wave` is the caller's wavefront index among the four that reduce together (see Team below).
 template <int BT, bool IS_MAX>
-__device__ __forceinline__ void block_reduce(float (&v)[BT], float *s_scratch) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__device__ __forceinline__ void block_reduce(float (&v)[BT], float *s_scratch, const int wave) {
+    const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int b = 0; b < BT; ++b) v[b] = IS_MAX ? wave_max(v[b]) : wave_sum(v[b]);
     if (lane == 0) {
@@ -244,7 +245,7 @@ __device__ __forceinline__ float finish_value(const int iacc, const float facc, 
 
 // Where the prologue takes a stream's activation row from.
 struct ActSource {
-    const float *rows[kBatchTile];   // plain device rows (one per stream of the tile) ...
+    const float *rows[kBatchTile];   // plain device rows, one per stream of the team (rows[0] = the team's first stream) ...
     // ... or the fold of split-L attention partials (resident step): row[b] = sum_u o_u e^(m_u-M) / sum_u l_u e^(m_u-M)
     const float *partial;            // non-null selects the fold: partial outputs [stream][head][max_units][head_width]
     const float *partial_ml;         // chunk maxima and sums [stream][head][2][max_units]
@@ -332,7 +333,19 @@ struct PrologueParams {
     float *probe_sx;
 };
 
-// Stages the activations of up to BT streams in LDS, all 256 threads cooperating on every stream:
+// Who stages which streams.  A team is four wavefronts acting as the 256 threads tid = 0..255 of the staging scheme
+// below for the streams [stream0, stream0 + its stream count).  A 256-thread workgroup is one team for all of its
+// streams.  A 1024-thread workgroup (matvec builds for more than two streams) is four teams that split the streams
+// between them: every thread then touches a quarter of the activations and reduces a quarter of the values, and since
+// a team's four wavefronts hold exactly what the four wavefronts of a one-team workgroup would hold, every sum is
+// formed in the same order -- a stream's staged bytes do not depend on how many teams there were.
+struct Team {
+    int tid;       // 0..255 within the team
+    int stream0;   // first stream of the team
+};
+__device__ __forceinline__ Team whole_workgroup() { return Team{(int)threadIdx.x, 0}; }
+
+// Stages the activations of up to BT streams in LDS, all 256 threads of a team cooperating on every stream:
 // load (or fold) -> optional LayerNorm -> for int8/int4 weights the per-vector absmax int8 quantisation
 // (quantize_act_int8, src/qmat.c:94-113; int4 additionally de-interleaves even/odd elements per run of 8
 // so they line up with the low/high nibbles of a weight dword).  NVT = float4 per thread per stream.
@@ -341,18 +354,19 @@ struct PrologueParams {
 // First half of the prologue: request (or fold) the activation rows and the LayerNorm vectors.  Split from the
 // arithmetic so that a kernel can put other requests between the two (they are served while these are in flight).
 template <int BT, int NVT>
-__device__ __forceinline__ void load_activations(const PrologueParams &p, const ActSource &src, float4 (&xr)[BT][NVT], float4 (&gv)[NVT],
-                                                 float4 (&bv)[NVT]) {
-    const int tid = threadIdx.x;
+__device__ __forceinline__ void load_activations(const PrologueParams &p, const ActSource &src, const Team team, float4 (&xr)[BT][NVT],
+                                                 float4 (&gv)[NVT], float4 (&bv)[NVT]) {
+    const int tid = team.tid;
     const int nf4 = p.k >> 2;
 #pragma unroll
     for (int b = 0; b < BT; ++b)
 #pragma unroll
         for (int i = 0; i < NVT; ++i) {
             const int f = tid + kThreads * i;
-            const bool on = b < p.batch && f < nf4;
+            const int stream = team.stream0 + b;
+            const bool on = stream < p.batch && f < nf4;
             if (!on) xr[b][i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            else if (src.partial != nullptr) xr[b][i] = fold_partials(src, src.stream0 + b, f);
+            else if (src.partial != nullptr) xr[b][i] = fold_partials(src, src.stream0 + stream, f);
             else xr[b][i] = reinterpret_cast<const float4 *>(src.rows[b])[f];
         }
 #pragma unroll
@@ -364,10 +378,13 @@ __device__ __forceinline__ void load_activations(const PrologueParams &p, const 
 }
 
 // Second half: optional LayerNorm -> quantisation (or plain copy) -> LDS.
+// s_scratch: kPrologueScratch floats per stream of the workgroup (all teams).
 template <int QT, int BT, int NVT>
-__device__ __forceinline__ void finish_activations(const PrologueParams &p, float4 (&xr)[BT][NVT], const float4 (&gv)[NVT],
-                                                   const float4 (&bv)[NVT], unsigned char *smem, float *s_sx, float *s_scratch) {
-    const int tid = threadIdx.x;
+__device__ __forceinline__ void finish_activations(const PrologueParams &p, const Team team, float4 (&xr)[BT][NVT], const float4 (&gv)[NVT],
+                                                   const float4 (&bv)[NVT], unsigned char *smem, float *s_sx, float *s_scratch_all) {
+    const int tid = team.tid;
+    const int wave = tid >> 6;
+    float *s_scratch = s_scratch_all + team.stream0 * kPrologueScratch;   // the team's own region
     const int nf4 = p.k >> 2;
     if (p.ln_gain != nullptr) {
         float s[BT];
@@ -377,7 +394,7 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, floa
 #pragma unroll
             for (int i = 0; i < NVT; ++i) s[b] += (xr[b][i].x + xr[b][i].y) + (xr[b][i].z + xr[b][i].w);
         }
-        block_reduce<BT, false>(s, s_scratch);
+        block_reduce<BT, false>(s, s_scratch, wave);
         float mean[BT], v[BT];
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
@@ -393,7 +410,7 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, floa
                     v[b] = __builtin_fmaf(d3, d3, v[b]);
                 }
         }
-        block_reduce<BT, false>(v, s_scratch + 4 * BT);
+        block_reduce<BT, false>(v, s_scratch + 4 * BT, wave);
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
             const float rstd = 1.0f / sqrtf(v[b] / (float)p.k + 1.0e-5f);
@@ -421,11 +438,12 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, floa
                 if (tid + kThreads * i < nf4)
                     amax[b] = fmaxf(fmaxf(amax[b], fmaxf(fabsf(xr[b][i].x), fabsf(xr[b][i].y))), fmaxf(fabsf(xr[b][i].z), fabsf(xr[b][i].w)));
         }
-        block_reduce<BT, true>(amax, s_scratch + 8 * BT);
+        block_reduce<BT, true>(amax, s_scratch + 8 * BT, wave);
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
             const float inv = amax[b] > 0.0f ? 127.0f / amax[b] : 0.0f;
-            unsigned char *dst = smem + (size_t)b * p.k;
+            const int stream = team.stream0 + b;
+            unsigned char *dst = smem + (size_t)stream * p.k;
 #pragma unroll
             for (int i = 0; i < NVT; ++i) {
                 const int f = tid + kThreads * i;
@@ -441,7 +459,7 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, floa
                         *reinterpret_cast<unsigned short *>(dst + block + half) = (unsigned short)((q0 & 0xff) | ((q2 & 0xff) << 8));
                         *reinterpret_cast<unsigned short *>(dst + block + 4 + half) = (unsigned short)((q1 & 0xff) | ((q3 & 0xff) << 8));
                     }
-                    if (p.probe_qx != nullptr && blockIdx.x == 0 && b == 0) {
+                    if (p.probe_qx != nullptr && blockIdx.x == 0 && stream == 0) {
                         p.probe_qx[idx] = (int8_t)q0; p.probe_qx[idx + 1] = (int8_t)q1;
                         p.probe_qx[idx + 2] = (int8_t)q2; p.probe_qx[idx + 3] = (int8_t)q3;
                     }
@@ -450,20 +468,20 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, floa
             if (tid == 0) {
                 // returned activation scale (src/qmat.c:112): amax/127, or amax * f32(1/127) as the stock build folds it
                 const float sx = amax[b] > 0.0f ? (p.arith == MYNAH_HIP_ARITH_STOCK ? amax[b] * (1.0f / 127.0f) : amax[b] / 127.0f) : 0.0f;
-                s_sx[b] = sx;
-                if (p.probe_sx != nullptr && blockIdx.x == 0 && b == 0) p.probe_sx[0] = sx;
+                s_sx[stream] = sx;
+                if (p.probe_sx != nullptr && blockIdx.x == 0 && stream == 0) p.probe_sx[0] = sx;
             }
         }
     } else {
 #pragma unroll
         for (int b = 0; b < BT; ++b) {
-            float4 *dst = reinterpret_cast<float4 *>(smem) + (size_t)b * nf4;
+            float4 *dst = reinterpret_cast<float4 *>(smem) + (size_t)(team.stream0 + b) * nf4;
 #pragma unroll
             for (int i = 0; i < NVT; ++i) {
                 const int f = tid + kThreads * i;
                 if (f < nf4) dst[f] = xr[b][i];
             }
-            if (tid == 0) s_sx[b] = 1.0f;
+            if (tid == 0) s_sx[team.stream0 + b] = 1.0f;
         }
     }
     __syncthreads();
@@ -473,8 +491,8 @@ template <int QT, int BT, int NVT>
 __device__ __forceinline__ void stage_activations(const PrologueParams &p, const ActSource &src, unsigned char *smem, float *s_sx,
                                                   float *s_scratch) {
     float4 xr[BT][NVT], gv[NVT], bv[NVT];
-    load_activations<BT, NVT>(p, src, xr, gv, bv);
-    finish_activations<QT, BT, NVT>(p, xr, gv, bv, smem, s_sx, s_scratch);
+    load_activations<BT, NVT>(p, src, whole_workgroup(), xr, gv, bv);
+    finish_activations<QT, BT, NVT>(p, whole_workgroup(), xr, gv, bv, smem, s_sx, s_scratch);
 }
 
 }  // namespace mynah

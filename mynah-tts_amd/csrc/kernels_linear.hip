@@ -50,8 +50,19 @@ __device__ __forceinline__ float *stream_out(const LinearArgs &a, int b) {
 // GELU epilogue (the step's FFN-up projection).
 enum { SPEC_ANY = 0, SPEC_RESIDUAL = 1, SPEC_UP = 2 };
 
+// More than two streams: the workgroup has four teams of 256 threads (device_common.h) that stage a quarter of the
+// streams each -- staging every stream's activations is what such a launch spends most of its time on, every workgroup
+// has to do all of it, and a quarter of it per thread takes a quarter of the time.  The first team then does the
+// matvec as the only team of a small-batch workgroup would; the others are done once the activations are staged.
+template <int BT>
+constexpr int kLinearTeams = BT > kConsumerFoldMaxBatch ? 4 : 1;
+
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
-__global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
+__global__ void __launch_bounds__(kThreads * kLinearTeams<BT>) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
+    constexpr int kTeams = kLinearTeams<BT>;
+    constexpr int SB = BT / kTeams;   // streams staged by one team
+    const Team team{(int)(threadIdx.x & (kThreads - 1)), (int)(threadIdx.x / kThreads) * SB};
+    const bool worker = kTeams == 1 || threadIdx.x < kThreads;
     // the arguments a specialised build does not look at
     const float *const arg_bias = SPEC != SPEC_ANY ? nullptr : a.bias;
     int8_t *const arg_probe_qx = SPEC != SPEC_ANY ? nullptr : a.probe_qx;
@@ -85,14 +96,20 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
     PrologueParams pro;
     pro.k = k; pro.batch = a.batch; pro.ln_gain = arg_ln_gain; pro.ln_bias = arg_ln_bias; pro.arith = a.arith;
     pro.probe_qx = arg_probe_qx; pro.probe_sx = arg_probe_sx;
-    float4 xr[BT][NVT], gv[NVT], bv[NVT];
+    float4 xr[SB][NVT], gv[NVT], bv[NVT];
     {
         ActSource src;
 #pragma unroll
-        for (int b = 0; b < kBatchTile; ++b) src.rows[b] = a.in[b];
+        for (int b = 0; b < kBatchTile; ++b) {   // the team's own rows first (select chain over the kernel arguments)
+            const float *row = a.in[0];
+#pragma unroll
+            for (int q = 1; q < BT; ++q)
+                if (team.stream0 + b == q) row = a.in[q];
+            src.rows[b] = row;
+        }
         src.partial = arg_fold_partial; src.partial_ml = a.fold_partial_ml; src.slots = a.fold_slots; src.heads = a.fold_heads; src.head_width = a.fold_head_width;
         src.max_units = a.fold_max_units; src.is_self = a.fold_is_self; src.stream0 = a.fold_stream0;
-        load_activations<BT, NVT>(pro, src, xr, gv, bv);
+        load_activations<SB, NVT>(pro, src, team, xr, gv, bv);
     }
     requests_issued();
 
@@ -103,7 +120,7 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
 #pragma unroll
     for (int b = 0; b < BT; ++b) pre_res[b] = 0.0f;
     const bool lanes_finish = BT > 1 && G >= BT;
-    {
+    if (worker) {
         const int row = row_begin + wave * rows_per_pass + gidx;
         const int rowc = row < row_end ? row : row_end - 1;
         const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(a.w) + (size_t)rowc * row_bytes);
@@ -132,7 +149,8 @@ __global__ void __launch_bounds__(kThreads) k_linear(const LinearArgs a, const i
     requests_issued();
 
     // ------------------------------------------------------------------ prologue arithmetic (the weight requests above stay in flight)
-    finish_activations<QT, BT, NVT>(pro, xr, gv, bv, smem, s_sx, s_scratch);
+    finish_activations<QT, SB, NVT>(pro, team, xr, gv, bv, smem, s_sx, s_scratch);
+    if (!worker) return;
 
     // ------------------------------------------------------------------ body
     bool first = true;
@@ -273,7 +291,7 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads), lds, st->stream, a, rows_per_wg, lg);
+    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT>), lds, st->stream, a, rows_per_wg, lg);
     return hip_check(hipGetLastError(), "linear launch", error, capacity);
 }
 

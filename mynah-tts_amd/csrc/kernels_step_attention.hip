@@ -220,7 +220,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     ActSource act;
     act.rows[0] = a.x + (size_t)b * a.width;
     act.partial = nullptr;
-    if constexpr (PF == kPrefetchLatency) load_activations<1, NVT>(pro, act, xr, gv, bv);
+    if constexpr (PF == kPrefetchLatency) load_activations<1, NVT>(pro, act, whole_workgroup(), xr, gv, bv);
     PassRegs pre[PF];
     if (role_qk) load_bank<QT, PF>(pre, a, 0, 0, 2 * kHw, head, lg, chunks);
     else if (role_v) load_bank<QT, PF>(pre, a, 0, 2 * kHw, kHw, head, lg, chunks);
@@ -287,8 +287,8 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     }
 
     // ---- LayerNorm + activation quantisation of x[b], staged in LDS (the cache rows requested above stay in flight)
-    if constexpr (PF != kPrefetchLatency) load_activations<1, NVT>(pro, act, xr, gv, bv);
-    finish_activations<QT, 1, NVT>(pro, xr, gv, bv, smem, s_sx, s_scratch);
+    if constexpr (PF != kPrefetchLatency) load_activations<1, NVT>(pro, act, whole_workgroup(), xr, gv, bv);
+    finish_activations<QT, 1, NVT>(pro, whole_workgroup(), xr, gv, bv, smem, s_sx, s_scratch);
 
     const size_t sh = (size_t)b * a.heads + head;
     float *out_m = a.partial_ml + sh * 2 * a.max_units;
