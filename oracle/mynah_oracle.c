@@ -794,3 +794,65 @@ int orc_local_frame(const orc_local *L, size_t batch, const float *const *decode
     free(row_in); free(row_out); free(logits); free(top_indices); free(top_values);
     return rc;
 }
+
+
+/* ---- codec operators ------------------------------------------------------------------------------------ */
+
+void orc_conv1d_causal(const float *input, float *output, size_t in_channels, size_t out_channels, size_t length,
+                       size_t kernel, size_t dilation, const float *weight, const float *bias) {
+    /* src/graph.c:2141-2154 */
+    for (size_t o = 0; o < out_channels; ++o) {
+        for (size_t t = 0; t < length; ++t) {
+            float value = bias != NULL ? bias[o] : 0.0f;
+            for (size_t i = 0; i < in_channels; ++i) {
+                for (size_t k = 0; k < kernel; ++k) {
+                    const long source = (long)t - (long)((kernel - 1u) * dilation) + (long)(k * dilation);
+                    if (source >= 0) value += weight[(o * in_channels + i) * kernel + k] * input[i * length + (size_t)source];
+                }
+            }
+            output[o * length + t] = value;
+        }
+    }
+}
+
+void orc_conv_transpose_causal(const float *input, float *output, size_t in_channels, size_t out_channels, size_t length,
+                               size_t output_length, size_t kernel, size_t stride, size_t groups, const float *weight,
+                               const float *bias) {
+    /* src/graph.c:2179-2198 */
+    const size_t in_per_group = in_channels / groups, out_per_group = out_channels / groups;
+    for (size_t o = 0; o < out_channels; ++o) {
+        const size_t group = o / out_per_group, o_local = o % out_per_group;
+        float *row = output + o * output_length;
+        for (size_t t = 0; t < output_length; ++t) row[t] = bias != NULL ? bias[o] : 0.0f;
+        for (size_t i = group * in_per_group; i < (group + 1) * in_per_group; ++i) {
+            const float *in_row = input + i * length;
+            const float *w = weight + (i * out_per_group + o_local) * kernel;
+            for (size_t t = 0; t < length; ++t) {
+                const float in_v = in_row[t];
+                for (size_t k = 0; k < kernel; ++k) {
+                    const size_t position = t * stride + k;
+                    if (position < output_length) row[position] += in_v * w[k];
+                }
+            }
+        }
+    }
+}
+
+void orc_snake(float *data, const float *alpha, size_t channels, size_t length, size_t snake_channels) {
+    /* src/backend.c:643-658 */
+    for (size_t c = 0; c < channels; ++c) {
+        float *row = data + c * length;
+        if (c < snake_channels) {
+            const float a = alpha[c];
+            const float inv_a = 1.0f / (a + 1e-9f);
+            for (size_t t = 0; t < length; ++t) {
+                const float v = row[t];
+                const float sn = sinf(a * v);
+                row[t] = v + sn * sn * inv_a;
+            }
+        } else {
+            for (size_t t = 0; t < length; ++t)
+                if (row[t] < 0.0f) row[t] *= 0.01f;
+        }
+    }
+}

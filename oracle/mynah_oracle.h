@@ -34,6 +34,10 @@
  *                                                     the sampled token against an independent numpy restatement
  *                                                     (stable sort, float32 sequential sums) on seeded rows with ties,
  *                                                     draw frequencies against softmax
+ *   codec conv1d / transposed conv / snake          -- compiled reference's conv1d_causal, conv_transpose_causal and
+ *                                                     mynah_backend_snake_dev on a synthetic safetensors file;
+ *                                                     Metal self-test KAT (gpu/metal/backend_metal_ops.m:1026-1106);
+ *                                                     float64 numpy convolution
  */
 #ifndef MYNAH_ORACLE_H
 #define MYNAH_ORACLE_H
@@ -173,6 +177,23 @@ typedef struct {
 int orc_local_frame(const orc_local *L, size_t batch, const float *const *decoder_last, orc_local_item *items,
                     float *const *k, float *const *v, unsigned *values, unsigned *stored, int *saw_eos,
                     size_t *eos_frame, float *logits_out);
+
+/* ---- codec operators (NanoCodec decoder), layout [channels, length] row-major ---- */
+
+/* conv1d_causal (src/graph.c:2010-2160): out[o][t] = bias[o] + sum_i sum_k w[(o*in + i)*kernel + k] *
+ * in[i][t - (kernel-1-k)*dilation], terms with a negative source index dropped.  Accumulates in the order of the
+ * reference's scalar loop (:2141-2154: i outer, k inner); its usual path is im2col + sgemm, whose order is the BLAS's. */
+void orc_conv1d_causal(const float *input, float *output, size_t in_channels, size_t out_channels, size_t length,
+                       size_t kernel, size_t dilation, const float *weight, const float *bias);
+/* conv_transpose_causal (src/graph.c:2179-2231): grouped transposed conv trimmed to output_length = length * stride
+ * when kernel = 2 * stride (in general (length-1)*stride + kernel - (kernel - stride)); per output row the
+ * contributions arrive in the reference's order (input channel, then input position, then tap). */
+void orc_conv_transpose_causal(const float *input, float *output, size_t in_channels, size_t out_channels, size_t length,
+                               size_t output_length, size_t kernel, size_t stride, size_t groups, const float *weight,
+                               const float *bias);
+/* snake_row (src/backend.c:643-658): channels below snake_channels get x + sin(a x)^2 * (1 / (a + 1e-9f)), the rest a
+ * leaky ReLU with slope 0.01. */
+void orc_snake(float *data, const float *alpha, size_t channels, size_t length, size_t snake_channels);
 
 #ifdef __cplusplus
 }

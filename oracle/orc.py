@@ -548,3 +548,77 @@ class RefDecoder:
         if self.h:
             self.r.ref_decoder_free(C.c_void_p(self.h))
             self.h = None
+
+
+# ----------------------------------------------------------------------------- codec operators
+_vp = C.c_void_p
+lib.orc_conv1d_causal.argtypes = [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp, _vp]
+lib.orc_conv1d_causal.restype = None
+lib.orc_conv_transpose_causal.argtypes = [_vp, _vp, _sz, _sz, _sz, _sz, _sz, _sz, _sz, _vp, _vp]
+lib.orc_conv_transpose_causal.restype = None
+lib.orc_snake.argtypes = [_vp, _vp, _sz, _sz, _sz]
+lib.orc_snake.restype = None
+
+
+def conv1d_causal(x, weight, bias, dilation):
+    """x [in, length], weight [out, in, kernel], bias [out] or None -> [out, length]."""
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(weight, np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    out = np.zeros((w.shape[0], x.shape[1]), np.float32)
+    lib.orc_conv1d_causal(_ptr(x), _ptr(out), x.shape[0], w.shape[0], x.shape[1], w.shape[2], dilation, _ptr(w), _ptr(b))
+    return out
+
+
+def conv_transpose_causal(x, weight, bias, stride, groups, output_length=None):
+    """x [in, length], weight [in, out / groups, kernel] -> [out, output_length] (default: length * stride)."""
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(weight, np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    out_ch = w.shape[1] * groups
+    kernel = w.shape[2]
+    if output_length is None:
+        output_length = (x.shape[1] - 1) * stride + kernel - (kernel - stride)
+    out = np.zeros((out_ch, output_length), np.float32)
+    lib.orc_conv_transpose_causal(_ptr(x), _ptr(out), x.shape[0], out_ch, x.shape[1], output_length, kernel, stride, groups, _ptr(w),
+                                  _ptr(b))
+    return out
+
+
+def snake(x, alpha, snake_channels):
+    out = np.array(x, np.float32, copy=True)
+    a = np.ascontiguousarray(alpha, np.float32)
+    lib.orc_snake(_ptr(out), _ptr(a), out.shape[0], out.shape[1], snake_channels)
+    return out
+
+
+def write_safetensors(path, tensors):
+    """A minimal safetensors file (8-byte little-endian header length, JSON header, raw little-endian f32 data) holding the
+    given name -> float32 array map: what the compiled reference's weight loader opens for the codec operators."""
+    import json
+    import struct
+    header, blobs, offset = {}, [], 0
+    for name, value in tensors.items():
+        a = np.ascontiguousarray(value, "<f4")
+        header[name] = {"dtype": "F32", "shape": list(a.shape), "data_offsets": [offset, offset + a.nbytes]}
+        blobs.append(a.tobytes())
+        offset += a.nbytes
+    text = json.dumps(header, separators=(",", ":")).encode()
+    text += b" " * ((8 - len(text) % 8) % 8)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(text)))
+        f.write(text)
+        for blob in blobs:
+            f.write(blob)
+
+
+def ref_codec(strict=False):
+    r = load_ref(strict)
+    fp = C.POINTER(C.c_float)
+    r.ref_conv1d.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, fp, fp, _sz, _sz, _sz, _sz, _sz, C.c_char_p, _sz]
+    r.ref_conv1d.restype = C.c_int
+    r.ref_conv_transpose.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, fp, fp, _sz, _sz, _sz, _sz, _sz, _sz, C.c_char_p, _sz]
+    r.ref_conv_transpose.restype = C.c_int
+    r.ref_snake.argtypes = [fp, fp, _sz, _sz, _sz]
+    r.ref_snake.restype = C.c_int
+    return r

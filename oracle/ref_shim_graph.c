@@ -257,3 +257,45 @@ int ref_local_step(ref_local *d, float *const *k, float *const *v, size_t *lengt
     }
     return rc;
 }
+
+/* ---- codec operators (NanoCodec decoder) -------------------------------------------------------------------
+ * Reference functions reached (file:line in the reference tree):
+ *   conv1d_causal             src/graph.c:2010-2160  (causal dilated conv: im2col + sgemm on the CPU backend)
+ *   conv_transpose_causal     src/graph.c:2200-2231  (grouped causal transposed conv, convt_channel :2179-2198)
+ *   mynah_backend_snake_dev   src/backend.c:660-680  (CPU fallback snake_row :643-658)
+ * The two convolutions look their weights up by name in a mynah_weights file; the caller passes the path of a
+ * safetensors file it wrote itself (synthetic tensors). */
+int ref_conv1d(const char *weights_path, const char *weight_name, const char *bias_name, const float *input, float *output,
+               size_t in_channels, size_t out_channels, size_t length, size_t kernel, size_t dilation, char *error,
+               size_t error_capacity) {
+    mynah_weights *file = NULL;
+    mynah_backend *backend = NULL;
+    int rc = -1;
+    if (mynah_weights_open(weights_path, &file, error, error_capacity) != 0) return -1;
+    if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &backend, error, error_capacity) == 0)
+        rc = conv1d_causal(file, backend, NULL, weight_name, bias_name, input, output, in_channels, out_channels, length, kernel,
+                           dilation, NULL, 0, NULL, error, error_capacity);
+    if (backend != NULL) mynah_backend_close(backend);
+    mynah_weights_close(file);
+    return rc;
+}
+
+int ref_conv_transpose(const char *weights_path, const char *weight_name, const char *bias_name, const float *input, float *output,
+                       size_t in_channels, size_t out_channels, size_t length, size_t kernel, size_t stride, size_t groups,
+                       char *error, size_t error_capacity) {
+    mynah_weights *file = NULL;
+    if (mynah_weights_open(weights_path, &file, error, error_capacity) != 0) return -1;
+    const int rc = conv_transpose_causal(file, weight_name, bias_name, input, output, in_channels, out_channels, length, kernel,
+                                         stride, groups, NULL, error, error_capacity);
+    mynah_weights_close(file);
+    return rc;
+}
+
+int ref_snake(float *data, const float *alpha, size_t channels, size_t length, size_t snake_channels) {
+    char error[256];
+    mynah_backend *backend = NULL;
+    if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &backend, error, sizeof error) != 0) return -1;
+    const int rc = mynah_backend_snake_dev(backend, data, alpha, channels, length, snake_channels, error, sizeof error);
+    mynah_backend_close(backend);
+    return rc;
+}
