@@ -120,6 +120,24 @@ int mynah_hip_clip_dev(void *state, float *dev_data, size_t n, char *error, size
 int mynah_hip_argmax_dev(void *state, const float *dev_logits, size_t vocab, size_t codebook_size, size_t eos_id,
                          int allow_eos, unsigned *argmax, char *error, size_t error_capacity);
 
+/* Codec operators of the resident NanoCodec decode (src/backend.h:60-61,129-133; called from src/graph.c:2463-2490,
+ * 2553-2616), rows of layout [channels, length] in device memory, weight / bias / alpha HOST pointers.  A backend
+ * that registers attention is also given the codec (src/graph.c:2514-2518), which fails hard without these
+ * (:2552-2555): with them MYNAH_METAL_CPU_CODEC is not needed.
+ * conv1d: causal, dilated; weight [out, in, kernel]; bias may be NULL (conv1d_causal, src/graph.c:2010-2160); runs
+ *   on the f32 matrix cores; kernel <= 16, (kernel - 1) * dilation <= 128.
+ * conv_transpose_dev: grouped, weight [in, out / groups, kernel], output trimmed to output_length; bit-identical to
+ *   the reference's scalar loop (convt_channel, src/graph.c:2179-2198).
+ * snake_dev: in place; rows below snake_channels get x + sin(a x)^2 / (a + 1e-9), the rest a leaky ReLU of slope 0.01
+ *   (snake_row, src/backend.c:643-658). */
+int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                     int kernel, int dilation, const float *weight, const float *bias, char *error, size_t error_capacity);
+int mynah_hip_conv_transpose_dev(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels,
+                                 int length, int output_length, int kernel, int stride, int groups, const float *weight,
+                                 const float *bias, char *error, size_t error_capacity);
+int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length,
+                        size_t snake_channels, char *error, size_t error_capacity);
+
 /* ------------------------------------------------------------------------------------------
  * Section 2 -- what the single-stream seam lacks
  * ------------------------------------------------------------------------------------------ */

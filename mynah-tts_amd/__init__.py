@@ -101,6 +101,10 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_scale_dev.argtypes = [_vp, _vp, _sz, C.c_float, *_err]
     lib.mynah_hip_clip_dev.argtypes = [_vp, _vp, _sz, *_err]
     lib.mynah_hip_argmax_dev.argtypes = [_vp, _vp, _sz, _sz, _sz, C.c_int, C.POINTER(C.c_uint), *_err]
+    lib.mynah_hip_conv1d.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp, *_err]
+    lib.mynah_hip_conv_transpose_dev.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp,
+                                                 *_err]
+    lib.mynah_hip_snake_dev.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, *_err]
     lib.mynah_hip_set_quant.argtypes = [_vp, C.c_int, C.c_int, *_err]
     lib.mynah_hip_quantize_weight_int8.argtypes = [_vp, _sz, _sz, _vp, _vp, C.c_int]
     lib.mynah_hip_quantize_weight_int8.restype = None
@@ -283,6 +287,17 @@ class Backend:
 
     def clip_dev(self, d, n):
         self._call("mynah_hip_clip_dev", _vp(d), _sz(n))
+
+    def conv1d(self, din, dout, in_ch, out_ch, length, kernel, dilation, weight, bias=None):
+        self._call("mynah_hip_conv1d", din, dout, in_ch, out_ch, length, kernel, dilation, _np_ptr(self.keep(weight)),
+                   None if bias is None else _np_ptr(self.keep(bias)))
+
+    def conv_transpose_dev(self, din, dout, in_ch, out_ch, length, output_length, kernel, stride, groups, weight, bias=None):
+        self._call("mynah_hip_conv_transpose_dev", din, dout, in_ch, out_ch, length, output_length, kernel, stride, groups,
+                   _np_ptr(self.keep(weight)), None if bias is None else _np_ptr(self.keep(bias)))
+
+    def snake_dev(self, d, alpha, channels, length, snake_channels):
+        self._call("mynah_hip_snake_dev", d, _np_ptr(self.keep(alpha)), _sz(channels), _sz(length), _sz(snake_channels))
 
     def argmax_dev(self, dlogits, vocab, codebook_size, eos_id, allow_eos):
         out = C.c_uint(0)

@@ -1,0 +1,262 @@
+// Codec operators of the resident NanoCodec decode (decode_codec_resident, src/graph.c:2504-2638; res_layer_device
+// :2423-2498): causal dilated conv1d, grouped causal transposed conv and the half-snake activation, on device rows of
+// layout [channels, length].  Weights, biases and snake alphas arrive as HOST pointers and are cached on the device at
+// first sight like every other weight (the seam's contract).  None of the three synchronises.
+//
+//   conv1d          out[o][t] = bias[o] + sum_i sum_k w[(o*in + i)*K + k] * in[i][t - (K-1-k)*dilation]   (conv1d_causal,
+//                   src/graph.c:2010-2160).  The reference builds an im2col matrix and calls sgemm; here the same GEMM
+//                   (M = out channels, N = length, inner = in channels x taps) runs on the f32 matrix cores with the
+//                   im2col done by addressing: a workgroup stages the input rows of eight channels once, with a halo of
+//                   (K-1)*dilation positions, and every tap reads the same rows at its own offset.  f32 operands,
+//                   f32 accumulation (v_mfma_f32_32x32x2_f32); only the order of the additions differs from the CPU's.
+//   conv_transpose  grouped, trimmed to output_length (conv_transpose_causal / convt_channel, src/graph.c:2179-2231):
+//                   one thread per output element, contributions added in the reference's order (input channel, then
+//                   input position), so the result is bit-identical to the scalar CPU loop.
+//   snake           x + sin(a x)^2 * (1 / (a + 1e-9)) on the first snake_channels rows, leaky ReLU (0.01) on the rest
+//                   (snake_row, src/backend.c:643-658).
+#include <limits.h>
+
+#include "kernels.h"
+
+using namespace mynah;
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kConvChannels = 8;      // input channels staged per step of the inner dimension
+constexpr int kConvMaxKernel = 16;
+constexpr int kConvMaxHalo = 128;     // (kernel - 1) * dilation
+
+struct ConvArgs {
+    const float *in;     // [in_ch, length]
+    float *out;          // [out_ch, length]
+    const float *w;      // [out_ch, in_ch * kernel]
+    const float *bias;   // [out_ch] or null
+    int in_ch, out_ch, length, kernel, dilation;
+};
+
+// Workgroup tile: (32 * WM) output channels x (64 * WN) positions; a wavefront owns 32 x 64 (two 32 x 32 accumulators).
+template <int WM, int WN>
+__global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a) {
+    constexpr int TM = 32 * WM, TN = 64 * WN;
+    extern __shared__ __align__(16) float lds[];
+    const int kb = kConvChannels * a.kernel;   // inner elements per step (even)
+    const int a_stride = kb | 1;               // odd row stride: the 32 rows a wavefront reads land in 32 different banks
+    const int halo = (a.kernel - 1) * a.dilation;
+    const int win = TN + halo;                 // staged positions per input channel
+    float *s_w = lds;                          // [TM][a_stride]
+    float *s_in = lds + TM * a_stride;         // [kConvChannels][win]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int m0 = blockIdx.y * TM, t0 = blockIdx.x * TN;
+    const int inner = a.in_ch * a.kernel;
+
+    // Staging slots of a thread: weights -- row (tid / 16) + 16 * g, column (tid % 16) + 16 * c of the step's TM x kb
+    // block; input rows -- channel ch, position tid + 256 * x of the window.  Fixed loops, no divisions.
+    constexpr int kRowGroups = TM / 16, kColGroups = kConvChannels * kConvMaxKernel / 16, kWinParts = (TN + kConvMaxHalo + 255) / 256;
+    float stage_w[kRowGroups][kColGroups], stage_in[kConvChannels][kWinParts];
+    const int srow = tid >> 4, scol = tid & 15;
+    const auto fetch = [&](int i0) {   // global -> registers: the weight columns and input rows of channels [i0, i0 + 8)
+#pragma unroll
+        for (int g = 0; g < kRowGroups; ++g) {
+            const int m = m0 + srow + 16 * g;
+#pragma unroll
+            for (int c = 0; c < kColGroups; ++c) {
+                const int cc = scol + 16 * c, ci = i0 * a.kernel + cc;
+                stage_w[g][c] = (cc < kb && m < a.out_ch && ci < inner) ? a.w[(size_t)m * inner + ci] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int ch = 0; ch < kConvChannels; ++ch) {
+            const int i = i0 + ch;
+#pragma unroll
+            for (int x = 0; x < kWinParts; ++x) {
+                const int xx = tid + 256 * x, t = t0 - halo + xx;
+                stage_in[ch][x] = (xx < win && i < a.in_ch && t >= 0 && t < a.length) ? a.in[(size_t)i * a.length + t] : 0.0f;
+            }
+        }
+    };
+    const auto publish = [&]() {   // registers -> LDS
+#pragma unroll
+        for (int g = 0; g < kRowGroups; ++g)
+#pragma unroll
+            for (int c = 0; c < kColGroups; ++c) {
+                const int cc = scol + 16 * c;
+                if (cc < kb) s_w[(srow + 16 * g) * a_stride + cc] = stage_w[g][c];
+            }
+#pragma unroll
+        for (int ch = 0; ch < kConvChannels; ++ch)
+#pragma unroll
+            for (int x = 0; x < kWinParts; ++x) {
+                const int xx = tid + 256 * x;
+                if (xx < win) s_in[ch * win + xx] = stage_in[ch][x];
+            }
+    };
+
+    floatx16 acc0, acc1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
+    const int half = lane >> 5, col = lane & 31;
+    fetch(0);
+    for (int i0 = 0; i0 < a.in_ch; i0 += kConvChannels) {
+        publish();
+        __syncthreads();
+        if (i0 + kConvChannels < a.in_ch) fetch(i0 + kConvChannels);   // in flight during the products below
+        // this lane's inner index runs half, half + 2, ...: (channel, tap) kept as counters instead of dividing
+        int ch = 0, k = half;
+        if (k >= a.kernel) { k -= a.kernel; ++ch; }
+        const float *wrow = s_w + (wm * 32 + col) * a_stride + half;
+        const float *irow = s_in + wn * 64 + col;
+#pragma unroll 4
+        for (int q = 0; q < kb; q += 2) {
+            const float wv = wrow[q];
+            const float *src = irow + ch * win + k * a.dilation;
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv, src[0], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv, src[32], acc1, 0, 0, 0);
+            k += 2;
+            if (k >= a.kernel) { k -= a.kernel; ++ch; }   // kernel 1 wraps twice
+            if (k >= a.kernel) { k -= a.kernel; ++ch; }
+        }
+        __syncthreads();
+    }
+    // accumulator element r of a lane: row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (m < a.out_ch) {
+            const float b = a.bias != nullptr ? a.bias[m] : 0.0f;
+            const int t = t0 + wn * 64 + col;
+            if (t < a.length) a.out[(size_t)m * a.length + t] = acc0[r] + b;
+            if (t + 32 < a.length) a.out[(size_t)m * a.length + t + 32] = acc1[r] + b;
+        }
+    }
+}
+
+struct ConvTransposeArgs {
+    const float *in;     // [in_ch, length]
+    float *out;          // [out_ch, output_length]
+    const float *w;      // [in_ch, out_ch / groups, kernel]
+    const float *bias;   // [out_ch] or null
+    int in_ch, out_ch, length, output_length, kernel, stride, groups;
+};
+
+__global__ void __launch_bounds__(256) k_conv_transpose(const ConvTransposeArgs a) {
+    const size_t index = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (index >= (size_t)a.out_ch * a.output_length) return;
+    const int p = (int)(index % a.output_length), o = (int)(index / a.output_length);
+    const int ipg = a.in_ch / a.groups, opg = a.out_ch / a.groups;
+    const int group = o / opg, o_local = o - group * opg;
+    float value = a.bias != nullptr ? a.bias[o] : 0.0f;
+    // input positions t with 0 <= p - t * stride < kernel
+    const int t_hi = min(a.length - 1, p / a.stride);
+    const int t_lo = p < a.kernel ? 0 : (p - a.kernel) / a.stride + 1;
+    for (int i = group * ipg; i < (group + 1) * ipg; ++i) {
+        const float *in_row = a.in + (size_t)i * a.length;
+        const float *w = a.w + ((size_t)i * opg + o_local) * a.kernel;
+        for (int t = t_lo; t <= t_hi; ++t) value += in_row[t] * w[p - t * a.stride];
+    }
+    a.out[index] = value;
+}
+
+__global__ void __launch_bounds__(256) k_snake(float *data, const float *alpha, size_t count, int length, int snake_channels) {
+    const size_t index = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (index >= count) return;
+    const int channel = (int)(index / (size_t)length);
+    const float v = data[index];
+    if (channel < snake_channels) {
+        const float al = alpha[channel];
+        const float inv_a = 1.0f / (al + 1e-9f);
+        const float sn = sinf(al * v);
+        data[index] = v + sn * sn * inv_a;
+    } else if (v < 0.0f) {
+        data[index] = v * 0.01f;
+    }
+}
+
+template <int WM, int WN>
+int launch_conv(State *st, const ConvArgs &a, char *error, size_t capacity) {
+    constexpr int TM = 32 * WM, TN = 64 * WN;
+    const int kb = kConvChannels * a.kernel;
+    const size_t lds = ((size_t)TM * (kb | 1) + (size_t)kConvChannels * (TN + (a.kernel - 1) * a.dilation)) * sizeof(float);
+    static bool raised = false;   // per instantiation
+    if (lds > 48 * 1024 && !raised) {
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        raised = true;
+    }
+    const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM));
+    hipLaunchKernelGGL((k_conv1d<WM, WN>), grid, dim3(256), lds, st->stream, a);
+    return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
+}
+
+}  // namespace
+
+extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                                int kernel, int dilation, const float *weight, const float *bias, char *error, size_t capacity) {
+    State *st = static_cast<State *>(state);
+    if (st == nullptr || dev_input == nullptr || dev_output == nullptr || weight == nullptr || in_channels <= 0 || out_channels <= 0 ||
+        length <= 0 || kernel <= 0 || dilation <= 0) {
+        set_error(error, capacity, "invalid conv1d arguments");   // the checks of metal_ops_conv1d, gpu/metal/backend_metal_ops.m:371-372
+        return -1;
+    }
+    if (kernel > kConvMaxKernel || (kernel - 1) * (long)dilation > kConvMaxHalo || (size_t)in_channels * kernel > (size_t)INT_MAX ||
+        (size_t)in_channels * (size_t)length > (size_t)INT_MAX * 4u || (size_t)out_channels * (size_t)length > (size_t)INT_MAX * 4u) {
+        set_error(error, capacity, "conv1d: kernel above 16 taps, reach above 128 positions or tensor too large");
+        return -1;
+    }
+    const CachedWeight *cw = nullptr;
+    if (cached_matrix(st, weight, (size_t)out_channels, (size_t)in_channels * kernel, MYNAH_HIP_F32, &cw, error, capacity) != 0) return -1;
+    if (cw->qtype != MYNAH_HIP_F32) {
+        set_error(error, capacity, "conv1d: weight could not be kept as f32");
+        return -1;
+    }
+    const float *dev_bias = nullptr;
+    if (cached_vector(st, bias, (size_t)out_channels, &dev_bias, error, capacity) != 0) return -1;
+    ConvArgs a{dev_input, dev_output, static_cast<const float *>(cw->data), dev_bias, in_channels, out_channels, length, kernel, dilation};
+    // few output channels: one row of wavefronts, wider in time
+    if (out_channels <= 32) return launch_conv<1, 4>(st, a, error, capacity);
+    return launch_conv<2, 2>(st, a, error, capacity);
+}
+
+extern "C" int mynah_hip_conv_transpose_dev(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels,
+                                            int length, int output_length, int kernel, int stride, int groups, const float *weight,
+                                            const float *bias, char *error, size_t capacity) {
+    State *st = static_cast<State *>(state);
+    if (st == nullptr || dev_input == nullptr || dev_output == nullptr || weight == nullptr || in_channels <= 0 || out_channels <= 0 ||
+        length <= 0 || output_length <= 0 || kernel <= 0 || stride <= 0 || groups <= 0 || in_channels % groups != 0 ||
+        out_channels % groups != 0) {
+        set_error(error, capacity, "invalid conv_transpose arguments");
+        return -1;
+    }
+    const size_t per_in = (size_t)(out_channels / groups) * kernel;
+    const CachedWeight *cw = nullptr;
+    if (cached_matrix(st, weight, (size_t)in_channels, per_in, MYNAH_HIP_F32, &cw, error, capacity) != 0) return -1;
+    if (cw->qtype != MYNAH_HIP_F32) {
+        set_error(error, capacity, "conv_transpose: weight could not be kept as f32");
+        return -1;
+    }
+    const float *dev_bias = nullptr;
+    if (cached_vector(st, bias, (size_t)out_channels, &dev_bias, error, capacity) != 0) return -1;
+    ConvTransposeArgs a{dev_input, dev_output, static_cast<const float *>(cw->data), dev_bias, in_channels, out_channels, length,
+                        output_length, kernel, stride, groups};
+    const size_t count = (size_t)out_channels * output_length;
+    hipLaunchKernelGGL(k_conv_transpose, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st->stream, a);
+    return hip_check(hipGetLastError(), "conv_transpose launch", error, capacity);
+}
+
+extern "C" int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length, size_t snake_channels,
+                                   char *error, size_t capacity) {
+    State *st = static_cast<State *>(state);
+    if (st == nullptr || dev_data == nullptr || channels > (size_t)INT_MAX || length > (size_t)INT_MAX || snake_channels > channels ||
+        (snake_channels != 0 && alpha == nullptr)) {
+        set_error(error, capacity, "invalid snake arguments");   // metal_ops_snake, gpu/metal/backend_metal_ops.m:343-346
+        return -1;
+    }
+    const size_t count = channels * length;
+    if (count == 0) return 0;
+    const float *dev_alpha = nullptr;
+    if (snake_channels != 0 && cached_vector(st, alpha, snake_channels, &dev_alpha, error, capacity) != 0) return -1;
+    hipLaunchKernelGGL(k_snake, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st->stream, dev_data, dev_alpha, count, (int)length,
+                       (int)snake_channels);
+    return hip_check(hipGetLastError(), "snake launch", error, capacity);
+}
