@@ -157,6 +157,84 @@ def time_local(pkg, synth, backend, qtype, batch, frames=40, warmup=5, streams=1
     return {"batch": batch, "frame_us": us, "position_us": us / streams, "bytes": nbytes, "gbps": nbytes / (us * 1e-6) / 1e9}
 
 
+def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
+    """The resident NanoCodec decode's operator sequence (decode_codec_resident / res_layer_device, src/graph.c:2423-2638)
+    on synthetic weights: 32 -> 864 pre-conv, five stages of half-snake, grouped transposed conv (rates 8 8 4 2 2, channels
+    halving) and a residual layer of 3 branches x 3 x (snake, conv k, snake, conv k) with k = 3 / 7 / 11 and dilations
+    1 / 3 / 5, then snake, the 1-channel post-conv and the clip.  f32 throughout; the convolutions run on the f32 matrix
+    cores.  Timed with HIP events on the backend's stream over whole decodes of `frames` raw frames."""
+    rng = np.random.default_rng(11)
+
+    def conv_w(out_ch, in_ch, k):
+        return (rng.standard_normal((out_ch, in_ch, k), dtype=np.float32) * np.float32(1.0 / np.sqrt(in_ch * k))), \
+               rng.standard_normal(out_ch, dtype=np.float32) * np.float32(0.1)
+
+    def alpha(c):
+        return (np.abs(rng.standard_normal(c // 2, dtype=np.float32)) + np.float32(0.1))
+
+    rates, kernels, dilations = (8, 8, 4, 2, 2), (3, 7, 11), (1, 3, 5)
+    pre = conv_w(864, 32, 7)
+    stages, flops = [], 2.0 * 864 * 32 * 7 * frames
+    C, L = 864, frames
+    for rate in rates:
+        nc, nl = C // 2, L * rate
+        up_w = rng.standard_normal((C, 1, 2 * rate), dtype=np.float32) * np.float32(0.3)
+        blocks = [[(alpha(nc), conv_w(nc, nc, k), alpha(nc), conv_w(nc, nc, k), d) for d in dilations] for k in kernels]
+        stages.append({"alpha": alpha(C), "up": (up_w, rng.standard_normal(nc, dtype=np.float32) * np.float32(0.1)), "blocks": blocks,
+                       "rate": rate})
+        flops += 2.0 * nc * 2 * 2 * nl + sum(2 * 2.0 * nc * nc * k * nl * len(dilations) for k in kernels)
+        C, L = nc, nl
+    post_alpha, post = alpha(C), conv_w(1, C, 3)
+    flops += 2.0 * C * 3 * L
+    latent = backend.alloc(32 * frames).write(rng.uniform(-1, 1, 32 * frames).astype(np.float32))
+    biggest = max((864 >> (i + 1)) * frames * int(np.prod(rates[:i + 1])) for i in range(5))
+    bufs = [backend.alloc(max(biggest, 864 * frames)) for _ in range(7)]
+    cur, up, out, act, res, br, work = bufs
+    audio = backend.alloc(L)
+
+    def decode():
+        nonlocal cur, up, out
+        C, L = 864, frames
+        backend.conv1d(latent.ptr, cur.ptr, 32, 864, L, 7, 1, *pre)
+        for st in stages:
+            nc, nl = C // 2, L * st["rate"]
+            backend.snake_dev(cur.ptr, st["alpha"], C, L, C // 2)
+            backend.conv_transpose_dev(cur.ptr, up.ptr, C, nc, L, nl, 2 * st["rate"], st["rate"], nc, *st["up"])
+            n = nc * nl
+            for index, (branch, k) in enumerate(zip(st["blocks"], kernels)):
+                backend.copy_dev(work.ptr, up.ptr, n)
+                for a1, c1, a2, c2, d in branch:
+                    backend.copy_dev(act.ptr, work.ptr, n)
+                    backend.snake_dev(act.ptr, a1, nc, nl, nc // 2)
+                    backend.conv1d(act.ptr, res.ptr, nc, nc, nl, k, d, *c1)
+                    backend.snake_dev(res.ptr, a2, nc, nl, nc // 2)
+                    backend.conv1d(res.ptr, br.ptr, nc, nc, nl, k, 1, *c2)
+                    backend.residual_inplace(work.ptr, br.ptr, n)
+                if index == 0:
+                    backend.copy_dev(out.ptr, work.ptr, n)          # the reference adds to uploaded zeros (:2441,2492)
+                else:
+                    backend.residual_inplace(out.ptr, work.ptr, n)
+            backend.scale_dev(out.ptr, n, 1.0 / 3.0)
+            cur, out = out, cur
+            C, L = nc, nl
+        backend.snake_dev(cur.ptr, post_alpha, C, L, C // 2)
+        backend.conv1d(cur.ptr, audio.ptr, C, 1, L, 3, 1, *post)
+        backend.clip_dev(audio.ptr, L)
+
+    for _ in range(warmup):
+        decode()
+    backend.sync()
+    backend.timer_begin()
+    for _ in range(runs):
+        decode()
+    ms = backend.timer_end() / runs
+    samples = audio.read()
+    assert np.all(np.isfinite(samples)) and np.abs(samples).max() <= 1.0, "codec output is not a clipped waveform"
+    for d in bufs + [latent, audio]:
+        d.free()
+    return {"frames": frames, "samples": int(L), "ms": ms, "flops": flops, "tflops": flops / (ms * 1e-3) / 1e12}
+
+
 STAGES = [("self-attention", "k_step_attention: LayerNorm + int8 act-quant + per-head Q/K/V rows + KV append + attention over the self cache"),
           ("self-out", "k_linear: fold of attention partials + act-quant + O matvec + residual"),
           ("cross-attention", "k_step_attention: LayerNorm + act-quant + per-head Q rows + attention over the cross cache"),
@@ -214,6 +292,7 @@ def main():
     ap.add_argument("--skip-b8", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
     ap.add_argument("--skip-local", action="store_true")
+    ap.add_argument("--skip-codec", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the library's plain read+write kernel over 256 MiB three times (a known-size reference for "
@@ -245,6 +324,7 @@ def main():
         b8["self_lengths"], b8["cross_lengths"] = self_len, cross_len
     prefill = None if args.skip_prefill else time_prefill(pkg, synth, backend)
     local = None if args.skip_local else [time_local(pkg, synth, backend, qtype, b) for b in (1, 8)]
+    codec = None if args.skip_codec else time_codec(pkg, backend)
     backend.close()
 
     result = {
@@ -287,6 +367,12 @@ def main():
                            "frames": [{"batch": r["batch"], "frame_us": round(r["frame_us"], 1), "position_us": round(r["position_us"], 2),
                                        "algorithmic_bytes_per_frame": r["bytes"], "gbps": round(r["gbps"], 1),
                                        "frac": round(r["gbps"] / PEAK_GBPS, 4)} for r in local]}
+    if codec is not None:
+        result["codec"] = {"workload": "NanoCodec decode operator sequence, %d raw frames -> %d samples, f32: causal conv1d (kernels 3/7/11, "
+                                       "dilations 1/3/5, 864..27 channels) on the f32 matrix cores, grouped transposed conv, half-snake"
+                                       % (codec["frames"], codec["samples"]),
+                           "ms": round(codec["ms"], 3), "flops": codec["flops"], "tflops": round(codec["tflops"], 2), "bound": "mfma",
+                           "peak_tflops": 157.3, "frac": round(codec["tflops"] / 157.3, 4)}
     if not args.no_cpu:
         cpu = cpu_baseline()
         allc = cpu.get("all", {})

@@ -49,7 +49,7 @@ typedef int (*mynah_backend_sgemm_fn)(void *, int trans_a, int trans_b, size_t m
  *         like mynah_qmat_linear_resolved (src/qmat.c:768-818); more rows use the f32 GEMM.
  * sgemm:  row-major C = alpha op(A) op(B) + beta C on HOST pointers (src/backend.h:15-25).
  * self_test: the matmul/sgemm KATs of gpu/cuda/backend_cuda.cu:514-529 and the resident-op KATs
- *         of gpu/metal/backend_metal_ops.m:1038-1107 (codec ops excluded). */
+ *         of gpu/metal/backend_metal_ops.m:1038-1107, codec operators included. */
 int mynah_backend_hip_open(void **state, mynah_backend_matmul_fn *matmul, mynah_backend_sgemm_fn *sgemm,
                            mynah_backend_close_fn *close, mynah_backend_self_test_fn *self_test,
                            char *error, size_t error_capacity);

@@ -747,7 +747,7 @@ namespace mynah {
 static bool near(float a, float b, float tol) { return fabsf(a - b) <= tol; }
 
 // The matmul/sgemm KATs of gpu/cuda/backend_cuda.cu:514-529 (same numbers as src/backend.c:290-310) and
-// the resident-op KATs of gpu/metal/backend_metal_ops.m:1038-1107 (codec ops excluded).
+// the resident-op KATs of gpu/metal/backend_metal_ops.m:1038-1107, codec operators included.
 // Arrays are static: the weight cache keys on the host address and never refreshes it.
 static int backend_self_test(void *opaque, char *error, size_t capacity) {
     static const float in[6] = {1, 2, 3, -1, 0.5f, 2};
@@ -834,6 +834,27 @@ static int backend_self_test(void *opaque, char *error, size_t capacity) {
             break;
         if (o[0] != -1.0f || o[1] != 0.0f) {
             if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP clip mismatch: %.8g %.8g (want -1 0)", o[0], o[1]);
+            break;
+        }
+        // codec operators (gpu/metal/backend_metal_ops.m:1026-1030,1085,1099-1106): snake with alpha 1 on the row the clip
+        // left (-1, 0), then the three-position causal conv with taps 1 2: 2 5 8
+        static const float alpha[2] = {1.0f, 1.0f};
+        static const float conv_input[3] = {1.0f, 2.0f, 3.0f};
+        static const float conv_weight[2] = {1.0f, 2.0f};
+        float c3[3];
+        if (mynah_hip_snake_dev(opaque, dtmp, alpha, 2, 1, 2, error, capacity) != 0 || mynah_hip_d2h(opaque, dtmp, o, 2, error, capacity) != 0)
+            break;
+        const float s1 = sinf(-1.0f);
+        if (!near(o[0], -1.0f + s1 * s1, 1e-5f) || !near(o[1], 0.0f, 1e-6f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP snake mismatch: %.8g %.8g", o[0], o[1]);
+            break;
+        }
+        if (mynah_hip_h2d(opaque, conv_input, dqkv, 3, error, capacity) != 0 ||
+            mynah_hip_conv1d(opaque, dqkv, dsk, 1, 1, 3, 2, 1, conv_weight, nullptr, error, capacity) != 0 ||
+            mynah_hip_d2h(opaque, dsk, c3, 3, error, capacity) != 0)
+            break;
+        if (!near(c3[0], 2.0f, 1e-5f) || !near(c3[1], 5.0f, 1e-5f) || !near(c3[2], 8.0f, 1e-5f)) {
+            if (error != nullptr && capacity > 0) snprintf(error, capacity, "HIP conv1d mismatch: %.8g %.8g %.8g (want 2 5 8)", c3[0], c3[1], c3[2]);
             break;
         }
         rc = 0;

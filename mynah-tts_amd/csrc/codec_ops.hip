@@ -36,12 +36,43 @@ struct ConvArgs {
     int in_ch, out_ch, length, kernel, dilation;
 };
 
+// The products of one staged block of eight input channels for a wavefront's 32 x 64 tile.  The two inner indices one
+// matrix instruction consumes are the same tap of two neighbouring channels (lanes 0-31: the even channel, lanes 32-63:
+// the odd one), so a lane walks its channel's taps with plain increments.  wrow: this lane's output row at its first
+// channel; irow: its first channel's staged row at its output position.  Operands of the next product are requested
+// before the current one is issued.
+template <int KF, int NT = 2>
+__device__ __forceinline__ void conv_products(const float *wrow, const float *irow, const int kernel_arg, const int dilation, const int win,
+                                              floatx16 &acc0, floatx16 &acc1) {
+    const int kernel = KF != 0 ? KF : kernel_arg;
+    float wv = wrow[0], x0 = irow[0], x1 = NT > 1 ? irow[32] : 0.0f;
+#pragma unroll
+    for (int pair = 0; pair < kConvChannels / 2; ++pair) {
+#pragma unroll
+        for (int k = 0; k < kernel; ++k) {
+            // the product after this one: the next tap, or the first tap of the next channel pair (past the last pair the
+            // addresses stay inside the staging area and the values are not used)
+            const bool wrap = k + 1 == kernel;
+            wrow += wrap ? kernel + 1 : 1;
+            irow += wrap ? 2 * win - (kernel - 1) * dilation : dilation;
+            const float nw = wrow[0], n0 = irow[0], n1 = NT > 1 ? irow[32] : 0.0f;
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv, x0, acc0, 0, 0, 0);
+            if constexpr (NT > 1) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv, x1, acc1, 0, 0, 0);
+            wv = nw; x0 = n0; x1 = n1;
+        }
+    }
+}
+
 // Workgroup tile: (32 * WM) output channels x (64 * WN) positions; a wavefront owns 32 x 64 (two 32 x 32 accumulators).
-template <int WM, int WN>
-__global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a) {
+// KF: number of taps known at compile time (0 = from the arguments): the staging loops then have exactly as many slots as
+// the block has columns and the product loop is straight-line code.  The codec's 3, 7 and 11 taps get such builds.
+template <int WM, int WN, int KF>
+__global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     extern __shared__ __align__(16) float lds[];
-    const int kb = kConvChannels * a.kernel;   // inner elements per step (even)
+    ConvArgs a = a_arg;
+    if constexpr (KF != 0) a.kernel = KF;
+    const int kb = kConvChannels * a.kernel;   // inner elements per step
     const int a_stride = kb | 1;               // odd row stride: the 32 rows a wavefront reads land in 32 different banks
     const int halo = (a.kernel - 1) * a.dilation;
     const int win = TN + halo;                 // staged positions per input channel
@@ -54,7 +85,8 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a) {
 
     // Staging slots of a thread: weights -- row (tid / 16) + 16 * g, column (tid % 16) + 16 * c of the step's TM x kb
     // block; input rows -- channel ch, position tid + 256 * x of the window.  Fixed loops, no divisions.
-    constexpr int kRowGroups = TM / 16, kColGroups = kConvChannels * kConvMaxKernel / 16, kWinParts = (TN + kConvMaxHalo + 255) / 256;
+    constexpr int kRowGroups = TM / 16, kColGroups = (kConvChannels * (KF != 0 ? KF : kConvMaxKernel) + 15) / 16;
+    constexpr int kWinParts = (TN + kConvMaxHalo + 255) / 256;
     float stage_w[kRowGroups][kColGroups], stage_in[kConvChannels][kWinParts];
     const int srow = tid >> 4, scol = tid & 15;
     const auto fetch = [&](int i0) {   // global -> registers: the weight columns and input rows of channels [i0, i0 + 8)
@@ -64,7 +96,9 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a) {
 #pragma unroll
             for (int c = 0; c < kColGroups; ++c) {
                 const int cc = scol + 16 * c, ci = i0 * a.kernel + cc;
-                stage_w[g][c] = (cc < kb && m < a.out_ch && ci < inner) ? a.w[(size_t)m * inner + ci] : 0.0f;
+                const bool valid = cc < kb && m < a.out_ch && ci < inner;
+                const float v = a.w[valid ? (size_t)m * inner + ci : 0];   // always a legal address: no branch around the load
+                stage_w[g][c] = valid ? v : 0.0f;
             }
         }
 #pragma unroll
@@ -73,7 +107,9 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a) {
 #pragma unroll
             for (int x = 0; x < kWinParts; ++x) {
                 const int xx = tid + 256 * x, t = t0 - halo + xx;
-                stage_in[ch][x] = (xx < win && i < a.in_ch && t >= 0 && t < a.length) ? a.in[(size_t)i * a.length + t] : 0.0f;
+                const bool valid = xx < win && i < a.in_ch && t >= 0 && t < a.length;
+                const float v = a.in[valid ? (size_t)i * a.length + t : 0];
+                stage_in[ch][x] = valid ? v : 0.0f;
             }
         }
     };
@@ -103,21 +139,8 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a) {
         publish();
         __syncthreads();
         if (i0 + kConvChannels < a.in_ch) fetch(i0 + kConvChannels);   // in flight during the products below
-        // this lane's inner index runs half, half + 2, ...: (channel, tap) kept as counters instead of dividing
-        int ch = 0, k = half;
-        if (k >= a.kernel) { k -= a.kernel; ++ch; }
-        const float *wrow = s_w + (wm * 32 + col) * a_stride + half;
-        const float *irow = s_in + wn * 64 + col;
-#pragma unroll 4
-        for (int q = 0; q < kb; q += 2) {
-            const float wv = wrow[q];
-            const float *src = irow + ch * win + k * a.dilation;
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv, src[0], acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv, src[32], acc1, 0, 0, 0);
-            k += 2;
-            if (k >= a.kernel) { k -= a.kernel; ++ch; }   // kernel 1 wraps twice
-            if (k >= a.kernel) { k -= a.kernel; ++ch; }
-        }
+        conv_products<KF>(s_w + (wm * 32 + col) * a_stride + half * a.kernel, s_in + half * win + wn * 64 + col, a.kernel, a.dilation,
+                          win, acc0, acc1);
         __syncthreads();
     }
     // accumulator element r of a lane: row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
@@ -130,6 +153,99 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a) {
             if (t < a.length) a.out[(size_t)m * a.length + t] = acc0[r] + b;
             if (t + 32 < a.length) a.out[(size_t)m * a.length + t + 32] = acc1[r] + b;
         }
+    }
+}
+
+// The same product for short rows (few positions, many channels: the codec's first stages), where 64 x 128 tiles would
+// leave most of the chip idle: a workgroup owns a 32 x 64 tile and its four wavefronts split the input channels between
+// them (wavefront w takes channel blocks w, w + 4, ...), each staging its own blocks in its own part of LDS; the four
+// partial tiles are added in wavefront order at the end, so the result does not depend on timing.  NT: 32-position
+// halves per tile (2, or 1 for the very shortest rows: twice the workgroups).
+template <int KF, int NT>
+__global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
+    constexpr int TM = 32, TN = 32 * NT;
+    extern __shared__ __align__(16) float lds[];
+    ConvArgs a = a_arg;
+    if constexpr (KF != 0) a.kernel = KF;
+    const int kb = kConvChannels * a.kernel;
+    const int a_stride = kb | 1;
+    const int halo = (a.kernel - 1) * a.dilation;
+    const int win = TN + halo;
+    const int per_wave = TM * a_stride + kConvChannels * win;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float *s_w = lds + wave * per_wave;        // [TM][a_stride] of this wavefront
+    float *s_in = s_w + TM * a_stride;         // [kConvChannels][win]
+    const int m0 = blockIdx.y * TM, t0 = blockIdx.x * TN;
+    const int inner = a.in_ch * a.kernel;
+    // staging slots of a lane: weights -- row (lane / 2) , column (lane % 2) + 2 * c; input rows -- channel ch, position lane + 64 * x
+    constexpr int kCols = kConvChannels * (KF != 0 ? KF : kConvMaxKernel) / 2, kWinParts = (TN + kConvMaxHalo + 63) / 64;
+    const int srow = lane >> 1, scol = lane & 1;
+
+    floatx16 acc0, acc1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
+    const int half = lane >> 5, col = lane & 31;
+    const int blocks = (a.in_ch + kConvChannels - 1) / kConvChannels;
+    const int rounds = (blocks + 3) / 4;   // the same count for every wavefront (a block past the end stages zeros)
+    float stage_w[kCols], stage_in[kConvChannels][kWinParts];
+    const auto fetch = [&](int round) {   // global -> registers: this wavefront's channel block of the round
+        const int i0 = (4 * round + wave) * kConvChannels;
+        const int m = m0 + srow;
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) {
+            const int cc = scol + 2 * c, ci = i0 * a.kernel + cc;
+            const bool valid = cc < kb && m < a.out_ch && ci < inner;
+            const float v = a.w[valid ? (size_t)m * inner + ci : 0];
+            stage_w[c] = valid ? v : 0.0f;
+        }
+#pragma unroll
+        for (int ch = 0; ch < kConvChannels; ++ch) {
+            const int i = i0 + ch;
+#pragma unroll
+            for (int x = 0; x < kWinParts; ++x) {
+                const int xx = lane + 64 * x, t = t0 - halo + xx;
+                const bool valid = xx < win && i < a.in_ch && t >= 0 && t < a.length;
+                const float v = a.in[valid ? (size_t)i * a.length + t : 0];
+                stage_in[ch][x] = valid ? v : 0.0f;
+            }
+        }
+    };
+    fetch(0);
+    for (int round = 0; round < rounds; ++round) {
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) {
+            const int cc = scol + 2 * c;
+            if (cc < kb) s_w[srow * a_stride + cc] = stage_w[c];
+        }
+#pragma unroll
+        for (int ch = 0; ch < kConvChannels; ++ch)
+#pragma unroll
+            for (int x = 0; x < kWinParts; ++x) {
+                const int xx = lane + 64 * x;
+                if (xx < win) s_in[ch * win + xx] = stage_in[ch][x];
+            }
+        __syncthreads();
+        if (round + 1 < rounds) fetch(round + 1);   // in flight during the products below
+        conv_products<KF, NT>(s_w + col * a_stride + half * a.kernel, s_in + half * win + col, a.kernel, a.dilation, win, acc0, acc1);
+        __syncthreads();
+    }
+    // partial tiles through LDS: [wavefront][element r][lane], then ((p0 + p1) + p2) + p3 + bias
+    float *s_part = lds;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        s_part[(wave * 32 + r) * 64 + lane] = acc0[r];
+        s_part[(wave * 32 + 16 + r) * 64 + lane] = acc1[r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int e = tid + 256 * j;       // element r of lane l of the tile: e = r * 64 + l
+        const int r = e >> 6, l = e & 63;
+        const float sum = ((s_part[e] + s_part[2048 + e]) + s_part[4096 + e]) + s_part[6144 + e];
+        const int rr = r & 15;
+        const int m = m0 + 8 * (rr >> 2) + 4 * (l >> 5) + (rr & 3);
+        const int t = t0 + (l & 31) + (r >= 16 ? 32 : 0);
+        if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length) a.out[(size_t)m * a.length + t] = sum + (a.bias != nullptr ? a.bias[m] : 0.0f);
     }
 }
 
@@ -174,19 +290,62 @@ __global__ void __launch_bounds__(256) k_snake(float *data, const float *alpha, 
     }
 }
 
-template <int WM, int WN>
-int launch_conv(State *st, const ConvArgs &a, char *error, size_t capacity) {
+template <int WM, int WN, int KF>
+int launch_conv_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     const int kb = kConvChannels * a.kernel;
-    const size_t lds = ((size_t)TM * (kb | 1) + (size_t)kConvChannels * (TN + (a.kernel - 1) * a.dilation)) * sizeof(float);
+    // two more staged rows than are filled: the product loop requests the operands after its last product before it stops
+    const size_t lds = ((size_t)TM * (kb | 1) + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
     static bool raised = false;   // per instantiation
     if (lds > 48 * 1024 && !raised) {
-        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
         raised = true;
     }
     const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM));
-    hipLaunchKernelGGL((k_conv1d<WM, WN>), grid, dim3(256), lds, st->stream, a);
+    hipLaunchKernelGGL((k_conv1d<WM, WN, KF>), grid, dim3(256), lds, st->stream, a);
     return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
+}
+
+template <int WM, int WN>
+int launch_conv(State *st, const ConvArgs &a, char *error, size_t capacity) {
+    switch (a.kernel) {
+        case 3: return launch_conv_k<WM, WN, 3>(st, a, error, capacity);
+        case 7: return launch_conv_k<WM, WN, 7>(st, a, error, capacity);
+        case 11: return launch_conv_k<WM, WN, 11>(st, a, error, capacity);
+        default: return launch_conv_k<WM, WN, 0>(st, a, error, capacity);
+    }
+}
+
+template <int KF, int NT>
+int launch_conv_split_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
+    const int kb = kConvChannels * a.kernel;
+    const size_t per_wave = (size_t)32 * (kb | 1) + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
+    size_t lds = (4 * per_wave + 2 * (32 * NT + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);   // see launch_conv about the two extra rows
+    if (lds < 4 * 32 * 64 * sizeof(float)) lds = 4 * 32 * 64 * sizeof(float);   // the partial tiles
+    static bool raised = false;
+    if (!raised) {
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d_split<KF, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+        raised = true;
+    }
+    const dim3 grid((unsigned)((a.length + 32 * NT - 1) / (32 * NT)), (unsigned)((a.out_ch + 31) / 32));
+    hipLaunchKernelGGL((k_conv1d_split<KF, NT>), grid, dim3(256), lds, st->stream, a);
+    return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
+}
+
+template <int NT>
+int launch_conv_split_n(State *st, const ConvArgs &a, char *error, size_t capacity) {
+    switch (a.kernel) {
+        case 3: return launch_conv_split_k<3, NT>(st, a, error, capacity);
+        case 7: return launch_conv_split_k<7, NT>(st, a, error, capacity);
+        case 11: return launch_conv_split_k<11, NT>(st, a, error, capacity);
+        default: return launch_conv_split_k<0, NT>(st, a, error, capacity);
+    }
+}
+
+int launch_conv_split(State *st, const ConvArgs &a, char *error, size_t capacity) {
+    const long tiles = (long)((a.out_ch + 31) / 32) * ((a.length + 63) / 64);
+    if (tiles < st->cu_count) return launch_conv_split_n<1>(st, a, error, capacity);
+    return launch_conv_split_n<2>(st, a, error, capacity);
 }
 
 }  // namespace
@@ -213,7 +372,10 @@ extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_
     const float *dev_bias = nullptr;
     if (cached_vector(st, bias, (size_t)out_channels, &dev_bias, error, capacity) != 0) return -1;
     ConvArgs a{dev_input, dev_output, static_cast<const float *>(cw->data), dev_bias, in_channels, out_channels, length, kernel, dilation};
-    // few output channels: one row of wavefronts, wider in time
+    // few output channels: one row of wavefronts, wider in time; too few large tiles to fill the chip (and enough input
+    // channels to share out): small tiles with the channels split over the wavefronts
+    const long tiles = out_channels <= 32 ? (long)((length + 255) / 256) : (long)((out_channels + 63) / 64) * ((length + 127) / 128);
+    if (tiles < st->cu_count && in_channels >= 4 * kConvChannels) return launch_conv_split(st, a, error, capacity);
     if (out_channels <= 32) return launch_conv<1, 4>(st, a, error, capacity);
     return launch_conv<2, 2>(st, a, error, capacity);
 }
