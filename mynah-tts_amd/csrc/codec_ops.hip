@@ -66,14 +66,16 @@ __device__ __forceinline__ void conv_products(const float *wrow, const float *ir
 // Workgroup tile: (32 * WM) output channels x (64 * WN) positions; a wavefront owns 32 x 64 (two 32 x 32 accumulators).
 // KF: number of taps known at compile time (0 = from the arguments): the staging loops then have exactly as many slots as
 // the block has columns and the product loop is straight-line code.  The codec's 3, 7 and 11 taps get such builds.
-template <int WM, int WN, int KF>
+// VEC: the weight rows are whole 16-byte pieces (in_ch * kernel a multiple of 4): the weight block is staged four
+// elements per request and kept in LDS with packed rows.
+template <int WM, int WN, int KF, int VEC>
 __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     extern __shared__ __align__(16) float lds[];
     ConvArgs a = a_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;   // inner elements per step
-    const int a_stride = kb | 1;               // odd row stride: the 32 rows a wavefront reads land in 32 different banks
+    const int a_stride = VEC ? kb : (kb | 1);  // odd row stride: the 32 rows a wavefront reads land in 32 different banks
     const int halo = (a.kernel - 1) * a.dilation;
     const int win = TN + halo;                 // staged positions per input channel
     float *s_w = lds;                          // [TM][a_stride]
@@ -87,11 +89,26 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
     // block; input rows -- channel ch, position tid + 256 * x of the window.  Fixed loops, no divisions.
     constexpr int kRowGroups = TM / 16, kColGroups = (kConvChannels * (KF != 0 ? KF : kConvMaxKernel) + 15) / 16;
     constexpr int kWinParts = (TN + kConvMaxHalo + 255) / 256;
-    float stage_w[kRowGroups][kColGroups], stage_in[kConvChannels][kWinParts];
+    constexpr int kVecSlots = (TM * kConvChannels * (KF != 0 ? KF : kConvMaxKernel) / 4 + 255) / 256;
+    float stage_w[VEC ? 1 : kRowGroups][VEC ? 1 : kColGroups], stage_in[kConvChannels][kWinParts];
+    float4 stage_w4[VEC ? kVecSlots : 1];
     const int srow = tid >> 4, scol = tid & 15;
+    const int kb4 = kb / 4;
     const auto fetch = [&](int i0) {   // global -> registers: the weight columns and input rows of channels [i0, i0 + 8)
+        if constexpr (VEC != 0) {
+            int tid_now = tid;
+            __asm__ volatile("" : "+v"(tid_now));   // slot rows recomputed per step rather than held in registers
 #pragma unroll
-        for (int g = 0; g < kRowGroups; ++g) {
+            for (int c = 0; c < kVecSlots; ++c) {
+                const int e = tid_now + 256 * c, row = e / kb4, cc = 4 * (e - row * kb4);
+                const int m = m0 + row, ci = i0 * a.kernel + cc;
+                const bool valid = row < TM && m < a.out_ch && ci < inner;
+                const float4 v = *reinterpret_cast<const float4 *>(a.w + (valid ? (size_t)m * inner + ci : 0));
+                stage_w4[c] = valid ? v : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < (VEC ? 0 : kRowGroups); ++g) {
             const int m = m0 + srow + 16 * g;
 #pragma unroll
             for (int c = 0; c < kColGroups; ++c) {
@@ -114,8 +131,15 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
         }
     };
     const auto publish = [&]() {   // registers -> LDS
+        if constexpr (VEC != 0) {
 #pragma unroll
-        for (int g = 0; g < kRowGroups; ++g)
+            for (int c = 0; c < kVecSlots; ++c) {
+                const int e = tid + 256 * c;
+                if (e < TM * kb4) reinterpret_cast<float4 *>(s_w)[e] = stage_w4[c];
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < (VEC ? 0 : kRowGroups); ++g)
 #pragma unroll
             for (int c = 0; c < kColGroups; ++c) {
                 const int cc = scol + 16 * c;
@@ -168,7 +192,8 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
     ConvArgs a = a_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;
-    const int a_stride = kb | 1;
+    const int a_stride = kb;   // rows packed: a request of 64 consecutive block elements lands on 64 consecutive words (the row reads
+                               // of the products then share banks four ways, which costs a few cycles per 64-cycle product)
     const int halo = (a.kernel - 1) * a.dilation;
     const int win = TN + halo;
     const int per_wave = TM * a_stride + kConvChannels * win;
@@ -177,9 +202,11 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
     float *s_in = s_w + TM * a_stride;         // [kConvChannels][win]
     const int m0 = blockIdx.y * TM, t0 = blockIdx.x * TN;
     const int inner = a.in_ch * a.kernel;
-    // staging slots of a lane: weights -- row (lane / 2) , column (lane % 2) + 2 * c; input rows -- channel ch, position lane + 64 * x
-    constexpr int kCols = kConvChannels * (KF != 0 ? KF : kConvMaxKernel) / 2, kWinParts = (TN + kConvMaxHalo + 63) / 64;
-    const int srow = lane >> 1, scol = lane & 1;
+    // staging slots of a lane: weights -- the four elements 4 * (lane + 64 * c) .. + 3 of the 32 x kb block taken row by
+    // row (rows are whole 16-byte pieces: the launch requires in_ch * kernel to be a multiple of 4, and kb is 8 * kernel);
+    // input rows -- channel ch, position lane + 64 * x
+    constexpr int kCols = kConvChannels * (KF != 0 ? KF : kConvMaxKernel) / 8, kWinParts = (TN + kConvMaxHalo + 63) / 64;
+    const int kb4 = kb / 4;
 
     floatx16 acc0, acc1;
 #pragma unroll
@@ -187,16 +214,20 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
     const int half = lane >> 5, col = lane & 31;
     const int blocks = (a.in_ch + kConvChannels - 1) / kConvChannels;
     const int rounds = (blocks + 3) / 4;   // the same count for every wavefront (a block past the end stages zeros)
-    float stage_w[kCols], stage_in[kConvChannels][kWinParts];
+    float4 stage_w[kCols];
+    float stage_in[kConvChannels][kWinParts];
     const auto fetch = [&](int round) {   // global -> registers: this wavefront's channel block of the round
         const int i0 = (4 * round + wave) * kConvChannels;
-        const int m = m0 + srow;
+        int lane_now = lane;
+        __asm__ volatile("" : "+v"(lane_now));   // the slots' rows are recomputed every round (a few instructions each) instead of
+                                                  // being kept in forty registers across the products
 #pragma unroll
         for (int c = 0; c < kCols; ++c) {
-            const int cc = scol + 2 * c, ci = i0 * a.kernel + cc;
-            const bool valid = cc < kb && m < a.out_ch && ci < inner;
-            const float v = a.w[valid ? (size_t)m * inner + ci : 0];
-            stage_w[c] = valid ? v : 0.0f;
+            const int e = lane_now + 64 * c, row = e / kb4, cc = 4 * (e - row * kb4);   // kb is a constant in the builds that matter
+            const int m = m0 + row, ci = i0 * a.kernel + cc;
+            const bool valid = row < TM && m < a.out_ch && ci < inner;
+            const float4 v = *reinterpret_cast<const float4 *>(a.w + (valid ? m * inner + ci : 0));   // offsets fit 31 bits (checked at launch)
+            stage_w[c] = valid ? v : make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
         for (int ch = 0; ch < kConvChannels; ++ch) {
@@ -205,7 +236,7 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
             for (int x = 0; x < kWinParts; ++x) {
                 const int xx = lane + 64 * x, t = t0 - halo + xx;
                 const bool valid = xx < win && i < a.in_ch && t >= 0 && t < a.length;
-                const float v = a.in[valid ? (size_t)i * a.length + t : 0];
+                const float v = a.in[valid ? i * a.length + t : 0];
                 stage_in[ch][x] = valid ? v : 0.0f;
             }
         }
@@ -214,8 +245,8 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
     for (int round = 0; round < rounds; ++round) {
 #pragma unroll
         for (int c = 0; c < kCols; ++c) {
-            const int cc = scol + 2 * c;
-            if (cc < kb) s_w[srow * a_stride + cc] = stage_w[c];
+            const int e = lane + 64 * c;
+            if (e < TM * kb4) reinterpret_cast<float4 *>(s_w)[e] = stage_w[c];
         }
 #pragma unroll
         for (int ch = 0; ch < kConvChannels; ++ch)
@@ -290,20 +321,26 @@ __global__ void __launch_bounds__(256) k_snake(float *data, const float *alpha, 
     }
 }
 
-template <int WM, int WN, int KF>
-int launch_conv_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
+template <int WM, int WN, int KF, int VEC>
+int launch_conv_v(State *st, const ConvArgs &a, char *error, size_t capacity) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     const int kb = kConvChannels * a.kernel;
     // two more staged rows than are filled: the product loop requests the operands after its last product before it stops
     const size_t lds = ((size_t)TM * (kb | 1) + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
     static bool raised = false;   // per instantiation
     if (lds > 48 * 1024 && !raised) {
-        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF, VEC>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
         raised = true;
     }
     const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM));
-    hipLaunchKernelGGL((k_conv1d<WM, WN, KF>), grid, dim3(256), lds, st->stream, a);
+    hipLaunchKernelGGL((k_conv1d<WM, WN, KF, VEC>), grid, dim3(256), lds, st->stream, a);
     return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
+}
+
+template <int WM, int WN, int KF>
+int launch_conv_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
+    if (((size_t)a.in_ch * a.kernel) % 4 == 0) return launch_conv_v<WM, WN, KF, 1>(st, a, error, capacity);
+    return launch_conv_v<WM, WN, KF, 0>(st, a, error, capacity);
 }
 
 template <int WM, int WN>
@@ -319,7 +356,7 @@ int launch_conv(State *st, const ConvArgs &a, char *error, size_t capacity) {
 template <int KF, int NT>
 int launch_conv_split_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
     const int kb = kConvChannels * a.kernel;
-    const size_t per_wave = (size_t)32 * (kb | 1) + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
+    const size_t per_wave = (size_t)32 * kb + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
     size_t lds = (4 * per_wave + 2 * (32 * NT + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);   // see launch_conv about the two extra rows
     if (lds < 4 * 32 * 64 * sizeof(float)) lds = 4 * 32 * 64 * sizeof(float);   // the partial tiles
     static bool raised = false;
@@ -375,7 +412,9 @@ extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_
     // few output channels: one row of wavefronts, wider in time; too few large tiles to fill the chip (and enough input
     // channels to share out): small tiles with the channels split over the wavefronts
     const long tiles = out_channels <= 32 ? (long)((length + 255) / 256) : (long)((out_channels + 63) / 64) * ((length + 127) / 128);
-    if (tiles < st->cu_count && in_channels >= 4 * kConvChannels) return launch_conv_split(st, a, error, capacity);
+    if (tiles < st->cu_count && in_channels >= 4 * kConvChannels && ((size_t)in_channels * kernel) % 4 == 0 &&
+        (size_t)out_channels * in_channels * kernel < (size_t)INT_MAX && (size_t)in_channels * length < (size_t)INT_MAX)
+        return launch_conv_split(st, a, error, capacity);
     if (out_channels <= 32) return launch_conv<1, 4>(st, a, error, capacity);
     return launch_conv<2, 2>(st, a, error, capacity);
 }
