@@ -33,7 +33,8 @@ def test_known_answer(backend):
 # (in, out, length, kernel, dilation): the codec's pre-conv, its residual convs at three stages (kernels 3/7/11, dilations
 # 1/3/5), the post-conv, and shapes that end inside a tile or are shorter than a tap's reach
 SHAPES = [(32, 864, 75, 7, 1), (432, 432, 600, 3, 1), (216, 216, 700, 7, 3), (108, 108, 1000, 11, 5), (54, 54, 3000, 11, 1),
-          (27, 27, 5000, 7, 5), (27, 1, 9000, 3, 1), (5, 70, 33, 1, 1), (9, 33, 20, 11, 5), (8, 64, 128, 2, 1)]
+          (27, 27, 5000, 7, 5), (27, 1, 9000, 3, 1), (5, 70, 33, 1, 1), (9, 33, 20, 11, 5), (8, 64, 128, 2, 1),
+          (40, 48, 300, 16, 8), (64, 40, 257, 5, 2), (33, 65, 129, 4, 1), (128, 96, 64, 1, 1)]   # generic tap counts, the largest reach, odd edges
 
 
 @pytest.mark.parametrize("shape", SHAPES)

@@ -163,6 +163,32 @@ def test_frame_model_shape_batch8(pkg, backend, orc, synth, nerr, qtype_name):
     backend.set_quant(0)
 
 
+def test_frame_batch16_two_tiles(pkg, backend, orc, synth, nerr):
+    """Sixteen items (two passes of eight through every matvec, the many-stream attention layout), alternating greedy and
+    sampling, f32: tokens and generator states equal to the oracle's frame."""
+    _announce("local frame batch 16 f32")
+    S, V, codebook, eos, cbc = 16, 512, 480, 481, 8
+    cfg, w, proj, bias, tables, rng = _setup(synth, 1, S, V, seed=71)
+    backend.set_quant(0)
+    loc = pkg.Local(backend, cfg, w, proj, bias, tables, codebook, eos, cbc)
+    B = 16
+    base = [dict(ITEMS[i % len(ITEMS)], rng_state=ITEMS[i % len(ITEMS)]["rng_state"] + 31 * i) for i in range(B)]
+    rows = [rng.standard_normal(cfg["width"]).astype(np.float32) for _ in range(B)]
+    drows = [backend.alloc(cfg["width"]).write(r) for r in rows]
+    dlogits = backend.alloc(B * S * V)
+    for attempt in range(2):     # eager frame, then the captured one
+        got = loc.frame([dict(it, row=d.ptr) for it, d in zip(base, drows)], dlogits.ptr)
+        logits = dlogits.read().reshape(B, S, V)
+        _replay_choices(orc, logits, base, got, codebook, eos, cbc)
+    oframe = orc.LocalFrame(orc.Decoder(cfg, w, 0), [orc.PackedWeight(p, 0) for p in proj], bias, tables, codebook, eos, cbc)
+    want = oframe.frame(rows, base, want_logits=True)
+    _compare_with_oracle_frame(nerr, got, logits, want, base, TOL["f32"])
+    assert np.array_equal(got["values"], want["values"]) and got["rng_state"] == want["rng_state"]
+    loc.destroy()
+    for d in drows + [dlogits]:
+        d.free()
+
+
 def test_frame_error_paths(pkg, backend, synth):
     _announce("local frame error paths")
     S, V = 4, 512
