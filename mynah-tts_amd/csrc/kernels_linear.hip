@@ -54,12 +54,14 @@ enum { SPEC_ANY = 0, SPEC_RESIDUAL = 1, SPEC_UP = 2 };
 // streams each -- staging every stream's activations is what such a launch spends most of its time on, every workgroup
 // has to do all of it, and a quarter of it per thread takes a quarter of the time.  The first team then does the
 // matvec as the only team of a small-batch workgroup would; the others are done once the activations are staged.
-template <int BT>
-constexpr int kLinearTeams = BT > kConsumerFoldMaxBatch ? 4 : 1;
+// Only for int8 / int4 weights, where staging includes the activation quantisation: for f16 / f32 weights it is a
+// LayerNorm or a copy, and the 128 registers a thread of a 1024-thread workgroup may use do not hold the wider products.
+template <int BT, int QT>
+constexpr int kLinearTeams = (BT > kConsumerFoldMaxBatch && kQuantised<QT>) ? 4 : 1;
 
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
-__global__ void __launch_bounds__(kThreads * kLinearTeams<BT>) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
-    constexpr int kTeams = kLinearTeams<BT>;
+__global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
+    constexpr int kTeams = kLinearTeams<BT, QT>;
     constexpr int SB = BT / kTeams;   // streams staged by one team
     const Team team{(int)(threadIdx.x & (kThreads - 1)), (int)(threadIdx.x / kThreads) * SB};
     const bool worker = kTeams == 1 || threadIdx.x < kThreads;
@@ -291,7 +293,7 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT>), lds, st->stream, a, rows_per_wg, lg);
+    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, a, rows_per_wg, lg);
     return hip_check(hipGetLastError(), "linear launch", error, capacity);
 }
 
