@@ -13,6 +13,10 @@ namespace mynah {
 // ------------------------------------------------------------------------------------------ helpers
 int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity) {
     if (st->pinned_bytes >= bytes) return 0;
+    if (bytes > (SIZE_MAX >> 1)) {   // the doubling below would never reach it
+        set_error(error, capacity, "staging request too large");
+        return -1;
+    }
     if (st->pinned != nullptr) {
         MYNAH_TRY(hipStreamSynchronize(st->stream));
         (void)hipHostFree(st->pinned);
@@ -28,6 +32,10 @@ int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity) {
 
 static int ensure_scratch(State *st, size_t bytes, char *error, size_t capacity) {
     if (st->scratch_bytes >= bytes) return 0;
+    if (bytes > (SIZE_MAX >> 1)) {   // the doubling below would never reach it
+        set_error(error, capacity, "staging request too large");
+        return -1;
+    }
     if (st->scratch != nullptr) {
         MYNAH_TRY(hipStreamSynchronize(st->stream));
         (void)hipFree(st->scratch);
@@ -41,12 +49,30 @@ static int ensure_scratch(State *st, size_t bytes, char *error, size_t capacity)
     return 0;
 }
 
-// Host memory -> device, stream ordered.  Sources of at most the pinned staging size are staged so
-// the call can return before the copy runs; larger ones (weights at load time) copy synchronously.
+// Host memory -> device, ordered on the backend's stream.  The source is pageable memory of the caller: the runtime has
+// taken its contents when the call returns, so the caller may reuse it at once.
 static int copy_to_device(State *st, void *dst, const void *src, size_t bytes, char *error, size_t capacity) {
     if (bytes == 0) return 0;
     MYNAH_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, st->stream));
-    // pageable source: the runtime has consumed `src` when the call returns
+    return 0;
+}
+
+// n floats as a byte count, or false when that does not fit a size_t
+static bool float_bytes(size_t n, size_t *bytes) {
+    if (n > SIZE_MAX / sizeof(float)) return false;
+    *bytes = n * sizeof(float);
+    return true;
+}
+
+// One device block holding a copy of `bytes` host bytes; nothing stays allocated when it fails.
+static int device_copy_of(const void *host, size_t bytes, void **dev, char *error, size_t capacity) {
+    *dev = nullptr;
+    MYNAH_TRY(hipMalloc(dev, bytes));
+    if (hip_check(hipMemcpy(*dev, host, bytes, hipMemcpyHostToDevice), "weight upload", error, capacity) != 0) {
+        (void)hipFree(*dev);
+        *dev = nullptr;
+        return -1;
+    }
     return 0;
 }
 
@@ -97,25 +123,22 @@ int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qty
     cw.n = n;
     cw.k = k;
     const size_t count = n * k;
+    int rc = 0;
     if (qtype == MYNAH_HIP_F32) {
         cw.bytes = count * sizeof(float);
-        MYNAH_TRY(hipMalloc(&cw.data, cw.bytes));
-        MYNAH_TRY(hipMemcpy(cw.data, host, cw.bytes, hipMemcpyHostToDevice));
+        rc = device_copy_of(host, cw.bytes, &cw.data, error, capacity);
     } else if (qtype == MYNAH_HIP_F16) {
         std::vector<uint16_t> packed(count);
         for (size_t i = 0; i < count; ++i) packed[i] = f32_to_f16_rne(host[i]);
         cw.bytes = count * sizeof(uint16_t);
-        MYNAH_TRY(hipMalloc(&cw.data, cw.bytes));
-        MYNAH_TRY(hipMemcpy(cw.data, packed.data(), cw.bytes, hipMemcpyHostToDevice));
+        rc = device_copy_of(packed.data(), cw.bytes, &cw.data, error, capacity);
     } else if (qtype == MYNAH_HIP_INT8) {
         std::vector<int8_t> packed(count);
         std::vector<float> scales(n);
         quantize_weight_int8(host, n, k, packed.data(), scales.data(), st->arith);
         cw.bytes = count + n * sizeof(float);
-        MYNAH_TRY(hipMalloc(&cw.data, count));
-        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&cw.scales), n * sizeof(float)));
-        MYNAH_TRY(hipMemcpy(cw.data, packed.data(), count, hipMemcpyHostToDevice));
-        MYNAH_TRY(hipMemcpy(cw.scales, scales.data(), n * sizeof(float), hipMemcpyHostToDevice));
+        rc = device_copy_of(packed.data(), count, &cw.data, error, capacity);
+        if (rc == 0) rc = device_copy_of(scales.data(), n * sizeof(float), reinterpret_cast<void **>(&cw.scales), error, capacity);
     } else {
         const size_t groups = k / 32u;
         std::vector<uint8_t> packed(count / 2u);
@@ -125,10 +148,13 @@ int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qty
             return -1;
         }
         cw.bytes = count / 2u + n * groups * sizeof(float);
-        MYNAH_TRY(hipMalloc(&cw.data, count / 2u));
-        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&cw.scales), n * groups * sizeof(float)));
-        MYNAH_TRY(hipMemcpy(cw.data, packed.data(), count / 2u, hipMemcpyHostToDevice));
-        MYNAH_TRY(hipMemcpy(cw.scales, scales.data(), n * groups * sizeof(float), hipMemcpyHostToDevice));
+        rc = device_copy_of(packed.data(), count / 2u, &cw.data, error, capacity);
+        if (rc == 0)
+            rc = device_copy_of(scales.data(), n * groups * sizeof(float), reinterpret_cast<void **>(&cw.scales), error, capacity);
+    }
+    if (rc != 0) {
+        if (cw.data != nullptr) (void)hipFree(cw.data);   // the scales failed after the values had gone up
+        return -1;
     }
     st->weight_bytes += cw.bytes;
     auto ins = st->weights.emplace(key, cw);
@@ -137,11 +163,16 @@ int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qty
 }
 
 int cached_vector(State *st, const float *host, size_t n, const float **dev, char *error, size_t capacity) {
-    if (host == nullptr) {
+    if (host == nullptr || n == 0) {
         *dev = nullptr;
         return 0;
     }
-    const WeightKey key{host, n * sizeof(float), 0};
+    size_t bytes = 0;
+    if (!float_bytes(n, &bytes)) {
+        set_error(error, capacity, "invalid vector size");
+        return -1;
+    }
+    const WeightKey key{host, bytes, 0};
     std::lock_guard<std::mutex> lock(st->mu);
     auto it = st->weights.find(key);
     if (it != st->weights.end()) {
@@ -151,9 +182,8 @@ int cached_vector(State *st, const float *host, size_t n, const float **dev, cha
     CachedWeight cw;
     cw.n = 1;
     cw.k = n;
-    cw.bytes = n * sizeof(float);
-    MYNAH_TRY(hipMalloc(&cw.data, cw.bytes));
-    MYNAH_TRY(hipMemcpy(cw.data, host, cw.bytes, hipMemcpyHostToDevice));
+    cw.bytes = bytes;
+    if (device_copy_of(host, cw.bytes, &cw.data, error, capacity) != 0) return -1;
     st->weight_bytes += cw.bytes;
     st->weights.emplace(key, cw);
     *dev = static_cast<const float *>(cw.data);
@@ -232,7 +262,8 @@ static int hip_matmul(void *opaque, const float *input, float *output, size_t ro
                       const float *weight, const float *bias, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
     if (check_rows(input, output, rows, iw, ow, weight, error, capacity) != 0) return -1;
-    const size_t in_n = rows * iw, out_n = rows * ow;
+    MYNAH_NEED_STATE(st);
+    const size_t in_n = rows * iw, out_n = rows * ow;   // each factor is below 2^31
     if (ensure_scratch(st, (in_n + out_n) * sizeof(float), error, capacity) != 0) return -1;
     float *din = st->scratch, *dout = st->scratch + in_n;
     MYNAH_TRY(hipMemcpyAsync(din, input, in_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
@@ -247,6 +278,12 @@ static int hip_sgemm(void *opaque, int ta, int tb, size_t m, size_t n, size_t k,
     State *st = static_cast<State *>(opaque);
     if (a == nullptr || b == nullptr || c == nullptr || m == 0 || n == 0) {
         set_error(error, capacity, "invalid sgemm arguments");
+        return -1;
+    }
+    MYNAH_NEED_STATE(st);
+    const size_t limit = (size_t)1 << 31;   // keeps every product below exact in a size_t
+    if (m >= limit || n >= limit || k >= limit || lda >= limit || ldb >= limit || ldc >= limit) {
+        set_error(error, capacity, "sgemm dimensions too large");
         return -1;
     }
     const size_t a_n = (ta ? k : m) * lda, b_n = (tb ? n : k) * ldb, c_n = m * ldc;
@@ -274,6 +311,7 @@ static void hip_close(void *opaque) {
     if (st->flush != nullptr) (void)hipFree(st->flush);
     if (st->attn_partial != nullptr) (void)hipFree(st->attn_partial);
     if (st->attn_counters != nullptr) (void)hipFree(st->attn_counters);
+    if (st->argmax_result != nullptr) (void)hipFree(st->argmax_result);
     if (st->ptr_table != nullptr) (void)hipFree(st->ptr_table);
     if (st->ptr_table_host != nullptr) (void)hipHostFree(st->ptr_table_host);
     if (st->ev0 != nullptr) (void)hipEventDestroy(st->ev0);
@@ -410,33 +448,36 @@ extern "C" void mynah_hip_dev_free(void *opaque, float *dev_ptr) {
 
 extern "C" int mynah_hip_h2d(void *opaque, const float *host, float *dev_ptr, size_t n, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
-    if (host == nullptr || dev_ptr == nullptr) {
+    size_t bytes = 0;
+    if (st == nullptr || host == nullptr || dev_ptr == nullptr || !float_bytes(n, &bytes)) {
         set_error(error, capacity, "invalid h2d arguments");
         return -1;
     }
-    return copy_to_device(st, dev_ptr, host, n * sizeof(float), error, capacity);
+    return copy_to_device(st, dev_ptr, host, bytes, error, capacity);
 }
 
 extern "C" int mynah_hip_d2h(void *opaque, const float *dev_ptr, float *host, size_t n, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
-    if (host == nullptr || dev_ptr == nullptr) {
+    size_t bytes = 0;
+    if (st == nullptr || host == nullptr || dev_ptr == nullptr || !float_bytes(n, &bytes)) {
         set_error(error, capacity, "invalid d2h arguments");
         return -1;
     }
-    MYNAH_TRY(hipMemcpyAsync(host, dev_ptr, n * sizeof(float), hipMemcpyDeviceToHost, st->stream));
+    if (bytes != 0) MYNAH_TRY(hipMemcpyAsync(host, dev_ptr, bytes, hipMemcpyDeviceToHost, st->stream));
     MYNAH_TRY(hipStreamSynchronize(st->stream));
     return 0;
 }
 
 extern "C" int mynah_hip_upload(void *opaque, const float *host, size_t n, float **dev_ptr, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
-    if (host == nullptr || dev_ptr == nullptr || n == 0) {
+    size_t bytes = 0;
+    if (st == nullptr || host == nullptr || dev_ptr == nullptr || n == 0 || !float_bytes(n, &bytes)) {
         set_error(error, capacity, "invalid upload arguments");
         return -1;
     }
-    if (ensure_scratch(st, n * sizeof(float), error, capacity) != 0) return -1;
+    if (ensure_scratch(st, bytes, error, capacity) != 0) return -1;
     *dev_ptr = st->scratch;
-    return copy_to_device(st, st->scratch, host, n * sizeof(float), error, capacity);
+    return copy_to_device(st, st->scratch, host, bytes, error, capacity);
 }
 
 extern "C" int mynah_hip_download(void *opaque, const float *dev_ptr, float *host, size_t n, char *error, size_t capacity) {
@@ -445,6 +486,7 @@ extern "C" int mynah_hip_download(void *opaque, const float *dev_ptr, float *hos
 
 extern "C" int mynah_hip_sync(void *opaque, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
     return hip_check(hipStreamSynchronize(st->stream), "sync", error, capacity);
 }
 
@@ -511,6 +553,7 @@ extern "C" int mynah_hip_matvec_dev(void *opaque, const float *din, float *dout,
 extern "C" int mynah_hip_matmul_to_dev(void *opaque, const float *host_in, float *dout, size_t rows, size_t iw, size_t ow,
                                        const float *weight, const float *bias, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
     if (check_rows(host_in, dout, rows, iw, ow, weight, error, capacity) != 0) return -1;
     if (ensure_scratch(st, rows * iw * sizeof(float), error, capacity) != 0) return -1;
     if (copy_to_device(st, st->scratch, host_in, rows * iw * sizeof(float), error, capacity) != 0) return -1;
@@ -541,14 +584,14 @@ extern "C" int mynah_hip_clip_dev(void *opaque, float *d, size_t n, char *error,
 extern "C" int mynah_hip_argmax_dev(void *opaque, const float *dlogits, size_t vocab, size_t codebook_size, size_t eos_id,
                                     int allow_eos, unsigned *argmax, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
-    if (dlogits == nullptr || argmax == nullptr || vocab == 0 || codebook_size > vocab || eos_id > 0xffffffffu ||
+    if (st == nullptr || dlogits == nullptr || argmax == nullptr || vocab == 0 || codebook_size > vocab || eos_id > 0xffffffffu ||
         vocab > 0x7fffffffu) {   // src/backend.c:829-830
         set_error(error, capacity, "invalid argmax arguments");
         return -1;
     }
-    if (ensure_scratch(st, 256, error, capacity) != 0) return -1;
+    if (st->argmax_result == nullptr) MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->argmax_result), 256));
     if (ensure_pinned(st, 256, error, capacity) != 0) return -1;
-    unsigned *dres = reinterpret_cast<unsigned *>(st->scratch);
+    unsigned *dres = st->argmax_result;
     if (launch_argmax(st, dlogits, vocab, codebook_size, eos_id >= 0x7fffffffu ? 0x7ffffffeu : eos_id, allow_eos, dres, error, capacity) != 0)
         return -1;
     MYNAH_TRY(hipMemcpyAsync(st->pinned, dres, sizeof(unsigned), hipMemcpyDeviceToHost, st->stream));
@@ -577,6 +620,7 @@ extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, cons
 // =========================================================================================== section 2
 extern "C" int mynah_hip_set_quant(void *opaque, int qtype, int arith, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
     if (qtype < MYNAH_HIP_F32 || qtype > MYNAH_HIP_F16 || arith < 0 || arith > 1) {
         set_error(error, capacity, "unknown quantisation mode");
         return -1;
@@ -708,10 +752,15 @@ __global__ void __launch_bounds__(256) k_flush(uint4 *p, size_t n16) {
 
 extern "C" int mynah_hip_timer_begin(void *opaque, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
     return hip_check(hipEventRecord(st->ev0, st->stream), "event record", error, capacity);
 }
 extern "C" int mynah_hip_timer_end(void *opaque, float *ms, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
+    if (st == nullptr || ms == nullptr) {
+        set_error(error, capacity, "invalid timer arguments");
+        return -1;
+    }
     MYNAH_TRY(hipEventRecord(st->ev1, st->stream));
     MYNAH_TRY(hipEventSynchronize(st->ev1));
     MYNAH_TRY(hipEventElapsedTime(ms, st->ev0, st->ev1));
@@ -719,6 +768,7 @@ extern "C" int mynah_hip_timer_end(void *opaque, float *ms, char *error, size_t 
 }
 extern "C" int mynah_hip_flush_cache(void *opaque, size_t bytes, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
     if (bytes < (1u << 20)) bytes = 1u << 20;
     if (st->flush_bytes < bytes) {
         if (st->flush != nullptr) {
@@ -735,11 +785,14 @@ extern "C" int mynah_hip_flush_cache(void *opaque, size_t bytes, char *error, si
     return hip_check(hipGetLastError(), "flush launch", error, capacity);
 }
 extern "C" int mynah_hip_set_graph_mode(void *opaque, int enabled, char *error, size_t capacity) {
-    (void)error; (void)capacity;
-    static_cast<State *>(opaque)->graph_mode = enabled ? 1 : 0;
+    State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
+    st->graph_mode = enabled ? 1 : 0;
     return 0;
 }
-extern "C" size_t mynah_hip_cached_weight_bytes(void *opaque) { return static_cast<State *>(opaque)->weight_bytes; }
+extern "C" size_t mynah_hip_cached_weight_bytes(void *opaque) {
+    return opaque != nullptr ? static_cast<State *>(opaque)->weight_bytes : 0;
+}
 
 // =========================================================================================== self test
 namespace mynah {

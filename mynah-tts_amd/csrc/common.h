@@ -37,6 +37,7 @@ inline int hip_check(hipError_t r, const char *what, char *error, size_t capacit
     return -1;
 }
 #define MYNAH_TRY(expr) do { if (hip_check((expr), #expr, error, capacity) != 0) return -1; } while (0)
+#define MYNAH_NEED_STATE(st) do { if ((st) == nullptr) { set_error(error, capacity, "backend state is null"); return -1; } } while (0)
 
 // ---- device-resident copy of one host tensor, converted at first sight ----
 struct CachedWeight {
@@ -97,6 +98,8 @@ struct State {
     // small device block for batched pointer tables of the section-2 calls
     void *ptr_table = nullptr;
     void *ptr_table_host = nullptr;   // pinned
+    // result word of the argmax operator: its own allocation, so that it can never alias a caller's upload buffer
+    unsigned *argmax_result = nullptr;
 };
 
 // weight cache (backend_hip.hip)

@@ -231,7 +231,7 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
                                         size_t capacity) {
     State *st = static_cast<State *>(opaque);
     if (out != nullptr) *out = nullptr;
-    if (st == nullptr || desc == nullptr || out == nullptr || desc->layers == 0 || desc->width == 0 || desc->heads == 0 ||
+    if (st == nullptr || desc == nullptr || out == nullptr || desc->layers == 0 || desc->layers > 4096 || desc->width == 0 || desc->heads == 0 ||
         desc->heads * desc->head_width != desc->width || desc->ffn_width == 0 || desc->capacity == 0 ||
         desc->capacity > 0x7ffffff0u || desc->norm_self == nullptr || desc->norm_pos_ff == nullptr || desc->qkv_w == nullptr ||
         desc->o_self_w == nullptr || desc->ffn_up_w == nullptr || desc->ffn_down_w == nullptr) {

@@ -182,11 +182,19 @@ __global__ void __launch_bounds__(256) k_step_end(const StepSlots *slots, int wi
 
 inline unsigned blocks_for(size_t n) { return (unsigned)((n + 255) / 256); }
 
+// one workgroup per row: the row count has to fit a grid dimension
+inline int check_grid_rows(size_t rows, const char *what, char *error, size_t capacity) {
+    if (rows <= 0x7fffffffu) return 0;
+    if (error != nullptr && capacity > 0) snprintf(error, capacity, "%s: too many rows", what);
+    return -1;
+}
+
 }  // namespace
 
 int launch_layernorm(State *st, const float *in, float *out, const float *gain, const float *bias, size_t rows,
                      size_t width, char *error, size_t capacity) {
     if (rows == 0 || width == 0) return 0;
+    if (check_grid_rows(rows, "layernorm", error, capacity) != 0) return -1;
     hipLaunchKernelGGL(k_layernorm, dim3((unsigned)rows), dim3(256), 0, st->stream, in, out, gain, bias, (int)width);
     return hip_check(hipGetLastError(), "layernorm launch", error, capacity);
 }
@@ -217,12 +225,15 @@ int launch_clip(State *st, float *data, size_t n, char *error, size_t capacity) 
 }
 int launch_softmax(State *st, float *data, size_t rows, size_t cols, size_t valid, char *error, size_t capacity) {
     if (rows == 0 || cols == 0) return 0;
+    if (check_grid_rows(rows, "softmax", error, capacity) != 0) return -1;
+    if (valid > cols) valid = cols;   // src/backend.c:609; also keeps the narrowing below exact
     hipLaunchKernelGGL(k_softmax_masked, dim3((unsigned)rows), dim3(256), 0, st->stream, data, (int)cols, (int)valid);
     return hip_check(hipGetLastError(), "softmax launch", error, capacity);
 }
 int launch_softmax_heads(State *st, const float *logits, float *probs, size_t rows, size_t cols, char *error,
                          size_t capacity) {
     if (rows == 0 || cols == 0) return 0;
+    if (check_grid_rows(rows, "softmax", error, capacity) != 0) return -1;
     hipLaunchKernelGGL(k_softmax_heads, dim3((unsigned)rows), dim3(256), 0, st->stream, logits, probs, (int)cols);
     return hip_check(hipGetLastError(), "softmax launch", error, capacity);
 }
@@ -239,6 +250,7 @@ int launch_gather(State *st, const float *const *dev_tables, size_t table_count,
         set_error(error, capacity, "gather: between 1 and 32 tables");
         return -1;
     }
+    if (check_grid_rows(tokens, "gather", error, capacity) != 0) return -1;
     GatherTables t;
     for (size_t j = 0; j < 32; ++j) t.t[j] = j < table_count ? dev_tables[j] : nullptr;
     hipLaunchKernelGGL(k_gather, dim3((unsigned)tokens), dim3(256), 0, st->stream, t, (int)table_count, dev_ids, (int)width, scale,

@@ -130,6 +130,41 @@ def test_two_layers_ragged_batch8_and_bit_identity(pkg, backend, orc, synth, ner
     backend.set_quant(0)
 
 
+@pytest.mark.parametrize("qtype_name", ["f32", "int8"])
+def test_streams_without_memory(pkg, backend, orc, synth, nerr, qtype_name):
+    """Streams whose encoder memory is empty (no cross cache at all) beside streams that have one: their
+    cross-attention context is zero (src/graph.c:3237-3244).  Batch 4 takes the workgroup numbering over live units
+    and the stand-alone fold, the pairs take the latency layout with the fold inside the output projection; a
+    stream's bits are the same in both."""
+    _announce("streams without memory %s" % qtype_name)
+    lengths = [3, 0, 128, 40]
+    mems = [0, 5, 0, 130]
+    cfg = synth.decoder_config(layers=2, capacity=136)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=2)
+    backend.set_quant(QT[qtype_name])
+    h = Harness(pkg, backend, cfg, weights, streams)
+    want, ks, vs = _oracle_step(orc, cfg, weights, streams, QT[qtype_name])
+    first = h.step()
+    for b in range(4):
+        assert np.isfinite(first[b]).all(), "stream %d" % b
+        assert nerr(first[b], want[b]) < TOL[qtype_name], "stream %d" % b
+    for replay in range(2):   # second call of this batch size is captured, third replays the graph
+        for b in range(4):
+            h.reset_cache(b)
+        again = h.step()
+        for b in range(4):
+            assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32)), "replay %d stream %d" % (replay, b)
+    for pair in ((0, 1), (2, 3), (0, 2)):
+        for b in pair:
+            h.reset_cache(b)
+        got = h.step(list(pair))
+        for out, b in zip(got, pair):
+            assert np.array_equal(out.view(np.uint32), first[b].view(np.uint32)), "stream %d in pair %s" % (b, pair)
+    h.close()
+    backend.set_quant(0)
+
+
 def test_twelve_layers_int8_multi_step(pkg, backend, orc, synth, nerr):
     """The benchmark stack (12 layers, 12x64 cross heads, int8) at reduced cache length, two consecutive steps
     so that the second step attends over the row the first one appended."""

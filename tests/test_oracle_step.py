@@ -62,6 +62,20 @@ def test_step_matches_reference_ragged_batch(orc, ref_strict, synth, nerr, qtype
         assert nerr(want[b], got[b]) < tol, "stream %d" % b
 
 
+@pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4"])
+def test_step_matches_reference_empty_memory(orc, ref_strict, synth, nerr, qtype_name):
+    """Streams without any encoder memory beside streams that have one: the cross-attention context of the former is
+    all zeros (src/graph.c:3237-3244: no row is ever added to the cleared output), so that sublayer leaves x as it was."""
+    qtype = {"f32": orc.F32, "int8": orc.INT8, "int4": orc.INT4}[qtype_name]
+    lengths = [3, 0, 12, 9]
+    mems = [0, 5, 0, 13]
+    cfg, want, got, _, _ = _run_both(orc, synth, qtype, 2, lengths, mems, True)
+    tol = 1e-5 if qtype == orc.F32 else 5e-3   # as in the ragged batch above
+    for b in range(len(lengths)):
+        assert np.isfinite(want[b]).all() and np.isfinite(got[b]).all()
+        assert nerr(want[b], got[b]) < tol, "stream %d" % b
+
+
 def test_reference_batched_equals_solo_bitwise(orc, ref, synth):
     """The contract the GPU path inherits (src/graph.h:33-38): a stream inside a batch of 8 is bit-identical
     to the same stream run alone -- shown here on the compiled reference itself."""
