@@ -441,6 +441,10 @@ extern "C" int mynah_hip_conv_transpose_dev(void *state, const float *dev_input,
     ConvTransposeArgs a{dev_input, dev_output, static_cast<const float *>(cw->data), dev_bias, in_channels, out_channels, length,
                         output_length, kernel, stride, groups};
     const size_t count = (size_t)out_channels * output_length;
+    if (count > (size_t)INT_MAX * 256u) {   // one thread per output value, 256 to a workgroup
+        set_error(error, capacity, "conv_transpose: output too large");
+        return -1;
+    }
     hipLaunchKernelGGL(k_conv_transpose, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st->stream, a);
     return hip_check(hipGetLastError(), "conv_transpose launch", error, capacity);
 }
@@ -455,6 +459,10 @@ extern "C" int mynah_hip_snake_dev(void *state, float *dev_data, const float *al
     }
     const size_t count = channels * length;
     if (count == 0) return 0;
+    if (count > (size_t)INT_MAX * 256u) {   // one thread per value, 256 to a workgroup
+        set_error(error, capacity, "snake: tensor too large");
+        return -1;
+    }
     const float *dev_alpha = nullptr;
     if (snake_channels != 0 && cached_vector(st, alpha, snake_channels, &dev_alpha, error, capacity) != 0) return -1;
     hipLaunchKernelGGL(k_snake, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st->stream, dev_data, dev_alpha, count, (int)length,

@@ -22,6 +22,8 @@
 // All products are "NT": C[m][n] = sum_k A[m][k] * W[n][k], both operands K-contiguous, which is how
 // the 32x32x16 MFMA wants them: lane l supplies row (l % 32) of A (or of W) and the eight consecutive
 // k values 8*(l / 32) .. +7 of the 16-deep step.
+#include <new>
+
 #include "device_common.h"
 
 using namespace mynah;
@@ -516,7 +518,11 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
         set_error(error, capacity, "encoder_create: unsupported shape (needs 64-wide heads, widths that are multiples of 64) or missing weights");
         return -1;
     }
-    auto *e = new mynah_hip_encoder();
+    auto *e = new (std::nothrow) mynah_hip_encoder();
+    if (e == nullptr) {
+        set_error(error, capacity, "out of memory creating the encoder");
+        return -1;
+    }
     e->layers = d->layers; e->width = d->width; e->heads = d->heads; e->head_width = d->head_width; e->ffn = d->ffn_width;
     e->vocab = d->vocab; e->max_positions = d->max_positions;
     e->tpad_max = (d->max_positions + kTile - 1) / kTile * kTile;

@@ -441,8 +441,12 @@ extern "C" int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc 
     auto fail = [&]() { mynah_hip_local_destroy(state, l); return -1; };
     if (mynah_hip_decoder_create(state, stack, &l->stack, error, capacity) != 0) return fail();
     l->layers = stack->layers; l->width = stack->width; l->capacity = stack->capacity; l->arith = st->arith;
-    l->streams = desc->streams; l->vocab = desc->vocab; l->codebook_size = desc->codebook_size; l->eos_id = desc->eos_id;
-    l->codebook_count = desc->codebook_count;
+    l->streams = desc->streams; l->vocab = desc->vocab;
+    // The kernels hold these as int.  Ids at or above the vocabulary do not exist, so a codebook larger than it allows the
+    // same ids as one of its size, and an end-of-sequence id outside it can match no id: keep that meaning after narrowing.
+    l->codebook_size = desc->codebook_size < desc->vocab ? desc->codebook_size : desc->vocab;
+    l->eos_id = desc->eos_id < desc->vocab ? desc->eos_id : (size_t)0x7fffffff;
+    l->codebook_count = desc->codebook_count < (size_t)0x7fffffff ? desc->codebook_count : (size_t)0x7fffffff;
     for (size_t s = 0; s < desc->streams; ++s) {
         if (desc->projection_w[s] == nullptr || desc->audio_table[s] == nullptr) {
             set_error(error, capacity, "local_create: missing projection weight or audio table");

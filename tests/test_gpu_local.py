@@ -189,6 +189,49 @@ def test_frame_batch16_two_tiles(pkg, backend, orc, synth, nerr):
         d.free()
 
 
+def test_frame_eos_outside_vocabulary(pkg, backend, orc, synth, nerr):
+    """An end-of-sequence id that is no id of the vocabulary (here one whose low 32 bits are 5, a real id) matches
+    nothing, as in the reference's full-width comparison (src/graph.c:1563-1574): only codebook ids are ever allowed,
+    allowed or forbidden makes no difference, and no end of sequence is reported.  Likewise a codebook size above the
+    vocabulary allows every id."""
+    _announce("local frame, eos id outside the vocabulary")
+    S, V, codebook, cbc = 8, 96, 80, 4
+    eos = 2 ** 32 + 5
+    cfg, w, proj, bias, tables, rng = _setup(synth, 2, S, V, seed=43)
+    for s in range(S):
+        bias[s][5] = 30.0       # id 5 is the greedy choice everywhere: a truncated eos id would report it as EOS
+        bias[s][90] = 40.0      # above the codebook: never allowed, since it is not the eos id either
+    backend.set_quant(QT["f32"])
+    loc = pkg.Local(backend, cfg, w, proj, bias, tables, codebook, eos, cbc)
+    B = len(ITEMS)
+    rows = [rng.standard_normal(cfg["width"]).astype(np.float32) for _ in range(B)]
+    drows = [backend.alloc(cfg["width"]).write(r) for r in rows]
+    dlogits = backend.alloc(B * S * V)
+    items = [dict(it, row=d.ptr) for it, d in zip(ITEMS, drows)]
+    got = loc.frame(items, dlogits.ptr)
+    logits = dlogits.read().reshape(B, S, V)
+    _replay_choices(orc, logits, ITEMS, got, codebook, eos, cbc)
+    assert not np.any(got["saw_eos"]) and np.all(got["values"] < codebook)
+    assert np.all(got["values"][0] == 5) and np.all(got["values"][4] == 5)      # the greedy items
+    stack = orc.Decoder(cfg, w, QT["f32"])
+    oframe = orc.LocalFrame(stack, [orc.PackedWeight(p, QT["f32"]) for p in proj], bias, tables, codebook, eos, cbc)
+    want = oframe.frame(rows, ITEMS, want_logits=True)
+    _compare_with_oracle_frame(nerr, got, logits, want, ITEMS, TOL["f32"])
+    assert np.array_equal(got["values"], want["values"]) and got["rng_state"] == want["rng_state"]
+    loc.destroy()
+
+    # a codebook size beyond the vocabulary: every id allowed, 90 wins everywhere for the greedy items
+    loc = pkg.Local(backend, cfg, w, proj, bias, tables, 2 ** 33, eos, cbc)
+    got = loc.frame(items, dlogits.ptr)
+    logits = dlogits.read().reshape(B, S, V)
+    _replay_choices(orc, logits, ITEMS, got, 2 ** 33, eos, cbc)
+    assert np.all(got["values"][0] == 90) and np.array_equal(got["stored"], got["values"]) and not np.any(got["saw_eos"])
+    loc.destroy()
+    for d in drows + [dlogits]:
+        d.free()
+    backend.set_quant(0)
+
+
 def test_frame_error_paths(pkg, backend, synth):
     _announce("local frame error paths")
     S, V = 4, 512
