@@ -12,7 +12,14 @@
  *     (gpu/cuda/backend_cuda.cu:133-143,193-219);
  *   - resident ops enqueue on one internal stream and return without synchronising; only
  *     mynah_hip_sync, mynah_hip_d2h, mynah_hip_download, mynah_hip_argmax_dev and the host-pointer
- *     matmul/sgemm block.
+ *     matmul/sgemm block;
+ *   - threads: a state, and every decoder, encoder and local frame created from it, serves one
+ *     thread at a time.  Its stream, upload buffer, staging memory and captured graphs are shared
+ *     by all its calls without locks, as in the reference's GPU backends, whose state belongs to
+ *     the one engine thread (gpu/cuda/backend_cuda.cu has no lock).  Separate states are
+ *     independent and may be used from separate threads.  The pointer returned by
+ *     mynah_hip_upload is the state's one upload buffer: the next upload, host-pointer
+ *     matmul/sgemm, matmul_to_dev or embed_gather reuses it.
  *
  * Section 1 mirrors, symbol for symbol, what src/backend.c declares for a GPU backend
  * (src/backend.c:72-135) so `#if defined(MYNAH_ENABLE_HIP)` blocks can bind it unchanged.
