@@ -165,6 +165,43 @@ def test_streams_without_memory(pkg, backend, orc, synth, nerr, qtype_name):
     backend.set_quant(0)
 
 
+@pytest.mark.parametrize("qtype_name", ["f32", "int8"])
+def test_last_row_of_the_cache(pkg, backend, orc, synth, nerr, qtype_name):
+    """length == capacity - 1 appends into the last row the cache has (one more is the capacity error of
+    src/graph.c:3152-3155); beside it a stream whose cache is exactly one full attention unit and one that is a row
+    short of it.  Outputs and appended rows against the oracle; every other cache row untouched."""
+    _announce("last cache row %s" % qtype_name)
+    capacity = 256
+    lengths = [capacity - 1, 128, 127]
+    mems = [9, 1, 128]
+    cfg = synth.decoder_config(layers=2, capacity=capacity)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=4)
+    backend.set_quant(QT[qtype_name])
+    h = Harness(pkg, backend, cfg, weights, streams)
+    want, ks, vs = _oracle_step(orc, cfg, weights, streams, QT[qtype_name])
+    got = h.step()
+    for b, L in enumerate(lengths):
+        assert nerr(got[b], want[b]) < TOL[qtype_name], "stream %d" % b
+        gk, gv = h.cache_rows(b)
+        for layer in range(2):
+            assert nerr(gk[layer, L], ks[b][layer, L]) < TOL[qtype_name]
+            assert nerr(gv[layer, L], vs[b][layer, L]) < TOL[qtype_name]
+        mask = np.ones(capacity, bool)
+        mask[L] = False
+        assert np.array_equal(gk[:, mask], streams[b]["k"][:, mask]) and np.array_equal(gv[:, mask], streams[b]["v"][:, mask])
+    # one row further is refused, and refusing it changes nothing
+    slots = h.slots()
+    slots[0]["length"] = capacity
+    with pytest.raises(pkg.BackendError, match="capacity exceeded"):
+        h.dec.step(slots)
+    for b in range(3):
+        gk, gv = h.cache_rows(b)
+        assert nerr(gk[0, lengths[b]], ks[b][0, lengths[b]]) < TOL[qtype_name]
+    h.close()
+    backend.set_quant(0)
+
+
 def test_twelve_layers_int8_multi_step(pkg, backend, orc, synth, nerr):
     """The benchmark stack (12 layers, 12x64 cross heads, int8) at reduced cache length, two consecutive steps
     so that the second step attends over the row the first one appended."""
