@@ -51,13 +51,16 @@ __device__ __forceinline__ float *stream_out(const LinearArgs &a, int b) {
 enum { SPEC_ANY = 0, SPEC_RESIDUAL = 1, SPEC_UP = 2 };
 
 // More than two streams: the workgroup has four teams of 256 threads (device_common.h) that stage a quarter of the
-// streams each -- staging every stream's activations is what such a launch spends most of its time on, every workgroup
+// streams each (two teams and half of them each in the case named below) -- staging every stream's activations is what such a launch spends most of its time on, every workgroup
 // has to do all of it, and a quarter of it per thread takes a quarter of the time.  The first team then does the
 // matvec as the only team of a small-batch workgroup would; the others are done once the activations are staged.
 // Only for int8 / int4 weights, where staging includes the activation quantisation: for f16 / f32 weights it is a
 // LayerNorm or a copy, and the 128 registers a thread of a 1024-thread workgroup may use do not hold the wider products.
+// int4 weights with eight streams take two teams of four streams: their products (group scales, eight streams of
+// accumulators) need about 240 registers, which a 512-thread workgroup may have and a 1024-thread one may not
+// (there: 430 to 570 bytes of scratch memory per thread).
 template <int BT, int QT>
-constexpr int kLinearTeams = (BT > kConsumerFoldMaxBatch && kQuantised<QT>) ? 4 : 1;
+constexpr int kLinearTeams = !(BT > kConsumerFoldMaxBatch && kQuantised<QT>) ? 1 : (QT == MYNAH_HIP_INT4 && BT == 8) ? 2 : 4;
 
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
 __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
