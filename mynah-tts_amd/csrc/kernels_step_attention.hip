@@ -135,8 +135,15 @@ template <int QT, int NVT, int PF, int WFIX, int SELF, int PACKED>
 __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a_arg, const int lg_arg, const int per_xcd_arg) {
     extern __shared__ __align__(16) unsigned char smem[];   // staged activations: width bytes (int8/int4) or floats
     __shared__ __align__(16) float s_proj[3 * kHw];         // q | k | v of this head
-    __shared__ __align__(16) float s_red[4 * kHw];          // per-wavefront weighted V sums
-    __shared__ float s_wave_ml[8];                          // per-wavefront max | sum
+    // CP: consecutive cache chunks of a stream per chunk workgroup; the code below is written for any CP.  With CP chunks one
+    // LayerNorm and one Q projection serve them all, their rows are requested at once, and each chunk still becomes a
+    // partial of its own, computed as a workgroup with that chunk alone would compute it, so results do not depend on CP.
+    // Measured with eight ragged streams, CP = 2 against 1: 42 % fewer workgroups and one round instead of two, yet the
+    // self-attention stage stays where it was (22.2 -> 21.8 us) and the cross-attention stage, whose memories are one or
+    // two chunks long, loses (9.4 -> 10.3 us): a workgroup's requests double as their number halves.
+    constexpr int CP = 1;
+    __shared__ __align__(16) float s_red[CP][4 * kHw];      // per-wavefront weighted V sums, per chunk
+    __shared__ float s_wave_ml[CP][8];                      // per-wavefront max | sum, per chunk
     __shared__ float s_sx[1];
     __shared__ float s_scratch[kPrologueScratch];
 
@@ -162,12 +169,12 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         b = hb % a.batch;
         head = hb / a.batch;
     } else {
-        // per head: [Q+K and V of every stream's new row (self only)] [the cache chunks that exist, stream by stream]
+        // per head: [Q+K and V of every stream's new row (self only)] [groups of CP cache chunks that exist, stream by stream]
         int chunk_items = 0;
         for (int s = 0; s < a.batch; ++s) {
             const int len = is_self ? slots->length[s] : slots->memory_length[s];
             const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-            chunk_items += is_self ? live : max(live, 1);
+            chunk_items += ((is_self ? live : max(live, 1)) + CP - 1) / CP;
         }
         const int row_items = is_self ? 2 * a.batch : 0;
         const int per_head = row_items + chunk_items;
@@ -188,7 +195,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
             for (int s = 0; s < a.batch; ++s) {
                 const int len = is_self ? slots->length[s] : slots->memory_length[s];
                 const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-                const int n = is_self ? live : max(live, 1);
+                const int n = ((is_self ? live : max(live, 1)) + CP - 1) / CP;
                 if (r >= before && r < before + n) { b = s; unit = r - before + (is_self ? 2 : 0); }
                 before += n;
             }
@@ -196,8 +203,8 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     }
     const bool role_qk = is_self && unit == 0;
     const bool role_v = is_self && unit == 1;
-    const int chunk = is_self ? unit - 2 : unit;   // cache chunk of this workgroup (chunk roles only)
-    const int pidx = is_self ? unit - 1 : unit;    // partial slot written by a chunk role (slot 0 = the new row)
+    const int chunk = CP * (is_self ? unit - 2 : unit);   // first cache chunk of this workgroup (chunk roles only)
+    const int pidx = is_self ? chunk + 1 : chunk;         // partial slot of that chunk (slot 0 of self-attention = the new row)
 
     const int chunks = a.width / kEpc;
 
@@ -245,11 +252,13 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const int g = tid / kPosLanes;
     const size_t col = (size_t)head * kHw + 4 * j;
     const int p0 = chunk * kStepUnitRows;
-    const int count = new_row ? 0 : max(0, min(kStepUnitRows, length - p0));
+    int count[CP];
+#pragma unroll
+    for (int cc = 0; cc < CP; ++cc) count[cc] = new_row ? 0 : max(0, min(kStepUnitRows, length - p0 - cc * kStepUnitRows));
     // A chunk role keeps its cache rows here.  The Q+K role has no cache rows and parks its second bank of weight
     // passes in the same registers (as raw bits), so that no role needs more registers than the largest one.
     static_assert(2 * kRowsPerThread >= 4 * PF, "the second weight bank must fit the cache-row registers");
-    float4 kv[kRowsPerThread], vv[kRowsPerThread];
+    float4 kv[CP][kRowsPerThread], vv[CP][kRowsPerThread];
     float sc2[4 * PF];   // int4 only: group scales of the second bank
     float ws2[PF];       // int8 only: row scales of the second bank
     if (role_qk) {
@@ -266,8 +275,8 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int idx = 4 * p + u;
-                if (idx < kRowsPerThread) kv[idx] = __builtin_bit_cast(float4, bank2[p].wv[u]);
-                else vv[idx - kRowsPerThread] = __builtin_bit_cast(float4, bank2[p].wv[u]);
+                if (idx < kRowsPerThread) kv[0][idx] = __builtin_bit_cast(float4, bank2[p].wv[u]);
+                else vv[0][idx - kRowsPerThread] = __builtin_bit_cast(float4, bank2[p].wv[u]);
                 sc2[idx] = bank2[p].sc[u];
             }
             ws2[p] = bank2[p].ws;
@@ -278,11 +287,15 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 #pragma unroll
         for (int i = 0; i < PF; ++i) ws2[i] = 1.0f;
 #pragma unroll
-        for (int i = 0; i < kRowsPerThread; ++i) {
-            const int pi = g + kPosPerPass * i;
-            const bool in_range = pi < count;
-            kv[i] = in_range ? *reinterpret_cast<const float4 *>(kc + (size_t)(p0 + pi) * stride + col) : make_float4(0.f, 0.f, 0.f, 0.f);
-            vv[i] = in_range ? *reinterpret_cast<const float4 *>(vc + (size_t)(p0 + pi) * stride + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int cc = 0; cc < CP; ++cc) {
+#pragma unroll
+            for (int i = 0; i < kRowsPerThread; ++i) {
+                const int pi = g + kPosPerPass * i;
+                const bool in_range = pi < count[cc];
+                const size_t at = (size_t)(p0 + cc * kStepUnitRows + pi) * stride + col;
+                kv[cc][i] = in_range ? *reinterpret_cast<const float4 *>(kc + at) : make_float4(0.f, 0.f, 0.f, 0.f);
+                vv[cc][i] = in_range ? *reinterpret_cast<const float4 *>(vc + at) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
         }
     }
 
@@ -303,7 +316,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int idx = 4 * p + u;
-                    bank2[p].wv[u] = __builtin_bit_cast(uint4, idx < kRowsPerThread ? kv[idx] : vv[idx - kRowsPerThread]);
+                    bank2[p].wv[u] = __builtin_bit_cast(uint4, idx < kRowsPerThread ? kv[0][idx] : vv[0][idx - kRowsPerThread]);
                     bank2[p].sc[u] = sc2[idx];
                 }
                 bank2[p].ws = ws2[p];
@@ -342,69 +355,78 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     // ---- cache chunk: this head's q, then the chunk's scores
     project_rows<QT, PF>(a, pre, PF, 0, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
     __syncthreads();
-    float *out_o = a.partial + (sh * a.max_units + pidx) * kHw;
-    if (count <= 0) {   // empty memory (cross only): the context stays zero (src/graph.c:3242)
+    float *out_o = a.partial + (sh * a.max_units + pidx) * kHw;   // the first chunk's partial; the second follows it
+    if (count[0] <= 0) {   // empty memory (cross only): the context stays zero (src/graph.c:3242)
         if (tid < kHw) out_o[tid] = 0.0f;
         if (tid == 0) { out_m[pidx] = 0.0f; out_l[pidx] = 1.0f; }
         return;
     }
 
-    // ---- scores, softmax statistics and weighted V rows, one wavefront at a time: a wavefront owns 32 rows of the unit
+    // ---- scores, softmax statistics and weighted V rows, one wavefront at a time: a wavefront owns 32 rows of a chunk
     // (its four 16-lane row groups x 8 passes) and nothing leaves it until its own (max, sum, out[64]) is complete;
-    // the four results meet once in LDS.
+    // the four results of a chunk meet once in LDS.
     const float4 qv = *reinterpret_cast<const float4 *>(s_proj + 4 * j);
-    float sc[kRowsPerThread];
-    float m = -3.0e38f;
-#pragma unroll
-    for (int i = 0; i < kRowsPerThread; ++i) {
-        const int pi = g + kPosPerPass * i;
-        float dot = 0.0f;
-        dot = __builtin_fmaf(qv.x, kv[i].x, dot);
-        dot = __builtin_fmaf(qv.y, kv[i].y, dot);
-        dot = __builtin_fmaf(qv.z, kv[i].z, dot);
-        dot = __builtin_fmaf(qv.w, kv[i].w, dot);
-        dot = row16_sum(dot);   // every lane of the row group holds the row's score
-        sc[i] = pi < count ? dot * a.scale : -3.0e38f;
-        m = fmaxf(m, sc[i]);
-    }
-    m = fmaxf(fmaxf(lane_f(m, 0), lane_f(m, 16)), fmaxf(lane_f(m, 32), lane_f(m, 48)));
-    float l = 0.0f;
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-    for (int i = 0; i < kRowsPerThread; ++i) {
-        // hardware exponential (2^(x log2 e), relative error about 1e-6 for the arguments met here) for the unit's 128 weights;
-        // the few exponentials that combine partial results stay exact
-        const float e = g + kPosPerPass * i < count ? __expf(sc[i] - m) : 0.0f;
-        l += e;
-        acc.x = __builtin_fmaf(e, vv[i].x, acc.x);
-        acc.y = __builtin_fmaf(e, vv[i].y, acc.y);
-        acc.z = __builtin_fmaf(e, vv[i].z, acc.z);
-        acc.w = __builtin_fmaf(e, vv[i].w, acc.w);
-    }
-    l = ((lane_f(l, 0) + lane_f(l, 16)) + lane_f(l, 32)) + lane_f(l, 48);
-    acc.x += __shfl_xor(acc.x, 16); acc.y += __shfl_xor(acc.y, 16); acc.z += __shfl_xor(acc.z, 16); acc.w += __shfl_xor(acc.w, 16);
-    acc.x += __shfl_xor(acc.x, 32); acc.y += __shfl_xor(acc.y, 32); acc.z += __shfl_xor(acc.z, 32); acc.w += __shfl_xor(acc.w, 32);
     const int lane = tid & 63, wave = tid >> 6;
-    if (lane < kPosLanes) *reinterpret_cast<float4 *>(s_red + wave * kHw + 4 * lane) = acc;
-    if (lane == 0) { s_wave_ml[wave] = m; s_wave_ml[4 + wave] = l; }
+#pragma unroll
+    for (int cc = 0; cc < CP; ++cc) {
+        if (count[cc] <= 0) continue;   // the stream's last group may hold one chunk only (same for the whole workgroup)
+        float sc[kRowsPerThread];
+        float m = -3.0e38f;
+#pragma unroll
+        for (int i = 0; i < kRowsPerThread; ++i) {
+            const int pi = g + kPosPerPass * i;
+            float dot = 0.0f;
+            dot = __builtin_fmaf(qv.x, kv[cc][i].x, dot);
+            dot = __builtin_fmaf(qv.y, kv[cc][i].y, dot);
+            dot = __builtin_fmaf(qv.z, kv[cc][i].z, dot);
+            dot = __builtin_fmaf(qv.w, kv[cc][i].w, dot);
+            dot = row16_sum(dot);   // every lane of the row group holds the row's score
+            sc[i] = pi < count[cc] ? dot * a.scale : -3.0e38f;
+            m = fmaxf(m, sc[i]);
+        }
+        m = fmaxf(fmaxf(lane_f(m, 0), lane_f(m, 16)), fmaxf(lane_f(m, 32), lane_f(m, 48)));
+        float l = 0.0f;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < kRowsPerThread; ++i) {
+            // hardware exponential (2^(x log2 e), relative error about 1e-6 for the arguments met here) for the chunk's 128 weights;
+            // the few exponentials that combine partial results stay exact
+            const float e = g + kPosPerPass * i < count[cc] ? __expf(sc[i] - m) : 0.0f;
+            l += e;
+            acc.x = __builtin_fmaf(e, vv[cc][i].x, acc.x);
+            acc.y = __builtin_fmaf(e, vv[cc][i].y, acc.y);
+            acc.z = __builtin_fmaf(e, vv[cc][i].z, acc.z);
+            acc.w = __builtin_fmaf(e, vv[cc][i].w, acc.w);
+        }
+        l = ((lane_f(l, 0) + lane_f(l, 16)) + lane_f(l, 32)) + lane_f(l, 48);
+        acc.x += __shfl_xor(acc.x, 16); acc.y += __shfl_xor(acc.y, 16); acc.z += __shfl_xor(acc.z, 16); acc.w += __shfl_xor(acc.w, 16);
+        acc.x += __shfl_xor(acc.x, 32); acc.y += __shfl_xor(acc.y, 32); acc.z += __shfl_xor(acc.z, 32); acc.w += __shfl_xor(acc.w, 32);
+        if (lane < kPosLanes) *reinterpret_cast<float4 *>(s_red[cc] + wave * kHw + 4 * lane) = acc;
+        if (lane == 0) { s_wave_ml[cc][wave] = m; s_wave_ml[cc][4 + wave] = l; }
+    }
     __syncthreads();
-    if (tid < kPosLanes) {   // merge the four wavefronts in order 0..3
-        const float m0 = s_wave_ml[0], m1 = s_wave_ml[1], m2 = s_wave_ml[2], m3 = s_wave_ml[3];
-        const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
-        const float w0 = expf(m0 - M), w1 = expf(m1 - M), w2 = expf(m2 - M), w3 = expf(m3 - M);   // a wavefront without rows: exp(-3e38 - M) = 0
-        float L = s_wave_ml[4] * w0;
-        L = __builtin_fmaf(s_wave_ml[5], w1, L);
-        L = __builtin_fmaf(s_wave_ml[6], w2, L);
-        L = __builtin_fmaf(s_wave_ml[7], w3, L);
-        const float4 o0 = *reinterpret_cast<const float4 *>(s_red + 4 * tid), o1 = *reinterpret_cast<const float4 *>(s_red + kHw + 4 * tid);
-        const float4 o2 = *reinterpret_cast<const float4 *>(s_red + 2 * kHw + 4 * tid), o3 = *reinterpret_cast<const float4 *>(s_red + 3 * kHw + 4 * tid);
-        float4 o;
-        o.x = __builtin_fmaf(o3.x, w3, __builtin_fmaf(o2.x, w2, __builtin_fmaf(o1.x, w1, o0.x * w0)));
-        o.y = __builtin_fmaf(o3.y, w3, __builtin_fmaf(o2.y, w2, __builtin_fmaf(o1.y, w1, o0.y * w0)));
-        o.z = __builtin_fmaf(o3.z, w3, __builtin_fmaf(o2.z, w2, __builtin_fmaf(o1.z, w1, o0.z * w0)));
-        o.w = __builtin_fmaf(o3.w, w3, __builtin_fmaf(o2.w, w2, __builtin_fmaf(o1.w, w1, o0.w * w0)));
-        *reinterpret_cast<float4 *>(out_o + 4 * tid) = o;
-        if (tid == 0) { out_m[pidx] = M; out_l[pidx] = L; }
+    if (tid < CP * kPosLanes) {   // merge a chunk's four wavefronts in order 0..3: lanes 0-15 the first chunk, 16-31 the second
+        const int cc = tid / kPosLanes, t = tid - cc * kPosLanes;
+        if (count[cc] > 0) {
+            const float *ml = s_wave_ml[cc];
+            const float *red = s_red[cc];
+            const float m0 = ml[0], m1 = ml[1], m2 = ml[2], m3 = ml[3];
+            const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+            const float w0 = expf(m0 - M), w1 = expf(m1 - M), w2 = expf(m2 - M), w3 = expf(m3 - M);   // a wavefront without rows: exp(-3e38 - M) = 0
+            float L = ml[4] * w0;
+            L = __builtin_fmaf(ml[5], w1, L);
+            L = __builtin_fmaf(ml[6], w2, L);
+            L = __builtin_fmaf(ml[7], w3, L);
+            const float4 o0 = *reinterpret_cast<const float4 *>(red + 4 * t), o1 = *reinterpret_cast<const float4 *>(red + kHw + 4 * t);
+            const float4 o2 = *reinterpret_cast<const float4 *>(red + 2 * kHw + 4 * t), o3 = *reinterpret_cast<const float4 *>(red + 3 * kHw + 4 * t);
+            float4 o;
+            o.x = __builtin_fmaf(o3.x, w3, __builtin_fmaf(o2.x, w2, __builtin_fmaf(o1.x, w1, o0.x * w0)));
+            o.y = __builtin_fmaf(o3.y, w3, __builtin_fmaf(o2.y, w2, __builtin_fmaf(o1.y, w1, o0.y * w0)));
+            o.z = __builtin_fmaf(o3.z, w3, __builtin_fmaf(o2.z, w2, __builtin_fmaf(o1.z, w1, o0.z * w0)));
+            o.w = __builtin_fmaf(o3.w, w3, __builtin_fmaf(o2.w, w2, __builtin_fmaf(o1.w, w1, o0.w * w0)));
+            *reinterpret_cast<float4 *>(out_o + (size_t)cc * kHw + 4 * t) = o;
+            if (t == 0) { out_m[pidx + cc] = M; out_l[pidx + cc] = L; }
+        }
     }
 }
 
