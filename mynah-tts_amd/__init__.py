@@ -222,6 +222,20 @@ class Backend:
     def sync(self):
         self._call("mynah_hip_sync")
 
+    def upload(self, array):
+        """mynah_backend_upload (src/backend.h:79-81): host floats into the backend's one upload buffer.  Returns the
+        device address, valid until the next upload or host-pointer matmul."""
+        a = np.ascontiguousarray(array, np.float32)
+        dev = _vp()
+        self._call("mynah_hip_upload", _np_ptr(a), _sz(a.size), C.byref(dev))
+        return dev.value
+
+    def download(self, dev_ptr, n):
+        """mynah_backend_download (src/backend.h:83-85): n floats from a device address, synchronous."""
+        out = np.empty(n, np.float32)
+        self._call("mynah_hip_download", _vp(dev_ptr), _np_ptr(out), _sz(n))
+        return out
+
     def set_quant(self, qtype, arith=ARITH_STRICT):
         self._call("mynah_hip_set_quant", C.c_int(qtype), C.c_int(arith))
 

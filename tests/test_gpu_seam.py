@@ -229,6 +229,30 @@ def test_layernorm_gelu_residual_softmax(backend, orc, nerr):
         d.free()
 
 
+def test_upload_operator_download(backend, orc):
+    """The engine's use of the upload buffer (src/graph.c:2263-2268): upload, one operator, download.  With argmax as
+    the operator the buffer must come back untouched -- its result has a word of its own -- and with snake as the
+    operator it must come back transformed."""
+    _announce("upload -> operator -> download")
+    rng = np.random.default_rng(701)
+    logits = rng.standard_normal(1024).astype(np.float32)
+    logits[0] = 3.25
+    logits[77] = 8.5
+    dev = backend.upload(logits)
+    assert backend.argmax_dev(dev, 1024, 1024, 0, False) == 77
+    assert backend.argmax_dev(dev, 1024, 50, 0, False) == orc.argmax_constrained(logits, 50, 0, False)[1]
+    assert np.array_equal(backend.download(dev, 1024).view(np.uint32), logits.view(np.uint32))
+    signal = rng.standard_normal(6 * 40).astype(np.float32)
+    alpha = (rng.random(3) + 0.5).astype(np.float32)
+    dev = backend.upload(signal)
+    backend.snake_dev(dev, alpha, 6, 40, 3)
+    got = backend.download(dev, signal.size)
+    want = orc.snake(signal.reshape(6, 40), alpha, 3).reshape(-1)
+    assert np.max(np.abs(got - want)) <= 1e-6 * max(1.0, float(np.max(np.abs(want))))
+    with pytest.raises(Exception):
+        backend.upload(np.zeros(0, np.float32))
+
+
 def test_argmax(backend, orc):
     _announce("argmax")
     rng = np.random.default_rng(700)
