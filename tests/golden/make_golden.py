@@ -24,6 +24,9 @@ import __graft_entry__ as entry  # noqa: E402
 STEP_LENGTHS = [5, 17, 0, 31, 9, 2, 25, 12]
 STEP_MEMS = [7, 19, 3, 32, 11, 1, 27, 16]
 STEP_LAYERS = 2
+# streams without any encoder memory beside streams that have one (src/graph.c:3237-3244: their context stays zero)
+NOMEM_LENGTHS = [3, 0, 12, 9]
+NOMEM_MEMS = [0, 5, 0, 13]
 
 
 def crc(*arrays):
@@ -47,6 +50,30 @@ def quant_inputs():
     rows.append(np.full(k, 1e-30, np.float32))
     rows.append((rng.standard_normal(k) * 0.02).astype(np.float32))
     return np.stack(rows)
+
+
+def step_case(orc, synth, out, prefix, lengths, mems, stream_seed, qnames):
+    """Outputs and appended cache rows of the compiled reference's decoder_step_batch on seeded synthetic streams."""
+    batch = len(lengths)
+    cfg = synth.decoder_config(layers=STEP_LAYERS, capacity=max(lengths) + 3, cross_heads=1)
+    weights = synth.decoder_weights(cfg, seed=0, ln_bias=False)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=stream_seed)
+    out[prefix + "_lengths"] = np.array(lengths, np.int64)
+    out[prefix + "_mems"] = np.array(mems, np.int64)
+    out[prefix + "_input_crc"] = crc(*[weights[k] for k in sorted(weights) if weights[k] is not None],
+                                     *[s[n] for s in streams for n in ("k", "v", "ck", "cv", "x")])
+    qtypes = {"f32": orc.F32, "int8": orc.INT8, "int4": orc.INT4}
+    for qname in qnames:
+        for tag, strict in (("stock", False), ("strict", True)):
+            dec = orc.RefDecoder(cfg, weights, qtypes[qname], batch, max(mems), strict=strict)
+            ks = [s["k"].copy() for s in streams]
+            vs = [s["v"].copy() for s in streams]
+            outs, _ = dec.step(ks, vs, [s["ck"] for s in streams], [s["cv"] for s in streams], lengths, mems,
+                               [s["x"] for s in streams])
+            dec.close()
+            out["%s_%s_%s_out" % (prefix, qname, tag)] = np.stack(outs)
+            out["%s_%s_%s_newk" % (prefix, qname, tag)] = np.stack([ks[b][:, lengths[b]] for b in range(batch)])
+            out["%s_%s_%s_newv" % (prefix, qname, tag)] = np.stack([vs[b][:, lengths[b]] for b in range(batch)])
 
 
 def main():
@@ -100,25 +127,10 @@ def main():
     assert lib.mynah_softmax_f32(np.ascontiguousarray(v[0]), sm, 64) == 0
     out.update(kern_x=v, kern_gain=gain, kern_beta=beta, kern_layernorm=ln, kern_gelu=g.reshape(v.shape), kern_softmax=sm)
 
-    # ---- the whole decode step (src/graph.c:3127-3284): 2 layers, ragged batch of 8 and stream 3 alone
-    cfg = synth.decoder_config(layers=STEP_LAYERS, capacity=max(STEP_LENGTHS) + 3, cross_heads=1)
-    weights = synth.decoder_weights(cfg, seed=0, ln_bias=False)
-    streams = synth.decoder_streams(cfg, STEP_LENGTHS, STEP_MEMS, seed=1)
-    out["step_lengths"] = np.array(STEP_LENGTHS, np.int64)
-    out["step_mems"] = np.array(STEP_MEMS, np.int64)
-    out["step_input_crc"] = crc(*[weights[k] for k in sorted(weights) if weights[k] is not None],
-                                *[s[n] for s in streams for n in ("k", "v", "ck", "cv", "x")])
-    for qname, qtype in (("f32", orc.F32), ("int8", orc.INT8), ("int4", orc.INT4)):
-        for tag, strict in (("stock", False), ("strict", True)):
-            dec = orc.RefDecoder(cfg, weights, qtype, 8, max(STEP_MEMS), strict=strict)
-            ks = [s["k"].copy() for s in streams]
-            vs = [s["v"].copy() for s in streams]
-            outs, _ = dec.step(ks, vs, [s["ck"] for s in streams], [s["cv"] for s in streams], STEP_LENGTHS, STEP_MEMS,
-                               [s["x"] for s in streams])
-            dec.close()
-            out["step_%s_%s_out" % (qname, tag)] = np.stack(outs)
-            out["step_%s_%s_newk" % (qname, tag)] = np.stack([ks[b][:, STEP_LENGTHS[b]] for b in range(8)])
-            out["step_%s_%s_newv" % (qname, tag)] = np.stack([vs[b][:, STEP_LENGTHS[b]] for b in range(8)])
+    # ---- the whole decode step (src/graph.c:3127-3284), 2 layers: a ragged batch of 8, and a batch of 4 in which two
+    # streams have no encoder memory
+    step_case(orc, synth, out, "step", STEP_LENGTHS, STEP_MEMS, 1, ("f32", "int8", "int4"))
+    step_case(orc, synth, out, "nomem", NOMEM_LENGTHS, NOMEM_MEMS, 2, ("f32", "int8", "int4"))
 
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **out)
