@@ -266,7 +266,10 @@ def roofline(r):
                            "kv_bytes": r["kv_bytes"], "gbps": round(r["gbps"], 2), "frac": round(r["gbps"] / PEAK_GBPS, 4)}}
 
 
-def cpu_baseline(steps=5, warmup=2):
+CPU_STEPS, CPU_WARMUP = 400, 20   # about 5 s per leg at 11.5 ms per step
+
+
+def cpu_baseline(steps=CPU_STEPS, warmup=CPU_WARMUP):
     """The reference's own CPU decode step (compiled from its sources into oracle/_ref), timed on this box's host
     cores in a child process: all online cores, then one thread."""
     out = {}
@@ -379,9 +382,9 @@ def main():
         result["cpu_baseline"] = {
             "value": round(allc.get("median_us", float("nan")), 1), "unit": "us per decode step (batch 1)",
             "cores": allc.get("threads"), "kind": allc.get("kind", "reference"),
-            "sample": "median of 5 steps after 2 warm-ups of the reference's own decoder_step_batch (stock flags, its pthread "
+            "sample": "median of %d steps after %d warm-ups of the reference's own decoder_step_batch (stock flags, its pthread "
                       "pool) on the same 12-layer int8 stack, self-KV 1024, cross-KV 256; that function has gain-only LayerNorm and "
-                      "one 768-wide cross head (same bytes and flops) and no output head",
+                      "one 768-wide cross head (same bytes and flops) and no output head" % (allc.get("steps", CPU_STEPS), allc.get("warmup", CPU_WARMUP)),
             "one_thread_us": round(cpu.get("one", {}).get("median_us", float("nan")), 1),
             "online_cores": allc.get("online_cores"),
             "gpu_speedup": round(allc.get("median_us", float("nan")) / b1["step_us"], 1) if "median_us" in allc else None,
