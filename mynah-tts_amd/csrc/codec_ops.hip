@@ -216,27 +216,46 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
     const int rounds = (blocks + 3) / 4;   // the same count for every wavefront (a block past the end stages zeros)
     float4 stage_w[kCols];
     float stage_in[kConvChannels][kWinParts];
+    // What a staging slot of this lane is does not change from round to round: kept as one 32-bit offset per slot (-1:
+    // outside the matrix or the row), so that a round's requests are an add, a load and a select each.  Working them out
+    // anew every round (a division, the range checks, 64-bit addresses) took 2.0 of a round's 5.0 us on the 432-channel
+    // stage: with one wavefront per SIMD the requests are bound by the instructions that form them, not by their round trip.
+    int w_slot[kCols];        // weights: offset of the slot's four floats from the block's first column
+    int in_slot[kWinParts];   // input: position in the row
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+        const int e = lane + 64 * c, row = e / kb4, cc = 4 * (e - row * kb4);   // kb is a constant in the builds that matter
+        const int m = m0 + row;
+        w_slot[c] = (row < TM && m < a.out_ch) ? m * inner + cc : -1;   // offsets fit 31 bits (checked at launch)
+    }
+#pragma unroll
+    for (int x = 0; x < kWinParts; ++x) {
+        const int xx = lane + 64 * x, t = t0 - halo + xx;
+        in_slot[x] = (xx < win && t >= 0 && t < a.length) ? t : -1;
+    }
     const auto fetch = [&](int round) {   // global -> registers: this wavefront's channel block of the round
         const int i0 = (4 * round + wave) * kConvChannels;
-        int lane_now = lane;
-        __asm__ volatile("" : "+v"(lane_now));   // the slots' rows are recomputed every round (a few instructions each) instead of
-                                                  // being kept in forty registers across the products
+        const int ci0 = i0 * a.kernel;
+        const bool whole_block = ci0 + kb <= inner;   // all but a ragged last block
 #pragma unroll
         for (int c = 0; c < kCols; ++c) {
-            const int e = lane_now + 64 * c, row = e / kb4, cc = 4 * (e - row * kb4);   // kb is a constant in the builds that matter
-            const int m = m0 + row, ci = i0 * a.kernel + cc;
-            const bool valid = row < TM && m < a.out_ch && ci < inner;
-            const float4 v = *reinterpret_cast<const float4 *>(a.w + (valid ? m * inner + ci : 0));   // offsets fit 31 bits (checked at launch)
+            bool valid = w_slot[c] >= 0;
+            if (!whole_block) {
+                const int e = lane + 64 * c;
+                valid = valid && ci0 + 4 * (e - (e / kb4) * kb4) < inner;
+            }
+            const float4 v = *reinterpret_cast<const float4 *>(a.w + (valid ? w_slot[c] + ci0 : 0));
             stage_w[c] = valid ? v : make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
         for (int ch = 0; ch < kConvChannels; ++ch) {
             const int i = i0 + ch;
+            const bool row_exists = i < a.in_ch;
+            const int row_at = i * a.length;
 #pragma unroll
             for (int x = 0; x < kWinParts; ++x) {
-                const int xx = lane + 64 * x, t = t0 - halo + xx;
-                const bool valid = xx < win && i < a.in_ch && t >= 0 && t < a.length;
-                const float v = a.in[valid ? i * a.length + t : 0];
+                const bool valid = row_exists && in_slot[x] >= 0;
+                const float v = a.in[valid ? row_at + in_slot[x] : 0];
                 stage_in[ch][x] = valid ? v : 0.0f;
             }
         }
