@@ -104,22 +104,32 @@ struct StagedTiles {
     }
 };
 
-// acc += A-tile fragment x W-tile fragment over one 64-deep K step (four 32x32x16 MFMAs).
-__device__ __forceinline__ void mma_tile(floatx16 &acc, const _Float16 *pa, const _Float16 *pw) {
+// The fragments of one 64-deep K step of a wavefront's 32 x 32 tile (four 32x32x16 MFMAs), read from LDS into registers
+// a step ahead of their use, so that the reads' round trip runs beside the previous step's matrix instructions.
+struct StepFragments {
+    half8 a[kTile / 16], w[kTile / 16];
+    __device__ __forceinline__ void read(const _Float16 *pa, const _Float16 *pw) {
 #pragma unroll
-    for (int j = 0; j < kTile / 16; ++j) {
-        const half8 fa = *reinterpret_cast<const half8 *>(pa + 16 * j);
-        const half8 fw = *reinterpret_cast<const half8 *>(pw + 16 * j);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fw, acc, 0, 0, 0);
+        for (int j = 0; j < kTile / 16; ++j) {
+            a[j] = *reinterpret_cast<const half8 *>(pa + 16 * j);
+            w[j] = *reinterpret_cast<const half8 *>(pw + 16 * j);
+        }
     }
-}
+    __device__ __forceinline__ void multiply(floatx16 &acc) const {
+#pragma unroll
+        for (int j = 0; j < kTile / 16; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j], w[j], acc, 0, 0, 0);
+    }
+};
 
 // D: K steps whose operand tiles are on their way from global memory at any time (even, so that a step's LDS buffer
-// is the parity of its register stage; 16 registers per step).  These launches put at most one workgroup on a CU, one
-// wavefront per SIMD, so nothing overlaps a step's own chain of LDS store, barrier, LDS reads and four dependent matrix
-// instructions, and that chain, not the global loads, is what the loop's time consists of: measured on the 256-token
-// prefill, D = 2 / 4 / 6 / 12 give 301 / 290 / 292 / 308 us.
-template <int EPI, int D>
+// is the parity of its register stage; 16 registers per step).
+// EXACT: the number of K steps is a multiple of D, and the loop body has no branch at all: every iteration stores,
+// requests, reads and multiplies, the requests past the last step repeating the last step's (never used).  This is what
+// makes the depth real.  Loads return in order and a wait names how many may still be out, so when a request is issued
+// under a condition the compiler must assume it was not, and the wait before storing the oldest block then drains every
+// younger one as well: with `if (kt + D < nk)` around the requests the pipeline was one step deep whatever D said.
+// Without EXACT (an odd number of steps) the guarded form is used, with that cost.
+template <int EPI, int D, bool EXACT>
 __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
     static_assert(D >= 2 && D % 2 == 0, "stage parity must equal step parity");
     __shared__ __align__(16) _Float16 s_a[2][kTile * kLdsStride];
@@ -140,26 +150,46 @@ __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
     const int kbase = (int)blockIdx.z * nk * (kTile / 8);   // in 16-byte chunks
     ga0 += kbase; ga1 += kbase; gw0 += kbase; gw1 += kbase;
 
-    // Global -> register -> LDS pipeline.  Step kt waits in register stage kt % D, is stored to LDS buffer kt % 2 and
-    // multiplied after one barrier; the same stage then requests step kt + D.  A buffer is overwritten two steps after
-    // it was read: every wavefront has passed the barrier in between, which it reaches only with those reads complete.
+    // Global -> register -> LDS -> register pipeline.  Step kt waits in register stage kt % D, is stored to LDS buffer
+    // kt % 2 one iteration before its products, and after that iteration's barrier its fragments are read into registers
+    // while the matrix instructions of step kt - 1 run from the other fragment set; the same stage then requests step
+    // kt + D.  A buffer is overwritten two steps after it was read: every wavefront has passed a barrier in between, which
+    // it reaches only with its LDS reads complete.  The products are issued in ascending K order.
     StagedTiles st[D];
+    const int last = nk - 1;
+    const auto chunk_of = [&](int step) { return (step < last ? step : last) * (kTile / 8); };   // past the end: the last step again
 #pragma unroll
     for (int d = 0; d < D; ++d)
-        if (d < nk) st[d].load(ga0, ga1, gw0, gw1, d * (kTile / 8));
+        if (EXACT || d < nk) st[d].load(ga0, ga1, gw0, gw1, chunk_of(d));
 
     floatx16 acc = {0};
     const int frag = (lane & 31) * kLdsStride + 8 * (lane >> 5);
     const int fa_off = wm * 32 * kLdsStride + frag, fw_off = wn * 32 * kLdsStride + frag;
+    StepFragments fr[2];   // fragments of step kt in fr[kt % 2]
+    st[0].store(&s_a[0][0], &s_w[0][0], soff0, soff1);
+    if (EXACT || D < nk) st[0].load(ga0, ga1, gw0, gw1, chunk_of(D));
+    __syncthreads();
+    fr[0].read(&s_a[0][fa_off], &s_w[0][fw_off]);
+    // iteration kt: stage step kt + 1, barrier, read its fragments, multiply step kt
     for (int base = 0; base < nk; base += D) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const int kt = base + d;
-            if (kt < nk) {   // the same for every thread of the grid
-                st[d].store(&s_a[d & 1][0], &s_w[d & 1][0], soff0, soff1);
-                if (kt + D < nk) st[d].load(ga0, ga1, gw0, gw1, (kt + D) * (kTile / 8));
+            const int dn = (d + 1) % D;   // register stage of step kt + 1 (a constant after unrolling)
+            if constexpr (EXACT) {
+                st[dn].store(&s_a[(d + 1) & 1][0], &s_w[(d + 1) & 1][0], soff0, soff1);
+                st[dn].load(ga0, ga1, gw0, gw1, chunk_of(kt + 1 + D));
                 __syncthreads();
-                mma_tile(acc, &s_a[d & 1][fa_off], &s_w[d & 1][fw_off]);
+                fr[(d + 1) & 1].read(&s_a[(d + 1) & 1][fa_off], &s_w[(d + 1) & 1][fw_off]);
+                fr[d & 1].multiply(acc);
+            } else if (kt < nk) {   // the same for every thread of the grid
+                if (kt + 1 < nk) {
+                    st[dn].store(&s_a[(d + 1) & 1][0], &s_w[(d + 1) & 1][0], soff0, soff1);
+                    if (kt + 1 + D < nk) st[dn].load(ga0, ga1, gw0, gw1, chunk_of(kt + 1 + D));
+                }
+                __syncthreads();
+                if (kt + 1 < nk) fr[(d + 1) & 1].read(&s_a[(d + 1) & 1][fa_off], &s_w[(d + 1) & 1][fw_off]);
+                fr[d & 1].multiply(acc);
             }
         }
     }
@@ -308,6 +338,9 @@ void launch_rows(State *st, int width, dim3 grid, float *x, const float *part, i
 // (f16, written over the row's own storage) and denominators -> O = P V / denom.
 // Wavefront w takes key tiles w, w+4, ... for the scores and, for PV, output columns 32*(w & 1) .. +31
 // over the key half (w >> 1); the two halves meet in LDS.
+// kKeyTiles, kValueSteps: score tiles and PV steps of a wavefront whose fragments are requested up front; the launch
+// picks the smallest pair that covers the padded length (up to 4 and 16: 512 tokens), so that none is requested in vain.
+template <int kKeyTiles, int kValueSteps>
 __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, const _Float16 *vt, _Float16 *ctx, const EncParams *params,
                                                             int tpad, int width, int vt_stride, float scale) {
     const int tokens = params->tokens;
@@ -322,7 +355,9 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
     // ---- every global request of this workgroup is independent of the others and is issued here: the query
     // fragments, the key fragments of this wavefront's first kKeyTiles score tiles and the V fragments of its first
     // kValueSteps PV steps (all of them up to 512 tokens); they are consumed in that order while the rest arrives.
-    constexpr int kKeyTiles = 4, kValueSteps = 16;
+    // None of the requests is under a condition -- a tile or step this call does not have repeats the last one it has and
+    // is never used -- so that the number of requests behind each one is a constant: loads return in order, a wait names
+    // how many may still be out, and behind a conditional request the compiler has to wait for everything.
     const int ld = 2 * width;
     const int ntiles = tpad / 32;
     const int wn = wave & 1, kh = wave >> 1;
@@ -335,14 +370,12 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
     for (int j = 0; j < 4; ++j) fq[j] = *reinterpret_cast<const half8 *>(qrow + 16 * j);
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) {
-        const int tile = wave + 4 * t;
+        const int tile = min(wave + 4 * t, ntiles - 1);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            fk[t][j] = tile < ntiles ? *reinterpret_cast<const half8 *>(kbase + (size_t)tile * 32 * ld + 16 * j) : half8{0, 0, 0, 0, 0, 0, 0, 0};
+        for (int j = 0; j < 4; ++j) fk[t][j] = *reinterpret_cast<const half8 *>(kbase + (size_t)tile * 32 * ld + 16 * j);
     }
 #pragma unroll
-    for (int st = 0; st < kValueSteps; ++st)
-        fv[st] = 16 * st < kspan ? *reinterpret_cast<const half8 *>(vrow + 16 * st) : half8{0, 0, 0, 0, 0, 0, 0, 0};
+    for (int st = 0; st < kValueSteps; ++st) fv[st] = *reinterpret_cast<const half8 *>(vrow + min(16 * st, kspan - 16));
 
     // ---- scores
     {
@@ -357,7 +390,7 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
 #pragma unroll
         for (int t = 0; t < kKeyTiles; ++t)
             if (wave + 4 * t < ntiles) score_tile(wave + 4 * t, fk[t]);
-        for (int tile = wave + 4 * kKeyTiles; tile < ntiles; tile += 4) {   // more than 512 tokens
+        for (int tile = wave + 4 * kKeyTiles; tile < ntiles; tile += 4) {   // beyond the tiles requested up front (more than 512 tokens)
             half8 k4[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) k4[j] = *reinterpret_cast<const half8 *>(kbase + (size_t)tile * 32 * ld + 16 * j);
@@ -419,7 +452,7 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fp, fv[st], acc, 0, 0, 0);
             }
         }
-        for (int k = 16 * kValueSteps; k < kspan; k += 16) {   // more than 512 tokens
+        for (int k = 16 * kValueSteps; k < kspan; k += 16) {   // beyond the steps requested up front (more than 512 tokens)
             const half8 fp = *reinterpret_cast<const half8 *>(prow + k);
             const half8 fvk = *reinterpret_cast<const half8 *>(vrow + k);
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fp, fvk, acc, 0, 0, 0);
@@ -447,7 +480,11 @@ int launch_gemm(State *st, const GemmArgs &g, int splits, char *error, size_t ca
         set_error(error, capacity, "encoder product: shape is not a multiple of the 64 x 64 x 64 tile");
         return -1;
     }
-    hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth>), dim3(g.N / kTile, g.M / kTile, splits), dim3(kThreads), 0, st->stream, g);
+    const int steps = g.K / kTile / splits;
+    const dim3 grid(g.N / kTile, g.M / kTile, splits), block(kThreads);
+    if (steps % kGemmDepth == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true>), grid, block, 0, st->stream, g);
+    else if (steps % 2 == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true>), grid, block, 0, st->stream, g);
+    else hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false>), grid, block, 0, st->stream, g);
     return hip_check(hipGetLastError(), "encoder product launch", error, capacity);
 }
 
@@ -463,9 +500,12 @@ int f16_matrix(State *st, const float *host, size_t n, size_t k, const CachedWei
 size_t attention_lds_bytes(size_t tpad) { return (size_t)kQTile * (tpad + kScorePad) * sizeof(float); }
 
 constexpr int kMaxSplits = 4;   // k_enc_rows reads exactly this many partial planes at most
+// Most splits that leave each workgroup at least three K steps, preferring a step count the products' pipeline takes
+// without guards: a multiple of its depth, else an even one.
 int pick_splits(int k) {
-    for (int s = kMaxSplits; s > 1; --s)
-        if (k % (kTile * s) == 0 && k / (kTile * s) >= 3) return s;
+    for (const int multiple : {kGemmDepth, 2, 1})
+        for (int s = kMaxSplits; s > 1; --s)
+            if (k % (kTile * s) == 0 && k / (kTile * s) >= 3 && (k / (kTile * s)) % multiple == 0) return s;
     return 1;
 }
 
@@ -490,8 +530,13 @@ int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size
         g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->qkv[l]->data); g.M = tpad; g.N = 3 * w; g.K = w;
         g.out = e->qk; g.vt = e->vt; g.width = w; g.vt_stride = vt_stride;
         if (launch_gemm<ENC_QKV>(st, g, 1, error, capacity) != 0) return -1;
-        hipLaunchKernelGGL(k_enc_attention, dim3(tpad / kQTile, (unsigned)e->heads), dim3(kThreads), lds, st->stream, e->qk, e->vt, e->ctx, e->params,
-                           tpad, w, vt_stride, scale);
+        {
+            // a wavefront scores every fourth 32-key tile and multiplies half of the keys in steps of 16
+            const dim3 agrid(tpad / kQTile, (unsigned)e->heads), ablock(kThreads);
+            if (tpad <= 128) hipLaunchKernelGGL((k_enc_attention<1, 4>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale);
+            else if (tpad <= 256) hipLaunchKernelGGL((k_enc_attention<2, 8>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale);
+            else hipLaunchKernelGGL((k_enc_attention<4, 16>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale);
+        }
         g = GemmArgs{};
         g.a = e->ctx; g.w = static_cast<const _Float16 *>(e->o[l]->data); g.M = tpad; g.N = w; g.K = w; g.part = e->part;
         if (launch_gemm<ENC_PARTIAL>(st, g, o_splits, error, capacity) != 0) return -1;
@@ -588,10 +633,13 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
                   "encoder ids staging", error, capacity) != 0)
         return fail();
     e->params = reinterpret_cast<EncParams *>(e->ids + tp);   // tp is a multiple of 64: 8-byte aligned
-    if (attention_lds_bytes(e->tpad_max) > 48 * 1024 &&
-        hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_enc_attention), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (int)attention_lds_bytes(e->tpad_max)), "encoder attention LDS size", error, capacity) != 0)
-        return fail();
+    if (attention_lds_bytes(e->tpad_max) > 48 * 1024) {
+        const int bytes = (int)attention_lds_bytes(e->tpad_max);
+        if (hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_enc_attention<1, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes), "encoder attention LDS size", error, capacity) != 0 ||
+            hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_enc_attention<2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes), "encoder attention LDS size", error, capacity) != 0 ||
+            hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_enc_attention<4, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes), "encoder attention LDS size", error, capacity) != 0)
+            return fail();
+    }
     if (hip_check(hipStreamSynchronize(st->stream), "encoder create", error, capacity) != 0) return fail();
     *out = e;
     return 0;
