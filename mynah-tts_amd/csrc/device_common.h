@@ -261,6 +261,21 @@ __device__ __forceinline__ int attention_units(const StepSlots *s, int stream, i
     return chunks > 0 ? chunks : 1;
 }
 
+// A pointer that comes out of memory (the slot table's cache, input and output rows) carries no address space, and a load
+// or store through it is a flat instruction, which counts against the LDS counter as well as the vector-memory one: every
+// wait in front of a barrier then also waits for it.  These go through the pointer as what it is, a global address.
+typedef float float_x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 load_global4(const float *p) {
+    const float_x4 v = *(const __attribute__((address_space(1))) float_x4 *)p;
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ float load_global(const float *p) { return *(const __attribute__((address_space(1))) float *)p; }
+__device__ __forceinline__ void store_global(float *p, float v) { *(__attribute__((address_space(1))) float *)p = v; }
+__device__ __forceinline__ void store_global4(float *p, float4 v) {
+    const float_x4 w = {v.x, v.y, v.z, v.w};
+    *(__attribute__((address_space(1))) float_x4 *)p = w;
+}
+
 // Keeps the memory requests written above this point above it: without it the compiler is free to sink a load to its
 // first use, i.e. behind whatever that use waits for.  Emits no instruction and waits for nothing.
 __device__ __forceinline__ void requests_issued() { __asm__ volatile("" ::: "memory"); }

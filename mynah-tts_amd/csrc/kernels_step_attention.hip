@@ -208,6 +208,13 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 
     const int chunks = a.width / kEpc;
 
+    // ---- slot table: read before any vector request.  The stream is the same for the whole workgroup and nothing has
+    // been stored yet, so these are scalar loads, whose answers do not queue behind the vector loads below (vector loads
+    // return in order: a table word requested after the weight rows could only be looked at once all of them had come).
+    const int length = is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
+    float *const k_base = is_self ? slots->self_k[b] : const_cast<float *>(slots->cross_k[b]);
+    float *const v_base = is_self ? slots->self_v[b] : const_cast<float *>(slots->cross_v[b]);
+
     // With many streams most of the grid belongs to units that short streams do not have: there the slot table is
     // looked at first, so that such a workgroup leaves without having requested anything.  With one or two streams
     // nearly every unit is live and the weight rows are requested before the table has arrived (latency matters more).
@@ -234,19 +241,18 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     else load_bank<QT, PF>(pre, a, 0, 0, kHw, head, lg, chunks);
     if constexpr (PF == kPrefetchLatency) requests_issued();
 
-    // ---- slot table: is this unit live, and where are its cache rows?
-    const int length = is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
+    // ---- is this unit live, and where are its cache rows?
     const int nchunks = (length + kStepUnitRows - 1) / kStepUnitRows;
     const bool new_row = role_qk || role_v;
     if (!new_row && chunk >= (is_self ? nchunks : max(nchunks, 1))) return;
     const int stride = a.heads * kHw;   // floats between cache rows
     float *kc, *vc;
     if (is_self) {
-        kc = slots->self_k[b] + a.layer * a.capacity * (size_t)stride;
-        vc = slots->self_v[b] + a.layer * a.capacity * (size_t)stride;
+        kc = k_base + a.layer * a.capacity * (size_t)stride;
+        vc = v_base + a.layer * a.capacity * (size_t)stride;
     } else {
-        kc = const_cast<float *>(slots->cross_k[b]) + a.layer * (size_t)length * stride;
-        vc = const_cast<float *>(slots->cross_v[b]) + a.layer * (size_t)length * stride;
+        kc = k_base + a.layer * (size_t)length * stride;
+        vc = v_base + a.layer * (size_t)length * stride;
     }
     const int j = tid & (kPosLanes - 1);
     const int g = tid / kPosLanes;
@@ -286,17 +292,27 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         for (int i = 0; i < 4 * PF; ++i) sc2[i] = 0.0f;
 #pragma unroll
         for (int i = 0; i < PF; ++i) ws2[i] = 1.0f;
+        // Every request is issued, whatever the lane's row: a row past the chunk's end repeats the chunk's last row, and a
+        // workgroup without cache rows (the new row's V role; an empty memory, whose pointers may be null) reads the
+        // activation buffer, which always holds heads x 64 floats.  Under a per-lane condition each request would sit in
+        // a branch of its own with a wait behind it, and the next one would leave only after it had come back.
+        const bool have_rows = count[0] > 0;
+        const float *const k_from = have_rows ? kc : a.x;
+        const float *const v_from = have_rows ? vc : a.x;
 #pragma unroll
         for (int cc = 0; cc < CP; ++cc) {
+            const int rows = count[cc];
 #pragma unroll
             for (int i = 0; i < kRowsPerThread; ++i) {
                 const int pi = g + kPosPerPass * i;
-                const bool in_range = pi < count[cc];
-                const size_t at = (size_t)(p0 + cc * kStepUnitRows + pi) * stride + col;
-                kv[cc][i] = in_range ? *reinterpret_cast<const float4 *>(kc + at) : make_float4(0.f, 0.f, 0.f, 0.f);
-                vv[cc][i] = in_range ? *reinterpret_cast<const float4 *>(vc + at) : make_float4(0.f, 0.f, 0.f, 0.f);
+                const int row = !have_rows ? 0 : rows > 0 ? p0 + cc * kStepUnitRows + min(pi, rows - 1) : p0;
+                const size_t at = (size_t)row * stride + col;
+                kv[cc][i] = load_global4(k_from + at);
+                vv[cc][i] = load_global4(v_from + at);
             }
         }
+        // The repeated rows need no clearing: further down a row past the chunk's end gets the score -3e38 and the weight
+        // exactly 0, and fma(0, v, acc) is acc for the finite v of a real cache row -- the bits a zero row would give.
     }
 
     // ---- LayerNorm + activation quantisation of x[b], staged in LDS (the cache rows requested above stay in flight)
@@ -333,7 +349,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         __syncthreads();
         if (tid < 64) {
             const float kval = s_proj[kHw + tid];
-            kc[(size_t)length * stride + (size_t)head * kHw + tid] = kval;
+            store_global(kc + (size_t)length * stride + (size_t)head * kHw + tid, kval);
             float d = s_proj[tid] * kval;
             d = wave_sum(d);
             if (tid == 0) { out_m[0] = d * a.scale; out_l[0] = 1.0f; }   // exp(score - max) = 1
@@ -346,7 +362,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         __syncthreads();
         if (tid < kHw) {
             const float vval = s_proj[2 * kHw + tid];
-            vc[(size_t)length * stride + (size_t)head * kHw + tid] = vval;
+            store_global(vc + (size_t)length * stride + (size_t)head * kHw + tid, vval);
             a.partial[sh * a.max_units * kHw + tid] = vval;
         }
         return;
