@@ -255,10 +255,12 @@ struct ActSource {
 
 // Units a stream's attention was split into: cache chunks of kStepUnitRows rows, plus the step's new row for
 // self-attention.  Depends on that stream's own length only.
+__device__ __forceinline__ int units_of_length(int rows, int is_self) {
+    const int chunks = (rows + kStepUnitRows - 1) / kStepUnitRows;
+    return is_self ? chunks + 1 : (chunks > 0 ? chunks : 1);
+}
 __device__ __forceinline__ int attention_units(const StepSlots *s, int stream, int is_self) {
-    if (is_self) return (s->length[stream] + kStepUnitRows - 1) / kStepUnitRows + 1;
-    const int chunks = (s->memory_length[stream] + kStepUnitRows - 1) / kStepUnitRows;
-    return chunks > 0 ? chunks : 1;
+    return units_of_length(is_self ? s->length[stream] : s->memory_length[stream], is_self);
 }
 
 // A pointer that comes out of memory (the slot table's cache, input and output rows) carries no address space, and a load
@@ -293,17 +295,29 @@ __device__ __forceinline__ float4 fold_partials(const ActSource &src, int stream
     const float *m = src.partial_ml + sh * 2 * src.max_units;
     const float *l = m + src.max_units;
     const float *o = src.partial + sh * src.max_units * hw + dh;
+    // The unit count is read first: the stream is the same for the whole workgroup and nothing has been stored yet, so it is
+    // a scalar load, whose answer neither queues behind the vector requests below nor makes them wait; it is looked at
+    // after they have all been issued.  (Read after them it was a vector load -- nothing after requests_issued() can be
+    // proven unwritten -- that could only be looked at once every partial had come back: a round trip on top of theirs.)
+    // (every caller's stream is the same for a whole wavefront -- it depends on the team and the loop index only -- which
+    // the compiler cannot see through the thread index: readfirstlane says so)
+    const int stream_u = __builtin_amdgcn_readfirstlane(stream);
+    int rows = src.is_self ? src.slots->length[stream_u] : src.slots->memory_length[stream_u];
     float pm[kFoldAhead], pl[kFoldAhead];
     float4 po[kFoldAhead];
 #pragma unroll
     for (int u = 0; u < kFoldAhead; ++u) {
-        const bool in = u < src.max_units;
-        pm[u] = in ? m[u] : -3.0e38f;
-        pl[u] = in ? l[u] : 0.0f;
-        po[u] = in ? *reinterpret_cast<const float4 *>(o + (size_t)u * hw) : make_float4(0.f, 0.f, 0.f, 0.f);
+        // no request under a condition (the compiler would have to wait for all of them at the first use): a slot the
+        // workspace does not have repeats its last one, and is never used since units <= max_units
+        const int uu = u < src.max_units ? u : src.max_units - 1;
+        pm[u] = m[uu];
+        pl[u] = l[uu];
+        po[u] = *reinterpret_cast<const float4 *>(o + (size_t)uu * hw);
     }
     requests_issued();
-    const int units = attention_units(src.slots, stream, src.is_self);
+    rows = __builtin_amdgcn_readfirstlane(rows);   // the same for the whole wavefront
+    __asm__ volatile("" : "+s"(rows));               // the table word is first looked at here, behind the requests (emits nothing)
+    const int units = units_of_length(rows, src.is_self);
     float M = -3.0e38f;
 #pragma unroll
     for (int u = 0; u < kFoldAhead; ++u)
