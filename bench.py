@@ -245,8 +245,8 @@ STAGES = [("self-attention", "k_step_attention: LayerNorm + int8 act-quant + per
 # HBM bytes per launch (batch 1) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same counter
 # reads for the library's plain 256 MiB read+write kernel: x2.000 and x1.000); the summary with the commands is
 # profiles/decode_step_int8_hbm_counters.md.  Valid for the int8 workload these were measured on.
-MEASURED_TRAFFIC = {"self-attention": 8548039, "cross-attention": 2716151, "self-out": 947146, "cross-out": 947146,
-                    "ffn-up": 2532256, "ffn-down": 2656088}
+MEASURED_TRAFFIC = {"self-attention": 8543923, "cross-attention": 2695632, "self-out": 942538, "cross-out": 942538,
+                    "ffn-up": 2540386, "ffn-down": 2656109}
 
 
 def roofline(r):
