@@ -75,7 +75,9 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
     ConvArgs a = a_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;   // inner elements per step
-    const int a_stride = VEC ? kb : (kb | 1);  // odd row stride: the 32 rows a wavefront reads land in 32 different banks
+    const int a_stride = VEC ? kb + 4 : (kb | 1);  // odd row stride: the 32 rows a wavefront reads land in 32 different banks;
+                                                   // with 16-byte staging rows stay 16-byte aligned and get four floats of padding
+                                                   // (a stride of 4 mod 8 words spreads them over eight banks instead of four)
     const int halo = (a.kernel - 1) * a.dilation;
     const int win = TN + halo;                 // staged positions per input channel
     float *s_w = lds;                          // [TM][a_stride]
@@ -134,8 +136,8 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
         if constexpr (VEC != 0) {
 #pragma unroll
             for (int c = 0; c < kVecSlots; ++c) {
-                const int e = tid + 256 * c;
-                if (e < TM * kb4) reinterpret_cast<float4 *>(s_w)[e] = stage_w4[c];
+                const int e = tid + 256 * c, row = e / kb4, c4 = e - row * kb4;
+                if (e < TM * kb4) reinterpret_cast<float4 *>(s_w + row * a_stride)[c4] = stage_w4[c];
             }
         }
 #pragma unroll
@@ -192,8 +194,8 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
     ConvArgs a = a_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;
-    const int a_stride = kb;   // rows packed: a request of 64 consecutive block elements lands on 64 consecutive words (the row reads
-                               // of the products then share banks four ways, which costs a few cycles per 64-cycle product)
+    const int a_stride = kb + 4;   // rows stay 16-byte aligned and get four floats of padding: a stride of 4 mod 8 words spreads the
+                                   // 32 rows a wavefront reads for a product over eight banks instead of four
     const int halo = (a.kernel - 1) * a.dilation;
     const int win = TN + halo;
     const int per_wave = TM * a_stride + kConvChannels * win;
@@ -264,8 +266,8 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
     for (int round = 0; round < rounds; ++round) {
 #pragma unroll
         for (int c = 0; c < kCols; ++c) {
-            const int e = lane + 64 * c;
-            if (e < TM * kb4) reinterpret_cast<float4 *>(s_w)[e] = stage_w[c];
+            const int e = lane + 64 * c, row = e / kb4, c4 = e - row * kb4;
+            if (e < TM * kb4) reinterpret_cast<float4 *>(s_w + row * a_stride)[c4] = stage_w[c];
         }
 #pragma unroll
         for (int ch = 0; ch < kConvChannels; ++ch)
@@ -345,7 +347,7 @@ int launch_conv_v(State *st, const ConvArgs &a, char *error, size_t capacity) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     const int kb = kConvChannels * a.kernel;
     // two more staged rows than are filled: the product loop requests the operands after its last product before it stops
-    const size_t lds = ((size_t)TM * (kb | 1) + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
+    const size_t lds = ((size_t)TM * (VEC ? kb + 4 : (kb | 1)) + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
     static bool raised = false;   // per instantiation
     if (lds > 48 * 1024 && !raised) {
         MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF, VEC>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
@@ -375,7 +377,7 @@ int launch_conv(State *st, const ConvArgs &a, char *error, size_t capacity) {
 template <int KF, int NT>
 int launch_conv_split_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
     const int kb = kConvChannels * a.kernel;
-    const size_t per_wave = (size_t)32 * kb + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
+    const size_t per_wave = (size_t)32 * (kb + 4) + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
     size_t lds = (4 * per_wave + 2 * (32 * NT + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);   // see launch_conv about the two extra rows
     if (lds < 4 * 32 * 64 * sizeof(float)) lds = 4 * 32 * 64 * sizeof(float);   // the partial tiles
     static bool raised = false;
