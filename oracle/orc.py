@@ -500,8 +500,30 @@ class RefLocal:
             raise RuntimeError(err.value.decode())
         return outs, list(lens)
 
+    def use_hip(self, library_path):
+        """Hands the reference engine this repository's library as its backend (oracle/ref_shim_backend.c)."""
+        err = C.create_string_buffer(512)
+        self.r.ref_local_use_hip.restype = C.c_int
+        if self.r.ref_local_use_hip(C.c_void_p(self.h), os.fsencode(library_path), err, _sz(512)) != 0:
+            raise RuntimeError(err.value.decode())
+        self.device = True
+
+    def device_step(self, slot, length, x):
+        """The reference's local_step_device (src/graph.c:1106-1158) for one slot; returns (row, new length)."""
+        out = np.empty(self.cfg["width"], np.float32)
+        x = np.ascontiguousarray(x, np.float32)
+        n = _sz(length)
+        err = C.create_string_buffer(512)
+        self.r.ref_local_device_step.restype = C.c_int
+        rc = self.r.ref_local_device_step(C.c_void_p(self.h), _sz(slot), C.byref(n), _ptr(x), _ptr(out), err, _sz(512))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        return out, int(n.value)
+
     def close(self):
         if self.h:
+            if getattr(self, "device", False):
+                self.r.ref_local_release(C.c_void_p(self.h))
             self.r.ref_local_free(C.c_void_p(self.h))
             self.h = None
 
@@ -544,8 +566,48 @@ class RefDecoder:
             raise RuntimeError(err.value.decode())
         return outs, list(lens)
 
+    def use_hip(self, library_path):
+        """Hands the reference engine this repository's library as its backend (oracle/ref_shim_backend.c)."""
+        err = C.create_string_buffer(512)
+        self.r.ref_decoder_use_hip.restype = C.c_int
+        if self.r.ref_decoder_use_hip(C.c_void_p(self.h), os.fsencode(library_path), err, _sz(512)) != 0:
+            raise RuntimeError(err.value.decode())
+        self.device = True
+
+    def self_test(self):
+        err = C.create_string_buffer(512)
+        self.r.ref_decoder_self_test.restype = C.c_int
+        if self.r.ref_decoder_self_test(C.c_void_p(self.h), err, _sz(512)) != 0:
+            raise RuntimeError(err.value.decode())
+
+    def run_one(self, slot, self_k, self_v, cross_k, cross_v, length, memory_length, x):
+        """The reference's decoder_run with one row (src/graph.c:3292-3654); returns (row, new length, resident)."""
+        out = np.empty(self.cfg["width"], np.float32)
+        x = np.ascontiguousarray(x, np.float32)
+        n = _sz(length)
+        resident = C.c_int(0)
+        err = C.create_string_buffer(512)
+        self.r.ref_decoder_run_one.restype = C.c_int
+        rc = self.r.ref_decoder_run_one(C.c_void_p(self.h), _sz(slot), _ptr(self_k), _ptr(self_v), _ptr(cross_k), _ptr(cross_v),
+                                        C.byref(n), _sz(memory_length), _ptr(x), _ptr(out), C.byref(resident), err, _sz(512))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        return out, int(n.value), bool(resident.value)
+
+    def device_kv_row(self, slot, layer, row):
+        k = np.empty(self.cfg["width"], np.float32)
+        v = np.empty(self.cfg["width"], np.float32)
+        err = C.create_string_buffer(512)
+        self.r.ref_decoder_read_device_kv.restype = C.c_int
+        if self.r.ref_decoder_read_device_kv(C.c_void_p(self.h), _sz(slot), _sz(layer), _sz(row), _ptr(k), _ptr(v), err,
+                                             _sz(512)) != 0:
+            raise RuntimeError(err.value.decode() or "no device caches")
+        return k, v
+
     def close(self):
         if self.h:
+            if getattr(self, "device", False):
+                self.r.ref_decoder_release(C.c_void_p(self.h))
             self.r.ref_decoder_free(C.c_void_p(self.h))
             self.h = None
 

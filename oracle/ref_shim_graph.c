@@ -299,3 +299,153 @@ int ref_snake(float *data, const float *alpha, size_t channels, size_t length, s
     mynah_backend_close(backend);
     return rc;
 }
+
+/* ---- the reference engine as a consumer of a device backend ---------------------------------------------------
+ * Reference functions reached (file:line in the reference tree):
+ *   decoder_run                 src/graph.c:3292-3654  count == 1 and a backend with device operators and attention:
+ *                                                      the resident step, 18 seam calls per layer (:3368-3491)
+ *   decoder_gpu_attention_init  src/graph.c:2901-2962  device K/V caches, uploaded from the host caches once
+ *   local_step_device           src/graph.c:1106-1158  one resident local-transformer position
+ * ref_backend_open_hip (ref_shim_backend.c) fills the reference's backend struct with the library's entry points. */
+mynah_backend *ref_backend_open_hip(const char *library_path, char *error, size_t error_capacity);
+
+static void ref_decoder_release_device(ref_decoder *d) {
+    for (size_t b = 0; b < MYNAH_MAX_BATCH; ++b) {
+        decoder_cache *c = &d->caches[b];
+        if (c->dev_backend == NULL) continue;
+        /* the device half of decoder_cache_free (src/graph.c:2881-2897); the host caches are the caller's */
+        mynah_backend_dev_free(c->dev_backend, c->dev_nrm);
+        mynah_backend_dev_free(c->dev_backend, c->dev_qkv);
+        mynah_backend_dev_free(c->dev_backend, c->dev_attn);
+        mynah_backend_dev_free(c->dev_backend, c->dev_proj);
+        mynah_backend_dev_free(c->dev_backend, c->dev_qx);
+        mynah_backend_dev_free(c->dev_backend, c->dev_xctx);
+        mynah_backend_dev_free(c->dev_backend, c->dev_hidden);
+        mynah_backend_dev_free(c->dev_backend, c->dev_x);
+        if (c->dev_attention_allocated) {
+            mynah_backend_dev_free(c->dev_backend, c->dev_self_k);
+            mynah_backend_dev_free(c->dev_backend, c->dev_self_v);
+            mynah_backend_dev_free(c->dev_backend, c->dev_cross_k);
+            mynah_backend_dev_free(c->dev_backend, c->dev_cross_v);
+        }
+        c->dev_nrm = c->dev_qkv = c->dev_attn = c->dev_proj = c->dev_qx = c->dev_xctx = c->dev_hidden = c->dev_x = NULL;
+        c->dev_self_k = c->dev_self_v = c->dev_cross_k = c->dev_cross_v = NULL;
+        c->dev_allocated = 0;
+        c->dev_attention_allocated = 0;
+        c->dev_backend = NULL;
+    }
+}
+
+/* Replaces the decoder's CPU backend by the library at library_path.  Device buffers of the previous backend are
+ * released first. */
+int ref_decoder_use_hip(ref_decoder *d, const char *library_path, char *error, size_t error_capacity) {
+    mynah_backend *hip = ref_backend_open_hip(library_path, error, error_capacity);
+    if (hip == NULL) return -1;
+    ref_decoder_release_device(d);
+    if (d->model.backend != NULL) mynah_backend_close(d->model.backend);
+    d->model.backend = hip;
+    return 0;
+}
+
+/* Call before ref_decoder_free when a device backend is attached (ref_decoder_free closes the backend). */
+void ref_decoder_release(ref_decoder *d) { if (d != NULL) ref_decoder_release_device(d); }
+
+/* The attached backend's own self-test through the struct's function pointer. */
+int ref_backend_self_test(const mynah_backend *backend, char *error, size_t error_capacity);
+int ref_decoder_self_test(ref_decoder *d, char *error, size_t error_capacity) {
+    return ref_backend_self_test(d->model.backend, error, error_capacity);
+}
+
+/* One single-row decoder_run of slot `slot`.  On the first call of a slot the host caches (rows [0, *length) of
+ * self_k/self_v, all of cross_k/cross_v) are what the engine uploads; afterwards the device caches are the live ones
+ * and the pointers are only kept for the engine's bookkeeping.  *resident comes back 1 when the slot's device
+ * buffers and device caches exist after the call, i.e. the resident path was taken. */
+int ref_decoder_run_one(ref_decoder *d, size_t slot, float *self_k, float *self_v, float *cross_k, float *cross_v,
+                        size_t *length, size_t memory_length, const float *input, float *out, int *resident,
+                        char *error, size_t error_capacity) {
+    if (slot >= d->batch) return -1;
+    decoder_cache *c = &d->caches[slot];
+    c->self_k = self_k; c->self_v = self_v; c->cross_k = cross_k; c->cross_v = cross_v;
+    c->length = *length;
+    c->memory_length = memory_length;
+    const int rc = decoder_run(&d->model, c, input, 1u, out, NULL, error, error_capacity);
+    *length = c->length;
+    if (resident != NULL) *resident = c->dev_allocated && c->dev_attention_allocated;
+    return rc;
+}
+
+/* Row `row` of layer `layer` of the slot's device K and V caches, through the backend's own d2h. */
+int ref_decoder_read_device_kv(ref_decoder *d, size_t slot, size_t layer, size_t row, float *k_row, float *v_row,
+                               char *error, size_t error_capacity) {
+    decoder_cache *c = &d->caches[slot];
+    if (!c->dev_attention_allocated) return -1;
+    const size_t offset = (layer * c->capacity + row) * c->width;
+    if (mynah_backend_d2h(c->dev_backend, c->dev_self_k + offset, k_row, c->width, error, error_capacity) != 0) return -1;
+    return mynah_backend_d2h(c->dev_backend, c->dev_self_v + offset, v_row, c->width, error, error_capacity);
+}
+
+/* -- local transformer, resident position ----------------------------------------------------------------------- */
+static void ref_local_release_device(ref_local *d) {
+    for (size_t b = 0; b < MYNAH_MAX_BATCH; ++b) {
+        local_cache *c = &d->caches[b];
+        if (c->dev_backend == NULL) continue;
+        mynah_backend_dev_free(c->dev_backend, c->dev_k);      mynah_backend_dev_free(c->dev_backend, c->dev_v);
+        mynah_backend_dev_free(c->dev_backend, c->dev_x);      mynah_backend_dev_free(c->dev_backend, c->dev_nrm);
+        mynah_backend_dev_free(c->dev_backend, c->dev_qkv);    mynah_backend_dev_free(c->dev_backend, c->dev_attn);
+        mynah_backend_dev_free(c->dev_backend, c->dev_proj);   mynah_backend_dev_free(c->dev_backend, c->dev_hidden);
+        mynah_backend_dev_free(c->dev_backend, c->dev_input);
+        c->dev_k = c->dev_v = c->dev_x = c->dev_nrm = c->dev_qkv = c->dev_attn = c->dev_proj = c->dev_hidden = NULL;
+        c->dev_input = NULL;
+        c->dev_backend = NULL;
+        c->gpu_ready = 0;
+    }
+}
+
+int ref_local_use_hip(ref_local *d, const char *library_path, char *error, size_t error_capacity) {
+    mynah_backend *hip = ref_backend_open_hip(library_path, error, error_capacity);
+    if (hip == NULL) return -1;
+    ref_local_release_device(d);
+    if (d->model.backend != NULL) mynah_backend_close(d->model.backend);
+    d->model.backend = hip;
+    return 0;
+}
+
+void ref_local_release(ref_local *d) { if (d != NULL) ref_local_release_device(d); }
+
+/* One resident position of slot `slot`: the buffers local_cache_init allocates for a device backend
+ * (src/graph.c:1058-1090; the logits buffer is not touched by the step and is left out), the input row uploaded,
+ * local_step_device, and the output row read back.  *length is the slot's position before / after. */
+int ref_local_device_step(ref_local *d, size_t slot, size_t *length, const float *input, float *out,
+                          char *error, size_t error_capacity) {
+    if (slot >= d->batch) return -1;
+    local_cache *c = &d->caches[slot];
+    const mynah_backend *bk = d->model.backend;
+    if (!mynah_backend_has_dev_ops(bk) || !mynah_backend_has_attention_dev(bk)) {
+        graph_error(error, error_capacity, "backend has no resident operators");
+        return -1;
+    }
+    if (!c->gpu_ready) {
+        const size_t kv_count = c->layers * c->capacity * c->width;
+        c->dev_backend = bk;
+        const int ok =
+            mynah_backend_dev_alloc(bk, kv_count, &c->dev_k, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, kv_count, &c->dev_v, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, c->width, &c->dev_x, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, c->width, &c->dev_nrm, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, c->width * 3u, &c->dev_qkv, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, c->width, &c->dev_attn, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, c->width, &c->dev_proj, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, c->ffn_width, &c->dev_hidden, error, error_capacity) == 0 &&
+            mynah_backend_dev_alloc(bk, c->width, &c->dev_input, error, error_capacity) == 0;
+        if (!ok) { ref_local_release_device(d); return -1; }
+        c->gpu_ready = 1;
+    }
+    c->length = *length;
+    float *dev_out = NULL;
+    if (mynah_backend_h2d(bk, input, c->dev_input, c->width, error, error_capacity) != 0) return -1;
+    if (local_step_device(&d->model, c, c->dev_input, &dev_out, error, error_capacity) != 0) return -1;
+    if (mynah_backend_sync(bk, error, error_capacity) != 0) return -1;
+    if (mynah_backend_d2h(bk, dev_out, out, c->width, error, error_capacity) != 0) return -1;
+    *length = c->length;
+    return 0;
+}
