@@ -684,3 +684,74 @@ def ref_codec(strict=False):
     r.ref_snake.argtypes = [fp, fp, _sz, _sz, _sz]
     r.ref_snake.restype = C.c_int
     return r
+
+
+class RefCodecEngine:
+    """The reference's decode_codec (src/graph.c:2640-2790) on a safetensors file of synthetic codec weights: with
+    hip_library=None its CPU sequence on the CPU backend, otherwise decode_codec_resident on that library."""
+
+    def __init__(self, weights_path, hip_library=None, strict=False):
+        self.r = load_ref(strict)
+        self.r.ref_codec_engine_new.restype = C.c_void_p
+        self.r.ref_codec_engine_new.argtypes = [C.c_char_p, C.c_char_p, C.c_char_p, _sz]
+        self.r.ref_codec_engine_free.argtypes = [C.c_void_p]
+        self.r.ref_codec_engine_decode.restype = C.c_int
+        err = C.create_string_buffer(512)
+        self.h = self.r.ref_codec_engine_new(os.fsencode(weights_path), None if hip_library is None else os.fsencode(hip_library),
+                                             err, 512)
+        if not self.h:
+            raise RuntimeError(err.value.decode())
+
+    def decode(self, codes):
+        codes = np.ascontiguousarray(codes, np.uint32)
+        assert codes.ndim == 2 and codes.shape[0] == 8
+        raw = codes.shape[1]
+        samples = np.empty(raw * 1024, np.float32)
+        count, resident = _sz(0), C.c_int(0)
+        err = C.create_string_buffer(512)
+        rc = self.r.ref_codec_engine_decode(C.c_void_p(self.h), _ptr(codes), _sz(raw), _ptr(samples), _sz(samples.size),
+                                            C.byref(count), C.byref(resident), err, _sz(512))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        assert count.value == samples.size
+        return samples, bool(resident.value)
+
+    def close(self):
+        if self.h:
+            self.r.ref_codec_engine_free(C.c_void_p(self.h))
+            self.h = None
+
+
+def codec_weights(seed=11):
+    """Synthetic NanoCodec decoder weights under the tensor names the reference's codec decode looks up
+    (src/graph.c:2345-2400,2444-2480,2547-2617): 32 -> 864 pre-conv (7 taps), five stages of half-snake alpha, grouped
+    transposed conv (rates 8 8 4 2 2, one group per output channel) and 3 x 3 residual blocks (taps 3 / 7 / 11), the post
+    snake alpha and the 1-channel post-conv (3 taps)."""
+    rng = np.random.default_rng(seed)
+    t = {}
+
+    def conv(prefix, out_ch, in_ch, k):
+        t[prefix + ".weight"] = rng.standard_normal((out_ch, in_ch, k), dtype=np.float32) * np.float32(1.0 / np.sqrt(in_ch * k))
+        t[prefix + ".bias"] = rng.standard_normal(out_ch, dtype=np.float32) * np.float32(0.1)
+
+    def alpha(name, channels):
+        t[name] = np.abs(rng.standard_normal(channels // 2, dtype=np.float32)) + np.float32(0.1)
+
+    conv("audio_decoder.pre_conv.conv", 864, 32, 7)
+    c = 864
+    for stage, rate in enumerate((8, 8, 4, 2, 2)):
+        alpha("audio_decoder.activations.%d.activation.snake_act.alpha" % stage, c)
+        nc = c // 2
+        t["audio_decoder.up_sample_conv_layers.%d.conv.weight" % stage] = rng.standard_normal((c, 1, 2 * rate), dtype=np.float32) * np.float32(0.3)
+        t["audio_decoder.up_sample_conv_layers.%d.conv.bias" % stage] = rng.standard_normal(nc, dtype=np.float32) * np.float32(0.1)
+        for branch, k in enumerate((3, 7, 11)):
+            for block in range(3):
+                p = "audio_decoder.res_layers.%d.res_blocks.%d.res_blocks.%d." % (stage, branch, block)
+                alpha(p + "input_activation.activation.snake_act.alpha", nc)
+                conv(p + "input_conv.conv", nc, nc, k)
+                alpha(p + "skip_activation.activation.snake_act.alpha", nc)
+                conv(p + "skip_conv.conv", nc, nc, k)
+        c = nc
+    alpha("audio_decoder.post_activation.activation.snake_act.alpha", c)
+    conv("audio_decoder.post_conv.conv", 1, c, 3)
+    return t

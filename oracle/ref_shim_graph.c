@@ -449,3 +449,50 @@ int ref_local_device_step(ref_local *d, size_t slot, size_t *length, const float
     *length = c->length;
     return 0;
 }
+
+/* -- the codec decode, CPU orchestration against resident orchestration ------------------------------------------
+ * Reference functions reached (file:line in the reference tree):
+ *   decode_codec            src/graph.c:2640-2790  tries decode_codec_resident first, else the CPU sequence
+ *   decode_codec_resident   src/graph.c:2508-2638  taken when the backend has device operators and attention
+ *   res_layer_device        src/graph.c:2423-2505
+ * The model is zero-filled except for its codec weight file (a safetensors file the caller wrote) and its backend. */
+typedef struct {
+    mynah_tts_model model;
+} ref_codec_engine;
+
+void ref_codec_engine_free(ref_codec_engine *e) {
+    if (e == NULL) return;
+    if (e->model.backend != NULL) mynah_backend_close(e->model.backend);
+    if (e->model.codec != NULL) mynah_weights_close(e->model.codec);
+    free(e);
+}
+
+/* hip_library == NULL: the reference's CPU backend. */
+ref_codec_engine *ref_codec_engine_new(const char *weights_path, const char *hip_library, char *error, size_t error_capacity) {
+    ref_codec_engine *e = (ref_codec_engine *)calloc(1, sizeof(*e));
+    if (e == NULL) return NULL;
+    if (mynah_weights_open(weights_path, &e->model.codec, error, error_capacity) != 0) { free(e); return NULL; }
+    if (hip_library != NULL) {
+        e->model.backend = ref_backend_open_hip(hip_library, error, error_capacity);
+        if (e->model.backend == NULL) { ref_codec_engine_free(e); return NULL; }
+    } else if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &e->model.backend, error, error_capacity) != 0) {
+        ref_codec_engine_free(e);
+        return NULL;
+    }
+    return e;
+}
+
+/* codes: [8 groups, raw_length].  Returns the sample count through *count (raw_length * 1024) and copies at most
+ * `capacity` samples into `samples`.  *resident says which of the two sequences the engine chose. */
+int ref_codec_engine_decode(ref_codec_engine *e, const unsigned *codes, size_t raw_length, float *samples, size_t capacity,
+                            size_t *count, int *resident, char *error, size_t error_capacity) {
+    float *audio = NULL;
+    size_t n = 0;
+    const mynah_backend *bk = e->model.backend;
+    if (resident != NULL) *resident = mynah_backend_has_dev_ops(bk) && mynah_backend_has_attention_dev(bk);
+    if (decode_codec(&e->model, codes, raw_length, &audio, &n, error, error_capacity) != 0) return -1;
+    memcpy(samples, audio, (n < capacity ? n : capacity) * sizeof(float));
+    free(audio);
+    *count = n;
+    return 0;
+}

@@ -133,3 +133,31 @@ def test_local_step_device(pkg, orc, ref_strict, synth, nerr, quant_env, qtype_n
     finally:
         hip.close()
         cpu.close()
+
+
+def test_codec_decode_resident(pkg, orc, ref_strict, nerr, quant_env, tmp_path):
+    """The reference's decode_codec on a file of synthetic codec weights (every tensor at the codec's real shape): on
+    the library it takes decode_codec_resident (src/graph.c:2508-2638: pre-conv, five stages of snake, grouped
+    transposed conv and res_layer_device, post-conv, clip -- about 290 operator calls), on the CPU backend its own CPU
+    sequence (im2col + sgemm convolutions).  Three raw frames -> 3072 samples.  Ninety-five convolutions in a row, each
+    adding in a different order on the matrix cores than the CPU does: 1e-4 normalised on the clipped waveform."""
+    _announce("engine: decode_codec resident, 3 raw frames")
+    quant_env("f32")
+    path = str(tmp_path / "codec.safetensors")
+    orc.write_safetensors(path, orc.codec_weights(seed=11))
+    codes = np.random.default_rng(1).integers(0, 2016, (8, 3)).astype(np.uint32)
+    cpu = orc.RefCodecEngine(path, None, strict=True)
+    hip = orc.RefCodecEngine(path, pkg.LIB_PATH, strict=True)
+    try:
+        want, cpu_resident = cpu.decode(codes)
+        got, resident = hip.decode(codes)
+        assert resident and not cpu_resident
+        assert np.all(np.isfinite(got)) and np.abs(got).max() <= 1.0
+        assert np.std(want) > 0.05, "degenerate waveform"
+        e = nerr(got, want)
+        assert e < 1e-4, "codec waveform: %.3g" % e
+        again, _ = hip.decode(codes)          # weights now come from the library's device cache
+        assert np.array_equal(again, got)
+    finally:
+        hip.close()
+        cpu.close()
