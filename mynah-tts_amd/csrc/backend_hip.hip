@@ -260,7 +260,7 @@ static int matmul_device(State *st, const float *din, float *dout, size_t rows, 
 // host in / host out, synchronous (mynah_backend_matmul, src/backend.h:32-35)
 static int hip_matmul(void *opaque, const float *input, float *output, size_t rows, size_t iw, size_t ow,
                       const float *weight, const float *bias, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (check_rows(input, output, rows, iw, ow, weight, error, capacity) != 0) return -1;
     MYNAH_NEED_STATE(st);
     const size_t in_n = rows * iw, out_n = rows * ow;   // each factor is below 2^31
@@ -275,7 +275,7 @@ static int hip_matmul(void *opaque, const float *input, float *output, size_t ro
 
 static int hip_sgemm(void *opaque, int ta, int tb, size_t m, size_t n, size_t k, float alpha, const float *a, size_t lda,
                      const float *b, size_t ldb, float beta, float *c, size_t ldc, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (a == nullptr || b == nullptr || c == nullptr || m == 0 || n == 0) {
         set_error(error, capacity, "invalid sgemm arguments");
         return -1;
@@ -299,7 +299,7 @@ static int hip_sgemm(void *opaque, int ta, int tb, size_t m, size_t n, size_t k,
 }
 
 static void hip_close(void *opaque) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (st == nullptr) return;
     (void)hipStreamSynchronize(st->stream);
     for (auto &kv : st->weights) {
@@ -418,6 +418,8 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
     else if (quant != nullptr && strcmp(quant, "f16") == 0) st->qtype = MYNAH_HIP_F16;
     const char *arith = getenv("MYNAH_QUANT_ARITH");
     if (arith != nullptr && strcmp(arith, "stock") == 0) st->arith = MYNAH_HIP_ARITH_STOCK;
+    const char *fuse = getenv("MYNAH_HIP_FUSE");   // 0: every seam call is a launch of its own
+    if (fuse != nullptr && strcmp(fuse, "0") == 0) st->fuse = 0;
     const char *graph = getenv("MYNAH_HIP_GRAPH");
     if (graph != nullptr && strcmp(graph, "0") == 0) st->graph_mode = 0;
     *state_out = st;
@@ -440,14 +442,14 @@ extern "C" int mynah_hip_dev_alloc(void *opaque, size_t n, float **dev_ptr, char
 }
 
 extern "C" void mynah_hip_dev_free(void *opaque, float *dev_ptr) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (dev_ptr == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
     (void)hipFree(dev_ptr);
 }
 
 extern "C" int mynah_hip_h2d(void *opaque, const float *host, float *dev_ptr, size_t n, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     size_t bytes = 0;
     if (st == nullptr || host == nullptr || dev_ptr == nullptr || !float_bytes(n, &bytes)) {
         set_error(error, capacity, "invalid h2d arguments");
@@ -457,7 +459,7 @@ extern "C" int mynah_hip_h2d(void *opaque, const float *host, float *dev_ptr, si
 }
 
 extern "C" int mynah_hip_d2h(void *opaque, const float *dev_ptr, float *host, size_t n, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     size_t bytes = 0;
     if (st == nullptr || host == nullptr || dev_ptr == nullptr || !float_bytes(n, &bytes)) {
         set_error(error, capacity, "invalid d2h arguments");
@@ -469,7 +471,7 @@ extern "C" int mynah_hip_d2h(void *opaque, const float *dev_ptr, float *host, si
 }
 
 extern "C" int mynah_hip_upload(void *opaque, const float *host, size_t n, float **dev_ptr, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     size_t bytes = 0;
     if (st == nullptr || host == nullptr || dev_ptr == nullptr || n == 0 || !float_bytes(n, &bytes)) {
         set_error(error, capacity, "invalid upload arguments");
@@ -485,8 +487,14 @@ extern "C" int mynah_hip_download(void *opaque, const float *dev_ptr, float *hos
 }
 
 extern "C" int mynah_hip_sync(void *opaque, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
+    if (st->deferred_error[0] != '\0') {   // a held-back launch failed inside a call that could not report it
+        set_error(error, capacity, st->deferred_error);
+        st->deferred_error[0] = '\0';
+        (void)hipStreamSynchronize(st->stream);
+        return -1;
+    }
     return hip_check(hipStreamSynchronize(st->stream), "sync", error, capacity);
 }
 
@@ -496,17 +504,94 @@ extern "C" int mynah_hip_batch_begin(void *opaque, char *error, size_t capacity)
     return 0;
 }
 
+// ---- seam fusion -------------------------------------------------------------------------------------------------
+// The engine's resident step makes 18 seam calls per layer (src/graph.c:3391-3476), most of them tiny dependent
+// launches: LayerNorm -> product, product -> GELU, product -> residual add.  A single-row LayerNorm or product is
+// therefore held back for one call.  When the next call continues the chain on the same buffers, the two (or three)
+// become one launch of the fused matvec kernel, which writes every buffer the separate calls would have written (the
+// LayerNorm row, the product before the residual add); any other call launches what is held back first
+// (enter_state).  Chains: LayerNorm + product, LayerNorm + product + GELU, product + GELU, product + residual.
+static bool ranges_overlap(const float *a, size_t na, const float *b, size_t nb) {
+    if (a == nullptr || b == nullptr) return false;
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a0 < b0 + nb * sizeof(float) && b0 < a0 + na * sizeof(float);
+}
+
+static int launch_pending_linear(State *st, const PendingOp &p, int epilogue, float *residual_row, char *error, size_t capacity) {
+    LinearArgs a{};
+    a.w = p.weight->data;
+    a.scales = p.weight->scales;
+    a.bias = p.bias;
+    a.qtype = p.weight->qtype;
+    a.n = (int)p.ow;
+    a.k = (int)p.iw;
+    a.batch = 1;
+    a.in[0] = p.has_ln ? p.ln_in : p.in;
+    a.arith = st->arith;
+    a.epilogue = epilogue;
+    if (p.has_ln) {
+        a.ln_gain = p.ln_gain;
+        a.ln_bias = p.ln_bias;
+        a.ln_out = p.ln_out;
+    }
+    if (epilogue == EPI_RESIDUAL) {
+        a.out[0] = residual_row;   // row += product
+        a.aux_out = p.out;         // the product itself, where the separate call would have left it
+    } else {
+        a.out[0] = p.out;
+    }
+    return launch_linear(st, a, error, capacity);
+}
+
+static int seam_flush(State *st, char *error, size_t capacity) {
+    const PendingOp p = st->pending;
+    st->pending = PendingOp{};
+    if (p.kind == PendingOp::kLayerNorm) return launch_layernorm(st, p.ln_in, p.ln_out, p.ln_gain, p.ln_bias, 1, p.iw, error, capacity);
+    if (p.kind == PendingOp::kLinear) return launch_pending_linear(st, p, EPI_NONE, nullptr, error, capacity);
+    return 0;
+}
+
+State *mynah::enter_state(void *opaque) {
+    State *st = static_cast<State *>(opaque);
+    if (st != nullptr && st->pending.kind != PendingOp::kNone) {
+        char message[sizeof st->deferred_error] = {0};
+        if (seam_flush(st, message, sizeof message) != 0 && st->deferred_error[0] == '\0')
+            snprintf(st->deferred_error, sizeof st->deferred_error, "%s", message[0] != '\0' ? message : "a held-back launch failed");
+    }
+    return st;
+}
+
 // =========================================================================================== resident ops
 extern "C" int mynah_hip_gelu_inplace(void *opaque, float *d, size_t n, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
     if (d == nullptr) { set_error(error, capacity, "invalid gelu arguments"); return -1; }
-    return launch_gelu(static_cast<State *>(opaque), d, n, error, capacity);
+    if (st->pending.kind == PendingOp::kLinear && st->pending.out == d && st->pending.ow == n) {
+        const PendingOp p = st->pending;
+        st->pending = PendingOp{};
+        return launch_pending_linear(st, p, EPI_GELU, nullptr, error, capacity);
+    }
+    if (seam_flush(st, error, capacity) != 0) return -1;
+    return launch_gelu(st, d, n, error, capacity);
 }
 extern "C" int mynah_hip_gelu_dev(void *opaque, float *d, size_t n, char *error, size_t capacity) {
     return mynah_hip_gelu_inplace(opaque, d, n, error, capacity);
 }
 extern "C" int mynah_hip_residual_inplace(void *opaque, float *dout, const float *din, size_t n, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
     if (dout == nullptr || din == nullptr) { set_error(error, capacity, "invalid residual arguments"); return -1; }
+    {
+        // product -> `dout += product`: one launch, unless the row being updated is one the product reads or writes
+        const PendingOp &p = st->pending;
+        if (p.kind == PendingOp::kLinear && p.out == din && p.ow == n && !ranges_overlap(dout, n, p.out, p.ow) &&
+            !ranges_overlap(dout, n, p.in, p.iw) && !(p.has_ln && (ranges_overlap(dout, n, p.ln_in, p.iw) || ranges_overlap(dout, n, p.ln_out, p.iw)))) {
+            const PendingOp q = p;
+            st->pending = PendingOp{};
+            return launch_pending_linear(st, q, EPI_RESIDUAL, dout, error, capacity);
+        }
+    }
+    if (seam_flush(st, error, capacity) != 0) return -1;
     // The engine passes a HOST row of the mmapped position table in the device slot (src/graph.c:1118-1120):
     // resolve it through the pointer-keyed cache when the address is not device memory.
     hipPointerAttribute_t attr;
@@ -524,7 +609,8 @@ extern "C" int mynah_hip_residual_add_dev(void *opaque, float *dout, const float
 }
 extern "C" int mynah_hip_layer_norm_dev(void *opaque, const float *din, float *dout, const float *gain, const float *bias,
                                         size_t rows, size_t width, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
     if (din == nullptr || dout == nullptr || gain == nullptr || width == 0 || width > 0x7fffffffu) {
         set_error(error, capacity, "invalid layer norm arguments");
         return -1;
@@ -532,27 +618,73 @@ extern "C" int mynah_hip_layer_norm_dev(void *opaque, const float *din, float *d
     const float *dgain = nullptr, *dbias = nullptr;
     if (cached_vector(st, gain, width, &dgain, error, capacity) != 0) return -1;
     if (cached_vector(st, bias, width, &dbias, error, capacity) != 0) return -1;
+    if (st->fuse && rows == 1 && !ranges_overlap(din, width, dout, width)) {   // held back: a product may follow
+        PendingOp &p = st->pending;
+        p.kind = PendingOp::kLayerNorm;
+        p.ln_in = din;
+        p.ln_out = dout;
+        p.ln_gain = dgain;
+        p.ln_bias = dbias;
+        p.iw = width;
+        return 0;
+    }
     return launch_layernorm(st, din, dout, dgain, dbias, rows, width, error, capacity);
 }
 extern "C" int mynah_hip_layer_norm_inplace(void *opaque, const float *din, float *dout, const float *gain, size_t rows,
                                             size_t width, char *error, size_t capacity) {
     return mynah_hip_layer_norm_dev(opaque, din, dout, gain, nullptr, rows, width, error, capacity);
 }
+
+// Single-row products of the seam: joins a held-back LayerNorm of its input row, and is itself held back for a GELU or
+// residual add of its output row.
+static int seam_matmul(void *opaque, const float *din, float *dout, size_t rows, size_t iw, size_t ow, const float *weight,
+                       const float *bias, char *error, size_t capacity) {
+    State *st = static_cast<State *>(opaque);
+    MYNAH_NEED_STATE(st);
+    if (check_rows(din, dout, rows, iw, ow, weight, error, capacity) != 0) return -1;
+    if (st->fuse && rows == 1) {
+        const float *dbias = nullptr;
+        const CachedWeight *cw = nullptr;
+        if (cached_vector(st, bias, ow, &dbias, error, capacity) != 0) return -1;
+        if (cached_matrix(st, weight, ow, iw, st->qtype, &cw, error, capacity) != 0) return -1;
+        if (linear_fast_supported(cw->qtype, ow, iw) && !ranges_overlap(din, iw, dout, ow)) {
+            PendingOp p = st->pending;
+            const bool joins = p.kind == PendingOp::kLayerNorm && p.ln_out == din && p.iw == iw &&
+                               !ranges_overlap(dout, ow, p.ln_in, iw) && !ranges_overlap(dout, ow, p.ln_out, iw);
+            if (!joins) {
+                if (seam_flush(st, error, capacity) != 0) return -1;
+                p = PendingOp{};
+            }
+            p.kind = PendingOp::kLinear;
+            p.has_ln = joins;
+            p.in = din;
+            p.out = dout;
+            p.iw = iw;
+            p.ow = ow;
+            p.weight = cw;
+            p.bias = dbias;
+            st->pending = p;
+            return 0;
+        }
+    }
+    if (seam_flush(st, error, capacity) != 0) return -1;
+    return matmul_device(st, din, dout, rows, iw, ow, weight, bias, error, capacity);
+}
 extern "C" int mynah_hip_matmul_d2d(void *opaque, const float *din, float *dout, size_t rows, size_t iw, size_t ow,
                                     const float *weight, const float *bias, char *error, size_t capacity) {
-    return matmul_device(static_cast<State *>(opaque), din, dout, rows, iw, ow, weight, bias, error, capacity);
+    return seam_matmul(opaque, din, dout, rows, iw, ow, weight, bias, error, capacity);
 }
 extern "C" int mynah_hip_matmul_dev(void *opaque, const float *din, float *dout, size_t rows, size_t iw, size_t ow,
                                     const float *weight, const float *bias, char *error, size_t capacity) {
-    return matmul_device(static_cast<State *>(opaque), din, dout, rows, iw, ow, weight, bias, error, capacity);
+    return seam_matmul(opaque, din, dout, rows, iw, ow, weight, bias, error, capacity);
 }
 extern "C" int mynah_hip_matvec_dev(void *opaque, const float *din, float *dout, size_t K, size_t N, const float *weight,
                                     const float *bias, char *error, size_t capacity) {
-    return matmul_device(static_cast<State *>(opaque), din, dout, 1, K, N, weight, bias, error, capacity);
+    return seam_matmul(opaque, din, dout, 1, K, N, weight, bias, error, capacity);
 }
 extern "C" int mynah_hip_matmul_to_dev(void *opaque, const float *host_in, float *dout, size_t rows, size_t iw, size_t ow,
                                        const float *weight, const float *bias, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
     if (check_rows(host_in, dout, rows, iw, ow, weight, error, capacity) != 0) return -1;
     if (ensure_scratch(st, rows * iw * sizeof(float), error, capacity) != 0) return -1;
@@ -563,27 +695,27 @@ extern "C" int mynah_hip_sgemm_dev(void *opaque, int ta, int tb, size_t m, size_
                                    size_t lda, const float *db, size_t ldb, float beta, float *dc, size_t ldc, char *error,
                                    size_t capacity) {
     if (da == nullptr || db == nullptr || dc == nullptr) { set_error(error, capacity, "invalid sgemm arguments"); return -1; }
-    return launch_sgemm(static_cast<State *>(opaque), ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc, error, capacity);
+    return launch_sgemm(enter_state(opaque), ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc, error, capacity);
 }
 extern "C" int mynah_hip_softmax_dev(void *opaque, float *d, size_t rows, size_t cols, size_t valid, char *error, size_t capacity) {
     if (d == nullptr || cols > 0x7fffffffu) { set_error(error, capacity, "invalid softmax arguments"); return -1; }
-    return launch_softmax(static_cast<State *>(opaque), d, rows, cols, valid, error, capacity);
+    return launch_softmax(enter_state(opaque), d, rows, cols, valid, error, capacity);
 }
 extern "C" int mynah_hip_copy_dev(void *opaque, float *dst, const float *src, size_t n, char *error, size_t capacity) {
     if (dst == nullptr || src == nullptr) { set_error(error, capacity, "invalid copy arguments"); return -1; }
-    return launch_copy(static_cast<State *>(opaque), dst, src, n, error, capacity);
+    return launch_copy(enter_state(opaque), dst, src, n, error, capacity);
 }
 extern "C" int mynah_hip_scale_dev(void *opaque, float *d, size_t n, float scale, char *error, size_t capacity) {
     if (d == nullptr) { set_error(error, capacity, "invalid scale arguments"); return -1; }
-    return launch_scale(static_cast<State *>(opaque), d, n, scale, error, capacity);
+    return launch_scale(enter_state(opaque), d, n, scale, error, capacity);
 }
 extern "C" int mynah_hip_clip_dev(void *opaque, float *d, size_t n, char *error, size_t capacity) {
     if (d == nullptr) { set_error(error, capacity, "invalid clip arguments"); return -1; }
-    return launch_clip(static_cast<State *>(opaque), d, n, error, capacity);
+    return launch_clip(enter_state(opaque), d, n, error, capacity);
 }
 extern "C" int mynah_hip_argmax_dev(void *opaque, const float *dlogits, size_t vocab, size_t codebook_size, size_t eos_id,
                                     int allow_eos, unsigned *argmax, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (st == nullptr || dlogits == nullptr || argmax == nullptr || vocab == 0 || codebook_size > vocab || eos_id > 0xffffffffu ||
         vocab > 0x7fffffffu) {   // src/backend.c:829-830
         set_error(error, capacity, "invalid argmax arguments");
@@ -605,7 +737,7 @@ extern "C" int mynah_hip_self_attention_dev(void *opaque, const float *dqkv, flo
                                             float *dout, char *error, size_t capacity) {
     const float *q[1] = {dqkv};
     float *k[1] = {dk}, *v[1] = {dv}, *o[1] = {dout};
-    return attention_table(static_cast<State *>(opaque), 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width,
+    return attention_table(enter_state(opaque), 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width,
                            scale, o, error, capacity);
 }
 extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, const float *dk, const float *dv, size_t valid,
@@ -613,13 +745,13 @@ extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, cons
                                              char *error, size_t capacity) {
     const float *q[1] = {dq};
     float *k[1] = {const_cast<float *>(dk)}, *v[1] = {const_cast<float *>(dv)}, *o[1] = {dout};
-    return attention_table(static_cast<State *>(opaque), 0, q, k, v, nullptr, &valid, cache_stride, 1, heads, head_width,
+    return attention_table(enter_state(opaque), 0, q, k, v, nullptr, &valid, cache_stride, 1, heads, head_width,
                            scale, o, error, capacity);
 }
 
 // =========================================================================================== section 2
 extern "C" int mynah_hip_set_quant(void *opaque, int qtype, int arith, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
     if (qtype < MYNAH_HIP_F32 || qtype > MYNAH_HIP_F16 || arith < 0 || arith > 1) {
         set_error(error, capacity, "unknown quantisation mode");
@@ -632,7 +764,7 @@ extern "C" int mynah_hip_set_quant(void *opaque, int qtype, int arith, char *err
 
 extern "C" int mynah_hip_matmul_d2d_batched(void *opaque, const float *const *din, float *const *dout, size_t batch, size_t iw,
                                             size_t ow, const float *weight, const float *bias, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (batch == 0) return 0;   // src/qmat.c:826
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "batch exceeds MYNAH_MAX_BATCH");
@@ -650,7 +782,7 @@ extern "C" int mynah_hip_matmul_d2d_batched(void *opaque, const float *const *di
 extern "C" int mynah_hip_matmul_d2d_probe(void *opaque, const float *din, float *dout, size_t iw, size_t ow,
                                           const float *weight, const float *bias, int8_t *dqx, float *dsx, int32_t *dacc,
                                           char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (check_rows(din, dout, 1, iw, ow, weight, error, capacity) != 0) return -1;
     const float *in[1] = {din};
     float *out[1] = {dout};
@@ -665,7 +797,7 @@ extern "C" int mynah_hip_self_attention_dev_batched(void *opaque, const float *c
         set_error(error, capacity, "attention: null buffer");
         return -1;
     }
-    return attention_table(static_cast<State *>(opaque), 1, dqkv, dk, dv, position, valid, cache_stride, batch, heads,
+    return attention_table(enter_state(opaque), 1, dqkv, dk, dv, position, valid, cache_stride, batch, heads,
                            head_width, scale, dout, error, capacity);
 }
 extern "C" int mynah_hip_cross_attention_dev_batched(void *opaque, const float *const *dq, const float *const *dk,
@@ -681,14 +813,14 @@ extern "C" int mynah_hip_cross_attention_dev_batched(void *opaque, const float *
         k[b] = const_cast<float *>(dk[b]);
         v[b] = const_cast<float *>(dv[b]);
     }
-    return attention_table(static_cast<State *>(opaque), 0, dq, k, v, nullptr, valid, cache_stride, batch, heads, head_width,
+    return attention_table(enter_state(opaque), 0, dq, k, v, nullptr, valid, cache_stride, batch, heads, head_width,
                            scale, dout, error, capacity);
 }
 
 extern "C" int mynah_hip_embed_gather(void *opaque, const float *const *tables, const size_t *table_rows, size_t table_count,
                                       const int32_t *ids, size_t tokens, size_t width, float scale, const float *position,
                                       size_t position_offset, float *dout, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (tables == nullptr || table_rows == nullptr || ids == nullptr || dout == nullptr || table_count == 0 || table_count > 32 ||
         width == 0 || width > 0x7fffffffu) {
         set_error(error, capacity, "invalid gather arguments");
@@ -723,7 +855,7 @@ extern "C" int mynah_hip_embed_gather(void *opaque, const float *const *tables, 
 extern "C" int mynah_hip_output_head(void *opaque, const float *const *dhidden, size_t batch, size_t width, const float *weight,
                                      const float *bias, size_t rows, size_t vocab, float *const *dlogits,
                                      float *const *dprobs, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (batch == 0) return 0;
     if (batch > (size_t)kMaxBatch || dhidden == nullptr || dlogits == nullptr || vocab == 0 || rows % vocab != 0) {
         set_error(error, capacity, "invalid output head arguments");
@@ -751,12 +883,12 @@ __global__ void __launch_bounds__(256) k_flush(uint4 *p, size_t n16) {
 }
 
 extern "C" int mynah_hip_timer_begin(void *opaque, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
     return hip_check(hipEventRecord(st->ev0, st->stream), "event record", error, capacity);
 }
 extern "C" int mynah_hip_timer_end(void *opaque, float *ms, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (st == nullptr || ms == nullptr) {
         set_error(error, capacity, "invalid timer arguments");
         return -1;
@@ -767,7 +899,7 @@ extern "C" int mynah_hip_timer_end(void *opaque, float *ms, char *error, size_t 
     return 0;
 }
 extern "C" int mynah_hip_flush_cache(void *opaque, size_t bytes, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
     if (bytes < (1u << 20)) bytes = 1u << 20;
     if (st->flush_bytes < bytes) {
@@ -785,7 +917,7 @@ extern "C" int mynah_hip_flush_cache(void *opaque, size_t bytes, char *error, si
     return hip_check(hipGetLastError(), "flush launch", error, capacity);
 }
 extern "C" int mynah_hip_set_graph_mode(void *opaque, int enabled, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
     st->graph_mode = enabled ? 1 : 0;
     return 0;

@@ -410,7 +410,7 @@ int launch_conv_split(State *st, const ConvArgs &a, char *error, size_t capacity
 
 extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
                                 int kernel, int dilation, const float *weight, const float *bias, char *error, size_t capacity) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (st == nullptr || dev_input == nullptr || dev_output == nullptr || weight == nullptr || in_channels <= 0 || out_channels <= 0 ||
         length <= 0 || kernel <= 0 || dilation <= 0) {
         set_error(error, capacity, "invalid conv1d arguments");   // the checks of metal_ops_conv1d, gpu/metal/backend_metal_ops.m:371-372
@@ -443,7 +443,7 @@ extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_
 extern "C" int mynah_hip_conv_transpose_dev(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels,
                                             int length, int output_length, int kernel, int stride, int groups, const float *weight,
                                             const float *bias, char *error, size_t capacity) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (st == nullptr || dev_input == nullptr || dev_output == nullptr || weight == nullptr || in_channels <= 0 || out_channels <= 0 ||
         length <= 0 || output_length <= 0 || kernel <= 0 || stride <= 0 || groups <= 0 || in_channels % groups != 0 ||
         out_channels % groups != 0) {
@@ -472,7 +472,7 @@ extern "C" int mynah_hip_conv_transpose_dev(void *state, const float *dev_input,
 
 extern "C" int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length, size_t snake_channels,
                                    char *error, size_t capacity) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (st == nullptr || dev_data == nullptr || channels > (size_t)INT_MAX || length > (size_t)INT_MAX || snake_channels > channels ||
         (snake_channels != 0 && alpha == nullptr)) {
         set_error(error, capacity, "invalid snake arguments");   // metal_ops_snake, gpu/metal/backend_metal_ops.m:343-346

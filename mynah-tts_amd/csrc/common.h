@@ -73,6 +73,23 @@ struct StepSlots {
     int memory_length[kMaxBatch];
 };
 
+// A seam call held back for one call so that the next one can join its launch (backend_hip.hip, "seam fusion").
+struct PendingOp {
+    enum { kNone = 0, kLayerNorm = 1, kLinear = 2 };
+    int kind = kNone;
+    // LayerNorm of one row (alone, or as the prologue of the product)
+    const float *ln_in = nullptr;
+    float *ln_out = nullptr;
+    const float *ln_gain = nullptr, *ln_bias = nullptr;   // device copies
+    // product of one row
+    bool has_ln = false;
+    const float *in = nullptr;
+    float *out = nullptr;
+    size_t iw = 0, ow = 0;
+    const CachedWeight *weight = nullptr;
+    const float *bias = nullptr;                           // device copy
+};
+
 struct State {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -100,7 +117,16 @@ struct State {
     void *ptr_table_host = nullptr;   // pinned
     // result word of the argmax operator: its own allocation, so that it can never alias a caller's upload buffer
     unsigned *argmax_result = nullptr;
+    // seam fusion: the held-back call, whether holding back is on (MYNAH_HIP_FUSE=0 turns it off), and the message of a
+    // held-back launch that failed where no caller could be told (reported by the next sync)
+    PendingOp pending;
+    int fuse = 1;
+    char deferred_error[160] = {0};
 };
+
+// First statement of every entry point that is not itself part of the seam fusion: launches what is held back, so that
+// the stream holds every earlier call's work before this one adds its own.
+State *enter_state(void *opaque);
 
 // weight cache (backend_hip.hip)
 int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qtype, const CachedWeight **out,

@@ -212,7 +212,7 @@ static int per_layer_vector(State *st, const float *const *arr, size_t layer, si
 using namespace mynah;
 
 extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (d == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
     for (auto &g : d->graphs)
@@ -229,7 +229,7 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
 
 extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_desc *desc, mynah_hip_decoder **out, char *error,
                                         size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (out != nullptr) *out = nullptr;
     if (st == nullptr || desc == nullptr || out == nullptr || desc->layers == 0 || desc->layers > 4096 || desc->width == 0 || desc->heads == 0 ||
         desc->heads * desc->head_width != desc->width || desc->ffn_width == 0 || desc->capacity == 0 ||
@@ -325,7 +325,7 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
 
 extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch,
                                       char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (batch == 0) return 0;   // src/graph.c:3132
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "decoder batch exceeds MYNAH_MAX_BATCH");   // src/graph.c:3133-3136
@@ -392,7 +392,7 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
 // step's own setting (dependent graph nodes, weights and caches coming from HBM).  It perturbs the decoder's
 // workspaces (x, hidden) like a step does and is not part of the decode path.
 extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *d, size_t batch, int stage, char *error, size_t capacity) {
-    State *st = static_cast<State *>(opaque);
+    State *st = enter_state(opaque);
     if (st == nullptr || d == nullptr || batch == 0 || batch > (size_t)kMaxBatch || stage < 0 || stage >= MYNAH_HIP_STAGE_COUNT) {
         set_error(error, capacity, "invalid stage arguments");
         return -1;

@@ -360,6 +360,7 @@ struct PrologueParams {
     int arith;
     int8_t *probe_qx;       // parity probes for stream 0 (written by workgroup 0 only)
     float *probe_sx;
+    float *ln_out = nullptr;   // non-null: workgroup 0 also stores stream 0's LayerNorm row here
 };
 
 // Who stages which streams.  A team is four wavefronts acting as the 256 threads tid = 0..255 of the staging scheme
@@ -454,6 +455,8 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, cons
                     y.x += bv[i].x; y.y += bv[i].y; y.z += bv[i].z; y.w += bv[i].w;
                 }
                 xr[b][i] = y;   // lanes beyond the row hold gain 0 -> 0
+                if (p.ln_out != nullptr && blockIdx.x == 0 && team.stream0 + b == 0 && tid + kThreads * i < nf4)
+                    reinterpret_cast<float4 *>(p.ln_out)[tid + kThreads * i] = y;
             }
         }
     }

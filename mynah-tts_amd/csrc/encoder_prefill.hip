@@ -558,7 +558,7 @@ int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size
 }  // namespace
 
 extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_desc *d, mynah_hip_encoder **out, char *error, size_t capacity) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (out != nullptr) *out = nullptr;
     if (st == nullptr || d == nullptr || out == nullptr) {
         set_error(error, capacity, "encoder_create: null argument");
@@ -646,7 +646,7 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
 }
 
 extern "C" void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *e) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (e == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
     for (auto &g : e->graphs)
@@ -659,7 +659,7 @@ extern "C" void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *e) {
 
 extern "C" int mynah_hip_encoder_prefill(void *state, mynah_hip_encoder *e, const int32_t *ids, size_t tokens, uint16_t *dev_embed_f16,
                                          float *dev_out, char *error, size_t capacity) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (st == nullptr || e == nullptr || ids == nullptr || dev_out == nullptr) {
         set_error(error, capacity, "encoder_prefill: null argument");
         return -1;

@@ -30,6 +30,10 @@ struct LinearArgs {
     int8_t *probe_qx;       // parity probes (null in production)
     float *probe_sx;
     int32_t *probe_acc;
+    // Seam calls folded into one launch (single row only): ln_out receives the LayerNorm prologue's row, aux_out the
+    // value of the product before the residual epilogue adds it -- the buffers the separate calls would have written.
+    float *ln_out;
+    float *aux_out;
 };
 
 // True when the fused matvec kernel supports this shape/storage; otherwise use linear_generic.

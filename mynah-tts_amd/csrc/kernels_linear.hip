@@ -73,6 +73,7 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
     int8_t *const arg_probe_qx = SPEC != SPEC_ANY ? nullptr : a.probe_qx;
     float *const arg_probe_sx = SPEC != SPEC_ANY ? nullptr : a.probe_sx;
     int32_t *const arg_probe_acc = SPEC != SPEC_ANY ? nullptr : a.probe_acc;
+    float *const arg_aux_out = SPEC != SPEC_ANY ? nullptr : a.aux_out;
     const int arg_epilogue = SPEC == SPEC_UP ? EPI_GELU : SPEC == SPEC_RESIDUAL ? EPI_RESIDUAL : a.epilogue;
     const float *const arg_ln_gain = SPEC == SPEC_RESIDUAL ? nullptr : a.ln_gain;
     const float *const arg_ln_bias = SPEC == SPEC_RESIDUAL ? nullptr : a.ln_bias;
@@ -101,6 +102,7 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
     PrologueParams pro;
     pro.k = k; pro.batch = a.batch; pro.ln_gain = arg_ln_gain; pro.ln_bias = arg_ln_bias; pro.arith = a.arith;
     pro.probe_qx = arg_probe_qx; pro.probe_sx = arg_probe_sx;
+    pro.ln_out = SPEC != SPEC_ANY ? nullptr : a.ln_out;
     float4 xr[SB][NVT], gv[NVT], bv[NVT];
     {
         ActSource src;
@@ -208,6 +210,7 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
                 if (arg_bias != nullptr) val += bias;
                 if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
                 float *o = stream_out<BT>(a, gl) + row;
+                if (arg_aux_out != nullptr && gl == 0) arg_aux_out[row] = val;
                 if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : *o) + val;
                 *o = val;
             }
@@ -228,6 +231,7 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
                     if (arg_bias != nullptr) val += bias;
                     if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
                     float *o = a.out[b] + row;
+                    if (arg_aux_out != nullptr && b == 0) arg_aux_out[row] = val;
                     if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[b] : *o) + val;
                     *o = val;
                 }
@@ -311,7 +315,8 @@ int launch_linear_b(State *st, const LinearArgs &a, char *error, size_t capacity
 template <int QT>
 int launch_linear_q(State *st, const LinearArgs &a, char *error, size_t capacity) {
     // what the arguments rule out decides the build (see SPEC above)
-    const bool plain = a.bias == nullptr && a.probe_qx == nullptr && a.probe_sx == nullptr && a.probe_acc == nullptr;
+    const bool plain = a.bias == nullptr && a.probe_qx == nullptr && a.probe_sx == nullptr && a.probe_acc == nullptr &&
+                       a.ln_out == nullptr && a.aux_out == nullptr;
     const bool residual = plain && a.epilogue == EPI_RESIDUAL && a.ln_gain == nullptr;
     const bool up = plain && a.epilogue == EPI_GELU && a.ln_gain != nullptr && a.fold_partial == nullptr;
     if (a.k == 768) {

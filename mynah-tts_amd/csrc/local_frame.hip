@@ -405,7 +405,7 @@ static int enqueue_frame(State *st, mynah_hip_local *l, int B, char *error, size
 }
 
 extern "C" void mynah_hip_local_destroy(void *state, mynah_hip_local *l) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (l == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
     for (auto &g : l->graphs)
@@ -420,7 +420,7 @@ extern "C" void mynah_hip_local_destroy(void *state, mynah_hip_local *l) {
 
 extern "C" int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc *stack, const mynah_hip_local_desc *desc,
                                       mynah_hip_local **out, char *error, size_t capacity) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (out != nullptr) *out = nullptr;
     if (st == nullptr || stack == nullptr || desc == nullptr || out == nullptr) {
         set_error(error, capacity, "local_create: null argument");
@@ -490,7 +490,7 @@ extern "C" int mynah_hip_local_create(void *state, const mynah_hip_decoder_desc 
 extern "C" int mynah_hip_local_frame(void *state, mynah_hip_local *l, mynah_hip_local_item *items, size_t batch, unsigned *values,
                                      unsigned *stored, int *saw_eos, size_t *eos_frame, float *dev_logits_copy, char *error,
                                      size_t capacity) {
-    State *st = static_cast<State *>(state);
+    State *st = enter_state(state);
     if (batch == 0) return 0;   // src/graph.c:1378
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "local frame batch exceeds MYNAH_MAX_BATCH");   // src/graph.c:1379-1382

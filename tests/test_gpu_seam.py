@@ -367,3 +367,88 @@ def test_embedding_gather_bit_exact(backend):
     with pytest.raises(Exception):
         backend.embed_gather([table], np.array([4096], np.int32), 768, 1.0, None, 0, dout.ptr)   # out of vocabulary
     dout.free()
+
+
+@pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4", "f16"])
+def test_fused_seam_chains_match_separate_launches(backend, pkg, nerr, qtype_name):
+    """Consecutive single-row seam calls that continue on each other's buffers run as one launch (LayerNorm + product
+    (+ GELU), product + GELU, product + residual).  Every buffer the separate calls write must hold what they would have
+    written: a synchronisation between two calls keeps them apart, which gives the reference values.  The product's own
+    arithmetic is the same kernel code in both cases: bit-identical; the LayerNorm row comes from the matvec's prologue
+    instead of the stand-alone kernel (other reduction tree): 1e-6 normalised, and what is computed from it 1e-5 (f32,
+    f16) or, with quantised activations, within one quantisation step of a weight row's reach (2e-2)."""
+    _announce("fused seam chains " + qtype_name)
+    qt = {"f32": pkg.F32, "int8": pkg.INT8, "int4": pkg.INT4, "f16": pkg.F16}[qtype_name]
+    tol = {"f32": 1e-5, "f16": 1e-5, "int8": 2e-2, "int4": 2e-2}[qtype_name]
+    backend.set_quant(qt)
+    rng = np.random.default_rng(77)
+    w, f = 768, 3072
+    gain = backend.keep((1 + 0.1 * rng.standard_normal(w)).astype(np.float32))
+    up = backend.keep((0.02 * rng.standard_normal((f, w))).astype(np.float32))
+    down = backend.keep((0.02 * rng.standard_normal((w, f))).astype(np.float32))
+    x0 = rng.standard_normal(w).astype(np.float32)
+    bufs = {n: backend.alloc(s) for n, s in (("x", w), ("nrm", w), ("hidden", f), ("proj", w))}
+
+    def run(separate):
+        gap = backend.sync if separate else (lambda: None)
+        bufs["x"].write(x0)
+        for b in ("nrm", "hidden", "proj"):
+            bufs[b].write(np.zeros(bufs[b].n, np.float32))
+        # the engine's feed-forward block (src/graph.c:3451-3476)
+        backend.layer_norm_inplace(bufs["x"].ptr, bufs["nrm"].ptr, gain, 1, w)
+        gap()
+        backend.matmul_d2d(bufs["nrm"].ptr, bufs["hidden"].ptr, 1, w, f, up)
+        gap()
+        backend.gelu_inplace(bufs["hidden"].ptr, f)
+        gap()
+        backend.matmul_d2d(bufs["hidden"].ptr, bufs["proj"].ptr, 1, f, w, down)
+        gap()
+        backend.residual_inplace(bufs["x"].ptr, bufs["proj"].ptr, w)
+        return {n: bufs[n].read() for n in bufs}
+
+    want = run(True)
+    got = run(False)
+    assert nerr(got["nrm"], want["nrm"]) < 1e-6
+    assert nerr(got["hidden"], want["hidden"]) < tol
+    assert nerr(got["proj"], want["proj"]) < tol
+    assert nerr(got["x"], want["x"]) < tol
+    assert np.array_equal(got["x"], x0 + got["proj"]), "residual row and product row disagree"
+
+    # product + GELU and product + residual on rows that are the same in both runs: bit-identical
+    h0 = rng.standard_normal(f).astype(np.float32)
+
+    def tail(separate):
+        gap = backend.sync if separate else (lambda: None)
+        bufs["x"].write(x0)
+        bufs["hidden"].write(h0)
+        backend.matmul_d2d(bufs["hidden"].ptr, bufs["proj"].ptr, 1, f, w, down)
+        gap()
+        backend.residual_inplace(bufs["x"].ptr, bufs["proj"].ptr, w)
+        backend.matmul_d2d(bufs["x"].ptr, bufs["hidden"].ptr, 1, w, f, up)
+        gap()
+        backend.gelu_inplace(bufs["hidden"].ptr, f)
+        return {n: bufs[n].read() for n in ("x", "proj", "hidden")}
+
+    want, got = tail(True), tail(False)
+    for n in want:
+        assert np.array_equal(got[n], want[n]), n
+
+    # chains that must NOT join: the residual add updates the row the product reads
+    def aliased(separate):
+        gap = backend.sync if separate else (lambda: None)
+        bufs["x"].write(x0)
+        backend.matmul_d2d(bufs["x"].ptr, bufs["proj"].ptr, 1, w, w, backend.keep(np.ascontiguousarray(down[:, :w])))
+        gap()
+        backend.residual_inplace(bufs["x"].ptr, bufs["proj"].ptr, w)
+        # a LayerNorm whose row nobody multiplies, then an unrelated call
+        backend.layer_norm_inplace(bufs["x"].ptr, bufs["nrm"].ptr, gain, 1, w)
+        gap()
+        backend.scale_dev(bufs["nrm"].ptr, w, 0.5)
+        return {n: bufs[n].read() for n in ("x", "proj", "nrm")}
+
+    want, got = aliased(True), aliased(False)
+    for n in want:
+        assert np.array_equal(got[n], want[n]), n
+    for b in bufs.values():
+        b.free()
+    backend.set_quant(pkg.F32)
