@@ -77,9 +77,9 @@ static int device_copy_of(const void *host, size_t bytes, void **dev, char *erro
 }
 
 int ensure_attention_workspace(State *st, size_t batch, size_t heads, size_t head_width, size_t max_valid,
-                               char *error, size_t capacity) {
-    const size_t chunks = (max_valid + kAttnChunk - 1) / kAttnChunk + 1;
-    const size_t need = batch * heads * chunks * (head_width + 2);
+                               char *error, size_t capacity, size_t chunk_rows) {
+    const size_t chunks = (max_valid + chunk_rows - 1) / chunk_rows + 1;
+    const size_t need = batch * heads * chunks * (head_width + 4);
     if (st->attn_partial_floats < need) {
         if (st->attn_partial != nullptr) {
             MYNAH_TRY(hipStreamSynchronize(st->stream));
@@ -351,7 +351,13 @@ static int attention_table(State *st, int is_self, const float *const *q, float 
         a.valid[b] = (int)valid[b];
         if (valid[b] > max_valid) max_valid = valid[b];
     }
-    if (ensure_attention_workspace(st, batch, heads, hw, max_valid, error, capacity) != 0) return -1;
+    // the vector paths need 16-byte aligned rows everywhere
+    bool aligned = true;
+    for (size_t b = 0; b < batch; ++b)
+        aligned = aligned && ((reinterpret_cast<uintptr_t>(q[b]) | reinterpret_cast<uintptr_t>(kc[b]) |
+                               reinterpret_cast<uintptr_t>(vc[b]) | reinterpret_cast<uintptr_t>(out[b])) & 15u) == 0;
+    const size_t chunk_rows = (size_t)attention_chunk_rows(is_self, hw, aligned && hw % 4 == 0 && stride % 4 == 0, max_valid);
+    if (ensure_attention_workspace(st, batch, heads, hw, max_valid, error, capacity, chunk_rows) != 0) return -1;
     a.slots = nullptr;
     a.batch = (int)batch;
     a.heads = (int)heads;
@@ -360,14 +366,10 @@ static int attention_table(State *st, int is_self, const float *const *q, float 
     a.q_stride = 0;
     a.scale = scale;
     a.is_self = is_self;
-    a.max_chunks = (int)((max_valid + kAttnChunk - 1) / kAttnChunk);
+    a.chunk_rows = (int)chunk_rows;
+    a.max_chunks = (int)((max_valid + chunk_rows - 1) / chunk_rows);
     a.partial = st->attn_partial;
     a.counters = st->attn_counters;
-    // the vector path needs 16-byte aligned rows everywhere
-    bool aligned = true;
-    for (size_t b = 0; b < batch; ++b)
-        aligned = aligned && ((reinterpret_cast<uintptr_t>(q[b]) | reinterpret_cast<uintptr_t>(kc[b]) |
-                               reinterpret_cast<uintptr_t>(vc[b]) | reinterpret_cast<uintptr_t>(out[b])) & 15u) == 0;
     if (!aligned) a.q_stride = 1;   // any value that is not a multiple of 4 selects the scalar path
     return launch_attention(st, a, error, capacity);
 }

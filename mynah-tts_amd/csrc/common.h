@@ -19,6 +19,7 @@ constexpr int kMaxBatch = MYNAH_HIP_MAX_BATCH;
 constexpr int kBatchTile = 8;        // streams served by one pass over a weight tile
 constexpr size_t kQuantMaxRows = 16; // QMAT_SMALL_COUNT, src/qmat.c:32
 constexpr size_t kQuantMaxK = 8192;  // QMAT_K_MAX, src/qmat.c:33
+constexpr int kWideRows = 16;        // the same for their wide-head form (one wavefront per row)
 constexpr int kAttnChunk = 64;       // cache positions handled by one workgroup of the stand-alone attention kernels
 constexpr int kStepUnitRows = 128;   // cache rows per attention unit (workgroup) of the fused resident step
 // Up to this many streams the resident step is laid out for latency: the output projection folds the attention
@@ -133,7 +134,7 @@ int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qty
                   char *error, size_t capacity);
 int cached_vector(State *st, const float *host, size_t n, const float **dev, char *error, size_t capacity);
 int ensure_attention_workspace(State *st, size_t batch, size_t heads, size_t head_width, size_t max_valid,
-                               char *error, size_t capacity);
+                               char *error, size_t capacity, size_t chunk_rows = kAttnChunk);
 int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity);
 
 // host quantisers (quantize_host.cpp)

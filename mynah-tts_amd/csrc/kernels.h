@@ -64,10 +64,12 @@ struct AttnArgs {
     float scale;
     int is_self;
     int max_chunks;                // grid.x
+    int chunk_rows;                // cache rows per workgroup: 0 / kAttnChunk, or kWideRows (from attention_chunk_rows)
     float *partial;                // [batch, heads, max_chunks, head_width + 2]
     unsigned *counters;            // [batch, heads], zero between launches
 };
 int launch_attention(State *st, const AttnArgs &args, char *error, size_t capacity);
+int attention_chunk_rows(int is_self, size_t head_width, bool vector_rows, size_t max_valid);
 
 // Resident step: LayerNorm + activation quantisation + this head's slice of the Q (self: Q, K, V) projection +
 // attention over one cache chunk, per workgroup; writes split-L partials that the next matvec folds.

@@ -339,7 +339,165 @@ __global__ void __launch_bounds__(kThreads) k_attention_any(const AttnArgs a) {
     publish_and_fold(a, b, head, chunk, nchunks, hw, s_red, m_c, l_c, outh, s_w, s_fold, &s_last);
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Wide heads (head_width = 256 * NV; the engine's cross attention is ONE head as wide as the model,
+// src/graph.c:3443-3448), read-only caches.  With one head there are only valid / 64 workgroups of
+// the kernel above, each walking 64 rows of 3 KB through a dozen dependent round trips.  Here a
+// workgroup takes kWideRows rows, a wavefront takes a whole row per pass (lane l holds the float4 at
+// columns 4 l + 256 i), and every row the workgroup will touch is requested before anything is used.
+// Partial layout per chunk: out[hw], max, sum, 2 floats of padding (rows stay 16-byte aligned).
+template <int NV>
+__global__ void __launch_bounds__(kThreads) k_attention_wide(const AttnArgs a) {
+    extern __shared__ __align__(16) float lds[];
+    constexpr int hw = 256 * NV;
+    constexpr int kPasses = kWideRows / 4;
+    float *s_score = lds;                    // [64]
+    float *s_red = s_score + kAttnChunk;     // [4][hw]
+    float *s_w = s_red + 4 * hw;             // [2 * max_chunks]
+    __shared__ float s_ml[2];
+    __shared__ int s_last;
+
+    const int chunk = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const Resolved r = resolve(a, b);
+    const int nchunks = r.valid > 0 ? (r.valid + kWideRows - 1) / kWideRows : 1;
+    if (chunk >= nchunks) return;
+    float *outh = r.out + (size_t)head * hw;
+    if (r.valid <= 0) {   // empty memory: the context stays zero (src/graph.c:3242)
+        for (int d = tid; d < hw; d += kThreads) outh[d] = 0.0f;
+        return;
+    }
+    const int p0 = chunk * kWideRows;
+    const int count = min(kWideRows, r.valid - p0);
+    const size_t col = (size_t)head * hw + 4 * lane;
+
+    // ---- every request first, from a row index clamped into the chunk (rows past its end get the weight 0)
+    float4 qv[NV], kv[kPasses][NV], vv[kPasses][NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) qv[i] = *reinterpret_cast<const float4 *>(r.q + col + 256 * i);
+#pragma unroll
+    for (int rr = 0; rr < kPasses; ++rr) {
+        const int p = p0 + min(wave + 4 * rr, count - 1);
+        const float *krow = r.kc + (size_t)p * a.stride + col;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) kv[rr][i] = *reinterpret_cast<const float4 *>(krow + 256 * i);
+    }
+#pragma unroll
+    for (int rr = 0; rr < kPasses; ++rr) {
+        const int p = p0 + min(wave + 4 * rr, count - 1);
+        const float *vrow = r.vc + (size_t)p * a.stride + col;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) vv[rr][i] = *reinterpret_cast<const float4 *>(vrow + 256 * i);
+    }
+    if (tid >= kWideRows && tid < kAttnChunk) s_score[tid] = -3.0e38f;
+#pragma unroll
+    for (int rr = 0; rr < kPasses; ++rr) {
+        const int pi = wave + 4 * rr;
+        float dot = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            dot = __builtin_fmaf(qv[i].x, kv[rr][i].x, dot);
+            dot = __builtin_fmaf(qv[i].y, kv[rr][i].y, dot);
+            dot = __builtin_fmaf(qv[i].z, kv[rr][i].z, dot);
+            dot = __builtin_fmaf(qv[i].w, kv[rr][i].w, dot);
+        }
+        dot = wave_sum(dot);
+        if (lane == 0) s_score[pi] = pi < count ? dot * a.scale : -3.0e38f;
+    }
+    __syncthreads();
+    chunk_stats(s_score, s_ml, count);
+    __syncthreads();
+    float4 acc[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int rr = 0; rr < kPasses; ++rr) {
+        const float e = s_score[wave + 4 * rr];   // 0 beyond `count`
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            acc[i].x = __builtin_fmaf(e, vv[rr][i].x, acc[i].x);
+            acc[i].y = __builtin_fmaf(e, vv[rr][i].y, acc[i].y);
+            acc[i].z = __builtin_fmaf(e, vv[rr][i].z, acc[i].z);
+            acc[i].w = __builtin_fmaf(e, vv[rr][i].w, acc[i].w);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) *reinterpret_cast<float4 *>(s_red + (size_t)wave * hw + 4 * lane + 256 * i) = acc[i];
+    __syncthreads();
+    const float m_c = s_ml[0], l_c = s_ml[1];
+    // the four wavefronts' sums, in order; thread t owns the float4 column t
+    const bool owner = tid < hw / 4;
+    float4 mine = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (owner) {
+        mine = *reinterpret_cast<const float4 *>(s_red + 4 * tid);
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const float4 o = *reinterpret_cast<const float4 *>(s_red + (size_t)w * hw + 4 * tid);
+            mine.x += o.x; mine.y += o.y; mine.z += o.z; mine.w += o.w;
+        }
+    }
+    if (nchunks == 1) {
+        if (owner) *reinterpret_cast<float4 *>(outh + 4 * tid) = make_float4(mine.x / l_c, mine.y / l_c, mine.z / l_c, mine.w / l_c);
+        return;
+    }
+    constexpr size_t pstride = hw + 4;
+    float *part = a.partial + (((size_t)b * a.heads + head) * a.max_chunks) * pstride;
+    float *slot = part + (size_t)chunk * pstride;
+    if (owner) *reinterpret_cast<float4 *>(slot + 4 * tid) = mine;
+    if (tid == 0) { slot[hw] = m_c; slot[hw + 1] = l_c; }
+    __syncthreads();   // the workgroup's stores are in the L2 ...
+    if (tid == 0) {
+        __threadfence();   // ... and one device-scope release publishes them
+        unsigned *counter = a.counters + (size_t)b * a.heads + head;
+        const unsigned before = atomicAdd(counter, 1u);
+        const int last = (before == (unsigned)(nchunks - 1)) ? 1 : 0;
+        if (last) *counter = 0u;   // every other chunk has arrived: ready for the next launch
+        s_last = last;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();   // acquire
+
+    // fold, chunks in index order: out = sum_c o_c e^(m_c - M) / sum_c l_c e^(m_c - M)
+    for (int c = tid; c < nchunks; c += kThreads) {
+        s_w[c] = part[(size_t)c * pstride + hw];
+        s_w[a.max_chunks + c] = part[(size_t)c * pstride + hw + 1];
+    }
+    __syncthreads();
+    float M = -3.0e38f;
+    for (int c = 0; c < nchunks; ++c) M = fmaxf(M, s_w[c]);
+    __syncthreads();
+    for (int c = tid; c < nchunks; c += kThreads) s_w[c] = expf(s_w[c] - M);
+    __syncthreads();
+    float L = 0.0f;
+    for (int c = 0; c < nchunks; ++c) L = __builtin_fmaf(s_w[a.max_chunks + c], s_w[c], L);
+    if (!owner) return;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int c0 = 0; c0 < nchunks; c0 += 8) {
+        float4 pv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) pv[u] = *reinterpret_cast<const float4 *>(part + (size_t)min(c0 + u, nchunks - 1) * pstride + 4 * tid);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float w = c0 + u < nchunks ? s_w[min(c0 + u, nchunks - 1)] : 0.0f;
+            o.x = __builtin_fmaf(pv[u].x, w, o.x);
+            o.y = __builtin_fmaf(pv[u].y, w, o.y);
+            o.z = __builtin_fmaf(pv[u].z, w, o.z);
+            o.w = __builtin_fmaf(pv[u].w, w, o.w);
+        }
+    }
+    *reinterpret_cast<float4 *>(outh + 4 * tid) = make_float4(o.x / L, o.y / L, o.z / L, o.w / L);
+}
+
 }  // namespace
+
+// Rows of the cache one workgroup takes for this call: kWideRows when the wide-head kernel applies, else kAttnChunk.
+int attention_chunk_rows(int is_self, size_t head_width, bool vector_rows, size_t max_valid) {
+    const bool wide = !is_self && vector_rows && head_width >= 256 && head_width <= 1024 && head_width % 256 == 0 &&
+                      (max_valid + kWideRows - 1) / kWideRows <= 4096;
+    return wide ? kWideRows : kAttnChunk;
+}
 
 int launch_attention(State *st, const AttnArgs &a, char *error, size_t capacity) {
     if (a.batch < 1 || a.batch > kMaxBatch || a.heads < 1 || a.head_width < 1 || a.head_width > 1024 ||
@@ -349,6 +507,21 @@ int launch_attention(State *st, const AttnArgs &a, char *error, size_t capacity)
     }
     const bool vec = (a.head_width % 4) == 0 && (a.stride % 4) == 0 && (a.q_stride % 4) == 0;
     const bool fast = vec && a.head_width == 64;
+    if (a.chunk_rows == kWideRows) {
+        if (a.chunk_rows != attention_chunk_rows(a.is_self, (size_t)a.head_width, vec, 1)) {
+            set_error(error, capacity, "attention: the wide-head kernel does not take this shape");
+            return -1;
+        }
+        const size_t wide_lds = (kAttnChunk + 4 * (size_t)a.head_width + 2 * (size_t)a.max_chunks) * sizeof(float);
+        const dim3 wide_grid((unsigned)a.max_chunks, (unsigned)a.heads, (unsigned)a.batch);
+        switch (a.head_width / 256) {
+            case 1: hipLaunchKernelGGL(k_attention_wide<1>, wide_grid, dim3(kThreads), wide_lds, st->stream, a); break;
+            case 2: hipLaunchKernelGGL(k_attention_wide<2>, wide_grid, dim3(kThreads), wide_lds, st->stream, a); break;
+            case 3: hipLaunchKernelGGL(k_attention_wide<3>, wide_grid, dim3(kThreads), wide_lds, st->stream, a); break;
+            default: hipLaunchKernelGGL(k_attention_wide<4>, wide_grid, dim3(kThreads), wide_lds, st->stream, a); break;
+        }
+        return hip_check(hipGetLastError(), "attention launch", error, capacity);
+    }
     const size_t hw = (size_t)a.head_width;
     const size_t lds = ((fast ? 0 : hw) + kAttnChunk + (size_t)kPosPerPass * hw + 2 * (size_t)a.max_chunks + kThreads) * sizeof(float);
     const dim3 grid((unsigned)a.max_chunks, (unsigned)a.heads, (unsigned)a.batch);

@@ -273,10 +273,12 @@ def test_argmax(backend, orc):
 
 
 @pytest.mark.parametrize("heads,hw,L", [(12, 64, 1), (12, 64, 63), (12, 64, 64), (12, 64, 65), (12, 64, 300),
-                                        (12, 64, 1024), (1, 768, 200), (3, 20, 70), (1, 2, 5)])
+                                        (12, 64, 1024), (1, 768, 200), (3, 20, 70), (1, 2, 5),
+                                        (1, 768, 16), (1, 768, 17), (1, 768, 256), (1, 256, 100), (2, 512, 33), (1, 1024, 40)])
 def test_self_and_cross_attention(backend, orc, nerr, heads, hw, L):
     """Split-L attention against the reference's two-pass order, incl. chunk edges (63/64/65), one wide head
-    (what the engine passes for cross attention) and head widths that are not multiples of 4."""
+    (what the engine passes for cross attention; its read-only form has a kernel of its own for head widths that are
+    multiples of 256, sixteen rows per workgroup: chunk edges 16/17) and head widths that are not multiples of 4."""
     _announce("attention heads=%d hw=%d L=%d" % (heads, hw, L))
     rng = np.random.default_rng(800 + heads + hw + L)
     width = heads * hw
@@ -452,3 +454,32 @@ def test_fused_seam_chains_match_separate_launches(backend, pkg, nerr, qtype_nam
     for b in bufs.values():
         b.free()
     backend.set_quant(pkg.F32)
+
+
+def test_batched_wide_head_cross_attention_bit_identical_to_solo(backend, orc, nerr):
+    """Ragged memories behind one 768-wide head: each stream in the batch equals the same stream alone, bit for bit, and
+    a stream without memory gets a zero context (src/graph.c:3237-3244)."""
+    _announce("batched wide-head cross attention")
+    rng = np.random.default_rng(901)
+    hw = 768
+    scale = 1.0 / math.sqrt(hw)
+    lens = [256, 1, 40, 0, 17, 133]
+    qs = [rng.standard_normal(hw).astype(np.float32) for _ in lens]
+    ks = [rng.standard_normal((max(n, 1), hw)).astype(np.float32) for n in lens]
+    vs = [rng.standard_normal((max(n, 1), hw)).astype(np.float32) for n in lens]
+    dq = [backend.alloc(hw).write(q) for q in qs]
+    dk = [backend.alloc(k.size).write(k) for k in ks]
+    dv = [backend.alloc(v.size).write(v) for v in vs]
+    do = [backend.alloc(hw) for _ in lens]
+    backend.cross_attention_dev_batched([d.ptr for d in dq], [d.ptr for d in dk], [d.ptr for d in dv], lens, hw, 1, hw, scale,
+                                        [d.ptr for d in do])
+    together = [d.read() for d in do]
+    for b, n in enumerate(lens):
+        if n == 0:
+            assert not together[b].any()
+            continue
+        assert nerr(together[b], orc.cross_attention(qs[b], ks[b], vs[b], n, hw, 1, hw, scale)) < 1e-5
+        backend.cross_attention_dev(dq[b].ptr, dk[b].ptr, dv[b].ptr, n, hw, 1, hw, scale, do[b].ptr)
+        assert np.array_equal(do[b].read(), together[b]), "stream %d" % b
+    for d in dq + dk + dv + do:
+        d.free()
