@@ -274,9 +274,9 @@ def cpu_baseline(steps=CPU_STEPS, warmup=CPU_WARMUP):
     cores in a child process: all online cores, then one thread."""
     out = {}
     cores = os.cpu_count() or 1
-    for label, threads in (("all", cores), ("one", 1)):
-        cmd = [sys.executable, os.path.join(ROOT, "oracle", "cpu_baseline.py"), "--kind", "reference", "--threads", str(threads),
-               "--steps", str(steps), "--warmup", str(warmup)]
+    for label, threads in (("all", cores), ("one", 1), ("engine", 1)):
+        cmd = [sys.executable, os.path.join(ROOT, "oracle", "cpu_baseline.py"), "--kind", "engine" if label == "engine" else "reference",
+               "--threads", str(threads), "--steps", str(steps), "--warmup", str(warmup)]
         try:
             proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=600)
             out[label] = json.loads(proc.stdout.strip().splitlines()[-1])
@@ -387,6 +387,9 @@ def main():
                       "one 768-wide cross head (same bytes and flops) and no output head" % (allc.get("steps", CPU_STEPS), allc.get("warmup", CPU_WARMUP)),
             "one_thread_us": round(cpu.get("one", {}).get("median_us", float("nan")), 1),
             "online_cores": allc.get("online_cores"),
+            # not a CPU figure: the same engine's single-row decoder_run (src/graph.c:3292-3654) with this library as its
+            # backend, through the reference's backend struct -- the per-operator seam, 18 calls per layer
+            "same_engine_on_this_library_us": round(cpu["engine"]["median_us"], 1) if "median_us" in cpu.get("engine", {}) else None,
             "gpu_speedup": round(allc.get("median_us", float("nan")) / b1["step_us"], 1) if "median_us" in allc else None,
         }
     print(json.dumps(result))

@@ -166,20 +166,24 @@ __global__ void __launch_bounds__(kThreads) k_attention_hw64(const AttnArgs a) {
     const int g = tid / kPosLanes;
     const size_t col = (size_t)head * hw + 4 * j;
 
-    // ---- every load this workgroup needs, issued before anything is consumed
-    const float4 qv = *reinterpret_cast<const float4 *>(r.q + col);
+    // ---- every load this workgroup needs, issued before anything is consumed: unconditional global loads from a row
+    // index clamped into the chunk (a request under a condition would make every later wait a wait for all of them);
+    // rows past the chunk's end get the score -3e38 and the weight 0 below
+    const float4 qv = load_global4(r.q + col);
     float4 kv[kRowsPerThread], vv[kRowsPerThread];
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
-        const int pi = g + kPosPerPass * i;
-        const int p = p0 + pi;
-        const bool in_range = pi < count;
-        const bool fresh = in_range && p == r.position;
-        const float *krow = fresh ? r.q + width + col : r.kc + (size_t)p * a.stride + col;
-        const float *vrow = fresh ? r.q + 2 * (size_t)width + col : r.vc + (size_t)p * a.stride + col;
-        kv[i] = in_range ? *reinterpret_cast<const float4 *>(krow) : make_float4(0.f, 0.f, 0.f, 0.f);
-        vv[i] = in_range ? *reinterpret_cast<const float4 *>(vrow) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int p = p0 + min(g + kPosPerPass * i, count - 1);
+        const bool fresh = p == r.position;
+        kv[i] = load_global4(fresh ? r.q + width + col : r.kc + (size_t)p * a.stride + col);
     }
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; ++i) {
+        const int p = p0 + min(g + kPosPerPass * i, count - 1);
+        const bool fresh = p == r.position;
+        vv[i] = load_global4(fresh ? r.q + 2 * (size_t)width + col : r.vc + (size_t)p * a.stride + col);
+    }
+    requests_issued();
     // ---- scores (+ append of the new row)
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
@@ -375,21 +379,22 @@ __global__ void __launch_bounds__(kThreads) k_attention_wide(const AttnArgs a) {
     // ---- every request first, from a row index clamped into the chunk (rows past its end get the weight 0)
     float4 qv[NV], kv[kPasses][NV], vv[kPasses][NV];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) qv[i] = *reinterpret_cast<const float4 *>(r.q + col + 256 * i);
+    for (int i = 0; i < NV; ++i) qv[i] = load_global4(r.q + col + 256 * i);
 #pragma unroll
     for (int rr = 0; rr < kPasses; ++rr) {
         const int p = p0 + min(wave + 4 * rr, count - 1);
         const float *krow = r.kc + (size_t)p * a.stride + col;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) kv[rr][i] = *reinterpret_cast<const float4 *>(krow + 256 * i);
+        for (int i = 0; i < NV; ++i) kv[rr][i] = load_global4(krow + 256 * i);
     }
 #pragma unroll
     for (int rr = 0; rr < kPasses; ++rr) {
         const int p = p0 + min(wave + 4 * rr, count - 1);
         const float *vrow = r.vc + (size_t)p * a.stride + col;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) vv[rr][i] = *reinterpret_cast<const float4 *>(vrow + 256 * i);
+        for (int i = 0; i < NV; ++i) vv[rr][i] = load_global4(vrow + 256 * i);
     }
+    requests_issued();
     if (tid >= kWideRows && tid < kAttnChunk) s_score[tid] = -3.0e38f;
 #pragma unroll
     for (int rr = 0; rr < kPasses; ++rr) {

@@ -8,6 +8,10 @@ process, src/threads.c:36-44, so each thread count needs its own process):
 kind=reference : the reference's own decoder_step_batch (oracle/_ref/libmynah_ref.so, stock flags, its pthread pool)
                  -- gain-only LayerNorm and ONE cross-attention head of width 768, the only form that function has;
                  same weight bytes, KV bytes and flops as the benchmark workload.
+kind=engine    : the same reference engine function one level up (decoder_run, src/graph.c:3292-3654, single row) with the
+                 gfx950 library as its backend through the reference's backend struct (oracle/ref_shim_backend.c): the
+                 resident path, 18 seam calls per layer.  Not a CPU figure: it is what the unmodified engine gets from the
+                 library, reported beside the CPU figure of the same engine.
 kind=port      : this repository's restatement (liboracle.so), single thread, exact benchmark workload.
 Protocol as the reference's own bench (cli/main.c:382-406): warm-ups, then the median of the measured runs.
 Prints one JSON line.
@@ -43,12 +47,30 @@ def main():
     kind = args.kind
     if kind == "reference" and not orc.ref_available():
         kind = "port"
-    cross_heads = 1 if kind == "reference" else 12
-    cfg = synth.decoder_config(layers=args.layers, capacity=args.length + 8, cross_heads=cross_heads)
-    weights = synth.decoder_weights(cfg, seed=0, ln_bias=(kind != "reference"))
+    if kind == "engine" and not orc.ref_available():
+        print(json.dumps({"kind": "engine", "error": "oracle/_ref is not built"}))
+        return
+    cross_heads = 1 if kind in ("reference", "engine") else 12
+    extra = args.steps + args.warmup if kind == "engine" else 0    # the engine run appends a row per step
+    cfg = synth.decoder_config(layers=args.layers, capacity=args.length + 8 + extra, cross_heads=cross_heads)
+    weights = synth.decoder_weights(cfg, seed=0, ln_bias=(kind == "port"))
     length = args.length - 1
     s = synth.decoder_streams(cfg, [length], [args.memory], seed=1)[0]
-    if kind == "reference":
+    if kind == "engine":
+        if args.quant == "f32":
+            os.environ.pop("MYNAH_QUANT", None)
+        else:
+            os.environ["MYNAH_QUANT"] = args.quant
+        os.environ["MYNAH_QUANT_ARITH"] = "stock"
+        dec = orc.RefDecoder(cfg, weights, qtype, 1, args.memory)
+        dec.use_hip(entry.load_package().LIB_PATH)
+        state = {"n": length}
+
+        def run():
+            _, state["n"], resident = dec.run_one(0, s["k"], s["v"], s["ck"], s["cv"], state["n"], args.memory, s["x"])
+            assert resident, "the engine fell back to its CPU path"
+        threads = 1
+    elif kind == "reference":
         dec = orc.RefDecoder(cfg, weights, qtype, 1, args.memory)
         run = lambda: dec.step([s["k"]], [s["v"]], [s["ck"]], [s["cv"]], [length], [args.memory], [s["x"]])
         threads = orc.load_ref().ref_num_threads()
