@@ -64,6 +64,7 @@ struct AttnArgs {
     float scale;
     int is_self;
     int max_chunks;                // grid.x
+    int two_pass;                  // set by launch_attention: the fold is a launch of its own (no arrival counters)
     int chunk_rows;                // cache rows per workgroup: 0 / kAttnChunk, or kWideRows (from attention_chunk_rows)
     float *partial;                // [batch, heads, max_chunks, head_width + 2]
     unsigned *counters;            // [batch, heads], zero between launches

@@ -74,6 +74,9 @@ __device__ __forceinline__ void chunk_stats(float *s_score, float *s_ml, int cou
     }
 }
 
+__device__ __forceinline__ void fold_chunks(const AttnArgs &a, const float *part, int nchunks, int hw, float *outh, float *s_w,
+                                            float *s_fold);
+
 // Publishes this chunk's (max, sum, partial output) and lets the last arrival of the (stream, head)
 // fold all chunks: out = sum_c o_c e^(m_c - M) / sum_c l_c e^(m_c - M), chunks taken in four interleaved
 // sequences (c = g, g+4, ...) that are then added in order g = 0..3 -- fixed, whoever folds.
@@ -91,6 +94,7 @@ __device__ __forceinline__ void publish_and_fold(const AttnArgs &a, int b, int h
         mine[2 + d] = o;
     }
     if (tid == 0) { mine[0] = m_c; mine[1] = l_c; }
+    if (a.two_pass) return;   // a launch of k_attention_fold follows: the kernel boundary publishes the partials
     __syncthreads();   // every store of this workgroup has reached the L2 (workgroup-scope release) ...
     if (tid == 0) {
         __threadfence();   // ... and one device-scope release publishes them: a fence per wave would serialise hundreds of L2 write-backs
@@ -103,7 +107,14 @@ __device__ __forceinline__ void publish_and_fold(const AttnArgs &a, int b, int h
     __syncthreads();
     if (!*s_last) return;
     __threadfence();   // acquire: the partials below are read with ordinary loads
+    fold_chunks(a, part, nchunks, hw, outh, s_w, s_fold);
+}
 
+// out = sum_c o_c e^(m_c - M) / sum_c l_c e^(m_c - M) over the chunks of one (stream, head), in a fixed order.
+__device__ __forceinline__ void fold_chunks(const AttnArgs &a, const float *part, int nchunks, int hw, float *outh, float *s_w,
+                                            float *s_fold) {
+    const int tid = threadIdx.x;
+    const size_t pstride = (size_t)hw + 2;
     // s_w[c] = m_c, s_w[max_chunks + c] = l_c
     for (int c = tid; c < nchunks; c += kThreads) {
         s_w[c] = part[(size_t)c * pstride];
@@ -345,6 +356,23 @@ __global__ void __launch_bounds__(kThreads) k_attention_any(const AttnArgs a) {
 
 
 // ------------------------------------------------------------------------------------------------
+// Second pass of the two-pass form: one workgroup per (stream, head) folds the chunks the first launch left in the
+// workspace.  A device-scope release per workgroup costs about 60 ns of serialised L2 write-back, so with hundreds of
+// chunk workgroups (twelve 64-wide heads over a long cache) two launches are shorter than one with a last-arrival fold.
+__global__ void __launch_bounds__(kThreads) k_attention_fold(const AttnArgs a) {
+    extern __shared__ __align__(16) float lds[];
+    float *s_w = lds;                          // [2 * max_chunks]
+    float *s_fold = s_w + 2 * a.max_chunks;    // [256]
+    const int head = blockIdx.x, b = blockIdx.y;
+    const Resolved r = resolve(a, b);
+    const int nchunks = r.valid > 0 ? (r.valid + kAttnChunk - 1) / kAttnChunk : 1;
+    if (nchunks <= 1) return;   // written by the first pass
+    const int hw = a.head_width;
+    const float *part = a.partial + (((size_t)b * a.heads + head) * a.max_chunks) * ((size_t)hw + 2);
+    fold_chunks(a, part, nchunks, hw, r.out + (size_t)head * hw, s_w, s_fold);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Wide heads (head_width = 256 * NV; the engine's cross attention is ONE head as wide as the model,
 // src/graph.c:3443-3448), read-only caches.  With one head there are only valid / 64 workgroups of
 // the kernel above, each walking 64 rows of 3 KB through a dozen dependent round trips.  Here a
@@ -540,9 +568,17 @@ int launch_attention(State *st, const AttnArgs &a, char *error, size_t capacity)
         set_error(error, capacity, "attention: head width and cache length exceed the workgroup's LDS");
         return -1;
     }
-    if (fast) hipLaunchKernelGGL(k_attention_hw64, grid, dim3(kThreads), lds, st->stream, a);
-    else if (vec) hipLaunchKernelGGL(k_attention_any<true>, grid, dim3(kThreads), lds, st->stream, a);
-    else hipLaunchKernelGGL(k_attention_any<false>, grid, dim3(kThreads), lds, st->stream, a);
+    // many chunk workgroups: fold in a second launch instead of a device-scope release per workgroup
+    AttnArgs args = a;
+    args.two_pass = a.max_chunks > 1 && (size_t)a.max_chunks * a.heads * a.batch >= 64 ? 1 : 0;
+    if (fast) hipLaunchKernelGGL(k_attention_hw64, grid, dim3(kThreads), lds, st->stream, args);
+    else if (vec) hipLaunchKernelGGL(k_attention_any<true>, grid, dim3(kThreads), lds, st->stream, args);
+    else hipLaunchKernelGGL(k_attention_any<false>, grid, dim3(kThreads), lds, st->stream, args);
+    if (args.two_pass) {
+        if (hip_check(hipGetLastError(), "attention launch", error, capacity) != 0) return -1;
+        const size_t fold_lds = (2 * (size_t)a.max_chunks + kThreads) * sizeof(float);
+        hipLaunchKernelGGL(k_attention_fold, dim3((unsigned)a.heads, (unsigned)a.batch), dim3(kThreads), fold_lds, st->stream, args);
+    }
     return hip_check(hipGetLastError(), "attention launch", error, capacity);
 }
 
