@@ -13,6 +13,14 @@
  *   - resident ops enqueue on one internal stream and return without synchronising; only
  *     mynah_hip_sync, mynah_hip_d2h, mynah_hip_download, mynah_hip_argmax_dev and the host-pointer
  *     matmul/sgemm block;
+ *   - a single-row LayerNorm or product (layer_norm_*, matmul_d2d / matmul_dev / matvec_dev with
+ *     rows == 1) may be held back until the next call of this library: when that call continues
+ *     on its buffers (LayerNorm -> product, product -> GELU, product -> residual add, as in
+ *     src/graph.c:3391-3476) the calls run as one launch that writes every buffer the separate
+ *     calls write; any other call first launches what is held back.  Nothing observable through
+ *     this interface changes, except that a held-back launch that fails is reported by the call
+ *     that launches it, or by the next mynah_hip_sync.  MYNAH_HIP_FUSE=0 in the environment at
+ *     open makes every call a launch of its own;
  *   - threads: a state, and every decoder, encoder and local frame created from it, serves one
  *     thread at a time.  Its stream, upload buffer, staging memory and captured graphs are shared
  *     by all its calls without locks, as in the reference's GPU backends, whose state belongs to
