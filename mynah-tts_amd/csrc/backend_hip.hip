@@ -311,6 +311,7 @@ static void hip_close(void *opaque) {
     if (st->flush != nullptr) (void)hipFree(st->flush);
     if (st->attn_partial != nullptr) (void)hipFree(st->attn_partial);
     if (st->attn_counters != nullptr) (void)hipFree(st->attn_counters);
+    if (st->seam_slots != nullptr) (void)hipFree(st->seam_slots);
     if (st->argmax_result != nullptr) (void)hipFree(st->argmax_result);
     if (st->ptr_table != nullptr) (void)hipFree(st->ptr_table);
     if (st->ptr_table_host != nullptr) (void)hipHostFree(st->ptr_table_host);
@@ -322,7 +323,7 @@ static void hip_close(void *opaque) {
 
 static int attention_table(State *st, int is_self, const float *const *q, float *const *kc, float *const *vc,
                            const size_t *position, const size_t *valid, size_t stride, size_t batch, size_t heads,
-                           size_t hw, float scale, float *const *out, char *error, size_t capacity) {
+                           size_t hw, float scale, float *const *out, char *error, size_t capacity, bool hold = false) {
     if (batch == 0) return 0;
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "attention batch exceeds MYNAH_MAX_BATCH");
@@ -371,6 +372,34 @@ static int attention_table(State *st, int is_self, const float *const *q, float 
     a.partial = st->attn_partial;
     a.counters = st->attn_counters;
     if (!aligned) a.q_stride = 1;   // any value that is not a multiple of 4 selects the scalar path
+    // A single-stream seam call over more than one chunk leaves its partials for the product that will read its output
+    // row (seam fusion): the fold becomes that product's prologue instead of a device-scope hand-over or a launch.
+    const bool unit_kernel = aligned && stride % 4 == 0 && (hw == 64 || chunk_rows == (size_t)kWideRows);
+    if (a.max_chunks > 1 && unit_kernel) {
+        // Whatever the batch, the chunks are folded by the one device function (fold_partials), so a stream's bits do not
+        // depend on who called: the batched twin folds in a launch of its own, a single-stream call is held back.
+        if (st->seam_slots == nullptr) {
+            MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->seam_slots), sizeof(StepSlots)));
+            MYNAH_TRY(hipMemsetAsync(st->seam_slots, 0, sizeof(StepSlots), st->stream));
+        }
+        a.unit_partial = st->attn_partial;
+        a.unit_ml = st->attn_partial + batch * heads * (size_t)a.max_chunks * hw;
+        a.unit_slots = st->seam_slots;
+        if (launch_attention(st, a, error, capacity) != 0) return -1;
+        if (!(hold && st->fuse && batch == 1)) return launch_unit_fold_streams(st, a, error, capacity);
+        PendingOp p;
+        p.kind = PendingOp::kAttentionFold;
+        p.has_fold = true;
+        p.fold_out = out[0];
+        p.fold_partial = a.unit_partial;
+        p.fold_ml = a.unit_ml;
+        p.fold_heads = (int)heads;
+        p.fold_head_width = (int)hw;
+        p.fold_max_units = a.max_chunks;
+        p.iw = heads * hw;
+        st->pending = p;
+        return 0;
+    }
     return launch_attention(st, a, error, capacity);
 }
 
@@ -529,6 +558,17 @@ static int launch_pending_linear(State *st, const PendingOp &p, int epilogue, fl
     a.k = (int)p.iw;
     a.batch = 1;
     a.in[0] = p.has_ln ? p.ln_in : p.in;
+    if (p.has_fold) {   // the row is the fold of the attention partials; workgroup 0 also leaves it where the attention call's output goes
+        a.fold_partial = p.fold_partial;
+        a.fold_partial_ml = p.fold_ml;
+        a.fold_slots = st->seam_slots;
+        a.fold_heads = p.fold_heads;
+        a.fold_head_width = p.fold_head_width;
+        a.fold_max_units = p.fold_max_units;
+        a.fold_is_self = 0;
+        a.fold_stream0 = 0;
+        a.act_out = p.fold_out;
+    }
     a.arith = st->arith;
     a.epilogue = epilogue;
     if (p.has_ln) {
@@ -550,6 +590,9 @@ static int seam_flush(State *st, char *error, size_t capacity) {
     st->pending = PendingOp{};
     if (p.kind == PendingOp::kLayerNorm) return launch_layernorm(st, p.ln_in, p.ln_out, p.ln_gain, p.ln_bias, 1, p.iw, error, capacity);
     if (p.kind == PendingOp::kLinear) return launch_pending_linear(st, p, EPI_NONE, nullptr, error, capacity);
+    if (p.kind == PendingOp::kAttentionFold)
+        return launch_unit_fold(st, p.fold_partial, p.fold_ml, st->seam_slots, p.fold_heads, p.fold_head_width, p.fold_max_units, p.fold_out,
+                                error, capacity);
     return 0;
 }
 
@@ -653,7 +696,8 @@ static int seam_matmul(void *opaque, const float *din, float *dout, size_t rows,
             PendingOp p = st->pending;
             const bool joins = p.kind == PendingOp::kLayerNorm && p.ln_out == din && p.iw == iw &&
                                !ranges_overlap(dout, ow, p.ln_in, iw) && !ranges_overlap(dout, ow, p.ln_out, iw);
-            if (!joins) {
+            const bool folds = p.kind == PendingOp::kAttentionFold && p.fold_out == din && p.iw == iw;
+            if (!joins && !folds) {
                 if (seam_flush(st, error, capacity) != 0) return -1;
                 p = PendingOp{};
             }
@@ -740,7 +784,7 @@ extern "C" int mynah_hip_self_attention_dev(void *opaque, const float *dqkv, flo
     const float *q[1] = {dqkv};
     float *k[1] = {dk}, *v[1] = {dv}, *o[1] = {dout};
     return attention_table(enter_state(opaque), 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width,
-                           scale, o, error, capacity);
+                           scale, o, error, capacity, true);
 }
 extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, const float *dk, const float *dv, size_t valid,
                                              size_t cache_stride, size_t heads, size_t head_width, float scale, float *dout,
@@ -748,7 +792,7 @@ extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, cons
     const float *q[1] = {dq};
     float *k[1] = {const_cast<float *>(dk)}, *v[1] = {const_cast<float *>(dv)}, *o[1] = {dout};
     return attention_table(enter_state(opaque), 0, q, k, v, nullptr, &valid, cache_stride, 1, heads, head_width,
-                           scale, o, error, capacity);
+                           scale, o, error, capacity, true);
 }
 
 // =========================================================================================== section 2

@@ -76,7 +76,7 @@ struct StepSlots {
 
 // A seam call held back for one call so that the next one can join its launch (backend_hip.hip, "seam fusion").
 struct PendingOp {
-    enum { kNone = 0, kLayerNorm = 1, kLinear = 2 };
+    enum { kNone = 0, kLayerNorm = 1, kLinear = 2, kAttentionFold = 3 };
     int kind = kNone;
     // LayerNorm of one row (alone, or as the prologue of the product)
     const float *ln_in = nullptr;
@@ -89,6 +89,11 @@ struct PendingOp {
     size_t iw = 0, ow = 0;
     const CachedWeight *weight = nullptr;
     const float *bias = nullptr;                           // device copy
+    // attention whose chunks are still to be folded (alone, or as the prologue of the product that reads its output row)
+    bool has_fold = false;
+    float *fold_out = nullptr;
+    const float *fold_partial = nullptr, *fold_ml = nullptr;
+    int fold_heads = 0, fold_head_width = 0, fold_max_units = 0;
 };
 
 struct State {
@@ -121,6 +126,7 @@ struct State {
     // seam fusion: the held-back call, whether holding back is on (MYNAH_HIP_FUSE=0 turns it off), and the message of a
     // held-back launch that failed where no caller could be told (reported by the next sync)
     PendingOp pending;
+    StepSlots *seam_slots = nullptr;   // device word the chunk count of a held-back fold travels in
     int fuse = 1;
     char deferred_error[160] = {0};
 };

@@ -361,6 +361,7 @@ struct PrologueParams {
     int8_t *probe_qx;       // parity probes for stream 0 (written by workgroup 0 only)
     float *probe_sx;
     float *ln_out = nullptr;   // non-null: workgroup 0 also stores stream 0's LayerNorm row here
+    float *act_out = nullptr;  // non-null: workgroup 0 also stores stream 0's row as loaded (after a fold, before LayerNorm)
 };
 
 // Who stages which streams.  A team is four wavefronts acting as the 256 threads tid = 0..255 of the staging scheme
@@ -416,6 +417,11 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, cons
     const int wave = tid >> 6;
     float *s_scratch = s_scratch_all + team.stream0 * kPrologueScratch;   // the team's own region
     const int nf4 = p.k >> 2;
+    if (p.act_out != nullptr && blockIdx.x == 0 && team.stream0 == 0) {
+#pragma unroll
+        for (int i = 0; i < NVT; ++i)
+            if (tid + kThreads * i < nf4) reinterpret_cast<float4 *>(p.act_out)[tid + kThreads * i] = xr[0][i];
+    }
     if (p.ln_gain != nullptr) {
         float s[BT];
 #pragma unroll

@@ -34,6 +34,7 @@ struct LinearArgs {
     // value of the product before the residual epilogue adds it -- the buffers the separate calls would have written.
     float *ln_out;
     float *aux_out;
+    float *act_out;         // the input row as the prologue formed it (the fold of attention partials), before any LayerNorm
 };
 
 // True when the fused matvec kernel supports this shape/storage; otherwise use linear_generic.
@@ -64,12 +65,22 @@ struct AttnArgs {
     float scale;
     int is_self;
     int max_chunks;                // grid.x
+    // Consumer-side fold (single-stream seam calls): instead of folding, every chunk leaves its partial in the layout
+    // the fused matvec's fold prologue reads -- unit_partial [stream][head][max_chunks][head_width], unit_ml [stream][head][2][max_chunks]
+    // -- per stream, and the stream's chunk count, as "rows" of kStepUnitRows per chunk, in unit_slots->memory_length[stream].
+    float *unit_partial;
+    float *unit_ml;
+    StepSlots *unit_slots;
     int two_pass;                  // set by launch_attention: the fold is a launch of its own (no arrival counters)
     int chunk_rows;                // cache rows per workgroup: 0 / kAttnChunk, or kWideRows (from attention_chunk_rows)
     float *partial;                // [batch, heads, max_chunks, head_width + 2]
     unsigned *counters;            // [batch, heads], zero between launches
 };
 int launch_attention(State *st, const AttnArgs &args, char *error, size_t capacity);
+// Folds partials left in the unit layout into out[heads * head_width] (what the consumer's prologue would have formed).
+int launch_unit_fold(State *st, const float *partial, const float *ml, const StepSlots *slots, int heads, int head_width,
+                     int max_units, float *out, char *error, size_t capacity);
+int launch_unit_fold_streams(State *st, const AttnArgs &args, char *error, size_t capacity);
 int attention_chunk_rows(int is_self, size_t head_width, bool vector_rows, size_t max_valid);
 
 // Resident step: LayerNorm + activation quantisation + this head's slice of the Q (self: Q, K, V) projection +

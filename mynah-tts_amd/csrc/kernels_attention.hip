@@ -61,6 +61,16 @@ __device__ __forceinline__ Resolved resolve(const AttnArgs &a, int b) {
     return r;
 }
 
+// Unit layout for a stream without memory: one unit of zeros with sum 1, which folds to the zero row.
+__device__ __forceinline__ void empty_unit(const AttnArgs &a, int b, int head, int hw) {
+    for (int d = threadIdx.x; d < hw; d += kThreads) a.unit_partial[((size_t)b * a.heads + head) * a.max_chunks * hw + d] = 0.0f;
+    if (threadIdx.x == 0) {
+        a.unit_ml[((size_t)b * a.heads + head) * 2 * a.max_chunks] = 0.0f;
+        a.unit_ml[((size_t)b * a.heads + head) * 2 * a.max_chunks + a.max_chunks] = 1.0f;
+        if (head == 0) a.unit_slots->memory_length[b] = kStepUnitRows;
+    }
+}
+
 // Softmax statistics of one chunk: s_score[0..63] holds scaled scores (-3e38 beyond `count`);
 // afterwards it holds exp(score - max), and (max, sum) are in s_ml.
 __device__ __forceinline__ void chunk_stats(float *s_score, float *s_ml, int count) {
@@ -169,6 +179,7 @@ __global__ void __launch_bounds__(kThreads) k_attention_hw64(const AttnArgs a) {
     float *outh = r.out + (size_t)head * hw;
     if (r.valid <= 0) {   // empty memory: the reference leaves the context at zero (src/graph.c:3242)
         if (tid < hw) outh[tid] = 0.0f;
+        if (a.unit_partial != nullptr) empty_unit(a, b, head, hw);
         return;
     }
     const int p0 = chunk * kAttnChunk;
@@ -228,6 +239,20 @@ __global__ void __launch_bounds__(kThreads) k_attention_hw64(const AttnArgs a) {
     *reinterpret_cast<float4 *>(s_red + (size_t)g * hw + 4 * j) = acc;
     __syncthreads();
     const float m_c = s_ml[0], l_c = s_ml[1];
+    if (a.unit_partial != nullptr) {   // the consumer folds: leave this chunk's partial in its layout
+        if (tid < hw) {
+            float o = 0.0f;
+#pragma unroll
+            for (int gg = 0; gg < kPosPerPass; ++gg) o += s_red[(size_t)gg * hw + tid];
+            a.unit_partial[(((size_t)b * a.heads + head) * a.max_chunks + chunk) * hw + tid] = o;
+        }
+        if (tid == 0) {
+            a.unit_ml[((size_t)b * a.heads + head) * 2 * a.max_chunks + chunk] = m_c;
+            a.unit_ml[((size_t)b * a.heads + head) * 2 * a.max_chunks + a.max_chunks + chunk] = l_c;
+            if (chunk == 0 && head == 0) a.unit_slots->memory_length[b] = nchunks * kStepUnitRows;
+        }
+        return;
+    }
     if (nchunks == 1) {
         if (tid < hw) {
             float o = 0.0f;
@@ -372,6 +397,20 @@ __global__ void __launch_bounds__(kThreads) k_attention_fold(const AttnArgs a) {
     fold_chunks(a, part, nchunks, hw, r.out + (size_t)head * hw, s_w, s_fold);
 }
 
+// Fold of partials in the unit layout by a launch of its own: what the fused matvec's prologue forms when it is the
+// consumer (the same device function), for the case that some other call comes next.
+__global__ void __launch_bounds__(kThreads) k_unit_fold(const float *partial, const float *ml, const StepSlots *slots, int heads, int hw,
+                                                        int max_units, const AttnArgs a, float *single_out) {
+    const int f4 = blockIdx.x * kThreads + threadIdx.x;
+    const int b = blockIdx.y;
+    if (f4 >= heads * hw / 4) return;
+    ActSource src;
+    src.partial = partial; src.partial_ml = ml; src.slots = slots; src.heads = heads; src.head_width = hw;
+    src.max_units = max_units; src.is_self = 0; src.stream0 = 0;
+    float *out = single_out != nullptr ? single_out : a.out[b];
+    reinterpret_cast<float4 *>(out)[f4] = fold_partials(src, b, f4);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Wide heads (head_width = 256 * NV; the engine's cross attention is ONE head as wide as the model,
 // src/graph.c:3443-3448), read-only caches.  With one head there are only valid / 64 workgroups of
@@ -398,6 +437,7 @@ __global__ void __launch_bounds__(kThreads) k_attention_wide(const AttnArgs a) {
     float *outh = r.out + (size_t)head * hw;
     if (r.valid <= 0) {   // empty memory: the context stays zero (src/graph.c:3242)
         for (int d = tid; d < hw; d += kThreads) outh[d] = 0.0f;
+        if (a.unit_partial != nullptr) empty_unit(a, b, head, hw);
         return;
     }
     const int p0 = chunk * kWideRows;
@@ -470,6 +510,15 @@ __global__ void __launch_bounds__(kThreads) k_attention_wide(const AttnArgs a) {
             mine.x += o.x; mine.y += o.y; mine.z += o.z; mine.w += o.w;
         }
     }
+    if (a.unit_partial != nullptr) {   // the consumer folds: leave this chunk's partial in its layout
+        if (owner) *reinterpret_cast<float4 *>(a.unit_partial + (((size_t)b * a.heads + head) * a.max_chunks + chunk) * hw + 4 * tid) = mine;
+        if (tid == 0) {
+            a.unit_ml[((size_t)b * a.heads + head) * 2 * a.max_chunks + chunk] = m_c;
+            a.unit_ml[((size_t)b * a.heads + head) * 2 * a.max_chunks + a.max_chunks + chunk] = l_c;
+            if (chunk == 0 && head == 0) a.unit_slots->memory_length[b] = nchunks * kStepUnitRows;
+        }
+        return;
+    }
     if (nchunks == 1) {
         if (owner) *reinterpret_cast<float4 *>(outh + 4 * tid) = make_float4(mine.x / l_c, mine.y / l_c, mine.z / l_c, mine.w / l_c);
         return;
@@ -525,6 +574,22 @@ __global__ void __launch_bounds__(kThreads) k_attention_wide(const AttnArgs a) {
 
 }  // namespace
 
+int launch_unit_fold(State *st, const float *partial, const float *ml, const StepSlots *slots, int heads, int head_width,
+                     int max_units, float *out, char *error, size_t capacity) {
+    const int f4 = heads * head_width / 4;
+    hipLaunchKernelGGL(k_unit_fold, dim3((unsigned)((f4 + kThreads - 1) / kThreads), 1u), dim3(kThreads), 0, st->stream, partial, ml, slots, heads,
+                       head_width, max_units, AttnArgs{}, out);
+    return hip_check(hipGetLastError(), "unit fold launch", error, capacity);
+}
+
+// The same for every stream of a table-mode call, into the call's own output rows.
+int launch_unit_fold_streams(State *st, const AttnArgs &a, char *error, size_t capacity) {
+    const int f4 = a.heads * a.head_width / 4;
+    hipLaunchKernelGGL(k_unit_fold, dim3((unsigned)((f4 + kThreads - 1) / kThreads), (unsigned)a.batch), dim3(kThreads), 0, st->stream,
+                       a.unit_partial, a.unit_ml, a.unit_slots, a.heads, a.head_width, a.max_chunks, a, static_cast<float *>(nullptr));
+    return hip_check(hipGetLastError(), "unit fold launch", error, capacity);
+}
+
 // Rows of the cache one workgroup takes for this call: kWideRows when the wide-head kernel applies, else kAttnChunk.
 int attention_chunk_rows(int is_self, size_t head_width, bool vector_rows, size_t max_valid) {
     const bool wide = !is_self && vector_rows && head_width >= 256 && head_width <= 1024 && head_width % 256 == 0 &&
@@ -570,7 +635,11 @@ int launch_attention(State *st, const AttnArgs &a, char *error, size_t capacity)
     }
     // many chunk workgroups: fold in a second launch instead of a device-scope release per workgroup
     AttnArgs args = a;
-    args.two_pass = a.max_chunks > 1 && (size_t)a.max_chunks * a.heads * a.batch >= 64 ? 1 : 0;
+    args.two_pass = a.unit_partial == nullptr && a.max_chunks > 1 && (size_t)a.max_chunks * a.heads * a.batch >= 64 ? 1 : 0;
+    if (a.unit_partial != nullptr && !fast) {
+        set_error(error, capacity, "attention: the unit layout is written by the 64-wide and the wide-head kernels only");
+        return -1;
+    }
     if (fast) hipLaunchKernelGGL(k_attention_hw64, grid, dim3(kThreads), lds, st->stream, args);
     else if (vec) hipLaunchKernelGGL(k_attention_any<true>, grid, dim3(kThreads), lds, st->stream, args);
     else hipLaunchKernelGGL(k_attention_any<false>, grid, dim3(kThreads), lds, st->stream, args);

@@ -103,6 +103,7 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
     pro.k = k; pro.batch = a.batch; pro.ln_gain = arg_ln_gain; pro.ln_bias = arg_ln_bias; pro.arith = a.arith;
     pro.probe_qx = arg_probe_qx; pro.probe_sx = arg_probe_sx;
     pro.ln_out = SPEC != SPEC_ANY ? nullptr : a.ln_out;
+    pro.act_out = SPEC != SPEC_ANY ? nullptr : a.act_out;
     float4 xr[SB][NVT], gv[NVT], bv[NVT];
     {
         ActSource src;
@@ -316,7 +317,7 @@ template <int QT>
 int launch_linear_q(State *st, const LinearArgs &a, char *error, size_t capacity) {
     // what the arguments rule out decides the build (see SPEC above)
     const bool plain = a.bias == nullptr && a.probe_qx == nullptr && a.probe_sx == nullptr && a.probe_acc == nullptr &&
-                       a.ln_out == nullptr && a.aux_out == nullptr;
+                       a.ln_out == nullptr && a.aux_out == nullptr && a.act_out == nullptr;
     const bool residual = plain && a.epilogue == EPI_RESIDUAL && a.ln_gain == nullptr;
     const bool up = plain && a.epilogue == EPI_GELU && a.ln_gain != nullptr && a.fold_partial == nullptr;
     if (a.k == 768) {

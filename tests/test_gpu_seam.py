@@ -483,3 +483,56 @@ def test_batched_wide_head_cross_attention_bit_identical_to_solo(backend, orc, n
         assert np.array_equal(do[b].read(), together[b]), "stream %d" % b
     for d in dq + dk + dv + do:
         d.free()
+
+
+@pytest.mark.parametrize("qtype_name", ["f32", "int8"])
+@pytest.mark.parametrize("heads,hw,L,is_self", [(12, 64, 300, True), (12, 64, 1100, True), (1, 768, 200, False), (12, 64, 90, False)])
+def test_fused_attention_fold_matches_separate_launches(backend, pkg, orc, nerr, qtype_name, heads, hw, L, is_self):
+    """A single-stream attention call over more than one chunk leaves the fold of its chunks to the product that reads
+    its output row (the engine's attention -> output projection -> residual add, src/graph.c:3416-3428).  The joined
+    launch must leave in every buffer what the separate calls leave: the attention row (folded in another order: 1e-6
+    against the separate call, 1e-5 against the oracle), the product and the updated residual row."""
+    _announce("fused attention fold %s heads=%d hw=%d L=%d self=%s" % (qtype_name, heads, hw, L, is_self))
+    qt = {"f32": pkg.F32, "int8": pkg.INT8}[qtype_name]
+    tol = {"f32": 1e-5, "int8": 2e-2}[qtype_name]
+    backend.set_quant(qt)
+    rng = np.random.default_rng(1234 + L + hw)
+    width = heads * hw
+    scale = 1.0 / math.sqrt(hw)
+    qkv = rng.standard_normal(3 * width).astype(np.float32)
+    kc = rng.standard_normal((L + 1, width)).astype(np.float32)
+    vc = rng.standard_normal((L + 1, width)).astype(np.float32)
+    wo = backend.keep((0.02 * rng.standard_normal((width, width))).astype(np.float32))
+    x0 = rng.standard_normal(width).astype(np.float32)
+    dq, dk, dv = backend.alloc(qkv.size).write(qkv), backend.alloc(kc.size), backend.alloc(vc.size)
+    dattn, dproj, dx = backend.alloc(width), backend.alloc(width), backend.alloc(width)
+
+    def run(separate):
+        gap = backend.sync if separate else (lambda: None)
+        dk.write(kc)
+        dv.write(vc)
+        dx.write(x0)
+        dattn.write(np.zeros(width, np.float32))
+        if is_self:
+            backend.self_attention_dev(dq.ptr, dk.ptr, dv.ptr, L - 1, width, L, heads, hw, scale, dattn.ptr)
+        else:
+            backend.cross_attention_dev(dq.ptr, dk.ptr, dv.ptr, L, width, heads, hw, scale, dattn.ptr)
+        gap()
+        backend.matmul_d2d(dattn.ptr, dproj.ptr, 1, width, width, wo)
+        gap()
+        backend.residual_inplace(dx.ptr, dproj.ptr, width)
+        return dattn.read(), dproj.read(), dx.read(), dk.read().reshape(kc.shape)
+
+    want = run(True)
+    got = run(False)
+    ok, ov = kc.copy(), vc.copy()
+    ref = orc.self_attention(qkv, ok, ov, L - 1, width, L, heads, hw, scale) if is_self else \
+        orc.cross_attention(qkv[:width], kc, vc, L, width, heads, hw, scale)
+    assert nerr(got[0], ref) < 1e-5
+    assert nerr(got[0], want[0]) < 1e-6
+    assert nerr(got[1], want[1]) < tol and nerr(got[2], want[2]) < tol
+    assert np.array_equal(got[2], x0 + got[1])
+    assert np.array_equal(got[3], want[3]), "cache rows"
+    for d in (dq, dk, dv, dattn, dproj, dx):
+        d.free()
+    backend.set_quant(pkg.F32)
