@@ -85,3 +85,20 @@ def test_host_f16_conversion_is_ieee(pkg, orc):
     got = pkg.convert_weight_f16(lib, x)
     assert np.array_equal(got, want)
     assert np.array_equal(got, orc.f32_to_f16_bits(x))
+
+
+def test_reference_backend_struct_binds_every_seam_symbol(orc, ref_strict, pkg, synth):
+    """oracle/ref_shim_backend.c fills the reference's own backend struct (src/backend.c:26-70) from the library by
+    symbol name, through pointers of the prototypes in include/mynah_hip.h: it compiled, so every prototype fits the
+    struct's field; here it must find every symbol and reach the library's open call.  Without a GPU that call refuses
+    with its own message (no CPU fallback); with one it succeeds."""
+    cfg = synth.decoder_config(layers=1, capacity=8, cross_heads=1)
+    w = synth.decoder_weights(cfg, seed=0, ln_bias=False)
+    dec = orc.RefDecoder(cfg, w, orc.F32, 1, 4, strict=True)
+    try:
+        dec.use_hip(pkg.LIB_PATH)
+    except RuntimeError as e:
+        assert "missing symbol" not in str(e) and "dlopen" not in str(e), str(e)
+        assert "HIP" in str(e) or "device" in str(e), str(e)
+    finally:
+        dec.close()
