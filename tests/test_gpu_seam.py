@@ -274,7 +274,7 @@ def test_argmax(backend, orc):
 
 @pytest.mark.parametrize("heads,hw,L", [(12, 64, 1), (12, 64, 63), (12, 64, 64), (12, 64, 65), (12, 64, 300),
                                         (12, 64, 1024), (1, 768, 200), (3, 20, 70), (1, 2, 5),
-                                        (1, 768, 16), (1, 768, 17), (1, 768, 256), (1, 256, 100), (2, 512, 33), (1, 1024, 40)])
+                                        (12, 64, 127), (12, 64, 128), (12, 64, 129), (12, 64, 257), (1, 768, 16), (1, 768, 17), (1, 768, 256), (1, 256, 100), (2, 512, 33), (1, 1024, 40)])
 def test_self_and_cross_attention(backend, orc, nerr, heads, hw, L):
     """Split-L attention against the reference's two-pass order, incl. chunk edges (63/64/65), one wide head
     (what the engine passes for cross attention; its read-only form has a kernel of its own for head widths that are
