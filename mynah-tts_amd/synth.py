@@ -91,6 +91,28 @@ def encoder_weights(cfg, seed=4):
     return out
 
 
+def encoder_weights_f16(cfg, seed, kernel=1, biases=False):
+    """Encoder tensors whose matrices and tables are exactly representable in f16 (as f32 arrays), so that a checker that
+    reads f32 weights and one that reads f16 bits multiply the same numbers.  kernel > 1: the FFN weights are those of
+    the causal conv FFN, up [L, ffn, width * kernel] and down [L, width, ffn * kernel] (rows [in][kernel] flattened).
+    LayerNorm gains stay f32; biases only when asked for (the reference's LayerNorm has none)."""
+    rng = np.random.default_rng(seed)
+    L, w, f = cfg["layers"], cfg["width"], cfg["ffn"]
+
+    def n(shape, std, mean=0.0):
+        return (rng.standard_normal(shape) * std + mean).astype(np.float32)
+
+    def h(a):
+        return a.astype(np.float16).astype(np.float32)
+    out = {"tok_table": h(n((cfg["vocab"], w), 0.02)), "pos_table": h(n((cfg["max_positions"], w), 0.02)),
+           "qkv": h(n((L, 3 * w, w), 0.02)), "o": h(n((L, w, w), 0.02)),
+           "up": h(n((L, f, w * kernel), 0.02)), "down": h(n((L, w, f * kernel), 0.02)),
+           "norm1_g": n((L, w), 0.1, 1.0), "norm2_g": n((L, w), 0.1, 1.0), "norm_out_g": n((w,), 0.1, 1.0)}
+    for name in ("norm1_b", "norm2_b", "norm_out_b"):
+        out[name] = n((L, w) if name != "norm_out_b" else (w,), 0.02) if biases else None
+    return out
+
+
 # ---- algorithmic bytes (what roofline.achieved is computed from) --------------------------------
 def weight_bytes(n, k, qtype):
     """Packed bytes of one [n, k] matrix incl. scales: f32 4nk; int8 nk + 4n; int4 nk/2 + 4nk/32; f16 2nk."""

@@ -602,11 +602,25 @@ void orc_gemm_nt(const float *a, const float *b, float *c, size_t m, size_t n, s
     for (int t = 0; t < started; ++t) pthread_join(tid[t], NULL);
 }
 
-/* Text-encoder prefill for the synthetic f16 configuration: gather (src/graph.c:729-737) + position
- * add (:649-651), then per layer pre-LN -> QKV -> per-head scaled QK^T -> row softmax
- * (softmax_row_inplace, :245-257, over the full row: bidirectional) -> PV -> O -> +res
- * (:387-470 without the causal mask) -> LN -> FFN with the scalar GELU (kernel == 1 branch, :302-316)
- * -> +res; optional final norm (:696-701).  Weights are f16 values widened exactly; all arithmetic f32. */
+/* Causal unfold of [T, channels] rows over `kernel` taps (unfold_causal, src/graph.c:271-286):
+ * col[t][i * kernel + j] = input[t - (kernel - 1) + j][i], zero before the start. */
+static void unfold_rows(const float *input, float *col, size_t T, size_t channels, size_t kernel) {
+    for (size_t t = 0; t < T; ++t)
+        for (size_t j = 0; j < kernel; ++j) {
+            const long src = (long)t - (long)(kernel - 1u) + (long)j;
+            for (size_t i = 0; i < channels; ++i)
+                col[(t * channels + i) * kernel + j] = src < 0 ? 0.0f : input[(size_t)src * channels + i];
+        }
+}
+
+/* Text-encoder prefill (transformer_stack, src/graph.c:634-711, as encode_text calls it, :738-740): gather
+ * (:729-737) + position add (:649-651), then per layer pre-LN -> QKV -> per-head scaled QK^T -> row softmax
+ * (softmax_row_inplace, :245-257) -> PV -> O -> +res (:387-470) -> LN -> FFN -> +res; optional final norm (:696-701).
+ *   causal != 0: row t attends rows [0, t] only and the rest of its weights are zero (:446-449), the reference's form;
+ *                causal == 0: the full row (the synthetic bidirectional configuration).
+ *   ffn_kernel == 1: plain FFN with the scalar GELU (:302-316); ffn_kernel > 1: the causal conv FFN as one product
+ *                over the unfolded rows, weights [out][in][kernel] (:317-352); 0 means 1.
+ * Weights are f16 values widened exactly; all arithmetic f32. */
 int orc_encoder_prefill(const orc_encoder *e, const int32_t *ids, size_t T, uint16_t *embed_out,
                         float *out, int threads) {
     const size_t w = e->width, f = e->ffn, H = e->heads, hw = e->head_width;
@@ -624,8 +638,10 @@ int orc_encoder_prefill(const orc_encoder *e, const int32_t *ids, size_t T, uint
     float *kh = (float *)malloc(T * hw * sizeof(float));
     float *vt = (float *)malloc(T * hw * sizeof(float));
     float *hc = (float *)malloc(T * hw * sizeof(float));
-    const size_t wmax = 3u * w * w > f * w ? 3u * w * w : f * w;
+    const size_t kn = e->ffn_kernel == 0 ? 1u : e->ffn_kernel;
+    const size_t wmax = 3u * w * w > f * w * kn ? 3u * w * w : f * w * kn;
     float *wf = (float *)malloc(wmax * sizeof(float));
+    float *col = kn > 1u ? (float *)malloc(T * (f > w ? f : w) * kn * sizeof(float)) : NULL;
     for (size_t t = 0; t < T; ++t) {
         const uint16_t *row = e->tok_table + (size_t)ids[t] * w;
         const uint16_t *pos = e->pos_table + t * w;
@@ -647,7 +663,12 @@ int orc_encoder_prefill(const orc_encoder *e, const int32_t *ids, size_t T, uint
             orc_gemm_nt(qh, kh, scores, T, T, hw, threads);
             for (size_t t = 0; t < T; ++t) {
                 for (size_t s = 0; s < T; ++s) scores[t * T + s] *= scale;
-                orc_softmax_row_inplace(scores + t * T, T);
+                if (e->causal) {
+                    orc_softmax_row_inplace(scores + t * T, t + 1u);
+                    for (size_t s = t + 1u; s < T; ++s) scores[t * T + s] = 0.0f;
+                } else {
+                    orc_softmax_row_inplace(scores + t * T, T);
+                }
             }
             orc_gemm_nt(scores, vt, hc, T, hw, T, threads);
             for (size_t t = 0; t < T; ++t) memcpy(ctx + t * w + h * hw, hc + t * hw, hw * sizeof(float));
@@ -656,17 +677,27 @@ int orc_encoder_prefill(const orc_encoder *e, const int32_t *ids, size_t T, uint
         orc_gemm_nt(ctx, wf, proj, T, w, w, threads);
         for (size_t i = 0; i < T * w; ++i) x[i] += proj[i];
         orc_layernorm(x, e->norm2_g + layer * w, e->norm2_b ? e->norm2_b + layer * w : NULL, nrm, T, w, 1.0e-5f);
-        for (size_t i = 0; i < f * w; ++i) wf[i] = orc_f16_to_f32(e->up_w[layer * f * w + i]);
-        orc_gemm_nt(nrm, wf, hidden, T, f, w, threads);
+        for (size_t i = 0; i < f * w * kn; ++i) wf[i] = orc_f16_to_f32(e->up_w[layer * f * w * kn + i]);
+        if (kn == 1u) {
+            orc_gemm_nt(nrm, wf, hidden, T, f, w, threads);
+        } else {
+            unfold_rows(nrm, col, T, w, kn);
+            orc_gemm_nt(col, wf, hidden, T, f, w * kn, threads);
+        }
         orc_gelu_scalar(hidden, T * f);
-        for (size_t i = 0; i < w * f; ++i) wf[i] = orc_f16_to_f32(e->down_w[layer * w * f + i]);
-        orc_gemm_nt(hidden, wf, proj, T, w, f, threads);
+        for (size_t i = 0; i < w * f * kn; ++i) wf[i] = orc_f16_to_f32(e->down_w[layer * w * f * kn + i]);
+        if (kn == 1u) {
+            orc_gemm_nt(hidden, wf, proj, T, w, f, threads);
+        } else {
+            unfold_rows(hidden, col, T, f, kn);
+            orc_gemm_nt(col, wf, proj, T, w, f * kn, threads);
+        }
         for (size_t i = 0; i < T * w; ++i) x[i] += proj[i];
     }
     if (e->norm_out_g != NULL) orc_layernorm(x, e->norm_out_g, e->norm_out_b, out, T, w, 1.0e-5f);
     else memcpy(out, x, T * w * sizeof(float));
     free(x); free(nrm); free(qkv); free(ctx); free(proj); free(hidden); free(scores);
-    free(qh); free(kh); free(vt); free(hc); free(wf);
+    free(qh); free(kh); free(vt); free(hc); free(wf); free(col);
     return 0;
 }
 

@@ -19,12 +19,16 @@
  *                                                     random floats; ingot KATs 0x3c00<->1.0
  *   matvec_f16                                      -- no x86 reference build exists (src/qmat.c:25-28);
  *                                                     pinned by float64 dot of exactly-widened halves
- *   encoder prefill (bidirectional, plain FFN, f16-rounded weights, synthetic config)
- *                                                   -- float64 numpy restatement + attention/LN/GELU pins
- *                                                     above; the reference has no function with this exact
- *                                                     composition (its encoder is causal with conv FFN), and
- *                                                     its rows>1 GEMM is OpenBLAS, absent here: parity of the
- *                                                     GEMM rounding order is UNPINNED, tolerance 2e-3.
+ *   encoder prefill                                 -- the reference's form (causal mask, gain-only LayerNorm, plain and
+ *                                                     kernel-3 conv FFN): compiled reference's transformer_stack
+ *                                                     (src/graph.c:634-711) on f16-representable weights, 1 / 37 / 130 / 256
+ *                                                     tokens, both flag sets, 1e-5; the same outputs committed as golden
+ *                                                     vectors.  The bidirectional form with LayerNorm biases (the synthetic
+ *                                                     prefill configuration, which the reference has no function for): a
+ *                                                     float64 numpy restatement written from the definition, 1e-5.
+ *   orc_gemm_nt                                     -- float64 matmul; a row equals orc_matvec_f32 of that row bit for bit
+ *   orc_output_head                                 -- equals orc_linear + orc_softmax per head bit for bit (both pinned
+ *                                                     above); float64 softmax and, for f32 weights, float64 logits
  *   local step (local_step_batch)                   -- compiled reference's own local_step_batch (f32/int8/int4, both
  *                                                     flag sets, three positions of a batch of three)
  *   local token choice and frame bookkeeping (sample_local_frame_batch)
@@ -129,7 +133,7 @@ int orc_decoder_step(const orc_decoder *d, size_t batch, float *const *self_k, f
 void orc_output_head(const orc_weight *w_out, const float *bias, const float *hidden, size_t heads_out,
                      size_t vocab, float *logits, float *probs, int act_variant);
 
-/* ---- encoder prefill (synthetic config: bidirectional, plain FFN, pre-LN, f16-rounded weights) ---- */
+/* ---- encoder prefill (pre-LN; causal or bidirectional; plain or causal conv FFN; f16-rounded weights) ---- */
 typedef struct {
     size_t layers, width, heads, head_width, ffn, vocab, max_positions;
     const uint16_t *tok_table;   /* f16 bits [vocab,width] */
@@ -137,6 +141,9 @@ typedef struct {
     const uint16_t *qkv_w, *o_w, *up_w, *down_w;   /* f16 bits, per layer concatenated */
     const float *norm1_g, *norm1_b, *norm2_g, *norm2_b;   /* [layers,width]; *_b may be NULL */
     const float *norm_out_g, *norm_out_b;          /* [width] or NULL gain => no final norm */
+    int causal;                  /* != 0: row t attends rows [0, t] (the reference's encoder); 0: the full row */
+    size_t ffn_kernel;           /* 0 or 1: plain FFN, up_w [ffn,width], down_w [width,ffn]; k > 1: causal conv FFN,
+                                    up_w [ffn,width,k], down_w [width,ffn,k] */
 } orc_encoder;
 
 /* embed_out: f16 bits [T,width] of the gathered token rows (bit-exact artefact);

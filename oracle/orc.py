@@ -101,7 +101,8 @@ class OrcEncoder(C.Structure):
                 ("tok_table", C.c_void_p), ("pos_table", C.c_void_p),
                 ("qkv_w", C.c_void_p), ("o_w", C.c_void_p), ("up_w", C.c_void_p), ("down_w", C.c_void_p),
                 ("norm1_g", C.c_void_p), ("norm1_b", C.c_void_p), ("norm2_g", C.c_void_p),
-                ("norm2_b", C.c_void_p), ("norm_out_g", C.c_void_p), ("norm_out_b", C.c_void_p)]
+                ("norm2_b", C.c_void_p), ("norm_out_g", C.c_void_p), ("norm_out_b", C.c_void_p),
+                ("causal", C.c_int), ("ffn_kernel", _sz)]
 
 
 # ----------------------------------------------------------------------------- numpy-level helpers
@@ -310,8 +311,12 @@ def output_head(pw, hidden, heads_out, vocab, bias=None, act_variant=STRICT):
 
 
 def encoder_prefill(cfg, w, ids, threads=8):
-    """w: dict with f16-bit tables/weights (uint16) and f32 norms.  Returns (embed_bits, out)."""
+    """w: dict with f16-bit tables/weights (uint16) and f32 norms.  cfg["causal"] (default False) masks row t to rows
+    [0, t]; cfg["ffn_kernel"] (default 1) > 1 takes up_w [ffn, width, k] / down_w [width, ffn, k] of the causal conv FFN.
+    Returns (embed_bits, out)."""
     e = OrcEncoder()
+    e.causal = 1 if cfg.get("causal") else 0
+    e.ffn_kernel = int(cfg.get("ffn_kernel", 1))
     e.layers, e.width, e.heads, e.head_width, e.ffn = cfg["layers"], cfg["width"], cfg["heads"], cfg["head_width"], cfg["ffn"]
     e.vocab, e.max_positions = cfg["vocab"], cfg["max_positions"]
     keep = []
@@ -672,6 +677,43 @@ def write_safetensors(path, tensors):
         f.write(text)
         for blob in blobs:
             f.write(blob)
+
+
+def ref_transformer_stack(cfg, w, states, kernel, strict=False, workdir=None):
+    """The compiled reference's transformer_stack (src/graph.c:634-711) exactly as encode_text calls it (:738-740):
+    causal self-attention, gain-only LayerNorm, FFN with `kernel` taps, final norm when w["norm_out_g"] is given.
+    w holds f32 arrays: pos_table [P, width], qkv [L, 3w, w], o [L, w, w], up [L, ffn, w(, kernel)],
+    down [L, w, ffn(, kernel)], norm1_g / norm2_g [L, w].  states: the gathered token rows [T, width]."""
+    import tempfile
+    r = load_ref(strict)
+    fp = C.POINTER(C.c_float)
+    r.ref_transformer_stack.argtypes = [C.c_char_p, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int, fp, fp, C.c_char_p, _sz]
+    r.ref_transformer_stack.restype = C.c_int
+    L, width, ffn = cfg["layers"], cfg["width"], cfg["ffn"]
+    tensors = {"encoder.position_embeddings.weight": w["pos_table"]}
+    for l in range(L):
+        base = "encoder.layers.%d." % l
+        tensors[base + "norm_self.weight"] = w["norm1_g"][l]
+        tensors[base + "self_attention.qkv_net.weight"] = w["qkv"][l]
+        tensors[base + "self_attention.o_net.weight"] = w["o"][l]
+        tensors[base + "norm_pos_ff.weight"] = w["norm2_g"][l]
+        tensors[base + "pos_ff.proj.conv.weight"] = np.asarray(w["up"][l]).reshape(ffn, width, kernel)
+        tensors[base + "pos_ff.o_net.conv.weight"] = np.asarray(w["down"][l]).reshape(width, ffn, kernel)
+    final = w.get("norm_out_g") is not None
+    if final:
+        tensors["encoder.norm_out.weight"] = w["norm_out_g"]
+    states = np.ascontiguousarray(states, np.float32)
+    T = states.shape[0]
+    out = np.empty((T, width), np.float32)
+    err = C.create_string_buffer(512)
+    with tempfile.TemporaryDirectory(dir=workdir) as tmp:
+        path = os.path.join(tmp, "encoder.safetensors")
+        write_safetensors(path, tensors)
+        rc = r.ref_transformer_stack(os.fsencode(path), L, T, width, ffn, cfg["heads"], kernel, 1 if final else 0,
+                                     states.ctypes.data_as(fp), out.ctypes.data_as(fp), err, 512)
+    if rc != 0:
+        raise RuntimeError(err.value.decode())
+    return out
 
 
 def ref_codec(strict=False):

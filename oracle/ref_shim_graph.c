@@ -9,6 +9,7 @@
  *   decoder_step_batch        src/graph.c:3127-3284  (B slots, weight-stationary projections)
  *   local_step_batch          src/graph.c:1234-1343  (the local transformer's batched step)
  *   layer_norm                src/graph.c:147-150    (gain only, eps 1e-5)
+ *   transformer_stack         src/graph.c:634-711    (the text encoder's layer stack)
  *   softmax_row_inplace       src/graph.c:245-257
  *   batch_scratch_init        src/graph.c:121-144
  *   mynah_backend_open(CPU)   src/backend.c:367-475
@@ -297,6 +298,36 @@ int ref_snake(float *data, const float *alpha, size_t channels, size_t length, s
     if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &backend, error, sizeof error) != 0) return -1;
     const int rc = mynah_backend_snake_dev(backend, data, alpha, channels, length, snake_channels, error, sizeof error);
     mynah_backend_close(backend);
+    return rc;
+}
+
+/* ---- encoder stack --------------------------------------------------------------------------------------------
+ * Reference function reached (file:line in the reference tree):
+ *   transformer_stack         src/graph.c:634-711  (position add, per layer gain-only LayerNorm -> causal self_attention
+ *                                                  :387-513 -> +res -> LayerNorm -> causal_conv_ffn :288-385 -> +res,
+ *                                                  final norm) exactly as encode_text calls it (:738-740), on the CPU
+ *                                                  backend, with `kernel` 1 (plain FFN) or 3 (the model's conv FFN).
+ * Weights are looked up by name ("encoder....") in a safetensors file the caller wrote itself (synthetic tensors).
+ * `states` are the gathered token rows [length, width]; `output` receives [length, width]. */
+int ref_transformer_stack(const char *weights_path, size_t layers, size_t length, size_t width, size_t ffn_width,
+                          size_t heads, size_t kernel, int apply_norm_out, const float *states, float *output, char *error,
+                          size_t error_capacity) {
+    mynah_weights *file = NULL;
+    mynah_backend *backend = NULL;
+    int rc = -1;
+    if (error != NULL && error_capacity > 0) error[0] = '\0';
+    if (mynah_weights_open(weights_path, &file, error, error_capacity) != 0) return -1;
+    if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &backend, error, error_capacity) == 0) {
+        float *copy = (float *)malloc(length * width * sizeof(float));   /* the function takes a non-const pointer */
+        if (copy != NULL) {
+            memcpy(copy, states, length * width * sizeof(float));
+            rc = transformer_stack(file, backend, "encoder", layers, length, width, ffn_width, heads, kernel, 0, apply_norm_out,
+                                   NULL, 0, copy, output, error, error_capacity);
+            free(copy);
+        }
+    }
+    if (backend != NULL) mynah_backend_close(backend);
+    mynah_weights_close(file);
     return rc;
 }
 

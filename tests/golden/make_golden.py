@@ -27,6 +27,11 @@ STEP_LAYERS = 2
 # streams without any encoder memory beside streams that have one (src/graph.c:3237-3244: their context stays zero)
 NOMEM_LENGTHS = [3, 0, 12, 9]
 NOMEM_MEMS = [0, 5, 0, 13]
+ENC_CFG = {"layers": 2, "width": 768, "heads": 12, "head_width": 64, "ffn": 3072, "vocab": 300, "max_positions": 64,
+           "causal": True}
+ENC_KERNELS = (1, 3)
+ENC_TOKENS = 19
+ENC_SEED = 50
 
 
 def crc(*arrays):
@@ -131,6 +136,16 @@ def main():
     # streams have no encoder memory
     step_case(orc, synth, out, "step", STEP_LENGTHS, STEP_MEMS, 1, ("f32", "int8", "int4"))
     step_case(orc, synth, out, "nomem", NOMEM_LENGTHS, NOMEM_MEMS, 2, ("f32", "int8", "int4"))
+
+    # ---- the text encoder's layer stack (transformer_stack, src/graph.c:634-711, as encode_text calls it): causal,
+    # gain-only LayerNorm, plain FFN and the model's kernel-3 conv FFN, 19 tokens, 2 layers
+    for kernel in ENC_KERNELS:
+        cfg = dict(ENC_CFG, ffn_kernel=kernel)
+        w = synth.encoder_weights_f16(cfg, seed=ENC_SEED + kernel, kernel=kernel)
+        ids = np.random.default_rng(ENC_SEED).integers(0, cfg["vocab"], size=ENC_TOKENS).astype(np.int32)
+        out["enc_k%d_input_crc" % kernel] = crc(ids, *[w[k] for k in sorted(w) if w[k] is not None])
+        for tag, strict in (("stock", False), ("strict", True)):
+            out["enc_k%d_%s_out" % (kernel, tag)] = orc.ref_transformer_stack(cfg, w, w["tok_table"][ids], kernel, strict=strict)
 
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **out)

@@ -98,3 +98,22 @@ def test_decode_step(orc, synth, gold, nerr, case, qname, tag):
         assert nerr(outs[b], gold["%s_%s_%s_out" % (case, qname, tag)][b]) < tol, "stream %d" % b
         assert nerr(ks[b][:, lengths[b]], gold["%s_%s_%s_newk" % (case, qname, tag)][b]) < tol
         assert nerr(vs[b][:, lengths[b]], gold["%s_%s_%s_newv" % (case, qname, tag)][b]) < tol
+
+
+@pytest.mark.parametrize("kernel", [1, 3])
+@pytest.mark.parametrize("tag", ["stock", "strict"])
+def test_encoder_stack(orc, synth, gold, nerr, kernel, tag):
+    """orc_encoder_prefill in the reference's form (causal, gain-only LayerNorm, plain / kernel-3 conv FFN) against the
+    committed outputs of the compiled reference's transformer_stack (src/graph.c:634-711)."""
+    from tests.golden import make_golden as mg
+    cfg = dict(mg.ENC_CFG, ffn_kernel=kernel)
+    w = synth.encoder_weights_f16(cfg, seed=mg.ENC_SEED + kernel, kernel=kernel)
+    ids = np.random.default_rng(mg.ENC_SEED).integers(0, cfg["vocab"], size=mg.ENC_TOKENS).astype(np.int32)
+    if mg.crc(ids, *[w[k] for k in sorted(w) if w[k] is not None]) != gold["enc_k%d_input_crc" % kernel]:
+        pytest.skip("numpy's generator produced different synthetic inputs than when the fixture was written")
+    h = lambda a: np.asarray(a, np.float32).astype(np.float16).view(np.uint16)
+    ow = {"tok_table": h(w["tok_table"]), "pos_table": h(w["pos_table"]), "qkv_w": h(w["qkv"]), "o_w": h(w["o"]),
+          "up_w": h(w["up"]), "down_w": h(w["down"]), "norm1_g": w["norm1_g"], "norm2_g": w["norm2_g"],
+          "norm_out_g": w["norm_out_g"]}
+    _, got = orc.encoder_prefill(cfg, ow, ids)
+    assert nerr(got, gold["enc_k%d_%s_out" % (kernel, tag)]) < 1e-5
