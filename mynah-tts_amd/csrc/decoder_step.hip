@@ -40,6 +40,10 @@ struct mynah_hip_decoder {
     mynah::StepSlots *dev_slots = nullptr;
     float *partial = nullptr;   // split-L attention partials of the fused path
     float *partial_ml = nullptr;
+    // Split-L partials of the stand-alone attention kernels (head widths the fused kernel does not take).  Owned by the
+    // decoder, not the backend's shared workspace: that one is freed and reallocated when a later call needs more room,
+    // and the captured graphs of this decoder hold the address they were recorded with.
+    float *seam_partial = nullptr;
     int max_units = 0;
     bool fused_attention = false;
     hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};
@@ -94,8 +98,8 @@ static int enqueue_attention(State *st, const mynah_hip_decoder *d, int is_self,
     a.capacity = d->capacity;
     a.batch = batch;
     a.is_self = is_self;
-    a.partial = st->attn_partial;
-    a.counters = st->attn_counters;
+    a.partial = d->seam_partial;
+    a.counters = st->attn_counters;   // allocated once per backend and never moved
     if (is_self) {
         a.q[0] = d->qkv;
         a.out[0] = d->attn;
@@ -220,7 +224,7 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
     for (auto &row : d->stage_graphs)
         for (auto &g : row)
             if (g != nullptr) (void)hipGraphExecDestroy(g);
-    float *bufs[] = {d->x, d->qkv, d->attn, d->qx, d->ctx, d->hidden, d->partial, d->partial_ml};
+    float *bufs[] = {d->x, d->qkv, d->attn, d->qx, d->ctx, d->hidden, d->partial, d->partial_ml, d->seam_partial};
     for (float *p : bufs)
         if (p != nullptr) (void)hipFree(p);
     if (d->dev_slots != nullptr) (void)hipFree(d->dev_slots);
@@ -307,6 +311,11 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
                              (xw == 0 || (l0.q_cross->qtype == l0.qkv->qtype &&
                                           step_attention_supported(l0.q_cross->qtype, w, d->cross_heads, d->cross_head_width)));
         d->max_units = (int)((d->capacity + kStepUnitRows - 1) / kStepUnitRows) + 1;
+        if (!d->fused_attention) {
+            const size_t chunks = (d->capacity + kAttnChunk - 1) / kAttnChunk + 1;
+            rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->seam_partial), B * heads_max * chunks * (hw_max + 4) * sizeof(float)),
+                            "malloc", error, capacity);
+        }
         if (d->fused_attention) {
             const size_t floats = B * heads_max * (size_t)d->max_units * hw_max;
             rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial), floats * sizeof(float)), "malloc", error, capacity);

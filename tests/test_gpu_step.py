@@ -58,10 +58,23 @@ def _oracle_step(orc, cfg, weights, streams, qtype):
 
 QT = {"f32": 0, "int8": 1, "int4": 2, "f16": 3}
 # f32/f16 activations stay f32 end to end: 1e-5 normalised (f16: against the oracle run on the same f16 bits).
-# int8/int4 re-quantise the activation of every projection; one last-bit difference in a LayerNorm output can move
-# an int8 activation by one step, which the next layers amplify, so whole-step agreement is bounded at 2e-2 while the
-# per-projection integers are checked bit-exactly in test_gpu_seam.py.
+# int8/int4 re-quantise the activation of every projection.  With the same int8 activations on both sides a quantised
+# step agrees like an f32 one (1e-5); but the GPU's LayerNorm adds in another order than the CPU's, and a last-bit
+# difference there moves an activation that sits on a rounding boundary by one int8 step -- about 1e-3 of the output's
+# scale, amplified by the layers that follow.  Roughly one (stream, layer) in thirty meets such a boundary.  So a
+# quantised whole-step comparison asserts the shape of that: every stream below OUTLIER, and at most a stated number of
+# streams above TOL["f32"] (quantised_errors_ok).  The per-projection integers are bit-exact in test_gpu_seam.py.
 TOL = {"f32": 1e-5, "f16": 1e-5, "int8": 2e-2, "int4": 2e-2}
+OUTLIER = 2e-2
+
+
+def quantised_errors_ok(errors, max_outliers, what=""):
+    """errors: normalised errors of the streams (or rows) of one quantised comparison."""
+    errors = [float(e) for e in errors]
+    above = [e for e in errors if e >= TOL["f32"]]
+    print("[quantised] %s errors %s" % (what, " ".join("%.1e" % e for e in errors)), flush=True)
+    assert all(e < OUTLIER for e in errors), "%s: a stream is beyond the outlier bound: %s" % (what, errors)
+    assert len(above) <= max_outliers, "%s: %d streams above 1e-5 (at most %d expected): %s" % (what, len(above), max_outliers, errors)
 
 
 @pytest.mark.parametrize("qtype_name", ["f32", "f16", "int8", "int4"])
@@ -100,8 +113,11 @@ def test_two_layers_ragged_batch8_and_bit_identity(pkg, backend, orc, synth, ner
     h = Harness(pkg, backend, cfg, weights, streams)
     want, ks, vs = _oracle_step(orc, cfg, weights, streams, QT[qtype_name])
     first = h.step()                        # eager (first use of this batch size)
-    for b in range(8):
-        assert nerr(first[b], want[b]) < TOL[qtype_name], "stream %d" % b
+    if qtype_name in ("int8", "int4"):      # 16 (stream, layer) pairs: at most two streams may have met a rounding boundary
+        quantised_errors_ok([nerr(first[b], want[b]) for b in range(8)], 2, "two layers b=8 " + qtype_name)
+    else:
+        for b in range(8):
+            assert nerr(first[b], want[b]) < TOL[qtype_name], "stream %d" % b
     for b in (0, 3, 6):
         gk, gv = h.cache_rows(b)
         L = lengths[b]
@@ -146,6 +162,8 @@ def test_streams_without_memory(pkg, backend, orc, synth, nerr, qtype_name):
     h = Harness(pkg, backend, cfg, weights, streams)
     want, ks, vs = _oracle_step(orc, cfg, weights, streams, QT[qtype_name])
     first = h.step()
+    if qtype_name == "int8":
+        quantised_errors_ok([nerr(first[b], want[b]) for b in range(4)], 1, "streams without memory int8")
     for b in range(4):
         assert np.isfinite(first[b]).all(), "stream %d" % b
         assert nerr(first[b], want[b]) < TOL[qtype_name], "stream %d" % b
@@ -220,8 +238,8 @@ def test_twelve_layers_int8_multi_step(pkg, backend, orc, synth, nerr):
             s["length"] = lengths[i]
         want = odec.step(ks, vs, [s["ck"] for s in streams], [s["cv"] for s in streams], lengths, [64, 48], [s["x"] for s in streams])
         got = h.step()
-        for b in range(2):
-            assert nerr(got[b], want[b]) < 5e-2, "step %d stream %d" % (step, b)
+        # 24 (stream, layer) pairs per step: either stream may have met a rounding boundary, neither may leave the bound
+        quantised_errors_ok([nerr(got[b], want[b]) for b in range(2)], 2, "12 layers int8 step %d" % step)
         lengths = [n + 1 for n in lengths]
     h.close()
     backend.set_quant(0)
@@ -296,6 +314,9 @@ def test_step_against_compiled_reference_fixture(pkg, backend, synth, nerr, qtyp
     h = Harness(pkg, backend, cfg, weights, streams)
     got = h.step()
     tol = TOL[qtype_name]
+    if qtype_name != "f32":   # 8 or 4 streams x 2 layers: at most two streams may have met a rounding boundary
+        quantised_errors_ok([nerr(got[b], gold["%s_%s_%s_out" % (case, qtype_name, arith_name)][b]) for b in range(len(lengths))], 2,
+                            "fixture %s %s %s" % (case, qtype_name, arith_name))
     for b in range(len(lengths)):
         assert np.isfinite(got[b]).all(), "stream %d" % b
         assert nerr(got[b], gold["%s_%s_%s_out" % (case, qtype_name, arith_name)][b]) < tol, "stream %d" % b
@@ -319,8 +340,7 @@ def test_batch16_two_tiles(pkg, backend, orc, synth, nerr):
     h = Harness(pkg, backend, cfg, weights, streams)
     want, ks, vs = _oracle_step(orc, cfg, weights, streams, 1)
     first = h.step()
-    for b in range(16):
-        assert nerr(first[b], want[b]) < TOL["int8"], "stream %d" % b
+    quantised_errors_ok([nerr(first[b], want[b]) for b in range(16)], 2, "b=16 int8, one layer")
     for b in range(16):
         h.reset_cache(b)
     again = h.step()                       # captured graph
@@ -375,10 +395,12 @@ def test_full_size_ragged_batch8_int8(pkg, backend, orc, synth, nerr):
     assert all(np.all(np.isfinite(o)) for o in first)
     check = (1, 6)                                      # the shortest and the longest stream
     odec = orc.Decoder(cfg, weights, orc.INT8)
+    errs = []
     for b in check:
         s = streams[b]
         want = odec.step([s["k"].copy()], [s["v"].copy()], [s["ck"]], [s["cv"]], [lengths[b]], [cross_len[b]], [s["x"]])[0]
-        assert nerr(first[b], want) < 5e-2, "stream %d" % b     # 12 layers of re-quantised activations, see TOL above
+        errs.append(nerr(first[b], want))
+    quantised_errors_ok(errs, 2, "full size b=8 int8")     # 12 layers each: both may have met a rounding boundary
     for b in range(8):
         h.reset_cache(b)
     again = h.step()                                    # captured graph
@@ -390,3 +412,72 @@ def test_full_size_ragged_batch8_int8(pkg, backend, orc, synth, nerr):
         assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
     h.close()
     backend.set_quant(0)
+
+
+def test_config2_int4_full_stack_with_head(pkg, backend, orc, synth, nerr):
+    """The benchmark's int4 configuration at full size: 12 layers, int4 group-32 weights, batch 1, self KV 1024 rows, 256
+    encoder states under 12 x 64 cross heads, LayerNorm gain and bias, final LayerNorm, then the 768 -> 8 x 1024 output
+    projection and a softmax per head.  Hidden row, logits and probabilities against the oracle; the captured graph's
+    replay against the eager step bit for bit."""
+    _announce("config 2: 12 layers int4 b=1 kv=1024/256 + head")
+    cfg = synth.decoder_config(layers=12, capacity=1025)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, [1024], [256], seed=1)
+    rng = np.random.default_rng(1102)
+    head_w = backend.keep((rng.standard_normal((8192, 768)) * 0.02).astype(np.float32))
+    backend.set_quant(pkg.INT4)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    want, ks, vs = _oracle_step(orc, cfg, weights, streams, orc.INT4)
+    first = h.step()
+    assert np.isfinite(first[0]).all()
+    quantised_errors_ok([nerr(first[0], want[0])], 1, "config 2 hidden row")
+    gk, gv = h.cache_rows(0)
+    quantised_errors_ok([nerr(gk[:, 1024], ks[0][:, 1024]), nerr(gv[:, 1024], vs[0][:, 1024])], 2, "config 2 appended rows")
+    mask = np.ones(1025, bool)
+    mask[1024] = False
+    assert np.array_equal(gk[:, mask], streams[0]["k"][:, mask]) and np.array_equal(gv[:, mask], streams[0]["v"][:, mask])
+    # the head on the device's own hidden row: checked against the oracle's head of that same row, so the head's bar is the
+    # matvec's (1e-5) whatever the stack did before it
+    dl, dp = backend.alloc(8192), backend.alloc(8192)
+    backend.output_head([h.bufs[0]["out"].ptr], 768, head_w, None, 8192, 1024, [dl.ptr], [dp.ptr])
+    logits, probs = orc.output_head(orc.PackedWeight(head_w, orc.INT4), first[0], 8, 1024)
+    assert nerr(dl.read(), logits) < 1e-5
+    got_probs = dp.read()
+    assert nerr(got_probs, probs) < 1e-5
+    assert np.allclose(got_probs.reshape(8, 1024).sum(-1), 1.0, atol=1e-5)
+    for replay in range(3):                  # second call captures, the others replay
+        h.reset_cache(0)
+        again = h.step()
+        assert np.array_equal(again[0].view(np.uint32), first[0].view(np.uint32)), "replay %d" % replay
+    dl.free()
+    dp.free()
+    h.close()
+    backend.set_quant(0)
+
+
+def test_captured_step_survives_a_growing_backend_workspace(pkg, backend, synth):
+    """A decoder whose cross head is not 64 wide runs the eight-kernel layer, whose attention partials are the decoder's own
+    memory: after its graph has been captured, a second decoder with a far larger cache (which makes the backend replace
+    its shared attention workspace) and a step of that one, the first decoder's graph still gives its first result."""
+    _announce("captured graph vs workspace growth")
+    cfg_a = synth.decoder_config(layers=2, capacity=70, cross_heads=1)
+    weights_a = synth.decoder_weights(cfg_a, seed=0, ln_bias=False)
+    streams_a = synth.decoder_streams(cfg_a, [66, 3], [9, 20], seed=1)
+    a = Harness(pkg, backend, cfg_a, weights_a, streams_a)
+    first = a.step()
+    for b in range(2):
+        a.reset_cache(b)
+    second = a.step()                                  # captured here
+    cfg_b = synth.decoder_config(layers=1, capacity=20000, cross_heads=1)
+    weights_b = synth.decoder_weights(cfg_b, seed=3, ln_bias=False, position=False)
+    streams_b = synth.decoder_streams(cfg_b, [19990], [40], seed=2)
+    bh = Harness(pkg, backend, cfg_b, weights_b, streams_b)
+    bh.step()
+    for b in range(2):
+        a.reset_cache(b)
+    third = a.step()                                   # replay of the graph captured before the workspace moved
+    for b in range(2):
+        assert np.array_equal(second[b].view(np.uint32), first[b].view(np.uint32))
+        assert np.array_equal(third[b].view(np.uint32), first[b].view(np.uint32)), "stream %d changed after the workspace grew" % b
+    bh.close()
+    a.close()
