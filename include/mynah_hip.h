@@ -126,6 +126,17 @@ int mynah_hip_cross_attention_dev(void *state, const float *dev_q, const float *
                                   size_t head_width, float scale, float *dev_out,
                                   char *error, size_t error_capacity);
 
+/* No counterpart in the reference.  mynah_hip_self_attention_dev for callers that cannot allocate (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc): same arguments, same result bit for bit, but the split-L
+ * partials live in a fixed array inside the library (about 1 MiB per GPU, held until the process ends) and the call makes
+ * no hipMalloc, hipFree or memset node.  It fails with "exceeds the allocation-free workspace" when
+ * heads * (ceil(valid / 64) + 1) * (head_width + 4) floats exceed 2^18 (12 heads of 64: valid up to 20,480 rows), or heads
+ * exceed 4096.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two states, two streams) race. */
+int mynah_hip_self_attention_dev_noalloc(void *state, const float *dev_qkv, float *dev_k_cache, float *dev_v_cache,
+                                         size_t position, size_t cache_stride, size_t valid, size_t heads,
+                                         size_t head_width, float scale, float *dev_out,
+                                         char *error, size_t error_capacity);
+
 /* src/backend.h:165-179.  clip: clamp to [-1, 1], NaN -> 0 (gpu/metal/backend_metal_ops.m:1090-1101).
  * argmax: candidates i < codebook_size plus eos_id iff allow_eos; strict > from -FLT_MAX, the first
  * index wins ties (src/backend.c:825-847).  Synchronises and returns one scalar. */

@@ -97,6 +97,7 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_softmax_dev.argtypes = [_vp, _vp, _sz, _sz, _sz, *_err]
     lib.mynah_hip_self_attention_dev.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_float, _vp, *_err]
     lib.mynah_hip_cross_attention_dev.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp, *_err]
+    lib.mynah_hip_self_attention_dev_noalloc.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, C.c_float, _vp, *_err]
     lib.mynah_hip_copy_dev.argtypes = [_vp, _vp, _vp, _sz, *_err]
     lib.mynah_hip_scale_dev.argtypes = [_vp, _vp, _sz, C.c_float, *_err]
     lib.mynah_hip_clip_dev.argtypes = [_vp, _vp, _sz, *_err]
@@ -321,6 +322,10 @@ class Backend:
 
     def self_attention_dev(self, dqkv, dk, dv, position, stride, valid, heads, hw, scale, dout):
         self._call("mynah_hip_self_attention_dev", _vp(dqkv), _vp(dk), _vp(dv), _sz(position), _sz(stride), _sz(valid),
+                   _sz(heads), _sz(hw), C.c_float(scale), _vp(dout))
+
+    def self_attention_dev_noalloc(self, dqkv, dk, dv, position, stride, valid, heads, hw, scale, dout):
+        self._call("mynah_hip_self_attention_dev_noalloc", _vp(dqkv), _vp(dk), _vp(dv), _sz(position), _sz(stride), _sz(valid),
                    _sz(heads), _sz(hw), C.c_float(scale), _vp(dout))
 
     def cross_attention_dev(self, dq, dk, dv, valid, stride, heads, hw, scale, dout):

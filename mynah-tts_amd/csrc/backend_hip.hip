@@ -10,6 +10,34 @@
 
 namespace mynah {
 
+// ------------------------------------------------------------------------------------------ allocation-free workspace
+// Scratch of mynah_hip_self_attention_dev_noalloc: split-L partials, the device word the chunk count travels in, and
+// arrival counters, in one file-scope device array so that the call never allocates.  Each GPU holds its own copy at its
+// own address; host code reaches it only through the pointer hipGetSymbolAddress returned with that device current
+// (State::noalloc) -- the array's name here is a host-side stand-in, never a device address.
+constexpr size_t kNoAllocPartialFloats = (size_t)1 << 18;   // 1 MiB of partials
+constexpr size_t kNoAllocCounters = 4096;                    // heads of one stream
+struct NoAllocScratch {
+    float partial[kNoAllocPartialFloats];
+    StepSlots slots;
+    unsigned counters[kNoAllocCounters];
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(NoAllocScratch)];
+
+// Where an attention call keeps its partials: the backend's growable workspace, or a fixed one that must suffice.
+struct AttnWorkspace {
+    float *partial;
+    size_t partial_floats;
+    unsigned *counters;
+    size_t counter_count;
+    StepSlots *slots;
+};
+
+__global__ void __launch_bounds__(256) k_zero_words(unsigned *p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 // ------------------------------------------------------------------------------------------ helpers
 int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity) {
     if (st->pinned_bytes >= bytes) return 0;
@@ -323,7 +351,8 @@ static void hip_close(void *opaque) {
 
 static int attention_table(State *st, int is_self, const float *const *q, float *const *kc, float *const *vc,
                            const size_t *position, const size_t *valid, size_t stride, size_t batch, size_t heads,
-                           size_t hw, float scale, float *const *out, char *error, size_t capacity, bool hold = false) {
+                           size_t hw, float scale, float *const *out, char *error, size_t capacity, bool hold = false,
+                           const AttnWorkspace *fixed = nullptr) {
     if (batch == 0) return 0;
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "attention batch exceeds MYNAH_MAX_BATCH");
@@ -358,7 +387,26 @@ static int attention_table(State *st, int is_self, const float *const *q, float 
         aligned = aligned && ((reinterpret_cast<uintptr_t>(q[b]) | reinterpret_cast<uintptr_t>(kc[b]) |
                                reinterpret_cast<uintptr_t>(vc[b]) | reinterpret_cast<uintptr_t>(out[b])) & 15u) == 0;
     const size_t chunk_rows = (size_t)attention_chunk_rows(is_self, hw, aligned && hw % 4 == 0 && stride % 4 == 0, max_valid);
-    if (ensure_attention_workspace(st, batch, heads, hw, max_valid, error, capacity, chunk_rows) != 0) return -1;
+    float *ws_partial = nullptr;
+    unsigned *ws_counters = nullptr;
+    if (fixed != nullptr) {
+        // same sizing as ensure_attention_workspace, but the memory is what it is: refuse what does not fit
+        const size_t chunks = (max_valid + chunk_rows - 1) / chunk_rows + 1;
+        if (batch * heads * chunks * (hw + 4) > fixed->partial_floats || batch * heads > fixed->counter_count) {
+            set_error(error, capacity, "attention: the call exceeds the allocation-free workspace (heads x chunks x (head width + 4) floats above 2^18)");
+            return -1;
+        }
+        ws_partial = fixed->partial;
+        ws_counters = fixed->counters;
+        // the counters must read zero when the kernel starts; whatever an earlier call left there is cleared by a kernel
+        // (a memset node would not survive a caller's graph capture)
+        hipLaunchKernelGGL(k_zero_words, dim3((unsigned)((batch * heads + 255) / 256)), dim3(256), 0, st->stream, ws_counters, batch * heads);
+        MYNAH_TRY(hipGetLastError());
+    } else {
+        if (ensure_attention_workspace(st, batch, heads, hw, max_valid, error, capacity, chunk_rows) != 0) return -1;
+        ws_partial = st->attn_partial;
+        ws_counters = st->attn_counters;
+    }
     a.slots = nullptr;
     a.batch = (int)batch;
     a.heads = (int)heads;
@@ -369,8 +417,8 @@ static int attention_table(State *st, int is_self, const float *const *q, float 
     a.is_self = is_self;
     a.chunk_rows = (int)chunk_rows;
     a.max_chunks = (int)((max_valid + chunk_rows - 1) / chunk_rows);
-    a.partial = st->attn_partial;
-    a.counters = st->attn_counters;
+    a.partial = ws_partial;
+    a.counters = ws_counters;
     if (!aligned) a.q_stride = 1;   // any value that is not a multiple of 4 selects the scalar path
     // A single-stream seam call over more than one chunk leaves its partials for the product that will read its output
     // row (seam fusion): the fold becomes that product's prologue instead of a device-scope hand-over or a launch.
@@ -378,15 +426,15 @@ static int attention_table(State *st, int is_self, const float *const *q, float 
     if (a.max_chunks > 1 && unit_kernel) {
         // Whatever the batch, the chunks are folded by the one device function (fold_partials), so a stream's bits do not
         // depend on who called: the batched twin folds in a launch of its own, a single-stream call is held back.
-        if (st->seam_slots == nullptr) {
+        if (fixed == nullptr && st->seam_slots == nullptr) {
             MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->seam_slots), sizeof(StepSlots)));
             MYNAH_TRY(hipMemsetAsync(st->seam_slots, 0, sizeof(StepSlots), st->stream));
         }
-        a.unit_partial = st->attn_partial;
-        a.unit_ml = st->attn_partial + batch * heads * (size_t)a.max_chunks * hw;
-        a.unit_slots = st->seam_slots;
+        a.unit_partial = ws_partial;
+        a.unit_ml = ws_partial + batch * heads * (size_t)a.max_chunks * hw;
+        a.unit_slots = fixed != nullptr ? fixed->slots : st->seam_slots;   // the kernel writes the one word the fold reads
         if (launch_attention(st, a, error, capacity) != 0) return -1;
-        if (!(hold && st->fuse && batch == 1)) return launch_unit_fold_streams(st, a, error, capacity);
+        if (fixed != nullptr || !(hold && st->fuse && batch == 1)) return launch_unit_fold_streams(st, a, error, capacity);
         PendingOp p;
         p.kind = PendingOp::kAttentionFold;
         p.has_fold = true;
@@ -440,6 +488,13 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
     if (hip_check(hipStreamCreate(&st->stream), "stream create", error, capacity) != 0 ||
         hip_check(hipEventCreate(&st->ev0), "event create", error, capacity) != 0 ||
         hip_check(hipEventCreate(&st->ev1), "event create", error, capacity) != 0) {
+        hip_close(st);
+        return -1;
+    }
+    // the allocation-free entry point's workspace: this device's copy of the file-scope array
+    if (hip_check(hipGetSymbolAddress(reinterpret_cast<void **>(&st->noalloc), HIP_SYMBOL(scratch)), "scratch symbol address", error, capacity) != 0 ||
+        st->noalloc == nullptr) {
+        if (error != nullptr && capacity > 0 && error[0] == '\0') set_error(error, capacity, "scratch symbol has no device address");
         hip_close(st);
         return -1;
     }
@@ -793,6 +848,20 @@ extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, cons
     float *k[1] = {const_cast<float *>(dk)}, *v[1] = {const_cast<float *>(dv)}, *o[1] = {dout};
     return attention_table(enter_state(opaque), 0, q, k, v, nullptr, &valid, cache_stride, 1, heads, head_width,
                            scale, o, error, capacity, true);
+}
+
+// The same call on the library's fixed workspace: no hipMalloc, no hipFree, no memset node.  It is never held back for
+// fusion, and refuses a shape whose partials do not fit instead of growing anything.
+extern "C" int mynah_hip_self_attention_dev_noalloc(void *opaque, const float *dqkv, float *dk, float *dv, size_t position,
+                                                    size_t cache_stride, size_t valid, size_t heads, size_t head_width, float scale,
+                                                    float *dout, char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    NoAllocScratch *ws = static_cast<NoAllocScratch *>(st->noalloc);
+    const AttnWorkspace fixed{ws->partial, kNoAllocPartialFloats, ws->counters, kNoAllocCounters, &ws->slots};
+    const float *q[1] = {dqkv};
+    float *k[1] = {dk}, *v[1] = {dv}, *o[1] = {dout};
+    return attention_table(st, 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width, scale, o, error, capacity, false, &fixed);
 }
 
 // =========================================================================================== section 2

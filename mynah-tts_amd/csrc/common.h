@@ -118,6 +118,8 @@ struct State {
     float *attn_partial = nullptr;
     size_t attn_partial_floats = 0;
     unsigned *attn_counters = nullptr;
+    // this device's address of the library's fixed scratch array (the allocation-free entry point's workspace)
+    void *noalloc = nullptr;
     // small device block for batched pointer tables of the section-2 calls
     void *ptr_table = nullptr;
     void *ptr_table_host = nullptr;   // pinned
