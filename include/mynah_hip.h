@@ -380,7 +380,10 @@ int mynah_hip_timer_end(void *state, float *milliseconds, char *error, size_t er
 /* Streams `bytes` of backend-owned scratch through the chip (read+write) so that the last-level
  * cache holds none of the caller's data: used between timed iterations. */
 int mynah_hip_flush_cache(void *state, size_t bytes, char *error, size_t error_capacity);
-/* 0 = launch every stage kernel individually, 1 (default) = replay the step as a captured HIP graph. */
+/* How mynah_hip_decoder_step runs: 0 = every stage kernel a launch of its own, 1 = the step replayed as a captured HIP
+ * graph, 2 (default) = one persistent launch for the whole step where it applies (one or two streams, int8 / int4
+ * weights, width 768 / FFN 3072 / 64-wide heads, at most one attention unit per compute unit), else as 1.  All three give
+ * the same bits.  MYNAH_HIP_GRAPH in the environment at open sets the initial value. */
 int mynah_hip_set_graph_mode(void *state, int enabled, char *error, size_t error_capacity);
 /* Bytes of device memory held by the weight cache (packed weights + scales + vectors). */
 size_t mynah_hip_cached_weight_bytes(void *state);

@@ -343,6 +343,7 @@ static void hip_close(void *opaque) {
     if (st->argmax_result != nullptr) (void)hipFree(st->argmax_result);
     if (st->ptr_table != nullptr) (void)hipFree(st->ptr_table);
     if (st->ptr_table_host != nullptr) (void)hipHostFree(st->ptr_table_host);
+    if (st->persist_abort_host != nullptr) (void)hipHostFree(st->persist_abort_host);
     if (st->ev0 != nullptr) (void)hipEventDestroy(st->ev0);
     if (st->ev1 != nullptr) (void)hipEventDestroy(st->ev1);
     if (st->stream != nullptr) (void)hipStreamDestroy(st->stream);
@@ -506,8 +507,19 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
     if (arith != nullptr && strcmp(arith, "stock") == 0) st->arith = MYNAH_HIP_ARITH_STOCK;
     const char *fuse = getenv("MYNAH_HIP_FUSE");   // 0: every seam call is a launch of its own
     if (fuse != nullptr && strcmp(fuse, "0") == 0) st->fuse = 0;
-    const char *graph = getenv("MYNAH_HIP_GRAPH");
-    if (graph != nullptr && strcmp(graph, "0") == 0) st->graph_mode = 0;
+    const char *graph = getenv("MYNAH_HIP_GRAPH");   // 0: every stage a launch, 1: captured graph, 2 (default): persistent launch where it applies
+    if (graph != nullptr && (strcmp(graph, "0") == 0 || strcmp(graph, "1") == 0 || strcmp(graph, "2") == 0)) st->graph_mode = graph[0] - '0';
+    const char *spin = getenv("MYNAH_HIP_PERSIST_SPIN");
+    if (spin != nullptr && spin[0] != '\0') st->persist_spin_limit = (unsigned)strtoul(spin, nullptr, 10);
+    const char *row_wgs = getenv("MYNAH_HIP_PERSIST_ROW_WGS");
+    if (row_wgs != nullptr && row_wgs[0] != '\0') st->persist_row_wgs = atoi(row_wgs);
+    // the word a persistent step sets when one of its bounded waits gave up: host memory the device writes directly
+    if (hip_check(hipHostMalloc(reinterpret_cast<void **>(&st->persist_abort_host), 64, hipHostMallocMapped), "abort word", error, capacity) != 0 ||
+        hip_check(hipHostGetDevicePointer(reinterpret_cast<void **>(&st->persist_abort_dev), st->persist_abort_host, 0), "abort word", error, capacity) != 0) {
+        hip_close(st);
+        return -1;
+    }
+    st->persist_abort_host[0] = 0u;
     *state_out = st;
     if (matmul != nullptr) *matmul = hip_matmul;
     if (sgemm != nullptr) *sgemm = hip_sgemm;
@@ -544,6 +556,18 @@ extern "C" int mynah_hip_h2d(void *opaque, const float *host, float *dev_ptr, si
     return copy_to_device(st, dev_ptr, host, bytes, error, capacity);
 }
 
+// Waits for the stream; a persistent step that gave up one of its bounded waits has left results that mean nothing, and is
+// reported here, by the first call that synchronises after it.
+static int synchronise(State *st, char *error, size_t capacity) {
+    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    if (st->persist_abort_host != nullptr && st->persist_abort_host[0] != 0u) {
+        st->persist_abort_host[0] = 0u;
+        set_error(error, capacity, "resident decode step gave up a bounded wait between its workgroups; its outputs are invalid");
+        return -1;
+    }
+    return 0;
+}
+
 extern "C" int mynah_hip_d2h(void *opaque, const float *dev_ptr, float *host, size_t n, char *error, size_t capacity) {
     State *st = enter_state(opaque);
     size_t bytes = 0;
@@ -552,8 +576,7 @@ extern "C" int mynah_hip_d2h(void *opaque, const float *dev_ptr, float *host, si
         return -1;
     }
     if (bytes != 0) MYNAH_TRY(hipMemcpyAsync(host, dev_ptr, bytes, hipMemcpyDeviceToHost, st->stream));
-    MYNAH_TRY(hipStreamSynchronize(st->stream));
-    return 0;
+    return synchronise(st, error, capacity);
 }
 
 extern "C" int mynah_hip_upload(void *opaque, const float *host, size_t n, float **dev_ptr, char *error, size_t capacity) {
@@ -581,7 +604,7 @@ extern "C" int mynah_hip_sync(void *opaque, char *error, size_t capacity) {
         (void)hipStreamSynchronize(st->stream);
         return -1;
     }
-    return hip_check(hipStreamSynchronize(st->stream), "sync", error, capacity);
+    return synchronise(st, error, capacity);
 }
 
 extern "C" int mynah_hip_batch_begin(void *opaque, char *error, size_t capacity) {
@@ -1034,7 +1057,11 @@ extern "C" int mynah_hip_flush_cache(void *opaque, size_t bytes, char *error, si
 extern "C" int mynah_hip_set_graph_mode(void *opaque, int enabled, char *error, size_t capacity) {
     State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
-    st->graph_mode = enabled ? 1 : 0;
+    if (enabled < 0 || enabled > 2) {
+        set_error(error, capacity, "graph mode is 0 (launches), 1 (captured graph) or 2 (persistent launch where it applies)");
+        return -1;
+    }
+    st->graph_mode = enabled;
     return 0;
 }
 extern "C" size_t mynah_hip_cached_weight_bytes(void *opaque) {

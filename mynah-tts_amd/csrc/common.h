@@ -27,6 +27,7 @@ constexpr int kStepUnitRows = 128;   // cache rows per attention unit (workgroup
 // separate fold kernel runs once (every workgroup folding every stream would outweigh one extra launch) and
 // workgroups of units a stream does not have leave before requesting anything.
 constexpr int kConsumerFoldMaxBatch = 2;
+constexpr int kStepRecord = 68;      // 64-bit slots of one attention partial of the persistent step: out[64] | max | sum | two unused
 
 // ---- error plumbing (0 / -1 + message, src/backend.c:137-139) ----
 inline void set_error(char *error, size_t capacity, const char *message) {
@@ -102,7 +103,13 @@ struct State {
     int cu_count = 256;
     int qtype = MYNAH_HIP_F32;
     int arith = MYNAH_HIP_ARITH_STRICT;
-    int graph_mode = 1;
+    int graph_mode = 2;   // resident step: 0 = every stage kernel a launch, 1 = captured graph, 2 = one persistent launch where it applies (else graph)
+    // persistent step: word a workgroup sets when a bounded wait gave up (pinned host memory, mapped), polls a wait may make,
+    // and an override of the row stages' workgroup count (0 = chosen from the batch)
+    unsigned *persist_abort_host = nullptr;
+    unsigned *persist_abort_dev = nullptr;
+    unsigned persist_spin_limit = 1u << 20;
+    int persist_row_wgs = 0;
     std::mutex mu;
     std::unordered_map<WeightKey, CachedWeight, WeightKeyHash> weights;
     size_t weight_bytes = 0;

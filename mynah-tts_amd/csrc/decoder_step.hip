@@ -20,7 +20,7 @@
 
 #include <new>
 
-#include "kernels.h"
+#include "device_common.h"
 
 namespace mynah {
 
@@ -50,6 +50,12 @@ struct mynah_hip_decoder {
     int eager_steps[mynah::kMaxBatch + 1] = {};   // a batch size runs eagerly once before it is captured
     hipGraphExec_t stage_graphs[MYNAH_HIP_STAGE_COUNT][mynah::kMaxBatch + 1] = {};   // single-stage graphs (measurement only)
     int arith = 0;
+    // the step as one persistent launch (one or two streams): per-layer pointer table, exchange area and its tag counter
+    mynah::PersistLayer *persist_layers = nullptr;
+    unsigned long long *persist_exchange = nullptr;
+    size_t persist_exchange_words = 0;
+    unsigned persist_epoch = 8;
+    int qtype = 0;
 };
 
 namespace mynah {
@@ -228,6 +234,8 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
     for (float *p : bufs)
         if (p != nullptr) (void)hipFree(p);
     if (d->dev_slots != nullptr) (void)hipFree(d->dev_slots);
+    if (d->persist_layers != nullptr) (void)hipFree(d->persist_layers);
+    if (d->persist_exchange != nullptr) (void)hipFree(d->persist_exchange);
     delete d;
 }
 
@@ -324,6 +332,48 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
                                 "malloc", error, capacity);
         }
     }
+    if (rc == 0) {
+        const LayerWeights &l0 = d->lw[0];
+        d->qtype = l0.qkv->qtype;
+        bool one_type = true;
+        for (const LayerWeights &lw : d->lw)
+            one_type = one_type && lw.qkv->qtype == d->qtype && lw.o_self->qtype == d->qtype && lw.up->qtype == d->qtype && lw.down->qtype == d->qtype &&
+                       (xw == 0 || (lw.q_cross->qtype == d->qtype && lw.o_cross->qtype == d->qtype));
+        if (d->fused_attention && one_type &&
+            step_persistent_supported(d->qtype, w, d->heads, d->head_width, d->ffn, d->cross_heads, d->cross_head_width)) {
+            std::vector<PersistLayer> table(d->layers);
+            for (size_t l = 0; l < d->layers; ++l) {
+                const LayerWeights &lw = d->lw[l];
+                PersistLayer &t = table[l];
+                memset(&t, 0, sizeof t);
+                t.qkv_w = lw.qkv->data; t.qkv_s = lw.qkv->scales;
+                t.o_w = lw.o_self->data; t.o_s = lw.o_self->scales;
+                if (xw != 0) {
+                    t.qx_w = lw.q_cross->data; t.qx_s = lw.q_cross->scales;
+                    t.ox_w = lw.o_cross->data; t.ox_s = lw.o_cross->scales;
+                }
+                t.up_w = lw.up->data; t.up_s = lw.up->scales;
+                t.down_w = lw.down->data; t.down_s = lw.down->scales;
+                t.norm_self = lw.norm_self; t.norm_self_b = lw.norm_self_b;
+                t.norm_cross = lw.norm_cross; t.norm_cross_b = lw.norm_cross_b;
+                t.norm_ff = lw.norm_ff; t.norm_ff_b = lw.norm_ff_b;
+            }
+            PersistArgs shape{};
+            shape.heads = (int)d->heads;
+            shape.cross_heads = (int)d->cross_heads;
+            shape.max_units = d->max_units;
+            d->persist_exchange_words = step_persistent_exchange_words(shape);
+            rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->persist_layers), table.size() * sizeof(PersistLayer)), "malloc", error, capacity);
+            if (rc == 0)
+                rc |= hip_check(hipMemcpy(d->persist_layers, table.data(), table.size() * sizeof(PersistLayer), hipMemcpyHostToDevice), "layer table upload",
+                                error, capacity);
+            if (rc == 0)
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->persist_exchange), d->persist_exchange_words * sizeof(unsigned long long)), "malloc",
+                                error, capacity);
+            if (rc == 0)   // tag 0 is never expected: a fresh area holds nothing that could be taken for a result
+                rc |= hip_check(hipMemset(d->persist_exchange, 0, d->persist_exchange_words * sizeof(unsigned long long)), "exchange clear", error, capacity);
+        }
+    }
     if (rc != 0) {
         mynah_hip_decoder_destroy(opaque, d);
         return -1;
@@ -331,6 +381,69 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
     *out = d;
     return 0;
 }
+
+namespace mynah {
+
+// The step as one persistent launch, when this batch fits it: one or two streams, int8 / int4 weights, the stack's own
+// shape, and few enough attention units for one workgroup each.  Returns 1 when launched, 0 when the step has to take
+// the launched-kernels path, -1 on error.
+static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch, char *error, size_t capacity) {
+    if (st->graph_mode != 2 || d->persist_layers == nullptr || batch > 2 || st->persist_abort_dev == nullptr) return 0;
+    PersistArgs a{};
+    a.layers = d->persist_layers;
+    a.n_layers = (int)d->layers;
+    a.batch = (int)batch;
+    a.heads = (int)d->heads;
+    a.cross_heads = (int)d->cross_heads;
+    a.arith = d->arith;
+    a.capacity = d->capacity;
+    a.max_units = d->max_units;
+    a.scale = 1.0f / sqrtf((float)d->head_width);
+    for (size_t b = 0; b < batch; ++b) {
+        a.self_k[b] = slots[b].dev_self_k;
+        a.self_v[b] = slots[b].dev_self_v;
+        a.cross_k[b] = slots[b].dev_cross_k;
+        a.cross_v[b] = slots[b].dev_cross_v;
+        a.input[b] = slots[b].dev_input;
+        a.output[b] = slots[b].dev_output;
+        a.length[b] = (int)slots[b].length;
+        a.memory_length[b] = (int)slots[b].memory_length;
+    }
+    a.position = d->position;
+    a.norm_out = d->norm_out;
+    a.norm_out_b = d->norm_out_b;
+    a.exchange = d->persist_exchange;
+    a.spin_limit = st->persist_spin_limit;
+    a.abort_word = st->persist_abort_dev;
+    const int grid = st->cu_count;
+    const int attn = step_persistent_attention_workgroups(a);
+    if (attn > grid) return 0;
+    // Row stages count their workgroups from the end of the grid, attention roles from its start: with room for both, a
+    // workgroup has one kind of role and requests its next stage's operands a whole stage ahead.
+    const int pass768 = 4 * (64 >> lane_group_log2(768 / (d->qtype == MYNAH_HIP_INT8 ? 16 : 32)));
+    int free_wgs = grid - attn;
+    int wide = st->persist_row_wgs > 0 ? st->persist_row_wgs : (free_wgs >= 96 ? (free_wgs < 192 ? free_wgs : 192) : 192);
+    if (wide > grid) wide = grid;
+    a.rows_out = pass768;
+    a.wgs_out = (768 + a.rows_out - 1) / a.rows_out;
+    a.rows_up = (3072 + wide - 1) / wide;
+    a.wgs_up = (3072 + a.rows_up - 1) / a.rows_up;
+    a.rows_down = (768 + wide - 1) / wide;
+    a.wgs_down = (768 + a.rows_down - 1) / a.rows_down;
+    const unsigned span = 8u * (unsigned)(d->layers + 2);
+    if (d->persist_epoch > 0xffffffffu - 2u * span) {   // the tag counter is about to wrap: start over on a cleared area
+        if (hip_check(hipMemsetAsync(d->persist_exchange, 0, d->persist_exchange_words * sizeof(unsigned long long), st->stream), "exchange clear", error,
+                      capacity) != 0)
+            return -1;
+        d->persist_epoch = 8;
+    }
+    a.epoch = d->persist_epoch;
+    d->persist_epoch += span;
+    if (launch_step_persistent(st, a, d->qtype, grid, error, capacity) != 0) return -1;
+    return 1;
+}
+
+}  // namespace mynah
 
 extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch,
                                       char *error, size_t capacity) {
@@ -371,8 +484,12 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
         s.memory_length[b] = (int)in.memory_length;
     }
     const int B = (int)batch;
+    {
+        const int taken = try_persistent_step(st, d, slots, batch, error, capacity);
+        if (taken != 0) return taken < 0 ? -1 : 0;
+    }
     if (launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
-    if (!st->graph_mode || d->eager_steps[B] == 0) {
+    if (st->graph_mode == 0 || d->eager_steps[B] == 0) {
         // the first step of a batch size also performs one-time kernel attribute set-up, which does not belong in a capture
         d->eager_steps[B] = 1;
         return enqueue_layers(st, d, B, error, capacity);

@@ -101,6 +101,43 @@ __device__ __forceinline__ void block_reduce(float (&v)[BT], float *s_scratch, c
     }
 }
 
+// Sum over a 256-thread workgroup in a fixed order: lanes by butterfly, then waves 0..3.
+__device__ __forceinline__ float block_sum(float v, float *s4) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return ((s4[0] + s4[1]) + s4[2]) + s4[3];
+}
+__device__ __forceinline__ float block_max(float v, float *s4) {
+    v = wave_max(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
+}
+
+// mynah_layernorm_f32 (src/kernels.c:186-244): mean, then the variance of (x - mean), eps inside the
+// square root, y = (x - mean) * scale * gain (+ bias).  One workgroup per row.
+__device__ __forceinline__ void layernorm_row(const float *x, float *y, const float *gain, const float *bias, int width,
+                                              float *s4) {
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < width; i += 256) s += x[i];
+    const float mean = block_sum(s, s4) / (float)width;
+    float v = 0.0f;
+    for (int i = threadIdx.x; i < width; i += 256) {
+        const float d = x[i] - mean;
+        v = __builtin_fmaf(d, d, v);
+    }
+    const float variance = block_sum(v, s4);
+    const float scale = 1.0f / sqrtf(variance / (float)width + 1.0e-5f);
+    for (int i = threadIdx.x; i < width; i += 256) {
+        float z = ((x[i] - mean) * scale) * gain[i];
+        if (bias != nullptr) z += bias[i];
+        y[i] = z;
+    }
+}
+
 // round half away from zero by truncation, clamp to +-127 (src/qmat.c:106-110)
 __device__ __forceinline__ int quant_act(float x, float inv) {
     const float v = x * inv;
@@ -270,6 +307,11 @@ typedef float float_x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float4 load_global4(const float *p) {
     const float_x4 v = *(const __attribute__((address_space(1))) float_x4 *)p;
     return make_float4(v.x, v.y, v.z, v.w);
+}
+typedef unsigned uint_x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_global_u4(const uint4 *p) {
+    const uint_x4 v = *(const __attribute__((address_space(1))) uint_x4 *)p;
+    return make_uint4(v.x, v.y, v.z, v.w);
 }
 __device__ __forceinline__ float load_global(const float *p) { return *(const __attribute__((address_space(1))) float *)p; }
 __device__ __forceinline__ void store_global(float *p, float v) { *(__attribute__((address_space(1))) float *)p = v; }

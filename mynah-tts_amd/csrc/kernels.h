@@ -106,6 +106,38 @@ int launch_step_attention(State *st, const StepAttnArgs &args, char *error, size
 int launch_step_fold(State *st, const StepAttnArgs &args, float *out, char *error, size_t capacity);
 bool step_attention_supported(int qtype, size_t width, size_t heads, size_t head_width);
 
+// The whole resident step as one persistent launch (kernels_step_persistent.hip): one or two streams, int8 / int4 weights,
+// the decoder stack's own shape (width 768, FFN 3072, 64-wide heads).
+struct PersistLayer {   // one per layer, in device memory
+    const void *qkv_w, *o_w, *qx_w, *ox_w, *up_w, *down_w;
+    const float *qkv_s, *o_s, *qx_s, *ox_s, *up_s, *down_s;
+    const float *norm_self, *norm_self_b, *norm_cross, *norm_cross_b, *norm_ff, *norm_ff_b;
+};
+struct PersistArgs {
+    const PersistLayer *layers;
+    int n_layers, batch, heads, cross_heads, arith;
+    size_t capacity;
+    int max_units;                  // partial records per (stream, head) the exchange area holds
+    float scale;
+    float *self_k[2], *self_v[2];
+    const float *cross_k[2], *cross_v[2];
+    const float *input[2];
+    float *output[2];
+    int length[2], memory_length[2];
+    const float *position, *norm_out, *norm_out_b;
+    unsigned long long *exchange;   // tagged vectors and partial records (step_persistent_exchange_words of them)
+    unsigned epoch;                 // tags of this step start here; a step uses 8 * (layers + 1) of them
+    unsigned spin_limit;            // polls a wait may make before the step is given up
+    unsigned *abort_word;           // set when a wait gave up (host-visible)
+    int wgs_out, rows_out;          // workgroups and rows per workgroup of the [768, 768] output projections
+    int wgs_up, rows_up;            // ... of FFN up [3072, 768]
+    int wgs_down, rows_down;        // ... of FFN down [768, 3072]
+};
+bool step_persistent_supported(int qtype, size_t width, size_t heads, size_t head_width, size_t ffn, size_t cross_heads, size_t cross_head_width);
+size_t step_persistent_exchange_words(const PersistArgs &args);
+int step_persistent_attention_workgroups(const PersistArgs &args);
+int launch_step_persistent(State *st, const PersistArgs &args, int qtype, int grid, char *error, size_t capacity);
+
 int launch_layernorm(State *st, const float *in, float *out, const float *gain, const float *bias, size_t rows,
                      size_t width, char *error, size_t capacity);
 int launch_gelu(State *st, float *data, size_t n, char *error, size_t capacity);

@@ -7,43 +7,6 @@
 namespace mynah {
 namespace {
 
-// Sum over a 256-thread workgroup in a fixed order: lanes by butterfly, then waves 0..3.
-__device__ __forceinline__ float block_sum(float v, float *s4) {
-    v = wave_sum(v);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return ((s4[0] + s4[1]) + s4[2]) + s4[3];
-}
-__device__ __forceinline__ float block_max(float v, float *s4) {
-    v = wave_max(v);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) s4[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return fmaxf(fmaxf(s4[0], s4[1]), fmaxf(s4[2], s4[3]));
-}
-
-// mynah_layernorm_f32 (src/kernels.c:186-244): mean, then the variance of (x - mean), eps inside the
-// square root, y = (x - mean) * scale * gain (+ bias).  One workgroup per row.
-__device__ __forceinline__ void layernorm_row(const float *x, float *y, const float *gain, const float *bias, int width,
-                                              float *s4) {
-    float s = 0.0f;
-    for (int i = threadIdx.x; i < width; i += 256) s += x[i];
-    const float mean = block_sum(s, s4) / (float)width;
-    float v = 0.0f;
-    for (int i = threadIdx.x; i < width; i += 256) {
-        const float d = x[i] - mean;
-        v = __builtin_fmaf(d, d, v);
-    }
-    const float variance = block_sum(v, s4);
-    const float scale = 1.0f / sqrtf(variance / (float)width + 1.0e-5f);
-    for (int i = threadIdx.x; i < width; i += 256) {
-        float z = ((x[i] - mean) * scale) * gain[i];
-        if (bias != nullptr) z += bias[i];
-        y[i] = z;
-    }
-}
-
 __global__ void __launch_bounds__(256) k_layernorm(const float *in, float *out, const float *gain, const float *bias, int width) {
     __shared__ float s4[4];
     layernorm_row(in + (size_t)blockIdx.x * width, out + (size_t)blockIdx.x * width, gain, bias, width, s4);

@@ -24,104 +24,10 @@
 //
 // The mapping from workgroup to (head, stream, unit) is static, so the weight slice and x are requested
 // before the slot table (lengths, cache pointers) has arrived; K and V rows follow as soon as it has.
-#include "device_common.h"
+#include "step_attention_core.h"
 
 namespace mynah {
 namespace {
-
-constexpr int kHw = 64;                          // head width handled by the fused kernel
-constexpr int kPosLanes = 16;                    // lanes cooperating on one cache row
-constexpr int kPosPerPass = kThreads / kPosLanes;
-constexpr int kRowsPerThread = kStepUnitRows / kPosPerPass;   // 8
-// PF = passes of weight rows per register bank: one bank is in flight for a cache-chunk or V workgroup, two for the
-// Q+K workgroup of the new row (twice the rows).  4 when one or two streams are stepped (every weight row of a head is
-// requested at once: shortest path), 2 for larger batches (fewer registers: three workgroups per CU instead of two,
-// which is what matters once there are more workgroups than the chip holds at a time).  The arithmetic is the same.
-constexpr int kPrefetchLatency = 4, kPrefetchThroughput = 2;
-
-struct PassRegs {
-    uint4 wv[4];
-    float sc[4];   // int4: group scales of the four chunks
-    float ws;      // int8: scale of the row
-};
-
-// Weight row of projection output r for this head: r = part * 64 + i, part 0/1/2 = q/k/v.
-__device__ __forceinline__ int weight_row(int r, int head, int width) { return (r >> 6) * width + head * kHw + (r & 63); }
-
-template <int QT, int PF>
-__device__ __forceinline__ void load_pass(PassRegs &p, const StepAttnArgs &a, int pass, int row0, int nrows, int head, int lg, int chunks) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int G = 1 << lg, gl = lane & (G - 1), gidx = lane >> lg;
-    const int rpp = 64 >> lg;
-    int r = row0 + pass * 4 * rpp + wave * rpp + gidx;
-    if (r >= row0 + nrows) r = row0 + nrows - 1;
-    const int wrow_id = weight_row(r, head, a.width);
-    const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(a.w) + (size_t)wrow_id * chunks * 16);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int c = gl + u * G;
-        p.wv[u] = c < chunks ? wrow[c] : make_uint4(0, 0, 0, 0);
-        p.sc[u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? a.scales[(size_t)wrow_id * chunks + c] : 0.0f;
-    }
-    // the row scale travels with the weights in the latency layout; the throughput layout fetches it at use (registers)
-    p.ws = (QT == MYNAH_HIP_INT8 && PF == kPrefetchLatency) ? a.scales[wrow_id] : 1.0f;
-}
-
-// Requests passes [pass0, pass0 + PF) of rows [row0, row0 + nrows) into `bank`.
-template <int QT, int PF>
-__device__ __forceinline__ void load_bank(PassRegs (&bank)[PF], const StepAttnArgs &a, int pass0, int row0, int nrows, int head,
-                                          int lg, int chunks) {
-    const int rpp = 64 >> lg;
-    const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
-#pragma unroll
-    for (int p = 0; p < PF; ++p)
-        if (pass0 + p < passes) load_pass<QT, PF>(bank[p], a, pass0 + p, row0, nrows, head, lg, chunks);
-}
-
-// Passes [pass0, pass0 + PF) of the projection rows [row0, row0 + nrows) of this head (row numbering
-// of weight_row), whose weights are in `bank` -> s_proj.
-template <int QT, int PF>
-__device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRegs (&bank)[PF], int pass0, int row0, int nrows,
-                                             int head, int lg, int chunks, const unsigned char *smem, const float sx, float *s_proj) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int G = 1 << lg, gl = lane & (G - 1), gidx = lane >> lg;
-    const int rpp = 64 >> lg;
-    const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
-#pragma unroll
-    for (int p = 0; p < PF; ++p) {
-        const int pass = pass0 + p;
-        if (pass < passes) {
-            const int r = row0 + pass * 4 * rpp + wave * rpp + gidx;
-            int iacc[1] = {0};
-            float facc[1] = {0.0f};
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int c = gl + u * G;
-                if (c < chunks) dot_chunk<QT, 1>(bank[p].wv[u], bank[p].sc[u], c, smem, a.width, iacc, facc, nullptr);
-            }
-            group_reduce<QT, 1>(iacc, facc, lg);
-            if (gl == 0 && r < row0 + nrows) {
-                float wscale = bank[p].ws;
-                if constexpr (QT == MYNAH_HIP_INT8 && PF != kPrefetchLatency) wscale = a.scales[weight_row(r, head, a.width)];
-                s_proj[r] = finish_value<QT>(iacc[0], facc[0], wscale, sx);
-            }
-        }
-    }
-}
-
-// Projection rows [row0, row0 + nrows): passes [0, PF) are in `bank` on entry, those from `next_pass`
-// on are fetched here, a bank at a time.
-template <int QT, int PF>
-__device__ __forceinline__ void project_rows(const StepAttnArgs &a, PassRegs (&bank)[PF], int next_pass, int row0, int nrows,
-                                             int head, int lg, int chunks, const unsigned char *smem, const float sx, float *s_proj) {
-    const int rpp = 64 >> lg;
-    const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
-    project_bank<QT, PF>(a, bank, 0, row0, nrows, head, lg, chunks, smem, sx, s_proj);
-    for (int pb = next_pass; pb < passes; pb += PF) {
-        load_bank<QT, PF>(bank, a, pb, row0, nrows, head, lg, chunks);
-        project_bank<QT, PF>(a, bank, pb, row0, nrows, head, lg, chunks, smem, sx, s_proj);
-    }
-}
 
 // WFIX: model width known at compile time (0 = taken from the arguments): lane-group width, chunks per lane and passes
 // per bank become constants and the per-chunk range checks fold away.  The decoder stack's width (768) gets such a build.
@@ -382,64 +288,18 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     // (its four 16-lane row groups x 8 passes) and nothing leaves it until its own (max, sum, out[64]) is complete;
     // the four results of a chunk meet once in LDS.
     const float4 qv = *reinterpret_cast<const float4 *>(s_proj + 4 * j);
-    const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
     for (int cc = 0; cc < CP; ++cc) {
         if (count[cc] <= 0) continue;   // the stream's last group may hold one chunk only (same for the whole workgroup)
-        float sc[kRowsPerThread];
-        float m = -3.0e38f;
-#pragma unroll
-        for (int i = 0; i < kRowsPerThread; ++i) {
-            const int pi = g + kPosPerPass * i;
-            float dot = 0.0f;
-            dot = __builtin_fmaf(qv.x, kv[cc][i].x, dot);
-            dot = __builtin_fmaf(qv.y, kv[cc][i].y, dot);
-            dot = __builtin_fmaf(qv.z, kv[cc][i].z, dot);
-            dot = __builtin_fmaf(qv.w, kv[cc][i].w, dot);
-            dot = row16_sum(dot);   // every lane of the row group holds the row's score
-            sc[i] = pi < count[cc] ? dot * a.scale : -3.0e38f;
-            m = fmaxf(m, sc[i]);
-        }
-        m = fmaxf(fmaxf(lane_f(m, 0), lane_f(m, 16)), fmaxf(lane_f(m, 32), lane_f(m, 48)));
-        float l = 0.0f;
-        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-        for (int i = 0; i < kRowsPerThread; ++i) {
-            // hardware exponential (2^(x log2 e), relative error about 1e-6 for the arguments met here) for the chunk's 128 weights;
-            // the few exponentials that combine partial results stay exact
-            const float e = g + kPosPerPass * i < count[cc] ? __expf(sc[i] - m) : 0.0f;
-            l += e;
-            acc.x = __builtin_fmaf(e, vv[cc][i].x, acc.x);
-            acc.y = __builtin_fmaf(e, vv[cc][i].y, acc.y);
-            acc.z = __builtin_fmaf(e, vv[cc][i].z, acc.z);
-            acc.w = __builtin_fmaf(e, vv[cc][i].w, acc.w);
-        }
-        l = ((lane_f(l, 0) + lane_f(l, 16)) + lane_f(l, 32)) + lane_f(l, 48);
-        acc.x += __shfl_xor(acc.x, 16); acc.y += __shfl_xor(acc.y, 16); acc.z += __shfl_xor(acc.z, 16); acc.w += __shfl_xor(acc.w, 16);
-        acc.x += __shfl_xor(acc.x, 32); acc.y += __shfl_xor(acc.y, 32); acc.z += __shfl_xor(acc.z, 32); acc.w += __shfl_xor(acc.w, 32);
-        if (lane < kPosLanes) *reinterpret_cast<float4 *>(s_red[cc] + wave * kHw + 4 * lane) = acc;
-        if (lane == 0) { s_wave_ml[cc][wave] = m; s_wave_ml[cc][4 + wave] = l; }
+        attend_chunk(qv, kv[cc], vv[cc], count[cc], a.scale, s_red[cc], s_wave_ml[cc]);
     }
     __syncthreads();
     if (tid < CP * kPosLanes) {   // merge a chunk's four wavefronts in order 0..3: lanes 0-15 the first chunk, 16-31 the second
         const int cc = tid / kPosLanes, t = tid - cc * kPosLanes;
         if (count[cc] > 0) {
-            const float *ml = s_wave_ml[cc];
-            const float *red = s_red[cc];
-            const float m0 = ml[0], m1 = ml[1], m2 = ml[2], m3 = ml[3];
-            const float M = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
-            const float w0 = expf(m0 - M), w1 = expf(m1 - M), w2 = expf(m2 - M), w3 = expf(m3 - M);   // a wavefront without rows: exp(-3e38 - M) = 0
-            float L = ml[4] * w0;
-            L = __builtin_fmaf(ml[5], w1, L);
-            L = __builtin_fmaf(ml[6], w2, L);
-            L = __builtin_fmaf(ml[7], w3, L);
-            const float4 o0 = *reinterpret_cast<const float4 *>(red + 4 * t), o1 = *reinterpret_cast<const float4 *>(red + kHw + 4 * t);
-            const float4 o2 = *reinterpret_cast<const float4 *>(red + 2 * kHw + 4 * t), o3 = *reinterpret_cast<const float4 *>(red + 3 * kHw + 4 * t);
             float4 o;
-            o.x = __builtin_fmaf(o3.x, w3, __builtin_fmaf(o2.x, w2, __builtin_fmaf(o1.x, w1, o0.x * w0)));
-            o.y = __builtin_fmaf(o3.y, w3, __builtin_fmaf(o2.y, w2, __builtin_fmaf(o1.y, w1, o0.y * w0)));
-            o.z = __builtin_fmaf(o3.z, w3, __builtin_fmaf(o2.z, w2, __builtin_fmaf(o1.z, w1, o0.z * w0)));
-            o.w = __builtin_fmaf(o3.w, w3, __builtin_fmaf(o2.w, w2, __builtin_fmaf(o1.w, w1, o0.w * w0)));
+            float M, L;
+            merge_chunk(t, s_red[cc], s_wave_ml[cc], o, M, L);
             *reinterpret_cast<float4 *>(out_o + (size_t)cc * kHw + 4 * t) = o;
             if (t == 0) { out_m[pidx + cc] = M; out_l[pidx + cc] = L; }
         }
