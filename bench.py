@@ -56,38 +56,54 @@ def build_sets(pkg, synth, backend, cfg, qtype, lengths, mems, head_rows, rotate
     return sets, streams
 
 
-def run_steps(backend, sets, cfg, head_rows, vocab, count, start=0):
+def run_steps(backend, sets, cfg, head_rows, vocab, count, start=0, with_head=True):
     for i in range(start, start + count):
         s = sets[i % len(sets)]
         s["dec"].step(s["slots"])
-        backend.output_head([o.ptr for o in s["outs"]], cfg["width"], s["head"], None, head_rows, vocab,
-                            [d.ptr for d in s["logits"]], [d.ptr for d in s["probs"]])
+        if with_head:
+            backend.output_head([o.ptr for o in s["outs"]], cfg["width"], s["head"], None, head_rows, vocab,
+                                [d.ptr for d in s["logits"]], [d.ptr for d in s["probs"]])
 
 
-def time_config(pkg, synth, backend, qtype, lengths, mems, capacity, steps, warmup, rotate=ROTATE):
+def timed_steps(backend, sets, cfg, head_rows, vocab, steps, warmup, with_head=True):
+    run_steps(backend, sets, cfg, head_rows, vocab, warmup, with_head=with_head)
+    backend.sync()
+    backend.timer_begin()
+    run_steps(backend, sets, cfg, head_rows, vocab, steps, with_head=with_head)
+    return backend.timer_end() * 1000.0 / steps
+
+
+def time_config(pkg, synth, backend, qtype, lengths, mems, capacity, steps, warmup, rotate=ROTATE, stages=True):
+    """Times the step of one configuration as the library runs it by default (a captured graph of stage kernels) with the
+    output head -- the figure `value` is made from --, the decoder stack's part of it alone, each stage kernel of the
+    graph alone, and, where it applies, the same step as one persistent launch (graph mode 2, opt-in)."""
     cfg = synth.decoder_config(layers=12, capacity=capacity)
     head_rows, vocab = 8 * 1024, 1024
     backend.set_quant(qtype)
     t0 = time.time()
     sets, streams = build_sets(pkg, synth, backend, cfg, qtype, lengths, mems, head_rows, rotate)
     setup_s = time.time() - t0
-    run_steps(backend, sets, cfg, head_rows, vocab, max(warmup, 2 * rotate))      # eager pass + graph capture for every set
-    backend.sync()
-    backend.timer_begin()
-    run_steps(backend, sets, cfg, head_rows, vocab, steps)
-    ms = backend.timer_end()
-    step_us = ms * 1000.0 / steps
+    warm = max(warmup, 2 * rotate)      # every set runs eagerly once and captures its graph before anything is timed
+    batch = len(streams)
+    backend.set_graph_mode(1)
+    step_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm)
+    probs = sets[0]["probs"][0].read()
+    assert np.all(np.isfinite(probs)) and abs(float(probs[:vocab].sum()) - 1.0) < 1e-3, "benchmark output is not a distribution"
+    stack_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm, with_head=False)
+    persistent_us = persistent_stack_us = None
+    if batch <= 2 and qtype in (pkg.INT8, pkg.INT4):      # the same step as one persistent launch (opt-in form)
+        backend.set_graph_mode(2)
+        persistent_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm)
+        persistent_stack_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm, with_head=False)
+        backend.set_graph_mode(1)
     b = synth.decoder_step_bytes(cfg, qtype, [s["length"] for s in streams], [s["memory_length"] for s in streams])
     head_bytes = synth.weight_bytes(head_rows, cfg["width"], qtype)
     total = b["total"] + head_bytes
-    probs = sets[0]["probs"][0].read()
-    assert np.all(np.isfinite(probs)) and abs(float(probs[:vocab].sum()) - 1.0) < 1e-3, "benchmark output is not a distribution"
-    # per-stage launch times: each of the six stage kernels alone (its 12 launches per step as one graph), rotating over
-    # the same weight/cache sets so its bytes come from HBM, timed with HIP events on the backend's stream
+    # per-stage launch times of the graph form: each of the six stage kernels alone (its 12 launches per step as one graph),
+    # rotating over the same weight/cache sets so its bytes come from HBM, timed with HIP events on the backend's stream
     stage_us = []
-    batch = len(streams)
     reps = max(4, steps // 4)
-    for stage in range(6):
+    for stage in range(6 if stages else 0):
         for i in range(2 * rotate):
             sets[i % rotate]["dec"].stage_enqueue(batch, stage)
         backend.sync()
@@ -97,7 +113,8 @@ def time_config(pkg, synth, backend, qtype, lengths, mems, capacity, steps, warm
         stage_us.append(backend.timer_end() * 1000.0 / (reps * cfg["layers"]))
     for s in sets:
         s["dec"].destroy()
-    return {"step_us": step_us, "bytes": total, "weight_bytes": b["weights"] + head_bytes, "kv_bytes": b["kv"],
+    return {"step_us": step_us, "stack_us": stack_us, "persistent_step_us": persistent_us, "persistent_stack_us": persistent_stack_us, "bytes": total,
+            "stack_bytes": b["total"], "weight_bytes": b["weights"] + head_bytes, "kv_bytes": b["kv"],
             "gbps": total / (step_us * 1e-6) / 1e9, "setup_s": setup_s, "stage_us": stage_us,
             "stage_bytes": b["stage_bytes_per_launch"], "layers": cfg["layers"]}
 
@@ -235,33 +252,57 @@ def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
     return {"frames": frames, "samples": int(L), "ms": ms, "flops": flops, "tflops": flops / (ms * 1e-3) / 1e12}
 
 
-STAGES = [("self-attention", "k_step_attention: LayerNorm + int8 act-quant + per-head Q/K/V rows + KV append + attention over the self cache"),
-          ("self-out", "k_linear: fold of attention partials + act-quant + O matvec + residual"),
-          ("cross-attention", "k_step_attention: LayerNorm + act-quant + per-head Q rows + attention over the cross cache"),
-          ("cross-out", "k_linear: fold + act-quant + O matvec + residual"),
-          ("ffn-up", "k_linear: LayerNorm + act-quant + up matvec + GELU"),
-          ("ffn-down", "k_linear: act-quant + down matvec + residual")]
+STAGES = [("self-attention", "k_step_attention<self>", "LayerNorm + int8 act-quant + per-head Q/K/V rows + KV append + attention over the self cache"),
+          ("self-out", "k_linear<k=768, residual>", "fold of attention partials + act-quant + O matvec + residual"),
+          ("cross-attention", "k_step_attention<cross>", "LayerNorm + act-quant + per-head Q rows + attention over the cross cache"),
+          ("cross-out", "k_linear<k=768, residual>", "fold + act-quant + O matvec + residual"),
+          ("ffn-up", "k_linear<k=768, LayerNorm, GELU>", "LayerNorm + act-quant + up matvec + GELU"),
+          ("ffn-down", "k_linear<k=3072, residual>", "act-quant + down matvec + residual")]
 
-# HBM bytes per launch (batch 1) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same counter
-# reads for the library's plain 256 MiB read+write kernel: x2.000 and x1.000); the summary with the commands is
-# profiles/decode_step_int8_hbm_counters.md.  Valid for the int8 workload these were measured on.
-MEASURED_TRAFFIC = {"self-attention": 8543923, "cross-attention": 2695632, "self-out": 942538, "cross-out": 942538,
-                    "ffn-up": 2540386, "ffn-down": 2656109}
+# HBM bytes per launch of the dominant kernel of the batch-1 int8 line, from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE), each scaled by what the same counter reads for the library's plain 256 MiB read+write kernel.  The figure
+# belongs to the kernel sources it was measured on: it is reported only while their hash is the one recorded here.
+MEASURED_TRAFFIC = {"kernel": None, "bytes": None, "profile": None, "csrc_sha256": None}
+
+
+def csrc_hash():
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(ROOT, "mynah-tts_amd", "csrc", "*"))):
+        with open(path, "rb") as f:
+            h.update(os.path.basename(path).encode())
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def roofline(r):
-    """The dominant kernel = the stage with the largest share of the step; achieved = its algorithmic bytes per launch
-    over its average launch time (HIP events around graphs holding only that stage, all layers, sets rotating)."""
+    """The dominant kernel is chosen by kernel symbol: launches of one template instance are summed (the two output
+    projections of a layer are the same kernel), and the instance with the largest share of the step is the one whose
+    achieved = average algorithmic bytes per launch over average launch time (HIP events around graphs holding only that
+    stage, all layers, sets rotating) goes into the line.  The per-stage list is given as well."""
     rows = []
-    for (name, what), us, nbytes in zip(STAGES, r["stage_us"], r["stage_bytes"]):
-        rows.append({"stage": name, "kernel": what, "launch_us": round(us, 3), "algorithmic_bytes_per_launch": nbytes,
+    for (name, symbol, what), us, nbytes in zip(STAGES, r["stage_us"], r["stage_bytes"]):
+        rows.append({"stage": name, "kernel": symbol, "does": what, "launch_us": round(us, 3), "algorithmic_bytes_per_launch": nbytes,
                      "gbps": round(nbytes / (us * 1e-6) / 1e9, 1), "frac": round(nbytes / (us * 1e-6) / 1e9 / PEAK_GBPS, 4),
                      "share_of_step": round(us * r["layers"] / r["step_us"], 3)})
-    top = max(rows, key=lambda x: x["share_of_step"])
-    return {"bound": "hbm", "kernel": top["stage"] + " stage = " + top["kernel"], "achieved": top["gbps"], "peak": PEAK_GBPS,
-            "unit": "GB/s", "frac": top["frac"], "traffic": MEASURED_TRAFFIC.get(top["stage"]) if r.get("traffic_valid") else None,
-            "launch_us": top["launch_us"], "algorithmic_bytes_per_launch": top["algorithmic_bytes_per_launch"],
-            "stages": rows,
+    groups = {}
+    for row in rows:
+        g = groups.setdefault(row["kernel"], {"us": 0.0, "bytes": 0, "launches": 0})
+        g["us"] += row["launch_us"]
+        g["bytes"] += row["algorithmic_bytes_per_launch"]
+        g["launches"] += 1
+    name, g = max(groups.items(), key=lambda kv: kv[1]["us"])
+    kernel, launch_us, nbytes = name, g["us"] / g["launches"], g["bytes"] // g["launches"]
+    share = g["us"] * r["layers"] / r["step_us"]
+    gbps = nbytes / (launch_us * 1e-6) / 1e9
+    traffic = None
+    if r.get("traffic_valid") and MEASURED_TRAFFIC["bytes"] is not None and MEASURED_TRAFFIC["csrc_sha256"] == csrc_hash():
+        traffic = MEASURED_TRAFFIC["bytes"]
+    return {"bound": "hbm", "kernel": kernel, "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / PEAK_GBPS, 4),
+            "traffic": traffic, "traffic_source": MEASURED_TRAFFIC["profile"] if traffic is not None else None,
+            "launch_us": round(launch_us, 3), "algorithmic_bytes_per_launch": nbytes, "share_of_step": round(share, 3),
+            "launches_per_step": g["launches"] * r["layers"], "stages": rows,
             "whole_step": {"step_us": round(r["step_us"], 2), "algorithmic_bytes_per_step": r["bytes"], "weight_bytes": r["weight_bytes"],
                            "kv_bytes": r["kv_bytes"], "gbps": round(r["gbps"], 2), "frac": round(r["gbps"] / PEAK_GBPS, 4)}}
 
@@ -293,10 +334,10 @@ def main():
     ap.add_argument("--quant", default="int8", choices=["int8", "int4", "f16", "f32"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--skip-b8", action="store_true")
+    ap.add_argument("--skip-int4", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true")
     ap.add_argument("--skip-local", action="store_true")
     ap.add_argument("--skip-codec", action="store_true")
-    ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the library's plain read+write kernel over 256 MiB three times (a known-size reference for "
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -310,8 +351,6 @@ def main():
     import mynah_tts_amd.synth as synth
     qtype = {"f32": pkg.F32, "int8": pkg.INT8, "int4": pkg.INT4, "f16": pkg.F16}[args.quant]
     backend = pkg.Backend(quant=qtype)
-    if args.no_graph:
-        backend.set_graph_mode(False)
     if args.calibrate:
         for _ in range(3):
             backend.flush_cache(256 << 20)
@@ -319,6 +358,10 @@ def main():
 
     b1 = time_config(pkg, synth, backend, qtype, [1023], [256], 1024, args.steps, args.warmup)
     b1["traffic_valid"] = args.quant == "int8"
+    int4 = None
+    if args.quant == "int8" and not args.skip_int4:
+        int4 = time_config(pkg, synth, backend, pkg.INT4, [1023], [256], 1024, max(args.steps // 3, 20), max(args.warmup // 3, 6), stages=False)
+        backend.set_quant(qtype)
     b8 = None
     if not args.skip_b8:
         self_len, cross_len = synth.ragged_lengths(8, seed=3)
@@ -349,9 +392,21 @@ def main():
         "config": {"workload": "12-layer d=768 decoder stack decode step, %s weights, batch 1, self-KV 1024, cross-KV 256 "
                                "(12x64 heads), final LayerNorm + 768->8x1024 output head + softmax" % args.quant,
                    "batch": 1, "layers": 12, "width": 768, "self_kv": 1024, "cross_kv": 256, "quant": args.quant,
-                   "graph": not args.no_graph, "rotating_sets": ROTATE},
+                   "step_form": "captured graph of stage kernels",
+                   "rotating_sets": ROTATE},
         "roofline": roofline(b1),
     }
+    if b1["persistent_step_us"] is not None:
+        result["persistent_form"] = {"what": "the same step as ONE persistent launch (graph mode 2, opt-in): stage hand-overs through tagged "
+                                             "(value, tag) pairs in memory instead of kernel boundaries",
+                                     "step_us": round(b1["persistent_step_us"], 2), "stack_launch_us": round(b1["persistent_stack_us"], 2),
+                                     "stack_algorithmic_bytes": b1["stack_bytes"],
+                                     "frac": round(b1["stack_bytes"] / (b1["persistent_stack_us"] * 1e-6) / 1e9 / PEAK_GBPS, 4)}
+    if int4 is not None:
+        result["int4_b1"] = {"workload": "the same stack and lengths with int4 group-32 weights, batch 1, + output head",
+                             "step_us": round(int4["step_us"], 2), "persistent_step_us": round(int4["persistent_step_us"], 2),
+                             "algorithmic_bytes_per_step": int4["bytes"], "gbps": round(int4["gbps"], 2),
+                             "pct_of_peak": round(100.0 * int4["gbps"] / PEAK_GBPS, 2)}
     if b8 is not None:
         result["b8"] = {"step_us": round(b8["step_us"], 2), "gbps": round(b8["gbps"], 2),
                         "pct_of_peak": round(100.0 * b8["gbps"] / PEAK_GBPS, 2), "algorithmic_bytes_per_step": b8["bytes"],

@@ -380,10 +380,12 @@ int mynah_hip_timer_end(void *state, float *milliseconds, char *error, size_t er
 /* Streams `bytes` of backend-owned scratch through the chip (read+write) so that the last-level
  * cache holds none of the caller's data: used between timed iterations. */
 int mynah_hip_flush_cache(void *state, size_t bytes, char *error, size_t error_capacity);
-/* How mynah_hip_decoder_step runs: 0 = every stage kernel a launch of its own, 1 = the step replayed as a captured HIP
- * graph, 2 (default) = one persistent launch for the whole step where it applies (one or two streams, int8 / int4
- * weights, width 768 / FFN 3072 / 64-wide heads, at most one attention unit per compute unit), else as 1.  All three give
- * the same bits.  MYNAH_HIP_GRAPH in the environment at open sets the initial value. */
+/* How mynah_hip_decoder_step runs: 0 = every stage kernel a launch of its own, 1 (default) = the step replayed as a
+ * captured HIP graph, 2 = one persistent launch for the whole step where it applies (one or two streams, int8 / int4
+ * weights, width 768 / FFN 3072 / 64-wide heads, attention units and row stages fitting the chip side by side), else as
+ * 1.  All three give the same bits.  Form 2 waits inside the kernel for other workgroups' results; every such wait is
+ * bounded (MYNAH_HIP_PERSIST_SPIN polls, default 2^20), and a step that gave one up is reported by the next call that
+ * synchronises.  MYNAH_HIP_GRAPH in the environment at open sets the initial value. */
 int mynah_hip_set_graph_mode(void *state, int enabled, char *error, size_t error_capacity);
 /* Bytes of device memory held by the weight cache (packed weights + scales + vectors). */
 size_t mynah_hip_cached_weight_bytes(void *state);

@@ -507,7 +507,7 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
     if (arith != nullptr && strcmp(arith, "stock") == 0) st->arith = MYNAH_HIP_ARITH_STOCK;
     const char *fuse = getenv("MYNAH_HIP_FUSE");   // 0: every seam call is a launch of its own
     if (fuse != nullptr && strcmp(fuse, "0") == 0) st->fuse = 0;
-    const char *graph = getenv("MYNAH_HIP_GRAPH");   // 0: every stage a launch, 1: captured graph, 2 (default): persistent launch where it applies
+    const char *graph = getenv("MYNAH_HIP_GRAPH");   // 0: every stage a launch, 1 (default): captured graph, 2: persistent launch where it applies
     if (graph != nullptr && (strcmp(graph, "0") == 0 || strcmp(graph, "1") == 0 || strcmp(graph, "2") == 0)) st->graph_mode = graph[0] - '0';
     const char *spin = getenv("MYNAH_HIP_PERSIST_SPIN");
     if (spin != nullptr && spin[0] != '\0') st->persist_spin_limit = (unsigned)strtoul(spin, nullptr, 10);

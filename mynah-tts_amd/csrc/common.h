@@ -103,7 +103,7 @@ struct State {
     int cu_count = 256;
     int qtype = MYNAH_HIP_F32;
     int arith = MYNAH_HIP_ARITH_STRICT;
-    int graph_mode = 2;   // resident step: 0 = every stage kernel a launch, 1 = captured graph, 2 = one persistent launch where it applies (else graph)
+    int graph_mode = 1;   // resident step: 0 = every stage kernel a launch, 1 = captured graph, 2 = one persistent launch where it applies (else graph)
     // persistent step: word a workgroup sets when a bounded wait gave up (pinned host memory, mapped), polls a wait may make,
     // and an override of the row stages' workgroup count (0 = chosen from the batch)
     unsigned *persist_abort_host = nullptr;

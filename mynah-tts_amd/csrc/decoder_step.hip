@@ -382,6 +382,14 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
     return 0;
 }
 
+#ifdef MYNAH_PERSIST_PROBE
+static unsigned long long *g_persist_probe = nullptr;
+extern "C" int mynah_hip_debug_probe(unsigned long long *host, size_t words) {   // development builds only
+    if (g_persist_probe == nullptr) return -1;
+    return hipMemcpy(host, g_persist_probe, words * sizeof(unsigned long long), hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
+}
+#endif
+
 namespace mynah {
 
 // The step as one persistent launch, when this batch fits it: one or two streams, int8 / int4 weights, the stack's own
@@ -417,19 +425,29 @@ static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_
     a.abort_word = st->persist_abort_dev;
     const int grid = st->cu_count;
     const int attn = step_persistent_attention_workgroups(a);
-    if (attn > grid) return 0;
+    a.attention_wgs = attn;
     // Row stages count their workgroups from the end of the grid, attention roles from its start: with room for both, a
     // workgroup has one kind of role and requests its next stage's operands a whole stage ahead.
-    const int pass768 = 4 * (64 >> lane_group_log2(768 / (d->qtype == MYNAH_HIP_INT8 ? 16 : 32)));
-    int free_wgs = grid - attn;
-    int wide = st->persist_row_wgs > 0 ? st->persist_row_wgs : (free_wgs >= 96 ? (free_wgs < 192 ? free_wgs : 192) : 192);
-    if (wide > grid) wide = grid;
-    a.rows_out = pass768;
+    // Row stages count their workgroups from the end of the grid, attention roles from its start: with room for both a
+    // workgroup has one kind of role.  Rows per workgroup are what the kernel requests ahead (32 rows of an output
+    // projection and of FFN up, 8 of FFN down); MYNAH_HIP_PERSIST_ROW_WGS spreads the FFN rows over more workgroups.
+    a.rows_out = 32;
     a.wgs_out = (768 + a.rows_out - 1) / a.rows_out;
-    a.rows_up = (3072 + wide - 1) / wide;
+    a.rows_up = 32;
+    a.rows_down = 8;
+    if (st->persist_row_wgs > 0) {
+        const int wide = st->persist_row_wgs < grid ? st->persist_row_wgs : grid;
+        a.rows_up = (3072 + wide - 1) / wide;
+        a.rows_down = (768 + wide - 1) / wide;
+    }
     a.wgs_up = (3072 + a.rows_up - 1) / a.rows_up;
-    a.rows_down = (768 + wide - 1) / wide;
     a.wgs_down = (768 + a.rows_down - 1) / a.rows_down;
+    {
+        // a workgroup has one kind of role: when the attention units of these lengths and the row stages do not fit the grid
+        // side by side, the step takes the launched-kernels path
+        const int rows = a.wgs_up > a.wgs_down ? (a.wgs_up > a.wgs_out ? a.wgs_up : a.wgs_out) : (a.wgs_down > a.wgs_out ? a.wgs_down : a.wgs_out);
+        if (attn + rows > grid || (int)batch > rows) return 0;
+    }
     const unsigned span = 8u * (unsigned)(d->layers + 2);
     if (d->persist_epoch > 0xffffffffu - 2u * span) {   // the tag counter is about to wrap: start over on a cleared area
         if (hip_check(hipMemsetAsync(d->persist_exchange, 0, d->persist_exchange_words * sizeof(unsigned long long), st->stream), "exchange clear", error,
@@ -439,6 +457,16 @@ static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_
     }
     a.epoch = d->persist_epoch;
     d->persist_epoch += span;
+#ifdef MYNAH_PERSIST_PROBE
+    {
+        static unsigned long long *probe = nullptr;
+        if (probe == nullptr && hipMalloc(reinterpret_cast<void **>(&probe), 1024 * 32 * sizeof(unsigned long long)) != hipSuccess) probe = nullptr;
+        const char *layer = getenv("MYNAH_PERSIST_PROBE_LAYER");
+        a.probe = probe;
+        a.probe_layer = layer != nullptr ? atoi(layer) : 5;
+        g_persist_probe = probe;
+    }
+#endif
     if (launch_step_persistent(st, a, d->qtype, grid, error, capacity) != 0) return -1;
     return 1;
 }

@@ -129,9 +129,14 @@ struct PersistArgs {
     unsigned epoch;                 // tags of this step start here; a step uses 8 * (layers + 1) of them
     unsigned spin_limit;            // polls a wait may make before the step is given up
     unsigned *abort_word;           // set when a wait gave up (host-visible)
+    int attention_wgs;              // workgroups [0, attention_wgs) run the attention stages, the row stages count from the grid's end
     int wgs_out, rows_out;          // workgroups and rows per workgroup of the [768, 768] output projections
     int wgs_up, rows_up;            // ... of FFN up [3072, 768]
     int wgs_down, rows_down;        // ... of FFN down [768, 3072]
+#ifdef MYNAH_PERSIST_PROBE
+    unsigned long long *probe;      // development builds only: [workgroup][32] clock readings of layer probe_layer
+    int probe_layer;
+#endif
 };
 bool step_persistent_supported(int qtype, size_t width, size_t heads, size_t head_width, size_t ffn, size_t cross_heads, size_t cross_head_width);
 size_t step_persistent_exchange_words(const PersistArgs &args);

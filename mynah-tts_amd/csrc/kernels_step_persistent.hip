@@ -53,28 +53,62 @@ __device__ __forceinline__ bool give_up(Waiter &w, unsigned &spins) {
     return false;
 }
 
-// n tagged values -> dst (LDS floats, same index), by the whole workgroup, N requests in flight per thread.  Every request
-// is issued whatever the index (clamped), so that none sits behind a branch.
-template <int N>
+// A poll is a request that bypasses the caches, about a microsecond there and back.  Polling one request at a time finds a
+// value, on average, half a round trip after it could have; two requests in flight, checked in turn, halve that.
+__device__ __forceinline__ void poll_until(const u64 *p, const unsigned tag, Waiter &w) {
+    unsigned spins = 0;
+    u64 first = get(p), second = get(p);
+    while (tag_of(first) != tag) {
+        if (give_up(w, spins)) { w.dead = true; break; }
+        first = second;
+        second = get(p);
+    }
+}
+
+// n tagged values -> dst (LDS floats, same index), by the whole workgroup, N values per thread and batch.  Every request
+// is issued whatever the index (clamped), so that none sits behind a branch.  The batch itself is the poll, and two
+// batches are in flight: while one is looked at the next is already on its way, so a value is found a fraction of a
+// round trip after it became visible instead of half a round trip (one batch in flight) or a whole one (poll one value,
+// then request the batch).  WAIT_FIRST: poll one value of the batch before the first batch is requested -- for batches of
+// tens of values, which many workgroups would otherwise request over and over while the producers are still at work.
+template <int N, bool WAIT_FIRST>
 __device__ __forceinline__ void fetch_tagged(const u64 *src, float *dst, const int n, const unsigned tag, Waiter &w) {
     const int tid = threadIdx.x;
     for (int base = 0; base < n; base += kThreads * N) {
-        u64 v[N];
+        u64 v[N], next[N];
         unsigned spins = 0;
-        for (;;) {
+        if (WAIT_FIRST) {
+            int last = base + (N - 1) * kThreads + tid;
+            while (last >= n) last -= kThreads;
+            if (last >= base) poll_until(src + last, tag, w);
+        }
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int i = base + j * kThreads + tid;
+            v[j] = get(src + (i < n ? i : n - 1));
+        }
+        if (!WAIT_FIRST) {
 #pragma unroll
             for (int j = 0; j < N; ++j) {
                 const int i = base + j * kThreads + tid;
-                v[j] = get(src + (i < n ? i : n - 1));
+                next[j] = get(src + (i < n ? i : n - 1));
             }
+        }
+        for (;;) {
             bool all = true;
 #pragma unroll
             for (int j = 0; j < N; ++j) {
                 const int i = base + j * kThreads + tid;
                 all = all && (i >= n || tag_of(v[j]) == tag);
             }
-            if (all) break;
+            if (all || w.dead) break;
             if (give_up(w, spins)) { w.dead = true; break; }
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                const int i = base + j * kThreads + tid;
+                v[j] = WAIT_FIRST ? get(src + (i < n ? i : n - 1)) : next[j];
+                if (!WAIT_FIRST) next[j] = get(src + (i < n ? i : n - 1));
+            }
         }
 #pragma unroll
         for (int j = 0; j < N; ++j) {
@@ -324,12 +358,14 @@ __device__ __forceinline__ void attention_compute(AttnRegs &g, const AttnRole &r
 
 // ---- matvec stages -------------------------------------------------------------------------------------------------------
 
-template <int BT, int NVT>
+// Operands of a row role requested ahead: the first P passes of its rows (a pass = the 4 x (64 / lane group) rows the
+// workgroup's four wavefronts take at a time); passes beyond P are requested when their turn comes.
+template <int BT, int NVT, int P>
 struct RowRegs {
-    uint4 wv[4];
-    float sc[4];
-    float ws;
-    u64 res;            // the residual value of this lane's (row, stream), tagged
+    uint4 wv[P][4];
+    float sc[P][4];
+    float ws[P];
+    u64 res[P];         // the residual value of this lane's (row, stream), tagged
     float4 gv[NVT], bv[NVT];
 };
 
@@ -348,29 +384,33 @@ __device__ __forceinline__ u64 residual_request(const Residual &src, const int s
     return ((u64)src.tag << 32) | (u64)__float_as_uint(v);
 }
 
-template <int QT, int BT, int NVT, int K>
-__device__ __forceinline__ void rows_request(RowRegs<BT, NVT> &g, const RowRole &r, const void *w, const float *scales, const bool with_res,
+template <int QT, int BT, int NVT, int K, int P>
+__device__ __forceinline__ void rows_request(RowRegs<BT, NVT, P> &g, const RowRole &r, const void *w, const float *scales, const bool with_res,
                                              const Residual &res, const int batch, const float *gain, const float *bias) {
     constexpr int kEpc = Chunk<QT>::n;
     constexpr int chunks = K / kEpc;
     constexpr int lg = lane_group_log2(chunks);
     constexpr int G = 1 << lg;
+    constexpr int rpp = 64 >> lg;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int gl = lane & (G - 1), gidx = lane >> lg;
-    const int row = r.row_begin + wave * (64 >> lg) + gidx;
-    const int rowc = row < r.row_end ? row : r.row_end - 1;
-    const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(w) + (size_t)rowc * chunks * 16);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const int c = gl + u * G;
-        g.wv[u] = c < chunks ? load_global_u4(wrow + c) : make_uint4(0, 0, 0, 0);
-        g.sc[u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? load_global(scales + (size_t)rowc * chunks + c) : 0.0f;
-    }
-    g.ws = 1.0f;
-    g.res = 0;
-    if (gl < BT) {
-        if constexpr (QT == MYNAH_HIP_INT8) g.ws = load_global(scales + rowc);
-        if (with_res && gl < batch) g.res = residual_request(res, gl, rowc);
+    for (int p = 0; p < P; ++p) {
+        const int row = r.row_begin + p * 4 * rpp + wave * rpp + gidx;
+        const int rowc = row < r.row_end ? row : r.row_end - 1;
+        const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(w) + (size_t)rowc * chunks * 16);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = gl + u * G;
+            g.wv[p][u] = c < chunks ? load_global_u4(wrow + c) : make_uint4(0, 0, 0, 0);
+            g.sc[p][u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? load_global(scales + (size_t)rowc * chunks + c) : 0.0f;
+        }
+        g.ws[p] = 1.0f;
+        g.res[p] = 0;
+        if (gl < BT) {
+            if constexpr (QT == MYNAH_HIP_INT8) g.ws[p] = load_global(scales + rowc);
+            if (with_res && gl < batch) g.res[p] = residual_request(res, gl, rowc);
+        }
     }
 #pragma unroll
     for (int i = 0; i < NVT; ++i) {
@@ -380,63 +420,99 @@ __device__ __forceinline__ void rows_request(RowRegs<BT, NVT> &g, const RowRole 
     }
 }
 
-// Products of the role's rows against the activations staged in smem, epilogue, tagged stores.  Lane b of a row's lane
-// group finishes stream b.  EPI: EPI_GELU or EPI_RESIDUAL.
-template <int QT, int BT, int NVT, int K, int EPI>
-__device__ __forceinline__ void rows_compute(RowRegs<BT, NVT> &g, const RowRole &r, const void *w, const float *scales, const Residual &res,
-                                             const int batch, const unsigned char *smem, const float *s_sx, u64 *dst, const int dst_stride,
-                                             const unsigned tag, Waiter &wt) {
+// The residual values of a role's requested passes alone (for a role whose weights were requested while the residual
+// stream was still being written).
+template <int QT, int BT, int NVT, int K, int P>
+__device__ __forceinline__ void rows_request_residual(RowRegs<BT, NVT, P> &g, const RowRole &r, const Residual &res, const int batch) {
+    constexpr int lg = lane_group_log2(K / Chunk<QT>::n);
+    constexpr int G = 1 << lg;
+    constexpr int rpp = 64 >> lg;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gl = lane & (G - 1), gidx = lane >> lg;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+        const int row = r.row_begin + p * 4 * rpp + wave * rpp + gidx;
+        const int rowc = row < r.row_end ? row : r.row_end - 1;
+        if (gl < BT && gl < batch) g.res[p] = residual_request(res, gl, rowc);
+    }
+}
+
+// One pass of rows: products against the activations staged in smem, lane-group reduction, epilogue, tagged stores.
+// Lane b of a row's lane group finishes stream b.  EPI: EPI_GELU or EPI_RESIDUAL.
+template <int QT, int BT, int K, int EPI>
+__device__ __forceinline__ void rows_pass(const uint4 (&wv)[4], const float (&sc)[4], const float ws, const u64 resv, const int row, const bool valid,
+                                          const Residual &res, const int batch, const unsigned char *smem, const float *s_sx, u64 *dst,
+                                          const int dst_stride, const unsigned tag, Waiter &wt) {
     constexpr int kEpc = Chunk<QT>::n;
     constexpr int chunks = K / kEpc;
     constexpr int lg = lane_group_log2(chunks);
     constexpr int G = 1 << lg;
     static_assert(G >= BT, "a lane group must have a lane per stream");
     static_assert((chunks + G - 1) / G <= 4, "one register group of four chunks per lane");
+    const int gl = (threadIdx.x & 63) & (G - 1);
+    int iacc[BT];
+    float facc[BT];
+#pragma unroll
+    for (int b = 0; b < BT; ++b) { iacc[b] = 0; facc[b] = 0.0f; }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int c = gl + u * G;
+        if (c < chunks) dot_chunk<QT, BT>(wv[u], sc[u], c, smem, K, iacc, facc, nullptr);
+    }
+    group_reduce<QT, BT>(iacc, facc, lg);
+    if (gl < batch && valid) {
+        int mi = iacc[0];
+        float mf = facc[0];
+#pragma unroll
+        for (int b = 1; b < BT; ++b)
+            if (gl == b) { mi = iacc[b]; mf = facc[b]; }
+        float val = finish_value<QT>(mi, mf, ws, s_sx[gl]);
+        if (EPI == EPI_GELU) val = gelu_tanh(val);
+        if (EPI == EPI_RESIDUAL) {
+            const float before = res.tagged != nullptr ? settle(resv, res.tagged + (size_t)gl * kW + row, res.tag, wt) : value_of(resv);
+            val = before + val;
+        }
+        put(dst + (size_t)gl * dst_stride + row, tag, val);
+    }
+}
+
+template <int QT, int BT, int NVT, int K, int P, int EPI>
+__device__ __forceinline__ void rows_compute(RowRegs<BT, NVT, P> &g, const RowRole &r, const void *w, const float *scales, const Residual &res,
+                                             const int batch, const unsigned char *smem, const float *s_sx, u64 *dst, const int dst_stride,
+                                             const unsigned tag, Waiter &wt) {
+    constexpr int kEpc = Chunk<QT>::n;
+    constexpr int chunks = K / kEpc;
+    constexpr int lg = lane_group_log2(chunks);
+    constexpr int G = 1 << lg;
+    constexpr int rpp = 64 >> lg;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int gl = lane & (G - 1), gidx = lane >> lg;
-    constexpr int rpp = 64 >> lg;
-    bool first = true;
-    for (int base = r.row_begin + wave * rpp; base < r.row_end; base += 4 * rpp) {
+#pragma unroll
+    for (int p = 0; p < P; ++p) {   // the passes requested ahead
+        const int row = r.row_begin + p * 4 * rpp + wave * rpp + gidx;
+        if (r.row_begin + p * 4 * rpp + wave * rpp < r.row_end)   // the same for the whole wavefront
+            rows_pass<QT, BT, K, EPI>(g.wv[p], g.sc[p], g.ws[p], g.res[p], row, row < r.row_end, res, batch, smem, s_sx, dst, dst_stride, tag, wt);
+    }
+    for (int base = r.row_begin + P * 4 * rpp + wave * rpp; base < r.row_end; base += 4 * rpp) {   // any further pass
         const int row = base + gidx;
         const bool valid = row < r.row_end;
         const int rowc = valid ? row : r.row_end - 1;
-        if (!first) {
-            const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(w) + (size_t)rowc * chunks * 16);
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int c = gl + u * G;
-                g.wv[u] = c < chunks ? load_global_u4(wrow + c) : make_uint4(0, 0, 0, 0);
-                g.sc[u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? load_global(scales + (size_t)rowc * chunks + c) : 0.0f;
-            }
-        }
-        int iacc[BT];
-        float facc[BT];
-#pragma unroll
-        for (int b = 0; b < BT; ++b) { iacc[b] = 0; facc[b] = 0.0f; }
+        const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(w) + (size_t)rowc * chunks * 16);
+        uint4 wv[4];
+        float sc[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int c = gl + u * G;
-            if (c < chunks) dot_chunk<QT, BT>(g.wv[u], g.sc[u], c, smem, K, iacc, facc, nullptr);
+            wv[u] = c < chunks ? load_global_u4(wrow + c) : make_uint4(0, 0, 0, 0);
+            sc[u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? load_global(scales + (size_t)rowc * chunks + c) : 0.0f;
         }
-        group_reduce<QT, BT>(iacc, facc, lg);
+        float ws = 1.0f;
+        u64 resv = 0;
         if (gl < batch && valid) {
-            int mi = iacc[0];
-            float mf = facc[0];
-#pragma unroll
-            for (int b = 1; b < BT; ++b)
-                if (gl == b) { mi = iacc[b]; mf = facc[b]; }
-            float wscale = 1.0f;
-            if constexpr (QT == MYNAH_HIP_INT8) wscale = first ? g.ws : load_global(scales + row);
-            float val = finish_value<QT>(mi, mf, wscale, s_sx[gl]);
-            if (EPI == EPI_GELU) val = gelu_tanh(val);
-            if (EPI == EPI_RESIDUAL) {
-                const u64 rv = first ? g.res : residual_request(res, gl, row);
-                const float before = res.tagged != nullptr ? settle(rv, res.tagged + (size_t)gl * kW + row, res.tag, wt) : value_of(rv);
-                val = before + val;
-            }
-            put(dst + (size_t)gl * dst_stride + row, tag, val);
+            if constexpr (QT == MYNAH_HIP_INT8) ws = load_global(scales + row);
+            if (EPI == EPI_RESIDUAL) resv = residual_request(res, gl, row);
         }
-        first = false;
+        rows_pass<QT, BT, K, EPI>(wv, sc, ws, resv, row, valid, res, batch, smem, s_sx, dst, dst_stride, tag, wt);
     }
 }
 
@@ -466,6 +542,306 @@ __device__ __forceinline__ float4 fold_from_lds(const float *rec, const int rec_
 
 // ---- the kernel ------------------------------------------------------------------------------------------------------------
 
+// What both kinds of workgroup need to find the exchange area's parts and the step's tags.
+struct Exchange {
+    u64 *X6, *X2, *X4, *H, *PS, *PC;
+    size_t ps_stream, pc_stream;
+};
+__device__ __forceinline__ Exchange exchange_of(const PersistArgs &a) {
+    Exchange e;
+    e.X6 = a.exchange;
+    e.X2 = e.X6 + 2 * kW;
+    e.X4 = e.X2 + 2 * kW;
+    e.H = e.X4 + 2 * kW;
+    e.PS = e.H + 2 * kF;
+    e.ps_stream = (size_t)a.max_units * a.heads * kStepRecord;
+    e.PC = e.PS + 2 * e.ps_stream;
+    e.pc_stream = (size_t)a.max_units * (a.cross_heads > 0 ? a.cross_heads : 1) * kStepRecord;
+    return e;
+}
+
+// One stream's kernel arguments as values (an argument array indexed by a run-time stream number would be read with
+// vector loads at every use).
+struct StreamArgs {
+    float *self_k, *self_v;
+    const float *cross_k, *cross_v, *input, *pos_row;
+    float *output;
+    int length, memory_length;
+};
+__device__ __forceinline__ StreamArgs stream_of(const PersistArgs &a, const int b) {
+    StreamArgs s;
+    s.self_k = b == 0 ? a.self_k[0] : a.self_k[1];
+    s.self_v = b == 0 ? a.self_v[0] : a.self_v[1];
+    s.cross_k = b == 0 ? a.cross_k[0] : a.cross_k[1];
+    s.cross_v = b == 0 ? a.cross_v[0] : a.cross_v[1];
+    s.input = b == 0 ? a.input[0] : a.input[1];
+    s.output = b == 0 ? a.output[0] : a.output[1];
+    s.length = b == 0 ? a.length[0] : a.length[1];
+    s.memory_length = b == 0 ? a.memory_length[0] : a.memory_length[1];
+    s.pos_row = a.position != nullptr ? a.position + (size_t)s.length * kW : nullptr;
+    return s;
+}
+
+// a workgroup that cannot go on: say so, and leave (every barrier of this kernel is passed by whole workgroups)
+#define MYNAH_LEAVE_IF_DEAD()                                                                                           \
+    if (__syncthreads_or(wt.dead ? 1 : 0)) {                                                                            \
+        if (threadIdx.x == 0) __hip_atomic_store(a.abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);         \
+        return;                                                                                                         \
+    }
+// development builds only: clock readings (100 MHz) of one layer, per workgroup: slot 3 (stage - 1) + {0 before the wait,
+// 1 input there, 2 stage done}
+#ifdef MYNAH_PERSIST_PROBE
+#define MYNAH_STAMP(slot) do { if (threadIdx.x == 0 && a.probe != nullptr && layer == a.probe_layer) a.probe[(size_t)blockIdx.x * 32 + (slot)] = wall_clock64(); } while (0)
+#else
+#define MYNAH_STAMP(slot) do { } while (0)
+#endif
+
+struct SharedBlocks {
+    float *s_in;
+    unsigned char *smem;
+    float *s_proj, *s_red, *s_wave_ml, *s_sx, *s_scratch, *s4;
+};
+
+// A workgroup of the attention stages: per layer, stage 1 (self) and stage 3 (cross).  Everything of a stage that does not
+// depend on the residual stream is requested as soon as the stage before it is done.
+template <int QT>
+__device__ __forceinline__ void attention_path(const PersistArgs &a, const SharedBlocks &sh, const AttnRole r1, const AttnRole r3) {
+    const int tid = threadIdx.x;
+    const Exchange ex = exchange_of(a);
+    Waiter wt{a.spin_limit, a.abort_word, false};
+    const StreamArgs s1 = stream_of(a, r1.b), s3 = stream_of(a, r3.b);
+    const int stride_self = a.heads * kHw, stride_cross = a.cross_heads * kHw;
+    StepAttnArgs aw{};
+    aw.width = kW;
+    aw.arith = a.arith;
+    aw.scale = a.scale;
+    AttnRegs g;
+    if (r1.active) {
+        const PersistLayer &lw = a.layers[0];
+        aw.w = lw.qkv_w; aw.scales = lw.qkv_s; aw.heads = a.heads;
+        attention_request<QT, true>(g, r1, aw, s1.self_k, s1.self_v, s1.input, lw.norm_self, lw.norm_self_b);
+        requests_issued();
+    }
+    for (int layer = 0; layer < a.n_layers; ++layer) {
+        const PersistLayer &lw = a.layers[layer];
+        const unsigned t0 = a.epoch + 8u * (unsigned)layer;
+        if (r1.active) {
+            MYNAH_STAMP(0);
+            if (layer == 0) {
+                for (int i = tid; i < kW; i += kThreads)
+                    sh.s_in[i] = s1.pos_row != nullptr ? load_global(s1.input + i) + load_global(s1.pos_row + i) : load_global(s1.input + i);
+            } else {
+                fetch_tagged<3, false>(ex.X6 + (size_t)r1.b * kW, sh.s_in, kW, t0, wt);
+            }
+            MYNAH_LEAVE_IF_DEAD();
+            MYNAH_STAMP(1);
+            aw.w = lw.qkv_w; aw.scales = lw.qkv_s; aw.heads = a.heads;
+            float *kc = s1.self_k + (size_t)layer * a.capacity * stride_self;
+            float *vc = s1.self_v + (size_t)layer * a.capacity * stride_self;
+            attention_compute<QT>(g, r1, aw, sh.s_in, kc, vc, s1.length, lw.norm_self_b != nullptr, ex.PS + (size_t)r1.b * ex.ps_stream, a.heads,
+                                  t0 + 1u, sh.smem, sh.s_sx, sh.s_scratch, sh.s_proj, sh.s_red, sh.s_wave_ml);
+            MYNAH_STAMP(2);
+        }
+        if (r3.active) {
+            aw.w = lw.qx_w; aw.scales = lw.qx_s; aw.heads = a.cross_heads;
+            const size_t at = (size_t)layer * s3.memory_length * stride_cross;
+            attention_request<QT, false>(g, r3, aw, s3.cross_k != nullptr ? s3.cross_k + at : nullptr, s3.cross_v != nullptr ? s3.cross_v + at : nullptr,
+                                         s3.input, lw.norm_cross, lw.norm_cross_b);
+            requests_issued();
+            MYNAH_STAMP(6);
+            fetch_tagged<3, false>(ex.X2 + (size_t)r3.b * kW, sh.s_in, kW, t0 + 2u, wt);
+            MYNAH_LEAVE_IF_DEAD();
+            MYNAH_STAMP(7);
+            attention_compute<QT>(g, r3, aw, sh.s_in, nullptr, nullptr, 0, lw.norm_cross_b != nullptr, ex.PC + (size_t)r3.b * ex.pc_stream, a.cross_heads,
+                                  t0 + 3u, sh.smem, sh.s_sx, sh.s_scratch, sh.s_proj, sh.s_red, sh.s_wave_ml);
+            MYNAH_STAMP(8);
+        }
+        if (r1.active && layer + 1 < a.n_layers) {
+            const PersistLayer &nx = a.layers[layer + 1];
+            aw.w = nx.qkv_w; aw.scales = nx.qkv_s; aw.heads = a.heads;
+            const size_t at = (size_t)(layer + 1) * a.capacity * stride_self;
+            attention_request<QT, true>(g, r1, aw, s1.self_k + at, s1.self_v + at, s1.input, nx.norm_self, nx.norm_self_b);
+            requests_issued();
+        }
+    }
+}
+
+// A workgroup of the row stages: per layer, stages 2, 4, 5, 6 for its rows, and at the end the final norm of one stream.
+// A stage's weight rows are requested when the stage before it has its input, i.e. they travel during that stage's
+// arithmetic and the wait that follows.
+template <int QT, int BT>
+__device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBlocks &sh, const RowRole r2, const RowRole r5, const RowRole r6,
+                                          const int final_stream) {
+    // passes of rows requested ahead per role: 32 rows of FFN up, 8 of FFN down, one pass of the output projections
+    constexpr int rpp768 = 64 >> lane_group_log2(kW / Chunk<QT>::n), rpp3072 = 64 >> lane_group_log2(kF / Chunk<QT>::n);
+    constexpr int kUpPasses = 32 / (4 * rpp768) > 0 ? 32 / (4 * rpp768) : 1, kDownPasses = 8 / (4 * rpp3072) > 0 ? 8 / (4 * rpp3072) : 1;
+    constexpr int kOutPasses = kUpPasses;   // 32 rows of an output projection: every partial record is read by 24 workgroups
+    const int tid = threadIdx.x;
+    const Exchange ex = exchange_of(a);
+    Waiter wt{a.spin_limit, a.abort_word, false};
+    const StreamArgs sa = stream_of(a, 0), sb = stream_of(a, 1);
+    const bool cross = a.cross_heads > 0;
+    PrologueParams pro;
+    pro.batch = a.batch; pro.arith = a.arith; pro.probe_qx = nullptr; pro.probe_sx = nullptr;
+
+    RowRegs<BT, 1, kOutPasses> g2;
+    if (r2.active) {
+        Residual res0;
+        res0.tagged = nullptr; res0.tag = a.epoch;
+        res0.input[0] = sa.input; res0.input[1] = sb.input; res0.position[0] = sa.pos_row; res0.position[1] = sb.pos_row;
+        rows_request<QT, BT, 1, kW, kOutPasses>(g2, r2, a.layers[0].o_w, a.layers[0].o_s, true, res0, a.batch, nullptr, nullptr);
+        requests_issued();
+    }
+    for (int layer = 0; layer < a.n_layers; ++layer) {
+        const PersistLayer &lw = a.layers[layer];
+        const unsigned t0 = a.epoch + 8u * (unsigned)layer;
+        Residual res_prev;   // x before this layer
+        res_prev.tagged = layer == 0 ? nullptr : ex.X6;
+        res_prev.tag = t0;
+        res_prev.input[0] = sa.input; res_prev.input[1] = sb.input; res_prev.position[0] = sa.pos_row; res_prev.position[1] = sb.pos_row;
+        Residual res2;
+        res2.tagged = ex.X2; res2.tag = t0 + 2u;
+        res2.input[0] = res2.input[1] = nullptr; res2.position[0] = res2.position[1] = nullptr;
+        Residual res_mid = res2;   // x before the FFN: after the cross sublayer when there is one
+        if (cross) { res_mid.tagged = ex.X4; res_mid.tag = t0 + 4u; }
+
+        // ---------------------------------------------------------------- 2: fold + O + residual
+        RowRegs<BT, 1, kOutPasses> g4;
+        if (r2.active) {
+            MYNAH_STAMP(3);
+            int off = 0;
+            for (int b = 0; b < a.batch; ++b) {
+                const int units = ((b == 0 ? sa.length : sb.length) + kStepUnitRows - 1) / kStepUnitRows + 1;
+                const int n = units * a.heads * kStepRecord;
+                fetch_tagged<32, true>(ex.PS + (size_t)b * ex.ps_stream, sh.s_in + off, n, t0 + 1u, wt);
+                off += n;
+            }
+            MYNAH_LEAVE_IF_DEAD();
+            MYNAH_STAMP(4);
+            if (layer > 0) rows_request_residual<QT, BT, 1, kW, kOutPasses>(g2, r2, res_prev, a.batch);   // the partials are there, so the stream they were made from is
+            if (cross) {
+                rows_request<QT, BT, 1, kW, kOutPasses>(g4, r2, lw.ox_w, lw.ox_s, true, res2, a.batch, nullptr, nullptr);
+                requests_issued();
+            }
+            float4 xr[BT][1];
+            off = 0;
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                xr[b][0] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (b < a.batch) {
+                    const int units = ((b == 0 ? sa.length : sb.length) + kStepUnitRows - 1) / kStepUnitRows + 1;
+                    if (tid < kW / 4) xr[b][0] = fold_from_lds(sh.s_in + off, a.heads, units, tid);
+                    off += units * a.heads * kStepRecord;
+                }
+            }
+            pro.k = kW; pro.ln_gain = nullptr; pro.ln_bias = nullptr;
+            finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g2.gv, g2.bv, sh.smem, sh.s_sx, sh.s_scratch);
+            rows_compute<QT, BT, 1, kW, kOutPasses, EPI_RESIDUAL>(g2, r2, lw.o_w, lw.o_s, res_prev, a.batch, sh.smem, sh.s_sx, ex.X2, kW, t0 + 2u, wt);
+            MYNAH_STAMP(5);
+        }
+        // ---------------------------------------------------------------- 4: fold + O + residual (cross)
+        RowRegs<BT, 1, kUpPasses> g5;
+        if (r2.active && cross) {
+            MYNAH_STAMP(9);
+            int off = 0;
+            for (int b = 0; b < a.batch; ++b) {
+                const int units = max(((b == 0 ? sa.memory_length : sb.memory_length) + kStepUnitRows - 1) / kStepUnitRows, 1);
+                const int n = units * a.cross_heads * kStepRecord;
+                fetch_tagged<32, true>(ex.PC + (size_t)b * ex.pc_stream, sh.s_in + off, n, t0 + 3u, wt);
+                off += n;
+            }
+            MYNAH_LEAVE_IF_DEAD();
+            MYNAH_STAMP(10);
+        }
+        if (r5.active) {
+            rows_request<QT, BT, 1, kW, kUpPasses>(g5, r5, lw.up_w, lw.up_s, false, res_mid, a.batch, lw.norm_ff, lw.norm_ff_b);
+            requests_issued();
+        }
+        if (r2.active && cross) {
+            float4 xr[BT][1];
+            int off = 0;
+#pragma unroll
+            for (int b = 0; b < BT; ++b) {
+                xr[b][0] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (b < a.batch) {
+                    const int units = max(((b == 0 ? sa.memory_length : sb.memory_length) + kStepUnitRows - 1) / kStepUnitRows, 1);
+                    if (tid < kW / 4) xr[b][0] = fold_from_lds(sh.s_in + off, a.cross_heads, units, tid);
+                    off += units * a.cross_heads * kStepRecord;
+                }
+            }
+            pro.k = kW; pro.ln_gain = nullptr; pro.ln_bias = nullptr;
+            finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g4.gv, g4.bv, sh.smem, sh.s_sx, sh.s_scratch);
+            rows_compute<QT, BT, 1, kW, kOutPasses, EPI_RESIDUAL>(g4, r2, lw.ox_w, lw.ox_s, res2, a.batch, sh.smem, sh.s_sx, ex.X4, kW, t0 + 4u, wt);
+            MYNAH_STAMP(11);
+        }
+        // ---------------------------------------------------------------- 5: LN + up + GELU
+        RowRegs<BT, 3, kDownPasses> g6;
+        if (r5.active) {
+            MYNAH_STAMP(12);
+            fetch_tagged<3 * BT, false>(res_mid.tagged, sh.s_in, a.batch * kW, res_mid.tag, wt);
+            MYNAH_LEAVE_IF_DEAD();
+            MYNAH_STAMP(13);
+        }
+        if (r6.active) {
+            rows_request<QT, BT, 3, kF, kDownPasses>(g6, r6, lw.down_w, lw.down_s, true, res_mid, a.batch, nullptr, nullptr);
+            requests_issued();
+        }
+        if (r5.active) {
+            float4 xr[BT][1];
+#pragma unroll
+            for (int b = 0; b < BT; ++b)
+                xr[b][0] = (b < a.batch && tid < kW / 4) ? reinterpret_cast<const float4 *>(sh.s_in)[b * (kW / 4) + tid] : make_float4(0.f, 0.f, 0.f, 0.f);
+            pro.k = kW; pro.ln_gain = lw.norm_ff; pro.ln_bias = lw.norm_ff_b;
+            finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g5.gv, g5.bv, sh.smem, sh.s_sx, sh.s_scratch);
+            MYNAH_STAMP(18);
+            rows_compute<QT, BT, 1, kW, kUpPasses, EPI_GELU>(g5, r5, lw.up_w, lw.up_s, res_mid, a.batch, sh.smem, sh.s_sx, ex.H, kF, t0 + 5u, wt);
+            MYNAH_STAMP(14);
+        }
+        // ---------------------------------------------------------------- 6: down + residual
+        if (r6.active) {
+            MYNAH_STAMP(15);
+            fetch_tagged<12 * BT, true>(ex.H, sh.s_in, a.batch * kF, t0 + 5u, wt);
+            MYNAH_LEAVE_IF_DEAD();
+            MYNAH_STAMP(16);
+        }
+        if (r2.active && layer + 1 < a.n_layers) {
+            Residual res_next;
+            res_next.tagged = ex.X6; res_next.tag = t0 + 8u;
+            res_next.input[0] = res_next.input[1] = nullptr; res_next.position[0] = res_next.position[1] = nullptr;
+            // the weights only: this layer's residual stream is still being written (the row's value is polled for at its use)
+            rows_request<QT, BT, 1, kW, kOutPasses>(g2, r2, a.layers[layer + 1].o_w, a.layers[layer + 1].o_s, false, res_next, a.batch, nullptr, nullptr);
+            requests_issued();
+        }
+        if (r6.active) {
+            float4 xr[BT][3];
+#pragma unroll
+            for (int b = 0; b < BT; ++b)
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    xr[b][i] = b < a.batch ? reinterpret_cast<const float4 *>(sh.s_in)[b * (kF / 4) + tid + kThreads * i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            pro.k = kF; pro.ln_gain = nullptr; pro.ln_bias = nullptr;
+            finish_activations<QT, BT, 3>(pro, whole_workgroup(), xr, g6.gv, g6.bv, sh.smem, sh.s_sx, sh.s_scratch);
+            MYNAH_STAMP(19);
+            rows_compute<QT, BT, 3, kF, kDownPasses, EPI_RESIDUAL>(g6, r6, lw.down_w, lw.down_s, res_mid, a.batch, sh.smem, sh.s_sx, ex.X6, kW, t0 + 8u, wt);
+            MYNAH_STAMP(17);
+        }
+    }
+    // ---------------------------------------------------------------- final norm of one stream's row
+    if (final_stream >= 0) {
+        const StreamArgs sf = stream_of(a, final_stream);
+        __syncthreads();
+        fetch_tagged<3, false>(ex.X6 + (size_t)final_stream * kW, sh.s_in, kW, a.epoch + 8u * (unsigned)a.n_layers, wt);
+        MYNAH_LEAVE_IF_DEAD();
+        if (a.norm_out == nullptr) {
+            for (int d = tid; d < kW; d += kThreads) store_global(sf.output + d, sh.s_in[d]);
+        } else {
+            layernorm_row(sh.s_in, sf.output, a.norm_out, a.norm_out_b, kW, sh.s4);
+        }
+    }
+}
+
+// The grid: attention workgroups [0, a.attention_wgs), row workgroups counted from the end.  The two ranges never overlap
+// (the host takes another path when they would), so a workgroup runs one of the two loops.
 template <int QT, int BT>
 __global__ void __launch_bounds__(kThreads) k_step_persistent(const PersistArgs a) {
     extern __shared__ __align__(16) float s_in[];               // what a stage waits for: residual rows, hidden rows or partial records
@@ -476,254 +852,27 @@ __global__ void __launch_bounds__(kThreads) k_step_persistent(const PersistArgs 
     __shared__ float s_sx[BT];
     __shared__ float s_scratch[kPrologueScratch * BT];
     __shared__ float s4[4];
-
-    const int wg = blockIdx.x, grid = gridDim.x, tid = threadIdx.x;
-    const AttnRole r1 = attention_role(a, wg, true);
-    AttnRole r3 = attention_role(a, wg, false);
-    if (a.cross_heads == 0) r3.active = false;
-    constexpr int rpp768 = 64 >> lane_group_log2(kW / Chunk<QT>::n), rpp3072 = 64 >> lane_group_log2(kF / Chunk<QT>::n);
+    const SharedBlocks sh{s_in, smem, s_proj, s_red, s_wave_ml, s_sx, s_scratch, s4};
+    const int wg = blockIdx.x, grid = gridDim.x;
+#ifdef MYNAH_PERSIST_PROBE
+    if (threadIdx.x == 0 && a.probe != nullptr) { a.probe[(size_t)wg * 32 + 28] = wall_clock64(); a.probe[(size_t)wg * 32 + 29] = clock64(); }
+    struct AtExit { const PersistArgs &a; int wg; __device__ ~AtExit() { if (threadIdx.x == 0 && a.probe != nullptr) { a.probe[(size_t)wg * 32 + 30] = wall_clock64(); a.probe[(size_t)wg * 32 + 31] = clock64(); } } } at_exit{a, wg};
+#endif
+    if (wg < a.attention_wgs) {
+        const AttnRole r1 = attention_role(a, wg, true);
+        AttnRole r3 = attention_role(a, wg, false);
+        if (a.cross_heads == 0) r3.active = false;
+        if (r1.active || r3.active) attention_path<QT>(a, sh, r1, r3);
+        return;
+    }
     const RowRole r2 = row_role(wg, grid, kW, a.wgs_out, a.rows_out);
-    RowRole r4 = r2;
-    if (a.cross_heads == 0) r4.active = false;
     const RowRole r5 = row_role(wg, grid, kF, a.wgs_up, a.rows_up);
     const RowRole r6 = row_role(wg, grid, kW, a.wgs_down, a.rows_down);
-    (void)rpp768; (void)rpp3072;
-    const bool final_role = grid - 1 - wg < a.batch;
-    if (!(r1.active || r3.active || r2.active || r5.active || r6.active || final_role)) return;
-
-    Waiter wt{a.spin_limit, a.abort_word, false};
-    u64 *const X6 = a.exchange, *const X2 = X6 + 2 * kW, *const X4 = X2 + 2 * kW, *const H = X4 + 2 * kW;
-    u64 *const PS = H + 2 * kF;
-    const size_t ps_stream = (size_t)a.max_units * a.heads * kStepRecord;
-    u64 *const PC = PS + 2 * ps_stream;
-    const size_t pc_stream = (size_t)a.max_units * (a.cross_heads > 0 ? a.cross_heads : 1) * kStepRecord;
-
-    StepAttnArgs aw{};   // what the projection passes read
-    aw.width = kW;
-    aw.arith = a.arith;
-    aw.scale = a.scale;
-
-    const int stride_self = a.heads * kHw, stride_cross = a.cross_heads * kHw;
-    const float *pos_row[2];
-#pragma unroll
-    for (int b = 0; b < 2; ++b) pos_row[b] = (a.position != nullptr && b < a.batch) ? a.position + (size_t)a.length[b] * kW : nullptr;
-
-    // a workgroup that cannot go on: say so, and leave (every barrier of this kernel is passed by whole workgroups)
-#define MYNAH_LEAVE_IF_DEAD()                                                                                           \
-    if (__syncthreads_or(wt.dead ? 1 : 0)) {                                                                            \
-        if (tid == 0) __hip_atomic_store(a.abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);             \
-        return;                                                                                                         \
-    }
-
-    AttnRegs g1;
-    {
-        const PersistLayer &lw = a.layers[0];
-        if (r1.active) {
-            aw.w = lw.qkv_w; aw.scales = lw.qkv_s; aw.heads = a.heads;
-            attention_request<QT, true>(g1, r1, aw, a.self_k[r1.b], a.self_v[r1.b], a.input[r1.b], lw.norm_self, lw.norm_self_b);
-        }
-    }
-    requests_issued();
-
-    for (int layer = 0; layer < a.n_layers; ++layer) {
-        const PersistLayer &lw = a.layers[layer];
-        const unsigned t0 = a.epoch + 8u * (unsigned)layer;   // tags of this layer: t0 + stage; the residual stream it starts from carries t0
-        Residual res_prev;   // x before this layer
-        res_prev.tagged = layer == 0 ? nullptr : X6;
-        res_prev.tag = t0;
-        res_prev.input[0] = a.input[0]; res_prev.input[1] = a.input[1];
-        res_prev.position[0] = pos_row[0]; res_prev.position[1] = pos_row[1];
-
-        // ---------------------------------------------------------------- 1: self attention
-        if (r1.active) {
-            const int b = r1.b;
-            if (layer == 0) {
-                const float *in = a.input[b];
-                const float *pe = pos_row[b];
-                for (int i = tid; i < kW; i += kThreads) s_in[i] = pe != nullptr ? load_global(in + i) + load_global(pe + i) : load_global(in + i);
-            } else {
-                fetch_tagged<3>(X6 + (size_t)b * kW, s_in, kW, t0, wt);
-            }
-            MYNAH_LEAVE_IF_DEAD();
-        }
-        RowRegs<BT, 1> g2;
-        if (r2.active) {
-            rows_request<QT, BT, 1, kW>(g2, r2, lw.o_w, lw.o_s, true, res_prev, a.batch, nullptr, nullptr);
-            requests_issued();
-        }
-        if (r1.active) {
-            const int b = r1.b;
-            aw.w = lw.qkv_w; aw.scales = lw.qkv_s; aw.heads = a.heads;
-            float *kc = a.self_k[b] + (size_t)layer * a.capacity * stride_self;
-            float *vc = a.self_v[b] + (size_t)layer * a.capacity * stride_self;
-            attention_compute<QT>(g1, r1, aw, s_in, kc, vc, a.length[b], lw.norm_self_b != nullptr, PS + (size_t)b * ps_stream, a.heads, t0 + 1u,
-                                  smem, s_sx, s_scratch, s_proj, s_red, s_wave_ml);
-        }
-        g1 = AttnRegs{};   // nothing of it is needed until the next layer's requests: its registers are free for the other stages
-
-        // ---------------------------------------------------------------- 2: fold + O + residual
-        if (r2.active) {
-            int off = 0;
-            for (int b = 0; b < a.batch; ++b) {
-                const int units = (a.length[b] + kStepUnitRows - 1) / kStepUnitRows + 1;
-                const int n = units * a.heads * kStepRecord;
-                fetch_tagged<32>(PS + (size_t)b * ps_stream, s_in + off, n, t0 + 1u, wt);
-                off += n;
-            }
-            MYNAH_LEAVE_IF_DEAD();
-        }
-        AttnRegs g3;
-        if (r3.active) {
-            const int b = r3.b;
-            aw.w = lw.qx_w; aw.scales = lw.qx_s; aw.heads = a.cross_heads;
-            const size_t at = (size_t)layer * a.memory_length[b] * stride_cross;
-            attention_request<QT, false>(g3, r3, aw, a.cross_k[b] != nullptr ? a.cross_k[b] + at : nullptr,
-                                  a.cross_v[b] != nullptr ? a.cross_v[b] + at : nullptr, a.input[b], lw.norm_cross, lw.norm_cross_b);
-            requests_issued();
-        }
-        if (r2.active) {
-            PrologueParams pro;
-            pro.k = kW; pro.batch = a.batch; pro.ln_gain = nullptr; pro.ln_bias = nullptr; pro.arith = a.arith;
-            pro.probe_qx = nullptr; pro.probe_sx = nullptr;
-            float4 xr[BT][1];
-            int off = 0;
-#pragma unroll
-            for (int b = 0; b < BT; ++b) {
-                xr[b][0] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (b < a.batch) {
-                    const int units = (a.length[b] + kStepUnitRows - 1) / kStepUnitRows + 1;
-                    if (tid < kW / 4) xr[b][0] = fold_from_lds(s_in + off, a.heads, units, tid);
-                    off += units * a.heads * kStepRecord;
-                }
-            }
-            __syncthreads();   // s_in has been read: the stage after this one may fill it again
-            finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g2.gv, g2.bv, smem, s_sx, s_scratch);
-            rows_compute<QT, BT, 1, kW, EPI_RESIDUAL>(g2, r2, lw.o_w, lw.o_s, res_prev, a.batch, smem, s_sx, X2, kW, t0 + 2u, wt);
-        }
-
-        Residual res2;
-        res2.tagged = X2; res2.tag = t0 + 2u;
-        res2.input[0] = res2.input[1] = nullptr; res2.position[0] = res2.position[1] = nullptr;
-        Residual res_mid = res2;   // x before the FFN: after the cross sublayer when there is one
-        if (a.cross_heads > 0) {
-            // ------------------------------------------------------------ 3: cross attention
-            if (r3.active) {
-                fetch_tagged<3>(X2 + (size_t)r3.b * kW, s_in, kW, t0 + 2u, wt);
-                MYNAH_LEAVE_IF_DEAD();
-            }
-            RowRegs<BT, 1> g4;
-            if (r4.active) {
-                rows_request<QT, BT, 1, kW>(g4, r4, lw.ox_w, lw.ox_s, true, res2, a.batch, nullptr, nullptr);
-                requests_issued();
-            }
-            if (r3.active) {
-                const int b = r3.b;
-                aw.w = lw.qx_w; aw.scales = lw.qx_s; aw.heads = a.cross_heads;
-                attention_compute<QT>(g3, r3, aw, s_in, nullptr, nullptr, 0, lw.norm_cross_b != nullptr, PC + (size_t)b * pc_stream, a.cross_heads,
-                                      t0 + 3u, smem, s_sx, s_scratch, s_proj, s_red, s_wave_ml);
-            }
-            // ------------------------------------------------------------ 4: fold + O + residual
-            if (r4.active) {
-                int off = 0;
-                for (int b = 0; b < a.batch; ++b) {
-                    const int units = max((a.memory_length[b] + kStepUnitRows - 1) / kStepUnitRows, 1);
-                    const int n = units * a.cross_heads * kStepRecord;
-                    fetch_tagged<32>(PC + (size_t)b * pc_stream, s_in + off, n, t0 + 3u, wt);
-                    off += n;
-                }
-                MYNAH_LEAVE_IF_DEAD();
-                PrologueParams pro;
-                pro.k = kW; pro.batch = a.batch; pro.ln_gain = nullptr; pro.ln_bias = nullptr; pro.arith = a.arith;
-                pro.probe_qx = nullptr; pro.probe_sx = nullptr;
-                float4 xr[BT][1];
-                off = 0;
-#pragma unroll
-                for (int b = 0; b < BT; ++b) {
-                    xr[b][0] = make_float4(0.f, 0.f, 0.f, 0.f);
-                    if (b < a.batch) {
-                        const int units = max((a.memory_length[b] + kStepUnitRows - 1) / kStepUnitRows, 1);
-                        if (tid < kW / 4) xr[b][0] = fold_from_lds(s_in + off, a.cross_heads, units, tid);
-                        off += units * a.cross_heads * kStepRecord;
-                    }
-                }
-                __syncthreads();
-                finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g4.gv, g4.bv, smem, s_sx, s_scratch);
-                rows_compute<QT, BT, 1, kW, EPI_RESIDUAL>(g4, r4, lw.ox_w, lw.ox_s, res2, a.batch, smem, s_sx, X4, kW, t0 + 4u, wt);
-            }
-            res_mid.tagged = X4;
-            res_mid.tag = t0 + 4u;
-        }
-
-        // ---------------------------------------------------------------- 5: LN + up + GELU
-        RowRegs<BT, 1> g5;
-        if (r5.active) {
-            rows_request<QT, BT, 1, kW>(g5, r5, lw.up_w, lw.up_s, false, res_mid, a.batch, lw.norm_ff, lw.norm_ff_b);
-            requests_issued();
-            fetch_tagged<3 * BT>(res_mid.tagged, s_in, a.batch * kW, res_mid.tag, wt);
-            MYNAH_LEAVE_IF_DEAD();
-        }
-        RowRegs<BT, 3> g6;
-        if (r6.active) {
-            rows_request<QT, BT, 3, kF>(g6, r6, lw.down_w, lw.down_s, true, res_mid, a.batch, nullptr, nullptr);
-            requests_issued();
-        }
-        if (r5.active) {
-            PrologueParams pro;
-            pro.k = kW; pro.batch = a.batch; pro.ln_gain = lw.norm_ff; pro.ln_bias = lw.norm_ff_b; pro.arith = a.arith;
-            pro.probe_qx = nullptr; pro.probe_sx = nullptr;
-            float4 xr[BT][1];
-#pragma unroll
-            for (int b = 0; b < BT; ++b)
-                xr[b][0] = (b < a.batch && tid < kW / 4) ? reinterpret_cast<const float4 *>(s_in)[b * (kW / 4) + tid] : make_float4(0.f, 0.f, 0.f, 0.f);
-            __syncthreads();
-            finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g5.gv, g5.bv, smem, s_sx, s_scratch);
-            rows_compute<QT, BT, 1, kW, EPI_GELU>(g5, r5, lw.up_w, lw.up_s, res_mid, a.batch, smem, s_sx, H, kF, t0 + 5u, wt);
-        }
-
-        // ---------------------------------------------------------------- 6: down + residual
-        if (r6.active) {
-            fetch_tagged<12 * BT>(H, s_in, a.batch * kF, t0 + 5u, wt);
-            MYNAH_LEAVE_IF_DEAD();
-        }
-        if (r1.active && layer + 1 < a.n_layers) {
-            const PersistLayer &nx = a.layers[layer + 1];
-            const int b = r1.b;
-            aw.w = nx.qkv_w; aw.scales = nx.qkv_s; aw.heads = a.heads;
-            const size_t at = (size_t)(layer + 1) * a.capacity * stride_self;
-            attention_request<QT, true>(g1, r1, aw, a.self_k[b] + at, a.self_v[b] + at, a.input[b], nx.norm_self, nx.norm_self_b);
-            requests_issued();
-        }
-        if (r6.active) {
-            PrologueParams pro;
-            pro.k = kF; pro.batch = a.batch; pro.ln_gain = nullptr; pro.ln_bias = nullptr; pro.arith = a.arith;
-            pro.probe_qx = nullptr; pro.probe_sx = nullptr;
-            float4 xr[BT][3];
-#pragma unroll
-            for (int b = 0; b < BT; ++b)
-#pragma unroll
-                for (int i = 0; i < 3; ++i)
-                    xr[b][i] = b < a.batch ? reinterpret_cast<const float4 *>(s_in)[b * (kF / 4) + tid + kThreads * i] : make_float4(0.f, 0.f, 0.f, 0.f);
-            __syncthreads();
-            finish_activations<QT, BT, 3>(pro, whole_workgroup(), xr, g6.gv, g6.bv, smem, s_sx, s_scratch);
-            rows_compute<QT, BT, 3, kF, EPI_RESIDUAL>(g6, r6, lw.down_w, lw.down_s, res_mid, a.batch, smem, s_sx, X6, kW, t0 + 8u, wt);
-        }
-    }
-
-    // ---------------------------------------------------------------- final norm of each stream's row
-    if (final_role) {
-        const int b = grid - 1 - wg;
-        __syncthreads();
-        fetch_tagged<3>(X6 + (size_t)b * kW, s_in, kW, a.epoch + 8u * (unsigned)a.n_layers, wt);
-        MYNAH_LEAVE_IF_DEAD();
-        float *out = a.output[b];
-        if (a.norm_out == nullptr) {
-            for (int d = tid; d < kW; d += kThreads) store_global(out + d, s_in[d]);
-        } else {
-            layernorm_row(s_in, out, a.norm_out, a.norm_out_b, kW, s4);
-        }
-    }
-#undef MYNAH_LEAVE_IF_DEAD
+    const int final_stream = grid - 1 - wg < a.batch ? grid - 1 - wg : -1;
+    if (r2.active || r5.active || r6.active || final_stream >= 0) rows_path<QT, BT>(a, sh, r2, r5, r6, final_stream);
 }
+#undef MYNAH_LEAVE_IF_DEAD
+#undef MYNAH_STAMP
 
 }  // namespace
 
@@ -788,8 +937,9 @@ static int launch_pt(State *st, const PersistArgs &a, int grid, char *error, siz
 }
 
 int launch_step_persistent(State *st, const PersistArgs &a, int qtype, int grid, char *error, size_t capacity) {
+    const int row_wgs = a.wgs_up > a.wgs_down ? (a.wgs_up > a.wgs_out ? a.wgs_up : a.wgs_out) : (a.wgs_down > a.wgs_out ? a.wgs_down : a.wgs_out);
     if (a.batch < 1 || a.batch > 2 || a.exchange == nullptr || a.abort_word == nullptr || a.layers == nullptr || a.n_layers < 1 ||
-        grid < step_persistent_attention_workgroups(a) || grid < a.wgs_up || grid < a.wgs_down || grid < a.wgs_out) {
+        a.attention_wgs != step_persistent_attention_workgroups(a) || a.attention_wgs + row_wgs > grid || a.batch > row_wgs) {
         set_error(error, capacity, "persistent step: invalid arguments or too few workgroups for these lengths");
         return -1;
     }
