@@ -122,7 +122,7 @@ def test_persistent_steps_in_a_row(pkg, backend, orc, synth, nerr):
     finally:
         for b in range(2):
             streams[b]["length"] = lengths[b]
-        backend.set_graph_mode(2)
+        backend.set_graph_mode(1)
         h.close()
         backend.set_quant(0)
 
