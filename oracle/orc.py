@@ -525,8 +525,44 @@ class RefLocal:
             raise RuntimeError(err.value.decode())
         return out, int(n.value)
 
+    def hip_frame(self, library_path, projections, biases, audio_tables, vocab, codebook_size, eos_id, codebook_count, items,
+                  code_stride, raw_offset):
+        """One device frame through the integration text's hip_sample_local_frame_batch (oracle/integration_batched.inc) on the
+        reference's own local_batch_item.  items: dicts with row, temperature, topk, rng_state (None = greedy),
+        generated_raw_length, min_raw_length.  Returns (codes [count, codebook_count, code_stride], saw_eos, eos_frame,
+        rng states)."""
+        streams, count = len(projections), len(items)
+        keep = [np.ascontiguousarray(a, np.float32) for a in projections]
+        keep_b = [None if biases is None or b is None else np.ascontiguousarray(b, np.float32) for b in (biases or [None] * streams)]
+        keep_t = [np.ascontiguousarray(a, np.float32) for a in audio_tables]
+        self._frame_keep = (keep, keep_b, keep_t)        # the device weight cache keys on these addresses
+        pp, pc = C.c_void_p * streams, C.c_void_p * count
+        rows = [np.ascontiguousarray(it["row"], np.float32) for it in items]
+        temperature = (C.c_float * count)(*[it["temperature"] for it in items])
+        topk = (C.c_uint * count)(*[it["topk"] for it in items])
+        rng = (C.c_uint64 * count)(*[it["rng_state"] or 0 for it in items])
+        has_rng = (C.c_int * count)(*[0 if it["rng_state"] is None else 1 for it in items])
+        generated = (_sz * count)(*[it["generated_raw_length"] for it in items])
+        minimum = (_sz * count)(*[it["min_raw_length"] for it in items])
+        codes = np.full((count, codebook_count, code_stride), 0xffffffff, np.uint32)
+        saw = (C.c_int * count)()
+        eos_frame = (_sz * count)()
+        err = C.create_string_buffer(512)
+        self.r.ref_local_hip_frame.restype = C.c_int
+        rc = self.r.ref_local_hip_frame(C.c_void_p(self.h), os.fsencode(library_path), _sz(streams), _sz(vocab), _sz(codebook_size),
+                                        _sz(eos_id), _sz(codebook_count), pp(*[_ptr(a) for a in keep]),
+                                        None if biases is None else pp(*[_ptr(a) for a in keep_b]), pp(*[_ptr(a) for a in keep_t]),
+                                        _sz(count), pc(*[_ptr(a) for a in rows]), temperature, topk, rng, has_rng, generated, minimum,
+                                        _ptr(codes), _sz(code_stride), _sz(raw_offset), saw, eos_frame, err, _sz(512))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        self.hip_batched = True
+        return codes, list(saw), list(eos_frame), list(rng)
+
     def close(self):
         if self.h:
+            if getattr(self, "hip_batched", False):
+                self.r.ref_local_hip_batch_release(C.c_void_p(self.h))
             if getattr(self, "device", False):
                 self.r.ref_local_release(C.c_void_p(self.h))
             self.r.ref_local_free(C.c_void_p(self.h))
@@ -609,8 +645,29 @@ class RefDecoder:
             raise RuntimeError(err.value.decode() or "no device caches")
         return k, v
 
+    def hip_step_batch(self, library_path, self_k, self_v, cross_k, cross_v, lengths, memory_lengths, inputs):
+        """One batched device step through the integration text's hip_decoder_step_batch (oracle/integration_batched.inc) on
+        the reference's own decoder_cache slots; returns (rows, new lengths)."""
+        B = self.batch
+        outs = [np.empty(self.cfg["width"], np.float32) for _ in range(B)]
+        pp, szs = C.c_void_p * B, _sz * B
+        lens = szs(*lengths)
+        err = C.create_string_buffer(512)
+        self.r.ref_decoder_hip_step_batch.restype = C.c_int
+        rc = self.r.ref_decoder_hip_step_batch(C.c_void_p(self.h), os.fsencode(library_path), pp(*[_ptr(a) for a in self_k]),
+                                               pp(*[_ptr(a) for a in self_v]), pp(*[_ptr(a) for a in cross_k]),
+                                               pp(*[_ptr(a) for a in cross_v]), lens, szs(*memory_lengths),
+                                               pp(*[_ptr(np.ascontiguousarray(a, np.float32)) for a in inputs]),
+                                               pp(*[_ptr(a) for a in outs]), err, _sz(512))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        self.hip_batched = True
+        return outs, list(lens)
+
     def close(self):
         if self.h:
+            if getattr(self, "hip_batched", False):
+                self.r.ref_decoder_hip_batch_release(C.c_void_p(self.h))
             if getattr(self, "device", False):
                 self.r.ref_decoder_release(C.c_void_p(self.h))
             self.r.ref_decoder_free(C.c_void_p(self.h))

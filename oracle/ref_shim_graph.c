@@ -43,6 +43,9 @@ typedef struct {
     decoder_cache caches[MYNAH_MAX_BATCH];
     batch_scratch scratch;
     size_t batch;
+    /* the batched device step of the integration text (set up at its first use) */
+    void *hip_batch;
+    float *hip_in[MYNAH_MAX_BATCH], *hip_out[MYNAH_MAX_BATCH];
 } ref_decoder;
 
 void ref_decoder_free(ref_decoder *d) {
@@ -178,6 +181,8 @@ typedef struct {
     local_workspace workspaces[MYNAH_MAX_BATCH];
     batch_scratch scratch;
     size_t batch;
+    void *hip_batch;                       /* the device frame of the integration text */
+    float *hip_last[MYNAH_MAX_BATCH];
 } ref_local;
 
 void ref_local_free(ref_local *d) {
@@ -526,4 +531,181 @@ int ref_codec_engine_decode(ref_codec_engine *e, const unsigned *codes, size_t r
     free(audio);
     *count = n;
     return 0;
+}
+
+
+/* ---- the integration text, compiled ------------------------------------------------------------------------------
+ * oracle/integration_batched.inc is the engine-side code INTEGRATION.md sections 6 and 6b quote.  In the engine its five
+ * library calls are linked symbols; here the library is found with dlopen (so that this file still loads where no GPU
+ * runtime is installed) and the calls go through pointers of the header's own prototype types.
+ * Reference types it is compiled against: decoder_cache / decoder_layer_resolved (src/graph.c:2795-2861), local_cache
+ * (:810-851), local_batch_item (:1346-1364); reference functions the drivers below use: decoder_gpu_attention_init
+ * (:2901-2962). */
+#include <dlfcn.h>
+
+#include "mynah_hip.h"
+
+static struct {
+    __typeof__(&mynah_hip_decoder_create) decoder_create;
+    __typeof__(&mynah_hip_decoder_destroy) decoder_destroy;
+    __typeof__(&mynah_hip_decoder_step) decoder_step;
+    __typeof__(&mynah_hip_local_create) local_create;
+    __typeof__(&mynah_hip_local_destroy) local_destroy;
+    __typeof__(&mynah_hip_local_frame) local_frame;
+} hip_calls;
+#define mynah_hip_decoder_create (*hip_calls.decoder_create)
+#define mynah_hip_decoder_destroy (*hip_calls.decoder_destroy)
+#define mynah_hip_decoder_step (*hip_calls.decoder_step)
+#define mynah_hip_local_create (*hip_calls.local_create)
+#define mynah_hip_local_destroy (*hip_calls.local_destroy)
+#define mynah_hip_local_frame (*hip_calls.local_frame)
+#include "integration_batched.inc"
+#undef mynah_hip_decoder_create
+#undef mynah_hip_decoder_destroy
+#undef mynah_hip_decoder_step
+#undef mynah_hip_local_create
+#undef mynah_hip_local_destroy
+#undef mynah_hip_local_frame
+
+void *ref_backend_state(const mynah_backend *backend);   /* ref_shim_backend.c: the accessor the integration text asks for */
+
+static int integration_bind(const char *library_path, char *error, size_t error_capacity) {
+    if (hip_calls.decoder_create != NULL) return 0;
+    void *handle = dlopen(library_path, RTLD_NOW | RTLD_GLOBAL);
+    if (handle == NULL) {
+        snprintf(error, error_capacity, "dlopen: %s", dlerror());
+        return -1;
+    }
+    hip_calls.decoder_create = (__typeof__(hip_calls.decoder_create))dlsym(handle, "mynah_hip_decoder_create");
+    hip_calls.decoder_destroy = (__typeof__(hip_calls.decoder_destroy))dlsym(handle, "mynah_hip_decoder_destroy");
+    hip_calls.decoder_step = (__typeof__(hip_calls.decoder_step))dlsym(handle, "mynah_hip_decoder_step");
+    hip_calls.local_create = (__typeof__(hip_calls.local_create))dlsym(handle, "mynah_hip_local_create");
+    hip_calls.local_destroy = (__typeof__(hip_calls.local_destroy))dlsym(handle, "mynah_hip_local_destroy");
+    hip_calls.local_frame = (__typeof__(hip_calls.local_frame))dlsym(handle, "mynah_hip_local_frame");
+    if (!hip_calls.decoder_create || !hip_calls.decoder_destroy || !hip_calls.decoder_step || !hip_calls.local_create ||
+        !hip_calls.local_destroy || !hip_calls.local_frame) {
+        snprintf(error, error_capacity, "the library lacks a batched entry point");
+        hip_calls.decoder_create = NULL;
+        return -1;
+    }
+    return 0;
+}
+
+/* One batched device step of the decoder's first `d->batch` slots through hip_decoder_step_batch.  The decoder must have
+ * the library attached (ref_decoder_use_hip).  At a slot's first call its host caches (rows [0, lengths[b]) of
+ * self_k / self_v, all of cross_k / cross_v) are uploaded by the reference's own decoder_gpu_attention_init; afterwards the
+ * device caches are the live ones.  lengths[b] comes back advanced by one. */
+int ref_decoder_hip_step_batch(ref_decoder *d, const char *library_path, float *const *self_k, float *const *self_v,
+                               float *const *cross_k, float *const *cross_v, size_t *lengths, const size_t *memory_lengths,
+                               const float *const *inputs, float *const *outs, char *error, size_t error_capacity) {
+    const mynah_backend *backend = d->model.backend;
+    void *state = ref_backend_state(backend);
+    if (integration_bind(library_path, error, error_capacity) != 0) return -1;
+    decoder_cache *ptrs[MYNAH_MAX_BATCH];
+    for (size_t b = 0; b < d->batch; ++b) {
+        decoder_cache *c = &d->caches[b];
+        c->self_k = self_k[b]; c->self_v = self_v[b]; c->cross_k = cross_k[b]; c->cross_v = cross_v[b];
+        c->length = lengths[b];
+        c->memory_length = memory_lengths[b];
+        if (decoder_gpu_attention_init(c, backend, error, error_capacity) != 0) return -1;
+        if (d->hip_in[b] == NULL &&
+            (mynah_backend_dev_alloc(backend, c->width, &d->hip_in[b], error, error_capacity) != 0 ||
+             mynah_backend_dev_alloc(backend, c->width, &d->hip_out[b], error, error_capacity) != 0))
+            return -1;
+        if (mynah_backend_h2d(backend, inputs[b], d->hip_in[b], c->width, error, error_capacity) != 0) return -1;
+        ptrs[b] = c;
+    }
+    if (d->hip_batch == NULL) {
+        hip_decoder_batch *h = (hip_decoder_batch *)calloc(1, sizeof(*h));
+        if (h == NULL || hip_decoder_batch_init(state, &d->caches[0], h, error, error_capacity) != 0) {
+            free(h);
+            return -1;
+        }
+        d->hip_batch = h;
+    }
+    if (hip_decoder_step_batch(state, (hip_decoder_batch *)d->hip_batch, ptrs, (const float *const *)d->hip_in, d->hip_out, d->batch,
+                               error, error_capacity) != 0)
+        return -1;
+    for (size_t b = 0; b < d->batch; ++b) {
+        if (mynah_backend_d2h(backend, d->hip_out[b], outs[b], d->caches[b].width, error, error_capacity) != 0) return -1;
+        lengths[b] = d->caches[b].length;
+    }
+    return 0;
+}
+
+/* Releases what ref_decoder_hip_step_batch set up; call before ref_decoder_release. */
+void ref_decoder_hip_batch_release(ref_decoder *d) {
+    if (d == NULL) return;
+    if (d->hip_batch != NULL) {
+        hip_decoder_batch_free(ref_backend_state(d->model.backend), (hip_decoder_batch *)d->hip_batch);
+        free(d->hip_batch);
+        d->hip_batch = NULL;
+    }
+    for (size_t b = 0; b < MYNAH_MAX_BATCH; ++b) {
+        if (d->hip_in[b] != NULL) mynah_backend_dev_free(d->model.backend, d->hip_in[b]);
+        if (d->hip_out[b] != NULL) mynah_backend_dev_free(d->model.backend, d->hip_out[b]);
+        d->hip_in[b] = d->hip_out[b] = NULL;
+    }
+}
+
+/* One device frame for `count` items through hip_sample_local_frame_batch, on the local stack of `d` (library attached
+ * with ref_local_use_hip).  The items are the reference's own local_batch_item: decoder_last[i] is uploaded to a device
+ * row; rng_states[i] is used when has_rng[i] (else the item is greedy, rng_state == NULL); codes is
+ * [count][codebook_count][code_stride] and receives the stored codes at column raw_offset + frame. */
+int ref_local_hip_frame(ref_local *d, const char *library_path, size_t streams, size_t vocab, size_t codebook_size, size_t eos_id,
+                        size_t codebook_count, const float *const *projection_w, const float *const *projection_bias,
+                        const float *const *audio_table, size_t count, const float *const *decoder_last, const float *temperature,
+                        const unsigned *topk, uint64_t *rng_states, const int *has_rng, const size_t *generated_raw_length,
+                        const size_t *min_raw_length, unsigned *codes, size_t code_stride, size_t raw_offset, int *saw_eos,
+                        size_t *eos_frame, char *error, size_t error_capacity) {
+    const mynah_backend *backend = d->model.backend;
+    void *state = ref_backend_state(backend);
+    if (integration_bind(library_path, error, error_capacity) != 0) return -1;
+    if (count > MYNAH_MAX_BATCH) return -1;
+    if (d->hip_batch == NULL) {
+        hip_local_batch *h = (hip_local_batch *)calloc(1, sizeof(*h));
+        if (h == NULL || hip_local_batch_init(state, &d->caches[0], streams, vocab, codebook_size, eos_id, codebook_count, projection_w,
+                                              projection_bias, audio_table, h, error, error_capacity) != 0) {
+            free(h);
+            return -1;
+        }
+        d->hip_batch = h;
+    }
+    local_batch_item items[MYNAH_MAX_BATCH];
+    memset(items, 0, sizeof items);
+    const size_t width = d->caches[0].width;
+    for (size_t i = 0; i < count; ++i) {
+        if (d->hip_last[i] == NULL && mynah_backend_dev_alloc(backend, width, &d->hip_last[i], error, error_capacity) != 0) return -1;
+        if (mynah_backend_h2d(backend, decoder_last[i], d->hip_last[i], width, error, error_capacity) != 0) return -1;
+        items[i].decoder_last = decoder_last[i];
+        items[i].decoder_dev_last = d->hip_last[i];
+        items[i].codes = codes + i * codebook_count * code_stride;
+        items[i].raw_offset = raw_offset;
+        items[i].code_stride = code_stride;
+        items[i].generated_raw_length = generated_raw_length[i];
+        items[i].min_raw_length = min_raw_length[i];
+        items[i].temperature = temperature[i];
+        items[i].topk = topk[i];
+        items[i].rng_state = has_rng[i] ? &rng_states[i] : NULL;
+    }
+    if (hip_sample_local_frame_batch(state, (hip_local_batch *)d->hip_batch, items, count, error, error_capacity) != 0) return -1;
+    for (size_t i = 0; i < count; ++i) {
+        saw_eos[i] = items[i].saw_eos;
+        eos_frame[i] = items[i].eos_frame;
+    }
+    return 0;
+}
+
+void ref_local_hip_batch_release(ref_local *d) {
+    if (d == NULL) return;
+    if (d->hip_batch != NULL) {
+        hip_local_batch *h = (hip_local_batch *)d->hip_batch;
+        if (h->local != NULL) (*hip_calls.local_destroy)(ref_backend_state(d->model.backend), h->local);
+        free(h);
+        d->hip_batch = NULL;
+    }
+    for (size_t b = 0; b < MYNAH_MAX_BATCH; ++b) {
+        if (d->hip_last[b] != NULL) mynah_backend_dev_free(d->model.backend, d->hip_last[b]);
+        d->hip_last[b] = NULL;
+    }
 }

@@ -161,3 +161,97 @@ def test_codec_decode_resident(pkg, orc, ref_strict, nerr, quant_env, tmp_path):
     finally:
         hip.close()
         cpu.close()
+
+
+@pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4"])
+def test_integration_text_batched_decoder_step(pkg, orc, ref_strict, synth, nerr, quant_env, qtype_name):
+    """The engine-side code INTEGRATION.md section 6 quotes (oracle/integration_batched.inc), compiled against the
+    reference's own decoder_cache: eight ragged streams, two consecutive steps through hip_decoder_step_batch on the
+    library, against the reference's CPU decoder_step_batch on the same caches and inputs.  The device caches are the
+    ones the reference's decoder_gpu_attention_init uploads; lengths advance as the reference's do; the rows the step
+    appended are read back through the backend."""
+    _announce("engine: integration text, batched decoder step, %s" % qtype_name)
+    from tests.test_gpu_step import quantised_errors_ok
+    qtype = QT[qtype_name]
+    lengths = [5, 17, 0, 31, 9, 2, 25, 12]
+    mems = [7, 19, 3, 32, 11, 1, 27, 16]
+    steps = 2
+    cfg = synth.decoder_config(layers=2, capacity=max(lengths) + steps + 1, cross_heads=1)
+    w = synth.decoder_weights(cfg, seed=0, ln_bias=False)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=1)
+    rng = np.random.default_rng(9)
+    xs = [[rng.standard_normal(cfg["width"]).astype(np.float32) for _ in streams] for _ in range(steps)]
+    quant_env(qtype_name)
+    cpu = orc.RefDecoder(cfg, w, qtype, len(streams), max(mems), strict=True)
+    hip = orc.RefDecoder(cfg, w, qtype, len(streams), max(mems), strict=True)
+    hip.use_hip(pkg.LIB_PATH)
+    try:
+        ck, cv = [s["k"].copy() for s in streams], [s["v"].copy() for s in streams]
+        hk, hv = [s["k"].copy() for s in streams], [s["v"].copy() for s in streams]
+        clens, hlens = list(lengths), list(lengths)
+        for t in range(steps):
+            want, clens = cpu.step(ck, cv, [s["ck"] for s in streams], [s["cv"] for s in streams], clens, mems, xs[t])
+            got, hlens = hip.hip_step_batch(pkg.LIB_PATH, hk, hv, [s["ck"] for s in streams], [s["cv"] for s in streams], hlens, mems, xs[t])
+            assert hlens == clens == [n + t + 1 for n in lengths]
+            errs = [nerr(got[b], want[b]) for b in range(len(streams))]
+            if qtype_name == "f32":
+                assert max(errs) < 1e-5, errs
+            else:   # 16 (stream, layer) pairs per step; the second step inherits what the first one's rounding did
+                quantised_errors_ok(errs, 2 + 2 * t, "integration text step %d %s" % (t, qtype_name))
+            for b in (0, 2, 7):
+                row = lengths[b] + t
+                for layer in range(cfg["layers"]):
+                    dk, dv = hip.device_kv_row(b, layer, row)
+                    assert nerr(dk, ck[b][layer, row]) < TOL[qtype_name] and nerr(dv, cv[b][layer, row]) < TOL[qtype_name]
+        for b in range(len(streams)):      # the host copies were uploaded once and never written
+            assert np.array_equal(hk[b], streams[b]["k"]) and np.array_equal(hv[b], streams[b]["v"])
+    finally:
+        hip.close()
+        cpu.close()
+
+
+def test_integration_text_local_frame(pkg, orc, ref_strict, synth, quant_env):
+    """The engine-side code INTEGRATION.md section 6b quotes, compiled against the reference's own local_cache and
+    local_batch_item: one frame of three items (greedy with rng_state == NULL, two sampling items, one of them with EOS
+    forbidden) through hip_sample_local_frame_batch on the library, f32 weights, against the oracle's frame: the codes
+    land where the reference's loop stores them (src/graph.c:1620-1628: codebook * code_stride + raw_offset + frame),
+    the generators advance in place, EOS flags and frames agree."""
+    _announce("engine: integration text, local frame")
+    S, V, codebook, eos, cbc = 16, 96, 80, 83, 8
+    cfg = synth.decoder_config(layers=2, capacity=S + 1, cross_heads=0)
+    w = synth.decoder_weights(cfg, seed=41, ln_bias=False)
+    w["norm_out_g"] = w["norm_out_b"] = None
+    rng = np.random.default_rng(42)
+    proj = [(rng.standard_normal((V, cfg["width"])) * 0.05).astype(np.float32) for _ in range(S)]
+    bias = [(rng.standard_normal(V) * 0.1).astype(np.float32) for _ in range(S)]
+    tables = [rng.standard_normal((V, cfg["width"])).astype(np.float32) for _ in range(S)]
+    bias[6][eos] = 50.0                        # position 6 chooses EOS unless it is forbidden
+    rows = [rng.standard_normal(cfg["width"]).astype(np.float32) for _ in range(3)]
+    items = [
+        {"row": rows[0], "temperature": 0.9, "topk": 40, "rng_state": None, "generated_raw_length": 10, "min_raw_length": 4},   # greedy
+        {"row": rows[1], "temperature": 0.8, "topk": 50, "rng_state": 0x1234567, "generated_raw_length": 1, "min_raw_length": 4},  # EOS forbidden
+        {"row": rows[2], "temperature": 1.1, "topk": 7, "rng_state": 99, "generated_raw_length": 4, "min_raw_length": 4},
+    ]
+    oracle_items = [{"temperature": it["temperature"], "topk": it["topk"] if it["rng_state"] is not None else 1,
+                     "rng_state": it["rng_state"] or 0, "forbid_eos": it["generated_raw_length"] < it["min_raw_length"]} for it in items]
+    quant_env("f32")
+    hip = orc.RefLocal(cfg, w, orc.F32, 3, strict=True)
+    hip.use_hip(pkg.LIB_PATH)
+    try:
+        code_stride, raw_offset = 11, 5
+        codes, saw, eos_frame, states = hip.hip_frame(pkg.LIB_PATH, proj, bias, tables, V, codebook, eos, cbc, items, code_stride, raw_offset)
+        stack = orc.Decoder(cfg, w, orc.F32)
+        want = orc.LocalFrame(stack, [orc.PackedWeight(p, orc.F32) for p in proj], bias, tables, codebook, eos, cbc).frame(rows, oracle_items)
+        for i in range(3):
+            for s in range(S):
+                assert codes[i, s % cbc, raw_offset + s // cbc] == want["stored"][i, s], "item %d position %d" % (i, s)
+            untouched = np.ones(code_stride, bool)
+            untouched[raw_offset:raw_offset + S // cbc] = False
+            assert np.all(codes[i][:, untouched] == 0xffffffff), "codes outside the frame's columns were written"
+            assert saw[i] == want["saw_eos"][i]
+            assert eos_frame[i] == want["eos_frame"][i]
+            if items[i]["rng_state"] is not None:
+                assert states[i] == want["rng_state"][i], "generator of item %d" % i
+        assert saw[0] == 1 and eos_frame[0] == 6 // cbc and saw[1] == 0
+    finally:
+        hip.close()

@@ -1,0 +1,17 @@
+"""INTEGRATION.md quotes the engine-side code of sections 6 and 6b from oracle/integration_batched.inc, the file the
+compiler sees (oracle/ref_shim_graph.c includes it against the reference's own structs).  The quotation must be the file."""
+import os
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_integration_md_quotes_the_compiled_file():
+    with open(os.path.join(ROOT, "oracle", "integration_batched.inc")) as f:
+        source = f.read()
+    with open(os.path.join(ROOT, "INTEGRATION.md")) as f:
+        doc = f.read()
+    marker6, marker6b = "/* ---- section 6: the batched decoder step", "/* ---- section 6b: the local-transformer frame"
+    part6 = source[source.index(marker6):source.index(marker6b)].strip()
+    part6b = source[source.index(marker6b):].strip()
+    assert part6 in doc, "INTEGRATION.md section 6 no longer quotes oracle/integration_batched.inc"
+    assert part6b in doc, "INTEGRATION.md section 6b no longer quotes oracle/integration_batched.inc"
