@@ -359,6 +359,9 @@ typedef struct {
     const float *const *qkv_w, *const *o_w, *const *up_w, *const *down_w;   /* [layers] HOST f32, stored f16 */
     const float *const *norm1, *const *norm1_bias, *const *norm2, *const *norm2_bias;
     const float *norm_out, *norm_out_bias;
+    int causal;                   /* nonzero: query t attends to keys 0 .. t (src/graph.c:446-449); 0: every key */
+    size_t ffn_kernel;            /* 0 or 1: plain FFN, up_w [ffn, width], down_w [width, ffn].  3: causal_conv_ffn
+                                   * (src/graph.c:302-352), up_w [ffn, width, 3], down_w [width, ffn, 3] */
 } mynah_hip_encoder_desc;
 typedef struct mynah_hip_encoder mynah_hip_encoder;
 

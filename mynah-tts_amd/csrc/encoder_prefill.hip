@@ -5,17 +5,21 @@
 // through an f32 BLAS.  Here the weights are f16 (converted once at load, IEEE round to nearest even,
 // third_party/ingot/src/dtype.c:246-268), the activations entering a product are rounded to f16, and
 // every product accumulates in f32 on v_mfma_f32_32x32x16_f16.  The residual stream, the LayerNorm
-// statistics, the softmax and the GELU stay f32.  Bidirectional attention and the plain FFN
-// (kernel == 1 branch of causal_conv_ffn, src/graph.c:302-316).
+// statistics, the softmax and the GELU stay f32.  Attention is bidirectional or causal (the mask of
+// src/graph.c:446-449: query t sees keys 0 .. t).  The FFN is causal_conv_ffn (src/graph.c:302-352) with kernel 1
+// (two plain products) or kernel 3: out[t][o] = sum_{i,j} W[o][i][j] * in[t - 2 + j][i], rows before the first
+// being zero.  The conv is an NT product too: its weights are stored tap-major, W'[o][j * in + i], so that the
+// A operand of token t is rows t-2, t-1, t of the activation side by side, and a K step of the product reads one
+// of those rows -- addressing only, no unfolded copy.  The two rows before row 0 of nrm and hid exist and stay zero.
 //
 // Layout in device memory (T tokens padded to a multiple of 64 rows; pad rows are kept finite and are
 // masked out as attention keys, so they never reach a real row):
 //   x    f32 [Tpad, w]       residual stream
-//   nrm  f16 [Tpad, w]       LayerNorm output = A operand of the QKV / FFN-up products
+//   nrm  f16 [2 + Tpad, w]   LayerNorm output = A operand of the QKV / FFN-up products (after two zero rows)
 //   qk   f16 [Tpad, 2w]      q | k of every token, row-major (K-contiguous operands of QK^T)
 //   vt   f16 [w, TpadMax]    v transposed: vt[h*64+d][t], so PV's B operand is K(=t)-contiguous too
 //   ctx  f16 [Tpad, w]       attention output = A operand of the O product
-//   hid  f16 [Tpad, ffn]     GELU(up) = A operand of the FFN-down product
+//   hid  f16 [2 + Tpad, ffn] GELU(up) = A operand of the FFN-down product (after two zero rows)
 //   part f32 [4, Tpad, w]    K-split partial sums of the O and FFN-down products; the row pass that follows
 //                            adds them to x in a fixed order (no atomics: results do not depend on scheduling)
 //
@@ -39,12 +43,16 @@ struct EncParams {
 
 struct mynah_hip_encoder {
     size_t layers = 0, width = 0, heads = 0, head_width = 0, ffn = 0, vocab = 0, max_positions = 0, tpad_max = 0;
+    size_t taps = 1;           // FFN conv kernel size, 1 or 3
+    int causal = 0;
     const CachedWeight *tok = nullptr, *pos = nullptr;
     std::vector<const CachedWeight *> qkv, o, up, down;
+    std::vector<_Float16 *> conv_up, conv_down;   // taps == 3: tap-major f16 copies owned by the encoder
     std::vector<const float *> n1g, n1b, n2g, n2b;
     const float *nog = nullptr, *nob = nullptr;
     float *x = nullptr, *part = nullptr;   // part: [splits, Tpad, w] partial products of the O and FFN-down products
     _Float16 *nrm = nullptr, *qk = nullptr, *vt = nullptr, *ctx = nullptr, *hid = nullptr;
+    _Float16 *nrm_alloc = nullptr, *hid_alloc = nullptr;   // nrm and hid begin kLeadRows rows into these
     int *ids = nullptr;        // [tpad_max] token ids, followed by one EncParams
     int *ids_host = nullptr;   // pinned twin of ids
     EncParams *params = nullptr;
@@ -65,6 +73,7 @@ constexpr int kLdsStride = 72;       // halfs per staged row: 64 + 8 keeps 16-by
 constexpr int kQTile = 32;           // queries per attention workgroup
 constexpr int kScorePad = 8;         // floats appended to a score row (bank spread for the row-wise softmax)
 constexpr int kGemmDepth = 4;        // K steps of operand tiles in flight in the products (see k_enc_gemm)
+constexpr int kLeadRows = 2;         // zero rows in front of the conv FFN's activations (kernel size 3 looks two rows back)
 
 enum { ENC_QKV = 0, ENC_PARTIAL = 1, ENC_GELU = 2 };
 
@@ -76,6 +85,7 @@ struct GemmArgs {
     _Float16 *out;         // ENC_QKV: qk [M, 2*width];  ENC_GELU: hid [M, N]
     _Float16 *vt;          // ENC_QKV: v transposed [width, vt_stride]
     int width, vt_stride;
+    int taps, cin;         // conv form: K = taps * cin, A is [M, cin] with (taps - 1) zero rows before row 0
 };
 
 // tanh-GELU (src/kernels.c:382-389) for a value that is rounded to f16 at once: 0.5 x (1 + tanh c) = x / (1 + e^(-2c)),
@@ -93,8 +103,8 @@ __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 
 // One K step of both operand tiles on its way from global memory to LDS (four 16-byte pieces per thread).
 struct StagedTiles {
     u32x4 a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0}, w0 = {0, 0, 0, 0}, w1 = {0, 0, 0, 0};
-    __device__ __forceinline__ void load(const u32x4 *ga0, const u32x4 *ga1, const u32x4 *gw0, const u32x4 *gw1, int chunk) {
-        a0 = ga0[chunk]; a1 = ga1[chunk]; w0 = gw0[chunk]; w1 = gw1[chunk];
+    __device__ __forceinline__ void load(const u32x4 *ga0, const u32x4 *ga1, const u32x4 *gw0, const u32x4 *gw1, int a_chunk, int w_chunk) {
+        a0 = ga0[a_chunk]; a1 = ga1[a_chunk]; w0 = gw0[w_chunk]; w1 = gw1[w_chunk];
     }
     __device__ __forceinline__ void store(_Float16 *sa, _Float16 *sw, int off0, int off1) const {
         *reinterpret_cast<u32x4 *>(sa + off0) = a0;
@@ -129,7 +139,8 @@ struct StepFragments {
 // under a condition the compiler must assume it was not, and the wait before storing the oldest block then drains every
 // younger one as well: with `if (kt + D < nk)` around the requests the pipeline was one step deep whatever D said.
 // Without EXACT (an odd number of steps) the guarded form is used, with that cost.
-template <int EPI, int D, bool EXACT>
+// CONV: the A operand of K step s is the 64 channels (s % (cin / 64)) * 64 .. of row m - (taps - 1) + s / (cin / 64).
+template <int EPI, int D, bool EXACT, bool CONV>
 __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
     static_assert(D >= 2 && D % 2 == 0, "stage parity must equal step parity");
     __shared__ __align__(16) _Float16 s_a[2][kTile * kLdsStride];
@@ -139,8 +150,9 @@ __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
     const int m0 = blockIdx.y * kTile, n0 = blockIdx.x * kTile;
     // staging: thread -> (row tid / 8 and + 32, 16-byte chunk tid % 8) of both tiles
     const int srow = tid >> 3, schunk = tid & 7;
-    const u32x4 *ga0 = reinterpret_cast<const u32x4 *>(g.a + (size_t)(m0 + srow) * g.K) + schunk;
-    const u32x4 *ga1 = reinterpret_cast<const u32x4 *>(g.a + (size_t)(m0 + srow + 32) * g.K) + schunk;
+    const int lda = CONV ? g.cin : g.K;
+    const u32x4 *ga0 = reinterpret_cast<const u32x4 *>(g.a + (ptrdiff_t)(m0 + srow) * lda) + schunk;
+    const u32x4 *ga1 = reinterpret_cast<const u32x4 *>(g.a + (ptrdiff_t)(m0 + srow + 32) * lda) + schunk;
     const u32x4 *gw0 = reinterpret_cast<const u32x4 *>(g.w + (size_t)(n0 + srow) * g.K) + schunk;
     const u32x4 *gw1 = reinterpret_cast<const u32x4 *>(g.w + (size_t)(n0 + srow + 32) * g.K) + schunk;
     const int soff0 = srow * kLdsStride + schunk * 8, soff1 = (srow + 32) * kLdsStride + schunk * 8;
@@ -148,7 +160,11 @@ __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
     // K range of this workgroup (blockIdx.z splits K; only ENC_PARTIAL launches more than one split)
     const int nk = g.K / kTile / (int)gridDim.z;
     const int kbase = (int)blockIdx.z * nk * (kTile / 8);   // in 16-byte chunks
-    ga0 += kbase; ga1 += kbase; gw0 += kbase; gw1 += kbase;
+    gw0 += kbase; gw1 += kbase;
+    if constexpr (!CONV) { ga0 += kbase; ga1 += kbase; }
+    const int first_step = (int)blockIdx.z * nk;
+    const int steps_per_tap = CONV ? g.cin / kTile : 1;
+    const int row_chunks = lda / 8;   // 16-byte chunks per row of A
 
     // Global -> register -> LDS -> register pipeline.  Step kt waits in register stage kt % D, is stored to LDS buffer
     // kt % 2 one iteration before its products, and after that iteration's barrier its fragments are read into registers
@@ -158,16 +174,25 @@ __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
     StagedTiles st[D];
     const int last = nk - 1;
     const auto chunk_of = [&](int step) { return (step < last ? step : last) * (kTile / 8); };   // past the end: the last step again
+    // chunk offset of a step's A operand from ga0 / ga1: along the row, or (conv form) to an earlier row as well
+    const auto a_chunk_of = [&](int step) {
+        if constexpr (!CONV) return chunk_of(step);
+        else {
+            const int s = first_step + (step < last ? step : last);
+            const int tap = (s >= steps_per_tap ? 1 : 0) + (s >= 2 * steps_per_tap ? 1 : 0);   // taps <= 3
+            return (tap - (g.taps - 1)) * row_chunks + (s - tap * steps_per_tap) * (kTile / 8);
+        }
+    };
 #pragma unroll
     for (int d = 0; d < D; ++d)
-        if (EXACT || d < nk) st[d].load(ga0, ga1, gw0, gw1, chunk_of(d));
+        if (EXACT || d < nk) st[d].load(ga0, ga1, gw0, gw1, a_chunk_of(d), chunk_of(d));
 
     floatx16 acc = {0};
     const int frag = (lane & 31) * kLdsStride + 8 * (lane >> 5);
     const int fa_off = wm * 32 * kLdsStride + frag, fw_off = wn * 32 * kLdsStride + frag;
     StepFragments fr[2];   // fragments of step kt in fr[kt % 2]
     st[0].store(&s_a[0][0], &s_w[0][0], soff0, soff1);
-    if (EXACT || D < nk) st[0].load(ga0, ga1, gw0, gw1, chunk_of(D));
+    if (EXACT || D < nk) st[0].load(ga0, ga1, gw0, gw1, a_chunk_of(D), chunk_of(D));
     __syncthreads();
     fr[0].read(&s_a[0][fa_off], &s_w[0][fw_off]);
     // iteration kt: stage step kt + 1, barrier, read its fragments, multiply step kt
@@ -178,14 +203,14 @@ __global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
             const int dn = (d + 1) % D;   // register stage of step kt + 1 (a constant after unrolling)
             if constexpr (EXACT) {
                 st[dn].store(&s_a[(d + 1) & 1][0], &s_w[(d + 1) & 1][0], soff0, soff1);
-                st[dn].load(ga0, ga1, gw0, gw1, chunk_of(kt + 1 + D));
+                st[dn].load(ga0, ga1, gw0, gw1, a_chunk_of(kt + 1 + D), chunk_of(kt + 1 + D));
                 __syncthreads();
                 fr[(d + 1) & 1].read(&s_a[(d + 1) & 1][fa_off], &s_w[(d + 1) & 1][fw_off]);
                 fr[d & 1].multiply(acc);
             } else if (kt < nk) {   // the same for every thread of the grid
                 if (kt + 1 < nk) {
                     st[dn].store(&s_a[(d + 1) & 1][0], &s_w[(d + 1) & 1][0], soff0, soff1);
-                    if (kt + 1 + D < nk) st[dn].load(ga0, ga1, gw0, gw1, chunk_of(kt + 1 + D));
+                    if (kt + 1 + D < nk) st[dn].load(ga0, ga1, gw0, gw1, a_chunk_of(kt + 1 + D), chunk_of(kt + 1 + D));
                 }
                 __syncthreads();
                 if (kt + 1 < nk) fr[(d + 1) & 1].read(&s_a[(d + 1) & 1][fa_off], &s_w[(d + 1) & 1][fw_off]);
@@ -342,7 +367,7 @@ void launch_rows(State *st, int width, dim3 grid, float *x, const float *part, i
 // picks the smallest pair that covers the padded length (up to 4 and 16: 512 tokens), so that none is requested in vain.
 template <int kKeyTiles, int kValueSteps>
 __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, const _Float16 *vt, _Float16 *ctx, const EncParams *params,
-                                                            int tpad, int width, int vt_stride, float scale) {
+                                                            int tpad, int width, int vt_stride, float scale, int causal) {
     const int tokens = params->tokens;
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_inv[kQTile];
@@ -385,7 +410,11 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
             for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fq[j], k4[j], acc, 0, 0, 0);
             const int key = tile * 32 + (lane & 31);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) S[acc_row(r, lane) * sstride + key] = key < tokens ? acc[r] * scale : -3.0e38f;
+            for (int r = 0; r < 16; ++r) {
+                // causal: query q0 + row sees keys up to itself (src/graph.c:446-449); its own key is always in range
+                const bool seen = key < tokens && (!causal || key <= q0 + acc_row(r, lane));
+                S[acc_row(r, lane) * sstride + key] = seen ? acc[r] * scale : -3.0e38f;
+            }
         };
 #pragma unroll
         for (int t = 0; t < kKeyTiles; ++t)
@@ -473,18 +502,19 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
     }
 }
 
-template <int EPI>
+template <int EPI, bool CONV = false>
 int launch_gemm(State *st, const GemmArgs &g, int splits, char *error, size_t capacity) {
     if (g.M % kTile != 0 || g.N % kTile != 0 || g.M <= 0 || g.N <= 0 || g.K <= 0 || splits < 1 || g.K % (kTile * splits) != 0 ||
-        (splits > 1 && EPI != ENC_PARTIAL)) {
+        (splits > 1 && EPI != ENC_PARTIAL) ||
+        (CONV && (g.taps < 1 || g.taps > kLeadRows + 1 || g.cin <= 0 || g.cin % kTile != 0 || g.taps * g.cin != g.K))) {
         set_error(error, capacity, "encoder product: shape is not a multiple of the 64 x 64 x 64 tile");
         return -1;
     }
     const int steps = g.K / kTile / splits;
     const dim3 grid(g.N / kTile, g.M / kTile, splits), block(kThreads);
-    if (steps % kGemmDepth == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true>), grid, block, 0, st->stream, g);
-    else if (steps % 2 == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true>), grid, block, 0, st->stream, g);
-    else hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false>), grid, block, 0, st->stream, g);
+    if (steps % kGemmDepth == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true, CONV>), grid, block, 0, st->stream, g);
+    else if (steps % 2 == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true, CONV>), grid, block, 0, st->stream, g);
+    else hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false, CONV>), grid, block, 0, st->stream, g);
     return hip_check(hipGetLastError(), "encoder product launch", error, capacity);
 }
 
@@ -494,6 +524,30 @@ int f16_matrix(State *st, const float *host, size_t n, size_t k, const CachedWei
         set_error(error, capacity, "encoder: weight shape cannot be stored as f16");
         return -1;
     }
+    return 0;
+}
+
+// Conv weight [n][cin][taps] (the reference's conv1d layout, src/graph.c:318-352) as f16 [n][taps][cin] in device memory:
+// the K order in which k_enc_gemm's conv form walks the activation rows.  The caller owns the allocation.
+int tap_major_f16(State *st, const float *host, size_t n, size_t cin, size_t taps, _Float16 **out, char *error, size_t capacity) {
+    *out = nullptr;
+    std::vector<uint16_t> packed;
+    try {
+        packed.resize(n * cin * taps);
+    } catch (...) {
+        set_error(error, capacity, "out of memory converting an encoder conv weight");
+        return -1;
+    }
+    for (size_t o = 0; o < n; ++o)
+        for (size_t i = 0; i < cin; ++i)
+            for (size_t j = 0; j < taps; ++j) packed[(o * taps + j) * cin + i] = f32_to_f16_rne(host[(o * cin + i) * taps + j]);
+    void *dev = nullptr;
+    if (hip_check(hipMalloc(&dev, packed.size() * sizeof(uint16_t)), "encoder conv weight", error, capacity) != 0) return -1;
+    if (hip_check(hipMemcpy(dev, packed.data(), packed.size() * sizeof(uint16_t), hipMemcpyHostToDevice), "encoder conv weight upload", error, capacity) != 0) {
+        (void)hipFree(dev);
+        return -1;
+    }
+    *out = static_cast<_Float16 *>(dev);
     return 0;
 }
 
@@ -521,7 +575,8 @@ int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size
     const size_t lds = attention_lds_bytes((size_t)tpad);
     const size_t split_stride = (size_t)tpad * w;
     // K splits of the two width-wide products (few output tiles, long K): enough workgroups to occupy the chip
-    const int o_splits = pick_splits(w), down_splits = pick_splits(f);
+    const int taps = (int)e->taps;
+    const int o_splits = pick_splits(w), down_splits = pick_splits(f * taps);
     const float *pending = nullptr;   // partials of the last product, not yet added to x
     int pending_splits = 0;
     for (size_t l = 0; l < e->layers; ++l) {
@@ -533,20 +588,24 @@ int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size
         {
             // a wavefront scores every fourth 32-key tile and multiplies half of the keys in steps of 16
             const dim3 agrid(tpad / kQTile, (unsigned)e->heads), ablock(kThreads);
-            if (tpad <= 128) hipLaunchKernelGGL((k_enc_attention<1, 4>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale);
-            else if (tpad <= 256) hipLaunchKernelGGL((k_enc_attention<2, 8>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale);
-            else hipLaunchKernelGGL((k_enc_attention<4, 16>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale);
+            if (tpad <= 128) hipLaunchKernelGGL((k_enc_attention<1, 4>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale, e->causal);
+            else if (tpad <= 256) hipLaunchKernelGGL((k_enc_attention<2, 8>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale, e->causal);
+            else hipLaunchKernelGGL((k_enc_attention<4, 16>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale, e->causal);
         }
         g = GemmArgs{};
         g.a = e->ctx; g.w = static_cast<const _Float16 *>(e->o[l]->data); g.M = tpad; g.N = w; g.K = w; g.part = e->part;
         if (launch_gemm<ENC_PARTIAL>(st, g, o_splits, error, capacity) != 0) return -1;
         launch_rows<true>(st, w, row_grid, e->x, e->part, o_splits, split_stride, e->n2g[l], e->n2b[l], e->nrm, e->params, tpad);
         g = GemmArgs{};
-        g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->up[l]->data); g.M = tpad; g.N = f; g.K = w; g.out = e->hid;
-        if (launch_gemm<ENC_GELU>(st, g, 1, error, capacity) != 0) return -1;
+        g.a = e->nrm; g.M = tpad; g.N = f; g.K = w * taps; g.out = e->hid; g.taps = taps; g.cin = w;
+        g.w = taps > 1 ? e->conv_up[l] : static_cast<const _Float16 *>(e->up[l]->data);
+        if ((taps > 1 ? launch_gemm<ENC_GELU, true>(st, g, 1, error, capacity) : launch_gemm<ENC_GELU>(st, g, 1, error, capacity)) != 0) return -1;
         g = GemmArgs{};
-        g.a = e->hid; g.w = static_cast<const _Float16 *>(e->down[l]->data); g.M = tpad; g.N = w; g.K = f; g.part = e->part;
-        if (launch_gemm<ENC_PARTIAL>(st, g, down_splits, error, capacity) != 0) return -1;
+        g.a = e->hid; g.M = tpad; g.N = w; g.K = f * taps; g.part = e->part; g.taps = taps; g.cin = f;
+        g.w = taps > 1 ? e->conv_down[l] : static_cast<const _Float16 *>(e->down[l]->data);
+        if ((taps > 1 ? launch_gemm<ENC_PARTIAL, true>(st, g, down_splits, error, capacity)
+                      : launch_gemm<ENC_PARTIAL>(st, g, down_splits, error, capacity)) != 0)
+            return -1;
         pending = e->part;
         pending_splits = down_splits;
     }
@@ -571,6 +630,10 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
         set_error(error, capacity, "encoder_create: unsupported shape (needs 64-wide heads, widths that are multiples of 64) or missing weights");
         return -1;
     }
+    if (d->ffn_kernel != 0 && d->ffn_kernel != 1 && d->ffn_kernel != 3) {
+        set_error(error, capacity, "encoder_create: ffn_kernel must be 1 or 3");
+        return -1;
+    }
     auto *e = new (std::nothrow) mynah_hip_encoder();
     if (e == nullptr) {
         set_error(error, capacity, "out of memory creating the encoder");
@@ -578,6 +641,8 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
     }
     e->layers = d->layers; e->width = d->width; e->heads = d->heads; e->head_width = d->head_width; e->ffn = d->ffn_width;
     e->vocab = d->vocab; e->max_positions = d->max_positions;
+    e->taps = d->ffn_kernel == 3 ? 3 : 1;
+    e->causal = d->causal != 0;
     e->tpad_max = (d->max_positions + kTile - 1) / kTile * kTile;
     int lds = 0;
     if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, 0) != hipSuccess || lds <= 0) lds = 65536;
@@ -601,10 +666,18 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
         e->qkv.push_back(cw);
         if (f16_matrix(st, d->o_w[l], d->width, d->width, &cw, error, capacity) != 0) return fail();
         e->o.push_back(cw);
-        if (f16_matrix(st, d->up_w[l], d->ffn_width, d->width, &cw, error, capacity) != 0) return fail();
-        e->up.push_back(cw);
-        if (f16_matrix(st, d->down_w[l], d->width, d->ffn_width, &cw, error, capacity) != 0) return fail();
-        e->down.push_back(cw);
+        if (e->taps == 1) {
+            if (f16_matrix(st, d->up_w[l], d->ffn_width, d->width, &cw, error, capacity) != 0) return fail();
+            e->up.push_back(cw);
+            if (f16_matrix(st, d->down_w[l], d->width, d->ffn_width, &cw, error, capacity) != 0) return fail();
+            e->down.push_back(cw);
+        } else {
+            _Float16 *dev = nullptr;
+            if (tap_major_f16(st, d->up_w[l], d->ffn_width, d->width, e->taps, &dev, error, capacity) != 0) return fail();
+            e->conv_up.push_back(dev);
+            if (tap_major_f16(st, d->down_w[l], d->width, d->ffn_width, e->taps, &dev, error, capacity) != 0) return fail();
+            e->conv_down.push_back(dev);
+        }
         if (cached_vector(st, d->norm1[l], d->width, &v, error, capacity) != 0) return fail();
         e->n1g.push_back(v);
         v = nullptr;
@@ -623,9 +696,9 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
         if (hip_check(hipMalloc(p, bytes), "encoder workspace", error, capacity) != 0) return -1;
         return hip_check(hipMemsetAsync(*p, 0, bytes, st->stream), "encoder workspace clear", error, capacity);
     };
-    if (alloc(reinterpret_cast<void **>(&e->x), tp * w * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->nrm), tp * w * 2) != 0 ||
+    if (alloc(reinterpret_cast<void **>(&e->x), tp * w * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->nrm_alloc), (kLeadRows + tp) * w * 2) != 0 ||
         alloc(reinterpret_cast<void **>(&e->qk), tp * 2 * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->vt), w * tp * 2) != 0 ||
-        alloc(reinterpret_cast<void **>(&e->ctx), tp * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->hid), tp * f * 2) != 0 ||
+        alloc(reinterpret_cast<void **>(&e->ctx), tp * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->hid_alloc), (kLeadRows + tp) * f * 2) != 0 ||
         alloc(reinterpret_cast<void **>(&e->ids), tp * sizeof(int) + sizeof(EncParams)) != 0 ||
         alloc(reinterpret_cast<void **>(&e->part), kMaxSplits * tp * w * sizeof(float)) != 0)
         return fail();
@@ -633,6 +706,8 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
                   "encoder ids staging", error, capacity) != 0)
         return fail();
     e->params = reinterpret_cast<EncParams *>(e->ids + tp);   // tp is a multiple of 64: 8-byte aligned
+    e->nrm = e->nrm_alloc + kLeadRows * w;   // rows -2 and -1 stay zero; widths are multiples of 64, so both stay 16-byte aligned
+    e->hid = e->hid_alloc + kLeadRows * f;
     if (attention_lds_bytes(e->tpad_max) > 48 * 1024) {
         const int bytes = (int)attention_lds_bytes(e->tpad_max);
         if (hip_check(hipFuncSetAttribute(reinterpret_cast<const void *>(k_enc_attention<1, 4>), hipFuncAttributeMaxDynamicSharedMemorySize, bytes), "encoder attention LDS size", error, capacity) != 0 ||
@@ -651,8 +726,10 @@ extern "C" void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *e) {
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
     for (auto &g : e->graphs)
         if (g.second != nullptr) (void)hipGraphExecDestroy(g.second);
-    for (void *p : {(void *)e->x, (void *)e->nrm, (void *)e->qk, (void *)e->vt, (void *)e->ctx, (void *)e->hid, (void *)e->ids, (void *)e->part})
+    for (void *p : {(void *)e->x, (void *)e->nrm_alloc, (void *)e->qk, (void *)e->vt, (void *)e->ctx, (void *)e->hid_alloc, (void *)e->ids, (void *)e->part})
         if (p != nullptr) (void)hipFree(p);
+    for (_Float16 *p : e->conv_up) (void)hipFree(p);
+    for (_Float16 *p : e->conv_down) (void)hipFree(p);
     if (e->ids_host != nullptr) (void)hipHostFree(e->ids_host);
     delete e;
 }

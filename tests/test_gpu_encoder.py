@@ -4,6 +4,8 @@ Tolerances, both as normalised max error max|a-b|/max|b| over the whole output: 
 bit-exact (a gather); the encoder output is within 2e-3 -- the GPU rounds the operands of every product to f16
 and accumulates in f32, the oracle keeps the activations in f32.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -87,3 +89,73 @@ def test_encoder_prefill_rejects_bad_input(pkg, backend, synth):
     bad = synth.encoder_config(layers=1, width=96, heads=2)      # 48-wide heads: not supported by the MFMA path
     with pytest.raises(pkg.BackendError):
         pkg.Encoder(backend, bad, synth.encoder_weights(bad, seed=4))
+
+
+def _f16_bits(w):
+    h = lambda a: np.asarray(a, np.float32).astype(np.float16).view(np.uint16)
+    out = {"tok_table": h(w["tok_table"]), "pos_table": h(w["pos_table"]), "qkv_w": h(w["qkv"]), "o_w": h(w["o"]),
+           "up_w": h(w["up"]), "down_w": h(w["down"])}
+    for name in ("norm1_g", "norm1_b", "norm2_g", "norm2_b", "norm_out_g", "norm_out_b"):
+        out[name] = w.get(name)
+    return out
+
+
+def _prefill(pkg, backend, cfg, w, ids):
+    enc = pkg.Encoder(backend, cfg, w)
+    try:
+        dout = backend.alloc(ids.size * cfg["width"])
+        outs = []
+        for _ in range(3):                       # eager, capture, replay
+            enc.prefill(ids, 0, dout.ptr)
+            outs.append(dout.read().reshape(ids.size, cfg["width"]).copy())
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+        assert np.array_equal(outs[0].view(np.uint32), outs[2].view(np.uint32))
+        return outs[0]
+    finally:
+        enc.destroy()
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("kernel", [1, 3])
+@pytest.mark.parametrize("tokens,layers", [(1, 1), (2, 1), (37, 2), (65, 1), (256, 2), (300, 1)])
+def test_encoder_reference_form_matches_oracle(pkg, backend, orc, synth, nerr, causal, kernel, tokens, layers):
+    """The stack as the reference builds it (src/graph.c:634-711): causal mask, causal conv FFN of kernel size 1 or 3,
+    LayerNorm with and without bias, against the oracle (itself checked against the compiled reference on CPU)."""
+    _announce("encoder reference form causal=%s kernel=%d tokens=%d layers=%d" % (causal, kernel, tokens, layers))
+    cfg = dict(synth.encoder_config(layers=layers), causal=causal, ffn_kernel=kernel)
+    w = synth.encoder_weights_f16(cfg, seed=60 + kernel, kernel=kernel, biases=(tokens % 2 == 0))
+    ids = np.random.default_rng(61).integers(0, cfg["vocab"], size=tokens).astype(np.int32)
+    got = _prefill(pkg, backend, cfg, w, ids)
+    _, want = orc.encoder_prefill(cfg, _f16_bits(w), ids)
+    assert np.isfinite(got).all()
+    assert nerr(got, want) < 2e-3
+    if causal and tokens > 2:
+        # a causal stack's first rows do not depend on what follows them: bit-equal to a shorter call's
+        # when both calls pad to the same number of rows (the products then see the same tiles)
+        shorter = tokens - 1 if (tokens - 1 + 63) // 64 == (tokens + 63) // 64 else None
+        if shorter:
+            head = _prefill(pkg, backend, cfg, w, ids[:shorter])
+            assert np.array_equal(head.view(np.uint32), got[:shorter].view(np.uint32))
+
+
+@pytest.mark.parametrize("kernel", [1, 3])
+def test_encoder_matches_the_reference_fixture(pkg, backend, synth, nerr, kernel):
+    """Against the committed outputs of the compiled reference's transformer_stack (strict build) on the same weights."""
+    from tests.golden import make_golden as mg
+    _announce("encoder against the reference fixture, kernel=%d" % kernel)
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(mg.__file__)), "reference_vectors.npz"), allow_pickle=False)
+    cfg = dict(mg.ENC_CFG, ffn_kernel=kernel)
+    w = synth.encoder_weights_f16(cfg, seed=mg.ENC_SEED + kernel, kernel=kernel)
+    ids = np.random.default_rng(mg.ENC_SEED).integers(0, cfg["vocab"], size=mg.ENC_TOKENS).astype(np.int32)
+    if mg.crc(ids, *[w[k] for k in sorted(w) if w[k] is not None]) != gold["enc_k%d_input_crc" % kernel]:
+        pytest.skip("numpy's generator produced different synthetic inputs than when the fixture was written")
+    got = _prefill(pkg, backend, cfg, w, ids)
+    for tag in ("strict", "stock"):
+        assert nerr(got, gold["enc_k%d_%s_out" % (kernel, tag)]) < 2e-3
+
+
+def test_encoder_rejects_other_conv_kernels(pkg, backend, synth):
+    _announce("encoder: ffn_kernel 2 is refused")
+    cfg = dict(synth.encoder_config(layers=1), ffn_kernel=2)
+    with pytest.raises(pkg.BackendError, match="ffn_kernel"):
+        pkg.Encoder(backend, cfg, synth.encoder_weights_f16(cfg, seed=1, kernel=2))
