@@ -73,6 +73,7 @@ struct StepSlots {
     float *output[kMaxBatch];
     int length[kMaxBatch];
     int memory_length[kMaxBatch];
+    unsigned epoch;   // step counter (24 bits, never 0): goes into the tags of what workgroups of one launch hand each other
 };
 
 // A seam call held back for one call so that the next one can join its launch (backend_hip.hip, "seam fusion").

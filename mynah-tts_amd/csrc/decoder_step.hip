@@ -44,6 +44,13 @@ struct mynah_hip_decoder {
     // decoder, not the backend's shared workspace: that one is freed and reallocated when a later call needs more room,
     // and the captured graphs of this decoder hold the address they were recorded with.
     float *seam_partial = nullptr;
+    mynah::StepItem *self_items = nullptr, *cross_items = nullptr;   // work tables of the many-stream attention launches
+    // many streams: the attention launches fold their own partials, which travel as tagged records
+    // [kMaxBatch, heads, max_units, kStepRecord] (one area per attention kind); null: a fold kernel follows each launch
+    unsigned long long *self_records = nullptr, *cross_records = nullptr;
+    size_t records_bytes = 0;
+    unsigned item_epoch = 0;                    // next step counter for the tables (24 bits, never 0)
+    mynah::StepSlots last_slots;                // of the last step (the single-stage measurement graphs rebuild the tables from it)
     int max_units = 0;
     bool fused_attention = false;
     hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};
@@ -133,6 +140,7 @@ static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_
                                   const float *ln_gain, const float *ln_bias, char *error, size_t capacity) {
     StepAttnArgs a{};
     a.slots = d->dev_slots;
+    a.items = is_self ? d->self_items : d->cross_items;
     a.x = d->x;
     a.batch = batch;
     a.width = (int)d->width;
@@ -151,8 +159,12 @@ static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_
     a.scale = 1.0f / sqrtf((float)a.head_width);
     a.partial = d->partial;
     a.partial_ml = d->partial_ml;
+    a.records = batch > kConsumerFoldMaxBatch ? (is_self ? d->self_records : d->cross_records) : nullptr;
+    a.fold_out = is_self ? d->attn : d->ctx;
+    a.spin_limit = st->persist_spin_limit;
+    a.abort_word = st->persist_abort_dev;
     if (launch_step_attention(st, a, error, capacity) != 0) return -1;
-    if (batch > kConsumerFoldMaxBatch) return launch_step_fold(st, a, is_self ? d->attn : d->ctx, error, capacity);
+    if (batch > kConsumerFoldMaxBatch && a.records == nullptr) return launch_step_fold(st, a, a.fold_out, error, capacity);
     return 0;
 }
 
@@ -206,7 +218,11 @@ static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char
 
 DecoderRows decoder_rows(mynah_hip_decoder *d) { return DecoderRows{d->x, d->dev_slots, d->position}; }
 
-int decoder_enqueue_layers(State *st, mynah_hip_decoder *d, int batch, char *error, size_t capacity) {
+int decoder_enqueue_layers(State *st, mynah_hip_decoder *d, int batch, unsigned epoch_offset, char *error, size_t capacity) {
+    if (d->fused_attention && batch > kConsumerFoldMaxBatch &&
+        launch_step_items(st, d->dev_slots, epoch_offset, batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items,
+                          d->self_records != nullptr, error, capacity) != 0)
+        return -1;
     return enqueue_layers(st, d, batch, error, capacity, kAllStages, false);
 }
 
@@ -234,6 +250,10 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
     for (float *p : bufs)
         if (p != nullptr) (void)hipFree(p);
     if (d->dev_slots != nullptr) (void)hipFree(d->dev_slots);
+    if (d->self_items != nullptr) (void)hipFree(d->self_items);
+    if (d->self_records != nullptr) (void)hipFree(d->self_records);
+    if (d->cross_records != nullptr) (void)hipFree(d->cross_records);
+    if (d->cross_items != nullptr) (void)hipFree(d->cross_items);
     if (d->persist_layers != nullptr) (void)hipFree(d->persist_layers);
     if (d->persist_exchange != nullptr) (void)hipFree(d->persist_exchange);
     delete d;
@@ -330,6 +350,27 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
             if (rc == 0)
                 rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial_ml), B * heads_max * 2 * (size_t)d->max_units * sizeof(float)),
                                 "malloc", error, capacity);
+            // one entry per workgroup of the largest attention grid (kMaxBatch streams), self and cross
+            if (rc == 0)
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->self_items),
+                                          (size_t)step_attention_grid((int)d->heads, kMaxBatch, d->max_units, 1) * sizeof(StepItem)), "malloc", error, capacity);
+            // The launches fold their own partials unless switched off, the wait has no abort word to report through, or
+            // a (stream, head)'s records do not fit the LDS every launch may use without asking (long caches: the fold kernel then)
+            const char *fold_env = getenv("MYNAH_HIP_FOLD_IN_LAUNCH");
+            const bool fold_in_launch = !(fold_env != nullptr && strcmp(fold_env, "0") == 0) && st->persist_abort_dev != nullptr &&
+                                        d->layers < 255 && step_fold_lds_bytes(d->max_units) <= 40 * 1024;
+            if (rc == 0 && fold_in_launch) {
+                d->records_bytes = B * heads_max * (size_t)d->max_units * kStepRecord * sizeof(unsigned long long);
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->self_records), d->records_bytes), "malloc", error, capacity);
+                if (rc == 0) rc |= hip_check(hipMemset(d->self_records, 0, d->records_bytes), "memset", error, capacity);   // tag 0 is never waited for
+                if (rc == 0 && xw != 0) {
+                    rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->cross_records), d->records_bytes), "malloc", error, capacity);
+                    if (rc == 0) rc |= hip_check(hipMemset(d->cross_records, 0, d->records_bytes), "memset", error, capacity);
+                }
+            }
+            if (rc == 0 && xw != 0)
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->cross_items),
+                                          (size_t)step_attention_grid((int)d->cross_heads, kMaxBatch, d->max_units, 0) * sizeof(StepItem)), "malloc", error, capacity);
         }
     }
     if (rc == 0) {
@@ -473,6 +514,21 @@ static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_
 
 }  // namespace mynah
 
+namespace mynah {
+// `count` consecutive step counters (24 bits, never 0).  When the counter wraps, the tags of 2^24 steps ago are forgotten
+// first (outside any capture; the stream orders it).
+int decoder_next_epochs(State *st, mynah_hip_decoder *d, unsigned count, unsigned *first, char *error, size_t capacity) {
+    if (d->item_epoch + count >= 0xffffffu || d->item_epoch == 0) {
+        if (d->self_records != nullptr) MYNAH_TRY(hipMemsetAsync(d->self_records, 0, d->records_bytes, st->stream));
+        if (d->cross_records != nullptr) MYNAH_TRY(hipMemsetAsync(d->cross_records, 0, d->records_bytes, st->stream));
+        d->item_epoch = 1;
+    }
+    *first = d->item_epoch;
+    d->item_epoch += count;
+    return 0;
+}
+}  // namespace mynah
+
 extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch,
                                       char *error, size_t capacity) {
     State *st = enter_state(opaque);
@@ -516,7 +572,12 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
         const int taken = try_persistent_step(st, d, slots, batch, error, capacity);
         if (taken != 0) return taken < 0 ? -1 : 0;
     }
+    if (decoder_next_epochs(st, d, 1, &s.epoch, error, capacity) != 0) return -1;
+    d->last_slots = s;
     if (launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
+    if (d->fused_attention && B > kConsumerFoldMaxBatch &&
+        launch_step_items(st, d->dev_slots, 0, B, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items, d->self_records != nullptr, error, capacity) != 0)
+        return -1;
     if (st->graph_mode == 0 || d->eager_steps[B] == 0) {
         // the first step of a batch size also performs one-time kernel attribute set-up, which does not belong in a capture
         d->eager_steps[B] = 1;
@@ -576,6 +637,14 @@ extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *
             exec = nullptr;
             return -1;
         }
+    }
+    // a fresh step counter, as every real step has one: the workgroups that wait for tagged values then really wait
+    if (batch > (size_t)kConsumerFoldMaxBatch) {
+        if (decoder_next_epochs(st, d, 1, &d->last_slots.epoch, error, capacity) != 0) return -1;
+        if (launch_step_begin(st, d->last_slots, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
+        if (launch_step_items(st, d->dev_slots, 0, (int)batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items,
+                              d->self_records != nullptr, error, capacity) != 0)
+            return -1;
     }
     return hip_check(hipGraphLaunch(exec, st->stream), "stage graph launch", error, capacity);
 }

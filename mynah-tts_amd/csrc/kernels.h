@@ -85,8 +85,17 @@ int attention_chunk_rows(int is_self, size_t head_width, bool vector_rows, size_
 
 // Resident step: LayerNorm + activation quantisation + this head's slice of the Q (self: Q, K, V) projection +
 // attention over one cache chunk, per workgroup; writes split-L partials that the next matvec folds.
+// What one workgroup of a many-stream attention grid does: written per step by k_step_items, read by that workgroup.
+struct StepItem {
+    float *k, *v;      // the stream's K and V cache (self or cross), all layers
+    int length;        // rows in it before this step
+    int code;          // head | stream << 8 | unit << 16, or -1: nothing to do
+    int epoch;         // step counter (24 bits): with the layer, the tag of what workgroups of one launch hand each other
+    int pad1;
+};
 struct StepAttnArgs {
     const StepSlots *slots;
+    const StepItem *items;    // batch > kConsumerFoldMaxBatch: one entry per workgroup of this launch's grid
     const float *x;           // [batch, width] residual stream
     int batch, width;
     const float *ln_gain, *ln_bias;
@@ -100,8 +109,22 @@ struct StepAttnArgs {
     float scale;
     float *partial;           // partial outputs [batch, heads, max_units, head_width]
     float *partial_ml;        // chunk maxima and sums [batch, heads, 2, max_units]
+    // many streams, fold inside the launch: the partials as tagged records [batch, heads, max_units, kStepRecord] (non-null
+    // selects this form), the folded rows [batch, heads * head_width], and the bound of the fold workgroups' wait
+    unsigned long long *records;
+    float *fold_out;
+    unsigned spin_limit;
+    unsigned *abort_word;
 };
 int launch_step_attention(State *st, const StepAttnArgs &args, char *error, size_t capacity);
+// Workgroups of the attention launch for this shape (the table below has as many entries).
+int step_attention_grid(int heads, int batch, int max_units, int is_self);
+// Fills the work tables of the many-stream attention launches for one step (both kinds) from the slot table in device
+// memory; the tables' step counter is the slot table's plus `epoch_offset`.
+int launch_step_items(State *st, const StepSlots *dev_slots, unsigned epoch_offset, int batch, int heads, int cross_heads, int max_units,
+                      StepItem *self_items, StepItem *cross_items, bool with_fold, char *error, size_t capacity);
+// LDS a fold workgroup needs: the launch's dynamic LDS is at least this when it folds its own partials.
+size_t step_fold_lds_bytes(int max_units);
 // Folds the partials of the same arguments into out[batch][heads * head_width] (large batches only).
 int launch_step_fold(State *st, const StepAttnArgs &args, float *out, char *error, size_t capacity);
 bool step_attention_supported(int qtype, size_t width, size_t heads, size_t head_width);
@@ -177,6 +200,9 @@ struct DecoderRows {
     const float *position;
 };
 DecoderRows decoder_rows(mynah_hip_decoder *decoder);
-int decoder_enqueue_layers(State *st, mynah_hip_decoder *decoder, int batch, char *error, size_t capacity);
+// `epoch_offset`: added to the slot table's step counter for this pass (a caller that runs the layers several times per
+// slot table gives each pass its own).  decoder_next_epochs reserves `count` consecutive counters and returns the first.
+int decoder_enqueue_layers(State *st, mynah_hip_decoder *decoder, int batch, unsigned epoch_offset, char *error, size_t capacity);
+int decoder_next_epochs(State *st, mynah_hip_decoder *decoder, unsigned count, unsigned *first, char *error, size_t capacity);
 
 }  // namespace mynah

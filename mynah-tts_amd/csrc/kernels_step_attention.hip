@@ -25,9 +25,46 @@
 // The mapping from workgroup to (head, stream, unit) is static, so the weight slice and x are requested
 // before the slot table (lengths, cache pointers) has arrived; K and V rows follow as soon as it has.
 #include "step_attention_core.h"
+#include "tagged_exchange.h"
 
 namespace mynah {
 namespace {
+
+// max | sum of a record, and its two unused words: a reader takes a record as 68 tagged words
+__device__ __forceinline__ void put_ml(u64 *rec, unsigned tag, float m, float l) {
+    put(rec + kHw, tag, m);
+    put(rec + kHw + 1, tag, l);
+    put(rec + kHw + 2, tag, 0.0f);
+    put(rec + kHw + 3, tag, 0.0f);
+}
+
+// The fold of one (stream, head)'s partial records (fold_partials' arithmetic, units in order) from LDS, by 16 threads.
+// weight[u] = expf(max[u] - M), M the largest max: computed beforehand, one unit per thread, instead of one after the
+// other by each of the sixteen.
+__device__ __forceinline__ float fold_max(const float *rec, const int units) {
+    float M = -3.0e38f;
+    for (int u = 0; u < units; ++u) M = fmaxf(M, rec[u * kStepRecord + kHw]);
+    return M;
+}
+__device__ __forceinline__ float4 fold_records(const float *rec, const float *weight, const int units, const int t) {
+    float L = 0.0f;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int u = 0; u < units; ++u) {
+        const float *p = rec + u * kStepRecord;
+        const float wgt = weight[u];
+        const float4 ou = *reinterpret_cast<const float4 *>(p + 4 * t);
+        L = __builtin_fmaf(p[kHw + 1], wgt, L);
+        acc.x = __builtin_fmaf(ou.x, wgt, acc.x);
+        acc.y = __builtin_fmaf(ou.y, wgt, acc.y);
+        acc.z = __builtin_fmaf(ou.z, wgt, acc.z);
+        acc.w = __builtin_fmaf(ou.w, wgt, acc.w);
+    }
+    acc.x /= L; acc.y /= L; acc.z /= L; acc.w /= L;
+    return acc;
+}
+
+constexpr bool kFoldWaitFirst = true;    // a fold workgroup polls one word per thread before it requests its records (continuous requests for all of them slowed the attending workgroups: step 650 -> 666 us)
+constexpr int kFoldUnit = 0x7fff;   // unit number of a table entry that folds instead of attending
 
 // WFIX: model width known at compile time (0 = taken from the arguments): lane-group width, chunks per lane and passes
 // per bank become constants and the per-chunk range checks fold away.  The decoder stack's width (768) gets such a build.
@@ -65,6 +102,9 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     // Self-attention: unit 0 = Q+K of the new row, unit 1 = V of the new row, unit 2 + c = cache chunk c.
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     int unit, b, head;
+    int item_length = 0;
+    unsigned item_epoch = 0;
+    float *item_k = nullptr, *item_v = nullptr;
     if constexpr (PACKED == 0) {
         const int wg_units = a.max_units + (is_self ? 1 : 0);
         const int items = a.heads * a.batch * wg_units;
@@ -75,36 +115,42 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         b = hb % a.batch;
         head = hb / a.batch;
     } else {
-        // per head: [Q+K and V of every stream's new row (self only)] [groups of CP cache chunks that exist, stream by stream]
-        int chunk_items = 0;
-        for (int s = 0; s < a.batch; ++s) {
-            const int len = is_self ? slots->length[s] : slots->memory_length[s];
-            const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-            chunk_items += ((is_self ? live : max(live, 1)) + CP - 1) / CP;
-        }
-        const int row_items = is_self ? 2 * a.batch : 0;
-        const int per_head = row_items + chunk_items;
-        const int items = a.heads * per_head;
-        const int per_xcd = (items + 7) / 8;
-        const int item = xcd * per_xcd + slot;
-        if (slot >= per_xcd || item >= items) return;
-        head = item / per_head;
-        int r = item - head * per_head;
-        if (r < row_items) {
-            b = r >> 1;
-            unit = r & 1;
-        } else {
-            r -= row_items;
-            b = 0;
-            unit = 0;
-            int before = 0;
-            for (int s = 0; s < a.batch; ++s) {
-                const int len = is_self ? slots->length[s] : slots->memory_length[s];
-                const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-                const int n = ((is_self ? live : max(live, 1)) + CP - 1) / CP;
-                if (r >= before && r < before + n) { b = s; unit = r - before + (is_self ? 2 : 0); }
-                before += n;
+        // one table entry, written at the step's start for this very workgroup index (k_step_items): one read instead of
+        // the lengths, two loops over the streams and then the stream's cache pointers, each a round trip of its own
+        typedef int int8v __attribute__((ext_vector_type(8)));
+        static_assert(sizeof(StepItem) == sizeof(int8v), "an entry is read as one 32-byte scalar load");
+        const int8v raw = *reinterpret_cast<const int8v *>(a.items + blockIdx.x);   // all of it before the first branch
+        const int code = raw[5];
+        if (code < 0) return;
+        head = code & 0xff;
+        b = (code >> 8) & 0xff;
+        unit = code >> 16;
+        item_length = raw[4];
+        item_epoch = (unsigned)raw[6];
+        item_k = reinterpret_cast<float *>(((unsigned long long)(unsigned)raw[1] << 32) | (unsigned)raw[0]);
+        item_v = reinterpret_cast<float *>(((unsigned long long)(unsigned)raw[3] << 32) | (unsigned)raw[2]);
+    }
+    // ---- many streams: the fold of one (stream, head), by a workgroup numbered behind every workgroup that writes one of
+    // its records -- those are running or done when this one starts.  The records arrive as tagged words (tagged_exchange.h),
+    // tag = step counter | layer; the wait is bounded.  The next kernel reads the folded rows as plain memory.
+    if constexpr (PACKED == 1) {
+        if (unit == kFoldUnit) {
+            const int live = (item_length + kStepUnitRows - 1) / kStepUnitRows;
+            const int units = is_self ? live + 1 : max(live, 1);
+            const size_t sh = (size_t)b * a.heads + head;
+            float *s_fold = reinterpret_cast<float *>(smem);
+            Waiter wt{a.spin_limit, a.abort_word, false};
+            float *s_weight = s_fold + (size_t)a.max_units * kStepRecord;
+            fetch_tagged<8, kFoldWaitFirst>(a.records + sh * a.max_units * kStepRecord, s_fold, units * kStepRecord, (item_epoch << 8) | (unsigned)(a.layer + 1), wt);
+            if (__syncthreads_or(wt.dead ? 1 : 0)) {   // gave up: say so and leave; the host reports it at its next synchronisation
+                if (tid == 0) __hip_atomic_store(a.abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                return;
             }
+            const float M = fold_max(s_fold, units);
+            for (int u = tid; u < units; u += kThreads) s_weight[u] = expf(s_fold[u * kStepRecord + kHw] - M);
+            __syncthreads();
+            if (tid < kPosLanes) *reinterpret_cast<float4 *>(a.fold_out + sh * kHw + 4 * tid) = fold_records(s_fold, s_weight, units, tid);
+            return;
         }
     }
     const bool role_qk = is_self && unit == 0;
@@ -117,9 +163,9 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     // ---- slot table: read before any vector request.  The stream is the same for the whole workgroup and nothing has
     // been stored yet, so these are scalar loads, whose answers do not queue behind the vector loads below (vector loads
     // return in order: a table word requested after the weight rows could only be looked at once all of them had come).
-    const int length = is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
-    float *const k_base = is_self ? slots->self_k[b] : const_cast<float *>(slots->cross_k[b]);
-    float *const v_base = is_self ? slots->self_v[b] : const_cast<float *>(slots->cross_v[b]);
+    const int length = PACKED ? item_length : is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
+    float *const k_base = PACKED ? item_k : is_self ? slots->self_k[b] : const_cast<float *>(slots->cross_k[b]);
+    float *const v_base = PACKED ? item_v : is_self ? slots->self_v[b] : const_cast<float *>(slots->cross_v[b]);
 
     // With many streams most of the grid belongs to units that short streams do not have: there the slot table is
     // looked at first, so that such a workgroup leaves without having requested anything.  With one or two streams
@@ -228,6 +274,10 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     const size_t sh = (size_t)b * a.heads + head;
     float *out_m = a.partial_ml + sh * 2 * a.max_units;
     float *out_l = out_m + a.max_units;
+    // many streams: the partials leave as tagged records that the fold workgroups of this same launch wait for
+    const bool tagged = PACKED == 1 && a.records != nullptr;
+    u64 *const rec0 = a.records + sh * a.max_units * kStepRecord;
+    const unsigned tag = (item_epoch << 8) | (unsigned)(a.layer + 1);
 
     if (role_qk) {
         // this head's q and k of the new row; append k; the new row's own score opens partial 0
@@ -258,7 +308,10 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
             store_global(kc + (size_t)length * stride + (size_t)head * kHw + tid, kval);
             float d = s_proj[tid] * kval;
             d = wave_sum(d);
-            if (tid == 0) { out_m[0] = d * a.scale; out_l[0] = 1.0f; }   // exp(score - max) = 1
+            if (tid == 0) {   // exp(score - max) = 1
+                if (tagged) put_ml(rec0, tag, d * a.scale, 1.0f);
+                else { out_m[0] = d * a.scale; out_l[0] = 1.0f; }
+            }
         }
         return;
     }
@@ -269,7 +322,8 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         if (tid < kHw) {
             const float vval = s_proj[2 * kHw + tid];
             store_global(vc + (size_t)length * stride + (size_t)head * kHw + tid, vval);
-            a.partial[sh * a.max_units * kHw + tid] = vval;
+            if (tagged) put(rec0 + tid, tag, vval);
+            else a.partial[sh * a.max_units * kHw + tid] = vval;
         }
         return;
     }
@@ -279,8 +333,13 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     __syncthreads();
     float *out_o = a.partial + (sh * a.max_units + pidx) * kHw;   // the first chunk's partial; the second follows it
     if (count[0] <= 0) {   // empty memory (cross only): the context stays zero (src/graph.c:3242)
-        if (tid < kHw) out_o[tid] = 0.0f;
-        if (tid == 0) { out_m[pidx] = 0.0f; out_l[pidx] = 1.0f; }
+        if (tagged) {
+            if (tid < kHw) put(rec0 + (size_t)pidx * kStepRecord + tid, tag, 0.0f);
+            if (tid == 0) put_ml(rec0 + (size_t)pidx * kStepRecord, tag, 0.0f, 1.0f);
+        } else {
+            if (tid < kHw) out_o[tid] = 0.0f;
+            if (tid == 0) { out_m[pidx] = 0.0f; out_l[pidx] = 1.0f; }
+        }
         return;
     }
 
@@ -300,10 +359,90 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
             float4 o;
             float M, L;
             merge_chunk(t, s_red[cc], s_wave_ml[cc], o, M, L);
-            *reinterpret_cast<float4 *>(out_o + (size_t)cc * kHw + 4 * t) = o;
-            if (t == 0) { out_m[pidx + cc] = M; out_l[pidx + cc] = L; }
+            if (tagged) {
+                u64 *rec = rec0 + (size_t)(pidx + cc) * kStepRecord;
+                put(rec + 4 * t, tag, o.x); put(rec + 4 * t + 1, tag, o.y); put(rec + 4 * t + 2, tag, o.z); put(rec + 4 * t + 3, tag, o.w);
+                if (t == 0) put_ml(rec, tag, M, L);
+            } else {
+                *reinterpret_cast<float4 *>(out_o + (size_t)cc * kHw + 4 * t) = o;
+                if (t == 0) { out_m[pidx + cc] = M; out_l[pidx + cc] = L; }
+            }
         }
     }
+}
+
+// Work table of the PACKED builds, one entry per workgroup index of the attention grid: which (head, stream, unit) the
+// workgroup takes and where that stream's cache is.  Self-attention: first the Q+K and V roles of every stream's new row,
+// head-major; then, per head, the cache chunks that exist, stream by stream.  Each of the two lists is cut into eight
+// contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so a head's weight slice is fetched by at most two XCDs.
+// Behind the chunks that exist: one fold entry per (stream, head) when the launch folds its own partials.  Workgroups
+// numbered past all of these get code -1: they are the last ones of the grid and leave after this one read.  Written once per step, before the layers, from the slot table in device memory (whose
+// lengths a caller's own kernels may have advanced since the host last saw it) and its step counter plus `epoch_offset`.
+__device__ StepItem make_item(const StepSlots &slots, int batch, int heads, bool is_self, int wg, int epoch, bool with_fold) {
+    const StepItem dead{nullptr, nullptr, 0, -1, 0, 0};
+    int chunk_items = 0;
+    for (int s = 0; s < batch; ++s) {
+        const int len = is_self ? slots.length[s] : slots.memory_length[s];
+        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+        chunk_items += is_self ? live : max(live, 1);
+    }
+    int head, b = 0, unit = 0;
+    const int producers = is_self ? 2 * batch * heads : 0;
+    const int producer_grid = 8 * ((producers + 7) / 8);
+    if (wg < producer_grid) {
+        // the new row's Q+K and V roles, head-major, before everything that waits for them
+        const int per_xcd = producer_grid / 8;
+        const int xcd = wg & 7, slot = wg >> 3;
+        const int p = xcd * per_xcd + slot;
+        if (p >= producers) return dead;
+        head = p / (2 * batch);
+        const int r = p - head * 2 * batch;
+        b = r >> 1;
+        unit = r & 1;
+    } else {
+        const int w2 = wg - producer_grid;
+        const int items = heads * chunk_items;
+        const int per_xcd = (items + 7) / 8;
+        const int xcd = w2 & 7, slot = w2 >> 3;
+        const int item = xcd * per_xcd + slot;
+        if (w2 >= 8 * per_xcd) {
+            // behind every workgroup that attends: one fold per (stream, head)
+            const int f = w2 - 8 * per_xcd;
+            if (!with_fold || f >= heads * batch) return dead;
+            head = f / batch;
+            b = f - head * batch;
+            unit = kFoldUnit;
+        } else {
+            if (item >= items) return dead;
+            head = item / chunk_items;
+            const int r = item - head * chunk_items;
+            int before = 0;
+            for (int s = 0; s < batch; ++s) {
+                const int len = is_self ? slots.length[s] : slots.memory_length[s];
+                const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+                const int n = is_self ? live : max(live, 1);
+                if (r >= before && r < before + n) { b = s; unit = r - before + (is_self ? 2 : 0); }
+                before += n;
+            }
+        }
+    }
+    StepItem it;
+    it.k = is_self ? slots.self_k[b] : const_cast<float *>(slots.cross_k[b]);
+    it.v = is_self ? slots.self_v[b] : const_cast<float *>(slots.cross_v[b]);
+    it.length = is_self ? slots.length[b] : slots.memory_length[b];
+    it.code = head | (b << 8) | (unit << 16);
+    it.epoch = epoch;
+    it.pad1 = 0;
+    return it;
+}
+
+__global__ void __launch_bounds__(kThreads) k_step_items(const StepSlots *slots, unsigned epoch_offset, int batch, int heads, int cross_heads,
+                                                         StepItem *self_items, int self_entries, StepItem *cross_items, int cross_entries,
+                                                         bool with_fold) {
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    const int epoch = (int)((slots->epoch + epoch_offset) & 0xffffffu);
+    if (i < self_entries) self_items[i] = make_item(*slots, batch, heads, true, i, epoch, with_fold);
+    else if (i - self_entries < cross_entries) cross_items[i - self_entries] = make_item(*slots, batch, cross_heads, false, i - self_entries, epoch, with_fold);
 }
 
 // Stand-alone fold of the partials into out[stream][heads * 64]: used instead of the consumer-side fold when
@@ -324,10 +463,13 @@ template <int QT>
 int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const int chunks = a.width / Chunk<QT>::n;
     const int lg = lane_group_log2(chunks);
-    const int items = a.heads * a.batch * (a.max_units + (a.is_self ? 1 : 0));   // self: the new row takes two workgroups
-    const int per_xcd = (items + 7) / 8;
-    const int grid = 8 * per_xcd;
-    const size_t lds = (size_t)a.width * (kQuantised<QT> ? 1 : 4);
+    const int grid = step_attention_grid(a.heads, a.batch, a.max_units, a.is_self);
+    const int per_xcd = grid / 8;
+    size_t lds = (size_t)a.width * (kQuantised<QT> ? 1 : 4);
+    if (a.batch > kConsumerFoldMaxBatch && a.records != nullptr) {   // the fold workgroups stage a (stream, head)'s records there
+        const size_t fold_bytes = step_fold_lds_bytes(a.max_units);
+        lds = lds > fold_bytes ? lds : fold_bytes;
+    }
     const bool latency = a.batch <= kConsumerFoldMaxBatch;
     const dim3 g(grid), t(kThreads);
     if (a.width == 768) {
@@ -364,8 +506,38 @@ int launch_step_fold(State *st, const StepAttnArgs &a, float *out, char *error, 
     return hip_check(hipGetLastError(), "step fold launch", error, capacity);
 }
 
+size_t step_fold_lds_bytes(int max_units) { return (size_t)max_units * (kStepRecord + 1) * sizeof(float); }   // records + one weight per unit
+
+int step_attention_grid(int heads, int batch, int max_units, int is_self) {
+    if (batch > kConsumerFoldMaxBatch) {
+        // table order: the new rows' two roles (self; max_units counts the new row), the cache chunks, the folds
+        const int producers = is_self ? 8 * ((2 * batch * heads + 7) / 8) : 0;
+        const int chunks = heads * batch * (max_units - (is_self ? 1 : 0));
+        return producers + 8 * ((chunks + 7) / 8) + 8 * ((heads * batch + 7) / 8);
+    }
+    const int items = heads * batch * (max_units + (is_self ? 1 : 0));   // self: the new row takes two workgroups
+    return 8 * ((items + 7) / 8);
+}
+
+int launch_step_items(State *st, const StepSlots *dev_slots, unsigned epoch_offset, int batch, int heads, int cross_heads, int max_units,
+                      StepItem *self_items, StepItem *cross_items, bool with_fold, char *error, size_t capacity) {
+    if (batch < 1 || batch > kMaxBatch || heads < 1 || heads > 255 || cross_heads < 0 || cross_heads > 255 || max_units < 1 || max_units > 32000 ||
+        dev_slots == nullptr || self_items == nullptr || (cross_heads > 0 && cross_items == nullptr)) {
+        set_error(error, capacity, "step items: invalid shape");
+        return -1;
+    }
+    const int self_entries = step_attention_grid(heads, batch, max_units, 1);
+    const int cross_entries = cross_heads > 0 ? step_attention_grid(cross_heads, batch, max_units, 0) : 0;
+    const int total = self_entries + cross_entries;
+    hipLaunchKernelGGL(k_step_items, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0, st->stream, dev_slots, epoch_offset, batch,
+                       heads, cross_heads, self_items, self_entries, cross_items, cross_entries, with_fold);
+    return hip_check(hipGetLastError(), "step items launch", error, capacity);
+}
+
 int launch_step_attention(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     if (a.batch < 1 || a.batch > kMaxBatch || a.max_units < 1 || a.partial == nullptr || a.partial_ml == nullptr || a.slots == nullptr ||
+        (a.batch > kConsumerFoldMaxBatch &&
+         (a.items == nullptr || a.layer >= 255 || (a.records != nullptr && (a.abort_word == nullptr || a.fold_out == nullptr)))) ||
         !step_attention_supported(a.qtype, (size_t)a.width, (size_t)a.heads, (size_t)a.head_width)) {
         set_error(error, capacity, "step attention: invalid or unsupported shape");
         return -1;

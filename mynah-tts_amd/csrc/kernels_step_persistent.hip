@@ -23,110 +23,14 @@
 // abort word and leave; every other workgroup then runs into the same bound or sees the word, so the grid always drains.
 // The host reports an aborted step at the next synchronisation.  The grid never exceeds what the chip holds at once.
 #include "step_attention_core.h"
+#include "tagged_exchange.h"
 
 namespace mynah {
 namespace {
 
-typedef unsigned long long u64;
-
 constexpr int kW = 768;        // model width of this build
 constexpr int kF = 3072;       // FFN width of this build
 constexpr int kPF = kPrefetchLatency;
-
-__device__ __forceinline__ void put(u64 *p, unsigned tag, float v) {
-    __hip_atomic_store(p, ((u64)tag << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ u64 get(const u64 *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ unsigned tag_of(u64 v) { return (unsigned)(v >> 32); }
-__device__ __forceinline__ float value_of(u64 v) { return __uint_as_float((unsigned)v); }
-
-struct Waiter {
-    unsigned limit;
-    unsigned *abort_word;
-    bool dead;
-};
-
-__device__ __forceinline__ bool give_up(Waiter &w, unsigned &spins) {
-    ++spins;
-    if (spins > w.limit) return true;
-    if ((spins & 255u) == 0u && __hip_atomic_load(w.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) return true;
-    return false;
-}
-
-// A poll is a request that bypasses the caches, about a microsecond there and back.  Polling one request at a time finds a
-// value, on average, half a round trip after it could have; two requests in flight, checked in turn, halve that.
-__device__ __forceinline__ void poll_until(const u64 *p, const unsigned tag, Waiter &w) {
-    unsigned spins = 0;
-    u64 first = get(p), second = get(p);
-    while (tag_of(first) != tag) {
-        if (give_up(w, spins)) { w.dead = true; break; }
-        first = second;
-        second = get(p);
-    }
-}
-
-// n tagged values -> dst (LDS floats, same index), by the whole workgroup, N values per thread and batch.  Every request
-// is issued whatever the index (clamped), so that none sits behind a branch.  The batch itself is the poll, and two
-// batches are in flight: while one is looked at the next is already on its way, so a value is found a fraction of a
-// round trip after it became visible instead of half a round trip (one batch in flight) or a whole one (poll one value,
-// then request the batch).  WAIT_FIRST: poll one value of the batch before the first batch is requested -- for batches of
-// tens of values, which many workgroups would otherwise request over and over while the producers are still at work.
-template <int N, bool WAIT_FIRST>
-__device__ __forceinline__ void fetch_tagged(const u64 *src, float *dst, const int n, const unsigned tag, Waiter &w) {
-    const int tid = threadIdx.x;
-    for (int base = 0; base < n; base += kThreads * N) {
-        u64 v[N], next[N];
-        unsigned spins = 0;
-        if (WAIT_FIRST) {
-            int last = base + (N - 1) * kThreads + tid;
-            while (last >= n) last -= kThreads;
-            if (last >= base) poll_until(src + last, tag, w);
-        }
-#pragma unroll
-        for (int j = 0; j < N; ++j) {
-            const int i = base + j * kThreads + tid;
-            v[j] = get(src + (i < n ? i : n - 1));
-        }
-        if (!WAIT_FIRST) {
-#pragma unroll
-            for (int j = 0; j < N; ++j) {
-                const int i = base + j * kThreads + tid;
-                next[j] = get(src + (i < n ? i : n - 1));
-            }
-        }
-        for (;;) {
-            bool all = true;
-#pragma unroll
-            for (int j = 0; j < N; ++j) {
-                const int i = base + j * kThreads + tid;
-                all = all && (i >= n || tag_of(v[j]) == tag);
-            }
-            if (all || w.dead) break;
-            if (give_up(w, spins)) { w.dead = true; break; }
-#pragma unroll
-            for (int j = 0; j < N; ++j) {
-                const int i = base + j * kThreads + tid;
-                v[j] = WAIT_FIRST ? get(src + (i < n ? i : n - 1)) : next[j];
-                if (!WAIT_FIRST) next[j] = get(src + (i < n ? i : n - 1));
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < N; ++j) {
-            const int i = base + j * kThreads + tid;
-            if (i < n) dst[i] = value_of(v[j]);
-        }
-    }
-}
-
-// One tagged value that is expected to be there already (it was requested ahead); polls if it is not.
-__device__ __forceinline__ float settle(u64 v, const u64 *p, const unsigned tag, Waiter &w) {
-    unsigned spins = 0;
-    while (tag_of(v) != tag) {
-        if (give_up(w, spins)) { w.dead = true; break; }
-        v = get(p);
-    }
-    return value_of(v);
-}
 
 // ---- workgroup roles ---------------------------------------------------------------------------------------------------
 

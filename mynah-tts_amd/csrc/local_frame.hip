@@ -45,6 +45,8 @@ struct LocalItemDev {
 // Everything a frame brings from the host, uploaded in one copy.
 struct LocalFrameDev {
     float *logits_copy;             // optional [batch, streams, vocab]: the masked logits, for parity tests
+    unsigned epoch_base;            // step counter of this frame's first pass through the stack (pass s uses base + s)
+    unsigned reserved;
     LocalItemDev items[kMaxBatch];  // generator state and EOS flags updated in place
 };
 
@@ -93,7 +95,10 @@ __device__ __forceinline__ int count_above(const unsigned long long *list, int n
 __global__ void __launch_bounds__(256) k_local_begin(LocalFrameDev *frame, const StepSlots slots, StepSlots *dev_slots, float *x,
                                                      const float *position, int width) {
     const int b = blockIdx.x;
-    if (b == 0 && threadIdx.x == 0) *dev_slots = slots;
+    if (b == 0 && threadIdx.x == 0) {
+        *dev_slots = slots;
+        dev_slots->epoch = frame->epoch_base;
+    }
     const float *src = frame->items[b].decoder_last;
     for (int d = threadIdx.x; d < width; d += 256) x[(size_t)b * width + d] = position != nullptr ? src[d] + position[d] : src[d];
     if (threadIdx.x == 0) {
@@ -373,7 +378,7 @@ static int enqueue_frame(State *st, mynah_hip_local *l, int B, char *error, size
     hipLaunchKernelGGL(k_local_begin, dim3(B), dim3(256), 0, st->stream, l->frame, slots, rows.slots, rows.x, rows.position, width);
     MYNAH_TRY(hipGetLastError());
     for (size_t stream = 0; stream < l->streams; ++stream) {
-        if (decoder_enqueue_layers(st, l->stack, B, error, capacity) != 0) return -1;
+        if (decoder_enqueue_layers(st, l->stack, B, (unsigned)stream, error, capacity) != 0) return -1;
         const CachedWeight *cw = l->projection[stream];
         for (int b0 = 0; b0 < B; b0 += kBatchTile) {
             LinearArgs p{};
@@ -515,6 +520,8 @@ extern "C" int mynah_hip_local_frame(void *state, mynah_hip_local *l, mynah_hip_
     const int B = (int)batch;
     MYNAH_TRY(hipStreamSynchronize(st->stream));   // the staging buffers of the previous frame may still be in flight
     l->frame_host->logits_copy = dev_logits_copy;
+    if (decoder_next_epochs(st, l->stack, (unsigned)l->streams, &l->frame_host->epoch_base, error, capacity) != 0) return -1;
+    l->frame_host->reserved = 0;
     for (size_t b = 0; b < batch; ++b) {
         LocalItemDev &d = l->frame_host->items[b];
         d.decoder_last = items[b].dev_decoder_last;
