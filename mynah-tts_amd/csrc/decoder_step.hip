@@ -49,6 +49,7 @@ struct mynah_hip_decoder {
     // [kMaxBatch, heads, max_units, kStepRecord] (one area per attention kind); null: a fold kernel follows each launch
     unsigned long long *self_records = nullptr, *cross_records = nullptr;
     size_t records_bytes = 0;
+    int self_slots = 0, cross_slots = 0;   // workgroups of the many-stream attention kernels that the device holds at once
     unsigned item_epoch = 0;                    // next step counter for the tables (24 bits, never 0)
     mynah::StepSlots last_slots;                // of the last step (the single-stage measurement graphs rebuild the tables from it)
     int max_units = 0;
@@ -221,7 +222,7 @@ DecoderRows decoder_rows(mynah_hip_decoder *d) { return DecoderRows{d->x, d->dev
 int decoder_enqueue_layers(State *st, mynah_hip_decoder *d, int batch, unsigned epoch_offset, char *error, size_t capacity) {
     if (d->fused_attention && batch > kConsumerFoldMaxBatch &&
         launch_step_items(st, d->dev_slots, epoch_offset, batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items,
-                          d->self_records != nullptr, error, capacity) != 0)
+                          d->self_records != nullptr, d->self_slots, d->cross_slots, error, capacity) != 0)
         return -1;
     return enqueue_layers(st, d, batch, error, capacity, kAllStages, false);
 }
@@ -353,7 +354,7 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
             // one entry per workgroup of the largest attention grid (kMaxBatch streams), self and cross
             if (rc == 0)
                 rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->self_items),
-                                          (size_t)step_attention_grid((int)d->heads, kMaxBatch, d->max_units, 1) * sizeof(StepItem)), "malloc", error, capacity);
+                                          (size_t)step_attention_grid((int)d->heads, kMaxBatch, d->max_units, 1, true) * sizeof(StepItem)), "malloc", error, capacity);
             // The launches fold their own partials unless switched off, the wait has no abort word to report through, or
             // a (stream, head)'s records do not fit the LDS every launch may use without asking (long caches: the fold kernel then)
             const char *fold_env = getenv("MYNAH_HIP_FOLD_IN_LAUNCH");
@@ -368,9 +369,23 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
                     if (rc == 0) rc |= hip_check(hipMemset(d->cross_records, 0, d->records_bytes), "memset", error, capacity);
                 }
             }
+            if (rc == 0) {
+                // Chunks per workgroup: one, unless MYNAH_HIP_ATTN_SLOTS names a number of workgroup slots to fit the launch into
+                // ("device": what the device holds of this kernel at once).  Measured with eight ragged streams, same box, twice
+                // each: grouped to fit the device (pairs of chunks, one round of workgroups instead of two) 654 us per step,
+                // one chunk per workgroup 649 us -- the second chunk of a pair waits for its rows a full round trip after the first.
+                d->self_slots = d->cross_slots = 1 << 30;
+                const char *slots_env = getenv("MYNAH_HIP_ATTN_SLOTS");
+                if (slots_env != nullptr && strcmp(slots_env, "device") == 0) {
+                    d->self_slots = step_attention_slots(l0.qkv->qtype, (int)w, d->max_units, 1, d->self_records != nullptr);
+                    d->cross_slots = xw != 0 ? step_attention_slots(l0.q_cross->qtype, (int)w, d->max_units, 0, d->cross_records != nullptr) : 0;
+                } else if (slots_env != nullptr && atoi(slots_env) > 0) {
+                    d->self_slots = d->cross_slots = atoi(slots_env);
+                }
+            }
             if (rc == 0 && xw != 0)
                 rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->cross_items),
-                                          (size_t)step_attention_grid((int)d->cross_heads, kMaxBatch, d->max_units, 0) * sizeof(StepItem)), "malloc", error, capacity);
+                                          (size_t)step_attention_grid((int)d->cross_heads, kMaxBatch, d->max_units, 0, true) * sizeof(StepItem)), "malloc", error, capacity);
         }
     }
     if (rc == 0) {
@@ -576,7 +591,7 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
     d->last_slots = s;
     if (launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
     if (d->fused_attention && B > kConsumerFoldMaxBatch &&
-        launch_step_items(st, d->dev_slots, 0, B, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items, d->self_records != nullptr, error, capacity) != 0)
+        launch_step_items(st, d->dev_slots, 0, B, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items, d->self_records != nullptr, d->self_slots, d->cross_slots, error, capacity) != 0)
         return -1;
     if (st->graph_mode == 0 || d->eager_steps[B] == 0) {
         // the first step of a batch size also performs one-time kernel attribute set-up, which does not belong in a capture
@@ -643,7 +658,7 @@ extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *
         if (decoder_next_epochs(st, d, 1, &d->last_slots.epoch, error, capacity) != 0) return -1;
         if (launch_step_begin(st, d->last_slots, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
         if (launch_step_items(st, d->dev_slots, 0, (int)batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items,
-                              d->self_records != nullptr, error, capacity) != 0)
+                              d->self_records != nullptr, d->self_slots, d->cross_slots, error, capacity) != 0)
             return -1;
     }
     return hip_check(hipGraphLaunch(exec, st->stream), "stage graph launch", error, capacity);

@@ -91,7 +91,7 @@ struct StepItem {
     int length;        // rows in it before this step
     int code;          // head | stream << 8 | unit << 16, or -1: nothing to do
     int epoch;         // step counter (24 bits): with the layer, the tag of what workgroups of one launch hand each other
-    int pad1;
+    int group;         // consecutive cache chunks a chunk workgroup takes (unit u: chunks group * (u - first) ..)
 };
 struct StepAttnArgs {
     const StepSlots *slots;
@@ -118,11 +118,13 @@ struct StepAttnArgs {
 };
 int launch_step_attention(State *st, const StepAttnArgs &args, char *error, size_t capacity);
 // Workgroups of the attention launch for this shape (the table below has as many entries).
-int step_attention_grid(int heads, int batch, int max_units, int is_self);
+int step_attention_grid(int heads, int batch, int max_units, int is_self, bool packed);
 // Fills the work tables of the many-stream attention launches for one step (both kinds) from the slot table in device
 // memory; the tables' step counter is the slot table's plus `epoch_offset`.
 int launch_step_items(State *st, const StepSlots *dev_slots, unsigned epoch_offset, int batch, int heads, int cross_heads, int max_units,
-                      StepItem *self_items, StepItem *cross_items, bool with_fold, char *error, size_t capacity);
+                      StepItem *self_items, StepItem *cross_items, bool with_fold, int self_slots, int cross_slots, char *error, size_t capacity);
+// Workgroups of the many-stream attention kernel for this weight storage and shape that the device holds at once.
+int step_attention_slots(int qtype, int width, int max_units, int is_self, bool with_fold);
 // LDS a fold workgroup needs: the launch's dynamic LDS is at least this when it folds its own partials.
 size_t step_fold_lds_bytes(int max_units);
 // Folds the partials of the same arguments into out[batch][heads * head_width] (large batches only).

@@ -63,7 +63,6 @@ __device__ __forceinline__ float4 fold_records(const float *rec, const float *we
     return acc;
 }
 
-constexpr bool kFoldWaitFirst = true;    // a fold workgroup polls one word per thread before it requests its records (continuous requests for all of them slowed the attending workgroups: step 650 -> 666 us)
 constexpr int kFoldUnit = 0x7fff;   // unit number of a table entry that folds instead of attending
 
 // WFIX: model width known at compile time (0 = taken from the arguments): lane-group width, chunks per lane and passes
@@ -104,6 +103,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     int unit, b, head;
     int item_length = 0;
     unsigned item_epoch = 0;
+    int item_group = 1;   // consecutive cache chunks this workgroup takes, one after the other
     float *item_k = nullptr, *item_v = nullptr;
     if constexpr (PACKED == 0) {
         const int wg_units = a.max_units + (is_self ? 1 : 0);
@@ -127,6 +127,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         unit = code >> 16;
         item_length = raw[4];
         item_epoch = (unsigned)raw[6];
+        item_group = raw[7];
         item_k = reinterpret_cast<float *>(((unsigned long long)(unsigned)raw[1] << 32) | (unsigned)raw[0]);
         item_v = reinterpret_cast<float *>(((unsigned long long)(unsigned)raw[3] << 32) | (unsigned)raw[2]);
     }
@@ -141,7 +142,12 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
             float *s_fold = reinterpret_cast<float *>(smem);
             Waiter wt{a.spin_limit, a.abort_word, false};
             float *s_weight = s_fold + (size_t)a.max_units * kStepRecord;
-            fetch_tagged<8, kFoldWaitFirst>(a.records + sh * a.max_units * kStepRecord, s_fold, units * kStepRecord, (item_epoch << 8) | (unsigned)(a.layer + 1), wt);
+            // (Measured and not kept: continuous requests for every word -- the polling took bandwidth from the workgroups
+            // that read the caches, batch-8 step 650 -> 666 us; one slow poll per record and then the fetch -- a second round
+            // trip behind the last record, 655 -> 672 us.)
+            const u64 *records = a.records + sh * a.max_units * kStepRecord;
+            const unsigned fold_tag = (item_epoch << 8) | (unsigned)(a.layer + 1);
+            fetch_tagged<8, true>(records, s_fold, units * kStepRecord, fold_tag, wt);
             if (__syncthreads_or(wt.dead ? 1 : 0)) {   // gave up: say so and leave; the host reports it at its next synchronisation
                 if (tid == 0) __hip_atomic_store(a.abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                 return;
@@ -155,7 +161,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     }
     const bool role_qk = is_self && unit == 0;
     const bool role_v = is_self && unit == 1;
-    const int chunk = CP * (is_self ? unit - 2 : unit);   // first cache chunk of this workgroup (chunk roles only)
+    const int chunk = (PACKED == 1 ? item_group : CP) * (is_self ? unit - 2 : unit);   // first cache chunk of this workgroup (chunk roles only)
     const int pidx = is_self ? chunk + 1 : chunk;         // partial slot of that chunk (slot 0 of self-attention = the new row)
 
     const int chunks = a.width / kEpc;
@@ -213,6 +219,76 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     int count[CP];
 #pragma unroll
     for (int cc = 0; cc < CP; ++cc) count[cc] = new_row ? 0 : max(0, min(kStepUnitRows, length - p0 - cc * kStepUnitRows));
+    // ---- many streams, cache chunks: the whole of this role here, ahead of the new row's roles.  Kept apart from the code
+    // below so that nothing of those roles (their second weight bank, parked in registers) is alive while this one runs:
+    // the chunk loop then fits the registers that one chunk needs.
+    if constexpr (PACKED == 1) {
+        if (!new_row) {
+            static_assert(CP == 1, "the chunk loop keeps one chunk's rows in registers");
+            const bool have_rows = count[0] > 0;   // an empty memory has none (its pointers may be null): read the activation buffer
+            const float *const k_from = have_rows ? kc : a.x;
+            const float *const v_from = have_rows ? vc : a.x;
+            float4 kv[kRowsPerThread], vv[kRowsPerThread];
+#pragma unroll
+            for (int i = 0; i < kRowsPerThread; ++i) {
+                // every request is issued, whatever the lane's row: a row past the chunk's end repeats the chunk's last row
+                const int row = have_rows ? p0 + min(g + kPosPerPass * i, count[0] - 1) : 0;
+                const size_t at = (size_t)row * stride + col;
+                kv[i] = load_global4(k_from + at);
+                vv[i] = load_global4(v_from + at);
+            }
+            if constexpr (PF != kPrefetchLatency) load_activations<1, NVT>(pro, act, whole_workgroup(), xr, gv, bv);
+            finish_activations<QT, 1, NVT>(pro, whole_workgroup(), xr, gv, bv, smem, s_sx, s_scratch);
+            const size_t sh = (size_t)b * a.heads + head;
+            u64 *const rec0 = a.records + sh * a.max_units * kStepRecord;   // the partials leave as tagged records (see the fold role)
+            const unsigned tag = (item_epoch << 8) | (unsigned)(a.layer + 1);
+            project_rows<QT, PF>(a, pre, PF, 0, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
+            __syncthreads();
+            if (!have_rows) {   // empty memory (cross only): the context stays zero (src/graph.c:3242)
+                if (tid < kHw) put(rec0 + (size_t)pidx * kStepRecord + tid, tag, 0.0f);
+                if (tid == 0) put_ml(rec0 + (size_t)pidx * kStepRecord, tag, 0.0f, 1.0f);
+                return;
+            }
+            const float4 qv = *reinterpret_cast<const float4 *>(s_proj + 4 * j);
+            const auto finish_chunk = [&](const int cc) {   // behind a barrier after attend_chunk: merge the four wavefronts in order 0..3
+                if (tid < kPosLanes) {
+                    float4 o;
+                    float M, L;
+                    merge_chunk(tid, s_red[0], s_wave_ml[0], o, M, L);
+                    u64 *rec = rec0 + (size_t)(pidx + cc) * kStepRecord;
+                    put(rec + 4 * tid, tag, o.x); put(rec + 4 * tid + 1, tag, o.y); put(rec + 4 * tid + 2, tag, o.z); put(rec + 4 * tid + 3, tag, o.w);
+                    if (tid == 0) put_ml(rec, tag, M, L);
+                }
+            };
+            attend_chunk(qv, kv, vv, count[0], a.scale, s_red[0], s_wave_ml[0]);
+            __syncthreads();
+            finish_chunk(0);
+            // The workgroup goes on to the next chunks of its group, one at a time in the same registers.  A chunk's partial
+            // is what a workgroup with that chunk alone computes, so the bits do not depend on how chunks are grouped; the
+            // group size only sets how many workgroups the launch has (few enough to be resident at once, see make_item).
+            // The stream's last group may be short; the count is the same for the whole workgroup.
+            const int trips = __builtin_amdgcn_readfirstlane(min(item_group, nchunks - chunk));
+            const int first_row = __builtin_amdgcn_readfirstlane(p0);
+            const int total_rows = __builtin_amdgcn_readfirstlane(length);
+#pragma nounroll
+            for (int cc = 1; cc < trips; ++cc) {
+                const int row0 = first_row + cc * kStepUnitRows;
+                const int rows = min(kStepUnitRows, total_rows - row0);
+#pragma unroll
+                for (int i = 0; i < kRowsPerThread; ++i) {
+                    const size_t at = (size_t)(row0 + min(g + kPosPerPass * i, rows - 1)) * stride + col;
+                    kv[i] = load_global4(kc + at);
+                    vv[i] = load_global4(vc + at);
+                }
+                __syncthreads();            // the merge of the chunk before has read what this one writes
+                attend_chunk(qv, kv, vv, rows, a.scale, s_red[0], s_wave_ml[0]);
+                __syncthreads();
+                finish_chunk(cc);
+            }
+            return;
+        }
+    }
+
     // A chunk role keeps its cache rows here.  The Q+K role has no cache rows and parks its second bank of weight
     // passes in the same registers (as raw bits), so that no role needs more registers than the largest one.
     static_assert(2 * kRowsPerThread >= 4 * PF, "the second weight bank must fit the cache-row registers");
@@ -275,7 +351,7 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
     float *out_m = a.partial_ml + sh * 2 * a.max_units;
     float *out_l = out_m + a.max_units;
     // many streams: the partials leave as tagged records that the fold workgroups of this same launch wait for
-    const bool tagged = PACKED == 1 && a.records != nullptr;
+    constexpr bool tagged = PACKED == 1;
     u64 *const rec0 = a.records + sh * a.max_units * kStepRecord;
     const unsigned tag = (item_epoch << 8) | (unsigned)(a.layer + 1);
 
@@ -328,18 +404,15 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
         return;
     }
 
+    if constexpr (PACKED == 1) return;   // the chunk role of the many-stream build is complete further up
+
     // ---- cache chunk: this head's q, then the chunk's scores
     project_rows<QT, PF>(a, pre, PF, 0, kHw, head, lg, chunks, smem, s_sx[0], s_proj);
     __syncthreads();
     float *out_o = a.partial + (sh * a.max_units + pidx) * kHw;   // the first chunk's partial; the second follows it
     if (count[0] <= 0) {   // empty memory (cross only): the context stays zero (src/graph.c:3242)
-        if (tagged) {
-            if (tid < kHw) put(rec0 + (size_t)pidx * kStepRecord + tid, tag, 0.0f);
-            if (tid == 0) put_ml(rec0 + (size_t)pidx * kStepRecord, tag, 0.0f, 1.0f);
-        } else {
-            if (tid < kHw) out_o[tid] = 0.0f;
-            if (tid == 0) { out_m[pidx] = 0.0f; out_l[pidx] = 1.0f; }
-        }
+        if (tid < kHw) out_o[tid] = 0.0f;
+        if (tid == 0) { out_m[pidx] = 0.0f; out_l[pidx] = 1.0f; }
         return;
     }
 
@@ -359,14 +432,8 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
             float4 o;
             float M, L;
             merge_chunk(t, s_red[cc], s_wave_ml[cc], o, M, L);
-            if (tagged) {
-                u64 *rec = rec0 + (size_t)(pidx + cc) * kStepRecord;
-                put(rec + 4 * t, tag, o.x); put(rec + 4 * t + 1, tag, o.y); put(rec + 4 * t + 2, tag, o.z); put(rec + 4 * t + 3, tag, o.w);
-                if (t == 0) put_ml(rec, tag, M, L);
-            } else {
-                *reinterpret_cast<float4 *>(out_o + (size_t)cc * kHw + 4 * t) = o;
-                if (t == 0) { out_m[pidx + cc] = M; out_l[pidx + cc] = L; }
-            }
+            *reinterpret_cast<float4 *>(out_o + (size_t)cc * kHw + 4 * t) = o;
+            if (t == 0) { out_m[pidx + cc] = M; out_l[pidx + cc] = L; }
         }
     }
 }
@@ -376,15 +443,27 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 // head-major; then, per head, the cache chunks that exist, stream by stream.  Each of the two lists is cut into eight
 // contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so a head's weight slice is fetched by at most two XCDs.
 // Behind the chunks that exist: one fold entry per (stream, head) when the launch folds its own partials.  Workgroups
-// numbered past all of these get code -1: they are the last ones of the grid and leave after this one read.  Written once per step, before the layers, from the slot table in device memory (whose
-// lengths a caller's own kernels may have advanced since the host last saw it) and its step counter plus `epoch_offset`.
-__device__ StepItem make_item(const StepSlots &slots, int batch, int heads, bool is_self, int wg, int epoch, bool with_fold) {
+// numbered past all of these get code -1: they are the last ones of the grid and leave after this one read.  Written once
+// per step, before the layers, from the slot table in device memory (whose lengths a caller's own kernels may have advanced
+// since the host last saw it) and its step counter plus `epoch_offset`.
+// A workgroup takes `group` consecutive chunks of its stream and head: the smallest number with which every workgroup of the
+// launch is resident at once (`budget` = the chip's workgroup slots for this kernel less the other roles).  A second round
+// of workgroups would start when the first ends and run its whole dependent chain again, some 5 us, for a fifth of the work.
+__device__ StepItem make_item(const StepSlots &slots, int batch, int heads, bool is_self, int wg, int epoch, bool with_fold, int budget) {
     const StepItem dead{nullptr, nullptr, 0, -1, 0, 0};
-    int chunk_items = 0;
+    // chunks per workgroup: the smallest group size with which the launch's chunk workgroups are at most `budget`
+    int all_chunks = 0;
     for (int s = 0; s < batch; ++s) {
         const int len = is_self ? slots.length[s] : slots.memory_length[s];
         const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-        chunk_items += is_self ? live : max(live, 1);
+        all_chunks += is_self ? live : max(live, 1);
+    }
+    const int group = max(1, (heads * all_chunks + budget - 1) / max(budget, 1));
+    int chunk_items = 0;   // groups per head
+    for (int s = 0; s < batch; ++s) {
+        const int len = is_self ? slots.length[s] : slots.memory_length[s];
+        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+        chunk_items += ((is_self ? live : max(live, 1)) + group - 1) / group;
     }
     int head, b = 0, unit = 0;
     const int producers = is_self ? 2 * batch * heads : 0;
@@ -420,7 +499,7 @@ __device__ StepItem make_item(const StepSlots &slots, int batch, int heads, bool
             for (int s = 0; s < batch; ++s) {
                 const int len = is_self ? slots.length[s] : slots.memory_length[s];
                 const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-                const int n = is_self ? live : max(live, 1);
+                const int n = ((is_self ? live : max(live, 1)) + group - 1) / group;
                 if (r >= before && r < before + n) { b = s; unit = r - before + (is_self ? 2 : 0); }
                 before += n;
             }
@@ -432,17 +511,18 @@ __device__ StepItem make_item(const StepSlots &slots, int batch, int heads, bool
     it.length = is_self ? slots.length[b] : slots.memory_length[b];
     it.code = head | (b << 8) | (unit << 16);
     it.epoch = epoch;
-    it.pad1 = 0;
+    it.group = group;
     return it;
 }
 
 __global__ void __launch_bounds__(kThreads) k_step_items(const StepSlots *slots, unsigned epoch_offset, int batch, int heads, int cross_heads,
                                                          StepItem *self_items, int self_entries, StepItem *cross_items, int cross_entries,
-                                                         bool with_fold) {
+                                                         bool with_fold, int self_budget, int cross_budget) {
     const int i = blockIdx.x * kThreads + threadIdx.x;
     const int epoch = (int)((slots->epoch + epoch_offset) & 0xffffffu);
-    if (i < self_entries) self_items[i] = make_item(*slots, batch, heads, true, i, epoch, with_fold);
-    else if (i - self_entries < cross_entries) cross_items[i - self_entries] = make_item(*slots, batch, cross_heads, false, i - self_entries, epoch, with_fold);
+    if (i < self_entries) self_items[i] = make_item(*slots, batch, heads, true, i, epoch, with_fold, self_budget);
+    else if (i - self_entries < cross_entries)
+        cross_items[i - self_entries] = make_item(*slots, batch, cross_heads, false, i - self_entries, epoch, with_fold, cross_budget);
 }
 
 // Stand-alone fold of the partials into out[stream][heads * 64]: used instead of the consumer-side fold when
@@ -459,33 +539,59 @@ __global__ void __launch_bounds__(kThreads) k_step_fold(const float *partial, co
     reinterpret_cast<float4 *>(out + (size_t)stream * heads * kHw)[f4] = fold_partials(src, stream, f4);
 }
 
+using StepAttnKernel = void (*)(const StepAttnArgs, const int, const int);
+
+// The build that runs a shape: fixed-width builds for the decoder stack's width; `latency`: the build for one or two
+// streams (work found from the workgroup index; it also serves more streams when the launch cannot fold its own partials),
+// else the many-stream build (work table, partials as tagged records, fold inside the launch).
+template <int QT>
+StepAttnKernel kernel_for(int width, bool is_self, bool latency) {
+    if (width == 768) {
+        // the fixed-shape build needs few enough registers (154 for int8) to hold three workgroups per CU with four-pass banks
+        if (is_self && latency) return k_step_attention<QT, 1, kPrefetchLatency, 768, 1, 0>;
+        if (is_self) return k_step_attention<QT, 1, kPrefetchLatency, 768, 1, 1>;
+        if (latency) return k_step_attention<QT, 1, kPrefetchLatency, 768, 0, 0>;
+        return k_step_attention<QT, 1, kPrefetchLatency, 768, 0, 1>;
+    }
+    if (width <= 1024) {
+        if (latency) return k_step_attention<QT, 1, kPrefetchLatency, 0, -1, 0>;
+        return k_step_attention<QT, 1, kPrefetchThroughput, 0, -1, 1>;
+    }
+    if (latency) return k_step_attention<QT, 3, kPrefetchLatency, 0, -1, 0>;
+    return k_step_attention<QT, 3, kPrefetchThroughput, 0, -1, 1>;
+}
+
+template <int QT>
+size_t lds_for(int width, int max_units, bool with_fold) {
+    size_t lds = (size_t)width * (kQuantised<QT> ? 1 : 4);
+    if (with_fold) {   // the fold workgroups stage a (stream, head)'s records there
+        const size_t fold_bytes = step_fold_lds_bytes(max_units);
+        lds = lds > fold_bytes ? lds : fold_bytes;
+    }
+    return lds;
+}
+
 template <int QT>
 int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const int chunks = a.width / Chunk<QT>::n;
     const int lg = lane_group_log2(chunks);
-    const int grid = step_attention_grid(a.heads, a.batch, a.max_units, a.is_self);
+    const bool packed_grid = a.records != nullptr;
+    const int grid = step_attention_grid(a.heads, a.batch, a.max_units, a.is_self, packed_grid);
     const int per_xcd = grid / 8;
-    size_t lds = (size_t)a.width * (kQuantised<QT> ? 1 : 4);
-    if (a.batch > kConsumerFoldMaxBatch && a.records != nullptr) {   // the fold workgroups stage a (stream, head)'s records there
-        const size_t fold_bytes = step_fold_lds_bytes(a.max_units);
-        lds = lds > fold_bytes ? lds : fold_bytes;
-    }
-    const bool latency = a.batch <= kConsumerFoldMaxBatch;
-    const dim3 g(grid), t(kThreads);
-    if (a.width == 768) {
-        // the fixed-shape build needs few enough registers (154 for int8) to hold three workgroups per CU with four-pass banks
-        if (a.is_self && latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 1, 0>), g, t, lds, st->stream, a, lg, per_xcd);
-        else if (a.is_self) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 1, 1>), g, t, lds, st->stream, a, lg, per_xcd);
-        else if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 0, 0>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 768, 0, 1>), g, t, lds, st->stream, a, lg, per_xcd);
-    } else if (a.width <= 1024) {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchLatency, 0, -1, 0>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 1, kPrefetchThroughput, 0, -1, 1>), g, t, lds, st->stream, a, lg, per_xcd);
-    } else {
-        if (latency) hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchLatency, 0, -1, 0>), g, t, lds, st->stream, a, lg, per_xcd);
-        else hipLaunchKernelGGL((k_step_attention<QT, 3, kPrefetchThroughput, 0, -1, 1>), g, t, lds, st->stream, a, lg, per_xcd);
-    }
+    const bool packed = a.records != nullptr;
+    const size_t lds = lds_for<QT>(a.width, a.max_units, packed);
+    hipLaunchKernelGGL(kernel_for<QT>(a.width, a.is_self != 0, !packed), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
     return hip_check(hipGetLastError(), "step attention launch", error, capacity);
+}
+
+template <int QT>
+int slots_t(int width, int max_units, bool is_self, bool with_fold) {
+    int per_cu = 0, device = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void *>(kernel_for<QT>(width, is_self, false)), kThreads,
+                                                     lds_for<QT>(width, max_units, with_fold)) != hipSuccess ||
+        hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+        return 0;
+    return per_cu * cus;
 }
 
 }  // namespace
@@ -499,6 +605,15 @@ bool step_attention_supported(int qtype, size_t width, size_t heads, size_t head
     return (chunks + group - 1) / group <= 4;   // one register group of four chunks per lane and pass
 }
 
+int step_attention_slots(int qtype, int width, int max_units, int is_self, bool with_fold) {
+    switch (qtype) {
+        case MYNAH_HIP_F32: return slots_t<MYNAH_HIP_F32>(width, max_units, is_self != 0, with_fold);
+        case MYNAH_HIP_F16: return slots_t<MYNAH_HIP_F16>(width, max_units, is_self != 0, with_fold);
+        case MYNAH_HIP_INT8: return slots_t<MYNAH_HIP_INT8>(width, max_units, is_self != 0, with_fold);
+        default: return slots_t<MYNAH_HIP_INT4>(width, max_units, is_self != 0, with_fold);
+    }
+}
+
 int launch_step_fold(State *st, const StepAttnArgs &a, float *out, char *error, size_t capacity) {
     const int f4 = a.heads * (kHw / 4);
     const dim3 grid((unsigned)((f4 + kThreads - 1) / kThreads), (unsigned)a.batch);
@@ -508,8 +623,8 @@ int launch_step_fold(State *st, const StepAttnArgs &a, float *out, char *error, 
 
 size_t step_fold_lds_bytes(int max_units) { return (size_t)max_units * (kStepRecord + 1) * sizeof(float); }   // records + one weight per unit
 
-int step_attention_grid(int heads, int batch, int max_units, int is_self) {
-    if (batch > kConsumerFoldMaxBatch) {
+int step_attention_grid(int heads, int batch, int max_units, int is_self, bool packed) {
+    if (packed) {
         // table order: the new rows' two roles (self; max_units counts the new row), the cache chunks, the folds
         const int producers = is_self ? 8 * ((2 * batch * heads + 7) / 8) : 0;
         const int chunks = heads * batch * (max_units - (is_self ? 1 : 0));
@@ -520,24 +635,25 @@ int step_attention_grid(int heads, int batch, int max_units, int is_self) {
 }
 
 int launch_step_items(State *st, const StepSlots *dev_slots, unsigned epoch_offset, int batch, int heads, int cross_heads, int max_units,
-                      StepItem *self_items, StepItem *cross_items, bool with_fold, char *error, size_t capacity) {
+                      StepItem *self_items, StepItem *cross_items, bool with_fold, int self_slots, int cross_slots, char *error, size_t capacity) {
     if (batch < 1 || batch > kMaxBatch || heads < 1 || heads > 255 || cross_heads < 0 || cross_heads > 255 || max_units < 1 || max_units > 32000 ||
         dev_slots == nullptr || self_items == nullptr || (cross_heads > 0 && cross_items == nullptr)) {
         set_error(error, capacity, "step items: invalid shape");
         return -1;
     }
-    const int self_entries = step_attention_grid(heads, batch, max_units, 1);
-    const int cross_entries = cross_heads > 0 ? step_attention_grid(cross_heads, batch, max_units, 0) : 0;
+    const int self_entries = step_attention_grid(heads, batch, max_units, 1, true);
+    const int cross_entries = cross_heads > 0 ? step_attention_grid(cross_heads, batch, max_units, 0, true) : 0;
     const int total = self_entries + cross_entries;
     hipLaunchKernelGGL(k_step_items, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0, st->stream, dev_slots, epoch_offset, batch,
-                       heads, cross_heads, self_items, self_entries, cross_items, cross_entries, with_fold);
+                       heads, cross_heads, self_items, self_entries, cross_items, cross_entries, with_fold,
+                       self_slots - 8 * ((2 * batch * heads + 7) / 8) - (with_fold ? heads * batch : 0), cross_slots - (with_fold ? cross_heads * batch : 0));
     return hip_check(hipGetLastError(), "step items launch", error, capacity);
 }
 
 int launch_step_attention(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     if (a.batch < 1 || a.batch > kMaxBatch || a.max_units < 1 || a.partial == nullptr || a.partial_ml == nullptr || a.slots == nullptr ||
-        (a.batch > kConsumerFoldMaxBatch &&
-         (a.items == nullptr || a.layer >= 255 || (a.records != nullptr && (a.abort_word == nullptr || a.fold_out == nullptr)))) ||
+        (a.records != nullptr && (a.batch <= kConsumerFoldMaxBatch || a.items == nullptr || a.layer >= 255 || a.abort_word == nullptr ||
+                                  a.fold_out == nullptr)) ||
         !step_attention_supported(a.qtype, (size_t)a.width, (size_t)a.heads, (size_t)a.head_width)) {
         set_error(error, capacity, "step attention: invalid or unsupported shape");
         return -1;

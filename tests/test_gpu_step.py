@@ -481,3 +481,46 @@ def test_captured_step_survives_a_growing_backend_workspace(pkg, backend, synth)
         assert np.array_equal(third[b].view(np.uint32), first[b].view(np.uint32)), "stream %d changed after the workspace grew" % b
     bh.close()
     a.close()
+
+
+@pytest.mark.parametrize("qtype_name", ["int8", "f32", "int4"])
+def test_many_stream_forms_agree(pkg, backend, synth, qtype_name):
+    """Five ragged streams (one with an empty cache, one without encoder memory) stepped by the many-stream attention launches
+    in each of their forms -- partials folded inside the launch (the default), by a fold kernel behind it, and with two or
+    more cache chunks per workgroup -- give the same bits, outputs and appended cache rows, eagerly and as a captured graph."""
+    import os
+    _announce("many-stream forms agree, %s" % qtype_name)
+    lengths, mems = [700, 0, 129, 383, 512], [40, 7, 0, 130, 129]
+    cfg = synth.decoder_config(layers=3, capacity=800)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=5)
+    backend.set_quant(QT[qtype_name])
+    results = {}
+    try:
+        for name, env in (("default", {}), ("fold kernel", {"MYNAH_HIP_FOLD_IN_LAUNCH": "0"}), ("grouped to the device", {"MYNAH_HIP_ATTN_SLOTS": "device"}),
+                          ("grouped into 100 slots", {"MYNAH_HIP_ATTN_SLOTS": "100"})):
+            os.environ.update(env)
+            try:
+                h = Harness(pkg, backend, cfg, weights, streams)     # the decoder reads the switches when it is created
+            finally:
+                for k in env:
+                    del os.environ[k]
+            outs = []
+            for _ in range(3):                                      # eager, capture, replay
+                for b in range(len(lengths)):
+                    h.reset_cache(b)
+                outs.append(h.step())
+            rows = [tuple(a[:, lengths[b]].copy() for a in h.cache_rows(b)) for b in range(len(lengths))]
+            h.close()
+            for b in range(len(lengths)):
+                assert np.isfinite(outs[0][b]).all()
+                for o in outs[1:]:
+                    assert np.array_equal(o[b].view(np.uint32), outs[0][b].view(np.uint32)), "%s: replay differs, stream %d" % (name, b)
+            results[name] = (outs[0], rows)
+        ref_out, ref_rows = results["default"]
+        for name, (out, rows) in results.items():
+            for b in range(len(lengths)):
+                assert np.array_equal(out[b].view(np.uint32), ref_out[b].view(np.uint32)), "%s differs from the default, stream %d" % (name, b)
+                assert np.array_equal(rows[b][0], ref_rows[b][0]) and np.array_equal(rows[b][1], ref_rows[b][1]), "%s: appended rows differ" % name
+    finally:
+        backend.set_quant(0)
