@@ -297,8 +297,7 @@ static int hip_matmul(void *opaque, const float *input, float *output, size_t ro
     MYNAH_TRY(hipMemcpyAsync(din, input, in_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
     if (matmul_device(st, din, dout, rows, iw, ow, weight, bias, error, capacity) != 0) return -1;
     MYNAH_TRY(hipMemcpyAsync(output, dout, out_n * sizeof(float), hipMemcpyDeviceToHost, st->stream));
-    MYNAH_TRY(hipStreamSynchronize(st->stream));
-    return 0;
+    return synchronise(st, error, capacity);
 }
 
 static int hip_sgemm(void *opaque, int ta, int tb, size_t m, size_t n, size_t k, float alpha, const float *a, size_t lda,
@@ -321,15 +320,27 @@ static int hip_sgemm(void *opaque, int ta, int tb, size_t m, size_t n, size_t k,
     MYNAH_TRY(hipMemcpyAsync(db, b, b_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
     if (beta != 0.0f) MYNAH_TRY(hipMemcpyAsync(dc, c, c_n * sizeof(float), hipMemcpyHostToDevice, st->stream));
     if (launch_sgemm(st, ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc, error, capacity) != 0) return -1;
-    MYNAH_TRY(hipMemcpyAsync(c, dc, c_n * sizeof(float), hipMemcpyDeviceToHost, st->stream));
-    MYNAH_TRY(hipStreamSynchronize(st->stream));
-    return 0;
+    // only the m x n result goes back: what lies between a row's end and the next row (ldc > n) is the caller's
+    MYNAH_TRY(hipMemcpy2DAsync(c, ldc * sizeof(float), dc, ldc * sizeof(float), n * sizeof(float), m, hipMemcpyDeviceToHost, st->stream));
+    return synchronise(st, error, capacity);
 }
+
+// Buffers handed to mynah_hip_dev_free wait here until the stream is next idle: work enqueued before the call may still
+// read them, nothing enqueued after it does, so any later synchronisation makes them safe to free -- and a caller that
+// frees per-utterance buffers in a loop does not stall the stream once per buffer.
+static void free_pending(State *st) {   // the stream is idle
+    for (void *p : st->pending_free) (void)hipFree(p);
+    st->pending_free.clear();
+}
+constexpr size_t kMaxPendingFrees = 64;
 
 static void hip_close(void *opaque) {
     State *st = enter_state(opaque);
     if (st == nullptr) return;
     (void)hipStreamSynchronize(st->stream);
+    free_pending(st);
+    for (auto &kv : st->position_tables)
+        if (kv.second.data != nullptr) (void)hipFree(kv.second.data);
     for (auto &kv : st->weights) {
         if (kv.second.data != nullptr) (void)hipFree(kv.second.data);
         if (kv.second.scales != nullptr) (void)hipFree(kv.second.scales);
@@ -531,19 +542,30 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
 
 // =========================================================================================== memory
 extern "C" int mynah_hip_dev_alloc(void *opaque, size_t n, float **dev_ptr, char *error, size_t capacity) {
-    (void)opaque;
+    State *st = opaque != nullptr ? enter_state(opaque) : nullptr;
     if (dev_ptr == nullptr || n == 0 || n > SIZE_MAX / sizeof(float)) {
         set_error(error, capacity, "invalid device allocation size");
         return -1;
     }
-    return hip_check(hipMalloc(reinterpret_cast<void **>(dev_ptr), n * sizeof(float)), "malloc", error, capacity);
+    hipError_t r = hipMalloc(reinterpret_cast<void **>(dev_ptr), n * sizeof(float));
+    if (r == hipErrorOutOfMemory && st != nullptr && !st->pending_free.empty()) {   // memory that is only waiting to be freed
+        (void)hipGetLastError();
+        if (hipStreamSynchronize(st->stream) == hipSuccess) free_pending(st);
+        r = hipMalloc(reinterpret_cast<void **>(dev_ptr), n * sizeof(float));
+    }
+    return hip_check(r, "malloc", error, capacity);
 }
 
 extern "C" void mynah_hip_dev_free(void *opaque, float *dev_ptr) {
     State *st = enter_state(opaque);
     if (dev_ptr == nullptr) return;
-    if (st != nullptr) (void)hipStreamSynchronize(st->stream);
-    (void)hipFree(dev_ptr);
+    if (st == nullptr) {
+        (void)hipDeviceSynchronize();
+        (void)hipFree(dev_ptr);
+        return;
+    }
+    st->pending_free.push_back(dev_ptr);
+    if (st->pending_free.size() >= kMaxPendingFrees && hipStreamSynchronize(st->stream) == hipSuccess) free_pending(st);
 }
 
 extern "C" int mynah_hip_h2d(void *opaque, const float *host, float *dev_ptr, size_t n, char *error, size_t capacity) {
@@ -556,10 +578,18 @@ extern "C" int mynah_hip_h2d(void *opaque, const float *host, float *dev_ptr, si
     return copy_to_device(st, dev_ptr, host, bytes, error, capacity);
 }
 
-// Waits for the stream; a persistent step that gave up one of its bounded waits has left results that mean nothing, and is
-// reported here, by the first call that synchronises after it.
-static int synchronise(State *st, char *error, size_t capacity) {
+// Waits for the stream, and reports what an earlier call could not: a held-back launch that failed inside a call with
+// no way to say so, and a step whose workgroups gave up one of their bounded waits (its results mean nothing).  Every
+// entry point that hands data or a completion to the host ends here, so the first of them after the failure returns it.
+int mynah::synchronise(State *st, char *error, size_t capacity) {
+    if (st->deferred_error[0] != '\0') {
+        set_error(error, capacity, st->deferred_error);
+        st->deferred_error[0] = '\0';
+        (void)hipStreamSynchronize(st->stream);
+        return -1;
+    }
     MYNAH_TRY(hipStreamSynchronize(st->stream));
+    free_pending(st);
     if (st->persist_abort_host != nullptr && st->persist_abort_host[0] != 0u) {
         st->persist_abort_host[0] = 0u;
         set_error(error, capacity, "resident decode step gave up a bounded wait between its workgroups; its outputs are invalid");
@@ -598,12 +628,6 @@ extern "C" int mynah_hip_download(void *opaque, const float *dev_ptr, float *hos
 extern "C" int mynah_hip_sync(void *opaque, char *error, size_t capacity) {
     State *st = enter_state(opaque);
     MYNAH_NEED_STATE(st);
-    if (st->deferred_error[0] != '\0') {   // a held-back launch failed inside a call that could not report it
-        set_error(error, capacity, st->deferred_error);
-        st->deferred_error[0] = '\0';
-        (void)hipStreamSynchronize(st->stream);
-        return -1;
-    }
     return synchronise(st, error, capacity);
 }
 
@@ -819,23 +843,33 @@ extern "C" int mynah_hip_sgemm_dev(void *opaque, int ta, int tb, size_t m, size_
                                    size_t lda, const float *db, size_t ldb, float beta, float *dc, size_t ldc, char *error,
                                    size_t capacity) {
     if (da == nullptr || db == nullptr || dc == nullptr) { set_error(error, capacity, "invalid sgemm arguments"); return -1; }
-    return launch_sgemm(enter_state(opaque), ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc, error, capacity);
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return launch_sgemm(st, ta, tb, m, n, k, alpha, da, lda, db, ldb, beta, dc, ldc, error, capacity);
 }
 extern "C" int mynah_hip_softmax_dev(void *opaque, float *d, size_t rows, size_t cols, size_t valid, char *error, size_t capacity) {
     if (d == nullptr || cols > 0x7fffffffu) { set_error(error, capacity, "invalid softmax arguments"); return -1; }
-    return launch_softmax(enter_state(opaque), d, rows, cols, valid, error, capacity);
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return launch_softmax(st, d, rows, cols, valid, error, capacity);
 }
 extern "C" int mynah_hip_copy_dev(void *opaque, float *dst, const float *src, size_t n, char *error, size_t capacity) {
     if (dst == nullptr || src == nullptr) { set_error(error, capacity, "invalid copy arguments"); return -1; }
-    return launch_copy(enter_state(opaque), dst, src, n, error, capacity);
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return launch_copy(st, dst, src, n, error, capacity);
 }
 extern "C" int mynah_hip_scale_dev(void *opaque, float *d, size_t n, float scale, char *error, size_t capacity) {
     if (d == nullptr) { set_error(error, capacity, "invalid scale arguments"); return -1; }
-    return launch_scale(enter_state(opaque), d, n, scale, error, capacity);
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return launch_scale(st, d, n, scale, error, capacity);
 }
 extern "C" int mynah_hip_clip_dev(void *opaque, float *d, size_t n, char *error, size_t capacity) {
     if (d == nullptr) { set_error(error, capacity, "invalid clip arguments"); return -1; }
-    return launch_clip(enter_state(opaque), d, n, error, capacity);
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return launch_clip(st, d, n, error, capacity);
 }
 extern "C" int mynah_hip_argmax_dev(void *opaque, const float *dlogits, size_t vocab, size_t codebook_size, size_t eos_id,
                                     int allow_eos, unsigned *argmax, char *error, size_t capacity) {
@@ -851,7 +885,7 @@ extern "C" int mynah_hip_argmax_dev(void *opaque, const float *dlogits, size_t v
     if (launch_argmax(st, dlogits, vocab, codebook_size, eos_id >= 0x7fffffffu ? 0x7ffffffeu : eos_id, allow_eos, dres, error, capacity) != 0)
         return -1;
     MYNAH_TRY(hipMemcpyAsync(st->pinned, dres, sizeof(unsigned), hipMemcpyDeviceToHost, st->stream));
-    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    if (synchronise(st, error, capacity) != 0) return -1;
     *argmax = *static_cast<unsigned *>(st->pinned);
     return 0;
 }
@@ -861,7 +895,9 @@ extern "C" int mynah_hip_self_attention_dev(void *opaque, const float *dqkv, flo
                                             float *dout, char *error, size_t capacity) {
     const float *q[1] = {dqkv};
     float *k[1] = {dk}, *v[1] = {dv}, *o[1] = {dout};
-    return attention_table(enter_state(opaque), 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width,
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return attention_table(st, 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width,
                            scale, o, error, capacity, true);
 }
 extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, const float *dk, const float *dv, size_t valid,
@@ -869,7 +905,9 @@ extern "C" int mynah_hip_cross_attention_dev(void *opaque, const float *dq, cons
                                              char *error, size_t capacity) {
     const float *q[1] = {dq};
     float *k[1] = {const_cast<float *>(dk)}, *v[1] = {const_cast<float *>(dv)}, *o[1] = {dout};
-    return attention_table(enter_state(opaque), 0, q, k, v, nullptr, &valid, cache_stride, 1, heads, head_width,
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return attention_table(st, 0, q, k, v, nullptr, &valid, cache_stride, 1, heads, head_width,
                            scale, o, error, capacity, true);
 }
 
@@ -903,6 +941,7 @@ extern "C" int mynah_hip_set_quant(void *opaque, int qtype, int arith, char *err
 extern "C" int mynah_hip_matmul_d2d_batched(void *opaque, const float *const *din, float *const *dout, size_t batch, size_t iw,
                                             size_t ow, const float *weight, const float *bias, char *error, size_t capacity) {
     State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
     if (batch == 0) return 0;   // src/qmat.c:826
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "batch exceeds MYNAH_MAX_BATCH");
@@ -935,7 +974,9 @@ extern "C" int mynah_hip_self_attention_dev_batched(void *opaque, const float *c
         set_error(error, capacity, "attention: null buffer");
         return -1;
     }
-    return attention_table(enter_state(opaque), 1, dqkv, dk, dv, position, valid, cache_stride, batch, heads,
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return attention_table(st, 1, dqkv, dk, dv, position, valid, cache_stride, batch, heads,
                            head_width, scale, dout, error, capacity);
 }
 extern "C" int mynah_hip_cross_attention_dev_batched(void *opaque, const float *const *dq, const float *const *dk,
@@ -951,8 +992,38 @@ extern "C" int mynah_hip_cross_attention_dev_batched(void *opaque, const float *
         k[b] = const_cast<float *>(dk[b]);
         v[b] = const_cast<float *>(dv[b]);
     }
-    return attention_table(enter_state(opaque), 0, dq, k, v, nullptr, valid, cache_stride, batch, heads, head_width,
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    return attention_table(st, 0, dq, k, v, nullptr, valid, cache_stride, batch, heads, head_width,
                            scale, dout, error, capacity);
+}
+
+// Device copy of rows [0, rows) of the host position table at `table`: one growing buffer per table, filled up to the
+// highest row any call has needed.  The table's own row count is not known here, so rows are uploaded as calls reach
+// them (a decode loop asks for one more row per step) and the buffer doubles when it runs out.
+static int position_rows(State *st, const float *table, size_t rows, size_t width, const float **dev, char *error, size_t capacity) {
+    if (rows > SIZE_MAX / sizeof(float) / width) {
+        set_error(error, capacity, "position table too large");
+        return -1;
+    }
+    PositionTable &t = st->position_tables[std::make_pair(table, width)];
+    if (rows > t.capacity_rows) {
+        const size_t grown = rows > 2 * t.capacity_rows ? rows : 2 * t.capacity_rows;
+        float *bigger = nullptr;
+        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&bigger), grown * width * sizeof(float)));
+        if (t.filled_rows != 0) MYNAH_TRY(hipMemcpyAsync(bigger, t.data, t.filled_rows * width * sizeof(float), hipMemcpyDeviceToDevice, st->stream));
+        if (t.data != nullptr) st->pending_free.push_back(t.data);   // earlier launches may still read it
+        t.data = bigger;
+        t.capacity_rows = grown;
+    }
+    if (rows > t.filled_rows) {
+        if (copy_to_device(st, t.data + t.filled_rows * width, table + t.filled_rows * width, (rows - t.filled_rows) * width * sizeof(float), error,
+                           capacity) != 0)
+            return -1;
+        t.filled_rows = rows;
+    }
+    *dev = t.data;
+    return 0;
 }
 
 extern "C" int mynah_hip_embed_gather(void *opaque, const float *const *tables, const size_t *table_rows, size_t table_count,
@@ -980,9 +1051,8 @@ extern "C" int mynah_hip_embed_gather(void *opaque, const float *const *tables, 
         dtables[j] = static_cast<const float *>(cw->data);
     }
     const float *dpos = nullptr;
-    if (position != nullptr) {
-        if (cached_vector(st, position + position_offset * width, tokens * width, &dpos, error, capacity) != 0) return -1;
-    }
+    if (position != nullptr && position_rows(st, position, position_offset + tokens, width, &dpos, error, capacity) != 0) return -1;
+    if (dpos != nullptr) dpos += position_offset * width;
     const size_t id_bytes = tokens * table_count * sizeof(int32_t);
     if (ensure_scratch(st, id_bytes, error, capacity) != 0) return -1;
     if (copy_to_device(st, st->scratch, ids, id_bytes, error, capacity) != 0) return -1;

@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include <cstdio>
+#include <map>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -39,6 +40,9 @@ inline int hip_check(hipError_t r, const char *what, char *error, size_t capacit
     return -1;
 }
 #define MYNAH_TRY(expr) do { if (hip_check((expr), #expr, error, capacity) != 0) return -1; } while (0)
+struct State;
+// Stream synchronisation that also reports a failure an earlier call could not return (backend_hip.hip).
+int synchronise(State *st, char *error, size_t capacity);
 #define MYNAH_NEED_STATE(st) do { if ((st) == nullptr) { set_error(error, capacity, "backend state is null"); return -1; } } while (0)
 
 // ---- device-resident copy of one host tensor, converted at first sight ----
@@ -98,6 +102,12 @@ struct PendingOp {
     int fold_heads = 0, fold_head_width = 0, fold_max_units = 0;
 };
 
+// Device copy of the leading rows of a host position table (mynah_hip_embed_gather).
+struct PositionTable {
+    float *data = nullptr;
+    size_t capacity_rows = 0, filled_rows = 0;
+};
+
 struct State {
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -114,6 +124,8 @@ struct State {
     std::mutex mu;
     std::unordered_map<WeightKey, CachedWeight, WeightKeyHash> weights;
     size_t weight_bytes = 0;
+    std::map<std::pair<const float *, size_t>, PositionTable> position_tables;   // by (host table, width)
+    std::vector<void *> pending_free;   // from mynah_hip_dev_free, freed at the next synchronisation
     // upload scratch (src/backend.h:78-81) and pinned staging for h2d/d2h
     float *scratch = nullptr;
     size_t scratch_bytes = 0;

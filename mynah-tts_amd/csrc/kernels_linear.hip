@@ -283,6 +283,116 @@ __global__ void __launch_bounds__(256) k_sgemm(int ta, int tb, int m, int n, int
     *dst = beta == 0.0f ? alpha * sum : alpha * sum + beta * *dst;
 }
 
+// The same products for many rows, on the matrix cores: C[m][n] = alpha * sum_k A[m][k] * B(n, k) + beta * C[m][n] + bias[n],
+// A row-major with row stride lda; TB = 1: B[n][k] (both operands K-contiguous, "NT" -- the seam's matmul and its scores
+// Q K^T), TB = 0: B[k][n] ("NN" -- P V).  f32 in, f32 multiply-add (v_mfma_f32_32x32x2_f32: lane l supplies row l % 32 and
+// k l / 32 of each operand), so the result differs from a serial sum only in the order of the additions.
+// Workgroup tile 64 x 64, a wavefront 32 x 32; K in steps of 32 through LDS (rows padded to 33 floats: the 32 rows a
+// wavefront reads fall into 32 banks).  The next step's operands are requested before the current step's products and
+// stored after them.  VEC: rows are whole aligned float4s (strides and K multiples of 4, 16-byte bases); otherwise the
+// staging is scalar with the same bounds.  Rows and columns past the matrix are staged as zeros and not written.
+constexpr int kGemmTile = 64, kGemmStep = 32, kGemmPad = 33;
+
+template <int TB, int VEC>
+__global__ void __launch_bounds__(256) k_gemm_f32_mfma(const float *__restrict__ A, int lda, const float *__restrict__ B, int ldb, float *__restrict__ C,
+                                                       int ldc, int M, int N, int K, float alpha, float beta, const float *__restrict__ bias) {
+    typedef float floatx16 __attribute__((ext_vector_type(16)));
+    __shared__ float s_a[kGemmTile * kGemmPad];
+    __shared__ float s_b[kGemmTile * kGemmPad];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+    const int m0 = blockIdx.y * kGemmTile, n0 = blockIdx.x * kGemmTile;
+
+    // staging slots.  K-contiguous operand (A, and B when TB): rows r and r + 32, four k from 4 * (tid % 8).
+    // N-contiguous operand (B when !TB): k rows kr and kr + 16, four n from 4 * (tid % 16).
+    const int kr = tid >> 3, kc = (tid & 7) * 4;
+    const int nr = tid >> 4, nc = (tid & 15) * 4;
+    float4 ra[2], rb[2];
+    const auto fetch_k_major = [&](const float *base, int ld, int row, int rows, int k0) -> float4 {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row < rows) {
+            const float *p = base + (size_t)row * ld + k0;
+            if (VEC && k0 + 3 < K) v = *reinterpret_cast<const float4 *>(p);
+            else {
+                if (k0 < K) v.x = p[0];
+                if (k0 + 1 < K) v.y = p[1];
+                if (k0 + 2 < K) v.z = p[2];
+                if (k0 + 3 < K) v.w = p[3];
+            }
+        }
+        return v;
+    };
+    const auto fetch_n_major = [&](int k, int n) -> float4 {   // B[k][n .. n + 3]
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (k < K) {
+            const float *p = B + (size_t)k * ldb + n;
+            if (VEC && n + 3 < N) v = *reinterpret_cast<const float4 *>(p);
+            else {
+                if (n < N) v.x = p[0];
+                if (n + 1 < N) v.y = p[1];
+                if (n + 2 < N) v.z = p[2];
+                if (n + 3 < N) v.w = p[3];
+            }
+        }
+        return v;
+    };
+    const auto request = [&](int k0) {
+        ra[0] = fetch_k_major(A, lda, m0 + kr, M, k0 + kc);
+        ra[1] = fetch_k_major(A, lda, m0 + kr + 32, M, k0 + kc);
+        if constexpr (TB) {
+            rb[0] = fetch_k_major(B, ldb, n0 + kr, N, k0 + kc);
+            rb[1] = fetch_k_major(B, ldb, n0 + kr + 32, N, k0 + kc);
+        } else {
+            rb[0] = fetch_n_major(k0 + nr, n0 + nc);
+            rb[1] = fetch_n_major(k0 + nr + 16, n0 + nc);
+        }
+    };
+    const auto stage = [&]() {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float *pa = s_a + (kr + 32 * h) * kGemmPad + kc;
+            pa[0] = ra[h].x; pa[1] = ra[h].y; pa[2] = ra[h].z; pa[3] = ra[h].w;
+            if constexpr (TB) {
+                float *pb = s_b + (kr + 32 * h) * kGemmPad + kc;
+                pb[0] = rb[h].x; pb[1] = rb[h].y; pb[2] = rb[h].z; pb[3] = rb[h].w;
+            } else {
+                float *pb = s_b + nc * kGemmPad + nr + 16 * h;   // transposed: s_b[n][k]
+                pb[0] = rb[h].x; pb[kGemmPad] = rb[h].y; pb[2 * kGemmPad] = rb[h].z; pb[3 * kGemmPad] = rb[h].w;
+            }
+        }
+    };
+
+    floatx16 acc = {0};
+    const float *fa = s_a + (wm * 32 + (lane & 31)) * kGemmPad + (lane >> 5);
+    const float *fb = s_b + (wn * 32 + (lane & 31)) * kGemmPad + (lane >> 5);
+    request(0);
+    for (int k0 = 0; k0 < K; k0 += kGemmStep) {
+        __syncthreads();   // the products of the step before have read the tiles
+        stage();
+        __syncthreads();
+        if (k0 + kGemmStep < K) request(k0 + kGemmStep);
+#pragma unroll
+        for (int s2 = 0; s2 < kGemmStep / 2; ++s2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[2 * s2], fb[2 * s2], acc, 0, 0, 0);
+    }
+    const int n = n0 + wn * 32 + (lane & 31);
+    if (n >= N) return;
+    const float add = bias != nullptr ? bias[n] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);   // row of accumulator register r
+        if (m < M) {
+            float *dst = C + (size_t)m * ldc + n;
+            const float v = alpha * acc[r] + add;
+            *dst = beta == 0.0f ? v : v + beta * *dst;
+        }
+    }
+}
+
+static bool gemm_vec_ok(const float *a, size_t lda, const float *b, size_t ldb, size_t k, size_t inner_b) {
+    return (reinterpret_cast<uintptr_t>(a) % 16 == 0) && (reinterpret_cast<uintptr_t>(b) % 16 == 0) && lda % 4 == 0 && ldb % 4 == 0 && k % 4 == 0 &&
+           inner_b % 4 == 0;
+}
+
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
 int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity) {
     constexpr int epc = Chunk<QT>::n;
@@ -363,9 +473,22 @@ int launch_linear(State *st, const LinearArgs &a, char *error, size_t capacity) 
     }
 }
 
+// Products of fewer rows than this stay on the scalar tile kernels (a 64-row tile would be mostly padding).
+constexpr size_t kGemmMfmaMinRows = 24;
+
 int launch_gemm_f32(State *st, const float *in, float *out, size_t rows, size_t k, size_t n, const float *w,
                     const float *bias, char *error, size_t capacity) {
     if (rows == 0 || n == 0) return 0;
+    if (rows >= kGemmMfmaMinRows && k > 0) {
+        const dim3 grid((unsigned)((n + kGemmTile - 1) / kGemmTile), (unsigned)((rows + kGemmTile - 1) / kGemmTile));
+        if (gemm_vec_ok(in, k, w, k, k, k))
+            hipLaunchKernelGGL((k_gemm_f32_mfma<1, 1>), grid, dim3(256), 0, st->stream, in, (int)k, w, (int)k, out, (int)n, (int)rows, (int)n, (int)k, 1.0f,
+                               0.0f, bias);
+        else
+            hipLaunchKernelGGL((k_gemm_f32_mfma<1, 0>), grid, dim3(256), 0, st->stream, in, (int)k, w, (int)k, out, (int)n, (int)rows, (int)n, (int)k, 1.0f,
+                               0.0f, bias);
+        return hip_check(hipGetLastError(), "gemm launch", error, capacity);
+    }
     const dim3 grid((unsigned)((n + 15) / 16), (unsigned)((rows + 15) / 16));
     hipLaunchKernelGGL(k_gemm_nt_f32, grid, dim3(256), 0, st->stream, in, w, bias, out, (int)rows, (int)k, (int)n);
     return hip_check(hipGetLastError(), "gemm launch", error, capacity);
@@ -374,6 +497,19 @@ int launch_gemm_f32(State *st, const float *in, float *out, size_t rows, size_t 
 int launch_sgemm(State *st, int ta, int tb, size_t m, size_t n, size_t k, float alpha, const float *a, size_t lda,
                  const float *b, size_t ldb, float beta, float *c, size_t ldc, char *error, size_t capacity) {
     if (m == 0 || n == 0) return 0;
+    if (!ta && m >= kGemmMfmaMinRows && k > 0) {   // op(A) = A: the forms the engine's attention makes (Q K^T, P V) and its row products
+        const dim3 grid((unsigned)((n + kGemmTile - 1) / kGemmTile), (unsigned)((m + kGemmTile - 1) / kGemmTile));
+        const bool vec = gemm_vec_ok(a, lda, b, ldb, tb ? k : 0, tb ? k : n);
+        if (tb && vec)
+            hipLaunchKernelGGL((k_gemm_f32_mfma<1, 1>), grid, dim3(256), 0, st->stream, a, (int)lda, b, (int)ldb, c, (int)ldc, (int)m, (int)n, (int)k, alpha, beta, nullptr);
+        else if (tb)
+            hipLaunchKernelGGL((k_gemm_f32_mfma<1, 0>), grid, dim3(256), 0, st->stream, a, (int)lda, b, (int)ldb, c, (int)ldc, (int)m, (int)n, (int)k, alpha, beta, nullptr);
+        else if (vec && k % 4 == 0)
+            hipLaunchKernelGGL((k_gemm_f32_mfma<0, 1>), grid, dim3(256), 0, st->stream, a, (int)lda, b, (int)ldb, c, (int)ldc, (int)m, (int)n, (int)k, alpha, beta, nullptr);
+        else
+            hipLaunchKernelGGL((k_gemm_f32_mfma<0, 0>), grid, dim3(256), 0, st->stream, a, (int)lda, b, (int)ldb, c, (int)ldc, (int)m, (int)n, (int)k, alpha, beta, nullptr);
+        return hip_check(hipGetLastError(), "sgemm launch", error, capacity);
+    }
     const dim3 grid((unsigned)((n + 15) / 16), (unsigned)((m + 15) / 16));
     hipLaunchKernelGGL(k_sgemm, grid, dim3(256), 0, st->stream, ta, tb, (int)m, (int)n, (int)k, alpha, a, (int)lda, b,
                        (int)ldb, beta, c, (int)ldc);

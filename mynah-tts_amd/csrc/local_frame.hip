@@ -558,7 +558,7 @@ extern "C" int mynah_hip_local_frame(void *state, mynah_hip_local *l, mynah_hip_
     }
     MYNAH_TRY(hipMemcpyAsync(l->values_host, l->values, 2 * (size_t)kMaxBatch * l->streams * sizeof(unsigned), hipMemcpyDeviceToHost, st->stream));
     MYNAH_TRY(hipMemcpyAsync(l->frame_host, l->frame, sizeof(LocalFrameDev), hipMemcpyDeviceToHost, st->stream));
-    MYNAH_TRY(hipStreamSynchronize(st->stream));
+    if (synchronise(st, error, capacity) != 0) return -1;
     for (size_t b = 0; b < batch; ++b) {
         for (size_t s = 0; s < l->streams; ++s) {
             values[b * l->streams + s] = l->values_host[b * l->streams + s];

@@ -102,3 +102,28 @@ def test_reference_backend_struct_binds_every_seam_symbol(orc, ref_strict, pkg, 
         assert "HIP" in str(e) or "device" in str(e), str(e)
     finally:
         dec.close()
+
+
+def test_entry_points_refuse_a_null_state(pkg):
+    """Every resident entry point that only forwards to a launch returns -1 with a message for a NULL state, before it
+    touches a device (no GPU is needed to see that)."""
+    import ctypes as C
+    lib = pkg.load_library()
+    err = C.create_string_buffer(256)
+    fake = C.c_void_p(0x1000)          # never dereferenced: the state is looked at first
+    one = C.c_size_t(1)
+    calls = {
+        "mynah_hip_sgemm_dev": (None, 0, 0, one, one, one, C.c_float(1.0), fake, one, fake, one, C.c_float(0.0), fake, one),
+        "mynah_hip_softmax_dev": (None, fake, one, one, one),
+        "mynah_hip_copy_dev": (None, fake, fake, one),
+        "mynah_hip_scale_dev": (None, fake, one, C.c_float(1.0)),
+        "mynah_hip_clip_dev": (None, fake, one),
+        "mynah_hip_self_attention_dev": (None, fake, fake, fake, C.c_size_t(0), one, one, one, C.c_size_t(64), C.c_float(1.0), fake),
+        "mynah_hip_cross_attention_dev": (None, fake, fake, fake, one, one, one, C.c_size_t(64), C.c_float(1.0), fake),
+        "mynah_hip_sync": (None,),
+    }
+    for name, args in calls.items():
+        err.value = b""
+        rc = getattr(lib, name)(*args, err, C.c_size_t(len(err)))
+        assert rc == -1, name
+        assert b"state is null" in err.value, (name, err.value)

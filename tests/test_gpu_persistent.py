@@ -172,5 +172,15 @@ def test_persistent_bounded_wait_reports_instead_of_hanging(pkg, synth):
         again = h.step()
         assert np.isfinite(first[0]).all() and _same_bits(first[0], again[0])
         h.close()
+        # the same bound holds the fold workgroups of the many-stream attention launches: eight long streams make more
+        # workgroups than the device holds at once, so the folds start while cache chunks are still being read, find
+        # records missing, and give up at their first look
+        cfg = synth.decoder_config(layers=1, capacity=2048)
+        weights = synth.decoder_weights(cfg, seed=0)
+        streams = synth.decoder_streams(cfg, [2000, 1990, 1980, 1970, 1960, 1950, 1940, 1930], [16] * 8, seed=2)
+        h = Harness(pkg, b2, cfg, weights, streams)
+        with pytest.raises(pkg.BackendError, match="bounded wait"):
+            h.step()
+        h.close()
     finally:
         b2.close()

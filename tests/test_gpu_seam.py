@@ -176,6 +176,38 @@ def test_matmul_rows_and_generic_shapes(backend, pkg, orc, nerr):
     backend.set_quant(pkg.F32)
 
 
+def test_many_row_products_on_the_matrix_cores(backend, nerr):
+    """Products of 24 rows and more take the f32 MFMA tile kernel: matmul (NT, bias) and sgemm with op(A) = A (NT and NN,
+    padded leading dimensions, alpha / beta), at tile-aligned and ragged shapes, against float64.  1e-5 normalised."""
+    _announce("many-row f32 products (MFMA)")
+    rng = np.random.default_rng(510)
+    for rows, k, n in ((24, 768, 2304), (64, 768, 768), (100, 3072, 768), (300, 70, 50), (33, 33, 65), (257, 129, 190), (512, 768, 3072)):
+        w = backend.keep((rng.standard_normal((n, k)) * 0.05).astype(np.float32))
+        bias = backend.keep(rng.standard_normal(n).astype(np.float32))
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        want = x.astype(np.float64) @ w.astype(np.float64).T + bias
+        din, dout = backend.alloc(rows * k).write(x), backend.alloc(rows * n)
+        backend.matmul_d2d(din.ptr, dout.ptr, rows, k, n, w, bias)
+        assert nerr(dout.read().reshape(rows, n), want) < 1e-5, (rows, k, n)
+        backend.matmul_d2d(din.ptr, dout.ptr, rows, k, n, w, None)
+        assert nerr(dout.read().reshape(rows, n), want - bias) < 1e-5, (rows, k, n)
+        din.free()
+        dout.free()
+    for tb in (1, 0):
+        for m, n, k, pad in ((64, 64, 64, 0), (128, 200, 64, 0), (37, 130, 64, 3), (200, 64, 257, 4), (25, 31, 7, 1), (256, 256, 768, 8)):
+            lda, ldb, ldc = k + pad, (k if tb else n) + pad, n + pad
+            a = rng.standard_normal((m, lda)).astype(np.float32)
+            b = rng.standard_normal(((n if tb else k), ldb)).astype(np.float32)
+            c0 = rng.standard_normal((m, ldc)).astype(np.float32)
+            a64, b64 = a[:, :k].astype(np.float64), (b[:, :k].T if tb else b[:, :n]).astype(np.float64)
+            for alpha, beta in ((1.0, 0.0), (0.125, 0.5)):
+                c = c0.copy()
+                backend.sgemm(0, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc)
+                want = alpha * (a64 @ b64) + beta * c0[:, :n]
+                assert nerr(c[:, :n], want) < 1e-5, (tb, m, n, k, pad, alpha, beta)
+                assert np.array_equal(c[:, n:], c0[:, n:]), "columns beyond n were written"
+
+
 def test_layernorm_gelu_residual_softmax(backend, orc, nerr):
     _announce("layernorm/gelu/residual/softmax")
     rng = np.random.default_rng(600)
@@ -369,6 +401,41 @@ def test_embedding_gather_bit_exact(backend):
     with pytest.raises(Exception):
         backend.embed_gather([table], np.array([4096], np.int32), 768, 1.0, None, 0, dout.ptr)   # out of vocabulary
     dout.free()
+
+
+def test_embedding_gather_decode_loop_positions(backend):
+    """One token per call at a growing position (a decode loop), then a prefill range over rows already seen and beyond:
+    every call adds the right position rows, from one device copy of the table that grows as rows are reached."""
+    _announce("gather: positions of a decode loop")
+    rng = np.random.default_rng(1001)
+    table = backend.keep((rng.standard_normal((300, 768)) * 0.02).astype(np.float32))
+    pos = backend.keep((rng.standard_normal((400, 768)) * 0.02).astype(np.float32))
+    dout = backend.alloc(64 * 768)
+    for step in range(130):
+        ids = np.array([step % 300], np.int32)
+        backend.embed_gather([table], ids, 768, 1.0, pos, step, dout.ptr)
+        assert np.array_equal(dout.read(768), table[ids[0]] + pos[step]), "step %d" % step
+    ids = rng.integers(0, 300, 64).astype(np.int32)
+    for offset in (0, 100, 336):
+        backend.embed_gather([table], ids, 768, 1.0, pos, offset, dout.ptr)
+        assert np.array_equal(dout.read().reshape(64, 768), table[ids] + pos[offset:offset + 64]), "offset %d" % offset
+    dout.free()
+
+
+def test_freed_buffers_outlive_the_work_that_reads_them(backend):
+    """mynah_hip_dev_free does not wait for the stream: a buffer freed right after a launch that reads it is still read
+    correctly, and hundreds of allocate-use-free rounds neither stall nor run out of memory."""
+    _announce("deferred frees")
+    rng = np.random.default_rng(1002)
+    n = 1 << 22
+    want = rng.standard_normal(n).astype(np.float32)
+    keep = backend.alloc(n)
+    for _ in range(200):
+        src = backend.alloc(n).write(want)
+        backend.copy_dev(keep.ptr, src.ptr, n)
+        src.free()
+    assert np.array_equal(keep.read(), want)
+    keep.free()
 
 
 @pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4", "f16"])
