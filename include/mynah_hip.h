@@ -217,6 +217,15 @@ int mynah_hip_cross_attention_dev_batched(void *state, const float *const *dev_q
                                           size_t batch, size_t heads, size_t head_width, float scale,
                                           float *const *dev_out, char *error, size_t error_capacity);
 
+/* Cross-attention K/V of an utterance for every decoder layer, from encoder memory that is resident on the device
+ * (decoder_cache_init, src/graph.c:3002-3028): per layer LayerNorm(memory; norm_xattn_memory) -> kv_net product -> K half
+ * and V half, written to dev_cross_k / dev_cross_v as [layers, memory_length, xattn_width] (the layout the decoder slots
+ * take).  norm_gain / norm_bias / kv_w are [layers] arrays of HOST pointers (kv_w[l]: [2 * xattn_width, width], K rows
+ * first; norm_bias may be NULL).  Asynchronous on the backend stream. */
+int mynah_hip_cross_kv_dev(void *state, const float *dev_memory, size_t memory_length, size_t width, size_t layers,
+                           const float *const *norm_gain, const float *const *norm_bias, const float *const *kv_w,
+                           size_t xattn_width, float *dev_cross_k, float *dev_cross_v, char *error, size_t error_capacity);
+
 /* Embedding gather (src/graph.c:729-737 text rows, :764-804 audio frame): out[t,:] = sum over `tables`
  * of table_j[ids[t*tables + j], :] scaled by `scale` (1 for text, 1/16 for the stacked audio frame),
  * optionally + position[t0 + t, :] (src/graph.c:649-651, :3156-3157).  f32 tables are HOST pointers

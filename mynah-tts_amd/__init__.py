@@ -118,6 +118,7 @@ def load_library(path=LIB_PATH):
                                                          _vp, *_err]
     lib.mynah_hip_cross_attention_dev_batched.argtypes = [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp,
                                                           *_err]
+    lib.mynah_hip_cross_kv_dev.argtypes = [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz, _vp, _vp, *_err]
     lib.mynah_hip_embed_gather.argtypes = [_vp, _vp, _vp, _sz, _vp, _sz, _sz, C.c_float, _vp, _sz, _vp, *_err]
     lib.mynah_hip_decoder_create.argtypes = [_vp, C.POINTER(DecoderDesc), C.POINTER(_vp), *_err]
     lib.mynah_hip_decoder_destroy.argtypes = [_vp, _vp]
@@ -293,6 +294,14 @@ class Backend:
 
     def softmax_dev(self, d, rows, cols, valid):
         self._call("mynah_hip_softmax_dev", _vp(d), _sz(rows), _sz(cols), _sz(valid))
+
+    def cross_kv_dev(self, dmemory, memory_length, width, norm_gains, norm_biases, kv_ws, xattn_width, dck, dcv):
+        """norm_gains / kv_ws: per-layer lists of kept host arrays (norm_biases may be None)."""
+        layers = len(kv_ws)
+        g, w = _ptr_array(norm_gains), _ptr_array(kv_ws)
+        b = _ptr_array(norm_biases) if norm_biases is not None else None
+        self._call("mynah_hip_cross_kv_dev", _vp(dmemory), _sz(memory_length), _sz(width), _sz(layers), C.cast(g, _vp),
+                   C.cast(b, _vp) if b is not None else None, C.cast(w, _vp), _sz(xattn_width), _vp(dck), _vp(dcv))
 
     def copy_dev(self, dst, src, n):
         self._call("mynah_hip_copy_dev", _vp(dst), _vp(src), _sz(n))

@@ -925,6 +925,44 @@ extern "C" int mynah_hip_self_attention_dev_noalloc(void *opaque, const float *d
     return attention_table(st, 1, q, k, v, &position, &valid, cache_stride, 1, heads, head_width, scale, o, error, capacity, false, &fixed);
 }
 
+// The cross-attention keys and values of an utterance, all layers, from the encoder memory that is already on the device
+// (decoder_cache_init, src/graph.c:3002-3028): per layer LayerNorm(memory) -> kv product [T, 2 * xw] -> K and V halves.
+// Here the two halves are two products, each writing its half straight into the cache (the rows of kv_net are independent,
+// so each half's weights -- and, for quantised storage, their scales -- are what they are in the whole matrix).  Products of
+// up to 16 rows take the current quantisation like every seam product, more rows are f32 (src/qmat.c row limit).
+// Everything is enqueued on the backend's stream; nothing is copied to the host.
+extern "C" int mynah_hip_cross_kv_dev(void *opaque, const float *dev_memory, size_t memory_length, size_t width, size_t layers,
+                                      const float *const *norm_gain, const float *const *norm_bias, const float *const *kv_w, size_t xattn_width,
+                                      float *dev_cross_k, float *dev_cross_v, char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    if (dev_memory == nullptr || norm_gain == nullptr || kv_w == nullptr || dev_cross_k == nullptr || dev_cross_v == nullptr || width == 0 ||
+        width > 0x7fffffffu || xattn_width == 0 || xattn_width > 0x7fffffffu || memory_length > 0x7fffffffu || layers > 4096) {
+        set_error(error, capacity, "invalid cross K/V arguments");
+        return -1;
+    }
+    if (memory_length == 0 || layers == 0) return 0;
+    float *normed = nullptr;
+    MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&normed), memory_length * width * sizeof(float)));
+    st->pending_free.push_back(normed);   // freed at a later synchronisation, when the launches below are done with it
+    const size_t per_layer = memory_length * xattn_width;
+    for (size_t l = 0; l < layers; ++l) {
+        if (norm_gain[l] == nullptr || kv_w[l] == nullptr) {
+            set_error(error, capacity, "cross K/V: missing layer weight");
+            return -1;
+        }
+        const float *dgain = nullptr, *dbias = nullptr;
+        if (cached_vector(st, norm_gain[l], width, &dgain, error, capacity) != 0) return -1;
+        if (norm_bias != nullptr && cached_vector(st, norm_bias[l], width, &dbias, error, capacity) != 0) return -1;
+        if (launch_layernorm(st, dev_memory, normed, dgain, dbias, memory_length, width, error, capacity) != 0) return -1;
+        if (matmul_device(st, normed, dev_cross_k + l * per_layer, memory_length, width, xattn_width, kv_w[l], nullptr, error, capacity) != 0) return -1;
+        if (matmul_device(st, normed, dev_cross_v + l * per_layer, memory_length, width, xattn_width, kv_w[l] + xattn_width * width, nullptr, error,
+                          capacity) != 0)
+            return -1;
+    }
+    return 0;
+}
+
 // =========================================================================================== section 2
 extern "C" int mynah_hip_set_quant(void *opaque, int qtype, int arith, char *error, size_t capacity) {
     State *st = enter_state(opaque);

@@ -208,6 +208,43 @@ def test_many_row_products_on_the_matrix_cores(backend, nerr):
                 assert np.array_equal(c[:, n:], c0[:, n:]), "columns beyond n were written"
 
 
+@pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4"])
+def test_cross_kv_from_resident_memory(backend, pkg, orc, nerr, qtype_name):
+    """decoder_cache_init's cross K/V (src/graph.c:3002-3028) from encoder memory on the device: per layer LayerNorm ->
+    kv product -> K | V halves, for memories of 1, 9 (<= 16 rows: the current quantisation, checked against the oracle's
+    quantised product of the whole kv matrix), 40 and 300 rows (f32, against float64)."""
+    _announce("cross K/V precompute, %s" % qtype_name)
+    qt = {"f32": pkg.F32, "int8": pkg.INT8, "int4": pkg.INT4}[qtype_name]
+    rng = np.random.default_rng(520)
+    layers, width, xw = 3, 768, 768
+    gains = [backend.keep((1.0 + 0.1 * rng.standard_normal(width)).astype(np.float32)) for _ in range(layers)]
+    biases = [backend.keep((0.02 * rng.standard_normal(width)).astype(np.float32)) for _ in range(layers)]
+    kvw = [backend.keep((0.02 * rng.standard_normal((2 * xw, width))).astype(np.float32)) for _ in range(layers)]
+    backend.set_quant(qt)
+    try:
+        for T, with_bias in ((1, False), (9, True), (40, False), (300, True)):
+            memory = rng.standard_normal((T, width)).astype(np.float32)
+            dmem = backend.alloc(T * width).write(memory)
+            dck, dcv = backend.alloc(layers * T * xw), backend.alloc(layers * T * xw)
+            backend.cross_kv_dev(dmem.ptr, T, width, gains, biases if with_bias else None, kvw, xw, dck.ptr, dcv.ptr)
+            gk, gv = dck.read().reshape(layers, T, xw), dcv.read().reshape(layers, T, xw)
+            for l in range(layers):
+                normed = np.stack([orc.layernorm(r, gains[l], biases[l] if with_bias else None) for r in memory])
+                if T <= 16 and qt != pkg.F32:
+                    pw = orc.PackedWeight(kvw[l], {pkg.INT8: orc.INT8, pkg.INT4: orc.INT4}[qt])
+                    want = np.stack([orc.linear(pw, r) for r in normed])
+                    tol = 1e-5
+                else:
+                    want = normed.astype(np.float64) @ kvw[l].astype(np.float64).T
+                    tol = 1e-5
+                assert nerr(gk[l], want[:, :xw]) < tol, (T, l, "k")
+                assert nerr(gv[l], want[:, xw:]) < tol, (T, l, "v")
+            for d in (dmem, dck, dcv):
+                d.free()
+    finally:
+        backend.set_quant(pkg.F32)
+
+
 def test_layernorm_gelu_residual_softmax(backend, orc, nerr):
     _announce("layernorm/gelu/residual/softmax")
     rng = np.random.default_rng(600)
