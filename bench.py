@@ -73,6 +73,9 @@ def timed_steps(backend, sets, cfg, head_rows, vocab, steps, warmup, with_head=T
     return backend.timer_end() * 1000.0 / steps
 
 
+GRAPH_MODE = 1   # 0 with --launches: every stage kernel a launch of its own (runs under a profiler)
+
+
 def time_config(pkg, synth, backend, qtype, lengths, mems, capacity, steps, warmup, rotate=ROTATE, stages=True):
     """Times the step of one configuration as the library runs it by default (a captured graph of stage kernels) with the
     output head -- the figure `value` is made from --, the decoder stack's part of it alone, each stage kernel of the
@@ -85,13 +88,14 @@ def time_config(pkg, synth, backend, qtype, lengths, mems, capacity, steps, warm
     setup_s = time.time() - t0
     warm = max(warmup, 2 * rotate)      # every set runs eagerly once and captures its graph before anything is timed
     batch = len(streams)
-    backend.set_graph_mode(1)
+    backend.set_graph_mode(GRAPH_MODE)
+    stages = stages and GRAPH_MODE == 1
     step_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm)
     probs = sets[0]["probs"][0].read()
     assert np.all(np.isfinite(probs)) and abs(float(probs[:vocab].sum()) - 1.0) < 1e-3, "benchmark output is not a distribution"
     stack_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm, with_head=False)
     persistent_us = persistent_stack_us = None
-    if batch <= 2 and qtype in (pkg.INT8, pkg.INT4):      # the same step as one persistent launch (opt-in form)
+    if GRAPH_MODE == 1 and batch <= 2 and qtype in (pkg.INT8, pkg.INT4):      # the same step as one persistent launch (opt-in form)
         backend.set_graph_mode(2)
         persistent_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm)
         persistent_stack_us = timed_steps(backend, sets, cfg, head_rows, vocab, steps, warm, with_head=False)
@@ -252,17 +256,21 @@ def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
     return {"frames": frames, "samples": int(L), "ms": ms, "flops": flops, "tflops": flops / (ms * 1e-3) / 1e12}
 
 
-STAGES = [("self-attention", "k_step_attention<self>", "LayerNorm + int8 act-quant + per-head Q/K/V rows + KV append + attention over the self cache"),
-          ("self-out", "k_linear<k=768, residual>", "fold of attention partials + act-quant + O matvec + residual"),
-          ("cross-attention", "k_step_attention<cross>", "LayerNorm + act-quant + per-head Q rows + attention over the cross cache"),
-          ("cross-out", "k_linear<k=768, residual>", "fold + act-quant + O matvec + residual"),
+# (with one or two streams the attention partials are folded by the output projection that follows; with more, by
+# workgroups of the attention launch itself, and the stage timing of those launches includes, per twelve launches, the two
+# small launches that give the step its counter)
+STAGES = [("self-attention", "k_step_attention<self>", "LayerNorm + int8 act-quant + per-head Q/K/V rows + KV append + attention over the self cache (+ fold of the partials when more than two streams)"),
+          ("self-out", "k_linear<k=768, residual>", "(fold of attention partials, up to two streams) + act-quant + O matvec + residual"),
+          ("cross-attention", "k_step_attention<cross>", "LayerNorm + act-quant + per-head Q rows + attention over the cross cache (+ fold when more than two streams)"),
+          ("cross-out", "k_linear<k=768, residual>", "(fold, up to two streams) + act-quant + O matvec + residual"),
           ("ffn-up", "k_linear<k=768, LayerNorm, GELU>", "LayerNorm + act-quant + up matvec + GELU"),
           ("ffn-down", "k_linear<k=3072, residual>", "act-quant + down matvec + residual")]
 
 # HBM bytes per launch of the dominant kernel of the batch-1 int8 line, from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE), each scaled by what the same counter reads for the library's plain 256 MiB read+write kernel.  The figure
 # belongs to the kernel sources it was measured on: it is reported only while their hash is the one recorded here.
-MEASURED_TRAFFIC = {"kernel": None, "bytes": None, "profile": None, "csrc_sha256": None}
+MEASURED_TRAFFIC = {"kernel": "k_linear<k=768, residual>", "bytes": 943567, "profile": "profiles/decode_step_int8_hbm_counters.md",
+                    "csrc_sha256": "8ead30e33a2025ea"}
 
 
 def csrc_hash():
@@ -297,7 +305,8 @@ def roofline(r):
     share = g["us"] * r["layers"] / r["step_us"]
     gbps = nbytes / (launch_us * 1e-6) / 1e9
     traffic = None
-    if r.get("traffic_valid") and MEASURED_TRAFFIC["bytes"] is not None and MEASURED_TRAFFIC["csrc_sha256"] == csrc_hash():
+    if (r.get("traffic_valid") and MEASURED_TRAFFIC["bytes"] is not None and MEASURED_TRAFFIC["kernel"] == kernel and
+            MEASURED_TRAFFIC["csrc_sha256"] == csrc_hash()):
         traffic = MEASURED_TRAFFIC["bytes"]
     return {"bound": "hbm", "kernel": kernel, "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / PEAK_GBPS, 4),
             "traffic": traffic, "traffic_source": MEASURED_TRAFFIC["profile"] if traffic is not None else None,
@@ -341,6 +350,9 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the library's plain read+write kernel over 256 MiB three times (a known-size reference for "
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--launches", action="store_true",
+                    help="run every kernel as a launch of its own instead of captured graphs, skip the per-stage and persistent timings "
+                         "and print a reduced line: for runs under rocprofv3, whose interception of graph launches has crashed here")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: the decode step has no multi-GPU form (streams shard by request, with no "
@@ -351,6 +363,10 @@ def main():
     import mynah_tts_amd.synth as synth
     qtype = {"f32": pkg.F32, "int8": pkg.INT8, "int4": pkg.INT4, "f16": pkg.F16}[args.quant]
     backend = pkg.Backend(quant=qtype)
+    if args.launches:
+        global GRAPH_MODE
+        GRAPH_MODE = 0
+        backend.set_graph_mode(0)
     if args.calibrate:
         for _ in range(3):
             backend.flush_cache(256 << 20)
@@ -372,6 +388,20 @@ def main():
     local = None if args.skip_local else [time_local(pkg, synth, backend, qtype, b) for b in (1, 8)]
     codec = None if args.skip_codec else time_codec(pkg, backend)
     backend.close()
+    if args.launches:
+        line = {"mode": "every kernel a launch of its own (profiling run: not the benchmark figure)", "b1_step_us": round(b1["step_us"], 2)}
+        if b8 is not None:
+            line["b8_step_us"] = round(b8["step_us"], 2)
+        if int4 is not None:
+            line["int4_b1_step_us"] = round(int4["step_us"], 2)
+        if prefill is not None:
+            line["prefill_us"] = round(prefill["us"], 2)
+        if local is not None:
+            line["local_frame_us"] = [round(f["frame_us"], 1) for f in local]
+        if codec is not None:
+            line["codec_ms"] = round(codec["ms"], 3)
+        print(json.dumps(line))
+        return
 
     result = {
         "metric": METRIC,

@@ -654,7 +654,7 @@ extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *
         }
     }
     // a fresh step counter, as every real step has one: the workgroups that wait for tagged values then really wait
-    if (batch > (size_t)kConsumerFoldMaxBatch) {
+    if (batch > (size_t)kConsumerFoldMaxBatch && (stage == MYNAH_HIP_STAGE_SELF_ATTENTION || stage == MYNAH_HIP_STAGE_CROSS_ATTENTION)) {
         if (decoder_next_epochs(st, d, 1, &d->last_slots.epoch, error, capacity) != 0) return -1;
         if (launch_step_begin(st, d->last_slots, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
         if (launch_step_items(st, d->dev_slots, 0, (int)batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items,
