@@ -524,3 +524,31 @@ def test_many_stream_forms_agree(pkg, backend, synth, qtype_name):
                 assert np.array_equal(rows[b][0], ref_rows[b][0]) and np.array_equal(rows[b][1], ref_rows[b][1]), "%s: appended rows differ" % name
     finally:
         backend.set_quant(0)
+
+
+def test_long_cache_takes_the_fold_kernel(pkg, backend, orc, synth, nerr):
+    """A capacity whose per-(stream, head) partial records exceed the LDS a launch may use without asking (more than
+    about 19,000 rows): the many-stream step then folds in a kernel of its own.  Three streams, one of them 20,000 rows
+    long, against the oracle and against each stream alone."""
+    _announce("long cache: fold kernel form")
+    lengths, mems = [20000, 5, 700], [33, 0, 129]
+    cfg = synth.decoder_config(layers=1, capacity=20480)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=8)
+    backend.set_quant(1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    try:
+        outs = h.step()
+        want, _, _ = _oracle_step(orc, cfg, weights, streams, QT["int8"])
+        quantised_errors_ok([nerr(outs[b], want[b]) for b in range(3)], 1, "long cache int8")
+        for b in range(3):
+            h.reset_cache(b)
+        again = h.step()
+        for b in range(3):
+            assert np.array_equal(again[b].view(np.uint32), outs[b].view(np.uint32))
+            h.reset_cache(b)
+            solo = h.step([b])[0]
+            assert np.array_equal(solo.view(np.uint32), outs[b].view(np.uint32)), "stream %d differs from its solo run" % b
+    finally:
+        h.close()
+        backend.set_quant(0)
