@@ -288,6 +288,18 @@ void mynah_hip_decoder_destroy(void *state, mynah_hip_decoder *decoder);
 int mynah_hip_decoder_step(void *state, mynah_hip_decoder *decoder, const mynah_hip_decoder_slot *slots,
                            size_t batch, char *error, size_t error_capacity);
 
+/* The decoder head's token choice when no local transformer follows (slot_advance, src/graph.c:3873-3905; the rule of
+ * mynah_matvec_argmax_f32, src/kernels.c:116-139, whose threaded form is src/qmat.c:500-536): for each of `batch` slots and each of
+ * `streams` stacked streams the first maximum of final_proj's logits W[streams * vocab, width] hidden + bias among the codes
+ * (candidate < codebook_size) and, unless forbid_eos[slot], eos_id; strict > from -FLT_MAX, 0 when nothing beats it.  HOST
+ * outputs as mynah_hip_local_frame's: values / stored [batch * streams] (stored = the value if it is a code, else 0), saw_eos
+ * [batch], eos_frame [batch] (stream / codebook_count of the earliest EOS, SIZE_MAX = none).  f32 arithmetic on the stored
+ * weights (HOST pointers, cached on the device); the logits never leave the device.  One synchronisation for all slots. */
+int mynah_hip_head_argmax(void *state, const float *const *dev_hidden, size_t batch, size_t width, const float *weight,
+                          const float *bias, size_t streams, size_t vocab, size_t codebook_size, size_t eos_id,
+                          size_t codebook_count, const int *forbid_eos, unsigned *values, unsigned *stored, int *saw_eos,
+                          size_t *eos_frame, char *error, size_t error_capacity);
+
 /* Output head for the step's final-normed rows: logits[b] = W[rows,width] hidden[b] + bias, then a
  * softmax over each consecutive group of `vocab` logits (mynah_softmax_f32, src/kernels.c:391-420).
  * dev_probs[b] may be NULL (logits only).  W/bias HOST pointers. */

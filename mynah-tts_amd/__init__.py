@@ -118,6 +118,7 @@ def load_library(path=LIB_PATH):
                                                          _vp, *_err]
     lib.mynah_hip_cross_attention_dev_batched.argtypes = [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.c_float, _vp,
                                                           *_err]
+    lib.mynah_hip_head_argmax.argtypes = [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, *_err]
     lib.mynah_hip_cross_kv_dev.argtypes = [_vp, _vp, _sz, _sz, _sz, _vp, _vp, _vp, _sz, _vp, _vp, *_err]
     lib.mynah_hip_embed_gather.argtypes = [_vp, _vp, _vp, _sz, _vp, _sz, _sz, C.c_float, _vp, _sz, _vp, *_err]
     lib.mynah_hip_decoder_create.argtypes = [_vp, C.POINTER(DecoderDesc), C.POINTER(_vp), *_err]
@@ -294,6 +295,18 @@ class Backend:
 
     def softmax_dev(self, d, rows, cols, valid):
         self._call("mynah_hip_softmax_dev", _vp(d), _sz(rows), _sz(cols), _sz(valid))
+
+    def head_argmax(self, dev_hidden, width, weight, bias, streams, vocab, codebook_size, eos_id, codebook_count, forbid_eos):
+        """Returns (values, stored) [batch, streams], saw_eos [batch], eos_frame [batch] (None where no EOS)."""
+        B = len(dev_hidden)
+        values, stored = np.zeros((B, streams), np.uint32), np.zeros((B, streams), np.uint32)
+        saw = np.zeros(B, np.int32)
+        frame = np.zeros(B, np.uint64)
+        forbid = np.ascontiguousarray(forbid_eos, np.int32)
+        self._call("mynah_hip_head_argmax", (_vp * B)(*dev_hidden), _sz(B), _sz(width), _np_ptr(weight), _np_ptr(bias), _sz(streams), _sz(vocab),
+                   _sz(codebook_size), _sz(eos_id), _sz(codebook_count), _np_ptr(forbid), _np_ptr(values), _np_ptr(stored), _np_ptr(saw),
+                   _np_ptr(frame))
+        return values, stored, saw, [None if f == np.iinfo(np.uint64).max else int(f) for f in frame]
 
     def cross_kv_dev(self, dmemory, memory_length, width, norm_gains, norm_biases, kv_ws, xattn_width, dck, dcv):
         """norm_gains / kv_ws: per-layer lists of kept host arrays (norm_biases may be None)."""

@@ -352,6 +352,8 @@ static void hip_close(void *opaque) {
     if (st->attn_counters != nullptr) (void)hipFree(st->attn_counters);
     if (st->seam_slots != nullptr) (void)hipFree(st->seam_slots);
     if (st->argmax_result != nullptr) (void)hipFree(st->argmax_result);
+    if (st->head_logits != nullptr) (void)hipFree(st->head_logits);
+    if (st->head_result != nullptr) (void)hipFree(st->head_result);
     if (st->ptr_table != nullptr) (void)hipFree(st->ptr_table);
     if (st->ptr_table_host != nullptr) (void)hipHostFree(st->ptr_table_host);
     if (st->persist_abort_host != nullptr) (void)hipHostFree(st->persist_abort_host);
@@ -1114,6 +1116,90 @@ extern "C" int mynah_hip_output_head(void *opaque, const float *const *dhidden, 
             if (dprobs[b] != nullptr &&
                 launch_softmax_heads(st, dlogits[b], dprobs[b], rows / vocab, vocab, error, capacity) != 0)
                 return -1;
+    return 0;
+}
+
+// The decoder head when no local transformer follows (slot_advance, src/graph.c:3873-3905): for every slot and every stacked
+// stream the constrained first maximum of final_proj's logits (mynah_matvec_argmax_f32's rule, src/kernels.c:116-139), the
+// stored code and the EOS bookkeeping.  The reference computes one stream of one slot at a time on the host; here all
+// slots and streams are two launches -- the f32 projection of every slot's row (weights read once for the batch; the
+// logits stay in a device buffer of the library and never travel) and one workgroup per slot that chooses -- and one
+// synchronisation.  f32 weights whatever the quantisation setting, like the reference's own loop.
+extern "C" int mynah_hip_head_argmax(void *opaque, const float *const *dev_hidden, size_t batch, size_t width, const float *weight,
+                                     const float *bias, size_t streams, size_t vocab, size_t codebook_size, size_t eos_id,
+                                     size_t codebook_count, const int *forbid_eos, unsigned *values, unsigned *stored, int *saw_eos,
+                                     size_t *eos_frame, char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    if (batch == 0) return 0;
+    if (batch > (size_t)kMaxBatch) {
+        set_error(error, capacity, "head argmax batch exceeds MYNAH_MAX_BATCH");
+        return -1;
+    }
+    if (dev_hidden == nullptr || weight == nullptr || forbid_eos == nullptr || values == nullptr || stored == nullptr || saw_eos == nullptr ||
+        eos_frame == nullptr || streams == 0 || vocab == 0 || vocab > 0x7fffffffu || streams > 0xffffu || codebook_count == 0 ||
+        codebook_size > vocab || streams * vocab > 0x7fffffffu || width == 0 || width > 0x7fffffffu) {
+        set_error(error, capacity, "invalid head argmax arguments");
+        return -1;
+    }
+    const size_t rows = streams * vocab;
+    if (st->head_logits_floats < (size_t)kMaxBatch * rows) {
+        if (st->head_logits != nullptr) st->pending_free.push_back(st->head_logits);
+        st->head_logits = nullptr;
+        st->head_logits_floats = 0;
+        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->head_logits), (size_t)kMaxBatch * rows * sizeof(float)));
+        st->head_logits_floats = (size_t)kMaxBatch * rows;
+    }
+    const size_t n = batch * streams;
+    const size_t result_bytes = 2 * n * sizeof(unsigned) + batch * sizeof(int) + 8 + batch * sizeof(unsigned long long);
+    if (st->head_result_bytes < result_bytes) {
+        if (st->head_result != nullptr) st->pending_free.push_back(st->head_result);
+        st->head_result = nullptr;
+        st->head_result_bytes = 0;
+        const size_t cap = (size_t)kMaxBatch * (2 * streams * sizeof(unsigned) + sizeof(int) + sizeof(unsigned long long)) + 64;
+        MYNAH_TRY(hipMalloc(&st->head_result, cap));
+        st->head_result_bytes = cap;
+    }
+    if (ensure_pinned(st, st->head_result_bytes, error, capacity) != 0) return -1;
+    float *dlogits[kMaxBatch];
+    HeadArgmaxArgs a{};
+    for (size_t b = 0; b < batch; ++b) {
+        if (dev_hidden[b] == nullptr) {
+            set_error(error, capacity, "invalid head argmax arguments");
+            return -1;
+        }
+        dlogits[b] = st->head_logits + b * rows;
+        a.logits[b] = dlogits[b];
+        a.forbid_eos[b] = forbid_eos[b] != 0;
+    }
+    const int saved_qtype = st->qtype;   // the reference's head loop is f32 arithmetic on the stored weights
+    st->qtype = MYNAH_HIP_F32;
+    const int rc = linear_rows(st, dev_hidden, dlogits, batch, width, rows, weight, bias, nullptr, nullptr, nullptr, error, capacity);
+    st->qtype = saved_qtype;
+    if (rc != 0) return -1;
+    unsigned char *res = static_cast<unsigned char *>(st->head_result);
+    a.values = reinterpret_cast<unsigned *>(res);
+    a.stored = a.values + n;
+    size_t off = 2 * n * sizeof(unsigned);
+    a.saw_eos = reinterpret_cast<int *>(res + off);
+    off = (off + batch * sizeof(int) + 7) & ~(size_t)7;
+    a.eos_frame = reinterpret_cast<unsigned long long *>(res + off);
+    a.streams = (int)streams; a.vocab = (int)vocab; a.codebook_size = (int)codebook_size;
+    a.eos_id = eos_id >= 0x7fffffffu ? 0x7ffffffe : (int)eos_id;   // an id beyond the vocabulary matches no candidate
+    a.codebook_count = (int)codebook_count;
+    if (launch_head_argmax(st, a, (int)batch, error, capacity) != 0) return -1;
+    const size_t used = off + batch * sizeof(unsigned long long);
+    MYNAH_TRY(hipMemcpyAsync(st->pinned, st->head_result, used, hipMemcpyDeviceToHost, st->stream));
+    if (synchronise(st, error, capacity) != 0) return -1;
+    const unsigned char *host = static_cast<const unsigned char *>(st->pinned);
+    memcpy(values, host, n * sizeof(unsigned));
+    memcpy(stored, host + n * sizeof(unsigned), n * sizeof(unsigned));
+    const int *hs = reinterpret_cast<const int *>(host + 2 * n * sizeof(unsigned));
+    const unsigned long long *hf = reinterpret_cast<const unsigned long long *>(host + off);
+    for (size_t b = 0; b < batch; ++b) {
+        saw_eos[b] = hs[b];
+        eos_frame[b] = hf[b] == ~0ull ? SIZE_MAX : (size_t)hf[b];
+    }
     return 0;
 }
 

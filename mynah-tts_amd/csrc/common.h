@@ -125,6 +125,10 @@ struct State {
     std::unordered_map<WeightKey, CachedWeight, WeightKeyHash> weights;
     size_t weight_bytes = 0;
     std::map<std::pair<const float *, size_t>, PositionTable> position_tables;   // by (host table, width)
+    float *head_logits = nullptr;        // logits of mynah_hip_head_argmax, [kMaxBatch, rows] (grown on demand)
+    size_t head_logits_floats = 0;
+    void *head_result = nullptr;         // its results on the device: values | stored | saw_eos | eos_frame
+    size_t head_result_bytes = 0;
     std::vector<void *> pending_free;   // from mynah_hip_dev_free, freed at the next synchronisation
     // upload scratch (src/backend.h:78-81) and pinned staging for h2d/d2h
     float *scratch = nullptr;

@@ -186,6 +186,16 @@ int launch_gather(State *st, const float *const *dev_tables, size_t table_count,
 int launch_stream_copy(State *st, const void *src, void *dst, size_t bytes, char *error, size_t capacity);
 
 // Resident step: writes the slot table to device memory and forms x[b] = input[b] + position[length[b]].
+// Token choice of the decoder head for `batch` slots (kernels_misc.hip).
+struct HeadArgmaxArgs {
+    const float *logits[kMaxBatch];   // [streams, vocab] per slot
+    int forbid_eos[kMaxBatch];
+    int streams, vocab, codebook_size, eos_id, codebook_count;
+    unsigned *values, *stored;        // device [batch, streams]
+    int *saw_eos;                     // device [batch]
+    unsigned long long *eos_frame;    // device [batch], ~0 = none
+};
+int launch_head_argmax(State *st, const HeadArgmaxArgs &args, int batch, char *error, size_t capacity);
 int launch_step_begin(State *st, const StepSlots &slots, StepSlots *dev_slots, int batch, size_t width,
                       const float *dev_position, float *x, size_t x_stride, char *error, size_t capacity);
 // Final norm of the step: out = slots->output[b]; gain may be null (plain copy).

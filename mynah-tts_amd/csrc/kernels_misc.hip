@@ -106,6 +106,54 @@ __global__ void __launch_bounds__(256) k_argmax(const float *logits, int vocab, 
     if (threadIdx.x == 0) result[0] = s_idx[0] == 0x7fffffff ? 0u : (unsigned)s_idx[0];
 }
 
+// The decoder head's token choice for every stream of every slot at once (slot_advance, src/graph.c:3873-3905; the rule of
+// mynah_matvec_argmax_f32, src/kernels.c:116-139): per (slot, stream) the first maximum among the codes and, unless forbidden
+// for that slot, the end-of-sequence id, strict > from -FLT_MAX, 0 when nothing beats it; then the slot's bookkeeping -- EOS seen,
+// the earliest frame it was seen in, the stored code.  One workgroup per slot; logits[slot] is [streams, vocab].
+__global__ void __launch_bounds__(256) k_head_argmax(HeadArgmaxArgs a) {
+    __shared__ float s_val[4];
+    __shared__ int s_idx[4];
+    const int b = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *logits = a.logits[b];
+    const bool allow_eos = a.forbid_eos[b] == 0;
+    int saw_eos = 0;
+    unsigned long long eos_frame = ~0ull;
+    for (int s = 0; s < a.streams; ++s) {
+        const float *row = logits + (size_t)s * a.vocab;
+        float best = -FLT_MAX;
+        int at = 0x7fffffff;
+        for (int i = tid; i < a.vocab; i += 256) {
+            if (!(i < a.codebook_size || (allow_eos && i == a.eos_id))) continue;
+            const float v = row[i];
+            if (v > best) { best = v; at = i; }   // ascending i inside a thread: the first maximum is kept
+        }
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(best, off);
+            const int oi = __shfl_xor(at, off);
+            if (ov > best || (ov == best && oi < at)) { best = ov; at = oi; }
+        }
+        __syncthreads();   // the slots below are free again
+        if (lane == 0) { s_val[wave] = best; s_idx[wave] = at; }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < 4; ++w)
+                if (s_val[w] > best || (s_val[w] == best && s_idx[w] < at)) { best = s_val[w]; at = s_idx[w]; }
+            const unsigned value = at == 0x7fffffff ? 0u : (unsigned)at;
+            if ((int)value == a.eos_id) {
+                saw_eos = 1;
+                const unsigned long long frame = (unsigned long long)(s / a.codebook_count);
+                if (frame < eos_frame) eos_frame = frame;
+            }
+            a.values[(size_t)b * a.streams + s] = value;
+            a.stored[(size_t)b * a.streams + s] = (int)value < a.codebook_size ? value : 0u;
+        }
+    }
+    if (tid == 0) {
+        a.saw_eos[b] = saw_eos;
+        a.eos_frame[b] = eos_frame;
+    }
+}
+
 // Embedding gather: sum of table rows (bit-exact copy for one table and scale 1) + optional position.
 struct GatherTables { const float *t[32]; };
 __global__ void __launch_bounds__(256) k_gather(GatherTables tables, int table_count, const int32_t *ids, int width, float scale,
@@ -205,6 +253,10 @@ int launch_argmax(State *st, const float *logits, size_t vocab, size_t codebook,
     hipLaunchKernelGGL(k_argmax, dim3(1), dim3(256), 0, st->stream, logits, (int)vocab, (int)codebook, (int)eos, allow_eos,
                        dev_result);
     return hip_check(hipGetLastError(), "argmax launch", error, capacity);
+}
+int launch_head_argmax(State *st, const HeadArgmaxArgs &a, int batch, char *error, size_t capacity) {
+    hipLaunchKernelGGL(k_head_argmax, dim3((unsigned)batch), dim3(256), 0, st->stream, a);
+    return hip_check(hipGetLastError(), "head argmax launch", error, capacity);
 }
 int launch_gather(State *st, const float *const *dev_tables, size_t table_count, const int32_t *dev_ids, size_t tokens,
                   size_t width, float scale, const float *dev_position, float *out, char *error, size_t capacity) {

@@ -245,6 +245,48 @@ def test_cross_kv_from_resident_memory(backend, pkg, orc, nerr, qtype_name):
         backend.set_quant(pkg.F32)
 
 
+def test_decoder_head_argmax_for_all_slots_and_streams(backend, pkg, orc):
+    """slot_advance's head (src/graph.c:3873-3905): per slot and stacked stream the constrained first maximum of
+    final_proj's logits, stored codes and EOS bookkeeping, for five slots in one call -- against the oracle's f32 matvec +
+    constrained argmax per stream.  EOS is forced into chosen streams through the bias; one of those slots forbids it.
+    Runs under int8 quantisation too: the head stays f32 like the reference's loop."""
+    _announce("decoder head: batched constrained argmax")
+    rng = np.random.default_rng(530)
+    width, streams, vocab, codebook, eos, per_frame = 768, 8, 1024, 1000, 1010, 4
+    w = backend.keep((rng.standard_normal((streams * vocab, width)) * 0.05).astype(np.float32))
+    bias = (rng.standard_normal(streams * vocab) * 0.1).astype(np.float32)
+    bias[5 * vocab + eos] = 50.0        # stream 5 (frame 1) says EOS wherever it is allowed
+    bias[2 * vocab + 1017] = 80.0       # a forbidden id with the largest logit of stream 2: never chosen
+    bias = backend.keep(bias)
+    hidden = rng.standard_normal((5, width)).astype(np.float32)
+    forbid = [0, 1, 0, 0, 1]
+    bufs = [backend.alloc(width).write(h) for h in hidden]
+    for qt in (pkg.F32, pkg.INT8):
+        backend.set_quant(qt)
+        values, stored, saw, frame = backend.head_argmax([d.ptr for d in bufs], width, w, bias, streams, vocab, codebook, eos, per_frame, forbid)
+        for b in range(5):
+            logits = orc.matvec_f32(hidden[b], w, bias).reshape(streams, vocab)
+            want_saw, want_frame = 0, None
+            for s in range(streams):
+                rc, want = orc.argmax_constrained(logits[s], codebook, eos, not forbid[b])
+                assert rc == 0
+                got = int(values[b, s])
+                if got != want:      # only a tie within rounding may differ
+                    assert abs(float(logits[s][got]) - float(logits[s][want])) <= 1e-5 * np.abs(logits[s]).max(), (b, s, got, want)
+                assert got < codebook or (got == eos and not forbid[b])
+                assert int(stored[b, s]) == (got if got < codebook else 0)
+                if got == eos:
+                    want_saw = 1
+                    want_frame = s // per_frame if want_frame is None else min(want_frame, s // per_frame)
+            assert int(saw[b]) == want_saw and frame[b] == want_frame, (b, saw[b], frame[b])
+        assert saw[0] == 1 and frame[0] == 1 and saw[1] == 0 and values[0, 5] == eos
+    backend.set_quant(pkg.F32)
+    with pytest.raises(pkg.BackendError):
+        backend.head_argmax([d.ptr for d in bufs], width, w, bias, streams, vocab, vocab + 1, eos, per_frame, forbid)   # more codes than vocabulary
+    for d in bufs:
+        d.free()
+
+
 def test_layernorm_gelu_residual_softmax(backend, orc, nerr):
     _announce("layernorm/gelu/residual/softmax")
     rng = np.random.default_rng(600)

@@ -167,3 +167,29 @@ def test_attention_kats_and_float64(orc, nerr):
     p1 = np.exp(s1 - s1.max())
     p1 /= p1.sum()
     assert nerr(out1, p1 @ vc[:L].astype(np.float64)) < 2e-6
+
+
+def test_head_choice_against_the_reference_fused_matvec_argmax(orc, ref_strict):
+    """What the GPU head test compares with -- the oracle's f32 matvec followed by its constrained first-max -- against
+    the compiled reference's own fused mynah_matvec_argmax_f32 (src/kernels.c:116-139, strict build: the same
+    sequential dot product), with and without the extra row, incl. a forbidden row that holds the largest value."""
+    rng = np.random.default_rng(77)
+    rows, cols, allowed, extra = 1024, 768, 1000, 1010
+    ref_strict.mynah_matvec_argmax_f32.restype = C.c_int
+    ref_strict.mynah_matvec_argmax_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int,
+                                                   C.POINTER(C.c_uint)]
+    for trial in range(6):
+        w = (rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)
+        x = rng.standard_normal(cols).astype(np.float32)
+        bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+        if trial % 2:
+            bias[extra] = 40.0                # the extra row wins wherever it is allowed
+        bias[1017] = 90.0                     # never allowed
+        logits = orc.matvec_f32(x, w, bias)
+        for allow in (0, 1):
+            out = C.c_uint(0)
+            rc = ref_strict.mynah_matvec_argmax_f32(w.ctypes.data, x.ctypes.data, bias.ctypes.data, rows, cols, allowed, extra, allow, C.byref(out))
+            assert rc == 0
+            orc_rc, got = orc.argmax_constrained(logits, allowed, extra, allow)
+            assert orc_rc == 0 and got == out.value, (trial, allow, got, out.value)
+            assert got != 1017 and (got == extra) == bool(allow and trial % 2)
