@@ -77,16 +77,20 @@ __device__ __forceinline__ unsigned long long candidate(unsigned key, int index)
 __device__ __forceinline__ int candidate_index(unsigned long long c) { return (int)(0xffffffffu - (unsigned)(c & 0xffffffffull)); }
 __device__ __forceinline__ unsigned candidate_key(unsigned long long c) { return (unsigned)(c >> 32); }
 
-// How many of list[0, n) are above `mine` (pairs of entries per LDS read; the list is 16-byte aligned).
-__device__ __forceinline__ int count_above(const unsigned long long *list, int n, unsigned long long mine) {
+// How many of list[0, n) are above `mine` (pairs of entries per LDS read; the list is 16-byte aligned), counted by four
+// adjacent threads: thread `part` of the four looks at pairs part, part + 4, ... and the four sums meet by shuffles.  Every
+// lane of the wavefront must call it.
+__device__ __forceinline__ int count_above_by_four(const unsigned long long *list, int n, unsigned long long mine, int part) {
     const ulonglong2 *pairs = reinterpret_cast<const ulonglong2 *>(list);
     int above = 0;
 #pragma unroll 4
-    for (int j = 0; j < n / 2; ++j) {
+    for (int j = part; j < n / 2; j += 4) {
         const ulonglong2 p = pairs[j];
         above += (p.x > mine ? 1 : 0) + (p.y > mine ? 1 : 0);
     }
-    if (n & 1) above += list[n - 1] > mine ? 1 : 0;
+    if ((n & 1) && part == 0) above += list[n - 1] > mine ? 1 : 0;
+    above += __shfl_xor(above, 1);
+    above += __shfl_xor(above, 2);
     return above;
 }
 
@@ -145,6 +149,11 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
 
     // ---- constraint mask (src/graph.c:1556-1563); eight candidates per thread are requested at a time
     unsigned long long mine = 0ull;
+    constexpr int kKeysInRegisters = 8;              // a vocabulary of up to 8 * 256 ids: a thread's keys stay in registers for the collection below
+    const bool keys_in_registers = V <= kKeysInRegisters * 256;
+    unsigned own_key[kKeysInRegisters];
+#pragma unroll
+    for (int i = 0; i < kKeysInRegisters; ++i) own_key[i] = 0u;
     for (int c0 = tid; c0 < V; c0 += 8 * 256) {
         float v[8];
 #pragma unroll
@@ -157,6 +166,7 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
                 const float masked = allowed ? v[i] : -FLT_MAX;
                 const unsigned key = order_key(masked);
                 s_key[c] = key;
+                if (c0 == tid) own_key[i] = key;
                 if (logits_copy != nullptr) logits_copy[((size_t)b * a.streams + a.stream) * V + c] = masked;
                 const unsigned long long cand = candidate(key, c);
                 mine = cand > mine ? cand : mine;
@@ -194,22 +204,43 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
 
     if (sampling) {
         // ---- collect the candidates at or above the bound: one LDS counter update per wavefront, places by ballot
-        unsigned in_wave = 0u;
-        for (int base = wave * 64; base < V; base += 256) {
-            const int c = base + lane;
-            in_wave += (unsigned)__popcll(__ballot(c < V && s_key[c] >= bound));
-        }
-        unsigned next_slot = 0u;
-        if (lane == 0) next_slot = atomicAdd(&s_count, in_wave);
-        next_slot = __shfl(next_slot, 0);
-        for (int base = wave * 64; base < V; base += 256) {
-            const int c = base + lane;
-            const unsigned key = c < V ? s_key[c] : 0u;
-            const bool take = c < V && key >= bound;
-            const unsigned long long mask = __ballot(take);
-            const unsigned slot = next_slot + (unsigned)__popcll(mask & ((1ull << lane) - 1ull));
-            if (take && slot < (unsigned)kFastCandidates) s_cand[slot] = candidate(key, c);
-            next_slot += (unsigned)__popcll(mask);
+        if (keys_in_registers) {
+            // from the keys the thread kept (ids tid + 256 i): eight ballots, no LDS read
+            unsigned long long masks[kKeysInRegisters];
+            unsigned in_wave = 0u;
+#pragma unroll
+            for (int i = 0; i < kKeysInRegisters; ++i) {
+                masks[i] = __ballot(tid + 256 * i < V && own_key[i] >= bound);
+                in_wave += (unsigned)__popcll(masks[i]);
+            }
+            unsigned next_slot = 0u;
+            if (lane == 0) next_slot = atomicAdd(&s_count, in_wave);
+            next_slot = __shfl(next_slot, 0);
+#pragma unroll
+            for (int i = 0; i < kKeysInRegisters; ++i) {
+                const bool take = (masks[i] >> lane) & 1ull;
+                const unsigned slot = next_slot + (unsigned)__popcll(masks[i] & ((1ull << lane) - 1ull));
+                if (take && slot < (unsigned)kFastCandidates) s_cand[slot] = candidate(own_key[i], tid + 256 * i);
+                next_slot += (unsigned)__popcll(masks[i]);
+            }
+        } else {
+            unsigned in_wave = 0u;
+            for (int base = wave * 64; base < V; base += 256) {
+                const int c = base + lane;
+                in_wave += (unsigned)__popcll(__ballot(c < V && s_key[c] >= bound));
+            }
+            unsigned next_slot = 0u;
+            if (lane == 0) next_slot = atomicAdd(&s_count, in_wave);
+            next_slot = __shfl(next_slot, 0);
+            for (int base = wave * 64; base < V; base += 256) {
+                const int c = base + lane;
+                const unsigned key = c < V ? s_key[c] : 0u;
+                const bool take = c < V && key >= bound;
+                const unsigned long long mask = __ballot(take);
+                const unsigned slot = next_slot + (unsigned)__popcll(mask & ((1ull << lane) - 1ull));
+                if (take && slot < (unsigned)kFastCandidates) s_cand[slot] = candidate(key, c);
+                next_slot += (unsigned)__popcll(mask);
+            }
         }
         __syncthreads();
         int listed = (int)s_count;
@@ -285,10 +316,11 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
             __syncthreads();
         }
         // ---- list position = how many collected candidates come before; numerators expf((l - max) / T) (src/graph.c:1599-1604)
-        for (int q = tid; q < listed; q += 256) {
-            const unsigned long long own = s_cand[q];
-            const int place = count_above(s_cand, listed, own);
-            if (place < top_count) {
+        for (int q0 = 0; q0 < listed; q0 += 64) {   // four adjacent threads per candidate; every lane takes part in the shuffles
+            const int q = q0 + (tid >> 2);
+            const unsigned long long own = s_cand[q < listed ? q : listed - 1];
+            const int place = count_above_by_four(s_cand, listed, own, tid & 3);
+            if (q < listed && (tid & 3) == 0 && place < top_count) {
                 s_top_idx[place] = candidate_index(own);
                 s_top_val[place] = expf((key_value(candidate_key(own)) - maximum) / temperature);
             }
