@@ -159,3 +159,16 @@ def test_encoder_rejects_other_conv_kernels(pkg, backend, synth):
     cfg = dict(synth.encoder_config(layers=1), ffn_kernel=2)
     with pytest.raises(pkg.BackendError, match="ffn_kernel"):
         pkg.Encoder(backend, cfg, synth.encoder_weights_f16(cfg, seed=1, kernel=2))
+
+
+@pytest.mark.parametrize("width,heads,ffn,kernel", [(64, 1, 192, 3), (320, 5, 704, 1), (1024, 16, 2048, 3), (1152, 18, 2304, 1)])
+def test_encoder_other_widths(pkg, backend, orc, synth, nerr, width, heads, ffn, kernel):
+    """Narrow, odd-multiple and wide rows (the row pass keeps 4 or 16 pieces of a row per lane), both FFN forms."""
+    _announce("encoder width=%d heads=%d ffn=%d kernel=%d" % (width, heads, ffn, kernel))
+    cfg = dict(synth.encoder_config(layers=2, width=width, heads=heads, ffn=ffn, vocab=512, max_positions=128), causal=True, ffn_kernel=kernel)
+    w = synth.encoder_weights_f16(cfg, seed=80, kernel=kernel)
+    ids = np.random.default_rng(81).integers(0, cfg["vocab"], size=70).astype(np.int32)
+    got = _prefill(pkg, backend, cfg, w, ids)
+    _, want = orc.encoder_prefill(cfg, _f16_bits(w), ids)
+    assert np.isfinite(got).all()
+    assert nerr(got, want) < 2e-3
