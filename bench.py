@@ -15,6 +15,7 @@ The JSON line also carries the same stack at batch 8 with ragged cache lengths (
 the roofline of the step and the CPU baseline (the reference's own CPU decode step, compiled from its sources).
 """
 import argparse
+import importlib
 import json
 import os
 import subprocess
@@ -213,47 +214,51 @@ def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
     cur, up, out, act, res, br, work = bufs
     audio = backend.alloc(L)
 
-    def decode():
+    codec = importlib.import_module(pkg.__name__ + ".codec")
+
+    def decode(fused):
+        """fused: the element-wise operators inside the convolutions' epilogues (mynah_hip_conv1d_fused); else the operator
+        sequence decode_codec_resident issues through the seam.  Both give the same samples, bit for bit."""
         nonlocal cur, up, out
         C, L = 864, frames
-        backend.conv1d(latent.ptr, cur.ptr, 32, 864, L, 7, 1, *pre)
-        for st in stages:
+        if fused:
+            backend.conv1d_fused(latent.ptr, cur.ptr, 32, 864, L, 7, 1, *pre, alpha=stages[0]["alpha"])
+        else:
+            backend.conv1d(latent.ptr, cur.ptr, 32, 864, L, 7, 1, *pre)
+        for index, st in enumerate(stages):
             nc, nl = C // 2, L * st["rate"]
-            backend.snake_dev(cur.ptr, st["alpha"], C, L, C // 2)
+            if not fused:
+                backend.snake_dev(cur.ptr, st["alpha"], C, L, C // 2)
             backend.conv_transpose_dev(cur.ptr, up.ptr, C, nc, L, nl, 2 * st["rate"], st["rate"], nc, *st["up"])
-            n = nc * nl
-            for index, (branch, k) in enumerate(zip(st["blocks"], kernels)):
-                backend.copy_dev(work.ptr, up.ptr, n)
-                for a1, c1, a2, c2, d in branch:
-                    backend.copy_dev(act.ptr, work.ptr, n)
-                    backend.snake_dev(act.ptr, a1, nc, nl, nc // 2)
-                    backend.conv1d(act.ptr, res.ptr, nc, nc, nl, k, d, *c1)
-                    backend.snake_dev(res.ptr, a2, nc, nl, nc // 2)
-                    backend.conv1d(res.ptr, br.ptr, nc, nc, nl, k, 1, *c2)
-                    backend.residual_inplace(work.ptr, br.ptr, n)
-                if index == 0:
-                    backend.copy_dev(out.ptr, work.ptr, n)          # the reference adds to uploaded zeros (:2441,2492)
-                else:
-                    backend.residual_inplace(out.ptr, work.ptr, n)
-            backend.scale_dev(out.ptr, n, 1.0 / 3.0)
+            if fused:
+                then_alpha = stages[index + 1]["alpha"] if index + 1 < len(stages) else post_alpha
+                codec.res_layer_fused(backend, st["blocks"], up.ptr, out.ptr, nc, nl, work.ptr, act.ptr, res.ptr, then_alpha=then_alpha)
+            else:
+                codec.res_layer(backend, st["blocks"], up.ptr, out.ptr, nc, nl, work.ptr, act.ptr, res.ptr, br.ptr)
             cur, out = out, cur
             C, L = nc, nl
-        backend.snake_dev(cur.ptr, post_alpha, C, L, C // 2)
+        if not fused:
+            backend.snake_dev(cur.ptr, post_alpha, C, L, C // 2)
         backend.conv1d(cur.ptr, audio.ptr, C, 1, L, 3, 1, *post)
         backend.clip_dev(audio.ptr, L)
 
-    for _ in range(warmup):
-        decode()
-    backend.sync()
-    backend.timer_begin()
-    for _ in range(runs):
-        decode()
-    ms = backend.timer_end() / runs
-    samples = audio.read()
+    timings, waves = {}, {}
+    for fused in (False, True):
+        for _ in range(warmup):
+            decode(fused)
+        backend.sync()
+        backend.timer_begin()
+        for _ in range(runs):
+            decode(fused)
+        timings[fused] = backend.timer_end() / runs
+        waves[fused] = audio.read()
+    assert np.array_equal(waves[False].view(np.uint32), waves[True].view(np.uint32)), "the fused sequence changed the samples"
+    ms, samples = timings[True], waves[True]
     assert np.all(np.isfinite(samples)) and np.abs(samples).max() <= 1.0, "codec output is not a clipped waveform"
     for d in bufs + [latent, audio]:
         d.free()
-    return {"frames": frames, "samples": int(L), "ms": ms, "flops": flops, "tflops": flops / (ms * 1e-3) / 1e12}
+    return {"frames": frames, "samples": int(L), "ms": ms, "flops": flops, "tflops": flops / (ms * 1e-3) / 1e12,
+            "ms_seam_operator_sequence": timings[False]}
 
 
 # (with one or two streams the attention partials are folded by the output projection that follows; with more, by
@@ -460,7 +465,10 @@ def main():
                                        "dilations 1/3/5, 864..27 channels) on the f32 matrix cores, grouped transposed conv, half-snake"
                                        % (codec["frames"], codec["samples"]),
                            "ms": round(codec["ms"], 3), "flops": codec["flops"], "tflops": round(codec["tflops"], 2), "bound": "mfma",
-                           "peak_tflops": 157.3, "frac": round(codec["tflops"] / 157.3, 4)}
+                           "peak_tflops": 157.3, "frac": round(codec["tflops"] / 157.3, 4),
+                           "form": "element-wise operators in the convolutions' epilogues (mynah_hip_conv1d_fused), samples bit-identical "
+                                   "to the seam's operator sequence",
+                           "ms_seam_operator_sequence": round(codec["ms_seam_operator_sequence"], 3)}
     if not args.no_cpu:
         cpu = cpu_baseline()
         allc = cpu.get("all", {})

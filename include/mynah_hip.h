@@ -164,6 +164,35 @@ int mynah_hip_conv_transpose_dev(void *state, const float *dev_input, float *dev
 int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length,
                         size_t snake_channels, char *error, size_t error_capacity);
 
+/* The residual layer of the codec (res_layer_device, src/graph.c:2423-2498) spends a fifth of its time in the element-wise
+ * operators between its convolutions: copy_dev, snake_dev, residual_inplace, scale_dev, each a pass over the rows in
+ * device memory.  conv1d_fused is conv1d followed, value by value before the store, by the arithmetic of those operators
+ * in this fixed order (every step optional), so that a sequence of fused calls gives the bits of the sequence it replaces:
+ *   v  = conv + bias
+ *   v  = dev_residual[i] + v          residual_inplace (src/backend.h:86-88); dev_residual may be dev_output
+ *   v  = dev_residual2[i] + v         a second one
+ *   v  = v * scale                    scale_dev, when scale != 1
+ *   activate == 0:                    dev_output[i] = v
+ *   activate != 0, dev_activated 0:   dev_output[i] = half-snake of v with the alpha of v's output channel (snake_dev on the result)
+ *   activate != 0, dev_activated set: dev_output[i] = v and dev_activated[i] = half-snake of v (the copy_dev + snake_dev
+ *                                     that prepare the next convolution's input while the plain value stays the residual)
+ * snake_alpha is a host pointer like every weight.  snake_copy_dev is snake_dev from one row set into another (copy_dev +
+ * snake_dev).  Neither has a counterpart in the reference's seam: they are for an engine whose residual layer calls them instead. */
+typedef struct mynah_hip_conv1d_extra {
+    const float *dev_residual;
+    const float *dev_residual2;
+    float scale;
+    int activate;
+    const float *snake_alpha;
+    size_t snake_channels;
+    float *dev_activated;
+} mynah_hip_conv1d_extra;
+int mynah_hip_conv1d_fused(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                           int kernel, int dilation, const float *weight, const float *bias, const mynah_hip_conv1d_extra *extra,
+                           char *error, size_t error_capacity);
+int mynah_hip_snake_copy_dev(void *state, const float *dev_input, float *dev_output, const float *alpha, size_t channels,
+                             size_t length, size_t snake_channels, char *error, size_t error_capacity);
+
 /* ------------------------------------------------------------------------------------------
  * Section 2 -- what the single-stream seam lacks
  * ------------------------------------------------------------------------------------------ */

@@ -47,6 +47,11 @@ class DecoderSlot(C.Structure):
                 ("length", _sz), ("memory_length", _sz), ("dev_input", _vp), ("dev_output", _vp)]
 
 
+class Conv1dExtra(C.Structure):
+    _fields_ = [("dev_residual", _vp), ("dev_residual2", _vp), ("scale", C.c_float), ("activate", C.c_int),
+                ("snake_alpha", _vp), ("snake_channels", _sz), ("dev_activated", _vp)]
+
+
 class EncoderDesc(C.Structure):
     _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn_width", _sz),
                 ("vocab", _sz), ("max_positions", _sz), ("tok_table", _vp), ("pos_table", _vp),
@@ -106,6 +111,9 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_conv_transpose_dev.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp,
                                                  *_err]
     lib.mynah_hip_snake_dev.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, *_err]
+    lib.mynah_hip_snake_copy_dev.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, *_err]
+    lib.mynah_hip_conv1d_fused.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp,
+                                           C.POINTER(Conv1dExtra), *_err]
     lib.mynah_hip_set_quant.argtypes = [_vp, C.c_int, C.c_int, *_err]
     lib.mynah_hip_quantize_weight_int8.argtypes = [_vp, _sz, _sz, _vp, _vp, C.c_int]
     lib.mynah_hip_quantize_weight_int8.restype = None
@@ -335,6 +343,19 @@ class Backend:
 
     def snake_dev(self, d, alpha, channels, length, snake_channels):
         self._call("mynah_hip_snake_dev", d, _np_ptr(self.keep(alpha)), _sz(channels), _sz(length), _sz(snake_channels))
+
+    def snake_copy_dev(self, din, dout, alpha, channels, length, snake_channels):
+        self._call("mynah_hip_snake_copy_dev", din, dout, _np_ptr(self.keep(alpha)), _sz(channels), _sz(length), _sz(snake_channels))
+
+    def conv1d_fused(self, din, dout, in_ch, out_ch, length, kernel, dilation, weight, bias=None, residual=None, residual2=None,
+                     scale=1.0, alpha=None, snake_channels=None, activated=None):
+        """conv1d, then per value: + residual, + residual2, * scale, and (alpha given) the half-snake, written to dout or,
+        with `activated`, beside the plain value."""
+        extra = Conv1dExtra(residual, residual2, scale, 0 if alpha is None else 1,
+                            None if alpha is None else _np_ptr(self.keep(alpha)),
+                            0 if alpha is None else (out_ch // 2 if snake_channels is None else snake_channels), activated)
+        self._call("mynah_hip_conv1d_fused", din, dout, in_ch, out_ch, length, kernel, dilation, _np_ptr(self.keep(weight)),
+                   None if bias is None else _np_ptr(self.keep(bias)), C.byref(extra))
 
     def argmax_dev(self, dlogits, vocab, codebook_size, eos_id, allow_eos):
         out = C.c_uint(0)

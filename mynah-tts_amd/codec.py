@@ -1,0 +1,52 @@
+"""The codec's residual layer as two sequences of backend calls.
+
+`res_layer` issues what res_layer_device issues (src/graph.c:2423-2498): per branch a copy of the input, per block
+copy, snake, conv, snake, conv, residual add, then the branch added to the output, and the sum scaled by a third at the
+end.  `res_layer_fused` computes the same values, bit for bit, from a third of the launches: the element-wise operators
+travel in the epilogue of the convolution before them (mynah_hip_conv1d_fused), and only a branch's first activation is a
+pass of its own (snake_copy_dev).
+
+blocks[branch][block] = (alpha_in, (w_in, b_in), alpha_skip, (w_skip, b_skip), dilation); the branch's kernel size is the
+weights' last dimension.  Buffers are device allocations of channels * length floats.
+"""
+
+
+def res_layer(backend, blocks, din, dout, channels, length, current, activated, residual, branch_out):
+    n = channels * length
+    for index, branch in enumerate(blocks):
+        backend.copy_dev(current, din, n)
+        for a_in, (w_in, b_in), a_skip, (w_skip, b_skip), dilation in branch:
+            kernel = w_in.shape[2]
+            backend.copy_dev(activated, current, n)
+            backend.snake_dev(activated, a_in, channels, length, channels // 2)
+            backend.conv1d(activated, residual, channels, channels, length, kernel, dilation, w_in, b_in)
+            backend.snake_dev(residual, a_skip, channels, length, channels // 2)
+            backend.conv1d(residual, branch_out, channels, channels, length, kernel, 1, w_skip, b_skip)
+            backend.residual_inplace(current, branch_out, n)
+        if index == 0:
+            backend.copy_dev(dout, current, n)          # the reference adds to uploaded zeros (src/graph.c:2441,2492)
+        else:
+            backend.residual_inplace(dout, current, n)
+    backend.scale_dev(dout, n, 1.0 / 3.0)
+
+
+def res_layer_fused(backend, blocks, din, dout, channels, length, current, activated, residual, then_alpha=None):
+    """then_alpha: the half-snake that the caller would apply to the layer's output next (decode_codec_resident's
+    activation before the next stage's transposed conv or the post-conv), applied by the layer's last call."""
+    for index, branch in enumerate(blocks):
+        backend.snake_copy_dev(din, activated, branch[0][0], channels, length, channels // 2)
+        for position, (a_in, (w_in, b_in), a_skip, (w_skip, b_skip), dilation) in enumerate(branch):
+            kernel = w_in.shape[2]
+            # input conv, its result activated for the skip conv
+            backend.conv1d_fused(activated, residual, channels, channels, length, kernel, dilation, w_in, b_in, alpha=a_skip)
+            before = din if position == 0 else current
+            if position + 1 < len(branch):
+                # skip conv + the block's residual add; the sum also leaves activated for the next block's input conv
+                backend.conv1d_fused(residual, current, channels, channels, length, kernel, 1, w_skip, b_skip, residual=before,
+                                     alpha=branch[position + 1][0], activated=activated)
+            else:
+                # the branch's last block adds the branch to the output, and the last branch scales the sum
+                backend.conv1d_fused(residual, dout, channels, channels, length, kernel, 1, w_skip, b_skip, residual=before,
+                                     residual2=None if index == 0 else dout,
+                                     scale=1.0 / 3.0 if index + 1 == len(blocks) else 1.0,
+                                     alpha=then_alpha if index + 1 == len(blocks) else None)

@@ -16,6 +16,8 @@
 //                   (snake_row, src/backend.c:643-658).
 #include <limits.h>
 
+#include <type_traits>
+
 #include "kernels.h"
 
 using namespace mynah;
@@ -27,6 +29,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int kConvChannels = 8;      // input channels staged per step of the inner dimension
 constexpr int kConvMaxKernel = 16;
 constexpr int kConvMaxHalo = 128;     // (kernel - 1) * dilation
+constexpr int kTileStride = 65;       // floats per row of a wavefront's 32 x 64 tile in LDS (fused epilogue)
 
 struct ConvArgs {
     const float *in;     // [in_ch, length]
@@ -34,7 +37,71 @@ struct ConvArgs {
     const float *w;      // [out_ch, in_ch * kernel]
     const float *bias;   // [out_ch] or null
     int in_ch, out_ch, length, kernel, dilation;
+    // what mynah_hip_conv1d_fused adds after conv + bias, in this order (each step is the arithmetic of the seam operator it replaces)
+    const float *residual = nullptr;    // [out_ch, length] added (residual_inplace); may be `out` itself
+    const float *residual2 = nullptr;   // then this one
+    float scale = 1.0f;                 // then multiplied (scale_dev) when `scaled`
+    int scaled = 0;
+    int activate = 0;                   // then the half-snake of the value's output channel (snake_dev)
+    const float *alpha = nullptr;       // [snake_channels]
+    int snake_channels = 0;
+    float *act_out = nullptr;           // null: `out` gets the activated value; else `out` keeps the value before it and this gets the activated one
 };
+
+// sin(x) in some twenty instructions for |x| < kShortSineLimit (the library routine, which also serves arguments of any
+// size, is about 150, and inside a convolution's epilogue nothing hides them): x = k * pi/2 + r with pi/2 in three pieces
+// and fused multiply-adds, then the sine or cosine polynomial of r on [-pi/4, pi/4] (Cephes' single-precision
+// coefficients).  Largest difference from the double-precision sine over every 7th float of (-8192, 8192): 9.3e-8, against
+// 6e-8 for a correctly rounded result near 1.
+constexpr float kShortSineLimit = 8192.0f;
+__device__ __forceinline__ float short_sine(float x) {
+    const float k = __builtin_rintf(x * 0.636619772367581343f);
+    float r = __builtin_fmaf(k, -1.57079637050628662109375f, x);
+    r = __builtin_fmaf(k, 4.37113882867379289e-8f, r);
+    r = __builtin_fmaf(k, 1.71512460692744033e-15f, r);
+    const float z = r * r;
+    const float s = __builtin_fmaf(r * z, __builtin_fmaf(z, __builtin_fmaf(z, -1.9515295891e-4f, 8.3321608736e-3f), -1.6666654611e-1f), r);
+    const float c = __builtin_fmaf(z * z, __builtin_fmaf(z, __builtin_fmaf(z, 2.443315711809948e-5f, -1.388731625493765e-3f), 4.166664568298827e-2f),
+                                   __builtin_fmaf(z, -0.5f, 1.0f));
+    const int q = (int)k;
+    const float v = (q & 1) ? c : s;
+    return (q & 2) ? -v : v;
+}
+// The codec's sine: the short routine where it holds, the library's beyond.
+__device__ __forceinline__ float snake_sine(float x) { return fabsf(x) < kShortSineLimit ? short_sine(x) : sinf(x); }
+
+// snake_row, src/backend.c:643-658.  inv_a = 1 / (alpha + 1e-9) for a snake row; a row past snake_channels is a leaky ReLU.
+__device__ __forceinline__ float half_snake(float v, bool snake_row, float al, float inv_a) {
+    if (snake_row) {
+        const float sn = snake_sine(al * v);
+        return v + sn * sn * inv_a;
+    }
+    return v < 0.0f ? v * 0.01f : v;
+}
+
+// One finished output value (conv + bias) on its way to memory, in two steps so that a kernel can run the first (two
+// requests and three operations) for all of a thread's values at once, requests side by side, and the second (some
+// hundred instructions when there is an activation) in a rolled loop.
+__device__ __forceinline__ float conv_combine(const ConvArgs &a, size_t index, float v) {
+    if (a.residual != nullptr) v = a.residual[index] + v;
+    if (a.residual2 != nullptr) v = a.residual2[index] + v;
+    return v * a.scale;   // 1.0f when there is no scaling: the value's own bits
+}
+// al, inv_a: the output channel's alpha and 1 / (alpha + 1e-9), which the kernels keep in LDS: read from global memory value
+// by value inside the rolled loops, that request was most of what an activation cost.
+__device__ __forceinline__ void conv_emit(const ConvArgs &a, int m, size_t index, float v, float al, float inv_a) {
+    if (a.activate) {
+        const float act = half_snake(v, m < a.snake_channels, al, inv_a);
+        if (a.act_out != nullptr) {
+            a.out[index] = v;
+            a.act_out[index] = act;
+        } else {
+            a.out[index] = act;
+        }
+    } else {
+        a.out[index] = v;
+    }
+}
 
 // The products of one staged block of eight input channels for a wavefront's 32 x 64 tile.  The two inner indices one
 // matrix instruction consumes are the same tap of two neighbouring channels (lanes 0-31: the even channel, lanes 32-63:
@@ -68,7 +135,9 @@ __device__ __forceinline__ void conv_products(const float *wrow, const float *ir
 // the block has columns and the product loop is straight-line code.  The codec's 3, 7 and 11 taps get such builds.
 // VEC: the weight rows are whole 16-byte pieces (in_ch * kernel a multiple of 4): the weight block is staged four
 // elements per request and kept in LDS with packed rows.
-template <int WM, int WN, int KF, int VEC>
+// FUSED: the build that mynah_hip_conv1d_fused launches (residuals, scale, activation after the products); the seam's
+// conv1d keeps a build without any of it.
+template <int WM, int WN, int KF, int VEC, bool FUSED>
 __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     extern __shared__ __align__(16) float lds[];
@@ -170,16 +239,99 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
         __syncthreads();
     }
     // accumulator element r of a lane: row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
+    // conv + bias, then the residuals and the scale (conv_combine's order), without a branch per value: requests go to a
+    // legal address whatever the value's place (element 0 when it lies outside the rows), side by side, and a request
+    // that is not wanted at all is left out by the build of this loop that runs.
+    const auto combine = [&](auto has_first, auto has_second) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+            const int t = t0 + wn * 64 + col;
+            const bool in0 = m < a.out_ch && t < a.length, in1 = m < a.out_ch && t + 32 < a.length;
+            const size_t i0 = in0 ? (size_t)m * a.length + t : 0, i1 = in1 ? (size_t)m * a.length + t + 32 : 0;
+            const float b = (a.bias != nullptr && m < a.out_ch) ? a.bias[m] : 0.0f;
+            float v0 = acc0[r] + b, v1 = acc1[r] + b;
+            if constexpr (decltype(has_first)::value) { v0 = a.residual[i0] + v0; v1 = a.residual[i1] + v1; }
+            if constexpr (decltype(has_second)::value) { v0 = a.residual2[i0] + v0; v1 = a.residual2[i1] + v1; }
+            if constexpr (FUSED) {
+                v0 = v0 * a.scale;   // 1.0f when there is no scaling: the value's own bits
+                v1 = v1 * a.scale;
+            }
+            acc0[r] = v0;
+            acc1[r] = v1;
+            if (!FUSED || !a.activate) {
+                if (in0) a.out[i0] = v0;
+                if (in1) a.out[i1] = v1;
+            }
+        }
+    };
+    if constexpr (!FUSED) {   // the seam's conv1d
+        combine(std::false_type{}, std::false_type{});
+        return;
+    }
+    if (a.residual2 != nullptr) combine(std::true_type{}, std::true_type{});    // the launch refuses a second residual without a first
+    else if (a.residual != nullptr) combine(std::true_type{}, std::false_type{});
+    else combine(std::false_type{}, std::false_type{});
+    if (!a.activate) return;
+    // The rows' alphas and 1 / (alpha + 1e-9) through the wavefront's own piece of LDS (free after the last products' barrier)
+    float *s_alpha = lds + 4 * (32 * kTileStride) + wave * 64;
+    if (lane < 32) {
+        const int m = m0 + wm * 32 + lane;
+        const float al = m < a.snake_channels ? a.alpha[m] : 0.0f;
+        s_alpha[lane] = al;
+        s_alpha[32 + lane] = 1.0f / (al + 1e-9f);
+    }
+    // Common case, every sine argument below the short routine's limit: the activation on the values where they are, in
+    // registers, the short sine inlined 32 times and no branch among them.
+    bool large = false;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-        if (m < a.out_ch) {
-            const float b = a.bias != nullptr ? a.bias[m] : 0.0f;
-            const int t = t0 + wn * 64 + col;
-            if (t < a.length) a.out[(size_t)m * a.length + t] = acc0[r] + b;
-            if (t + 32 < a.length) a.out[(size_t)m * a.length + t + 32] = acc1[r] + b;
-        }
+        const float al = s_alpha[8 * (r >> 2) + 4 * half + (r & 3)];
+        large = large || !(fabsf(al * acc0[r]) < kShortSineLimit) || !(fabsf(al * acc1[r]) < kShortSineLimit);
     }
+    if (!__any(large)) {
+        const auto finish = [&](auto has_copy) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = 8 * (r >> 2) + 4 * half + (r & 3), m = m0 + wm * 32 + row;
+                const int t = t0 + wn * 64 + col;
+                const bool in0 = m < a.out_ch && t < a.length, in1 = m < a.out_ch && t + 32 < a.length;
+                const size_t i0 = (size_t)m * a.length + t, i1 = i0 + 32;
+                const float al = s_alpha[row], inv_a = s_alpha[32 + row];
+                const float v0 = acc0[r], v1 = acc1[r];
+                const float s0 = short_sine(al * v0), s1 = short_sine(al * v1);
+                const bool snake_row = m < a.snake_channels;
+                const float y0 = snake_row ? v0 + s0 * s0 * inv_a : (v0 < 0.0f ? v0 * 0.01f : v0);
+                const float y1 = snake_row ? v1 + s1 * s1 * inv_a : (v1 < 0.0f ? v1 * 0.01f : v1);
+                if constexpr (decltype(has_copy)::value) {
+                    if (in0) { a.out[i0] = v0; a.act_out[i0] = y0; }
+                    if (in1) { a.out[i1] = v1; a.act_out[i1] = y1; }
+                } else {
+                    if (in0) a.out[i0] = y0;
+                    if (in1) a.out[i1] = y1;
+                }
+            }
+        };
+        if (a.act_out != nullptr) finish(std::true_type{});
+        else finish(std::false_type{});
+        return;
+    }
+    // Some argument needs the library's sine: the wavefront's 32 x 64 tile goes through LDS and a rolled loop finishes it
+    // a row at a time, with one copy of that long routine.
+    float *s_tile = lds + wave * (32 * kTileStride);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int row = 8 * (r >> 2) + 4 * half + (r & 3);
+        s_tile[row * kTileStride + col] = acc0[r];
+        s_tile[row * kTileStride + col + 32] = acc1[r];
+    }
+    const int t = t0 + wn * 64 + lane;
+    if (t >= a.length) return;
+    const int rows = min(32, a.out_ch - (m0 + wm * 32));   // the same for the whole wavefront
+    size_t index = (size_t)(m0 + wm * 32) * a.length + t;
+#pragma unroll 1
+    for (int row = 0; row < rows; ++row, index += a.length)
+        conv_emit(a, m0 + wm * 32 + row, index, s_tile[row * kTileStride + lane], s_alpha[row], s_alpha[32 + row]);
 }
 
 // The same product for short rows (few positions, many channels: the codec's first stages), where 64 x 128 tiles would
@@ -289,6 +441,7 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
         s_part[(wave * 32 + 16 + r) * 64 + lane] = acc1[r];
     }
     __syncthreads();
+    float value[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int e = tid + 256 * j;       // element r of lane l of the tile: e = r * 64 + l
@@ -297,7 +450,37 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
         const int rr = r & 15;
         const int m = m0 + 8 * (rr >> 2) + 4 * (l >> 5) + (rr & 3);
         const int t = t0 + (l & 31) + (r >= 16 ? 32 : 0);
-        if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length) a.out[(size_t)m * a.length + t] = sum + (a.bias != nullptr ? a.bias[m] : 0.0f);
+        value[j] = 0.0f;
+        if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length)
+            value[j] = conv_combine(a, (size_t)m * a.length + t, sum + (a.bias != nullptr ? a.bias[m] : 0.0f));
+    }
+    if (!a.activate) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int e = tid + 256 * j, r = e >> 6, l = e & 63, rr = r & 15;
+            const int m = m0 + 8 * (rr >> 2) + 4 * (l >> 5) + (rr & 3);
+            const int t = t0 + (l & 31) + (r >= 16 ? 32 : 0);
+            if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length) a.out[(size_t)m * a.length + t] = value[j];
+        }
+        return;
+    }
+    // with an activation: the values go back through LDS (a thread reads what it wrote) so that one copy of the
+    // activation's code serves the eight of them
+    float *s_alpha = lds + 4 * 32 * 64;   // [32] alpha, [32] 1 / (alpha + 1e-9) of the tile's rows
+    if (tid < 32) {
+        const float al = m0 + tid < a.snake_channels ? a.alpha[m0 + tid] : 0.0f;
+        s_alpha[tid] = al;
+        s_alpha[32 + tid] = 1.0f / (al + 1e-9f);
+    }
+    __syncthreads();   // every sum has been read
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s_part[tid + 256 * j] = value[j];
+#pragma unroll 2
+    for (int j = 0; j < 8; ++j) {
+        const int e = tid + 256 * j, r = e >> 6, l = e & 63, rr = r & 15;
+        const int row = 8 * (rr >> 2) + 4 * (l >> 5) + (rr & 3), m = m0 + row;
+        const int t = t0 + (l & 31) + (r >= 16 ? 32 : 0);
+        if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length) conv_emit(a, m, (size_t)m * a.length + t, s_part[e], s_alpha[row], s_alpha[32 + row]);
     }
 }
 
@@ -327,35 +510,38 @@ __global__ void __launch_bounds__(256) k_conv_transpose(const ConvTransposeArgs 
     a.out[index] = value;
 }
 
-__global__ void __launch_bounds__(256) k_snake(float *data, const float *alpha, size_t count, int length, int snake_channels) {
+__global__ void __launch_bounds__(256) k_snake(const float *in, float *out, const float *alpha, size_t count, int length, int snake_channels) {
     const size_t index = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (index >= count) return;
     const int channel = (int)(index / (size_t)length);
-    const float v = data[index];
-    if (channel < snake_channels) {
-        const float al = alpha[channel];
-        const float inv_a = 1.0f / (al + 1e-9f);
-        const float sn = sinf(al * v);
-        data[index] = v + sn * sn * inv_a;
-    } else if (v < 0.0f) {
-        data[index] = v * 0.01f;
+    const bool snake_row = channel < snake_channels;
+    const float al = snake_row ? alpha[channel] : 0.0f;
+    const float v = in[index];
+    if (in == out && !snake_row && !(v < 0.0f)) return;   // in place, a leaky row's value that stays as it is: no store
+    out[index] = half_snake(v, snake_row, al, 1.0f / (al + 1e-9f));
+}
+
+template <int WM, int WN, int KF, int VEC, bool FUSED>
+int launch_conv_f(State *st, const ConvArgs &a, char *error, size_t capacity) {
+    constexpr int TM = 32 * WM, TN = 64 * WN;
+    const int kb = kConvChannels * a.kernel;
+    // two more staged rows than are filled: the product loop requests the operands after its last product before it stops
+    size_t lds = ((size_t)TM * (VEC ? kb + 4 : (kb | 1)) + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
+    if (lds < (4 * 32 * kTileStride + 4 * 64) * sizeof(float)) lds = (4 * 32 * kTileStride + 4 * 64) * sizeof(float);   // the fused epilogue's tiles and alphas
+    static bool raised = false;   // per instantiation
+    if (lds > 48 * 1024 && !raised) {
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF, VEC, FUSED>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        raised = true;
     }
+    const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM));
+    hipLaunchKernelGGL((k_conv1d<WM, WN, KF, VEC, FUSED>), grid, dim3(256), lds, st->stream, a);
+    return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
 }
 
 template <int WM, int WN, int KF, int VEC>
 int launch_conv_v(State *st, const ConvArgs &a, char *error, size_t capacity) {
-    constexpr int TM = 32 * WM, TN = 64 * WN;
-    const int kb = kConvChannels * a.kernel;
-    // two more staged rows than are filled: the product loop requests the operands after its last product before it stops
-    const size_t lds = ((size_t)TM * (VEC ? kb + 4 : (kb | 1)) + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
-    static bool raised = false;   // per instantiation
-    if (lds > 48 * 1024 && !raised) {
-        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF, VEC>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
-        raised = true;
-    }
-    const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM));
-    hipLaunchKernelGGL((k_conv1d<WM, WN, KF, VEC>), grid, dim3(256), lds, st->stream, a);
-    return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
+    if (a.residual != nullptr || a.residual2 != nullptr || a.scaled || a.activate) return launch_conv_f<WM, WN, KF, VEC, true>(st, a, error, capacity);
+    return launch_conv_f<WM, WN, KF, VEC, false>(st, a, error, capacity);
 }
 
 template <int WM, int WN, int KF>
@@ -379,7 +565,7 @@ int launch_conv_split_k(State *st, const ConvArgs &a, char *error, size_t capaci
     const int kb = kConvChannels * a.kernel;
     const size_t per_wave = (size_t)32 * (kb + 4) + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
     size_t lds = (4 * per_wave + 2 * (32 * NT + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);   // see launch_conv about the two extra rows
-    if (lds < 4 * 32 * 64 * sizeof(float)) lds = 4 * 32 * 64 * sizeof(float);   // the partial tiles
+    if (lds < (4 * 32 * 64 + 64) * sizeof(float)) lds = (4 * 32 * 64 + 64) * sizeof(float);   // the partial tiles, and the rows' alphas behind them
     static bool raised = false;
     if (!raised) {
         MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d_split<KF, NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
@@ -408,8 +594,9 @@ int launch_conv_split(State *st, const ConvArgs &a, char *error, size_t capacity
 
 }  // namespace
 
-extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
-                                int kernel, int dilation, const float *weight, const float *bias, char *error, size_t capacity) {
+static int conv1d_entry(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                        int kernel, int dilation, const float *weight, const float *bias, const mynah_hip_conv1d_extra *extra,
+                        char *error, size_t capacity) {
     State *st = enter_state(state);
     if (st == nullptr || dev_input == nullptr || dev_output == nullptr || weight == nullptr || in_channels <= 0 || out_channels <= 0 ||
         length <= 0 || kernel <= 0 || dilation <= 0) {
@@ -430,6 +617,23 @@ extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_
     const float *dev_bias = nullptr;
     if (cached_vector(st, bias, (size_t)out_channels, &dev_bias, error, capacity) != 0) return -1;
     ConvArgs a{dev_input, dev_output, static_cast<const float *>(cw->data), dev_bias, in_channels, out_channels, length, kernel, dilation};
+    if (extra != nullptr) {
+        if (extra->snake_channels > (size_t)out_channels || (extra->snake_channels != 0 && extra->snake_alpha == nullptr) ||
+            (extra->dev_activated != nullptr && !extra->activate) || extra->dev_activated == dev_output || dev_input == dev_output ||
+            (extra->dev_residual2 != nullptr && extra->dev_residual == nullptr) || !(extra->scale == extra->scale) ||
+            extra->dev_activated == dev_input) {
+            set_error(error, capacity, "conv1d_fused: invalid activation or residual arguments, or the input is also an output");
+            return -1;
+        }
+        a.residual = extra->dev_residual;
+        a.residual2 = extra->dev_residual2;
+        a.scaled = extra->scale != 1.0f;
+        a.scale = extra->scale;
+        a.activate = extra->activate != 0;
+        a.snake_channels = (int)extra->snake_channels;
+        a.act_out = extra->dev_activated;
+        if (a.activate && a.snake_channels != 0 && cached_vector(st, extra->snake_alpha, extra->snake_channels, &a.alpha, error, capacity) != 0) return -1;
+    }
     // few output channels: one row of wavefronts, wider in time; too few large tiles to fill the chip (and enough input
     // channels to share out): small tiles with the channels split over the wavefronts
     const long tiles = out_channels <= 32 ? (long)((length + 255) / 256) : (long)((out_channels + 63) / 64) * ((length + 127) / 128);
@@ -438,6 +642,21 @@ extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_
         return launch_conv_split(st, a, error, capacity);
     if (out_channels <= 32) return launch_conv<1, 4>(st, a, error, capacity);
     return launch_conv<2, 2>(st, a, error, capacity);
+}
+
+extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                                int kernel, int dilation, const float *weight, const float *bias, char *error, size_t capacity) {
+    return conv1d_entry(state, dev_input, dev_output, in_channels, out_channels, length, kernel, dilation, weight, bias, nullptr, error, capacity);
+}
+
+extern "C" int mynah_hip_conv1d_fused(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                                      int kernel, int dilation, const float *weight, const float *bias, const mynah_hip_conv1d_extra *extra,
+                                      char *error, size_t capacity) {
+    if (extra == nullptr) {
+        set_error(error, capacity, "conv1d_fused: null extra");
+        return -1;
+    }
+    return conv1d_entry(state, dev_input, dev_output, in_channels, out_channels, length, kernel, dilation, weight, bias, extra, error, capacity);
 }
 
 extern "C" int mynah_hip_conv_transpose_dev(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels,
@@ -470,11 +689,11 @@ extern "C" int mynah_hip_conv_transpose_dev(void *state, const float *dev_input,
     return hip_check(hipGetLastError(), "conv_transpose launch", error, capacity);
 }
 
-extern "C" int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length, size_t snake_channels,
-                                   char *error, size_t capacity) {
+static int snake_entry(void *state, const float *dev_input, float *dev_output, const float *alpha, size_t channels, size_t length,
+                       size_t snake_channels, char *error, size_t capacity) {
     State *st = enter_state(state);
-    if (st == nullptr || dev_data == nullptr || channels > (size_t)INT_MAX || length > (size_t)INT_MAX || snake_channels > channels ||
-        (snake_channels != 0 && alpha == nullptr)) {
+    if (st == nullptr || dev_input == nullptr || dev_output == nullptr || channels > (size_t)INT_MAX || length > (size_t)INT_MAX ||
+        snake_channels > channels || (snake_channels != 0 && alpha == nullptr)) {
         set_error(error, capacity, "invalid snake arguments");   // metal_ops_snake, gpu/metal/backend_metal_ops.m:343-346
         return -1;
     }
@@ -486,7 +705,17 @@ extern "C" int mynah_hip_snake_dev(void *state, float *dev_data, const float *al
     }
     const float *dev_alpha = nullptr;
     if (snake_channels != 0 && cached_vector(st, alpha, snake_channels, &dev_alpha, error, capacity) != 0) return -1;
-    hipLaunchKernelGGL(k_snake, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st->stream, dev_data, dev_alpha, count, (int)length,
-                       (int)snake_channels);
+    hipLaunchKernelGGL(k_snake, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st->stream, dev_input, dev_output, dev_alpha, count,
+                       (int)length, (int)snake_channels);
     return hip_check(hipGetLastError(), "snake launch", error, capacity);
+}
+
+extern "C" int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length, size_t snake_channels,
+                                   char *error, size_t capacity) {
+    return snake_entry(state, dev_data, dev_data, alpha, channels, length, snake_channels, error, capacity);
+}
+
+extern "C" int mynah_hip_snake_copy_dev(void *state, const float *dev_input, float *dev_output, const float *alpha, size_t channels,
+                                        size_t length, size_t snake_channels, char *error, size_t capacity) {
+    return snake_entry(state, dev_input, dev_output, alpha, channels, length, snake_channels, error, capacity);
 }

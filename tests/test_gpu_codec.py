@@ -110,6 +110,92 @@ def test_res_block_chain(backend, orc, nerr):
         d.free()
 
 
+def _res_layer_inputs(C, L, seed):
+    rng = np.random.default_rng(seed)
+    alpha = lambda: (np.abs(rng.standard_normal(C // 2)) + 0.1).astype(np.float32)
+    conv = lambda k: ((rng.standard_normal((C, C, k)) / np.sqrt(C * k)).astype(np.float32), rng.standard_normal(C).astype(np.float32) * np.float32(0.1))
+    blocks = [[(alpha(), conv(k), alpha(), conv(k), d) for d in (1, 3, 5)] for k in (3, 7, 11)]
+    return rng.standard_normal((C, L)).astype(np.float32), blocks
+
+
+# channels x length: the 64 x 128 tiles, the channel-split small tiles in both widths, at most 32 output channels, ragged edges
+@pytest.mark.parametrize("C,L", [(108, 1000), (432, 96), (216, 300), (54, 700), (28, 1300), (70, 33)])
+def test_fused_res_layer_is_the_operator_sequence(pkg, backend, orc, nerr, C, L):
+    """The residual layer from fused calls (conv1d_fused, snake_copy_dev) against the same layer from the seam's operators
+    in res_layer_device's order (src/graph.c:2423-2498): every value bit for bit.  And, for one shape, both against the oracle."""
+    import importlib
+    codec = importlib.import_module(pkg.__name__ + ".codec")
+    _announce("fused residual layer %d x %d" % (C, L))
+    x, blocks = _res_layer_inputs(C, L, 20 + C)
+    n = C * L
+    din = backend.alloc(n).write(x)
+    bufs = [backend.alloc(n) for _ in range(8)]
+    out_a, out_b = bufs[0], bufs[1]
+    codec.res_layer(backend, blocks, din.ptr, out_a.ptr, C, L, *(b.ptr for b in bufs[2:6]))
+    codec.res_layer_fused(backend, blocks, din.ptr, out_b.ptr, C, L, *(b.ptr for b in bufs[5:8]))
+    seq, fused = out_a.read().reshape(C, L), out_b.read().reshape(C, L)
+    assert np.isfinite(seq).all()
+    assert np.array_equal(seq.view(np.uint32), fused.view(np.uint32))
+    assert np.array_equal(din.read().reshape(C, L), x), "the layer's input was written"
+    if C == 70:
+        total = np.zeros_like(x)
+        for branch in blocks:
+            cur = x.copy()
+            for a_in, (w_in, b_in), a_skip, (w_skip, b_skip), d in branch:
+                cur = cur + orc.conv1d_causal(orc.snake(orc.conv1d_causal(orc.snake(cur, a_in, C // 2), w_in, b_in, d), a_skip, C // 2), w_skip, b_skip, 1)
+            total += cur
+        assert nerr(fused, total * np.float32(1.0 / 3.0)) < 1e-5
+    for d in bufs + [din]:
+        d.free()
+
+
+def test_fused_conv_pieces(backend, orc, nerr):
+    """Each optional step of conv1d_fused alone against the operator it stands for, bit for bit."""
+    _announce("conv1d_fused steps")
+    rng = np.random.default_rng(31)
+    C, O, L, K, D = 40, 72, 210, 7, 3
+    x = rng.standard_normal((C, L)).astype(np.float32)
+    w = (rng.standard_normal((O, C, K)) / np.sqrt(C * K)).astype(np.float32)
+    b = rng.standard_normal(O).astype(np.float32)
+    r1, r2 = rng.standard_normal((2, O, L)).astype(np.float32)
+    alpha = (np.abs(rng.standard_normal(O // 2)) + 0.1).astype(np.float32)
+    din, dr1, dr2 = backend.alloc(x.size).write(x), backend.alloc(r1.size).write(r1), backend.alloc(r2.size).write(r2)
+    plain, got, act = backend.alloc(O * L), backend.alloc(O * L), backend.alloc(O * L)
+    bits = lambda d: d.read().view(np.uint32)
+
+    backend.conv1d(din.ptr, plain.ptr, C, O, L, K, D, w, b)
+    backend.conv1d_fused(din.ptr, got.ptr, C, O, L, K, D, w, b)                       # nothing added: the plain operator
+    assert np.array_equal(bits(got), bits(plain))
+
+    backend.conv1d_fused(din.ptr, got.ptr, C, O, L, K, D, w, b, residual=dr1.ptr, residual2=dr2.ptr, scale=0.25)
+    backend.residual_inplace(dr1.ptr, plain.ptr, O * L)                                # dr1 += conv
+    backend.residual_inplace(dr2.ptr, dr1.ptr, O * L)                                  # dr2 += that
+    backend.scale_dev(dr2.ptr, O * L, 0.25)
+    assert np.array_equal(bits(got), bits(dr2))
+
+    backend.conv1d_fused(din.ptr, got.ptr, C, O, L, K, D, w, b, alpha=alpha, snake_channels=O // 2, activated=act.ptr)
+    assert np.array_equal(bits(got), bits(plain)), "the plain value must stay beside the activated one"
+    backend.snake_dev(plain.ptr, alpha, O, L, O // 2)
+    assert np.array_equal(bits(act), bits(plain))
+    backend.conv1d_fused(din.ptr, got.ptr, C, O, L, K, D, w, b, alpha=alpha, snake_channels=O // 2)
+    assert np.array_equal(bits(got), bits(plain))
+
+    # sine arguments beyond the short routine's range take the epilogue's other path (and the library's sine in both kernels)
+    big = (alpha * np.float32(3.0e4)).astype(np.float32)
+    backend.conv1d(din.ptr, plain.ptr, C, O, L, K, D, w, b)
+    backend.snake_dev(plain.ptr, big, O, L, O // 2)
+    backend.conv1d_fused(din.ptr, got.ptr, C, O, L, K, D, w, b, alpha=big, snake_channels=O // 2)
+    assert np.array_equal(bits(got), bits(plain))
+    conv = _run_conv1d(backend, x, w, b, D)
+    assert nerr(got.read().reshape(O, L), orc.snake(conv, big, O // 2)) < 1e-6
+
+    backend.snake_copy_dev(din.ptr, got.ptr, alpha[:C // 2], C, L, C // 2)
+    assert nerr(got.read(x.size).reshape(C, L), orc.snake(x, alpha[:C // 2], C // 2)) < 1e-6
+    assert np.array_equal(din.read().reshape(C, L), x)
+    for d in (din, dr1, dr2, plain, got, act):
+        d.free()
+
+
 def test_error_paths(pkg, backend):
     _announce("codec error paths")
     d = backend.alloc(64)
@@ -122,4 +208,11 @@ def test_error_paths(pkg, backend):
         backend.conv_transpose_dev(d.ptr, d.ptr, 3, 2, 4, 8, 4, 2, 2, w)
     with pytest.raises(pkg.BackendError, match="invalid snake arguments"):
         backend.snake_dev(d.ptr, np.ones(4, np.float32), 2, 8, 3)
+    e = backend.alloc(64)
+    w3 = np.zeros((1, 1, 3), np.float32)
+    with pytest.raises(pkg.BackendError, match="conv1d_fused"):      # the activated copy may not be the output itself
+        backend.conv1d_fused(d.ptr, e.ptr, 1, 1, 8, 3, 1, w3, alpha=np.ones(1, np.float32), snake_channels=1, activated=e.ptr)
+    with pytest.raises(pkg.BackendError, match="conv1d_fused"):      # more snake channels than output channels
+        backend.conv1d_fused(d.ptr, e.ptr, 1, 1, 8, 3, 1, w3, alpha=np.ones(2, np.float32), snake_channels=2)
+    e.free()
     d.free()
