@@ -140,17 +140,19 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
         }
         // Epilogue operands.  One stream: lane 0 of a group finishes the row.  Several streams: lane b of a group
         // finishes stream b (when the group has that many lanes), so the epilogues of a row run side by side.
+        // Requested by every lane, whichever of them finishes the row: a request under a per-lane condition cannot be
+        // counted by the waits that follow, and the prologue's wait for the activation rows then also waited for the
+        // first weight pieces.  (Lanes of a group ask for the same address; the conditions left are the same for the
+        // whole launch.)
         if (lanes_finish) {
-            if (gl < BT) {
-                if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
-                if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
-                if (arg_epilogue == EPI_RESIDUAL && gl < a.batch) pre_res[0] = stream_out<BT>(a, gl)[rowc];
-            }
-        } else if (gl == 0) {
+            if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
+            if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
+            if (arg_epilogue == EPI_RESIDUAL) pre_res[0] = stream_out<BT>(a, gl < a.batch ? gl : 0)[rowc];
+        } else {
             if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
             if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
 #pragma unroll
-            for (int b = 0; b < BT; ++b) pre_res[b] = (arg_epilogue == EPI_RESIDUAL && b < a.batch) ? a.out[b][rowc] : 0.0f;
+            for (int b = 0; b < BT; ++b) pre_res[b] = (arg_epilogue == EPI_RESIDUAL && (b == 0 || b < a.batch)) ? a.out[b][rowc] : 0.0f;   // a launch has at least one stream
         }
     }
 
