@@ -119,8 +119,51 @@ __device__ __forceinline__ float block_max(float v, float *s4) {
 
 // mynah_layernorm_f32 (src/kernels.c:186-244): mean, then the variance of (x - mean), eps inside the
 // square root, y = (x - mean) * scale * gain (+ bias).  One workgroup per row.
+// Rows of up to 256 * NV values stay in registers: one round trip for the row, its gain and its bias (requested side by
+// side, none under a condition) instead of three passes over memory with a round trip per 256 values each.  A thread
+// adds its values in the order of the loop below, so the results are the same bits.
+template <int NV>
+__device__ __forceinline__ void layernorm_row_in_registers(const float *x, float *y, const float *gain, const float *bias, int width,
+                                                           float *s4) {
+    float xv[NV], gv[NV], bv[NV];
+    const float *bias_or_gain = bias != nullptr ? bias : gain;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = threadIdx.x + 256 * u, at = i < width ? i : width - 1;
+        xv[u] = x[at];
+        gv[u] = gain[at];
+        bv[u] = bias_or_gain[at];
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+        if ((int)threadIdx.x + 256 * u < width) s += xv[u];
+    const float mean = block_sum(s, s4) / (float)width;
+    float v = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        if ((int)threadIdx.x + 256 * u < width) {
+            const float d = xv[u] - mean;
+            v = __builtin_fmaf(d, d, v);
+        }
+    }
+    const float variance = block_sum(v, s4);
+    const float scale = 1.0f / sqrtf(variance / (float)width + 1.0e-5f);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = threadIdx.x + 256 * u;
+        if (i < width) {
+            float z = ((xv[u] - mean) * scale) * gv[u];
+            if (bias != nullptr) z += bv[u];
+            y[i] = z;
+        }
+    }
+}
+
 __device__ __forceinline__ void layernorm_row(const float *x, float *y, const float *gain, const float *bias, int width,
                                               float *s4) {
+    if (width <= 1024) return layernorm_row_in_registers<4>(x, y, gain, bias, width, s4);
+    if (width <= 4096) return layernorm_row_in_registers<16>(x, y, gain, bias, width, s4);
     float s = 0.0f;
     for (int i = threadIdx.x; i < width; i += 256) s += x[i];
     const float mean = block_sum(s, s4) / (float)width;

@@ -63,10 +63,42 @@ __global__ void __launch_bounds__(256) k_softmax_masked(float *data, int cols, i
 }
 
 // mynah_softmax_f32 (src/kernels.c:391-420) per head: p = expf(x - max) * (1 / total).
+// Rows of up to 256 * NV values stay in registers (one round trip instead of three passes over memory; a thread's
+// values are taken in the same order, so the bits are the same).
+template <int NV>
+__device__ __forceinline__ void softmax_row_in_registers(const float *row, float *prow, int cols, float *s4) {
+    float v[NV];
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = threadIdx.x + 256 * u;
+        v[u] = row[i < cols ? i : cols - 1];
+    }
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+        if ((int)threadIdx.x + 256 * u < cols) mx = fmaxf(mx, v[u]);
+    mx = block_max(mx, s4);
+    float sum = 0.0f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        v[u] = expf(v[u] - mx);
+        if ((int)threadIdx.x + 256 * u < cols) sum += v[u];
+    }
+    sum = block_sum(sum, s4);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const int i = threadIdx.x + 256 * u;
+        if (i < cols) prow[i] = v[u] * inv;
+    }
+}
+
 __global__ void __launch_bounds__(256) k_softmax_heads(const float *logits, float *probs, int cols) {
     __shared__ float s4[4];
     const float *row = logits + (size_t)blockIdx.x * cols;
     float *prow = probs + (size_t)blockIdx.x * cols;
+    if (cols <= 1024) return softmax_row_in_registers<4>(row, prow, cols, s4);
+    if (cols <= 4096) return softmax_row_in_registers<16>(row, prow, cols, s4);
     float mx = -FLT_MAX;
     for (int i = threadIdx.x; i < cols; i += 256) mx = fmaxf(mx, row[i]);
     mx = block_max(mx, s4);
@@ -175,6 +207,22 @@ __global__ void __launch_bounds__(256) k_step_begin(const StepSlots slots, StepS
     if (b == 0 && threadIdx.x == 0) *dev_slots = slots;
     const float *in = slots.input[b];
     const float *pe = position != nullptr ? position + (size_t)slots.length[b] * width : nullptr;
+    if (width <= 1024) {   // one round trip: every request issued before the first sum
+        float iv[4], pv[4];
+        const float *second = pe != nullptr ? pe : in;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int d = threadIdx.x + 256 * u, at = d < width ? d : width - 1;
+            iv[u] = in[at];
+            pv[u] = second[at];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int d = threadIdx.x + 256 * u;
+            if (d < width) x[(size_t)b * x_stride + d] = pe != nullptr ? iv[u] + pv[u] : iv[u];
+        }
+        return;
+    }
     for (int d = threadIdx.x; d < width; d += 256) x[(size_t)b * x_stride + d] = pe != nullptr ? in[d] + pe[d] : in[d];
 }
 
