@@ -66,6 +66,12 @@ template <int QT, int BT, int NVT, int KFIX, int SPEC>
 __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
     constexpr int kTeams = kLinearTeams<BT, QT>;
     constexpr int SB = BT / kTeams;   // streams staged by one team
+    // The kernel arguments that the first requests are formed from, fetched here in one go: left to the compiler each is
+    // fetched where it is first used, with a wait of its own, and three such round trips stood in a row in front of the
+    // first request for an activation row.
+    __asm__ volatile("" ::"s"(a.w), "s"(a.scales), "s"(a.in[0]), "s"(a.out[0]), "s"(a.fold_partial), "s"(a.fold_partial_ml), "s"(a.fold_slots),
+                     "s"(a.ln_gain), "s"(a.ln_bias), "s"(a.n), "s"(a.k), "s"(a.batch), "s"(a.fold_heads), "s"(a.fold_head_width),
+                     "s"(a.fold_max_units), "s"(a.fold_is_self), "s"(a.fold_stream0), "s"(rows_per_wg), "s"(a.arith), "s"(a.epilogue));
     const Team team{(int)(threadIdx.x & (kThreads - 1)), (int)(threadIdx.x / kThreads) * SB};
     const bool worker = kTeams == 1 || threadIdx.x < kThreads;
     // the arguments a specialised build does not look at
