@@ -535,7 +535,7 @@ int ref_codec_engine_decode(ref_codec_engine *e, const unsigned *codes, size_t r
 
 
 /* ---- the integration text, compiled ------------------------------------------------------------------------------
- * oracle/integration_batched.inc is the engine-side code INTEGRATION.md sections 6 and 6b quote.  In the engine its five
+ * oracle/integration_batched.inc is the engine-side code that the repository's integration notes quote.  In the engine its five
  * library calls are linked symbols; here the library is found with dlopen (so that this file still loads where no GPU
  * runtime is installed) and the calls go through pointers of the header's own prototype types.
  * Reference types it is compiled against: decoder_cache / decoder_layer_resolved (src/graph.c:2795-2861), local_cache

@@ -165,7 +165,7 @@ def test_codec_decode_resident(pkg, orc, ref_strict, nerr, quant_env, tmp_path):
 
 @pytest.mark.parametrize("qtype_name", ["f32", "int8", "int4"])
 def test_integration_text_batched_decoder_step(pkg, orc, ref_strict, synth, nerr, quant_env, qtype_name):
-    """The engine-side code INTEGRATION.md section 6 quotes (oracle/integration_batched.inc), compiled against the
+    """The engine-side code that the integration notes quote for the batched step (oracle/integration_batched.inc), compiled against the
     reference's own decoder_cache: eight ragged streams, two consecutive steps through hip_decoder_step_batch on the
     library, against the reference's CPU decoder_step_batch on the same caches and inputs.  The device caches are the
     ones the reference's decoder_gpu_attention_init uploads; lengths advance as the reference's do; the rows the step
@@ -211,7 +211,7 @@ def test_integration_text_batched_decoder_step(pkg, orc, ref_strict, synth, nerr
 
 
 def test_integration_text_local_frame(pkg, orc, ref_strict, synth, quant_env):
-    """The engine-side code INTEGRATION.md section 6b quotes, compiled against the reference's own local_cache and
+    """The engine-side code that the integration notes quote for the local frame, compiled against the reference's own local_cache and
     local_batch_item: one frame of three items (greedy with rng_state == NULL, two sampling items, one of them with EOS
     forbidden) through hip_sample_local_frame_batch on the library, f32 weights, against the oracle's frame: the codes
     land where the reference's loop stores them (src/graph.c:1620-1628: codebook * code_stride + raw_offset + frame),

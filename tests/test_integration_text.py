@@ -1,4 +1,4 @@
-"""INTEGRATION.md quotes the engine-side code of sections 6 and 6b from oracle/integration_batched.inc, the file the
+"""The integration notes quote the engine-side code of the batched step and of the local frame from oracle/integration_batched.inc, the file the
 compiler sees (oracle/ref_shim_graph.c includes it against the reference's own structs).  The quotation must be the file."""
 import os
 
@@ -13,5 +13,5 @@ def test_integration_md_quotes_the_compiled_file():
     marker6, marker6b = "/* ---- section 6: the batched decoder step", "/* ---- section 6b: the local-transformer frame"
     part6 = source[source.index(marker6):source.index(marker6b)].strip()
     part6b = source[source.index(marker6b):].strip()
-    assert part6 in doc, "INTEGRATION.md section 6 no longer quotes oracle/integration_batched.inc"
-    assert part6b in doc, "INTEGRATION.md section 6b no longer quotes oracle/integration_batched.inc"
+    assert part6 in doc, "the integration notes no longer quote the batched-step part of oracle/integration_batched.inc"
+    assert part6b in doc, "the integration notes no longer quote the local-frame part of oracle/integration_batched.inc"
