@@ -69,9 +69,19 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
     // The kernel arguments that the first requests are formed from, fetched here in one go: left to the compiler each is
     // fetched where it is first used, with a wait of its own, and three such round trips stood in a row in front of the
     // first request for an activation row.
-    __asm__ volatile("" ::"s"(a.w), "s"(a.scales), "s"(a.in[0]), "s"(a.out[0]), "s"(a.fold_partial), "s"(a.fold_partial_ml), "s"(a.fold_slots),
-                     "s"(a.ln_gain), "s"(a.ln_bias), "s"(a.n), "s"(a.k), "s"(a.batch), "s"(a.fold_heads), "s"(a.fold_head_width),
-                     "s"(a.fold_max_units), "s"(a.fold_is_self), "s"(a.fold_stream0), "s"(rows_per_wg), "s"(a.arith), "s"(a.epilogue));
+    // (One or two streams: only what the first requests are formed from -- fetching every argument first delays them.
+    // More streams: the eight row pointers of a.in and a.out as one operand each, or they are fetched in rounds of their own.)
+    if constexpr (BT <= 2) {
+        __asm__ volatile("" ::"s"(a.w), "s"(a.scales), "s"(a.in[0]), "s"(a.out[0]), "s"(a.fold_partial), "s"(a.fold_partial_ml), "s"(a.fold_slots),
+                         "s"(a.ln_gain), "s"(a.ln_bias), "s"(a.n), "s"(a.k), "s"(a.batch), "s"(a.fold_heads), "s"(a.fold_head_width),
+                         "s"(a.fold_max_units), "s"(a.fold_is_self), "s"(a.fold_stream0), "s"(rows_per_wg), "s"(a.arith), "s"(a.epilogue));
+    } else {
+        typedef unsigned row_pointers __attribute__((ext_vector_type(2 * BT)));
+        const row_pointers ins = *reinterpret_cast<const row_pointers *>(&a.in[0]), outs = *reinterpret_cast<const row_pointers *>(&a.out[0]);
+        __asm__ volatile("" ::"s"(a.w), "s"(a.scales), "s"(ins), "s"(outs), "s"(a.fold_partial), "s"(a.fold_partial_ml), "s"(a.fold_slots),
+                         "s"(a.ln_gain), "s"(a.ln_bias), "s"(a.n), "s"(a.k), "s"(a.batch), "s"(a.fold_heads), "s"(a.fold_head_width),
+                         "s"(a.fold_max_units), "s"(a.fold_is_self), "s"(a.fold_stream0), "s"(rows_per_wg), "s"(a.arith), "s"(a.epilogue));
+    }
     const Team team{(int)(threadIdx.x & (kThreads - 1)), (int)(threadIdx.x / kThreads) * SB};
     const bool worker = kTeams == 1 || threadIdx.x < kThreads;
     // the arguments a specialised build does not look at
