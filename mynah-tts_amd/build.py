@@ -21,6 +21,7 @@ FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC",
     "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",   # leading scalar kernel arguments arrive in registers (no fetch at kernel start)
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
 ]
 

@@ -63,7 +63,20 @@ template <int BT, int QT>
 constexpr int kLinearTeams = !(BT > kConsumerFoldMaxBatch && kQuantised<QT>) ? 1 : (QT == MYNAH_HIP_INT4 && BT == 8) ? 2 : 4;
 
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
-__global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(const LinearArgs a, const int rows_per_wg, const int lg_arg) {
+__global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>))
+k_linear(const float *const in0, const float *const fold_partial, const float *const fold_partial_ml, const StepSlots *const fold_slots,
+         const void *const w, const float *const scales, float *const out0, const int n, const int batch, const LinearArgs a_arg,
+         const int rows_per_wg, const int lg_arg) {
+    // The seven pointers and two counts in front repeat fields of a_arg: the first sixteen dwords of the kernel arguments are
+    // in registers when a wavefront starts (the build asks for that), the structure behind them is fetched from memory, and
+    // these are what the first requests are formed from.
+    // (Only for one or two streams: with more, the rows of a.in and a.out are picked by a run-time index, and a structure that
+    // has been written to is then kept in scratch memory -- the eight-stream matvecs took 20 us instead of 4.5.)
+    LinearArgs a = a_arg;
+    if constexpr (BT <= 2) {
+        a.in[0] = in0; a.fold_partial = fold_partial; a.fold_partial_ml = fold_partial_ml; a.fold_slots = fold_slots;
+        a.w = w; a.scales = scales; a.out[0] = out0; a.n = n; a.batch = batch;
+    }
     constexpr int kTeams = kLinearTeams<BT, QT>;
     constexpr int SB = BT / kTeams;   // streams staged by one team
     // The kernel arguments that the first requests are formed from, fetched here in one go: left to the compiler each is
@@ -71,11 +84,7 @@ __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>)) k_linear(co
     // first request for an activation row.
     // (One or two streams: only what the first requests are formed from -- fetching every argument first delays them.
     // More streams: the eight row pointers of a.in and a.out as one operand each, or they are fetched in rounds of their own.)
-    if constexpr (BT <= 2) {
-        __asm__ volatile("" ::"s"(a.w), "s"(a.scales), "s"(a.in[0]), "s"(a.out[0]), "s"(a.fold_partial), "s"(a.fold_partial_ml), "s"(a.fold_slots),
-                         "s"(a.ln_gain), "s"(a.ln_bias), "s"(a.n), "s"(a.k), "s"(a.batch), "s"(a.fold_heads), "s"(a.fold_head_width),
-                         "s"(a.fold_max_units), "s"(a.fold_is_self), "s"(a.fold_stream0), "s"(rows_per_wg), "s"(a.arith), "s"(a.epilogue));
-    } else {
+    if constexpr (BT > 2) {
         typedef unsigned row_pointers __attribute__((ext_vector_type(2 * BT)));
         const row_pointers ins = *reinterpret_cast<const row_pointers *>(&a.in[0]), outs = *reinterpret_cast<const row_pointers *>(&a.out[0]);
         __asm__ volatile("" ::"s"(a.w), "s"(a.scales), "s"(ins), "s"(outs), "s"(a.fold_partial), "s"(a.fold_partial_ml), "s"(a.fold_slots),
@@ -429,7 +438,8 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, a, rows_per_wg, lg);
+    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, a.in[0], a.fold_partial,
+                       a.fold_partial_ml, a.fold_slots, a.w, a.scales, a.out[0], a.n, a.batch, a, rows_per_wg, lg);
     return hip_check(hipGetLastError(), "linear launch", error, capacity);
 }
 
