@@ -74,7 +74,10 @@ constexpr int kFoldUnit = 0x7fff;   // unit number of a table entry that folds i
 // short streams do not have; here the workgroups are numbered over the units that exist, so those with nothing to do
 // are the last ones of the grid and leave after one read instead of holding places among the working ones).
 template <int QT, int NVT, int PF, int WFIX, int SELF, int PACKED>
-__global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs a_arg, const int lg_arg, const int per_xcd_arg) {
+__global__ void __launch_bounds__(kThreads)
+k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, const void *const w_arg, const float *const scales_arg,
+                 const float *const ln_gain_arg, const float *const ln_bias_arg, const StepItem *const items_arg, const int per_xcd_arg,
+                 const int lg_arg, const StepAttnArgs a_arg) {
     extern __shared__ __align__(16) unsigned char smem[];   // staged activations: width bytes (int8/int4) or floats
     __shared__ __align__(16) float s_proj[3 * kHw];         // q | k | v of this head
     // CP: consecutive cache chunks of a stream per chunk workgroup; the code below is written for any CP.  With CP chunks one
@@ -91,7 +94,10 @@ __global__ void __launch_bounds__(kThreads) k_step_attention(const StepAttnArgs 
 
     constexpr int kEpc = Chunk<QT>::n;
     const int lg = WFIX != 0 ? lane_group_log2(WFIX / kEpc) : lg_arg;
+    // The seven pointers and two counts in front repeat fields of a_arg: the first sixteen dwords of the kernel arguments are
+    // in registers when a wavefront starts (the build asks for that); the structure behind them is fetched from memory.
     StepAttnArgs a = a_arg;
+    a.slots = slots_arg; a.x = x_arg; a.w = w_arg; a.scales = scales_arg; a.ln_gain = ln_gain_arg; a.ln_bias = ln_bias_arg; a.items = items_arg;
     if constexpr (WFIX != 0) a.width = WFIX;
     const bool is_self = SELF >= 0 ? SELF == 1 : a.is_self != 0;
     const int tid = threadIdx.x;
@@ -539,7 +545,8 @@ __global__ void __launch_bounds__(kThreads) k_step_fold(const float *partial, co
     reinterpret_cast<float4 *>(out + (size_t)stream * heads * kHw)[f4] = fold_partials(src, stream, f4);
 }
 
-using StepAttnKernel = void (*)(const StepAttnArgs, const int, const int);
+using StepAttnKernel = void (*)(const StepSlots *, const float *, const void *, const float *, const float *, const float *, const StepItem *, const int,
+                                const int, const StepAttnArgs);
 
 // The build that runs a shape: fixed-width builds for the decoder stack's width; `latency`: the build for one or two
 // streams (work found from the workgroup index; it also serves more streams when the launch cannot fold its own partials),
@@ -580,7 +587,8 @@ int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const int per_xcd = grid / 8;
     const bool packed = a.records != nullptr;
     const size_t lds = lds_for<QT>(a.width, a.max_units, packed);
-    hipLaunchKernelGGL(kernel_for<QT>(a.width, a.is_self != 0, !packed), dim3(grid), dim3(kThreads), lds, st->stream, a, lg, per_xcd);
+    hipLaunchKernelGGL(kernel_for<QT>(a.width, a.is_self != 0, !packed), dim3(grid), dim3(kThreads), lds, st->stream, a.slots, a.x, a.w, a.scales, a.ln_gain,
+                       a.ln_bias, a.items, per_xcd, lg, a);
     return hip_check(hipGetLastError(), "step attention launch", error, capacity);
 }
 
