@@ -140,8 +140,16 @@ struct StepFragments {
 // younger one as well: with `if (kt + D < nk)` around the requests the pipeline was one step deep whatever D said.
 // Without EXACT (an odd number of steps) the guarded form is used, with that cost.
 // CONV: the A operand of K step s is the 64 channels (s % (cin / 64)) * 64 .. of row m - (taps - 1) + s / (cin / 64).
+// The fields of GemmArgs as scalar arguments, in the order in which the kernel needs them: the first sixteen dwords of
+// scalar kernel arguments are in registers when a wavefront starts (the build asks for that), a structure passed by value
+// is fetched from memory.
 template <int EPI, int D, bool EXACT, bool CONV>
-__global__ void __launch_bounds__(kThreads) k_enc_gemm(const GemmArgs g) {
+__global__ void __launch_bounds__(kThreads)
+k_enc_gemm(const _Float16 *const a_arg, const _Float16 *const w_arg, const int M, const int N, const int K, const int taps, const int cin,
+           float *const part, _Float16 *const out, _Float16 *const vt, const int width, const int vt_stride) {
+    GemmArgs g;
+    g.a = a_arg; g.w = w_arg; g.M = M; g.N = N; g.K = K; g.part = part; g.out = out; g.vt = vt; g.width = width; g.vt_stride = vt_stride;
+    g.taps = taps; g.cin = cin;
     static_assert(D >= 2 && D % 2 == 0, "stage parity must equal step parity");
     __shared__ __align__(16) _Float16 s_a[2][kTile * kLdsStride];
     __shared__ __align__(16) _Float16 s_w[2][kTile * kLdsStride];
@@ -512,9 +520,15 @@ int launch_gemm(State *st, const GemmArgs &g, int splits, char *error, size_t ca
     }
     const int steps = g.K / kTile / splits;
     const dim3 grid(g.N / kTile, g.M / kTile, splits), block(kThreads);
-    if (steps % kGemmDepth == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true, CONV>), grid, block, 0, st->stream, g);
-    else if (steps % 2 == 0) hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true, CONV>), grid, block, 0, st->stream, g);
-    else hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false, CONV>), grid, block, 0, st->stream, g);
+    if (steps % kGemmDepth == 0)
+        hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt,
+                           g.width, g.vt_stride);
+    else if (steps % 2 == 0)
+        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width,
+                           g.vt_stride);
+    else
+        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width,
+                           g.vt_stride);
     return hip_check(hipGetLastError(), "encoder product launch", error, capacity);
 }
 
