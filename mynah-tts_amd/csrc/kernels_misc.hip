@@ -201,8 +201,9 @@ __global__ void __launch_bounds__(256) k_gather(GatherTables tables, int table_c
 }
 
 // Decode-step begin: record the slot table, x[b] = input[b] + position[length[b]] (src/graph.c:3156-3157).
-__global__ void __launch_bounds__(256) k_step_begin(const StepSlots slots, StepSlots *dev_slots, int width, const float *position,
-                                                    float *x, size_t x_stride) {
+// (The scalar arguments stand in front of the table: leading scalars are in registers when a wavefront starts.)
+__global__ void __launch_bounds__(256) k_step_begin(StepSlots *dev_slots, int width, const float *position, float *x, size_t x_stride,
+                                                    const StepSlots slots) {
     const int b = blockIdx.x;
     if (b == 0 && threadIdx.x == 0) *dev_slots = slots;
     const float *in = slots.input[b];
@@ -322,8 +323,8 @@ int launch_gather(State *st, const float *const *dev_tables, size_t table_count,
 }
 int launch_step_begin(State *st, const StepSlots &slots, StepSlots *dev_slots, int batch, size_t width,
                       const float *dev_position, float *x, size_t x_stride, char *error, size_t capacity) {
-    hipLaunchKernelGGL(k_step_begin, dim3((unsigned)batch), dim3(256), 0, st->stream, slots, dev_slots, (int)width, dev_position, x,
-                       x_stride);
+    hipLaunchKernelGGL(k_step_begin, dim3((unsigned)batch), dim3(256), 0, st->stream, dev_slots, (int)width, dev_position, x, x_stride,
+                       slots);
     return hip_check(hipGetLastError(), "step begin launch", error, capacity);
 }
 int launch_step_end(State *st, const StepSlots *dev_slots, int batch, size_t width, const float *x, size_t x_stride,
