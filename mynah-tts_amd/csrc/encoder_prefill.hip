@@ -16,8 +16,13 @@
 // masked out as attention keys, so they never reach a real row):
 //   x    f32 [Tpad, w]       residual stream
 //   nrm  f16 [2 + Tpad, w]   LayerNorm output = A operand of the QKV / FFN-up products (after two zero rows)
-//   qk   f16 [Tpad, 2w]      q | k of every token, row-major (K-contiguous operands of QK^T)
-//   vt   f16 [w, TpadMax]    v transposed: vt[h*64+d][t], so PV's B operand is K(=t)-contiguous too
+//   qk   f16 [2, heads, Tpad/32][2048]   q, then k, operand-major: per (head, 32-token tile) the 32 x 64 block in the order in
+//                            which a wavefront's four matrix instructions take it -- element (token r of the tile, d) at
+//                            ((d / 16) * 64 + ((d % 16) / 8) * 32 + r) * 8 + d % 8 -- so that one operand request of
+//                            the attention kernel is 1 KiB of consecutive bytes (read row-major, lane l: 16 bytes of row
+//                            l % 32, a request touches 32 cache lines for 32 bytes each)
+//   vt   f16 [heads*2, Tpad/16][512]     v, operand-major for PV (rows = 32 output columns, inner index = 16 keys): element
+//                            (d, t) at block (d / 32, t / 16), ((t % 16) / 8 * 32 + d % 32) * 8 + t % 8
 //   ctx  f16 [Tpad, w]       attention output = A operand of the O product
 //   hid  f16 [2 + Tpad, ffn] GELU(up) = A operand of the FFN-down product (after two zero rows)
 //   part f32 [4, Tpad, w]    K-split partial sums of the O and FFN-down products; the row pass that follows
@@ -83,8 +88,8 @@ struct GemmArgs {
     int M, N, K;
     float *part;           // ENC_PARTIAL: part[z][m][n] = this K split's share of the product (summed by the next LayerNorm pass)
     _Float16 *out;         // ENC_QKV: qk [M, 2*width];  ENC_GELU: hid [M, N]
-    _Float16 *vt;          // ENC_QKV: v transposed [width, vt_stride]
-    int width, vt_stride;
+    _Float16 *vt;          // ENC_QKV: v, operand-major (see the layout note)
+    int width;
     int taps, cin;         // conv form: K = taps * cin, A is [M, cin] with (taps - 1) zero rows before row 0
 };
 
@@ -146,9 +151,9 @@ struct StepFragments {
 template <int EPI, int D, bool EXACT, bool CONV>
 __global__ void __launch_bounds__(kThreads)
 k_enc_gemm(const _Float16 *const a_arg, const _Float16 *const w_arg, const int M, const int N, const int K, const int taps, const int cin,
-           float *const part, _Float16 *const out, _Float16 *const vt, const int width, const int vt_stride) {
+           float *const part, _Float16 *const out, _Float16 *const vt, const int width) {
     GemmArgs g;
-    g.a = a_arg; g.w = w_arg; g.M = M; g.N = N; g.K = K; g.part = part; g.out = out; g.vt = vt; g.width = width; g.vt_stride = vt_stride;
+    g.a = a_arg; g.w = w_arg; g.M = M; g.N = N; g.K = K; g.part = part; g.out = out; g.vt = vt; g.width = width;
     g.taps = taps; g.cin = cin;
     static_assert(D >= 2 && D % 2 == 0, "stage parity must equal step parity");
     __shared__ __align__(16) _Float16 s_a[2][kTile * kLdsStride];
@@ -237,15 +242,21 @@ k_enc_gemm(const _Float16 *const a_arg, const _Float16 *const w_arg, const int M
 #pragma unroll
         for (int r = 0; r < 16; ++r) g.out[(size_t)(mbase + acc_row(r, lane)) * g.N + n] = (_Float16)gelu_tanh_for_f16(acc[r]);
     } else {
+        // q, k and v leave in the order in which the attention kernel's matrix instructions take them (see the layout
+        // note at the top): a wavefront's 32 x 32 piece lies inside one (part, head, 32-token tile) block.
+        const int heads = g.width / 64;
         if (n < 2 * g.width) {   // uniform per workgroup: width is a multiple of the tile
+            const int part = n >= g.width ? 1 : 0, d = n & 63, head = (n - part * g.width) >> 6;
+            _Float16 *block = g.out + ((size_t)(part * heads + head) * (g.M / 32) + mbase / 32) * 2048 + ((d >> 4) * 64 + ((d >> 3) & 1) * 32) * 8 + (d & 7);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) g.out[(size_t)(mbase + acc_row(r, lane)) * (2 * g.width) + n] = (_Float16)acc[r];
+            for (int r = 0; r < 16; ++r) block[acc_row(r, lane) * 8] = (_Float16)acc[r];
         } else {
-            _Float16 *col = g.vt + (size_t)(n - 2 * g.width) * g.vt_stride + mbase;
+            const int d = n - 2 * g.width;   // d / 32: the (head, 32-column half) block row; d % 32 = lane % 32
+            _Float16 *block = g.vt + ((size_t)(d >> 5) * (g.M / 16) + mbase / 16) * 512 + (d & 31) * 8 + 4 * (lane >> 5);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {   // registers 4q .. 4q+3 are four consecutive tokens
+            for (int q = 0; q < 4; ++q) {   // registers 4q .. 4q+3 are the four consecutive tokens mbase + 8q + 4 (lane / 32) ..
                 half4 v = {(_Float16)acc[4 * q], (_Float16)acc[4 * q + 1], (_Float16)acc[4 * q + 2], (_Float16)acc[4 * q + 3]};
-                *reinterpret_cast<half4 *>(col + 8 * q + 4 * (lane >> 5)) = v;
+                *reinterpret_cast<half4 *>(block + (q >> 1) * 512 + (q & 1) * 256) = v;
             }
         }
     }
@@ -375,7 +386,7 @@ void launch_rows(State *st, int width, dim3 grid, float *x, const float *part, i
 // picks the smallest pair that covers the padded length (up to 4 and 16: 512 tokens), so that none is requested in vain.
 template <int kKeyTiles, int kValueSteps>
 __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, const _Float16 *vt, _Float16 *ctx, const EncParams *params,
-                                                            int tpad, int width, int vt_stride, float scale, int causal) {
+                                                            int tpad, int width, float scale, int causal) {
     const int tokens = params->tokens;
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ float s_inv[kQTile];
@@ -391,24 +402,26 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
     // None of the requests is under a condition -- a tile or step this call does not have repeats the last one it has and
     // is never used -- so that the number of requests behind each one is a constant: loads return in order, a wait names
     // how many may still be out, and behind a conditional request the compiler has to wait for everything.
-    const int ld = 2 * width;
+    const int heads = width / 64;
     const int ntiles = tpad / 32;
     const int wn = wave & 1, kh = wave >> 1;
     const int kspan = tpad / 2;                              // keys per PV half, multiple of 32
-    const _Float16 *qrow = qk + (size_t)(q0 + (lane & 31)) * ld + head * 64 + 8 * (lane >> 5);
-    const _Float16 *kbase = qk + (size_t)(lane & 31) * ld + width + head * 64 + 8 * (lane >> 5);
-    const _Float16 *vrow = vt + (size_t)(head * 64 + wn * 32 + (lane & 31)) * vt_stride + kh * kspan + 8 * (lane >> 5);
+    // Every request is one operand of one matrix instruction for the whole wavefront, 1 KiB of consecutive bytes (see the
+    // layout note at the top).
+    const half8 *qblock = reinterpret_cast<const half8 *>(qk + ((size_t)head * ntiles + q0 / 32) * 2048) + lane;
+    const half8 *kblocks = reinterpret_cast<const half8 *>(qk + (size_t)(heads + head) * ntiles * 2048) + lane;
+    const half8 *vblocks = reinterpret_cast<const half8 *>(vt + ((size_t)(head * 2 + wn) * (tpad / 16) + kh * (kspan / 16)) * 512) + lane;
     half8 fq[4], fk[kKeyTiles][4], fv[kValueSteps];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) fq[j] = *reinterpret_cast<const half8 *>(qrow + 16 * j);
+    for (int j = 0; j < 4; ++j) fq[j] = qblock[j * 64];
 #pragma unroll
     for (int t = 0; t < kKeyTiles; ++t) {
         const int tile = min(wave + 4 * t, ntiles - 1);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) fk[t][j] = *reinterpret_cast<const half8 *>(kbase + (size_t)tile * 32 * ld + 16 * j);
+        for (int j = 0; j < 4; ++j) fk[t][j] = kblocks[(size_t)tile * 256 + j * 64];
     }
 #pragma unroll
-    for (int st = 0; st < kValueSteps; ++st) fv[st] = *reinterpret_cast<const half8 *>(vrow + min(16 * st, kspan - 16));
+    for (int st = 0; st < kValueSteps; ++st) fv[st] = vblocks[min(st, kspan / 16 - 1) * 64];
 
     // ---- scores
     {
@@ -430,7 +443,7 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
         for (int tile = wave + 4 * kKeyTiles; tile < ntiles; tile += 4) {   // beyond the tiles requested up front (more than 512 tokens)
             half8 k4[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) k4[j] = *reinterpret_cast<const half8 *>(kbase + (size_t)tile * 32 * ld + 16 * j);
+            for (int j = 0; j < 4; ++j) k4[j] = kblocks[(size_t)tile * 256 + j * 64];
             score_tile(tile, k4);
         }
     }
@@ -491,7 +504,7 @@ __global__ void __launch_bounds__(kThreads) k_enc_attention(const _Float16 *qk, 
         }
         for (int k = 16 * kValueSteps; k < kspan; k += 16) {   // beyond the steps requested up front (more than 512 tokens)
             const half8 fp = *reinterpret_cast<const half8 *>(prow + k);
-            const half8 fvk = *reinterpret_cast<const half8 *>(vrow + k);
+            const half8 fvk = vblocks[(k / 16) * 64];
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fp, fvk, acc, 0, 0, 0);
         }
         if (kh == 1) {
@@ -522,13 +535,11 @@ int launch_gemm(State *st, const GemmArgs &g, int splits, char *error, size_t ca
     const dim3 grid(g.N / kTile, g.M / kTile, splits), block(kThreads);
     if (steps % kGemmDepth == 0)
         hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt,
-                           g.width, g.vt_stride);
+                           g.width);
     else if (steps % 2 == 0)
-        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width,
-                           g.vt_stride);
+        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width);
     else
-        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width,
-                           g.vt_stride);
+        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width);
     return hip_check(hipGetLastError(), "encoder product launch", error, capacity);
 }
 
@@ -581,7 +592,6 @@ int pick_splits(int k) {
 // call (token count, output pointers) is read from e->params on the device, so the sequence can be captured once.
 int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size_t capacity) {
     const int w = (int)e->width, f = (int)e->ffn;
-    const int vt_stride = (int)e->tpad_max;
     hipLaunchKernelGGL(k_enc_embed, dim3(tpad), dim3(kThreads), 0, st->stream, e->ids, e->params, static_cast<const _Float16 *>(e->tok->data),
                        static_cast<const _Float16 *>(e->pos->data), e->x, w);
     const dim3 row_grid((tpad + 3) / 4);
@@ -597,14 +607,14 @@ int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size
         launch_rows<true>(st, w, row_grid, e->x, pending, pending_splits, split_stride, e->n1g[l], e->n1b[l], e->nrm, e->params, tpad);
         GemmArgs g{};
         g.a = e->nrm; g.w = static_cast<const _Float16 *>(e->qkv[l]->data); g.M = tpad; g.N = 3 * w; g.K = w;
-        g.out = e->qk; g.vt = e->vt; g.width = w; g.vt_stride = vt_stride;
+        g.out = e->qk; g.vt = e->vt; g.width = w;
         if (launch_gemm<ENC_QKV>(st, g, 1, error, capacity) != 0) return -1;
         {
             // a wavefront scores every fourth 32-key tile and multiplies half of the keys in steps of 16
             const dim3 agrid(tpad / kQTile, (unsigned)e->heads), ablock(kThreads);
-            if (tpad <= 128) hipLaunchKernelGGL((k_enc_attention<1, 4>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale, e->causal);
-            else if (tpad <= 256) hipLaunchKernelGGL((k_enc_attention<2, 8>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale, e->causal);
-            else hipLaunchKernelGGL((k_enc_attention<4, 16>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, vt_stride, scale, e->causal);
+            if (tpad <= 128) hipLaunchKernelGGL((k_enc_attention<1, 4>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, scale, e->causal);
+            else if (tpad <= 256) hipLaunchKernelGGL((k_enc_attention<2, 8>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, scale, e->causal);
+            else hipLaunchKernelGGL((k_enc_attention<4, 16>), agrid, ablock, lds, st->stream, e->qk, e->vt, e->ctx, e->params, tpad, w, scale, e->causal);
         }
         g = GemmArgs{};
         g.a = e->ctx; g.w = static_cast<const _Float16 *>(e->o[l]->data); g.M = tpad; g.N = w; g.K = w; g.part = e->part;
