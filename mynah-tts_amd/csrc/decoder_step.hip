@@ -219,11 +219,13 @@ static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char
 
 DecoderRows decoder_rows(mynah_hip_decoder *d) { return DecoderRows{d->x, d->dev_slots, d->position}; }
 
-int decoder_enqueue_layers(State *st, mynah_hip_decoder *d, int batch, unsigned epoch_offset, char *error, size_t capacity) {
-    if (d->fused_attention && batch > kConsumerFoldMaxBatch &&
-        launch_step_items(st, d->dev_slots, epoch_offset, batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items,
-                          d->self_records != nullptr, d->self_slots, d->cross_slots, error, capacity) != 0)
-        return -1;
+StepItemTables decoder_item_tables(mynah_hip_decoder *d, int batch) {
+    if (!d->fused_attention || batch <= kConsumerFoldMaxBatch) return StepItemTables{};
+    return step_item_tables(batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items, d->self_records != nullptr,
+                            d->self_slots, d->cross_slots);
+}
+
+int decoder_enqueue_layers(State *st, mynah_hip_decoder *d, int batch, char *error, size_t capacity) {
     return enqueue_layers(st, d, batch, error, capacity, kAllStages, false);
 }
 
@@ -589,10 +591,7 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
     }
     if (decoder_next_epochs(st, d, 1, &s.epoch, error, capacity) != 0) return -1;
     d->last_slots = s;
-    if (launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
-    if (d->fused_attention && B > kConsumerFoldMaxBatch &&
-        launch_step_items(st, d->dev_slots, 0, B, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items, d->self_records != nullptr, d->self_slots, d->cross_slots, error, capacity) != 0)
-        return -1;
+    if (launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, decoder_item_tables(d, B), error, capacity) != 0) return -1;
     if (st->graph_mode == 0 || d->eager_steps[B] == 0) {
         // the first step of a batch size also performs one-time kernel attribute set-up, which does not belong in a capture
         d->eager_steps[B] = 1;
@@ -656,9 +655,8 @@ extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *
     // a fresh step counter, as every real step has one: the workgroups that wait for tagged values then really wait
     if (batch > (size_t)kConsumerFoldMaxBatch && (stage == MYNAH_HIP_STAGE_SELF_ATTENTION || stage == MYNAH_HIP_STAGE_CROSS_ATTENTION)) {
         if (decoder_next_epochs(st, d, 1, &d->last_slots.epoch, error, capacity) != 0) return -1;
-        if (launch_step_begin(st, d->last_slots, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, error, capacity) != 0) return -1;
-        if (launch_step_items(st, d->dev_slots, 0, (int)batch, (int)d->heads, (int)d->cross_heads, d->max_units, d->self_items, d->cross_items,
-                              d->self_records != nullptr, d->self_slots, d->cross_slots, error, capacity) != 0)
+        if (launch_step_begin(st, d->last_slots, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, decoder_item_tables(d, (int)batch),
+                              error, capacity) != 0)
             return -1;
     }
     return hip_check(hipGraphLaunch(exec, st->stream), "stage graph launch", error, capacity);

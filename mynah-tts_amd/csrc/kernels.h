@@ -85,7 +85,7 @@ int attention_chunk_rows(int is_self, size_t head_width, bool vector_rows, size_
 
 // Resident step: LayerNorm + activation quantisation + this head's slice of the Q (self: Q, K, V) projection +
 // attention over one cache chunk, per workgroup; writes split-L partials that the next matvec folds.
-// What one workgroup of a many-stream attention grid does: written per step by k_step_items, read by that workgroup.
+// What one workgroup of a many-stream attention grid does: written once per pass through the layers, read by that workgroup.
 struct StepItem {
     float *k, *v;      // the stream's K and V cache (self or cross), all layers
     int length;        // rows in it before this step
@@ -119,10 +119,18 @@ struct StepAttnArgs {
 int launch_step_attention(State *st, const StepAttnArgs &args, char *error, size_t capacity);
 // Workgroups of the attention launch for this shape (the table below has as many entries).
 int step_attention_grid(int heads, int batch, int max_units, int is_self, bool packed);
-// Fills the work tables of the many-stream attention launches for one step (both kinds) from the slot table in device
-// memory; the tables' step counter is the slot table's plus `epoch_offset`.
-int launch_step_items(State *st, const StepSlots *dev_slots, unsigned epoch_offset, int batch, int heads, int cross_heads, int max_units,
-                      StepItem *self_items, StepItem *cross_items, bool with_fold, int self_slots, int cross_slots, char *error, size_t capacity);
+// Both work tables of one pass through the layers, as the kernel that starts the pass needs them to fill them (extra
+// workgroups of its grid run write_step_item of step_items.h, one entry per thread).  No entries: the batch size takes no
+// tables.  self_slots / cross_slots: workgroups of the attention kernel that the device holds at once.
+struct StepItemTables {
+    StepItem *self_items, *cross_items;
+    int self_entries, cross_entries;
+    int batch, heads, cross_heads;
+    int with_fold, self_budget, cross_budget;
+};
+StepItemTables step_item_tables(int batch, int heads, int cross_heads, int max_units, StepItem *self_items, StepItem *cross_items, bool with_fold,
+                                int self_slots, int cross_slots);
+inline unsigned step_item_workgroups(const StepItemTables &t) { return (unsigned)((t.self_entries + t.cross_entries + 255) / 256); }
 // Workgroups of the many-stream attention kernel for this weight storage and shape that the device holds at once.
 int step_attention_slots(int qtype, int width, int max_units, int is_self, bool with_fold);
 // LDS a fold workgroup needs: the launch's dynamic LDS is at least this when it folds its own partials.
@@ -185,7 +193,6 @@ int launch_gather(State *st, const float *const *dev_tables, size_t table_count,
                   size_t capacity);
 int launch_stream_copy(State *st, const void *src, void *dst, size_t bytes, char *error, size_t capacity);
 
-// Resident step: writes the slot table to device memory and forms x[b] = input[b] + position[length[b]].
 // Token choice of the decoder head for `batch` slots (kernels_misc.hip).
 struct HeadArgmaxArgs {
     const float *logits[kMaxBatch];   // [streams, vocab] per slot
@@ -196,8 +203,10 @@ struct HeadArgmaxArgs {
     unsigned long long *eos_frame;    // device [batch], ~0 = none
 };
 int launch_head_argmax(State *st, const HeadArgmaxArgs &args, int batch, char *error, size_t capacity);
+// Resident step: writes the slot table to device memory, forms x[b] = input[b] + position[length[b]] and fills the work
+// tables of the step's many-stream attention launches (step counter: the slot table's).
 int launch_step_begin(State *st, const StepSlots &slots, StepSlots *dev_slots, int batch, size_t width,
-                      const float *dev_position, float *x, size_t x_stride, char *error, size_t capacity);
+                      const float *dev_position, float *x, size_t x_stride, const StepItemTables &tables, char *error, size_t capacity);
 // Final norm of the step: out = slots->output[b]; gain may be null (plain copy).
 int launch_step_end(State *st, const StepSlots *dev_slots, int batch, size_t width, const float *x, size_t x_stride,
                     const float *gain, const float *bias, char *error, size_t capacity);
@@ -205,16 +214,18 @@ int launch_step_end(State *st, const StepSlots *dev_slots, int batch, size_t wid
 // Resident decoder internals for a caller that drives the layers itself (the local frame): the residual rows
 // x[kMaxBatch][width] the layer kernels read and update, the device slot table they take caches and lengths from,
 // and the device position table.  decoder_enqueue_layers puts one step's layer kernels on the stream -- no begin
-// kernel, no output kernel, no graph launch -- and may be captured once every kernel shape has run eagerly.
+// kernel, no output kernel, no graph launch -- and may be captured once every kernel shape has run eagerly.  The caller's
+// own kernels fill the work tables decoder_item_tables names before each pass (no entries: none needed at this batch size).
 struct DecoderRows {
     float *x;
     StepSlots *slots;
     const float *position;
 };
 DecoderRows decoder_rows(mynah_hip_decoder *decoder);
-// `epoch_offset`: added to the slot table's step counter for this pass (a caller that runs the layers several times per
-// slot table gives each pass its own).  decoder_next_epochs reserves `count` consecutive counters and returns the first.
-int decoder_enqueue_layers(State *st, mynah_hip_decoder *decoder, int batch, unsigned epoch_offset, char *error, size_t capacity);
+// A caller that runs the layers several times per slot table gives each pass's tables a step counter of its own:
+// decoder_next_epochs reserves `count` consecutive counters and returns the first.
+StepItemTables decoder_item_tables(mynah_hip_decoder *decoder, int batch);
+int decoder_enqueue_layers(State *st, mynah_hip_decoder *decoder, int batch, char *error, size_t capacity);
 int decoder_next_epochs(State *st, mynah_hip_decoder *decoder, unsigned count, unsigned *first, char *error, size_t capacity);
 
 }  // namespace mynah

@@ -3,6 +3,7 @@
 #include <float.h>
 
 #include "device_common.h"
+#include "step_items.h"
 
 namespace mynah {
 namespace {
@@ -202,9 +203,15 @@ __global__ void __launch_bounds__(256) k_gather(GatherTables tables, int table_c
 
 // Decode-step begin: record the slot table, x[b] = input[b] + position[length[b]] (src/graph.c:3156-3157).
 // (The scalar arguments stand in front of the table: leading scalars are in registers when a wavefront starts.)
-__global__ void __launch_bounds__(256) k_step_begin(StepSlots *dev_slots, int width, const float *position, float *x, size_t x_stride,
-                                                    const StepSlots slots) {
+// Workgroups behind the streams' fill the work tables of the step's many-stream attention launches, from the table in the
+// kernel's arguments.
+__global__ void __launch_bounds__(256) k_step_begin(StepSlots *dev_slots, int width, const float *position, float *x, size_t x_stride, int batch,
+                                                    const StepSlots slots, const StepItemTables tables) {
     const int b = blockIdx.x;
+    if (b >= batch) {
+        write_step_item(tables, slots, -1, (int)(slots.epoch & 0xffffffu), (b - batch) * 256 + (int)threadIdx.x);
+        return;
+    }
     if (b == 0 && threadIdx.x == 0) *dev_slots = slots;
     const float *in = slots.input[b];
     const float *pe = position != nullptr ? position + (size_t)slots.length[b] * width : nullptr;
@@ -322,9 +329,9 @@ int launch_gather(State *st, const float *const *dev_tables, size_t table_count,
     return hip_check(hipGetLastError(), "gather launch", error, capacity);
 }
 int launch_step_begin(State *st, const StepSlots &slots, StepSlots *dev_slots, int batch, size_t width,
-                      const float *dev_position, float *x, size_t x_stride, char *error, size_t capacity) {
-    hipLaunchKernelGGL(k_step_begin, dim3((unsigned)batch), dim3(256), 0, st->stream, dev_slots, (int)width, dev_position, x, x_stride,
-                       slots);
+                      const float *dev_position, float *x, size_t x_stride, const StepItemTables &tables, char *error, size_t capacity) {
+    hipLaunchKernelGGL(k_step_begin, dim3((unsigned)batch + step_item_workgroups(tables)), dim3(256), 0, st->stream, dev_slots, (int)width, dev_position, x,
+                       x_stride, batch, slots, tables);
     return hip_check(hipGetLastError(), "step begin launch", error, capacity);
 }
 int launch_step_end(State *st, const StepSlots *dev_slots, int batch, size_t width, const float *x, size_t x_stride,

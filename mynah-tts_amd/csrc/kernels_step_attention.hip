@@ -25,6 +25,7 @@
 // The mapping from workgroup to (head, stream, unit) is static, so the weight slice and x are requested
 // before the slot table (lengths, cache pointers) has arrived; K and V rows follow as soon as it has.
 #include "step_attention_core.h"
+#include "step_items.h"
 #include "tagged_exchange.h"
 
 namespace mynah {
@@ -63,7 +64,6 @@ __device__ __forceinline__ float4 fold_records(const float *rec, const float *we
     return acc;
 }
 
-constexpr int kFoldUnit = 0x7fff;   // unit number of a table entry that folds instead of attending
 
 // WFIX: model width known at compile time (0 = taken from the arguments): lane-group width, chunks per lane and passes
 // per bank become constants and the per-chunk range checks fold away.  The decoder stack's width (768) gets such a build.
@@ -444,93 +444,6 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     }
 }
 
-// Work table of the PACKED builds, one entry per workgroup index of the attention grid: which (head, stream, unit) the
-// workgroup takes and where that stream's cache is.  Self-attention: first the Q+K and V roles of every stream's new row,
-// head-major; then, per head, the cache chunks that exist, stream by stream.  Each of the two lists is cut into eight
-// contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so a head's weight slice is fetched by at most two XCDs.
-// Behind the chunks that exist: one fold entry per (stream, head) when the launch folds its own partials.  Workgroups
-// numbered past all of these get code -1: they are the last ones of the grid and leave after this one read.  Written once
-// per step, before the layers, from the slot table in device memory (whose lengths a caller's own kernels may have advanced
-// since the host last saw it) and its step counter plus `epoch_offset`.
-// A workgroup takes `group` consecutive chunks of its stream and head: the smallest number with which every workgroup of the
-// launch is resident at once (`budget` = the chip's workgroup slots for this kernel less the other roles).  A second round
-// of workgroups would start when the first ends and run its whole dependent chain again, some 5 us, for a fifth of the work.
-__device__ StepItem make_item(const StepSlots &slots, int batch, int heads, bool is_self, int wg, int epoch, bool with_fold, int budget) {
-    const StepItem dead{nullptr, nullptr, 0, -1, 0, 0};
-    // chunks per workgroup: the smallest group size with which the launch's chunk workgroups are at most `budget`
-    int all_chunks = 0;
-    for (int s = 0; s < batch; ++s) {
-        const int len = is_self ? slots.length[s] : slots.memory_length[s];
-        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-        all_chunks += is_self ? live : max(live, 1);
-    }
-    const int group = max(1, (heads * all_chunks + budget - 1) / max(budget, 1));
-    int chunk_items = 0;   // groups per head
-    for (int s = 0; s < batch; ++s) {
-        const int len = is_self ? slots.length[s] : slots.memory_length[s];
-        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-        chunk_items += ((is_self ? live : max(live, 1)) + group - 1) / group;
-    }
-    int head, b = 0, unit = 0;
-    const int producers = is_self ? 2 * batch * heads : 0;
-    const int producer_grid = 8 * ((producers + 7) / 8);
-    if (wg < producer_grid) {
-        // the new row's Q+K and V roles, head-major, before everything that waits for them
-        const int per_xcd = producer_grid / 8;
-        const int xcd = wg & 7, slot = wg >> 3;
-        const int p = xcd * per_xcd + slot;
-        if (p >= producers) return dead;
-        head = p / (2 * batch);
-        const int r = p - head * 2 * batch;
-        b = r >> 1;
-        unit = r & 1;
-    } else {
-        const int w2 = wg - producer_grid;
-        const int items = heads * chunk_items;
-        const int per_xcd = (items + 7) / 8;
-        const int xcd = w2 & 7, slot = w2 >> 3;
-        const int item = xcd * per_xcd + slot;
-        if (w2 >= 8 * per_xcd) {
-            // behind every workgroup that attends: one fold per (stream, head)
-            const int f = w2 - 8 * per_xcd;
-            if (!with_fold || f >= heads * batch) return dead;
-            head = f / batch;
-            b = f - head * batch;
-            unit = kFoldUnit;
-        } else {
-            if (item >= items) return dead;
-            head = item / chunk_items;
-            const int r = item - head * chunk_items;
-            int before = 0;
-            for (int s = 0; s < batch; ++s) {
-                const int len = is_self ? slots.length[s] : slots.memory_length[s];
-                const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-                const int n = ((is_self ? live : max(live, 1)) + group - 1) / group;
-                if (r >= before && r < before + n) { b = s; unit = r - before + (is_self ? 2 : 0); }
-                before += n;
-            }
-        }
-    }
-    StepItem it;
-    it.k = is_self ? slots.self_k[b] : const_cast<float *>(slots.cross_k[b]);
-    it.v = is_self ? slots.self_v[b] : const_cast<float *>(slots.cross_v[b]);
-    it.length = is_self ? slots.length[b] : slots.memory_length[b];
-    it.code = head | (b << 8) | (unit << 16);
-    it.epoch = epoch;
-    it.group = group;
-    return it;
-}
-
-__global__ void __launch_bounds__(kThreads) k_step_items(const StepSlots *slots, unsigned epoch_offset, int batch, int heads, int cross_heads,
-                                                         StepItem *self_items, int self_entries, StepItem *cross_items, int cross_entries,
-                                                         bool with_fold, int self_budget, int cross_budget) {
-    const int i = blockIdx.x * kThreads + threadIdx.x;
-    const int epoch = (int)((slots->epoch + epoch_offset) & 0xffffffu);
-    if (i < self_entries) self_items[i] = make_item(*slots, batch, heads, true, i, epoch, with_fold, self_budget);
-    else if (i - self_entries < cross_entries)
-        cross_items[i - self_entries] = make_item(*slots, batch, cross_heads, false, i - self_entries, epoch, with_fold, cross_budget);
-}
-
 // Stand-alone fold of the partials into out[stream][heads * 64]: used instead of the consumer-side fold when
 // the batch is large enough that every workgroup of the output projection folding every stream would cost more
 // than one extra launch.  Same arithmetic (fold_partials), so the result does not depend on which path ran.
@@ -642,20 +555,23 @@ int step_attention_grid(int heads, int batch, int max_units, int is_self, bool p
     return 8 * ((items + 7) / 8);
 }
 
-int launch_step_items(State *st, const StepSlots *dev_slots, unsigned epoch_offset, int batch, int heads, int cross_heads, int max_units,
-                      StepItem *self_items, StepItem *cross_items, bool with_fold, int self_slots, int cross_slots, char *error, size_t capacity) {
+StepItemTables step_item_tables(int batch, int heads, int cross_heads, int max_units, StepItem *self_items, StepItem *cross_items, bool with_fold,
+                                int self_slots, int cross_slots) {
+    StepItemTables t{};
     if (batch < 1 || batch > kMaxBatch || heads < 1 || heads > 255 || cross_heads < 0 || cross_heads > 255 || max_units < 1 || max_units > 32000 ||
-        dev_slots == nullptr || self_items == nullptr || (cross_heads > 0 && cross_items == nullptr)) {
-        set_error(error, capacity, "step items: invalid shape");
-        return -1;
-    }
-    const int self_entries = step_attention_grid(heads, batch, max_units, 1, true);
-    const int cross_entries = cross_heads > 0 ? step_attention_grid(cross_heads, batch, max_units, 0, true) : 0;
-    const int total = self_entries + cross_entries;
-    hipLaunchKernelGGL(k_step_items, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0, st->stream, dev_slots, epoch_offset, batch,
-                       heads, cross_heads, self_items, self_entries, cross_items, cross_entries, with_fold,
-                       self_slots - 8 * ((2 * batch * heads + 7) / 8) - (with_fold ? heads * batch : 0), cross_slots - (with_fold ? cross_heads * batch : 0));
-    return hip_check(hipGetLastError(), "step items launch", error, capacity);
+        self_items == nullptr || (cross_heads > 0 && cross_items == nullptr))
+        return t;
+    t.self_items = self_items;
+    t.cross_items = cross_items;
+    t.self_entries = step_attention_grid(heads, batch, max_units, 1, true);
+    t.cross_entries = cross_heads > 0 ? step_attention_grid(cross_heads, batch, max_units, 0, true) : 0;
+    t.batch = batch;
+    t.heads = heads;
+    t.cross_heads = cross_heads;
+    t.with_fold = with_fold ? 1 : 0;
+    t.self_budget = self_slots - 8 * ((2 * batch * heads + 7) / 8) - (with_fold ? heads * batch : 0);
+    t.cross_budget = cross_slots - (with_fold ? cross_heads * batch : 0);
+    return t;
 }
 
 int launch_step_attention(State *st, const StepAttnArgs &a, char *error, size_t capacity) {

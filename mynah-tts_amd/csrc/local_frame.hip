@@ -24,6 +24,7 @@
 #include <new>
 
 #include "kernels.h"
+#include "step_items.h"
 
 using namespace mynah;
 
@@ -59,6 +60,8 @@ struct SampleArgs {
     StepSlots *slots;             // cache lengths advance here
     unsigned *values, *stored;    // [batch, streams]
     int stream, streams, vocab, codebook_size, eos_id, codebook_count, width;
+    int batch;                    // workgroups behind the items' fill `tables` for the next pass through the stack
+    StepItemTables tables;
 };
 
 // Monotone map float -> unsigned: a > b  <=>  key(a) > key(b)  (no NaNs among logits that matter), and back.
@@ -96,9 +99,14 @@ __device__ __forceinline__ int count_above_by_four(const unsigned long long *lis
 
 // Frame start: the slot table (caches of this object, every length 0), x[b] = decoder_last[b] + position[0]
 // (src/graph.c:1420-1422 and :1262-1264), EOS flags cleared (:1409-1410).
+// Workgroups behind the items' fill the work tables of the first pass's many-stream attention launch (every cache empty).
 __global__ void __launch_bounds__(256) k_local_begin(LocalFrameDev *frame, const StepSlots slots, StepSlots *dev_slots, float *x,
-                                                     const float *position, int width) {
+                                                     const float *position, int width, int batch, const StepItemTables tables) {
     const int b = blockIdx.x;
+    if (b >= batch) {
+        write_step_item(tables, slots, 0, (int)(frame->epoch_base & 0xffffffu), (b - batch) * 256 + (int)threadIdx.x);
+        return;
+    }
     if (b == 0 && threadIdx.x == 0) {
         *dev_slots = slots;
         dev_slots->epoch = frame->epoch_base;
@@ -137,6 +145,12 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
     __shared__ float s_draw;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, b = blockIdx.x;
+    if (b >= a.batch) {
+        // the next pass's caches hold stream + 1 rows each whatever is chosen here; the slot table's pointers are the frame's
+        if (a.stream + 1 < a.streams)
+            write_step_item(a.tables, *a.slots, a.stream + 1, (int)((a.frame->epoch_base + (unsigned)a.stream + 1u) & 0xffffffu), (b - a.batch) * 256 + tid);
+        return;
+    }
     LocalItemDev &item = a.frame->items[b];
     const int V = a.vocab;
     const float *lg = a.logits + (size_t)b * V;
@@ -407,10 +421,13 @@ static int enqueue_frame(State *st, mynah_hip_local *l, int B, char *error, size
         slots.input[b] = rows.x + (size_t)b * width;
         slots.output[b] = rows.x + (size_t)b * width;
     }
-    hipLaunchKernelGGL(k_local_begin, dim3(B), dim3(256), 0, st->stream, l->frame, slots, rows.slots, rows.x, rows.position, width);
+    const StepItemTables tables = decoder_item_tables(l->stack, B);
+    const unsigned table_workgroups = step_item_workgroups(tables);
+    hipLaunchKernelGGL(k_local_begin, dim3(B + table_workgroups), dim3(256), 0, st->stream, l->frame, slots, rows.slots, rows.x, rows.position, width, B,
+                       tables);
     MYNAH_TRY(hipGetLastError());
     for (size_t stream = 0; stream < l->streams; ++stream) {
-        if (decoder_enqueue_layers(st, l->stack, B, (unsigned)stream, error, capacity) != 0) return -1;
+        if (decoder_enqueue_layers(st, l->stack, B, error, capacity) != 0) return -1;
         const CachedWeight *cw = l->projection[stream];
         for (int b0 = 0; b0 < B; b0 += kBatchTile) {
             LinearArgs p{};
@@ -435,7 +452,8 @@ static int enqueue_frame(State *st, mynah_hip_local *l, int B, char *error, size
         a.x = rows.x; a.slots = rows.slots; a.values = l->values; a.stored = l->values + (size_t)kMaxBatch * l->streams;
         a.stream = (int)stream; a.streams = (int)l->streams; a.vocab = (int)l->vocab; a.codebook_size = (int)l->codebook_size;
         a.eos_id = (int)l->eos_id; a.codebook_count = (int)l->codebook_count; a.width = width;
-        hipLaunchKernelGGL(k_local_sample, dim3(B), dim3(256), l->vocab * sizeof(float), st->stream, a);
+        a.batch = B; a.tables = tables;
+        hipLaunchKernelGGL(k_local_sample, dim3(B + (stream + 1 < l->streams ? table_workgroups : 0u)), dim3(256), l->vocab * sizeof(float), st->stream, a);
         MYNAH_TRY(hipGetLastError());
     }
     return 0;
