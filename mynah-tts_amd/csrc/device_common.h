@@ -181,10 +181,11 @@ __device__ __forceinline__ void layernorm_row(const float *x, float *y, const fl
     }
 }
 
-// round half away from zero by truncation, clamp to +-127 (src/qmat.c:106-110)
+// round half away from zero by truncation, clamp to +-127 (src/qmat.c:106-110); the half with v's sign is one bit-field
+// instruction where the comparison and selection of the reference's form are two, with the same sum for every v
 __device__ __forceinline__ int quant_act(float x, float inv) {
     const float v = x * inv;
-    int q = (int)(v >= 0.0f ? v + 0.5f : v - 0.5f);
+    int q = (int)(v + __builtin_copysignf(0.5f, v));
     q = q > 127 ? 127 : q;
     q = q < -127 ? -127 : q;
     return q;
