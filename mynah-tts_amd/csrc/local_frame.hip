@@ -23,6 +23,7 @@
 
 #include <new>
 
+#include "device_common.h"
 #include "kernels.h"
 #include "step_items.h"
 
@@ -80,6 +81,18 @@ __device__ __forceinline__ unsigned long long candidate(unsigned key, int index)
 __device__ __forceinline__ int candidate_index(unsigned long long c) { return (int)(0xffffffffu - (unsigned)(c & 0xffffffffull)); }
 __device__ __forceinline__ unsigned candidate_key(unsigned long long c) { return (unsigned)(c >> 32); }
 
+// Largest value over the wavefront, in every lane: four steps inside the rows of sixteen lanes on the DPP path, then the
+// four rows through scalar registers.  All 64 lanes must be active.
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+    v = max(v, (unsigned)dpp_i<kDppXor1>((int)v));
+    v = max(v, (unsigned)dpp_i<kDppXor2>((int)v));
+    v = max(v, (unsigned)dpp_i<kDppHalfMirror>((int)v));
+    v = max(v, (unsigned)dpp_i<kDppMirror>((int)v));
+    const unsigned r0 = (unsigned)__builtin_amdgcn_readlane((int)v, 0), r1 = (unsigned)__builtin_amdgcn_readlane((int)v, 16);
+    const unsigned r2 = (unsigned)__builtin_amdgcn_readlane((int)v, 32), r3 = (unsigned)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(r0, r1), max(r2, r3));
+}
+
 // How many of list[0, n) are above `mine` (pairs of entries per LDS read; the list is 16-byte aligned), counted by four
 // adjacent threads: thread `part` of the four looks at pairs part, part + 4, ... and the four sums meet by shuffles.  Every
 // lane of the wavefront must call it.
@@ -92,8 +105,23 @@ __device__ __forceinline__ int count_above_by_four(const unsigned long long *lis
         above += (p.x > mine ? 1 : 0) + (p.y > mine ? 1 : 0);
     }
     if ((n & 1) && part == 0) above += list[n - 1] > mine ? 1 : 0;
-    above += __shfl_xor(above, 1);
-    above += __shfl_xor(above, 2);
+    above += dpp_i<kDppXor1>(above);
+    above += dpp_i<kDppXor2>(above);
+    return above;
+}
+
+// The same for a list of at most 64 entries followed by zeros up to 64 (no candidate is zero): every thread's eight reads
+// are requested at once.
+__device__ __forceinline__ int count_above_in_64(const unsigned long long *list, unsigned long long mine, int part) {
+    const ulonglong2 *pairs = reinterpret_cast<const ulonglong2 *>(list);
+    ulonglong2 p[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p[j] = pairs[part + 4 * j];
+    int above = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) above += (p[j].x > mine ? 1 : 0) + (p[j].y > mine ? 1 : 0);
+    above += dpp_i<kDppXor1>(above);
+    above += dpp_i<kDppXor2>(above);
     return above;
 }
 
@@ -137,7 +165,7 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
     __shared__ unsigned s_bound[4];
     __shared__ __align__(16) unsigned long long s_cand[kFastCandidates];
     __shared__ unsigned s_hist[4][256];
-    __shared__ __align__(16) float s_top_val[kMaxTopK + 8];
+    __shared__ __align__(16) float s_top_val[kMaxTopK + 32];
     __shared__ int s_top_idx[kMaxTopK];
     __shared__ unsigned s_wave_total[4];
     __shared__ unsigned s_prefix, s_count;
@@ -154,53 +182,63 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
     LocalItemDev &item = a.frame->items[b];
     const int V = a.vocab;
     const float *lg = a.logits + (size_t)b * V;
+    // Everything the kernel takes from memory before the choice is requested here, side by side and under no condition
+    // (ids past the vocabulary repeat its last one): one round trip.  Requested where they are used, the item's fields, the
+    // frame's pointer and the logits were three round trips one after the other, and the generator state a fourth.
+    float first_logits[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) first_logits[i] = lg[min(tid + 256 * i, V - 1)];
     const int forbid_eos = item.forbid_eos;
     const float temperature = item.temperature;
     const unsigned topk = item.topk;
+    const unsigned long long rng_before = item.rng_state;
     float *logits_copy = a.frame->logits_copy;
-    const int top_count = min((int)min(topk, (unsigned)V), kMaxTopK);
-    const bool sampling = temperature > 0.0f && topk > 1u;
 
-    // ---- constraint mask (src/graph.c:1556-1563); eight candidates per thread are requested at a time
+    // ---- constraint mask (src/graph.c:1556-1563); eight candidates per thread at a time, the first eight already requested
     unsigned long long mine = 0ull;
     constexpr int kKeysInRegisters = 8;              // a vocabulary of up to 8 * 256 ids: a thread's keys stay in registers for the collection below
     const bool keys_in_registers = V <= kKeysInRegisters * 256;
     unsigned own_key[kKeysInRegisters];
-#pragma unroll
-    for (int i = 0; i < kKeysInRegisters; ++i) own_key[i] = 0u;
-    for (int c0 = tid; c0 < V; c0 += 8 * 256) {
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = c0 + 256 * i < V ? lg[c0 + 256 * i] : 0.0f;
+    const auto mask_eight = [&](const int c0, const float (&v)[8], const bool keep) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int c = c0 + 256 * i;
+            const bool allowed = c < a.codebook_size || (c == a.eos_id && !forbid_eos);
+            const float masked = allowed ? v[i] : -FLT_MAX;
+            const unsigned key = order_key(masked);
+            if (keep) own_key[i] = c < V ? key : 0u;
             if (c < V) {
-                const bool allowed = c < a.codebook_size || (c == a.eos_id && !forbid_eos);
-                const float masked = allowed ? v[i] : -FLT_MAX;
-                const unsigned key = order_key(masked);
                 s_key[c] = key;
-                if (c0 == tid) own_key[i] = key;
                 if (logits_copy != nullptr) logits_copy[((size_t)b * a.streams + a.stream) * V + c] = masked;
                 const unsigned long long cand = candidate(key, c);
                 mine = cand > mine ? cand : mine;
             }
         }
+    };
+    mask_eight(tid, first_logits, true);
+    for (int c0 = tid + 8 * 256; c0 < V; c0 += 8 * 256) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = c0 + 256 * i < V ? lg[c0 + 256 * i] : 0.0f;
+        mask_eight(c0, v, false);
     }
+    const int top_count = min((int)min(topk, (unsigned)V), kMaxTopK);
+    const bool sampling = temperature > 0.0f && topk > 1u;
     for (int p = 0; p < 4; ++p) s_hist[p][tid] = 0u;
+    if (tid < 64) s_cand[tid] = 0ull;   // a list of up to 64 candidates is followed by zeros (see count_above_in_64)
     if (tid == 0) { s_prefix = 0u; s_remaining = top_count; s_count = 0u; s_pick = top_count - 1; }
-    // ---- the head of the list: the largest candidate of the wavefront, then of the four
-    unsigned long long head = mine;
-    for (int off = 32; off >= 1; off >>= 1) {
-        const unsigned long long other = __shfl_xor(head, off);
-        head = other > head ? other : head;
-    }
-    // (sampling) the largest key that at least `want` of the wavefront's 64 bests reach
+    // ---- the head of the list: the largest candidate of the wavefront (the largest key, and among the lanes that hold it the
+    // largest low word = the smallest id), then of the four
+    const unsigned head_key = wave_max_u32(candidate_key(mine));
+    const unsigned head_low = wave_max_u32(candidate_key(mine) == head_key ? (unsigned)(mine & 0xffffffffull) : 0u);
+    unsigned long long head = ((unsigned long long)head_key << 32) | (unsigned long long)head_low;
+    // (sampling) the largest key with its low half clear that at least `want` of the wavefront's 64 bests reach: sixteen
+    // ballots; the keys between this bound and the exact one (1/128 of the logit's magnitude) add a candidate or two
     unsigned bound = 0u;
     if (sampling) {
         const int want = (top_count + 3) / 4;
         const unsigned own = candidate_key(mine);
-        for (int bit = 31; bit >= 0; --bit) {
+        for (int bit = 31; bit >= 16; --bit) {
             const unsigned trial = bound | (1u << bit);
             if (__popcll(__ballot(own >= trial)) >= want) bound = trial;
         }
@@ -229,7 +267,7 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
             }
             unsigned next_slot = 0u;
             if (lane == 0) next_slot = atomicAdd(&s_count, in_wave);
-            next_slot = __shfl(next_slot, 0);
+            next_slot = (unsigned)__builtin_amdgcn_readfirstlane((int)next_slot);
 #pragma unroll
             for (int i = 0; i < kKeysInRegisters; ++i) {
                 const bool take = (masks[i] >> lane) & 1ull;
@@ -327,35 +365,40 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
                 }
             }
             listed = top_count;
+            if (tid >= top_count && tid < 64) s_cand[tid] = 0ull;   // behind a short list: zeros again (count_above_in_64)
             __syncthreads();
         }
         // ---- list position = how many collected candidates come before; numerators expf((l - max) / T) (src/graph.c:1599-1604)
-        for (int q0 = 0; q0 < listed; q0 += 64) {   // four adjacent threads per candidate; every lane takes part in the shuffles
+        for (int q0 = 0; q0 < listed; q0 += 64) {   // four adjacent threads per candidate; every lane takes part in the exchanges
             const int q = q0 + (tid >> 2);
             const unsigned long long own = s_cand[q < listed ? q : listed - 1];
-            const int place = count_above_by_four(s_cand, listed, own, tid & 3);
+            const int place = listed <= 64 ? count_above_in_64(s_cand, own, tid & 3) : count_above_by_four(s_cand, listed, own, tid & 3);
             if (q < listed && (tid & 3) == 0 && place < top_count) {
                 s_top_idx[place] = candidate_index(own);
                 s_top_val[place] = expf((key_value(candidate_key(own)) - maximum) / temperature);
             }
         }
-        if (tid < 8) s_top_val[top_count + tid] = 0.0f;   // lets the running sum below go in whole groups of eight
+        if (tid < 32) s_top_val[top_count + tid] = 0.0f;   // lets the running sum below go in whole groups of 32
         __syncthreads();
         // ---- running sums in list order by one thread, kept in place (src/graph.c:1605-1616): float32 sums depend on
         // the order, and the last running sum is the reference's total
         if (tid == 0) {
             float running = 0.0f;
-            for (int q0 = 0; q0 < top_count; q0 += 8) {
-                float part[8];
+            for (int q0 = 0; q0 < top_count; q0 += 32) {   // a group's reads are requested together, its sums stay in registers
+                float4 part[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) part[i] = s_top_val[q0 + i];
+                for (int i = 0; i < 8; ++i) part[i] = *reinterpret_cast<const float4 *>(&s_top_val[q0 + 4 * i]);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    running += part[i];
-                    s_top_val[q0 + i] = running;
+                    running += part[i].x; part[i].x = running;
+                    running += part[i].y; part[i].y = running;
+                    running += part[i].z; part[i].z = running;
+                    running += part[i].w; part[i].w = running;
                 }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) *reinterpret_cast<float4 *>(&s_top_val[q0 + 4 * i]) = part[i];
             }
-            unsigned long long bits = item.rng_state;
+            unsigned long long bits = rng_before;
             bits ^= bits << 13;
             bits ^= bits >> 7;
             bits ^= bits << 17;
@@ -386,7 +429,23 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
         const unsigned emit = value < (unsigned)V ? value : 0u;                                          // :1626
         const float *row = a.audio_table + (size_t)emit * a.width;                                      // :1651
         const float *pe = a.next_position;                                                             // :1262-1264
-        for (int d = tid; d < a.width; d += 256) a.x[(size_t)b * a.width + d] = pe != nullptr ? row[d] + pe[d] : row[d];
+        if (a.width <= 1024) {   // one round trip: every request before the first sum
+            float rv[4], pv[4];
+            const float *second = pe != nullptr ? pe : row;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int d = tid + 256 * u, at = d < a.width ? d : a.width - 1;
+                rv[u] = row[at];
+                pv[u] = second[at];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int d = tid + 256 * u;
+                if (d < a.width) a.x[(size_t)b * a.width + d] = pe != nullptr ? rv[u] + pv[u] : rv[u];
+            }
+        } else {
+            for (int d = tid; d < a.width; d += 256) a.x[(size_t)b * a.width + d] = pe != nullptr ? row[d] + pe[d] : row[d];
+        }
     }
 }
 
