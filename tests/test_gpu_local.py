@@ -189,6 +189,35 @@ def test_frame_batch16_two_tiles(pkg, backend, orc, synth, nerr):
         d.free()
 
 
+def test_frame_many_tied_candidates(pkg, backend, orc, synth, nerr):
+    """Seven hundred ids share the largest logit, so more candidates reach the sampler's first bound than its fast list
+    holds and the exact selection runs with short lists (top-k 2, 7, 50) as well as a long one (256): the list is the
+    tied ids in ascending order, as the reference's insertion keeps the earlier id first (src/graph.c:1580-1598)."""
+    _announce("local frame, 700 tied largest logits")
+    S, V, codebook, eos, cbc = 4, 2048, 2016, 2017, 4
+    cfg, w, proj, bias, tables, rng = _setup(synth, 1, S, V, seed=67)
+    for s in range(S):
+        proj[s][200:900] = proj[s][7]
+        bias[s][200:900] = bias[s][7] = 25.0
+    backend.set_quant(QT["f32"])
+    loc = pkg.Local(backend, cfg, w, proj, bias, tables, codebook, eos, cbc)
+    B = len(ITEMS)
+    rows = [rng.standard_normal(cfg["width"]).astype(np.float32) for _ in range(B)]
+    drows = [backend.alloc(cfg["width"]).write(r) for r in rows]
+    dlogits = backend.alloc(B * S * V)
+    got = loc.frame([dict(it, row=d.ptr) for it, d in zip(ITEMS, drows)], dlogits.ptr)
+    logits = dlogits.read().reshape(B, S, V)
+    assert np.all(logits[:, :, 200:900] == logits[:, :, 7:8]) and np.all(logits.max(axis=2) == logits[:, :, 7])
+    _replay_choices(orc, logits, ITEMS, got, codebook, eos, cbc)
+    for b, it in enumerate(ITEMS):   # a list of k tied ids starts 7, 200, 201, ...: nothing beyond its k-th id can be chosen
+        k = it["topk"]
+        assert np.all((got["values"][b] == 7) | ((got["values"][b] >= 200) & (got["values"][b] < 200 + max(k - 1, 0)))), (b, got["values"][b])
+    loc.destroy()
+    for d in drows + [dlogits]:
+        d.free()
+    backend.set_quant(0)
+
+
 def test_frame_eos_outside_vocabulary(pkg, backend, orc, synth, nerr):
     """An end-of-sequence id that is no id of the vocabulary (here one whose low 32 bits are 5, a real id) matches
     nothing, as in the reference's full-width comparison (src/graph.c:1563-1574): only codebook ids are ever allowed,
