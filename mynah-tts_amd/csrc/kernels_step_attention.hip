@@ -121,7 +121,7 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
         b = hb % a.batch;
         head = hb / a.batch;
     } else {
-        // one table entry, written at the step's start for this very workgroup index (k_step_items): one read instead of
+        // one table entry, written at the step's start for this very workgroup index (write_step_item): one read instead of
         // the lengths, two loops over the streams and then the stream's cache pointers, each a round trip of its own
         typedef int int8v __attribute__((ext_vector_type(8)));
         static_assert(sizeof(StepItem) == sizeof(int8v), "an entry is read as one 32-byte scalar load");
