@@ -278,6 +278,22 @@ MEASURED_TRAFFIC = {"kernel": "k_linear<k=768, residual>", "bytes": 921584, "pro
                     "csrc_sha256": "66534d40a965041e"}
 
 
+def latency_floor(backend, step_us, launches):
+    """What the step's chain of dependent launches costs with every byte taken out: the library's probe runs graph nodes
+    that only hand a 768-float vector (3072 for one stage in six) from all workgroups of one node to all workgroups of the
+    next -- the skeleton of a matvec stage -- and the floor is that node time x the step's dependent launches."""
+    node768 = backend.dependent_launch_probe(72, 192, 768, 1, 40)
+    node3072 = backend.dependent_launch_probe(72, 192, 3072, 1, 40)
+    two = backend.dependent_launch_probe(72, 192, 768, 2, 40)
+    three = backend.dependent_launch_probe(72, 192, 768, 3, 40)
+    floor_us = node768 * launches
+    return {"what": "dependent graph nodes that only hand a 768-float vector from 192 workgroups to the next node's 192 (mynah_hip_dependent_launch_probe): "
+                    "no weights, no caches",
+            "node_us": round(node768, 3), "node_us_3072_floats": round(node3072, 3), "dependent_launches_per_step": launches,
+            "floor_us": round(floor_us, 1), "step_over_floor": round(step_us / floor_us, 3),
+            "node_us_two_chains_side_by_side": round(two, 3), "node_us_three_chains_side_by_side": round(three, 3)}
+
+
 def csrc_hash():
     import glob
     import hashlib
@@ -379,6 +395,8 @@ def main():
 
     b1 = time_config(pkg, synth, backend, qtype, [1023], [256], 1024, args.steps, args.warmup)
     b1["traffic_valid"] = args.quant == "int8"
+    # 6 stage kernels x 12 layers + begin, end, head projection, head softmax
+    floor = None if args.launches else latency_floor(backend, b1["step_us"], 6 * b1["layers"] + 4)
     int4 = None
     if args.quant == "int8" and not args.skip_int4:
         int4 = time_config(pkg, synth, backend, pkg.INT4, [1023], [256], 1024, max(args.steps // 3, 20), max(args.warmup // 3, 6), stages=False)
@@ -431,6 +449,8 @@ def main():
                    "rotating_sets": ROTATE},
         "roofline": roofline(b1),
     }
+    result["roofline"]["latency_floor"] = floor
+    result["config"]["step_over_latency_floor"] = floor["step_over_floor"]
     if b1["persistent_step_us"] is not None:
         result["persistent_form"] = {"what": "the same step as ONE persistent launch (graph mode 2, opt-in): stage hand-overs through tagged "
                                              "(value, tag) pairs in memory instead of kernel boundaries",

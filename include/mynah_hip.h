@@ -433,6 +433,16 @@ int mynah_hip_timer_end(void *state, float *milliseconds, char *error, size_t er
 /* Streams `bytes` of backend-owned scratch through the chip (read+write) so that the last-level
  * cache holds none of the caller's data: used between timed iterations. */
 int mynah_hip_flush_cache(void *state, size_t bytes, char *error, size_t error_capacity);
+/* What one dependent stage costs on this device with the bytes taken out (no counterpart in the reference: a measurement
+ * helper like the timers above).  Runs `nodes` kernel nodes as one captured graph on the backend's stream, `repeats` times:
+ * every one of a node's `workgroups` workgroups reads the whole `floats`-long vector the node before it wrote (as a matvec
+ * stage of the decode step reads its activation row, written by workgroups on every XCD), reduces it and writes its share
+ * of the next vector.  *node_us = elapsed time (HIP events on the backend's stream) / (repeats * nodes).  chains > 1 (up
+ * to 3) runs that many independent chains side by side, each on a stream of its own, forked from and joined to the
+ * backend's stream once per repeat; *node_us is still elapsed / (repeats * nodes), so a value equal to the one-chain
+ * figure means the chains overlap fully and `chains` times it that they do not overlap at all.  Synchronises. */
+int mynah_hip_dependent_launch_probe(void *state, int nodes, int workgroups, int floats, int chains, int repeats, float *node_us,
+                                     char *error, size_t error_capacity);
 /* How mynah_hip_decoder_step runs: 0 = every stage kernel a launch of its own, 1 (default) = the step replayed as a
  * captured HIP graph, 2 = one persistent launch for the whole step where it applies (one or two streams, int8 / int4
  * weights, width 768 / FFN 3072 / 64-wide heads, attention units and row stages fitting the chip side by side), else as
@@ -440,6 +450,13 @@ int mynah_hip_flush_cache(void *state, size_t bytes, char *error, size_t error_c
  * bounded (MYNAH_HIP_PERSIST_SPIN polls, default 2^20), and a step that gave one up is reported by the next call that
  * synchronises.  MYNAH_HIP_GRAPH in the environment at open sets the initial value. */
 int mynah_hip_set_graph_mode(void *state, int enabled, char *error, size_t error_capacity);
+/* Lanes of mynah_hip_decoder_step above two streams: the batch is cut into `lanes` groups (1..3) that step side by side,
+ * each on a HIP stream of its own with rows and work tables of its own, forked from and joined to the backend's stream
+ * (one captured graph with a branch per lane).  The reference serves up to MYNAH_MAX_BATCH streams in one pass over
+ * each weight (src/qmat.c:820-888); here a lane is such a pass, and the lanes overlap each other's launch gaps.  A
+ * stream's arithmetic does not depend on which streams share its lane, so every lane count gives the same bits.
+ * 0 (default): chosen from the batch size.  MYNAH_HIP_LANES in the environment at open sets the initial value. */
+int mynah_hip_set_step_lanes(void *state, int lanes, char *error, size_t error_capacity);
 /* Bytes of device memory held by the weight cache (packed weights + scales + vectors). */
 size_t mynah_hip_cached_weight_bytes(void *state);
 

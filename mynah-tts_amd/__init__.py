@@ -147,6 +147,8 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_timer_end.argtypes = [_vp, C.POINTER(C.c_float), *_err]
     lib.mynah_hip_flush_cache.argtypes = [_vp, _sz, *_err]
     lib.mynah_hip_set_graph_mode.argtypes = [_vp, C.c_int, *_err]
+    lib.mynah_hip_set_step_lanes.argtypes = [_vp, C.c_int, *_err]
+    lib.mynah_hip_dependent_launch_probe.argtypes = [_vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), *_err]
     lib.mynah_hip_cached_weight_bytes.argtypes = [_vp]
     lib.mynah_hip_cached_weight_bytes.restype = _sz
     return lib
@@ -416,6 +418,17 @@ class Backend:
 
     def set_graph_mode(self, enabled):
         self._call("mynah_hip_set_graph_mode", C.c_int(int(enabled)))
+
+    def dependent_launch_probe(self, nodes=72, workgroups=192, floats=768, chains=1, repeats=20):
+        """Microseconds per dependent graph node that only hands a `floats`-long vector to the next node (no weights, no caches)."""
+        us = C.c_float(0.0)
+        self._call("mynah_hip_dependent_launch_probe", C.c_int(nodes), C.c_int(workgroups), C.c_int(floats), C.c_int(chains), C.c_int(repeats),
+                   C.byref(us))
+        return float(us.value)
+
+    def set_step_lanes(self, lanes):
+        """Groups a resident step above two streams is cut into, each stepping on a stream of its own (0: chosen from the batch size)."""
+        self._call("mynah_hip_set_step_lanes", C.c_int(int(lanes)))
 
     def cached_weight_bytes(self):
         return self.lib.mynah_hip_cached_weight_bytes(self.state)

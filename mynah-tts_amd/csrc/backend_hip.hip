@@ -359,8 +359,32 @@ static void hip_close(void *opaque) {
     if (st->persist_abort_host != nullptr) (void)hipHostFree(st->persist_abort_host);
     if (st->ev0 != nullptr) (void)hipEventDestroy(st->ev0);
     if (st->ev1 != nullptr) (void)hipEventDestroy(st->ev1);
+    for (int i = 1; i < kMaxLanes; ++i) {
+        if (st->lane_streams[i] != nullptr) {
+            (void)hipStreamSynchronize(st->lane_streams[i]);
+            (void)hipStreamDestroy(st->lane_streams[i]);
+        }
+        if (st->lane_done[i] != nullptr) (void)hipEventDestroy(st->lane_done[i]);
+    }
+    if (st->lane_fork != nullptr) (void)hipEventDestroy(st->lane_fork);
     if (st->stream != nullptr) (void)hipStreamDestroy(st->stream);
     delete st;
+}
+
+int lane_stream(State *st, int lane, hipStream_t *stream, char *error, size_t capacity) {
+    if (lane < 0 || lane >= kMaxLanes) {
+        set_error(error, capacity, "no such lane");
+        return -1;
+    }
+    if (lane == 0) {
+        *stream = st->stream;
+        return 0;
+    }
+    if (st->lane_fork == nullptr) MYNAH_TRY(hipEventCreateWithFlags(&st->lane_fork, hipEventDisableTiming));
+    if (st->lane_streams[lane] == nullptr) MYNAH_TRY(hipStreamCreateWithFlags(&st->lane_streams[lane], hipStreamNonBlocking));   // default priority
+    if (st->lane_done[lane] == nullptr) MYNAH_TRY(hipEventCreateWithFlags(&st->lane_done[lane], hipEventDisableTiming));
+    *stream = st->lane_streams[lane];
+    return 0;
 }
 
 static int attention_table(State *st, int is_self, const float *const *q, float *const *kc, float *const *vc,
@@ -522,6 +546,8 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
     if (fuse != nullptr && strcmp(fuse, "0") == 0) st->fuse = 0;
     const char *graph = getenv("MYNAH_HIP_GRAPH");   // 0: every stage a launch, 1 (default): captured graph, 2: persistent launch where it applies
     if (graph != nullptr && (strcmp(graph, "0") == 0 || strcmp(graph, "1") == 0 || strcmp(graph, "2") == 0)) st->graph_mode = graph[0] - '0';
+    const char *lanes = getenv("MYNAH_HIP_LANES");   // lanes of a resident step above two streams; unset or 0: chosen from the batch size
+    if (lanes != nullptr && lanes[0] >= '0' && lanes[0] <= '0' + kMaxLanes && lanes[1] == '\0') st->step_lanes = lanes[0] - '0';
     const char *spin = getenv("MYNAH_HIP_PERSIST_SPIN");
     if (spin != nullptr && spin[0] != '\0') st->persist_spin_limit = (unsigned)strtoul(spin, nullptr, 10);
     const char *row_wgs = getenv("MYNAH_HIP_PERSIST_ROW_WGS");
@@ -1256,6 +1282,16 @@ extern "C" int mynah_hip_set_graph_mode(void *opaque, int enabled, char *error, 
         return -1;
     }
     st->graph_mode = enabled;
+    return 0;
+}
+extern "C" int mynah_hip_set_step_lanes(void *opaque, int lanes, char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    if (lanes < 0 || lanes > kMaxLanes) {
+        set_error(error, capacity, "step lanes: 0 (chosen from the batch size) to 3");
+        return -1;
+    }
+    st->step_lanes = lanes;
     return 0;
 }
 extern "C" size_t mynah_hip_cached_weight_bytes(void *opaque) {

@@ -28,6 +28,11 @@ constexpr int kStepUnitRows = 128;   // cache rows per attention unit (workgroup
 // separate fold kernel runs once (every workgroup folding every stream would outweigh one extra launch) and
 // workgroups of units a stream does not have leave before requesting anything.
 constexpr int kConsumerFoldMaxBatch = 2;
+constexpr int kMaxLanes = 3;         // groups of a batch's streams that step side by side, each on a stream of its own (a process has four
+                                     // hardware queues here: with a fourth stream in use two of them share one, and chains that share a queue run one after the other)
+constexpr int kLaneStreams = 8;      // streams per lane when the caller names no lane count: one weight pass serves eight, so nine to sixteen streams step
+                                     // as two lanes (measured, sixteen uniform streams: 1048 us in one lane, 856 us in two, 942 us in three; eight ragged
+                                     // streams: 602 / 596 / 633 us -- a lane of four takes 480 us alone, and two chains side by side 1.24 times one)
 constexpr int kStepRecord = 68;      // 64-bit slots of one attention partial of the persistent step: out[64] | max | sum | two unused
 
 // ---- error plumbing (0 / -1 + message, src/backend.c:137-139) ----
@@ -114,6 +119,11 @@ struct State {
     int cu_count = 256;
     int qtype = MYNAH_HIP_F32;
     int arith = MYNAH_HIP_ARITH_STRICT;
+    int step_lanes = 0;   // lanes of a resident step above two streams (0: chosen from the batch size)
+    // the streams lanes 1.. step on, and the events that fork them from and join them to `stream` (created at first use, shared
+    // by every decoder of the backend: more streams would not mean more hardware queues)
+    hipStream_t lane_streams[kMaxLanes] = {};
+    hipEvent_t lane_fork = nullptr, lane_done[kMaxLanes] = {};
     int graph_mode = 1;   // resident step: 0 = every stage kernel a launch, 1 = captured graph, 2 = one persistent launch where it applies (else graph)
     // persistent step: word a workgroup sets when a bounded wait gave up (pinned host memory, mapped), polls a wait may make,
     // and an override of the row stages' workgroup count (0 = chosen from the batch)
@@ -156,6 +166,9 @@ struct State {
     int fuse = 1;
     char deferred_error[160] = {0};
 };
+
+// The stream of lane `lane` (0: the backend's own), created at first use (backend_hip.hip).
+int lane_stream(State *st, int lane, hipStream_t *stream, char *error, size_t capacity);
 
 // First statement of every entry point that is not itself part of the seam fusion: launches what is held back, so that
 // the stream holds every earlier call's work before this one adds its own.

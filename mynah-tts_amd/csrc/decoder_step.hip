@@ -51,13 +51,22 @@ struct mynah_hip_decoder {
     size_t records_bytes = 0;
     int self_slots = 0, cross_slots = 0;   // workgroups of the many-stream attention kernels that the device holds at once
     unsigned item_epoch = 0;                    // next step counter for the tables (24 bits, never 0)
-    mynah::StepSlots last_slots;                // of the last step (the single-stage measurement graphs rebuild the tables from it)
+    mynah::StepSlots last_slots;                // of the last step of this lane
+    mynah::StepSlots last_batch_slots;          // of the last step, every stream of it (the single-stage measurement graphs rebuild the tables from it)
+    int last_lanes = 1;                         // lanes the last step ran in
+    int last_batch = 0;                         // streams of the last step
     int max_units = 0;
     bool fused_attention = false;
-    hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};
-    int eager_steps[mynah::kMaxBatch + 1] = {};   // a batch size runs eagerly once before it is captured
+    hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};   // by stream count: this lane's layer kernels as one chain of kernel nodes
+    int eager_steps[mynah::kMaxBatch + 1] = {};   // a stream count runs eagerly once before it is captured
     hipGraphExec_t stage_graphs[MYNAH_HIP_STAGE_COUNT][mynah::kMaxBatch + 1] = {};   // single-stage graphs (measurement only)
     int arith = 0;
+    // Lanes: a batch above two streams is cut into groups that step side by side, each on a stream of its own with
+    // workspaces, slot table and work tables of its own (a sibling decoder that shares this one's weights).  A stream's
+    // arithmetic does not depend on who else is in its group, so the cut changes no bit of any output; what it buys is
+    // that one group's launch gaps and staging phases are filled by the others' work.  lanes[0] is this decoder.
+    std::vector<mynah_hip_decoder *> lanes;
+    bool is_lane = false;
     // the step as one persistent launch (one or two streams): per-layer pointer table, exchange area and its tag counter
     mynah::PersistLayer *persist_layers = nullptr;
     unsigned long long *persist_exchange = nullptr;
@@ -229,6 +238,80 @@ int decoder_enqueue_layers(State *st, mynah_hip_decoder *d, int batch, char *err
     return enqueue_layers(st, d, batch, error, capacity, kAllStages, false);
 }
 
+// The rows, slot table, partial areas and work tables one group of streams steps on: the owner's, and each lane's.
+static int allocate_workspaces(State *st, mynah_hip_decoder *d, char *error, size_t capacity) {
+    int rc = 0;
+    const size_t w = d->width, xw = d->xw;
+    const size_t B = kMaxBatch;
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->x), B * w * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->qkv), B * 3 * w * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->attn), B * w * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->qx), B * (xw ? xw : 4) * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->ctx), B * (xw ? xw : 4) * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->hidden), B * d->ffn * sizeof(float)), "malloc", error, capacity);
+    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->dev_slots), sizeof(StepSlots)), "malloc", error, capacity);
+    const size_t hw_max = d->head_width > d->cross_head_width ? d->head_width : d->cross_head_width;
+    const size_t heads_max = d->heads > d->cross_heads ? d->heads : d->cross_heads;
+    if (rc == 0) rc |= ensure_attention_workspace(st, B, heads_max, hw_max, d->capacity, error, capacity);
+    if (rc == 0) {
+        const char *env = getenv("MYNAH_HIP_FUSED_ATTENTION");
+        const LayerWeights &l0 = d->lw[0];
+        d->fused_attention = !(env != nullptr && strcmp(env, "0") == 0) &&
+                             step_attention_supported(l0.qkv->qtype, w, d->heads, d->head_width) &&
+                             (xw == 0 || (l0.q_cross->qtype == l0.qkv->qtype &&
+                                          step_attention_supported(l0.q_cross->qtype, w, d->cross_heads, d->cross_head_width)));
+        d->max_units = (int)((d->capacity + kStepUnitRows - 1) / kStepUnitRows) + 1;
+        if (!d->fused_attention) {
+            const size_t chunks = (d->capacity + kAttnChunk - 1) / kAttnChunk + 1;
+            rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->seam_partial), B * heads_max * chunks * (hw_max + 4) * sizeof(float)),
+                            "malloc", error, capacity);
+        }
+        if (d->fused_attention) {
+            const size_t floats = B * heads_max * (size_t)d->max_units * hw_max;
+            rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial), floats * sizeof(float)), "malloc", error, capacity);
+            if (rc == 0)
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial_ml), B * heads_max * 2 * (size_t)d->max_units * sizeof(float)),
+                                "malloc", error, capacity);
+            // one entry per workgroup of the largest attention grid (kMaxBatch streams), self and cross
+            if (rc == 0)
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->self_items),
+                                          (size_t)step_attention_grid((int)d->heads, kMaxBatch, d->max_units, 1, true) * sizeof(StepItem)), "malloc", error, capacity);
+            // The launches fold their own partials unless switched off, the wait has no abort word to report through, or
+            // a (stream, head)'s records do not fit the LDS every launch may use without asking (long caches: the fold kernel then)
+            const char *fold_env = getenv("MYNAH_HIP_FOLD_IN_LAUNCH");
+            const bool fold_in_launch = !(fold_env != nullptr && strcmp(fold_env, "0") == 0) && st->persist_abort_dev != nullptr &&
+                                        d->layers < 255 && step_fold_lds_bytes(d->max_units) <= 40 * 1024;
+            if (rc == 0 && fold_in_launch) {
+                d->records_bytes = B * heads_max * (size_t)d->max_units * kStepRecord * sizeof(unsigned long long);
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->self_records), d->records_bytes), "malloc", error, capacity);
+                if (rc == 0) rc |= hip_check(hipMemset(d->self_records, 0, d->records_bytes), "memset", error, capacity);   // tag 0 is never waited for
+                if (rc == 0 && xw != 0) {
+                    rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->cross_records), d->records_bytes), "malloc", error, capacity);
+                    if (rc == 0) rc |= hip_check(hipMemset(d->cross_records, 0, d->records_bytes), "memset", error, capacity);
+                }
+            }
+            if (rc == 0) {
+                // Chunks per workgroup: one, unless MYNAH_HIP_ATTN_SLOTS names a number of workgroup slots to fit the launch into
+                // ("device": what the device holds of this kernel at once).  Measured with eight ragged streams, same box, twice
+                // each: grouped to fit the device (pairs of chunks, one round of workgroups instead of two) 654 us per step,
+                // one chunk per workgroup 649 us -- the second chunk of a pair waits for its rows a full round trip after the first.
+                d->self_slots = d->cross_slots = 1 << 30;
+                const char *slots_env = getenv("MYNAH_HIP_ATTN_SLOTS");
+                if (slots_env != nullptr && strcmp(slots_env, "device") == 0) {
+                    d->self_slots = step_attention_slots(l0.qkv->qtype, (int)w, d->max_units, 1, d->self_records != nullptr);
+                    d->cross_slots = xw != 0 ? step_attention_slots(l0.q_cross->qtype, (int)w, d->max_units, 0, d->cross_records != nullptr) : 0;
+                } else if (slots_env != nullptr && atoi(slots_env) > 0) {
+                    d->self_slots = d->cross_slots = atoi(slots_env);
+                }
+            }
+            if (rc == 0 && xw != 0)
+                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->cross_items),
+                                          (size_t)step_attention_grid((int)d->cross_heads, kMaxBatch, d->max_units, 0, true) * sizeof(StepItem)), "malloc", error, capacity);
+        }
+    }
+    return rc;
+}
+
 static int per_layer_vector(State *st, const float *const *arr, size_t layer, size_t n, const float **dev, char *error,
                             size_t capacity) {
     *dev = nullptr;
@@ -244,6 +327,11 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
     State *st = enter_state(opaque);
     if (d == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
+    for (size_t i = 1; i < d->lanes.size(); ++i) {   // the lanes' streams have joined the backend's stream after every step
+        d->lanes[i]->lanes.clear();
+        mynah_hip_decoder_destroy(opaque, d->lanes[i]);
+    }
+    d->lanes.clear();
     for (auto &g : d->graphs)
         if (g != nullptr) (void)hipGraphExecDestroy(g);
     for (auto &row : d->stage_graphs)
@@ -323,73 +411,7 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
     if (rc == 0) rc |= cached_vector(st, desc->norm_out, w, &d->norm_out, error, capacity);
     if (rc == 0) rc |= cached_vector(st, desc->norm_out_bias, w, &d->norm_out_b, error, capacity);
     if (rc == 0 && desc->position != nullptr) rc |= cached_vector(st, desc->position, d->capacity * w, &d->position, error, capacity);
-    const size_t B = kMaxBatch;
-    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->x), B * w * sizeof(float)), "malloc", error, capacity);
-    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->qkv), B * 3 * w * sizeof(float)), "malloc", error, capacity);
-    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->attn), B * w * sizeof(float)), "malloc", error, capacity);
-    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->qx), B * (xw ? xw : 4) * sizeof(float)), "malloc", error, capacity);
-    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->ctx), B * (xw ? xw : 4) * sizeof(float)), "malloc", error, capacity);
-    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->hidden), B * d->ffn * sizeof(float)), "malloc", error, capacity);
-    if (rc == 0) rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->dev_slots), sizeof(StepSlots)), "malloc", error, capacity);
-    const size_t hw_max = d->head_width > d->cross_head_width ? d->head_width : d->cross_head_width;
-    const size_t heads_max = d->heads > d->cross_heads ? d->heads : d->cross_heads;
-    if (rc == 0) rc |= ensure_attention_workspace(st, B, heads_max, hw_max, d->capacity, error, capacity);
-    if (rc == 0) {
-        const char *env = getenv("MYNAH_HIP_FUSED_ATTENTION");
-        const LayerWeights &l0 = d->lw[0];
-        d->fused_attention = !(env != nullptr && strcmp(env, "0") == 0) &&
-                             step_attention_supported(l0.qkv->qtype, w, d->heads, d->head_width) &&
-                             (xw == 0 || (l0.q_cross->qtype == l0.qkv->qtype &&
-                                          step_attention_supported(l0.q_cross->qtype, w, d->cross_heads, d->cross_head_width)));
-        d->max_units = (int)((d->capacity + kStepUnitRows - 1) / kStepUnitRows) + 1;
-        if (!d->fused_attention) {
-            const size_t chunks = (d->capacity + kAttnChunk - 1) / kAttnChunk + 1;
-            rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->seam_partial), B * heads_max * chunks * (hw_max + 4) * sizeof(float)),
-                            "malloc", error, capacity);
-        }
-        if (d->fused_attention) {
-            const size_t floats = B * heads_max * (size_t)d->max_units * hw_max;
-            rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial), floats * sizeof(float)), "malloc", error, capacity);
-            if (rc == 0)
-                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->partial_ml), B * heads_max * 2 * (size_t)d->max_units * sizeof(float)),
-                                "malloc", error, capacity);
-            // one entry per workgroup of the largest attention grid (kMaxBatch streams), self and cross
-            if (rc == 0)
-                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->self_items),
-                                          (size_t)step_attention_grid((int)d->heads, kMaxBatch, d->max_units, 1, true) * sizeof(StepItem)), "malloc", error, capacity);
-            // The launches fold their own partials unless switched off, the wait has no abort word to report through, or
-            // a (stream, head)'s records do not fit the LDS every launch may use without asking (long caches: the fold kernel then)
-            const char *fold_env = getenv("MYNAH_HIP_FOLD_IN_LAUNCH");
-            const bool fold_in_launch = !(fold_env != nullptr && strcmp(fold_env, "0") == 0) && st->persist_abort_dev != nullptr &&
-                                        d->layers < 255 && step_fold_lds_bytes(d->max_units) <= 40 * 1024;
-            if (rc == 0 && fold_in_launch) {
-                d->records_bytes = B * heads_max * (size_t)d->max_units * kStepRecord * sizeof(unsigned long long);
-                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->self_records), d->records_bytes), "malloc", error, capacity);
-                if (rc == 0) rc |= hip_check(hipMemset(d->self_records, 0, d->records_bytes), "memset", error, capacity);   // tag 0 is never waited for
-                if (rc == 0 && xw != 0) {
-                    rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->cross_records), d->records_bytes), "malloc", error, capacity);
-                    if (rc == 0) rc |= hip_check(hipMemset(d->cross_records, 0, d->records_bytes), "memset", error, capacity);
-                }
-            }
-            if (rc == 0) {
-                // Chunks per workgroup: one, unless MYNAH_HIP_ATTN_SLOTS names a number of workgroup slots to fit the launch into
-                // ("device": what the device holds of this kernel at once).  Measured with eight ragged streams, same box, twice
-                // each: grouped to fit the device (pairs of chunks, one round of workgroups instead of two) 654 us per step,
-                // one chunk per workgroup 649 us -- the second chunk of a pair waits for its rows a full round trip after the first.
-                d->self_slots = d->cross_slots = 1 << 30;
-                const char *slots_env = getenv("MYNAH_HIP_ATTN_SLOTS");
-                if (slots_env != nullptr && strcmp(slots_env, "device") == 0) {
-                    d->self_slots = step_attention_slots(l0.qkv->qtype, (int)w, d->max_units, 1, d->self_records != nullptr);
-                    d->cross_slots = xw != 0 ? step_attention_slots(l0.q_cross->qtype, (int)w, d->max_units, 0, d->cross_records != nullptr) : 0;
-                } else if (slots_env != nullptr && atoi(slots_env) > 0) {
-                    d->self_slots = d->cross_slots = atoi(slots_env);
-                }
-            }
-            if (rc == 0 && xw != 0)
-                rc |= hip_check(hipMalloc(reinterpret_cast<void **>(&d->cross_items),
-                                          (size_t)step_attention_grid((int)d->cross_heads, kMaxBatch, d->max_units, 0, true) * sizeof(StepItem)), "malloc", error, capacity);
-        }
-    }
+    if (rc == 0) rc |= allocate_workspaces(st, d, error, capacity);
     if (rc == 0) {
         const LayerWeights &l0 = d->lw[0];
         d->qtype = l0.qkv->qtype;
@@ -532,6 +554,147 @@ static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_
 }  // namespace mynah
 
 namespace mynah {
+
+// ---- lanes: groups of a batch's streams that step side by side --------------------------------------------------
+// A sibling decoder for one lane: the owner's shape and (cached, shared) weights, rows and tables of its own.
+static mynah_hip_decoder *new_lane(State *st, const mynah_hip_decoder *owner, char *error, size_t capacity) {
+    mynah_hip_decoder *l = new (std::nothrow) mynah_hip_decoder();
+    if (l == nullptr) {
+        set_error(error, capacity, "out of memory creating a decoder lane");
+        return nullptr;
+    }
+    l->layers = owner->layers; l->width = owner->width; l->heads = owner->heads; l->head_width = owner->head_width;
+    l->ffn = owner->ffn; l->cross_heads = owner->cross_heads; l->cross_head_width = owner->cross_head_width;
+    l->xw = owner->xw; l->capacity = owner->capacity; l->arith = owner->arith; l->qtype = owner->qtype;
+    l->lw = owner->lw;
+    l->norm_out = owner->norm_out; l->norm_out_b = owner->norm_out_b; l->position = owner->position;
+    l->is_lane = true;
+    if (allocate_workspaces(st, l, error, capacity) != 0) {
+        mynah_hip_decoder_destroy(st, l);
+        return nullptr;
+    }
+    return l;
+}
+
+static int ensure_lanes(State *st, mynah_hip_decoder *d, int n, char *error, size_t capacity) {
+    if (d->lanes.empty()) d->lanes.push_back(d);
+    for (int i = 1; i < n; ++i) {
+        hipStream_t unused;
+        if (lane_stream(st, i, &unused, error, capacity) != 0) return -1;
+    }
+    while ((int)d->lanes.size() < n) {
+        mynah_hip_decoder *l = new_lane(st, d, error, capacity);
+        if (l == nullptr) return -1;
+        d->lanes.push_back(l);
+    }
+    return 0;
+}
+
+// How many lanes a batch of this size steps in.  One or two streams run the latency layout in one lane; the head shapes
+// the fused attention kernel does not take share one backend-wide counter area and stay in one lane too.
+static int lanes_for(const State *st, const mynah_hip_decoder *d, int batch) {
+    if (d->is_lane || !d->fused_attention || batch <= kConsumerFoldMaxBatch) return 1;
+    int n = st->step_lanes > 0 ? st->step_lanes : (batch + kLaneStreams - 1) / kLaneStreams;
+    if (n > kMaxLanes) n = kMaxLanes;
+    if (n > batch) n = batch;
+    return n < 1 ? 1 : n;
+}
+
+// Which stream steps in which lane.  Lane sizes are fixed by (batch, lanes) -- the captured graph holds them as kernel
+// arguments -- and the streams are dealt longest first to the lane with the least cache rows so far that still has room,
+// so that ragged batches give the lanes equal work.  Any assignment yields the same bits for every stream.
+struct LanePlan {
+    int lanes;
+    int count[kMaxLanes];
+    int member[kMaxLanes][kMaxBatch];
+};
+static LanePlan plan_lanes(const StepSlots &s, int batch, int lanes) {
+    LanePlan p{};
+    p.lanes = lanes;
+    for (int i = 0; i < lanes; ++i) p.count[i] = batch / lanes + (i < batch % lanes ? 1 : 0);
+    int order[kMaxBatch];
+    for (int b = 0; b < batch; ++b) order[b] = b;
+    const auto cost = [&s](int b) { return (long)s.length[b] + (long)s.memory_length[b]; };
+    for (int i = 1; i < batch; ++i) {   // insertion sort, descending cost, stable
+        const int v = order[i];
+        int j = i;
+        while (j > 0 && cost(order[j - 1]) < cost(v)) { order[j] = order[j - 1]; --j; }
+        order[j] = v;
+    }
+    int filled[kMaxLanes] = {};
+    long load[kMaxLanes] = {};
+    for (int i = 0; i < batch; ++i) {
+        int best = -1;
+        for (int l = 0; l < lanes; ++l)
+            if (filled[l] < p.count[l] && (best < 0 || load[l] < load[best])) best = l;
+        p.member[best][filled[best]++] = order[i];
+        load[best] += cost(order[i]);
+    }
+    return p;
+}
+
+static StepSlots lane_slots(const StepSlots &s, const LanePlan &p, int lane) {
+    StepSlots out;
+    memset(&out, 0, sizeof out);
+    for (int i = 0; i < p.count[lane]; ++i) {
+        const int b = p.member[lane][i];
+        out.self_k[i] = s.self_k[b]; out.self_v[i] = s.self_v[b];
+        out.cross_k[i] = s.cross_k[b]; out.cross_v[i] = s.cross_v[b];
+        out.input[i] = s.input[b]; out.output[i] = s.output[b];
+        out.length[i] = s.length[b]; out.memory_length[i] = s.memory_length[b];
+    }
+    return out;
+}
+
+// One lane's layer kernels for `count` streams on `stream`: as plain launches the first time a lane meets a count (one-time
+// kernel attribute set-up does not belong in a capture) and in graph mode 0, else as the lane's captured graph of that count.
+// A graph is a single chain of kernel nodes -- the form the runtime replays without touching each node on the host; one
+// graph with a branch per lane was measured at 4.2 us of host time per node, 670 us for the two chains of a batch of eight.
+static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t stream, char *error, size_t capacity) {
+    hipStream_t main_stream = st->stream;
+    st->stream = stream;   // the launch wrappers enqueue on the state's stream
+    int rc = 0;
+    if (st->graph_mode == 0 || lane->eager_steps[count] == 0) {
+        lane->eager_steps[count] = 1;
+        rc = enqueue_layers(st, lane, count, error, capacity);
+    } else {
+        if (lane->graphs[count] == nullptr) {
+            hipGraph_t graph = nullptr;
+            rc = hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal), "begin capture", error, capacity);
+            if (rc == 0) {
+                rc = enqueue_layers(st, lane, count, error, capacity);
+                const hipError_t end = hipStreamEndCapture(stream, &graph);
+                if (rc == 0) rc = hip_check(end, "end capture", error, capacity);
+                if (rc == 0) rc = hip_check(hipGraphInstantiate(&lane->graphs[count], graph, nullptr, nullptr, 0), "graph instantiate", error, capacity);
+                if (graph != nullptr) (void)hipGraphDestroy(graph);
+                if (rc != 0) lane->graphs[count] = nullptr;
+            }
+        }
+        if (rc == 0) rc = hip_check(hipGraphLaunch(lane->graphs[count], stream), "graph launch", error, capacity);
+    }
+    st->stream = main_stream;
+    return rc;
+}
+
+// Every lane of a step: lane 0 on the backend's stream, the others on theirs, forked from and joined to it by events.
+static int run_lanes(State *st, mynah_hip_decoder *d, const LanePlan &p, char *error, size_t capacity) {
+    hipStream_t main_stream = st->stream;
+    if (p.lanes > 1) {
+        MYNAH_TRY(hipEventRecord(st->lane_fork, main_stream));
+        for (int i = 1; i < p.lanes; ++i) MYNAH_TRY(hipStreamWaitEvent(st->lane_streams[i], st->lane_fork, 0));
+    }
+    int rc = 0;
+    for (int i = p.lanes - 1; i >= 0 && rc == 0; --i) {   // the owner's lane last: its stream is the one the caller's next work queues behind
+        rc = run_lane(st, d->lanes[i], p.count[i], i == 0 ? main_stream : st->lane_streams[i], error, capacity);
+        if (i > 0 && rc == 0) rc = hip_check(hipEventRecord(st->lane_done[i], st->lane_streams[i]), "lane event", error, capacity);
+    }
+    for (int i = 1; i < p.lanes && rc == 0; ++i) rc = hip_check(hipStreamWaitEvent(main_stream, st->lane_done[i], 0), "lane join", error, capacity);
+    return rc;
+}
+
+}  // namespace mynah
+
+namespace mynah {
 // `count` consecutive step counters (24 bits, never 0).  When the counter wraps, the tags of 2^24 steps ago are forgotten
 // first (outside any capture; the stream orders it).
 int decoder_next_epochs(State *st, mynah_hip_decoder *d, unsigned count, unsigned *first, char *error, size_t capacity) {
@@ -589,29 +752,22 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
         const int taken = try_persistent_step(st, d, slots, batch, error, capacity);
         if (taken != 0) return taken < 0 ? -1 : 0;
     }
-    if (decoder_next_epochs(st, d, 1, &s.epoch, error, capacity) != 0) return -1;
-    d->last_slots = s;
-    if (launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, decoder_item_tables(d, B), error, capacity) != 0) return -1;
-    if (st->graph_mode == 0 || d->eager_steps[B] == 0) {
-        // the first step of a batch size also performs one-time kernel attribute set-up, which does not belong in a capture
-        d->eager_steps[B] = 1;
-        return enqueue_layers(st, d, B, error, capacity);
-    }
-    if (d->graphs[B] == nullptr) {
-        hipGraph_t graph = nullptr;
-        MYNAH_TRY(hipStreamBeginCapture(st->stream, hipStreamCaptureModeThreadLocal));
-        const int rc = enqueue_layers(st, d, B, error, capacity);
-        const hipError_t end = hipStreamEndCapture(st->stream, &graph);
-        if (rc != 0) {
-            if (graph != nullptr) (void)hipGraphDestroy(graph);
+    const int lanes = lanes_for(st, d, B);
+    if (ensure_lanes(st, d, lanes, error, capacity) != 0) return -1;
+    const LanePlan plan = plan_lanes(s, B, lanes);
+    d->last_batch_slots = s;
+    d->last_lanes = lanes;
+    d->last_batch = B;
+    for (int i = 0; i < lanes; ++i) {
+        mynah_hip_decoder *lane = d->lanes[i];
+        StepSlots ls = lanes == 1 ? s : lane_slots(s, plan, i);
+        if (decoder_next_epochs(st, lane, 1, &ls.epoch, error, capacity) != 0) return -1;
+        lane->last_slots = ls;
+        if (launch_step_begin(st, ls, lane->dev_slots, plan.count[i], d->width, d->position, lane->x, d->width, decoder_item_tables(lane, plan.count[i]), error,
+                              capacity) != 0)
             return -1;
-        }
-        MYNAH_TRY(end);
-        const hipError_t inst = hipGraphInstantiate(&d->graphs[B], graph, nullptr, nullptr, 0);
-        (void)hipGraphDestroy(graph);
-        MYNAH_TRY(inst);
     }
-    return hip_check(hipGraphLaunch(d->graphs[B], st->stream), "graph launch", error, capacity);
+    return run_lanes(st, d, plan, error, capacity);
 }
 
 // Measurement helper: enqueue ONE stage of the step (all layers, back to back, as its own captured graph) on the
@@ -626,8 +782,8 @@ extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *
         set_error(error, capacity, "invalid stage arguments");
         return -1;
     }
-    if (!d->fused_attention || d->eager_steps[batch] == 0) {
-        set_error(error, capacity, "stage timing needs the fused step and one earlier step with this batch size");
+    if (!d->fused_attention || d->last_batch != (int)batch) {
+        set_error(error, capacity, "stage timing needs the fused step and follows a step with this batch size");
         return -1;
     }
     if ((stage == MYNAH_HIP_STAGE_CROSS_ATTENTION || stage == MYNAH_HIP_STAGE_CROSS_OUT) && d->xw == 0) {
@@ -635,7 +791,19 @@ extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *
         return -1;
     }
     hipGraphExec_t &exec = d->stage_graphs[stage][batch];
+    // The stage runs in one lane whatever the step does: when the last step ran in several, the owner's slot table holds one
+    // lane's streams only and is rewritten for the whole batch first.  A fresh step counter, as every real step has one, for the
+    // attention launches that fold their own partials: the workgroups that wait for tagged values then really wait.
+    const bool attention_stage = stage == MYNAH_HIP_STAGE_SELF_ATTENTION || stage == MYNAH_HIP_STAGE_CROSS_ATTENTION;
+    if (d->last_lanes > 1 || exec == nullptr || (batch > (size_t)kConsumerFoldMaxBatch && attention_stage)) {
+        if (decoder_next_epochs(st, d, 1, &d->last_batch_slots.epoch, error, capacity) != 0) return -1;
+        if (launch_step_begin(st, d->last_batch_slots, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, decoder_item_tables(d, (int)batch),
+                              error, capacity) != 0)
+            return -1;
+    }
     if (exec == nullptr) {
+        // once as plain launches (one-time kernel attributes of this batch size's builds do not belong in a capture)
+        if (enqueue_layers(st, d, (int)batch, error, capacity, 1u << stage) != 0) return -1;
         hipGraph_t graph = nullptr;
         MYNAH_TRY(hipStreamBeginCapture(st->stream, hipStreamCaptureModeThreadLocal));
         const int rc = enqueue_layers(st, d, (int)batch, error, capacity, 1u << stage);
@@ -651,13 +819,6 @@ extern "C" int mynah_hip_decoder_stage_enqueue(void *opaque, mynah_hip_decoder *
             exec = nullptr;
             return -1;
         }
-    }
-    // a fresh step counter, as every real step has one: the workgroups that wait for tagged values then really wait
-    if (batch > (size_t)kConsumerFoldMaxBatch && (stage == MYNAH_HIP_STAGE_SELF_ATTENTION || stage == MYNAH_HIP_STAGE_CROSS_ATTENTION)) {
-        if (decoder_next_epochs(st, d, 1, &d->last_slots.epoch, error, capacity) != 0) return -1;
-        if (launch_step_begin(st, d->last_slots, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, decoder_item_tables(d, (int)batch),
-                              error, capacity) != 0)
-            return -1;
     }
     return hip_check(hipGraphLaunch(exec, st->stream), "stage graph launch", error, capacity);
 }

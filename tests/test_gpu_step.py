@@ -327,8 +327,9 @@ def test_step_against_compiled_reference_fixture(pkg, backend, synth, nerr, qtyp
     backend.set_quant(0)
 
 
-def test_batch16_two_tiles(pkg, backend, orc, synth, nerr):
-    """MYNAH_MAX_BATCH streams: two weight passes of eight streams each; oracle parity and batched == solo bitwise."""
+def test_batch16_two_lanes(pkg, backend, orc, synth, nerr):
+    """MYNAH_MAX_BATCH streams: two lanes of eight streams side by side (each one pass over the weights); oracle parity,
+    graph replay == eager, batched == solo bitwise, and the same bits in one lane (two passes one after the other) and in three."""
     _announce("one layer ragged b=16 int8")
     rng = np.random.default_rng(16)
     lengths = [int(n) for n in rng.integers(0, 200, size=16)]
@@ -338,20 +339,71 @@ def test_batch16_two_tiles(pkg, backend, orc, synth, nerr):
     streams = synth.decoder_streams(cfg, lengths, mems, seed=6)
     backend.set_quant(1)
     h = Harness(pkg, backend, cfg, weights, streams)
-    want, ks, vs = _oracle_step(orc, cfg, weights, streams, 1)
-    first = h.step()
-    quantised_errors_ok([nerr(first[b], want[b]) for b in range(16)], 2, "b=16 int8, one layer")
-    for b in range(16):
-        h.reset_cache(b)
-    again = h.step()                       # captured graph
-    for b in range(16):
-        assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32))
-    for b in (0, 7, 8, 15):
-        h.reset_cache(b)
-        solo = h.step([b])[0]
-        assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
-    h.close()
-    backend.set_quant(0)
+    try:
+        want, ks, vs = _oracle_step(orc, cfg, weights, streams, 1)
+        first = h.step()
+        quantised_errors_ok([nerr(first[b], want[b]) for b in range(16)], 2, "b=16 int8, one layer")
+        for replay in range(2):                # captured graphs, then their replay
+            for b in range(16):
+                h.reset_cache(b)
+            again = h.step()
+            for b in range(16):
+                assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32)), "replay %d stream %d" % (replay, b)
+        for b in (0, 7, 8, 15):
+            h.reset_cache(b)
+            solo = h.step([b])[0]
+            assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
+        for lanes in (1, 3):
+            backend.set_step_lanes(lanes)
+            for attempt in range(3):           # eager, capture, replay in this lane layout
+                for b in range(16):
+                    h.reset_cache(b)
+                got = h.step()
+                for b in range(16):
+                    assert np.array_equal(got[b].view(np.uint32), first[b].view(np.uint32)), "%d lanes, attempt %d, stream %d" % (lanes, attempt, b)
+    finally:
+        backend.set_step_lanes(0)
+        h.close()
+        backend.set_quant(0)
+
+
+@pytest.mark.parametrize("qtype_name", ["int8", "f32"])
+def test_lanes_keep_every_bit(pkg, backend, synth, qtype_name):
+    """A ragged batch of eight stepped in one, two and three lanes (groups of streams on HIP streams of their own, dealt by
+    cache length): outputs and appended cache rows are the same bits in every layout, eagerly, at capture and on replay, and
+    so is a batch of five that follows on the same decoder (other lane sizes, the lanes' graphs of those sizes)."""
+    _announce("lanes keep every bit, %s" % qtype_name)
+    lengths = [5, 640, 0, 129, 63, 2, 300, 65]
+    mems = [7, 64, 3, 32, 65, 0, 27, 200]
+    cfg = synth.decoder_config(layers=3, capacity=648)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=11)
+    backend.set_quant(QT[qtype_name])
+    h = Harness(pkg, backend, cfg, weights, streams)
+    try:
+        ref = {}
+        for lanes in (1, 2, 3, 2):
+            backend.set_step_lanes(lanes)
+            for which in (list(range(8)), [6, 1, 3, 7, 0]):
+                for attempt in range(3):
+                    for b in which:
+                        h.reset_cache(b)
+                    got = h.step(which)
+                    rows = [tuple(a[:, lengths[b]].copy() for a in h.cache_rows(b)) for b in which]
+                    key = len(which)
+                    if key not in ref:
+                        ref[key] = (got, rows)
+                        assert all(np.isfinite(o).all() for o in got)
+                    for i, b in enumerate(which):
+                        what = "%d lanes, batch %d, attempt %d, stream %d" % (lanes, key, attempt, b)
+                        assert np.array_equal(got[i].view(np.uint32), ref[key][0][i].view(np.uint32)), what
+                        assert np.array_equal(rows[i][0], ref[key][1][i][0]) and np.array_equal(rows[i][1], ref[key][1][i][1]), what + " (appended rows)"
+        for i, b in enumerate([6, 1, 3, 7, 0]):   # and a stream's bits do not depend on the batch it is in
+            assert np.array_equal(ref[5][0][i].view(np.uint32), ref[8][0][b].view(np.uint32))
+    finally:
+        backend.set_step_lanes(0)
+        h.close()
+        backend.set_quant(0)
 
 
 def test_stage_enqueue_leaves_the_step_intact(pkg, backend, synth):
@@ -382,7 +434,7 @@ def test_stage_enqueue_leaves_the_step_intact(pkg, backend, synth):
 
 def test_full_size_ragged_batch8_int8(pkg, backend, orc, synth, nerr):
     """The benchmark's batch-8 configuration at full size (12 layers, self KV up to 2048 rows, 12x64 cross heads, int8):
-    two streams against the oracle, graph replay == eager and batched == solo bit for bit."""
+    four streams against the oracle, graph replay == eager, and EVERY stream bit-identical to the same stream alone."""
     _announce("12 layers int8 ragged b=8 full size")
     self_len, cross_len = synth.ragged_lengths(8, seed=3)
     lengths = [n - 1 for n in self_len]
@@ -393,25 +445,65 @@ def test_full_size_ragged_batch8_int8(pkg, backend, orc, synth, nerr):
     h = Harness(pkg, backend, cfg, weights, streams)
     first = h.step()
     assert all(np.all(np.isfinite(o)) for o in first)
-    check = (1, 6)                                      # the shortest and the longest stream
+    check = (1, 6, 3, 7)                                # the shortest and the longest stream, and two in between
     odec = orc.Decoder(cfg, weights, orc.INT8)
     errs = []
     for b in check:
         s = streams[b]
         want = odec.step([s["k"].copy()], [s["v"].copy()], [s["ck"]], [s["cv"]], [lengths[b]], [cross_len[b]], [s["x"]])[0]
         errs.append(nerr(first[b], want))
-    quantised_errors_ok(errs, 2, "full size b=8 int8")     # 12 layers each: both may have met a rounding boundary
+    quantised_errors_ok(errs, 3, "full size b=8 int8")     # 12 layers each: roughly one (stream, layer) in thirty meets a rounding boundary
     for b in range(8):
         h.reset_cache(b)
     again = h.step()                                    # captured graph
     for b in range(8):
         assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32)), "replay differs for stream %d" % b
-    for b in check:
+    for b in range(8):
         h.reset_cache(b)
         solo = h.step([b])[0]
         assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
     h.close()
     backend.set_quant(0)
+
+
+def test_full_size_batch16_int8(pkg, backend, orc, synth, nerr):
+    """Sixteen streams of the 12-layer int8 stack at full size (self caches of 700 to 1023 rows, memories of 100 to 256 rows), stepped
+    as two lanes of eight: three streams against the oracle, graph replay == eager, and four streams (both lanes, both ends
+    of the length order) bit-identical to themselves alone."""
+    _announce("12 layers int8 b=16 full size")
+    rng = np.random.default_rng(160)
+    lengths = [int(n) for n in rng.integers(700, 1024, size=16)]
+    mems = [int(n) for n in rng.integers(100, 257, size=16)]
+    lengths[5], mems[5] = 1023, 256
+    cfg = synth.decoder_config(layers=12, capacity=1024)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=21)
+    backend.set_quant(1)
+    h = Harness(pkg, backend, cfg, weights, streams)
+    try:
+        first = h.step()
+        assert all(np.all(np.isfinite(o)) for o in first)
+        odec = orc.Decoder(cfg, weights, orc.INT8)
+        errs = []
+        for b in (5, 0, 11):
+            s = streams[b]
+            want = odec.step([s["k"].copy()], [s["v"].copy()], [s["ck"]], [s["cv"]], [lengths[b]], [mems[b]], [s["x"]])[0]
+            errs.append(nerr(first[b], want))
+        quantised_errors_ok(errs, 2, "full size b=16 int8")
+        for replay in range(2):
+            for b in range(16):
+                h.reset_cache(b)
+            again = h.step()
+            for b in range(16):
+                assert np.array_equal(again[b].view(np.uint32), first[b].view(np.uint32)), "replay %d differs for stream %d" % (replay, b)
+        order = sorted(range(16), key=lambda b: lengths[b] + mems[b])
+        for b in (order[0], order[1], order[-1], order[-2]):
+            h.reset_cache(b)
+            solo = h.step([b])[0]
+            assert np.array_equal(solo.view(np.uint32), first[b].view(np.uint32)), "stream %d differs from its solo run" % b
+    finally:
+        h.close()
+        backend.set_quant(0)
 
 
 def test_config2_int4_full_stack_with_head(pkg, backend, orc, synth, nerr):
