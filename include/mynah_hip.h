@@ -447,16 +447,31 @@ int mynah_hip_dependent_launch_probe(void *state, int nodes, int workgroups, int
  * captured HIP graph, 2 = one persistent launch for the whole step where it applies (one or two streams, int8 / int4
  * weights, width 768 / FFN 3072 / 64-wide heads, attention units and row stages fitting the chip side by side), else as
  * 1.  All three give the same bits.  Form 2 waits inside the kernel for other workgroups' results; every such wait is
- * bounded (MYNAH_HIP_PERSIST_SPIN polls, default 2^20), and a step that gave one up is reported by the next call that
- * synchronises.  MYNAH_HIP_GRAPH in the environment at open sets the initial value. */
+ * bounded (MYNAH_HIP_PERSIST_SPIN polls, default 2^20; a value that is not a number fails the open), and a step that gave
+ * one up is repeated in form 0 by the next call that synchronises (mynah_hip_wait_fallbacks).  MYNAH_HIP_GRAPH in the environment at open sets the initial value. */
 int mynah_hip_set_graph_mode(void *state, int enabled, char *error, size_t error_capacity);
 /* Lanes of mynah_hip_decoder_step above two streams: the batch is cut into `lanes` groups (1..3) that step side by side,
  * each on a HIP stream of its own with rows and work tables of its own, forked from and joined to the backend's stream
- * (one captured graph with a branch per lane).  The reference serves up to MYNAH_MAX_BATCH streams in one pass over
+ * by events (every lane replays a captured graph of its own: a chain of kernel nodes).  The reference serves up to MYNAH_MAX_BATCH streams in one pass over
  * each weight (src/qmat.c:820-888); here a lane is such a pass, and the lanes overlap each other's launch gaps.  A
  * stream's arithmetic does not depend on which streams share its lane, so every lane count gives the same bits.
  * 0 (default): chosen from the batch size.  MYNAH_HIP_LANES in the environment at open sets the initial value. */
 int mynah_hip_set_step_lanes(void *state, int lanes, char *error, size_t error_capacity);
+/* How often a resident step was run a second time because one of its workgroups had given up a bounded wait for another
+ * one's result.  Two forms of mynah_hip_decoder_step wait inside a kernel: the persistent launch (graph mode 2) and, in
+ * every mode, the attention launches of more than two streams, whose fold workgroups wait for the attending workgroups
+ * of the same launch (they are numbered behind them and the device starts workgroups in index order, so the ones waited
+ * for are running or done; the bound -- MYNAH_HIP_PERSIST_SPIN polls, default 2^20 -- is there for a device that does
+ * otherwise, or is shared with other work).  A workgroup that gives up sets a host-visible word and leaves, so the launch
+ * always drains.  The next call that synchronises finds the word and, when that step is the only one since the stream
+ * was last idle and no other call has put work behind it, repeats it as plain launches in the form without such waits
+ * (fold kernel, MYNAH_HIP_FOLD_IN_LAUNCH=0's form; the cache rows it appends are the ones the first run wrote to) and
+ * returns its results -- the same bits, later.  So a step followed by mynah_hip_sync, mynah_hip_d2h or mynah_hip_download
+ * never fails for this reason.  With several steps since the last synchronisation, or with work enqueued behind the step
+ * (an output head, a local frame: it has read rows that meant nothing), the synchronising call fails with "gave up a
+ * bounded wait" as before; a caller that wants the repeat there synchronises right after the step.  No counterpart in the
+ * reference, whose CPU step cannot give up. */
+size_t mynah_hip_wait_fallbacks(void *state);
 /* Bytes of device memory held by the weight cache (packed weights + scales + vectors). */
 size_t mynah_hip_cached_weight_bytes(void *state);
 

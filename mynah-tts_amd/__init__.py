@@ -148,6 +148,8 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_flush_cache.argtypes = [_vp, _sz, *_err]
     lib.mynah_hip_set_graph_mode.argtypes = [_vp, C.c_int, *_err]
     lib.mynah_hip_set_step_lanes.argtypes = [_vp, C.c_int, *_err]
+    lib.mynah_hip_wait_fallbacks.argtypes = [_vp]
+    lib.mynah_hip_wait_fallbacks.restype = C.c_size_t
     lib.mynah_hip_dependent_launch_probe.argtypes = [_vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), *_err]
     lib.mynah_hip_cached_weight_bytes.argtypes = [_vp]
     lib.mynah_hip_cached_weight_bytes.restype = _sz
@@ -425,6 +427,10 @@ class Backend:
         self._call("mynah_hip_dependent_launch_probe", C.c_int(nodes), C.c_int(workgroups), C.c_int(floats), C.c_int(chains), C.c_int(repeats),
                    C.byref(us))
         return float(us.value)
+
+    def wait_fallbacks(self):
+        """Steps that were repeated in the wait-free form because a workgroup had given up a bounded wait."""
+        return int(self.lib.mynah_hip_wait_fallbacks(self.state))
 
     def set_step_lanes(self, lanes):
         """Groups a resident step above two streams is cut into, each stepping on a stream of its own (0: chosen from the batch size)."""

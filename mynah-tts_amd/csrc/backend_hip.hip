@@ -549,7 +549,16 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
     const char *lanes = getenv("MYNAH_HIP_LANES");   // lanes of a resident step above two streams; unset or 0: chosen from the batch size
     if (lanes != nullptr && lanes[0] >= '0' && lanes[0] <= '0' + kMaxLanes && lanes[1] == '\0') st->step_lanes = lanes[0] - '0';
     const char *spin = getenv("MYNAH_HIP_PERSIST_SPIN");
-    if (spin != nullptr && spin[0] != '\0') st->persist_spin_limit = (unsigned)strtoul(spin, nullptr, 10);
+    if (spin != nullptr && spin[0] != '\0') {   // a value that is not a number would read as 0: every wait giving up at once
+        char *end = nullptr;
+        const unsigned long polls = strtoul(spin, &end, 10);
+        if (end == spin || *end != '\0' || polls > 0xffffffffUL) {
+            set_error(error, capacity, "MYNAH_HIP_PERSIST_SPIN is not a number of polls");
+            hip_close(st);
+            return -1;
+        }
+        st->persist_spin_limit = (unsigned)polls;
+    }
     const char *row_wgs = getenv("MYNAH_HIP_PERSIST_ROW_WGS");
     if (row_wgs != nullptr && row_wgs[0] != '\0') st->persist_row_wgs = atoi(row_wgs);
     // the word a persistent step sets when one of its bounded waits gave up: host memory the device writes directly
@@ -614,12 +623,33 @@ int mynah::synchronise(State *st, char *error, size_t capacity) {
         set_error(error, capacity, st->deferred_error);
         st->deferred_error[0] = '\0';
         (void)hipStreamSynchronize(st->stream);
+        st->steps_since_sync = 0;
         return -1;
     }
     MYNAH_TRY(hipStreamSynchronize(st->stream));
     free_pending(st);
+    const unsigned steps = st->steps_since_sync;
+    st->steps_since_sync = 0;
     if (st->persist_abort_host != nullptr && st->persist_abort_host[0] != 0u) {
         st->persist_abort_host[0] = 0u;
+        // A workgroup of a resident step gave up waiting for another one's result (it never hangs: every such wait is bounded).
+        // When that step is the only one since the stream was last idle and nothing was enqueued behind it, its inputs are
+        // still where they were and nobody has read its rows: it runs again here in the form without such waits and the caller
+        // never sees the difference, apart from the time.  With several steps in between, which of them it was cannot be told
+        // and the earlier ones' inputs may be gone; work enqueued behind the step has used rows that meant nothing: an error.
+        if (steps == 1 && st->calls_since_step == 0 && !st->rerunning && st->last_step_decoder != nullptr) {
+            st->rerunning = true;
+            int rc = rerun_last_step_without_waits(st, error, capacity);
+            if (rc == 0) rc = hip_check(hipStreamSynchronize(st->stream), "synchronise", error, capacity);
+            st->rerunning = false;
+            st->steps_since_sync = 0;
+            if (rc == 0 && st->persist_abort_host[0] == 0u) {
+                ++st->wait_fallbacks;
+                return 0;
+            }
+            st->persist_abort_host[0] = 0u;
+            if (rc != 0) return -1;
+        }
         set_error(error, capacity, "resident decode step gave up a bounded wait between its workgroups; its outputs are invalid");
         return -1;
     }
@@ -627,12 +657,14 @@ int mynah::synchronise(State *st, char *error, size_t capacity) {
 }
 
 extern "C" int mynah_hip_d2h(void *opaque, const float *dev_ptr, float *host, size_t n, char *error, size_t capacity) {
-    State *st = enter_state(opaque);
+    State *st = enter_state(opaque, false);
     size_t bytes = 0;
     if (st == nullptr || host == nullptr || dev_ptr == nullptr || !float_bytes(n, &bytes)) {
         set_error(error, capacity, "invalid d2h arguments");
         return -1;
     }
+    // a resident step still on the stream is waited for first: should it have given up a wait it is repeated before its rows are copied
+    if (st->steps_since_sync != 0 && synchronise(st, error, capacity) != 0) return -1;
     if (bytes != 0) MYNAH_TRY(hipMemcpyAsync(host, dev_ptr, bytes, hipMemcpyDeviceToHost, st->stream));
     return synchronise(st, error, capacity);
 }
@@ -654,7 +686,7 @@ extern "C" int mynah_hip_download(void *opaque, const float *dev_ptr, float *hos
 }
 
 extern "C" int mynah_hip_sync(void *opaque, char *error, size_t capacity) {
-    State *st = enter_state(opaque);
+    State *st = enter_state(opaque, false);
     MYNAH_NEED_STATE(st);
     return synchronise(st, error, capacity);
 }
@@ -726,8 +758,9 @@ static int seam_flush(State *st, char *error, size_t capacity) {
     return 0;
 }
 
-State *mynah::enter_state(void *opaque) {
+State *mynah::enter_state(void *opaque, bool enqueues) {
     State *st = static_cast<State *>(opaque);
+    if (st != nullptr && enqueues) ++st->calls_since_step;
     if (st != nullptr && st->pending.kind != PendingOp::kNone) {
         char message[sizeof st->deferred_error] = {0};
         if (seam_flush(st, message, sizeof message) != 0 && st->deferred_error[0] == '\0')
@@ -1293,6 +1326,9 @@ extern "C" int mynah_hip_set_step_lanes(void *opaque, int lanes, char *error, si
     }
     st->step_lanes = lanes;
     return 0;
+}
+extern "C" size_t mynah_hip_wait_fallbacks(void *opaque) {
+    return opaque != nullptr ? (size_t)static_cast<State *>(opaque)->wait_fallbacks : 0;
 }
 extern "C" size_t mynah_hip_cached_weight_bytes(void *opaque) {
     return opaque != nullptr ? static_cast<State *>(opaque)->weight_bytes : 0;

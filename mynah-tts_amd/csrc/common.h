@@ -119,6 +119,18 @@ struct State {
     int cu_count = 256;
     int qtype = MYNAH_HIP_F32;
     int arith = MYNAH_HIP_ARITH_STRICT;
+    // The last resident step since the stream was last waited for, kept so that it can be run again in the form without waits
+    // between workgroups should one of its bounded waits give up: its decoder, every stream's slot, how many steps were
+    // enqueued since the last synchronisation (only a single one can be repeated: the inputs of earlier ones may be gone),
+    // whether anything was enqueued behind it (that work has read the step's rows and cannot be repeated from here), and how
+    // often a step was repeated.
+    mynah_hip_decoder *last_step_decoder = nullptr;
+    StepSlots last_step_slots;
+    int last_step_batch = 0;
+    unsigned steps_since_sync = 0;
+    unsigned calls_since_step = 0;   // entry points since that step that may have put work behind it (work that has read its rows)
+    bool rerunning = false;
+    unsigned long long wait_fallbacks = 0;
     int step_lanes = 0;   // lanes of a resident step above two streams (0: chosen from the batch size)
     // the streams lanes 1.. step on, and the events that fork them from and join them to `stream` (created at first use, shared
     // by every decoder of the backend: more streams would not mean more hardware queues)
@@ -170,9 +182,15 @@ struct State {
 // The stream of lane `lane` (0: the backend's own), created at first use (backend_hip.hip).
 int lane_stream(State *st, int lane, hipStream_t *stream, char *error, size_t capacity);
 
+// Runs the step recorded in the state again, as plain launches in the form whose workgroups never wait for each other (fold
+// kernel behind the attention launches, no persistent launch); the cache rows it appends are the ones the first run wrote to
+// (decoder_step.hip).
+int rerun_last_step_without_waits(State *st, char *error, size_t capacity);
+
 // First statement of every entry point that is not itself part of the seam fusion: launches what is held back, so that
 // the stream holds every earlier call's work before this one adds its own.
-State *enter_state(void *opaque);
+// `enqueues`: the entry point may put work on the stream (false for those that only wait or copy to the host).
+State *enter_state(void *opaque, bool enqueues = true);
 
 // weight cache (backend_hip.hip)
 int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qtype, const CachedWeight **out,

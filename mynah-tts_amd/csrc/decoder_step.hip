@@ -327,6 +327,7 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
     State *st = enter_state(opaque);
     if (d == nullptr) return;
     if (st != nullptr) (void)hipStreamSynchronize(st->stream);
+    if (st != nullptr && st->last_step_decoder == d) st->last_step_decoder = nullptr;
     for (size_t i = 1; i < d->lanes.size(); ++i) {   // the lanes' streams have joined the backend's stream after every step
         d->lanes[i]->lanes.clear();
         mynah_hip_decoder_destroy(opaque, d->lanes[i]);
@@ -462,14 +463,6 @@ extern "C" int mynah_hip_decoder_create(void *opaque, const mynah_hip_decoder_de
     return 0;
 }
 
-#ifdef MYNAH_PERSIST_PROBE
-static unsigned long long *g_persist_probe = nullptr;
-extern "C" int mynah_hip_debug_probe(unsigned long long *host, size_t words) {   // development builds only
-    if (g_persist_probe == nullptr) return -1;
-    return hipMemcpy(host, g_persist_probe, words * sizeof(unsigned long long), hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
-}
-#endif
-
 namespace mynah {
 
 // The step as one persistent launch, when this batch fits it: one or two streams, int8 / int4 weights, the stack's own
@@ -506,11 +499,10 @@ static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_
     const int grid = st->cu_count;
     const int attn = step_persistent_attention_workgroups(a);
     a.attention_wgs = attn;
-    // Row stages count their workgroups from the end of the grid, attention roles from its start: with room for both, a
-    // workgroup has one kind of role and requests its next stage's operands a whole stage ahead.
     // Row stages count their workgroups from the end of the grid, attention roles from its start: with room for both a
-    // workgroup has one kind of role.  Rows per workgroup are what the kernel requests ahead (32 rows of an output
-    // projection and of FFN up, 8 of FFN down); MYNAH_HIP_PERSIST_ROW_WGS spreads the FFN rows over more workgroups.
+    // workgroup has one kind of role and requests its next stage's operands a whole stage ahead.  Rows per workgroup are what
+    // the kernel requests ahead (32 rows of an output projection and of FFN up, 8 of FFN down); MYNAH_HIP_PERSIST_ROW_WGS
+    // spreads the FFN rows over more workgroups.
     a.rows_out = 32;
     a.wgs_out = (768 + a.rows_out - 1) / a.rows_out;
     a.rows_up = 32;
@@ -522,12 +514,9 @@ static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_
     }
     a.wgs_up = (3072 + a.rows_up - 1) / a.rows_up;
     a.wgs_down = (768 + a.rows_down - 1) / a.rows_down;
-    {
-        // a workgroup has one kind of role: when the attention units of these lengths and the row stages do not fit the grid
-        // side by side, the step takes the launched-kernels path
-        const int rows = a.wgs_up > a.wgs_down ? (a.wgs_up > a.wgs_out ? a.wgs_up : a.wgs_out) : (a.wgs_down > a.wgs_out ? a.wgs_down : a.wgs_out);
-        if (attn + rows > grid || (int)batch > rows) return 0;
-    }
+    // When the attention units of these lengths and the row stages do not fit the grid side by side, or a stream's partial
+    // records do not fit a workgroup's LDS, the step takes the launched-kernels path -- decided before a tag range is used up.
+    if (!step_persistent_fits(a, grid)) return 0;
     const unsigned span = 8u * (unsigned)(d->layers + 2);
     if (d->persist_epoch > 0xffffffffu - 2u * span) {   // the tag counter is about to wrap: start over on a cleared area
         if (hip_check(hipMemsetAsync(d->persist_exchange, 0, d->persist_exchange_words * sizeof(unsigned long long), st->stream), "exchange clear", error,
@@ -537,16 +526,6 @@ static int try_persistent_step(State *st, mynah_hip_decoder *d, const mynah_hip_
     }
     a.epoch = d->persist_epoch;
     d->persist_epoch += span;
-#ifdef MYNAH_PERSIST_PROBE
-    {
-        static unsigned long long *probe = nullptr;
-        if (probe == nullptr && hipMalloc(reinterpret_cast<void **>(&probe), 1024 * 32 * sizeof(unsigned long long)) != hipSuccess) probe = nullptr;
-        const char *layer = getenv("MYNAH_PERSIST_PROBE_LAYER");
-        a.probe = probe;
-        a.probe_layer = layer != nullptr ? atoi(layer) : 5;
-        g_persist_probe = probe;
-    }
-#endif
     if (launch_step_persistent(st, a, d->qtype, grid, error, capacity) != 0) return -1;
     return 1;
 }
@@ -748,6 +727,11 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
         s.memory_length[b] = (int)in.memory_length;
     }
     const int B = (int)batch;
+    st->last_step_decoder = d;   // kept so that the step can be repeated should one of its bounded waits give up (synchronise)
+    st->last_step_slots = s;
+    st->last_step_batch = B;
+    ++st->steps_since_sync;
+    st->calls_since_step = 0;
     {
         const int taken = try_persistent_step(st, d, slots, batch, error, capacity);
         if (taken != 0) return taken < 0 ? -1 : 0;
@@ -768,6 +752,30 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
             return -1;
     }
     return run_lanes(st, d, plan, error, capacity);
+}
+
+int mynah::rerun_last_step_without_waits(State *st, char *error, size_t capacity) {
+    mynah_hip_decoder *d = st->last_step_decoder;
+    const int B = st->last_step_batch;
+    if (d == nullptr || B < 1 || B > kMaxBatch) {
+        set_error(error, capacity, "no resident step to repeat");
+        return -1;
+    }
+    StepSlots s = st->last_step_slots;
+    s.epoch = 1;
+    // One lane, every kernel a launch of its own, and no record areas: the attention launches then take the build that
+    // finds its work from the workgroup index and a fold kernel follows each of them -- nothing in this form waits for
+    // another workgroup.  The arithmetic is the one of every other form, so these are the bits the step would have given.
+    unsigned long long *const self_records = d->self_records, *const cross_records = d->cross_records;
+    d->self_records = d->cross_records = nullptr;
+    int rc = launch_step_begin(st, s, d->dev_slots, B, d->width, d->position, d->x, d->width, StepItemTables{}, error, capacity);
+    if (rc == 0) rc = enqueue_layers(st, d, B, error, capacity);
+    d->self_records = self_records;
+    d->cross_records = cross_records;
+    d->last_batch_slots = s;
+    d->last_lanes = 1;
+    d->last_batch = B;
+    return rc;
 }
 
 // Measurement helper: enqueue ONE stage of the step (all layers, back to back, as its own captured graph) on the

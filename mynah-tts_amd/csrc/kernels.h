@@ -166,14 +166,11 @@ struct PersistArgs {
     int wgs_out, rows_out;          // workgroups and rows per workgroup of the [768, 768] output projections
     int wgs_up, rows_up;            // ... of FFN up [3072, 768]
     int wgs_down, rows_down;        // ... of FFN down [768, 3072]
-#ifdef MYNAH_PERSIST_PROBE
-    unsigned long long *probe;      // development builds only: [workgroup][32] clock readings of layer probe_layer
-    int probe_layer;
-#endif
 };
 bool step_persistent_supported(int qtype, size_t width, size_t heads, size_t head_width, size_t ffn, size_t cross_heads, size_t cross_head_width);
 size_t step_persistent_exchange_words(const PersistArgs &args);
 int step_persistent_attention_workgroups(const PersistArgs &args);
+bool step_persistent_fits(const PersistArgs &args, int grid);
 int launch_step_persistent(State *st, const PersistArgs &args, int qtype, int grid, char *error, size_t capacity);
 
 int launch_layernorm(State *st, const float *in, float *out, const float *gain, const float *bias, size_t rows,

@@ -1,6 +1,10 @@
 // The resident decode step as ONE launch: every layer, every stage, in a kernel whose workgroups stay on the chip and hand
 // vectors to each other through memory instead of through kernel boundaries.
 //
+// OPT-IN (graph mode 2), and slower than the default: measured at one stream, int8, 12 layers, 400 us per step against 331 us
+// for the captured graph of stage kernels.  It is kept as the measured answer to "are the kernel boundaries what holds the
+// step": they are not -- a hand-over through memory costs what a graph node's boundary costs.
+//
 // decoder_step_batch (src/graph.c:3127-3284) is a chain of dependent stages, per layer
 //     1  LN + Q/K/V rows + KV append + split-L self-attention  -> partials      (k_step_attention as a launch)
 //     2  fold + O matvec + residual                            -> x             (k_linear)
@@ -21,7 +25,8 @@
 //
 // Every wait is bounded: a poll that exceeds its spin limit (or sees the abort word set) makes its workgroup set the
 // abort word and leave; every other workgroup then runs into the same bound or sees the word, so the grid always drains.
-// The host reports an aborted step at the next synchronisation.  The grid never exceeds what the chip holds at once.
+// The host finds the word at its next synchronisation and repeats the step as launched kernels.  The grid never exceeds
+// what the chip holds at once.
 #include "step_attention_core.h"
 #include "tagged_exchange.h"
 
@@ -494,12 +499,6 @@ __device__ __forceinline__ StreamArgs stream_of(const PersistArgs &a, const int 
     }
 // development builds only: clock readings (100 MHz) of one layer, per workgroup: slot 3 (stage - 1) + {0 before the wait,
 // 1 input there, 2 stage done}
-#ifdef MYNAH_PERSIST_PROBE
-#define MYNAH_STAMP(slot) do { if (threadIdx.x == 0 && a.probe != nullptr && layer == a.probe_layer) a.probe[(size_t)blockIdx.x * 32 + (slot)] = wall_clock64(); } while (0)
-#else
-#define MYNAH_STAMP(slot) do { } while (0)
-#endif
-
 struct SharedBlocks {
     float *s_in;
     unsigned char *smem;
@@ -530,7 +529,6 @@ __device__ __forceinline__ void attention_path(const PersistArgs &a, const Share
         const PersistLayer &lw = a.layers[layer];
         const unsigned t0 = a.epoch + 8u * (unsigned)layer;
         if (r1.active) {
-            MYNAH_STAMP(0);
             if (layer == 0) {
                 for (int i = tid; i < kW; i += kThreads)
                     sh.s_in[i] = s1.pos_row != nullptr ? load_global(s1.input + i) + load_global(s1.pos_row + i) : load_global(s1.input + i);
@@ -538,13 +536,11 @@ __device__ __forceinline__ void attention_path(const PersistArgs &a, const Share
                 fetch_tagged<3, false>(ex.X6 + (size_t)r1.b * kW, sh.s_in, kW, t0, wt);
             }
             MYNAH_LEAVE_IF_DEAD();
-            MYNAH_STAMP(1);
             aw.w = lw.qkv_w; aw.scales = lw.qkv_s; aw.heads = a.heads;
             float *kc = s1.self_k + (size_t)layer * a.capacity * stride_self;
             float *vc = s1.self_v + (size_t)layer * a.capacity * stride_self;
             attention_compute<QT>(g, r1, aw, sh.s_in, kc, vc, s1.length, lw.norm_self_b != nullptr, ex.PS + (size_t)r1.b * ex.ps_stream, a.heads,
                                   t0 + 1u, sh.smem, sh.s_sx, sh.s_scratch, sh.s_proj, sh.s_red, sh.s_wave_ml);
-            MYNAH_STAMP(2);
         }
         if (r3.active) {
             aw.w = lw.qx_w; aw.scales = lw.qx_s; aw.heads = a.cross_heads;
@@ -552,13 +548,10 @@ __device__ __forceinline__ void attention_path(const PersistArgs &a, const Share
             attention_request<QT, false>(g, r3, aw, s3.cross_k != nullptr ? s3.cross_k + at : nullptr, s3.cross_v != nullptr ? s3.cross_v + at : nullptr,
                                          s3.input, lw.norm_cross, lw.norm_cross_b);
             requests_issued();
-            MYNAH_STAMP(6);
             fetch_tagged<3, false>(ex.X2 + (size_t)r3.b * kW, sh.s_in, kW, t0 + 2u, wt);
             MYNAH_LEAVE_IF_DEAD();
-            MYNAH_STAMP(7);
             attention_compute<QT>(g, r3, aw, sh.s_in, nullptr, nullptr, 0, lw.norm_cross_b != nullptr, ex.PC + (size_t)r3.b * ex.pc_stream, a.cross_heads,
                                   t0 + 3u, sh.smem, sh.s_sx, sh.s_scratch, sh.s_proj, sh.s_red, sh.s_wave_ml);
-            MYNAH_STAMP(8);
         }
         if (r1.active && layer + 1 < a.n_layers) {
             const PersistLayer &nx = a.layers[layer + 1];
@@ -612,7 +605,6 @@ __device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBloc
         // ---------------------------------------------------------------- 2: fold + O + residual
         RowRegs<BT, 1, kOutPasses> g4;
         if (r2.active) {
-            MYNAH_STAMP(3);
             int off = 0;
             for (int b = 0; b < a.batch; ++b) {
                 const int units = ((b == 0 ? sa.length : sb.length) + kStepUnitRows - 1) / kStepUnitRows + 1;
@@ -621,7 +613,6 @@ __device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBloc
                 off += n;
             }
             MYNAH_LEAVE_IF_DEAD();
-            MYNAH_STAMP(4);
             if (layer > 0) rows_request_residual<QT, BT, 1, kW, kOutPasses>(g2, r2, res_prev, a.batch);   // the partials are there, so the stream they were made from is
             if (cross) {
                 rows_request<QT, BT, 1, kW, kOutPasses>(g4, r2, lw.ox_w, lw.ox_s, true, res2, a.batch, nullptr, nullptr);
@@ -641,12 +632,10 @@ __device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBloc
             pro.k = kW; pro.ln_gain = nullptr; pro.ln_bias = nullptr;
             finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g2.gv, g2.bv, sh.smem, sh.s_sx, sh.s_scratch);
             rows_compute<QT, BT, 1, kW, kOutPasses, EPI_RESIDUAL>(g2, r2, lw.o_w, lw.o_s, res_prev, a.batch, sh.smem, sh.s_sx, ex.X2, kW, t0 + 2u, wt);
-            MYNAH_STAMP(5);
         }
         // ---------------------------------------------------------------- 4: fold + O + residual (cross)
         RowRegs<BT, 1, kUpPasses> g5;
         if (r2.active && cross) {
-            MYNAH_STAMP(9);
             int off = 0;
             for (int b = 0; b < a.batch; ++b) {
                 const int units = max(((b == 0 ? sa.memory_length : sb.memory_length) + kStepUnitRows - 1) / kStepUnitRows, 1);
@@ -655,7 +644,6 @@ __device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBloc
                 off += n;
             }
             MYNAH_LEAVE_IF_DEAD();
-            MYNAH_STAMP(10);
         }
         if (r5.active) {
             rows_request<QT, BT, 1, kW, kUpPasses>(g5, r5, lw.up_w, lw.up_s, false, res_mid, a.batch, lw.norm_ff, lw.norm_ff_b);
@@ -676,15 +664,12 @@ __device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBloc
             pro.k = kW; pro.ln_gain = nullptr; pro.ln_bias = nullptr;
             finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g4.gv, g4.bv, sh.smem, sh.s_sx, sh.s_scratch);
             rows_compute<QT, BT, 1, kW, kOutPasses, EPI_RESIDUAL>(g4, r2, lw.ox_w, lw.ox_s, res2, a.batch, sh.smem, sh.s_sx, ex.X4, kW, t0 + 4u, wt);
-            MYNAH_STAMP(11);
         }
         // ---------------------------------------------------------------- 5: LN + up + GELU
         RowRegs<BT, 3, kDownPasses> g6;
         if (r5.active) {
-            MYNAH_STAMP(12);
             fetch_tagged<3 * BT, false>(res_mid.tagged, sh.s_in, a.batch * kW, res_mid.tag, wt);
             MYNAH_LEAVE_IF_DEAD();
-            MYNAH_STAMP(13);
         }
         if (r6.active) {
             rows_request<QT, BT, 3, kF, kDownPasses>(g6, r6, lw.down_w, lw.down_s, true, res_mid, a.batch, nullptr, nullptr);
@@ -697,16 +682,12 @@ __device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBloc
                 xr[b][0] = (b < a.batch && tid < kW / 4) ? reinterpret_cast<const float4 *>(sh.s_in)[b * (kW / 4) + tid] : make_float4(0.f, 0.f, 0.f, 0.f);
             pro.k = kW; pro.ln_gain = lw.norm_ff; pro.ln_bias = lw.norm_ff_b;
             finish_activations<QT, BT, 1>(pro, whole_workgroup(), xr, g5.gv, g5.bv, sh.smem, sh.s_sx, sh.s_scratch);
-            MYNAH_STAMP(18);
             rows_compute<QT, BT, 1, kW, kUpPasses, EPI_GELU>(g5, r5, lw.up_w, lw.up_s, res_mid, a.batch, sh.smem, sh.s_sx, ex.H, kF, t0 + 5u, wt);
-            MYNAH_STAMP(14);
         }
         // ---------------------------------------------------------------- 6: down + residual
         if (r6.active) {
-            MYNAH_STAMP(15);
             fetch_tagged<12 * BT, true>(ex.H, sh.s_in, a.batch * kF, t0 + 5u, wt);
             MYNAH_LEAVE_IF_DEAD();
-            MYNAH_STAMP(16);
         }
         if (r2.active && layer + 1 < a.n_layers) {
             Residual res_next;
@@ -725,9 +706,7 @@ __device__ __forceinline__ void rows_path(const PersistArgs &a, const SharedBloc
                     xr[b][i] = b < a.batch ? reinterpret_cast<const float4 *>(sh.s_in)[b * (kF / 4) + tid + kThreads * i] : make_float4(0.f, 0.f, 0.f, 0.f);
             pro.k = kF; pro.ln_gain = nullptr; pro.ln_bias = nullptr;
             finish_activations<QT, BT, 3>(pro, whole_workgroup(), xr, g6.gv, g6.bv, sh.smem, sh.s_sx, sh.s_scratch);
-            MYNAH_STAMP(19);
             rows_compute<QT, BT, 3, kF, kDownPasses, EPI_RESIDUAL>(g6, r6, lw.down_w, lw.down_s, res_mid, a.batch, sh.smem, sh.s_sx, ex.X6, kW, t0 + 8u, wt);
-            MYNAH_STAMP(17);
         }
     }
     // ---------------------------------------------------------------- final norm of one stream's row
@@ -758,10 +737,6 @@ __global__ void __launch_bounds__(kThreads) k_step_persistent(const PersistArgs 
     __shared__ float s4[4];
     const SharedBlocks sh{s_in, smem, s_proj, s_red, s_wave_ml, s_sx, s_scratch, s4};
     const int wg = blockIdx.x, grid = gridDim.x;
-#ifdef MYNAH_PERSIST_PROBE
-    if (threadIdx.x == 0 && a.probe != nullptr) { a.probe[(size_t)wg * 32 + 28] = wall_clock64(); a.probe[(size_t)wg * 32 + 29] = clock64(); }
-    struct AtExit { const PersistArgs &a; int wg; __device__ ~AtExit() { if (threadIdx.x == 0 && a.probe != nullptr) { a.probe[(size_t)wg * 32 + 30] = wall_clock64(); a.probe[(size_t)wg * 32 + 31] = clock64(); } } } at_exit{a, wg};
-#endif
     if (wg < a.attention_wgs) {
         const AttnRole r1 = attention_role(a, wg, true);
         AttnRole r3 = attention_role(a, wg, false);
@@ -776,7 +751,6 @@ __global__ void __launch_bounds__(kThreads) k_step_persistent(const PersistArgs 
     if (r2.active || r5.active || r6.active || final_stream >= 0) rows_path<QT, BT>(a, sh, r2, r5, r6, final_stream);
 }
 #undef MYNAH_LEAVE_IF_DEAD
-#undef MYNAH_STAMP
 
 }  // namespace
 
@@ -805,9 +779,8 @@ int step_persistent_attention_workgroups(const PersistArgs &a) {
     return self_wgs > cross_wgs ? self_wgs : cross_wgs;
 }
 
-template <int QT, int BT>
-static int launch_pt(State *st, const PersistArgs &a, int grid, char *error, size_t capacity) {
-    // LDS for the largest thing a stage waits for: all partial records of the streams, or their hidden rows
+// LDS for the largest thing a stage waits for: all partial records of the streams, or their hidden rows
+static size_t persistent_lds_bytes(const PersistArgs &a) {
     size_t floats = (size_t)a.batch * kF;
     size_t rec = 0;
     for (int s = 0; s < a.batch; ++s) {
@@ -818,8 +791,14 @@ static int launch_pt(State *st, const PersistArgs &a, int grid, char *error, siz
         rec += (self_rec > cross_rec ? self_rec : cross_rec) * kStepRecord;
     }
     if (rec > floats) floats = rec;
-    const size_t lds = floats * sizeof(float);
-    if (lds > 120 * 1024) {
+    return floats * sizeof(float);
+}
+constexpr size_t kPersistentLdsLimit = 120 * 1024;
+
+template <int QT, int BT>
+static int launch_pt(State *st, const PersistArgs &a, int grid, char *error, size_t capacity) {
+    const size_t lds = persistent_lds_bytes(a);
+    if (lds > kPersistentLdsLimit) {
         set_error(error, capacity, "persistent step: the attention partials of these lengths exceed the workgroup's LDS");
         return -1;
     }
@@ -838,6 +817,15 @@ static int launch_pt(State *st, const PersistArgs &a, int grid, char *error, siz
     }
     hipLaunchKernelGGL((k_step_persistent<QT, BT>), dim3(grid), dim3(kThreads), lds, st->stream, a);
     return hip_check(hipGetLastError(), "persistent step launch", error, capacity);
+}
+
+// Whether these lengths and workgroup counts fit the launch (what launch_step_persistent would refuse for its shape): asked
+// before a step commits to this form, so that a step that does not fit runs as launched kernels instead of failing.
+bool step_persistent_fits(const PersistArgs &a, int grid) {
+    const int row_wgs = a.wgs_up > a.wgs_down ? (a.wgs_up > a.wgs_out ? a.wgs_up : a.wgs_out) : (a.wgs_down > a.wgs_out ? a.wgs_down : a.wgs_out);
+    return a.batch >= 1 && a.batch <= 2 && a.rows_out > 0 && a.rows_up > 0 && a.rows_down > 0 && a.wgs_out > 0 && a.wgs_up > 0 && a.wgs_down > 0 &&
+           a.attention_wgs == step_persistent_attention_workgroups(a) && a.attention_wgs + row_wgs <= grid && a.batch <= row_wgs &&
+           persistent_lds_bytes(a) <= kPersistentLdsLimit;
 }
 
 int launch_step_persistent(State *st, const PersistArgs &a, int qtype, int grid, char *error, size_t capacity) {

@@ -629,6 +629,10 @@ extern "C" int mynah_hip_local_frame(void *state, mynah_hip_local *l, mynah_hip_
     const int B = (int)batch;
     MYNAH_TRY(hipStreamSynchronize(st->stream));   // the staging buffers of the previous frame may still be in flight
     l->frame_host->logits_copy = dev_logits_copy;
+    // a frame's many-stream attention launches wait like a decode step's, but a frame cannot be repeated from here (its
+    // generator states have moved on): a wait given up inside it is reported as the error it is, never taken for a decode step's
+    st->last_step_decoder = nullptr;
+    st->steps_since_sync += 2;
     if (decoder_next_epochs(st, l->stack, (unsigned)l->streams, &l->frame_host->epoch_base, error, capacity) != 0) return -1;
     l->frame_host->reserved = 0;
     for (size_t b = 0; b < batch; ++b) {
