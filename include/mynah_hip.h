@@ -457,6 +457,9 @@ int mynah_hip_set_graph_mode(void *state, int enabled, char *error, size_t error
  * stream's arithmetic does not depend on which streams share its lane, so every lane count gives the same bits.
  * 0 (default): chosen from the batch size.  MYNAH_HIP_LANES in the environment at open sets the initial value. */
 int mynah_hip_set_step_lanes(void *state, int lanes, char *error, size_t error_capacity);
+/* Free and total bytes of the backend's device (hipMemGetInfo); either pointer may be NULL.  Lets a caller, or a test,
+ * check that a call it relies on not to allocate left the device's free memory where it was. */
+int mynah_hip_device_memory(void *state, size_t *free_bytes, size_t *total_bytes, char *error, size_t error_capacity);
 /* How often a resident step was run a second time because one of its workgroups had given up a bounded wait for another
  * one's result.  Two forms of mynah_hip_decoder_step wait inside a kernel: the persistent launch (graph mode 2) and, in
  * every mode, the attention launches of more than two streams, whose fold workgroups wait for the attending workgroups

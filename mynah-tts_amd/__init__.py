@@ -148,6 +148,7 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_flush_cache.argtypes = [_vp, _sz, *_err]
     lib.mynah_hip_set_graph_mode.argtypes = [_vp, C.c_int, *_err]
     lib.mynah_hip_set_step_lanes.argtypes = [_vp, C.c_int, *_err]
+    lib.mynah_hip_device_memory.argtypes = [_vp, C.POINTER(_sz), C.POINTER(_sz), *_err]
     lib.mynah_hip_wait_fallbacks.argtypes = [_vp]
     lib.mynah_hip_wait_fallbacks.restype = C.c_size_t
     lib.mynah_hip_dependent_launch_probe.argtypes = [_vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), *_err]
@@ -427,6 +428,12 @@ class Backend:
         self._call("mynah_hip_dependent_launch_probe", C.c_int(nodes), C.c_int(workgroups), C.c_int(floats), C.c_int(chains), C.c_int(repeats),
                    C.byref(us))
         return float(us.value)
+
+    def device_memory(self):
+        """(free bytes, total bytes) of the device."""
+        free, total = _sz(0), _sz(0)
+        self._call("mynah_hip_device_memory", C.byref(free), C.byref(total))
+        return int(free.value), int(total.value)
 
     def wait_fallbacks(self):
         """Steps that were repeated in the wait-free form because a workgroup had given up a bounded wait."""

@@ -348,6 +348,7 @@ static void hip_close(void *opaque) {
     if (st->scratch != nullptr) (void)hipFree(st->scratch);
     if (st->pinned != nullptr) (void)hipHostFree(st->pinned);
     if (st->flush != nullptr) (void)hipFree(st->flush);
+    if (st->cross_norm != nullptr) (void)hipFree(st->cross_norm);
     if (st->attn_partial != nullptr) (void)hipFree(st->attn_partial);
     if (st->attn_counters != nullptr) (void)hipFree(st->attn_counters);
     if (st->seam_slots != nullptr) (void)hipFree(st->seam_slots);
@@ -1003,9 +1004,20 @@ extern "C" int mynah_hip_cross_kv_dev(void *opaque, const float *dev_memory, siz
         return -1;
     }
     if (memory_length == 0 || layers == 0) return 0;
-    float *normed = nullptr;
-    MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&normed), memory_length * width * sizeof(float)));
-    st->pending_free.push_back(normed);   // freed at a later synchronisation, when the launches below are done with it
+    // The normalised rows live in a buffer the backend keeps and grows: one allocation per call would add up between
+    // synchronisations when a caller prepares many utterances in a row.  An outgrown buffer may still be read by earlier
+    // launches: it waits in the list that the next idle stream frees (bounded like mynah_hip_dev_free's).
+    if (st->cross_norm_floats < memory_length * width) {
+        if (st->cross_norm != nullptr) {
+            st->pending_free.push_back(st->cross_norm);
+            st->cross_norm = nullptr;
+            st->cross_norm_floats = 0;
+            if (st->pending_free.size() >= kMaxPendingFrees && hipStreamSynchronize(st->stream) == hipSuccess) free_pending(st);
+        }
+        MYNAH_TRY(hipMalloc(reinterpret_cast<void **>(&st->cross_norm), memory_length * width * sizeof(float)));
+        st->cross_norm_floats = memory_length * width;
+    }
+    float *const normed = st->cross_norm;
     const size_t per_layer = memory_length * xattn_width;
     for (size_t l = 0; l < layers; ++l) {
         if (norm_gain[l] == nullptr || kv_w[l] == nullptr) {
@@ -1325,6 +1337,15 @@ extern "C" int mynah_hip_set_step_lanes(void *opaque, int lanes, char *error, si
         return -1;
     }
     st->step_lanes = lanes;
+    return 0;
+}
+extern "C" int mynah_hip_device_memory(void *opaque, size_t *free_bytes, size_t *total_bytes, char *error, size_t capacity) {
+    State *st = enter_state(opaque, false);
+    MYNAH_NEED_STATE(st);
+    size_t f = 0, t = 0;
+    MYNAH_TRY(hipMemGetInfo(&f, &t));
+    if (free_bytes != nullptr) *free_bytes = f;
+    if (total_bytes != nullptr) *total_bytes = t;
     return 0;
 }
 extern "C" size_t mynah_hip_wait_fallbacks(void *opaque) {

@@ -157,6 +157,9 @@ struct State {
     size_t scratch_bytes = 0;
     void *pinned = nullptr;
     size_t pinned_bytes = 0;
+    // normalised encoder memory of mynah_hip_cross_kv_dev (grown on demand; an outgrown one waits in pending_free)
+    float *cross_norm = nullptr;
+    size_t cross_norm_floats = 0;
     // cache-flush buffer
     void *flush = nullptr;
     size_t flush_bytes = 0;

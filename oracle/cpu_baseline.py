@@ -87,8 +87,11 @@ def main():
         times.append(time.perf_counter() - t0)
     times.sort()
     median = times[len(times) // 2]
+    # cores this process may run on (a container's share can be smaller than the machine's count) beside the machine's count
+    affinity = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else None
     print(json.dumps({"kind": kind, "threads": threads, "median_us": median * 1e6, "min_us": times[0] * 1e6,
-                      "steps": args.steps, "warmup": args.warmup, "online_cores": os.cpu_count()}))
+                      "steps": args.steps, "warmup": args.warmup, "online_cores": os.cpu_count(), "affinity_cores": affinity,
+                      "length": args.length, "memory": args.memory}))
 
 
 if __name__ == "__main__":

@@ -68,3 +68,36 @@ def test_noalloc_refuses_what_does_not_fit(pkg, backend):
         backend.self_attention_dev_noalloc(dq.ptr, dk.ptr, dv.ptr, L - 1, width, L, heads, hw, 0.125, do.ptr)
     for d in (dq, dk, dv, do):
         d.free()
+
+
+def test_noalloc_allocates_nothing(pkg):
+    """What names the entry point: on a backend whose first attention call it is (no workspace, no counters, no chunk-count
+    word exist yet), two calls leave the device's free memory exactly where it was, and a call of the allocating entry
+    afterwards does take some (so the reading would have shown an allocation)."""
+    _announce("no-alloc self attention: device memory before and after")
+    fresh = pkg.Backend()
+    try:
+        heads, hw = 12, 64
+        width = heads * hw
+        rng = np.random.default_rng(4300)
+        bufs = []
+        for L in (1100, 70):
+            qkv, kc, vc = _case(fresh, rng, heads, hw, L)
+            bufs.append((L, fresh.alloc(qkv.size).write(qkv), fresh.alloc(kc.size).write(kc), fresh.alloc(vc.size).write(vc), fresh.alloc(width)))
+        fresh.sync()
+        before = fresh.device_memory()[0]
+        for L, dq, dk, dv, do in bufs:
+            fresh.self_attention_dev_noalloc(dq.ptr, dk.ptr, dv.ptr, L - 1, width, L, heads, hw, 1.0 / math.sqrt(hw), do.ptr)
+        fresh.sync()
+        after = fresh.device_memory()[0]
+        assert after == before, "the allocation-free entry point changed the device's free memory by %d bytes" % (before - after)
+        L, dq, dk, dv, do = bufs[0]
+        dbig = [fresh.alloc(32 << 20) for _ in range(2)]      # an allocation of a size the reading cannot miss
+        assert fresh.device_memory()[0] < after
+        for d in dbig:
+            d.free()
+        for L, dq, dk, dv, do in bufs:
+            for d in (dq, dk, dv, do):
+                d.free()
+    finally:
+        fresh.close()
