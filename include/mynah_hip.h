@@ -351,6 +351,15 @@ enum {
 };
 int mynah_hip_decoder_stage_enqueue(void *state, mynah_hip_decoder *decoder, size_t batch, int stage,
                                     char *error, size_t error_capacity);
+/* Parity probe for the whole step (no counterpart in the reference): one step of ONE or TWO streams as plain launches,
+ * like mynah_hip_decoder_step, which also stores, for stream 0, the int8 activation vector and the activation scale the
+ * device formed at each of a layer's six projections (quantize_act_int8, src/qmat.c:94-113), in the order qkv, o_self,
+ * q_cross, o_cross, ffn_up, ffn_down: dev_qx [layers][6][ffn_width] bytes (a projection's first k bytes are used),
+ * dev_sx [layers][6] floats.  A CPU restatement fed these integers instead of its own reproduces the step to the f32
+ * tolerance, which is how the tests separate arithmetic from the occasional int8 activation that a last-bit LayerNorm
+ * difference moves across a rounding boundary.  int8 / int4 weights and 64-wide heads only. */
+int mynah_hip_decoder_step_probe(void *state, mynah_hip_decoder *decoder, const mynah_hip_decoder_slot *slots, size_t batch,
+                                 int8_t *dev_qx, float *dev_sx, char *error, size_t error_capacity);
 
 /* ---- local-transformer frame ---------------------------------------------------------------- */
 

@@ -135,6 +135,7 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_decoder_step.argtypes = [_vp, _vp, C.POINTER(DecoderSlot), _sz, *_err]
     lib.mynah_hip_output_head.argtypes = [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _vp, *_err]
     lib.mynah_hip_decoder_stage_enqueue.argtypes = [_vp, _vp, _sz, C.c_int, *_err]
+    lib.mynah_hip_decoder_step_probe.argtypes = [_vp, _vp, C.POINTER(DecoderSlot), _sz, _vp, _vp, *_err]
     lib.mynah_hip_local_create.argtypes = [_vp, C.POINTER(DecoderDesc), C.POINTER(LocalDesc), C.POINTER(_vp), *_err]
     lib.mynah_hip_local_destroy.argtypes = [_vp, _vp]
     lib.mynah_hip_local_destroy.restype = None
@@ -503,6 +504,26 @@ class Decoder:
             arr[i] = DecoderSlot(s["k"], s["v"], s.get("ck"), s.get("cv"), s["length"], s.get("memory_length", 0),
                                  s["inp"], s["out"])
         self.backend._call("mynah_hip_decoder_step", self.handle, arr, _sz(B))
+
+    def step_probe(self, slots):
+        """One step of one or two streams as plain launches; returns (qx [layers, 6, ffn] int8, sx [layers, 6] f32) of stream 0:
+        the int8 activations and scales the device formed at each projection (qkv, o_self, q_cross, o_cross, up, down)."""
+        B = len(slots)
+        arr = (DecoderSlot * B)()
+        for i, s in enumerate(slots):
+            arr[i] = DecoderSlot(s["k"], s["v"], s.get("ck"), s.get("cv"), s["length"], s.get("memory_length", 0), s["inp"], s["out"])
+        layers, ffn = int(self.desc.layers), int(self.desc.ffn_width)
+        dqx = self.backend.alloc((layers * 6 * ffn + 3) // 4)
+        dsx = self.backend.alloc(layers * 6)
+        dqx.write(np.zeros((layers * 6 * ffn + 3) // 4, np.float32))
+        try:
+            self.backend._call("mynah_hip_decoder_step_probe", self.handle, arr, _sz(B), _vp(dqx.ptr), _vp(dsx.ptr))
+            qx = dqx.read().view(np.int8)[:layers * 6 * ffn].reshape(layers, 6, ffn).copy()
+            sx = dsx.read().reshape(layers, 6).copy()
+        finally:
+            dqx.free()
+            dsx.free()
+        return qx, sx
 
     def stage_enqueue(self, batch, stage):
         """Measurement helper: one stage of the step (all layers) as its own graph, see mynah_hip_decoder_stage_enqueue."""

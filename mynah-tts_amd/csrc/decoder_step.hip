@@ -55,6 +55,10 @@ struct mynah_hip_decoder {
     mynah::StepSlots last_batch_slots;          // of the last step, every stream of it (the single-stage measurement graphs rebuild the tables from it)
     int last_lanes = 1;                         // lanes the last step ran in
     int last_batch = 0;                         // streams of the last step
+    // parity probe (mynah_hip_decoder_step_probe only, null otherwise): [layers][6][ffn] int8 activations and [layers][6]
+    // activation scales of stream 0, one slot per projection in the order qkv, o_self, q_cross, o_cross, up, down
+    int8_t *probe_qx = nullptr;
+    float *probe_sx = nullptr;
     int max_units = 0;
     bool fused_attention = false;
     hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};   // by stream count: this lane's layer kernels as one chain of kernel nodes
@@ -80,9 +84,13 @@ namespace mynah {
 // fold: 0 = plain input rows, 1 = fold of the self-attention partials, 2 = fold of the cross-attention partials
 static int enqueue_linear(State *st, const mynah_hip_decoder *d, const CachedWeight *w, const float *in, size_t in_stride,
                           float *out, size_t out_stride, int batch, const float *ln_gain, const float *ln_bias, int epilogue,
-                          char *error, size_t capacity, int fold = 0) {
+                          char *error, size_t capacity, int fold = 0, int probe_slot = -1) {
     for (int b0 = 0; b0 < batch; b0 += kBatchTile) {
         LinearArgs a{};
+        if (d->probe_qx != nullptr && probe_slot >= 0 && b0 == 0) {
+            a.probe_qx = d->probe_qx + (size_t)probe_slot * d->ffn;
+            a.probe_sx = d->probe_sx + probe_slot;
+        }
         if (fold != 0) {
             a.fold_partial = d->partial;
             a.fold_partial_ml = d->partial_ml;
@@ -149,6 +157,11 @@ static int enqueue_attention(State *st, const mynah_hip_decoder *d, int is_self,
 static int enqueue_step_attention(State *st, const mynah_hip_decoder *d, int is_self, size_t layer, int batch, const CachedWeight *w,
                                   const float *ln_gain, const float *ln_bias, char *error, size_t capacity) {
     StepAttnArgs a{};
+    if (d->probe_qx != nullptr) {
+        const size_t slot = layer * 6 + (is_self ? 0 : 2);
+        a.probe_qx = d->probe_qx + slot * d->ffn;
+        a.probe_sx = d->probe_sx + slot;
+    }
     a.slots = d->dev_slots;
     a.items = is_self ? d->self_items : d->cross_items;
     a.x = d->x;
@@ -193,18 +206,19 @@ static int enqueue_layers(State *st, const mynah_hip_decoder *d, int batch, char
             if (on(MYNAH_HIP_STAGE_SELF_ATTENTION) &&
                 enqueue_step_attention(st, d, 1, l, batch, lw.qkv, lw.norm_self, lw.norm_self_b, error, capacity) != 0) return -1;
             const bool consumer_fold = batch <= kConsumerFoldMaxBatch;
+            const int slot0 = (int)l * 6;
             if (on(MYNAH_HIP_STAGE_SELF_OUT) &&
-                enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 1 : 0) != 0) return -1;
+                enqueue_linear(st, d, lw.o_self, d->attn, w, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 1 : 0, slot0 + 1) != 0) return -1;
             if (d->xw != 0) {
                 if (on(MYNAH_HIP_STAGE_CROSS_ATTENTION) &&
                     enqueue_step_attention(st, d, 0, l, batch, lw.q_cross, lw.norm_cross, lw.norm_cross_b, error, capacity) != 0) return -1;
                 if (on(MYNAH_HIP_STAGE_CROSS_OUT) &&
-                    enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 2 : 0) != 0) return -1;
+                    enqueue_linear(st, d, lw.o_cross, d->ctx, d->xw, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, consumer_fold ? 2 : 0, slot0 + 3) != 0) return -1;
             }
             if (on(MYNAH_HIP_STAGE_FFN_UP) &&
-                enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity) != 0) return -1;
+                enqueue_linear(st, d, lw.up, d->x, w, d->hidden, d->ffn, batch, lw.norm_ff, lw.norm_ff_b, EPI_GELU, error, capacity, 0, slot0 + 4) != 0) return -1;
             if (on(MYNAH_HIP_STAGE_FFN_DOWN) &&
-                enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity) != 0) return -1;
+                enqueue_linear(st, d, lw.down, d->hidden, d->ffn, d->x, w, batch, nullptr, nullptr, EPI_RESIDUAL, error, capacity, 0, slot0 + 5) != 0) return -1;
         }
         if (stages != kAllStages || !with_end) return 0;
         return launch_step_end(st, d->dev_slots, batch, w, d->x, w, d->norm_out, d->norm_out_b, error, capacity);
@@ -775,6 +789,46 @@ int mynah::rerun_last_step_without_waits(State *st, char *error, size_t capacity
     d->last_batch_slots = s;
     d->last_lanes = 1;
     d->last_batch = B;
+    return rc;
+}
+
+// Parity probe: one step of one or two streams as plain launches in one lane, with the int8 activations and activation scale
+// of stream 0 at every projection written to the caller's device buffers -- what lets a CPU restatement be run on the very
+// integers the device used.  Same kernels and arithmetic as mynah_hip_decoder_step (the matvec launches take the build that
+// carries the probe stores); not part of the decode path.
+extern "C" int mynah_hip_decoder_step_probe(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch, int8_t *dev_qx,
+                                            float *dev_sx, char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    if (st == nullptr || d == nullptr || slots == nullptr || dev_qx == nullptr || dev_sx == nullptr || batch < 1 || batch > (size_t)kConsumerFoldMaxBatch) {
+        set_error(error, capacity, "step probe: one or two streams and both probe buffers");
+        return -1;
+    }
+    if (!d->fused_attention || (d->qtype != MYNAH_HIP_INT8 && d->qtype != MYNAH_HIP_INT4)) {
+        set_error(error, capacity, "step probe: int8 / int4 weights and 64-wide heads only");
+        return -1;
+    }
+    StepSlots s;
+    memset(&s, 0, sizeof s);
+    for (size_t b = 0; b < batch; ++b) {
+        const mynah_hip_decoder_slot &in = slots[b];
+        if (in.length >= d->capacity || in.memory_length > d->capacity || in.dev_self_k == nullptr || in.dev_self_v == nullptr || in.dev_input == nullptr ||
+            in.dev_output == nullptr || (d->xw != 0 && in.memory_length != 0 && (in.dev_cross_k == nullptr || in.dev_cross_v == nullptr))) {
+            set_error(error, capacity, "step probe: invalid slot");
+            return -1;
+        }
+        s.self_k[b] = in.dev_self_k; s.self_v[b] = in.dev_self_v; s.cross_k[b] = in.dev_cross_k; s.cross_v[b] = in.dev_cross_v;
+        s.input[b] = in.dev_input; s.output[b] = in.dev_output; s.length[b] = (int)in.length; s.memory_length[b] = (int)in.memory_length;
+    }
+    s.epoch = 1;
+    d->last_batch_slots = s;
+    d->last_lanes = 1;
+    d->last_batch = (int)batch;
+    if (launch_step_begin(st, s, d->dev_slots, (int)batch, d->width, d->position, d->x, d->width, StepItemTables{}, error, capacity) != 0) return -1;
+    d->probe_qx = dev_qx;
+    d->probe_sx = dev_sx;
+    const int rc = enqueue_layers(st, d, (int)batch, error, capacity);
+    d->probe_qx = nullptr;
+    d->probe_sx = nullptr;
     return rc;
 }
 

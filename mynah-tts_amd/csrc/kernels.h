@@ -115,6 +115,9 @@ struct StepAttnArgs {
     float *fold_out;
     unsigned spin_limit;
     unsigned *abort_word;
+    // parity probes (null in production): the int8 activations and the activation scale of stream 0, as this launch quantised them
+    int8_t *probe_qx;
+    float *probe_sx;
 };
 int launch_step_attention(State *st, const StepAttnArgs &args, char *error, size_t capacity);
 // Workgroups of the attention launch for this shape (the table below has as many entries).

@@ -193,7 +193,8 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     // requested right after, are still on their way.  Throughput layout: after the cache rows (fewer live registers).
     PrologueParams pro;
     pro.k = a.width; pro.batch = 1; pro.ln_gain = a.ln_gain; pro.ln_bias = a.ln_bias; pro.arith = a.arith;
-    pro.probe_qx = nullptr; pro.probe_sx = nullptr;
+    // (the probes name stream 0: finish_activations writes them from workgroup 0, which always belongs to it)
+    pro.probe_qx = PACKED == 0 ? a.probe_qx : nullptr; pro.probe_sx = PACKED == 0 ? a.probe_sx : nullptr;
     float4 xr[1][NVT], gv[NVT], bv[NVT];
     ActSource act;
     act.rows[0] = a.x + (size_t)b * a.width;

@@ -257,21 +257,43 @@ void orc_matvec_f32(float *out, const float *x, const float *weights, const floa
     }
 }
 
-/* src/qmat.c:768-818 for one activation row (count == 1). */
-void orc_linear(const orc_weight *w, const float *x, float *out, const float *bias, int act_variant) {
+/* src/qmat.c:768-818 for one activation row (count == 1).
+ * forced_qx / forced_sx (test hook, both or neither): use this int8 activation vector and scale instead of quantising x --
+ * what another implementation formed at this very projection.  *flips, when given, is increased by the number of
+ * elements in which the forced vector differs from the one quantised here, *max_step raised to the largest such
+ * difference: a forced vector from a correct implementation differs only where x sits on a rounding boundary, by 1. */
+static void linear_forced(const orc_weight *w, const float *x, float *out, const float *bias, int act_variant,
+                          const int8_t *forced_qx, const float *forced_sx, size_t *flips, int *max_step, int8_t *capture_qx, float *capture_sx) {
     if (w->qtype == ORC_F32) {
         orc_matvec_f32(out, x, (const float *)w->data, bias, w->n, w->k);
     } else if (w->qtype == ORC_F16) {
         orc_matvec_f16(out, x, (const uint16_t *)w->data, bias, w->n, w->k);
     } else {
         int8_t *qx = (int8_t *)malloc(w->k);
-        const float sx = orc_quantize_act_int8(qx, x, w->k, act_variant);
+        float sx = orc_quantize_act_int8(qx, x, w->k, act_variant);
+        if (capture_qx != NULL && capture_sx != NULL) {   /* what was quantised here, before any forcing */
+            memcpy(capture_qx, qx, w->k);
+            *capture_sx = sx;
+        }
+        if (forced_qx != NULL && forced_sx != NULL) {
+            for (size_t i = 0; i < w->k; ++i) {
+                const int step = abs((int)qx[i] - (int)forced_qx[i]);
+                if (step != 0 && flips != NULL) ++*flips;
+                if (max_step != NULL && step > *max_step) *max_step = step;
+            }
+            memcpy(qx, forced_qx, w->k);
+            sx = *forced_sx;
+        }
         if (w->qtype == ORC_INT8)
             orc_matvec_q8(out, NULL, qx, sx, (const int8_t *)w->data, w->scales, bias, w->n, w->k);
         else
             orc_matvec_q4(out, NULL, qx, sx, (const uint8_t *)w->data, w->scales, bias, w->n, w->k);
         free(qx);
     }
+}
+
+void orc_linear(const orc_weight *w, const float *x, float *out, const float *bias, int act_variant) {
+    linear_forced(w, x, out, bias, act_variant, NULL, NULL, NULL, NULL, NULL, NULL);
 }
 
 /* ===================================================================== f32 kernels */
@@ -474,10 +496,18 @@ void orc_cross_attention(const float *q, const float *k_cache, const float *v_ca
 /* src/graph.c:3127-3284, one slot at a time (the reference's batched form is bit-identical to this
  * per-slot form by its own contract, src/qmat.c:1107-1179).  Generalisations for the synthetic
  * configurations: optional LayerNorm bias, cross_heads x cross_head_width cross attention. */
-int orc_decoder_step(const orc_decoder *d, size_t batch, float *const *self_k, float *const *self_v,
-                     const float *const *cross_k, const float *const *cross_v,
-                     const size_t *lengths, const size_t *memory_lengths,
-                     const float *const *inputs, float *const *outs) {
+static int decoder_step_body(const orc_decoder *d, size_t batch, float *const *self_k, float *const *self_v,
+                             const float *const *cross_k, const float *const *cross_v,
+                             const size_t *lengths, const size_t *memory_lengths,
+                             const float *const *inputs, float *const *outs,
+                             const int8_t *forced_qx, const float *forced_sx, size_t *flips, int *max_step, int8_t *capture_qx,
+                             float *capture_sx) {
+    /* forced_qx [layers][6][ffn], forced_sx [layers][6]: stream 0's int8 activations per projection (qkv, o_self, q_cross,
+     * o_cross, ffn_up, ffn_down), or NULL */
+#define FORCED(slot) (forced_qx != NULL && b == 0 ? forced_qx + (layer * 6u + (slot)) * ffn : NULL), \
+                     (forced_sx != NULL && b == 0 ? forced_sx + layer * 6u + (slot) : NULL), flips, max_step, \
+                     (capture_qx != NULL && b == 0 ? capture_qx + (layer * 6u + (slot)) * ffn : NULL), \
+                     (capture_sx != NULL && b == 0 ? capture_sx + layer * 6u + (slot) : NULL)
     const size_t width = d->width, ffn = d->ffn;
     const size_t xw = d->cross_heads * d->cross_head_width;
     const float self_scale = 1.0f / sqrtf((float)d->head_width);
@@ -509,31 +539,56 @@ int orc_decoder_step(const orc_decoder *d, size_t batch, float *const *self_k, f
             const float *bc = d->norm_cross_b ? d->norm_cross_b + layer * width : NULL;
             const float *bf = d->norm_ff_b ? d->norm_ff_b + layer * width : NULL;
             orc_layernorm(x, d->norm_self_g + layer * width, bs, nrm, 1, width, 1.0e-5f);
-            orc_linear(&d->qkv[layer], nrm, qkv, NULL, d->act_variant);
+            linear_forced(&d->qkv[layer], nrm, qkv, NULL, d->act_variant, FORCED(0));
             orc_self_attention(qkv, self_k[b] + layer * d->capacity * width,
                                self_v[b] + layer * d->capacity * width, start, width, start + 1u,
                                d->heads, d->head_width, self_scale, attn, scores);
-            orc_linear(&d->o_self[layer], attn, proj, NULL, d->act_variant);
+            linear_forced(&d->o_self[layer], attn, proj, NULL, d->act_variant, FORCED(1));
             for (size_t i = 0; i < width; ++i) x[i] += proj[i];
             if (xw != 0) {
                 orc_layernorm(x, d->norm_cross_g + layer * width, bc, nrm, 1, width, 1.0e-5f);
-                orc_linear(&d->q_cross[layer], nrm, qx, NULL, d->act_variant);
+                linear_forced(&d->q_cross[layer], nrm, qx, NULL, d->act_variant, FORCED(2));
                 orc_cross_attention(qx, cross_k[b] + layer * memory_lengths[b] * xw,
                                     cross_v[b] + layer * memory_lengths[b] * xw, memory_lengths[b], xw,
                                     d->cross_heads, d->cross_head_width, cross_scale, xctx, scores);
-                orc_linear(&d->o_cross[layer], xctx, proj, NULL, d->act_variant);
+                linear_forced(&d->o_cross[layer], xctx, proj, NULL, d->act_variant, FORCED(3));
                 for (size_t i = 0; i < width; ++i) x[i] += proj[i];
             }
             orc_layernorm(x, d->norm_ff_g + layer * width, bf, nrm, 1, width, 1.0e-5f);
-            orc_linear(&d->ffn_up[layer], nrm, hidden, NULL, d->act_variant);
+            linear_forced(&d->ffn_up[layer], nrm, hidden, NULL, d->act_variant, FORCED(4));
             orc_gelu_scalar(hidden, ffn);
-            orc_linear(&d->ffn_down[layer], hidden, proj, NULL, d->act_variant);
+            linear_forced(&d->ffn_down[layer], hidden, proj, NULL, d->act_variant, FORCED(5));
             for (size_t i = 0; i < width; ++i) x[i] += proj[i];
         }
         if (d->norm_out_g != NULL) orc_layernorm(x, d->norm_out_g, d->norm_out_b, outs[b], 1, width, 1.0e-5f);
         else memcpy(outs[b], x, width * sizeof(float));
     }
     free(x); free(nrm); free(qkv); free(attn); free(proj); free(qx); free(xctx); free(hidden); free(scores);
+    return rc;
+#undef FORCED
+}
+
+int orc_decoder_step(const orc_decoder *d, size_t batch, float *const *self_k, float *const *self_v,
+                     const float *const *cross_k, const float *const *cross_v,
+                     const size_t *lengths, const size_t *memory_lengths,
+                     const float *const *inputs, float *const *outs) {
+    return decoder_step_body(d, batch, self_k, self_v, cross_k, cross_v, lengths, memory_lengths, inputs, outs, NULL, NULL, NULL, NULL, NULL, NULL);
+}
+
+/* Test hook: the same step with stream 0's int8 activations at every projection taken from the caller (see linear_forced;
+ * forced_qx / forced_sx may be NULL: nothing forced); counts[0] receives the number of activation elements in which they
+ * differ from the ones quantised here, counts[1] the largest difference in int8 steps.  capture_qx / capture_sx (same
+ * layout, may be NULL) receive the activations this implementation quantised itself at each projection. */
+int orc_decoder_step_forced(const orc_decoder *d, size_t batch, float *const *self_k, float *const *self_v,
+                            const float *const *cross_k, const float *const *cross_v,
+                            const size_t *lengths, const size_t *memory_lengths,
+                            const float *const *inputs, float *const *outs,
+                            const int8_t *forced_qx, const float *forced_sx, size_t *counts, int8_t *capture_qx, float *capture_sx) {
+    size_t flips = 0;
+    int max_step = 0;
+    const int rc = decoder_step_body(d, batch, self_k, self_v, cross_k, cross_v, lengths, memory_lengths, inputs, outs, forced_qx, forced_sx,
+                                     &flips, &max_step, capture_qx, capture_sx);
+    if (counts != NULL) { counts[0] = flips; counts[1] = (size_t)max_step; }
     return rc;
 }
 

@@ -129,6 +129,17 @@ int orc_decoder_step(const orc_decoder *d, size_t batch, float *const *self_k, f
                      const size_t *lengths, const size_t *memory_lengths,
                      const float *const *inputs, float *const *outs);
 
+/* Test hook: the same step, with stream 0's int8 activations at each projection optionally taken from the caller
+ * (forced_qx [layers][6][ffn] bytes, forced_sx [layers][6]; projections in the order qkv, o_self, q_cross, o_cross,
+ * ffn_up, ffn_down; both NULL: nothing forced) and the ones quantised here optionally written out (capture_*, same
+ * layout).  counts[0]: elements in which the forced vectors differ from the ones quantised here; counts[1]: the largest
+ * such difference in int8 steps. */
+int orc_decoder_step_forced(const orc_decoder *d, size_t batch, float *const *self_k, float *const *self_v,
+                            const float *const *cross_k, const float *const *cross_v,
+                            const size_t *lengths, const size_t *memory_lengths,
+                            const float *const *inputs, float *const *outs,
+                            const int8_t *forced_qx, const float *forced_sx, size_t *counts, int8_t *capture_qx, float *capture_sx);
+
 /* final-normed hidden [width] -> logits [heads_out*vocab] -> softmax per head. */
 void orc_output_head(const orc_weight *w_out, const float *bias, const float *hidden, size_t heads_out,
                      size_t vocab, float *logits, float *probs, int act_variant);

@@ -67,6 +67,7 @@ def _load_oracle():
     lib.orc_self_attention.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, _sz, _sz, C.c_float, _f32p, _f32p]
     lib.orc_cross_attention.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, _sz, C.c_float, _f32p, _f32p]
     lib.orc_decoder_step.restype = C.c_int
+    lib.orc_decoder_step_forced.restype = C.c_int
     lib.orc_output_head.restype = None
     lib.orc_encoder_prefill.restype = C.c_int
     lib.orc_gemm_nt.argtypes = [_f32p, _f32p, _f32p, _sz, _sz, _sz, C.c_int]
@@ -299,6 +300,30 @@ class Decoder:
         if rc != 0:
             raise RuntimeError("decoder cache capacity exceeded")
         return outs
+
+    def step_forced(self, self_k, self_v, cross_k, cross_v, lengths, memory_lengths, inputs, qx=None, sx=None):
+        """The same step with stream 0's int8 activations taken from the caller: qx [layers, 6, ffn] int8 and sx [layers, 6] f32,
+        one slot per projection (qkv, o_self, q_cross, o_cross, ffn_up, ffn_down); None: nothing forced.  Returns (outs,
+        elements in which qx differs from the oracle's own quantisation, the largest such difference in int8 steps, and the
+        activations the oracle quantised itself, in the same layout: (own_qx, own_sx))."""
+        B = len(inputs)
+        L, ffn = self.cfg["layers"], self.cfg["ffn"]
+        if qx is not None:
+            qx = np.ascontiguousarray(qx, np.int8)
+            sx = np.ascontiguousarray(sx, np.float32)
+            assert qx.shape == (L, 6, ffn) and sx.shape == (L, 6)
+        own_qx, own_sx = np.zeros((L, 6, ffn), np.int8), np.zeros((L, 6), np.float32)
+        outs = [np.empty(self.cfg["width"], np.float32) for _ in range(B)]
+        pp = C.c_void_p * B
+        szs = _sz * B
+        counts = (_sz * 2)(0, 0)
+        rc = lib.orc_decoder_step_forced(C.byref(self.d), _sz(B), pp(*[_ptr(a) for a in self_k]), pp(*[_ptr(a) for a in self_v]),
+                                         pp(*[_ptr(a) for a in cross_k]), pp(*[_ptr(a) for a in cross_v]),
+                                         szs(*lengths), szs(*memory_lengths), pp(*[_ptr(a) for a in inputs]),
+                                         pp(*[_ptr(a) for a in outs]), _ptr(qx), _ptr(sx), counts, _ptr(own_qx), _ptr(own_sx))
+        if rc != 0:
+            raise RuntimeError("decoder cache capacity exceeded")
+        return outs, int(counts[0]), int(counts[1]), (own_qx, own_sx)
 
 
 def output_head(pw, hidden, heads_out, vocab, bias=None, act_variant=STRICT):

@@ -220,6 +220,56 @@ def test_last_row_of_the_cache(pkg, backend, orc, synth, nerr, qtype_name):
     backend.set_quant(0)
 
 
+@pytest.mark.parametrize("qtype_name", ["int8", "int4"])
+@pytest.mark.parametrize("layers,length,mem,seeds", [(2, 300, 65, 10), (12, 1023, 256, 2)])
+def test_teacher_forced_quantised_step(pkg, backend, orc, synth, nerr, qtype_name, layers, length, mem, seeds):
+    """What the 2e-2 bar of the quantised whole-step comparisons stands for, turned into an assertion: the device reports the
+    int8 activation vector and scale it formed at every projection of every layer (mynah_hip_decoder_step_probe), the
+    oracle runs the same step on THOSE integers instead of its own, and the two outputs then agree like an f32 step --
+    1e-5, no outlier allowance, appended cache rows included, for every one of a row of seeded inputs.  The device's
+    integers differ from the oracle's own in a handful of elements at most, each by one int8 step (an activation on a
+    rounding boundary that a last-bit difference in the LayerNorm sums moves), and the probing step gives the bits of the
+    ordinary step."""
+    _announce("teacher-forced %s step, %d layers, kv %d/%d" % (qtype_name, layers, length, mem))
+    cfg = synth.decoder_config(layers=layers, capacity=length + 2)
+    weights = synth.decoder_weights(cfg, seed=0)
+    backend.set_quant(QT[qtype_name])
+    odec = orc.Decoder(cfg, weights, QT[qtype_name])
+    elements = layers * (5 * 768 + 3072)
+    total_flips, unforced_outliers = 0, 0
+    try:
+        for seed in range(seeds):
+            streams = synth.decoder_streams(cfg, [length], [mem], seed=90 + seed)
+            h = Harness(pkg, backend, cfg, weights, streams)
+            try:
+                ordinary = h.step()[0]
+                rows_ordinary = [a[:, length].copy() for a in h.cache_rows(0)]
+                h.reset_cache(0)
+                qx, sx = h.dec.step_probe(h.slots())
+                probed = h.bufs[0]["out"].read()
+                assert np.array_equal(probed.view(np.uint32), ordinary.view(np.uint32)), "the probing step is not the ordinary step"
+                s = streams[0]
+                ks, vs = [s["k"].copy()], [s["v"].copy()]
+                want, flips, step, (own_qx, own_sx) = odec.step_forced(ks, vs, [s["ck"]], [s["cv"]], [length], [mem], [s["x"]], qx=qx, sx=sx)
+                plain = odec.step([s["k"].copy()], [s["v"].copy()], [s["ck"]], [s["cv"]], [length], [mem], [s["x"]])[0]
+                total_flips += flips
+                unforced_outliers += nerr(ordinary, plain) >= 1e-5
+                print("[teacher-forced] %s seed %d: %d of %d int8 activations differ from the oracle's own (largest difference %d); error forced "
+                      "%.2e, unforced %.2e" % (qtype_name, seed, flips, elements, step, nerr(ordinary, want[0]), nerr(ordinary, plain)), flush=True)
+                assert nerr(ordinary, want[0]) < 1e-5, "seed %d" % seed
+                assert nerr(rows_ordinary[0], ks[0][:, length]) < 1e-5 and nerr(rows_ordinary[1], vs[0][:, length]) < 1e-5
+                assert step <= 1, "an int8 activation differs from the oracle's by more than one step"
+                assert flips <= max(4, elements // 500), "too many int8 activations differ from the oracle's own: %d" % flips
+                assert np.abs(sx - own_sx).max() <= 1e-5 * np.abs(own_sx).max()
+                assert flips > 0 or nerr(ordinary, plain) < 1e-5, "the unforced oracle differs although every int8 activation agrees"
+            finally:
+                h.close()
+        print("[teacher-forced] %s: %d differing activations over %d inputs, %d inputs above 1e-5 unforced" % (qtype_name, total_flips, seeds, unforced_outliers),
+              flush=True)
+    finally:
+        backend.set_quant(0)
+
+
 def test_twelve_layers_int8_multi_step(pkg, backend, orc, synth, nerr):
     """The benchmark stack (12 layers, 12x64 cross heads, int8) at reduced cache length, two consecutive steps
     so that the second step attends over the row the first one appended."""

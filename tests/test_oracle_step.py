@@ -146,3 +146,33 @@ def test_multi_head_cross_and_bias_generalisation(orc, synth, nerr):
     x = x + f(w["ffn_down"][0]) @ h
     want = ln(x, f(w["norm_out_g"]), f(w["norm_out_b"]))
     assert nerr(out, want) < 1e-5
+
+
+def test_forced_activations_hook(orc, synth):
+    """The hook the GPU's teacher-forced comparison rests on: a step fed its own captured int8 activations is the plain step
+    bit for bit with no element counted as different; moving one activation by one step is counted as exactly that and
+    changes the output; the captured vectors obey quantize_act_int8's invariants (|q| <= 127, the largest is 127, scale =
+    absmax / 127 > 0)."""
+    cfg = synth.decoder_config(layers=2, capacity=40)
+    weights = synth.decoder_weights(cfg, seed=0)
+    s = synth.decoder_streams(cfg, [33], [17], seed=1)[0]
+    for qtype in (orc.INT8, orc.INT4):
+        dec = orc.Decoder(cfg, weights, qtype)
+        args = lambda: ([s["k"].copy()], [s["v"].copy()], [s["ck"]], [s["cv"]], [33], [17], [s["x"]])
+        plain = dec.step(*args())[0]
+        outs, flips, step, (qx, sx) = dec.step_forced(*args())
+        assert np.array_equal(outs[0].view(np.uint32), plain.view(np.uint32)) and flips == 0 and step == 0
+        widths = [768, 768, 768, 768, 768, 3072]
+        for layer in range(2):
+            for slot, k in enumerate(widths):
+                q = qx[layer, slot, :k].astype(np.int32)
+                assert np.abs(q).max() == 127 and sx[layer, slot] > 0.0
+                assert not qx[layer, slot, k:].any()
+        again, flips, step, _ = dec.step_forced(*args(), qx=qx, sx=sx)
+        assert np.array_equal(again[0].view(np.uint32), plain.view(np.uint32)) and flips == 0 and step == 0
+        moved = qx.copy()
+        at = int(np.argmin(np.abs(moved[1, 5, :3072].astype(np.int32))))     # an element away from the clamp, in the step's last projection
+        moved[1, 5, at] += 1                                                 # (earlier ones would also move what the later ones quantise)
+        other, flips, step, _ = dec.step_forced(*args(), qx=moved, sx=sx)
+        assert flips == 1 and step == 1
+        assert not np.array_equal(other[0].view(np.uint32), plain.view(np.uint32))
