@@ -62,18 +62,65 @@ enum { SPEC_ANY = 0, SPEC_RESIDUAL = 1, SPEC_UP = 2 };
 template <int BT, int QT>
 constexpr int kLinearTeams = !(BT > kConsumerFoldMaxBatch && kQuantised<QT>) ? 1 : (QT == MYNAH_HIP_INT4 && BT == 8) ? 2 : 4;
 
+// The builds whose leading arguments are repacked (see the kernel): specialised ones, one or two streams.
+template <int BT, int SPEC>
+constexpr bool kPackedLead = BT <= 2 && SPEC != SPEC_ANY;
+
+// The small numbers such a launch needs before its first request, in the 64 bits of one pointer argument.
+struct LeadShape {
+    int n, rows_per_wg, batch, folding, is_self, stream0, heads, max_units, head_width;
+};
+__host__ __device__ inline bool lead_fits(const LeadShape &s) {
+    return s.n >= 0 && s.n < (1 << 20) && s.rows_per_wg >= 0 && s.rows_per_wg < (1 << 12) && s.batch >= 0 && s.batch < 16 && s.stream0 >= 0 && s.stream0 < 32 &&
+           s.heads >= 0 && s.heads < 64 && s.max_units >= 0 && s.max_units < (1 << 11) && s.head_width >= 0 && s.head_width % 64 == 0 && s.head_width / 64 < 16;
+}
+__host__ __device__ inline unsigned long long pack_lead(const LeadShape &s) {
+    return (unsigned long long)s.n | ((unsigned long long)s.rows_per_wg << 20) | ((unsigned long long)s.batch << 32) | ((unsigned long long)(s.folding & 1) << 36) |
+           ((unsigned long long)(s.is_self & 1) << 37) | ((unsigned long long)s.stream0 << 38) | ((unsigned long long)s.heads << 43) |
+           ((unsigned long long)s.max_units << 49) | ((unsigned long long)(s.head_width / 64) << 60);
+}
+__device__ __forceinline__ LeadShape unpack_lead(const unsigned long long v) {
+    LeadShape s;
+    s.n = (int)(v & 0xfffffu); s.rows_per_wg = (int)((v >> 20) & 0xfffu); s.batch = (int)((v >> 32) & 0xfu); s.folding = (int)((v >> 36) & 1u);
+    s.is_self = (int)((v >> 37) & 1u); s.stream0 = (int)((v >> 38) & 0x1fu); s.heads = (int)((v >> 43) & 0x3fu); s.max_units = (int)((v >> 49) & 0x7ffu);
+    s.head_width = (int)((v >> 60) & 0xfu) * 64;
+    return s;
+}
+
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
 __global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>))
 k_linear(const float *const in0, const float *const fold_partial, const float *const fold_partial_ml, const StepSlots *const fold_slots,
          const void *const w, const float *const scales, float *const out0, const int n, const int batch, const LinearArgs a_arg,
-         const int rows_per_wg, const int lg_arg) {
+         const int rows_per_wg_arg, const int lg_arg) {
     // The seven pointers and two counts in front repeat fields of a_arg: the first sixteen dwords of the kernel arguments are
     // in registers when a wavefront starts (the build asks for that), the structure behind them is fetched from memory, and
     // these are what the first requests are formed from.
     // (Only for one or two streams: with more, the rows of a.in and a.out are picked by a run-time index, and a structure that
     // has been written to is then kept in scratch memory -- the eight-stream matvecs took 20 us instead of 4.5.)
     LinearArgs a = a_arg;
-    if constexpr (BT <= 2) {
+    int rows_per_wg = rows_per_wg_arg;
+    if constexpr (kPackedLead<BT, SPEC>) {
+        // Fourteen dwords of arguments -- the seven pointers -- are in registers at wavefront start; n, batch, the structure and
+        // rows_per_wg_arg come out of memory, a round trip that stood in front of the first request.  The specialised builds for
+        // one or two streams never use all seven pointers at once, so the launch (pack_lead) passes in the free places what
+        // the first requests are formed from: LayerNorm vectors where nothing is folded, the slot table's address in the place
+        // of the unused input row where something is, and every small number in the place of the slot table's pointer.
+        const LeadShape shape = unpack_lead(reinterpret_cast<unsigned long long>(fold_slots));
+        a.w = w; a.scales = scales; a.out[0] = out0; a.n = shape.n; a.batch = shape.batch;
+        rows_per_wg = shape.rows_per_wg;
+        a.fold_partial = nullptr; a.fold_partial_ml = nullptr; a.fold_slots = nullptr;
+        a.in[0] = in0;   // (never read as a row when something is folded)
+        // assigned whatever the case, so that no field of the structure in memory is asked for on their account
+        a.fold_heads = shape.heads; a.fold_head_width = shape.head_width; a.fold_max_units = shape.max_units;
+        a.fold_is_self = shape.is_self; a.fold_stream0 = shape.stream0;
+        if constexpr (SPEC == SPEC_UP) {
+            a.ln_gain = fold_partial; a.ln_bias = fold_partial_ml;
+        } else {
+            if (shape.folding) {
+                a.fold_partial = fold_partial; a.fold_partial_ml = fold_partial_ml; a.fold_slots = reinterpret_cast<const StepSlots *>(in0);
+            }
+        }
+    } else if constexpr (BT <= 2) {
         a.in[0] = in0; a.fold_partial = fold_partial; a.fold_partial_ml = fold_partial_ml; a.fold_slots = fold_slots;
         a.w = w; a.scales = scales; a.out[0] = out0; a.n = n; a.batch = batch;
     }
@@ -438,8 +485,29 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised = true;
     }
-    hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, a.in[0], a.fold_partial,
-                       a.fold_partial_ml, a.fold_slots, a.w, a.scales, a.out[0], a.n, a.batch, a, rows_per_wg, lg);
+    if constexpr (kPackedLead<BT, SPEC>) {
+        // the launch's small numbers in the slot table pointer's place, and what the free pointer places carry (see the kernel)
+        LeadShape shape{};
+        shape.n = a.n; shape.rows_per_wg = rows_per_wg; shape.batch = a.batch;
+        const bool folding = SPEC == SPEC_RESIDUAL && a.fold_partial != nullptr;
+        if (folding) {
+            shape.folding = 1; shape.is_self = a.fold_is_self; shape.stream0 = a.fold_stream0; shape.heads = a.fold_heads;
+            shape.max_units = a.fold_max_units; shape.head_width = a.fold_head_width;
+        }
+        if (!lead_fits(shape)) {   // launch_linear_q sends what does not fit to the general build; this is the backstop
+            set_error(error, capacity, "linear: shape does not fit the packed launch arguments");
+            return -1;
+        }
+        const StepSlots *const packed = reinterpret_cast<const StepSlots *>(pack_lead(shape));
+        const float *lead0 = a.in[0], *lead1 = nullptr, *lead2 = nullptr;
+        if (SPEC == SPEC_UP) { lead1 = a.ln_gain; lead2 = a.ln_bias; }
+        else if (folding) { lead0 = reinterpret_cast<const float *>(a.fold_slots); lead1 = a.fold_partial; lead2 = a.fold_partial_ml; }
+        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, lead0, lead1, lead2, packed,
+                           a.w, a.scales, a.out[0], a.n, a.batch, a, rows_per_wg, lg);
+    } else {
+        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, a.in[0], a.fold_partial,
+                           a.fold_partial_ml, a.fold_slots, a.w, a.scales, a.out[0], a.n, a.batch, a, rows_per_wg, lg);
+    }
     return hip_check(hipGetLastError(), "linear launch", error, capacity);
 }
 
@@ -456,8 +524,16 @@ int launch_linear_q(State *st, const LinearArgs &a, char *error, size_t capacity
     // what the arguments rule out decides the build (see SPEC above)
     const bool plain = a.bias == nullptr && a.probe_qx == nullptr && a.probe_sx == nullptr && a.probe_acc == nullptr &&
                        a.ln_out == nullptr && a.aux_out == nullptr && a.act_out == nullptr;
-    const bool residual = plain && a.epilogue == EPI_RESIDUAL && a.ln_gain == nullptr;
-    const bool up = plain && a.epilogue == EPI_GELU && a.ln_gain != nullptr && a.fold_partial == nullptr;
+    // (the specialised builds for one or two streams take their small numbers packed into one argument: when one of them
+    // does not fit its bit field the launch takes the general build, with the same arithmetic)
+    LeadShape fit{};
+    fit.n = a.n; fit.batch = a.batch; fit.rows_per_wg = 2048;   // above what launch_linear_t chooses for any n that fits (256 rows per 196,608 of n)
+    if (a.fold_partial != nullptr) {
+        fit.is_self = a.fold_is_self; fit.stream0 = a.fold_stream0; fit.heads = a.fold_heads; fit.max_units = a.fold_max_units; fit.head_width = a.fold_head_width;
+    }
+    const bool packs = a.batch > 2 || lead_fits(fit);
+    const bool residual = plain && packs && a.epilogue == EPI_RESIDUAL && a.ln_gain == nullptr;
+    const bool up = plain && packs && a.epilogue == EPI_GELU && a.ln_gain != nullptr && a.fold_partial == nullptr;
     if (a.k == 768) {
         if (residual) return launch_linear_b<QT, 1, 768, SPEC_RESIDUAL>(st, a, error, capacity);
         if (up) return launch_linear_b<QT, 1, 768, SPEC_UP>(st, a, error, capacity);

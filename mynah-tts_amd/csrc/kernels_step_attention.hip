@@ -99,6 +99,20 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     StepAttnArgs a = a_arg;
     a.slots = slots_arg; a.x = x_arg; a.w = w_arg; a.scales = scales_arg; a.ln_gain = ln_gain_arg; a.ln_bias = ln_bias_arg; a.items = items_arg;
     if constexpr (WFIX != 0) a.width = WFIX;
+    // Only fourteen dwords of arguments are in registers at wavefront start (the seven pointers): per_xcd_arg, lg_arg and every
+    // field of a_arg come out of memory, and the first request for the activation row cannot be formed before the stream
+    // index is known.  The builds that find their work from the workgroup index have no use for the work table's pointer, so
+    // there the launch passes in its place the few small numbers that decide a workgroup's role (pack_grid_shape): the
+    // activation row, its LayerNorm vectors and the head's weight rows are then requested without waiting for anything.
+    int per_xcd = per_xcd_arg;
+    if constexpr (PACKED == 0) {
+        const unsigned long long shape = reinterpret_cast<unsigned long long>(items_arg);
+        per_xcd = (int)(shape & 0xffffu);
+        a.max_units = (int)((shape >> 16) & 0xffffu);
+        a.batch = (int)((shape >> 32) & 0xffu);
+        a.heads = (int)((shape >> 40) & 0xffu);
+        a.items = nullptr;
+    }
     const bool is_self = SELF >= 0 ? SELF == 1 : a.is_self != 0;
     const int tid = threadIdx.x;
     const StepSlots *slots = a.slots;
@@ -114,8 +128,8 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     if constexpr (PACKED == 0) {
         const int wg_units = a.max_units + (is_self ? 1 : 0);
         const int items = a.heads * a.batch * wg_units;
-        const int item = xcd * per_xcd_arg + slot;
-        if (slot >= per_xcd_arg || item >= items) return;
+        const int item = xcd * per_xcd + slot;
+        if (slot >= per_xcd || item >= items) return;
         unit = item % wg_units;
         const int hb = item / wg_units;
         b = hb % a.batch;
@@ -501,8 +515,20 @@ int launch_t(State *st, const StepAttnArgs &a, char *error, size_t capacity) {
     const int per_xcd = grid / 8;
     const bool packed = a.records != nullptr;
     const size_t lds = lds_for<QT>(a.width, a.max_units, packed);
+    // the builds without a work table take the grid's shape in the table pointer's place (see the kernel): 16 bits each for the
+    // workgroups per XCD and the units per stream, 8 each for streams and heads
+    const StepItem *items_or_shape = a.items;
+    if (!packed) {
+        if (per_xcd > 0xffff || a.max_units > 0xffff || a.batch > 0xff || a.heads > 0xff) {
+            set_error(error, capacity, "step attention: grid too large for the launch's packed shape");
+            return -1;
+        }
+        const unsigned long long shape = (unsigned long long)per_xcd | ((unsigned long long)a.max_units << 16) | ((unsigned long long)a.batch << 32) |
+                                         ((unsigned long long)a.heads << 40);
+        items_or_shape = reinterpret_cast<const StepItem *>(shape);
+    }
     hipLaunchKernelGGL(kernel_for<QT>(a.width, a.is_self != 0, !packed), dim3(grid), dim3(kThreads), lds, st->stream, a.slots, a.x, a.w, a.scales, a.ln_gain,
-                       a.ln_bias, a.items, per_xcd, lg, a);
+                       a.ln_bias, items_or_shape, per_xcd, lg, a);
     return hip_check(hipGetLastError(), "step attention launch", error, capacity);
 }
 
