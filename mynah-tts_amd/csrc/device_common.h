@@ -364,6 +364,28 @@ __device__ __forceinline__ void store_global4(float *p, float4 v) {
     *(__attribute__((address_space(1))) float_x4 *)p = w;
 }
 
+// Kernel arguments beyond the fourteen dwords that are in registers at wavefront start are read from memory where the
+// compiler first needs them, and the first read of every 64-byte line of them is a round trip of a few hundred nanoseconds --
+// wherever it stands: in front of the cache-row requests, between two barriers of the activation quantisation.  This asks
+// for one dword of each of the first LINES lines at the top of a kernel, without waiting: when the fields are needed they
+// come out of the scalar cache.  The four destination registers must stay reserved until a wait the compiler emits for its
+// own scalar or LDS reads has certainly passed (any such wait covers these too, or is stricter for them): release_warm,
+// placed behind the first barrier, does that and emits nothing.  A wavefront that ends before that waits for what it has
+// outstanding as part of ending.
+struct WarmArguments { unsigned r0, r1, r2, r3; };
+template <int LINES>
+__device__ __forceinline__ WarmArguments warm_kernel_arguments() {
+    static_assert(LINES >= 1 && LINES <= 4, "one dword from each of up to four lines behind the first");
+    WarmArguments w{0u, 0u, 0u, 0u};
+    const auto args = __builtin_amdgcn_kernarg_segment_ptr();   // a constant-address-space pointer: two scalar registers
+    if constexpr (LINES >= 1) __asm__ volatile("s_load_dword %0, %1, 0x40" : "=&s"(w.r0) : "s"(args));
+    if constexpr (LINES >= 2) __asm__ volatile("s_load_dword %0, %1, 0x80" : "=&s"(w.r1) : "s"(args));
+    if constexpr (LINES >= 3) __asm__ volatile("s_load_dword %0, %1, 0xc0" : "=&s"(w.r2) : "s"(args));
+    if constexpr (LINES >= 4) __asm__ volatile("s_load_dword %0, %1, 0x100" : "=&s"(w.r3) : "s"(args));
+    return w;
+}
+__device__ __forceinline__ void release_warm(const WarmArguments &w) { __asm__ volatile("" ::"s"(w.r0), "s"(w.r1), "s"(w.r2), "s"(w.r3)); }
+
 // Keeps the memory requests written above this point above it: without it the compiler is free to sink a load to its
 // first use, i.e. behind whatever that use waits for.  Emits no instruction and waits for nothing.
 __device__ __forceinline__ void requests_issued() { __asm__ volatile("" ::: "memory"); }

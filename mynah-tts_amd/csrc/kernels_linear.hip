@@ -97,6 +97,9 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     // these are what the first requests are formed from.
     // (Only for one or two streams: with more, the rows of a.in and a.out are picked by a run-time index, and a structure that
     // has been written to is then kept in scratch memory -- the eight-stream matvecs took 20 us instead of 4.5.)
+    static_assert(64 + sizeof(LinearArgs) > 0x100 + 4, "the warmed lines lie inside the kernel arguments");
+    WarmArguments warm{0u, 0u, 0u, 0u};
+    if constexpr (BT <= 2) warm = warm_kernel_arguments<4>();
     LinearArgs a = a_arg;
     int rows_per_wg = rows_per_wg_arg;
     if constexpr (kPackedLead<BT, SPEC>) {
@@ -232,6 +235,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
 
     // ------------------------------------------------------------------ prologue arithmetic (the weight requests above stay in flight)
     finish_activations<QT, SB, NVT>(pro, team, xr, gv, bv, smem, s_sx, s_scratch);
+    release_warm(warm);
     if (!worker) return;
 
     // ------------------------------------------------------------------ body

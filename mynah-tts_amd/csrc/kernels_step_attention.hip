@@ -104,6 +104,10 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     // index is known.  The builds that find their work from the workgroup index have no use for the work table's pointer, so
     // there the launch passes in its place the few small numbers that decide a workgroup's role (pack_grid_shape): the
     // activation row, its LayerNorm vectors and the head's weight rows are then requested without waiting for anything.
+    // (the argument structure ends 0xf8 bytes into the kernel arguments: three lines behind the first)
+    static_assert(64 + sizeof(StepAttnArgs) > 0xc0 + 4, "the warmed lines lie inside the kernel arguments");
+    WarmArguments warm{0u, 0u, 0u, 0u};
+    if constexpr (PACKED == 0) warm = warm_kernel_arguments<3>();
     int per_xcd = per_xcd_arg;
     if constexpr (PACKED == 0) {
         const unsigned long long shape = reinterpret_cast<unsigned long long>(items_arg);
@@ -367,6 +371,7 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     // ---- LayerNorm + activation quantisation of x[b], staged in LDS (the cache rows requested above stay in flight)
     if constexpr (PF != kPrefetchLatency) load_activations<1, NVT>(pro, act, whole_workgroup(), xr, gv, bv);
     finish_activations<QT, 1, NVT>(pro, whole_workgroup(), xr, gv, bv, smem, s_sx, s_scratch);
+    release_warm(warm);
 
     const size_t sh = (size_t)b * a.heads + head;
     float *out_m = a.partial_ml + sh * 2 * a.max_units;
