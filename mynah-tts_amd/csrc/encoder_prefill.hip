@@ -151,7 +151,7 @@ struct StepFragments {
 template <int EPI, int D, bool EXACT, bool CONV>
 __global__ void __launch_bounds__(kThreads)
 k_enc_gemm(const _Float16 *const a_arg, const _Float16 *const w_arg, const int M, const int N, const int K, const int taps, const int cin,
-           float *const part, _Float16 *const out, _Float16 *const vt, const int width) {
+           const int splits, float *const part, _Float16 *const out, _Float16 *const vt, const int width) {
     GemmArgs g;
     g.a = a_arg; g.w = w_arg; g.M = M; g.N = N; g.K = K; g.part = part; g.out = out; g.vt = vt; g.width = width;
     g.taps = taps; g.cin = cin;
@@ -171,7 +171,9 @@ k_enc_gemm(const _Float16 *const a_arg, const _Float16 *const w_arg, const int M
     const int soff0 = srow * kLdsStride + schunk * 8, soff1 = (srow + 32) * kLdsStride + schunk * 8;
 
     // K range of this workgroup (blockIdx.z splits K; only ENC_PARTIAL launches more than one split)
-    const int nk = g.K / kTile / (int)gridDim.z;
+    // (the K split is an argument among the first fourteen dwords, which are in registers at wavefront start; the grid's own
+    // dimensions would come out of memory, a round trip in front of the first request)
+    const int nk = g.K / kTile / splits;
     const int kbase = (int)blockIdx.z * nk * (kTile / 8);   // in 16-byte chunks
     gw0 += kbase; gw1 += kbase;
     if constexpr (!CONV) { ga0 += kbase; ga1 += kbase; }
@@ -289,9 +291,11 @@ __global__ void __launch_bounds__(kThreads) k_enc_embed(const int *ids, const En
 // f32 (the encoder's output, to params->out, rows below params->tokens only).  gain == nullptr: no
 // LayerNorm, the updated row is copied out as f32.  A lane keeps its NV float4 pieces of the row in
 // registers (width <= 256 * NV; the widest supported row, 4096, takes NV = 16).
+// (Argument order: what the row's first requests are formed from stands among the first fourteen dwords, which are in registers
+// at wavefront start; bias and the f16 destination, needed last, come out of memory.)
 template <bool F16_OUT, int NV>
-__global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *part, int splits, size_t split_stride, const float *gain,
-                                                       const float *bias, _Float16 *out_f16, const EncParams *params, int rows, int width) {
+__global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *part, const EncParams *params, int rows, int width, int splits,
+                                                       size_t split_stride, const float *gain, const float *bias, _Float16 *out_f16) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -373,9 +377,9 @@ template <bool F16_OUT>
 void launch_rows(State *st, int width, dim3 grid, float *x, const float *part, int splits, size_t split_stride, const float *gain,
                  const float *bias, _Float16 *out_f16, const EncParams *params, int rows) {
     if (width <= 1024)
-        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 4>), grid, dim3(kThreads), 0, st->stream, x, part, splits, split_stride, gain, bias, out_f16, params, rows, width);
+        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 4>), grid, dim3(kThreads), 0, st->stream, x, part, params, rows, width, splits, split_stride, gain, bias, out_f16);
     else
-        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 16>), grid, dim3(kThreads), 0, st->stream, x, part, splits, split_stride, gain, bias, out_f16, params, rows, width);
+        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 16>), grid, dim3(kThreads), 0, st->stream, x, part, params, rows, width, splits, split_stride, gain, bias, out_f16);
 }
 
 // One (32-query tile, head): S = scale * Q K^T over all keys (f32, in LDS) -> row softmax numerators
@@ -534,12 +538,12 @@ int launch_gemm(State *st, const GemmArgs &g, int splits, char *error, size_t ca
     const int steps = g.K / kTile / splits;
     const dim3 grid(g.N / kTile, g.M / kTile, splits), block(kThreads);
     if (steps % kGemmDepth == 0)
-        hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt,
-                           g.width);
+        hipLaunchKernelGGL((k_enc_gemm<EPI, kGemmDepth, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, splits, g.part, g.out,
+                           g.vt, g.width);
     else if (steps % 2 == 0)
-        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width);
+        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, true, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, splits, g.part, g.out, g.vt, g.width);
     else
-        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, g.part, g.out, g.vt, g.width);
+        hipLaunchKernelGGL((k_enc_gemm<EPI, 2, false, CONV>), grid, block, 0, st->stream, g.a, g.w, g.M, g.N, g.K, g.taps, g.cin, splits, g.part, g.out, g.vt, g.width);
     return hip_check(hipGetLastError(), "encoder product launch", error, capacity);
 }
 

@@ -127,6 +127,9 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
         a.in[0] = in0; a.fold_partial = fold_partial; a.fold_partial_ml = fold_partial_ml; a.fold_slots = fold_slots;
         a.w = w; a.scales = scales; a.out[0] = out0; a.n = n; a.batch = batch;
     }
+    // a one-stream build is launched for exactly one stream (launch_linear_b): its first request then depends on no argument
+    // that comes out of memory (n and batch are the fifteenth and sixteenth dword, one past what is in registers at start)
+    if constexpr (BT == 1) a.batch = 1;
     constexpr int kTeams = kLinearTeams<BT, QT>;
     constexpr int SB = BT / kTeams;   // streams staged by one team
     // The kernel arguments that the first requests are formed from, fetched here in one go: left to the compiler each is
