@@ -164,6 +164,21 @@ int mynah_hip_conv_transpose_dev(void *state, const float *dev_input, float *dev
 int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length,
                         size_t snake_channels, char *error, size_t error_capacity);
 
+/* The seam's remaining optional slots (src/backend.h:59,62-64; src/backend.c:60,63-65; CUDA: gpu/cuda/backend_cuda.cu:708-735,
+ * :813-851, :874-950).  graph.c calls none of them today and the wrappers fall back when a slot is NULL (src/backend.c:900-952);
+ * they exist so that the HIP block of backend.c can fill every field the CUDA block fills.
+ * im2col: device rows [in_channels, length] -> columns [in_channels * kernel, length], columns[(i*kernel + k)*length + l] =
+ *   input[i*length + l - (kernel-1-k)*dilation] or 0 in front of the row; no synchronisation.
+ * gelu_host / gelu_host_f64: HOST data in place: upload, tanh-GELU (f32 as everywhere else / evaluated in double and rounded
+ *   once), download, synchronise.
+ * matmul_graph: the host-pointer matmul (same arguments and result as the `matmul` of mynah_backend_hip_open). */
+int mynah_hip_im2col(void *state, const float *dev_input, float *dev_columns, int in_channels, int length, int kernel, int dilation,
+                     char *error, size_t error_capacity);
+int mynah_hip_gelu_host(void *state, float *data, size_t n, char *error, size_t error_capacity);
+int mynah_hip_gelu_host_f64(void *state, float *data, size_t n, char *error, size_t error_capacity);
+int mynah_hip_matmul_graph(void *state, const float *input, float *output, size_t rows, size_t input_width, size_t output_width,
+                           const float *weight, const float *bias, char *error, size_t error_capacity);
+
 /* The residual layer of the codec (res_layer_device, src/graph.c:2423-2498) spends a fifth of its time in the element-wise
  * operators between its convolutions: copy_dev, snake_dev, residual_inplace, scale_dev, each a pass over the rows in
  * device memory.  conv1d_fused is conv1d followed, value by value before the store, by the arithmetic of those operators

@@ -149,6 +149,10 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_flush_cache.argtypes = [_vp, _sz, *_err]
     lib.mynah_hip_set_graph_mode.argtypes = [_vp, C.c_int, *_err]
     lib.mynah_hip_set_step_lanes.argtypes = [_vp, C.c_int, *_err]
+    lib.mynah_hip_im2col.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, *_err]
+    lib.mynah_hip_gelu_host.argtypes = [_vp, _vp, _sz, *_err]
+    lib.mynah_hip_gelu_host_f64.argtypes = [_vp, _vp, _sz, *_err]
+    lib.mynah_hip_matmul_graph.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, *_err]
     lib.mynah_hip_device_memory.argtypes = [_vp, C.POINTER(_sz), C.POINTER(_sz), *_err]
     lib.mynah_hip_wait_fallbacks.argtypes = [_vp]
     lib.mynah_hip_wait_fallbacks.restype = C.c_size_t
@@ -439,6 +443,22 @@ class Backend:
     def wait_fallbacks(self):
         """Steps that were repeated in the wait-free form because a workgroup had given up a bounded wait."""
         return int(self.lib.mynah_hip_wait_fallbacks(self.state))
+
+    def im2col(self, din, dcolumns, in_channels, length, kernel, dilation):
+        self._call("mynah_hip_im2col", _vp(din), _vp(dcolumns), C.c_int(in_channels), C.c_int(length), C.c_int(kernel), C.c_int(dilation))
+
+    def gelu_host(self, data, in_double=False):
+        """tanh-GELU of a host float32 array, in place (upload, kernel, download, synchronise)."""
+        assert data.dtype == np.float32 and data.flags["C_CONTIGUOUS"]
+        self._call("mynah_hip_gelu_host_f64" if in_double else "mynah_hip_gelu_host", _np_ptr(data), _sz(data.size))
+        return data
+
+    def matmul_graph(self, x, weight, bias=None):
+        x = np.ascontiguousarray(x, np.float32)
+        rows, iw = x.shape
+        out = np.empty((rows, weight.shape[0]), np.float32)
+        self._call("mynah_hip_matmul_graph", _np_ptr(x), _np_ptr(out), _sz(rows), _sz(iw), _sz(weight.shape[0]), _np_ptr(weight), _np_ptr(bias))
+        return out
 
     def set_step_lanes(self, lanes):
         """Groups a resident step above two streams is cut into, each stepping on a stream of its own (0: chosen from the batch size)."""

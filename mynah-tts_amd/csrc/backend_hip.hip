@@ -786,6 +786,83 @@ extern "C" int mynah_hip_gelu_inplace(void *opaque, float *d, size_t n, char *er
 extern "C" int mynah_hip_gelu_dev(void *opaque, float *d, size_t n, char *error, size_t capacity) {
     return mynah_hip_gelu_inplace(opaque, d, n, error, capacity);
 }
+// ---- the seam's remaining optional slots (src/backend.h:59,62-64; CUDA forms gpu/cuda/backend_cuda.cu:708-735,813-851,874-950).
+// graph.c calls none of them and a backend may leave them null; they are here so that a HIP block in backend.c can fill
+// every field the CUDA block fills.
+namespace mynah {
+namespace {
+// columns[(i * kernel + k) * length + l] = input[i * length + l - (kernel - 1 - k) * dilation], 0 in front of the row
+__global__ void __launch_bounds__(256) k_im2col_causal(const float *__restrict__ input, float *__restrict__ columns, size_t total, int length,
+                                                       int kernel, int dilation) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int l = (int)(idx % (size_t)length);
+    const size_t ik = idx / (size_t)length;
+    const int k = (int)(ik % (size_t)kernel);
+    const size_t i = ik / (size_t)kernel;
+    const long src = (long)l - (long)(kernel - 1 - k) * dilation;
+    columns[idx] = src >= 0 ? input[i * (size_t)length + (size_t)src] : 0.0f;
+}
+// tanh-GELU evaluated in double, rounded once (gpu/cuda/backend_cuda.cu:827-837)
+__global__ void __launch_bounds__(256) k_gelu_f64(float *data, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const double x = (double)data[i];
+    const double inner = 0.7978845608028654 * (x + 0.044715 * (x * x * x));
+    data[i] = (float)(0.5 * x * (1.0 + tanh(inner)));
+}
+int gelu_on_host_rows(State *st, float *data, size_t n, bool in_double, char *error, size_t capacity) {
+    size_t bytes = 0;
+    if (st == nullptr || data == nullptr || !float_bytes(n, &bytes)) {
+        set_error(error, capacity, "invalid gelu arguments");
+        return -1;
+    }
+    if (n == 0) return 0;
+    if (ensure_scratch(st, bytes, error, capacity) != 0) return -1;
+    if (copy_to_device(st, st->scratch, data, bytes, error, capacity) != 0) return -1;
+    if (in_double) {
+        hipLaunchKernelGGL(k_gelu_f64, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st->stream, st->scratch, n);
+        MYNAH_TRY(hipGetLastError());
+    } else if (launch_gelu(st, st->scratch, n, error, capacity) != 0) {
+        return -1;
+    }
+    MYNAH_TRY(hipMemcpyAsync(data, st->scratch, bytes, hipMemcpyDeviceToHost, st->stream));
+    return synchronise(st, error, capacity);
+}
+}  // namespace
+}  // namespace mynah
+
+extern "C" int mynah_hip_im2col(void *opaque, const float *dev_input, float *dev_columns, int in_channels, int length, int kernel, int dilation,
+                                char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    MYNAH_NEED_STATE(st);
+    if (dev_input == nullptr || dev_columns == nullptr || in_channels < 0 || length < 0 || kernel < 1 || dilation < 1) {
+        set_error(error, capacity, "invalid im2col arguments");
+        return -1;
+    }
+    const size_t total = (size_t)in_channels * (size_t)kernel * (size_t)length;
+    if (total == 0) return 0;
+    if ((total + 255) / 256 > 0x7fffffffu) {
+        set_error(error, capacity, "im2col: too many elements");
+        return -1;
+    }
+    hipLaunchKernelGGL(k_im2col_causal, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st->stream, dev_input, dev_columns, total, length, kernel,
+                       dilation);
+    return hip_check(hipGetLastError(), "im2col launch", error, capacity);
+}
+extern "C" int mynah_hip_gelu_host(void *opaque, float *data, size_t n, char *error, size_t capacity) {
+    return gelu_on_host_rows(enter_state(opaque), data, n, false, error, capacity);
+}
+extern "C" int mynah_hip_gelu_host_f64(void *opaque, float *data, size_t n, char *error, size_t capacity) {
+    return gelu_on_host_rows(enter_state(opaque), data, n, true, error, capacity);
+}
+// The CUDA backend replays a captured graph of its upload, product and download to save launch overhead and falls back to
+// its plain matmul; here the plain host-pointer matmul is already one launch between two copies, so this is that call.
+extern "C" int mynah_hip_matmul_graph(void *opaque, const float *input, float *output, size_t rows, size_t iw, size_t ow, const float *weight,
+                                      const float *bias, char *error, size_t capacity) {
+    return hip_matmul(opaque, input, output, rows, iw, ow, weight, bias, error, capacity);
+}
+
 extern "C" int mynah_hip_residual_inplace(void *opaque, float *dout, const float *din, size_t n, char *error, size_t capacity) {
     State *st = static_cast<State *>(opaque);
     MYNAH_NEED_STATE(st);

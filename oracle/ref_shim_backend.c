@@ -85,6 +85,10 @@ mynah_backend *ref_backend_open_hip(const char *library_path, char *error, size_
     REF_BIND(conv1d, mynah_hip_conv1d);
     REF_BIND(conv_transpose_dev, mynah_hip_conv_transpose_dev);
     REF_BIND(snake_dev, mynah_hip_snake_dev);
+    REF_BIND(im2col, mynah_hip_im2col);
+    REF_BIND(gelu_host, mynah_hip_gelu_host);
+    REF_BIND(gelu_host_f64, mynah_hip_gelu_host_f64);
+    REF_BIND(matmul_graph, mynah_hip_matmul_graph);
     if (error != NULL && error_capacity > 0) error[0] = '\0';
     return backend;
 }

@@ -682,3 +682,39 @@ def test_fused_attention_fold_matches_separate_launches(backend, pkg, orc, nerr,
     for d in (dq, dk, dv, dattn, dproj, dx):
         d.free()
     backend.set_quant(pkg.F32)
+
+
+def test_optional_seam_slots(pkg, backend, orc, nerr):
+    """The four seam slots graph.c does not call (src/backend.h:59,62-64): causal im2col against its definition, the
+    host-pointer GELU in f32 against the oracle's and in double against a float64 evaluation rounded once, and the
+    "graph" matmul against the plain host-pointer matmul bit for bit."""
+    _announce("optional seam slots")
+    rng = np.random.default_rng(777)
+    for in_ch, length, kernel, dilation in ((3, 17, 3, 1), (5, 64, 7, 3), (2, 9, 11, 5), (1, 1, 1, 1)):
+        x = rng.standard_normal((in_ch, length)).astype(np.float32)
+        want = np.zeros((in_ch, kernel, length), np.float32)
+        for k in range(kernel):
+            shift = (kernel - 1 - k) * dilation
+            if shift < length:
+                want[:, k, shift:] = x[:, :length - shift]
+        din, dcol = backend.alloc(x.size).write(x), backend.alloc(want.size)
+        backend.im2col(din.ptr, dcol.ptr, in_ch, length, kernel, dilation)
+        got = dcol.read().reshape(want.shape)
+        assert np.array_equal(got, want), (in_ch, length, kernel, dilation)
+        din.free()
+        dcol.free()
+    v = (rng.standard_normal(5000) * 3).astype(np.float32)
+    v[:4] = [0.0, 1.0, -1.0, 6.5]
+    got32 = backend.gelu_host(v.copy())
+    assert nerr(got32, orc.gelu_scalar(v.copy())) < 1e-6
+    assert abs(float(got32[1]) - 0.8411920) < 1e-6 and got32[0] == 0.0            # src/kernels.c:493-499
+    got64 = backend.gelu_host(v.copy(), in_double=True)
+    x64 = v.astype(np.float64)
+    want64 = (0.5 * x64 * (1.0 + np.tanh(0.7978845608028654 * (x64 + 0.044715 * x64 ** 3)))).astype(np.float32)
+    # one rounding of a double result; where 1 + tanh cancels (x below about -5) the two double evaluations may differ in their
+    # last bits, which is an absolute difference far below the smallest value compared here
+    assert np.allclose(got64, want64, rtol=1.2e-7, atol=1e-12), "double-precision GELU differs from the float64 evaluation by more than a rounding"
+    w = backend.keep((rng.standard_normal((40, 96)) * 0.1).astype(np.float32))
+    b = backend.keep(rng.standard_normal(40).astype(np.float32))
+    rows = rng.standard_normal((3, 96)).astype(np.float32)
+    assert np.array_equal(backend.matmul_graph(rows, w, b).view(np.uint32), backend.matmul(rows, w, b).view(np.uint32))
