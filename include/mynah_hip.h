@@ -436,6 +436,10 @@ typedef struct {
     int causal;                   /* nonzero: query t attends to keys 0 .. t (src/graph.c:446-449); 0: every key */
     size_t ffn_kernel;            /* 0 or 1: plain FFN, up_w [ffn, width], down_w [width, ffn].  3: causal_conv_ffn
                                    * (src/graph.c:302-352), up_w [ffn, width, 3], down_w [width, ffn, 3] */
+    int operands_f32;             /* nonzero: tables, weights and every product operand stay f32 -- transformer_stack's own
+                                   * arithmetic (src/graph.c:634-711: f32 sgemm per head, f32 linears), to 1e-5 of the CPU.  The
+                                   * accuracy form: the library's f32 operators one after the other, no graph, several times the
+                                   * time of the f16 form.  0: f16 operands, f32 accumulation (2e-3) */
 } mynah_hip_encoder_desc;
 typedef struct mynah_hip_encoder mynah_hip_encoder;
 
@@ -443,8 +447,8 @@ int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_desc *desc, my
                              char *error, size_t error_capacity);
 void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *encoder);
 /* ids: HOST int32 [tokens]; dev_embed_f16 (optional): [tokens,width] f16 bits of the gathered token rows;
- * dev_out: f32 [tokens,width].  Bidirectional attention, plain FFN (the kernel == 1 branch of
- * causal_conv_ffn, src/graph.c:302-316), pre-LayerNorm, f16 operands with f32 accumulation. */
+ * dev_out: f32 [tokens,width].  Attention bidirectional or causal, FFN plain or the kernel-3 causal conv, as the
+ * description says; pre-LayerNorm; f16 operands with f32 accumulation, or f32 operands (then dev_embed_f16 must be NULL). */
 int mynah_hip_encoder_prefill(void *state, mynah_hip_encoder *encoder, const int32_t *ids, size_t tokens,
                               uint16_t *dev_embed_f16, float *dev_out, char *error, size_t error_capacity);
 

@@ -57,7 +57,7 @@ class EncoderDesc(C.Structure):
                 ("vocab", _sz), ("max_positions", _sz), ("tok_table", _vp), ("pos_table", _vp),
                 ("qkv_w", _vp), ("o_w", _vp), ("up_w", _vp), ("down_w", _vp),
                 ("norm1", _vp), ("norm1_bias", _vp), ("norm2", _vp), ("norm2_bias", _vp),
-                ("norm_out", _vp), ("norm_out_bias", _vp), ("causal", C.c_int), ("ffn_kernel", _sz)]
+                ("norm_out", _vp), ("norm_out_bias", _vp), ("causal", C.c_int), ("ffn_kernel", _sz), ("operands_f32", C.c_int)]
 
 
 class LocalItem(C.Structure):
@@ -626,6 +626,7 @@ class Encoder:
         e.norm2, e.norm2_bias = per_layer("norm2_g"), per_layer("norm2_b")
         e.norm_out, e.norm_out_bias = single("norm_out_g"), single("norm_out_b")
         e.causal, e.ffn_kernel = int(bool(cfg.get("causal", False))), int(cfg.get("ffn_kernel", 1))
+        e.operands_f32 = int(bool(cfg.get("operands_f32", False)))
         self.desc = e
         h = _vp()
         backend._call("mynah_hip_encoder_create", C.byref(e), C.byref(h))

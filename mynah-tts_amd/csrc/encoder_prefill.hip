@@ -64,6 +64,14 @@ struct mynah_hip_encoder {
     std::unordered_map<int, hipGraphExec_t> graphs;   // by padded length
     std::unordered_map<int, int> eager_runs;          // a padded length runs eagerly once before it is captured
     size_t max_lds = 0;
+    // f32 operands (the reference's own arithmetic, src/graph.c:634-711: every product an f32 GEMM): f32 copies of the tables
+    // and weights (conv weights tap-major, owned here), and f32 workspaces for exactly max_positions rows
+    bool f32 = false;
+    const CachedWeight *tok32 = nullptr, *pos32 = nullptr;
+    std::vector<const float *> qkv32, o32, up32, down32;
+    std::vector<float *> conv32;   // owned tap-major copies behind up32 / down32 when taps == 3
+    float *f_nrm = nullptr, *f_qkv = nullptr, *f_scores = nullptr, *f_ctx = nullptr, *f_hid = nullptr, *f_col = nullptr, *f_tmp = nullptr;
+    int *f_ids = nullptr;
 };
 
 namespace {
@@ -642,6 +650,116 @@ int enqueue_prefill(State *st, mynah_hip_encoder *e, int tpad, char *error, size
     return hip_check(hipGetLastError(), "encoder prefill launch", error, capacity);
 }
 
+// ---- f32 operands: the stack as the reference computes it ---------------------------------------------------------------
+// transformer_stack (src/graph.c:634-711) is LayerNorm -> QKV linear -> per head sgemm(Q K^T, alpha = scale) -> masked row
+// softmax -> sgemm(P V) -> O linear -> residual -> LayerNorm -> causal_conv_ffn -> residual, all f32.  This form runs exactly
+// that sequence on the library's f32 operators (LayerNorm rows, the f32 matrix-core product, GELU with tanhf, residual add),
+// so that only the order of additions inside a product differs from the CPU: 1e-5 instead of the 2e-3 of f16 operands.
+// It is the accuracy form, not the fast one: some forty launches per layer, no graph.
+
+// Row r = h * T + t of the scores [heads, T, T]: softmax over the keys the query may see (src/graph.c:446-449 masks key > query;
+// softmax_row_inplace, src/graph.c:245-257: max, exp, sum, divide), zeros behind them.
+__global__ void __launch_bounds__(256) k_enc_softmax_rows(float *scores, int T, int causal) {
+    __shared__ float s4[4];
+    const int t = (int)(blockIdx.x % (unsigned)T);
+    float *row = scores + (size_t)blockIdx.x * T;
+    const int valid = causal ? t + 1 : T;
+    float m = -3.0e38f;
+    for (int i = threadIdx.x; i < valid; i += 256) m = fmaxf(m, row[i]);
+    m = block_max(m, s4);
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < valid; i += 256) {
+        const float e = expf(row[i] - m);
+        row[i] = e;
+        sum += e;
+    }
+    sum = block_sum(sum, s4);
+    for (int i = threadIdx.x; i < T; i += 256) row[i] = i < valid ? row[i] / sum : 0.0f;
+}
+
+// unfold_causal (src/graph.c:271-286) in the tap-major order of the conv weights here: col[t][j * C + i] = in[t - (taps - 1) + j][i],
+// zero for rows before the first.
+__global__ void __launch_bounds__(256) k_enc_unfold(const float *in, float *col, int T, int C, int taps) {
+    const size_t n = (size_t)T * taps * C;
+    for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < n; idx += (size_t)gridDim.x * 256) {
+        const int i = (int)(idx % (size_t)C);
+        const size_t tj = idx / (size_t)C;
+        const int j = (int)(tj % (size_t)taps);
+        const int t = (int)(tj / (size_t)taps);
+        const int src = t - (taps - 1) + j;
+        col[idx] = src >= 0 ? in[(size_t)src * C + i] : 0.0f;
+    }
+}
+
+// Conv weight [n][cin][taps] as f32 [n][taps][cin] in device memory (the caller owns it).
+int tap_major_f32(const float *host, size_t n, size_t cin, size_t taps, float **out, char *error, size_t capacity) {
+    *out = nullptr;
+    std::vector<float> packed;
+    try {
+        packed.resize(n * cin * taps);
+    } catch (...) {
+        set_error(error, capacity, "out of memory converting an encoder conv weight");
+        return -1;
+    }
+    for (size_t o = 0; o < n; ++o)
+        for (size_t i = 0; i < cin; ++i)
+            for (size_t j = 0; j < taps; ++j) packed[(o * taps + j) * cin + i] = host[(o * cin + i) * taps + j];
+    void *dev = nullptr;
+    if (hip_check(hipMalloc(&dev, packed.size() * sizeof(float)), "encoder conv weight", error, capacity) != 0) return -1;
+    if (hip_check(hipMemcpy(dev, packed.data(), packed.size() * sizeof(float), hipMemcpyHostToDevice), "encoder conv weight upload", error, capacity) != 0) {
+        (void)hipFree(dev);
+        return -1;
+    }
+    *out = static_cast<float *>(dev);
+    return 0;
+}
+
+int f32_matrix(State *st, const float *host, size_t n, size_t k, const CachedWeight **out, char *error, size_t capacity) {
+    return cached_matrix(st, host, n, k, MYNAH_HIP_F32, out, error, capacity);
+}
+
+int prefill_f32(State *st, mynah_hip_encoder *e, int T, float *dev_out, char *error, size_t capacity) {
+    const size_t w = e->width, f = e->ffn, taps = e->taps, heads = e->heads, hw = e->head_width;
+    const float scale = 1.0f / sqrtf((float)hw);
+    const float *tables[1] = {static_cast<const float *>(e->tok32->data)};
+    if (launch_gather(st, tables, 1, e->f_ids, (size_t)T, w, 1.0f, static_cast<const float *>(e->pos32->data), e->x, error, capacity) != 0) return -1;
+    for (size_t l = 0; l < e->layers; ++l) {
+        if (launch_layernorm(st, e->x, e->f_nrm, e->n1g[l], e->n1b[l], (size_t)T, w, error, capacity) != 0) return -1;
+        if (launch_gemm_f32(st, e->f_nrm, e->f_qkv, (size_t)T, w, 3 * w, e->qkv32[l], nullptr, error, capacity) != 0) return -1;
+        for (size_t h = 0; h < heads; ++h)   // scores_h = scale * Q_h K_h^T (src/graph.c:428-445)
+            if (launch_sgemm(st, 0, 1, (size_t)T, (size_t)T, hw, scale, e->f_qkv + h * hw, 3 * w, e->f_qkv + w + h * hw, 3 * w, 0.0f,
+                             e->f_scores + h * (size_t)T * T, (size_t)T, error, capacity) != 0)
+                return -1;
+        hipLaunchKernelGGL(k_enc_softmax_rows, dim3((unsigned)(heads * (size_t)T)), dim3(256), 0, st->stream, e->f_scores, T, e->causal);
+        MYNAH_TRY(hipGetLastError());
+        for (size_t h = 0; h < heads; ++h)   // ctx_h = P_h V_h (src/graph.c:451-462)
+            if (launch_sgemm(st, 0, 0, (size_t)T, hw, (size_t)T, 1.0f, e->f_scores + h * (size_t)T * T, (size_t)T, e->f_qkv + 2 * w + h * hw, 3 * w, 0.0f,
+                             e->f_ctx + h * hw, w, error, capacity) != 0)
+                return -1;
+        if (launch_gemm_f32(st, e->f_ctx, e->f_tmp, (size_t)T, w, w, e->o32[l], nullptr, error, capacity) != 0) return -1;
+        if (launch_residual(st, e->x, e->f_tmp, (size_t)T * w, error, capacity) != 0) return -1;
+        if (launch_layernorm(st, e->x, e->f_nrm, e->n2g[l], e->n2b[l], (size_t)T, w, error, capacity) != 0) return -1;
+        const float *up_in = e->f_nrm;
+        if (taps > 1) {
+            hipLaunchKernelGGL(k_enc_unfold, dim3(1024), dim3(256), 0, st->stream, e->f_nrm, e->f_col, T, (int)w, (int)taps);
+            MYNAH_TRY(hipGetLastError());
+            up_in = e->f_col;
+        }
+        if (launch_gemm_f32(st, up_in, e->f_hid, (size_t)T, w * taps, f, e->up32[l], nullptr, error, capacity) != 0) return -1;
+        if (launch_gelu(st, e->f_hid, (size_t)T * f, error, capacity) != 0) return -1;
+        const float *down_in = e->f_hid;
+        if (taps > 1) {
+            hipLaunchKernelGGL(k_enc_unfold, dim3(1024), dim3(256), 0, st->stream, e->f_hid, e->f_col, T, (int)f, (int)taps);
+            MYNAH_TRY(hipGetLastError());
+            down_in = e->f_col;
+        }
+        if (launch_gemm_f32(st, down_in, e->f_tmp, (size_t)T, f * taps, w, e->down32[l], nullptr, error, capacity) != 0) return -1;
+        if (launch_residual(st, e->x, e->f_tmp, (size_t)T * w, error, capacity) != 0) return -1;
+    }
+    if (e->nog != nullptr) return launch_layernorm(st, e->x, dev_out, e->nog, e->nob, (size_t)T, w, error, capacity);
+    return launch_copy(st, dev_out, e->x, (size_t)T * w, error, capacity);
+}
+
 }  // namespace
 
 extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_desc *d, mynah_hip_encoder **out, char *error, size_t capacity) {
@@ -680,8 +798,14 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
         set_error(error, capacity, "encoder_create: max_positions beyond 1024, or more LDS per workgroup than this device has");
         return fail();
     }
-    if (f16_matrix(st, d->tok_table, d->vocab, d->width, &e->tok, error, capacity) != 0) return fail();
-    if (f16_matrix(st, d->pos_table, d->max_positions, d->width, &e->pos, error, capacity) != 0) return fail();
+    e->f32 = d->operands_f32 != 0;
+    if (e->f32) {
+        if (f32_matrix(st, d->tok_table, d->vocab, d->width, &e->tok32, error, capacity) != 0) return fail();
+        if (f32_matrix(st, d->pos_table, d->max_positions, d->width, &e->pos32, error, capacity) != 0) return fail();
+    } else {
+        if (f16_matrix(st, d->tok_table, d->vocab, d->width, &e->tok, error, capacity) != 0) return fail();
+        if (f16_matrix(st, d->pos_table, d->max_positions, d->width, &e->pos, error, capacity) != 0) return fail();
+    }
     for (size_t l = 0; l < d->layers; ++l) {
         const CachedWeight *cw = nullptr;
         const float *v = nullptr;
@@ -690,6 +814,26 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
             set_error(error, capacity, "encoder_create: missing layer weight");
             return fail();
         }
+        if (e->f32) {
+            if (f32_matrix(st, d->qkv_w[l], 3 * d->width, d->width, &cw, error, capacity) != 0) return fail();
+            e->qkv32.push_back(static_cast<const float *>(cw->data));
+            if (f32_matrix(st, d->o_w[l], d->width, d->width, &cw, error, capacity) != 0) return fail();
+            e->o32.push_back(static_cast<const float *>(cw->data));
+            if (e->taps == 1) {
+                if (f32_matrix(st, d->up_w[l], d->ffn_width, d->width, &cw, error, capacity) != 0) return fail();
+                e->up32.push_back(static_cast<const float *>(cw->data));
+                if (f32_matrix(st, d->down_w[l], d->width, d->ffn_width, &cw, error, capacity) != 0) return fail();
+                e->down32.push_back(static_cast<const float *>(cw->data));
+            } else {
+                float *dev = nullptr;
+                if (tap_major_f32(d->up_w[l], d->ffn_width, d->width, e->taps, &dev, error, capacity) != 0) return fail();
+                e->conv32.push_back(dev);
+                e->up32.push_back(dev);
+                if (tap_major_f32(d->down_w[l], d->width, d->ffn_width, e->taps, &dev, error, capacity) != 0) return fail();
+                e->conv32.push_back(dev);
+                e->down32.push_back(dev);
+            }
+        } else {
         if (f16_matrix(st, d->qkv_w[l], 3 * d->width, d->width, &cw, error, capacity) != 0) return fail();
         e->qkv.push_back(cw);
         if (f16_matrix(st, d->o_w[l], d->width, d->width, &cw, error, capacity) != 0) return fail();
@@ -705,6 +849,7 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
             e->conv_up.push_back(dev);
             if (tap_major_f16(st, d->down_w[l], d->width, d->ffn_width, e->taps, &dev, error, capacity) != 0) return fail();
             e->conv_down.push_back(dev);
+        }
         }
         if (cached_vector(st, d->norm1[l], d->width, &v, error, capacity) != 0) return fail();
         e->n1g.push_back(v);
@@ -724,6 +869,21 @@ extern "C" int mynah_hip_encoder_create(void *state, const mynah_hip_encoder_des
         if (hip_check(hipMalloc(p, bytes), "encoder workspace", error, capacity) != 0) return -1;
         return hip_check(hipMemsetAsync(*p, 0, bytes, st->stream), "encoder workspace clear", error, capacity);
     };
+    if (e->f32) {
+        const size_t T = d->max_positions, wide = (w > f ? w : f) * e->taps;
+        if (alloc(reinterpret_cast<void **>(&e->x), T * w * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->f_nrm), T * w * sizeof(float)) != 0 ||
+            alloc(reinterpret_cast<void **>(&e->f_qkv), T * 3 * w * sizeof(float)) != 0 ||
+            alloc(reinterpret_cast<void **>(&e->f_scores), e->heads * T * T * sizeof(float)) != 0 ||
+            alloc(reinterpret_cast<void **>(&e->f_ctx), T * w * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->f_hid), T * f * sizeof(float)) != 0 ||
+            alloc(reinterpret_cast<void **>(&e->f_col), T * wide * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->f_tmp), T * w * sizeof(float)) != 0 ||
+            alloc(reinterpret_cast<void **>(&e->f_ids), T * sizeof(int)) != 0)
+            return fail();
+        if (hip_check(hipHostMalloc(reinterpret_cast<void **>(&e->ids_host), T * sizeof(int), hipHostMallocDefault), "encoder ids staging", error, capacity) != 0)
+            return fail();
+        if (hip_check(hipStreamSynchronize(st->stream), "encoder create", error, capacity) != 0) return fail();
+        *out = e;
+        return 0;
+    }
     if (alloc(reinterpret_cast<void **>(&e->x), tp * w * sizeof(float)) != 0 || alloc(reinterpret_cast<void **>(&e->nrm_alloc), (kLeadRows + tp) * w * 2) != 0 ||
         alloc(reinterpret_cast<void **>(&e->qk), tp * 2 * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->vt), w * tp * 2) != 0 ||
         alloc(reinterpret_cast<void **>(&e->ctx), tp * w * 2) != 0 || alloc(reinterpret_cast<void **>(&e->hid_alloc), (kLeadRows + tp) * f * 2) != 0 ||
@@ -758,6 +918,9 @@ extern "C" void mynah_hip_encoder_destroy(void *state, mynah_hip_encoder *e) {
         if (p != nullptr) (void)hipFree(p);
     for (_Float16 *p : e->conv_up) (void)hipFree(p);
     for (_Float16 *p : e->conv_down) (void)hipFree(p);
+    for (float *p : e->conv32) (void)hipFree(p);
+    for (void *p : {(void *)e->f_nrm, (void *)e->f_qkv, (void *)e->f_scores, (void *)e->f_ctx, (void *)e->f_hid, (void *)e->f_col, (void *)e->f_tmp, (void *)e->f_ids})
+        if (p != nullptr) (void)hipFree(p);
     if (e->ids_host != nullptr) (void)hipHostFree(e->ids_host);
     delete e;
 }
@@ -781,6 +944,15 @@ extern "C" int mynah_hip_encoder_prefill(void *state, mynah_hip_encoder *e, cons
     }
     // the staging buffer of the previous call may still be in flight
     MYNAH_TRY(hipStreamSynchronize(st->stream));
+    if (e->f32) {
+        if (dev_embed_f16 != nullptr) {
+            set_error(error, capacity, "encoder_prefill: with f32 operands there are no f16 token rows to return");
+            return -1;
+        }
+        for (size_t t = 0; t < tokens; ++t) e->ids_host[t] = ids[t];
+        MYNAH_TRY(hipMemcpyAsync(e->f_ids, e->ids_host, tokens * sizeof(int), hipMemcpyHostToDevice, st->stream));
+        return prefill_f32(st, e, (int)tokens, dev_out, error, capacity);
+    }
     const size_t tp = e->tpad_max;
     for (size_t t = 0; t < tokens; ++t) e->ids_host[t] = ids[t];
     EncParams *hp = reinterpret_cast<EncParams *>(e->ids_host + tp);

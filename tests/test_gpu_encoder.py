@@ -172,3 +172,60 @@ def test_encoder_other_widths(pkg, backend, orc, synth, nerr, width, heads, ffn,
     _, want = orc.encoder_prefill(cfg, _f16_bits(w), ids)
     assert np.isfinite(got).all()
     assert nerr(got, want) < 2e-3
+
+
+def _prefill_f32(pkg, backend, cfg, w, ids):
+    enc = pkg.Encoder(backend, dict(cfg, operands_f32=True), w)
+    try:
+        dout = backend.alloc(ids.size * cfg["width"])
+        outs = []
+        for _ in range(2):
+            enc.prefill(ids, 0, dout.ptr)
+            outs.append(dout.read().reshape(ids.size, cfg["width"]).copy())
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), "the f32 form is not repeatable"
+        return outs[0]
+    finally:
+        enc.destroy()
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("kernel", [1, 3])
+@pytest.mark.parametrize("tokens,layers", [(1, 1), (19, 2), (130, 2), (256, 1)])
+def test_encoder_f32_operands_match_oracle(pkg, backend, orc, synth, nerr, causal, kernel, tokens, layers):
+    """The f32-operand form (transformer_stack's own arithmetic, src/graph.c:634-711) against the oracle on weights that are
+    exactly representable in f16, so that both sides multiply the same numbers: 1e-5, the bar of an f32 operator."""
+    _announce("encoder f32 operands causal=%s kernel=%d tokens=%d layers=%d" % (causal, kernel, tokens, layers))
+    cfg = dict(synth.encoder_config(layers=layers), causal=causal, ffn_kernel=kernel)
+    w = synth.encoder_weights_f16(cfg, seed=70 + kernel, kernel=kernel, biases=(tokens % 2 == 0))
+    ids = np.random.default_rng(71).integers(0, cfg["vocab"], size=tokens).astype(np.int32)
+    got = _prefill_f32(pkg, backend, cfg, w, ids)
+    _, want = orc.encoder_prefill(cfg, _f16_bits(w), ids)
+    assert np.isfinite(got).all()
+    assert nerr(got, want) < 1e-5
+    half = _prefill(pkg, backend, cfg, w, ids)            # and the f16-operand form stays within its own bar of it
+    assert nerr(half, got) < 2e-3
+
+
+@pytest.mark.parametrize("kernel", [1, 3])
+def test_encoder_f32_operands_match_the_reference_fixture(pkg, backend, synth, nerr, kernel):
+    """Against the committed outputs of the compiled reference's transformer_stack, both builds, at the f32 bar."""
+    from tests.golden import make_golden as mg
+    _announce("encoder f32 operands against the reference fixture, kernel=%d" % kernel)
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(mg.__file__)), "reference_vectors.npz"), allow_pickle=False)
+    cfg = dict(mg.ENC_CFG, ffn_kernel=kernel)
+    w = synth.encoder_weights_f16(cfg, seed=mg.ENC_SEED + kernel, kernel=kernel)
+    ids = np.random.default_rng(mg.ENC_SEED).integers(0, cfg["vocab"], size=mg.ENC_TOKENS).astype(np.int32)
+    if mg.crc(ids, *[w[k] for k in sorted(w) if w[k] is not None]) != gold["enc_k%d_input_crc" % kernel]:
+        pytest.skip("numpy's generator produced different synthetic inputs than when the fixture was written")
+    got = _prefill_f32(pkg, backend, cfg, w, ids)
+    for tag in ("strict", "stock"):
+        assert nerr(got, gold["enc_k%d_%s_out" % (kernel, tag)]) < 1e-5, tag
+
+
+def test_encoder_f32_operands_return_no_f16_rows(pkg, backend, synth):
+    cfg = dict(synth.encoder_config(layers=1, max_positions=64), operands_f32=True)
+    enc = pkg.Encoder(backend, cfg, synth.encoder_weights(cfg, seed=4))
+    dout, dembed = backend.alloc(4 * cfg["width"]), backend.alloc(4 * cfg["width"])
+    with pytest.raises(pkg.BackendError, match="f32 operands"):
+        enc.prefill(np.zeros(4, np.int32), dembed.ptr, dout.ptr)
+    enc.destroy()
