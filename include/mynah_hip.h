@@ -503,6 +503,17 @@ int mynah_hip_device_memory(void *state, size_t *free_bytes, size_t *total_bytes
  * bounded wait" as before; a caller that wants the repeat there synchronises right after the step.  No counterpart in the
  * reference, whose CPU step cannot give up. */
 size_t mynah_hip_wait_fallbacks(void *state);
+/* Packed-weight file (the optional "pre-packed sidecar"; no counterpart in the reference, which converts every tensor at
+ * its first use in every process, src/qmat.c:779-782).  export writes every converted weight the backend holds -- int8 /
+ * int4 values and scales, f16 values -- to `path`; import reads such a file, and from then on a tensor whose shape,
+ * storage type, quantiser arithmetic and content fingerprint (FNV-1a over its shape and 1,536 sampled f32 values) match an
+ * entry is uploaded from the file instead of being converted.  Tensors the file does not hold are converted as always, so
+ * a stale or partial file costs nothing but its reading.  *entries (may be NULL): entries written / read.
+ * mynah_hip_weights_from_pack counts the weights taken from files.  MYNAH_HIP_PACK_VERIFY=1 at open: convert all the same
+ * and fail the call that meets a difference. */
+int mynah_hip_weights_export(void *state, const char *path, size_t *entries, char *error, size_t error_capacity);
+int mynah_hip_weights_import(void *state, const char *path, size_t *entries, char *error, size_t error_capacity);
+size_t mynah_hip_weights_from_pack(void *state);
 /* Bytes of device memory held by the weight cache (packed weights + scales + vectors). */
 size_t mynah_hip_cached_weight_bytes(void *state);
 

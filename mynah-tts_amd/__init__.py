@@ -154,6 +154,10 @@ def load_library(path=LIB_PATH):
     lib.mynah_hip_gelu_host_f64.argtypes = [_vp, _vp, _sz, *_err]
     lib.mynah_hip_matmul_graph.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, _vp, _vp, *_err]
     lib.mynah_hip_device_memory.argtypes = [_vp, C.POINTER(_sz), C.POINTER(_sz), *_err]
+    lib.mynah_hip_weights_export.argtypes = [_vp, C.c_char_p, C.POINTER(_sz), *_err]
+    lib.mynah_hip_weights_import.argtypes = [_vp, C.c_char_p, C.POINTER(_sz), *_err]
+    lib.mynah_hip_weights_from_pack.argtypes = [_vp]
+    lib.mynah_hip_weights_from_pack.restype = C.c_size_t
     lib.mynah_hip_wait_fallbacks.argtypes = [_vp]
     lib.mynah_hip_wait_fallbacks.restype = C.c_size_t
     lib.mynah_hip_dependent_launch_probe.argtypes = [_vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float), *_err]
@@ -439,6 +443,21 @@ class Backend:
         free, total = _sz(0), _sz(0)
         self._call("mynah_hip_device_memory", C.byref(free), C.byref(total))
         return int(free.value), int(total.value)
+
+    def weights_export(self, path):
+        """Writes every converted weight the backend holds to a packed-weight file; returns the number of entries."""
+        n = _sz(0)
+        self._call("mynah_hip_weights_export", os.fsencode(path), C.byref(n))
+        return int(n.value)
+
+    def weights_import(self, path):
+        """Reads a packed-weight file: matching tensors are then uploaded from it instead of being converted."""
+        n = _sz(0)
+        self._call("mynah_hip_weights_import", os.fsencode(path), C.byref(n))
+        return int(n.value)
+
+    def weights_from_pack(self):
+        return int(self.lib.mynah_hip_weights_from_pack(self.state))
 
     def wait_fallbacks(self):
         """Steps that were repeated in the wait-free form because a workgroup had given up a bounded wait."""

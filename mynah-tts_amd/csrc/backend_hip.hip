@@ -150,9 +150,25 @@ int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qty
     cw.qtype = qtype;
     cw.n = n;
     cw.k = k;
+    cw.arith = (qtype == MYNAH_HIP_INT8 || qtype == MYNAH_HIP_INT4) ? st->arith : 0;
     const size_t count = n * k;
     int rc = 0;
-    if (qtype == MYNAH_HIP_F32) {
+    const PackedWeight *pack = nullptr;
+    if (qtype != MYNAH_HIP_F32) {
+        cw.fingerprint = weight_fingerprint(host, n, k);
+        (void)pack_lookup(st, host, n, k, qtype, cw.arith, cw.fingerprint, &pack);
+    }
+    if (pack != nullptr && !st->pack_verify) {
+        // converted in an earlier process and read from a packed-weight file: upload, nothing to convert
+        cw.bytes = pack->values.size() + pack->scales.size() * sizeof(float);
+        rc = device_copy_of(pack->values.data(), pack->values.size(), &cw.data, error, capacity);
+        if (rc == 0 && !pack->scales.empty())
+            rc = device_copy_of(pack->scales.data(), pack->scales.size() * sizeof(float), reinterpret_cast<void **>(&cw.scales), error, capacity);
+        if (rc == 0) {
+            ++st->pack_hits;
+            st->packs.erase(PackKey{cw.fingerprint, (uint64_t)n, (uint64_t)k, qtype, cw.arith});
+        }
+    } else if (qtype == MYNAH_HIP_F32) {
         cw.bytes = count * sizeof(float);
         rc = device_copy_of(host, cw.bytes, &cw.data, error, capacity);
     } else if (qtype == MYNAH_HIP_F16) {
@@ -180,8 +196,25 @@ int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qty
         if (rc == 0)
             rc = device_copy_of(scales.data(), n * groups * sizeof(float), reinterpret_cast<void **>(&cw.scales), error, capacity);
     }
+    if (rc == 0 && pack != nullptr && st->pack_verify) {
+        // the file's bytes against the conversion just made (read back from the device: one comparison for every storage)
+        std::vector<unsigned char> values(pack->values.size());
+        std::vector<float> scales(pack->scales.size());
+        const size_t made = cw.bytes - scales.size() * sizeof(float);
+        if (made != values.size() || hipMemcpy(values.data(), cw.data, values.size(), hipMemcpyDeviceToHost) != hipSuccess ||
+            (!scales.empty() && hipMemcpy(scales.data(), cw.scales, scales.size() * sizeof(float), hipMemcpyDeviceToHost) != hipSuccess) ||
+            memcmp(values.data(), pack->values.data(), values.size()) != 0 ||
+            (!scales.empty() && memcmp(scales.data(), pack->scales.data(), scales.size() * sizeof(float)) != 0)) {
+            set_error(error, capacity, "packed-weight file does not hold what this tensor converts to");
+            rc = -1;
+        } else {
+            ++st->pack_hits;
+            st->packs.erase(PackKey{cw.fingerprint, (uint64_t)n, (uint64_t)k, qtype, cw.arith});
+        }
+    }
     if (rc != 0) {
         if (cw.data != nullptr) (void)hipFree(cw.data);   // the scales failed after the values had gone up
+        if (cw.scales != nullptr) (void)hipFree(cw.scales);
         return -1;
     }
     st->weight_bytes += cw.bytes;
@@ -547,6 +580,8 @@ extern "C" int mynah_backend_hip_open(void **state_out, mynah_backend_matmul_fn 
     if (fuse != nullptr && strcmp(fuse, "0") == 0) st->fuse = 0;
     const char *graph = getenv("MYNAH_HIP_GRAPH");   // 0: every stage a launch, 1 (default): captured graph, 2: persistent launch where it applies
     if (graph != nullptr && (strcmp(graph, "0") == 0 || strcmp(graph, "1") == 0 || strcmp(graph, "2") == 0)) st->graph_mode = graph[0] - '0';
+    const char *verify = getenv("MYNAH_HIP_PACK_VERIFY");   // 1: weights found in a packed-weight file are converted anyway and compared
+    if (verify != nullptr && strcmp(verify, "1") == 0) st->pack_verify = 1;
     const char *lanes = getenv("MYNAH_HIP_LANES");   // lanes of a resident step above two streams; unset or 0: chosen from the batch size
     if (lanes != nullptr && lanes[0] >= '0' && lanes[0] <= '0' + kMaxLanes && lanes[1] == '\0') st->step_lanes = lanes[0] - '0';
     const char *spin = getenv("MYNAH_HIP_PERSIST_SPIN");

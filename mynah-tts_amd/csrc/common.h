@@ -57,6 +57,22 @@ struct CachedWeight {
     void *data = nullptr;        // f32 [n,k] | int8 [n,k] | nibbles [n,k/2] | f16 [n,k]
     float *scales = nullptr;     // int8 [n] | int4 [n,k/32]
     size_t bytes = 0;
+    int arith = 0;               // quantiser arithmetic the values were formed with (int8 / int4)
+    uint64_t fingerprint = 0;    // of the f32 tensor it was converted from (converted storages only; weight_pack.cpp)
+};
+
+// One entry of a packed-weight file, waiting in host memory for the tensor it belongs to (weight_pack.cpp).
+struct PackKey {
+    uint64_t fingerprint, n, k;
+    int qtype, arith;
+    bool operator==(const PackKey &o) const { return fingerprint == o.fingerprint && n == o.n && k == o.k && qtype == o.qtype && arith == o.arith; }
+};
+struct PackKeyHash {
+    size_t operator()(const PackKey &p) const { return (size_t)(p.fingerprint ^ (p.n * 0x9e3779b97f4a7c15ull) ^ (p.k << 20) ^ ((uint64_t)p.qtype << 60) ^ ((uint64_t)p.arith << 59)); }
+};
+struct PackedWeight {
+    std::vector<unsigned char> values;
+    std::vector<float> scales;
 };
 
 struct WeightKey {
@@ -146,6 +162,9 @@ struct State {
     std::mutex mu;
     std::unordered_map<WeightKey, CachedWeight, WeightKeyHash> weights;
     size_t weight_bytes = 0;
+    std::unordered_map<PackKey, PackedWeight, PackKeyHash> packs;   // entries of imported packed-weight files not yet taken
+    size_t pack_hits = 0;                                           // weights that came out of such a file instead of a conversion
+    int pack_verify = 0;                                            // MYNAH_HIP_PACK_VERIFY: convert anyway and compare
     std::map<std::pair<const float *, size_t>, PositionTable> position_tables;   // by (host table, width)
     float *head_logits = nullptr;        // logits of mynah_hip_head_argmax, [kMaxBatch, rows] (grown on demand)
     size_t head_logits_floats = 0;
@@ -202,6 +221,10 @@ int cached_vector(State *st, const float *host, size_t n, const float **dev, cha
 int ensure_attention_workspace(State *st, size_t batch, size_t heads, size_t head_width, size_t max_valid,
                                char *error, size_t capacity, size_t chunk_rows = kAttnChunk);
 int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity);
+
+// packed-weight files (weight_pack.cpp)
+uint64_t weight_fingerprint(const float *host, size_t n, size_t k);
+int pack_lookup(State *st, const float *host, size_t n, size_t k, int qtype, int arith, uint64_t fingerprint, const PackedWeight **found);
 
 // host quantisers (quantize_host.cpp)
 void quantize_weight_int8(const float *w, size_t n, size_t k, int8_t *q, float *scales, int arith);
