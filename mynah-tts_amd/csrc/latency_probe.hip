@@ -16,7 +16,15 @@ __global__ void __launch_bounds__(256) k_probe_node(const float *__restrict__ in
     __shared__ float s_wave[4];
     const int tid = threadIdx.x;
     float acc = 0.0f;
-    for (int i = tid; i < floats; i += 256) acc += in[i];
+    if ((floats & 3) == 0) {   // 16-byte requests, as the stage kernels read their activation rows
+        const float4 *in4 = reinterpret_cast<const float4 *>(in);
+        for (int i = tid; i < (floats >> 2); i += 256) {
+            const float4 v = in4[i];
+            acc += (v.x + v.y) + (v.z + v.w);
+        }
+    } else {
+        for (int i = tid; i < floats; i += 256) acc += in[i];
+    }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off);
     if ((tid & 63) == 0) s_wave[tid >> 6] = acc;
