@@ -472,17 +472,16 @@ struct PrologueParams {
     float *act_out = nullptr;  // non-null: workgroup 0 also stores stream 0's row as loaded (after a fold, before LayerNorm)
 };
 
-// Who stages which streams.  A team is four wavefronts acting as the 256 threads tid = 0..255 of the staging scheme
-// below for the streams [stream0, stream0 + its stream count).  A 256-thread workgroup is one team for all of its
-// streams.  A 1024-thread workgroup (matvec builds for more than two streams) is four teams that split the streams
-// between them: every thread then touches a quarter of the activations and reduces a quarter of the values, and since
-// a team's four wavefronts hold exactly what the four wavefronts of a one-team workgroup would hold, every sum is
-// formed in the same order -- a stream's staged bytes do not depend on how many teams there were.
+// Who stages which streams: the 256 threads tid = 0..255 of a workgroup stage the streams [stream0, stream0 + count) together
+// with the scheme below.  (Matvec builds for more than two streams with quantised weights stage a stream per wavefront
+// instead: load_stream_row / finish_stream_row further down, same bytes.)
 struct Team {
     int tid;       // 0..255 within the team
     int stream0;   // first stream of the team
 };
-__device__ __forceinline__ Team whole_workgroup() { return Team{(int)threadIdx.x, 0}; }
+// (every kernel that stages this way has 256 threads; the mask says so to the compiler, which then drops the range checks of a
+// row that fills the workgroup's places exactly -- k = 3072 -- and requests it unconditionally)
+__device__ __forceinline__ Team whole_workgroup() { return Team{(int)(threadIdx.x & (kThreads - 1)), 0}; }
 
 // Stages the activations of up to BT streams in LDS, all 256 threads of a team cooperating on every stream:
 // load (or fold) -> optional LayerNorm -> for int8/int4 weights the per-vector absmax int8 quantisation
@@ -631,6 +630,147 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, cons
         }
     }
     __syncthreads();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// One wavefront stages one stream (matvec builds for more than two streams with int8 / int4 weights).  Lane l holds, for
+// each of the four "virtual wavefronts" v of the 256-thread scheme above and each i < NVT, the float4 f = 64 v + l + 256 i:
+// what thread 64 v + l of that scheme holds, at xr[v * NVT + i].  Every sum is formed per virtual wavefront in that
+// thread's order, reduced over the lanes by the same butterfly and combined ((a0 + a1) + a2) + a3 as block_reduce does, so
+// the staged bytes of a stream are those of the 256-thread scheme bit for bit -- with no barrier and no exchange through
+// LDS: the wavefronts of a workgroup stage their streams independently of each other, where sixteen wavefronts used to
+// meet at three workgroup barriers.  (The maximum is exact in any order.)
+template <int NVT>
+__device__ __forceinline__ void load_stream_row(const PrologueParams &p, const float *row, const bool live, const int lane, float4 (&xr)[4 * NVT],
+                                                float4 (&gv)[4 * NVT], float4 (&bv)[4 * NVT]) {
+    const int nf4 = p.k >> 2;
+    // no request under a condition: a place beyond the row asks for the row's last float4 and is zeroed afterwards
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+        for (int i = 0; i < NVT; ++i) {
+            const int f = 64 * v + lane + kThreads * i;
+            xr[v * NVT + i] = reinterpret_cast<const float4 *>(row)[f < nf4 ? f : nf4 - 1];
+        }
+    if (p.ln_gain != nullptr) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int i = 0; i < NVT; ++i) {
+                const int f = 64 * v + lane + kThreads * i;
+                gv[v * NVT + i] = reinterpret_cast<const float4 *>(p.ln_gain)[f < nf4 ? f : nf4 - 1];
+                bv[v * NVT + i] = reinterpret_cast<const float4 *>(p.ln_bias != nullptr ? p.ln_bias : p.ln_gain)[f < nf4 ? f : nf4 - 1];
+            }
+    }
+    (void)live;
+}
+
+// Second half for one wavefront and its stream: LayerNorm (optional) -> quantisation -> the stream's bytes in LDS.  The caller
+// puts one workgroup barrier behind it.  live == false (a place of the batch tile without a stream): zeros are staged.
+template <int QT, int NVT>
+__device__ __forceinline__ void finish_stream_row(const PrologueParams &p, const int stream, const bool live, const int lane, float4 (&xr)[4 * NVT],
+                                                  const float4 (&gv)[4 * NVT], const float4 (&bv)[4 * NVT], unsigned char *smem, float *s_sx) {
+    static_assert(kQuantised<QT>, "only the quantising builds stage a stream per wavefront");
+    const int nf4 = p.k >> 2;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+        for (int i = 0; i < NVT; ++i)
+            if (!live || 64 * v + lane + kThreads * i >= nf4) xr[v * NVT + i] = zero;
+    const bool first = blockIdx.x == 0 && stream == 0 && live;
+    if (p.act_out != nullptr && first) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int i = 0; i < NVT; ++i)
+                if (64 * v + lane + kThreads * i < nf4) reinterpret_cast<float4 *>(p.act_out)[64 * v + lane + kThreads * i] = xr[v * NVT + i];
+    }
+    if (p.ln_gain != nullptr) {
+        float part[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float s = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NVT; ++i) s += (xr[v * NVT + i].x + xr[v * NVT + i].y) + (xr[v * NVT + i].z + xr[v * NVT + i].w);
+            part[v] = wave_sum(s);
+        }
+        const float mean = (((part[0] + part[1]) + part[2]) + part[3]) / (float)p.k;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float q = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NVT; ++i)
+                if (64 * v + lane + kThreads * i < nf4) {
+                    const float4 x = xr[v * NVT + i];
+                    const float d0 = x.x - mean, d1 = x.y - mean, d2 = x.z - mean, d3 = x.w - mean;
+                    q = __builtin_fmaf(d0, d0, q);
+                    q = __builtin_fmaf(d1, d1, q);
+                    q = __builtin_fmaf(d2, d2, q);
+                    q = __builtin_fmaf(d3, d3, q);
+                }
+            part[v] = wave_sum(q);
+        }
+        const float rstd = 1.0f / sqrtf((((part[0] + part[1]) + part[2]) + part[3]) / (float)p.k + 1.0e-5f);
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+            for (int i = 0; i < NVT; ++i) {
+                const int f = 64 * v + lane + kThreads * i;
+                const float4 x = xr[v * NVT + i], g = f < nf4 ? gv[v * NVT + i] : zero;   // places beyond the row: gain 0 -> 0
+                float4 y;
+                y.x = ((x.x - mean) * rstd) * g.x;
+                y.y = ((x.y - mean) * rstd) * g.y;
+                y.z = ((x.z - mean) * rstd) * g.z;
+                y.w = ((x.w - mean) * rstd) * g.w;
+                if (p.ln_bias != nullptr && f < nf4) {
+                    const float4 b = bv[v * NVT + i];
+                    y.x += b.x; y.y += b.y; y.z += b.z; y.w += b.w;
+                }
+                xr[v * NVT + i] = y;
+                if (p.ln_out != nullptr && first && f < nf4) reinterpret_cast<float4 *>(p.ln_out)[f] = y;
+            }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+        for (int i = 0; i < NVT; ++i)
+            if (64 * v + lane + kThreads * i < nf4) {
+                const float4 x = xr[v * NVT + i];
+                amax = fmaxf(fmaxf(amax, fmaxf(fabsf(x.x), fabsf(x.y))), fmaxf(fabsf(x.z), fabsf(x.w)));
+            }
+    amax = wave_max(amax);
+    const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+    unsigned char *dst = smem + (size_t)stream * p.k;
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+        for (int i = 0; i < NVT; ++i) {
+            const int f = 64 * v + lane + kThreads * i;
+            if (f < nf4) {
+                const float4 x = xr[v * NVT + i];
+                const int q0 = quant_act(x.x, inv), q1 = quant_act(x.y, inv), q2 = quant_act(x.z, inv), q3 = quant_act(x.w, inv);
+                const int idx = 4 * f;
+                if constexpr (QT == MYNAH_HIP_INT8) {
+                    *reinterpret_cast<unsigned *>(dst + idx) = (unsigned)(q0 & 0xff) | ((unsigned)(q1 & 0xff) << 8) | ((unsigned)(q2 & 0xff) << 16) |
+                                                               ((unsigned)(q3 & 0xff) << 24);
+                } else {
+                    const int block = idx & ~7, half = (idx & 4) >> 1;
+                    *reinterpret_cast<unsigned short *>(dst + block + half) = (unsigned short)((q0 & 0xff) | ((q2 & 0xff) << 8));
+                    *reinterpret_cast<unsigned short *>(dst + block + 4 + half) = (unsigned short)((q1 & 0xff) | ((q3 & 0xff) << 8));
+                }
+                if (p.probe_qx != nullptr && first) {
+                    p.probe_qx[idx] = (int8_t)q0; p.probe_qx[idx + 1] = (int8_t)q1;
+                    p.probe_qx[idx + 2] = (int8_t)q2; p.probe_qx[idx + 3] = (int8_t)q3;
+                }
+            }
+        }
+    if (lane == 0) {
+        const float sx = amax > 0.0f ? (p.arith == MYNAH_HIP_ARITH_STOCK ? amax * (1.0f / 127.0f) : amax / 127.0f) : 0.0f;
+        s_sx[stream] = sx;
+        if (p.probe_sx != nullptr && first) p.probe_sx[0] = sx;
+    }
 }
 
 template <int QT, int BT, int NVT>

@@ -50,17 +50,16 @@ __device__ __forceinline__ float *stream_out(const LinearArgs &a, int b) {
 // GELU epilogue (the step's FFN-up projection).
 enum { SPEC_ANY = 0, SPEC_RESIDUAL = 1, SPEC_UP = 2 };
 
-// More than two streams: the workgroup has four teams of 256 threads (device_common.h) that stage a quarter of the
-// streams each (two teams and half of them each in the case named below) -- staging every stream's activations is what such a launch spends most of its time on, every workgroup
-// has to do all of it, and a quarter of it per thread takes a quarter of the time.  The first team then does the
-// matvec as the only team of a small-batch workgroup would; the others are done once the activations are staged.
-// Only for int8 / int4 weights, where staging includes the activation quantisation: for f16 / f32 weights it is a
-// LayerNorm or a copy, and the 128 registers a thread of a 1024-thread workgroup may use do not hold the wider products.
-// int4 weights with eight streams take two teams of four streams: their products (group scales, eight streams of
-// accumulators) need about 240 registers, which a 512-thread workgroup may have and a 1024-thread one may not
-// (there: 430 to 570 bytes of scratch memory per thread).
+// More than two streams with int8 / int4 weights: one wavefront stages one stream (load_stream_row / finish_stream_row,
+// device_common.h) -- staging every stream's activations is what such a launch spends most of its time on, every workgroup
+// has to do all of it, and a wavefront that owns a whole row needs no barrier and no exchange to normalise and quantise it.
+// The workgroup has as many wavefronts as the batch tile has streams (at least four); the first four then do the matvec as
+// the four wavefronts of a small-batch workgroup would, the others are done once the activations are staged.
+// For f16 / f32 weights staging is a LayerNorm or a copy by the 256 threads together.
 template <int BT, int QT>
-constexpr int kLinearTeams = !(BT > kConsumerFoldMaxBatch && kQuantised<QT>) ? 1 : (QT == MYNAH_HIP_INT4 && BT == 8) ? 2 : 4;
+constexpr bool kWaveStaging = BT > kConsumerFoldMaxBatch && kQuantised<QT>;
+template <int BT, int QT>
+constexpr int kLinearThreads = kWaveStaging<BT, QT> ? 64 * (BT > 4 ? BT : 4) : kThreads;
 
 // The builds whose leading arguments are repacked (see the kernel): specialised ones, one or two streams.
 template <int BT, int SPEC>
@@ -88,7 +87,7 @@ __device__ __forceinline__ LeadShape unpack_lead(const unsigned long long v) {
 }
 
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
-__global__ void __launch_bounds__((kThreads * kLinearTeams<BT, QT>))
+__global__ void __launch_bounds__((kLinearThreads<BT, QT>))
 k_linear(const float *const in0, const float *const fold_partial, const float *const fold_partial_ml, const StepSlots *const fold_slots,
          const void *const w, const float *const scales, float *const out0, const int n, const int batch, const LinearArgs a_arg,
          const int rows_per_wg_arg, const int lg_arg) {
@@ -130,8 +129,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     // a one-stream build is launched for exactly one stream (launch_linear_b): its first request then depends on no argument
     // that comes out of memory (n and batch are the fifteenth and sixteenth dword, one past what is in registers at start)
     if constexpr (BT == 1) a.batch = 1;
-    constexpr int kTeams = kLinearTeams<BT, QT>;
-    constexpr int SB = BT / kTeams;   // streams staged by one team
+    constexpr bool kWaves = kWaveStaging<BT, QT>;   // a wavefront per stream (see above); otherwise the 256 threads stage every stream together
     // The kernel arguments that the first requests are formed from, fetched here in one go: left to the compiler each is
     // fetched where it is first used, with a wait of its own, and three such round trips stood in a row in front of the
     // first request for an activation row.
@@ -144,8 +142,8 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                          "s"(a.ln_gain), "s"(a.ln_bias), "s"(a.n), "s"(a.k), "s"(a.batch), "s"(a.fold_heads), "s"(a.fold_head_width),
                          "s"(a.fold_max_units), "s"(a.fold_is_self), "s"(a.fold_stream0), "s"(rows_per_wg), "s"(a.arith), "s"(a.epilogue));
     }
-    const Team team{(int)(threadIdx.x & (kThreads - 1)), (int)(threadIdx.x / kThreads) * SB};
-    const bool worker = kTeams == 1 || threadIdx.x < kThreads;
+    const Team team = whole_workgroup();
+    const bool worker = !kWaves || threadIdx.x < kThreads;   // (a constant where every wavefront works: no request stands under a condition then)
     // the arguments a specialised build does not look at
     const float *const arg_bias = SPEC != SPEC_ANY ? nullptr : a.bias;
     int8_t *const arg_probe_qx = SPEC != SPEC_ANY ? nullptr : a.probe_qx;
@@ -182,20 +180,23 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     pro.probe_qx = arg_probe_qx; pro.probe_sx = arg_probe_sx;
     pro.ln_out = SPEC != SPEC_ANY ? nullptr : a.ln_out;
     pro.act_out = SPEC != SPEC_ANY ? nullptr : a.act_out;
-    float4 xr[SB][NVT], gv[NVT], bv[NVT];
-    {
+    constexpr int XB = kWaves ? 1 : BT, XN = kWaves ? 4 * NVT : NVT;
+    float4 xr[XB][XN], gv[XN], bv[XN];
+    const int stream = __builtin_amdgcn_readfirstlane(wave);   // a wavefront's stream is its index (the same for all of its lanes)
+    const bool live = !kWaves || stream < a.batch;
+    if constexpr (kWaves) {
+        const float *row = a.in[0];   // a place of the tile without a stream reads stream 0's row and stages zeros
+#pragma unroll
+        for (int q = 1; q < BT; ++q)
+            if (stream == q && q < a.batch) row = a.in[q];   // (select chain over the kernel arguments)
+        load_stream_row<NVT>(pro, row, live, lane, xr[0], gv, bv);
+    } else {
         ActSource src;
 #pragma unroll
-        for (int b = 0; b < kBatchTile; ++b) {   // the team's own rows first (select chain over the kernel arguments)
-            const float *row = a.in[0];
-#pragma unroll
-            for (int q = 1; q < BT; ++q)
-                if (team.stream0 + b == q) row = a.in[q];
-            src.rows[b] = row;
-        }
+        for (int b = 0; b < kBatchTile; ++b) src.rows[b] = a.in[b < BT ? b : 0];
         src.partial = arg_fold_partial; src.partial_ml = a.fold_partial_ml; src.slots = a.fold_slots; src.heads = a.fold_heads; src.head_width = a.fold_head_width;
         src.max_units = a.fold_max_units; src.is_self = a.fold_is_self; src.stream0 = a.fold_stream0;
-        load_activations<SB, NVT>(pro, src, team, xr, gv, bv);
+        load_activations<BT, NVT>(pro, src, team, xr, gv, bv);
     }
     requests_issued();
 
@@ -237,7 +238,12 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     requests_issued();
 
     // ------------------------------------------------------------------ prologue arithmetic (the weight requests above stay in flight)
-    finish_activations<QT, SB, NVT>(pro, team, xr, gv, bv, smem, s_sx, s_scratch);
+    if constexpr (kWaves) {
+        finish_stream_row<QT, NVT>(pro, stream, live, lane, xr[0], gv, bv, smem, s_sx);
+        __syncthreads();
+    } else {
+        finish_activations<QT, BT, NVT>(pro, team, xr, gv, bv, smem, s_sx, s_scratch);
+    }
     release_warm(warm);
     if (!worker) return;
 
@@ -509,10 +515,10 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
         const float *lead0 = a.in[0], *lead1 = nullptr, *lead2 = nullptr;
         if (SPEC == SPEC_UP) { lead1 = a.ln_gain; lead2 = a.ln_bias; }
         else if (folding) { lead0 = reinterpret_cast<const float *>(a.fold_slots); lead1 = a.fold_partial; lead2 = a.fold_partial_ml; }
-        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, lead0, lead1, lead2, packed,
+        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kLinearThreads<BT, QT>), lds, st->stream, lead0, lead1, lead2, packed,
                            a.w, a.scales, a.out[0], a.n, a.batch, a, rows_per_wg, lg);
     } else {
-        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kThreads * kLinearTeams<BT, QT>), lds, st->stream, a.in[0], a.fold_partial,
+        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kLinearThreads<BT, QT>), lds, st->stream, a.in[0], a.fold_partial,
                            a.fold_partial_ml, a.fold_slots, a.w, a.scales, a.out[0], a.n, a.batch, a, rows_per_wg, lg);
     }
     return hip_check(hipGetLastError(), "linear launch", error, capacity);
