@@ -181,14 +181,19 @@ __device__ __forceinline__ void layernorm_row(const float *x, float *y, const fl
     }
 }
 
-// round half away from zero by truncation, clamp to +-127 (src/qmat.c:106-110); the half with v's sign is one bit-field
-// instruction where the comparison and selection of the reference's form are two, with the same sum for every v
+// round half away from zero by truncation (src/qmat.c:106-110); the half with v's sign is one bit-field instruction where
+// the comparison and selection of the reference's form are two, with the same sum for every v.  The reference then clamps
+// to +-127, which changes nothing when inv is 127 / amax and amax the largest |x| of the row this x belongs to -- the only
+// way this is called: |x * inv| <= 127 (1 + 2^-23), plus a half stays below 128, and truncation gives at most 127.
 __device__ __forceinline__ int quant_act(float x, float inv) {
     const float v = x * inv;
-    int q = (int)(v + __builtin_copysignf(0.5f, v));
-    q = q > 127 ? 127 : q;
-    q = q < -127 ? -127 : q;
-    return q;
+    return (int)(v + __builtin_copysignf(0.5f, v));
+}
+// the low bytes of four such integers in one dword, q0 lowest (three byte-permute instructions)
+__device__ __forceinline__ unsigned pack_bytes(int q0, int q1, int q2, int q3) {
+    const unsigned lo = __builtin_amdgcn_perm((unsigned)q1, (unsigned)q0, 0x0c0c0400u);   // [q0.b0, q1.b0, 0, 0]
+    const unsigned hi = __builtin_amdgcn_perm((unsigned)q3, (unsigned)q2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);                                    // [lo.b0, lo.b1, hi.b0, hi.b1]
 }
 
 // src/kernels.c:382-389
@@ -597,8 +602,7 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, cons
                     const int q2 = quant_act(xr[b][i].z, inv), q3 = quant_act(xr[b][i].w, inv);
                     const int idx = 4 * f;
                     if constexpr (QT == MYNAH_HIP_INT8) {
-                        *reinterpret_cast<unsigned *>(dst + idx) = (unsigned)(q0 & 0xff) | ((unsigned)(q1 & 0xff) << 8) |
-                                                                   ((unsigned)(q2 & 0xff) << 16) | ((unsigned)(q3 & 0xff) << 24);
+                        *reinterpret_cast<unsigned *>(dst + idx) = pack_bytes(q0, q1, q2, q3);
                     } else {
                         const int block = idx & ~7, half = (idx & 4) >> 1;
                         *reinterpret_cast<unsigned short *>(dst + block + half) = (unsigned short)((q0 & 0xff) | ((q2 & 0xff) << 8));
@@ -753,8 +757,7 @@ __device__ __forceinline__ void finish_stream_row(const PrologueParams &p, const
                 const int q0 = quant_act(x.x, inv), q1 = quant_act(x.y, inv), q2 = quant_act(x.z, inv), q3 = quant_act(x.w, inv);
                 const int idx = 4 * f;
                 if constexpr (QT == MYNAH_HIP_INT8) {
-                    *reinterpret_cast<unsigned *>(dst + idx) = (unsigned)(q0 & 0xff) | ((unsigned)(q1 & 0xff) << 8) | ((unsigned)(q2 & 0xff) << 16) |
-                                                               ((unsigned)(q3 & 0xff) << 24);
+                    *reinterpret_cast<unsigned *>(dst + idx) = pack_bytes(q0, q1, q2, q3);
                 } else {
                     const int block = idx & ~7, half = (idx & 4) >> 1;
                     *reinterpret_cast<unsigned short *>(dst + block + half) = (unsigned short)((q0 & 0xff) | ((q2 & 0xff) << 8));

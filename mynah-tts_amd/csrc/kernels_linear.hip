@@ -64,6 +64,41 @@ constexpr int kLinearThreads = kWaveStaging<BT, QT> ? 64 * (BT > 4 ? BT : 4) : k
 // The builds whose leading arguments are repacked (see the kernel): specialised ones, one or two streams.
 template <int BT, int SPEC>
 constexpr bool kPackedLead = BT <= 2 && SPEC != SPEC_ANY;
+// The same for more streams, when the rows of a launch lie at a fixed stride (the step's workspaces do): the specialised
+// builds that stage a stream per wavefront take two row pointers and two strides instead of sixteen row pointers.
+template <int BT, int QT, int SPEC>
+constexpr bool kStridedLead = kWaveStaging<BT, QT> && SPEC != SPEC_ANY;
+
+// n:20 | rows per workgroup:12 | streams:4 | input stride / 4:14 | output stride / 4:14 (strides in floats)
+struct StridedShape {
+    int n, rows_per_wg, batch;
+    size_t in_stride, out_stride;
+};
+__host__ __device__ inline bool strided_fits(const StridedShape &s) {
+    return s.n >= 0 && s.n < (1 << 20) && s.rows_per_wg >= 0 && s.rows_per_wg < (1 << 12) && s.batch >= 0 && s.batch < 16 && s.in_stride % 4 == 0 &&
+           s.in_stride / 4 < (1u << 14) && s.out_stride % 4 == 0 && s.out_stride / 4 < (1u << 14);
+}
+__host__ __device__ inline unsigned long long pack_strided(const StridedShape &s) {
+    return (unsigned long long)s.n | ((unsigned long long)s.rows_per_wg << 20) | ((unsigned long long)s.batch << 32) |
+           ((unsigned long long)(s.in_stride / 4) << 36) | ((unsigned long long)(s.out_stride / 4) << 50);
+}
+__device__ __forceinline__ StridedShape unpack_strided(const unsigned long long v) {
+    StridedShape s;
+    s.n = (int)(v & 0xfffffu); s.rows_per_wg = (int)((v >> 20) & 0xfffu); s.batch = (int)((v >> 32) & 0xfu);
+    s.in_stride = (size_t)((v >> 36) & 0x3fffu) * 4; s.out_stride = (size_t)((v >> 50) & 0x3fffu) * 4;
+    return s;
+}
+// rows of a launch at one stride (floats) from the first, or no stride at all
+inline bool rows_strided(const LinearArgs &a, size_t *in_stride, size_t *out_stride) {
+    *in_stride = *out_stride = 0;
+    if (a.batch < 2) return true;
+    if (a.in[1] < a.in[0] || a.out[1] < a.out[0]) return false;
+    const size_t si = (size_t)(a.in[1] - a.in[0]), so = (size_t)(a.out[1] - a.out[0]);
+    for (int b = 2; b < a.batch; ++b)
+        if (a.in[b] != a.in[0] + (size_t)b * si || a.out[b] != a.out[0] + (size_t)b * so) return false;
+    *in_stride = si; *out_stride = so;
+    return true;
+}
 
 // The small numbers such a launch needs before its first request, in the 64 bits of one pointer argument.
 struct LeadShape {
@@ -97,10 +132,26 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     // (Only for one or two streams: with more, the rows of a.in and a.out are picked by a run-time index, and a structure that
     // has been written to is then kept in scratch memory -- the eight-stream matvecs took 20 us instead of 4.5.)
     static_assert(64 + sizeof(LinearArgs) > 0x100 + 4, "the warmed lines lie inside the kernel arguments");
+    constexpr bool kStrided = kStridedLead<BT, QT, SPEC>;
     WarmArguments warm{0u, 0u, 0u, 0u};
-    if constexpr (BT <= 2) warm = warm_kernel_arguments<4>();
+    if constexpr (BT <= 2 || kStrided) warm = warm_kernel_arguments<4>();
     LinearArgs a = a_arg;
     int rows_per_wg = rows_per_wg_arg;
+    size_t in_stride = 0, out_stride = 0;   // (strided builds: rows b of the launch are in0 + b * in_stride, out0 + b * out_stride)
+    if constexpr (kStrided) {
+        // As for one or two streams below: what the first requests are formed from arrives in the fourteen dwords that are in
+        // registers at wavefront start -- first rows, weights, scales, the LayerNorm vectors in the two places that carry fold
+        // arguments for fewer streams, every small number in the slot table pointer's place (pack_strided).
+        const StridedShape shape = unpack_strided(reinterpret_cast<unsigned long long>(fold_slots));
+        a.w = w; a.scales = scales; a.n = shape.n; a.batch = shape.batch;
+        rows_per_wg = shape.rows_per_wg;
+        in_stride = shape.in_stride; out_stride = shape.out_stride;
+        a.fold_partial = nullptr; a.fold_partial_ml = nullptr; a.fold_slots = nullptr;
+        a.fold_heads = 0; a.fold_head_width = 0; a.fold_max_units = 0; a.fold_is_self = 0; a.fold_stream0 = 0;
+        if constexpr (SPEC == SPEC_UP) {
+            a.ln_gain = fold_partial; a.ln_bias = fold_partial_ml;
+        }
+    }
     if constexpr (kPackedLead<BT, SPEC>) {
         // Fourteen dwords of arguments -- the seven pointers -- are in registers at wavefront start; n, batch, the structure and
         // rows_per_wg_arg come out of memory, a round trip that stood in front of the first request.  The specialised builds for
@@ -135,7 +186,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     // first request for an activation row.
     // (One or two streams: only what the first requests are formed from -- fetching every argument first delays them.
     // More streams: the eight row pointers of a.in and a.out as one operand each, or they are fetched in rounds of their own.)
-    if constexpr (BT > 2) {
+    if constexpr (BT > 2 && !kStrided) {
         typedef unsigned row_pointers __attribute__((ext_vector_type(2 * BT)));
         const row_pointers ins = *reinterpret_cast<const row_pointers *>(&a.in[0]), outs = *reinterpret_cast<const row_pointers *>(&a.out[0]);
         __asm__ volatile("" ::"s"(a.w), "s"(a.scales), "s"(ins), "s"(outs), "s"(a.fold_partial), "s"(a.fold_partial_ml), "s"(a.fold_slots),
@@ -184,11 +235,20 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     float4 xr[XB][XN], gv[XN], bv[XN];
     const int stream = __builtin_amdgcn_readfirstlane(wave);   // a wavefront's stream is its index (the same for all of its lanes)
     const bool live = !kWaves || stream < a.batch;
+    // output row of stream b
+    const auto out_of = [&](const int b) -> float * {
+        if constexpr (kStrided) return out0 + (size_t)b * out_stride;
+        else return stream_out<BT>(a, b);
+    };
     if constexpr (kWaves) {
-        const float *row = a.in[0];   // a place of the tile without a stream reads stream 0's row and stages zeros
+        const float *row = kStrided ? in0 : a.in[0];   // a place of the tile without a stream reads stream 0's row and stages zeros
+        if constexpr (kStrided) {
+            if (live) row = in0 + (size_t)stream * in_stride;
+        } else {
 #pragma unroll
-        for (int q = 1; q < BT; ++q)
-            if (stream == q && q < a.batch) row = a.in[q];   // (select chain over the kernel arguments)
+            for (int q = 1; q < BT; ++q)
+                if (stream == q && q < a.batch) row = a.in[q];   // (select chain over the kernel arguments)
+        }
         load_stream_row<NVT>(pro, row, live, lane, xr[0], gv, bv);
     } else {
         ActSource src;
@@ -226,12 +286,12 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
         if (lanes_finish) {
             if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
             if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
-            if (arg_epilogue == EPI_RESIDUAL) pre_res[0] = stream_out<BT>(a, gl < a.batch ? gl : 0)[rowc];
+            if (arg_epilogue == EPI_RESIDUAL) pre_res[0] = out_of(gl < a.batch ? gl : 0)[rowc];
         } else {
             if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
             if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
 #pragma unroll
-            for (int b = 0; b < BT; ++b) pre_res[b] = (arg_epilogue == EPI_RESIDUAL && (b == 0 || b < a.batch)) ? a.out[b][rowc] : 0.0f;   // a launch has at least one stream
+            for (int b = 0; b < BT; ++b) pre_res[b] = (arg_epilogue == EPI_RESIDUAL && (b == 0 || b < a.batch)) ? out_of(b)[rowc] : 0.0f;   // a launch has at least one stream
         }
     }
 
@@ -297,7 +357,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                 if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && gl == 0) arg_probe_acc[row] = mi;
                 if (arg_bias != nullptr) val += bias;
                 if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
-                float *o = stream_out<BT>(a, gl) + row;
+                float *o = out_of(gl) + row;
                 if (arg_aux_out != nullptr && gl == 0) arg_aux_out[row] = val;
                 if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : *o) + val;
                 *o = val;
@@ -318,7 +378,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                     if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && b == 0) arg_probe_acc[row] = iacc[b];
                     if (arg_bias != nullptr) val += bias;
                     if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
-                    float *o = a.out[b] + row;
+                    float *o = out_of(b) + row;
                     if (arg_aux_out != nullptr && b == 0) arg_aux_out[row] = val;
                     if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[b] : *o) + val;
                     *o = val;
@@ -498,7 +558,18 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
         raised = true;
     }
-    if constexpr (kPackedLead<BT, SPEC>) {
+    if constexpr (kStridedLead<BT, QT, SPEC>) {
+        StridedShape shape{};
+        shape.n = a.n; shape.rows_per_wg = rows_per_wg; shape.batch = a.batch;
+        if (!rows_strided(a, &shape.in_stride, &shape.out_stride) || !strided_fits(shape)) {   // launch_linear_q sends such launches to the general build; this is the backstop
+            set_error(error, capacity, "linear: rows do not fit the strided launch arguments");
+            return -1;
+        }
+        const StepSlots *const packed = reinterpret_cast<const StepSlots *>(pack_strided(shape));
+        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kLinearThreads<BT, QT>), lds, st->stream, a.in[0],
+                           SPEC == SPEC_UP ? a.ln_gain : nullptr, SPEC == SPEC_UP ? a.ln_bias : nullptr, packed, a.w, a.scales, a.out[0], a.n, a.batch, a,
+                           rows_per_wg, lg);
+    } else if constexpr (kPackedLead<BT, SPEC>) {
         // the launch's small numbers in the slot table pointer's place, and what the free pointer places carry (see the kernel)
         LeadShape shape{};
         shape.n = a.n; shape.rows_per_wg = rows_per_wg; shape.batch = a.batch;
@@ -544,7 +615,12 @@ int launch_linear_q(State *st, const LinearArgs &a, char *error, size_t capacity
     if (a.fold_partial != nullptr) {
         fit.is_self = a.fold_is_self; fit.stream0 = a.fold_stream0; fit.heads = a.fold_heads; fit.max_units = a.fold_max_units; fit.head_width = a.fold_head_width;
     }
-    const bool packs = a.batch > 2 || lead_fits(fit);
+    bool packs = lead_fits(fit);
+    if (a.batch > 2) {   // more streams: the specialised builds of quantised weights take rows at a fixed stride
+        StridedShape strided{};
+        strided.n = a.n; strided.batch = a.batch; strided.rows_per_wg = 2048;
+        packs = !kQuantised<QT> || (rows_strided(a, &strided.in_stride, &strided.out_stride) && strided_fits(strided));
+    }
     const bool residual = plain && packs && a.epilogue == EPI_RESIDUAL && a.ln_gain == nullptr;
     const bool up = plain && packs && a.epilogue == EPI_GELU && a.ln_gain != nullptr && a.fold_partial == nullptr;
     if (a.k == 768) {
