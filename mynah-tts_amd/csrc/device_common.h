@@ -373,9 +373,8 @@ __device__ __forceinline__ void store_global4(float *p, float4 v) {
 // compiler first needs them, and the first read of every 64-byte line of them is a round trip of a few hundred nanoseconds --
 // wherever it stands: in front of the cache-row requests, between two barriers of the activation quantisation.  This asks
 // for one dword of each of the first LINES lines at the top of a kernel, without waiting: when the fields are needed they
-// come out of the scalar cache.  The four destination registers must stay reserved until a wait the compiler emits for its
-// own scalar or LDS reads has certainly passed (any such wait covers these too, or is stricter for them): release_warm,
-// placed behind the first barrier, does that and emits nothing.  A wavefront that ends before that waits for what it has
+// come out of the scalar cache.  The four destination registers must stay reserved until the answers are in: release_warm
+// (below) ends the reservation with a wait of its own.  A wavefront that ends before that waits for what it has
 // outstanding as part of ending.
 struct WarmArguments { unsigned r0, r1, r2, r3; };
 template <int LINES>
@@ -389,7 +388,31 @@ __device__ __forceinline__ WarmArguments warm_kernel_arguments() {
     if constexpr (LINES >= 4) __asm__ volatile("s_load_dword %0, %1, 0x100" : "=&s"(w.r3) : "s"(args));
     return w;
 }
-__device__ __forceinline__ void release_warm(const WarmArguments &w) { __asm__ volatile("" ::"s"(w.r0), "s"(w.r1), "s"(w.r2), "s"(w.r3)); }
+// Lets go of the registers the lines were asked into.  The compiler does not know that the statements above are loads, so it
+// would hand these registers to other values while the answers are still on their way: they stay reserved up to here, and
+// the wait makes sure the answers are in (placed where the kernel has long waited for later requests, it costs nothing).
+__device__ __forceinline__ void release_warm(const WarmArguments &w) {
+    __asm__ volatile("s_waitcnt lgkmcnt(0)" ::"s"(w.r0), "s"(w.r1), "s"(w.r2), "s"(w.r3));
+}
+// Table words through the scalar cache, whatever the compiler can prove.  A wavefront-uniform word from memory is a scalar
+// load only when the compiler can show that nothing before it may have written memory; behind any of the statements above
+// (which it must take for writes) it becomes a vector load, and vector loads return in order -- a table word then arrives
+// behind every row requested before it, or, requested first, makes the kernel wait a whole round trip before its first
+// row request.  These ask for the word as a scalar load outright; scalar_words_arrived() is the wait, to be placed in front
+// of the first use (the answers of scalar loads do not queue behind vector requests).
+__device__ __forceinline__ int scalar_load_int(const int *p) {
+    int v;
+    __asm__ volatile("s_load_dword %0, %1, 0x0" : "=&s"(v) : "s"(p));
+    return v;
+}
+__device__ __forceinline__ unsigned long long scalar_load_u64(const void *p) {
+    unsigned long long v;
+    __asm__ volatile("s_load_dwordx2 %0, %1, 0x0" : "=&s"(v) : "s"(p));
+    return v;
+}
+__device__ __forceinline__ void scalar_words_arrived(int &a, unsigned long long &b, unsigned long long &c) {
+    __asm__ volatile("s_waitcnt lgkmcnt(0)" : "+s"(a), "+s"(b), "+s"(c));
+}
 
 // Keeps the memory requests written above this point above it: without it the compiler is free to sink a load to its
 // first use, i.e. behind whatever that use waits for.  Emits no instruction and waits for nothing.

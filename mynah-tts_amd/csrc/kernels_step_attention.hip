@@ -106,6 +106,7 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     // activation row, its LayerNorm vectors and the head's weight rows are then requested without waiting for anything.
     // (the argument structure ends 0xf8 bytes into the kernel arguments: three lines behind the first)
     static_assert(64 + sizeof(StepAttnArgs) > 0xc0 + 4, "the warmed lines lie inside the kernel arguments");
+    // (one or two streams only: with more, 1,800 workgroups asking for three more lines each made both attention stages 0.2 us slower)
     WarmArguments warm{0u, 0u, 0u, 0u};
     if constexpr (PACKED == 0) warm = warm_kernel_arguments<3>();
     int per_xcd = per_xcd_arg;
@@ -193,16 +194,22 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     // ---- slot table: read before any vector request.  The stream is the same for the whole workgroup and nothing has
     // been stored yet, so these are scalar loads, whose answers do not queue behind the vector loads below (vector loads
     // return in order: a table word requested after the weight rows could only be looked at once all of them had come).
-    const int length = PACKED ? item_length : is_self ? slots->length[b] : slots->memory_length[b];   // cache rows that exist before this step
-    float *const k_base = PACKED ? item_k : is_self ? slots->self_k[b] : const_cast<float *>(slots->cross_k[b]);
-    float *const v_base = PACKED ? item_v : is_self ? slots->self_v[b] : const_cast<float *>(slots->cross_v[b]);
+    // (asked for as scalar loads outright -- scalar_load_int, device_common.h -- and first looked at behind the row requests)
+    int length = item_length;   // cache rows that exist before this step
+    unsigned long long k_bits = reinterpret_cast<unsigned long long>(item_k), v_bits = reinterpret_cast<unsigned long long>(item_v);
+    if constexpr (PACKED == 0) {
+        const int bu = __builtin_amdgcn_readfirstlane(b);
+        length = scalar_load_int(is_self ? &slots->length[bu] : &slots->memory_length[bu]);
+        k_bits = scalar_load_u64(is_self ? static_cast<const void *>(&slots->self_k[bu]) : static_cast<const void *>(&slots->cross_k[bu]));
+        v_bits = scalar_load_u64(is_self ? static_cast<const void *>(&slots->self_v[bu]) : static_cast<const void *>(&slots->cross_v[bu]));
+    }
 
     // With many streams most of the grid belongs to units that short streams do not have: there the slot table is
     // looked at first, so that such a workgroup leaves without having requested anything.  With one or two streams
     // nearly every unit is live and the weight rows are requested before the table has arrived (latency matters more).
     if (PACKED == 0 && a.batch > kConsumerFoldMaxBatch && !(is_self && unit < 2)) {
-        const int len = is_self ? slots->length[b] : slots->memory_length[b];
-        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+        scalar_words_arrived(length, k_bits, v_bits);   // (only on this path: with one or two streams the table is first looked at behind the requests)
+        const int live = (length + kStepUnitRows - 1) / kStepUnitRows;
         if (chunk >= (is_self ? live : max(live, 1))) return;
     }
 
@@ -225,6 +232,8 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     if constexpr (PF == kPrefetchLatency) requests_issued();
 
     // ---- is this unit live, and where are its cache rows?
+    if constexpr (PACKED == 0) scalar_words_arrived(length, k_bits, v_bits);
+    float *const k_base = reinterpret_cast<float *>(k_bits), *const v_base = reinterpret_cast<float *>(v_bits);
     const int nchunks = (length + kStepUnitRows - 1) / kStepUnitRows;
     const bool new_row = role_qk || role_v;
     if (!new_row && chunk >= (is_self ? nchunks : max(nchunks, 1))) return;
@@ -371,7 +380,7 @@ k_step_attention(const StepSlots *const slots_arg, const float *const x_arg, con
     // ---- LayerNorm + activation quantisation of x[b], staged in LDS (the cache rows requested above stay in flight)
     if constexpr (PF != kPrefetchLatency) load_activations<1, NVT>(pro, act, whole_workgroup(), xr, gv, bv);
     finish_activations<QT, 1, NVT>(pro, whole_workgroup(), xr, gv, bv, smem, s_sx, s_scratch);
-    release_warm(warm);
+    if constexpr (PACKED == 0) release_warm(warm);
 
     const size_t sh = (size_t)b * a.heads + head;
     float *out_m = a.partial_ml + sh * 2 * a.max_units;
