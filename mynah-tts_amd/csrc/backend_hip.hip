@@ -1294,11 +1294,14 @@ extern "C" int mynah_hip_output_head(void *opaque, const float *const *dhidden, 
     }
     if (linear_rows(st, dhidden, dlogits, batch, width, rows, weight, bias, nullptr, nullptr, nullptr, error, capacity) != 0)
         return -1;
-    if (dprobs != nullptr)
+    if (dprobs != nullptr) {   // every stream that wants probabilities, in one launch
+        const float *from[kMaxBatch];
+        float *to[kMaxBatch];
+        size_t wanted = 0;
         for (size_t b = 0; b < batch; ++b)
-            if (dprobs[b] != nullptr &&
-                launch_softmax_heads(st, dlogits[b], dprobs[b], rows / vocab, vocab, error, capacity) != 0)
-                return -1;
+            if (dprobs[b] != nullptr) { from[wanted] = dlogits[b]; to[wanted] = dprobs[b]; ++wanted; }
+        if (launch_softmax_heads(st, from, to, wanted, rows / vocab, vocab, error, capacity) != 0) return -1;
+    }
     return 0;
 }
 

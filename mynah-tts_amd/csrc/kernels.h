@@ -184,7 +184,7 @@ int launch_copy(State *st, float *dst, const float *src, size_t n, char *error, 
 int launch_scale(State *st, float *data, size_t n, float scale, char *error, size_t capacity);
 int launch_clip(State *st, float *data, size_t n, char *error, size_t capacity);
 int launch_softmax(State *st, float *data, size_t rows, size_t cols, size_t valid, char *error, size_t capacity);
-int launch_softmax_heads(State *st, const float *logits, float *probs, size_t rows, size_t cols, char *error,
+int launch_softmax_heads(State *st, const float *const *logits, float *const *probs, size_t streams, size_t rows, size_t cols, char *error,
                          size_t capacity);
 int launch_argmax(State *st, const float *logits, size_t vocab, size_t codebook, size_t eos, int allow_eos,
                   unsigned *dev_result, char *error, size_t capacity);

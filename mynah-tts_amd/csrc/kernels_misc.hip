@@ -94,8 +94,20 @@ __device__ __forceinline__ void softmax_row_in_registers(const float *row, float
     }
 }
 
-__global__ void __launch_bounds__(256) k_softmax_heads(const float *logits, float *probs, int cols) {
+// The rows of up to kMaxBatch streams in one launch: blockIdx.y names the stream (a select over the kernel arguments).
+struct SoftmaxStreams {
+    const float *logits[kMaxBatch];
+    float *probs[kMaxBatch];
+};
+// (the first stream's rows and the row length lead the arguments: those are in registers when a wavefront starts, the
+// structure behind them is fetched from memory by the streams that need it)
+__global__ void __launch_bounds__(256) k_softmax_heads(const float *logits0, float *probs0, int cols, const SoftmaxStreams streams) {
     __shared__ float s4[4];
+    const float *logits = logits0;
+    float *probs = probs0;
+#pragma unroll
+    for (int b = 1; b < kMaxBatch; ++b)
+        if ((int)blockIdx.y == b) { logits = streams.logits[b]; probs = streams.probs[b]; }
     const float *row = logits + (size_t)blockIdx.x * cols;
     float *prow = probs + (size_t)blockIdx.x * cols;
     if (cols <= 1024) return softmax_row_in_registers<4>(row, prow, cols, s4);
@@ -297,11 +309,17 @@ int launch_softmax(State *st, float *data, size_t rows, size_t cols, size_t vali
     hipLaunchKernelGGL(k_softmax_masked, dim3((unsigned)rows), dim3(256), 0, st->stream, data, (int)cols, (int)valid);
     return hip_check(hipGetLastError(), "softmax launch", error, capacity);
 }
-int launch_softmax_heads(State *st, const float *logits, float *probs, size_t rows, size_t cols, char *error,
+int launch_softmax_heads(State *st, const float *const *logits, float *const *probs, size_t streams, size_t rows, size_t cols, char *error,
                          size_t capacity) {
-    if (rows == 0 || cols == 0) return 0;
+    if (rows == 0 || cols == 0 || streams == 0) return 0;
+    if (streams > (size_t)kMaxBatch) {
+        set_error(error, capacity, "softmax: more streams than one launch takes");
+        return -1;
+    }
     if (check_grid_rows(rows, "softmax", error, capacity) != 0) return -1;
-    hipLaunchKernelGGL(k_softmax_heads, dim3((unsigned)rows), dim3(256), 0, st->stream, logits, probs, (int)cols);
+    SoftmaxStreams s{};
+    for (size_t b = 0; b < streams; ++b) { s.logits[b] = logits[b]; s.probs[b] = probs[b]; }
+    hipLaunchKernelGGL(k_softmax_heads, dim3((unsigned)rows, (unsigned)streams), dim3(256), 0, st->stream, s.logits[0], s.probs[0], (int)cols, s);
     return hip_check(hipGetLastError(), "softmax launch", error, capacity);
 }
 int launch_argmax(State *st, const float *logits, size_t vocab, size_t codebook, size_t eos, int allow_eos,
