@@ -53,8 +53,8 @@ enum { SPEC_ANY = 0, SPEC_RESIDUAL = 1, SPEC_UP = 2 };
 // More than two streams with int8 / int4 weights: one wavefront stages one stream (load_stream_row / finish_stream_row,
 // device_common.h) -- staging every stream's activations is what such a launch spends most of its time on, every workgroup
 // has to do all of it, and a wavefront that owns a whole row needs no barrier and no exchange to normalise and quantise it.
-// The workgroup has as many wavefronts as the batch tile has streams (at least four); the first four then do the matvec as
-// the four wavefronts of a small-batch workgroup would, the others are done once the activations are staged.
+// The workgroup has as many wavefronts as the batch tile has streams (at least four); the products then go to sets of four
+// wavefronts, each set doing the matvec as the four wavefronts of a small-batch workgroup would for four of the streams.
 // For f16 / f32 weights staging is a LayerNorm or a copy by the 256 threads together.
 template <int BT, int QT>
 constexpr bool kWaveStaging = BT > kConsumerFoldMaxBatch && kQuantised<QT>;
@@ -194,7 +194,11 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                          "s"(a.fold_max_units), "s"(a.fold_is_self), "s"(a.fold_stream0), "s"(rows_per_wg), "s"(a.arith), "s"(a.epilogue));
     }
     const Team team = whole_workgroup();
-    const bool worker = !kWaves || threadIdx.x < kThreads;   // (a constant where every wavefront works: no request stands under a condition then)
+    // Products.  A workgroup's rows go to four wavefronts (wave_row); where the stream-per-wavefront builds have eight, the
+    // second four take the same rows for the upper half of the streams: PB streams per wavefront, from stream_base on.  Every
+    // wavefront works, so no request stands under a condition.
+    constexpr int PB = (kWaves && BT > 4) ? BT / 2 : BT;
+    static_assert(!kWaves || kLinearThreads<BT, QT> == kThreads * (BT / PB), "one set of four wavefronts per PB streams");
     // the arguments a specialised build does not look at
     const float *const arg_bias = SPEC != SPEC_ANY ? nullptr : a.bias;
     int8_t *const arg_probe_qx = SPEC != SPEC_ANY ? nullptr : a.probe_qx;
@@ -211,6 +215,9 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     constexpr int kEpc = Chunk<QT>::n;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
+    // (constants where the workgroup has four wavefronts, so that the small-batch builds are the code they were)
+    const int wave_row = PB != BT ? (wave & 3) : wave;
+    const int stream_base = PB != BT ? __builtin_amdgcn_readfirstlane(wave >> 2) * PB : 0;
     const int k = KFIX != 0 ? KFIX : a.k;
     const int lg = KFIX != 0 ? lane_group_log2(KFIX / kEpc) : lg_arg;
 
@@ -263,12 +270,12 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     // ------------------------------------------------------------------ loads that need no activation
     uint4 wv[4];
     float sc[4];
-    float pre_scale = 1.0f, pre_bias = 0.0f, pre_res[BT];
+    float pre_scale = 1.0f, pre_bias = 0.0f, pre_res[PB];
 #pragma unroll
-    for (int b = 0; b < BT; ++b) pre_res[b] = 0.0f;
-    const bool lanes_finish = BT > 1 && G >= BT;
-    if (worker) {
-        const int row = row_begin + wave * rows_per_pass + gidx;
+    for (int b = 0; b < PB; ++b) pre_res[b] = 0.0f;
+    const bool lanes_finish = BT > 1 && G >= PB;
+    {
+        const int row = row_begin + wave_row * rows_per_pass + gidx;
         const int rowc = row < row_end ? row : row_end - 1;
         const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(a.w) + (size_t)rowc * row_bytes);
 #pragma unroll
@@ -286,12 +293,12 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
         if (lanes_finish) {
             if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
             if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
-            if (arg_epilogue == EPI_RESIDUAL) pre_res[0] = out_of(gl < a.batch ? gl : 0)[rowc];
+            if (arg_epilogue == EPI_RESIDUAL) pre_res[0] = out_of(stream_base + gl < a.batch ? stream_base + gl : 0)[rowc];
         } else {
             if constexpr (QT == MYNAH_HIP_INT8) pre_scale = a.scales[rowc];
             if (arg_bias != nullptr) pre_bias = arg_bias[rowc];
 #pragma unroll
-            for (int b = 0; b < BT; ++b) pre_res[b] = (arg_epilogue == EPI_RESIDUAL && (b == 0 || b < a.batch)) ? out_of(b)[rowc] : 0.0f;   // a launch has at least one stream
+            for (int b = 0; b < PB; ++b) pre_res[b] = (arg_epilogue == EPI_RESIDUAL && stream_base + b < a.batch) ? out_of(stream_base + b)[rowc] : 0.0f;
         }
     }
 
@@ -305,19 +312,19 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
         finish_activations<QT, BT, NVT>(pro, team, xr, gv, bv, smem, s_sx, s_scratch);
     }
     release_warm(warm);
-    if (!worker) return;
 
     // ------------------------------------------------------------------ body
     bool first = true;
-    for (int base = row_begin + wave * rows_per_pass; base < row_end; base += pass_stride) {
+    const unsigned char *const staged = smem + (size_t)stream_base * k * (kQuantised<QT> ? 1 : 4);   // this wavefront's streams
+    for (int base = row_begin + wave_row * rows_per_pass; base < row_end; base += pass_stride) {
         const int row = base + gidx;
         const bool valid = row < row_end;
         const int rowc = valid ? row : row_end - 1;
         const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(a.w) + (size_t)rowc * row_bytes);
-        int iacc[BT];
-        float facc[BT];
+        int iacc[PB];
+        float facc[PB];
 #pragma unroll
-        for (int b = 0; b < BT; ++b) { iacc[b] = 0; facc[b] = 0.0f; }
+        for (int b = 0; b < PB; ++b) { iacc[b] = 0; facc[b] = 0.0f; }
         for (int c0 = gl; c0 < chunks; c0 += 4 * G) {
             if (!(first && c0 == gl)) {   // the first group of the first pass was loaded before the prologue
 #pragma unroll
@@ -332,18 +339,19 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                 const int c = c0 + u * G;
                 if (c < chunks) {
                     int group_int = 0;
-                    dot_chunk<QT, BT>(wv[u], sc[u], c, smem, k, iacc, facc, &group_int);
-                    if (QT == MYNAH_HIP_INT4 && arg_probe_acc != nullptr && valid) arg_probe_acc[(size_t)row * chunks + c] = group_int;
+                    dot_chunk<QT, PB>(wv[u], sc[u], c, staged, k, iacc, facc, &group_int);
+                    if (QT == MYNAH_HIP_INT4 && arg_probe_acc != nullptr && valid && stream_base == 0) arg_probe_acc[(size_t)row * chunks + c] = group_int;
                 }
             }
         }
-        group_reduce<QT, BT>(iacc, facc, lg);
+        group_reduce<QT, PB>(iacc, facc, lg);
         if (lanes_finish) {
-            if (gl < a.batch && valid) {
+            const int sb = stream_base + gl;   // the stream this lane finishes
+            if (gl < PB && sb < a.batch && valid) {
                 int mi = iacc[0];
                 float mf = facc[0];
 #pragma unroll
-                for (int b = 1; b < BT; ++b)
+                for (int b = 1; b < PB; ++b)
                     if (gl == b) { mi = iacc[b]; mf = facc[b]; }
                 float wscale = 1.0f, bias = 0.0f;
                 if (first) {
@@ -353,12 +361,12 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                     if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[row];
                     if (arg_bias != nullptr) bias = arg_bias[row];
                 }
-                float val = finish_value<QT>(mi, mf, wscale, s_sx[gl]);
-                if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && gl == 0) arg_probe_acc[row] = mi;
+                float val = finish_value<QT>(mi, mf, wscale, s_sx[sb]);
+                if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && sb == 0) arg_probe_acc[row] = mi;
                 if (arg_bias != nullptr) val += bias;
                 if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
-                float *o = out_of(gl) + row;
-                if (arg_aux_out != nullptr && gl == 0) arg_aux_out[row] = val;
+                float *o = out_of(sb) + row;
+                if (arg_aux_out != nullptr && sb == 0) arg_aux_out[row] = val;
                 if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : *o) + val;
                 *o = val;
             }
@@ -372,14 +380,15 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                 if (arg_bias != nullptr) bias = arg_bias[row];
             }
 #pragma unroll
-            for (int b = 0; b < BT; ++b) {
-                if (b < a.batch) {
-                    float val = finish_value<QT>(iacc[b], facc[b], wscale, s_sx[b]);
-                    if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && b == 0) arg_probe_acc[row] = iacc[b];
+            for (int b = 0; b < PB; ++b) {
+                const int sb = stream_base + b;
+                if (sb < a.batch) {
+                    float val = finish_value<QT>(iacc[b], facc[b], wscale, s_sx[sb]);
+                    if (QT == MYNAH_HIP_INT8 && arg_probe_acc != nullptr && sb == 0) arg_probe_acc[row] = iacc[b];
                     if (arg_bias != nullptr) val += bias;
                     if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
-                    float *o = out_of(b) + row;
-                    if (arg_aux_out != nullptr && b == 0) arg_aux_out[row] = val;
+                    float *o = out_of(sb) + row;
+                    if (arg_aux_out != nullptr && sb == 0) arg_aux_out[row] = val;
                     if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[b] : *o) + val;
                     *o = val;
                 }
