@@ -105,9 +105,11 @@ __global__ void __launch_bounds__(256) k_softmax_heads(const float *logits0, flo
     __shared__ float s4[4];
     const float *logits = logits0;
     float *probs = probs0;
+    if (blockIdx.y != 0) {   // (a branch, so that the first stream's workgroups do not wait for the structure)
 #pragma unroll
-    for (int b = 1; b < kMaxBatch; ++b)
-        if ((int)blockIdx.y == b) { logits = streams.logits[b]; probs = streams.probs[b]; }
+        for (int b = 1; b < kMaxBatch; ++b)
+            if ((int)blockIdx.y == b) { logits = streams.logits[b]; probs = streams.probs[b]; }
+    }
     const float *row = logits + (size_t)blockIdx.x * cols;
     float *prow = probs + (size_t)blockIdx.x * cols;
     if (cols <= 1024) return softmax_row_in_registers<4>(row, prow, cols, s4);
