@@ -60,10 +60,10 @@ def build_sets(pkg, synth, backend, cfg, qtype, lengths, mems, head_rows, rotate
 def run_steps(backend, sets, cfg, head_rows, vocab, count, start=0, with_head=True):
     for i in range(start, start + count):
         s = sets[i % len(sets)]
-        s["dec"].step(s["slots"])
-        if with_head:
-            backend.output_head([o.ptr for o in s["outs"]], cfg["width"], s["head"], None, head_rows, vocab,
-                                [d.ptr for d in s["logits"]], [d.ptr for d in s["probs"]])
+        if with_head:   # the step and the output head on its rows, as the one call a serving loop makes per step
+            s["dec"].step_head(s["slots"], s["head"], None, head_rows, vocab, [d.ptr for d in s["logits"]], [d.ptr for d in s["probs"]])
+        else:
+            s["dec"].step(s["slots"])
 
 
 def timed_steps(backend, sets, cfg, head_rows, vocab, steps, warmup, with_head=True):
@@ -408,8 +408,8 @@ def main():
 
     b1 = time_config(pkg, synth, backend, qtype, [1023], [256], 1024, args.steps, args.warmup)
     b1["traffic_valid"] = args.quant == "int8"
-    # 6 stage kernels x 12 layers + begin, end, head projection, head softmax
-    floor = None if args.launches else latency_floor(backend, b1["step_us"], 6 * b1["layers"] + 4)
+    # dependent launches of a step: six stages a layer, begin, the head product (which also does the final LayerNorm), its softmax
+    floor = None if args.launches else latency_floor(backend, b1["step_us"], 6 * b1["layers"] + 3)
     int4 = None
     if args.quant == "int8" and not args.skip_int4:
         int4 = time_config(pkg, synth, backend, pkg.INT4, [1023], [256], 1024, max(args.steps // 3, 20), max(args.warmup // 3, 6), stages=False)

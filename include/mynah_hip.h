@@ -351,6 +351,17 @@ int mynah_hip_output_head(void *state, const float *const *dev_hidden, size_t ba
                           const float *weight, const float *bias, size_t rows, size_t vocab,
                           float *const *dev_logits, float *const *dev_probs, char *error, size_t error_capacity);
 
+/* mynah_hip_decoder_step followed by mynah_hip_output_head on the slots' outputs, as one call: what slot_advance does with every
+ * step's rows (src/graph.c:3873-3905 takes final_proj of the step's output).  Same results in the same places -- every slot's
+ * dev_output holds the final-normed row, dev_logits / dev_probs what the head gives -- within the head's own tolerance: where
+ * the step runs as one group of stage kernels with a final LayerNorm (up to 8 streams, head shapes the fused matvec takes),
+ * the LayerNorm is the head product's prologue instead of a kernel of its own, one dependent launch less per step; the
+ * normalised rows are the bits of the separate form.  Elsewhere the two calls run one after the other.  A step of this
+ * entry whose bounded wait gives up is reported at the next synchronising call and not repeated (its rows have been consumed). */
+int mynah_hip_decoder_step_head(void *state, mynah_hip_decoder *decoder, const mynah_hip_decoder_slot *slots, size_t batch,
+                                const float *weight, const float *bias, size_t rows, size_t vocab, float *const *dev_logits,
+                                float *const *dev_probs, char *error, size_t error_capacity);
+
 /* Measurement helper (no counterpart in the reference): enqueue one stage of the step -- all layers, as its own
  * captured graph, with the slot table of the last mynah_hip_decoder_step of this batch size -- so that a caller can
  * time that kernel alone in the step's own setting between mynah_hip_timer_begin / _end.  Overwrites the decoder's

@@ -544,6 +544,16 @@ class Decoder:
                                  s["inp"], s["out"])
         self.backend._call("mynah_hip_decoder_step", self.handle, arr, _sz(B))
 
+    def step_head(self, slots, weight, bias, rows, vocab, dlogits, dprobs):
+        """The step and the output head on the slots' outputs as one call (mynah_hip_decoder_step_head)."""
+        B = len(slots)
+        arr = (DecoderSlot * B)()
+        for i, s in enumerate(slots):
+            arr[i] = DecoderSlot(s["k"], s["v"], s.get("ck"), s.get("cv"), s["length"], s.get("memory_length", 0), s["inp"], s["out"])
+        ptrs = _vp * B
+        self.backend._call("mynah_hip_decoder_step_head", self.handle, arr, _sz(B), _np_ptr(weight), _np_ptr(bias), _sz(rows), _sz(vocab),
+                           ptrs(*dlogits), None if dprobs is None else ptrs(*dprobs))
+
     def step_probe(self, slots):
         """One step of one or two streams as plain launches; returns (qx [layers, 6, ffn] int8, sx [layers, 6] f32) of stream 0:
         the int8 activations and scales the device formed at each projection (qkv, o_self, q_cross, o_cross, up, down)."""

@@ -252,14 +252,21 @@ int cached_vector(State *st, const float *host, size_t n, const float **dev, cha
 }
 
 // out[b] = W in[b] (+bias) for `batch` device rows: fused matvec tiles, or the generic f32 GEMM.
+// ln_gain (device vector) non-null: the rows are normalised first (LayerNorm prologue of the product; one weight pass only), and
+// with ln_out_slots every stream's normalised row is also stored at that device table's output[stream].
 static int linear_rows(State *st, const float *const *in, float *const *out, size_t batch, size_t iw, size_t ow,
                        const float *weight, const float *bias, int8_t *probe_qx, float *probe_sx, int32_t *probe_acc,
-                       char *error, size_t capacity) {
+                       char *error, size_t capacity, const float *ln_gain = nullptr, const float *ln_bias = nullptr,
+                       const StepSlots *ln_out_slots = nullptr) {
     const float *dbias = nullptr;
     if (cached_vector(st, bias, ow, &dbias, error, capacity) != 0) return -1;
     const CachedWeight *cw = nullptr;
     const int want = batch <= kQuantMaxRows ? st->qtype : MYNAH_HIP_F32;
     if (cached_matrix(st, weight, ow, iw, want, &cw, error, capacity) != 0) return -1;
+    if (ln_gain != nullptr && (!linear_fast_supported(cw->qtype, ow, iw) || batch > (size_t)kBatchTile)) {
+        set_error(error, capacity, "linear: a LayerNorm prologue takes one weight pass of the fused matvec");
+        return -1;
+    }
     if (!linear_fast_supported(cw->qtype, ow, iw)) {
         for (size_t b = 0; b < batch; ++b)
             if (launch_gemm_f32(st, in[b], out[b], 1, iw, ow, static_cast<const float *>(cw->data), dbias, error, capacity) != 0)
@@ -281,6 +288,9 @@ static int linear_rows(State *st, const float *const *in, float *const *out, siz
         }
         a.arith = st->arith;
         a.epilogue = EPI_NONE;
+        a.ln_gain = ln_gain;
+        a.ln_bias = ln_bias;
+        a.ln_out_slots = ln_out_slots;
         a.probe_qx = probe_qx;
         a.probe_sx = probe_sx;
         a.probe_acc = probe_acc;
@@ -1283,16 +1293,21 @@ extern "C" int mynah_hip_embed_gather(void *opaque, const float *const *tables, 
                          dout, error, capacity);
 }
 
-extern "C" int mynah_hip_output_head(void *opaque, const float *const *dhidden, size_t batch, size_t width, const float *weight,
-                                     const float *bias, size_t rows, size_t vocab, float *const *dlogits,
-                                     float *const *dprobs, char *error, size_t capacity) {
-    State *st = enter_state(opaque);
+// The output head on rows that are already normalised (x_rows null), or on the residual rows x_rows[b * width] with the final
+// LayerNorm as the product's prologue, the normalised rows written through ln_out_slots (mynah_hip_decoder_step_head).
+int mynah::output_head_rows(State *st, const float *const *dhidden, size_t batch, size_t width, const float *weight, const float *bias, size_t rows,
+                            size_t vocab, float *const *dlogits, float *const *dprobs, const float *x_rows, const float *ln_gain, const float *ln_bias,
+                            char *error, size_t capacity, const StepSlots *ln_out_slots) {
     if (batch == 0) return 0;
     if (batch > (size_t)kMaxBatch || dhidden == nullptr || dlogits == nullptr || vocab == 0 || rows % vocab != 0) {
         set_error(error, capacity, "invalid output head arguments");
         return -1;
     }
-    if (linear_rows(st, dhidden, dlogits, batch, width, rows, weight, bias, nullptr, nullptr, nullptr, error, capacity) != 0)
+    const float *residual[kMaxBatch];
+    if (x_rows != nullptr)
+        for (size_t b = 0; b < batch; ++b) residual[b] = x_rows + b * width;
+    if (linear_rows(st, x_rows != nullptr ? residual : dhidden, dlogits, batch, width, rows, weight, bias, nullptr, nullptr, nullptr, error, capacity,
+                    x_rows != nullptr ? ln_gain : nullptr, x_rows != nullptr ? ln_bias : nullptr, x_rows != nullptr ? ln_out_slots : nullptr) != 0)
         return -1;
     if (dprobs != nullptr) {   // every stream that wants probabilities, in one launch
         const float *from[kMaxBatch];
@@ -1303,6 +1318,13 @@ extern "C" int mynah_hip_output_head(void *opaque, const float *const *dhidden, 
         if (launch_softmax_heads(st, from, to, wanted, rows / vocab, vocab, error, capacity) != 0) return -1;
     }
     return 0;
+}
+
+extern "C" int mynah_hip_output_head(void *opaque, const float *const *dhidden, size_t batch, size_t width, const float *weight,
+                                     const float *bias, size_t rows, size_t vocab, float *const *dlogits,
+                                     float *const *dprobs, char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    return output_head_rows(st, dhidden, batch, width, weight, bias, rows, vocab, dlogits, dprobs, nullptr, nullptr, nullptr, error, capacity);
 }
 
 // The decoder head when no local transformer follows (slot_advance, src/graph.c:3873-3905): for every slot and every stacked

@@ -207,6 +207,10 @@ int lane_stream(State *st, int lane, hipStream_t *stream, char *error, size_t ca
 // Runs the step recorded in the state again, as plain launches in the form whose workgroups never wait for each other (fold
 // kernel behind the attention launches, no persistent launch); the cache rows it appends are the ones the first run wrote to
 // (decoder_step.hip).
+// The output head on normalised rows, or on residual rows with the final LayerNorm as the product's prologue (backend_hip.hip).
+int output_head_rows(State *st, const float *const *dhidden, size_t batch, size_t width, const float *weight, const float *bias, size_t rows,
+                     size_t vocab, float *const *dlogits, float *const *dprobs, const float *x_rows, const float *ln_gain, const float *ln_bias,
+                     char *error, size_t capacity, const StepSlots *ln_out_slots = nullptr);
 int rerun_last_step_without_waits(State *st, char *error, size_t capacity);
 
 // First statement of every entry point that is not itself part of the seam fusion: launches what is held back, so that

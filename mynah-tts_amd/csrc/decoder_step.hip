@@ -61,8 +61,10 @@ struct mynah_hip_decoder {
     float *probe_sx = nullptr;
     int max_units = 0;
     bool fused_attention = false;
-    hipGraphExec_t graphs[mynah::kMaxBatch + 1] = {};   // by stream count: this lane's layer kernels as one chain of kernel nodes
-    int eager_steps[mynah::kMaxBatch + 1] = {};   // a stream count runs eagerly once before it is captured
+    // [with the end kernel or without it][stream count]: this lane's layer kernels as one chain of kernel nodes (without the
+    // end kernel: the step whose final LayerNorm the output head's product does, mynah_hip_decoder_step_head)
+    hipGraphExec_t graphs[2][mynah::kMaxBatch + 1] = {};
+    int eager_steps[2][mynah::kMaxBatch + 1] = {};   // a stream count runs eagerly once before it is captured
     hipGraphExec_t stage_graphs[MYNAH_HIP_STAGE_COUNT][mynah::kMaxBatch + 1] = {};   // single-stage graphs (measurement only)
     int arith = 0;
     // Lanes: a batch above two streams is cut into groups that step side by side, each on a stream of its own with
@@ -347,8 +349,9 @@ extern "C" void mynah_hip_decoder_destroy(void *opaque, mynah_hip_decoder *d) {
         mynah_hip_decoder_destroy(opaque, d->lanes[i]);
     }
     d->lanes.clear();
-    for (auto &g : d->graphs)
-        if (g != nullptr) (void)hipGraphExecDestroy(g);
+    for (auto &form : d->graphs)
+        for (auto &g : form)
+            if (g != nullptr) (void)hipGraphExecDestroy(g);
     for (auto &row : d->stage_graphs)
         for (auto &g : row)
             if (g != nullptr) (void)hipGraphExecDestroy(g);
@@ -643,34 +646,36 @@ static StepSlots lane_slots(const StepSlots &s, const LanePlan &p, int lane) {
 // kernel attribute set-up does not belong in a capture) and in graph mode 0, else as the lane's captured graph of that count.
 // A graph is a single chain of kernel nodes -- the form the runtime replays without touching each node on the host; one
 // graph with a branch per lane was measured at 4.2 us of host time per node, 670 us for the two chains of a batch of eight.
-static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t stream, char *error, size_t capacity) {
+static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t stream, char *error, size_t capacity, bool with_end = true) {
     hipStream_t main_stream = st->stream;
     st->stream = stream;   // the launch wrappers enqueue on the state's stream
     int rc = 0;
-    if (st->graph_mode == 0 || lane->eager_steps[count] == 0) {
-        lane->eager_steps[count] = 1;
-        rc = enqueue_layers(st, lane, count, error, capacity);
+    const int form = with_end ? 0 : 1;
+    if (st->graph_mode == 0 || lane->eager_steps[form][count] == 0) {
+        lane->eager_steps[form][count] = 1;
+        rc = enqueue_layers(st, lane, count, error, capacity, kAllStages, with_end);
     } else {
-        if (lane->graphs[count] == nullptr) {
+        hipGraphExec_t &exec = lane->graphs[form][count];
+        if (exec == nullptr) {
             hipGraph_t graph = nullptr;
             rc = hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal), "begin capture", error, capacity);
             if (rc == 0) {
-                rc = enqueue_layers(st, lane, count, error, capacity);
+                rc = enqueue_layers(st, lane, count, error, capacity, kAllStages, with_end);
                 const hipError_t end = hipStreamEndCapture(stream, &graph);
                 if (rc == 0) rc = hip_check(end, "end capture", error, capacity);
-                if (rc == 0) rc = hip_check(hipGraphInstantiate(&lane->graphs[count], graph, nullptr, nullptr, 0), "graph instantiate", error, capacity);
+                if (rc == 0) rc = hip_check(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "graph instantiate", error, capacity);
                 if (graph != nullptr) (void)hipGraphDestroy(graph);
-                if (rc != 0) lane->graphs[count] = nullptr;
+                if (rc != 0) exec = nullptr;
             }
         }
-        if (rc == 0) rc = hip_check(hipGraphLaunch(lane->graphs[count], stream), "graph launch", error, capacity);
+        if (rc == 0) rc = hip_check(hipGraphLaunch(exec, stream), "graph launch", error, capacity);
     }
     st->stream = main_stream;
     return rc;
 }
 
 // Every lane of a step: lane 0 on the backend's stream, the others on theirs, forked from and joined to it by events.
-static int run_lanes(State *st, mynah_hip_decoder *d, const LanePlan &p, char *error, size_t capacity) {
+static int run_lanes(State *st, mynah_hip_decoder *d, const LanePlan &p, char *error, size_t capacity, bool with_end = true) {
     hipStream_t main_stream = st->stream;
     if (p.lanes > 1) {
         MYNAH_TRY(hipEventRecord(st->lane_fork, main_stream));
@@ -678,7 +683,7 @@ static int run_lanes(State *st, mynah_hip_decoder *d, const LanePlan &p, char *e
     }
     int rc = 0;
     for (int i = p.lanes - 1; i >= 0 && rc == 0; --i) {   // the owner's lane last: its stream is the one the caller's next work queues behind
-        rc = run_lane(st, d->lanes[i], p.count[i], i == 0 ? main_stream : st->lane_streams[i], error, capacity);
+        rc = run_lane(st, d->lanes[i], p.count[i], i == 0 ? main_stream : st->lane_streams[i], error, capacity, with_end);
         if (i > 0 && rc == 0) rc = hip_check(hipEventRecord(st->lane_done[i], st->lane_streams[i]), "lane event", error, capacity);
     }
     for (int i = 1; i < p.lanes && rc == 0; ++i) rc = hip_check(hipStreamWaitEvent(main_stream, st->lane_done[i], 0), "lane join", error, capacity);
@@ -702,9 +707,11 @@ int decoder_next_epochs(State *st, mynah_hip_decoder *d, unsigned count, unsigne
 }
 }  // namespace mynah
 
-extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch,
-                                      char *error, size_t capacity) {
-    State *st = enter_state(opaque);
+// The step, with its end kernel (the final LayerNorm into every slot's output) or -- one lane, no persistent form -- without:
+// *ended says which it was.
+static int decoder_step(State *st, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch, bool want_end, bool *ended, char *error,
+                        size_t capacity) {
+    *ended = true;
     if (batch == 0) return 0;   // src/graph.c:3132
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "decoder batch exceeds MYNAH_MAX_BATCH");   // src/graph.c:3133-3136
@@ -752,6 +759,8 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
     }
     const int lanes = lanes_for(st, d, B);
     if (ensure_lanes(st, d, lanes, error, capacity) != 0) return -1;
+    const bool with_end = want_end || lanes != 1 || !d->fused_attention;
+    *ended = with_end;
     const LanePlan plan = plan_lanes(s, B, lanes);
     d->last_batch_slots = s;
     d->last_lanes = lanes;
@@ -765,7 +774,41 @@ extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const 
                               capacity) != 0)
             return -1;
     }
-    return run_lanes(st, d, plan, error, capacity);
+    return run_lanes(st, d, plan, error, capacity, with_end);
+}
+
+extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch,
+                                      char *error, size_t capacity) {
+    State *st = enter_state(opaque);
+    bool ended = true;
+    return decoder_step(st, d, slots, batch, true, &ended, error, capacity);
+}
+
+// The step and the output head in one call.  Where the step runs as one lane of stage kernels, its end kernel is left out and
+// the head's product does the final LayerNorm in its prologue -- it reads the residual rows, and its first workgroup writes
+// every stream's normalised row to the slot's output, so the caller finds there what mynah_hip_decoder_step leaves -- which
+// takes one dependent launch off the step.  Elsewhere (lanes, the persistent form, head shapes the matvec does not take) the
+// two calls run one after the other.  A step whose bounded wait gives up is reported, not repeated: the head has consumed it.
+extern "C" int mynah_hip_decoder_step_head(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch, const float *weight,
+                                           const float *bias, size_t rows, size_t vocab, float *const *dlogits, float *const *dprobs, char *error,
+                                           size_t capacity) {
+    State *st = enter_state(opaque);
+    if (batch == 0) return 0;
+    if (st == nullptr || d == nullptr || slots == nullptr || weight == nullptr || dlogits == nullptr || vocab == 0 || rows % vocab != 0 || rows == 0 ||
+        batch > (size_t)kMaxBatch) {
+        set_error(error, capacity, "invalid decoder step + head arguments");
+        return -1;
+    }
+    const float *hidden[kMaxBatch];
+    for (size_t b = 0; b < batch; ++b) hidden[b] = slots[b].dev_output;
+    // (the fused form's product takes one weight pass and the matvec's shapes; the decision must precede the step)
+    const bool fusable = batch <= (size_t)kBatchTile && d->norm_out != nullptr && linear_fast_supported(st->qtype, rows, d->width) && rows <= 0x7fffffffu;
+    bool ended = true;
+    if (decoder_step(st, d, slots, batch, !fusable, &ended, error, capacity) != 0) return -1;
+    if (ended) return output_head_rows(st, hidden, batch, d->width, weight, bias, rows, vocab, dlogits, dprobs, nullptr, nullptr, nullptr, error, capacity);
+    st->last_step_decoder = nullptr;   // (not repeatable behind the head)
+    return output_head_rows(st, hidden, batch, d->width, weight, bias, rows, vocab, dlogits, dprobs, d->x, d->norm_out, d->norm_out_b, error, capacity,
+                            d->dev_slots);
 }
 
 int mynah::rerun_last_step_without_waits(State *st, char *error, size_t capacity) {

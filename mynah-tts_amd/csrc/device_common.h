@@ -160,8 +160,63 @@ __device__ __forceinline__ void layernorm_row_in_registers(const float *x, float
     }
 }
 
+// The same for rows of whole float4s (width a multiple of 4, at most 1024 * NV4 values, 16-byte aligned rows), with every sum
+// formed exactly as the fused matvec's LayerNorm prologue forms it (finish_activations below: a thread's float4s f = tid + 256 i,
+// each added as (x + y) + (z + w), lanes by butterfly, wavefronts 0..3) -- so a row normalised here and a row normalised by a
+// product's prologue are the same bits, whichever of the two a caller's sequence of calls ends up in.
+template <int NV4>
+__device__ __forceinline__ void layernorm_row_as_prologue(const float *x, float *y, const float *gain, const float *bias, int width, float *s4) {
+    const int nf4 = width >> 2;
+    const int tid = threadIdx.x & 255;
+    float4 xv[NV4], gv[NV4], bv[NV4];
+    const float *bias_or_gain = bias != nullptr ? bias : gain;
+#pragma unroll
+    for (int i = 0; i < NV4; ++i) {
+        const int f = tid + 256 * i, at = f < nf4 ? f : nf4 - 1;
+        xv[i] = reinterpret_cast<const float4 *>(x)[at];
+        gv[i] = reinterpret_cast<const float4 *>(gain)[at];
+        bv[i] = reinterpret_cast<const float4 *>(bias_or_gain)[at];
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV4; ++i) {
+        const float4 v = tid + 256 * i < nf4 ? xv[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        s += (v.x + v.y) + (v.z + v.w);
+    }
+    const float mean = block_sum(s, s4) / (float)width;
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV4; ++i)
+        if (tid + 256 * i < nf4) {
+            const float d0 = xv[i].x - mean, d1 = xv[i].y - mean, d2 = xv[i].z - mean, d3 = xv[i].w - mean;
+            q = __builtin_fmaf(d0, d0, q);
+            q = __builtin_fmaf(d1, d1, q);
+            q = __builtin_fmaf(d2, d2, q);
+            q = __builtin_fmaf(d3, d3, q);
+        }
+    const float variance = block_sum(q, s4);
+    const float scale = 1.0f / sqrtf(variance / (float)width + 1.0e-5f);
+#pragma unroll
+    for (int i = 0; i < NV4; ++i) {
+        const int f = tid + 256 * i;
+        if (f < nf4) {
+            float4 z;
+            z.x = ((xv[i].x - mean) * scale) * gv[i].x;
+            z.y = ((xv[i].y - mean) * scale) * gv[i].y;
+            z.z = ((xv[i].z - mean) * scale) * gv[i].z;
+            z.w = ((xv[i].w - mean) * scale) * gv[i].w;
+            if (bias != nullptr) { z.x += bv[i].x; z.y += bv[i].y; z.z += bv[i].z; z.w += bv[i].w; }
+            reinterpret_cast<float4 *>(y)[f] = z;
+        }
+    }
+}
+
 __device__ __forceinline__ void layernorm_row(const float *x, float *y, const float *gain, const float *bias, int width,
                                               float *s4) {
+    const bool whole4 = (width & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(gain) |
+                                              reinterpret_cast<uintptr_t>(bias)) & 15) == 0;
+    if (whole4 && width <= 1024) return layernorm_row_as_prologue<1>(x, y, gain, bias, width, s4);
+    if (whole4 && width <= 3072) return layernorm_row_as_prologue<3>(x, y, gain, bias, width, s4);
     if (width <= 1024) return layernorm_row_in_registers<4>(x, y, gain, bias, width, s4);
     if (width <= 4096) return layernorm_row_in_registers<16>(x, y, gain, bias, width, s4);
     float s = 0.0f;
@@ -497,6 +552,7 @@ struct PrologueParams {
     int8_t *probe_qx;       // parity probes for stream 0 (written by workgroup 0 only)
     float *probe_sx;
     float *ln_out = nullptr;   // non-null: workgroup 0 also stores stream 0's LayerNorm row here
+    const StepSlots *ln_out_slots = nullptr;   // non-null: workgroup 0 stores every stream's LayerNorm row at this table's output[stream]
     float *act_out = nullptr;  // non-null: workgroup 0 also stores stream 0's row as loaded (after a fold, before LayerNorm)
 };
 
@@ -598,6 +654,8 @@ __device__ __forceinline__ void finish_activations(const PrologueParams &p, cons
                 xr[b][i] = y;   // lanes beyond the row hold gain 0 -> 0
                 if (p.ln_out != nullptr && blockIdx.x == 0 && team.stream0 + b == 0 && tid + kThreads * i < nf4)
                     reinterpret_cast<float4 *>(p.ln_out)[tid + kThreads * i] = y;
+                if (p.ln_out_slots != nullptr && blockIdx.x == 0 && team.stream0 + b < p.batch && tid + kThreads * i < nf4)
+                    reinterpret_cast<float4 *>(p.ln_out_slots->output[team.stream0 + b])[tid + kThreads * i] = y;
             }
         }
     }
@@ -756,6 +814,7 @@ __device__ __forceinline__ void finish_stream_row(const PrologueParams &p, const
                 }
                 xr[v * NVT + i] = y;
                 if (p.ln_out != nullptr && first && f < nf4) reinterpret_cast<float4 *>(p.ln_out)[f] = y;
+                if (p.ln_out_slots != nullptr && blockIdx.x == 0 && live && f < nf4) reinterpret_cast<float4 *>(p.ln_out_slots->output[stream])[f] = y;
             }
     }
     float amax = 0.0f;

@@ -33,6 +33,9 @@ struct LinearArgs {
     // Seam calls folded into one launch (single row only): ln_out receives the LayerNorm prologue's row, aux_out the
     // value of the product before the residual epilogue adds it -- the buffers the separate calls would have written.
     float *ln_out;
+    // The same for every stream of a launch: stream b's LayerNorm row goes to ln_out_slots->output[b] (the resident step's
+    // final LayerNorm done by the output head's product, which then stands in for the step's end kernel).
+    const StepSlots *ln_out_slots;
     float *aux_out;
     float *act_out;         // the input row as the prologue formed it (the fold of attention partials), before any LayerNorm
 };

@@ -237,6 +237,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     pro.k = k; pro.batch = a.batch; pro.ln_gain = arg_ln_gain; pro.ln_bias = arg_ln_bias; pro.arith = a.arith;
     pro.probe_qx = arg_probe_qx; pro.probe_sx = arg_probe_sx;
     pro.ln_out = SPEC != SPEC_ANY ? nullptr : a.ln_out;
+    pro.ln_out_slots = SPEC != SPEC_ANY ? nullptr : a.ln_out_slots;
     pro.act_out = SPEC != SPEC_ANY ? nullptr : a.act_out;
     constexpr int XB = kWaves ? 1 : BT, XN = kWaves ? 4 * NVT : NVT;
     float4 xr[XB][XN], gv[XN], bv[XN];
@@ -616,7 +617,7 @@ template <int QT>
 int launch_linear_q(State *st, const LinearArgs &a, char *error, size_t capacity) {
     // what the arguments rule out decides the build (see SPEC above)
     const bool plain = a.bias == nullptr && a.probe_qx == nullptr && a.probe_sx == nullptr && a.probe_acc == nullptr &&
-                       a.ln_out == nullptr && a.aux_out == nullptr && a.act_out == nullptr;
+                       a.ln_out == nullptr && a.ln_out_slots == nullptr && a.aux_out == nullptr && a.act_out == nullptr;
     // (the specialised builds for one or two streams take their small numbers packed into one argument: when one of them
     // does not fit its bit field the launch takes the general build, with the same arithmetic)
     LeadShape fit{};

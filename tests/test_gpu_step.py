@@ -694,3 +694,50 @@ def test_long_cache_takes_the_fold_kernel(pkg, backend, orc, synth, nerr):
     finally:
         h.close()
         backend.set_quant(0)
+
+
+@pytest.mark.parametrize("qtype_name,batch", [("int8", 1), ("int8", 2), ("int8", 5), ("int8", 8), ("int4", 3), ("f32", 2), ("f16", 4), ("int8", 11)])
+def test_step_and_head_in_one_call(pkg, backend, synth, nerr, qtype_name, batch):
+    """mynah_hip_decoder_step_head against mynah_hip_decoder_step followed by mynah_hip_output_head on the same streams: the
+    slots' outputs (the final-normed rows), the appended cache rows, logits and probabilities, all bit for bit -- the head
+    product's LayerNorm prologue forms its sums as the end kernel does; three steps in a row (eager, captured, replayed);
+    eleven streams take the two-call form inside the library (two lanes)."""
+    _announce("step + head in one call %s b=%d" % (qtype_name, batch))
+    rng = np.random.default_rng(11)
+    lengths = [int(v) for v in rng.integers(0, 290, batch)]
+    mems = [int(v) for v in rng.integers(0, 200, batch)]
+    cfg = synth.decoder_config(layers=2, capacity=304)
+    weights = synth.decoder_weights(cfg, seed=0)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=1)
+    head_w = (rng.standard_normal((2 * 256, cfg["width"])) * 0.02).astype(np.float32)
+    head_b = (rng.standard_normal(2 * 256) * 0.1).astype(np.float32)
+    backend.set_quant(QT[qtype_name])
+    h = Harness(pkg, backend, cfg, weights, streams)
+    dl = [backend.alloc(512) for _ in range(batch)]
+    dp = [backend.alloc(512) for _ in range(batch)]
+    for step in range(3):
+        for i in range(batch):
+            h.reset_cache(i)
+        rows = h.step()
+        backend.output_head([b["out"].ptr for b in h.bufs], cfg["width"], head_w, head_b, 512, 256, [d.ptr for d in dl], [d.ptr for d in dp])
+        want_logits = [d.read() for d in dl]
+        want_probs = [d.read() for d in dp]
+        want_cache = [h.cache_rows(i) for i in range(batch)]
+        for i in range(batch):
+            h.reset_cache(i)
+            h.bufs[i]["out"].write(np.zeros(cfg["width"], np.float32))
+            dl[i].write(np.zeros(512, np.float32))
+            dp[i].write(np.zeros(512, np.float32))
+        h.dec.step_head(h.slots(), head_w, head_b, 512, 256, [d.ptr for d in dl], [d.ptr for d in dp])
+        got_rows = [b["out"].read() for b in h.bufs]
+        for i in range(batch):
+            assert np.array_equal(got_rows[i].view(np.uint32), rows[i].view(np.uint32)), "step %d stream %d: output row" % (step, i)
+            gk, gv = h.cache_rows(i)
+            assert np.array_equal(gk, want_cache[i][0]) and np.array_equal(gv, want_cache[i][1]), "step %d stream %d: cache" % (step, i)
+            gl, gp = dl[i].read(), dp[i].read()
+            assert np.array_equal(gl.view(np.uint32), want_logits[i].view(np.uint32)), "step %d stream %d: logits" % (step, i)
+            assert np.array_equal(gp.view(np.uint32), want_probs[i].view(np.uint32)), "step %d stream %d: probabilities" % (step, i)
+    for d in dl + dp:
+        d.free()
+    h.close()
+    backend.set_quant(0)
