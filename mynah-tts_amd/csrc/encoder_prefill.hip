@@ -301,25 +301,32 @@ __global__ void __launch_bounds__(kThreads) k_enc_embed(const int *ids, const En
 // registers (width <= 256 * NV; the widest supported row, 4096, takes NV = 16).
 // (Argument order: what the row's first requests are formed from stands among the first fourteen dwords, which are in registers
 // at wavefront start; bias and the f16 destination, needed last, come out of memory.)
-template <bool F16_OUT, int NV>
-__global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *part, const EncParams *params, int rows, int width, int splits,
-                                                       size_t split_stride, const float *gain, const float *bias, _Float16 *out_f16) {
+// RPW: rows (wavefronts) per workgroup.  One: a row's 3 KB and the up to four partial planes that go with it are 15 KB of
+// requests, and four rows to a workgroup put 60 KB through one CU's L1 while three quarters of the CUs have nothing to do
+// (256 rows: 64 workgroups) -- a row per workgroup spreads them over the chip.
+// No request stands under a condition (a place beyond the row, or a partial plane the product did not write, asks for a
+// place that exists and is set to zero afterwards): the waits then name exactly the requests they need.
+template <bool F16_OUT, int NV, int RPW>
+__global__ void __launch_bounds__(64 * RPW) k_enc_rows(float *x, const float *part, const EncParams *params, int rows, int width, int splits,
+                                                        size_t split_stride, const float *gain, const float *bias, _Float16 *out_f16) {
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    const int row = blockIdx.x * RPW + (threadIdx.x >> 6);
     if (row >= rows) return;
     if constexpr (!F16_OUT) {
         if (row >= params->tokens) return;
     }
     float4 *xr = reinterpret_cast<float4 *>(x + (size_t)row * width);
     const int n4 = width / 4;
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
     float4 v[NV], gg[NV], bb[NV];
+    const float4 *const gain4 = reinterpret_cast<const float4 *>(gain != nullptr ? gain : x);   // (x: a place that exists)
+    const float4 *const bias4 = reinterpret_cast<const float4 *>(bias != nullptr ? bias : x);
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-        const int i = lane + 64 * u;
-        const bool in = i < n4;
-        v[u] = in ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        gg[u] = (in && gain != nullptr) ? reinterpret_cast<const float4 *>(gain)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        bb[u] = (in && bias != nullptr) ? reinterpret_cast<const float4 *>(bias)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        const int i = lane + 64 * u, at = i < n4 ? i : n4 - 1;
+        v[u] = xr[at];
+        gg[u] = gain4[at];
+        bb[u] = bias4[at];
     }
     if (part != nullptr) {
         // all splits are requested at once and added in split order: the sum does not depend on how the splits were scheduled
@@ -327,12 +334,19 @@ __global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *pa
         float4 p[kSplits][NV];
 #pragma unroll
         for (int z = 0; z < kSplits; ++z) {
+            const float4 *const plane = reinterpret_cast<const float4 *>(part + (z < splits ? z : splits - 1) * split_stride + (size_t)row * width);
 #pragma unroll
             for (int u = 0; u < NV; ++u) {
                 const int i = lane + 64 * u;
-                p[z][u] = (z < splits && i < n4) ? reinterpret_cast<const float4 *>(part + z * split_stride + (size_t)row * width)[i]
-                                                : make_float4(0.f, 0.f, 0.f, 0.f);
+                p[z][u] = plane[i < n4 ? i : n4 - 1];
             }
+        }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            if (lane + 64 * u >= n4) v[u] = zero4;
+#pragma unroll
+            for (int z = 0; z < kSplits; ++z)
+                if (z >= splits || lane + 64 * u >= n4) p[z][u] = zero4;
         }
 #pragma unroll
         for (int u = 0; u < NV; ++u) {
@@ -343,6 +357,13 @@ __global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *pa
             v[u].x += t.x; v[u].y += t.y; v[u].z += t.z; v[u].w += t.w;
             if (i < n4) xr[i] = v[u];
         }
+    }
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+        const bool in = lane + 64 * u < n4;
+        if (!in) v[u] = zero4;
+        if (!in || gain == nullptr) gg[u] = zero4;
+        if (!in || bias == nullptr) bb[u] = zero4;
     }
     if (gain == nullptr) {
         if constexpr (!F16_OUT) {
@@ -384,10 +405,15 @@ __global__ void __launch_bounds__(kThreads) k_enc_rows(float *x, const float *pa
 template <bool F16_OUT>
 void launch_rows(State *st, int width, dim3 grid, float *x, const float *part, int splits, size_t split_stride, const float *gain,
                  const float *bias, _Float16 *out_f16, const EncParams *params, int rows) {
+    (void)grid;
+    constexpr int kRowsPerWg = 1;
+    const dim3 rows_grid((unsigned)((rows + kRowsPerWg - 1) / kRowsPerWg));
     if (width <= 1024)
-        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 4>), grid, dim3(kThreads), 0, st->stream, x, part, params, rows, width, splits, split_stride, gain, bias, out_f16);
+        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 4, kRowsPerWg>), rows_grid, dim3(64 * kRowsPerWg), 0, st->stream, x, part, params, rows, width, splits, split_stride,
+                           gain, bias, out_f16);
     else
-        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 16>), grid, dim3(kThreads), 0, st->stream, x, part, params, rows, width, splits, split_stride, gain, bias, out_f16);
+        hipLaunchKernelGGL((k_enc_rows<F16_OUT, 16, kRowsPerWg>), rows_grid, dim3(64 * kRowsPerWg), 0, st->stream, x, part, params, rows, width, splits, split_stride,
+                           gain, bias, out_f16);
 }
 
 // One (32-query tile, head): S = scale * Q K^T over all keys (f32, in LDS) -> row softmax numerators
