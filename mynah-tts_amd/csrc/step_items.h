@@ -22,22 +22,24 @@ constexpr int kFoldUnit = 0x7fff;   // unit number of a table entry that folds i
 // kernel that advances them in the same launch can still write the next pass's tables).
 __device__ inline StepItem make_item(const StepSlots &slots, int uniform_length, int batch, int heads, bool is_self, int wg, int epoch, bool with_fold,
                                      int budget) {
-    const auto rows_of = [&](int s) { return !is_self ? slots.memory_length[s] : uniform_length >= 0 ? uniform_length : slots.length[s]; };
+    // Every stream's unit count first, from places of the table known at compile time: the loops below then run on registers.
+    // (Read inside the loops, a length was one dependent fetch from the kernel's arguments per iteration, two dozen in a row.)
+    int units[kMaxBatch];
+#pragma unroll
+    for (int s = 0; s < kMaxBatch; ++s) {
+        const int len = !is_self ? slots.memory_length[s] : uniform_length >= 0 ? uniform_length : slots.length[s];
+        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
+        units[s] = s < batch ? (is_self ? live : max(live, 1)) : 0;
+    }
     const StepItem dead{nullptr, nullptr, 0, -1, 0, 0};
     // chunks per workgroup: the smallest group size with which the launch's chunk workgroups are at most `budget`
     int all_chunks = 0;
-    for (int s = 0; s < batch; ++s) {
-        const int len = rows_of(s);
-        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-        all_chunks += is_self ? live : max(live, 1);
-    }
+#pragma unroll
+    for (int s = 0; s < kMaxBatch; ++s) all_chunks += units[s];
     const int group = max(1, (heads * all_chunks + budget - 1) / max(budget, 1));
     int chunk_items = 0;   // groups per head
-    for (int s = 0; s < batch; ++s) {
-        const int len = rows_of(s);
-        const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-        chunk_items += ((is_self ? live : max(live, 1)) + group - 1) / group;
-    }
+#pragma unroll
+    for (int s = 0; s < kMaxBatch; ++s) chunk_items += (units[s] + group - 1) / group;
     int head, b = 0, unit = 0;
     const int producers = is_self ? 2 * batch * heads : 0;
     const int producer_grid = 8 * ((producers + 7) / 8);
@@ -69,10 +71,9 @@ __device__ inline StepItem make_item(const StepSlots &slots, int uniform_length,
             head = item / chunk_items;
             const int r = item - head * chunk_items;
             int before = 0;
-            for (int s = 0; s < batch; ++s) {
-                const int len = rows_of(s);
-                const int live = (len + kStepUnitRows - 1) / kStepUnitRows;
-                const int n = ((is_self ? live : max(live, 1)) + group - 1) / group;
+#pragma unroll
+            for (int s = 0; s < kMaxBatch; ++s) {
+                const int n = (units[s] + group - 1) / group;   // (no units beyond the batch: nothing matches there)
                 if (r >= before && r < before + n) { b = s; unit = r - before + (is_self ? 2 : 0); }
                 before += n;
             }
@@ -81,7 +82,7 @@ __device__ inline StepItem make_item(const StepSlots &slots, int uniform_length,
     StepItem it;
     it.k = is_self ? slots.self_k[b] : const_cast<float *>(slots.cross_k[b]);
     it.v = is_self ? slots.self_v[b] : const_cast<float *>(slots.cross_v[b]);
-    it.length = rows_of(b);
+    it.length = !is_self ? slots.memory_length[b] : uniform_length >= 0 ? uniform_length : slots.length[b];
     it.code = head | (b << 8) | (unit << 16);
     it.epoch = epoch;
     it.group = group;
