@@ -428,11 +428,14 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
                 const int xx = lane + 64 * x;
                 if (xx < win) s_in[ch * win + xx] = stage_in[ch][x];
             }
-        __syncthreads();
+        // (no workgroup barrier in the loop: a wavefront stages into its own part of LDS and reads nothing else, and its own
+        // LDS accesses complete in the order it issued them -- the four wavefronts walk their channel blocks independently)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         if (round + 1 < rounds) fetch(round + 1);   // in flight during the products below
         conv_products<KF, NT>(s_w + col * a_stride + half * a.kernel, s_in + half * win + col, a.kernel, a.dilation, win, acc0, acc1);
-        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
+    __syncthreads();   // the partial tiles below overwrite every wavefront's staging area
     // partial tiles through LDS: [wavefront][element r][lane], then ((p0 + p1) + p2) + p3 + bias
     float *s_part = lds;
 #pragma unroll
