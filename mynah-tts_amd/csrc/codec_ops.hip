@@ -138,10 +138,15 @@ __device__ __forceinline__ void conv_products(const float *wrow, const float *ir
 // FUSED: the build that mynah_hip_conv1d_fused launches (residuals, scale, activation after the products); the seam's
 // conv1d keeps a build without any of it.
 template <int WM, int WN, int KF, int VEC, bool FUSED>
-__global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
+__global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float *const out_arg, const float *const w_arg, const float *const bias_arg, const int in_ch_arg,
+                                                const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const ConvArgs a_arg) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     extern __shared__ __align__(16) float lds[];
+    // (the rows, the weights and the shape lead the arguments and repeat fields of a_arg: leading scalar arguments are in
+    // registers when a wavefront starts, a structure passed by value is fetched from memory where its fields are first used)
     ConvArgs a = a_arg;
+    a.in = in_arg; a.out = out_arg; a.w = w_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
+    a.kernel = kernel_arg; a.dilation = dilation_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;   // inner elements per step
     const int a_stride = VEC ? kb + 4 : (kb | 1);  // odd row stride: the 32 rows a wavefront reads land in 32 different banks;
@@ -340,10 +345,15 @@ __global__ void __launch_bounds__(256) k_conv1d(const ConvArgs a_arg) {
 // partial tiles are added in wavefront order at the end, so the result does not depend on timing.  NT: 32-position
 // halves per tile (2, or 1 for the very shortest rows: twice the workgroups).
 template <int KF, int NT>
-__global__ void __launch_bounds__(256) k_conv1d_split(const ConvArgs a_arg) {
+__global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg, float *const out_arg, const float *const w_arg, const float *const bias_arg, const int in_ch_arg,
+                                                const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const ConvArgs a_arg) {
     constexpr int TM = 32, TN = 32 * NT;
     extern __shared__ __align__(16) float lds[];
+    // (the rows, the weights and the shape lead the arguments and repeat fields of a_arg: leading scalar arguments are in
+    // registers when a wavefront starts, a structure passed by value is fetched from memory where its fields are first used)
     ConvArgs a = a_arg;
+    a.in = in_arg; a.out = out_arg; a.w = w_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
+    a.kernel = kernel_arg; a.dilation = dilation_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;
     const int a_stride = kb + 4;   // rows stay 16-byte aligned and get four floats of padding: a stride of 4 mod 8 words spreads the
@@ -537,7 +547,7 @@ int launch_conv_f(State *st, const ConvArgs &a, char *error, size_t capacity) {
         raised = true;
     }
     const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM));
-    hipLaunchKernelGGL((k_conv1d<WM, WN, KF, VEC, FUSED>), grid, dim3(256), lds, st->stream, a);
+    hipLaunchKernelGGL((k_conv1d<WM, WN, KF, VEC, FUSED>), grid, dim3(256), lds, st->stream, a.in, a.out, a.w, a.bias, a.in_ch, a.out_ch, a.length, a.kernel, a.dilation, a);
     return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
 }
 
@@ -575,7 +585,7 @@ int launch_conv_split_k(State *st, const ConvArgs &a, char *error, size_t capaci
         raised = true;
     }
     const dim3 grid((unsigned)((a.length + 32 * NT - 1) / (32 * NT)), (unsigned)((a.out_ch + 31) / 32));
-    hipLaunchKernelGGL((k_conv1d_split<KF, NT>), grid, dim3(256), lds, st->stream, a);
+    hipLaunchKernelGGL((k_conv1d_split<KF, NT>), grid, dim3(256), lds, st->stream, a.in, a.out, a.w, a.bias, a.in_ch, a.out_ch, a.length, a.kernel, a.dilation, a);
     return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
 }
 
