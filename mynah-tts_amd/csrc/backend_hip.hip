@@ -1,5 +1,6 @@
 // C ABI of the gfx950 backend: state, pointer-keyed weight cache, and the seam's resident ops.
 #include <float.h>
+#include <limits.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -220,6 +221,45 @@ int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qty
     st->weight_bytes += cw.bytes;
     auto ins = st->weights.emplace(key, cw);
     *out = &ins.first->second;   // unordered_map never moves its nodes: the pointer stays valid
+    return 0;
+}
+
+int cached_conv_blocks(State *st, const float *host, size_t out_ch, size_t in_ch, size_t kernel, ConvBlocks *out, char *error, size_t capacity) {
+    if (host == nullptr || out_ch == 0 || in_ch == 0 || kernel == 0 || kernel > 64 || in_ch > (size_t)(INT_MAX / 64) ||
+        out_ch > SIZE_MAX / in_ch / kernel / sizeof(float)) {
+        set_error(error, capacity, "invalid convolution weight");
+        return -1;
+    }
+    const size_t tiles = ((out_ch + 31) / 32 + 1) & ~(size_t)1, blocks = ((in_ch + kConvChannels - 1) / kConvChannels + 3) & ~(size_t)3;
+    const size_t row = kConvChannels * kernel + 4, chunk = conv_chunk_floats(kernel);
+    out->tiles = (int)tiles;
+    out->blocks = (int)blocks;
+    const WeightKey key{host, out_ch * in_ch * kernel * sizeof(float), (int)(64 + kernel + 32 * in_ch)};
+    std::lock_guard<std::mutex> lock(st->mu);
+    auto it = st->weights.find(key);
+    if (it != st->weights.end()) {
+        out->data = static_cast<const float *>(it->second.data);
+        return 0;
+    }
+    if (tiles > (size_t)INT_MAX || tiles * blocks > SIZE_MAX / sizeof(float) / chunk / 2) {
+        set_error(error, capacity, "convolution weight too large");
+        return -1;
+    }
+    std::vector<float> packed(tiles * blocks * chunk + 1024, 0.0f);
+    for (size_t o = 0; o < out_ch; ++o)
+        for (size_t i = 0; i < in_ch; ++i) {
+            float *dst = packed.data() + ((i / kConvChannels) * tiles + o / 32) * chunk + (o % 32) * row + (i % kConvChannels) * kernel;
+            const float *src = host + (o * in_ch + i) * kernel;
+            for (size_t k = 0; k < kernel; ++k) dst[k] = src[k];
+        }
+    CachedWeight cw;
+    cw.n = out_ch;
+    cw.k = in_ch * kernel;
+    cw.bytes = packed.size() * sizeof(float);
+    if (device_copy_of(packed.data(), cw.bytes, &cw.data, error, capacity) != 0) return -1;
+    st->weight_bytes += cw.bytes;
+    st->weights.emplace(key, cw);
+    out->data = static_cast<const float *>(cw.data);
     return 0;
 }
 

@@ -25,8 +25,8 @@ using namespace mynah;
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kConvChannels = 8;      // input channels staged per step of the inner dimension
 constexpr int kConvMaxKernel = 16;
 constexpr int kConvMaxHalo = 128;     // (kernel - 1) * dilation
 constexpr int kTileStride = 65;       // floats per row of a wavefront's 32 x 64 tile in LDS (fused epilogue)
@@ -34,7 +34,6 @@ constexpr int kTileStride = 65;       // floats per row of a wavefront's 32 x 64
 struct ConvArgs {
     const float *in;     // [in_ch, length]
     float *out;          // [out_ch, length]
-    const float *w;      // [out_ch, in_ch * kernel]
     const float *bias;   // [out_ch] or null
     int in_ch, out_ch, length, kernel, dilation;
     // what mynah_hip_conv1d_fused adds after conv + bias, in this order (each step is the arithmetic of the seam operator it replaces)
@@ -106,19 +105,45 @@ __device__ __forceinline__ void conv_emit(const ConvArgs &a, int m, size_t index
 // The products of one staged block of eight input channels for a wavefront's 32 x 64 tile.  The two inner indices one
 // matrix instruction consumes are the same tap of two neighbouring channels (lanes 0-31: the even channel, lanes 32-63:
 // the odd one), so a lane walks its channel's taps with plain increments.  wrow: this lane's output row at its first
-// channel; irow: its first channel's staged row at its output position.  Operands of the next product are requested
-// before the current one is issued.
+// channel; irow: its first channel's staged row at its output position.
+// With the tap count known at compile time the operands are requested TWO products ahead and the scheduler is fenced
+// around every product: left to itself the compiler reads a product's input operand into one and the same register right
+// before it, and with one wavefront on a SIMD every product then waits out an LDS read (some 120 cycles against the 64
+// of the instruction itself).  Past the last product the requests stay inside the staging area and are not used.
 template <int KF, int NT = 2>
 __device__ __forceinline__ void conv_products(const float *wrow, const float *irow, const int kernel_arg, const int dilation, const int win,
                                               floatx16 &acc0, floatx16 &acc1) {
-    const int kernel = KF != 0 ? KF : kernel_arg;
+    if constexpr (KF != 0) {
+        constexpr int kSteps = (kConvChannels / 2) * KF;
+        float wv[3], x0[3], x1[3];
+        int tap = 0;
+        const auto request = [&](int slot) {
+            wv[slot] = wrow[0];
+            x0[slot] = irow[0];
+            x1[slot] = NT > 1 ? irow[32] : 0.0f;
+            const bool wrap = tap + 1 == KF;   // then: the first tap of the next channel pair
+            wrow += wrap ? KF + 1 : 1;
+            irow += wrap ? 2 * win - (KF - 1) * dilation : dilation;
+            tap = wrap ? 0 : tap + 1;
+        };
+        request(0);
+        request(1);
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            request((s + 2) % 3);
+            __builtin_amdgcn_sched_barrier(0x77);
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[s % 3], x0[s % 3], acc0, 0, 0, 0);
+            if constexpr (NT > 1) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[s % 3], x1[s % 3], acc1, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0x77);
+        }
+        return;
+    }
+    const int kernel = kernel_arg;
     float wv = wrow[0], x0 = irow[0], x1 = NT > 1 ? irow[32] : 0.0f;
 #pragma unroll
     for (int pair = 0; pair < kConvChannels / 2; ++pair) {
-#pragma unroll
         for (int k = 0; k < kernel; ++k) {
-            // the product after this one: the next tap, or the first tap of the next channel pair (past the last pair the
-            // addresses stay inside the staging area and the values are not used)
+            // the product after this one: the next tap, or the first tap of the next channel pair
             const bool wrap = k + 1 == kernel;
             wrow += wrap ? kernel + 1 : 1;
             irow += wrap ? 2 * win - (kernel - 1) * dilation : dilation;
@@ -132,102 +157,78 @@ __device__ __forceinline__ void conv_products(const float *wrow, const float *ir
 
 // Workgroup tile: (32 * WM) output channels x (64 * WN) positions; a wavefront owns 32 x 64 (two 32 x 32 accumulators).
 // KF: number of taps known at compile time (0 = from the arguments): the staging loops then have exactly as many slots as
-// the block has columns and the product loop is straight-line code.  The codec's 3, 7 and 11 taps get such builds.
-// VEC: the weight rows are whole 16-byte pieces (in_ch * kernel a multiple of 4): the weight block is staged four
-// elements per request and kept in LDS with packed rows.
+// the block has 16-byte pieces and the product loop is straight-line code.  The codec's 3, 7 and 11 taps get such builds.
+// The weights arrive cut into chunks (ConvBlocks): the tile's block of a step is WM whole chunks in a row, already in the
+// layout LDS keeps, so staging it is a plain copy -- no index arithmetic, no bounds.
 // FUSED: the build that mynah_hip_conv1d_fused launches (residuals, scale, activation after the products); the seam's
 // conv1d keeps a build without any of it.
-template <int WM, int WN, int KF, int VEC, bool FUSED>
-__global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float *const out_arg, const float *const w_arg, const float *const bias_arg, const int in_ch_arg,
-                                                const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const ConvArgs a_arg) {
+template <int WM, int WN, int KF, bool FUSED>
+__global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float *const out_arg, const float *const chunks_arg, const float *const bias_arg, const int in_ch_arg,
+                                                const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const int tiles_arg,
+                                                const ConvArgs a_arg) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
     extern __shared__ __align__(16) float lds[];
     // (the rows, the weights and the shape lead the arguments and repeat fields of a_arg: leading scalar arguments are in
     // registers when a wavefront starts, a structure passed by value is fetched from memory where its fields are first used)
     ConvArgs a = a_arg;
-    a.in = in_arg; a.out = out_arg; a.w = w_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
+    a.in = in_arg; a.out = out_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
     a.kernel = kernel_arg; a.dilation = dilation_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;   // inner elements per step
-    const int a_stride = VEC ? kb + 4 : (kb | 1);  // odd row stride: the 32 rows a wavefront reads land in 32 different banks;
-                                                   // with 16-byte staging rows stay 16-byte aligned and get four floats of padding
-                                                   // (a stride of 4 mod 8 words spreads them over eight banks instead of four)
+    const int a_stride = kb + 4;               // the chunks' row stride: rows stay 16-byte aligned, and a stride of 4 mod 8 words
+                                               // spreads the 32 rows a wavefront reads for a product over eight banks
     const int halo = (a.kernel - 1) * a.dilation;
     const int win = TN + halo;                 // staged positions per input channel
-    float *s_w = lds;                          // [TM][a_stride]
-    float *s_in = lds + TM * a_stride;         // [kConvChannels][win]
+    // 16-byte pieces of the tile's weight block, and the slots (one piece per thread) that cover them; the last slot may
+    // reach past the block, into the next chunk or the zeros after the last one, and lands in LDS the products never read
+    constexpr int kSlots = (WM * 8 * (kConvChannels * (KF != 0 ? KF : kConvMaxKernel) + 4) + 255) / 256;
+    const int pieces = WM * 8 * a_stride;
+    const int slots = KF != 0 ? kSlots : (pieces + 255) / 256;
+    float *s_w = lds;                          // [TM][a_stride], then the last slot's excess
+    float *s_in = lds + slots * 1024;          // [kConvChannels][win]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int m0 = blockIdx.y * TM, t0 = blockIdx.x * TN;
-    const int inner = a.in_ch * a.kernel;
 
-    // Staging slots of a thread: weights -- row (tid / 16) + 16 * g, column (tid % 16) + 16 * c of the step's TM x kb
-    // block; input rows -- channel ch, position tid + 256 * x of the window.  Fixed loops, no divisions.
-    constexpr int kRowGroups = TM / 16, kColGroups = (kConvChannels * (KF != 0 ? KF : kConvMaxKernel) + 15) / 16;
+    // Staging slots of a thread: weights -- piece tid + 256 * c of the block; input rows -- channel ch, position
+    // tid + 256 * x of the window (its place in the row is the same for every block: kept, -1 outside the row).
     constexpr int kWinParts = (TN + kConvMaxHalo + 255) / 256;
-    constexpr int kVecSlots = (TM * kConvChannels * (KF != 0 ? KF : kConvMaxKernel) / 4 + 255) / 256;
-    float stage_w[VEC ? 1 : kRowGroups][VEC ? 1 : kColGroups], stage_in[kConvChannels][kWinParts];
-    float4 stage_w4[VEC ? kVecSlots : 1];
-    const int srow = tid >> 4, scol = tid & 15;
-    const int kb4 = kb / 4;
-    const auto fetch = [&](int i0) {   // global -> registers: the weight columns and input rows of channels [i0, i0 + 8)
-        if constexpr (VEC != 0) {
-            int tid_now = tid;
-            __asm__ volatile("" : "+v"(tid_now));   // slot rows recomputed per step rather than held in registers
+    floatx4 stage_w[kSlots];
+    float stage_in[kConvChannels][kWinParts];
+    int in_pos[kWinParts];
 #pragma unroll
-            for (int c = 0; c < kVecSlots; ++c) {
-                const int e = tid_now + 256 * c, row = e / kb4, cc = 4 * (e - row * kb4);
-                const int m = m0 + row, ci = i0 * a.kernel + cc;
-                const bool valid = row < TM && m < a.out_ch && ci < inner;
-                const float4 v = *reinterpret_cast<const float4 *>(a.w + (valid ? (size_t)m * inner + ci : 0));
-                stage_w4[c] = valid ? v : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-        }
+    for (int x = 0; x < kWinParts; ++x) {
+        const int xx = tid + 256 * x, t = t0 - halo + xx;
+        in_pos[x] = (xx < win && t >= 0 && t < a.length) ? t : -1;
+    }
+    const floatx4 *w_next = reinterpret_cast<const floatx4 *>(chunks_arg) + (size_t)(WM * blockIdx.y) * (8 * a_stride) + tid;   // this thread's first piece
+    const size_t w_step = (size_t)tiles_arg * (8 * a_stride);   // pieces from a block to the next
+    const auto fetch = [&](int i0) {   // global -> registers: the weight block and input rows of channels [i0, i0 + 8); nothing waits here
 #pragma unroll
-        for (int g = 0; g < (VEC ? 0 : kRowGroups); ++g) {
-            const int m = m0 + srow + 16 * g;
-#pragma unroll
-            for (int c = 0; c < kColGroups; ++c) {
-                const int cc = scol + 16 * c, ci = i0 * a.kernel + cc;
-                const bool valid = cc < kb && m < a.out_ch && ci < inner;
-                const float v = a.w[valid ? (size_t)m * inner + ci : 0];   // always a legal address: no branch around the load
-                stage_w[g][c] = valid ? v : 0.0f;
-            }
-        }
+        for (int c = 0; c < kSlots; ++c)
+            if (KF != 0 || c < slots) stage_w[c] = w_next[256 * c];
+        w_next += w_step;
 #pragma unroll
         for (int ch = 0; ch < kConvChannels; ++ch) {
-            const int i = i0 + ch;
+            const bool row_exists = i0 + ch < a.in_ch;
+            const float *row = a.in + (row_exists ? (size_t)(i0 + ch) * a.length : 0);
 #pragma unroll
-            for (int x = 0; x < kWinParts; ++x) {
-                const int xx = tid + 256 * x, t = t0 - halo + xx;
-                const bool valid = xx < win && i < a.in_ch && t >= 0 && t < a.length;
-                const float v = a.in[valid ? (size_t)i * a.length + t : 0];
-                stage_in[ch][x] = valid ? v : 0.0f;
-            }
+            for (int x = 0; x < kWinParts; ++x) stage_in[ch][x] = row[in_pos[x] >= 0 ? in_pos[x] : 0];   // always a legal address
         }
     };
-    const auto publish = [&]() {   // registers -> LDS
-        if constexpr (VEC != 0) {
+    const auto publish = [&](int i0) {   // registers -> LDS (zeros where the input has no such channel or position)
 #pragma unroll
-            for (int c = 0; c < kVecSlots; ++c) {
-                const int e = tid + 256 * c, row = e / kb4, c4 = e - row * kb4;
-                if (e < TM * kb4) reinterpret_cast<float4 *>(s_w + row * a_stride)[c4] = stage_w4[c];
-            }
-        }
+        for (int c = 0; c < kSlots; ++c)
+            if (KF != 0 || c < slots) reinterpret_cast<floatx4 *>(s_w)[tid + 256 * c] = stage_w[c];
 #pragma unroll
-        for (int g = 0; g < (VEC ? 0 : kRowGroups); ++g)
-#pragma unroll
-            for (int c = 0; c < kColGroups; ++c) {
-                const int cc = scol + 16 * c;
-                if (cc < kb) s_w[(srow + 16 * g) * a_stride + cc] = stage_w[g][c];
-            }
-#pragma unroll
-        for (int ch = 0; ch < kConvChannels; ++ch)
+        for (int ch = 0; ch < kConvChannels; ++ch) {
+            const bool row_exists = i0 + ch < a.in_ch;
 #pragma unroll
             for (int x = 0; x < kWinParts; ++x) {
                 const int xx = tid + 256 * x;
-                if (xx < win) s_in[ch * win + xx] = stage_in[ch][x];
+                if (xx < win) s_in[ch * win + xx] = (row_exists && in_pos[x] >= 0) ? stage_in[ch][x] : 0.0f;
             }
+        }
     };
 
     floatx16 acc0, acc1;
@@ -236,7 +237,7 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
     const int half = lane >> 5, col = lane & 31;
     fetch(0);
     for (int i0 = 0; i0 < a.in_ch; i0 += kConvChannels) {
-        publish();
+        publish(i0);
         __syncthreads();
         if (i0 + kConvChannels < a.in_ch) fetch(i0 + kConvChannels);   // in flight during the products below
         conv_products<KF>(s_w + (wm * 32 + col) * a_stride + half * a.kernel, s_in + half * win + wn * 64 + col, a.kernel, a.dilation,
@@ -341,103 +342,82 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
 
 // The same product for short rows (few positions, many channels: the codec's first stages), where 64 x 128 tiles would
 // leave most of the chip idle: a workgroup owns a 32 x 64 tile and its four wavefronts split the input channels between
-// them (wavefront w takes channel blocks w, w + 4, ...), each staging its own blocks in its own part of LDS; the four
-// partial tiles are added in wavefront order at the end, so the result does not depend on timing.  NT: 32-position
-// halves per tile (2, or 1 for the very shortest rows: twice the workgroups).
+// them (wavefront w takes channel blocks w, w + 4, ...: one weight chunk each), each staging its own blocks in its own
+// part of LDS; the four partial tiles are added in wavefront order at the end, so the result does not depend on timing.
+// NT: 32-position halves per tile (2, or 1 for the very shortest rows: twice the workgroups).
 template <int KF, int NT>
-__global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg, float *const out_arg, const float *const w_arg, const float *const bias_arg, const int in_ch_arg,
-                                                const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const ConvArgs a_arg) {
+__global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg, float *const out_arg, const float *const chunks_arg, const float *const bias_arg, const int in_ch_arg,
+                                                      const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const int tiles_arg,
+                                                      const ConvArgs a_arg) {
     constexpr int TM = 32, TN = 32 * NT;
     extern __shared__ __align__(16) float lds[];
     // (the rows, the weights and the shape lead the arguments and repeat fields of a_arg: leading scalar arguments are in
     // registers when a wavefront starts, a structure passed by value is fetched from memory where its fields are first used)
     ConvArgs a = a_arg;
-    a.in = in_arg; a.out = out_arg; a.w = w_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
+    a.in = in_arg; a.out = out_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
     a.kernel = kernel_arg; a.dilation = dilation_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;
-    const int a_stride = kb + 4;   // rows stay 16-byte aligned and get four floats of padding: a stride of 4 mod 8 words spreads the
-                                   // 32 rows a wavefront reads for a product over eight banks instead of four
+    const int a_stride = kb + 4;   // the chunks' row stride (see k_conv1d)
     const int halo = (a.kernel - 1) * a.dilation;
     const int win = TN + halo;
-    const int per_wave = TM * a_stride + kConvChannels * win;
+    // a chunk is 8 * a_stride 16-byte pieces; a lane's slots (one piece each) cover it, the last one possibly reaching past
+    // it (into the next chunk or the zeros after the last one: LDS the products never read)
+    constexpr int kSlots = (8 * (kConvChannels * (KF != 0 ? KF : kConvMaxKernel) + 4) + 63) / 64;
+    const int slots = KF != 0 ? kSlots : (8 * a_stride + 63) / 64;
+    const int per_wave = slots * 256 + kConvChannels * win;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    float *s_w = lds + wave * per_wave;        // [TM][a_stride] of this wavefront
-    float *s_in = s_w + TM * a_stride;         // [kConvChannels][win]
+    float *s_w = lds + wave * per_wave;        // [TM][a_stride] of this wavefront, then the last slot's excess
+    float *s_in = s_w + slots * 256;           // [kConvChannels][win]
     const int m0 = blockIdx.y * TM, t0 = blockIdx.x * TN;
-    const int inner = a.in_ch * a.kernel;
-    // staging slots of a lane: weights -- the four elements 4 * (lane + 64 * c) .. + 3 of the 32 x kb block taken row by
-    // row (rows are whole 16-byte pieces: the launch requires in_ch * kernel to be a multiple of 4, and kb is 8 * kernel);
-    // input rows -- channel ch, position lane + 64 * x
-    constexpr int kCols = kConvChannels * (KF != 0 ? KF : kConvMaxKernel) / 8, kWinParts = (TN + kConvMaxHalo + 63) / 64;
-    const int kb4 = kb / 4;
+    constexpr int kWinParts = (TN + kConvMaxHalo + 63) / 64;
 
     floatx16 acc0, acc1;
 #pragma unroll
     for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
     const int half = lane >> 5, col = lane & 31;
     const int blocks = (a.in_ch + kConvChannels - 1) / kConvChannels;
-    const int rounds = (blocks + 3) / 4;   // the same count for every wavefront (a block past the end stages zeros)
-    float4 stage_w[kCols];
+    const int rounds = (blocks + 3) / 4;   // the same count for every wavefront (a block past the end is a chunk of zeros)
+    floatx4 stage_w[kSlots];
     float stage_in[kConvChannels][kWinParts];
-    // What a staging slot of this lane is does not change from round to round: kept as one 32-bit offset per slot (-1:
-    // outside the matrix or the row), so that a round's requests are an add, a load and a select each.  Working them out
-    // anew every round (a division, the range checks, 64-bit addresses) took 2.0 of a round's 5.0 us on the 432-channel
-    // stage: with one wavefront per SIMD the requests are bound by the instructions that form them, not by their round trip.
-    int w_slot[kCols];        // weights: offset of the slot's four floats from the block's first column
-    int in_slot[kWinParts];   // input: position in the row
-#pragma unroll
-    for (int c = 0; c < kCols; ++c) {
-        const int e = lane + 64 * c, row = e / kb4, cc = 4 * (e - row * kb4);   // kb is a constant in the builds that matter
-        const int m = m0 + row;
-        w_slot[c] = (row < TM && m < a.out_ch) ? m * inner + cc : -1;   // offsets fit 31 bits (checked at launch)
-    }
+    int in_pos[kWinParts];    // input: position in the row, the same in every round (-1: outside the row or the window)
 #pragma unroll
     for (int x = 0; x < kWinParts; ++x) {
         const int xx = lane + 64 * x, t = t0 - halo + xx;
-        in_slot[x] = (xx < win && t >= 0 && t < a.length) ? t : -1;
+        in_pos[x] = (xx < win && t >= 0 && t < a.length) ? t : -1;
     }
-    const auto fetch = [&](int round) {   // global -> registers: this wavefront's channel block of the round
+    // this lane's first piece of the wavefront's first chunk; four blocks on from round to round
+    const floatx4 *w_next = reinterpret_cast<const floatx4 *>(chunks_arg) + ((size_t)wave * tiles_arg + blockIdx.y) * (8 * a_stride) + lane;
+    const size_t w_step = (size_t)4 * tiles_arg * (8 * a_stride);
+    const auto fetch = [&](int round) {   // global -> registers: this wavefront's channel block of the round; nothing waits here
         const int i0 = (4 * round + wave) * kConvChannels;
-        const int ci0 = i0 * a.kernel;
-        const bool whole_block = ci0 + kb <= inner;   // all but a ragged last block
 #pragma unroll
-        for (int c = 0; c < kCols; ++c) {
-            bool valid = w_slot[c] >= 0;
-            if (!whole_block) {
-                const int e = lane + 64 * c;
-                valid = valid && ci0 + 4 * (e - (e / kb4) * kb4) < inner;
-            }
-            const float4 v = *reinterpret_cast<const float4 *>(a.w + (valid ? w_slot[c] + ci0 : 0));
-            stage_w[c] = valid ? v : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+        for (int c = 0; c < kSlots; ++c)
+            if (KF != 0 || c < slots) stage_w[c] = w_next[64 * c];
+        w_next += w_step;
 #pragma unroll
         for (int ch = 0; ch < kConvChannels; ++ch) {
-            const int i = i0 + ch;
-            const bool row_exists = i < a.in_ch;
-            const int row_at = i * a.length;
+            const bool row_exists = i0 + ch < a.in_ch;
+            const float *row = a.in + (row_exists ? (size_t)(i0 + ch) * a.length : 0);
 #pragma unroll
-            for (int x = 0; x < kWinParts; ++x) {
-                const bool valid = row_exists && in_slot[x] >= 0;
-                const float v = a.in[valid ? row_at + in_slot[x] : 0];
-                stage_in[ch][x] = valid ? v : 0.0f;
-            }
+            for (int x = 0; x < kWinParts; ++x) stage_in[ch][x] = row[in_pos[x] >= 0 ? in_pos[x] : 0];   // always a legal address
         }
     };
     fetch(0);
     for (int round = 0; round < rounds; ++round) {
+        const int i0 = (4 * round + wave) * kConvChannels;
 #pragma unroll
-        for (int c = 0; c < kCols; ++c) {
-            const int e = lane + 64 * c, row = e / kb4, c4 = e - row * kb4;
-            if (e < TM * kb4) reinterpret_cast<float4 *>(s_w + row * a_stride)[c4] = stage_w[c];
-        }
+        for (int c = 0; c < kSlots; ++c)
+            if (KF != 0 || c < slots) reinterpret_cast<floatx4 *>(s_w)[lane + 64 * c] = stage_w[c];
 #pragma unroll
-        for (int ch = 0; ch < kConvChannels; ++ch)
+        for (int ch = 0; ch < kConvChannels; ++ch) {
+            const bool row_exists = i0 + ch < a.in_ch;
 #pragma unroll
             for (int x = 0; x < kWinParts; ++x) {
                 const int xx = lane + 64 * x;
-                if (xx < win) s_in[ch * win + xx] = stage_in[ch][x];
+                if (xx < win) s_in[ch * win + xx] = (row_exists && in_pos[x] >= 0) ? stage_in[ch][x] : 0.0f;
             }
+        }
         // (no workgroup barrier in the loop: a wavefront stages into its own part of LDS and reads nothing else, and its own
         // LDS accesses complete in the order it issued them -- the four wavefronts walk their channel blocks independently)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -534,50 +514,45 @@ __global__ void __launch_bounds__(256) k_snake(const float *in, float *out, cons
     out[index] = half_snake(v, snake_row, al, 1.0f / (al + 1e-9f));
 }
 
-template <int WM, int WN, int KF, int VEC, bool FUSED>
-int launch_conv_f(State *st, const ConvArgs &a, char *error, size_t capacity) {
+template <int WM, int WN, int KF, bool FUSED>
+int launch_conv_f(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
-    const int kb = kConvChannels * a.kernel;
-    // two more staged rows than are filled: the product loop requests the operands after its last product before it stops
-    size_t lds = ((size_t)TM * (VEC ? kb + 4 : (kb | 1)) + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
+    const int slots = (WM * 8 * (kConvChannels * a.kernel + 4) + 255) / 256;
+    // two more staged rows than are filled: the product loop requests the operands of two products past its last one
+    size_t lds = ((size_t)slots * 1024 + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
     if (lds < (4 * 32 * kTileStride + 4 * 64) * sizeof(float)) lds = (4 * 32 * kTileStride + 4 * 64) * sizeof(float);   // the fused epilogue's tiles and alphas
     static bool raised = false;   // per instantiation
     if (lds > 48 * 1024 && !raised) {
-        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF, VEC, FUSED>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d<WM, WN, KF, FUSED>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
         raised = true;
     }
     const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM));
-    hipLaunchKernelGGL((k_conv1d<WM, WN, KF, VEC, FUSED>), grid, dim3(256), lds, st->stream, a.in, a.out, a.w, a.bias, a.in_ch, a.out_ch, a.length, a.kernel, a.dilation, a);
+    hipLaunchKernelGGL((k_conv1d<WM, WN, KF, FUSED>), grid, dim3(256), lds, st->stream, a.in, a.out, chunks.data, a.bias, a.in_ch, a.out_ch, a.length, a.kernel, a.dilation,
+                       chunks.tiles, a);
     return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
 }
 
-template <int WM, int WN, int KF, int VEC>
-int launch_conv_v(State *st, const ConvArgs &a, char *error, size_t capacity) {
-    if (a.residual != nullptr || a.residual2 != nullptr || a.scaled || a.activate) return launch_conv_f<WM, WN, KF, VEC, true>(st, a, error, capacity);
-    return launch_conv_f<WM, WN, KF, VEC, false>(st, a, error, capacity);
-}
-
 template <int WM, int WN, int KF>
-int launch_conv_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
-    if (((size_t)a.in_ch * a.kernel) % 4 == 0) return launch_conv_v<WM, WN, KF, 1>(st, a, error, capacity);
-    return launch_conv_v<WM, WN, KF, 0>(st, a, error, capacity);
+int launch_conv_k(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
+    if (a.residual != nullptr || a.residual2 != nullptr || a.scaled || a.activate) return launch_conv_f<WM, WN, KF, true>(st, a, chunks, error, capacity);
+    return launch_conv_f<WM, WN, KF, false>(st, a, chunks, error, capacity);
 }
 
 template <int WM, int WN>
-int launch_conv(State *st, const ConvArgs &a, char *error, size_t capacity) {
+int launch_conv(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
     switch (a.kernel) {
-        case 3: return launch_conv_k<WM, WN, 3>(st, a, error, capacity);
-        case 7: return launch_conv_k<WM, WN, 7>(st, a, error, capacity);
-        case 11: return launch_conv_k<WM, WN, 11>(st, a, error, capacity);
-        default: return launch_conv_k<WM, WN, 0>(st, a, error, capacity);
+        case 3: return launch_conv_k<WM, WN, 3>(st, a, chunks, error, capacity);
+        case 7: return launch_conv_k<WM, WN, 7>(st, a, chunks, error, capacity);
+        case 11: return launch_conv_k<WM, WN, 11>(st, a, chunks, error, capacity);
+        default: return launch_conv_k<WM, WN, 0>(st, a, chunks, error, capacity);
     }
 }
 
 template <int KF, int NT>
-int launch_conv_split_k(State *st, const ConvArgs &a, char *error, size_t capacity) {
-    const int kb = kConvChannels * a.kernel;
-    const size_t per_wave = (size_t)32 * (kb + 4) + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
-    size_t lds = (4 * per_wave + 2 * (32 * NT + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);   // see launch_conv about the two extra rows
+int launch_conv_split_k(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
+    const int slots = (8 * (kConvChannels * a.kernel + 4) + 63) / 64;
+    const size_t per_wave = (size_t)slots * 256 + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
+    size_t lds = (4 * per_wave + 2 * (32 * NT + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);   // see launch_conv_f about the two extra rows
     if (lds < (4 * 32 * 64 + 64) * sizeof(float)) lds = (4 * 32 * 64 + 64) * sizeof(float);   // the partial tiles, and the rows' alphas behind them
     static bool raised = false;
     if (!raised) {
@@ -585,24 +560,25 @@ int launch_conv_split_k(State *st, const ConvArgs &a, char *error, size_t capaci
         raised = true;
     }
     const dim3 grid((unsigned)((a.length + 32 * NT - 1) / (32 * NT)), (unsigned)((a.out_ch + 31) / 32));
-    hipLaunchKernelGGL((k_conv1d_split<KF, NT>), grid, dim3(256), lds, st->stream, a.in, a.out, a.w, a.bias, a.in_ch, a.out_ch, a.length, a.kernel, a.dilation, a);
+    hipLaunchKernelGGL((k_conv1d_split<KF, NT>), grid, dim3(256), lds, st->stream, a.in, a.out, chunks.data, a.bias, a.in_ch, a.out_ch, a.length, a.kernel, a.dilation,
+                       chunks.tiles, a);
     return hip_check(hipGetLastError(), "conv1d launch", error, capacity);
 }
 
 template <int NT>
-int launch_conv_split_n(State *st, const ConvArgs &a, char *error, size_t capacity) {
+int launch_conv_split_n(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
     switch (a.kernel) {
-        case 3: return launch_conv_split_k<3, NT>(st, a, error, capacity);
-        case 7: return launch_conv_split_k<7, NT>(st, a, error, capacity);
-        case 11: return launch_conv_split_k<11, NT>(st, a, error, capacity);
-        default: return launch_conv_split_k<0, NT>(st, a, error, capacity);
+        case 3: return launch_conv_split_k<3, NT>(st, a, chunks, error, capacity);
+        case 7: return launch_conv_split_k<7, NT>(st, a, chunks, error, capacity);
+        case 11: return launch_conv_split_k<11, NT>(st, a, chunks, error, capacity);
+        default: return launch_conv_split_k<0, NT>(st, a, chunks, error, capacity);
     }
 }
 
-int launch_conv_split(State *st, const ConvArgs &a, char *error, size_t capacity) {
+int launch_conv_split(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
     const long tiles = (long)((a.out_ch + 31) / 32) * ((a.length + 63) / 64);
-    if (tiles < st->cu_count) return launch_conv_split_n<1>(st, a, error, capacity);
-    return launch_conv_split_n<2>(st, a, error, capacity);
+    if (tiles < st->cu_count) return launch_conv_split_n<1>(st, a, chunks, error, capacity);
+    return launch_conv_split_n<2>(st, a, chunks, error, capacity);
 }
 
 }  // namespace
@@ -621,15 +597,11 @@ static int conv1d_entry(void *state, const float *dev_input, float *dev_output, 
         set_error(error, capacity, "conv1d: kernel above 16 taps, reach above 128 positions or tensor too large");
         return -1;
     }
-    const CachedWeight *cw = nullptr;
-    if (cached_matrix(st, weight, (size_t)out_channels, (size_t)in_channels * kernel, MYNAH_HIP_F32, &cw, error, capacity) != 0) return -1;
-    if (cw->qtype != MYNAH_HIP_F32) {
-        set_error(error, capacity, "conv1d: weight could not be kept as f32");
-        return -1;
-    }
+    ConvBlocks chunks;
+    if (cached_conv_blocks(st, weight, (size_t)out_channels, (size_t)in_channels, (size_t)kernel, &chunks, error, capacity) != 0) return -1;
     const float *dev_bias = nullptr;
     if (cached_vector(st, bias, (size_t)out_channels, &dev_bias, error, capacity) != 0) return -1;
-    ConvArgs a{dev_input, dev_output, static_cast<const float *>(cw->data), dev_bias, in_channels, out_channels, length, kernel, dilation};
+    ConvArgs a{dev_input, dev_output, dev_bias, in_channels, out_channels, length, kernel, dilation};
     if (extra != nullptr) {
         if (extra->snake_channels > (size_t)out_channels || (extra->snake_channels != 0 && extra->snake_alpha == nullptr) ||
             (extra->dev_activated != nullptr && !extra->activate) || extra->dev_activated == dev_output || dev_input == dev_output ||
@@ -650,11 +622,9 @@ static int conv1d_entry(void *state, const float *dev_input, float *dev_output, 
     // few output channels: one row of wavefronts, wider in time; too few large tiles to fill the chip (and enough input
     // channels to share out): small tiles with the channels split over the wavefronts
     const long tiles = out_channels <= 32 ? (long)((length + 255) / 256) : (long)((out_channels + 63) / 64) * ((length + 127) / 128);
-    if (tiles < st->cu_count && in_channels >= 4 * kConvChannels && ((size_t)in_channels * kernel) % 4 == 0 &&
-        (size_t)out_channels * in_channels * kernel < (size_t)INT_MAX && (size_t)in_channels * length < (size_t)INT_MAX)
-        return launch_conv_split(st, a, error, capacity);
-    if (out_channels <= 32) return launch_conv<1, 4>(st, a, error, capacity);
-    return launch_conv<2, 2>(st, a, error, capacity);
+    if (tiles < st->cu_count && in_channels >= 4 * kConvChannels) return launch_conv_split(st, a, chunks, error, capacity);
+    if (out_channels <= 32) return launch_conv<1, 4>(st, a, chunks, error, capacity);
+    return launch_conv<2, 2>(st, a, chunks, error, capacity);
 }
 
 extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,

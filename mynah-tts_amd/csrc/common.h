@@ -78,7 +78,7 @@ struct PackedWeight {
 struct WeightKey {
     const void *host;
     size_t bytes;
-    int kind;   // 0 plain f32 vector/matrix, 1 + qtype*2 + arith for converted matrices
+    int kind;   // 0 plain f32 vector/matrix, 1 + qtype*2 + arith for converted matrices, 64 + kernel + 32 * in_ch for conv1d chunks
     bool operator==(const WeightKey &o) const { return host == o.host && bytes == o.bytes && kind == o.kind; }
 };
 struct WeightKeyHash {
@@ -222,6 +222,19 @@ State *enter_state(void *opaque, bool enqueues = true);
 int cached_matrix(State *st, const float *host, size_t n, size_t k, int want_qtype, const CachedWeight **out,
                   char *error, size_t capacity);
 int cached_vector(State *st, const float *host, size_t n, const float **dev, char *error, size_t capacity);
+// A conv1d weight [out_ch, in_ch, kernel] in the form the convolution kernels stage it (codec_ops.hip): cut into chunks of
+// 32 output channels x 8 input channels, each chunk 32 rows of 8 * kernel + 4 floats (a row holds the taps of its eight
+// channels one after the other, then four floats of padding: the row stride the kernels keep in LDS), zeros where the
+// tensor has no row or channel.  Chunk (block b of input channels, tile t of output channels) starts at float
+// (b * tiles + t) * conv_chunk_floats(kernel); `tiles` is even and `blocks` a multiple of four (whole chunks of zeros
+// past the tensor), and four kilobytes of zeros follow the last chunk, so a kernel copies whole chunks without a bounds check.
+struct ConvBlocks {
+    const float *data = nullptr;
+    int tiles = 0, blocks = 0;
+};
+constexpr int kConvChannels = 8;      // input channels per chunk: the convolution kernels' step along the inner dimension
+inline size_t conv_chunk_floats(size_t kernel) { return 32u * (kConvChannels * kernel + 4u); }
+int cached_conv_blocks(State *st, const float *host, size_t out_ch, size_t in_ch, size_t kernel, ConvBlocks *out, char *error, size_t capacity);
 int ensure_attention_workspace(State *st, size_t batch, size_t heads, size_t head_width, size_t max_valid,
                                char *error, size_t capacity, size_t chunk_rows = kAttnChunk);
 int ensure_pinned(State *st, size_t bytes, char *error, size_t capacity);
