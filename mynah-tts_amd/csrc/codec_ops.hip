@@ -184,8 +184,9 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
     constexpr int kSlots = (WM * 8 * (kConvChannels * (KF != 0 ? KF : kConvMaxKernel) + 4) + 255) / 256;
     const int pieces = WM * 8 * a_stride;
     const int slots = KF != 0 ? kSlots : (pieces + 255) / 256;
-    float *s_w = lds;                          // [TM][a_stride], then the last slot's excess
-    float *s_in = lds + slots * 1024;          // [kConvChannels][win]
+    // (the input rows first: their LDS addresses are then the staged positions themselves, with nothing to add per request)
+    float *s_in = lds;                         // [kConvChannels][win]
+    float *s_w = lds + kConvChannels * win;    // [TM][a_stride], then the last slot's excess; 16-byte aligned
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int m0 = blockIdx.y * TM, t0 = blockIdx.x * TN;
@@ -367,8 +368,8 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg,
     const int slots = KF != 0 ? kSlots : (8 * a_stride + 63) / 64;
     const int per_wave = slots * 256 + kConvChannels * win;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    float *s_w = lds + wave * per_wave;        // [TM][a_stride] of this wavefront, then the last slot's excess
-    float *s_in = s_w + slots * 256;           // [kConvChannels][win]
+    float *s_in = lds + wave * per_wave;       // [kConvChannels][win] of this wavefront
+    float *s_w = s_in + kConvChannels * win;   // [TM][a_stride], then the last slot's excess; 16-byte aligned
     const int m0 = blockIdx.y * TM, t0 = blockIdx.x * TN;
     constexpr int kWinParts = (TN + kConvMaxHalo + 63) / 64;
 
