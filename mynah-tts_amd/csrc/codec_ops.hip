@@ -232,10 +232,16 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
         }
     };
 
+    // The accumulators start from the rows' biases (requested here, beside the first block: at the end each would be a
+    // round trip of its own in front of the stores), so a value is bias + products in the products' order.
+    const int half = lane >> 5, col = lane & 31;
     floatx16 acc0, acc1;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
-    const int half = lane >> 5, col = lane & 31;
+    for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+        acc0[r] = (a.bias != nullptr && m < a.out_ch) ? a.bias[m] : 0.0f;
+    }
+    acc1 = acc0;
     fetch(0);
     for (int i0 = 0; i0 < a.in_ch; i0 += kConvChannels) {
         publish(i0);
@@ -256,8 +262,7 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
             const int t = t0 + wn * 64 + col;
             const bool in0 = m < a.out_ch && t < a.length, in1 = m < a.out_ch && t + 32 < a.length;
             const size_t i0 = in0 ? (size_t)m * a.length + t : 0, i1 = in1 ? (size_t)m * a.length + t + 32 : 0;
-            const float b = (a.bias != nullptr && m < a.out_ch) ? a.bias[m] : 0.0f;
-            float v0 = acc0[r] + b, v1 = acc1[r] + b;
+            float v0 = acc0[r], v1 = acc1[r];
             if constexpr (decltype(has_first)::value) { v0 = a.residual[i0] + v0; v1 = a.residual[i1] + v1; }
             if constexpr (decltype(has_second)::value) { v0 = a.residual2[i0] + v0; v1 = a.residual2[i1] + v1; }
             if constexpr (FUSED) {
