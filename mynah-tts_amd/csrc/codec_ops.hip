@@ -110,9 +110,11 @@ __device__ __forceinline__ void conv_emit(const ConvArgs &a, int m, size_t index
 // around every product: left to itself the compiler reads a product's input operand into one and the same register right
 // before it, and with one wavefront on a SIMD every product then waits out an LDS read (some 120 cycles against the 64
 // of the instruction itself).  Past the last product the requests stay inside the staging area and are not used.
+// pairs: channel pairs of the block that exist (the tensor's last block may hold fewer than four; the rest is zeros in
+// both operands and is left out -- the same for every lane of the wavefront).
 template <int KF, int NT = 2>
 __device__ __forceinline__ void conv_products(const float *wrow, const float *irow, const int kernel_arg, const int dilation, const int win,
-                                              floatx16 &acc0, floatx16 &acc1) {
+                                              floatx16 &acc0, floatx16 &acc1, const int pairs = kConvChannels / 2) {
     if constexpr (KF != 0) {
         constexpr int kSteps = (kConvChannels / 2) * KF;
         float wv[3], x0[3], x1[3];
@@ -130,6 +132,7 @@ __device__ __forceinline__ void conv_products(const float *wrow, const float *ir
         request(1);
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
+            if (s % KF == 0 && s != 0 && s / KF >= pairs) break;   // (looked at where a pair begins)
             request((s + 2) % 3);
             __builtin_amdgcn_sched_barrier(0x77);
             acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[s % 3], x0[s % 3], acc0, 0, 0, 0);
@@ -248,7 +251,7 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
         __syncthreads();
         if (i0 + kConvChannels < a.in_ch) fetch(i0 + kConvChannels);   // in flight during the products below
         conv_products<KF>(s_w + (wm * 32 + col) * a_stride + half * a.kernel, s_in + half * win + wn * 64 + col, a.kernel, a.dilation,
-                          win, acc0, acc1);
+                          win, acc0, acc1, min(kConvChannels / 2, (a.in_ch - i0 + 1) / 2));
         __syncthreads();
     }
     // accumulator element r of a lane: row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
