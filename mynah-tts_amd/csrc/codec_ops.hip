@@ -245,11 +245,29 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
         acc0[r] = (a.bias != nullptr && m < a.out_ch) ? a.bias[m] : 0.0f;
     }
     acc1 = acc0;
+    // The fused build's residual values are requested before the last block's products instead of behind them (a round
+    // trip in front of the stores otherwise); a residual may be the output itself -- every workgroup reads and writes its
+    // own tile only.
+    float res_first[FUSED ? 32 : 1], res_second[FUSED ? 32 : 1];
+    const auto request_residuals = [&]() {
+        if constexpr (FUSED) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const int t = t0 + wn * 64 + col;
+                const bool in0 = m < a.out_ch && t < a.length, in1 = m < a.out_ch && t + 32 < a.length;
+                const size_t i0 = in0 ? (size_t)m * a.length + t : 0, i1 = in1 ? (size_t)m * a.length + t + 32 : 0;
+                if (a.residual != nullptr) { res_first[r] = a.residual[i0]; res_first[16 + r] = a.residual[i1]; }
+                if (a.residual2 != nullptr) { res_second[r] = a.residual2[i0]; res_second[16 + r] = a.residual2[i1]; }
+            }
+        }
+    };
     fetch(0);
     for (int i0 = 0; i0 < a.in_ch; i0 += kConvChannels) {
         publish(i0);
         __syncthreads();
         if (i0 + kConvChannels < a.in_ch) fetch(i0 + kConvChannels);   // in flight during the products below
+        else request_residuals();
         conv_products<KF>(s_w + (wm * 32 + col) * a_stride + half * a.kernel, s_in + half * win + wn * 64 + col, a.kernel, a.dilation,
                           win, acc0, acc1, min(kConvChannels / 2, (a.in_ch - i0 + 1) / 2));
         __syncthreads();
@@ -266,8 +284,8 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
             const bool in0 = m < a.out_ch && t < a.length, in1 = m < a.out_ch && t + 32 < a.length;
             const size_t i0 = in0 ? (size_t)m * a.length + t : 0, i1 = in1 ? (size_t)m * a.length + t + 32 : 0;
             float v0 = acc0[r], v1 = acc1[r];
-            if constexpr (decltype(has_first)::value) { v0 = a.residual[i0] + v0; v1 = a.residual[i1] + v1; }
-            if constexpr (decltype(has_second)::value) { v0 = a.residual2[i0] + v0; v1 = a.residual2[i1] + v1; }
+            if constexpr (decltype(has_first)::value) { v0 = res_first[r] + v0; v1 = res_first[16 + r] + v1; }
+            if constexpr (decltype(has_second)::value) { v0 = res_second[r] + v0; v1 = res_second[16 + r] + v1; }
             if constexpr (FUSED) {
                 v0 = v0 * a.scale;   // 1.0f when there is no scaling: the value's own bits
                 v1 = v1 * a.scale;
