@@ -273,16 +273,32 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
         __syncthreads();
     }
     // accumulator element r of a lane: row 8 * (r / 4) + 4 * (lane / 32) + r % 4, column lane % 32
-    // conv + bias, then the residuals and the scale (conv_combine's order), without a branch per value: requests go to a
-    // legal address whatever the value's place (element 0 when it lies outside the rows), side by side, and a request
-    // that is not wanted at all is left out by the build of this loop that runs.
+    // conv + bias, then the residuals (requested before the last products, to a legal address whatever the value's place)
+    // and the scale, in conv_combine's order, without a branch per value: an addition that is not wanted at all is left out
+    // by the build of this loop that runs.
+    // A finished tile on its way to memory: from the accumulators' layout (a store instruction there covers 32 positions of
+    // two rows, and a row's validity differs between the halves of a wavefront: a mask and a branch per store) through the
+    // wavefront's own piece of LDS (free after the last products' barrier) to whole rows of 64 consecutive positions, whose
+    // validity is the same for every lane -- a loop over the rows that exist, the positions' own check once around it.
+    const auto store_tile = [&](float *dst, const floatx16 &first, const floatx16 &second) {
+        float *s_tile = lds + wave * (32 * kTileStride);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 8 * (r >> 2) + 4 * half + (r & 3);
+            s_tile[row * kTileStride + col] = first[r];
+            s_tile[row * kTileStride + col + 32] = second[r];
+        }
+        const int t = t0 + wn * 64 + lane;
+        const int rows = min(32, a.out_ch - (m0 + wm * 32));   // the same for the whole wavefront
+        if (t < a.length) {
+            float *p = dst + (size_t)(m0 + wm * 32) * a.length + t;
+#pragma unroll 8
+            for (int row = 0; row < rows; ++row, p += a.length) *p = s_tile[row * kTileStride + lane];
+        }
+    };
     const auto combine = [&](auto has_first, auto has_second) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-            const int t = t0 + wn * 64 + col;
-            const bool in0 = m < a.out_ch && t < a.length, in1 = m < a.out_ch && t + 32 < a.length;
-            const size_t i0 = in0 ? (size_t)m * a.length + t : 0, i1 = in1 ? (size_t)m * a.length + t + 32 : 0;
             float v0 = acc0[r], v1 = acc1[r];
             if constexpr (decltype(has_first)::value) { v0 = res_first[r] + v0; v1 = res_first[16 + r] + v1; }
             if constexpr (decltype(has_second)::value) { v0 = res_second[r] + v0; v1 = res_second[16 + r] + v1; }
@@ -292,11 +308,8 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
             }
             acc0[r] = v0;
             acc1[r] = v1;
-            if (!FUSED || !a.activate) {
-                if (in0) a.out[i0] = v0;
-                if (in1) a.out[i1] = v1;
-            }
         }
+        if (!FUSED || !a.activate) store_tile(a.out, acc0, acc1);
     };
     if constexpr (!FUSED) {   // the seam's conv1d
         combine(std::false_type{}, std::false_type{});
@@ -323,30 +336,23 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
         large = large || !(fabsf(al * acc0[r]) < kShortSineLimit) || !(fabsf(al * acc1[r]) < kShortSineLimit);
     }
     if (!__any(large)) {
-        const auto finish = [&](auto has_copy) {
+        floatx16 act0, act1;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = 8 * (r >> 2) + 4 * half + (r & 3), m = m0 + wm * 32 + row;
-                const int t = t0 + wn * 64 + col;
-                const bool in0 = m < a.out_ch && t < a.length, in1 = m < a.out_ch && t + 32 < a.length;
-                const size_t i0 = (size_t)m * a.length + t, i1 = i0 + 32;
-                const float al = s_alpha[row], inv_a = s_alpha[32 + row];
-                const float v0 = acc0[r], v1 = acc1[r];
-                const float s0 = short_sine(al * v0), s1 = short_sine(al * v1);
-                const bool snake_row = m < a.snake_channels;
-                const float y0 = snake_row ? v0 + s0 * s0 * inv_a : (v0 < 0.0f ? v0 * 0.01f : v0);
-                const float y1 = snake_row ? v1 + s1 * s1 * inv_a : (v1 < 0.0f ? v1 * 0.01f : v1);
-                if constexpr (decltype(has_copy)::value) {
-                    if (in0) { a.out[i0] = v0; a.act_out[i0] = y0; }
-                    if (in1) { a.out[i1] = v1; a.act_out[i1] = y1; }
-                } else {
-                    if (in0) a.out[i0] = y0;
-                    if (in1) a.out[i1] = y1;
-                }
-            }
-        };
-        if (a.act_out != nullptr) finish(std::true_type{});
-        else finish(std::false_type{});
+        for (int r = 0; r < 16; ++r) {
+            const int row = 8 * (r >> 2) + 4 * half + (r & 3), m = m0 + wm * 32 + row;
+            const float al = s_alpha[row], inv_a = s_alpha[32 + row];
+            const float v0 = acc0[r], v1 = acc1[r];
+            const float s0 = short_sine(al * v0), s1 = short_sine(al * v1);
+            const bool snake_row = m < a.snake_channels;
+            act0[r] = snake_row ? v0 + s0 * s0 * inv_a : (v0 < 0.0f ? v0 * 0.01f : v0);
+            act1[r] = snake_row ? v1 + s1 * s1 * inv_a : (v1 < 0.0f ? v1 * 0.01f : v1);
+        }
+        if (a.act_out != nullptr) {
+            store_tile(a.out, acc0, acc1);
+            store_tile(a.act_out, act0, act1);
+        } else {
+            store_tile(a.out, act0, act1);
+        }
         return;
     }
     // Some argument needs the library's sine: the wavefront's 32 x 64 tile goes through LDS and a rolled loop finishes it
@@ -461,26 +467,26 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg,
         s_part[(wave * 32 + 16 + r) * 64 + lane] = acc1[r];
     }
     __syncthreads();
+    // A thread finishes the tile's values at (row (tid / 64) + 4 j, position tid % 64): a store instruction then covers one
+    // row's 64 consecutive positions and whether the row exists is the same for all its lanes (in the accumulators' order an
+    // instruction covers halves of two rows, four apart).  e: where that value sits in a partial tile (element r of lane l).
+    const int pos = tid & 63;
+    const int t = t0 + pos;
+    const bool t_ok = (NT > 1 || pos < 32) && t < a.length;
     float value[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        const int e = tid + 256 * j;       // element r of lane l of the tile: e = r * 64 + l
-        const int r = e >> 6, l = e & 63;
+        const int row = (tid >> 6) + 4 * j, m = m0 + row;
+        const int e = ((((row >> 3) << 2) | (row & 3)) + 16 * (pos >> 5)) * 64 + ((row >> 2) & 1) * 32 + (pos & 31);
         const float sum = ((s_part[e] + s_part[2048 + e]) + s_part[4096 + e]) + s_part[6144 + e];
-        const int rr = r & 15;
-        const int m = m0 + 8 * (rr >> 2) + 4 * (l >> 5) + (rr & 3);
-        const int t = t0 + (l & 31) + (r >= 16 ? 32 : 0);
         value[j] = 0.0f;
-        if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length)
-            value[j] = conv_combine(a, (size_t)m * a.length + t, sum + (a.bias != nullptr ? a.bias[m] : 0.0f));
+        if (t_ok && m < a.out_ch) value[j] = conv_combine(a, (size_t)m * a.length + t, sum + (a.bias != nullptr ? a.bias[m] : 0.0f));
     }
     if (!a.activate) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int e = tid + 256 * j, r = e >> 6, l = e & 63, rr = r & 15;
-            const int m = m0 + 8 * (rr >> 2) + 4 * (l >> 5) + (rr & 3);
-            const int t = t0 + (l & 31) + (r >= 16 ? 32 : 0);
-            if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length) a.out[(size_t)m * a.length + t] = value[j];
+            const int m = m0 + (tid >> 6) + 4 * j;
+            if (t_ok && m < a.out_ch) a.out[(size_t)m * a.length + t] = value[j];
         }
         return;
     }
@@ -497,10 +503,8 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg,
     for (int j = 0; j < 8; ++j) s_part[tid + 256 * j] = value[j];
 #pragma unroll 2
     for (int j = 0; j < 8; ++j) {
-        const int e = tid + 256 * j, r = e >> 6, l = e & 63, rr = r & 15;
-        const int row = 8 * (rr >> 2) + 4 * (l >> 5) + (rr & 3), m = m0 + row;
-        const int t = t0 + (l & 31) + (r >= 16 ? 32 : 0);
-        if ((NT > 1 || r < 16) && m < a.out_ch && t < a.length) conv_emit(a, m, (size_t)m * a.length + t, s_part[e], s_alpha[row], s_alpha[32 + row]);
+        const int row = (tid >> 6) + 4 * j, m = m0 + row;
+        if (t_ok && m < a.out_ch) conv_emit(a, m, (size_t)m * a.length + t, s_part[tid + 256 * j], s_alpha[row], s_alpha[32 + row]);
     }
 }
 
