@@ -210,15 +210,17 @@ def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
     flops += 2.0 * C * 3 * L
     latent = backend.alloc(32 * frames).write(rng.uniform(-1, 1, 32 * frames).astype(np.float32))
     biggest = max((864 >> (i + 1)) * frames * int(np.prod(rates[:i + 1])) for i in range(5))
-    bufs = [backend.alloc(max(biggest, 864 * frames)) for _ in range(7)]
-    cur, up, out, act, res, br, work = bufs
+    bufs = [backend.alloc(max(biggest, 864 * frames)) for _ in range(13)]
+    cur, up, out, act, res, br, work = bufs[:7]
+    side = [b.ptr for b in bufs[4:13]]   # the batched form's buffers: three each of current, activated, residual
     audio = backend.alloc(L)
 
     codec = importlib.import_module(pkg.__name__ + ".codec")
 
     def decode(fused):
-        """fused: the element-wise operators inside the convolutions' epilogues (mynah_hip_conv1d_fused); else the operator
-        sequence decode_codec_resident issues through the seam.  Both give the same samples, bit for bit."""
+        """fused: the element-wise operators inside the convolutions' epilogues (mynah_hip_conv1d_fused), with "batched" also a
+        residual layer's three branches side by side in one launch per block and position (mynah_hip_conv1d_fused_batch);
+        else the operator sequence decode_codec_resident issues through the seam.  All give the same samples, bit for bit."""
         nonlocal cur, up, out
         C, L = 864, frames
         if fused:
@@ -232,7 +234,10 @@ def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
             backend.conv_transpose_dev(cur.ptr, up.ptr, C, nc, L, nl, 2 * st["rate"], st["rate"], nc, *st["up"])
             if fused:
                 then_alpha = stages[index + 1]["alpha"] if index + 1 < len(stages) else post_alpha
-                codec.res_layer_fused(backend, st["blocks"], up.ptr, out.ptr, nc, nl, work.ptr, act.ptr, res.ptr, then_alpha=then_alpha)
+                if fused == "batched":
+                    codec.res_layer_batched(backend, st["blocks"], up.ptr, out.ptr, nc, nl, side[0:3], side[3:6], side[6:9], then_alpha=then_alpha)
+                else:
+                    codec.res_layer_fused(backend, st["blocks"], up.ptr, out.ptr, nc, nl, work.ptr, act.ptr, res.ptr, then_alpha=then_alpha)
             else:
                 codec.res_layer(backend, st["blocks"], up.ptr, out.ptr, nc, nl, work.ptr, act.ptr, res.ptr, br.ptr)
             cur, out = out, cur
@@ -243,7 +248,7 @@ def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
         backend.clip_dev(audio.ptr, L)
 
     timings, waves = {}, {}
-    for fused in (False, True):
+    for fused in (False, True, "batched"):
         for _ in range(warmup):
             decode(fused)
         backend.sync()
@@ -253,12 +258,13 @@ def time_codec(pkg, backend, frames=64, runs=4, warmup=2):
         timings[fused] = backend.timer_end() / runs
         waves[fused] = audio.read()
     assert np.array_equal(waves[False].view(np.uint32), waves[True].view(np.uint32)), "the fused sequence changed the samples"
-    ms, samples = timings[True], waves[True]
+    assert np.array_equal(waves[False].view(np.uint32), waves["batched"].view(np.uint32)), "the batched sequence changed the samples"
+    ms, samples = timings["batched"], waves["batched"]
     assert np.all(np.isfinite(samples)) and np.abs(samples).max() <= 1.0, "codec output is not a clipped waveform"
     for d in bufs + [latent, audio]:
         d.free()
     return {"frames": frames, "samples": int(L), "ms": ms, "flops": flops, "tflops": flops / (ms * 1e-3) / 1e12,
-            "ms_seam_operator_sequence": timings[False]}
+            "ms_seam_operator_sequence": timings[False], "ms_one_launch_per_convolution": timings[True]}
 
 
 # (with one or two streams the attention partials are folded by the output projection that follows; with more, by
@@ -499,8 +505,10 @@ def main():
                                        % (codec["frames"], codec["samples"]),
                            "ms": round(codec["ms"], 3), "flops": codec["flops"], "tflops": round(codec["tflops"], 2), "bound": "mfma",
                            "peak_tflops": 157.3, "frac": round(codec["tflops"] / 157.3, 4),
-                           "form": "element-wise operators in the convolutions' epilogues (mynah_hip_conv1d_fused), samples bit-identical "
-                                   "to the seam's operator sequence",
+                           "form": "element-wise operators in the convolutions' epilogues and a residual layer's three branches side by side, "
+                                   "one launch per block and position (mynah_hip_conv1d_fused_batch); samples bit-identical to the seam's "
+                                   "operator sequence",
+                           "ms_one_launch_per_convolution": round(codec["ms_one_launch_per_convolution"], 3),
                            "ms_seam_operator_sequence": round(codec["ms_seam_operator_sequence"], 3)}
     if not args.no_cpu:
         cpu = cpu_baseline()

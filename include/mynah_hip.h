@@ -207,6 +207,21 @@ int mynah_hip_conv1d_fused(void *state, const float *dev_input, float *dev_outpu
                            char *error, size_t error_capacity);
 int mynah_hip_snake_copy_dev(void *state, const float *dev_input, float *dev_output, const float *alpha, size_t channels,
                              size_t length, size_t snake_channels, char *error, size_t error_capacity);
+/* Up to four conv1d_fused calls of one shape (in_channels, out_channels, length) in ONE launch -- the three branches of a
+ * residual layer (res_layer_device, src/graph.c:2423-2498, walks them one after the other) at the same block and position.
+ * Each member has its own rows, weights, taps, dilation and epilogue and gets the values its own conv1d_fused call would
+ * give, bit for bit; the members run at the same time, so no member may write rows that another reads or writes (refused).
+ * With 3, 7 or 11 taps in every member the launch is shared; other tap counts run the members one after the other.
+ * No counterpart in the reference's seam. */
+typedef struct mynah_hip_conv1d_item {
+    const float *dev_input;
+    float *dev_output;
+    int kernel, dilation;
+    const float *weight, *bias;   /* host pointers, cached like every weight */
+    mynah_hip_conv1d_extra extra;
+} mynah_hip_conv1d_item;
+int mynah_hip_conv1d_fused_batch(void *state, const mynah_hip_conv1d_item *items, size_t count, int in_channels, int out_channels,
+                                 int length, char *error, size_t error_capacity);
 
 /* ------------------------------------------------------------------------------------------
  * Section 2 -- what the single-stream seam lacks

@@ -52,6 +52,11 @@ class Conv1dExtra(C.Structure):
                 ("snake_alpha", _vp), ("snake_channels", _sz), ("dev_activated", _vp)]
 
 
+class Conv1dItem(C.Structure):
+    _fields_ = [("dev_input", _vp), ("dev_output", _vp), ("kernel", C.c_int), ("dilation", C.c_int), ("weight", _vp), ("bias", _vp),
+                ("extra", Conv1dExtra)]
+
+
 class EncoderDesc(C.Structure):
     _fields_ = [("layers", _sz), ("width", _sz), ("heads", _sz), ("head_width", _sz), ("ffn_width", _sz),
                 ("vocab", _sz), ("max_positions", _sz), ("tok_table", _vp), ("pos_table", _vp),
@@ -112,6 +117,7 @@ def load_library(path=LIB_PATH):
                                                  *_err]
     lib.mynah_hip_snake_dev.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, *_err]
     lib.mynah_hip_snake_copy_dev.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, *_err]
+    lib.mynah_hip_conv1d_fused_batch.argtypes = [_vp, C.POINTER(Conv1dItem), _sz, C.c_int, C.c_int, C.c_int, *_err]
     lib.mynah_hip_conv1d_fused.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp,
                                            C.POINTER(Conv1dExtra), *_err]
     lib.mynah_hip_set_quant.argtypes = [_vp, C.c_int, C.c_int, *_err]
@@ -370,6 +376,20 @@ class Backend:
                             0 if alpha is None else (out_ch // 2 if snake_channels is None else snake_channels), activated)
         self._call("mynah_hip_conv1d_fused", din, dout, in_ch, out_ch, length, kernel, dilation, _np_ptr(self.keep(weight)),
                    None if bias is None else _np_ptr(self.keep(bias)), C.byref(extra))
+
+    def conv1d_fused_batch(self, items, in_ch, out_ch, length):
+        """Up to four conv1d_fused calls of one shape in one launch.  items: dicts with din, dout, kernel, dilation, weight and,
+        optionally, bias, residual, residual2, scale, alpha, snake_channels, activated (conv1d_fused's arguments)."""
+        arr = (Conv1dItem * len(items))()
+        for slot, it in zip(arr, items):
+            alpha = it.get("alpha")
+            snake = 0 if alpha is None else (out_ch // 2 if it.get("snake_channels") is None else it["snake_channels"])
+            slot.dev_input, slot.dev_output, slot.kernel, slot.dilation = it["din"], it["dout"], it["kernel"], it["dilation"]
+            slot.weight = _np_ptr(self.keep(it["weight"]))
+            slot.bias = None if it.get("bias") is None else _np_ptr(self.keep(it["bias"]))
+            slot.extra = Conv1dExtra(it.get("residual"), it.get("residual2"), it.get("scale", 1.0), 0 if alpha is None else 1,
+                                     None if alpha is None else _np_ptr(self.keep(alpha)), snake, it.get("activated"))
+        self._call("mynah_hip_conv1d_fused_batch", arr, _sz(len(items)), in_ch, out_ch, length)
 
     def argmax_dev(self, dlogits, vocab, codebook_size, eos_id, allow_eos):
         out = C.c_uint(0)

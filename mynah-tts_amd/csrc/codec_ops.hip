@@ -165,17 +165,13 @@ __device__ __forceinline__ void conv_products(const float *wrow, const float *ir
 // layout LDS keeps, so staging it is a plain copy -- no index arithmetic, no bounds.
 // FUSED: the build that mynah_hip_conv1d_fused launches (residuals, scale, activation after the products); the seam's
 // conv1d keeps a build without any of it.
-template <int WM, int WN, int KF, bool FUSED>
-__global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float *const out_arg, const float *const chunks_arg, const float *const bias_arg, const int in_ch_arg,
-                                                const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const int tiles_arg,
-                                                const ConvArgs a_arg) {
+// (the tile's work as a function: the kernel of one convolution and the kernel of several side by side both run it)
+// LEAN: the residual values are requested in the epilogue instead of before the last block's products (64 registers less:
+// the build that runs several convolutions side by side wants three workgroups on a CU).
+template <int WM, int WN, int KF, bool FUSED, bool LEAN = false>
+__device__ __forceinline__ void conv_tile(const ConvArgs &a_arg, const float *const chunks_arg, const int tiles_arg, float *const lds) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
-    extern __shared__ __align__(16) float lds[];
-    // (the rows, the weights and the shape lead the arguments and repeat fields of a_arg: leading scalar arguments are in
-    // registers when a wavefront starts, a structure passed by value is fetched from memory where its fields are first used)
     ConvArgs a = a_arg;
-    a.in = in_arg; a.out = out_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
-    a.kernel = kernel_arg; a.dilation = dilation_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;   // inner elements per step
     const int a_stride = kb + 4;               // the chunks' row stride: rows stay 16-byte aligned, and a stride of 4 mod 8 words
@@ -267,7 +263,7 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
         publish(i0);
         __syncthreads();
         if (i0 + kConvChannels < a.in_ch) fetch(i0 + kConvChannels);   // in flight during the products below
-        else request_residuals();
+        else if constexpr (!LEAN) request_residuals();
         conv_products<KF>(s_w + (wm * 32 + col) * a_stride + half * a.kernel, s_in + half * win + wn * 64 + col, a.kernel, a.dilation,
                           win, acc0, acc1, min(kConvChannels / 2, (a.in_ch - i0 + 1) / 2));
         __syncthreads();
@@ -296,6 +292,7 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
             for (int row = 0; row < rows; ++row, p += a.length) *p = s_tile[row * kTileStride + lane];
         }
     };
+    if constexpr (LEAN) request_residuals();
     const auto combine = [&](auto has_first, auto has_second) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -373,22 +370,28 @@ __global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float
         conv_emit(a, m0 + wm * 32 + row, index, s_tile[row * kTileStride + lane], s_alpha[row], s_alpha[32 + row]);
 }
 
-// The same product for short rows (few positions, many channels: the codec's first stages), where 64 x 128 tiles would
-// leave most of the chip idle: a workgroup owns a 32 x 64 tile and its four wavefronts split the input channels between
-// them (wavefront w takes channel blocks w, w + 4, ...: one weight chunk each), each staging its own blocks in its own
-// part of LDS; the four partial tiles are added in wavefront order at the end, so the result does not depend on timing.
-// NT: 32-position halves per tile (2, or 1 for the very shortest rows: twice the workgroups).
-template <int KF, int NT>
-__global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg, float *const out_arg, const float *const chunks_arg, const float *const bias_arg, const int in_ch_arg,
-                                                      const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const int tiles_arg,
-                                                      const ConvArgs a_arg) {
-    constexpr int TM = 32, TN = 32 * NT;
+template <int WM, int WN, int KF, bool FUSED>
+__global__ void __launch_bounds__(256) k_conv1d(const float *const in_arg, float *const out_arg, const float *const chunks_arg, const float *const bias_arg, const int in_ch_arg,
+                                                const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const int tiles_arg,
+                                                const ConvArgs a_arg) {
     extern __shared__ __align__(16) float lds[];
     // (the rows, the weights and the shape lead the arguments and repeat fields of a_arg: leading scalar arguments are in
     // registers when a wavefront starts, a structure passed by value is fetched from memory where its fields are first used)
     ConvArgs a = a_arg;
     a.in = in_arg; a.out = out_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
     a.kernel = kernel_arg; a.dilation = dilation_arg;
+    conv_tile<WM, WN, KF, FUSED>(a, chunks_arg, tiles_arg, lds);
+}
+
+// The same product for short rows (few positions, many channels: the codec's first stages), where 64 x 128 tiles would
+// leave most of the chip idle: a workgroup owns a 32 x 64 tile and its four wavefronts split the input channels between
+// them (wavefront w takes channel blocks w, w + 4, ...: one weight chunk each), each staging its own blocks in its own
+// part of LDS; the four partial tiles are added in wavefront order at the end, so the result does not depend on timing.
+// NT: 32-position halves per tile (2, or 1 for the very shortest rows: twice the workgroups).
+template <int KF, int NT>
+__device__ __forceinline__ void conv_split_tile(const ConvArgs &a_arg, const float *const chunks_arg, const int tiles_arg, float *const lds) {
+    constexpr int TM = 32, TN = 32 * NT;
+    ConvArgs a = a_arg;
     if constexpr (KF != 0) a.kernel = KF;
     const int kb = kConvChannels * a.kernel;
     const int a_stride = kb + 4;   // the chunks' row stride (see k_conv1d)
@@ -508,6 +511,54 @@ __global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg,
     }
 }
 
+template <int KF, int NT>
+__global__ void __launch_bounds__(256) k_conv1d_split(const float *const in_arg, float *const out_arg, const float *const chunks_arg, const float *const bias_arg, const int in_ch_arg,
+                                                      const int out_ch_arg, const int length_arg, const int kernel_arg, const int dilation_arg, const int tiles_arg,
+                                                      const ConvArgs a_arg) {
+    extern __shared__ __align__(16) float lds[];
+    // (leading scalar arguments: see k_conv1d)
+    ConvArgs a = a_arg;
+    a.in = in_arg; a.out = out_arg; a.bias = bias_arg; a.in_ch = in_ch_arg; a.out_ch = out_ch_arg; a.length = length_arg;
+    a.kernel = kernel_arg; a.dilation = dilation_arg;
+    conv_split_tile<KF, NT>(a, chunks_arg, tiles_arg, lds);
+}
+
+// Several convolutions of one shape side by side in one launch (the three branches of a residual layer: same rows in and
+// out, own weights, taps, dilation and epilogue): blockIdx.z names the convolution, every workgroup runs the tile's work of
+// its own, so the values are those of the single launches.  A launch's fixed cost (dispatch, kernel start, the first
+// block's round trip, the stores behind the last product) is paid once for all of them, and a CU holds workgroups of
+// different convolutions whose staging and products overlap.  Tap counts 3, 7 and 11 only (the builds with straight-line
+// products); always the build with the fused epilogue (with nothing to add it leaves the product's own bits).
+constexpr int kConvBatchMax = 4;
+struct ConvBatchArgs {
+    ConvArgs item[kConvBatchMax];
+    const float *chunks[kConvBatchMax];
+    int tiles;
+};
+
+// (three wavefronts per SIMD asked of the compiler: alone, a 256-thread workgroup is given every register of the CU)
+template <int WM, int WN>
+__global__ void __launch_bounds__(256, 3) k_conv1d_batch(const ConvBatchArgs b) {
+    extern __shared__ __align__(16) float lds[];
+    const int z = blockIdx.z;
+    switch (b.item[z].kernel) {
+        case 3: conv_tile<WM, WN, 3, true, true>(b.item[z], b.chunks[z], b.tiles, lds); break;
+        case 7: conv_tile<WM, WN, 7, true, true>(b.item[z], b.chunks[z], b.tiles, lds); break;
+        default: conv_tile<WM, WN, 11, true, true>(b.item[z], b.chunks[z], b.tiles, lds); break;
+    }
+}
+
+template <int NT>
+__global__ void __launch_bounds__(256, 2) k_conv1d_split_batch(const ConvBatchArgs b) {
+    extern __shared__ __align__(16) float lds[];
+    const int z = blockIdx.z;
+    switch (b.item[z].kernel) {
+        case 3: conv_split_tile<3, NT>(b.item[z], b.chunks[z], b.tiles, lds); break;
+        case 7: conv_split_tile<7, NT>(b.item[z], b.chunks[z], b.tiles, lds); break;
+        default: conv_split_tile<11, NT>(b.item[z], b.chunks[z], b.tiles, lds); break;
+    }
+}
+
 struct ConvTransposeArgs {
     const float *in;     // [in_ch, length]
     float *out;          // [out_ch, output_length]
@@ -612,12 +663,55 @@ int launch_conv_split(State *st, const ConvArgs &a, const ConvBlocks &chunks, ch
     return launch_conv_split_n<2>(st, a, chunks, error, capacity);
 }
 
+// LDS of the largest member, as the single launches size it
+template <int WM, int WN>
+int launch_conv_batch(State *st, const ConvBatchArgs &b, int count, char *error, size_t capacity) {
+    constexpr int TM = 32 * WM, TN = 64 * WN;
+    size_t lds = (4 * 32 * kTileStride + 4 * 64) * sizeof(float);
+    for (int i = 0; i < count; ++i) {
+        const ConvArgs &a = b.item[i];
+        const int slots = (WM * 8 * (kConvChannels * a.kernel + 4) + 255) / 256;
+        const size_t need = ((size_t)slots * 1024 + (size_t)(kConvChannels + 2) * (TN + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
+        lds = need > lds ? need : lds;
+    }
+    static bool raised = false;   // per instantiation
+    if (!raised) {
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d_batch<WM, WN>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+        raised = true;
+    }
+    const ConvArgs &a = b.item[0];
+    const dim3 grid((unsigned)((a.length + TN - 1) / TN), (unsigned)((a.out_ch + TM - 1) / TM), (unsigned)count);
+    hipLaunchKernelGGL((k_conv1d_batch<WM, WN>), grid, dim3(256), lds, st->stream, b);
+    return hip_check(hipGetLastError(), "conv1d batch launch", error, capacity);
+}
+
+template <int NT>
+int launch_conv_split_batch(State *st, const ConvBatchArgs &b, int count, char *error, size_t capacity) {
+    size_t lds = (4 * 32 * 64 + 64) * sizeof(float);
+    for (int i = 0; i < count; ++i) {
+        const ConvArgs &a = b.item[i];
+        const int slots = (8 * (kConvChannels * a.kernel + 4) + 63) / 64;
+        const size_t per_wave = (size_t)slots * 256 + (size_t)kConvChannels * (32 * NT + (a.kernel - 1) * a.dilation);
+        const size_t need = (4 * per_wave + 2 * (32 * NT + (a.kernel - 1) * a.dilation) + 64) * sizeof(float);
+        lds = need > lds ? need : lds;
+    }
+    static bool raised = false;
+    if (!raised) {
+        MYNAH_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&k_conv1d_split_batch<NT>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+        raised = true;
+    }
+    const ConvArgs &a = b.item[0];
+    const dim3 grid((unsigned)((a.length + 32 * NT - 1) / (32 * NT)), (unsigned)((a.out_ch + 31) / 32), (unsigned)count);
+    hipLaunchKernelGGL((k_conv1d_split_batch<NT>), grid, dim3(256), lds, st->stream, b);
+    return hip_check(hipGetLastError(), "conv1d batch launch", error, capacity);
+}
+
 }  // namespace
 
-static int conv1d_entry(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
-                        int kernel, int dilation, const float *weight, const float *bias, const mynah_hip_conv1d_extra *extra,
-                        char *error, size_t capacity) {
-    State *st = enter_state(state);
+// Checks one convolution's arguments, caches its weights and fills the kernels' argument block.
+static int conv1d_prepare(State *st, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                          int kernel, int dilation, const float *weight, const float *bias, const mynah_hip_conv1d_extra *extra,
+                          ConvArgs *out_args, ConvBlocks *out_chunks, char *error, size_t capacity) {
     if (st == nullptr || dev_input == nullptr || dev_output == nullptr || weight == nullptr || in_channels <= 0 || out_channels <= 0 ||
         length <= 0 || kernel <= 0 || dilation <= 0) {
         set_error(error, capacity, "invalid conv1d arguments");   // the checks of metal_ops_conv1d, gpu/metal/backend_metal_ops.m:371-372
@@ -650,12 +744,33 @@ static int conv1d_entry(void *state, const float *dev_input, float *dev_output, 
         a.act_out = extra->dev_activated;
         if (a.activate && a.snake_channels != 0 && cached_vector(st, extra->snake_alpha, extra->snake_channels, &a.alpha, error, capacity) != 0) return -1;
     }
-    // few output channels: one row of wavefronts, wider in time; too few large tiles to fill the chip (and enough input
-    // channels to share out): small tiles with the channels split over the wavefronts
+    *out_args = a;
+    *out_chunks = chunks;
+    return 0;
+}
+
+// few output channels: one row of wavefronts, wider in time; too few large tiles to fill the chip (and enough input
+// channels to share out): small tiles with the channels split over the wavefronts
+static bool conv_takes_split(const State *st, int in_channels, int out_channels, int length) {
     const long tiles = out_channels <= 32 ? (long)((length + 255) / 256) : (long)((out_channels + 63) / 64) * ((length + 127) / 128);
-    if (tiles < st->cu_count && in_channels >= 4 * kConvChannels) return launch_conv_split(st, a, chunks, error, capacity);
-    if (out_channels <= 32) return launch_conv<1, 4>(st, a, chunks, error, capacity);
+    return tiles < st->cu_count && in_channels >= 4 * kConvChannels;
+}
+
+static int conv1d_launch(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
+    if (conv_takes_split(st, a.in_ch, a.out_ch, a.length)) return launch_conv_split(st, a, chunks, error, capacity);
+    if (a.out_ch <= 32) return launch_conv<1, 4>(st, a, chunks, error, capacity);
     return launch_conv<2, 2>(st, a, chunks, error, capacity);
+}
+
+static int conv1d_entry(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
+                        int kernel, int dilation, const float *weight, const float *bias, const mynah_hip_conv1d_extra *extra,
+                        char *error, size_t capacity) {
+    State *st = enter_state(state);
+    ConvArgs a;
+    ConvBlocks chunks;
+    if (conv1d_prepare(st, dev_input, dev_output, in_channels, out_channels, length, kernel, dilation, weight, bias, extra, &a, &chunks, error, capacity) != 0)
+        return -1;
+    return conv1d_launch(st, a, chunks, error, capacity);
 }
 
 extern "C" int mynah_hip_conv1d(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels, int length,
@@ -671,6 +786,52 @@ extern "C" int mynah_hip_conv1d_fused(void *state, const float *dev_input, float
         return -1;
     }
     return conv1d_entry(state, dev_input, dev_output, in_channels, out_channels, length, kernel, dilation, weight, bias, extra, error, capacity);
+}
+
+extern "C" int mynah_hip_conv1d_fused_batch(void *state, const mynah_hip_conv1d_item *items, size_t count, int in_channels, int out_channels,
+                                            int length, char *error, size_t capacity) {
+    State *st = enter_state(state);
+    if (st == nullptr || items == nullptr || count == 0 || count > (size_t)kConvBatchMax) {
+        set_error(error, capacity, "conv1d_fused_batch: one to four convolutions");
+        return -1;
+    }
+    ConvBatchArgs b{};
+    ConvBlocks chunks[kConvBatchMax];
+    bool side_by_side = true;
+    for (size_t i = 0; i < count; ++i) {
+        const mynah_hip_conv1d_item &it = items[i];
+        if (conv1d_prepare(st, it.dev_input, it.dev_output, in_channels, out_channels, length, it.kernel, it.dilation, it.weight, it.bias, &it.extra,
+                           &b.item[i], &chunks[i], error, capacity) != 0)
+            return -1;
+        b.chunks[i] = chunks[i].data;
+        side_by_side = side_by_side && (it.kernel == 3 || it.kernel == 7 || it.kernel == 11) && chunks[i].tiles == chunks[0].tiles;
+        // the members run at the same time: what one writes, no other may read or write
+        for (size_t j = 0; j < count; ++j) {
+            if (j == i) continue;
+            const mynah_hip_conv1d_item &o = items[j];
+            const float *const written[2] = {it.dev_output, it.extra.dev_activated};
+            for (const float *w : written) {
+                if (w == nullptr) continue;
+                if (w == o.dev_input || w == o.dev_output || w == o.extra.dev_residual || w == o.extra.dev_residual2 || w == o.extra.dev_activated) {
+                    set_error(error, capacity, "conv1d_fused_batch: a member writes rows that another member reads or writes");
+                    return -1;
+                }
+            }
+        }
+    }
+    b.tiles = chunks[0].tiles;
+    if (!side_by_side || count == 1) {   // other tap counts: one after the other (the same values)
+        for (size_t i = 0; i < count; ++i)
+            if (conv1d_launch(st, b.item[i], chunks[i], error, capacity) != 0) return -1;
+        return 0;
+    }
+    if (conv_takes_split(st, in_channels, out_channels, length)) {
+        const long tiles = (long)((out_channels + 31) / 32) * ((length + 63) / 64);
+        if (tiles < st->cu_count) return launch_conv_split_batch<1>(st, b, (int)count, error, capacity);
+        return launch_conv_split_batch<2>(st, b, (int)count, error, capacity);
+    }
+    if (out_channels <= 32) return launch_conv_batch<1, 4>(st, b, (int)count, error, capacity);
+    return launch_conv_batch<2, 2>(st, b, (int)count, error, capacity);
 }
 
 extern "C" int mynah_hip_conv_transpose_dev(void *state, const float *dev_input, float *dev_output, int in_channels, int out_channels,

@@ -137,6 +137,15 @@ def test_fused_res_layer_is_the_operator_sequence(pkg, backend, orc, nerr, C, L)
     assert np.isfinite(seq).all()
     assert np.array_equal(seq.view(np.uint32), fused.view(np.uint32))
     assert np.array_equal(din.read().reshape(C, L), x), "the layer's input was written"
+    # the three branches' convolutions of a block and position in one launch each (conv1d_fused_batch): the same bits again
+    more = [backend.alloc(n) for _ in range(10)]
+    codec.res_layer_batched(backend, blocks, din.ptr, more[0].ptr, C, L, [b.ptr for b in more[1:4]], [b.ptr for b in more[4:7]],
+                            [b.ptr for b in more[7:10]])
+    batched = more[0].read().reshape(C, L)
+    assert np.array_equal(seq.view(np.uint32), batched.view(np.uint32))
+    assert np.array_equal(din.read().reshape(C, L), x), "the layer's input was written"
+    for d in more:
+        d.free()
     if C == 70:
         total = np.zeros_like(x)
         for branch in blocks:
@@ -146,6 +155,45 @@ def test_fused_res_layer_is_the_operator_sequence(pkg, backend, orc, nerr, C, L)
             total += cur
         assert nerr(fused, total * np.float32(1.0 / 3.0)) < 1e-5
     for d in bufs + [din]:
+        d.free()
+
+
+def test_conv_batch_members_and_refusals(pkg, backend):
+    """conv1d_fused_batch: members with tap counts outside 3 / 7 / 11 (run one after the other) and with them (one launch)
+    give their own conv1d_fused results bit for bit; a member that writes what another reads is refused."""
+    _announce("conv1d_fused_batch members")
+    rng = np.random.default_rng(77)
+    C, O, L = 40, 72, 210
+    x = rng.standard_normal((3, C, L)).astype(np.float32)
+    r = rng.standard_normal((O, L)).astype(np.float32)
+    alpha = (np.abs(rng.standard_normal(O // 2)) + 0.1).astype(np.float32)
+    dins = [backend.alloc(C * L).write(x[i]) for i in range(3)]
+    dres = backend.alloc(O * L).write(r)
+    for taps in ((3, 7, 11), (11, 11, 3), (5, 7, 11)):
+        ws = [(rng.standard_normal((O, C, k)) / np.sqrt(C * k)).astype(np.float32) for k in taps]
+        bs = [rng.standard_normal(O).astype(np.float32) for _ in taps]
+        single = [backend.alloc(O * L) for _ in taps]
+        together = [backend.alloc(O * L) for _ in taps]
+        acts = [backend.alloc(O * L) for _ in range(2)]
+        extras = [dict(residual=dres.ptr, scale=0.5), dict(alpha=alpha, activated=acts[0].ptr), dict()]
+        for i, k in enumerate(taps):
+            e = dict(extras[i])
+            if "activated" in e:
+                e["activated"] = acts[1].ptr
+            backend.conv1d_fused(dins[i].ptr, single[i].ptr, C, O, L, k, 1 + i, ws[i], bs[i], **e)
+        backend.conv1d_fused_batch([dict(din=dins[i].ptr, dout=together[i].ptr, kernel=k, dilation=1 + i, weight=ws[i], bias=bs[i], **extras[i])
+                                    for i, k in enumerate(taps)], C, O, L)
+        for a, b in zip(single, together):
+            assert np.array_equal(a.read().view(np.uint32), b.read().view(np.uint32)), taps
+        assert np.array_equal(acts[0].read().view(np.uint32), acts[1].read().view(np.uint32)), taps
+        with pytest.raises(pkg.BackendError, match="another member"):
+            backend.conv1d_fused_batch([dict(din=dins[0].ptr, dout=together[0].ptr, kernel=taps[0], dilation=1, weight=ws[0]),
+                                        dict(din=together[0].ptr, dout=together[1].ptr, kernel=taps[1], dilation=1, weight=ws[1])], C, O, L)
+        for d in single + together + acts:
+            d.free()
+    with pytest.raises(pkg.BackendError, match="one to four"):
+        backend.conv1d_fused_batch([], C, O, L)
+    for d in dins + [dres]:
         d.free()
 
 
