@@ -222,6 +222,15 @@ typedef struct mynah_hip_conv1d_item {
 } mynah_hip_conv1d_item;
 int mynah_hip_conv1d_fused_batch(void *state, const mynah_hip_conv1d_item *items, size_t count, int in_channels, int out_channels,
                                  int length, char *error, size_t error_capacity);
+/* One pass over up to four row sets [channels, length]: v = ((in0 + in1) + in2 ...) * scale, then every output j gets v, or
+ * half-snake(v) with alphas[j] when that is non-null (host pointer, cached; alphas itself may be NULL) -- the arithmetic of
+ * residual_inplace per addend, scale_dev and snake_dev / snake_copy_dev in that order, value by value.  An output may be one
+ * of the inputs (a value is read before it is written); no output may be named twice.  It serves the residual layer with its
+ * branches side by side: one input and three activated outputs at the layer's start, three branch results summed, scaled
+ * by a third and activated at its end.  No counterpart in the reference's seam. */
+int mynah_hip_rows_combine_dev(void *state, const float *const *dev_inputs, size_t inputs, float scale, float *const *dev_outputs,
+                               const float *const *alphas, size_t outputs, size_t channels, size_t length, size_t snake_channels,
+                               char *error, size_t error_capacity);
 
 /* ------------------------------------------------------------------------------------------
  * Section 2 -- what the single-stream seam lacks

@@ -117,6 +117,7 @@ def load_library(path=LIB_PATH):
                                                  *_err]
     lib.mynah_hip_snake_dev.argtypes = [_vp, _vp, _vp, _sz, _sz, _sz, *_err]
     lib.mynah_hip_snake_copy_dev.argtypes = [_vp, _vp, _vp, _vp, _sz, _sz, _sz, *_err]
+    lib.mynah_hip_rows_combine_dev.argtypes = [_vp, C.POINTER(_vp), _sz, C.c_float, C.POINTER(_vp), C.POINTER(_vp), _sz, _sz, _sz, _sz, *_err]
     lib.mynah_hip_conv1d_fused_batch.argtypes = [_vp, C.POINTER(Conv1dItem), _sz, C.c_int, C.c_int, C.c_int, *_err]
     lib.mynah_hip_conv1d_fused.argtypes = [_vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp,
                                            C.POINTER(Conv1dExtra), *_err]
@@ -390,6 +391,13 @@ class Backend:
             slot.extra = Conv1dExtra(it.get("residual"), it.get("residual2"), it.get("scale", 1.0), 0 if alpha is None else 1,
                                      None if alpha is None else _np_ptr(self.keep(alpha)), snake, it.get("activated"))
         self._call("mynah_hip_conv1d_fused_batch", arr, _sz(len(items)), in_ch, out_ch, length)
+
+    def rows_combine_dev(self, dins, scale, douts, alphas, channels, length, snake_channels=None):
+        """((in0 + in1) + ...) * scale into every output, through the half-snake of alphas[j] where that is not None."""
+        arr_in, arr_out = (_vp * len(dins))(*dins), (_vp * len(douts))(*douts)
+        arr_al = (_vp * len(douts))(*[None if a is None else _np_ptr(self.keep(a)) for a in alphas])
+        self._call("mynah_hip_rows_combine_dev", arr_in, _sz(len(dins)), C.c_float(scale), arr_out, arr_al, _sz(len(douts)), _sz(channels),
+                   _sz(length), _sz(channels // 2 if snake_channels is None else snake_channels))
 
     def argmax_dev(self, dlogits, vocab, codebook_size, eos_id, allow_eos):
         out = C.c_uint(0)

@@ -6,7 +6,8 @@ end.  `res_layer_fused` computes the same values, bit for bit, from a third of t
 travel in the epilogue of the convolution before them (mynah_hip_conv1d_fused), and only a branch's first activation is a
 pass of its own (snake_copy_dev).  `res_layer_batched` issues res_layer_fused's calls with the three branches' convolutions
 of one block and position in one launch each (mynah_hip_conv1d_fused_batch): the branches do not depend on each other until
-their last convolutions, which add into the output one after the other as before.  Same values again, bit for bit.
+their last convolutions; those run side by side as well, each into its own rows, and one pass (rows_combine_dev) adds the
+branches in order, scales and activates.  Same values again, bit for bit.
 
 blocks[branch][block] = (alpha_in, (w_in, b_in), alpha_skip, (w_skip, b_skip), dilation); the branch's kernel size is the
 weights' last dimension.  Buffers are device allocations of channels * length floats.
@@ -57,8 +58,8 @@ def res_layer_fused(backend, blocks, din, dout, channels, length, current, activ
 def res_layer_batched(backend, blocks, din, dout, channels, length, currents, activateds, residuals, then_alpha=None):
     """currents, activateds, residuals: one buffer per branch each (the branches run side by side)."""
     branches = len(blocks)
-    for index, branch in enumerate(blocks):
-        backend.snake_copy_dev(din, activateds[index], branch[0][0], channels, length, channels // 2)
+    # the input through every branch's first activation: one pass, one output per branch
+    backend.rows_combine_dev([din], 1.0, activateds, [branch[0][0] for branch in blocks], channels, length)
     positions = len(blocks[0])
     for position in range(positions):
         # input convs of every branch, their results activated for the skip convs
@@ -72,10 +73,10 @@ def res_layer_batched(backend, blocks, din, dout, channels, length, currents, ac
                                          "residual": din if position == 0 else currents[i], "alpha": blocks[i][position + 1][0],
                                          "activated": activateds[i]} for i in range(branches)], channels, channels, length)
         else:
-            # the branches' last convs add into the output in branch order, the last one scales the sum: one after the other
-            for index in range(branches):
-                a_in, (w_in, b_in), a_skip, (w_skip, b_skip), dilation = blocks[index][position]
-                backend.conv1d_fused(residuals[index], dout, channels, channels, length, w_skip.shape[2], 1, w_skip, b_skip,
-                                     residual=din if position == 0 else currents[index], residual2=None if index == 0 else dout,
-                                     scale=1.0 / 3.0 if index + 1 == branches else 1.0,
-                                     alpha=then_alpha if index + 1 == branches else None)
+            # the branches' last skip convs + residual adds side by side too (each into its own rows), then one pass that adds
+            # the branches in branch order, scales the sum and applies the caller's activation: ((b0 + b1) + b2) * 1/3, which
+            # is what the one-after-the-other form computes in its last convolutions' epilogues
+            backend.conv1d_fused_batch([{"din": residuals[i], "dout": currents[i], "kernel": blocks[i][position][3][0].shape[2], "dilation": 1,
+                                         "weight": blocks[i][position][3][0], "bias": blocks[i][position][3][1],
+                                         "residual": din if position == 0 else currents[i]} for i in range(branches)], channels, channels, length)
+            backend.rows_combine_dev(currents, 1.0 / branches, [dout], [then_alpha], channels, length)

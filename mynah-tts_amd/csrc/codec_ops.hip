@@ -596,6 +596,42 @@ __global__ void __launch_bounds__(256) k_snake(const float *in, float *out, cons
     out[index] = half_snake(v, snake_row, al, 1.0f / (al + 1e-9f));
 }
 
+// Row sets added in order, scaled, and written to one or more outputs, each plain or through its own half-snake:
+// v = ((in0 + in1) + in2 ...) * scale; out_j = alpha_j ? half_snake(v) : v.  One pass instead of residual_inplace per
+// addend, scale_dev and snake_dev (or snake_copy_dev per output), with the same arithmetic in the same order.
+constexpr int kRowsMax = 4;
+struct RowsCombineArgs {
+    const float *in[kRowsMax];
+    float *out[kRowsMax];
+    const float *alpha[kRowsMax];   // null: the value as it is
+    int inputs, outputs;
+    float scale;
+    size_t count;
+    int length, snake_channels;
+};
+
+__global__ void __launch_bounds__(256) k_rows_combine(const RowsCombineArgs a) {
+    const size_t index = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (index >= a.count) return;
+    float v = a.in[0][index];
+    if (a.inputs > 1) v = v + a.in[1][index];
+    if (a.inputs > 2) v = v + a.in[2][index];
+    if (a.inputs > 3) v = v + a.in[3][index];
+    v = v * a.scale;   // 1.0f keeps the bits
+    const int channel = (int)(index / (size_t)a.length);
+    const bool snake_row = channel < a.snake_channels;
+#pragma unroll
+    for (int j = 0; j < kRowsMax; ++j) {
+        if (j >= a.outputs) break;
+        float y = v;
+        if (a.alpha[j] != nullptr) {
+            const float al = snake_row ? a.alpha[j][channel] : 0.0f;
+            y = half_snake(v, snake_row, al, 1.0f / (al + 1e-9f));
+        }
+        a.out[j][index] = y;
+    }
+}
+
 template <int WM, int WN, int KF, bool FUSED>
 int launch_conv_f(State *st, const ConvArgs &a, const ConvBlocks &chunks, char *error, size_t capacity) {
     constexpr int TM = 32 * WM, TN = 64 * WN;
@@ -883,6 +919,45 @@ static int snake_entry(void *state, const float *dev_input, float *dev_output, c
     hipLaunchKernelGGL(k_snake, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st->stream, dev_input, dev_output, dev_alpha, count,
                        (int)length, (int)snake_channels);
     return hip_check(hipGetLastError(), "snake launch", error, capacity);
+}
+
+extern "C" int mynah_hip_rows_combine_dev(void *state, const float *const *dev_inputs, size_t inputs, float scale, float *const *dev_outputs,
+                                          const float *const *alphas, size_t outputs, size_t channels, size_t length, size_t snake_channels,
+                                          char *error, size_t capacity) {
+    State *st = enter_state(state);
+    if (st == nullptr || dev_inputs == nullptr || dev_outputs == nullptr || inputs == 0 || inputs > (size_t)kRowsMax || outputs == 0 ||
+        outputs > (size_t)kRowsMax || channels > (size_t)INT_MAX || length > (size_t)INT_MAX || snake_channels > channels || !(scale == scale)) {
+        set_error(error, capacity, "invalid rows_combine arguments (one to four inputs and outputs)");
+        return -1;
+    }
+    RowsCombineArgs a{};
+    a.inputs = (int)inputs;
+    a.outputs = (int)outputs;
+    a.scale = scale;
+    a.count = channels * length;
+    a.length = (int)length;
+    a.snake_channels = (int)snake_channels;
+    if (a.count == 0) return 0;
+    if (a.count > (size_t)INT_MAX * 256u) {
+        set_error(error, capacity, "rows_combine: tensor too large");
+        return -1;
+    }
+    for (size_t i = 0; i < inputs; ++i) {
+        if (dev_inputs[i] == nullptr) { set_error(error, capacity, "rows_combine: null input"); return -1; }
+        a.in[i] = dev_inputs[i];
+    }
+    for (size_t j = 0; j < outputs; ++j) {
+        if (dev_outputs[j] == nullptr) { set_error(error, capacity, "rows_combine: null output"); return -1; }
+        for (size_t k = 0; k < j; ++k)
+            if (dev_outputs[k] == dev_outputs[j]) { set_error(error, capacity, "rows_combine: an output named twice"); return -1; }
+        a.out[j] = dev_outputs[j];
+        if (alphas != nullptr && alphas[j] != nullptr) {
+            if (snake_channels == 0) { a.alpha[j] = reinterpret_cast<const float *>(a.in[0]); continue; }   // only leaky rows: any non-null pointer, never read
+            if (cached_vector(st, alphas[j], snake_channels, &a.alpha[j], error, capacity) != 0) return -1;
+        }
+    }
+    hipLaunchKernelGGL(k_rows_combine, dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, st->stream, a);
+    return hip_check(hipGetLastError(), "rows_combine launch", error, capacity);
 }
 
 extern "C" int mynah_hip_snake_dev(void *state, float *dev_data, const float *alpha, size_t channels, size_t length, size_t snake_channels,

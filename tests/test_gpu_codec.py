@@ -197,6 +197,42 @@ def test_conv_batch_members_and_refusals(pkg, backend):
         d.free()
 
 
+def test_rows_combine_is_the_operator_sequence(pkg, backend):
+    """rows_combine_dev against residual_inplace per addend, scale_dev and snake_dev / snake_copy_dev: bit for bit."""
+    _announce("rows_combine_dev")
+    rng = np.random.default_rng(91)
+    C, L = 54, 333
+    rows = (rng.standard_normal((3, C, L)) * 3).astype(np.float32)
+    alphas = [(np.abs(rng.standard_normal(C // 2)) + 0.1).astype(np.float32) for _ in range(3)]
+    dins = [backend.alloc(C * L).write(rows[i]) for i in range(3)]
+    outs = [backend.alloc(C * L) for _ in range(3)]
+    want = backend.alloc(C * L)
+    bits = lambda d: d.read().view(np.uint32)
+    # one input, three activated outputs
+    backend.rows_combine_dev([dins[0].ptr], 1.0, [o.ptr for o in outs], alphas, C, L)
+    for o, al in zip(outs, alphas):
+        backend.snake_copy_dev(dins[0].ptr, want.ptr, al, C, L, C // 2)
+        assert np.array_equal(bits(o), bits(want))
+    # three inputs summed in order, scaled, one output plain and one activated
+    backend.rows_combine_dev([d.ptr for d in dins], 1.0 / 3.0, [outs[0].ptr, outs[1].ptr], [None, alphas[1]], C, L)
+    backend.copy_dev(want.ptr, dins[0].ptr, C * L)
+    backend.residual_inplace(want.ptr, dins[1].ptr, C * L)
+    backend.residual_inplace(want.ptr, dins[2].ptr, C * L)
+    backend.scale_dev(want.ptr, C * L, 1.0 / 3.0)
+    assert np.array_equal(bits(outs[0]), bits(want))
+    backend.snake_dev(want.ptr, alphas[1], C, L, C // 2)
+    assert np.array_equal(bits(outs[1]), bits(want))
+    # an output that is also the first input
+    backend.rows_combine_dev([d.ptr for d in dins], 1.0 / 3.0, [dins[0].ptr], [alphas[1]], C, L)
+    assert np.array_equal(bits(dins[0]), bits(want))
+    with pytest.raises(pkg.BackendError, match="named twice"):
+        backend.rows_combine_dev([dins[1].ptr], 1.0, [outs[0].ptr, outs[0].ptr], [None, None], C, L)
+    with pytest.raises(pkg.BackendError, match="one to four"):
+        backend.rows_combine_dev([], 1.0, [outs[0].ptr], [None], C, L)
+    for d in dins + outs + [want]:
+        d.free()
+
+
 def test_fused_conv_pieces(backend, orc, nerr):
     """Each optional step of conv1d_fused alone against the operator it stands for, bit for bit."""
     _announce("conv1d_fused steps")
