@@ -862,8 +862,10 @@ extern "C" int mynah_hip_conv1d_fused_batch(void *state, const mynah_hip_conv1d_
         return 0;
     }
     if (conv_takes_split(st, in_channels, out_channels, length)) {
+        // (the tile's width does not enter a value's arithmetic -- same channel blocks per wavefront, same order -- so the
+        // members may take the wider tile, half the weight traffic per product, as soon as all of them together fill the chip)
         const long tiles = (long)((out_channels + 31) / 32) * ((length + 63) / 64);
-        if (tiles < st->cu_count) return launch_conv_split_batch<1>(st, b, (int)count, error, capacity);
+        if (tiles * (long)count < st->cu_count) return launch_conv_split_batch<1>(st, b, (int)count, error, capacity);
         return launch_conv_split_batch<2>(st, b, (int)count, error, capacity);
     }
     if (out_channels <= 32) return launch_conv_batch<1, 4>(st, b, (int)count, error, capacity);

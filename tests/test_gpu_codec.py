@@ -197,6 +197,30 @@ def test_conv_batch_members_and_refusals(pkg, backend):
         d.free()
 
 
+def test_conv_batch_on_the_wider_split_tiles(backend):
+    """432 channels x 512 positions: alone a convolution takes the channel-split kernel's 32 x 32 tiles, three side by side
+    its 32 x 64 tiles.  The tile's width is not part of a value's arithmetic: every member keeps its single call's bits."""
+    _announce("conv1d_fused_batch on 432 x 512")
+    rng = np.random.default_rng(78)
+    C, L, taps = 432, 512, (3, 7, 11)
+    x = rng.standard_normal((C, L)).astype(np.float32)
+    din = backend.alloc(C * L).write(x)
+    ws = [(rng.standard_normal((C, C, k)) / np.sqrt(C * k)).astype(np.float32) for k in taps]
+    bs = [rng.standard_normal(C).astype(np.float32) for _ in taps]
+    single = [backend.alloc(C * L) for _ in taps]
+    together = [backend.alloc(C * L) for _ in taps]
+    for i, k in enumerate(taps):
+        backend.conv1d_fused(din.ptr, single[i].ptr, C, C, L, k, 1 + 2 * i, ws[i], bs[i], residual=din.ptr)
+    backend.conv1d_fused_batch([dict(din=din.ptr, dout=together[i].ptr, kernel=k, dilation=1 + 2 * i, weight=ws[i], bias=bs[i], residual=din.ptr)
+                                for i, k in enumerate(taps)], C, C, L)
+    for a, b in zip(single, together):
+        got = b.read()
+        assert np.isfinite(got).all()
+        assert np.array_equal(a.read().view(np.uint32), got.view(np.uint32))
+    for d in single + together + [din]:
+        d.free()
+
+
 def test_rows_combine_is_the_operator_sequence(pkg, backend):
     """rows_combine_dev against residual_inplace per addend, scale_dev and snake_dev / snake_copy_dev: bit for bit."""
     _announce("rows_combine_dev")
