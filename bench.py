@@ -280,7 +280,7 @@ STAGES = [("self-attention", "k_step_attention<self>", "LayerNorm + int8 act-qua
 # HBM bytes per launch of the dominant kernel of the batch-1 int8 line, from two rocprofv3 --pmc runs (FETCH_SIZE, then
 # WRITE_SIZE), each scaled by what the same counter reads for the library's plain 256 MiB read+write kernel.  The figure
 # belongs to the kernel sources it was measured on: it is reported only while their hash is the one recorded here.
-MEASURED_TRAFFIC = {"kernel": "k_linear<k=768, residual>", "bytes": 937934, "profile": "profiles/decode_step_int8_hbm_counters.md",
+MEASURED_TRAFFIC = {"kernel": "k_linear<k=768, residual>", "bytes": 937914, "profile": "profiles/decode_step_int8_hbm_counters.md",
                     "csrc_sha256": "b24c335f5817caf8"}
 
 
