@@ -159,23 +159,23 @@ def test_fused_res_layer_is_the_operator_sequence(pkg, backend, orc, nerr, C, L)
 
 
 def test_conv_batch_members_and_refusals(pkg, backend):
-    """conv1d_fused_batch: members with tap counts outside 3 / 7 / 11 (run one after the other) and with them (one launch)
-    give their own conv1d_fused results bit for bit; a member that writes what another reads is refused."""
+    """conv1d_fused_batch, two to four members: with tap counts outside 3 / 7 / 11 (run one after the other) and with them
+    (one launch) every member gets its own conv1d_fused result bit for bit; a member that writes what another reads is refused."""
     _announce("conv1d_fused_batch members")
     rng = np.random.default_rng(77)
     C, O, L = 40, 72, 210
-    x = rng.standard_normal((3, C, L)).astype(np.float32)
+    x = rng.standard_normal((4, C, L)).astype(np.float32)
     r = rng.standard_normal((O, L)).astype(np.float32)
     alpha = (np.abs(rng.standard_normal(O // 2)) + 0.1).astype(np.float32)
-    dins = [backend.alloc(C * L).write(x[i]) for i in range(3)]
+    dins = [backend.alloc(C * L).write(x[i]) for i in range(4)]
     dres = backend.alloc(O * L).write(r)
-    for taps in ((3, 7, 11), (11, 11, 3), (5, 7, 11)):
+    for taps in ((3, 7, 11), (11, 11, 3), (5, 7, 11), (7, 3), (11, 3, 7, 11)):
         ws = [(rng.standard_normal((O, C, k)) / np.sqrt(C * k)).astype(np.float32) for k in taps]
         bs = [rng.standard_normal(O).astype(np.float32) for _ in taps]
         single = [backend.alloc(O * L) for _ in taps]
         together = [backend.alloc(O * L) for _ in taps]
         acts = [backend.alloc(O * L) for _ in range(2)]
-        extras = [dict(residual=dres.ptr, scale=0.5), dict(alpha=alpha, activated=acts[0].ptr), dict()]
+        extras = [dict(residual=dres.ptr, scale=0.5), dict(alpha=alpha, activated=acts[0].ptr), dict(), dict(alpha=alpha)][:len(taps)]
         for i, k in enumerate(taps):
             e = dict(extras[i])
             if "activated" in e:
