@@ -380,7 +380,9 @@ int mynah_hip_output_head(void *state, const float *const *dev_hidden, size_t ba
  * dev_output holds the final-normed row, dev_logits / dev_probs what the head gives -- within the head's own tolerance: where
  * the step runs as one group of stage kernels with a final LayerNorm (up to 8 streams, head shapes the fused matvec takes),
  * the LayerNorm is the head product's prologue instead of a kernel of its own, one dependent launch less per step; the
- * normalised rows are the bits of the separate form.  Elsewhere the two calls run one after the other.  A step of this
+ * normalised rows are the bits of the separate form, and the head's launches are nodes of the step's captured graph (captured
+ * again when weight, bias, dev_logits or dev_probs differ from the step before: keep them stable).  Elsewhere the two calls run
+ * one after the other.  A step of this
  * entry whose bounded wait gives up is reported at the next synchronising call and not repeated (its rows have been consumed). */
 int mynah_hip_decoder_step_head(void *state, mynah_hip_decoder *decoder, const mynah_hip_decoder_slot *slots, size_t batch,
                                 const float *weight, const float *bias, size_t rows, size_t vocab, float *const *dev_logits,

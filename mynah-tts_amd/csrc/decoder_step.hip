@@ -63,8 +63,12 @@ struct mynah_hip_decoder {
     bool fused_attention = false;
     // [with the end kernel or without it][stream count]: this lane's layer kernels as one chain of kernel nodes (without the
     // end kernel: the step whose final LayerNorm the output head's product does, mynah_hip_decoder_step_head)
-    hipGraphExec_t graphs[2][mynah::kMaxBatch + 1] = {};
-    int eager_steps[2][mynah::kMaxBatch + 1] = {};   // a stream count runs eagerly once before it is captured
+    // forms: 0 the layers and the end kernel, 1 the layers alone, 2 the layers and the output head of HeadCall (its pointers are
+    // part of the captured nodes: head_signature says whose they are, and the graph is captured again when they change)
+    hipGraphExec_t graphs[3][mynah::kMaxBatch + 1] = {};
+    int eager_steps[3][mynah::kMaxBatch + 1] = {};   // a stream count runs eagerly once before it is captured
+    unsigned long long head_signature[mynah::kMaxBatch + 1] = {};
+    int head_recaptures = 0;
     hipGraphExec_t stage_graphs[MYNAH_HIP_STAGE_COUNT][mynah::kMaxBatch + 1] = {};   // single-stage graphs (measurement only)
     int arith = 0;
     // Lanes: a batch above two streams is cut into groups that step side by side, each on a stream of its own with
@@ -646,21 +650,57 @@ static StepSlots lane_slots(const StepSlots &s, const LanePlan &p, int lane) {
 // kernel attribute set-up does not belong in a capture) and in graph mode 0, else as the lane's captured graph of that count.
 // A graph is a single chain of kernel nodes -- the form the runtime replays without touching each node on the host; one
 // graph with a branch per lane was measured at 4.2 us of host time per node, 670 us for the two chains of a batch of eight.
-static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t stream, char *error, size_t capacity, bool with_end = true) {
+// The output head that follows a step in the same call (mynah_hip_decoder_step_head): with one lane it is enqueued behind the
+// layers inside the lane's graph, two dependent graph nodes instead of two launches behind the graph.
+struct HeadCall {
+    const float *weight, *bias;
+    size_t rows, vocab;
+    float *const *dlogits;
+    float *const *dprobs;
+};
+static unsigned long long head_signature_of(const HeadCall &h, int count) {
+    unsigned long long x = 0xcbf29ce484222325ull;
+    const auto mix = [&](unsigned long long v) { x = (x ^ v) * 0x100000001b3ull; };
+    mix(reinterpret_cast<unsigned long long>(h.weight)); mix(reinterpret_cast<unsigned long long>(h.bias)); mix(h.rows); mix(h.vocab);
+    for (int b = 0; b < count; ++b) {
+        mix(reinterpret_cast<unsigned long long>(h.dlogits[b]));
+        mix(h.dprobs != nullptr ? reinterpret_cast<unsigned long long>(h.dprobs[b]) : 0ull);
+    }
+    return x | 1ull;   // never 0
+}
+static int enqueue_head(State *st, mynah_hip_decoder *d, int count, const HeadCall &h, char *error, size_t capacity) {
+    const float *hidden[kMaxBatch] = {};   // (not read: the product takes the residual rows and normalises them itself)
+    return output_head_rows(st, hidden, (size_t)count, d->width, h.weight, h.bias, h.rows, h.vocab, h.dlogits, h.dprobs, d->x, d->norm_out, d->norm_out_b,
+                            error, capacity, d->dev_slots);
+}
+
+static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t stream, char *error, size_t capacity, bool with_end = true,
+                    const HeadCall *head = nullptr) {
     hipStream_t main_stream = st->stream;
     st->stream = stream;   // the launch wrappers enqueue on the state's stream
     int rc = 0;
-    const int form = with_end ? 0 : 1;
+    const int form = head != nullptr ? 2 : with_end ? 0 : 1;
+    const auto enqueue = [&]() {
+        int r = enqueue_layers(st, lane, count, error, capacity, kAllStages, with_end);
+        if (r == 0 && head != nullptr) r = enqueue_head(st, lane, count, *head, error, capacity);
+        return r;
+    };
+    if (head != nullptr && lane->graphs[2][count] != nullptr && lane->head_signature[count] != head_signature_of(*head, count)) {
+        (void)hipGraphExecDestroy(lane->graphs[2][count]);   // another head, or other rows for its results: captured again
+        lane->graphs[2][count] = nullptr;
+        ++lane->head_recaptures;
+    }
     if (st->graph_mode == 0 || lane->eager_steps[form][count] == 0) {
         lane->eager_steps[form][count] = 1;
-        rc = enqueue_layers(st, lane, count, error, capacity, kAllStages, with_end);
+        rc = enqueue();
     } else {
         hipGraphExec_t &exec = lane->graphs[form][count];
         if (exec == nullptr) {
             hipGraph_t graph = nullptr;
             rc = hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal), "begin capture", error, capacity);
             if (rc == 0) {
-                rc = enqueue_layers(st, lane, count, error, capacity, kAllStages, with_end);
+                if (head != nullptr) lane->head_signature[count] = head_signature_of(*head, count);
+                rc = enqueue();
                 const hipError_t end = hipStreamEndCapture(stream, &graph);
                 if (rc == 0) rc = hip_check(end, "end capture", error, capacity);
                 if (rc == 0) rc = hip_check(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "graph instantiate", error, capacity);
@@ -675,7 +715,8 @@ static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t s
 }
 
 // Every lane of a step: lane 0 on the backend's stream, the others on theirs, forked from and joined to it by events.
-static int run_lanes(State *st, mynah_hip_decoder *d, const LanePlan &p, char *error, size_t capacity, bool with_end = true) {
+static int run_lanes(State *st, mynah_hip_decoder *d, const LanePlan &p, char *error, size_t capacity, bool with_end = true,
+                     const HeadCall *head = nullptr) {
     hipStream_t main_stream = st->stream;
     if (p.lanes > 1) {
         MYNAH_TRY(hipEventRecord(st->lane_fork, main_stream));
@@ -683,7 +724,7 @@ static int run_lanes(State *st, mynah_hip_decoder *d, const LanePlan &p, char *e
     }
     int rc = 0;
     for (int i = p.lanes - 1; i >= 0 && rc == 0; --i) {   // the owner's lane last: its stream is the one the caller's next work queues behind
-        rc = run_lane(st, d->lanes[i], p.count[i], i == 0 ? main_stream : st->lane_streams[i], error, capacity, with_end);
+        rc = run_lane(st, d->lanes[i], p.count[i], i == 0 ? main_stream : st->lane_streams[i], error, capacity, with_end, p.lanes == 1 ? head : nullptr);
         if (i > 0 && rc == 0) rc = hip_check(hipEventRecord(st->lane_done[i], st->lane_streams[i]), "lane event", error, capacity);
     }
     for (int i = 1; i < p.lanes && rc == 0; ++i) rc = hip_check(hipStreamWaitEvent(main_stream, st->lane_done[i], 0), "lane join", error, capacity);
@@ -709,9 +750,12 @@ int decoder_next_epochs(State *st, mynah_hip_decoder *d, unsigned count, unsigne
 
 // The step, with its end kernel (the final LayerNorm into every slot's output) or -- one lane, no persistent form -- without:
 // *ended says which it was.
+// head (optional): the output head to run behind the step; *head_done says whether the step took it along (one lane of stage
+// kernels without the end kernel: the head is then part of the lane's graph), else the caller runs it.
 static int decoder_step(State *st, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch, bool want_end, bool *ended, char *error,
-                        size_t capacity) {
+                        size_t capacity, const HeadCall *head = nullptr, bool *head_done = nullptr) {
     *ended = true;
+    if (head_done != nullptr) *head_done = false;
     if (batch == 0) return 0;   // src/graph.c:3132
     if (batch > (size_t)kMaxBatch) {
         set_error(error, capacity, "decoder batch exceeds MYNAH_MAX_BATCH");   // src/graph.c:3133-3136
@@ -761,6 +805,10 @@ static int decoder_step(State *st, mynah_hip_decoder *d, const mynah_hip_decoder
     if (ensure_lanes(st, d, lanes, error, capacity) != 0) return -1;
     const bool with_end = want_end || lanes != 1 || !d->fused_attention;
     *ended = with_end;
+    // (a caller that hands over other rows for the results at every step would have the graph captured at every step)
+    static const bool head_in_graph = !(getenv("MYNAH_HIP_HEAD_IN_GRAPH") != nullptr && strcmp(getenv("MYNAH_HIP_HEAD_IN_GRAPH"), "0") == 0);
+    const bool head_along = head_in_graph && head != nullptr && !with_end && head_done != nullptr && d->head_recaptures < 8;
+    if (head_along) *head_done = true;
     const LanePlan plan = plan_lanes(s, B, lanes);
     d->last_batch_slots = s;
     d->last_lanes = lanes;
@@ -774,7 +822,7 @@ static int decoder_step(State *st, mynah_hip_decoder *d, const mynah_hip_decoder
                               capacity) != 0)
             return -1;
     }
-    return run_lanes(st, d, plan, error, capacity, with_end);
+    return run_lanes(st, d, plan, error, capacity, with_end, head_along ? head : nullptr);
 }
 
 extern "C" int mynah_hip_decoder_step(void *opaque, mynah_hip_decoder *d, const mynah_hip_decoder_slot *slots, size_t batch,
@@ -803,8 +851,13 @@ extern "C" int mynah_hip_decoder_step_head(void *opaque, mynah_hip_decoder *d, c
     for (size_t b = 0; b < batch; ++b) hidden[b] = slots[b].dev_output;
     // (the fused form's product takes one weight pass and the matvec's shapes; the decision must precede the step)
     const bool fusable = batch <= (size_t)kBatchTile && d->norm_out != nullptr && linear_fast_supported(st->qtype, rows, d->width) && rows <= 0x7fffffffu;
-    bool ended = true;
-    if (decoder_step(st, d, slots, batch, !fusable, &ended, error, capacity) != 0) return -1;
+    bool ended = true, head_done = false;
+    const HeadCall head{weight, bias, rows, vocab, dlogits, dprobs};
+    if (decoder_step(st, d, slots, batch, !fusable, &ended, error, capacity, fusable ? &head : nullptr, &head_done) != 0) return -1;
+    if (head_done) {
+        st->last_step_decoder = nullptr;   // (not repeatable behind the head)
+        return 0;
+    }
     if (ended) return output_head_rows(st, hidden, batch, d->width, weight, bias, rows, vocab, dlogits, dprobs, nullptr, nullptr, nullptr, error, capacity);
     st->last_step_decoder = nullptr;   // (not repeatable behind the head)
     return output_head_rows(st, hidden, batch, d->width, weight, bias, rows, vocab, dlogits, dprobs, d->x, d->norm_out, d->norm_out_b, error, capacity,

@@ -700,7 +700,8 @@ def test_long_cache_takes_the_fold_kernel(pkg, backend, orc, synth, nerr):
 def test_step_and_head_in_one_call(pkg, backend, synth, nerr, qtype_name, batch):
     """mynah_hip_decoder_step_head against mynah_hip_decoder_step followed by mynah_hip_output_head on the same streams: the
     slots' outputs (the final-normed rows), the appended cache rows, logits and probabilities, all bit for bit -- the head
-    product's LayerNorm prologue forms its sums as the end kernel does; three steps in a row (eager, captured, replayed);
+    product's LayerNorm prologue forms its sums as the end kernel does; five steps in a row (eager, captured, replayed, and two
+    with other rows for the results: the head travels in the step's graph, which is captured again for them);
     eleven streams take the two-call form inside the library (two lanes)."""
     _announce("step + head in one call %s b=%d" % (qtype_name, batch))
     rng = np.random.default_rng(11)
@@ -713,9 +714,10 @@ def test_step_and_head_in_one_call(pkg, backend, synth, nerr, qtype_name, batch)
     head_b = (rng.standard_normal(2 * 256) * 0.1).astype(np.float32)
     backend.set_quant(QT[qtype_name])
     h = Harness(pkg, backend, cfg, weights, streams)
-    dl = [backend.alloc(512) for _ in range(batch)]
-    dp = [backend.alloc(512) for _ in range(batch)]
-    for step in range(3):
+    first = [backend.alloc(512) for _ in range(2 * batch)]
+    other = [backend.alloc(512) for _ in range(2 * batch)]
+    for step in range(5):
+        dl, dp = (first[:batch], first[batch:]) if step < 3 else (other[:batch], other[batch:])
         for i in range(batch):
             h.reset_cache(i)
         rows = h.step()
@@ -737,7 +739,7 @@ def test_step_and_head_in_one_call(pkg, backend, synth, nerr, qtype_name, batch)
             gl, gp = dl[i].read(), dp[i].read()
             assert np.array_equal(gl.view(np.uint32), want_logits[i].view(np.uint32)), "step %d stream %d: logits" % (step, i)
             assert np.array_equal(gp.view(np.uint32), want_probs[i].view(np.uint32)), "step %d stream %d: probabilities" % (step, i)
-    for d in dl + dp:
+    for d in first + other:
         d.free()
     h.close()
     backend.set_quant(0)
