@@ -277,11 +277,16 @@ STAGES = [("self-attention", "k_step_attention<self>", "LayerNorm + int8 act-qua
           ("ffn-up", "k_linear<k=768, LayerNorm, GELU>", "LayerNorm + act-quant + up matvec + GELU"),
           ("ffn-down", "k_linear<k=3072, residual>", "act-quant + down matvec + residual")]
 
-# HBM bytes per launch of the dominant kernel of the batch-1 int8 line, from two rocprofv3 --pmc runs (FETCH_SIZE, then
-# WRITE_SIZE), each scaled by what the same counter reads for the library's plain 256 MiB read+write kernel.  The figure
+# HBM bytes per launch of the dominant kernels of the batch-1 and batch-8 int8 lines, from two rocprofv3 --pmc runs (FETCH_SIZE,
+# then WRITE_SIZE), each scaled by what the same counter reads for the library's plain 256 MiB read+write kernel.  A figure
 # belongs to the kernel sources it was measured on: it is reported only while their hash is the one recorded here.
-MEASURED_TRAFFIC = {"kernel": "k_linear<k=768, residual>", "bytes": 937914, "profile": "profiles/decode_step_int8_hbm_counters.md",
-                    "csrc_sha256": "b24c335f5817caf8"}
+MEASURED_TRAFFIC = {
+    1: {"kernel": "k_linear<k=768, residual>", "bytes": 937914, "profile": "profiles/decode_step_int8_hbm_counters.md",
+        "sources": ("kernels_linear.hip", "device_common.h", "kernels.h", "common.h"), "csrc_sha256": "b24c335f5817caf8"},
+    8: {"kernel": "k_step_attention<self>", "bytes": 54473544, "profile": "profiles/decode_step_int8_hbm_counters.md",
+        "sources": ("kernels_step_attention.hip", "step_attention_core.h", "step_items.h", "tagged_exchange.h", "device_common.h",
+                    "kernels.h", "common.h"), "csrc_sha256": "80f36709dc78482e"},
+}
 
 
 def latency_floor(backend, step_us, launches):
@@ -300,14 +305,10 @@ def latency_floor(backend, step_us, launches):
             "node_us_two_chains_side_by_side": round(two, 3), "node_us_three_chains_side_by_side": round(three, 3)}
 
 
-# the sources the roofline kernel (the fused matvec) is built from: its counter figure stands for exactly these
-TRAFFIC_SOURCES = ("kernels_linear.hip", "device_common.h", "kernels.h", "common.h")
-
-
-def csrc_hash():
+def csrc_hash(sources):
     import hashlib
     h = hashlib.sha256()
-    for name in TRAFFIC_SOURCES:
+    for name in sources:
         with open(os.path.join(ROOT, "mynah-tts_amd", "csrc", name), "rb") as f:
             h.update(name.encode())
             h.update(f.read())
@@ -334,12 +335,11 @@ def roofline(r):
     kernel, launch_us, nbytes = name, g["us"] / g["launches"], g["bytes"] // g["launches"]
     share = g["us"] * r["layers"] / r["step_us"]
     gbps = nbytes / (launch_us * 1e-6) / 1e9
-    traffic = None
-    if (r.get("traffic_valid") and MEASURED_TRAFFIC["bytes"] is not None and MEASURED_TRAFFIC["kernel"] == kernel and
-            MEASURED_TRAFFIC["csrc_sha256"] == csrc_hash()):
-        traffic = MEASURED_TRAFFIC["bytes"]
+    traffic, measured = None, MEASURED_TRAFFIC.get(r.get("traffic_batch"))
+    if measured is not None and measured["kernel"] == kernel and measured["csrc_sha256"] == csrc_hash(measured["sources"]):
+        traffic = measured["bytes"]
     return {"bound": "hbm", "kernel": kernel, "achieved": round(gbps, 1), "peak": PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / PEAK_GBPS, 4),
-            "traffic": traffic, "traffic_source": MEASURED_TRAFFIC["profile"] if traffic is not None else None,
+            "traffic": traffic, "traffic_source": measured["profile"] if traffic is not None else None,
             "launch_us": round(launch_us, 3), "algorithmic_bytes_per_launch": nbytes, "share_of_step": round(share, 3),
             "launches_per_step": g["launches"] * r["layers"], "stages": rows,
             "whole_step": {"step_us": round(r["step_us"], 2), "algorithmic_bytes_per_step": r["bytes"], "weight_bytes": r["weight_bytes"],
@@ -413,7 +413,7 @@ def main():
         backend.sync()
 
     b1 = time_config(pkg, synth, backend, qtype, [1023], [256], 1024, args.steps, args.warmup)
-    b1["traffic_valid"] = args.quant == "int8"
+    b1["traffic_batch"] = 1 if args.quant == "int8" else None
     # dependent launches of a step: six stages a layer, begin, the head product (which also does the final LayerNorm), its softmax
     floor = None if args.launches else latency_floor(backend, b1["step_us"], 6 * b1["layers"] + 3)
     int4 = None
@@ -426,6 +426,7 @@ def main():
         b8 = time_config(pkg, synth, backend, qtype, [n - 1 for n in self_len], cross_len, 2048, max(args.steps // 3, 20),
                          max(args.warmup // 3, 6), rotate=ROTATE)
         b8["self_lengths"], b8["cross_lengths"] = self_len, cross_len
+        b8["traffic_batch"] = 8 if args.quant == "int8" else None   # the counters were taken on these ragged lengths
     prefill = None if args.skip_prefill else time_prefill(pkg, synth, backend)
     local = None if args.skip_local else [time_local(pkg, synth, backend, qtype, b) for b in (1, 8)]
     codec = None if args.skip_codec else time_codec(pkg, backend)
