@@ -658,9 +658,10 @@ struct HeadCall {
     float *const *dlogits;
     float *const *dprobs;
 };
-static unsigned long long head_signature_of(const HeadCall &h, int count) {
+static unsigned long long head_signature_of(const State *st, const HeadCall &h, int count) {
     unsigned long long x = 0xcbf29ce484222325ull;
     const auto mix = [&](unsigned long long v) { x = (x ^ v) * 0x100000001b3ull; };
+    mix((unsigned long long)st->qtype);   // the storage the head's weight is looked up under
     mix(reinterpret_cast<unsigned long long>(h.weight)); mix(reinterpret_cast<unsigned long long>(h.bias)); mix(h.rows); mix(h.vocab);
     for (int b = 0; b < count; ++b) {
         mix(reinterpret_cast<unsigned long long>(h.dlogits[b]));
@@ -685,10 +686,19 @@ static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t s
         if (r == 0 && head != nullptr) r = enqueue_head(st, lane, count, *head, error, capacity);
         return r;
     };
-    if (head != nullptr && lane->graphs[2][count] != nullptr && lane->head_signature[count] != head_signature_of(*head, count)) {
-        (void)hipGraphExecDestroy(lane->graphs[2][count]);   // another head, or other rows for its results: captured again
-        lane->graphs[2][count] = nullptr;
-        ++lane->head_recaptures;
+    if (head != nullptr) {
+        // another head, or other rows for its results, than this stream count's last step had: captured again, behind one
+        // eager step (a weight seen for the first time is converted and uploaded there: no part of a capture)
+        const unsigned long long signature = head_signature_of(st, *head, count);
+        if (lane->head_signature[count] != signature) {
+            if (lane->graphs[2][count] != nullptr) {
+                (void)hipGraphExecDestroy(lane->graphs[2][count]);
+                lane->graphs[2][count] = nullptr;
+            }
+            if (lane->head_signature[count] != 0) ++lane->head_recaptures;
+            lane->eager_steps[2][count] = 0;
+            lane->head_signature[count] = signature;
+        }
     }
     if (st->graph_mode == 0 || lane->eager_steps[form][count] == 0) {
         lane->eager_steps[form][count] = 1;
@@ -699,7 +709,6 @@ static int run_lane(State *st, mynah_hip_decoder *lane, int count, hipStream_t s
             hipGraph_t graph = nullptr;
             rc = hip_check(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal), "begin capture", error, capacity);
             if (rc == 0) {
-                if (head != nullptr) lane->head_signature[count] = head_signature_of(*head, count);
                 rc = enqueue();
                 const hipError_t end = hipStreamEndCapture(stream, &graph);
                 if (rc == 0) rc = hip_check(end, "end capture", error, capacity);

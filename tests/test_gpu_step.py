@@ -700,8 +700,10 @@ def test_long_cache_takes_the_fold_kernel(pkg, backend, orc, synth, nerr):
 def test_step_and_head_in_one_call(pkg, backend, synth, nerr, qtype_name, batch):
     """mynah_hip_decoder_step_head against mynah_hip_decoder_step followed by mynah_hip_output_head on the same streams: the
     slots' outputs (the final-normed rows), the appended cache rows, logits and probabilities, all bit for bit -- the head
-    product's LayerNorm prologue forms its sums as the end kernel does; five steps in a row (eager, captured, replayed, and two
-    with other rows for the results: the head travels in the step's graph, which is captured again for them);
+    product's LayerNorm prologue forms its sums as the end kernel does; eight steps in a row: eager, captured, replayed; the
+    same three with other rows for the results (the head travels in the step's graph, whose nodes hold its pointers: one eager
+    step, then captured again); and two with a head whose weight the library has not seen before (converted and uploaded in
+    the eager step, outside any capture);
     eleven streams take the two-call form inside the library (two lanes)."""
     _announce("step + head in one call %s b=%d" % (qtype_name, batch))
     rng = np.random.default_rng(11)
@@ -710,35 +712,42 @@ def test_step_and_head_in_one_call(pkg, backend, synth, nerr, qtype_name, batch)
     cfg = synth.decoder_config(layers=2, capacity=304)
     weights = synth.decoder_weights(cfg, seed=0)
     streams = synth.decoder_streams(cfg, lengths, mems, seed=1)
-    head_w = (rng.standard_normal((2 * 256, cfg["width"])) * 0.02).astype(np.float32)
-    head_b = (rng.standard_normal(2 * 256) * 0.1).astype(np.float32)
+    first_w = (rng.standard_normal((2 * 256, cfg["width"])) * 0.02).astype(np.float32)
+    first_b = (rng.standard_normal(2 * 256) * 0.1).astype(np.float32)
     backend.set_quant(QT[qtype_name])
     h = Harness(pkg, backend, cfg, weights, streams)
+    later_w = (rng.standard_normal((2 * 256, cfg["width"])) * 0.02).astype(np.float32)
+    later_b = (rng.standard_normal(2 * 256) * 0.1).astype(np.float32)
     first = [backend.alloc(512) for _ in range(2 * batch)]
     other = [backend.alloc(512) for _ in range(2 * batch)]
-    for step in range(5):
-        dl, dp = (first[:batch], first[batch:]) if step < 3 else (other[:batch], other[batch:])
+    for step in range(8):
+        dl, dp = (other[:batch], other[batch:]) if 3 <= step < 6 else (first[:batch], first[batch:])
+        head_w, head_b = (later_w, later_b) if step >= 6 else (first_w, first_b)
+        def two_calls():
+            for i in range(batch):
+                h.reset_cache(i)
+            rows = h.step()
+            backend.output_head([b["out"].ptr for b in h.bufs], cfg["width"], head_w, head_b, 512, 256, [d.ptr for d in dl], [d.ptr for d in dp])
+            return rows, [d.read() for d in dl], [d.read() for d in dp], [h.cache_rows(i) for i in range(batch)]
+
+        def one_call():
+            for i in range(batch):
+                h.reset_cache(i)
+                h.bufs[i]["out"].write(np.zeros(cfg["width"], np.float32))
+                dl[i].write(np.zeros(512, np.float32))
+                dp[i].write(np.zeros(512, np.float32))
+            h.dec.step_head(h.slots(), head_w, head_b, 512, 256, [d.ptr for d in dl], [d.ptr for d in dp])
+            return [b["out"].read() for b in h.bufs], [d.read() for d in dl], [d.read() for d in dp], [h.cache_rows(i) for i in range(batch)]
+
+        if step == 6:   # the new head's first sight is the one-call form's
+            got, want = one_call(), two_calls()
+        else:
+            want, got = two_calls(), one_call()
         for i in range(batch):
-            h.reset_cache(i)
-        rows = h.step()
-        backend.output_head([b["out"].ptr for b in h.bufs], cfg["width"], head_w, head_b, 512, 256, [d.ptr for d in dl], [d.ptr for d in dp])
-        want_logits = [d.read() for d in dl]
-        want_probs = [d.read() for d in dp]
-        want_cache = [h.cache_rows(i) for i in range(batch)]
-        for i in range(batch):
-            h.reset_cache(i)
-            h.bufs[i]["out"].write(np.zeros(cfg["width"], np.float32))
-            dl[i].write(np.zeros(512, np.float32))
-            dp[i].write(np.zeros(512, np.float32))
-        h.dec.step_head(h.slots(), head_w, head_b, 512, 256, [d.ptr for d in dl], [d.ptr for d in dp])
-        got_rows = [b["out"].read() for b in h.bufs]
-        for i in range(batch):
-            assert np.array_equal(got_rows[i].view(np.uint32), rows[i].view(np.uint32)), "step %d stream %d: output row" % (step, i)
-            gk, gv = h.cache_rows(i)
-            assert np.array_equal(gk, want_cache[i][0]) and np.array_equal(gv, want_cache[i][1]), "step %d stream %d: cache" % (step, i)
-            gl, gp = dl[i].read(), dp[i].read()
-            assert np.array_equal(gl.view(np.uint32), want_logits[i].view(np.uint32)), "step %d stream %d: logits" % (step, i)
-            assert np.array_equal(gp.view(np.uint32), want_probs[i].view(np.uint32)), "step %d stream %d: probabilities" % (step, i)
+            assert np.array_equal(got[0][i].view(np.uint32), want[0][i].view(np.uint32)), "step %d stream %d: output row" % (step, i)
+            assert np.array_equal(got[3][i][0], want[3][i][0]) and np.array_equal(got[3][i][1], want[3][i][1]), "step %d stream %d: cache" % (step, i)
+            assert np.array_equal(got[1][i].view(np.uint32), want[1][i].view(np.uint32)), "step %d stream %d: logits" % (step, i)
+            assert np.array_equal(got[2][i].view(np.uint32), want[2][i].view(np.uint32)), "step %d stream %d: probabilities" % (step, i)
     for d in first + other:
         d.free()
     h.close()
