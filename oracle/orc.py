@@ -660,6 +660,20 @@ class RefDecoder:
             raise RuntimeError(err.value.decode())
         return out, int(n.value), bool(resident.value)
 
+    def run_rows(self, slot, self_k, self_v, cross_k, cross_v, length, memory_length, rows):
+        """The reference's decoder_run with several rows, its context prefill (src/graph.c:3506-3654): the host caches are
+        appended in place; returns (the last row after the final norm, new length)."""
+        rows = np.ascontiguousarray(rows, np.float32)
+        out = np.empty(self.cfg["width"], np.float32)
+        n = _sz(length)
+        err = C.create_string_buffer(512)
+        self.r.ref_decoder_run_rows.restype = C.c_int
+        rc = self.r.ref_decoder_run_rows(C.c_void_p(self.h), _sz(slot), _ptr(self_k), _ptr(self_v), _ptr(cross_k), _ptr(cross_v),
+                                         C.byref(n), _sz(memory_length), _ptr(rows), _sz(rows.shape[0]), _ptr(out), err, _sz(512))
+        if rc != 0:
+            raise RuntimeError(err.value.decode())
+        return out, int(n.value)
+
     def device_kv_row(self, slot, layer, row):
         k = np.empty(self.cfg["width"], np.float32)
         v = np.empty(self.cfg["width"], np.float32)

@@ -410,6 +410,45 @@ int ref_decoder_run_one(ref_decoder *d, size_t slot, float *self_k, float *self_
     return rc;
 }
 
+/* A decoder_run of `count` > 1 rows of slot `slot` (the context prefill, src/graph.c:3506-3654): the projections go to the
+ * backend as host-pointer products of `count` rows (or to the quantised CPU path when the cache is on and count <= 16,
+ * src/qmat.c:768-818), self-attention as two sgemm calls per head (:3532-3545); the host caches are appended in place.  The
+ * slot's one-row scratch is replaced by buffers of `count` rows for the call (decoder_cache_init sizes them so, :3086-3105). */
+int ref_decoder_run_rows(ref_decoder *d, size_t slot, float *self_k, float *self_v, float *cross_k, float *cross_v,
+                         size_t *length, size_t memory_length, const float *input_rows, size_t count, float *out_last,
+                         char *error, size_t error_capacity) {
+    if (slot >= d->batch || count < 2) return -1;
+    decoder_cache *c = &d->caches[slot];
+    const decoder_cache saved = *c;
+    const size_t w = c->width, f = c->ffn_width, xw = c->xattn_width;
+    const size_t score_len = c->capacity > memory_length ? c->capacity : memory_length;
+    float *bufs[11] = {0};
+    const size_t sizes[11] = {count * w, count * w, count * 3u * w, count * w, count * w, count * xw, count * xw, count * f,
+                              score_len + 1u, count * c->capacity, count * c->head_width};
+    int rc = -1;
+    for (int i = 0; i < 11; ++i) {
+        bufs[i] = (float *)calloc(sizes[i], sizeof(float));
+        if (bufs[i] == NULL) { graph_error(error, error_capacity, "out of memory"); goto done; }
+    }
+    c->scratch_rows = count;
+    c->scratch_x = bufs[0]; c->scratch_nrm = bufs[1]; c->scratch_qkv = bufs[2]; c->scratch_attn = bufs[3];
+    c->scratch_proj = bufs[4]; c->scratch_q_x = bufs[5]; c->scratch_xctx = bufs[6]; c->scratch_hidden = bufs[7];
+    c->scratch_scores = bufs[8]; c->scratch_score_matrix = bufs[9]; c->scratch_head_ctx = bufs[10];
+    c->self_k = self_k; c->self_v = self_v; c->cross_k = cross_k; c->cross_v = cross_v;
+    c->length = *length;
+    c->memory_length = memory_length;
+    rc = decoder_run(&d->model, c, input_rows, count, out_last, NULL, error, error_capacity);
+    *length = c->length;
+done:
+    {
+        const size_t new_length = c->length;
+        *c = saved;               /* the one-row scratch again; the call leaves no device state behind */
+        c->length = new_length;
+    }
+    for (int i = 0; i < 11; ++i) free(bufs[i]);
+    return rc;
+}
+
 /* Row `row` of layer `layer` of the slot's device K and V caches, through the backend's own d2h. */
 int ref_decoder_read_device_kv(ref_decoder *d, size_t slot, size_t layer, size_t row, float *k_row, float *v_row,
                                char *error, size_t error_capacity) {

@@ -104,6 +104,54 @@ def test_decoder_run_resident_path(pkg, orc, ref_strict, synth, nerr, quant_env,
 
 
 @pytest.mark.parametrize("qtype_name", ["f32", "int8"])
+def test_decoder_run_prefill_then_resident_steps(pkg, orc, ref_strict, synth, nerr, quant_env, qtype_name):
+    """decoder_run with 24 rows at once -- the reference's context prefill (src/graph.c:3506-3654) -- on the library and
+    on the CPU backend: with more than sixteen rows every projection is a host-pointer f32 product of 24 rows through the
+    backend's `matmul`, and self-attention two `sgemm` calls per head (QK^T over the rows the cache already holds plus the
+    new ones, then PV), so this is the seam's many-row side as the engine drives it.  Then two single-row calls per stream,
+    which on the library upload the prefilled host caches once and continue resident."""
+    _announce("engine: decoder_run prefill of 24 rows, then resident steps, %s" % qtype_name)
+    qtype = QT[qtype_name]
+    tol = TOL[qtype_name]
+    lengths, mems = [0, 6], [9, 19]
+    rows, steps = 24, 2
+    cfg = synth.decoder_config(layers=2, capacity=max(lengths) + rows + steps + 1, cross_heads=1)
+    w = synth.decoder_weights(cfg, seed=0, ln_bias=False)
+    streams = synth.decoder_streams(cfg, lengths, mems, seed=7)
+    rng = np.random.default_rng(8)
+    prompts = [rng.standard_normal((rows, cfg["width"])).astype(np.float32) for _ in streams]
+    xs = [[rng.standard_normal(cfg["width"]).astype(np.float32) for _ in range(steps)] for _ in streams]
+
+    quant_env(qtype_name)
+    cpu = orc.RefDecoder(cfg, w, qtype, len(streams), max(mems), strict=True)
+    hip = orc.RefDecoder(cfg, w, qtype, len(streams), max(mems), strict=True)
+    hip.use_hip(pkg.LIB_PATH)
+    try:
+        for slot, s in enumerate(streams):
+            ck, cv = s["k"].copy(), s["v"].copy()
+            hk, hv = s["k"].copy(), s["v"].copy()
+            want, clen = cpu.run_rows(slot, ck, cv, s["ck"], s["cv"], s["length"], s["memory_length"], prompts[slot])
+            got, hlen = hip.run_rows(slot, hk, hv, s["ck"], s["cv"], s["length"], s["memory_length"], prompts[slot])
+            assert hlen == clen == s["length"] + rows
+            e = nerr(got, want)
+            assert e < 1e-5, "stream %d prefill: %.3g" % (slot, e)   # f32 products on both sides whatever the weight storage
+            new = slice(s["length"], s["length"] + rows)
+            for layer in range(cfg["layers"]):
+                assert nerr(hk[layer, new], ck[layer, new]) < 1e-5 and nerr(hv[layer, new], cv[layer, new]) < 1e-5
+            assert np.array_equal(hk[:, :s["length"]], s["k"][:, :s["length"]])
+            for t in range(steps):
+                want, clen, _ = cpu.run_one(slot, ck, cv, s["ck"], s["cv"], clen, s["memory_length"], xs[slot][t])
+                got, hlen, resident = hip.run_one(slot, hk, hv, s["ck"], s["cv"], hlen, s["memory_length"], xs[slot][t])
+                assert resident, "the engine fell back to its CPU path"
+                assert hlen == clen == s["length"] + rows + t + 1
+                e = nerr(got, want)
+                assert e < tol, "stream %d step %d after the prefill: %.3g" % (slot, t, e)
+    finally:
+        hip.close()
+        cpu.close()
+
+
+@pytest.mark.parametrize("qtype_name", ["f32", "int8"])
 def test_local_step_device(pkg, orc, ref_strict, synth, nerr, quant_env, qtype_name):
     """Four positions of the local transformer: the reference's local_step_device on the library against its
     local_step_batch on the CPU backend.  The engine passes the position row, a pointer into host weight memory, in a
