@@ -775,16 +775,17 @@ def write_safetensors(path, tensors):
             f.write(blob)
 
 
-def ref_transformer_stack(cfg, w, states, kernel, strict=False, workdir=None):
+def ref_transformer_stack(cfg, w, states, kernel, strict=False, workdir=None, hip_library=None):
     """The compiled reference's transformer_stack (src/graph.c:634-711) exactly as encode_text calls it (:738-740):
     causal self-attention, gain-only LayerNorm, FFN with `kernel` taps, final norm when w["norm_out_g"] is given.
     w holds f32 arrays: pos_table [P, width], qkv [L, 3w, w], o [L, w, w], up [L, ffn, w(, kernel)],
-    down [L, w, ffn(, kernel)], norm1_g / norm2_g [L, w].  states: the gathered token rows [T, width]."""
+    down [L, w, ffn(, kernel)], norm1_g / norm2_g [L, w].  states: the gathered token rows [T, width].
+    hip_library: the same function on the reference's backend struct filled with that library's entry points."""
     import tempfile
     r = load_ref(strict)
     fp = C.POINTER(C.c_float)
-    r.ref_transformer_stack.argtypes = [C.c_char_p, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int, fp, fp, C.c_char_p, _sz]
-    r.ref_transformer_stack.restype = C.c_int
+    r.ref_transformer_stack_on.argtypes = [C.c_char_p, C.c_char_p, _sz, _sz, _sz, _sz, _sz, _sz, C.c_int, fp, fp, C.c_char_p, _sz]
+    r.ref_transformer_stack_on.restype = C.c_int
     L, width, ffn = cfg["layers"], cfg["width"], cfg["ffn"]
     tensors = {"encoder.position_embeddings.weight": w["pos_table"]}
     for l in range(L):
@@ -805,8 +806,8 @@ def ref_transformer_stack(cfg, w, states, kernel, strict=False, workdir=None):
     with tempfile.TemporaryDirectory(dir=workdir) as tmp:
         path = os.path.join(tmp, "encoder.safetensors")
         write_safetensors(path, tensors)
-        rc = r.ref_transformer_stack(os.fsencode(path), L, T, width, ffn, cfg["heads"], kernel, 1 if final else 0,
-                                     states.ctypes.data_as(fp), out.ctypes.data_as(fp), err, 512)
+        rc = r.ref_transformer_stack_on(os.fsencode(path), None if hip_library is None else os.fsencode(hip_library), L, T, width, ffn,
+                                        cfg["heads"], kernel, 1 if final else 0, states.ctypes.data_as(fp), out.ctypes.data_as(fp), err, 512)
     if rc != 0:
         raise RuntimeError(err.value.decode())
     return out

@@ -314,15 +314,22 @@ int ref_snake(float *data, const float *alpha, size_t channels, size_t length, s
  *                                                  backend, with `kernel` 1 (plain FFN) or 3 (the model's conv FFN).
  * Weights are looked up by name ("encoder....") in a safetensors file the caller wrote itself (synthetic tensors).
  * `states` are the gathered token rows [length, width]; `output` receives [length, width]. */
-int ref_transformer_stack(const char *weights_path, size_t layers, size_t length, size_t width, size_t ffn_width,
-                          size_t heads, size_t kernel, int apply_norm_out, const float *states, float *output, char *error,
-                          size_t error_capacity) {
+mynah_backend *ref_backend_open_hip(const char *library_path, char *error, size_t error_capacity);
+
+/* hip_library NULL: the CPU backend; else the reference's backend struct filled with that library's entry points
+ * (ref_shim_backend.c): every product of the stack is then a host-pointer `matmul` (the `linear` calls) or `sgemm`
+ * (QK^T and PV per head, the unfolded conv FFN) of `length` rows through the seam. */
+int ref_transformer_stack_on(const char *weights_path, const char *hip_library, size_t layers, size_t length, size_t width,
+                             size_t ffn_width, size_t heads, size_t kernel, int apply_norm_out, const float *states, float *output,
+                             char *error, size_t error_capacity) {
     mynah_weights *file = NULL;
     mynah_backend *backend = NULL;
     int rc = -1;
     if (error != NULL && error_capacity > 0) error[0] = '\0';
     if (mynah_weights_open(weights_path, &file, error, error_capacity) != 0) return -1;
-    if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &backend, error, error_capacity) == 0) {
+    if (hip_library != NULL) backend = ref_backend_open_hip(hip_library, error, error_capacity);
+    else if (mynah_backend_open(MYNAH_TTS_DEVICE_CPU, &backend, error, error_capacity) != 0) backend = NULL;
+    if (backend != NULL) {
         float *copy = (float *)malloc(length * width * sizeof(float));   /* the function takes a non-const pointer */
         if (copy != NULL) {
             memcpy(copy, states, length * width * sizeof(float));
@@ -334,6 +341,13 @@ int ref_transformer_stack(const char *weights_path, size_t layers, size_t length
     if (backend != NULL) mynah_backend_close(backend);
     mynah_weights_close(file);
     return rc;
+}
+
+int ref_transformer_stack(const char *weights_path, size_t layers, size_t length, size_t width, size_t ffn_width,
+                          size_t heads, size_t kernel, int apply_norm_out, const float *states, float *output, char *error,
+                          size_t error_capacity) {
+    return ref_transformer_stack_on(weights_path, NULL, layers, length, width, ffn_width, heads, kernel, apply_norm_out, states, output,
+                                    error, error_capacity);
 }
 
 /* ---- the reference engine as a consumer of a device backend ---------------------------------------------------

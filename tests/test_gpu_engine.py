@@ -103,6 +103,26 @@ def test_decoder_run_resident_path(pkg, orc, ref_strict, synth, nerr, quant_env,
         cpu.close()
 
 
+@pytest.mark.parametrize("tokens,layers,kernel", [(37, 2, 1), (130, 1, 3), (256, 2, 3)])
+def test_transformer_stack_on_the_library(pkg, orc, ref_strict, synth, nerr, tmp_path, tokens, layers, kernel):
+    """The reference's own text-encoder stack (transformer_stack as encode_text calls it, src/graph.c:634-711, :738-740:
+    causal attention, gain-only LayerNorm, plain or kernel-3 conv FFN) with the library as its backend against the same
+    function on the CPU backend: every projection is a host-pointer `matmul` of `tokens` rows, QK^T and PV one `sgemm` each
+    per head, the conv FFN two `sgemm` calls over the unfolded rows -- the seam's many-row products (f32 matrix cores from 24
+    rows on, the scalar kernels below) as the unmodified engine drives them.  f32 on both sides: 1e-5 normalised."""
+    _announce("engine: transformer_stack on the library, %d tokens, %d layers, kernel %d" % (tokens, layers, kernel))
+    cfg = {"layers": layers, "width": 768, "heads": 12, "head_width": 64, "ffn": 3072, "vocab": 300, "max_positions": 256,
+           "causal": True, "ffn_kernel": kernel}
+    w = synth.encoder_weights_f16(cfg, seed=30 + kernel, kernel=kernel)
+    ids = np.random.default_rng(6).integers(0, cfg["vocab"], size=tokens).astype(np.int32)
+    states = w["tok_table"][ids]
+    want = orc.ref_transformer_stack(cfg, w, states, kernel, strict=True, workdir=str(tmp_path))
+    got = orc.ref_transformer_stack(cfg, w, states, kernel, strict=True, workdir=str(tmp_path), hip_library=pkg.LIB_PATH)
+    assert np.isfinite(got).all()
+    e = nerr(got, want)
+    assert e < 1e-5, "%.3g" % e
+
+
 @pytest.mark.parametrize("qtype_name", ["f32", "int8"])
 def test_decoder_run_prefill_then_resident_steps(pkg, orc, ref_strict, synth, nerr, quant_env, qtype_name):
     """decoder_run with 24 rows at once -- the reference's context prefill (src/graph.c:3506-3654) -- on the library and
