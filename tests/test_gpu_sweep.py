@@ -2,7 +2,8 @@
 cross attention, 1-8 streams, every storage type; lengths drawn from {0, 1, capacity - 1, anything} and memories from the chunk
 edges) against the oracle, batched against solo bit for bit, the caches' untouched rows unchanged and a replay equal to the
 first run; and the local frame (vocabularies from 96 to 8192 ids, 2-16 positions, 1-8 items, planted ties, an end-of-sequence
-id that wins wherever it is allowed) with every token choice replayed on the CPU from the device's own masked logits."""
+id that wins wherever it is allowed) with every token choice replayed on the CPU from the device's own masked logits; and the
+codec's causal convolution at channel counts, lengths and tap counts between the named cases, with guard values around the output."""
 import numpy as np
 import pytest
 
@@ -96,3 +97,52 @@ def test_local_frame_shape_sweep(pkg, backend, orc, synth, seed):
         for d in drows + [dlogits]:
             d.free()
         backend.set_quant(0)
+
+
+@pytest.mark.parametrize("seed", [31])
+def test_codec_conv_shape_sweep(backend, orc, nerr, seed):
+    """Twenty seeded causal convolutions at shapes the named cases leave out -- channel counts that end inside a block of
+    eight or a tile of 32, rows shorter than a tap's reach or ending one position into a tile, every tap count from 1 to 16
+    within the reach limit of 128 positions -- against the oracle (1e-5 normalised: the matrix cores add in another order);
+    the output buffer carries guard values on both sides, which must survive; and with 3, 7 or 11 taps three convolutions
+    side by side in one launch give the bits of three launches."""
+    import test_gpu_codec as K
+    rng = np.random.default_rng(seed)
+    guard = 256
+    for case in range(20):
+        in_ch = int(rng.choice([1, 7, 8, 9, 31, 33, 64, 108, int(rng.integers(1, 261))]))
+        out_ch = int(rng.choice([1, 31, 32, 33, 63, 65, 108, int(rng.integers(1, 261))]))
+        length = int(rng.choice([1, 2, 31, 33, 63, 64, 65, 127, 129, 255, 257, int(rng.integers(1, 1501))]))
+        kernel = int(rng.choice([1, 2, 3, 3, 5, 7, 7, 11, 11, 16]))
+        dilation = int(rng.choice([d for d in (1, 2, 3, 5, 8) if (kernel - 1) * d <= 128]))
+        what = "conv sweep %d/%d: in %d out %d length %d kernel %d dilation %d" % (seed, case, in_ch, out_ch, length, kernel, dilation)
+        K._announce(what)
+        x = rng.standard_normal((in_ch, length)).astype(np.float32)
+        w = (rng.standard_normal((out_ch, in_ch, kernel)) / np.sqrt(in_ch * kernel)).astype(np.float32)
+        b = rng.standard_normal(out_ch).astype(np.float32)
+        want = orc.conv1d_causal(x, w, b, dilation)
+        din = backend.alloc(x.size).write(x)
+        fence = np.full(guard, 12345.0, np.float32)
+        padded = np.concatenate([fence, np.zeros(out_ch * length, np.float32), fence])
+        dbuf = backend.alloc(padded.size).write(padded)
+        backend.conv1d(din.ptr, dbuf.ptr + 4 * guard, in_ch, out_ch, length, kernel, dilation, w, b)
+        back = dbuf.read()
+        assert np.array_equal(back[:guard], fence) and np.array_equal(back[-guard:], fence), what + ": wrote outside its rows"
+        single = back[guard:-guard].reshape(out_ch, length)
+        e = nerr(single, want)
+        assert e < 1e-5, (what, e)
+        if kernel in (3, 7, 11):
+            outs = [backend.alloc(out_ch * length) for _ in range(3)]
+            weights = [w, (w * 0.5).astype(np.float32), (w[::-1] * 1.0).astype(np.float32).copy()]
+            items = [{"din": din.ptr, "dout": o.ptr, "kernel": kernel, "dilation": dilation, "weight": wt, "bias": b} for o, wt in zip(outs, weights)]
+            backend.conv1d_fused_batch(items, in_ch, out_ch, length)
+            together = [o.read() for o in outs]
+            for o, wt in zip(outs, weights):
+                backend.conv1d_fused(din.ptr, o.ptr, in_ch, out_ch, length, kernel, dilation, wt, b)
+            for got, o in zip(together, outs):
+                assert np.array_equal(got.view(np.uint32), o.read().view(np.uint32)), what + ": side by side"
+            assert np.array_equal(together[0].view(np.uint32), single.reshape(-1).view(np.uint32)), what + ": fused against the seam's conv1d"
+            for o in outs:
+                o.free()
+        din.free()
+        dbuf.free()
