@@ -141,7 +141,7 @@ __global__ void __launch_bounds__(256) k_argmax(const float *logits, int vocab, 
     s_idx[threadIdx.x] = at;
     __syncthreads();
     for (int half = 128; half > 0; half >>= 1) {
-        if (threadIdx.x < half) {
+        if ((int)threadIdx.x < half) {
             const float ov = s_val[threadIdx.x + half];
             const int oi = s_idx[threadIdx.x + half];
             const float mv = s_val[threadIdx.x];

@@ -240,7 +240,7 @@ __global__ void __launch_bounds__(256) k_local_sample(const SampleArgs a) {
         const unsigned own = candidate_key(mine);
         for (int bit = 31; bit >= 16; --bit) {
             const unsigned trial = bound | (1u << bit);
-            if (__popcll(__ballot(own >= trial)) >= want) bound = trial;
+            if ((int)__popcll(__ballot(own >= trial)) >= want) bound = trial;
         }
     }
     if (lane == 0) { s_head[wave] = head; s_bound[wave] = bound; }
