@@ -294,6 +294,29 @@ __host__ __device__ constexpr int lane_group_log2(int chunks) {
     return lg;
 }
 
+// int4, one stream, the group's activations already in registers (xa | xb: its 32 staged bytes; sum8: eight times their sum):
+// facc += (float)(sum n x - 8 sum x) * scale with n the offset-binary nibbles -- the integer of dot_q4 (src/qmat.c:156-185),
+// since n = q + 8.  A caller whose lanes keep their chunk columns over many rows reads and sums the activations once.
+__device__ __forceinline__ void dot_chunk_q4_held(const uint4 wv, const float sc, const uint4 xa, const uint4 xb, const int sum8, float &facc) {
+    const unsigned m = 0x0f0f0f0fu;
+    int gi = 0;
+    gi = dot4(wv.x & m, xa.x, gi); gi = dot4((wv.x >> 4) & m, xa.y, gi);
+    gi = dot4(wv.y & m, xa.z, gi); gi = dot4((wv.y >> 4) & m, xa.w, gi);
+    gi = dot4(wv.z & m, xb.x, gi); gi = dot4((wv.z >> 4) & m, xb.y, gi);
+    gi = dot4(wv.w & m, xb.z, gi); gi = dot4((wv.w >> 4) & m, xb.w, gi);
+    gi -= sum8;
+    const float term = (float)gi * sc;
+    facc = facc + term;
+}
+// eight times the sum of a group's 32 staged int8 activations
+__device__ __forceinline__ int group_sum8(const uint4 xa, const uint4 xb) {
+    const unsigned ones = 0x01010101u;
+    int s = 0;
+    s = dot4(ones, xa.x, s); s = dot4(ones, xa.y, s); s = dot4(ones, xa.z, s); s = dot4(ones, xa.w, s);
+    s = dot4(ones, xb.x, s); s = dot4(ones, xb.y, s); s = dot4(ones, xb.z, s); s = dot4(ones, xb.w, s);
+    return 8 * s;
+}
+
 // One 16-byte weight chunk against the staged activations of BT streams.
 //   int8 : iacc += sum w*qx                         (dot_q8, src/qmat.c:136-152)
 //   int4 : facc += (float)(group int32) * scale[g]  (dot_q4, src/qmat.c:156-185; one chunk = one group of 32)
@@ -314,6 +337,22 @@ __device__ __forceinline__ void dot_chunk(const uint4 wv, const float sc, const 
             s = dot4(wv.w, xv.w, s);
             iacc[b] = s;
         }
+    } else if constexpr (QT == MYNAH_HIP_INT4 && BT == 1) {
+        // One stream: the nibbles stay offset-binary (q + 8, 0 .. 15 -- a signed byte as well) and the offset comes off the
+        // group's integer at the end: sum (n - 8) x = sum n x - 8 sum x, exact in int32 (|sum n x| <= 32 * 15 * 127).  Twelve
+        // mask / shift operations and eight more dot products instead of the thirty-six that make signed bytes of the nibbles.
+        const uint4 *xp = reinterpret_cast<const uint4 *>(smem + (size_t)c * 32);
+        const uint4 xa = xp[0], xb = xp[1];
+        const unsigned m = 0x0f0f0f0fu;
+        int gi = 0;
+        gi = dot4(wv.x & m, xa.x, gi); gi = dot4((wv.x >> 4) & m, xa.y, gi);
+        gi = dot4(wv.y & m, xa.z, gi); gi = dot4((wv.y >> 4) & m, xa.w, gi);
+        gi = dot4(wv.z & m, xb.x, gi); gi = dot4((wv.z >> 4) & m, xb.y, gi);
+        gi = dot4(wv.w & m, xb.z, gi); gi = dot4((wv.w >> 4) & m, xb.w, gi);
+        gi -= group_sum8(xa, xb);
+        const float term = (float)gi * sc;   // acc += (float)gi * scales[g]  (src/qmat.c:181)
+        facc[0] = facc[0] + term;
+        if (group_out != nullptr) *group_out = gi;
     } else if constexpr (QT == MYNAH_HIP_INT4) {
         unsigned e0, o0, e1, o1, e2, o2, e3, o3;
         unpack_q4(wv.x, e0, o0);

@@ -66,6 +66,20 @@ __device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRe
     const int G = 1 << lg, gl = lane & (G - 1), gidx = lane >> lg;
     const int rpp = 64 >> lg;
     const int passes = (nrows + 4 * rpp - 1) / (4 * rpp);
+    // int4: a lane's chunk columns are the same in every pass, so their staged activations (and eight times their sums, what
+    // the offset-binary nibbles need taken off) are read once here instead of once per row
+    uint4 held_a[QT == MYNAH_HIP_INT4 ? 4 : 1], held_b[QT == MYNAH_HIP_INT4 ? 4 : 1];
+    int held_sum8[QT == MYNAH_HIP_INT4 ? 4 : 1];
+    if constexpr (QT == MYNAH_HIP_INT4) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = gl + u * G;
+            const uint4 *xp = reinterpret_cast<const uint4 *>(smem + (size_t)(c < chunks ? c : 0) * 32);
+            held_a[u] = xp[0];
+            held_b[u] = xp[1];
+            held_sum8[u] = group_sum8(held_a[u], held_b[u]);
+        }
+    }
 #pragma unroll
     for (int p = 0; p < PF; ++p) {
         const int pass = pass0 + p;
@@ -76,7 +90,11 @@ __device__ __forceinline__ void project_bank(const StepAttnArgs &a, const PassRe
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int c = gl + u * G;
-                if (c < chunks) dot_chunk<QT, 1>(bank[p].wv[u], bank[p].sc[u], c, smem, a.width, iacc, facc, nullptr);
+                if constexpr (QT == MYNAH_HIP_INT4) {
+                    if (c < chunks) dot_chunk_q4_held(bank[p].wv[u], bank[p].sc[u], held_a[u], held_b[u], held_sum8[u], facc[0]);
+                } else {
+                    if (c < chunks) dot_chunk<QT, 1>(bank[p].wv[u], bank[p].sc[u], c, smem, a.width, iacc, facc, nullptr);
+                }
             }
             group_reduce<QT, 1>(iacc, facc, lg);
             if (gl == 0 && r < row0 + nrows) {
