@@ -26,6 +26,9 @@
 // (the contract of src/qmat.c:1107-1179).
 #include <stdlib.h>
 
+#include <stdlib.h>
+#include <string.h>
+
 #include "device_common.h"
 
 namespace mynah {
@@ -138,14 +141,22 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     LinearArgs a = a_arg;
     int rows_per_wg = rows_per_wg_arg;
     size_t in_stride = 0, out_stride = 0;   // (strided builds: rows b of the launch are in0 + b * in_stride, out0 + b * out_stride)
+    // Strided builds: the grid's second dimension names a group of BT streams (launch_linear_t): five to eight streams run as
+    // two groups of four side by side, each workgroup staging four rows instead of eight.
+    const float *in_base = in0;
+    float *out_base = out0;
     if constexpr (kStrided) {
         // As for one or two streams below: what the first requests are formed from arrives in the fourteen dwords that are in
         // registers at wavefront start -- first rows, weights, scales, the LayerNorm vectors in the two places that carry fold
         // arguments for fewer streams, every small number in the slot table pointer's place (pack_strided).
         const StridedShape shape = unpack_strided(reinterpret_cast<unsigned long long>(fold_slots));
-        a.w = w; a.scales = scales; a.n = shape.n; a.batch = shape.batch;
+        a.w = w; a.scales = scales; a.n = shape.n;
         rows_per_wg = shape.rows_per_wg;
         in_stride = shape.in_stride; out_stride = shape.out_stride;
+        const int first_stream = (int)blockIdx.y * BT;
+        a.batch = min(BT, shape.batch - first_stream);
+        in_base = in0 + (size_t)first_stream * in_stride;
+        out_base = out0 + (size_t)first_stream * out_stride;
         a.fold_partial = nullptr; a.fold_partial_ml = nullptr; a.fold_slots = nullptr;
         a.fold_heads = 0; a.fold_head_width = 0; a.fold_max_units = 0; a.fold_is_self = 0; a.fold_stream0 = 0;
         if constexpr (SPEC == SPEC_UP) {
@@ -245,13 +256,13 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
     const bool live = !kWaves || stream < a.batch;
     // output row of stream b
     const auto out_of = [&](const int b) -> float * {
-        if constexpr (kStrided) return out0 + (size_t)b * out_stride;
+        if constexpr (kStrided) return out_base + (size_t)b * out_stride;
         else return stream_out<BT>(a, b);
     };
     if constexpr (kWaves) {
-        const float *row = kStrided ? in0 : a.in[0];   // a place of the tile without a stream reads stream 0's row and stages zeros
+        const float *row = kStrided ? in_base : a.in[0];   // a place of the tile without a stream reads stream 0's row and stages zeros
         if constexpr (kStrided) {
-            if (live) row = in0 + (size_t)stream * in_stride;
+            if (live) row = in_base + (size_t)stream * in_stride;
         } else {
 #pragma unroll
             for (int q = 1; q < BT; ++q)
@@ -550,6 +561,12 @@ static bool gemm_vec_ok(const float *a, size_t lda, const float *b, size_t ldb, 
            inner_b % 4 == 0;
 }
 
+// MYNAH_HIP_STREAM_GROUPS=0: five to eight streams as one tile of eight again
+static bool stream_groups_enabled() {
+    static const bool on = !(getenv("MYNAH_HIP_STREAM_GROUPS") != nullptr && strcmp(getenv("MYNAH_HIP_STREAM_GROUPS"), "0") == 0);
+    return on;
+}
+
 template <int QT, int BT, int NVT, int KFIX, int SPEC>
 int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity) {
     constexpr int epc = Chunk<QT>::n;
@@ -559,6 +576,10 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
     const int target_wgs = st->cu_count * 3;
     int passes = (a.n + rows_per_wg_pass * target_wgs - 1) / (rows_per_wg_pass * target_wgs);
     if (passes < 1) passes = 1;
+    // strided builds take more streams than their tile holds as groups of BT side by side (the grid's second dimension);
+    // with twice the rows per workgroup when the groups together would otherwise be more workgroups than the chip has CUs
+    const int groups = kStridedLead<BT, QT, SPEC> ? (a.batch + BT - 1) / BT : 1;
+    if (groups > 1 && (long)((a.n + rows_per_wg_pass * passes - 1) / (rows_per_wg_pass * passes)) * groups > st->cu_count) passes *= 2;
     const int rows_per_wg = rows_per_wg_pass * passes;
     const int grid = (a.n + rows_per_wg - 1) / rows_per_wg;
     const size_t lds = (size_t)BT * a.k * (kQuantised<QT> ? 1 : 4);
@@ -576,7 +597,7 @@ int launch_linear_t(State *st, const LinearArgs &a, char *error, size_t capacity
             return -1;
         }
         const StepSlots *const packed = reinterpret_cast<const StepSlots *>(pack_strided(shape));
-        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid), dim3(kLinearThreads<BT, QT>), lds, st->stream, a.in[0],
+        hipLaunchKernelGGL((k_linear<QT, BT, NVT, KFIX, SPEC>), dim3(grid, groups), dim3(kLinearThreads<BT, QT>), lds, st->stream, a.in[0],
                            SPEC == SPEC_UP ? a.ln_gain : nullptr, SPEC == SPEC_UP ? a.ln_bias : nullptr, packed, a.w, a.scales, a.out[0], a.n, a.batch, a,
                            rows_per_wg, lg);
     } else if constexpr (kPackedLead<BT, SPEC>) {
@@ -610,6 +631,12 @@ int launch_linear_b(State *st, const LinearArgs &a, char *error, size_t capacity
     if (a.batch <= 1) return launch_linear_t<QT, 1, NVT, KFIX, SPEC>(st, a, error, capacity);
     if (a.batch == 2) return launch_linear_t<QT, 2, NVT, KFIX, SPEC>(st, a, error, capacity);
     if (a.batch <= 4) return launch_linear_t<QT, 4, NVT, KFIX, SPEC>(st, a, error, capacity);
+    // five to eight streams, rows at a fixed stride, int8 / int4 weights, residual epilogue (the output projections and the
+    // FFN-down product): two groups of four in one launch -- what a workgroup stages, every stream of its tile, halves, and a
+    // stream's bits do not depend on the tile it runs in.  (Measured with eight ragged streams: step 497 -> 483 us; the FFN-up
+    // product the same way, whose LayerNorm prologue each group then runs for its four rows, 497 us with twice the rows per
+    // workgroup and 486 us with twice the workgroups: it keeps the tile of eight.)
+    if (kStridedLead<4, QT, SPEC> && SPEC == SPEC_RESIDUAL && stream_groups_enabled()) return launch_linear_t<QT, 4, NVT, KFIX, SPEC>(st, a, error, capacity);
     return launch_linear_t<QT, 8, NVT, KFIX, SPEC>(st, a, error, capacity);
 }
 
