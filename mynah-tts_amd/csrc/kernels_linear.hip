@@ -314,6 +314,34 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
         }
     }
 
+    // The stream-group builds (strided rows, residual epilogue) may be launched with two row passes per workgroup: the second
+    // pass's first weight group and its epilogue operands are requested here as well -- asked for inside the row loop they
+    // are two dependent round trips behind the first pass's products.  Requested whatever the launch (rows past the
+    // workgroup's range repeat its last row): a request under a condition could not be counted by the waits below.
+    // (not in the build for rows of 768: the stack's output projections, whose 48 row blocks never need a second pass)
+    constexpr bool kSecondAhead = kStrided && SPEC == SPEC_RESIDUAL && KFIX != 768;
+    uint4 wv_second[kSecondAhead ? 4 : 1];
+    float sc_second[kSecondAhead ? 4 : 1];
+    float scale_second = 1.0f, res_second[kSecondAhead ? PB : 1];
+    if constexpr (kSecondAhead) {
+        const int row = row_begin + pass_stride + wave_row * rows_per_pass + gidx;
+        const int rowc = row < row_end ? row : row_end - 1;
+        const uint4 *wrow = reinterpret_cast<const uint4 *>(static_cast<const unsigned char *>(a.w) + (size_t)rowc * row_bytes);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = gl + u * G;
+            wv_second[u] = c < chunks ? wrow[c] : make_uint4(0, 0, 0, 0);
+            sc_second[u] = (QT == MYNAH_HIP_INT4 && c < chunks) ? a.scales[(size_t)rowc * chunks + c] : 0.0f;
+        }
+        if constexpr (QT == MYNAH_HIP_INT8) scale_second = a.scales[rowc];
+        if (lanes_finish) {
+            res_second[0] = out_of(stream_base + gl < a.batch ? stream_base + gl : 0)[rowc];
+        } else {
+#pragma unroll
+            for (int b = 0; b < PB; ++b) res_second[b] = stream_base + b < a.batch ? out_of(stream_base + b)[rowc] : 0.0f;
+        }
+    }
+
     requests_issued();
 
     // ------------------------------------------------------------------ prologue arithmetic (the weight requests above stay in flight)
@@ -327,6 +355,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
 
     // ------------------------------------------------------------------ body
     bool first = true;
+    bool second = false;   // (stream-group builds) the pass whose operands were requested ahead as well
     const unsigned char *const staged = smem + (size_t)stream_base * k * (kQuantised<QT> ? 1 : 4);   // this wavefront's streams
     for (int base = row_begin + wave_row * rows_per_pass; base < row_end; base += pass_stride) {
         const int row = base + gidx;
@@ -338,7 +367,10 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
 #pragma unroll
         for (int b = 0; b < PB; ++b) { iacc[b] = 0; facc[b] = 0.0f; }
         for (int c0 = gl; c0 < chunks; c0 += 4 * G) {
-            if (!(first && c0 == gl)) {   // the first group of the first pass was loaded before the prologue
+            if (kSecondAhead && second && c0 == gl) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) { wv[u] = wv_second[kSecondAhead ? u : 0]; sc[u] = sc_second[kSecondAhead ? u : 0]; }
+            } else if (!(first && c0 == gl)) {   // the first group of the first pass was loaded before the prologue
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int c = c0 + u * G;
@@ -369,6 +401,8 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                 if (first) {
                     wscale = pre_scale;
                     bias = pre_bias;
+                } else if (kSecondAhead && second) {
+                    wscale = scale_second;
                 } else {
                     if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[row];
                     if (arg_bias != nullptr) bias = arg_bias[row];
@@ -379,7 +413,7 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                 if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
                 float *o = out_of(sb) + row;
                 if (arg_aux_out != nullptr && sb == 0) arg_aux_out[row] = val;
-                if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : *o) + val;
+                if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[0] : (kSecondAhead && second) ? res_second[0] : *o) + val;
                 *o = val;
             }
         } else if (gl == 0 && valid) {
@@ -387,6 +421,8 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
             if (first) {
                 wscale = pre_scale;
                 bias = pre_bias;
+            } else if (kSecondAhead && second) {
+                wscale = scale_second;
             } else {
                 if constexpr (QT == MYNAH_HIP_INT8) wscale = a.scales[row];
                 if (arg_bias != nullptr) bias = arg_bias[row];
@@ -401,11 +437,12 @@ k_linear(const float *const in0, const float *const fold_partial, const float *c
                     if (arg_epilogue == EPI_GELU) val = gelu_tanh(val);
                     float *o = out_of(sb) + row;
                     if (arg_aux_out != nullptr && sb == 0) arg_aux_out[row] = val;
-                    if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[b] : *o) + val;
+                    if (arg_epilogue == EPI_RESIDUAL) val = (first ? pre_res[b] : (kSecondAhead && second) ? res_second[kSecondAhead ? b : 0] : *o) + val;
                     *o = val;
                 }
             }
         }
+        second = first;   // the pass behind the first
         first = false;
     }
 }
@@ -635,7 +672,8 @@ int launch_linear_b(State *st, const LinearArgs &a, char *error, size_t capacity
     // FFN-down product): two groups of four in one launch -- what a workgroup stages, every stream of its tile, halves, and a
     // stream's bits do not depend on the tile it runs in.  (Measured with eight ragged streams: step 497 -> 483 us; the FFN-up
     // product the same way, whose LayerNorm prologue each group then runs for its four rows, 497 us with twice the rows per
-    // workgroup and 486 us with twice the workgroups: it keeps the tile of eight.)
+    // workgroup and 486 us with twice the workgroups; with the second pass's operands requested ahead as below, 476 against 477 us:
+    // it keeps the tile of eight.)
     if (kStridedLead<4, QT, SPEC> && SPEC == SPEC_RESIDUAL && stream_groups_enabled()) return launch_linear_t<QT, 4, NVT, KFIX, SPEC>(st, a, error, capacity);
     return launch_linear_t<QT, 8, NVT, KFIX, SPEC>(st, a, error, capacity);
 }
