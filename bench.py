@@ -281,9 +281,9 @@ STAGES = [("self-attention", "k_step_attention<self>", "LayerNorm + int8 act-qua
 # then WRITE_SIZE), each scaled by what the same counter reads for the library's plain 256 MiB read+write kernel.  A figure
 # belongs to the kernel sources it was measured on: it is reported only while their hash is the one recorded here.
 MEASURED_TRAFFIC = {
-    1: {"kernel": "k_linear<k=768, residual>", "bytes": 937914, "profile": "profiles/decode_step_int8_hbm_counters.md",
-        "sources": ("kernels_linear.hip", "device_common.h", "kernels.h", "common.h"), "csrc_sha256": "24a9df8e6041b334"},
-    8: {"kernel": "k_step_attention<self>", "bytes": 54465378, "profile": "profiles/decode_step_int8_hbm_counters.md",
+    1: {"kernel": "k_linear<k=768, residual>", "bytes": 937934, "profile": "profiles/decode_step_int8_hbm_counters.md",
+        "sources": ("kernels_linear.hip", "device_common.h", "kernels.h", "common.h"), "csrc_sha256": "21040170f4024ffc"},
+    8: {"kernel": "k_step_attention<self>", "bytes": 54469598, "profile": "profiles/decode_step_int8_hbm_counters.md",
         "sources": ("kernels_step_attention.hip", "step_attention_core.h", "step_items.h", "tagged_exchange.h", "device_common.h",
                     "kernels.h", "common.h"), "csrc_sha256": "186dff1ded534a42"},
 }
